@@ -1,0 +1,353 @@
+"""ctypes loader for the CPU oracle (test infrastructure only).
+
+The oracle is a plain-C restatement of the reference engine's CPU algorithms for
+the DFlash step; see ``dflash_oracle.h`` for what each function follows and how it
+is pinned.  Only the test-suite, the smoke check and the benchmark's CPU-baseline
+leg import this module.  The shipped library never does.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_DIR, "liboracle.so")
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+RNG_XOSHIRO, RNG_PHILOX = 0, 1
+CARRY_NONE, CARRY_CORRECTION, CARRY_BONUS = 0, 1, 2
+STOP_NONE, STOP_EOS, STOP_TOKEN_LIMIT = 0, 1, 2
+
+ERR = {
+    0: "Ok", 1: "EmptyLogits", 2: "InvalidTemperature", 3: "InvalidTopP", 4: "InvalidMinP",
+    5: "NanLogit", 6: "VocabularyTooLarge", 7: "NoCandidates", 8: "ProposalTokenOutOfRange",
+    9: "InvalidProposalWeight", 10: "MissingProposalToken", 11: "InvalidInput", 12: "InvalidToken",
+    13: "ProposalMismatch",
+}
+
+
+def build(force: bool = False) -> str:
+    """Compile liboracle.so with gcc (a few seconds)."""
+    srcs = [os.path.join(_DIR, f) for f in ("quant.c", "rng.c", "sampler.c", "forward.c", "dflash_oracle.h")]
+    stale = force or not os.path.exists(_LIB_PATH) or any(
+        os.path.getmtime(s) > os.path.getmtime(_LIB_PATH) for s in srcs)
+    if stale:
+        subprocess.run(["make", "-C", _DIR, "-B", "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+class SamplingConfig(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("min_p", C.c_float),
+                ("rng_kind", C.c_int32), ("top_k", C.c_uint64), ("seed", C.c_uint64)]
+
+
+class Sampler(C.Structure):
+    _fields_ = [("cfg", SamplingConfig), ("s", C.c_uint64 * 4), ("draws", C.c_uint64)]
+
+
+class WeightedCandidate(C.Structure):
+    _fields_ = [("token", C.c_int32), ("pad", C.c_int32), ("weight", C.c_double)]
+
+
+class AcceptDecision(C.Structure):
+    _fields_ = [("n_accepted", C.c_int32), ("accepted_drafts", C.c_int32 * 64), ("carry_kind", C.c_int32),
+                ("carry_token", C.c_int32), ("stop_reason", C.c_int32), ("retain_input_count", C.c_int32),
+                ("err_row", C.c_int32), ("err_code", C.c_int32), ("err_index", C.c_int64)]
+
+    def accepted(self):
+        return list(self.accepted_drafts[: self.n_accepted])
+
+    def key(self):
+        return (self.accepted(), self.carry_kind, self.carry_token if self.carry_kind else 0, self.stop_reason,
+                self.retain_input_count)
+
+
+class ModelCfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "n_q", "n_kv", "head_dim", "ffn", "vocab",
+                                          "n_expert", "n_expert_used", "ffn_expert", "ffn_shared")] + \
+               [("eps", C.c_float), ("rope_theta", C.c_float)]
+
+
+class QTensor(C.Structure):
+    _fields_ = [("type", C.c_int32), ("pad", C.c_int32), ("data", C.c_void_p)]
+
+
+class Layer(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("post_norm", C.c_void_p),
+                ("wq", QTensor), ("wk", QTensor), ("wv", QTensor), ("wo", QTensor), ("gate", QTensor), ("up", QTensor),
+                ("down", QTensor), ("router", QTensor), ("shexp_gate", C.c_void_p), ("gate_exps", QTensor),
+                ("up_exps", QTensor), ("down_exps", QTensor)]
+
+
+class Model(C.Structure):
+    _fields_ = [("cfg", ModelCfg), ("layers", C.POINTER(Layer)), ("token_embd", QTensor), ("output", QTensor),
+                ("output_norm", C.c_void_p)]
+
+
+class DraftCfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "n_q", "n_kv", "head_dim", "ffn", "block_size",
+                                          "n_taps", "causal")] + \
+               [("swa_window", C.c_uint32), ("eps", C.c_float), ("rope_theta", C.c_float)]
+
+
+class DraftLayer(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("post_norm", C.c_void_p),
+                ("wq", QTensor), ("wk", QTensor), ("wv", QTensor), ("wo", QTensor), ("gate", QTensor), ("up", QTensor),
+                ("down", QTensor), ("is_swa", C.c_int32), ("pad", C.c_int32)]
+
+
+class DraftHead(C.Structure):
+    _fields_ = [("cfg", DraftCfg), ("layers", C.POINTER(DraftLayer)), ("fc", QTensor), ("hidden_norm", C.c_void_p),
+                ("output_norm", C.c_void_p)]
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _declare(_lib)
+    return _lib
+
+
+def _declare(L):
+    vp, sz, i32, i64, u64, f32, f64 = C.c_void_p, C.c_size_t, C.c_int32, C.c_int64, C.c_uint64, C.c_float, C.c_double
+    L.orc_f16_to_f32.restype = f32
+    L.orc_f16_to_f32.argtypes = [C.c_uint16]
+    L.orc_f32_to_f16.restype = C.c_uint16
+    L.orc_f32_to_f16.argtypes = [f32]
+    L.orc_dequant.restype = C.c_int
+    L.orc_dequant.argtypes = [C.c_int, vp, sz, vp]
+    L.orc_row_bytes.restype = sz
+    L.orc_row_bytes.argtypes = [C.c_int, sz]
+    L.orc_splitmix64_next.restype = u64
+    L.orc_splitmix64_next.argtypes = [C.POINTER(u64)]
+    L.orc_xoshiro_seed.argtypes = [u64, C.POINTER(u64)]
+    L.orc_xoshiro_next.restype = u64
+    L.orc_xoshiro_next.argtypes = [C.POINTER(u64)]
+    L.orc_unit_f64.restype = f64
+    L.orc_unit_f64.argtypes = [u64]
+    L.orc_philox4x32_10.argtypes = [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+    L.orc_sampler_init.argtypes = [C.POINTER(Sampler), C.POINTER(SamplingConfig)]
+    L.orc_sampler_at_draw.argtypes = [C.POINTER(Sampler), C.POINTER(SamplingConfig), u64]
+    L.orc_sampler_next_unit.restype = f64
+    L.orc_sampler_next_unit.argtypes = [C.POINTER(Sampler)]
+    L.orc_greedy_token.argtypes = [vp, sz, C.POINTER(i32), C.POINTER(i64)]
+    L.orc_argmax_top2.argtypes = [vp, sz, C.POINTER(i32), C.POINTER(f32)]
+    L.orc_top16.argtypes = [vp, sz, vp, vp]
+    L.orc_sampler_diagnose.argtypes = [C.POINTER(Sampler), vp, sz, f64, C.POINTER(WeightedCandidate), sz,
+                                       C.POINTER(sz), C.POINTER(f64), C.POINTER(i32), C.POINTER(sz), C.POINTER(i64)]
+    L.orc_sampler_sample.argtypes = [C.POINTER(Sampler), vp, sz, C.POINTER(i32), C.POINTER(sz), C.POINTER(i64)]
+    L.orc_couple_deterministic_proposal.argtypes = [C.POINTER(Sampler), vp, sz, i32, C.POINTER(C.c_int),
+                                                    C.POINTER(i32), C.POINTER(i64)]
+    L.orc_couple_sparse_proposal.argtypes = [C.POINTER(Sampler), vp, sz, i32, C.POINTER(WeightedCandidate), sz,
+                                             C.POINTER(C.c_int), C.POINTER(i32), C.POINTER(i64)]
+    L.orc_couple_dense_proposal.argtypes = [C.POINTER(Sampler), vp, vp, sz, f32, i32, C.POINTER(C.c_int),
+                                            C.POINTER(i32), C.POINTER(i64)]
+    L.orc_dense_proposal_total.restype = f64
+    L.orc_dense_proposal_total.argtypes = [vp, sz, f32, C.POINTER(i64)]
+    L.orc_decide_accept_prefix.argtypes = [vp, sz, vp, sz, sz, C.c_int, sz, vp, vp, vp, vp, C.POINTER(Sampler), sz,
+                                           vp, sz, C.POINTER(AcceptDecision)]
+    L.orc_decide_accept_prefix_dense.argtypes = [vp, sz, vp, vp, sz, f32, C.POINTER(Sampler), sz, vp, sz,
+                                                 C.POINTER(AcceptDecision)]
+    L.orc_rms_norm.argtypes = [vp, vp, sz, f32, vp]
+    L.orc_silu.restype = f32
+    L.orc_silu.argtypes = [f32]
+    L.orc_softmax_in_place.argtypes = [vp, sz]
+    L.orc_mat_vec.argtypes = [vp, sz, sz, vp, vp]
+    L.orc_rope_in_place.argtypes = [vp, sz, sz, sz, C.c_uint32, f32]
+    L.orc_gemm_fewrow.argtypes = [C.c_int, vp, vp, vp, sz, sz, sz]
+    L.orc_attn_verify_block.argtypes = [vp, vp, vp, sz, sz, sz, sz, sz, f32, vp]
+    L.orc_attn_draft.argtypes = [vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, C.c_uint32, C.c_int, C.c_uint32, vp]
+    L.orc_target_verify.argtypes = [C.POINTER(Model), vp, sz, sz, vp, vp, sz, vp, vp, sz, vp]
+    L.orc_dflash_draft.argtypes = [C.POINTER(Model), C.POINTER(DraftHead), vp, vp, sz, vp, C.c_uint32, vp]
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+# ---------------------------------------------------------------- numpy-level helpers
+
+
+def row_bytes(qtype: int, n_in: int) -> int:
+    return int(lib().orc_row_bytes(qtype, n_in))
+
+
+def dequant(qtype: int, blocks: np.ndarray, n_elems: int) -> np.ndarray:
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    out = np.empty(n_elems, dtype=np.float32)
+    rc = lib().orc_dequant(qtype, _p(blocks), n_elems, _p(out))
+    if rc:
+        raise ValueError("orc_dequant: bad geometry")
+    return out
+
+
+def gemm_fewrow(qtype: int, w: np.ndarray, x: np.ndarray, n_in: int, n_out: int) -> np.ndarray:
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n_rows = x.shape[0]
+    y = np.empty((n_rows, n_out), dtype=np.float32)
+    rc = lib().orc_gemm_fewrow(qtype, _p(w), _p(x), _p(y), n_in, n_out, n_rows)
+    if rc:
+        raise ValueError("orc_gemm_fewrow failed")
+    return y
+
+
+def attn_verify_block(q, k_cache, v_cache, ctx_len, scale):
+    """q [n_rows,n_q,hd] f32; k/v cache [ctx_len+n_rows, n_kv, hd] float16."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k_cache, dtype=np.float16)
+    v = np.ascontiguousarray(v_cache, dtype=np.float16)
+    n_rows, n_q, hd = q.shape
+    n_kv = k.shape[1]
+    out = np.empty_like(q)
+    lib().orc_attn_verify_block(_p(q), _p(k), _p(v), ctx_len, n_rows, n_q, n_kv, hd, scale, _p(out))
+    return out
+
+
+def attn_draft(q, k_ctx, v_ctx, k_noise, v_noise, pos_ctx, noise_start_pos, causal, swa_window):
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    n, n_q, hd = q.shape
+    k_ctx = np.ascontiguousarray(k_ctx, dtype=np.float32)
+    v_ctx = np.ascontiguousarray(v_ctx, dtype=np.float32)
+    k_noise = np.ascontiguousarray(k_noise, dtype=np.float32)
+    v_noise = np.ascontiguousarray(v_noise, dtype=np.float32)
+    pos_ctx = np.ascontiguousarray(pos_ctx, dtype=np.int32)
+    n_kv = k_noise.shape[1]
+    out = np.empty_like(q)
+    lib().orc_attn_draft(_p(q), _p(k_ctx), _p(v_ctx), _p(k_noise), _p(v_noise), _p(pos_ctx), len(pos_ctx), n, n_q,
+                         n_kv, hd, noise_start_pos, int(causal), swa_window, _p(out))
+    return out
+
+
+def make_sampler(temperature=0.0, top_k=0, top_p=1.0, min_p=0.0, seed=0, rng_kind=RNG_XOSHIRO, draws=0):
+    cfg = SamplingConfig(temperature, top_p, min_p, rng_kind, top_k, seed)
+    s = Sampler()
+    rc = lib().orc_sampler_at_draw(C.byref(s), C.byref(cfg), draws)
+    if rc:
+        raise ValueError(ERR[rc])
+    return s
+
+
+def clone_sampler(s: Sampler) -> Sampler:
+    t = Sampler()
+    C.memmove(C.byref(t), C.byref(s), C.sizeof(Sampler))
+    return t
+
+
+def sampler_state(s: Sampler):
+    return (tuple(s.s), int(s.draws))
+
+
+def greedy_token(logits):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    tok, err = C.c_int32(), C.c_int64(-1)
+    rc = lib().orc_greedy_token(_p(logits), logits.size, C.byref(tok), C.byref(err))
+    return rc, tok.value, err.value
+
+
+def argmax_top2(logits):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    idx, gap = C.c_int32(), C.c_float()
+    lib().orc_argmax_top2(_p(logits), logits.size, C.byref(idx), C.byref(gap))
+    return idx.value, gap.value
+
+
+def top16(logits):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    ids = np.empty(16, dtype=np.int32)
+    vals = np.empty(16, dtype=np.float32)
+    lib().orc_top16(_p(logits), logits.size, _p(ids), _p(vals))
+    return ids, vals
+
+
+def sample(s: Sampler, logits):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    tok, idx, err = C.c_int32(), C.c_size_t(), C.c_int64(-1)
+    rc = lib().orc_sampler_sample(C.byref(s), _p(logits), logits.size, C.byref(tok), C.byref(idx), C.byref(err))
+    return rc, tok.value, idx.value, err.value
+
+
+def diagnose(s: Sampler, logits, uniform=0.0, cap=None):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    cap = cap or logits.size
+    cands = (WeightedCandidate * cap)()
+    n, total, tok, idx, err = C.c_size_t(), C.c_double(), C.c_int32(), C.c_size_t(), C.c_int64(-1)
+    rc = lib().orc_sampler_diagnose(C.byref(s), _p(logits), logits.size, uniform, cands, cap, C.byref(n),
+                                    C.byref(total), C.byref(tok), C.byref(idx), C.byref(err))
+    if rc:
+        return rc, [], 0.0, -1, err.value
+    return rc, [(cands[i].token, cands[i].weight) for i in range(min(n.value, cap))], total.value, tok.value, idx.value
+
+
+def _cands(pairs):
+    arr = (WeightedCandidate * max(1, len(pairs)))()
+    for i, (t, w) in enumerate(pairs):
+        arr[i].token, arr[i].weight = t, w
+    return arr
+
+
+def couple_deterministic(s, logits, proposal):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    acc, corr, err = C.c_int(), C.c_int32(), C.c_int64(-1)
+    rc = lib().orc_couple_deterministic_proposal(C.byref(s), _p(logits), logits.size, proposal, C.byref(acc),
+                                                 C.byref(corr), C.byref(err))
+    return rc, bool(acc.value), corr.value
+
+
+def couple_sparse(s, logits, token, pairs):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    acc, corr, err = C.c_int(), C.c_int32(), C.c_int64(-1)
+    rc = lib().orc_couple_sparse_proposal(C.byref(s), _p(logits), logits.size, token, _cands(pairs), len(pairs),
+                                          C.byref(acc), C.byref(corr), C.byref(err))
+    return rc, bool(acc.value), corr.value
+
+
+def couple_dense(s, target_logits, draft_logits, draft_temperature, token):
+    t = np.ascontiguousarray(target_logits, dtype=np.float32)
+    d = np.ascontiguousarray(draft_logits, dtype=np.float32)
+    acc, corr, err = C.c_int(), C.c_int32(), C.c_int64(-1)
+    rc = lib().orc_couple_dense_proposal(C.byref(s), _p(t), _p(d), t.size, draft_temperature, token, C.byref(acc),
+                                         C.byref(corr), C.byref(err))
+    return rc, bool(acc.value), corr.value
+
+
+def decide_accept_prefix(verified_tokens, target_logits, vocab, proposals, sampler, budget, stop_ids):
+    """proposals: None or list of (token, [(token, weight), ...]) with one entry per draft row."""
+    toks = np.ascontiguousarray(verified_tokens, dtype=np.int32)
+    logits = np.ascontiguousarray(target_logits, dtype=np.float32)
+    stops = np.ascontiguousarray(stop_ids, dtype=np.int32)
+    out = AcceptDecision()
+    if proposals is None:
+        rc = lib().orc_decide_accept_prefix(_p(toks), toks.size, _p(logits), logits.size, vocab, 0, 0, None, None,
+                                            None, None, C.byref(sampler), budget, _p(stops), stops.size,
+                                            C.byref(out))
+        return rc, out
+    ptoks = np.array([p[0] for p in proposals], dtype=np.int32)
+    counts = np.array([len(p[1]) for p in proposals], dtype=np.uint64)
+    offsets = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.uint64) if len(proposals) else \
+        np.zeros(0, dtype=np.uint64)
+    flat = [c for p in proposals for c in p[1]]
+    rc = lib().orc_decide_accept_prefix(_p(toks), toks.size, _p(logits), logits.size, vocab, 1, len(proposals),
+                                        _p(ptoks), _p(offsets), _p(counts), _cands(flat), C.byref(sampler), budget,
+                                        _p(stops), stops.size, C.byref(out))
+    return rc, out
+
+
+def decide_accept_prefix_dense(verified_tokens, target_logits, draft_logits, vocab, draft_temperature, sampler,
+                               budget, stop_ids):
+    toks = np.ascontiguousarray(verified_tokens, dtype=np.int32)
+    t = np.ascontiguousarray(target_logits, dtype=np.float32)
+    d = np.ascontiguousarray(draft_logits, dtype=np.float32)
+    stops = np.ascontiguousarray(stop_ids, dtype=np.int32)
+    out = AcceptDecision()
+    rc = lib().orc_decide_accept_prefix_dense(_p(toks), toks.size, _p(t), _p(d), vocab, draft_temperature,
+                                              C.byref(sampler), budget, _p(stops), stops.size, C.byref(out))
+    return rc, out
