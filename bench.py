@@ -1,0 +1,141 @@
+#!/usr/bin/env python3
+"""Benchmark of the DFlash verify hot path on one MI355X.
+
+A step is one pass of the few-row Q4_K dequant-GEMM over the three Qwen3.6-27B-shaped
+projections of a 16-row verify block (gate/up 5120->17408, down 17408->5120, fused QKV
+5120->6144), synthetic inputs resident in HBM.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "accepted tokens/s @ batch1 block16; verify Q4_K GEMM HBM GB/s (% of peak)"
+SHAPES = [(5120, 17408), (17408, 5120), (5120, 6144)]  # (n_in, n_out)
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(shapes, weights, xs):
+    """The oracle's dequant + f32 GEMM (OpenMP over output rows) on the same weights: a bounded
+    sample of the workload (the first `rows` output rows of every shape), scaled to GB/s."""
+    import numpy as np
+
+    import oracle
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    rows_frac = 0.25
+    total_bytes, total_s = 0, 0.0
+    for (n_in, n_out), w, x in zip(shapes, weights, xs):
+        rows = max(16, int(n_out * rows_frac))
+        ws = np.ascontiguousarray(w[:rows])
+        xf = x.astype(np.float32)
+        oracle.gemm_fewrow(oracle.Q4_K, ws, xf, n_in, rows)  # warm-up
+        best = 1e30
+        for _ in range(3):
+            t0 = time.perf_counter()
+            oracle.gemm_fewrow(oracle.Q4_K, ws, xf, n_in, rows)
+            best = min(best, time.perf_counter() - t0)
+        total_bytes += ws.size
+        total_s += best
+    return {"value": total_bytes / total_s / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"first {int(rows_frac * 100)}% of the output rows of each of the 3 GEMMs, best of 3"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the DFlash step is batch-1 and this build has no multi-GPU path; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import qwen_llm_amd as dfl
+
+    torch.cuda.set_device(0)
+    ctx = dfl.Context(0)
+    rng = np.random.default_rng(1)
+    weights, xs, wd, xd, yd = [], [], [], [], []
+    for n_in, n_out in SHAPES:
+        w = dfl.synth.random_weight(dfl.synth.Q4_K, n_out, n_in, seed=1)
+        x = rng.standard_normal((16, n_in)).astype(np.float16)
+        weights.append(w)
+        xs.append(x)
+        wd.append(torch.from_numpy(w).cuda())
+        xd.append(torch.from_numpy(x).cuda())
+        yd.append(torch.empty((16, n_out), dtype=torch.float32, device="cuda"))
+    w_bytes = [int(w.size) for w in weights]
+
+    def step():
+        for (n_in, n_out), w, x, y in zip(SHAPES, wd, xd, yd):
+            ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q4_K, x, y, n_in, n_out, 16)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+
+    # dominant kernel alone: events inside the library around gemm_q4k_kernel, on its stream
+    ctx.set_kernel_timing(True)
+    per_shape = []
+    for (n_in, n_out), w, x, y, nbytes in zip(SHAPES, wd, xd, yd, w_bytes):
+        ctx.set_kernel_timing(True)
+        for _ in range(max(20, args.steps // 4)):
+            ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q4_K, x, y, n_in, n_out, 16)
+        ms, n = ctx.kernel_timing(ctx.T_GEMM)
+        per_shape.append({"n_in": n_in, "n_out": n_out, "weight_bytes": nbytes, "kernel_us": ms / n * 1e3,
+                          "GBps": nbytes / (ms / n * 1e-3) / 1e9})
+    ctx.set_kernel_timing(False)
+    k_bytes = sum(p["weight_bytes"] for p in per_shape) / len(per_shape)
+    k_us = sum(p["kernel_us"] for p in per_shape) / len(per_shape)
+    achieved = k_bytes / (k_us * 1e-6) / 1e9
+
+    out = {
+        "metric": METRIC,
+        "value": sum(w_bytes) / (ms_per_step * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "few-row Q4_K dequant GEMM, M=16, (K,N) in {(5120,17408),(17408,5120),(5120,6144)}, "
+                               "X f16 N(0,1), W Q4_K from N(0,0.02) seed 1, f32 accumulation",
+                   "weight_bytes_per_step": sum(w_bytes), "block": 16, "batch": 1},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "gemm_q4k_kernel", "bytes_per_launch": k_bytes, "us_per_launch": k_us},
+        "shapes": per_shape,
+        "pct_of_hbm_peak": 100.0 * sum(w_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "accepted_tokens_per_s": None,
+        "wall_ms_per_step": wall_ms / args.steps,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(SHAPES, weights, xs)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,99 @@
+/*
+ * dflash_hip.h - C ABI of the MI355X (gfx950) DFlash speculative-decoding step.
+ *
+ * Plain C: pointers and sizes only.  Unless a parameter is suffixed `_host`, every
+ * pointer is a caller-owned DEVICE pointer; the library never frees or retains
+ * caller memory.  Every function returns a DFLASH_* status (0 = OK) and records a
+ * message retrievable with dflash_last_error().  Calls enqueue work on the stream
+ * passed in (a hipStream_t, given as void*; NULL = the default stream) and do not
+ * synchronise unless their name ends in `_sync` or their comment says they return
+ * host-side results.
+ *
+ * Each entry point cites the interface of the reference engine
+ * (brittlewis12/qwen-llm, paths relative to its root) that it replaces.
+ */
+#ifndef DFLASH_HIP_H
+#define DFLASH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dflash_ctx dflash_ctx;
+typedef void *dflash_stream_t; /* hipStream_t */
+
+/* status codes (the reference's Result enums: MetalError::BadShape, DFlashError
+ * metal_dflash.rs:2698-2732, SamplingError sampling.rs:278-302, DFlashAcceptError
+ * metal_dflash/accept.rs:34-52) */
+enum {
+    DFLASH_OK = 0,
+    DFLASH_ERR_BAD_SHAPE = 1,       /* MetalError::BadShape */
+    DFLASH_ERR_UNSUPPORTED = 2,     /* "decline": no kernel for this dtype / size */
+    DFLASH_ERR_ALIAS = 3,           /* output aliases an input (dispatch.rs:221-225, 522-526) */
+    DFLASH_ERR_ALIGNMENT = 4,
+    DFLASH_ERR_WORKSPACE = 5,       /* context workspace too small for this call */
+    DFLASH_ERR_HIP = 6,             /* a HIP runtime call failed */
+    DFLASH_ERR_INVALID_INPUT = 7,   /* DFlashAcceptError::InvalidInput */
+    DFLASH_ERR_INVALID_TOKEN = 8,   /* DFlashAcceptError::InvalidToken / ForwardError::BadToken */
+    DFLASH_ERR_PROPOSAL_MISMATCH = 9,
+    DFLASH_ERR_STATE = 10,          /* kv_n_pos != start_position and similar guard walls */
+    /* sampling errors, numbered 32 + the sampler's own code */
+    DFLASH_ERR_EMPTY_LOGITS = 33,
+    DFLASH_ERR_INVALID_TEMPERATURE = 34,
+    DFLASH_ERR_INVALID_TOP_P = 35,
+    DFLASH_ERR_INVALID_MIN_P = 36,
+    DFLASH_ERR_NAN_LOGIT = 37,
+    DFLASH_ERR_VOCAB_TOO_LARGE = 38,
+    DFLASH_ERR_NO_CANDIDATES = 39,
+    DFLASH_ERR_PROPOSAL_TOKEN_OUT_OF_RANGE = 40,
+    DFLASH_ERR_INVALID_PROPOSAL_WEIGHT = 41,
+    DFLASH_ERR_MISSING_PROPOSAL_TOKEN = 42
+};
+
+/* ggml tensor type tags (crates/qwen-llm/src/tensor.rs:164-208) */
+enum { DFLASH_TYPE_F32 = 0, DFLASH_TYPE_F16 = 1, DFLASH_TYPE_Q8_0 = 8, DFLASH_TYPE_Q4_K = 12, DFLASH_TYPE_Q6_K = 14 };
+
+/* ---- context ------------------------------------------------------------------
+ * Replaces MetalContext + the per-call scratch the reference keeps in
+ * MetalDFlashVerifyScratch / MetalDFlashLayerMajorScratch (metal_dflash.rs:5863-5905,
+ * 7240-7443).  `workspace_bytes` of device memory are allocated once here (0 = 128 MiB)
+ * and reused by every call; calls on one context must not overlap. */
+int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **out);
+void dflash_ctx_destroy(dflash_ctx *ctx);
+const char *dflash_last_error(const dflash_ctx *ctx);
+const char *dflash_status_name(int32_t status);
+const char *dflash_version(void);
+
+/* Per-kernel GPU timers: enable_phase_timers / maybe_record (metal_dflash.rs:5181-5190, 5622).
+ * While enabled, each call brackets its dominant kernel with events on the call's stream and
+ * waits for it, accumulating into a slot: 0 few-row GEMM, 1 verify attention, 2 acceptance,
+ * 3 argmax/top-k, 4 activation re-layout.  Enabling or disabling clears the slots. */
+void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable);
+int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms_host,
+                                 int64_t *launches_host);
+
+/* ---- block dequantisation -------------------------------------------------------
+ * codec::dequant_to_f32{,_into,_in_place} (codec.rs:256-302): ggml blocks -> f32,
+ * bit-exact with ggml's dequantize_row_{q4_K,q6_K,q8_0}.  n_elems must be a multiple
+ * of the block size (codec.rs:91-103). */
+int32_t dflash_dequant(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_elems, float *out_f32,
+                       dflash_stream_t stream);
+size_t dflash_row_bytes(int32_t type, size_t n_in);
+
+/* ---- few-row quantised GEMM ---------------------------------------------------
+ * encode_mat_mat_dispatch_dflash_verify(ctx, enc, weight, x, y, n_in, n_out, n_query)
+ * (metal_forward/dispatch.rs:365-378; kernel kernels/mat_mat_fewrow_gen.metal:374-474).
+ *   Y[n_rows][n_out] = X[n_rows][n_in] . W^T,  W = quant blocks, row-major [n_out][n_in/blk]
+ * x_type: DFLASH_TYPE_F32 (the reference's activations) or DFLASH_TYPE_F16; Y is f32.
+ * 1 <= n_rows <= 16; n_in % 256 == 0 (Q4_K, Q6_K) or % 32 == 0 (Q8_0); W 16-byte aligned
+ * (2-byte for Q8_0); Y must not alias X or W.  Enqueue-only. */
+int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
+                           int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

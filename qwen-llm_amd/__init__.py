@@ -1,0 +1,26 @@
+"""MI355X-native DFlash speculative-decoding step.
+
+Host-side mirror of the reference engine's interfaces for this path, over the C ABI
+of ``libdflash_hip.so`` (hand-written HIP for gfx950, declared in
+``include/dflash_hip.h``).  Device memory and streams come from PyTorch-ROCm; every
+array argument that reaches the library is a device tensor.
+
+There is no CPU fallback: if the HIP library is missing or no GPU is present, the
+calls raise.
+"""
+from __future__ import annotations
+
+from . import synth  # noqa: F401
+from .binding import (  # noqa: F401
+    DFlashError,
+    LIB_PATH,
+    STATUS,
+    TYPE_F16,
+    TYPE_F32,
+    TYPE_Q4_K,
+    TYPE_Q6_K,
+    TYPE_Q8_0,
+    Context,
+    declared_symbols,
+    lib,
+)

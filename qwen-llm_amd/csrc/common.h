@@ -1,0 +1,73 @@
+// Internal declarations shared by the HIP translation units of libdflash_hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/dflash_hip.h"
+
+struct dflash_ctx {
+    int device = 0;
+    char *workspace = nullptr;  // device scratch, owned
+    size_t workspace_bytes = 0;
+    int n_cu = 256;
+    char err[512] = {0};
+    // per-kernel timers (off by default; when on, timed launches synchronise)
+    bool timing = false;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    double timed_ms[8] = {0};
+    int64_t timed_launches[8] = {0};
+};
+
+// Slots of the per-kernel timers.
+enum { DFL_T_GEMM = 0, DFL_T_ATTN = 1, DFL_T_ACCEPT = 2, DFL_T_ARGMAX = 3, DFL_T_PREP = 4 };
+
+// Brackets the dominant kernel of a call with events on its stream when timing is on.
+struct dfl_timed {
+    dflash_ctx *ctx;
+    hipStream_t st;
+    int slot;
+    dfl_timed(dflash_ctx *c, hipStream_t s, int k) : ctx(c), st(s), slot(k) {
+        if (ctx->timing) (void)hipEventRecord(ctx->ev0, st);
+    }
+    ~dfl_timed() {
+        if (!ctx->timing) return;
+        (void)hipEventRecord(ctx->ev1, st);
+        (void)hipEventSynchronize(ctx->ev1);
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1) == hipSuccess) {
+            ctx->timed_ms[slot] += ms;
+            ctx->timed_launches[slot] += 1;
+        }
+    }
+};
+
+// Records a message on the context and returns `status`.
+int32_t dfl_fail(dflash_ctx *ctx, int32_t status, const char *fmt, ...);
+
+#define DFL_HIP_CHECK(ctx, expr)                                                          \
+    do {                                                                                  \
+        hipError_t e_ = (expr);                                                           \
+        if (e_ != hipSuccess)                                                             \
+            return dfl_fail((ctx), DFLASH_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+// Carves `bytes` (256-aligned) out of the context workspace starting at *offset.
+template <typename T>
+static inline T *dfl_ws_take(dflash_ctx *ctx, size_t *offset, size_t bytes) {
+    size_t start = (*offset + 255) & ~size_t(255);
+    if (start + bytes > ctx->workspace_bytes) return nullptr;
+    *offset = start + bytes;
+    return reinterpret_cast<T *>(ctx->workspace + start);
+}
+
+static inline bool dfl_ranges_overlap(const void *a, size_t na, const void *b, size_t nb) {
+    const char *pa = static_cast<const char *>(a), *pb = static_cast<const char *>(b);
+    return pa < pb + nb && pb < pa + na;
+}
+
+enum { DFL_QK_K = 256, DFL_Q4_K_BYTES = 144, DFL_Q6_K_BYTES = 210, DFL_Q8_0_BYTES = 34, DFL_QK8_0 = 32 };

@@ -1,0 +1,110 @@
+// Context lifetime, error reporting and block geometry of libdflash_hip.
+#include "common.h"
+
+#include <cstring>
+#include <new>
+
+int32_t dfl_fail(dflash_ctx *ctx, int32_t status, const char *fmt, ...) {
+    if (ctx) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(ctx->err, sizeof(ctx->err), fmt, ap);
+        va_end(ap);
+    }
+    return status;
+}
+
+extern "C" {
+
+int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **out) {
+    if (!out) return DFLASH_ERR_INVALID_INPUT;
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count) return DFLASH_ERR_HIP;
+    if (hipSetDevice(device) != hipSuccess) return DFLASH_ERR_HIP;
+    dflash_ctx *ctx = new (std::nothrow) dflash_ctx();
+    if (!ctx) return DFLASH_ERR_HIP;
+    ctx->device = device;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->n_cu = prop.multiProcessorCount;
+    ctx->workspace_bytes = workspace_bytes ? workspace_bytes : (size_t(128) << 20);
+    if (hipMalloc(reinterpret_cast<void **>(&ctx->workspace), ctx->workspace_bytes) != hipSuccess) {
+        delete ctx;
+        return DFLASH_ERR_HIP;
+    }
+    if (hipEventCreate(&ctx->ev0) != hipSuccess || hipEventCreate(&ctx->ev1) != hipSuccess) {
+        dflash_ctx_destroy(ctx);
+        return DFLASH_ERR_HIP;
+    }
+    *out = ctx;
+    return DFLASH_OK;
+}
+
+void dflash_ctx_destroy(dflash_ctx *ctx) {
+    if (!ctx) return;
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
+    if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    delete ctx;
+}
+
+void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable) {
+    if (!ctx) return;
+    ctx->timing = enable != 0;
+    for (int i = 0; i < 8; i++) {
+        ctx->timed_ms[i] = 0.0;
+        ctx->timed_launches[i] = 0;
+    }
+}
+
+int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms, int64_t *launches) {
+    if (!ctx || slot < 0 || slot >= 8 || !total_ms || !launches) return DFLASH_ERR_INVALID_INPUT;
+    *total_ms = ctx->timed_ms[slot];
+    *launches = ctx->timed_launches[slot];
+    return DFLASH_OK;
+}
+
+const char *dflash_last_error(const dflash_ctx *ctx) { return ctx ? ctx->err : "no context"; }
+
+const char *dflash_status_name(int32_t s) {
+    switch (s) {
+    case DFLASH_OK: return "Ok";
+    case DFLASH_ERR_BAD_SHAPE: return "BadShape";
+    case DFLASH_ERR_UNSUPPORTED: return "Unsupported";
+    case DFLASH_ERR_ALIAS: return "Alias";
+    case DFLASH_ERR_ALIGNMENT: return "Alignment";
+    case DFLASH_ERR_WORKSPACE: return "Workspace";
+    case DFLASH_ERR_HIP: return "Hip";
+    case DFLASH_ERR_INVALID_INPUT: return "InvalidInput";
+    case DFLASH_ERR_INVALID_TOKEN: return "InvalidToken";
+    case DFLASH_ERR_PROPOSAL_MISMATCH: return "ProposalMismatch";
+    case DFLASH_ERR_STATE: return "State";
+    case DFLASH_ERR_EMPTY_LOGITS: return "EmptyLogits";
+    case DFLASH_ERR_INVALID_TEMPERATURE: return "InvalidTemperature";
+    case DFLASH_ERR_INVALID_TOP_P: return "InvalidTopP";
+    case DFLASH_ERR_INVALID_MIN_P: return "InvalidMinP";
+    case DFLASH_ERR_NAN_LOGIT: return "NanLogit";
+    case DFLASH_ERR_VOCAB_TOO_LARGE: return "VocabularyTooLarge";
+    case DFLASH_ERR_NO_CANDIDATES: return "NoCandidates";
+    case DFLASH_ERR_PROPOSAL_TOKEN_OUT_OF_RANGE: return "ProposalTokenOutOfRange";
+    case DFLASH_ERR_INVALID_PROPOSAL_WEIGHT: return "InvalidProposalWeight";
+    case DFLASH_ERR_MISSING_PROPOSAL_TOKEN: return "MissingProposalToken";
+    default: return "Unknown";
+    }
+}
+
+const char *dflash_version(void) { return "dflash_hip 0.1 (gfx950)"; }
+
+// tensor.rs:164-208
+size_t dflash_row_bytes(int32_t type, size_t n_in) {
+    switch (type) {
+    case DFLASH_TYPE_Q4_K: return n_in % DFL_QK_K ? 0 : n_in / DFL_QK_K * DFL_Q4_K_BYTES;
+    case DFLASH_TYPE_Q6_K: return n_in % DFL_QK_K ? 0 : n_in / DFL_QK_K * DFL_Q6_K_BYTES;
+    case DFLASH_TYPE_Q8_0: return n_in % DFL_QK8_0 ? 0 : n_in / DFL_QK8_0 * DFL_Q8_0_BYTES;
+    case DFLASH_TYPE_F32: return n_in * 4;
+    case DFLASH_TYPE_F16: return n_in * 2;
+    default: return 0;
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,98 @@
+// Block dequantisation kernels: ggml Q4_K / Q6_K / Q8_0 -> f32, bit-exact with
+// ggml's dequantize_row_* (closed forms pinned by the reference's tests,
+// codec.rs:474-577 and metal/tests/q6_k_f32_tile.rs:46-107).  Every value is built
+// from round-to-nearest f32 products and one subtraction, never a fused
+// multiply-add, so __fmul_rn / __fsub_rn are used throughout.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float h2f(const uint8_t *p) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(p[0] | (p[1] << 8))));
+}
+
+// One thread per element; one 256-thread workgroup per super-block.
+__global__ void __launch_bounds__(256) dequant_q4_k_kernel(const uint8_t *__restrict__ blocks, float *__restrict__ out,
+                                                           size_t n_blocks) {
+    size_t b = blockIdx.x;
+    if (b >= n_blocks) return;
+    const uint8_t *blk = blocks + b * DFL_Q4_K_BYTES;
+    int e = threadIdx.x;
+    int j = e >> 5;  // sub-block
+    int l = e & 31;
+    const uint8_t *s = blk + 4;
+    int sc, m;
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (s[j + 4] & 0x0f) | ((s[j - 4] >> 6) << 4);
+        m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+    }
+    uint8_t byte = blk[16 + 32 * (j >> 1) + l];
+    int q = (j & 1) ? (byte >> 4) : (byte & 0x0f);
+    float d1 = __fmul_rn(h2f(blk), static_cast<float>(sc));
+    float m1 = __fmul_rn(h2f(blk + 2), static_cast<float>(m));
+    out[b * DFL_QK_K + e] = __fsub_rn(__fmul_rn(d1, static_cast<float>(q)), m1);
+}
+
+__global__ void __launch_bounds__(256) dequant_q6_k_kernel(const uint8_t *__restrict__ blocks, float *__restrict__ out,
+                                                           size_t n_blocks) {
+    size_t b = blockIdx.x;
+    if (b >= n_blocks) return;
+    const uint8_t *blk = blocks + b * DFL_Q6_K_BYTES;
+    int e = threadIdx.x;
+    int n = e >> 7;         // 128-element half
+    int r = e & 127;
+    int k = r >> 5;         // which of q1..q4
+    int l = r & 31;
+    const uint8_t *ql = blk + 64 * n;
+    const uint8_t *qh = blk + 128 + 32 * n;
+    const int8_t *sc = reinterpret_cast<const int8_t *>(blk + 192 + 8 * n);
+    int lo = (k & 1) ? ql[l + 32] : ql[l];
+    lo = (k & 2) ? (lo >> 4) : (lo & 0x0f);
+    int hi = (qh[l] >> (2 * k)) & 3;
+    int q = (lo | (hi << 4)) - 32;
+    float ds = __fmul_rn(h2f(blk + 208), static_cast<float>(sc[(l >> 4) + 2 * k]));
+    out[b * DFL_QK_K + e] = __fmul_rn(ds, static_cast<float>(q));
+}
+
+// Q8_0 blocks hold 32 elements; eight blocks per 256-thread workgroup.
+__global__ void __launch_bounds__(256) dequant_q8_0_kernel(const uint8_t *__restrict__ blocks, float *__restrict__ out,
+                                                           size_t n_blocks) {
+    size_t b = static_cast<size_t>(blockIdx.x) * 8 + (threadIdx.x >> 5);
+    if (b >= n_blocks) return;
+    const uint8_t *blk = blocks + b * DFL_Q8_0_BYTES;
+    int i = threadIdx.x & 31;
+    float q = static_cast<float>(reinterpret_cast<const int8_t *>(blk + 2)[i]);
+    out[b * DFL_QK8_0 + i] = __fmul_rn(h2f(blk), q);
+}
+
+}  // namespace
+
+extern "C" int32_t dflash_dequant(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_elems, float *out_f32,
+                                  dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!blocks || !out_f32) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "dequant: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint8_t *src = static_cast<const uint8_t *>(blocks);
+    size_t blk = (type == DFLASH_TYPE_Q8_0) ? DFL_QK8_0 : DFL_QK_K;
+    if (type != DFLASH_TYPE_Q4_K && type != DFLASH_TYPE_Q6_K && type != DFLASH_TYPE_Q8_0)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "dequant: unsupported type %d", type);
+    if (n_elems % blk)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "dequant: %zu elements is not a multiple of the block size %zu",
+                        n_elems, blk);
+    size_t n_blocks = n_elems / blk;
+    if (n_blocks == 0) return DFLASH_OK;
+    if (n_blocks > 0x7fffffffull) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "dequant: too many blocks");
+    if (dfl_ranges_overlap(out_f32, n_elems * 4, blocks, dflash_row_bytes(type, n_elems)))
+        return dfl_fail(ctx, DFLASH_ERR_ALIAS, "dequant: output aliases the blocks");
+    if (type == DFLASH_TYPE_Q4_K)
+        dequant_q4_k_kernel<<<dim3(static_cast<unsigned>(n_blocks)), 256, 0, st>>>(src, out_f32, n_blocks);
+    else if (type == DFLASH_TYPE_Q6_K)
+        dequant_q6_k_kernel<<<dim3(static_cast<unsigned>(n_blocks)), 256, 0, st>>>(src, out_f32, n_blocks);
+    else
+        dequant_q8_0_kernel<<<dim3(static_cast<unsigned>((n_blocks + 7) / 8)), 256, 0, st>>>(src, out_f32, n_blocks);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}

@@ -1,0 +1,171 @@
+"""GPU parity: block dequantisation (bit-exact) and the few-row quantised GEMM
+(<= 1e-2 relative, f32 accumulation) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import qwen_llm_amd as dfl
+
+pytestmark = pytest.mark.gpu
+
+QTYPES = [dfl.synth.Q4_K, dfl.synth.Q6_K, dfl.synth.Q8_0]
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = dfl.Context(0)
+    yield c
+    c.close()
+
+
+def dev(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("qtype", QTYPES)
+@pytest.mark.parametrize("kind", ["random", "extreme", "quantised"])
+def test_dequant_bit_exact(ctx, oracle, qtype, kind):
+    """codec.rs:474-577 / q6_k_f32_tile.rs:46-107: every element identical to ggml's value"""
+    n_blocks = 1031
+    be = dfl.synth.BLOCK_ELEMS[qtype]
+    if kind == "random":
+        blocks = dfl.synth.random_blocks(qtype, n_blocks, seed=1)
+    elif kind == "extreme":
+        blocks = dfl.synth.extreme_blocks(qtype, n_blocks, seed=2)
+    else:
+        w = (np.random.default_rng(3).standard_normal((n_blocks, be)) * 0.02).astype(np.float32)
+        blocks = dfl.synth.quantize(qtype, w)
+    want = oracle.dequant(qtype, blocks, n_blocks * be)
+    got = ctx.dequant_to_f32(qtype, dev(blocks), n_blocks * be).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_rejects_bad_geometry(ctx):
+    import torch
+
+    buf = torch.zeros(144, dtype=torch.uint8, device="cuda")
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.dequant_to_f32(dfl.TYPE_Q4_K, buf, 100)
+    assert e.value.kind == "BadShape"
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.dequant_to_f32(3, buf, 256)
+    assert e.value.kind == "Unsupported"
+
+
+def check_gemm(y, ref, label):
+    """north-star bar: <= 1e-2 relative (norm-wise and element-wise against max(|ref|, rms));
+    the reference's own bar (metal/mat_mat.rs:4285-4309) is reported alongside."""
+    y = y.astype(np.float64)
+    assert np.all(np.isfinite(y)), f"{label}: non-finite output"
+    rel_l2 = np.linalg.norm(y - ref) / max(np.linalg.norm(ref), 1e-30)
+    rms = np.sqrt(np.mean(ref ** 2))
+    elem = np.max(np.abs(y - ref) / np.maximum(np.abs(ref), rms))
+    assert rel_l2 <= 1e-2 and elem <= 1e-2, f"{label}: rel_l2 {rel_l2:.3e} elem {elem:.3e}"
+    max_ref = np.max(np.abs(ref))
+    atol, rtol = 1e-3 * max(max_ref, 1.0), 5e-3
+    assert np.all(np.abs(y - ref) <= atol + rtol * np.abs(ref)), f"{label}: reference tolerance"
+    assert rel_l2 <= 2e-3, f"{label}: RMS relative error {rel_l2:.3e}"
+    return rel_l2
+
+
+def f64_reference(oracle, qtype, w, x, n_in, n_out):
+    wf = oracle.dequant(qtype, w, n_in * n_out).reshape(n_out, n_in).astype(np.float64)
+    return x.astype(np.float64) @ wf.T
+
+
+SHAPES = [(256, 16, 16), (256, 1, 1), (512, 17, 3), (1024, 33, 16), (2560, 100, 8), (5120, 64, 16), (768, 2049, 5),
+          (4352, 130, 16), (256, 8, 9)]
+
+
+@pytest.mark.parametrize("qtype", QTYPES)
+@pytest.mark.parametrize("n_in,n_out,n_rows", SHAPES)
+@pytest.mark.parametrize("x_dtype", ["f32", "f16"])
+def test_gemm_fewrow_small_shapes(ctx, oracle, qtype, n_in, n_out, n_rows, x_dtype):
+    """tile edges, ragged n_out, every row count class, random + extreme blocks"""
+    rng = np.random.default_rng(n_in * 31 + n_out * 7 + n_rows)
+    nblk = n_in // dfl.synth.BLOCK_ELEMS[qtype] * n_out
+    w = dfl.synth.random_blocks(qtype, nblk, seed=n_out)
+    x = rng.standard_normal((n_rows, n_in)).astype(np.float32)
+    if x_dtype == "f16":
+        x = x.astype(np.float16)
+    ref = f64_reference(oracle, qtype, w, x.astype(np.float32), n_in, n_out)
+    y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+    check_gemm(y, ref, f"q{qtype} {n_in}x{n_out}x{n_rows} {x_dtype}")
+
+
+@pytest.mark.parametrize("qtype", QTYPES)
+def test_gemm_fewrow_extreme_blocks(ctx, oracle, qtype):
+    """metal/mat_mat.rs:4228-4265: large minima / saturated codes must stay finite and accurate"""
+    n_in, n_out, n_rows = 1024, 48, 16
+    nblk = n_in // dfl.synth.BLOCK_ELEMS[qtype] * n_out
+    w = dfl.synth.extreme_blocks(qtype, nblk, seed=5)
+    x = np.random.default_rng(5).standard_normal((n_rows, n_in)).astype(np.float32)
+    ref = f64_reference(oracle, qtype, w, x, n_in, n_out)
+    y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+    check_gemm(y, ref, f"extreme q{qtype}")
+
+
+def test_gemm_matches_oracle_f32_path(ctx, oracle):
+    """the oracle's own f32 dequant + mat_vec (forward.rs:1321-1334) on the same bytes"""
+    n_in, n_out, n_rows = 2048, 96, 16
+    w = dfl.synth.random_weight(dfl.synth.Q4_K, n_out, n_in, seed=1)
+    x = np.random.default_rng(1).standard_normal((n_rows, n_in)).astype(np.float32)
+    want = oracle.gemm_fewrow(dfl.synth.Q4_K, w, x, n_in, n_out)
+    got = ctx.gemm_fewrow(dev(w), dfl.synth.Q4_K, dev(x), n_in, n_out).cpu().numpy()
+    rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), rms)) <= 1e-2
+
+
+def test_gemm_deterministic_and_linear(ctx):
+    """size-independent properties at a full-size shape: run-to-run identical bits; linear in X"""
+    import torch
+
+    n_in, n_out = 5120, 6144
+    w = dev(dfl.synth.random_weight(dfl.synth.Q4_K, n_out, n_in, seed=1))
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x1 = torch.randn((16, n_in), device="cuda", generator=g, dtype=torch.float32).half()
+    x2 = torch.randn((16, n_in), device="cuda", generator=g, dtype=torch.float32).half()
+    y1 = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, x1, n_in, n_out)
+    y1b = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, x1, n_in, n_out)
+    assert torch.equal(y1, y1b)
+    y2 = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, x2, n_in, n_out)
+    xs = (x1.float() + x2.float())
+    ys = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, xs, n_in, n_out)
+    scale = ys.abs().max().item()
+    assert (ys - (y1 + y2)).abs().max().item() <= 4e-3 * scale
+
+
+@pytest.mark.parametrize("n_in,n_out", [(5120, 17408), (17408, 5120), (5120, 6144)])
+def test_gemm_fewrow_full_size_q4k(ctx, oracle, n_in, n_out):
+    """the three production shapes, X f16 N(0,1), W = Q4_K(N(0,0.02)), seed 1; checked on a
+    sample of output columns against the f64 reference (the oracle takes seconds per 256 rows)"""
+    w = dfl.synth.random_weight(dfl.synth.Q4_K, n_out, n_in, seed=1)
+    x = np.random.default_rng(1).standard_normal((16, n_in)).astype(np.float16)
+    y = ctx.gemm_fewrow(dev(w), dfl.synth.Q4_K, dev(x), n_in, n_out).cpu().numpy()
+    rows = np.unique(np.concatenate([np.arange(0, 64), np.arange(n_out - 64, n_out),
+                                     np.random.default_rng(2).integers(0, n_out, 384)]))
+    ref = f64_reference(oracle, dfl.synth.Q4_K, w[rows], x.astype(np.float32), n_in, len(rows))
+    check_gemm(y[:, rows], ref, f"full {n_in}x{n_out}")
+
+
+def test_gemm_guards(ctx):
+    """dispatch.rs:256-327, 522-526: shape / alias / dtype refusals are errors, not crashes"""
+    import torch
+
+    w = torch.zeros(16 * 144, dtype=torch.uint8, device="cuda")
+    x = torch.zeros((17, 256), device="cuda")
+    y = torch.zeros((17, 16), device="cuda")
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q4_K, x, y, 256, 16, 17)
+    assert e.value.kind == "BadShape"
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q4_K, x, y, 100, 16, 4)
+    assert e.value.kind == "BadShape"
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.encode_mat_mat_dispatch_dflash_verify(w, 3, x, y, 256, 16, 4)
+    assert e.value.kind == "Unsupported"
+    xy = torch.zeros(4 * 256, device="cuda")
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q4_K, xy, xy, 256, 16, 4)
+    assert e.value.kind == "Alias"
