@@ -15,6 +15,8 @@ struct dflash_ctx {
     char *workspace = nullptr;  // device scratch, owned
     size_t workspace_bytes = 0;
     int n_cu = 256;
+    int *counters = nullptr;  // zero-initialised arrival counters; every kernel leaves them zero
+    int n_counters = 0;
     char err[512] = {0};
     // per-kernel timers (off by default; when on, timed launches synchronise)
     bool timing = false;

@@ -32,6 +32,12 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
         delete ctx;
         return DFLASH_ERR_HIP;
     }
+    ctx->n_counters = 1 << 16;
+    if (hipMalloc(reinterpret_cast<void **>(&ctx->counters), ctx->n_counters * sizeof(int)) != hipSuccess ||
+        hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(int)) != hipSuccess) {
+        dflash_ctx_destroy(ctx);
+        return DFLASH_ERR_HIP;
+    }
     if (hipEventCreate(&ctx->ev0) != hipSuccess || hipEventCreate(&ctx->ev1) != hipSuccess) {
         dflash_ctx_destroy(ctx);
         return DFLASH_ERR_HIP;
@@ -43,6 +49,7 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
 void dflash_ctx_destroy(dflash_ctx *ctx) {
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     delete ctx;
