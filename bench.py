@@ -93,7 +93,7 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = e0.elapsed_time(e1) / args.steps
 
-    # dominant kernel alone: events inside the library around gemm_q4k_kernel, on its stream
+    # dominant kernel alone: events inside the library around gemm_q4k_stream_kernel, on its stream
     ctx.set_kernel_timing(True)
     per_shape = []
     for (n_in, n_out), w, x, y, nbytes in zip(SHAPES, wd, xd, yd, w_bytes):
@@ -126,7 +126,7 @@ def main():
                    "weight_bytes_per_step": sum(w_bytes), "block": 16, "batch": 1},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "gemm_q4k_kernel", "bytes_per_launch": k_bytes, "us_per_launch": k_us},
+                     "kernel": "gemm_q4k_stream_kernel", "bytes_per_launch": k_bytes, "us_per_launch": k_us},
         "shapes": per_shape,
         "pct_of_hbm_peak": 100.0 * sum(w_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "accepted_tokens_per_s": None,

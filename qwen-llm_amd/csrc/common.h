@@ -17,6 +17,11 @@ struct dflash_ctx {
     int n_cu = 256;
     int *counters = nullptr;  // zero-initialised arrival counters; every kernel leaves them zero
     int n_counters = 0;
+    // split-K partial tiles of the Q4_K GEMM: {value, epoch tag} pairs, persistent across calls
+    void *tagged_partials = nullptr;
+    int n_partial_wgs = 0;
+    uint32_t epoch = 0;
+    size_t lds_bytes = 65536;  // LDS available to one workgroup
     char err[512] = {0};
     // per-kernel timers (off by default; when on, timed launches synchronise)
     bool timing = false;

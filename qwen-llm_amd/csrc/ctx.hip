@@ -26,7 +26,10 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
     if (!ctx) return DFLASH_ERR_HIP;
     ctx->device = device;
     hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->n_cu = prop.multiProcessorCount;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) {
+        ctx->n_cu = prop.multiProcessorCount;
+        ctx->lds_bytes = prop.sharedMemPerBlock;
+    }
     ctx->workspace_bytes = workspace_bytes ? workspace_bytes : (size_t(128) << 20);
     if (hipMalloc(reinterpret_cast<void **>(&ctx->workspace), ctx->workspace_bytes) != hipSuccess) {
         delete ctx;
@@ -37,6 +40,14 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
         hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(int)) != hipSuccess) {
         dflash_ctx_destroy(ctx);
         return DFLASH_ERR_HIP;
+    }
+    ctx->n_partial_wgs = 1024;
+    {
+        const size_t bytes = static_cast<size_t>(ctx->n_partial_wgs) * 2 * 8 * 256 * 8;
+        if (hipMalloc(&ctx->tagged_partials, bytes) != hipSuccess || hipMemset(ctx->tagged_partials, 0, bytes) != hipSuccess) {
+            dflash_ctx_destroy(ctx);
+            return DFLASH_ERR_HIP;
+        }
     }
     if (hipEventCreate(&ctx->ev0) != hipSuccess || hipEventCreate(&ctx->ev1) != hipSuccess) {
         dflash_ctx_destroy(ctx);
@@ -50,6 +61,7 @@ void dflash_ctx_destroy(dflash_ctx *ctx) {
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->counters) (void)hipFree(ctx->counters);
+    if (ctx->tagged_partials) (void)hipFree(ctx->tagged_partials);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     delete ctx;

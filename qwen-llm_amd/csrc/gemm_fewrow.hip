@@ -39,6 +39,7 @@ namespace {
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxSplit = 16;
 constexpr int kWavesQ4K = 8;  // output tiles (waves) per workgroup of the Q4_K kernel
@@ -120,13 +121,17 @@ __device__ __forceinline__ half2_t splat(_Float16 v) {
     return r;
 }
 
-// (a & mask) | magic in one VALU instruction.  The compiler splits this into two
-// because both constants are literals; with the mask in an SGPR and the magic in a
-// VGPR it is a single v_and_or_b32.
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) {
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(magic));
-    return r;
+// The f16 constants 1024.0 and 64.0 (as pairs) whose mantissas receive the nibbles.  They are
+// passed through an empty asm once per kernel so the compiler sees VGPR values, not literals:
+// (w & mask) | magic then selects as one v_and_or_b32 (mask in an SGPR) instead of two
+// instructions with a literal each.
+struct Q4KMagic {
+    uint32_t lo, hi;
+};
+__device__ __forceinline__ Q4KMagic q4k_magic() {
+    Q4KMagic m = {0x64006400u, 0x54005400u};
+    asm volatile("" : "+v"(m.lo), "+v"(m.hi));
+    return m;
 }
 
 // Eight f16 weights of one MFMA from two dwords of quant bytes.
@@ -134,13 +139,12 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t m
 //   HIGH = true : high nibbles,   64 + q  via magic 0x5400, mask 0x00F0
 // s2 = (s, s), c2 = (-1024 s, -1024 s) or (-64 s, -64 s).
 template <bool HIGH>
-__device__ __forceinline__ half8_t unpack_scale(uint32_t w0, uint32_t w1, half2_t s2, half2_t c2) {
+__device__ __forceinline__ half8_t unpack_scale(uint32_t w0, uint32_t w1, half2_t s2, half2_t c2, uint32_t magic) {
     constexpr uint32_t mask = HIGH ? 0x00F000F0u : 0x000F000Fu;
-    constexpr uint32_t magic = HIGH ? 0x54005400u : 0x64006400u;
-    half2_t p0 = __builtin_elementwise_fma(as_half2(and_or(w0, mask, magic)), s2, c2);
-    half2_t p1 = __builtin_elementwise_fma(as_half2(and_or(w0 >> 8, mask, magic)), s2, c2);
-    half2_t p2 = __builtin_elementwise_fma(as_half2(and_or(w1, mask, magic)), s2, c2);
-    half2_t p3 = __builtin_elementwise_fma(as_half2(and_or(w1 >> 8, mask, magic)), s2, c2);
+    half2_t p0 = __builtin_elementwise_fma(as_half2((w0 & mask) | magic), s2, c2);
+    half2_t p1 = __builtin_elementwise_fma(as_half2(((w0 >> 8) & mask) | magic), s2, c2);
+    half2_t p2 = __builtin_elementwise_fma(as_half2((w1 & mask) | magic), s2, c2);
+    half2_t p3 = __builtin_elementwise_fma(as_half2(((w1 >> 8) & mask) | magic), s2, c2);
     half8_t r = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
     return r;
 }
@@ -150,161 +154,343 @@ __device__ __forceinline__ _Float16 byte_to_half(uint32_t v, int j) {
     return static_cast<_Float16>(static_cast<float>((v >> (8 * j)) & 0xffu));
 }
 
-// Grid: (tile groups) x (K slices); a workgroup is kWavesQ4K waves = kWavesQ4K output
-// tiles over one K-slice of at most KB super-blocks.
-// LDS: the slice's prepared activations, kQ4KBlockFrags half8 per super-block.
-template <int KB>
-__global__ void __launch_bounds__(64 * kWavesQ4K)
-    gemm_q4k_kernel(const uint8_t *__restrict__ w, const half8_t *__restrict__ xp, float *__restrict__ y,
-                    float *__restrict__ partials, int *__restrict__ counters, int n_out, int nb, int n_rows, int kb,
-                    int n_slices) {
-    extern __shared__ half8_t lds[];
-    __shared__ int s_last;
+// One super-block of one output tile: 8 MFMAs.  hdr = {d|dmin, scales[0..3], [4..7], [8..11]},
+// q0/q1 = the lane's 32 quant bytes (chunk g), a = this super-block's A fragments in LDS.
+// A super-block slot past the end of a short stage (`live` false) holds a re-read of the last
+// one; its scales are forced to zero so it adds nothing and the code stays straight-line.
+// After every second MFMA the wave issues one load of a later stage (`next`, loads j0 ..): spread
+// over the MFMAs, the loads never queue up behind each other in the address unit, which would
+// otherwise stall all eight waves at once at the top of each stage.
+struct Q4KIssue;
+__device__ __forceinline__ void q4k_issue_one(const Q4KIssue &d, int j, int tid);
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int n = lane & 15, g = lane >> 4;
-    const int group = blockIdx.x / n_slices;
-    const int slice = blockIdx.x - group * n_slices;
-    const int b0 = slice * kb;
-    const int nblk = min(kb, nb - b0);
-    const int tile = group * kWavesQ4K + wave;
-    const int n_tiles = (n_out + 15) >> 4;
-    const bool active = tile < n_tiles;
-    const size_t row_bytes = static_cast<size_t>(nb) * DFL_Q4_K_BYTES;
-
-    // Loads are unconditional (indices clamped into the slice) so that no control flow sits
-    // between them: all of them are issued back to back and only then waited for.
-    // 1. the K-slice's prepared activations: global -> registers (flat copy, tail clamped)
-    constexpr int kCopies = (KB * kQ4KBlockFrags + 64 * kWavesQ4K - 1) / (64 * kWavesQ4K);
-    const int n_frags = nblk * kQ4KBlockFrags;
-    const half8_t *xsrc = xp + static_cast<int64_t>(b0) * kQ4KBlockFrags;
-    half8_t xr[kCopies];
+__device__ __forceinline__ float4_t q4k_block(u32x4_t hdr, u32x4_t q0, u32x4_t q1, const half8_t *a, int g,
+                                              bool live, Q4KMagic magic, float4_t acc, const Q4KIssue &next, int j0,
+                                              int tid) {
+    // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles)
+    uint32_t lo_sc = hdr.y & 0x3F3F3F3Fu;
+    uint32_t hi_sc = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    uint32_t sel = (g < 2 ? lo_sc : hi_sc) >> (16 * (g & 1));
+    _Float16 d = live ? __builtin_bit_cast(half2_t, hdr.x)[0] : static_cast<_Float16>(0.0f);
+    _Float16 s_lo = byte_to_half(sel, 0) * d;
+    _Float16 s_hi = byte_to_half(sel, 1) * d;
+    half2_t s2l = splat(s_lo), c2l = splat(s_lo * static_cast<_Float16>(-1024.0f));
+    half2_t s2h = splat(s_hi), c2h = splat(s_hi * static_cast<_Float16>(-64.0f));
+    uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
-    for (int i = 0; i < kCopies; i++) xr[i] = xsrc[min(i * 64 * kWavesQ4K + tid, n_frags - 1)];
-
-    // 2. every weight byte of this wave's tile and slice
-    int row = tile * 16 + n;
-    row = row < n_out ? row : n_out - 1;
-    const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
-    uint4 hdr[KB], q0[KB], q1[KB];
-#pragma unroll
-    for (int i = 0; i < KB; i++) {
-        const uint8_t *blk = rowp + min(i, nblk - 1) * DFL_Q4_K_BYTES;
-        hdr[i] = *reinterpret_cast<const uint4 *>(blk);
-        q0[i] = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * g);
-        q1[i] = *reinterpret_cast<const uint4 *>(blk + 32 + 32 * g);
-    }
-    __builtin_amdgcn_sched_barrier(0);  // everything above is in flight before anything below waits
-
-    // 3. activations -> LDS (clamped duplicates rewrite the last entry with the same value)
-#pragma unroll
-    for (int i = 0; i < kCopies; i++) lds[min(i * 64 * kWavesQ4K + tid, n_frags - 1)] = xr[i];
-    __syncthreads();
-
-    // 4. main MFMAs.  Straight-line on purpose (a branch here lets the compiler sink the loads
-    //    above into it): a slot past the end of a short slice re-reads the last super-block with
-    //    its scales forced to zero, so it adds nothing.
-    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0};
-    const _Float16 zero = static_cast<_Float16>(0.0f);
-#pragma unroll
-    for (int i = 0; i < KB; i++) {
-        // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles)
-        uint32_t lo_sc = hdr[i].y & 0x3F3F3F3Fu;
-        uint32_t hi_sc = (hdr[i].w & 0x0F0F0F0Fu) | ((hdr[i].y >> 2) & 0x30303030u);
-        uint32_t sel = (g < 2 ? lo_sc : hi_sc) >> (16 * (g & 1));
-        _Float16 d = (i < nblk) ? __builtin_bit_cast(half2_t, hdr[i].x)[0] : zero;
-        _Float16 s_lo = byte_to_half(sel, 0) * d;
-        _Float16 s_hi = byte_to_half(sel, 1) * d;
-        half2_t s2l = splat(s_lo), c2l = splat(s_lo * static_cast<_Float16>(-1024.0f));
-        half2_t s2h = splat(s_hi), c2h = splat(s_hi * static_cast<_Float16>(-64.0f));
-        uint32_t qw[8] = {q0[i].x, q0[i].y, q0[i].z, q0[i].w, q1[i].x, q1[i].y, q1[i].z, q1[i].w};
-        const half8_t *a = lds + min(i, nblk - 1) * kQ4KBlockFrags + lane;
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t * 64], bl, acc, 0, 0, 0);
-        }
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(4 + t) * 64], bh, acc, 0, 0, 0);
+    for (int t = 0; t < 4; t++) {
+        half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t * 64], bl, acc, 0, 0, 0);
+        if (t & 1) {
+            q4k_issue_one(next, j0 + (t >> 1), tid);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
-
-    // 5. minima: lane (n, g) supplies the eight dmin*m_j of super-block 4q+g, against the
-    //    sub-block sums of the same super-block
 #pragma unroll
-    for (int q = 0; q < (KB + 3) / 4; q++) {
-        uint4 h = hdr[4 * q];
-#pragma unroll
-        for (int u = 1; u < 4; u++)
-            if (4 * q + u < KB && g == u) h = hdr[4 * q + u];
-        int blk = 4 * q + g;
-        bool valid = blk < nblk;
-        blk = valid ? blk : 0;
-        _Float16 dmin = valid ? __builtin_bit_cast(half2_t, h.x)[1] : zero;
-        uint32_t lo_m = h.z & 0x3F3F3F3Fu;
-        uint32_t hi_m = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-        half8_t bm;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            bm[j] = byte_to_half(lo_m, j) * dmin;
-            bm[4 + j] = byte_to_half(hi_m, j) * dmin;
+    for (int t = 0; t < 4; t++) {
+        half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(4 + t) * 64], bh, acc, 0, 0, 0);
+        if (t & 1) {
+            q4k_issue_one(next, j0 + 2 + (t >> 1), tid);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        const half8_t *sums = lds + blk * kQ4KBlockFrags + 512 + n;
-        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[0], bm, acc_min, 0, 0, 0);
-        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[16], bm, acc_min, 0, 0, 0);
     }
+    return acc;
+}
 
-    // 6. output: direct when K is not split, else partial tiles + last-arriver sum in slice order
+// The eight dmin*m_j of one super-block as an MFMA B operand.
+__device__ __forceinline__ half8_t q4k_mins(u32x4_t h, bool valid) {
+    _Float16 dmin = valid ? __builtin_bit_cast(half2_t, h.x)[1] : static_cast<_Float16>(0.0f);
+    uint32_t lo_m = h.z & 0x3F3F3F3Fu;
+    uint32_t hi_m = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+    half8_t bm;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        bm[j] = byte_to_half(lo_m, j) * dmin;
+        bm[4 + j] = byte_to_half(hi_m, j) * dmin;
+    }
+    return bm;
+}
+
+// Streaming Q4_K kernel.
+//
+// Work split.  The iteration space is (tile group) x (super-block), flattened group-major; a
+// tile group is kWavesQ4K consecutive output tiles, one per wave of a workgroup.  The grid is
+// one workgroup per CU and workgroup i owns the contiguous range [T i / G, T (i+1) / G) of that
+// space, so every CU streams the same number of weight bytes whatever the shape.
+//
+// Data path.  A workgroup walks its range in stages of up to kStage super-blocks that stay
+// inside one tile group.  Per stage, the group's 128 weight rows (a row-contiguous slice of
+// kStage*144 bytes each) and the prepared activations are copied global -> LDS by
+// global_load_lds_dwordx4: consecutive lanes take consecutive 16-byte pieces, so HBM sees
+// row-contiguous requests and no VGPR is held while a load is in flight.  The stages rotate
+// through kBufs LDS buffers; the loads of stage j + kBufs - 1 are issued before stage j is
+// computed, so HBM never idles.  Each wave issues exactly kLoadsPerStage load instructions per
+// stage (surplus ones land in a spare LDS slot), which makes "stage j has landed" a constant
+// s_waitcnt.  Waves then read their tile's quant bytes and A fragments with ds_read_b128.
+//
+// Split K.  When a range leaves a tile group, the accumulators are flushed: straight to Y if
+// this workgroup covered the group's whole K, else as a partial tile whose every value carries
+// the call's epoch tag in the same 8-byte store.  The highest-numbered workgroup that touches a
+// group owns it: at the end of its own range it reads the group's partial tiles in workgroup
+// order, polling each value until its tag is the current epoch, and writes Y.  No fences, no
+// atomics, deterministic sums; a poll only ever waits for lower-numbered workgroups, which were
+// dispatched first, and gives up (writing NaN) after a bounded number of tries.
+constexpr int kStage = 2;
+constexpr int kThreadsQ4K = 64 * kWavesQ4K;
+constexpr int kGroupRows = 16 * kWavesQ4K;
+constexpr int kRowPieces = 9 * kStage + 1;  // LDS row stride in pieces: one pad piece staggers the banks
+constexpr int kStageWPieces = kGroupRows * kRowPieces;          // 16-byte pieces of weights per stage
+constexpr int kStageXPieces = kStage * kQ4KBlockFrags;          // 16-byte pieces of activations per stage
+constexpr int kBufPieces = kStageWPieces + kStageXPieces;       // one LDS buffer
+constexpr int kWLoads = (kStageWPieces + kThreadsQ4K - 1) / kThreadsQ4K;
+constexpr int kXLoads = (kStageXPieces + kThreadsQ4K - 1) / kThreadsQ4K;
+constexpr int kLoadsPerStage = kWLoads + kXLoads;
+constexpr uint32_t kSpinLimit = 1u << 22;
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// index of the workgroup whose range contains flattened iteration `it`
+// (all of this index arithmetic fits 32 bits: the host checks total * n_wg < 2^31)
+__device__ __forceinline__ int q4k_wg_of(int it, int total, int n_wg) {
+    return static_cast<int>((static_cast<uint32_t>(it + 1) * n_wg + total - 1) / static_cast<uint32_t>(total)) - 1;
+}
+
+struct Q4KRange {
+    int total, it_begin, it_end;
+    int nb, n_wg, first_group;
+};
+
+__device__ __forceinline__ void q4k_stage_at(const Q4KRange &rg, int it, int &group, int &b, int &len) {
+    group = static_cast<int>(static_cast<uint32_t>(it) / static_cast<uint32_t>(rg.nb));
+    b = it - group * rg.nb;
+    len = min(kStage, min(rg.nb - b, rg.it_end - it));
+}
+
+// Everything a wave needs to issue its kLoadsPerStage direct-to-LDS loads of one stage.
+// `buf` is the stage's LDS buffer (kBufPieces pieces), `spare` a 1 KiB slot that absorbs the
+// surplus loads of short stages.
+struct Q4KIssue {
+    const uint8_t *wbase;   // first super-block of the stage in weight row 0
+    const half8_t *xsrc;    // the stage's prepared activations
+    half8_t *buf, *spare;
+    size_t row_bytes;
+    int row0, n_out, ppr, n_x;
+    bool on;
+};
+
+__device__ __forceinline__ Q4KIssue q4k_issue_desc(const uint8_t *__restrict__ w, const half8_t *__restrict__ xp,
+                                                   half8_t *buf, half8_t *spare, int group, int b, int len,
+                                                   int n_out, size_t row_bytes, bool on) {
+    Q4KIssue d;
+    d.wbase = w + static_cast<size_t>(b) * DFL_Q4_K_BYTES;
+    d.xsrc = xp + static_cast<size_t>(b) * kQ4KBlockFrags;
+    d.buf = buf;
+    d.spare = spare;
+    d.row_bytes = row_bytes;
+    d.row0 = group * kGroupRows;
+    d.n_out = n_out;
+    d.ppr = 9 * len;  // real pieces per weight row; the rest of the row's kRowPieces re-read piece 0
+    d.n_x = len * kQ4KBlockFrags;
+    d.on = on;
+    return d;
+}
+
+// Load number j (0 .. kLoadsPerStage-1) of the stage: kWLoads weight loads, then kXLoads
+// activation loads.  Consecutive lanes take consecutive 16-byte pieces.
+__device__ __forceinline__ void q4k_issue_one(const Q4KIssue &d, int j, int tid) {
+    if (!d.on) return;
+    const int lane = tid & 63, wave = tid >> 6;
+    if (j < kWLoads) {
+        const int p0 = (j * kWavesQ4K + wave) * 64;  // wave-uniform
+        const int p = min(p0 + lane, kStageWPieces - 1);
+        const int r = static_cast<int>(static_cast<uint32_t>(p) / static_cast<uint32_t>(kRowPieces));
+        int o = p - r * kRowPieces;
+        o = o < d.ppr ? o : 0;
+        const int row = min(d.row0 + r, d.n_out - 1);
+        const uint8_t *src = d.wbase + static_cast<size_t>(row) * d.row_bytes + o * 16;
+        half8_t *dst = (p0 < kStageWPieces) ? d.buf + p0 : d.spare;
+        __builtin_amdgcn_global_load_lds((gptr_t)(src), (lptr_t)(dst), 16, 0, 0);
+    } else {
+        const int p0 = ((j - kWLoads) * kWavesQ4K + wave) * 64;
+        const int p = min(p0 + lane, d.n_x - 1);
+        half8_t *dst = (p0 < d.n_x) ? d.buf + kStageWPieces + p0 : d.spare;
+        __builtin_amdgcn_global_load_lds((gptr_t)(d.xsrc + p), (lptr_t)(dst), 16, 0, 0);
+    }
+}
+
+__device__ __forceinline__ void q4k_issue_all(const Q4KIssue &d, int tid) {
+#pragma unroll
+    for (int j = 0; j < kLoadsPerStage; j++) q4k_issue_one(d, j, tid);
+}
+
+// One stage of MFMAs for this wave's tile, out of LDS buffer `buf`.
+static_assert(kLoadsPerStage == 4 * kStage, "one load is issued after every second of a stage's 8*kStage MFMAs");
+
+__device__ __forceinline__ void q4k_compute(const half8_t *buf, int len, int tid, Q4KMagic magic, float4_t &acc,
+                                            float4_t &acc_min, const Q4KIssue &next) {
+    const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
+    const u32x4_t *wrow = reinterpret_cast<const u32x4_t *>(buf) + (wave * 16 + n) * kRowPieces;
+    const half8_t *xbuf = buf + kStageWPieces;
+#pragma unroll
+    for (int u = 0; u < kStage; u++) {
+        const int ub = min(u, len - 1);
+        const u32x4_t *blk = wrow + ub * 9;
+        acc = q4k_block(blk[0], blk[1 + 2 * g], blk[2 + 2 * g], xbuf + ub * kQ4KBlockFrags + lane, g, u < len, magic,
+                        acc, next, 4 * u, tid);
+    }
+    // minima: lane (n, g) supplies super-block g of the stage
+    const bool valid = g < len;
+    const int gb = valid ? g : 0;
+    half8_t bm = q4k_mins(wrow[gb * 9], valid);
+    const half8_t *sums = xbuf + gb * kQ4KBlockFrags + 512 + n;
+    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[0], bm, acc_min, 0, 0, 0);
+    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[16], bm, acc_min, 0, 0, 0);
+}
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt low bits [3:0],
+// high bits [15:14]; expcnt [6:4] and lgkmcnt [11:8] at their maxima)
+constexpr int q4k_vmcnt(int n) { return ((n & 0xF) | ((n & 0x30) << 10)) | 0x0F70; }
+
+struct Q4KTagged {
+    float value;
+    uint32_t tag;
+};
+
+// Ends a tile group's segment: Y directly if this workgroup covered the group's whole K, else a
+// tagged partial tile.
+__device__ __forceinline__ void q4k_flush(const Q4KRange &rg, int group, float4_t &acc, float4_t &acc_min,
+                                          float *__restrict__ y, Q4KTagged *__restrict__ partials, uint32_t epoch,
+                                          int n_out, int n_rows, int tid) {
+    const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
     float4_t res = acc - acc_min;
-    if (n_slices == 1) {
-        if (active) {
-            int orow = tile * 16 + n;
+    acc = float4_t{0, 0, 0, 0};
+    acc_min = float4_t{0, 0, 0, 0};
+    const int orow = (group * kWavesQ4K + wave) * 16 + n;
+    const int wg_first = q4k_wg_of(group * rg.nb, rg.total, rg.n_wg);
+    const int wg_last = q4k_wg_of((group + 1) * rg.nb - 1, rg.total, rg.n_wg);
+    if (wg_first == wg_last) {
+        if (orow < n_out) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                int m = 4 * g + i;
-                if (m < n_rows && orow < n_out) y[static_cast<size_t>(m) * n_out + orow] = res[i];
-            }
+            for (int i = 0; i < 4; i++)
+                if (4 * g + i < n_rows) y[static_cast<size_t>(4 * g + i) * n_out + orow] = res[i];
         }
         return;
     }
-    // Partial tiles cross workgroups (and XCDs, whose L2s are not coherent with each other)
-    // through agent-scope atomic stores and loads, which are performed at the coherent level
-    // instruction by instruction.  A release fence here would write back the whole L2 once per
-    // wave; waiting for this wave's own stores to complete before the arrival counter is
-    // bumped gives the same ordering for the only data that matters.
-    if (active) {
-        float *p = partials + (static_cast<size_t>(slice) * n_tiles + tile) * 256;
+    const int slot = (group == rg.first_group) ? 0 : 1;
+    Q4KTagged *p = partials + ((static_cast<size_t>(blockIdx.x) * 2 + slot) * kWavesQ4K + wave) * 256;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            __hip_atomic_store(&p[(4 * g + i) * 16 + n], res[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int i = 0; i < 4; i++) {
+        Q4KTagged t = {res[i], epoch};
+        __hip_atomic_store(reinterpret_cast<uint64_t *>(&p[(4 * g + i) * 16 + n]), __builtin_bit_cast(uint64_t, t),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0)
-        s_last = (__hip_atomic_fetch_add(&counters[group], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                  n_slices - 1);
-    __syncthreads();
-    if (!s_last) return;
-    if (active) {
-        float4_t sum = {0, 0, 0, 0};
-        for (int s = 0; s < n_slices; s++) {
-            const float *p = partials + (static_cast<size_t>(s) * n_tiles + tile) * 256;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                sum[i] += __hip_atomic_load(&p[(4 * g + i) * 16 + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        int orow = tile * 16 + n;
+}
+
+// Runs once, at the end of a workgroup's range: if its first tile group is split over several
+// workgroups and this is the highest-numbered one, add the group's partial tiles in workgroup
+// order and write Y.
+__device__ __forceinline__ void q4k_reduce_owned(const Q4KRange &rg, float *__restrict__ y,
+                                                 const Q4KTagged *__restrict__ partials, uint32_t epoch, int n_out,
+                                                 int n_rows, int tid) {
+    const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
+    const int group = rg.first_group;
+    const int wg_first = q4k_wg_of(group * rg.nb, rg.total, rg.n_wg);
+    const int wg_last = q4k_wg_of((group + 1) * rg.nb - 1, rg.total, rg.n_wg);
+    if (wg_first == wg_last || wg_last != static_cast<int>(blockIdx.x)) return;
+    const int orow = (group * kWavesQ4K + wave) * 16 + n;
+    if (orow >= n_out) return;
+    float4_t sum = {0, 0, 0, 0};
+    for (int wg = wg_first; wg <= wg_last; wg++) {
+        const int wg_first_group = static_cast<int>(static_cast<uint32_t>(rg.total) * wg / rg.n_wg / rg.nb);
+        const int slot = (group == wg_first_group) ? 0 : 1;
+        const Q4KTagged *p = partials + ((static_cast<size_t>(wg) * 2 + slot) * kWavesQ4K + wave) * 256;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            int m = 4 * g + i;
-            if (m < n_rows && orow < n_out) y[static_cast<size_t>(m) * n_out + orow] = sum[i];
+            const uint64_t *src = reinterpret_cast<const uint64_t *>(&p[(4 * g + i) * 16 + n]);
+            Q4KTagged t = __builtin_bit_cast(Q4KTagged, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            for (uint32_t spin = 0; t.tag != epoch && spin < kSpinLimit; spin++) {
+                __builtin_amdgcn_s_sleep(2);
+                t = __builtin_bit_cast(Q4KTagged, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            }
+            sum[i] += (t.tag == epoch) ? t.value : __builtin_nanf("");
         }
     }
-    if (tid == 0) __hip_atomic_store(&counters[group], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (4 * g + i < n_rows) y[static_cast<size_t>(4 * g + i) * n_out + orow] = sum[i];
+}
+
+template <int kBufs>
+__global__ void __launch_bounds__(kThreadsQ4K)
+    gemm_q4k_stream_kernel(const uint8_t *__restrict__ w, const half8_t *__restrict__ xp, float *__restrict__ y,
+                           Q4KTagged *__restrict__ partials, uint32_t epoch, int n_out, int nb, int n_rows,
+                           int n_groups) {
+    extern __shared__ half8_t lds[];  // kBufs buffers of kBufPieces, then a 64-piece spare slot
+    half8_t *spare = lds + kBufs * kBufPieces;
+
+    const int tid = threadIdx.x;
+    Q4KRange rg;
+    rg.nb = nb;
+    rg.n_wg = gridDim.x;
+    rg.total = n_groups * nb;
+    rg.it_begin = static_cast<int>(static_cast<uint32_t>(rg.total) * blockIdx.x / rg.n_wg);
+    rg.it_end = static_cast<int>(static_cast<uint32_t>(rg.total) * (blockIdx.x + 1) / rg.n_wg);
+    if (rg.it_begin >= rg.it_end) return;
+    rg.first_group = static_cast<int>(static_cast<uint32_t>(rg.it_begin) / static_cast<uint32_t>(nb));
+    const size_t row_bytes = static_cast<size_t>(nb) * DFL_Q4_K_BYTES;
+
+    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0};
+    const Q4KMagic magic = q4k_magic();
+
+    // prologue: kBufs - 1 stages in flight
+    int it_issue = rg.it_begin;  // next iteration to issue loads for
+    int issued = 0;              // stages issued so far
+#pragma unroll
+    for (int s = 0; s < kBufs - 1; s++) {
+        if (it_issue < rg.it_end) {
+            int gi, bi, li;
+            q4k_stage_at(rg, it_issue, gi, bi, li);
+            q4k_issue_all(q4k_issue_desc(w, xp, lds + (issued % kBufs) * kBufPieces, spare, gi, bi, li, n_out,
+                                         row_bytes, true),
+                          tid);
+            it_issue += li;
+            issued++;
+        }
+    }
+    int it = rg.it_begin;
+    int done = 0;  // stages computed so far
+    while (it < rg.it_end) {
+        int gc, bc, lc;
+        q4k_stage_at(rg, it, gc, bc, lc);
+        // stage `done` has landed once at most (issued - done - 1) younger stages are in flight
+        if (issued - done - 1 >= kBufs - 2 && kBufs > 2)
+            __builtin_amdgcn_s_waitcnt(q4k_vmcnt((kBufs - 2) * kLoadsPerStage));
+        else
+            __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+        // A bare barrier, not __syncthreads(): that one carries a workgroup-scope fence, which waits
+        // for every load in flight and would undo the prefetch.  The s_waitcnt above is the only
+        // ordering this needs: each wave's own pieces have landed before it arrives here.
+        __builtin_amdgcn_s_barrier();  // the whole stage is in LDS; buffer (done-1) % kBufs is free
+        // the stage kBufs-1 ahead is loaded into that free buffer while this one is computed
+        const bool more = it_issue < rg.it_end;
+        int gi = gc, bi = bc, li = lc;
+        if (more) q4k_stage_at(rg, it_issue, gi, bi, li);
+        const Q4KIssue next =
+            q4k_issue_desc(w, xp, lds + (issued % kBufs) * kBufPieces, spare, gi, bi, li, n_out, row_bytes, more);
+        q4k_compute(lds + (done % kBufs) * kBufPieces, lc, tid, magic, acc, acc_min, next);
+        if (more) {
+            it_issue += li;
+            issued++;
+        }
+        it += lc;
+        done++;
+        int gn = gc;
+        if (it < rg.it_end) gn = static_cast<int>(static_cast<uint32_t>(it) / static_cast<uint32_t>(nb));
+        if (it >= rg.it_end || gn != gc) q4k_flush(rg, gc, acc, acc_min, y, partials, epoch, n_out, n_rows, tid);
+    }
+    q4k_reduce_owned(rg, y, partials, epoch, n_out, n_rows, tid);
 }
 
 // ----------------------------------------------------------------------------
@@ -425,23 +611,17 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
 
     if (w_type == DFLASH_TYPE_Q4_K) {
         const int nb = static_cast<int>(n_in / DFL_QK_K);
+        const int groups = (tiles + kWavesQ4K - 1) / kWavesQ4K;
+        int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
+        const int64_t total = static_cast<int64_t>(groups) * nb;
+        if (n_wg > total) n_wg = static_cast<int>(total);
+        if (n_wg > ctx->n_partial_wgs) n_wg = ctx->n_partial_wgs;
+        if (n_wg < 1) n_wg = 1;
+        if (total * (n_wg + 1) >= (int64_t(1) << 31))
+            return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: problem too large for 32-bit work indices");
         off = 0;
         xp = dfl_ws_take<half8_t>(ctx, &off, static_cast<size_t>(nb) * kQ4KBlockFrags * sizeof(half8_t));
-        // K-slice length: 5 super-blocks when that divides K evenly, else 4
-        int kb = env_int("DFLASH_GEMM_KB", (nb % 5 == 0) ? 5 : 4);
-        if (kb < 1) kb = 1;
-        if (kb > 8) kb = 8;
-        if (kb > nb) kb = nb;
-        const int n_slices = (nb + kb - 1) / kb;
-        const int groups = (tiles + kWavesQ4K - 1) / kWavesQ4K;
-        float *partials = nullptr;
-        if (n_slices > 1)
-            partials = dfl_ws_take<float>(ctx, &off, static_cast<size_t>(n_slices) * tiles * 256 * sizeof(float));
-        if (!xp || (n_slices > 1 && !partials))
-            return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");
-        if (groups > ctx->n_counters)
-            return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: n_out %lld needs more than %d tile groups",
-                            static_cast<long long>(n_out), ctx->n_counters);
+        if (!xp) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");
         {
             dfl_timed timer(ctx, st, DFL_T_PREP);
             if (x_type == DFLASH_TYPE_F32)
@@ -449,21 +629,36 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
             else
                 prep_x_q4k_kernel<_Float16><<<nb, 256, 0, st>>>(static_cast<const _Float16 *>(x), xp, n_rows, n_in);
         }
-        const uint8_t *wb = static_cast<const uint8_t *>(w);
-        const int kbt = kb <= 4 ? 4 : (kb == 5 ? 5 : 8);
-        const size_t lds = static_cast<size_t>(kbt) * kQ4KBlockFrags * sizeof(half8_t);
-        const dim3 grid(static_cast<unsigned>(groups * n_slices));
+        // three LDS buffers when the device has the full 160 KiB per workgroup, else two
+        const int bufs = env_int("DFLASH_GEMM_BUFS", ctx->lds_bytes >= (3 * kBufPieces + 64) * 16 ? 3 : 2);
+        const size_t lds = static_cast<size_t>(bufs * kBufPieces + 64) * sizeof(half8_t);
+        ctx->epoch += 1;
+        if (ctx->epoch == 0) ctx->epoch = 1;
+        Q4KTagged *partials = reinterpret_cast<Q4KTagged *>(ctx->tagged_partials);
         dfl_timed timer(ctx, st, DFL_T_GEMM);
-#define DFL_LAUNCH_Q4K(KBT)                                                                                      \
-    gemm_q4k_kernel<KBT><<<grid, 64 * kWavesQ4K, lds, st>>>(wb, xp, y, partials, ctx->counters,                  \
-                                                           static_cast<int>(n_out), nb, n_rows, kb, n_slices)
-        if (kbt == 4)
-            DFL_LAUNCH_Q4K(4);
-        else if (kbt == 5)
-            DFL_LAUNCH_Q4K(5);
-        else
-            DFL_LAUNCH_Q4K(8);
-#undef DFL_LAUNCH_Q4K
+        if (bufs == 3) {
+            static bool attr3 = false;
+            if (!attr3) {
+                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<3>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       static_cast<int>(lds)));
+                attr3 = true;
+            }
+            gemm_q4k_stream_kernel<3><<<n_wg, kThreadsQ4K, lds, st>>>(static_cast<const uint8_t *>(w), xp, y, partials,
+                                                                      ctx->epoch, static_cast<int>(n_out), nb, n_rows,
+                                                                      groups);
+        } else {
+            static bool attr2 = false;
+            if (!attr2) {
+                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<2>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       static_cast<int>(lds)));
+                attr2 = true;
+            }
+            gemm_q4k_stream_kernel<2><<<n_wg, kThreadsQ4K, lds, st>>>(static_cast<const uint8_t *>(w), xp, y, partials,
+                                                                      ctx->epoch, static_cast<int>(n_out), nb, n_rows,
+                                                                      groups);
+        }
     } else {
         if (!xp) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");
         unsigned prep_grid = static_cast<unsigned>((n_steps * 64 + 255) / 256);
