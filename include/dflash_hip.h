@@ -93,6 +93,24 @@ size_t dflash_row_bytes(int32_t type, size_t n_in);
 int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
                            int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream);
 
+/* ---- block-causal verify attention ------------------------------------------------
+ * The reference verifies a block with a per-row loop: encode_scatter_offset_f32_to_f16_kv +
+ * encode_attn_decode_v4_f32 / encode_attn_decode_f16kv_f32, once per row
+ * (metal_dflash.rs:9963-10062; kernels/attn_v4.metal, kernels/attn.metal:266-336; CPU form
+ * forward.rs:893-922).  This call is those n_rows launches in one: row i attends cache
+ * positions [0, ctx_len + i].
+ *   q        [n_rows][n_q][head_dim], f32 or f16 (q_type)
+ *   k_cache  [kv_capacity][n_kv][head_dim] f16; rows ctx_len .. ctx_len+n_rows-1 hold the block
+ *   v_cache  v_layout 0: same layout as k_cache (transposed into workspace first; small caches)
+ *            v_layout 1: transposed [n_kv][head_dim][kv_capacity] f16 (native; capacity % 32 == 0)
+ *   out      [n_rows][n_q][head_dim] f32
+ * 1 <= n_rows <= 16; n_q % n_kv == 0 with at most 16 query heads per KV head; head_dim 64, 128
+ * or 256.  Enqueue-only. */
+int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache,
+                                 const void *v_cache, int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q,
+                                 int32_t n_kv, int32_t head_dim, int64_t kv_capacity, float scale, float *out,
+                                 dflash_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -75,6 +75,8 @@ def _declare(L):
     L.dflash_dequant.argtypes = [vp, i32, vp, sz, vp, vp]
     L.dflash_gemm_fewrow.restype = i32
     L.dflash_gemm_fewrow.argtypes = [vp, i32, vp, vp, i32, vp, i64, i64, i32, vp]
+    L.dflash_attn_verify_block.restype = i32
+    L.dflash_attn_verify_block.argtypes = [vp, vp, i32, vp, vp, i32, i64, i32, i32, i32, i32, i64, f32, vp, vp]
 
 
 def _torch():
@@ -156,3 +158,19 @@ class Context:
         torch = _torch()
         y = torch.empty((x.shape[0], n_out), dtype=torch.float32, device=x.device)
         return self.encode_mat_mat_dispatch_dflash_verify(weight, w_type, x, y, n_in, n_out, x.shape[0])
+
+    # ---- per-row scatter + decode attention loop of packed verify (metal_dflash.rs:9963-10062)
+    def attn_verify_block(self, q, k_cache, v_cache, ctx_len: int, scale: float, v_transposed: bool = False,
+                          out=None):
+        """q [n_rows, n_q, hd] f32/f16; k_cache [cap, n_kv, hd] f16; v_cache the same, or
+        [n_kv, hd, cap] when v_transposed.  Row i attends positions [0, ctx_len + i]."""
+        torch = _torch()
+        n_rows, n_q, hd = q.shape
+        cap, n_kv = k_cache.shape[0], k_cache.shape[1]
+        q_type = TYPE_F32 if q.dtype == torch.float32 else TYPE_F16
+        if out is None:
+            out = torch.empty((n_rows, n_q, hd), dtype=torch.float32, device=q.device)
+        self._check(self._lib.dflash_attn_verify_block(self._h, q.data_ptr(), q_type, k_cache.data_ptr(),
+                                                       v_cache.data_ptr(), 1 if v_transposed else 0, ctx_len, n_rows,
+                                                       n_q, n_kv, hd, cap, scale, out.data_ptr(), _stream_ptr()))
+        return out
