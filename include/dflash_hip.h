@@ -111,6 +111,94 @@ int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int32_t q_type,
                                  int32_t n_kv, int32_t head_dim, int64_t kv_capacity, float scale, float *out,
                                  dflash_stream_t stream);
 
+/* ---- row-wise selection over logits -------------------------------------------------
+ * logits [n_rows][stride] f32 (stride >= vocab).  All enqueue-only, outputs on the device.
+ *
+ * dflash_argmax_top2: kernel_argmax_top2_f32 (kernels/elementwise.metal:1231-1286, encoder
+ *   metal/elementwise.rs:1196-1318): IEEE comparisons, lowest index on ties, gap = top1 - top2
+ *   (0 when the maximum occurs twice, +inf for vocab == 1), an all-NaN row gives index -1.
+ * dflash_argmax_greedy: kernel_argmax_f32_greedy (elementwise.metal:1300-1359) == greedy_token
+ *   (sampling.rs:1159-1181): f32 total order, lowest index on ties, a row with a NaN gives
+ *   ~(lowest NaN index).
+ * dflash_top16: kernel_topk16_f32 (kernels/dflash2.metal:96-170): the 16 best (value, index)
+ *   pairs by total order, ties to the lower index; unfilled slots are (-inf, -1). */
+int32_t dflash_argmax_top2(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64_t vocab, int64_t stride,
+                           int32_t *idx, float *gap, dflash_stream_t stream);
+int32_t dflash_argmax_greedy(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64_t vocab, int64_t stride,
+                             int32_t *idx, dflash_stream_t stream);
+int32_t dflash_top16(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64_t vocab, int64_t stride,
+                     int32_t *ids, float *vals, dflash_stream_t stream);
+
+/* ---- sampler state (host side) ------------------------------------------------------
+ * SamplingConfig / Sampler (sampling.rs:18-145, 304-366): one request-local random stream.
+ * rng_kind 0 = xoshiro256++ seeded by SplitMix64 (the reference's generator, sampling.rs:1621-1670),
+ * 1 = Philox4x32-10 counter stream (key = seed, counter = draw index; u64 = word0 | word1 << 32).
+ * A unit draw is (u64 >> 11) / 2^53. */
+typedef struct {
+    float temperature; /* 0 = greedy */
+    float top_p;       /* (0, 1] */
+    float min_p;       /* [0, 1] */
+    int32_t rng_kind;
+    uint64_t top_k;    /* 0 = off */
+    uint64_t seed;
+} dflash_sampling_config;
+
+typedef struct {
+    dflash_sampling_config cfg;
+    uint64_t s[4];  /* xoshiro state, or s[0] = Philox stream position */
+    uint64_t draws;
+} dflash_sampler;
+
+int32_t dflash_sampler_init(dflash_sampler *s, const dflash_sampling_config *cfg);             /* Sampler::new */
+int32_t dflash_sampler_at_draw(dflash_sampler *s, const dflash_sampling_config *cfg, uint64_t draws); /* ::at_draw */
+/* the next `n` unit draws of the stream, without advancing it (Sampler::gpu_uniform, sampling.rs:317-326) */
+void dflash_sampler_peek(const dflash_sampler *s, int32_t n, double *out_host);
+void dflash_sampler_advance(dflash_sampler *s, uint64_t draws);
+
+/* ---- accept-prefix decision ---------------------------------------------------------
+ * decide_dflash_accept_prefix (metal_dflash/accept.rs:76-183) with the Sampler's couplings
+ * (sampling.rs:530-603, 692-790), evaluated on the GPU.  Row r of target_logits predicts
+ * verified_tokens[r+1]; the last reached row supplies the bonus.
+ *   proposal_mode 0: deterministic drafts (couple_deterministic_proposal)
+ *                 1: sparse proposals: n_proposals (= n_tokens - 1) rows; row r has
+ *                    prop_counts_host[r] (token, weight) candidates, stored back to back
+ *                    (couple_sparse_proposal; prop_tokens_host[r] must equal verified_tokens[r+1])
+ *                 2: vocabulary-wide draft distribution softmax(draft_logits / draft_temperature)
+ *                    (sum order: 1024-token tiles, 256 four-element slots, halving tree, tiles
+ *                    added in order)
+ * The whole block is validated before anything is drawn; the sampler advances by the draws
+ * actually consumed and only on DFLASH_OK.  top_k must be in 1..64 (or vocab <= 64) when
+ * temperature > 0.  Synchronises: the decision is returned on the host. */
+enum { DFLASH_CARRY_NONE = 0, DFLASH_CARRY_CORRECTION = 1, DFLASH_CARRY_BONUS = 2 };
+enum { DFLASH_STOP_NONE = 0, DFLASH_STOP_EOS = 1, DFLASH_STOP_TOKEN_LIMIT = 2 };
+
+typedef struct {
+    int32_t n_accepted;
+    int32_t accepted_drafts[16];
+    int32_t carry_kind;
+    int32_t carry_token;
+    int32_t stop_reason;
+    int32_t retain_input_count;
+    int32_t draws_used;
+    int32_t err_row;    /* row of a sampling error, else -1 */
+    int32_t err_code;   /* DFLASH_ERR_* of that error */
+    int64_t err_index;  /* offending token / NaN index, else -1 */
+} dflash_accept_decision;
+
+typedef struct {
+    int32_t token;
+    int32_t pad;
+    double weight;
+} dflash_weighted_candidate;
+
+int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified_tokens_host, int32_t n_tokens,
+                             const float *target_logits, int64_t vocab, int32_t proposal_mode, int32_t n_proposals,
+                             const int32_t *prop_tokens_host, const int32_t *prop_counts_host,
+                             const dflash_weighted_candidate *prop_cands_host, const float *draft_logits,
+                             float draft_temperature, dflash_sampler *sampler, int64_t remaining_output_budget,
+                             const int32_t *stop_ids_host, int32_t n_stop, dflash_accept_decision *out_host,
+                             dflash_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,7 +20,17 @@ from .binding import (  # noqa: F401
     TYPE_Q4_K,
     TYPE_Q6_K,
     TYPE_Q8_0,
+    AcceptDecision,
+    CARRY_BONUS,
+    CARRY_CORRECTION,
+    CARRY_NONE,
     Context,
+    RNG_PHILOX,
+    RNG_XOSHIRO,
+    STOP_EOS,
+    STOP_NONE,
+    STOP_TOKEN_LIMIT,
+    Sampler,
     declared_symbols,
     lib,
 )

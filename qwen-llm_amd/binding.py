@@ -33,6 +33,30 @@ class DFlashError(RuntimeError):
         self.message = message
 
 
+class SamplingConfigC(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("min_p", C.c_float), ("rng_kind", C.c_int32),
+                ("top_k", C.c_uint64), ("seed", C.c_uint64)]
+
+
+class SamplerC(C.Structure):
+    _fields_ = [("cfg", SamplingConfigC), ("s", C.c_uint64 * 4), ("draws", C.c_uint64)]
+
+
+class WeightedCandidateC(C.Structure):
+    _fields_ = [("token", C.c_int32), ("pad", C.c_int32), ("weight", C.c_double)]
+
+
+class AcceptDecisionC(C.Structure):
+    _fields_ = [("n_accepted", C.c_int32), ("accepted_drafts", C.c_int32 * 16), ("carry_kind", C.c_int32),
+                ("carry_token", C.c_int32), ("stop_reason", C.c_int32), ("retain_input_count", C.c_int32),
+                ("draws_used", C.c_int32), ("err_row", C.c_int32), ("err_code", C.c_int32), ("err_index", C.c_int64)]
+
+
+RNG_XOSHIRO, RNG_PHILOX = 0, 1
+CARRY_NONE, CARRY_CORRECTION, CARRY_BONUS = 0, 1, 2
+STOP_NONE, STOP_EOS, STOP_TOKEN_LIMIT = 0, 1, 2
+
+
 def declared_symbols() -> list[str]:
     """Every function name the public header declares."""
     text = open(HEADER_PATH).read()
@@ -75,8 +99,75 @@ def _declare(L):
     L.dflash_dequant.argtypes = [vp, i32, vp, sz, vp, vp]
     L.dflash_gemm_fewrow.restype = i32
     L.dflash_gemm_fewrow.argtypes = [vp, i32, vp, vp, i32, vp, i64, i64, i32, vp]
+    for name in ("dflash_argmax_top2", "dflash_top16"):
+        getattr(L, name).restype = i32
+        getattr(L, name).argtypes = [vp, vp, i32, i64, i64, vp, vp, vp]
+    L.dflash_argmax_greedy.restype = i32
+    L.dflash_argmax_greedy.argtypes = [vp, vp, i32, i64, i64, vp, vp]
+    L.dflash_sampler_init.restype = i32
+    L.dflash_sampler_init.argtypes = [C.POINTER(SamplerC), C.POINTER(SamplingConfigC)]
+    L.dflash_sampler_at_draw.restype = i32
+    L.dflash_sampler_at_draw.argtypes = [C.POINTER(SamplerC), C.POINTER(SamplingConfigC), C.c_uint64]
+    L.dflash_sampler_peek.restype = None
+    L.dflash_sampler_peek.argtypes = [C.POINTER(SamplerC), i32, C.POINTER(C.c_double)]
+    L.dflash_sampler_advance.restype = None
+    L.dflash_sampler_advance.argtypes = [C.POINTER(SamplerC), C.c_uint64]
+    L.dflash_accept_prefix.restype = i32
+    L.dflash_accept_prefix.argtypes = [vp, C.POINTER(i32), i32, vp, i64, i32, i32, C.POINTER(i32), C.POINTER(i32),
+                                       C.POINTER(WeightedCandidateC), vp, f32, C.POINTER(SamplerC), i64,
+                                       C.POINTER(i32), i32, C.POINTER(AcceptDecisionC), vp]
     L.dflash_attn_verify_block.restype = i32
     L.dflash_attn_verify_block.argtypes = [vp, vp, i32, vp, vp, i32, i64, i32, i32, i32, i32, i64, f32, vp, vp]
+
+
+class Sampler:
+    """Request-local sampler state (sampling.rs:304-366): config + random stream + draw count."""
+
+    def __init__(self, temperature=0.0, top_k=0, top_p=1.0, min_p=0.0, seed=0, rng_kind=RNG_XOSHIRO, draws=0):
+        self.c = SamplerC()
+        cfg = SamplingConfigC(temperature, top_p, min_p, rng_kind, top_k, seed)
+        rc = lib().dflash_sampler_at_draw(C.byref(self.c), C.byref(cfg), draws)
+        if rc:
+            raise DFlashError(rc, "invalid sampling configuration")
+
+    @classmethod
+    def at_draw(cls, other: "Sampler", draws: int) -> "Sampler":
+        c = other.c.cfg
+        return cls(c.temperature, c.top_k, c.top_p, c.min_p, c.seed, c.rng_kind, draws)
+
+    def clone(self) -> "Sampler":
+        t = Sampler.__new__(Sampler)
+        t.c = SamplerC()
+        C.memmove(C.byref(t.c), C.byref(self.c), C.sizeof(SamplerC))
+        return t
+
+    @property
+    def draws(self) -> int:
+        return int(self.c.draws)
+
+    def state(self):
+        return (tuple(self.c.s), int(self.c.draws))
+
+    def peek(self, n: int):
+        out = (C.c_double * n)()
+        lib().dflash_sampler_peek(C.byref(self.c), n, out)
+        return list(out)
+
+
+class AcceptDecision:
+    """DFlashAcceptDecision (metal_dflash/accept.rs:17-32)."""
+
+    def __init__(self, c: AcceptDecisionC):
+        self.accepted_drafts = list(c.accepted_drafts[: c.n_accepted])
+        self.carry_kind = c.carry_kind
+        self.carry_token = c.carry_token if c.carry_kind else 0
+        self.stop_reason = c.stop_reason
+        self.retain_input_count = c.retain_input_count
+        self.draws_used = c.draws_used
+        self.err_row, self.err_code, self.err_index = c.err_row, c.err_code, c.err_index
+
+    def key(self):
+        return (self.accepted_drafts, self.carry_kind, self.carry_token, self.stop_reason, self.retain_input_count)
 
 
 def _torch():
@@ -174,3 +265,69 @@ class Context:
                                                        v_cache.data_ptr(), 1 if v_transposed else 0, ctx_len, n_rows,
                                                        n_q, n_kv, hd, cap, scale, out.data_ptr(), _stream_ptr()))
         return out
+
+    # ---- argmax family (metal/elementwise.rs:1196-1318) and top-16 (metal/elementwise.rs:1370-1386)
+    def _rows(self, logits):
+        if logits.dim() == 1:
+            logits = logits.unsqueeze(0)
+        return logits, logits.shape[0], logits.shape[1], logits.stride(0)
+
+    def argmax_top2(self, logits):
+        torch = _torch()
+        logits, n, v, stride = self._rows(logits)
+        idx = torch.empty(n, dtype=torch.int32, device=logits.device)
+        gap = torch.empty(n, dtype=torch.float32, device=logits.device)
+        self._check(self._lib.dflash_argmax_top2(self._h, logits.data_ptr(), n, v, stride, idx.data_ptr(),
+                                                 gap.data_ptr(), _stream_ptr()))
+        return idx, gap
+
+    def argmax_greedy(self, logits):
+        torch = _torch()
+        logits, n, v, stride = self._rows(logits)
+        idx = torch.empty(n, dtype=torch.int32, device=logits.device)
+        self._check(self._lib.dflash_argmax_greedy(self._h, logits.data_ptr(), n, v, stride, idx.data_ptr(),
+                                                   _stream_ptr()))
+        return idx
+
+    def top16(self, logits):
+        torch = _torch()
+        logits, n, v, stride = self._rows(logits)
+        ids = torch.empty((n, 16), dtype=torch.int32, device=logits.device)
+        vals = torch.empty((n, 16), dtype=torch.float32, device=logits.device)
+        self._check(self._lib.dflash_top16(self._h, logits.data_ptr(), n, v, stride, ids.data_ptr(), vals.data_ptr(),
+                                           _stream_ptr()))
+        return ids, vals
+
+    # ---- decide_dflash_accept_prefix (metal_dflash/accept.rs:76-84)
+    def decide_dflash_accept_prefix(self, verified_tokens, target_logits, vocab, proposals, sampler: Sampler,
+                                    remaining_output_budget, stop_ids, draft_logits=None, draft_temperature=0.0):
+        """verified_tokens: [carry, drafts...] (host ints); target_logits: device f32 [len, vocab];
+        proposals: None (deterministic drafts) or a list of (token, [(token, weight), ...]) per draft row;
+        draft_logits: device f32 [len-1, vocab] selects the vocabulary-wide proposal instead.
+        Returns an AcceptDecision; raises DFlashError (sampler unchanged) on any error."""
+        n = len(verified_tokens)
+        toks = (C.c_int32 * max(1, n))(*verified_tokens)
+        stops = (C.c_int32 * max(1, len(stop_ids)))(*stop_ids)
+        mode, n_props, ptoks, pcnts, pcands = 0, 0, None, None, None
+        if draft_logits is not None:
+            mode = 2
+        elif proposals is not None:
+            mode, n_props = 1, len(proposals)
+            ptoks = (C.c_int32 * max(1, n_props))(*[p[0] for p in proposals])
+            pcnts = (C.c_int32 * max(1, n_props))(*[len(p[1]) for p in proposals])
+            flat = [c for p in proposals for c in p[1]]
+            pcands = (WeightedCandidateC * max(1, len(flat)))()
+            for i, (t, w) in enumerate(flat):
+                pcands[i].token, pcands[i].weight = t, w
+        if target_logits is not None and n > 0 and vocab > 0 and target_logits.numel() != n * vocab:
+            raise DFlashError(7, "target logits extent mismatch")
+        out = AcceptDecisionC()
+        rc = self._lib.dflash_accept_prefix(
+            self._h, toks, n, target_logits.data_ptr() if target_logits is not None else None, vocab, mode, n_props,
+            ptoks, pcnts, pcands, draft_logits.data_ptr() if draft_logits is not None else None, draft_temperature,
+            C.byref(sampler.c), remaining_output_budget, stops, len(stop_ids), C.byref(out), _stream_ptr())
+        if rc:
+            err = DFlashError(rc, self._lib.dflash_last_error(self._h).decode())
+            err.decision = AcceptDecision(out)
+            raise err
+        return AcceptDecision(out)

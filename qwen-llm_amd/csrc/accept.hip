@@ -1,0 +1,963 @@
+// Acceptance: row-wise argmax / top-k over logits, the sampler-v1 filter chain and the
+// speculative couplings, and the accept-prefix block decision, on the GPU.
+//
+// Reference: kernels/elementwise.metal:1153-1359 (argmax family), kernels/dflash2.metal:73-170
+// (top-16), crates/qwen-llm/src/sampling.rs (chain :1541-1615, couplings :692-790, ordering keys
+// :1206-1235, RNG :1621-1670), crates/qwen-llm/src/metal_dflash/accept.rs:76-183 (block decision,
+// CPU-only in the reference).
+//
+// Everything here is HBM-bound streaming over [rows][vocab] f32 plus O(top_k) arithmetic:
+//  * a row is cut into chunks of 8192 tokens so that rows x chunks workgroups cover the chip;
+//    each workgroup streams its chunk once with coalesced loads;
+//  * order decisions use the reference's integer keys (descending f32 total order above ascending
+//    token id), so the selected candidates and their order are exact, not approximately sorted;
+//  * top-k of a chunk: the k-th best of the 1024 per-thread bests bounds every winner, so only
+//    the <= 8k elements of the k winning threads are sorted (bitonic, in LDS);
+//  * everything that feeds a comparison with a uniform draw is f64 and sequential, in the order
+//    of the reference's loops: one thread walks the <= 64 candidates of a row, one thread walks
+//    the rows of the block.
+#include "common.h"
+
+#include <cmath>
+#include <cstring>
+
+namespace {
+
+constexpr int kChunk = 8192;       // tokens per workgroup
+constexpr int kSelThreads = 1024;  // 8 tokens per thread
+constexpr int kMaxK = 64;          // largest supported top-k
+constexpr int kMaxRows = 16;
+constexpr uint64_t kNoKey = ~0ull;
+constexpr int kNoNan = 0x7fffffff;
+
+// sampling.rs:1206-1220: a u32 whose ascending order is descending f32 total order
+__device__ __host__ __forceinline__ uint32_t desc_bits(uint32_t bits) {
+    uint32_t asc = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+    return ~asc;
+}
+__device__ __forceinline__ uint64_t cand_key(uint32_t token, float logit) {
+    return (static_cast<uint64_t>(desc_bits(__float_as_uint(logit))) << 32) | token;
+}
+// sampling.rs:1223-1231
+__device__ __forceinline__ float key_logit(uint64_t key) {
+    uint32_t asc = ~static_cast<uint32_t>(key >> 32);
+    uint32_t bits = (asc & 0x80000000u) ? (asc & 0x7fffffffu) : ~asc;
+    return __uint_as_float(bits);
+}
+__device__ __forceinline__ int32_t key_token(uint64_t key) { return static_cast<int32_t>(static_cast<uint32_t>(key)); }
+
+// Ascending bitonic sort of n (power of two, <= 2 * blockDim.x) keys in LDS.
+__device__ void bitonic_sort(uint64_t *keys, int n) {
+    for (int size = 2; size <= n; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = threadIdx.x; i < n / 2; i += blockDim.x) {
+                int lo = 2 * i - (i & (stride - 1));  // index with the `stride` bit clear
+                int hi = lo + stride;
+                bool up = (lo & size) == 0;
+                uint64_t a = keys[lo], b = keys[hi];
+                if ((a > b) == up) {
+                    keys[lo] = b;
+                    keys[hi] = a;
+                }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// ------------------------------------------------------------------------------------------
+// argmax_top2: IEEE comparisons, lowest index on ties, second value counts duplicates
+// ------------------------------------------------------------------------------------------
+struct Top2 {
+    float v1;
+    uint32_t i1;
+    float v2;
+};
+
+__device__ __forceinline__ Top2 top2_merge(Top2 a, Top2 b) {
+    if (b.v1 > a.v1 || (b.v1 == a.v1 && b.i1 < a.i1)) {
+        Top2 t = a;
+        a = b;
+        b = t;
+    }
+    if (b.v1 > a.v2) a.v2 = b.v1;
+    if (b.v2 > a.v2) a.v2 = b.v2;
+    return a;
+}
+
+__global__ void __launch_bounds__(kSelThreads)
+    top2_chunk_kernel(const float *__restrict__ logits, int64_t vocab, int64_t stride, Top2 *__restrict__ part) {
+    __shared__ Top2 sh[kSelThreads];
+    const int row = blockIdx.y, chunk = blockIdx.x;
+    const float *x = logits + row * stride;
+    Top2 t = {-INFINITY, 0xffffffffu, -INFINITY};
+#pragma unroll
+    for (int j = 0; j < kChunk / kSelThreads; j++) {
+        int64_t i = static_cast<int64_t>(chunk) * kChunk + j * kSelThreads + threadIdx.x;
+        if (i < vocab) {
+            float v = x[i];
+            if (v > t.v1) {
+                t.v2 = t.v1;
+                t.v1 = v;
+                t.i1 = static_cast<uint32_t>(i);
+            } else if (v == t.v1 && static_cast<uint32_t>(i) < t.i1) {
+                t.v2 = t.v1;
+                t.i1 = static_cast<uint32_t>(i);
+            } else if (v > t.v2) {
+                t.v2 = v;
+            }
+        }
+    }
+    sh[threadIdx.x] = t;
+    for (int s = kSelThreads / 2; s > 0; s >>= 1) {
+        __syncthreads();
+        if (threadIdx.x < s) sh[threadIdx.x] = top2_merge(sh[threadIdx.x], sh[threadIdx.x + s]);
+    }
+    if (threadIdx.x == 0) part[row * gridDim.x + chunk] = sh[0];
+}
+
+__global__ void top2_final_kernel(const Top2 *__restrict__ part, int n_chunks, int32_t *__restrict__ idx,
+                                  float *__restrict__ gap) {
+    const int row = blockIdx.x;
+    if (threadIdx.x != 0) return;
+    Top2 t = part[row * n_chunks];
+    for (int c = 1; c < n_chunks; c++) t = top2_merge(t, part[row * n_chunks + c]);
+    idx[row] = static_cast<int32_t>(t.i1);
+    gap[row] = t.v1 - t.v2;
+}
+
+// ------------------------------------------------------------------------------------------
+// chunk selection: best K keys of a chunk (sorted), lowest NaN index, optional second row set
+// ------------------------------------------------------------------------------------------
+struct ChunkOut {
+    uint64_t keys[kMaxK];
+    int32_t nan_first;
+    int32_t pad;
+};
+
+// min over the workgroup of a key / an int, result broadcast
+__device__ uint64_t block_min_u64(uint64_t v, uint64_t *sh) {
+    for (int off = 32; off > 0; off >>= 1) {
+        uint64_t o = __shfl_xor(v, off, 64);
+        v = o < v ? o : v;
+    }
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    uint64_t r = sh[0];
+    for (int w = 1; w < static_cast<int>(blockDim.x >> 6); w++) r = sh[w] < r ? sh[w] : r;
+    return r;
+}
+
+// K == 1 fast path is the greedy / draft-max case: only the minimum key is needed.
+__global__ void __launch_bounds__(kSelThreads)
+    select_chunk_kernel(const float *__restrict__ logits, int64_t vocab, int64_t stride, int k,
+                        ChunkOut *__restrict__ out, bool nan_is_candidate) {
+    __shared__ uint64_t sk[kSelThreads];
+    __shared__ uint64_t cand[8 * kMaxK];
+    __shared__ int cnt;
+    __shared__ int nan_sh;
+    const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    const float *x = logits + row * stride;
+    uint64_t keys[kChunk / kSelThreads];
+    uint64_t best = kNoKey;
+    int nan_first = kNoNan;
+    if (tid == 0) {
+        cnt = 0;
+        nan_sh = kNoNan;
+    }
+#pragma unroll
+    for (int j = 0; j < kChunk / kSelThreads; j++) {
+        int64_t i = static_cast<int64_t>(chunk) * kChunk + j * kSelThreads + tid;
+        uint64_t key = kNoKey;
+        if (i < vocab) {
+            float v = x[i];
+            if (v != v) {
+                nan_first = nan_first < static_cast<int>(i) ? nan_first : static_cast<int>(i);
+                if (nan_is_candidate) key = cand_key(static_cast<uint32_t>(i), v);
+            } else {
+                key = cand_key(static_cast<uint32_t>(i), v);
+            }
+        }
+        keys[j] = key;
+        best = key < best ? key : best;
+    }
+    __syncthreads();
+    if (nan_first != kNoNan) atomicMin(&nan_sh, nan_first);
+    ChunkOut *o = out + (row * gridDim.x + chunk);
+    if (k == 1) {
+        uint64_t m = block_min_u64(best, sk);
+        if (tid == 0) {
+            o->keys[0] = m;
+            o->nan_first = nan_sh;
+        }
+        return;
+    }
+    // k-th best of the per-thread bests bounds every winner of the chunk
+    sk[tid] = best;
+    bitonic_sort(sk, kSelThreads);
+    const uint64_t tau = sk[k - 1];
+    if (best <= tau && best != kNoKey) {
+#pragma unroll
+        for (int j = 0; j < kChunk / kSelThreads; j++)
+            if (keys[j] <= tau && keys[j] != kNoKey) cand[atomicAdd(&cnt, 1)] = keys[j];
+    }
+    __syncthreads();
+    const int n_cand = cnt;  // <= 8 k
+    int n_sort = 2;
+    while (n_sort < n_cand) n_sort <<= 1;
+    for (int i = n_cand + tid; i < n_sort; i += kSelThreads) cand[i] = kNoKey;
+    bitonic_sort(cand, n_sort);
+    if (tid < k) o->keys[tid] = tid < n_sort ? cand[tid] : kNoKey;
+    if (tid == 0) o->nan_first = nan_sh;
+}
+
+// ------------------------------------------------------------------------------------------
+// per-row results
+// ------------------------------------------------------------------------------------------
+struct RowDist {
+    int32_t n_keep;     // candidates after every filter
+    int32_t err;        // DFLASH_ERR_* or 0
+    int64_t err_index;  // NaN index etc.
+    double total;       // sum of the kept weights (sequential)
+    int32_t tokens[kMaxK];
+    double weights[kMaxK];
+    // dense proposal side
+    int32_t d_err;
+    int32_t d_pad;
+    int64_t d_err_index;
+    double d_max_scaled;  // f64(max draft logit) / T
+    double d_total;       // P
+};
+
+struct ChainCfg {
+    float temperature, top_p, min_p;
+    int32_t k;          // effective top-k (<= kMaxK)
+    double ln_min_p;    // ln(f64(min_p)), computed on the host
+    float draft_temperature;
+    int32_t mode;       // proposal mode
+};
+
+// sampling.rs:1541-1615 on the ordered candidates of one row (keys ascending = best first)
+__device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowDist *d) {
+    double l[kMaxK];
+    int tok[kMaxK];
+    for (int i = 0; i < len; i++) {
+        l[i] = static_cast<double>(key_logit(keys[i]));
+        tok[i] = key_token(keys[i]);
+    }
+    if (c.min_p > 0.0f) {
+        double max_logit = l[0];
+        if (isfinite(max_logit)) {
+            double threshold = max_logit + c.ln_min_p;
+            int keep = 0;
+            for (int i = 0; i < len; i++)
+                if (l[i] >= threshold) {
+                    l[keep] = l[i];
+                    tok[keep] = tok[i];
+                    keep++;
+                }
+            len = keep;
+        }
+    }
+    if (len == 0) {
+        d->err = DFLASH_ERR_NO_CANDIDATES;
+        return;
+    }
+    if (l[0] == INFINITY) {
+        int keep = 0;
+        for (int i = 0; i < len; i++)
+            if (l[i] == INFINITY) {
+                l[keep] = l[i];
+                tok[keep] = tok[i];
+                keep++;
+            }
+        len = keep;
+    }
+    const double temperature = static_cast<double>(c.temperature);
+    for (int i = 0; i < len; i++) l[i] /= temperature;
+    double w[kMaxK];
+    int n_inf = 0;
+    for (int i = 0; i < len; i++) n_inf += (l[i] == INFINITY);
+    if (n_inf > 0) {
+        for (int i = 0; i < len; i++) w[i] = (l[i] == INFINITY) ? 1.0 : 0.0;
+    } else {
+        double max_logit = l[0];
+        if (max_logit == -INFINITY) {
+            d->err = DFLASH_ERR_NO_CANDIDATES;
+            return;
+        }
+        bool finite = true;
+        for (int i = 0; i < len; i++) {
+            w[i] = exp(l[i] - max_logit);
+            finite = finite && isfinite(w[i]);
+        }
+        if (!finite) {
+            d->err = DFLASH_ERR_NO_CANDIDATES;
+            return;
+        }
+    }
+    if (c.top_p < 1.0f) {
+        double total = -0.0;
+        for (int i = 0; i < len; i++) total += w[i];
+        double target = total * static_cast<double>(c.top_p);
+        double cumulative = 0.0;
+        int keep = 0;
+        for (int i = 0; i < len; i++) {
+            cumulative += w[i];
+            keep++;
+            if (cumulative >= target) break;
+        }
+        len = keep < 1 ? 1 : keep;
+    }
+    double total_weight = -0.0;
+    for (int i = 0; i < len; i++) total_weight += w[i];
+    if (!(isfinite(total_weight) && total_weight > 0.0)) {
+        d->err = DFLASH_ERR_NO_CANDIDATES;
+        return;
+    }
+    d->n_keep = len;
+    d->total = total_weight;
+    for (int i = 0; i < len; i++) {
+        d->tokens[i] = tok[i];
+        d->weights[i] = w[i];
+    }
+}
+
+// One workgroup per row: merge the chunk lists, order the best k, run the chain.
+__global__ void __launch_bounds__(kSelThreads)
+    row_merge_kernel(const ChunkOut *__restrict__ chunks, int n_chunks, const ChunkOut *__restrict__ draft_chunks,
+                     ChainCfg cfg, RowDist *__restrict__ rows, int32_t *__restrict__ greedy_out) {
+    __shared__ uint64_t sk[2 * kSelThreads];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int k = cfg.k;
+    const int n_in = n_chunks * k;  // <= 2048, checked on the host
+    int n_sort = 2;
+    while (n_sort < n_in) n_sort <<= 1;
+    for (int i = tid; i < n_sort; i += kSelThreads) {
+        uint64_t key = kNoKey;
+        if (i < n_in) key = chunks[row * n_chunks + i / k].keys[i % k];
+        sk[i] = key;
+    }
+    bitonic_sort(sk, n_sort);
+    if (tid != 0) return;
+    RowDist *d = rows + row;
+    d->n_keep = 0;
+    d->err = 0;
+    d->err_index = -1;
+    d->total = 0.0;
+    d->d_err = 0;
+    d->d_err_index = -1;
+    int nan_first = kNoNan;
+    for (int c = 0; c < n_chunks; c++) {
+        int nf = chunks[row * n_chunks + c].nan_first;
+        nan_first = nf < nan_first ? nf : nan_first;
+    }
+    if (greedy_out) greedy_out[row] = nan_first != kNoNan ? ~nan_first : key_token(sk[0]);
+    if (nan_first != kNoNan) {
+        d->err = DFLASH_ERR_NAN_LOGIT;
+        d->err_index = nan_first;
+    } else if (cfg.temperature == 0.0f) {
+        // greedy target: one-hot on the total-order argmax (sampling.rs:391-400)
+        d->n_keep = 1;
+        d->total = 1.0;
+        d->tokens[0] = key_token(sk[0]);
+        d->weights[0] = 1.0;
+    } else {
+        int len = 0;
+        while (len < k && sk[len] != kNoKey) len++;
+        run_chain(sk, len, cfg, d);
+    }
+    if (draft_chunks) {
+        uint64_t best = kNoKey;
+        int dn = kNoNan;
+        for (int c = 0; c < n_chunks; c++) {
+            const ChunkOut &dc = draft_chunks[row * n_chunks + c];
+            best = dc.keys[0] < best ? dc.keys[0] : best;
+            dn = dc.nan_first < dn ? dc.nan_first : dn;
+        }
+        d->d_max_scaled = static_cast<double>(key_logit(best)) / static_cast<double>(cfg.draft_temperature);
+        if (dn != kNoNan) {
+            d->d_err = DFLASH_ERR_NAN_LOGIT;
+            d->d_err_index = dn;
+        } else if (!isfinite(d->d_max_scaled)) {
+            d->d_err = DFLASH_ERR_NO_CANDIDATES;
+        }
+    }
+}
+
+// top-16 output from the merged order
+__global__ void __launch_bounds__(kSelThreads)
+    top16_merge_kernel(const ChunkOut *__restrict__ chunks, int n_chunks, int32_t *__restrict__ ids,
+                       float *__restrict__ vals) {
+    __shared__ uint64_t sk[2 * kSelThreads];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int n_in = n_chunks * 16;
+    int n_sort = 16;
+    while (n_sort < n_in) n_sort <<= 1;
+    for (int i = tid; i < n_sort; i += kSelThreads) sk[i] = i < n_in ? chunks[row * n_chunks + i / 16].keys[i % 16] : kNoKey;
+    bitonic_sort(sk, n_sort);
+    if (tid < 16) {
+        uint64_t key = sk[tid];
+        ids[row * 16 + tid] = key == kNoKey ? -1 : key_token(key);
+        vals[row * 16 + tid] = key == kNoKey ? -INFINITY : key_logit(key);
+    }
+}
+
+// Dense proposal: tile sums of exp(d/T - max/T) in the fixed shape: 1024-token tiles, slot t
+// holds ((e[4t]+e[4t+1])+e[4t+2])+e[4t+3], then a halving tree over the 256 slots.
+__global__ void __launch_bounds__(256) dense_tile_sum_kernel(const float *__restrict__ draft, int64_t vocab,
+                                                             int64_t stride, float temperature,
+                                                             const RowDist *__restrict__ rows,
+                                                             double *__restrict__ tile_sums) {
+    __shared__ double slot[256];
+    const int row = blockIdx.y, tile = blockIdx.x, t = threadIdx.x;
+    const double T = static_cast<double>(temperature);
+    const double mx = rows[row].d_max_scaled;
+    const float *x = draft + row * stride;
+    const int64_t base = static_cast<int64_t>(tile) * 1024 + 4 * t;
+    double acc = 0.0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        int64_t i = base + e;
+        double v = (i < vocab) ? exp(static_cast<double>(x[i]) / T - mx) : 0.0;
+        acc = (e == 0) ? v : acc + v;
+    }
+    slot[t] = acc;
+    for (int s = 128; s >= 1; s >>= 1) {
+        __syncthreads();
+        if (t < s) slot[t] += slot[t + s];
+    }
+    if (t == 0) tile_sums[row * gridDim.x + tile] = slot[0];
+}
+
+struct DecideArgs {
+    int32_t n_tokens, n_stop, mode, vocab;
+    int64_t budget;
+    const int32_t *verified;   // [n_tokens]
+    const int32_t *stop_ids;   // [n_stop]
+    const double *uniforms;    // [n_tokens + 1]
+    const RowDist *rows;
+    // sparse proposals
+    const int32_t *prop_tokens, *prop_offsets, *prop_counts;
+    const dflash_weighted_candidate *prop_cands;
+    // dense proposals
+    const float *draft;
+    int64_t draft_stride;
+    const double *tile_sums;
+    int32_t n_tiles;
+    float temperature, draft_temperature;
+};
+
+__device__ bool in_list(const int32_t *ids, int n, int32_t v) {
+    for (int i = 0; i < n; i++)
+        if (ids[i] == v) return true;
+    return false;
+}
+
+// first candidate whose running sum exceeds x, else the last (sampling.rs:1587-1596)
+__device__ int pick_index(const double *w, int n, double x) {
+    double cumulative = 0.0;
+    for (int i = 0; i < n; i++) {
+        cumulative += w[i];
+        if (x < cumulative) return i;
+    }
+    return n - 1;
+}
+
+// accept.rs:147-183 with the couplings of sampling.rs:692-790; one thread.
+__global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__ out) {
+    __shared__ double p_total[kMaxRows];
+    const int n_drafts = a.n_tokens - 1;
+    if (a.mode == 2 && static_cast<int>(threadIdx.x) < n_drafts) {
+        // P = sequential sum of the tile sums, tile order
+        double P = 0.0;
+        for (int t = 0; t < a.n_tiles; t++) P += a.tile_sums[threadIdx.x * a.n_tiles + t];
+        p_total[threadIdx.x] = P;
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    dflash_accept_decision d;
+    memset(&d, 0, sizeof(d));
+    d.err_row = -1;
+    d.err_index = -1;
+    int accepted = 0, draws = 0, carry_kind = DFLASH_CARRY_NONE, stop = DFLASH_STOP_NONE, carry_token = 0;
+    int err = 0;
+    const bool greedy = a.temperature == 0.0f;
+    for (;;) {
+        const int row = accepted;
+        const RowDist &rd = a.rows[row];
+        if (row == n_drafts) {  // bonus = sample(last reached row)
+            if (rd.err) {
+                err = rd.err;
+                d.err_index = rd.err_index;
+                d.err_row = row;
+                break;
+            }
+            int idx = 0;
+            if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
+            carry_kind = DFLASH_CARRY_BONUS;
+            carry_token = rd.tokens[idx];
+            break;
+        }
+        const int32_t draft = a.verified[row + 1];
+        bool acc = false;
+        int32_t correction = 0;
+        if (a.mode == 0) {  // deterministic coupling: draw the target token, accept iff it is the draft
+            if (rd.err) {
+                err = rd.err;
+                d.err_index = rd.err_index;
+                d.err_row = row;
+                break;
+            }
+            int idx = 0;
+            if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
+            correction = rd.tokens[idx];
+            acc = correction == draft;
+        } else {
+            // proposal probability q(draft) and, per target candidate, q(candidate)
+            double prop_total = 0.0, prop_tok_w = 0.0;
+            const dflash_weighted_candidate *pc = nullptr;
+            int n_pc = 0;
+            if (a.mode == 1) {
+                pc = a.prop_cands + a.prop_offsets[row];
+                n_pc = a.prop_counts[row];
+                if (n_pc == 0) err = DFLASH_ERR_NO_CANDIDATES;
+                for (int j = 0; j < n_pc && !err; j++) {
+                    if (!isfinite(pc[j].weight) || pc[j].weight < 0.0) {
+                        err = DFLASH_ERR_INVALID_PROPOSAL_WEIGHT;
+                        d.err_index = pc[j].token;
+                        break;
+                    }
+                    prop_total += pc[j].weight;
+                    if (pc[j].token == draft) prop_tok_w += pc[j].weight;
+                }
+                if (!err && !(isfinite(prop_total) && prop_total > 0.0)) err = DFLASH_ERR_NO_CANDIDATES;
+                if (!err && !(isfinite(prop_tok_w) && prop_tok_w > 0.0)) {
+                    err = DFLASH_ERR_MISSING_PROPOSAL_TOKEN;
+                    d.err_index = draft;
+                }
+            } else {
+                if (rd.d_err) {
+                    err = rd.d_err;
+                    d.err_index = rd.d_err_index;
+                }
+                prop_total = p_total[row];
+                if (!err && !(isfinite(prop_total) && prop_total > 0.0)) err = DFLASH_ERR_NO_CANDIDATES;
+                if (!err) {
+                    prop_tok_w = exp(static_cast<double>(a.draft[row * a.draft_stride + draft]) /
+                                         static_cast<double>(a.draft_temperature) -
+                                     rd.d_max_scaled);
+                    if (!(isfinite(prop_tok_w) && prop_tok_w > 0.0)) {
+                        err = DFLASH_ERR_MISSING_PROPOSAL_TOKEN;
+                        d.err_index = draft;
+                    }
+                }
+            }
+            if (!err && rd.err) {
+                err = rd.err;
+                d.err_index = rd.err_index;
+            }
+            if (err) {
+                d.err_row = row;
+                break;
+            }
+            double tp = -0.0;
+            for (int i = 0; i < rd.n_keep; i++)
+                if (rd.tokens[i] == draft) tp += rd.weights[i];
+            const double target_probability = tp / rd.total;
+            const double proposal_probability = prop_tok_w / prop_total;
+            const double acceptance = fmin(target_probability / proposal_probability, 1.0);
+            if (a.uniforms[draws++] < acceptance) {
+                acc = true;
+            } else {
+                double residual[kMaxK];
+                double residual_total = 0.0;
+                for (int i = 0; i < rd.n_keep; i++) {
+                    const double p = rd.weights[i] / rd.total;
+                    double q;
+                    if (a.mode == 1) {
+                        double qs = -0.0;
+                        for (int j = 0; j < n_pc; j++)
+                            if (pc[j].token == rd.tokens[i]) qs += pc[j].weight;
+                        q = qs / prop_total;
+                    } else {
+                        q = exp(static_cast<double>(a.draft[row * a.draft_stride + rd.tokens[i]]) /
+                                    static_cast<double>(a.draft_temperature) -
+                                rd.d_max_scaled) /
+                            prop_total;
+                    }
+                    const double wgt = fmax(p - q, 0.0);
+                    residual_total += wgt;
+                    residual[i] = wgt;
+                }
+                if (!(isfinite(residual_total) && residual_total > 0.0)) {
+                    err = DFLASH_ERR_NO_CANDIDATES;
+                    d.err_row = row;
+                    draws--;  // reported only; nothing is committed on an error
+                    break;
+                }
+                correction = rd.tokens[pick_index(residual, rd.n_keep, a.uniforms[draws++] * residual_total)];
+            }
+        }
+        if (!acc) {
+            carry_kind = DFLASH_CARRY_CORRECTION;
+            carry_token = correction;
+            break;
+        }
+        d.accepted_drafts[accepted++] = draft;
+        if (in_list(a.stop_ids, a.n_stop, draft)) {
+            stop = DFLASH_STOP_EOS;
+            break;
+        }
+        if (accepted == a.budget) {
+            stop = DFLASH_STOP_TOKEN_LIMIT;
+            break;
+        }
+    }
+    if (err) {
+        const int er = d.err_row;
+        const int64_t ei = d.err_index;
+        memset(&d, 0, sizeof(d));
+        d.err_row = er;
+        d.err_index = ei;
+        d.err_code = err;
+    } else {
+        d.n_accepted = accepted;
+        d.carry_kind = carry_kind;
+        d.carry_token = carry_token;
+        d.stop_reason = stop;
+        d.retain_input_count = 1 + accepted - (stop != DFLASH_STOP_NONE ? 1 : 0);
+        d.draws_used = draws;
+    }
+    *out = d;
+}
+
+// ------------------------------------------------------------------------------------------
+// host: random streams (sampling.rs:1621-1670; Philox4x32-10 after Salmon et al.)
+// ------------------------------------------------------------------------------------------
+uint64_t splitmix_next(uint64_t &state) {
+    state += 0x9e3779b97f4a7c15ull;
+    uint64_t v = state;
+    v = (v ^ (v >> 30)) * 0xbf58476d1ce4e5b9ull;
+    v = (v ^ (v >> 27)) * 0x94d049bb133111ebull;
+    return v ^ (v >> 31);
+}
+uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+uint64_t xoshiro_next(uint64_t s[4]) {
+    uint64_t result = rotl64(s[0] + s[3], 23) + s[0];
+    uint64_t t = s[1] << 17;
+    s[2] ^= s[0];
+    s[3] ^= s[1];
+    s[1] ^= s[2];
+    s[0] ^= s[3];
+    s[2] ^= t;
+    s[3] = rotl64(s[3], 45);
+    return result;
+}
+void philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; r++) {
+        uint64_t p0 = static_cast<uint64_t>(0xD2511F53u) * c0;
+        uint64_t p1 = static_cast<uint64_t>(0xCD9E8D57u) * c2;
+        uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0, n1 = static_cast<uint32_t>(p1);
+        uint32_t n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1, n3 = static_cast<uint32_t>(p0);
+        c0 = n0;
+        c1 = n1;
+        c2 = n2;
+        c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0;
+    out[1] = c1;
+    out[2] = c2;
+    out[3] = c3;
+}
+uint64_t sampler_raw_next(dflash_sampler *s) {
+    if (s->cfg.rng_kind == 1) {
+        uint64_t pos = s->s[0]++;
+        uint32_t ctr[4] = {static_cast<uint32_t>(pos), static_cast<uint32_t>(pos >> 32), 0, 0};
+        uint32_t key[2] = {static_cast<uint32_t>(s->cfg.seed), static_cast<uint32_t>(s->cfg.seed >> 32)};
+        uint32_t out[4];
+        philox4x32_10(ctr, key, out);
+        return static_cast<uint64_t>(out[0]) | (static_cast<uint64_t>(out[1]) << 32);
+    }
+    return xoshiro_next(s->s);
+}
+
+int32_t status_of_hip(hipError_t e) { return e == hipSuccess ? DFLASH_OK : DFLASH_ERR_HIP; }
+
+int32_t check_rows(dflash_ctx *ctx, const char *what, const float *logits, int32_t n_rows, int64_t vocab,
+                   int64_t stride) {
+    if (!logits) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "%s: null pointer", what);
+    if (n_rows < 1 || n_rows > 4096) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "%s: n_rows %d", what, n_rows);
+    if (vocab < 1) return dfl_fail(ctx, DFLASH_ERR_EMPTY_LOGITS, "%s: empty logits row", what);
+    if (vocab > 0x7fffffffll) return dfl_fail(ctx, DFLASH_ERR_VOCAB_TOO_LARGE, "%s: vocabulary %lld", what, static_cast<long long>(vocab));
+    if (stride < vocab) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "%s: stride %lld < vocab", what, static_cast<long long>(stride));
+    return DFLASH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t dflash_argmax_top2(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64_t vocab, int64_t stride,
+                           int32_t *idx, float *gap, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    int32_t rc = check_rows(ctx, "argmax_top2", logits, n_rows, vocab, stride);
+    if (rc) return rc;
+    if (!idx || !gap) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "argmax_top2: null output");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
+    size_t off = 0;
+    Top2 *part = dfl_ws_take<Top2>(ctx, &off, sizeof(Top2) * n_rows * n_chunks);
+    if (!part) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "argmax_top2: workspace too small");
+    dfl_timed timer(ctx, st, DFL_T_ARGMAX);
+    top2_chunk_kernel<<<dim3(n_chunks, n_rows), kSelThreads, 0, st>>>(logits, vocab, stride, part);
+    top2_final_kernel<<<n_rows, 64, 0, st>>>(part, n_chunks, idx, gap);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+int32_t dflash_argmax_greedy(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64_t vocab, int64_t stride,
+                             int32_t *idx, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    int32_t rc = check_rows(ctx, "argmax_greedy", logits, n_rows, vocab, stride);
+    if (rc) return rc;
+    if (!idx) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "argmax_greedy: null output");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
+    if (n_chunks > 2 * kSelThreads) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "argmax_greedy: vocabulary too large");
+    size_t off = 0;
+    ChunkOut *chunks = dfl_ws_take<ChunkOut>(ctx, &off, sizeof(ChunkOut) * n_rows * n_chunks);
+    RowDist *rows = dfl_ws_take<RowDist>(ctx, &off, sizeof(RowDist) * n_rows);
+    if (!chunks || !rows) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "argmax_greedy: workspace too small");
+    ChainCfg cfg = {};
+    cfg.k = 1;
+    dfl_timed timer(ctx, st, DFL_T_ARGMAX);
+    select_chunk_kernel<<<dim3(n_chunks, n_rows), kSelThreads, 0, st>>>(logits, vocab, stride, 1, chunks, false);
+    row_merge_kernel<<<n_rows, kSelThreads, 0, st>>>(chunks, n_chunks, nullptr, cfg, rows, idx);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+int32_t dflash_top16(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64_t vocab, int64_t stride,
+                     int32_t *ids, float *vals, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    int32_t rc = check_rows(ctx, "top16", logits, n_rows, vocab, stride);
+    if (rc) return rc;
+    if (!ids || !vals) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "top16: null output");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
+    if (n_chunks * 16 > 2 * kSelThreads) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "top16: vocabulary too large");
+    size_t off = 0;
+    ChunkOut *chunks = dfl_ws_take<ChunkOut>(ctx, &off, sizeof(ChunkOut) * n_rows * n_chunks);
+    if (!chunks) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "top16: workspace too small");
+    dfl_timed timer(ctx, st, DFL_T_ARGMAX);
+    select_chunk_kernel<<<dim3(n_chunks, n_rows), kSelThreads, 0, st>>>(logits, vocab, stride, 16, chunks, true);
+    top16_merge_kernel<<<n_rows, kSelThreads, 0, st>>>(chunks, n_chunks, ids, vals);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+// sampling.rs:133-144, 346-366
+int32_t dflash_sampler_init(dflash_sampler *s, const dflash_sampling_config *cfg) {
+    if (!s || !cfg) return DFLASH_ERR_INVALID_INPUT;
+    if (!std::isfinite(cfg->temperature) || cfg->temperature < 0.0f) return DFLASH_ERR_INVALID_TEMPERATURE;
+    if (!std::isfinite(cfg->top_p) || !(0.0f < cfg->top_p && cfg->top_p <= 1.0f)) return DFLASH_ERR_INVALID_TOP_P;
+    if (!std::isfinite(cfg->min_p) || !(0.0f <= cfg->min_p && cfg->min_p <= 1.0f)) return DFLASH_ERR_INVALID_MIN_P;
+    s->cfg = *cfg;
+    s->draws = 0;
+    if (cfg->rng_kind == 1) {
+        s->s[0] = s->s[1] = s->s[2] = s->s[3] = 0;
+    } else {
+        uint64_t sm = cfg->seed;
+        for (int i = 0; i < 4; i++) s->s[i] = splitmix_next(sm);
+    }
+    return DFLASH_OK;
+}
+
+int32_t dflash_sampler_at_draw(dflash_sampler *s, const dflash_sampling_config *cfg, uint64_t draws) {
+    int32_t rc = dflash_sampler_init(s, cfg);
+    if (rc) return rc;
+    dflash_sampler_advance(s, draws);
+    return DFLASH_OK;
+}
+
+void dflash_sampler_peek(const dflash_sampler *s, int32_t n, double *out_host) {
+    dflash_sampler copy = *s;
+    for (int32_t i = 0; i < n; i++)
+        out_host[i] = static_cast<double>(sampler_raw_next(&copy) >> 11) / 9007199254740992.0;
+}
+
+void dflash_sampler_advance(dflash_sampler *s, uint64_t draws) {
+    for (uint64_t i = 0; i < draws; i++) sampler_raw_next(s);
+    s->draws += draws;
+}
+
+int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n_tokens, const float *target_logits,
+                             int64_t vocab, int32_t mode, int32_t n_proposals, const int32_t *prop_tokens,
+                             const int32_t *prop_counts, const dflash_weighted_candidate *prop_cands,
+                             const float *draft_logits, float draft_temperature, dflash_sampler *sampler,
+                             int64_t budget, const int32_t *stop_ids, int32_t n_stop, dflash_accept_decision *out,
+                             dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!out || !sampler) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "accept_prefix: null sampler / output");
+    memset(out, 0, sizeof(*out));
+    out->err_row = -1;
+    out->err_index = -1;
+    // ---- whole-block validation before anything is drawn (accept.rs:85-130)
+    if (n_tokens < 1 || !verified) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "missing carry token");
+    if (vocab <= 0 || vocab > 0x7fffffffll) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "invalid vocabulary size");
+    if (n_tokens > kMaxRows)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "accept_prefix: %d verified tokens (at most %d)", n_tokens, kMaxRows);
+    if (!target_logits) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "target logits extent mismatch");
+    if (mode < 0 || mode > 2) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "accept_prefix: proposal mode %d", mode);
+    if (n_stop < 0 || (n_stop > 0 && !stop_ids)) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "accept_prefix: stop ids");
+    for (int i = 0; i < n_tokens; i++) {
+        if (verified[i] < 0 || verified[i] >= vocab) {
+            out->err_row = i;
+            out->err_index = verified[i];
+            return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "verified input token %d at index %d is outside vocabulary %lld",
+                            verified[i], i, static_cast<long long>(vocab));
+        }
+    }
+    const int n_drafts = n_tokens - 1;
+    int prop_offsets[kMaxRows] = {0};
+    int n_cands = 0;
+    if (mode == 1) {
+        if (n_proposals != n_drafts || (n_drafts > 0 && (!prop_tokens || !prop_counts)))
+            return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "proposal row count mismatch");
+        for (int r = 0; r < n_drafts; r++) {
+            if (prop_tokens[r] != verified[r + 1]) {
+                out->err_row = r;
+                out->err_index = prop_tokens[r];
+                return dfl_fail(ctx, DFLASH_ERR_PROPOSAL_MISMATCH, "proposal row %d sampled token %d, but verified draft is %d",
+                                r, prop_tokens[r], verified[r + 1]);
+            }
+            if (prop_counts[r] < 0 || (prop_counts[r] > 0 && !prop_cands))
+                return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "accept_prefix: proposal candidates");
+            prop_offsets[r] = n_cands;
+            for (int j = 0; j < prop_counts[r]; j++) {
+                int32_t t = prop_cands[n_cands + j].token;
+                if (t < 0 || t >= vocab) {
+                    out->err_row = r;
+                    out->err_code = DFLASH_ERR_PROPOSAL_TOKEN_OUT_OF_RANGE;
+                    out->err_index = t;
+                    return dfl_fail(ctx, DFLASH_ERR_PROPOSAL_TOKEN_OUT_OF_RANGE, "proposal token %d is outside the target vocabulary", t);
+                }
+            }
+            n_cands += prop_counts[r];
+        }
+    }
+    if (mode == 2) {
+        if (!draft_logits) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "accept_prefix: draft logits");
+        if (!(std::isfinite(draft_temperature) && draft_temperature > 0.0f))
+            return dfl_fail(ctx, DFLASH_ERR_INVALID_TEMPERATURE, "accept_prefix: draft temperature %f", draft_temperature);
+    }
+    // ---- terminal anchor / exhausted budget: no draw, nothing retained (accept.rs:131-145)
+    bool anchor_eos = false;
+    for (int i = 0; i < n_stop; i++) anchor_eos = anchor_eos || stop_ids[i] == verified[0];
+    if (anchor_eos || budget == 0) {
+        out->stop_reason = anchor_eos ? DFLASH_STOP_EOS : DFLASH_STOP_TOKEN_LIMIT;
+        return DFLASH_OK;
+    }
+    const dflash_sampling_config &sc = sampler->cfg;
+    int64_t k_eff = (sc.temperature == 0.0f) ? 1 : ((sc.top_k == 0 || static_cast<int64_t>(sc.top_k) >= vocab) ? vocab : static_cast<int64_t>(sc.top_k));
+    if (k_eff > kMaxK)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "accept_prefix: top_k %lld candidates (1..%d supported on the GPU)",
+                        static_cast<long long>(k_eff), kMaxK);
+    const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
+    if (n_chunks * k_eff > 2 * kSelThreads)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "accept_prefix: vocabulary %lld x top_k %lld too large", static_cast<long long>(vocab), static_cast<long long>(k_eff));
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int n_tiles = static_cast<int>((vocab + 1023) / 1024);
+    size_t off = 0;
+    ChunkOut *chunks = dfl_ws_take<ChunkOut>(ctx, &off, sizeof(ChunkOut) * n_tokens * n_chunks);
+    ChunkOut *dchunks = dfl_ws_take<ChunkOut>(ctx, &off, sizeof(ChunkOut) * n_tokens * n_chunks);
+    RowDist *rows = dfl_ws_take<RowDist>(ctx, &off, sizeof(RowDist) * n_tokens);
+    double *tile_sums = dfl_ws_take<double>(ctx, &off, sizeof(double) * n_tokens * n_tiles);
+    double *d_uniforms = dfl_ws_take<double>(ctx, &off, sizeof(double) * (kMaxRows + 2));
+    int32_t *d_small = dfl_ws_take<int32_t>(ctx, &off, sizeof(int32_t) * (4 * kMaxRows + n_stop + 8));
+    dflash_weighted_candidate *d_cands =
+        dfl_ws_take<dflash_weighted_candidate>(ctx, &off, sizeof(dflash_weighted_candidate) * (n_cands + 1));
+    dflash_accept_decision *d_out = dfl_ws_take<dflash_accept_decision>(ctx, &off, sizeof(dflash_accept_decision));
+    if (!chunks || !dchunks || !rows || !tile_sums || !d_uniforms || !d_small || !d_cands || !d_out)
+        return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "accept_prefix: workspace too small");
+
+    // small host inputs -> device
+    double uniforms[kMaxRows + 2];
+    dflash_sampler_peek(sampler, n_tokens + 1, uniforms);
+    int32_t small[4 * kMaxRows + 8];
+    int32_t *h_verified = small, *h_ptok = small + kMaxRows, *h_poff = small + 2 * kMaxRows, *h_pcnt = small + 3 * kMaxRows;
+    memset(small, 0, sizeof(small));
+    for (int i = 0; i < n_tokens; i++) h_verified[i] = verified[i];
+    for (int r = 0; r < n_drafts && mode == 1; r++) {
+        h_ptok[r] = prop_tokens[r];
+        h_poff[r] = prop_offsets[r];
+        h_pcnt[r] = prop_counts[r];
+    }
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(d_uniforms, uniforms, sizeof(double) * (n_tokens + 1), hipMemcpyHostToDevice, st));
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(d_small, small, sizeof(int32_t) * 4 * kMaxRows, hipMemcpyHostToDevice, st));
+    int32_t *d_stop = d_small + 4 * kMaxRows;
+    if (n_stop > 0)
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(d_stop, stop_ids, sizeof(int32_t) * n_stop, hipMemcpyHostToDevice, st));
+    if (n_cands > 0)
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(d_cands, prop_cands, sizeof(dflash_weighted_candidate) * n_cands,
+                                          hipMemcpyHostToDevice, st));
+
+    ChainCfg cfg;
+    cfg.temperature = sc.temperature;
+    cfg.top_p = sc.top_p;
+    cfg.min_p = sc.min_p;
+    cfg.k = static_cast<int32_t>(k_eff);
+    cfg.ln_min_p = sc.min_p > 0.0f ? std::log(static_cast<double>(sc.min_p)) : 0.0;
+    cfg.draft_temperature = draft_temperature;
+    cfg.mode = mode;
+    {
+        dfl_timed timer(ctx, st, DFL_T_ACCEPT);
+        select_chunk_kernel<<<dim3(n_chunks, n_tokens), kSelThreads, 0, st>>>(target_logits, vocab, vocab, cfg.k, chunks, false);
+        if (mode == 2 && n_drafts > 0)
+            select_chunk_kernel<<<dim3(n_chunks, n_drafts), kSelThreads, 0, st>>>(draft_logits, vocab, vocab, 1, dchunks, false);
+        row_merge_kernel<<<n_tokens, kSelThreads, 0, st>>>(chunks, n_chunks, (mode == 2 && n_drafts > 0) ? dchunks : nullptr,
+                                                          cfg, rows, nullptr);
+        if (mode == 2 && n_drafts > 0)
+            dense_tile_sum_kernel<<<dim3(n_tiles, n_drafts), 256, 0, st>>>(draft_logits, vocab, vocab, draft_temperature, rows, tile_sums);
+        DecideArgs a;
+        a.n_tokens = n_tokens;
+        a.n_stop = n_stop;
+        a.mode = mode;
+        a.vocab = static_cast<int32_t>(vocab);
+        a.budget = budget;
+        a.verified = d_small;
+        a.stop_ids = d_stop;
+        a.uniforms = d_uniforms;
+        a.rows = rows;
+        a.prop_tokens = d_small + kMaxRows;
+        a.prop_offsets = d_small + 2 * kMaxRows;
+        a.prop_counts = d_small + 3 * kMaxRows;
+        a.prop_cands = d_cands;
+        a.draft = draft_logits;
+        a.draft_stride = vocab;
+        a.tile_sums = tile_sums;
+        a.n_tiles = n_tiles;
+        a.temperature = sc.temperature;
+        a.draft_temperature = draft_temperature;
+        decide_kernel<<<1, 64, 0, st>>>(a, d_out);
+    }
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(out, d_out, sizeof(*out), hipMemcpyDeviceToHost, st));
+    DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+    if (out->err_code) {
+        int32_t code = out->err_code;
+        return dfl_fail(ctx, code, "DFlash target row %d: %s (index %lld)", out->err_row, dflash_status_name(code),
+                        static_cast<long long>(out->err_index));
+    }
+    dflash_sampler_advance(sampler, static_cast<uint64_t>(out->draws_used));  // committed only on success
+    return DFLASH_OK;
+}
+
+}  // extern "C"
