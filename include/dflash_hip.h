@@ -199,6 +199,112 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified_tokens_hos
                              const int32_t *stop_ids_host, int32_t n_stop, dflash_accept_decision *out_host,
                              dflash_stream_t stream);
 
+/* ---- target model, session, packed verify -----------------------------------------------
+ * Weights stay GGUF quant blocks used in place (crates/qwen-llm/src/lib.rs:17-18): a tensor is
+ * a type tag and a device pointer to row-major [n_out][n_in/blk] blocks.  Norm weights are f32.
+ * The block structure is the plain pre-norm decoder of forward.rs:96-163 with per-head q/k
+ * RMSNorm and full-width NeoX RoPE (attn_step, forward.rs:834-932, without the q-gate and the
+ * Gated-DeltaNet layers of the hybrid target, which the synthetic configurations do not have). */
+typedef struct {
+    int32_t type;
+    int32_t pad;
+    const void *data; /* device */
+} dflash_qtensor;
+
+typedef struct {
+    int32_t n_layers, hidden, n_q, n_kv, head_dim, ffn, vocab;
+    int32_t n_expert, n_expert_used, ffn_expert, ffn_shared; /* n_expert == 0: dense FFN */
+    float eps, rope_theta;
+} dflash_model_cfg;
+
+typedef struct {
+    const float *attn_norm, *q_norm, *k_norm, *post_norm; /* device f32 */
+    dflash_qtensor wq, wk, wv, wo, gate, up, down;        /* dense FFN, or the shared expert */
+    dflash_qtensor router;                                /* [hidden -> n_expert] (MoE) */
+    const float *shexp_gate;                              /* [hidden] f32 (MoE) */
+    dflash_qtensor gate_exps, up_exps, down_exps;         /* n_expert stacked matrices (MoE) */
+} dflash_layer;
+
+typedef struct {
+    dflash_model_cfg cfg;
+    const dflash_layer *layers; /* host array of n_layers */
+    dflash_qtensor token_embd, output;
+    const float *output_norm;
+} dflash_model;
+
+/* MetalSession for the target (KV f16, kv_n_pos) plus MetalDFlashVerifyScratch /
+ * MetalDFlashLayerMajorScratch (metal_dflash.rs:5863-5905, 7240-7443).  K is cached as
+ * [layer][capacity][n_kv][head_dim], V transposed as [layer][n_kv][head_dim][capacity]; capacity
+ * is rounded up to a multiple of 32. */
+typedef struct dflash_session dflash_session;
+int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int64_t kv_capacity, int32_t n_taps,
+                              dflash_session **out);
+void dflash_session_destroy(dflash_session *s);
+int64_t dflash_session_kv_n_pos(const dflash_session *s);
+
+/* encode_packed_verify_layer_major_inner(base, target_layer_ids, tokens, start_position, ...,
+ * debug_logits_dst, n_eff_override) (metal_dflash.rs:10696-10719): forward of tokens[n] at
+ * positions start_position .. start_position+n-1, layer-major, K/V appended to the session.
+ * Guards: kv_n_pos == start_position, start+n <= capacity, tokens in the vocabulary.
+ * Outputs (device, may be NULL): argmax[n] i32 and gap[n] f32 (argmax_top2 of each row),
+ * hidden_capture[n][n_taps][hidden] f32 (residual stream after the tapped layers, :10535-10551),
+ * logits[n][vocab] f32.  If argmax_host is non-NULL the call waits and copies the n indices
+ * there (the reference returns Vec<i32>).  1 <= n <= 16. */
+int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,
+                            const int32_t *tokens_host, int32_t n, int64_t start_position,
+                            const int32_t *tap_layers_host, int32_t n_taps, int32_t *argmax, float *gap,
+                            float *hidden_capture, float *logits, int32_t *argmax_host, dflash_stream_t stream);
+
+/* encode_restore_after_partial_accept_inner (metal_dflash.rs:15649-15777): must directly follow
+ * the matching verify; 1 <= n_keep <= n; sets kv_n_pos = start_position + n_keep (stale KV rows
+ * stay in place and are overwritten by the next verify).  n_keep == 0 restores the pre-block
+ * state (encode_restore_to_pre_block, :15789-15905). */
+int32_t dflash_restore(dflash_ctx *ctx, dflash_session *session, int64_t start_position, int32_t n, int32_t n_keep);
+
+/* ---- block drafter ----------------------------------------------------------------------
+ * DFlashConfig / DFlashHead / DFlashLayer (loader.rs:342-399), MetalDFlashSession
+ * (metal_dflash.rs:5053-5191). */
+typedef struct {
+    int32_t n_layers, hidden, n_q, n_kv, head_dim, ffn, block_size, n_taps;
+    int32_t causal;
+    uint32_t swa_window; /* 0 = full */
+    float eps, rope_theta;
+} dflash_draft_cfg;
+
+typedef struct {
+    const float *attn_norm, *q_norm, *k_norm, *post_norm;
+    dflash_qtensor wq, wk, wv, wo, gate, up, down;
+    int32_t is_swa;
+    int32_t pad;
+} dflash_draft_layer;
+
+typedef struct {
+    dflash_draft_cfg cfg;
+    const dflash_draft_layer *layers; /* host array */
+    dflash_qtensor fc;                /* [n_taps*hidden -> hidden] */
+    const float *hidden_norm, *output_norm;
+} dflash_draft_head;
+
+typedef struct dflash_draft_session dflash_draft_session;
+int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg, int64_t ctx_capacity,
+                                    int64_t vocab, dflash_draft_session **out);
+void dflash_draft_session_destroy(dflash_draft_session *s);
+int64_t dflash_draft_session_ctx_len(const dflash_draft_session *s);
+
+/* append_target_ctx_columns_now (metal_dflash.rs:5798-5860): append n_cols captured hidden rows
+ * (hidden_capture layout [col][n_taps][hidden], device f32) with their positions. */
+int32_t dflash_draft_append_ctx(dflash_ctx *ctx, dflash_draft_session *s, const float *hidden_capture, int32_t n_cols,
+                                const int32_t *positions_host, dflash_stream_t stream);
+
+/* MetalDFlashDraftDecoder::draft_block / draft_block_with_logits (metal_dflash.rs:17257-17513;
+ * CPU oracle Forward::dflash_draft, forward.rs:380-662): noise ids [carry, mask x (block-1)] at
+ * positions noise_start_pos.., attention over ctx || noise, shared embedding and lm_head of the
+ * target.  Outputs (device, may be NULL): draft_argmax[block] i32 (slot 0 unused by callers),
+ * draft_logits[block][vocab].  If argmax_host is non-NULL the call waits and copies. */
+int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
+                           dflash_draft_session *s, int32_t carry_token, int32_t mask_token, int64_t noise_start_pos,
+                           int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -351,3 +351,97 @@ def decide_accept_prefix_dense(verified_tokens, target_logits, draft_logits, voc
     rc = lib().orc_decide_accept_prefix_dense(_p(toks), toks.size, _p(t), _p(d), vocab, draft_temperature,
                                               C.byref(sampler), budget, _p(stops), stops.size, C.byref(out))
     return rc, out
+
+
+# ---- synthetic decoder / drafter (plain dictionaries of numpy arrays in, numpy out) ----
+
+class _Keep:
+    """Owns the numpy buffers a ctypes descriptor points into."""
+
+    def __init__(self):
+        self.bufs = []
+
+    def f32(self, a):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        self.bufs.append(a)
+        return a.ctypes.data
+
+    def q(self, pair):
+        if pair is None:
+            return QTensor(0, 0, None)
+        qtype, blocks = pair
+        b = np.ascontiguousarray(blocks, dtype=np.uint8)
+        self.bufs.append(b)
+        return QTensor(int(qtype), 0, b.ctypes.data)
+
+
+def build_model(cfg: dict, weights: dict):
+    """cfg: the dflash_model_cfg fields by name; weights: {'token_embd': (type, blocks), 'output', 'output_norm',
+    'layers': [{'attn_norm', 'q_norm', 'k_norm', 'post_norm', 'wq', ... }]}.  Returns (Model, keepalive)."""
+    keep = _Keep()
+    layers = (Layer * cfg["n_layers"])()
+    for il, Lw in enumerate(weights["layers"]):
+        L = layers[il]
+        for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
+            setattr(L, k, keep.f32(Lw[k]))
+        for k in ("wq", "wk", "wv", "wo", "gate", "up", "down", "router", "gate_exps", "up_exps", "down_exps"):
+            setattr(L, k, keep.q(Lw.get(k)))
+        L.shexp_gate = keep.f32(Lw["shexp_gate"]) if "shexp_gate" in Lw else None
+    m = Model(ModelCfg(**cfg), layers, keep.q(weights["token_embd"]), keep.q(weights["output"]),
+              keep.f32(weights["output_norm"]))
+    keep.bufs.append(layers)
+    return m, keep
+
+
+def build_draft_head(cfg: dict, weights: dict):
+    keep = _Keep()
+    layers = (DraftLayer * cfg["n_layers"])()
+    for il, Lw in enumerate(weights["layers"]):
+        L = layers[il]
+        for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
+            setattr(L, k, keep.f32(Lw[k]))
+        for k in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
+            setattr(L, k, keep.q(Lw[k]))
+        L.is_swa = int(Lw.get("is_swa", 0))
+    h = DraftHead(DraftCfg(**cfg), layers, keep.q(weights["fc"]), keep.f32(weights["hidden_norm"]),
+                  keep.f32(weights["output_norm"]))
+    keep.bufs.append(layers)
+    return h, keep
+
+
+class TargetState:
+    """KV cache of the CPU target: f16 bits [layer][capacity][n_kv*head_dim]."""
+
+    def __init__(self, cfg: dict, capacity: int):
+        kv_dim = cfg["n_kv"] * cfg["head_dim"]
+        self.capacity = capacity
+        self.k = np.zeros((cfg["n_layers"], capacity, kv_dim), np.uint16)
+        self.v = np.zeros((cfg["n_layers"], capacity, kv_dim), np.uint16)
+
+
+def target_verify(model: Model, state: TargetState, tokens, start_pos: int, tap_layers=()):
+    """Token-by-token forward of tokens at start_pos..; returns (logits [n, V], hidden [n, n_taps, H])."""
+    c = model.cfg
+    n = len(tokens)
+    toks = np.asarray(tokens, np.int32)
+    taps = np.asarray(list(tap_layers) or [0], np.int32)
+    logits = np.zeros((n, c.vocab), np.float32)
+    hidden = np.zeros((n, max(len(tap_layers), 1), c.hidden), np.float32)
+    rc = lib().orc_target_verify(C.byref(model), _p(toks), n, start_pos, _p(state.k), _p(state.v), state.capacity,
+                                 _p(logits), _p(taps), len(tap_layers), _p(hidden))
+    if rc:
+        raise RuntimeError(f"orc_target_verify failed: {rc}")
+    return logits, hidden[:, :len(tap_layers)]
+
+
+def dflash_draft(target: Model, head: DraftHead, noise_ids, ctx_stacked, pos_ctx, noise_start_pos: int):
+    """ctx_stacked [ctx_len, n_taps*hidden]; returns logits [block, V]."""
+    ids = np.asarray(noise_ids, np.int32)
+    ctx_stacked = np.ascontiguousarray(ctx_stacked, dtype=np.float32)
+    pos = np.asarray(pos_ctx if len(pos_ctx) else [0], np.int32)
+    logits = np.zeros((head.cfg.block_size, target.cfg.vocab), np.float32)
+    rc = lib().orc_dflash_draft(C.byref(target), C.byref(head), _p(ids), _p(ctx_stacked), len(pos_ctx), _p(pos),
+                                noise_start_pos, _p(logits))
+    if rc:
+        raise RuntimeError(f"orc_dflash_draft failed: {rc}")
+    return logits

@@ -34,3 +34,13 @@ from .binding import (  # noqa: F401
     declared_symbols,
     lib,
 )
+from .model import (  # noqa: F401,E402
+    DraftConfig,
+    DraftHead,
+    DraftSession,
+    ModelConfig,
+    Session,
+    TargetModel,
+    synth_draft_weights,
+    synth_target_weights,
+)

@@ -1,0 +1,517 @@
+// Target packed verify, KV rollback and the block drafter, built from the few-row GEMM, the
+// block-causal attention and small glue kernels.
+//
+// Reference: encode_packed_verify_layer_major_inner_for (metal_dflash.rs:9045-10690),
+// encode_restore_after_partial_accept_inner (:15649-15777), draft_block_inner (:15952-17164),
+// append_target_ctx_columns_now (:5798-5860); CPU forms forward.rs:96-163, 380-662, 725-932,
+// 1256-1371.  Glue: kernels/attn.metal:35-69 (RMSNorm), :137-196 (q/k norm + RoPE),
+// kernels/rope.metal:96-121, kernels/elementwise.metal:89, 193, 674-685, 727-900.
+#include "common.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <vector>
+
+namespace {
+
+__device__ __forceinline__ float h2f(const uint8_t *p) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(p[0] | (p[1] << 8))));
+}
+
+// One element of a quantised row, bit-exact with ggml's dequantize_row_* (see dequant.hip).
+__device__ float dequant_elem(int type, const uint8_t *row, int e) {
+    if (type == DFLASH_TYPE_F32) return reinterpret_cast<const float *>(row)[e];
+    if (type == DFLASH_TYPE_Q8_0) {
+        const uint8_t *blk = row + (e >> 5) * DFL_Q8_0_BYTES;
+        return __fmul_rn(h2f(blk), static_cast<float>(reinterpret_cast<const int8_t *>(blk + 2)[e & 31]));
+    }
+    if (type == DFLASH_TYPE_Q4_K) {
+        const uint8_t *blk = row + (e >> 8) * DFL_Q4_K_BYTES;
+        int i = e & 255, j = i >> 5, l = i & 31;
+        const uint8_t *s = blk + 4;
+        int sc, m;
+        if (j < 4) {
+            sc = s[j] & 63;
+            m = s[j + 4] & 63;
+        } else {
+            sc = (s[j + 4] & 0x0f) | ((s[j - 4] >> 6) << 4);
+            m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+        }
+        uint8_t byte = blk[16 + 32 * (j >> 1) + l];
+        int q = (j & 1) ? (byte >> 4) : (byte & 0x0f);
+        float d1 = __fmul_rn(h2f(blk), static_cast<float>(sc));
+        float m1 = __fmul_rn(h2f(blk + 2), static_cast<float>(m));
+        return __fsub_rn(__fmul_rn(d1, static_cast<float>(q)), m1);
+    }
+    // Q6_K
+    const uint8_t *blk = row + (e >> 8) * DFL_Q6_K_BYTES;
+    int i = e & 255, n = i >> 7, r = i & 127, k = r >> 5, l = r & 31;
+    const uint8_t *ql = blk + 64 * n;
+    const uint8_t *qh = blk + 128 + 32 * n;
+    const int8_t *sc = reinterpret_cast<const int8_t *>(blk + 192 + 8 * n);
+    int lo = (k & 1) ? ql[l + 32] : ql[l];
+    lo = (k & 2) ? (lo >> 4) : (lo & 0x0f);
+    int hi = (qh[l] >> (2 * k)) & 3;
+    float ds = __fmul_rn(h2f(blk + 208), static_cast<float>(sc[(l >> 4) + 2 * k]));
+    return __fmul_rn(ds, static_cast<float>((lo | (hi << 4)) - 32));
+}
+
+// kernel_get_rows_{f32,q4_K,q6_K,q8_0} (elementwise.metal:727-900): out[r][:] = deq(table[ids[r]])
+__global__ void get_rows_kernel(int type, const uint8_t *__restrict__ table, size_t row_bytes,
+                                const int32_t *__restrict__ ids, int hidden, float *__restrict__ out) {
+    const int r = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= hidden) return;
+    out[static_cast<size_t>(r) * hidden + e] = dequant_elem(type, table + static_cast<size_t>(ids[r]) * row_bytes, e);
+}
+
+__device__ float block_sum(float v, float *sh) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = 0.0f;
+    for (int w = 0; w < static_cast<int>(blockDim.x >> 6); w++) r += sh[w];
+    return r;
+}
+
+// kernel_rms_norm_batched_f32 (attn.metal:35-69): y = x * rsqrt(mean(x^2) + eps) * w, one row per workgroup
+__global__ void __launch_bounds__(256) rms_norm_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                       float *__restrict__ y, int n, float eps) {
+    __shared__ float sh[4];
+    const float *xr = x + static_cast<size_t>(blockIdx.x) * n;
+    float *yr = y + static_cast<size_t>(blockIdx.x) * n;
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) s += xr[i] * xr[i];
+    s = block_sum(s, sh);
+    const float scale = 1.0f / sqrtf(s / static_cast<float>(n) + eps);
+    for (int i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * scale * w[i];
+}
+
+// kernel_qk_rms_norm_rope_f32_packed_consecutive (attn.metal:137-196) + the f32 -> f16 KV scatter
+// (elementwise.metal:674-685).  One wave per (row, head): per-head RMSNorm (weight may be null),
+// NeoX RoPE over the full head (pairs (i, i + hd/2), angle = pos / theta^(2i/hd)).
+// Heads [0, n_q) are queries (rewritten in place, f32); heads [n_q, n_q+n_kv) are keys, written
+// as f16 into k_dst[pos][kv head][:] (k_dst == null: rewritten in place as f32 instead).
+__global__ void __launch_bounds__(64)
+    qk_norm_rope_kernel(float *__restrict__ q, float *__restrict__ k, const float *__restrict__ q_w,
+                        const float *__restrict__ k_w, _Float16 *__restrict__ k_dst, const int32_t *__restrict__ pos,
+                        int n_q, int n_kv, int hd, float eps, float theta) {
+    const int row = blockIdx.y, head = blockIdx.x, lane = threadIdx.x;
+    const bool is_q = head < n_q;
+    float *v = is_q ? q + (static_cast<size_t>(row) * n_q + head) * hd
+                    : k + (static_cast<size_t>(row) * n_kv + (head - n_q)) * hd;
+    const float *w = is_q ? q_w : k_w;
+    const int half = hd / 2;
+    float s = 0.0f;
+    for (int i = lane; i < hd; i += 64) s += v[i] * v[i];
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    const float scale = 1.0f / sqrtf(s / static_cast<float>(hd) + eps);
+    const float p = static_cast<float>(pos[row]);
+    for (int i = lane; i < half; i += 64) {
+        float a = v[i] * scale, b = v[i + half] * scale;
+        if (w) {
+            a *= w[i];
+            b *= w[i + half];
+        }
+        const float freq = p / powf(theta, static_cast<float>(2 * i) / static_cast<float>(hd));
+        float sn, cs;
+        sincosf(freq, &sn, &cs);
+        const float ra = a * cs - b * sn, rb = a * sn + b * cs;
+        if (is_q || !k_dst) {
+            v[i] = ra;
+            v[i + half] = rb;
+        } else {
+            _Float16 *dst = k_dst + (static_cast<size_t>(pos[row]) * n_kv + (head - n_q)) * hd;
+            dst[i] = static_cast<_Float16>(ra);
+            dst[i + half] = static_cast<_Float16>(rb);
+        }
+    }
+}
+
+// V rows f32 -> transposed f16 cache [kv head][dim][capacity] at column pos[row]
+__global__ void v_scatter_t_kernel(const float *__restrict__ v, _Float16 *__restrict__ vt, const int32_t *__restrict__ pos,
+                                   int kv_dim, int64_t capacity) {
+    const int row = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= kv_dim) return;
+    vt[static_cast<size_t>(e) * capacity + pos[row]] = static_cast<_Float16>(v[static_cast<size_t>(row) * kv_dim + e]);
+}
+
+// kernel_silu_mul_f32 (elementwise.metal:193): g = silu(g) * u
+__global__ void silu_mul_kernel(float *__restrict__ g, const float *__restrict__ u, size_t n) {
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        float x = g[i];
+        g[i] = x / (1.0f + expf(-x)) * u[i];
+    }
+}
+
+// kernel_add_inplace_f32 (elementwise.metal:89)
+__global__ void add_kernel(float *__restrict__ x, const float *__restrict__ y, size_t n) {
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) x[i] += y[i];
+}
+
+// hidden capture: dst[(row * n_taps + tap) * hidden + :] = x[row][:]
+__global__ void capture_kernel(const float *__restrict__ x, float *__restrict__ dst, int hidden, int n_taps, int tap) {
+    const int row = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < hidden) dst[(static_cast<size_t>(row) * n_taps + tap) * hidden + e] = x[static_cast<size_t>(row) * hidden + e];
+}
+
+// Drafter attention (kernels/dflash_attn.metal:99-307; CPU forward.rs:559-606): query row i of the
+// noise block over ctx || noise keys, f32, mask = (!causal || k_pos <= q_pos) &&
+// (window == 0 || |q_pos - k_pos| < window).  One wave per (q head, row), online softmax.
+__global__ void __launch_bounds__(64)
+    draft_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_ctx, const float *__restrict__ v_ctx,
+                      const float *__restrict__ k_noise, const float *__restrict__ v_noise,
+                      const int32_t *__restrict__ pos_ctx, int ctx_len, int n, int n_q, int n_kv, int hd,
+                      int noise_start, int causal, int window, float *__restrict__ out) {
+    const int head = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
+    const int kvh = head / (n_q / n_kv);
+    const int kv_dim = n_kv * hd;
+    const int per = hd / 64;  // dims per lane (hd in {64,128,256})
+    float qv[4], acc[4] = {0, 0, 0, 0};
+    const float scale = 1.0f / sqrtf(static_cast<float>(hd));
+    for (int i = 0; i < per; i++) qv[i] = q[(static_cast<size_t>(row) * n_q + head) * hd + lane * per + i];
+    const int q_pos = noise_start + row;
+    float m = -INFINITY, l = 0.0f;
+    for (int kk = 0; kk < ctx_len + n; kk++) {
+        const int k_pos = kk < ctx_len ? pos_ctx[kk] : noise_start + (kk - ctx_len);
+        const int dist = q_pos > k_pos ? q_pos - k_pos : k_pos - q_pos;
+        if ((causal && k_pos > q_pos) || (window != 0 && dist >= window)) continue;
+        const float *kr = (kk < ctx_len ? k_ctx + static_cast<size_t>(kk) * kv_dim
+                                        : k_noise + static_cast<size_t>(kk - ctx_len) * kv_dim) + kvh * hd + lane * per;
+        const float *vr = (kk < ctx_len ? v_ctx + static_cast<size_t>(kk) * kv_dim
+                                        : v_noise + static_cast<size_t>(kk - ctx_len) * kv_dim) + kvh * hd + lane * per;
+        float s = 0.0f;
+        for (int i = 0; i < per; i++) s += qv[i] * kr[i];
+        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        s *= scale;
+        const float m_new = fmaxf(m, s);
+        const float alpha = expf(m - m_new), p = expf(s - m_new);
+        l = l * alpha + p;
+        for (int i = 0; i < per; i++) acc[i] = acc[i] * alpha + p * vr[i];
+        m = m_new;
+    }
+    for (int i = 0; i < per; i++) out[(static_cast<size_t>(row) * n_q + head) * hd + lane * per + i] = acc[i] / l;
+}
+
+template <typename T>
+bool dev_alloc(T **p, size_t count) {
+    return hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T) + 256) == hipSuccess;
+}
+
+inline unsigned blocks_for(size_t n, int threads = 256) { return static_cast<unsigned>((n + threads - 1) / threads); }
+
+int32_t gemm(dflash_ctx *ctx, const dflash_qtensor &w, const float *x, float *y, int64_t n_in, int64_t n_out, int n,
+             hipStream_t st) {
+    return dflash_gemm_fewrow(ctx, w.type, w.data, x, DFLASH_TYPE_F32, y, n_in, n_out, n, st);
+}
+
+int32_t embed_rows(dflash_ctx *ctx, const dflash_qtensor &t, const int32_t *ids_dev, int n, int hidden, float *out,
+                   hipStream_t st) {
+    size_t rb = dflash_row_bytes(t.type, hidden);
+    if (rb == 0) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "embedding type %d", t.type);
+    get_rows_kernel<<<dim3(blocks_for(hidden), n), 256, 0, st>>>(t.type, static_cast<const uint8_t *>(t.data), rb, ids_dev,
+                                                               hidden, out);
+    return DFLASH_OK;
+}
+
+}  // namespace
+
+struct dflash_session {
+    dflash_model_cfg cfg;
+    int64_t capacity = 0, kv_n_pos = 0;
+    int n_taps = 0;
+    _Float16 *k_cache = nullptr, *vt_cache = nullptr;
+    float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
+    float *g = nullptr, *u = nullptr, *logits = nullptr, *gap = nullptr;
+    int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
+};
+
+struct dflash_draft_session {
+    dflash_draft_cfg cfg;
+    int64_t capacity = 0, ctx_len = 0, vocab = 0;
+    int64_t ctx_h_ready = 0;  // columns whose fc + hidden_norm are done
+    int64_t kv_ready = 0;     // columns whose per-layer K/V are done
+    float *ctx_raw = nullptr;  // [cap][n_taps*H] captured target hiddens
+    float *ctx_h = nullptr;    // [cap][H]
+    float *k_ctx = nullptr, *v_ctx = nullptr;  // [layer][cap][kv_dim]
+    int32_t *pos_ctx = nullptr;                // [cap]
+    float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
+    float *g = nullptr, *u = nullptr, *logits = nullptr, *tmp = nullptr;
+    int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
+};
+
+extern "C" {
+
+int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int64_t kv_capacity, int32_t n_taps,
+                              dflash_session **out) {
+    if (!ctx || !cfg || !out) return DFLASH_ERR_INVALID_INPUT;
+    *out = nullptr;
+    if (cfg->n_layers < 1 || cfg->hidden < 1 || cfg->n_q < 1 || cfg->n_kv < 1 || cfg->n_q % cfg->n_kv ||
+        (cfg->head_dim != 64 && cfg->head_dim != 128 && cfg->head_dim != 256) || cfg->vocab < 1 || kv_capacity < 1)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "session_create: unsupported model shape");
+    dflash_session *s = new (std::nothrow) dflash_session();
+    if (!s) return DFLASH_ERR_HIP;
+    s->cfg = *cfg;
+    s->capacity = (kv_capacity + 31) / 32 * 32;
+    s->n_taps = n_taps;
+    const size_t kv_dim = static_cast<size_t>(cfg->n_kv) * cfg->head_dim, q_dim = static_cast<size_t>(cfg->n_q) * cfg->head_dim;
+    const size_t f = std::max(std::max(cfg->ffn, cfg->ffn_shared), cfg->ffn_expert);
+    const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
+    bool ok = dev_alloc(&s->k_cache, per_layer * cfg->n_layers) && dev_alloc(&s->vt_cache, per_layer * cfg->n_layers) &&
+              dev_alloc(&s->x, 16 * cfg->hidden) && dev_alloc(&s->cur, 16 * cfg->hidden) && dev_alloc(&s->q, 16 * q_dim) &&
+              dev_alloc(&s->k, 16 * kv_dim) && dev_alloc(&s->v, 16 * kv_dim) && dev_alloc(&s->attn, 16 * q_dim) &&
+              dev_alloc(&s->mix, 16 * cfg->hidden) && dev_alloc(&s->g, 16 * f) && dev_alloc(&s->u, 16 * f) &&
+              dev_alloc(&s->logits, 16 * static_cast<size_t>(cfg->vocab)) && dev_alloc(&s->gap, 16) &&
+              dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) && dev_alloc(&s->argmax, 16);
+    if (ok) ok = hipMemset(s->vt_cache, 0, per_layer * cfg->n_layers * 2) == hipSuccess;
+    if (!ok) {
+        dflash_session_destroy(s);
+        return dfl_fail(ctx, DFLASH_ERR_HIP, "session_create: out of device memory");
+    }
+    *out = s;
+    return DFLASH_OK;
+}
+
+void dflash_session_destroy(dflash_session *s) {
+    if (!s) return;
+    void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
+                    s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    delete s;
+}
+
+int64_t dflash_session_kv_n_pos(const dflash_session *s) { return s ? s->kv_n_pos : -1; }
+
+int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
+                            int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps, int32_t *argmax,
+                            float *gap, float *hidden_capture, float *logits, int32_t *argmax_host,
+                            dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!model || !s || !tokens) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "verify_block: null argument");
+    const dflash_model_cfg &c = model->cfg;
+    // guard walls (metal_dflash.rs:9080-9186)
+    if (n < 1 || n > 16) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "verify_block: n %d outside 1..16", n);
+    if (s->kv_n_pos != start)
+        return dfl_fail(ctx, DFLASH_ERR_STATE, "verify_block: kv_n_pos %lld != start_position %lld",
+                        static_cast<long long>(s->kv_n_pos), static_cast<long long>(start));
+    if (start < 0 || start + n > s->capacity)
+        return dfl_fail(ctx, DFLASH_ERR_STATE, "verify_block: positions %lld..%lld exceed the KV capacity %lld",
+                        static_cast<long long>(start), static_cast<long long>(start + n), static_cast<long long>(s->capacity));
+    for (int i = 0; i < n; i++)
+        if (tokens[i] < 0 || tokens[i] >= c.vocab)
+            return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "verify_block: token %d at index %d outside vocabulary %d",
+                            tokens[i], i, c.vocab);
+    if (n_taps < 0 || n_taps > s->n_taps || (n_taps > 0 && (!tap_layers || !hidden_capture)))
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "verify_block: hidden capture arguments");
+    if (c.n_expert > 0) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "verify_block: the MoE FFN arm is not built yet");
+    if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "verify_block: session/model shape mismatch");
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int H = c.hidden, hd = c.head_dim;
+    const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
+    int32_t pos_host[16];
+    for (int i = 0; i < n; i++) pos_host[i] = static_cast<int32_t>(start + i);
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ids, tokens, n * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos, pos_host, n * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    int32_t rc = embed_rows(ctx, model->token_embd, s->ids, n, H, s->x, st);
+    if (rc) return rc;
+    const float scale = 1.0f / sqrtf(static_cast<float>(hd));
+    const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
+    for (int il = 0; il < c.n_layers; il++) {
+        const dflash_layer &L = model->layers[il];
+        _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
+        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, L.attn_norm, s->cur, H, c.eps);
+        if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, n, st))) return rc;
+        if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, n, st))) return rc;
+        if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, n, st))) return rc;
+        qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, n), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, kc, s->pos, c.n_q, c.n_kv,
+                                                                  hd, c.eps, c.rope_theta);
+        v_scatter_t_kernel<<<dim3(blocks_for(kv_dim), n), 256, 0, st>>>(s->v, vtc, s->pos, static_cast<int>(kv_dim), s->capacity);
+        if ((rc = dflash_attn_verify_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity,
+                                           scale, s->attn, st)))
+            return rc;
+        if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
+        add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
+        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, L.post_norm, s->cur, H, c.eps);
+        if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, n, st))) return rc;
+        if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, n, st))) return rc;
+        silu_mul_kernel<<<blocks_for(static_cast<size_t>(n) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(n) * c.ffn);
+        if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
+        add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
+        for (int t = 0; t < n_taps; t++)
+            if (tap_layers[t] == il)
+                capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
+    }
+    rms_norm_kernel<<<n, 256, 0, st>>>(s->x, model->output_norm, s->cur, H, c.eps);
+    float *lg = logits ? logits : s->logits;
+    if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
+    int32_t *am = argmax ? argmax : s->argmax;
+    if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gap ? gap : s->gap, st))) return rc;
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    s->kv_n_pos = start + n;
+    if (argmax_host) {
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(argmax_host, am, n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+    }
+    return DFLASH_OK;
+}
+
+int32_t dflash_restore(dflash_ctx *ctx, dflash_session *s, int64_t start, int32_t n, int32_t n_keep) {
+    if (!ctx || !s) return DFLASH_ERR_INVALID_INPUT;
+    if (n < 1 || n_keep < 0 || n_keep > n)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "restore: n_keep %d outside 0..%d", n_keep, n);
+    if (s->kv_n_pos != start + n)
+        return dfl_fail(ctx, DFLASH_ERR_STATE, "restore: kv_n_pos %lld != start %lld + n %d (must follow the matching verify)",
+                        static_cast<long long>(s->kv_n_pos), static_cast<long long>(start), n);
+    s->kv_n_pos = start + n_keep;  // stale rows stay in place; the next verify overwrites them
+    return DFLASH_OK;
+}
+
+int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg, int64_t ctx_capacity, int64_t vocab,
+                                    dflash_draft_session **out) {
+    if (!ctx || !cfg || !out) return DFLASH_ERR_INVALID_INPUT;
+    *out = nullptr;
+    if (cfg->n_layers < 1 || cfg->block_size < 1 || cfg->block_size > 16 || cfg->n_q % cfg->n_kv ||
+        (cfg->head_dim != 64 && cfg->head_dim != 128 && cfg->head_dim != 256) || cfg->n_taps < 1 || ctx_capacity < 1)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "draft_session_create: unsupported drafter shape");
+    dflash_draft_session *s = new (std::nothrow) dflash_draft_session();
+    if (!s) return DFLASH_ERR_HIP;
+    s->cfg = *cfg;
+    s->capacity = ctx_capacity;
+    s->vocab = vocab;
+    const size_t H = cfg->hidden, kv_dim = static_cast<size_t>(cfg->n_kv) * cfg->head_dim,
+                 q_dim = static_cast<size_t>(cfg->n_q) * cfg->head_dim, cap = ctx_capacity;
+    bool ok = dev_alloc(&s->ctx_raw, cap * cfg->n_taps * H) && dev_alloc(&s->ctx_h, cap * H) &&
+              dev_alloc(&s->k_ctx, cap * kv_dim * cfg->n_layers) && dev_alloc(&s->v_ctx, cap * kv_dim * cfg->n_layers) &&
+              dev_alloc(&s->pos_ctx, cap) && dev_alloc(&s->x, 16 * H) && dev_alloc(&s->cur, 16 * H) &&
+              dev_alloc(&s->q, 16 * q_dim) && dev_alloc(&s->k, 16 * kv_dim) && dev_alloc(&s->v, 16 * kv_dim) &&
+              dev_alloc(&s->attn, 16 * q_dim) && dev_alloc(&s->mix, 16 * H) && dev_alloc(&s->g, 16 * static_cast<size_t>(cfg->ffn)) &&
+              dev_alloc(&s->u, 16 * static_cast<size_t>(cfg->ffn)) && dev_alloc(&s->logits, 16 * static_cast<size_t>(vocab)) &&
+              dev_alloc(&s->tmp, 16 * std::max(H, kv_dim)) && dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) &&
+              dev_alloc(&s->argmax, 16);
+    if (!ok) {
+        dflash_draft_session_destroy(s);
+        return dfl_fail(ctx, DFLASH_ERR_HIP, "draft_session_create: out of device memory");
+    }
+    *out = s;
+    return DFLASH_OK;
+}
+
+void dflash_draft_session_destroy(dflash_draft_session *s) {
+    if (!s) return;
+    void *ptrs[] = {s->ctx_raw, s->ctx_h, s->k_ctx, s->v_ctx, s->pos_ctx, s->x, s->cur, s->q, s->k, s->v,
+                    s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    delete s;
+}
+
+int64_t dflash_draft_session_ctx_len(const dflash_draft_session *s) { return s ? s->ctx_len : -1; }
+
+int32_t dflash_draft_append_ctx(dflash_ctx *ctx, dflash_draft_session *s, const float *hidden_capture, int32_t n_cols,
+                                const int32_t *positions, dflash_stream_t stream) {
+    if (!ctx || !s) return DFLASH_ERR_INVALID_INPUT;
+    if (n_cols < 0 || (n_cols > 0 && (!hidden_capture || !positions)))
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "append_ctx: null argument");
+    if (s->ctx_len + n_cols > s->capacity)
+        return dfl_fail(ctx, DFLASH_ERR_STATE, "append_ctx: %lld + %d columns exceed the context capacity %lld",
+                        static_cast<long long>(s->ctx_len), n_cols, static_cast<long long>(s->capacity));
+    if (n_cols == 0) return DFLASH_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t feat = static_cast<size_t>(s->cfg.n_taps) * s->cfg.hidden;
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ctx_raw + s->ctx_len * feat, hidden_capture, n_cols * feat * sizeof(float),
+                                      hipMemcpyDeviceToDevice, st));
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos_ctx + s->ctx_len, positions, n_cols * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    s->ctx_len += n_cols;
+    return DFLASH_OK;
+}
+
+int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
+                           dflash_draft_session *s, int32_t carry, int32_t mask_token, int64_t noise_start,
+                           int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!target || !head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_block: null argument");
+    const dflash_draft_cfg &c = head->cfg;
+    if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_block: session/head shape mismatch");
+    if (c.hidden != target->cfg.hidden) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "draft_block: drafter and target hidden sizes differ");
+    const int V = target->cfg.vocab;
+    if (V != s->vocab) return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_block: vocabulary mismatch");
+    if (carry < 0 || carry >= V || mask_token < 0 || mask_token >= V)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "draft_block: carry %d / mask %d outside vocabulary %d", carry, mask_token, V);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int N = c.block_size, H = c.hidden, hd = c.head_dim;
+    const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
+    const size_t feat = static_cast<size_t>(c.n_taps) * H;
+    int32_t rc;
+
+    // phase 1: fc + hidden_norm on the NEW context columns only (metal_dflash.rs:16045-16143)
+    for (int64_t c0 = s->ctx_h_ready; c0 < s->ctx_len; c0 += 16) {
+        const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
+        if ((rc = gemm(ctx, head->fc, s->ctx_raw + c0 * feat, s->tmp, feat, H, m, st))) return rc;
+        rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps);
+    }
+    // phase 2: noise embedding
+    int32_t ids_host[16], pos_host[16];
+    for (int i = 0; i < N; i++) {
+        ids_host[i] = i == 0 ? carry : mask_token;
+        pos_host[i] = static_cast<int32_t>(noise_start + i);
+    }
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ids, ids_host, N * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos, pos_host, N * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    if ((rc = embed_rows(ctx, target->token_embd, s->ids, N, H, s->x, st))) return rc;
+
+    for (int il = 0; il < c.n_layers; il++) {
+        const dflash_draft_layer &L = head->layers[il];
+        float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
+        float *vc = s->v_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
+        // context K/V for the delta only, normed and rotated at the columns' own positions
+        for (int64_t c0 = s->kv_ready; c0 < s->ctx_len; c0 += 16) {
+            const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
+            if ((rc = gemm(ctx, L.wk, s->ctx_h + c0 * H, kc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
+            if ((rc = gemm(ctx, L.wv, s->ctx_h + c0 * H, vc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
+            qk_norm_rope_kernel<<<dim3(c.n_kv, m), 64, 0, st>>>(nullptr, kc + c0 * kv_dim, nullptr, L.k_norm, nullptr,
+                                                               s->pos_ctx + c0, 0, c.n_kv, hd, c.eps, c.rope_theta);
+        }
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, L.attn_norm, s->cur, H, c.eps);
+        if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, N, st))) return rc;
+        if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, N, st))) return rc;
+        if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, N, st))) return rc;
+        qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, nullptr, s->pos, c.n_q,
+                                                                  c.n_kv, hd, c.eps, c.rope_theta);
+        draft_attn_kernel<<<dim3(c.n_q, N), 64, 0, st>>>(s->q, kc, vc, s->k, s->v, s->pos_ctx, static_cast<int>(s->ctx_len), N,
+                                                        c.n_q, c.n_kv, hd, static_cast<int>(noise_start), c.causal,
+                                                        L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
+        if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st))) return rc;
+        add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, L.post_norm, s->cur, H, c.eps);
+        if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, N, st))) return rc;
+        if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, N, st))) return rc;
+        silu_mul_kernel<<<blocks_for(static_cast<size_t>(N) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(N) * c.ffn);
+        if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st))) return rc;
+        add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
+    }
+    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, head->output_norm, s->cur, H, c.eps);
+    float *lg = draft_logits ? draft_logits : s->logits;
+    if ((rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st))) return rc;
+    int32_t *am = draft_argmax ? draft_argmax : s->argmax;
+    if ((rc = dflash_argmax_greedy(ctx, lg, N, V, V, am, st))) return rc;
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    // watermarks advance only once everything was enqueued without error (metal_dflash.rs:17143-17150)
+    s->ctx_h_ready = s->ctx_len;
+    s->kv_ready = s->ctx_len;
+    if (argmax_host) {
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(argmax_host, am, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+    }
+    return DFLASH_OK;
+}
+
+}  // extern "C"

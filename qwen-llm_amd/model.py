@@ -1,0 +1,358 @@
+"""Host mirror of the target session, packed verify, rollback and the block drafter.
+
+Names follow the reference: ``MetalSession`` / ``encode_packed_verify_layer_major``
+(metal_dflash.rs:10696-10719), ``encode_restore_after_partial_accept`` (:15649-15777),
+``MetalDFlashSession`` / ``append_target_ctx_columns_now`` (:5053-5191, 5798-5860) and
+``MetalDFlashDraftDecoder::draft_block`` (:17257-17513).  Weights are plain dictionaries of
+numpy arrays (GGUF quant blocks as uint8 rows), uploaded once and used in place.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import asdict, dataclass
+
+import numpy as np
+
+from . import synth
+from .binding import Context, DFlashError, _stream_ptr, _torch, lib
+
+
+@dataclass
+class ModelConfig:
+    n_layers: int
+    hidden: int
+    n_q: int
+    n_kv: int
+    head_dim: int
+    ffn: int
+    vocab: int
+    n_expert: int = 0
+    n_expert_used: int = 0
+    ffn_expert: int = 0
+    ffn_shared: int = 0
+    eps: float = 1e-6
+    rope_theta: float = 1e6
+
+    def as_dict(self):
+        return asdict(self)
+
+
+@dataclass
+class DraftConfig:
+    n_layers: int
+    hidden: int
+    n_q: int
+    n_kv: int
+    head_dim: int
+    ffn: int
+    block_size: int = 16
+    n_taps: int = 5
+    causal: int = 0
+    swa_window: int = 0
+    eps: float = 1e-6
+    rope_theta: float = 1e6
+
+    def as_dict(self):
+        return asdict(self)
+
+
+class QTensorC(C.Structure):
+    _fields_ = [("type", C.c_int32), ("pad", C.c_int32), ("data", C.c_void_p)]
+
+
+class ModelCfgC(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "n_q", "n_kv", "head_dim", "ffn", "vocab", "n_expert",
+                                          "n_expert_used", "ffn_expert", "ffn_shared")] + \
+               [("eps", C.c_float), ("rope_theta", C.c_float)]
+
+
+class LayerC(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("post_norm", C.c_void_p),
+                ("wq", QTensorC), ("wk", QTensorC), ("wv", QTensorC), ("wo", QTensorC), ("gate", QTensorC),
+                ("up", QTensorC), ("down", QTensorC), ("router", QTensorC), ("shexp_gate", C.c_void_p),
+                ("gate_exps", QTensorC), ("up_exps", QTensorC), ("down_exps", QTensorC)]
+
+
+class ModelC(C.Structure):
+    _fields_ = [("cfg", ModelCfgC), ("layers", C.POINTER(LayerC)), ("token_embd", QTensorC), ("output", QTensorC),
+                ("output_norm", C.c_void_p)]
+
+
+class DraftCfgC(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "n_q", "n_kv", "head_dim", "ffn", "block_size", "n_taps",
+                                          "causal")] + \
+               [("swa_window", C.c_uint32), ("eps", C.c_float), ("rope_theta", C.c_float)]
+
+
+class DraftLayerC(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("post_norm", C.c_void_p),
+                ("wq", QTensorC), ("wk", QTensorC), ("wv", QTensorC), ("wo", QTensorC), ("gate", QTensorC),
+                ("up", QTensorC), ("down", QTensorC), ("is_swa", C.c_int32), ("pad", C.c_int32)]
+
+
+class DraftHeadC(C.Structure):
+    _fields_ = [("cfg", DraftCfgC), ("layers", C.POINTER(DraftLayerC)), ("fc", QTensorC), ("hidden_norm", C.c_void_p),
+                ("output_norm", C.c_void_p)]
+
+
+_declared = False
+
+
+def _lib():
+    global _declared
+    L = lib()
+    if not _declared:
+        vp, i32, i64, f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float
+        L.dflash_session_create.restype = i32
+        L.dflash_session_create.argtypes = [vp, C.POINTER(ModelCfgC), i64, i32, C.POINTER(vp)]
+        L.dflash_session_destroy.restype = None
+        L.dflash_session_destroy.argtypes = [vp]
+        L.dflash_session_kv_n_pos.restype = i64
+        L.dflash_session_kv_n_pos.argtypes = [vp]
+        L.dflash_verify_block.restype = i32
+        L.dflash_verify_block.argtypes = [vp, C.POINTER(ModelC), vp, C.POINTER(i32), i32, i64, C.POINTER(i32), i32, vp,
+                                          vp, vp, vp, C.POINTER(i32), vp]
+        L.dflash_restore.restype = i32
+        L.dflash_restore.argtypes = [vp, vp, i64, i32, i32]
+        L.dflash_draft_session_create.restype = i32
+        L.dflash_draft_session_create.argtypes = [vp, C.POINTER(DraftCfgC), i64, i64, C.POINTER(vp)]
+        L.dflash_draft_session_destroy.restype = None
+        L.dflash_draft_session_destroy.argtypes = [vp]
+        L.dflash_draft_session_ctx_len.restype = i64
+        L.dflash_draft_session_ctx_len.argtypes = [vp]
+        L.dflash_draft_append_ctx.restype = i32
+        L.dflash_draft_append_ctx.argtypes = [vp, vp, vp, i32, C.POINTER(i32), vp]
+        L.dflash_draft_block.restype = i32
+        L.dflash_draft_block.argtypes = [vp, C.POINTER(ModelC), C.POINTER(DraftHeadC), vp, i32, i32, i64, vp, vp,
+                                         C.POINTER(i32), vp]
+        _declared = True
+    return L
+
+
+# ---- synthetic weights (numpy; the same dictionaries feed the CPU checker in the tests) ----
+
+_ATTN_MATS = ("wq", "wk", "wv", "wo")
+
+
+def _norm_w(rng, n):
+    return (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+
+
+def _mat(qtype, n_out, n_in, seed):
+    return (qtype, synth.random_weight(qtype, n_out, n_in, seed, std=1.0 / np.sqrt(n_in)))
+
+
+def synth_target_weights(cfg: ModelConfig, seed: int, wtype: int = synth.Q4_K, embd_type: int = synth.Q6_K):
+    """Random-init weights of the synthetic decoder: Q4_K projections, Q6_K embedding / lm_head."""
+    rng = np.random.default_rng(seed)
+    q_dim, kv_dim = cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
+    s = seed * 1000003
+    w = {"token_embd": (embd_type, synth.random_weight(embd_type, cfg.vocab, cfg.hidden, s + 1, std=1.0)),
+         "output": _mat(embd_type, cfg.vocab, cfg.hidden, s + 2), "output_norm": _norm_w(rng, cfg.hidden), "layers": []}
+    for il in range(cfg.n_layers):
+        b = s + 100 * (il + 1)
+        ffn = cfg.ffn_shared if cfg.n_expert else cfg.ffn
+        L = {"attn_norm": _norm_w(rng, cfg.hidden), "q_norm": _norm_w(rng, cfg.head_dim),
+             "k_norm": _norm_w(rng, cfg.head_dim), "post_norm": _norm_w(rng, cfg.hidden),
+             "wq": _mat(wtype, q_dim, cfg.hidden, b + 1), "wk": _mat(wtype, kv_dim, cfg.hidden, b + 2),
+             "wv": _mat(wtype, kv_dim, cfg.hidden, b + 3), "wo": _mat(wtype, cfg.hidden, q_dim, b + 4),
+             "gate": _mat(wtype, ffn, cfg.hidden, b + 5), "up": _mat(wtype, ffn, cfg.hidden, b + 6),
+             "down": _mat(wtype, cfg.hidden, ffn, b + 7)}
+        if cfg.n_expert:
+            fe = cfg.ffn_expert
+            L["router"] = _mat(synth.Q8_0, cfg.n_expert, cfg.hidden, b + 8)
+            L["shexp_gate"] = (rng.standard_normal(cfg.hidden) / np.sqrt(cfg.hidden)).astype(np.float32)
+            L["gate_exps"] = _mat(wtype, cfg.n_expert * fe, cfg.hidden, b + 9)
+            L["up_exps"] = _mat(wtype, cfg.n_expert * fe, cfg.hidden, b + 10)
+            L["down_exps"] = _mat(wtype, cfg.n_expert * cfg.hidden, fe, b + 11)
+        w["layers"].append(L)
+    return w
+
+
+def synth_draft_weights(cfg: DraftConfig, seed: int, wtype: int = synth.Q4_K, swa_layers=()):
+    rng = np.random.default_rng(seed + 7919)
+    q_dim, kv_dim = cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
+    s = seed * 1000003 + 500000
+    w = {"fc": _mat(wtype, cfg.hidden, cfg.n_taps * cfg.hidden, s + 1), "hidden_norm": _norm_w(rng, cfg.hidden),
+         "output_norm": _norm_w(rng, cfg.hidden), "layers": []}
+    for il in range(cfg.n_layers):
+        b = s + 100 * (il + 1)
+        w["layers"].append({
+            "attn_norm": _norm_w(rng, cfg.hidden), "q_norm": _norm_w(rng, cfg.head_dim),
+            "k_norm": _norm_w(rng, cfg.head_dim), "post_norm": _norm_w(rng, cfg.hidden),
+            "wq": _mat(wtype, q_dim, cfg.hidden, b + 1), "wk": _mat(wtype, kv_dim, cfg.hidden, b + 2),
+            "wv": _mat(wtype, kv_dim, cfg.hidden, b + 3), "wo": _mat(wtype, cfg.hidden, q_dim, b + 4),
+            "gate": _mat(wtype, cfg.ffn, cfg.hidden, b + 5), "up": _mat(wtype, cfg.ffn, cfg.hidden, b + 6),
+            "down": _mat(wtype, cfg.hidden, cfg.ffn, b + 7), "is_swa": int(il in swa_layers)})
+    return w
+
+
+# ---- device-resident weights ----
+
+class _Uploader:
+    def __init__(self, device):
+        self.torch = _torch()
+        self.device = device
+        self.keep = []
+
+    def f32(self, a):
+        t = self.torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device)
+        self.keep.append(t)
+        return t.data_ptr()
+
+    def q(self, pair):
+        if pair is None:
+            return QTensorC(0, 0, None)
+        qtype, blocks = pair
+        t = self.torch.from_numpy(np.ascontiguousarray(blocks)).to(self.device)
+        self.keep.append(t)
+        return QTensorC(int(qtype), 0, t.data_ptr())
+
+
+class TargetModel:
+    """Device copy of a weight dictionary plus the ``dflash_model`` descriptor."""
+
+    def __init__(self, ctx: Context, cfg: ModelConfig, weights: dict):
+        self.ctx, self.cfg = ctx, cfg
+        up = _Uploader(f"cuda:{ctx.device}")
+        self._up = up
+        self._layers = (LayerC * cfg.n_layers)()
+        for il, Lw in enumerate(weights["layers"]):
+            L = self._layers[il]
+            for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
+                setattr(L, k, up.f32(Lw[k]))
+            for k in ("wq", "wk", "wv", "wo", "gate", "up", "down", "router", "gate_exps", "up_exps", "down_exps"):
+                setattr(L, k, up.q(Lw.get(k)))
+            L.shexp_gate = up.f32(Lw["shexp_gate"]) if "shexp_gate" in Lw else None
+        self.c = ModelC(ModelCfgC(**cfg.as_dict()), self._layers, up.q(weights["token_embd"]), up.q(weights["output"]),
+                        up.f32(weights["output_norm"]))
+
+    def weight_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._up.keep)
+
+
+class VerifyOutput:
+    def __init__(self, argmax, gap, hidden_capture, logits, argmax_host):
+        self.argmax, self.gap, self.hidden_capture, self.logits, self.argmax_host = argmax, gap, hidden_capture, logits, argmax_host
+
+
+class Session:
+    """Target session: f16 KV cache and ``kv_n_pos``."""
+
+    def __init__(self, ctx: Context, model: TargetModel, kv_capacity: int, tap_layers=()):
+        self.ctx, self.model = ctx, model
+        self.tap_layers = list(tap_layers)
+        self._L = _lib()
+        h = C.c_void_p()
+        cfgc = ModelCfgC(**model.cfg.as_dict())
+        ctx._check(self._L.dflash_session_create(ctx._h, C.byref(cfgc), kv_capacity, len(self.tap_layers), C.byref(h)))
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._L.dflash_session_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def kv_n_pos(self) -> int:
+        return self._L.dflash_session_kv_n_pos(self._h)
+
+    def encode_packed_verify_layer_major(self, tokens, start_position: int, want_logits=False, want_hidden=True,
+                                         sync=True) -> VerifyOutput:
+        """Forward of ``tokens`` at positions start_position.. ; appends K/V; returns argmax, top-2
+        gap, the tapped hidden rows [n][n_taps][hidden] and (optionally) the logits."""
+        torch = _torch()
+        cfg = self.model.cfg
+        n = len(tokens)
+        dev = f"cuda:{self.ctx.device}"
+        toks = (C.c_int32 * max(n, 1))(*[int(t) for t in tokens])
+        n_taps = len(self.tap_layers) if want_hidden else 0
+        taps = (C.c_int32 * max(n_taps, 1))(*self.tap_layers[:n_taps])
+        argmax = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
+        gap = torch.empty(max(n, 1), dtype=torch.float32, device=dev)
+        hidden = torch.empty((n, n_taps, cfg.hidden), dtype=torch.float32, device=dev) if n_taps else None
+        logits = torch.empty((n, cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
+        host = (C.c_int32 * max(n, 1))() if sync else None
+        self.ctx._check(self._L.dflash_verify_block(
+            self.ctx._h, C.byref(self.model.c), self._h, toks, n, start_position, taps, n_taps, argmax.data_ptr(),
+            gap.data_ptr(), hidden.data_ptr() if hidden is not None else None,
+            logits.data_ptr() if logits is not None else None, host, _stream_ptr()))
+        return VerifyOutput(argmax[:n], gap[:n], hidden, logits, list(host[:n]) if sync else None)
+
+    def encode_restore_after_partial_accept(self, start_position: int, n: int, n_keep: int):
+        self.ctx._check(self._L.dflash_restore(self.ctx._h, self._h, start_position, n, n_keep))
+
+
+class DraftHead:
+    def __init__(self, ctx: Context, cfg: DraftConfig, weights: dict):
+        self.ctx, self.cfg = ctx, cfg
+        up = _Uploader(f"cuda:{ctx.device}")
+        self._up = up
+        self._layers = (DraftLayerC * cfg.n_layers)()
+        for il, Lw in enumerate(weights["layers"]):
+            L = self._layers[il]
+            for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
+                setattr(L, k, up.f32(Lw[k]))
+            for k in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
+                setattr(L, k, up.q(Lw[k]))
+            L.is_swa = int(Lw.get("is_swa", 0))
+        self.c = DraftHeadC(DraftCfgC(**cfg.as_dict()), self._layers, up.q(weights["fc"]), up.f32(weights["hidden_norm"]),
+                            up.f32(weights["output_norm"]))
+
+    def weight_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._up.keep)
+
+
+class DraftSession:
+    """Drafter session: accumulated target context columns and their per-layer K/V."""
+
+    def __init__(self, ctx: Context, head: DraftHead, target: TargetModel, ctx_capacity: int):
+        self.ctx, self.head, self.target = ctx, head, target
+        self._L = _lib()
+        h = C.c_void_p()
+        cfgc = DraftCfgC(**head.cfg.as_dict())
+        ctx._check(self._L.dflash_draft_session_create(ctx._h, C.byref(cfgc), ctx_capacity, target.cfg.vocab, C.byref(h)))
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._L.dflash_draft_session_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def ctx_len(self) -> int:
+        return self._L.dflash_draft_session_ctx_len(self._h)
+
+    def append_target_ctx_columns(self, hidden_capture, positions):
+        """hidden_capture: device f32 [n_cols][n_taps][hidden]; positions: their token positions."""
+        n = len(positions)
+        if n and tuple(hidden_capture.shape) != (n, self.head.cfg.n_taps, self.head.cfg.hidden):
+            raise DFlashError(1, f"hidden_capture shape {tuple(hidden_capture.shape)}")
+        pos = (C.c_int32 * max(n, 1))(*[int(p) for p in positions])
+        hc = hidden_capture.contiguous() if n else None
+        self.ctx._check(self._L.dflash_draft_append_ctx(self.ctx._h, self._h, hc.data_ptr() if n else None, n, pos,
+                                                        _stream_ptr()))
+
+    def draft_block(self, carry_token: int, mask_token: int, noise_start_pos: int, want_logits=False, sync=True):
+        torch = _torch()
+        dev = f"cuda:{self.ctx.device}"
+        N = self.head.cfg.block_size
+        argmax = torch.empty(N, dtype=torch.int32, device=dev)
+        logits = torch.empty((N, self.target.cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
+        host = (C.c_int32 * N)() if sync else None
+        self.ctx._check(self._L.dflash_draft_block(
+            self.ctx._h, C.byref(self.target.c), C.byref(self.head.c), self._h, carry_token, mask_token, noise_start_pos,
+            argmax.data_ptr(), logits.data_ptr() if logits is not None else None, host, _stream_ptr()))
+        return argmax, logits, (list(host) if sync else None)

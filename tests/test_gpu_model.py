@@ -1,0 +1,170 @@
+"""GPU parity: packed 16-row verify, KV rollback and the block drafter against the CPU oracle
+(token-by-token attn_step / ffn of forward.rs:96-163, 834-932 and Forward::dflash_draft,
+forward.rs:380-662) on the reference's own synthetic shape (metal_dflash.rs tests: 4 layers,
+hidden 1024, 16 q / 8 kv heads of 128, FFN 3072, vocabulary 32000, Q4_K weights).
+
+Tolerance: each GEMM and each attention call is held to 1e-2 by its own test; here the error of
+4 layers x 8 such calls compounds, so the stack is held to a relative l2 error of 5e-3 and a
+worst element (over ~10^6 values, relative to max(|ref|, rms)) of 3e-2; argmax identical wherever
+the oracle's own top-2 gap exceeds the logit error bound."""
+import numpy as np
+import pytest
+
+import qwen_llm_amd as dfl
+
+pytestmark = pytest.mark.gpu
+
+C1 = dfl.ModelConfig(n_layers=4, hidden=1024, n_q=16, n_kv=8, head_dim=128, ffn=3072, vocab=32000)
+TAPS = [0, 1, 2, 3, 3]
+D1 = dfl.DraftConfig(n_layers=2, hidden=1024, n_q=16, n_kv=8, head_dim=128, ffn=3072, block_size=16, n_taps=5)
+PREFIX = 96
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = dfl.Context(0, workspace_bytes=256 << 20)
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def target(ctx, oracle):
+    w = dfl.synth_target_weights(C1, seed=11)
+    return dfl.TargetModel(ctx, C1, w), oracle.build_model(C1.as_dict(), w)
+
+
+def close(got, want, label, tol=3e-2, l2_tol=5e-3):
+    got, want = np.asarray(got, np.float32), np.asarray(want, np.float32)
+    assert got.shape == want.shape, f"{label}: shape {got.shape} vs {want.shape}"
+    assert np.all(np.isfinite(got)), f"{label}: non-finite"
+    rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    err = np.max(np.abs(got - want) / np.maximum(np.abs(want), rms))
+    l2 = np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want.astype(np.float64))
+    print(f"{label}: max err {err:.3e} l2 {l2:.3e}")
+    assert err <= tol, f"{label}: max err {err:.3e} (rms {rms:.3e})"
+    assert l2 <= l2_tol, f"{label}: rel l2 {l2:.3e}"
+    return err
+
+
+def argmax_agrees(argmax, logits_ref, label):
+    top = np.sort(logits_ref, axis=1)
+    gap = top[:, -1] - top[:, -2]
+    rms = np.sqrt(np.mean(logits_ref.astype(np.float64) ** 2))
+    decided = gap > 2e-2 * rms
+    assert decided.sum() >= len(gap) // 2, f"{label}: synthetic logits too flat to test the argmax"
+    want = logits_ref.argmax(axis=1)
+    assert np.array_equal(np.asarray(argmax)[decided], want[decided]), f"{label}: argmax differs on a decided row"
+
+
+def prefill(sess, ostate, omodel, oracle, tokens):
+    """Fill both caches with the prompt in blocks of 16 through the same verify path."""
+    hid_g, hid_o = [], []
+    for s in range(0, len(tokens), 16):
+        blk = tokens[s:s + 16]
+        out = sess.encode_packed_verify_layer_major(blk, s)
+        hid_g.append(out.hidden_capture.cpu().numpy())
+        hid_o.append(oracle.target_verify(omodel, ostate, blk, s, TAPS)[1])
+    return np.concatenate(hid_g), np.concatenate(hid_o)
+
+
+def test_verify_block_matches_oracle_and_restore(ctx, oracle, target):
+    model, (omodel, _keep) = target
+    rng = np.random.default_rng(5)
+    cap = PREFIX + 64
+    sess = dfl.Session(ctx, model, cap, TAPS)
+    ostate = oracle.TargetState(C1.as_dict(), cap)
+    prompt = rng.integers(0, C1.vocab, PREFIX).tolist()
+    hg, ho = prefill(sess, ostate, omodel, oracle, prompt)
+    close(hg, ho, "prefill hidden")
+    assert sess.kv_n_pos == PREFIX
+
+    pos = PREFIX
+    for n, n_keep in ((16, 7), (16, 0), (1, 1), (5, 5), (16, 16), (3, 1)):
+        blk = rng.integers(0, C1.vocab, n).tolist()
+        out = sess.encode_packed_verify_layer_major(blk, pos, want_logits=True)
+        lo, hid_o = oracle.target_verify(omodel, ostate, blk, pos, TAPS)
+        close(out.logits.cpu().numpy(), lo, f"logits n={n} pos={pos}")
+        close(out.hidden_capture.cpu().numpy(), hid_o, f"hidden n={n} pos={pos}")
+        lg = out.logits.cpu().numpy()
+        assert np.array_equal(out.argmax.cpu().numpy(), lg.argmax(axis=1)), "argmax is not the argmax of the logits"
+        assert out.argmax_host == out.argmax.cpu().tolist()
+        top = np.sort(lg, axis=1)
+        np.testing.assert_array_equal(out.gap.cpu().numpy(), top[:, -1] - top[:, -2])
+        if n >= 5:
+            argmax_agrees(out.argmax.cpu().numpy(), lo, f"n={n}")
+        assert sess.kv_n_pos == pos + n
+        sess.encode_restore_after_partial_accept(pos, n, n_keep)
+        assert sess.kv_n_pos == pos + n_keep
+        pos += n_keep
+    sess.close()
+
+
+def test_verify_guard_walls(ctx, target):
+    model, _ = target
+    sess = dfl.Session(ctx, model, 64, TAPS)
+    with pytest.raises(dfl.DFlashError) as e:
+        sess.encode_packed_verify_layer_major([1, 2, 3], 5)
+    assert e.value.status == 10 and "kv_n_pos" in str(e.value)
+    with pytest.raises(dfl.DFlashError) as e:
+        sess.encode_packed_verify_layer_major([1, C1.vocab], 0)
+    assert e.value.status == 8
+    with pytest.raises(dfl.DFlashError) as e:
+        sess.encode_packed_verify_layer_major(list(range(17)), 0)
+    assert e.value.status == 1
+    with pytest.raises(dfl.DFlashError):
+        sess.encode_packed_verify_layer_major([], 0)
+    assert sess.kv_n_pos == 0
+    sess.encode_packed_verify_layer_major(list(range(16)), 0)
+    with pytest.raises(dfl.DFlashError) as e:
+        sess.encode_restore_after_partial_accept(0, 16, 17)
+    assert e.value.status == 1
+    with pytest.raises(dfl.DFlashError) as e:
+        sess.encode_restore_after_partial_accept(3, 16, 4)
+    assert e.value.status == 10
+    for s in range(16, 64, 16):
+        sess.encode_packed_verify_layer_major(list(range(16)), s)
+    with pytest.raises(dfl.DFlashError) as e:
+        sess.encode_packed_verify_layer_major([1], 64)
+    assert e.value.status == 10 and "capacity" in str(e.value)
+    sess.close()
+
+
+@pytest.mark.parametrize("causal,swa", [(0, 0), (1, 0), (0, 24), (1, 8)])
+def test_draft_block_matches_oracle(ctx, oracle, target, causal, swa):
+    model, (omodel, _keep) = target
+    dcfg = dfl.DraftConfig(**{**D1.as_dict(), "causal": causal, "swa_window": swa})
+    dw = dfl.synth_draft_weights(dcfg, seed=3, swa_layers=(1,) if swa else ())
+    head = dfl.DraftHead(ctx, dcfg, dw)
+    ohead, _k2 = oracle.build_draft_head(dcfg.as_dict(), dw)
+    rng = np.random.default_rng(17 + causal + swa)
+    cap = 128
+    sess = dfl.Session(ctx, model, cap, TAPS)
+    ostate = oracle.TargetState(C1.as_dict(), cap)
+    dsess = dfl.DraftSession(ctx, head, model, cap)
+    mask_token = C1.vocab - 1
+
+    # incremental context: a 40-token prompt, then two accepted stretches of 5 and 16 columns
+    all_hidden_o = []
+    pos = 0
+    for n_new in (40, 5, 16):
+        toks = rng.integers(0, C1.vocab, n_new).tolist()
+        for s in range(0, n_new, 16):
+            blk = toks[s:s + 16]
+            out = sess.encode_packed_verify_layer_major(blk, pos)
+            dsess.append_target_ctx_columns(out.hidden_capture, list(range(pos, pos + len(blk))))
+            all_hidden_o.append(oracle.target_verify(omodel, ostate, blk, pos, TAPS)[1])
+            pos += len(blk)
+        assert dsess.ctx_len == pos
+        carry = int(rng.integers(0, C1.vocab))
+        argmax, logits, host = dsess.draft_block(carry, mask_token, pos, want_logits=True)
+        ctx_o = np.concatenate(all_hidden_o).reshape(pos, -1)
+        want = oracle.dflash_draft(omodel, ohead, [carry] + [mask_token] * 15, ctx_o, list(range(pos)), pos)
+        close(logits.cpu().numpy(), want, f"draft logits ctx={pos} causal={causal} swa={swa}")
+        lg = logits.cpu().numpy()
+        assert host == lg.argmax(axis=1).tolist() == argmax.cpu().tolist()
+        argmax_agrees(host, want, f"draft ctx={pos}")
+    with pytest.raises(dfl.DFlashError) as e:
+        dsess.draft_block(C1.vocab, mask_token, pos)
+    assert e.value.status == 8
+    dsess.close()
+    sess.close()
