@@ -78,3 +78,19 @@ static inline bool dfl_ranges_overlap(const void *a, size_t na, const void *b, s
 }
 
 enum { DFL_QK_K = 256, DFL_Q4_K_BYTES = 144, DFL_Q6_K_BYTES = 210, DFL_Q8_0_BYTES = 34, DFL_QK8_0 = 32 };
+
+// Device scratch of the mixture-of-experts FFN (owned by the target session).
+struct dfl_moe_scratch {
+    float *probs = nullptr;   // [16][n_expert] router logits
+    int32_t *sel_e = nullptr; // [16][n_used]
+    float *sel_w = nullptr;   // [16][n_used]
+    float *sg = nullptr;      // [16] shared-expert gate
+    float *act = nullptr;     // [16*n_used][ffn_expert]
+    float *eo = nullptr;      // [16*n_used][hidden]
+    float *shared = nullptr;  // [16][hidden]
+    float *g = nullptr, *u = nullptr;  // [16][ffn_shared]
+};
+
+// x_resid[n][hidden] += moe_ffn(cur[n][hidden]) for one layer; enqueue only.
+int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, const float *cur, int n,
+                    const dfl_moe_scratch &scratch, float *x_resid, hipStream_t stream);

@@ -7,6 +7,7 @@
 // 1256-1371.  Glue: kernels/attn.metal:35-69 (RMSNorm), :137-196 (q/k norm + RoPE),
 // kernels/rope.metal:96-121, kernels/elementwise.metal:89, 193, 674-685, 727-900.
 #include "common.h"
+#include "device_quant.h"
 
 #include <algorithm>
 #include <cmath>
@@ -16,55 +17,13 @@
 
 namespace {
 
-__device__ __forceinline__ float h2f(const uint8_t *p) {
-    return __half2float(__ushort_as_half(static_cast<unsigned short>(p[0] | (p[1] << 8))));
-}
-
-// One element of a quantised row, bit-exact with ggml's dequantize_row_* (see dequant.hip).
-__device__ float dequant_elem(int type, const uint8_t *row, int e) {
-    if (type == DFLASH_TYPE_F32) return reinterpret_cast<const float *>(row)[e];
-    if (type == DFLASH_TYPE_Q8_0) {
-        const uint8_t *blk = row + (e >> 5) * DFL_Q8_0_BYTES;
-        return __fmul_rn(h2f(blk), static_cast<float>(reinterpret_cast<const int8_t *>(blk + 2)[e & 31]));
-    }
-    if (type == DFLASH_TYPE_Q4_K) {
-        const uint8_t *blk = row + (e >> 8) * DFL_Q4_K_BYTES;
-        int i = e & 255, j = i >> 5, l = i & 31;
-        const uint8_t *s = blk + 4;
-        int sc, m;
-        if (j < 4) {
-            sc = s[j] & 63;
-            m = s[j + 4] & 63;
-        } else {
-            sc = (s[j + 4] & 0x0f) | ((s[j - 4] >> 6) << 4);
-            m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
-        }
-        uint8_t byte = blk[16 + 32 * (j >> 1) + l];
-        int q = (j & 1) ? (byte >> 4) : (byte & 0x0f);
-        float d1 = __fmul_rn(h2f(blk), static_cast<float>(sc));
-        float m1 = __fmul_rn(h2f(blk + 2), static_cast<float>(m));
-        return __fsub_rn(__fmul_rn(d1, static_cast<float>(q)), m1);
-    }
-    // Q6_K
-    const uint8_t *blk = row + (e >> 8) * DFL_Q6_K_BYTES;
-    int i = e & 255, n = i >> 7, r = i & 127, k = r >> 5, l = r & 31;
-    const uint8_t *ql = blk + 64 * n;
-    const uint8_t *qh = blk + 128 + 32 * n;
-    const int8_t *sc = reinterpret_cast<const int8_t *>(blk + 192 + 8 * n);
-    int lo = (k & 1) ? ql[l + 32] : ql[l];
-    lo = (k & 2) ? (lo >> 4) : (lo & 0x0f);
-    int hi = (qh[l] >> (2 * k)) & 3;
-    float ds = __fmul_rn(h2f(blk + 208), static_cast<float>(sc[(l >> 4) + 2 * k]));
-    return __fmul_rn(ds, static_cast<float>((lo | (hi << 4)) - 32));
-}
-
 // kernel_get_rows_{f32,q4_K,q6_K,q8_0} (elementwise.metal:727-900): out[r][:] = deq(table[ids[r]])
 __global__ void get_rows_kernel(int type, const uint8_t *__restrict__ table, size_t row_bytes,
                                 const int32_t *__restrict__ ids, int hidden, float *__restrict__ out) {
     const int r = blockIdx.y;
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= hidden) return;
-    out[static_cast<size_t>(r) * hidden + e] = dequant_elem(type, table + static_cast<size_t>(ids[r]) * row_bytes, e);
+    out[static_cast<size_t>(r) * hidden + e] = dfl_dequant_elem(type, table + static_cast<size_t>(ids[r]) * row_bytes, e);
 }
 
 __device__ float block_sum(float v, float *sh) {
@@ -231,6 +190,7 @@ struct dflash_session {
     float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
     float *g = nullptr, *u = nullptr, *logits = nullptr, *gap = nullptr;
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
+    dfl_moe_scratch moe;
 };
 
 struct dflash_draft_session {
@@ -270,6 +230,15 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
               dev_alloc(&s->mix, 16 * cfg->hidden) && dev_alloc(&s->g, 16 * f) && dev_alloc(&s->u, 16 * f) &&
               dev_alloc(&s->logits, 16 * static_cast<size_t>(cfg->vocab)) && dev_alloc(&s->gap, 16) &&
               dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) && dev_alloc(&s->argmax, 16);
+    if (ok && cfg->n_expert > 0) {
+        const size_t used = std::min(cfg->n_expert_used, cfg->n_expert);
+        ok = dev_alloc(&s->moe.probs, 16 * static_cast<size_t>(cfg->n_expert)) && dev_alloc(&s->moe.sel_e, 16 * used) &&
+             dev_alloc(&s->moe.sel_w, 16 * used) && dev_alloc(&s->moe.sg, 16) &&
+             dev_alloc(&s->moe.act, 16 * used * cfg->ffn_expert) && dev_alloc(&s->moe.eo, 16 * used * cfg->hidden) &&
+             dev_alloc(&s->moe.shared, 16 * cfg->hidden);
+        s->moe.g = s->g;
+        s->moe.u = s->u;
+    }
     if (ok) ok = hipMemset(s->vt_cache, 0, per_layer * cfg->n_layers * 2) == hipSuccess;
     if (!ok) {
         dflash_session_destroy(s);
@@ -282,7 +251,8 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
 void dflash_session_destroy(dflash_session *s) {
     if (!s) return;
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
-                    s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax};
+                    s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax,
+                    s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;
@@ -311,7 +281,6 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
                             tokens[i], i, c.vocab);
     if (n_taps < 0 || n_taps > s->n_taps || (n_taps > 0 && (!tap_layers || !hidden_capture)))
         return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "verify_block: hidden capture arguments");
-    if (c.n_expert > 0) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "verify_block: the MoE FFN arm is not built yet");
     if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "verify_block: session/model shape mismatch");
 
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -341,11 +310,15 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
         add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
         rms_norm_kernel<<<n, 256, 0, st>>>(s->x, L.post_norm, s->cur, H, c.eps);
-        if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, n, st))) return rc;
-        if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, n, st))) return rc;
-        silu_mul_kernel<<<blocks_for(static_cast<size_t>(n) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(n) * c.ffn);
-        if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
-        add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
+        if (c.n_expert > 0) {
+            if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, st))) return rc;
+        } else {
+            if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, n, st))) return rc;
+            if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, n, st))) return rc;
+            silu_mul_kernel<<<blocks_for(static_cast<size_t>(n) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(n) * c.ffn);
+            if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
+            add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
+        }
         for (int t = 0; t < n_taps; t++)
             if (tap_layers[t] == il)
                 capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);

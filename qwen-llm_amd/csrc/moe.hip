@@ -1,0 +1,231 @@
+// Mixture-of-experts FFN of the packed verify: route on the device, then read every selected
+// expert's weights ONCE for all block rows that picked it (the reference runs the experts per
+// row after a packed route, metal_dflash.rs:10184-10403; CPU form ffn_moe, forward.rs:749-824).
+//
+//   probs   = softmax(router . x)                       over all experts
+//   picks   = top-k by probability, ties to the lower expert id
+//   weights = probs[pick] / max(sum(probs[picks]), 2^-14)
+//   out     = sum_k weights[k] * down_e(silu(gate_e x) * up_e x)  +  sigmoid(x . w_shexp) * shared(x)
+//
+// Work items are "slots": slot = row * n_used + k.  The expert kernels run one workgroup column
+// per expert; a workgroup first collects the slots that picked its expert and leaves at once
+// if there are none, so HBM traffic is the distinct experts of the block, not rows x k.
+#include "common.h"
+#include "device_quant.h"
+
+namespace {
+
+constexpr int kMaxSlots = 16;  // a row picks an expert at most once, and a block has at most 16 rows
+
+// One wave per block row: softmax, top-k, renormalised weights, shared-expert gate.
+__global__ void __launch_bounds__(64)
+    moe_route_kernel(const float *__restrict__ logits, const float *__restrict__ x, const float *__restrict__ shexp_gate,
+                     int n_expert, int n_used, int hidden, int32_t *__restrict__ sel_e, float *__restrict__ sel_w,
+                     float *__restrict__ sg) {
+    extern __shared__ float probs[];  // [n_expert]
+    __shared__ float pick_w[64];
+    const int row = blockIdx.x, lane = threadIdx.x;
+    const float *lr = logits + static_cast<size_t>(row) * n_expert;
+    float mx = -INFINITY;
+    for (int e = lane; e < n_expert; e += 64) mx = fmaxf(mx, lr[e]);
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.0f;
+    for (int e = lane; e < n_expert; e += 64) {
+        const float p = expf(lr[e] - mx);
+        probs[e] = p;
+        sum += p;
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float inv = 1.0f / sum;
+    __syncthreads();
+    for (int e = lane; e < n_expert; e += 64) probs[e] *= inv;
+    __syncthreads();
+    float wsum = 0.0f;
+    for (int k = 0; k < n_used; k++) {
+        float best = -1.0f;
+        int best_e = 0x7fffffff;
+        for (int e = lane; e < n_expert; e += 64) {
+            const float p = probs[e];
+            if (p > best) {  // ascending e per lane: strict > keeps the lower id
+                best = p;
+                best_e = e;
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, 64);
+            const int oe = __shfl_xor(best_e, off, 64);
+            if (ob > best || (ob == best && oe < best_e)) {
+                best = ob;
+                best_e = oe;
+            }
+        }
+        if (lane == 0) {
+            sel_e[row * n_used + k] = best_e;
+            pick_w[k] = best;
+            probs[best_e] = -2.0f;  // taken
+        }
+        wsum += best;
+        __syncthreads();
+    }
+    wsum = fmaxf(wsum, 6.103515625e-05f);  // 2^-14
+    if (lane < n_used) sel_w[row * n_used + lane] = pick_w[lane] / wsum;
+    float dot = 0.0f;
+    for (int i = lane; i < hidden; i += 64) dot += x[static_cast<size_t>(row) * hidden + i] * shexp_gate[i];
+    for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+    if (lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
+}
+
+// Collects the slots whose pick is `expert`; returns the count (uniform over the workgroup).
+__device__ int collect_slots(const int32_t *__restrict__ sel_e, int n_slots, int expert, int *list, int *count) {
+    if (threadIdx.x == 0) *count = 0;
+    __syncthreads();
+    for (int s = threadIdx.x; s < n_slots; s += blockDim.x)
+        if (sel_e[s] == expert) list[atomicAdd(count, 1)] = s;
+    __syncthreads();
+    return *count;
+}
+
+// y[slot][o] = W_expert[o][:] . xin[src(slot)][:]  for the slots of this expert.
+// GATE_UP: two stacked matrices, y = silu(gate) * up, xin row = slot / n_used (the block row).
+// Otherwise: one matrix, xin row = slot.
+// A row of n_in/32 sub-blocks is spread over LPR lanes (32 or 64); a wave does 64/LPR rows at once.
+template <bool GATE_UP, int LPR>
+__global__ void __launch_bounds__(256)
+    moe_expert_kernel(int type, const uint8_t *__restrict__ w0, const uint8_t *__restrict__ w1, size_t row_bytes,
+                      const float *__restrict__ xin, const int32_t *__restrict__ sel_e, int n_slots, int n_used, int n_in,
+                      int n_out, float *__restrict__ y) {
+    __shared__ int list[kMaxSlots];
+    __shared__ int count;
+    const int expert = blockIdx.y;
+    const int n = collect_slots(sel_e, n_slots, expert, list, &count);
+    if (n == 0) return;
+    constexpr int kRowsPerWave = 64 / LPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub_lane = lane % LPR, sub_row = lane / LPR;
+    const int n_sub = n_in / 32;
+    const int rows_per_wg = 4 * kRowsPerWave * 4;  // 4 waves x rows at once x 4 passes
+    const int o0 = blockIdx.x * rows_per_wg;
+    const size_t expert_off = static_cast<size_t>(expert) * n_out * row_bytes;
+    for (int pass = 0; pass < 4; pass++) {
+        const int o = o0 + (pass * 4 + wave) * kRowsPerWave + sub_row;
+        const bool live = o < n_out;
+        const uint8_t *r0 = w0 + expert_off + static_cast<size_t>(live ? o : 0) * row_bytes;
+        const uint8_t *r1 = GATE_UP ? w1 + expert_off + static_cast<size_t>(live ? o : 0) * row_bytes : nullptr;
+        for (int s0 = 0; s0 < n; s0 += 4) {  // up to 4 slots share one dequantisation
+            float acc0[4] = {0, 0, 0, 0}, acc1[4] = {0, 0, 0, 0};
+            for (int sb = sub_lane; sb < n_sub; sb += LPR) {
+                float wa[32], wb[32];
+                dfl_dequant_sub32(type, r0, sb, wa);
+                if (GATE_UP) dfl_dequant_sub32(type, r1, sb, wb);
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    if (s0 + t >= n) break;
+                    const int slot = list[s0 + t];
+                    const float4 *xr = reinterpret_cast<const float4 *>(
+                        xin + static_cast<size_t>(GATE_UP ? slot / n_used : slot) * n_in + 32 * sb);
+#pragma unroll
+                    for (int v = 0; v < 8; v++) {
+                        const float4 xv = xr[v];
+                        acc0[t] += wa[4 * v] * xv.x + wa[4 * v + 1] * xv.y + wa[4 * v + 2] * xv.z + wa[4 * v + 3] * xv.w;
+                        if (GATE_UP)
+                            acc1[t] += wb[4 * v] * xv.x + wb[4 * v + 1] * xv.y + wb[4 * v + 2] * xv.z + wb[4 * v + 3] * xv.w;
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                float a = acc0[t], b = acc1[t];
+                for (int off = LPR / 2; off > 0; off >>= 1) {
+                    a += __shfl_xor(a, off, 64);
+                    if (GATE_UP) b += __shfl_xor(b, off, 64);
+                }
+                if (sub_lane == 0 && live && s0 + t < n) {
+                    const float r = GATE_UP ? a / (1.0f + expf(-a)) * b : a;
+                    y[static_cast<size_t>(list[s0 + t]) * n_out + o] = r;
+                }
+            }
+        }
+    }
+}
+
+// x[row] += sum_k w[row][k] * eo[row*n_used + k]  +  sg[row] * shared[row]
+__global__ void moe_combine_kernel(const float *__restrict__ eo, const float *__restrict__ sel_w, const float *__restrict__ sg,
+                                   const float *__restrict__ shared, int n_used, int hidden, float *__restrict__ x) {
+    const int row = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= hidden) return;
+    float out = 0.0f;
+    for (int k = 0; k < n_used; k++)
+        out += sel_w[row * n_used + k] * eo[(static_cast<size_t>(row) * n_used + k) * hidden + i];
+    out += sg[row] * shared[static_cast<size_t>(row) * hidden + i];
+    x[static_cast<size_t>(row) * hidden + i] += out;
+}
+
+__global__ void silu_mul_rows_kernel(float *__restrict__ g, const float *__restrict__ u, size_t n) {
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float v = g[i];
+        g[i] = v / (1.0f + expf(-v)) * u[i];
+    }
+}
+
+}  // namespace
+
+int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, const float *cur, int n,
+                    const dfl_moe_scratch &s, float *x_resid, hipStream_t st) {
+    const int E = c.n_expert, used = c.n_expert_used < E ? c.n_expert_used : E;
+    const int H = c.hidden, fe = c.ffn_expert, fs = c.ffn_shared;
+    const int n_slots = n * used;
+    if (used < 1 || used > 64 || E > 8192 || fe % 32 || H % 32)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: n_expert %d / n_expert_used %d / ffn_expert %d unsupported", E, used, fe);
+    const int et = L.gate_exps.type;
+    if (et != L.up_exps.type || (et != DFLASH_TYPE_Q4_K && et != DFLASH_TYPE_Q6_K && et != DFLASH_TYPE_Q8_0))
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: expert weight type %d", et);
+    const int dt = L.down_exps.type;
+    if (dt != DFLASH_TYPE_Q4_K && dt != DFLASH_TYPE_Q6_K && dt != DFLASH_TYPE_Q8_0)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: expert weight type %d", dt);
+    const size_t rb_in = dflash_row_bytes(et, H), rb_dn = dflash_row_bytes(dt, fe);
+    if (rb_in == 0 || rb_dn == 0) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "moe: row sizes do not fit the block size");
+
+    int32_t rc = dflash_gemm_fewrow(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
+    if (rc) return rc;
+    moe_route_kernel<<<n, 64, E * sizeof(float), st>>>(s.probs, cur, L.shexp_gate, E, used, H, s.sel_e, s.sel_w, s.sg);
+
+    {
+        dim3 grid(1, E);  // x: 16 * (64 / LPR) output rows per workgroup
+        const int n_sub = H / 32;
+        if (n_sub <= 32) {
+            grid.x = (fe + 31) / 32;
+            moe_expert_kernel<true, 32><<<grid, 256, 0, st>>>(et, static_cast<const uint8_t *>(L.gate_exps.data),
+                                                             static_cast<const uint8_t *>(L.up_exps.data), rb_in, cur, s.sel_e,
+                                                             n_slots, used, H, fe, s.act);
+        } else {
+            grid.x = (fe + 15) / 16;
+            moe_expert_kernel<true, 64><<<grid, 256, 0, st>>>(et, static_cast<const uint8_t *>(L.gate_exps.data),
+                                                             static_cast<const uint8_t *>(L.up_exps.data), rb_in, cur, s.sel_e,
+                                                             n_slots, used, H, fe, s.act);
+        }
+    }
+    {
+        dim3 grid(1, E);
+        const int n_sub = fe / 32;
+        if (n_sub <= 32) {
+            grid.x = (H + 31) / 32;
+            moe_expert_kernel<false, 32><<<grid, 256, 0, st>>>(dt, static_cast<const uint8_t *>(L.down_exps.data), nullptr, rb_dn,
+                                                              s.act, s.sel_e, n_slots, used, fe, H, s.eo);
+        } else {
+            grid.x = (H + 15) / 16;
+            moe_expert_kernel<false, 64><<<grid, 256, 0, st>>>(dt, static_cast<const uint8_t *>(L.down_exps.data), nullptr, rb_dn,
+                                                              s.act, s.sel_e, n_slots, used, fe, H, s.eo);
+        }
+    }
+    // shared expert: plain dense SwiGLU through the few-row GEMM
+    if ((rc = dflash_gemm_fewrow(ctx, L.gate.type, L.gate.data, cur, DFLASH_TYPE_F32, s.g, H, fs, n, st))) return rc;
+    if ((rc = dflash_gemm_fewrow(ctx, L.up.type, L.up.data, cur, DFLASH_TYPE_F32, s.u, H, fs, n, st))) return rc;
+    const size_t nf = static_cast<size_t>(n) * fs;
+    silu_mul_rows_kernel<<<static_cast<unsigned>((nf + 255) / 256), 256, 0, st>>>(s.g, s.u, nf);
+    if ((rc = dflash_gemm_fewrow(ctx, L.down.type, L.down.data, s.g, DFLASH_TYPE_F32, s.shared, fs, H, n, st))) return rc;
+    moe_combine_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.sel_w, s.sg, s.shared, used, H, x_resid);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}

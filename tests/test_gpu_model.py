@@ -168,3 +168,33 @@ def test_draft_block_matches_oracle(ctx, oracle, target, causal, swa):
     assert e.value.status == 8
     dsess.close()
     sess.close()
+
+
+MOE_CASES = {
+    # hidden 512: 16 sub-blocks per row (half-wave rows); hidden 2048 / F_exp 768: the end-to-end shape's widths
+    "small": dfl.ModelConfig(n_layers=2, hidden=512, n_q=8, n_kv=2, head_dim=64, ffn=0, vocab=4096, n_expert=16,
+                             n_expert_used=4, ffn_expert=256, ffn_shared=512),
+    "wide": dfl.ModelConfig(n_layers=2, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=8192, n_expert=32,
+                            n_expert_used=8, ffn_expert=768, ffn_shared=768),
+}
+
+
+@pytest.mark.parametrize("name", list(MOE_CASES))
+def test_moe_verify_matches_oracle(ctx, oracle, name):
+    cfg = MOE_CASES[name]
+    w = dfl.synth_target_weights(cfg, seed=23)
+    model = dfl.TargetModel(ctx, cfg, w)
+    omodel, _keep = oracle.build_model(cfg.as_dict(), w)
+    taps = [0, 1]
+    sess = dfl.Session(ctx, model, 64, taps)
+    ostate = oracle.TargetState(cfg.as_dict(), 64)
+    rng = np.random.default_rng(29)
+    pos = 0
+    for n in (16, 16, 1, 7):
+        blk = rng.integers(0, cfg.vocab, n).tolist()
+        out = sess.encode_packed_verify_layer_major(blk, pos, want_logits=True)
+        lo, hid = oracle.target_verify(omodel, ostate, blk, pos, taps)
+        close(out.hidden_capture.cpu().numpy(), hid, f"moe {name} hidden n={n}")
+        close(out.logits.cpu().numpy(), lo, f"moe {name} logits n={n}")
+        pos += n
+    sess.close()
