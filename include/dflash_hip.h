@@ -305,6 +305,49 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                            dflash_draft_session *s, int32_t carry_token, int32_t mask_token, int64_t noise_start_pos,
                            int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream);
 
+/* ---- one speculative transition -----------------------------------------------------------
+ * The body of the generation loop of crates/qwen-cli/src/qwen/dflash.rs:700-1241: draft a block
+ * from `carry` at `position`, verify [carry, drafts...] in one packed pass, accept a prefix,
+ * append the committed hidden columns to the drafter context, roll the target KV back.
+ *
+ * dflash_accept_greedy: the argmax accept loop (qwen/dflash.rs:838-858) in the decision format of
+ * decide_dflash_accept_prefix: accept while verify_input[i+1] == verify_argmax[i]; stop on a stop
+ * id or when `remaining_output_budget` accepted tokens are reached; otherwise the carry is
+ * verify_argmax[n_accepted] (a correction, or the bonus when every draft was accepted). */
+int32_t dflash_accept_greedy(const int32_t *verify_input_host, const int32_t *verify_argmax_host, int32_t n_tokens,
+                             int64_t remaining_output_budget, const int32_t *stop_ids_host, int32_t n_stop,
+                             dflash_accept_decision *out_host);
+
+typedef struct {
+    int32_t mask_token;
+    int32_t sampled_mode;           /* 0: greedy argmax accept; 1: sampler-coupled accept of the drafter's argmax
+                                       (couple_deterministic_proposal), logits stay on the device */
+    float fallback_margin;          /* greedy only: replay when a committed row's packed top-2 gap is below this
+                                       (DFLASH_VERIFY_FALLBACK_MARGIN_DEFAULT = 0.1); <= 0 disables */
+    int32_t fallback_partial;       /* 1: keep rows before the first flagged row (QWEN_DFLASH_VERIFY_FALLBACK_PARTIAL) */
+    float fallback_partial_min_gap; /* a partially replayed row below this gap escalates to a whole-block replay (0.15) */
+} dflash_step_cfg;
+
+typedef struct {
+    dflash_accept_decision decision; /* accepted drafts, next carry, stop reason, n_keep = retain_input_count */
+    int32_t n_block;
+    int32_t draft_tokens[16];        /* slot 0 = carry */
+    int32_t verify_argmax[16];       /* packed argmax; rows replayed by the fallback hold the replayed argmax */
+    float verify_gap[16];            /* packed top-2 gaps */
+    int32_t fallback_ran, fallback_rows_replayed, fallback_escalations, fallback_rows_kept;
+    double draft_ms, verify_ms, accept_ms, fallback_ms, append_ms, restore_ms; /* host wall clock per phase */
+} dflash_step_result;
+
+/* draft_override_host (may be NULL): block_size-1 token ids replacing the drafter's proposals for slots
+ * 1.. (entries < 0 keep the drafter's token): the loop's prefix-replay drafts (qwen/dflash.rs:700-712).
+ * sampler is required when sampled_mode != 0.  Blocking. */
+int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
+                         dflash_session *session, dflash_draft_session *draft_session,
+                         const int32_t *tap_layers_host, int32_t n_taps, int32_t carry_token, int64_t position,
+                         const dflash_step_cfg *cfg, dflash_sampler *sampler, int64_t remaining_output_budget,
+                         const int32_t *stop_ids_host, int32_t n_stop, const int32_t *draft_override_host,
+                         dflash_step_result *out_host, dflash_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -40,7 +40,9 @@ from .model import (  # noqa: F401,E402
     DraftSession,
     ModelConfig,
     Session,
+    SpeculativeDecoder,
     TargetModel,
+    accept_greedy,
     synth_draft_weights,
     synth_target_weights,
 )

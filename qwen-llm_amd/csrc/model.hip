@@ -10,6 +10,7 @@
 #include "device_quant.h"
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstring>
 #include <new>
@@ -189,6 +190,7 @@ struct dflash_session {
     _Float16 *k_cache = nullptr, *vt_cache = nullptr;
     float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
     float *g = nullptr, *u = nullptr, *logits = nullptr, *gap = nullptr;
+    float *hidden = nullptr;  // [16][n_taps][hidden] capture slots of the speculative step
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
     dfl_moe_scratch moe;
 };
@@ -229,7 +231,8 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
               dev_alloc(&s->k, 16 * kv_dim) && dev_alloc(&s->v, 16 * kv_dim) && dev_alloc(&s->attn, 16 * q_dim) &&
               dev_alloc(&s->mix, 16 * cfg->hidden) && dev_alloc(&s->g, 16 * f) && dev_alloc(&s->u, 16 * f) &&
               dev_alloc(&s->logits, 16 * static_cast<size_t>(cfg->vocab)) && dev_alloc(&s->gap, 16) &&
-              dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) && dev_alloc(&s->argmax, 16);
+              dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) && dev_alloc(&s->argmax, 16) &&
+              dev_alloc(&s->hidden, 16 * static_cast<size_t>(std::max(n_taps, 1)) * cfg->hidden);
     if (ok && cfg->n_expert > 0) {
         const size_t used = std::min(cfg->n_expert_used, cfg->n_expert);
         ok = dev_alloc(&s->moe.probs, 16 * static_cast<size_t>(cfg->n_expert)) && dev_alloc(&s->moe.sel_e, 16 * used) &&
@@ -251,7 +254,7 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
 void dflash_session_destroy(dflash_session *s) {
     if (!s) return;
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
-                    s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax,
+                    s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax, s->hidden,
                     s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -483,6 +486,229 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
     if (argmax_host) {
         DFL_HIP_CHECK(ctx, hipMemcpyAsync(argmax_host, am, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
         DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+    }
+    return DFLASH_OK;
+}
+
+int32_t dflash_accept_greedy(const int32_t *verify_input, const int32_t *verify_argmax, int32_t n, int64_t budget,
+                             const int32_t *stop_ids, int32_t n_stop, dflash_accept_decision *out) {
+    if (!verify_input || !verify_argmax || !out || n < 1 || n > 16 || budget < 0 || (n_stop > 0 && !stop_ids))
+        return DFLASH_ERR_INVALID_INPUT;
+    auto is_stop = [&](int32_t t) {
+        for (int i = 0; i < n_stop; i++)
+            if (stop_ids[i] == t) return true;
+        return false;
+    };
+    memset(out, 0, sizeof(*out));
+    out->err_row = -1;
+    out->err_index = -1;
+    if (is_stop(verify_input[0]) || budget == 0) {  // terminal anchor (accept.rs:131-145)
+        out->stop_reason = is_stop(verify_input[0]) ? DFLASH_STOP_EOS : DFLASH_STOP_TOKEN_LIMIT;
+        return DFLASH_OK;
+    }
+    int a = 0;
+    for (;;) {
+        if (a == n - 1) {
+            out->carry_kind = DFLASH_CARRY_BONUS;
+            out->carry_token = verify_argmax[a];
+            break;
+        }
+        const int32_t draft = verify_input[a + 1];
+        if (draft != verify_argmax[a]) {
+            out->carry_kind = DFLASH_CARRY_CORRECTION;
+            out->carry_token = verify_argmax[a];
+            break;
+        }
+        out->accepted_drafts[a++] = draft;
+        if (is_stop(draft)) {
+            out->stop_reason = DFLASH_STOP_EOS;
+            break;
+        }
+        if (a == budget) {
+            out->stop_reason = DFLASH_STOP_TOKEN_LIMIT;
+            break;
+        }
+    }
+    out->n_accepted = a;
+    out->retain_input_count = 1 + a - (out->stop_reason != DFLASH_STOP_NONE ? 1 : 0);
+    return DFLASH_OK;
+}
+
+namespace {
+
+double ms_since(std::chrono::steady_clock::time_point t0) {
+    return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+}
+
+// Margin-guarded exact fallback of the greedy accept (qwen/dflash.rs:859-1057): when a committed
+// row's packed top-2 gap is under the margin, roll the KV back and replay token by token.
+int32_t margin_fallback(dflash_ctx *ctx, const dflash_model *target, dflash_session *sess, const int32_t *taps, int n_taps,
+                        const int32_t *verify_input, int n_eff, int64_t pos, const dflash_step_cfg *cfg, int64_t budget,
+                        const int32_t *stop_ids, int n_stop, dflash_step_result *res, hipStream_t st) {
+    dflash_accept_decision &d = res->decision;
+    if (d.retain_input_count == 0 && d.n_accepted == 0 && d.carry_kind == DFLASH_CARRY_NONE) return DFLASH_OK;  // anchor stop
+    int n_accepted = d.n_accepted;
+    int first_flagged = -1;
+    for (int i = 0; i <= n_accepted && i < n_eff; i++) {
+        const float g = res->verify_gap[i];
+        if (!(std::isfinite(g) && g >= cfg->fallback_margin)) {
+            first_flagged = i;
+            break;
+        }
+    }
+    if (first_flagged < 0) return DFLASH_OK;
+    auto is_stop = [&](int32_t t) {
+        for (int i = 0; i < n_stop; i++)
+            if (stop_ids[i] == t) return true;
+        return false;
+    };
+    res->fallback_ran = 1;
+    int replay_start = cfg->fallback_partial ? first_flagged : 0;
+    int32_t rc = dflash_restore(ctx, sess, pos, n_eff, replay_start);
+    if (rc) return rc;
+    const int packed_terminal = d.stop_reason;
+    const size_t slot = static_cast<size_t>(std::max(n_taps, 1)) * target->cfg.hidden;
+    int32_t targets[17];
+    int accepted = 0, terminal = DFLASH_STOP_NONE, n_targets = 0;
+    for (;;) {
+        const bool partial = replay_start > 0;
+        accepted = replay_start;
+        terminal = replay_start == n_accepted ? packed_terminal : DFLASH_STOP_NONE;
+        n_targets = replay_start;
+        for (int i = 0; i < replay_start; i++) targets[i] = res->verify_argmax[i];
+        int escalate = 0, rows = 0;
+        auto replay_row = [&](int row, int32_t token, int32_t *arg, float *gap) -> int32_t {
+            int32_t r = dflash_verify_block(ctx, target, sess, &token, 1, pos + row, taps, n_taps, nullptr, nullptr,
+                                            n_taps ? sess->hidden + row * slot : nullptr, nullptr, arg, st);
+            if (r) return r;
+            if (hipMemcpy(gap, sess->gap, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess)
+                return dfl_fail(ctx, DFLASH_ERR_HIP, "fallback: gap read-back failed");
+            rows++;
+            return DFLASH_OK;
+        };
+        auto near_tie = [&](float g) { return !(std::isfinite(g) && g >= cfg->fallback_partial_min_gap); };
+        if (terminal == DFLASH_STOP_NONE) {
+            int32_t t;
+            float g;
+            if ((rc = replay_row(replay_start, verify_input[replay_start], &t, &g))) return rc;
+            if (partial && near_tie(g)) {
+                escalate = 1;
+            } else {
+                targets[n_targets++] = t;
+                for (int i = replay_start; i + 1 < n_eff; i++) {
+                    const int32_t draft = verify_input[i + 1];
+                    if (draft != targets[i]) break;
+                    accepted++;
+                    if (is_stop(draft)) {
+                        terminal = DFLASH_STOP_EOS;
+                        break;
+                    }
+                    if (accepted == budget) {
+                        terminal = DFLASH_STOP_TOKEN_LIMIT;
+                        break;
+                    }
+                    if ((rc = replay_row(i + 1, draft, &t, &g))) return rc;
+                    if (partial && near_tie(g)) {
+                        escalate = 1;
+                        break;
+                    }
+                    targets[n_targets++] = t;
+                }
+            }
+        }
+        res->fallback_rows_replayed += rows;
+        if (!escalate) break;
+        res->fallback_escalations++;
+        const int64_t done = dflash_session_kv_n_pos(sess) - pos;
+        if (done > 0 && (rc = dflash_restore(ctx, sess, pos, static_cast<int32_t>(done), 0))) return rc;
+        replay_start = 0;
+    }
+    res->fallback_rows_kept = replay_start;
+    for (int i = 0; i < n_targets; i++) res->verify_argmax[i] = targets[i];
+    memset(&d, 0, sizeof(d));
+    d.err_row = -1;
+    d.err_index = -1;
+    d.n_accepted = accepted;
+    for (int i = 0; i < accepted; i++) d.accepted_drafts[i] = verify_input[i + 1];
+    d.stop_reason = terminal;
+    d.retain_input_count = terminal != DFLASH_STOP_NONE ? accepted : accepted + 1;
+    if (terminal == DFLASH_STOP_NONE) {
+        d.carry_kind = accepted == n_eff - 1 ? DFLASH_CARRY_BONUS : DFLASH_CARRY_CORRECTION;
+        d.carry_token = targets[accepted];
+    }
+    return DFLASH_OK;
+}
+
+}  // namespace
+
+int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head, dflash_session *sess,
+                         dflash_draft_session *dsess, const int32_t *taps, int32_t n_taps, int32_t carry, int64_t position,
+                         const dflash_step_cfg *cfg, dflash_sampler *sampler, int64_t budget, const int32_t *stop_ids,
+                         int32_t n_stop, const int32_t *draft_override, dflash_step_result *res, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!target || !head || !sess || !dsess || !cfg || !res || (n_stop > 0 && !stop_ids) || budget < 0)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "spec_step: null or invalid argument");
+    if (cfg->sampled_mode != 0 && !sampler) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "spec_step: sampled mode needs a sampler");
+    if (n_taps != head->cfg.n_taps || n_taps > sess->n_taps || !taps)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "spec_step: %d tapped layers, the drafter expects %d", n_taps, head->cfg.n_taps);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    memset(res, 0, sizeof(*res));
+    const int N = head->cfg.block_size;
+    res->n_block = N;
+    int32_t rc;
+
+    auto t0 = std::chrono::steady_clock::now();
+    if ((rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, nullptr, nullptr,
+                                 res->draft_tokens, st)))
+        return rc;
+    res->draft_ms = ms_since(t0);
+    res->draft_tokens[0] = carry;
+    if (draft_override)
+        for (int i = 1; i < N; i++)
+            if (draft_override[i - 1] >= 0) res->draft_tokens[i] = draft_override[i - 1];
+
+    t0 = std::chrono::steady_clock::now();
+    const int32_t *verify_input = res->draft_tokens;
+    if ((rc = dflash_verify_block(ctx, target, sess, verify_input, N, position, taps, n_taps, nullptr, nullptr, sess->hidden,
+                                  nullptr, res->verify_argmax, st)))
+        return rc;
+    DFL_HIP_CHECK(ctx, hipMemcpy(res->verify_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost));
+    res->verify_ms = ms_since(t0);
+
+    t0 = std::chrono::steady_clock::now();
+    if (cfg->sampled_mode != 0) {
+        rc = dflash_accept_prefix(ctx, verify_input, N, sess->logits, target->cfg.vocab, 0, 0, nullptr, nullptr, nullptr,
+                                  nullptr, 0.0f, sampler, budget, stop_ids, n_stop, &res->decision, st);
+    } else {
+        rc = dflash_accept_greedy(verify_input, res->verify_argmax, N, budget, stop_ids, n_stop, &res->decision);
+        if (rc) dfl_fail(ctx, rc, "spec_step: greedy accept rejected its input");
+    }
+    if (rc) {  // nothing is committed: put the KV back where the block started
+        (void)dflash_restore(ctx, sess, position, N, 0);
+        return rc;
+    }
+    res->accept_ms = ms_since(t0);
+
+    if (cfg->sampled_mode == 0 && cfg->fallback_margin > 0.0f) {
+        t0 = std::chrono::steady_clock::now();
+        if ((rc = margin_fallback(ctx, target, sess, taps, n_taps, verify_input, N, position, cfg, budget, stop_ids, n_stop, res, st)))
+            return rc;
+        if (res->fallback_ran) res->fallback_ms = ms_since(t0);
+    }
+
+    const int n_keep = res->decision.retain_input_count;
+    if (n_keep > 0) {  // columns 0..n_keep-1 are the carry and the accepted drafts (qwen/dflash.rs:1066-1084)
+        t0 = std::chrono::steady_clock::now();
+        int32_t positions[16];
+        for (int i = 0; i < n_keep; i++) positions[i] = static_cast<int32_t>(position + i);
+        if ((rc = dflash_draft_append_ctx(ctx, dsess, sess->hidden, n_keep, positions, st))) return rc;
+        DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        res->append_ms = ms_since(t0);
+    }
+    if (!res->fallback_ran && n_keep < N) {
+        t0 = std::chrono::steady_clock::now();
+        if ((rc = dflash_restore(ctx, sess, position, N, n_keep))) return rc;
+        res->restore_ms = ms_since(t0);
     }
     return DFLASH_OK;
 }

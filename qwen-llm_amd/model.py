@@ -356,3 +356,129 @@ class DraftSession:
             self.ctx._h, C.byref(self.target.c), C.byref(self.head.c), self._h, carry_token, mask_token, noise_start_pos,
             argmax.data_ptr(), logits.data_ptr() if logits is not None else None, host, _stream_ptr()))
         return argmax, logits, (list(host) if sync else None)
+
+
+# ---- one speculative transition and the generation loop (qwen/dflash.rs:700-1241) ----
+
+from .binding import AcceptDecision, AcceptDecisionC, Sampler, SamplerC  # noqa: E402
+
+
+class StepCfgC(C.Structure):
+    _fields_ = [("mask_token", C.c_int32), ("sampled_mode", C.c_int32), ("fallback_margin", C.c_float),
+                ("fallback_partial", C.c_int32), ("fallback_partial_min_gap", C.c_float)]
+
+
+class StepResultC(C.Structure):
+    _fields_ = [("decision", AcceptDecisionC), ("n_block", C.c_int32), ("draft_tokens", C.c_int32 * 16),
+                ("verify_argmax", C.c_int32 * 16), ("verify_gap", C.c_float * 16), ("fallback_ran", C.c_int32),
+                ("fallback_rows_replayed", C.c_int32), ("fallback_escalations", C.c_int32),
+                ("fallback_rows_kept", C.c_int32), ("draft_ms", C.c_double), ("verify_ms", C.c_double),
+                ("accept_ms", C.c_double), ("fallback_ms", C.c_double), ("append_ms", C.c_double),
+                ("restore_ms", C.c_double)]
+
+
+DFLASH_VERIFY_FALLBACK_MARGIN_DEFAULT = 0.1       # qwen/dflash.rs:104
+DFLASH_VERIFY_FALLBACK_PARTIAL_MIN_GAP = 0.15     # qwen/dflash.rs:139
+
+
+def accept_greedy(verify_input, verify_argmax, budget: int, stop_ids=()) -> AcceptDecision:
+    L = _lib()
+    n = len(verify_input)
+    L.dflash_accept_greedy.restype = C.c_int32
+    L.dflash_accept_greedy.argtypes = [C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.c_int32, C.c_int64,
+                                       C.POINTER(C.c_int32), C.c_int32, C.POINTER(AcceptDecisionC)]
+    out = AcceptDecisionC()
+    rc = L.dflash_accept_greedy((C.c_int32 * max(n, 1))(*verify_input), (C.c_int32 * max(n, 1))(*verify_argmax), n, budget,
+                                (C.c_int32 * max(len(stop_ids), 1))(*stop_ids), len(stop_ids), C.byref(out))
+    if rc:
+        raise DFlashError(rc, "dflash_accept_greedy: invalid input")
+    return AcceptDecision(out)
+
+
+class SpeculativeDecoder:
+    """Target + drafter sessions driven one packed-verify transition at a time."""
+
+    def __init__(self, ctx: Context, target: TargetModel, head: DraftHead, tap_layers, kv_capacity: int,
+                 mask_token: int, sampler: Sampler | None = None, fallback_margin: float = 0.0,
+                 fallback_partial: bool = True, stop_ids=()):
+        self.ctx, self.target, self.head = ctx, target, head
+        self.tap_layers = list(tap_layers)
+        self.session = Session(ctx, target, kv_capacity, self.tap_layers)
+        self.draft_session = DraftSession(ctx, head, target, kv_capacity)
+        self.sampler = sampler
+        self.stop_ids = list(stop_ids)
+        self.cfg = StepCfgC(mask_token, int(sampler is not None), fallback_margin, int(fallback_partial),
+                            DFLASH_VERIFY_FALLBACK_PARTIAL_MIN_GAP)
+        self._L = _lib()
+        self._L.dflash_spec_step.restype = C.c_int32
+        self._L.dflash_spec_step.argtypes = [
+            C.c_void_p, C.POINTER(ModelC), C.POINTER(DraftHeadC), C.c_void_p, C.c_void_p, C.POINTER(C.c_int32),
+            C.c_int32, C.c_int32, C.c_int64, C.POINTER(StepCfgC), C.POINTER(SamplerC), C.c_int64,
+            C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_int32), C.POINTER(StepResultC), C.c_void_p]
+        self.position = 0
+
+    def close(self):
+        self.session.close()
+        self.draft_session.close()
+
+    def prefill(self, prompt):
+        """Run the prompt through the packed verify in blocks of 16, feed the tapped hidden rows to
+        the drafter context, and return the argmax after the last prompt token."""
+        assert len(prompt) > 0 and self.position == 0
+        last = None
+        for s in range(0, len(prompt), 16):
+            blk = list(prompt[s:s + 16])
+            out = self.session.encode_packed_verify_layer_major(blk, s)
+            self.draft_session.append_target_ctx_columns(out.hidden_capture, list(range(s, s + len(blk))))
+            last = out
+        self.position = len(prompt)
+        return last.argmax_host[-1]
+
+    def step(self, carry: int, budget: int, draft_override=None) -> StepResultC:
+        res = StepResultC()
+        n = self.head.cfg.block_size
+        ov = None
+        if draft_override is not None:
+            ov = (C.c_int32 * (n - 1))(*(list(draft_override) + [-1] * (n - 1))[: n - 1])
+        taps = (C.c_int32 * len(self.tap_layers))(*self.tap_layers)
+        stops = (C.c_int32 * max(len(self.stop_ids), 1))(*self.stop_ids)
+        self.ctx._check(self._L.dflash_spec_step(
+            self.ctx._h, C.byref(self.target.c), C.byref(self.head.c), self.session._h, self.draft_session._h, taps,
+            len(self.tap_layers), carry, self.position, C.byref(self.cfg),
+            C.byref(self.sampler.c) if self.sampler is not None else None, budget, stops, len(self.stop_ids), ov,
+            C.byref(res), _stream_ptr()))
+        self.position += res.decision.retain_input_count
+        return res
+
+    def generate(self, first_carry: int, max_tokens: int, on_step=None, draft_override_fn=None):
+        """Emit up to max_tokens tokens starting with first_carry.  Returns (tokens, stats)."""
+        tokens = [first_carry]
+        stats = {"spec_steps": 0, "accepted_drafts": 0, "drafts_scored": 0, "fallback_calls": 0, "draft_ms": 0.0,
+                 "verify_ms": 0.0, "accept_ms": 0.0, "fallback_ms": 0.0, "append_ms": 0.0, "restore_ms": 0.0,
+                 "stop_reason": None}
+        carry = first_carry
+        while True:
+            if carry in self.stop_ids:
+                stats["stop_reason"] = "eos"
+                break
+            if len(tokens) >= max_tokens:
+                stats["stop_reason"] = "token_limit"
+                break
+            ov = draft_override_fn(tokens, self.position) if draft_override_fn else None
+            res = self.step(carry, max_tokens - len(tokens), ov)
+            d = res.decision
+            stats["spec_steps"] += 1
+            stats["accepted_drafts"] += d.n_accepted
+            stats["drafts_scored"] += res.n_block - 1
+            stats["fallback_calls"] += res.fallback_ran
+            for k in ("draft_ms", "verify_ms", "accept_ms", "fallback_ms", "append_ms", "restore_ms"):
+                stats[k] += getattr(res, k)
+            tokens.extend(d.accepted_drafts[: d.n_accepted])
+            if on_step:
+                on_step(res)
+            if d.stop_reason:
+                stats["stop_reason"] = "eos" if d.stop_reason == 1 else "token_limit"
+                break
+            carry = d.carry_token
+            tokens.append(carry)
+        return tokens, stats

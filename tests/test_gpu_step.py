@@ -1,0 +1,138 @@
+"""GPU parity of one speculative transition and of the generation loop (qwen/dflash.rs:700-1241).
+
+Invariant used as the oracle: whatever the drafter proposes, greedy speculative decoding emits the
+target's own greedy continuation, and sampler-coupled decoding with deterministic proposals emits
+the serial sampler's stream (sampling.rs:2837-2865).  The continuation itself comes from the CPU
+oracle's token-by-token forward; rows whose oracle top-2 gap is within the logit error are not
+compared (none occur for the seeds below)."""
+import numpy as np
+import pytest
+
+import qwen_llm_amd as dfl
+
+pytestmark = pytest.mark.gpu
+
+C1 = dfl.ModelConfig(n_layers=4, hidden=1024, n_q=16, n_kv=8, head_dim=128, ffn=3072, vocab=32000)
+TAPS = [0, 1, 2, 3, 3]
+D1 = dfl.DraftConfig(n_layers=2, hidden=1024, n_q=16, n_kv=8, head_dim=128, ffn=3072, block_size=16, n_taps=5)
+PROMPT_LEN = 40
+MASK = C1.vocab - 1
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = dfl.Context(0, workspace_bytes=256 << 20)
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def world(ctx, oracle):
+    w = dfl.synth_target_weights(C1, seed=11)
+    dw = dfl.synth_draft_weights(D1, seed=3)
+    model, head = dfl.TargetModel(ctx, C1, w), dfl.DraftHead(ctx, D1, dw)
+    omodel, keep = oracle.build_model(C1.as_dict(), w)
+    prompt = np.random.default_rng(1).integers(0, C1.vocab - 1, PROMPT_LEN).tolist()
+    # the oracle's serial greedy continuation and every row's logits
+    ostate = oracle.TargetState(C1.as_dict(), 256)
+    lo, _ = oracle.target_verify(omodel, ostate, prompt, 0, TAPS)
+    cont, rows = [int(lo[-1].argmax())], []
+    for i in range(72):
+        lg, _ = oracle.target_verify(omodel, ostate, [cont[-1]], PROMPT_LEN + i, TAPS)
+        rows.append(lg[0])
+        cont.append(int(lg[0].argmax()))
+    rows = np.stack(rows)
+    top = np.sort(rows, axis=1)
+    decided = (top[:, -1] - top[:, -2]) > 2e-2 * rows.std()
+    return dict(model=model, head=head, omodel=omodel, keep=keep, prompt=prompt, cont=cont, rows=rows, decided=decided)
+
+
+def new_decoder(ctx, world, **kw):
+    dec = dfl.SpeculativeDecoder(ctx, world["model"], world["head"], TAPS, 256, MASK, **kw)
+    first = dec.prefill(world["prompt"])
+    return dec, first
+
+
+@pytest.mark.parametrize("k", [0, 1, 7, 15])
+def test_forced_prefix_is_accepted_exactly(ctx, world, k):
+    cont = world["cont"]
+    assert world["decided"][:16].all(), "seed gives an undecided row in the first block"
+    dec, first = new_decoder(ctx, world)
+    assert first == cont[0]
+    wrong = [(t + 1) % (C1.vocab - 1) for t in cont[1:16]]
+    override = cont[1:1 + k] + wrong[k:]
+    res = dec.step(first, budget=1000, draft_override=override)
+    d = res.decision
+    assert d.n_accepted == k and list(d.accepted_drafts[:k]) == cont[1:1 + k]
+    assert d.carry_token == cont[k + 1]
+    assert d.carry_kind == (dfl.CARRY_BONUS if k == 15 else dfl.CARRY_CORRECTION)
+    assert d.retain_input_count == k + 1 and d.stop_reason == dfl.STOP_NONE
+    assert dec.session.kv_n_pos == PROMPT_LEN + k + 1 == dec.position
+    assert dec.draft_session.ctx_len == PROMPT_LEN + k + 1
+    assert list(res.verify_argmax[:k + 1]) == cont[1:k + 2]
+    dec.close()
+
+
+def test_step_stops_on_eos_and_budget(ctx, world):
+    cont = world["cont"]
+    dec, first = new_decoder(ctx, world, stop_ids=[cont[3]])
+    res = dec.step(first, budget=1000, draft_override=cont[1:16])
+    d = res.decision
+    assert d.n_accepted == 3 and d.stop_reason == dfl.STOP_EOS and d.carry_kind == dfl.CARRY_NONE
+    assert d.retain_input_count == 3 and dec.session.kv_n_pos == PROMPT_LEN + 3
+    dec.close()
+    dec, first = new_decoder(ctx, world)
+    res = dec.step(first, budget=5, draft_override=cont[1:16])
+    d = res.decision
+    assert d.n_accepted == 5 and d.stop_reason == dfl.STOP_TOKEN_LIMIT and d.retain_input_count == 5
+    dec.close()
+
+
+@pytest.mark.parametrize("margin,partial", [(0.0, True), (1e9, False), (1e9, True), (0.5, True)])
+def test_generate_greedy_equals_serial_greedy(ctx, world, margin, partial):
+    cont = world["cont"]
+    undecided = np.flatnonzero(~world["decided"])
+    n_tok = int(min(60, undecided[0] if len(undecided) else 60))  # compare up to the first near-tie of the oracle
+    assert n_tok >= 30
+    dec, first = new_decoder(ctx, world, fallback_margin=margin, fallback_partial=partial)
+    # every third step gets the true continuation as drafts so that long accepts and rollbacks mix
+    def override(tokens, position):
+        done = len(tokens)
+        if (position // 3) % 2 == 0:
+            return cont[done:done + 9] + [-1] * 6
+        return None
+    tokens, stats = dec.generate(first, n_tok, draft_override_fn=override)
+    assert tokens == cont[:n_tok], f"diverged at {next(i for i, (a, b) in enumerate(zip(tokens, cont)) if a != b)}"
+    assert stats["stop_reason"] == "token_limit"
+    assert dec.session.kv_n_pos == PROMPT_LEN + n_tok - 1
+    assert stats["accepted_drafts"] > 0
+    if margin >= 1e9:
+        assert stats["fallback_calls"] == stats["spec_steps"]
+    dec.close()
+
+
+def test_generate_sampled_equals_serial_sampler(ctx, world, oracle):
+    """Deterministic-proposal coupling == serial sampling with the same stream (sampling.rs:2837-2865).
+    The serial stream is the CPU oracle's sampler applied to the logits of a token-by-token pass through
+    the same device kernels: with random-init weights the top-20 logits are near ties, so a stream
+    drawn from the oracle's own logits (1e-3 away) is not a usable expectation."""
+    n_tok = 40
+    kw = dict(temperature=0.8, top_k=20, top_p=0.95, min_p=0.0, seed=1234)
+    osamp = oracle.make_sampler(**kw)
+    serial = dfl.Session(ctx, world["model"], 256, TAPS)
+    out = None
+    for s in range(0, PROMPT_LEN, 16):
+        out = serial.encode_packed_verify_layer_major(world["prompt"][s:s + 16], s)
+    want = [out.argmax_host[-1]]
+    while len(want) < n_tok:
+        out = serial.encode_packed_verify_layer_major([want[-1]], PROMPT_LEN + len(want) - 1, want_logits=True)
+        rc, tok, _idx, _err = oracle.sample(osamp, out.logits.cpu().numpy()[0])
+        assert rc == 0
+        want.append(tok)
+    serial.close()
+    dec, first = new_decoder(ctx, world, sampler=dfl.Sampler(**kw))
+    tokens, stats = dec.generate(first, n_tok, draft_override_fn=lambda t, p: want[len(t):len(t) + 6] + [-1] * 9)
+    assert tokens == want
+    assert stats["accepted_drafts"] > 0
+    assert dec.sampler.draws == n_tok - 1 == oracle.sampler_state(osamp)[1]
+    dec.close()
