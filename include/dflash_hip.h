@@ -70,7 +70,7 @@ const char *dflash_version(void);
 /* Per-kernel GPU timers: enable_phase_timers / maybe_record (metal_dflash.rs:5181-5190, 5622).
  * While enabled, each call brackets its dominant kernel with events on the call's stream and
  * waits for it, accumulating into a slot: 0 few-row GEMM, 1 verify attention, 2 acceptance,
- * 3 argmax/top-k, 4 activation re-layout.  Enabling or disabling clears the slots. */
+ * 3 argmax/top-k, 4 split-K reduction of the few-row GEMM.  Enabling or disabling clears the slots. */
 void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable);
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms_host,
                                  int64_t *launches_host);

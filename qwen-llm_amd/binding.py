@@ -212,7 +212,7 @@ class Context:
             raise DFlashError(rc, self._lib.dflash_last_error(self._h).decode())
 
     # ---- enable_phase_timers (metal_dflash.rs:5181-5190)
-    T_GEMM, T_ATTN, T_ACCEPT, T_ARGMAX, T_PREP = 0, 1, 2, 3, 4
+    T_GEMM, T_ATTN, T_ACCEPT, T_ARGMAX, T_REDUCE = 0, 1, 2, 3, 4
 
     def set_kernel_timing(self, enable: bool):
         self._lib.dflash_ctx_set_kernel_timing(self._h, int(enable))

@@ -31,7 +31,7 @@ struct dflash_ctx {
 };
 
 // Slots of the per-kernel timers.
-enum { DFL_T_GEMM = 0, DFL_T_ATTN = 1, DFL_T_ACCEPT = 2, DFL_T_ARGMAX = 3, DFL_T_PREP = 4 };
+enum { DFL_T_GEMM = 0, DFL_T_ATTN = 1, DFL_T_ACCEPT = 2, DFL_T_ARGMAX = 3, DFL_T_REDUCE = 4 };
 
 // Brackets the dominant kernel of a call with events on its stream when timing is on.
 struct dfl_timed {

@@ -7,27 +7,19 @@
 // v_mfma_f32_16x16x32_f16, so a wave owns 16 weight rows (one output tile) and
 // streams them along K; lane l serves weight row l%16 and the k-octet l/16.
 //
-//  * Q4_K: a lane reads the 32 quant bytes of "its" chunk of a super-block (two
-//    sub-blocks: low and high nibbles) straight from HBM.  Nibbles are turned into
-//    exact f16 integers by OR-ing them into the mantissa of 1024.0 (low nibble) or
-//    64.0 (high nibble, which sits four bits up), and one packed f16 fma per value
-//    pair, fma(1024+q, s, -1024*s), yields round(q*s) with a single rounding
-//    (s = d*sc_j in f16).  The per-sub-block minimum never touches the nibbles:
-//    sum_k dmin*m_j*x[k] = dmin*m_j * (sum of x over the sub-block), so the eight
-//    minima of a super-block meet eight pre-summed activations in one extra MFMA
-//    per four super-blocks.  That keeps the vector ALU near 10 instructions per
-//    MFMA, below what the HBM stream needs.
-//  * X is re-laid out once per call by a small kernel into the exact per-lane
-//    fragment order the MFMA wants (and its sub-block sums are taken there).  A
-//    workgroup of eight waves (eight output tiles) copies the fragments of its
-//    K-slice into LDS once and every wave reads its A operands from there, so the
-//    activation traffic out of L2 stays well below the weight stream.
-//  * A wave issues the loads of every super-block of its K-slice before it computes
-//    anything: the whole weight matrix is in flight at once and the kernel runs as a
-//    single pass at the memory system's pace.
-//  * K is split over workgroups; each writes its partial tiles and the last one to
-//    arrive (a counter per tile group) adds them in slice order, so results are
-//    run-to-run deterministic.
+//  * Q4_K: nibbles are turned into exact f16 integers by OR-ing them into the mantissa
+//    of 1024.0 (low nibble) or 64.0 (high nibble, which sits four bits up), and one
+//    packed f16 fma per value pair, fma(1024+q, s, -1024*s), yields round(q*s) with a
+//    single rounding (s = d*sc_j in f16).  The per-sub-block minimum never touches the
+//    nibbles: sum_k dmin*m_j*x[k] = dmin*m_j * (sum of x over the sub-block), so the
+//    eight minima of a super-block meet eight pre-summed activations in one extra MFMA
+//    (two: the sums are carried as a high and a low f16 part).
+//  * The kernel is a persistent stream: one workgroup per CU walks a contiguous range of
+//    (tile group x super-block) work, weights go HBM -> LDS with direct-to-LDS loads
+//    through a ring of buffers, activations are converted to f16 MFMA fragments on the
+//    way into the same ring.  See the comment on the kernel for the pipeline.
+//  * K is split where the ranges cut a tile group; partial tiles are added by a second
+//    small kernel in a fixed order, so results are run-to-run deterministic.
 //  * Q6_K / Q8_0 share a generic kernel: eight consecutive weights per lane are
 //    dequantised to f16 and fed to the same MFMA.
 #include "common.h"
@@ -37,62 +29,17 @@
 namespace {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxSplit = 16;
-constexpr int kWavesQ4K = 8;  // output tiles (waves) per workgroup of the Q4_K kernel
-
-// ----------------------------------------------------------------------------
-// X preparation
-// ----------------------------------------------------------------------------
 
 template <typename T>
 __device__ __forceinline__ _Float16 load_x(const T *x, int m, int n_rows, int64_t n_in, int64_t k) {
     if (m >= n_rows) return static_cast<_Float16>(0.0f);
     return static_cast<_Float16>(x[static_cast<int64_t>(m) * n_in + k]);
-}
-
-// Q4_K layout: kQ4KBlockFrags (= 544) half8 entries per super-block b:
-//   [t*64 + lane], t = 0..7 : A fragment of MFMA t for lane (m = lane%16, g = lane/16),
-//        value i:  k = 256 b + 64 g + (t < 4 ? 8 t : 32 + 8 (t-4)) + perm[i],
-//        perm = {0,2,1,3,4,6,5,7}: the order in which the nibble unpack emits a lane's values;
-//   [512 + m], [528 + m]    : the eight sub-block sums of row m's f16-rounded activations,
-//        split into a high and a low f16 part.
-// One workgroup per super-block.
-constexpr int kQ4KBlockFrags = 544;
-
-template <typename T>
-__global__ void __launch_bounds__(256) prep_x_q4k_kernel(const T *__restrict__ x, half8_t *__restrict__ xp,
-                                                         int n_rows, int64_t n_in) {
-    __shared__ _Float16 tile[16][256 + 8];
-    const int b = blockIdx.x;
-    const int tid = threadIdx.x;
-    half8_t *out = xp + static_cast<int64_t>(b) * kQ4KBlockFrags;
-#pragma unroll
-    for (int m = 0; m < 16; m++) tile[m][tid] = load_x(x, m, n_rows, n_in, 256ll * b + tid);
-    __syncthreads();
-#pragma unroll
-    for (int it = 0; it < 2; it++) {
-        int item = tid + 256 * it;
-        int t = item >> 6, lane = item & 63;
-        int m = lane & 15, g = lane >> 4;
-        int k0 = 64 * g + (t < 4 ? 8 * t : 32 + 8 * (t - 4));
-        const _Float16 *src = &tile[m][k0];
-        half8_t v = {src[0], src[2], src[1], src[3], src[4], src[6], src[5], src[7]};
-        out[item] = v;
-    }
-    if (tid < 128) {
-        int m = tid >> 3, j = tid & 7;
-        float s = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 32; e++) s += static_cast<float>(tile[m][32 * j + e]);
-        _Float16 h = static_cast<_Float16>(s);
-        _Float16 *sums = reinterpret_cast<_Float16 *>(out + 512);
-        sums[m * 8 + j] = h;
-        sums[128 + m * 8 + j] = static_cast<_Float16>(s - static_cast<float>(h));
-    }
 }
 
 // Natural layout for the generic kernel: step s (32 k), lane (m, g), value i: k = 32 s + 8 g + i.
@@ -113,6 +60,15 @@ __global__ void __launch_bounds__(256) prep_x_natural_kernel(const T *__restrict
 // ----------------------------------------------------------------------------
 // Q4_K kernel
 // ----------------------------------------------------------------------------
+
+// Activation fragments of one super-block b in LDS: kQ4KBlockFrags (= 640) half8 entries:
+//   [t*64 + lane], t = 0..7 : A fragment of MFMA t for lane (m = lane%16, g = lane/16),
+//        value i:  k = 256 b + 64 g + 8 t + perm[i],
+//        perm = {0,2,1,3,4,6,5,7}: the order in which the nibble unpack emits a lane's values;
+//   [512 + lane], [576 + lane] : A fragment of the minima MFMA for lane (m, g): values 0 and 1
+//        are the sums of row m's f16-rounded activations over sub-blocks 2g and 2g+1 (a high and
+//        a low f16 part in the two entries), values 2..7 stay zero.
+constexpr int kQ4KBlockFrags = 640;
 
 __device__ __forceinline__ half2_t as_half2(uint32_t bits) { return __builtin_bit_cast(half2_t, bits); }
 
@@ -154,99 +110,47 @@ __device__ __forceinline__ _Float16 byte_to_half(uint32_t v, int j) {
     return static_cast<_Float16>(static_cast<float>((v >> (8 * j)) & 0xffu));
 }
 
-// One super-block of one output tile: 8 MFMAs.  hdr = {d|dmin, scales[0..3], [4..7], [8..11]},
-// q0/q1 = the lane's 32 quant bytes (chunk g), a = this super-block's A fragments in LDS.
-// A super-block slot past the end of a short stage (`live` false) holds a re-read of the last
-// one; its scales are forced to zero so it adds nothing and the code stays straight-line.
-// After every second MFMA the wave issues one load of a later stage (`next`, loads j0 ..): spread
-// over the MFMAs, the loads never queue up behind each other in the address unit, which would
-// otherwise stall all eight waves at once at the top of each stage.
-struct Q4KIssue;
-__device__ __forceinline__ void q4k_issue_one(const Q4KIssue &d, int j, int tid);
-
-__device__ __forceinline__ float4_t q4k_block(u32x4_t hdr, u32x4_t q0, u32x4_t q1, const half8_t *a, int g,
-                                              bool live, Q4KMagic magic, float4_t acc, const Q4KIssue &next, int j0,
-                                              int tid) {
-    // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles)
-    uint32_t lo_sc = hdr.y & 0x3F3F3F3Fu;
-    uint32_t hi_sc = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
-    uint32_t sel = (g < 2 ? lo_sc : hi_sc) >> (16 * (g & 1));
-    _Float16 d = live ? __builtin_bit_cast(half2_t, hdr.x)[0] : static_cast<_Float16>(0.0f);
-    _Float16 s_lo = byte_to_half(sel, 0) * d;
-    _Float16 s_hi = byte_to_half(sel, 1) * d;
-    half2_t s2l = splat(s_lo), c2l = splat(s_lo * static_cast<_Float16>(-1024.0f));
-    half2_t s2h = splat(s_hi), c2h = splat(s_hi * static_cast<_Float16>(-64.0f));
-    uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t * 64], bl, acc, 0, 0, 0);
-        if (t & 1) {
-            q4k_issue_one(next, j0 + (t >> 1), tid);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(4 + t) * 64], bh, acc, 0, 0, 0);
-        if (t & 1) {
-            q4k_issue_one(next, j0 + 2 + (t >> 1), tid);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    return acc;
-}
-
-// The eight dmin*m_j of one super-block as an MFMA B operand.
-__device__ __forceinline__ half8_t q4k_mins(u32x4_t h, bool valid) {
-    _Float16 dmin = valid ? __builtin_bit_cast(half2_t, h.x)[1] : static_cast<_Float16>(0.0f);
-    uint32_t lo_m = h.z & 0x3F3F3F3Fu;
-    uint32_t hi_m = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-    half8_t bm;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        bm[j] = byte_to_half(lo_m, j) * dmin;
-        bm[4 + j] = byte_to_half(hi_m, j) * dmin;
-    }
-    return bm;
-}
-
 // Streaming Q4_K kernel.
 //
 // Work split.  The iteration space is (tile group) x (super-block), flattened group-major; a
-// tile group is kWavesQ4K consecutive output tiles, one per wave of a workgroup.  The grid is
-// one workgroup per CU and workgroup i owns the contiguous range [T i / G, T (i+1) / G) of that
-// space, so every CU streams the same number of weight bytes whatever the shape.
+// tile group is kWaves consecutive output tiles (16 weight rows each), one per wave of a
+// workgroup.  The grid is one workgroup per CU and workgroup i owns the contiguous range
+// [T i / G, T (i+1) / G) of that space, so every CU streams the same number of weight bytes
+// whatever the shape.
 //
-// Data path.  A workgroup walks its range in stages of up to kStage super-blocks that stay
-// inside one tile group.  Per stage, the group's 128 weight rows (a row-contiguous slice of
-// kStage*144 bytes each) and the prepared activations are copied global -> LDS by
-// global_load_lds_dwordx4: consecutive lanes take consecutive 16-byte pieces, so HBM sees
-// row-contiguous requests and no VGPR is held while a load is in flight.  The stages rotate
-// through kBufs LDS buffers; the loads of stage j + kBufs - 1 are issued before stage j is
-// computed, so HBM never idles.  Each wave issues exactly kLoadsPerStage load instructions per
-// stage (surplus ones land in a spare LDS slot), which makes "stage j has landed" a constant
-// s_waitcnt.  Waves then read their tile's quant bytes and A fragments with ds_read_b128.
+// Data path.  A stage is one super-block of one tile group.  Its 16*kWaves weight rows (144
+// contiguous bytes each) are copied global -> LDS by global_load_lds_dwordx4: consecutive lanes
+// take consecutive 16-byte pieces, so HBM sees row-contiguous requests and no VGPR is held
+// while a load is in flight; the piece -> address map of a lane is the same in every stage
+// (only a uniform base moves), so a load costs no vector ALU work.  The stage's activations
+// (16 rows x 256 values, straight from the caller's f32 or f16 matrix, L2-resident) are loaded
+// into registers three stages ahead, rounded to f16, and written to LDS in MFMA fragment order
+// together with their sub-block sums one stage ahead.  Three LDS buffers rotate: while stage d
+// is computed out of one, the activations of d+1 are already in the second and the weights of
+// d+1 and d+2 are landing in the second and third.  The loads are issued between the MFMAs of
+// the stage being computed (one weight load after every second MFMA, then the activations), in
+// the same order in every wave, which makes "everything but the youngest group of loads has
+// landed" a constant s_waitcnt at the top of a stage.  Waves then read their tile's quant bytes
+// and A fragments with ds_read_b128 (row stride 9 pieces: conflict-free).  All per-stage
+// bookkeeping is a handful of scalar additions: the scalar unit is shared by the CU's waves.
 //
 // Split K.  When a range leaves a tile group, the accumulators are flushed: straight to Y if
-// this workgroup covered the group's whole K, else as a partial tile whose every value carries
-// the call's epoch tag in the same 8-byte store.  The highest-numbered workgroup that touches a
-// group owns it: at the end of its own range it reads the group's partial tiles in workgroup
-// order, polling each value until its tag is the current epoch, and writes Y.  No fences, no
-// atomics, deterministic sums; a poll only ever waits for lower-numbered workgroups, which were
-// dispatched first, and gives up (writing NaN) after a bounded number of tries.
-constexpr int kStage = 2;
-constexpr int kThreadsQ4K = 64 * kWavesQ4K;
-constexpr int kGroupRows = 16 * kWavesQ4K;
-constexpr int kRowPieces = 9 * kStage + 1;  // LDS row stride in pieces: one pad piece staggers the banks
-constexpr int kStageWPieces = kGroupRows * kRowPieces;          // 16-byte pieces of weights per stage
-constexpr int kStageXPieces = kStage * kQ4KBlockFrags;          // 16-byte pieces of activations per stage
-constexpr int kBufPieces = kStageWPieces + kStageXPieces;       // one LDS buffer
-constexpr int kWLoads = (kStageWPieces + kThreadsQ4K - 1) / kThreadsQ4K;
-constexpr int kXLoads = (kStageXPieces + kThreadsQ4K - 1) / kThreadsQ4K;
-constexpr int kLoadsPerStage = kWLoads + kXLoads;
-constexpr uint32_t kSpinLimit = 1u << 22;
+// this workgroup covered the group's whole K, else as a partial tile, which a second, chip-wide
+// kernel adds up in workgroup order (deterministic sums, no spinning, no atomics).
+template <int kWaves>
+struct Q4KGeom {
+    static constexpr int kThreads = 64 * kWaves;
+    static constexpr int kRows = 16 * kWaves;
+    static constexpr int kWPieces = kRows * 9;              // 16-byte pieces of weights per stage
+    static constexpr int kWaveLoads = kWPieces / 64;        // weight wave-loads per stage
+    static constexpr int kFull = kWaveLoads / kWaves;       // ... every wave issues this many,
+    static constexpr int kExtra = kWaveLoads % kWaves;      // ... and waves below kExtra one more
+    static constexpr int kXLoads = 16 / kWaves;             // activation loads per thread and stage
+    static constexpr int kBufPieces = kWPieces + kQ4KBlockFrags;
+    static_assert(kWPieces % 64 == 0, "whole wave-loads");
+    static_assert(kFull + (kExtra ? 1 : 0) <= 4, "one weight load is issued after every second of a stage's 8 MFMAs");
+    static_assert(kXLoads == 1 || kXLoads == 2, "8 or 16 waves");
+};
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -262,112 +166,193 @@ struct Q4KRange {
     int nb, n_wg, first_group;
 };
 
-__device__ __forceinline__ void q4k_stage_at(const Q4KRange &rg, int it, int &group, int &b, int &len) {
-    group = static_cast<int>(static_cast<uint32_t>(it) / static_cast<uint32_t>(rg.nb));
-    b = it - group * rg.nb;
-    len = min(kStage, min(rg.nb - b, rg.it_end - it));
-}
-
-// Everything a wave needs to issue its kLoadsPerStage direct-to-LDS loads of one stage.
-// `buf` is the stage's LDS buffer (kBufPieces pieces), `spare` a 1 KiB slot that absorbs the
-// surplus loads of short stages.
-struct Q4KIssue {
-    const uint8_t *wbase;   // first super-block of the stage in weight row 0
-    const half8_t *xsrc;    // the stage's prepared activations
-    half8_t *buf, *spare;
-    size_t row_bytes;
-    int row0, n_out, ppr, n_x;
-    bool on;
+// Per-lane constants of the loads and of the activation write, set up once per kernel.
+template <int kWaves>
+struct Q4KLane {
+    uint32_t w_off[Q4KGeom<kWaves>::kFull + 1];  // weight piece: byte offset from (group's first row, super-block)
+    uint32_t x_off[Q4KGeom<kWaves>::kXLoads];    // activation vector: byte offset from x[0][256 b]
+    uint32_t xw_off[Q4KGeom<kWaves>::kXLoads];   // its fragment half in LDS: byte offset from the buffer
+    uint32_t xs_off[Q4KGeom<kWaves>::kXLoads];   // its sums slot in LDS (lanes with sums_lane only)
+    bool x_live[Q4KGeom<kWaves>::kXLoads];       // the row is below n_rows
+    bool sums_lane;
 };
 
-__device__ __forceinline__ Q4KIssue q4k_issue_desc(const uint8_t *__restrict__ w, const half8_t *__restrict__ xp,
-                                                   half8_t *buf, half8_t *spare, int group, int b, int len,
-                                                   int n_out, size_t row_bytes, bool on) {
-    Q4KIssue d;
-    d.wbase = w + static_cast<size_t>(b) * DFL_Q4_K_BYTES;
-    d.xsrc = xp + static_cast<size_t>(b) * kQ4KBlockFrags;
-    d.buf = buf;
-    d.spare = spare;
-    d.row_bytes = row_bytes;
-    d.row0 = group * kGroupRows;
-    d.n_out = n_out;
-    d.ppr = 9 * len;  // real pieces per weight row; the rest of the row's kRowPieces re-read piece 0
-    d.n_x = len * kQ4KBlockFrags;
-    d.on = on;
-    return d;
-}
-
-// Load number j (0 .. kLoadsPerStage-1) of the stage: kWLoads weight loads, then kXLoads
-// activation loads.  Consecutive lanes take consecutive 16-byte pieces.
-__device__ __forceinline__ void q4k_issue_one(const Q4KIssue &d, int j, int tid) {
-    if (!d.on) return;
+// Rows past n_out (ragged last group) re-read the last row; their results are never stored.
+template <int kWaves>
+__device__ __forceinline__ void q4k_lane_w_offsets(Q4KLane<kWaves> &L, int tid, int row0, int n_out,
+                                                   uint32_t row_bytes) {
+    using G = Q4KGeom<kWaves>;
     const int lane = tid & 63, wave = tid >> 6;
-    if (j < kWLoads) {
-        const int p0 = (j * kWavesQ4K + wave) * 64;  // wave-uniform
-        const int p = min(p0 + lane, kStageWPieces - 1);
-        const int r = static_cast<int>(static_cast<uint32_t>(p) / static_cast<uint32_t>(kRowPieces));
-        int o = p - r * kRowPieces;
-        o = o < d.ppr ? o : 0;
-        const int row = min(d.row0 + r, d.n_out - 1);
-        const uint8_t *src = d.wbase + static_cast<size_t>(row) * d.row_bytes + o * 16;
-        half8_t *dst = (p0 < kStageWPieces) ? d.buf + p0 : d.spare;
-        __builtin_amdgcn_global_load_lds((gptr_t)(src), (lptr_t)(dst), 16, 0, 0);
-    } else {
-        const int p0 = ((j - kWLoads) * kWavesQ4K + wave) * 64;
-        const int p = min(p0 + lane, d.n_x - 1);
-        half8_t *dst = (p0 < d.n_x) ? d.buf + kStageWPieces + p0 : d.spare;
-        __builtin_amdgcn_global_load_lds((gptr_t)(d.xsrc + p), (lptr_t)(dst), 16, 0, 0);
+    const int last = n_out - 1 - row0;
+#pragma unroll
+    for (int j = 0; j <= G::kFull; j++) {
+        const int p = min((j * kWaves + wave) * 64 + lane, G::kWPieces - 1);
+        const int r = min(p / 9, last);
+        L.w_off[j] = static_cast<uint32_t>(r) * row_bytes + static_cast<uint32_t>(p % 9) * 16u;
     }
 }
 
-__device__ __forceinline__ void q4k_issue_all(const Q4KIssue &d, int tid) {
+// Activation item of (virtual wave vw = wave + kWaves r, lane l): row m = 8 (vw & 1) + (l & 7),
+// four values k = 4c .. 4c+3 with c = 8 (vw >> 1) + (l >> 3): a virtual wave is one sub-block of
+// eight rows, its global loads are eight 128-byte runs, its LDS writes are conflict-free, and a
+// sub-block sum is a reduction over lane bits 3..5.
+template <int kWaves, typename XT>
+__device__ __forceinline__ void q4k_lane_x_offsets(Q4KLane<kWaves> &L, int tid, int n_rows, uint32_t n_in) {
+    using G = Q4KGeom<kWaves>;
+    const int lane = tid & 63, wave = tid >> 6;
+    L.sums_lane = (lane >> 3) == 0;
 #pragma unroll
-    for (int j = 0; j < kLoadsPerStage; j++) q4k_issue_one(d, j, tid);
+    for (int r = 0; r < G::kXLoads; r++) {
+        const int vw = wave + kWaves * r;
+        const int m = 8 * (vw & 1) + (lane & 7), c = 8 * (vw >> 1) + (lane >> 3);
+        const int g = c >> 4, c15 = c & 15, j = c >> 3;
+        L.x_live[r] = m < n_rows;
+        L.x_off[r] = (static_cast<uint32_t>(min(m, n_rows - 1)) * n_in + 4u * c) * static_cast<uint32_t>(sizeof(XT));
+        L.xw_off[r] = static_cast<uint32_t>((G::kWPieces + (c15 >> 1) * 64 + m + 16 * g) * 16 + 8 * (c15 & 1));
+        L.xs_off[r] = static_cast<uint32_t>((G::kWPieces + 512 + m + 16 * (j >> 1)) * 16 + 2 * (j & 1));
+    }
 }
 
-// One stage of MFMAs for this wave's tile, out of LDS buffer `buf`.
-static_assert(kLoadsPerStage == 4 * kStage, "one load is issued after every second of a stage's 8*kStage MFMAs");
+template <typename XT>
+struct Q4KXVec;
+template <>
+struct Q4KXVec<float> {
+    typedef float4_t type;
+};
+template <>
+struct Q4KXVec<_Float16> {
+    typedef half4_t type;
+};
 
-__device__ __forceinline__ void q4k_compute(const half8_t *buf, int len, int tid, Q4KMagic magic, float4_t &acc,
-                                            float4_t &acc_min, const Q4KIssue &next) {
-    const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
-    const u32x4_t *wrow = reinterpret_cast<const u32x4_t *>(buf) + (wave * 16 + n) * kRowPieces;
-    const half8_t *xbuf = buf + kStageWPieces;
+// Raw activations of one stage held by a thread.
+template <int kWaves, typename XT>
+struct Q4KXRaw {
+    typename Q4KXVec<XT>::type v[Q4KGeom<kWaves>::kXLoads];
+};
+
+template <int kWaves, typename XT>
+__device__ __forceinline__ void q4k_load_x(const uint8_t *xblock, const Q4KLane<kWaves> &L, Q4KXRaw<kWaves, XT> &raw) {
+    typedef typename Q4KXVec<XT>::type vec_t;
 #pragma unroll
-    for (int u = 0; u < kStage; u++) {
-        const int ub = min(u, len - 1);
-        const u32x4_t *blk = wrow + ub * 9;
-        acc = q4k_block(blk[0], blk[1 + 2 * g], blk[2 + 2 * g], xbuf + ub * kQ4KBlockFrags + lane, g, u < len, magic,
-                        acc, next, 4 * u, tid);
+    for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) raw.v[r] = *reinterpret_cast<const vec_t *>(xblock + L.x_off[r]);
+}
+
+// Rounds a stage's raw activations to f16 and writes this thread's share of the fragments and
+// sub-block sums into the buffer at `buf`.
+template <int kWaves, typename XT>
+__device__ __forceinline__ void q4k_write_x(half8_t *buf, const Q4KLane<kWaves> &L, const Q4KXRaw<kWaves, XT> &raw,
+                                            bool full_rows) {
+    uint8_t *base = reinterpret_cast<uint8_t *>(buf);
+#pragma unroll
+    for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) {
+        _Float16 h[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) h[i] = static_cast<_Float16>(raw.v[r][i]);
+        if (!full_rows && !L.x_live[r]) {  // full_rows is uniform: a 16-row block never takes this
+#pragma unroll
+            for (int i = 0; i < 4; i++) h[i] = static_cast<_Float16>(0.0f);
+        }
+        half4_t frag = {h[0], h[2], h[1], h[3]};
+        *reinterpret_cast<half4_t *>(base + L.xw_off[r]) = frag;
+        float s = (static_cast<float>(h[0]) + static_cast<float>(h[1])) + (static_cast<float>(h[2]) + static_cast<float>(h[3]));
+        s += __shfl_xor(s, 8, 64);
+        s += __shfl_xor(s, 16, 64);
+        s += __shfl_xor(s, 32, 64);
+        if (L.sums_lane) {
+            const _Float16 hi = static_cast<_Float16>(s);
+            *reinterpret_cast<_Float16 *>(base + L.xs_off[r]) = hi;
+            *reinterpret_cast<_Float16 *>(base + L.xs_off[r] + 64 * 16) = static_cast<_Float16>(s - static_cast<float>(hi));
+        }
     }
-    // minima: lane (n, g) supplies super-block g of the stage
-    const bool valid = g < len;
-    const int gb = valid ? g : 0;
-    half8_t bm = q4k_mins(wrow[gb * 9], valid);
-    const half8_t *sums = xbuf + gb * kQ4KBlockFrags + 512 + n;
-    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[0], bm, acc_min, 0, 0, 0);
-    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[16], bm, acc_min, 0, 0, 0);
+}
+
+// One weight wave-load of the stage at `wstage` (uniform) into the buffer at `buf`.
+template <int kWaves>
+__device__ __forceinline__ void q4k_issue_w(const uint8_t *wstage, half8_t *buf, const Q4KLane<kWaves> &L, int j, int wave) {
+    __builtin_amdgcn_global_load_lds((gptr_t)(wstage + L.w_off[j]), (lptr_t)(buf + (j * kWaves + wave) * 64), 16, 0, 0);
+}
+
+// One stage (one super-block) of this wave's tile out of the LDS buffer `buf`: 8 MFMAs plus 2 for
+// the minima.  hdr = {d|dmin, scales[0..3], [4..7], [8..11]}, q0/q1 = the lane's 32 quant bytes
+// (chunk g: sub-blocks 2g in the low and 2g+1 in the high nibbles).  The loads of later stages
+// are issued in between: one weight load after every second MFMA (spread over the MFMAs, the
+// loads never queue up behind each other in the address unit), then the activations; the
+// activations of the next stage are converted and written to LDS half way through.
+template <int kWaves, typename XT>
+__device__ __forceinline__ void q4k_compute(const half8_t *buf, int lane, int wave, Q4KMagic magic, float4_t &acc,
+                                            float4_t &acc_min, bool issue_w, const uint8_t *wstage, half8_t *wbuf,
+                                            bool issue_x, const uint8_t *xblock, const Q4KLane<kWaves> &L,
+                                            Q4KXRaw<kWaves, XT> &raw, bool write_x, half8_t *xbuf, bool full_rows) {
+    using G = Q4KGeom<kWaves>;
+    const int n = lane & 15, g = lane >> 4;
+    const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(buf) + (wave * 16 + n) * 9;
+    const half8_t *a = buf + G::kWPieces + lane;
+    const u32x4_t hdr = blk[0], q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
+    // scales and minima of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles); the 6-bit codes of
+    // sub-blocks 0..3 sit in one dword, those of 4..7 are split over two: select by bit mask,
+    // not by branch
+    const int sh = 16 * (g & 1);
+    const uint32_t upper = 0u - static_cast<uint32_t>(g >> 1);  // all ones for g = 2, 3
+    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu, mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t sc_sel = ((sc_hi & upper) | (sc_lo & ~upper)) >> sh;
+    const uint32_t mn_sel = ((mn_hi & upper) | (mn_lo & ~upper)) >> sh;
+    const half2_t dm = __builtin_bit_cast(half2_t, hdr.x);
+    const _Float16 s_lo = byte_to_half(sc_sel, 0) * dm[0];
+    const _Float16 s_hi = byte_to_half(sc_sel, 1) * dm[0];
+    const half2_t s2l = splat(s_lo), c2l = splat(s_lo * static_cast<_Float16>(-1024.0f));
+    const half2_t s2h = splat(s_hi), c2h = splat(s_hi * static_cast<_Float16>(-64.0f));
+    const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t * 64], bl, acc, 0, 0, 0);
+        if (t & 1) {
+            const int j = t >> 1;
+            if (issue_w && (j < G::kFull || (j == G::kFull && wave < G::kExtra))) q4k_issue_w<kWaves>(wstage, wbuf, L, j, wave);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // the next stage's activations (in registers since the wait at the top of this stage) go to
+    // LDS here, off the critical path between that wait and the barrier
+    if (write_x) q4k_write_x<kWaves, XT>(xbuf, L, raw, full_rows);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(4 + t) * 64], bh, acc, 0, 0, 0);
+        if (t & 1) {
+            const int j = 2 + (t >> 1);
+            if (issue_w && (j < G::kFull || (j == G::kFull && wave < G::kExtra))) q4k_issue_w<kWaves>(wstage, wbuf, L, j, wave);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (issue_x) q4k_load_x<kWaves, XT>(xblock, L, raw);
+    __builtin_amdgcn_sched_barrier(0);
+    // minima: lane (n, g) carries dmin*m of sub-blocks 2g and 2g+1 in values 0 and 1 of the B operand
+    const half8_t bm = {byte_to_half(mn_sel, 0) * dm[1], byte_to_half(mn_sel, 1) * dm[1], 0, 0, 0, 0, 0, 0};
+    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[512], bm, acc_min, 0, 0, 0);
+    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[576], bm, acc_min, 0, 0, 0);
 }
 
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt low bits [3:0],
 // high bits [15:14]; expcnt [6:4] and lgkmcnt [11:8] at their maxima)
 constexpr int q4k_vmcnt(int n) { return ((n & 0xF) | ((n & 0x30) << 10)) | 0x0F70; }
-
-struct Q4KTagged {
-    float value;
-    uint32_t tag;
-};
+// s_waitcnt lgkmcnt(0) alone
+constexpr int kWaitLds = 0xC07F;
 
 // Ends a tile group's segment: Y directly if this workgroup covered the group's whole K, else a
-// tagged partial tile.
+// partial tile for the reduce kernel (slot 0: the range's first group, slot 1: its last).
+template <int kWaves>
 __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, int group, float4_t &acc, float4_t &acc_min,
-                                          float *__restrict__ y, Q4KTagged *__restrict__ partials, uint32_t epoch,
-                                          int n_out, int n_rows, int tid) {
+                                          float *__restrict__ y, float *__restrict__ partials, int n_out, int n_rows,
+                                          int tid) {
+    // rare path: an opaque copy of the thread index keeps its index arithmetic out of the stage loop
+    asm volatile("" : "+v"(tid));
     const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
     float4_t res = acc - acc_min;
     acc = float4_t{0, 0, 0, 0};
     acc_min = float4_t{0, 0, 0, 0};
-    const int orow = (group * kWavesQ4K + wave) * 16 + n;
+    const int orow = (group * kWaves + wave) * 16 + n;
     const int wg_first = q4k_wg_of(group * rg.nb, rg.total, rg.n_wg);
     const int wg_last = q4k_wg_of((group + 1) * rg.nb - 1, rg.total, rg.n_wg);
     if (wg_first == wg_last) {
@@ -379,58 +364,67 @@ __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, int group, float4_
         return;
     }
     const int slot = (group == rg.first_group) ? 0 : 1;
-    Q4KTagged *p = partials + ((static_cast<size_t>(blockIdx.x) * 2 + slot) * kWavesQ4K + wave) * 256;
+    float *p = partials + ((static_cast<size_t>(blockIdx.x) * 2 + slot) * kWaves + wave) * 256;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        Q4KTagged t = {res[i], epoch};
-        __hip_atomic_store(reinterpret_cast<uint64_t *>(&p[(4 * g + i) * 16 + n]), __builtin_bit_cast(uint64_t, t),
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    for (int i = 0; i < 4; i++) p[(4 * g + i) * 16 + n] = res[i];
 }
 
-// Runs once, at the end of a workgroup's range: if its first tile group is split over several
-// workgroups and this is the highest-numbered one, add the group's partial tiles in workgroup
-// order and write Y.
-__device__ __forceinline__ void q4k_reduce_owned(const Q4KRange &rg, float *__restrict__ y,
-                                                 const Q4KTagged *__restrict__ partials, uint32_t epoch, int n_out,
-                                                 int n_rows, int tid) {
-    const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
-    const int group = rg.first_group;
-    const int wg_first = q4k_wg_of(group * rg.nb, rg.total, rg.n_wg);
-    const int wg_last = q4k_wg_of((group + 1) * rg.nb - 1, rg.total, rg.n_wg);
-    if (wg_first == wg_last || wg_last != static_cast<int>(blockIdx.x)) return;
-    const int orow = (group * kWavesQ4K + wave) * 16 + n;
-    if (orow >= n_out) return;
-    float4_t sum = {0, 0, 0, 0};
-    for (int wg = wg_first; wg <= wg_last; wg++) {
-        const int wg_first_group = static_cast<int>(static_cast<uint32_t>(rg.total) * wg / rg.n_wg / rg.nb);
-        const int slot = (group == wg_first_group) ? 0 : 1;
-        const Q4KTagged *p = partials + ((static_cast<size_t>(wg) * 2 + slot) * kWavesQ4K + wave) * 256;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint64_t *src = reinterpret_cast<const uint64_t *>(&p[(4 * g + i) * 16 + n]);
-            Q4KTagged t = __builtin_bit_cast(Q4KTagged, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            for (uint32_t spin = 0; t.tag != epoch && spin < kSpinLimit; spin++) {
-                __builtin_amdgcn_s_sleep(2);
-                t = __builtin_bit_cast(Q4KTagged, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            }
-            sum[i] += (t.tag == epoch) ? t.value : __builtin_nanf("");
-        }
+// Second kernel of a split-K call: one workgroup per output tile of every tile group that was
+// split over several workgroups of the streaming kernel; adds the partial tiles in workgroup
+// order (so sums are run-to-run deterministic) and writes Y.  Spreading this over the chip
+// instead of leaving it to the group's last contributor matters when K is long: a group then
+// has a dozen partial tiles.
+template <int kWaves>
+__global__ void __launch_bounds__(256)
+    q4k_reduce_kernel(const float *__restrict__ partials, float *__restrict__ y, int n_out, int nb, int n_rows,
+                      int n_groups, int n_wg) {
+    const int group = blockIdx.x / kWaves, wave = blockIdx.x % kWaves;
+    const int total = n_groups * nb;
+    const int wg_first = q4k_wg_of(group * nb, total, n_wg);
+    const int wg_last = q4k_wg_of((group + 1) * nb - 1, total, n_wg);
+    if (wg_first == wg_last) return;
+    const int e = threadIdx.x, m = e >> 4, n = e & 15;
+    const int orow = (group * kWaves + wave) * 16 + n;
+    if (m >= n_rows || orow >= n_out) return;
+    // a contributor's partial sits in slot 0 if its range starts inside this group (true for all
+    // but possibly the first contributor), else in slot 1
+    const int first_begin = static_cast<int>(static_cast<uint32_t>(total) * wg_first / n_wg);
+    const int first_slot = first_begin >= group * nb ? 0 : 1;
+    const size_t stride = static_cast<size_t>(2) * kWaves * 256;  // floats per workgroup
+    const float *p = partials + static_cast<size_t>(wave) * 256 + e;
+    float sum = p[wg_first * stride + static_cast<size_t>(first_slot) * kWaves * 256];
+    int wg = wg_first + 1;
+    for (; wg + 3 <= wg_last; wg += 4) {
+        const float a0 = p[wg * stride], a1 = p[(wg + 1) * stride], a2 = p[(wg + 2) * stride], a3 = p[(wg + 3) * stride];
+        sum = (((sum + a0) + a1) + a2) + a3;
     }
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-        if (4 * g + i < n_rows) y[static_cast<size_t>(4 * g + i) * n_out + orow] = sum[i];
+    for (; wg <= wg_last; wg++) sum += p[wg * stride];
+    y[static_cast<size_t>(m) * n_out + orow] = sum;
 }
 
-template <int kBufs>
-__global__ void __launch_bounds__(kThreadsQ4K)
-    gemm_q4k_stream_kernel(const uint8_t *__restrict__ w, const half8_t *__restrict__ xp, float *__restrict__ y,
-                           Q4KTagged *__restrict__ partials, uint32_t epoch, int n_out, int nb, int n_rows,
-                           int n_groups) {
-    extern __shared__ half8_t lds[];  // kBufs buffers of kBufPieces, then a 64-piece spare slot
-    half8_t *spare = lds + kBufs * kBufPieces;
+#ifdef DFLASH_TRACE
+// Debug build only: per-workgroup time stamps (100 MHz constant clock) of the streaming kernel.
+__device__ unsigned long long *g_trace = nullptr;  // [n_wg][16]
+#define DFL_TR(i)                                                                          \
+    do {                                                                                   \
+        if (threadIdx.x == 0 && g_trace) g_trace[blockIdx.x * 16 + (i)] = wall_clock64();  \
+    } while (0)
+#else
+#define DFL_TR(i) \
+    do {          \
+    } while (0)
+#endif
+
+template <int kWaves, typename XT>
+__global__ void __launch_bounds__(64 * kWaves)
+    gemm_q4k_stream_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
+                           float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups) {
+    using G = Q4KGeom<kWaves>;
+    extern __shared__ half8_t lds[];  // three buffers of kBufPieces
 
     const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    DFL_TR(0);
     Q4KRange rg;
     rg.nb = nb;
     rg.n_wg = gridDim.x;
@@ -439,58 +433,135 @@ __global__ void __launch_bounds__(kThreadsQ4K)
     rg.it_end = static_cast<int>(static_cast<uint32_t>(rg.total) * (blockIdx.x + 1) / rg.n_wg);
     if (rg.it_begin >= rg.it_end) return;
     rg.first_group = static_cast<int>(static_cast<uint32_t>(rg.it_begin) / static_cast<uint32_t>(nb));
-    const size_t row_bytes = static_cast<size_t>(nb) * DFL_Q4_K_BYTES;
+    const int b0 = rg.it_begin - rg.first_group * nb;
+    const uint32_t row_bytes = static_cast<uint32_t>(nb) * DFL_Q4_K_BYTES;
+    const uint32_t n_in = static_cast<uint32_t>(nb) * DFL_QK_K;
+    const size_t group_bytes = static_cast<size_t>(G::kRows) * row_bytes;
+    const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(x);
+    constexpr uint32_t kXBlockBytes = DFL_QK_K * sizeof(XT);
 
+    Q4KLane<kWaves> L;
+    q4k_lane_w_offsets<kWaves>(L, tid, rg.first_group * G::kRows, n_out, row_bytes);
+    q4k_lane_x_offsets<kWaves, XT>(L, tid, n_rows, n_in);
     float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0};
     const Q4KMagic magic = q4k_magic();
 
-    // prologue: kBufs - 1 stages in flight
-    int it_issue = rg.it_begin;  // next iteration to issue loads for
-    int issued = 0;              // stages issued so far
+    // Cursors.  Weights: wstage = first byte of the next stage to load in its group's first row,
+    // bw its super-block, gw its group, w_left the stages not loaded yet.  Activations run one
+    // stage further ahead: xblock / bx / x_left.
+    const uint8_t *wstage = w + static_cast<size_t>(rg.first_group) * group_bytes + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
+    int bw = b0, gw = rg.first_group, w_left = rg.it_end - rg.it_begin;
+    const uint8_t *xblock = xbytes + static_cast<size_t>(b0) * kXBlockBytes;
+    int bx = b0, x_left = w_left;
+    auto advance_w = [&]() {
+        wstage += DFL_Q4_K_BYTES;
+        w_left--;
+        if (++bw == nb) {
+            bw = 0;
+            gw++;
+            wstage += group_bytes - row_bytes;
+            if (w_left > 0 && (gw + 1) * G::kRows > n_out)  // ragged last group: re-clamp the rows
+                q4k_lane_w_offsets<kWaves>(L, tid, gw * G::kRows, n_out, row_bytes);
+        }
+    };
+    auto advance_x = [&]() {
+        xblock += kXBlockBytes;
+        x_left--;
+        if (++bx == nb) {
+            bx = 0;
+            xblock = xbytes;
+        }
+    };
+    auto issue_w_all = [&](half8_t *buf) {
 #pragma unroll
-    for (int s = 0; s < kBufs - 1; s++) {
-        if (it_issue < rg.it_end) {
-            int gi, bi, li;
-            q4k_stage_at(rg, it_issue, gi, bi, li);
-            q4k_issue_all(q4k_issue_desc(w, xp, lds + (issued % kBufs) * kBufPieces, spare, gi, bi, li, n_out,
-                                         row_bytes, true),
-                          tid);
-            it_issue += li;
-            issued++;
+        for (int j = 0; j < G::kFull; j++) q4k_issue_w<kWaves>(wstage, buf, L, j, wave);
+        if (wave < G::kExtra) q4k_issue_w<kWaves>(wstage, buf, L, G::kFull, wave);
+    };
+    half8_t *buf_c = lds, *buf_n = lds + G::kBufPieces, *buf_f = lds + 2 * G::kBufPieces;
+
+    // Prologue, in this order: activations of stages 0 and 1, weights of stage 0 | weights of
+    // stage 1, activations of stage 2.  From then on stage d issues one group [weights of d+2,
+    // activations of d+3], and "all but the youngest group have landed" is what the top of each
+    // stage waits for; young_w / young_x say what the youngest group holds.
+    Q4KXRaw<kWaves, XT> raw_first, raw_a, raw_b;  // activations of stage 0 / odd stages / even stages >= 2
+    bool young_w = false, young_x = false;
+    q4k_load_x<kWaves, XT>(xblock, L, raw_first);
+    advance_x();
+    if (x_left > 0) {
+        q4k_load_x<kWaves, XT>(xblock, L, raw_a);
+        advance_x();
+    }
+    issue_w_all(buf_c);
+    advance_w();
+    if (w_left > 0) {
+        issue_w_all(buf_n);
+        advance_w();
+        young_w = true;
+        if (x_left > 0) {
+            q4k_load_x<kWaves, XT>(xblock, L, raw_b);
+            advance_x();
+            young_x = true;
         }
     }
-    int it = rg.it_begin;
-    int done = 0;  // stages computed so far
-    while (it < rg.it_end) {
-        int gc, bc, lc;
-        q4k_stage_at(rg, it, gc, bc, lc);
-        // stage `done` has landed once at most (issued - done - 1) younger stages are in flight
-        if (issued - done - 1 >= kBufs - 2 && kBufs > 2)
-            __builtin_amdgcn_s_waitcnt(q4k_vmcnt((kBufs - 2) * kLoadsPerStage));
-        else
+    // the unused values of the minima fragments must be finite: zero them once (ordered before the
+    // first sums writes by a barrier that does not wait for the loads just issued)
+    for (int e = tid; e < 3 * 128; e += G::kThreads)
+        lds[(e >> 7) * G::kBufPieces + G::kWPieces + 512 + (e & 127)] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    __builtin_amdgcn_s_waitcnt(kWaitLds);
+    __builtin_amdgcn_s_barrier();
+    DFL_TR(1);
+    int gc = rg.first_group, bc = b0, n_left = rg.it_end - rg.it_begin;
+    bool first = true;
+    int done = 0;
+    // One stage; `raw` holds the activations of the next stage and is refilled with those three ahead.
+    auto stage = [&](Q4KXRaw<kWaves, XT> &raw) {
+        constexpr int kW0 = G::kFull, kW1 = G::kFull + 1, kX = G::kXLoads;
+        if (young_w && young_x) {
+            if (wave < G::kExtra)
+                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW1 + kX));
+            else
+                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW0 + kX));
+        } else if (young_w) {
+            if (wave < G::kExtra)
+                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW1));
+            else
+                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW0));
+        } else {
             __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
-        // A bare barrier, not __syncthreads(): that one carries a workgroup-scope fence, which waits
-        // for every load in flight and would undo the prefetch.  The s_waitcnt above is the only
-        // ordering this needs: each wave's own pieces have landed before it arrives here.
-        __builtin_amdgcn_s_barrier();  // the whole stage is in LDS; buffer (done-1) % kBufs is free
-        // the stage kBufs-1 ahead is loaded into that free buffer while this one is computed
-        const bool more = it_issue < rg.it_end;
-        int gi = gc, bi = bc, li = lc;
-        if (more) q4k_stage_at(rg, it_issue, gi, bi, li);
-        const Q4KIssue next =
-            q4k_issue_desc(w, xp, lds + (issued % kBufs) * kBufPieces, spare, gi, bi, li, n_out, row_bytes, more);
-        q4k_compute(lds + (done % kBufs) * kBufPieces, lc, tid, magic, acc, acc_min, next);
-        if (more) {
-            it_issue += li;
-            issued++;
         }
-        it += lc;
+        if (first) q4k_write_x<kWaves, XT>(buf_c, L, raw_first, n_rows == 16);
+        first = false;
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        // A bare barrier, not __syncthreads(): that one carries a workgroup-scope fence, which waits
+        // for every load in flight and would undo the prefetch.  The waits above are the only
+        // ordering this needs: each wave's own pieces have landed before it arrives here.
+        __builtin_amdgcn_s_barrier();  // stage d is complete in buf_c; buf_f (stage d-1) is free
+        const bool iw = w_left > 0, ix = x_left > 0;
+        q4k_compute<kWaves, XT>(buf_c, lane, wave, magic, acc, acc_min, iw, wstage, buf_f, ix, xblock, L, raw, n_left > 1,
+                                buf_n, n_rows == 16);
+        if (iw) advance_w();
+        if (ix) advance_x();
+        young_w = iw;
+        young_x = ix;
+        half8_t *t = buf_c;
+        buf_c = buf_n;
+        buf_n = buf_f;
+        buf_f = t;
+        n_left--;
         done++;
-        int gn = gc;
-        if (it < rg.it_end) gn = static_cast<int>(static_cast<uint32_t>(it) / static_cast<uint32_t>(nb));
-        if (it >= rg.it_end || gn != gc) q4k_flush(rg, gc, acc, acc_min, y, partials, epoch, n_out, n_rows, tid);
+        if (done <= 8) DFL_TR(1 + done);
+        if (++bc == nb || n_left == 0) {
+            q4k_flush<kWaves>(rg, gc, acc, acc_min, y, partials, n_out, n_rows, tid);
+            bc = 0;
+            gc++;
+        }
+    };
+    while (n_left > 0) {
+        stage(raw_a);
+        if (n_left == 0) break;
+        stage(raw_b);
     }
-    q4k_reduce_owned(rg, y, partials, epoch, n_out, n_rows, tid);
+    DFL_TR(13);
 }
 
 // ----------------------------------------------------------------------------
@@ -568,6 +639,17 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
     }
 }
 
+}  // namespace
+
+#ifdef DFLASH_TRACE
+extern "C" void dflash_dbg_set_trace(uint64_t p) {
+    unsigned long long *v = reinterpret_cast<unsigned long long *>(p);
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &v, sizeof(v));
+}
+#endif
+
+namespace {
+
 int env_int(const char *name, int fallback) {
     const char *v = getenv(name);
     return (v && *v) ? atoi(v) : fallback;
@@ -605,61 +687,62 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t n_steps = n_in / 32;
     size_t off = 0;
-    half8_t *xp = dfl_ws_take<half8_t>(ctx, &off, static_cast<size_t>(n_steps) * 64 * sizeof(half8_t));
     const int tiles = static_cast<int>((n_out + 15) / 16);
     const int target_waves = 8 * ctx->n_cu;
 
     if (w_type == DFLASH_TYPE_Q4_K) {
         const int nb = static_cast<int>(n_in / DFL_QK_K);
-        const int groups = (tiles + kWavesQ4K - 1) / kWavesQ4K;
+        if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
+            return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
+        // 16-wave workgroups (256 weight rows per stage) when that still leaves every CU a few
+        // stages of work, else 8-wave ones
+        int waves = (static_cast<int64_t>((tiles + 15) / 16) * nb >= 2ll * ctx->n_cu) ? 16 : 8;
+        waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
+        const int groups = (tiles + waves - 1) / waves;
         int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
         const int64_t total = static_cast<int64_t>(groups) * nb;
+        const int max_wgs = ctx->n_partial_wgs * 8 / waves;
         if (n_wg > total) n_wg = static_cast<int>(total);
-        if (n_wg > ctx->n_partial_wgs) n_wg = ctx->n_partial_wgs;
+        if (n_wg > max_wgs) n_wg = max_wgs;
         if (n_wg < 1) n_wg = 1;
-        if (total * (n_wg + 1) >= (int64_t(1) << 31))
+        if (total * (n_wg + 1) >= (int64_t(1) << 31) || row_bytes * 256 >= (size_t(1) << 32))
             return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: problem too large for 32-bit work indices");
-        off = 0;
-        xp = dfl_ws_take<half8_t>(ctx, &off, static_cast<size_t>(nb) * kQ4KBlockFrags * sizeof(half8_t));
-        if (!xp) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");
-        {
-            dfl_timed timer(ctx, st, DFL_T_PREP);
-            if (x_type == DFLASH_TYPE_F32)
-                prep_x_q4k_kernel<float><<<nb, 256, 0, st>>>(static_cast<const float *>(x), xp, n_rows, n_in);
-            else
-                prep_x_q4k_kernel<_Float16><<<nb, 256, 0, st>>>(static_cast<const _Float16 *>(x), xp, n_rows, n_in);
-        }
-        // three LDS buffers when the device has the full 160 KiB per workgroup, else two
-        const int bufs = env_int("DFLASH_GEMM_BUFS", ctx->lds_bytes >= (3 * kBufPieces + 64) * 16 ? 3 : 2);
-        const size_t lds = static_cast<size_t>(bufs * kBufPieces + 64) * sizeof(half8_t);
-        ctx->epoch += 1;
-        if (ctx->epoch == 0) ctx->epoch = 1;
-        Q4KTagged *partials = reinterpret_cast<Q4KTagged *>(ctx->tagged_partials);
-        dfl_timed timer(ctx, st, DFL_T_GEMM);
-        if (bufs == 3) {
-            static bool attr3 = false;
-            if (!attr3) {
-                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<3>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                       static_cast<int>(lds)));
-                attr3 = true;
-            }
-            gemm_q4k_stream_kernel<3><<<n_wg, kThreadsQ4K, lds, st>>>(static_cast<const uint8_t *>(w), xp, y, partials,
-                                                                      ctx->epoch, static_cast<int>(n_out), nb, n_rows,
-                                                                      groups);
-        } else {
-            static bool attr2 = false;
-            if (!attr2) {
-                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<2>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                       static_cast<int>(lds)));
-                attr2 = true;
-            }
-            gemm_q4k_stream_kernel<2><<<n_wg, kThreadsQ4K, lds, st>>>(static_cast<const uint8_t *>(w), xp, y, partials,
-                                                                      ctx->epoch, static_cast<int>(n_out), nb, n_rows,
-                                                                      groups);
-        }
+        float *partials = reinterpret_cast<float *>(ctx->tagged_partials);
+        const bool split = groups % n_wg != 0;  // else every range is a whole number of tile groups
+        const uint8_t *wb = static_cast<const uint8_t *>(w);
+        const int no = static_cast<int>(n_out);
+#define DFL_LAUNCH_Q4K(WAVES, XT)                                                                                      \
+    do {                                                                                                               \
+        const size_t lds = static_cast<size_t>(3 * Q4KGeom<WAVES>::kBufPieces) * sizeof(half8_t);                      \
+        if (lds > ctx->lds_bytes)                                                                                      \
+            return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: %zu bytes of LDS needed", lds);                 \
+        static bool attr = false;                                                                                      \
+        if (!attr) {                                                                                                   \
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<WAVES, XT>), \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+            attr = true;                                                                                               \
+        }                                                                                                              \
+        {                                                                                                              \
+            dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                      \
+            gemm_q4k_stream_kernel<WAVES, XT>                                                                          \
+                <<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, no, nb, n_rows, groups);  \
+        }                                                                                                              \
+        if (split) {                                                                                                   \
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                      \
+            q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg);       \
+        }                                                                                                              \
+    } while (0)
+        if (waves == 16 && x_type == DFLASH_TYPE_F32)
+            DFL_LAUNCH_Q4K(16, float);
+        else if (waves == 16)
+            DFL_LAUNCH_Q4K(16, _Float16);
+        else if (x_type == DFLASH_TYPE_F32)
+            DFL_LAUNCH_Q4K(8, float);
+        else
+            DFL_LAUNCH_Q4K(8, _Float16);
+#undef DFL_LAUNCH_Q4K
     } else {
+        half8_t *xp = dfl_ws_take<half8_t>(ctx, &off, static_cast<size_t>(n_steps) * 64 * sizeof(half8_t));
         if (!xp) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");
         unsigned prep_grid = static_cast<unsigned>((n_steps * 64 + 255) / 256);
         if (x_type == DFLASH_TYPE_F32)
