@@ -17,6 +17,10 @@ sys.path.insert(0, ROOT)
 METRIC = "accepted tokens/s @ batch1 block16; verify Q4_K GEMM HBM GB/s (% of peak)"
 SHAPES = [(5120, 17408), (17408, 5120), (5120, 6144)]  # (n_in, n_out)
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, averaged over the three shapes of a step: FETCH_SIZE + WRITE_SIZE from
+# two rocprofv3 --pmc runs of this file, each scaled by what the same counter reads for a plain 256 MiB copy
+# (profiles/gemm_q4k_stream_kernel__hbm_traffic.txt).  A counter figure, not measured by this run.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 52.03e6
 
 
 def cpu_baseline(shapes, weights, xs):
@@ -45,13 +49,49 @@ def cpu_baseline(shapes, weights, xs):
             "sample": f"first {int(rows_frac * 100)}% of the output rows of each of the 3 GEMMs, best of 3"}
 
 
+def rocprof_summary(directory):
+    """Text summary of a rocprofv3 CSV output directory: per-kernel durations from *_kernel_trace.csv and
+    per-kernel counter averages from *_counter_collection.csv (whichever exist)."""
+    import collections
+    import csv
+    import glob
+
+    for path in sorted(glob.glob(os.path.join(directory, "**", "*_kernel_trace.csv"), recursive=True)):
+        per = collections.defaultdict(list)
+        for r in csv.DictReader(open(path)):
+            name = r["Kernel_Name"].split("(")[0]
+            per[(name, r["Grid_Size_X"], r["Workgroup_Size_X"])].append(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
+        print(f"# {os.path.basename(path)}: kernel, grid, workgroup, launches, avg / min / median / max duration (us)")
+        for (name, grid, wg), d in sorted(per.items(), key=lambda kv: -sum(kv[1])):
+            d.sort()
+            print(f"{name[-72:]:72s} grid {grid:>8s} wg {wg:>5s} n {len(d):5d}  avg {sum(d) / len(d) / 1e3:8.2f}  "
+                  f"min {d[0] / 1e3:8.2f}  med {d[len(d) // 2] / 1e3:8.2f}  max {d[-1] / 1e3:8.2f}")
+    for path in sorted(glob.glob(os.path.join(directory, "**", "*_counter_collection.csv"), recursive=True)):
+        per = collections.defaultdict(lambda: collections.defaultdict(list))
+        for r in csv.DictReader(open(path)):
+            name = r["Kernel_Name"].split("(")[0]
+            per[(name, r.get("Grid_Size", r.get("Grid_Size_X", "")))][r["Counter_Name"]].append(float(r["Counter_Value"]))
+        print(f"# {os.path.basename(path)}: kernel, grid, dispatches, average counter value per dispatch")
+        for (name, grid), ctrs in sorted(per.items()):
+            vals = "  ".join(f"{c} {sum(v) / len(v):.1f}" for c, v in sorted(ctrs.items()))
+            n = max(len(v) for v in ctrs.values())
+            print(f"{name[-72:]:72s} grid {grid:>8s} n {n:4d}  {vals}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times (outside the timed region): the reference "
+                         "dispatch for scaling FETCH_SIZE / WRITE_SIZE counter readings")
+    ap.add_argument("--rocprof-summary", metavar="DIR", help="print a text summary of a rocprofv3 CSV output directory and exit")
     args = ap.parse_args()
+    if args.rocprof_summary:
+        rocprof_summary(args.rocprof_summary)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: the DFlash step is batch-1 and this build has no multi-GPU path; "
               "run with --gpus 1", file=sys.stderr)
@@ -80,6 +120,13 @@ def main():
         for (n_in, n_out), w, x, y in zip(SHAPES, wd, xd, yd):
             ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q4_K, x, y, n_in, n_out, 16)
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -125,7 +172,7 @@ def main():
                                "X f16 N(0,1), W Q4_K from N(0,0.02) seed 1, f32 accumulation",
                    "weight_bytes_per_step": sum(w_bytes), "block": 16, "batch": 1},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "gemm_q4k_stream_kernel", "bytes_per_launch": k_bytes, "us_per_launch": k_us},
         "shapes": per_shape,
         "pct_of_hbm_peak": 100.0 * sum(w_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
