@@ -49,6 +49,78 @@ def cpu_baseline(shapes, weights, xs):
             "sample": f"first {int(rows_frac * 100)}% of the output rows of each of the 3 GEMMs, best of 3"}
 
 
+def e2e_speculative(ctx, n_generate, sweep, log):
+    """End-to-end DFlash speculative decode on the 35B-A3B-shaped synthetic MoE target (40 layers, hidden 2048,
+    16 q / 2 kv heads of 256, 128 experts top-8 with F_exp 768 plus a shared expert; experts Q4_K, attention Q6_K,
+    vocabulary 151936) with a 5-layer drafter fed by 3 tapped layers, batch 1, block 16, prompt 2048, greedy accept.
+    Random-init weights: the drafter never agrees with the target by itself, so acceptance is forced: the target's
+    own serial greedy continuation replaces the first k drafts of every block, wrong tokens the rest (the drafter
+    still runs and is timed).  Margin fallback off (random-init logits are all near ties)."""
+    import numpy as np
+    import torch
+
+    import qwen_llm_amd as dfl
+
+    cfg = dfl.ModelConfig(n_layers=40, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=151936, n_expert=128,
+                          n_expert_used=8, ffn_expert=768, ffn_shared=768)
+    dcfg = dfl.DraftConfig(n_layers=5, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=6144, block_size=16, n_taps=3)
+    taps = [1, 19, 38]
+    prompt_len, cap = 2048, 2048 + n_generate + 64
+    t0 = time.perf_counter()
+    target = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_device(cfg, 0, "cuda"))
+    head = dfl.DraftHead(ctx, dcfg, dfl.synth_draft_weights_device(dcfg, 0, "cuda"))
+    torch.cuda.synchronize()
+    log(f"e2e: weights on device in {time.perf_counter() - t0:.1f} s "
+        f"({(target.weight_bytes() + head.weight_bytes()) / 1e9:.2f} GB)")
+    prompt = np.random.default_rng(0).integers(0, cfg.vocab - 1, prompt_len).tolist()
+    mask = cfg.vocab - 1
+
+    # the target's serial greedy continuation (token by token through the same kernels)
+    serial = dfl.Session(ctx, target, cap, taps)
+    t0 = time.perf_counter()
+    for s0 in range(0, prompt_len, 16):
+        out = serial.encode_packed_verify_layer_major(prompt[s0:s0 + 16], s0, want_hidden=False)
+    prefill_s = time.perf_counter() - t0
+    cont = [out.argmax_host[-1]]
+    t0 = time.perf_counter()
+    while len(cont) < n_generate + 16:
+        out = serial.encode_packed_verify_layer_major([cont[-1]], prompt_len + len(cont) - 1, want_hidden=False)
+        cont.append(out.argmax_host[0])
+    serial_s = time.perf_counter() - t0
+    serial.close()
+    res = {"prompt": prompt_len, "generated": n_generate, "prefill_tokens_per_s": prompt_len / prefill_s,
+           "serial_tokens_per_s": (len(cont) - 1) / serial_s, "weights_GB": (target.weight_bytes() + head.weight_bytes()) / 1e9,
+           "sweep": []}
+    log(f"e2e: prefill {res['prefill_tokens_per_s']:.0f} tok/s, serial decode {res['serial_tokens_per_s']:.1f} tok/s")
+    for k in sweep:
+        dec = dfl.SpeculativeDecoder(ctx, target, head, taps, cap, mask)
+        first = dec.prefill(prompt)
+
+        def override(tokens, position, k=k):
+            done = len(tokens)
+            good = cont[done:done + k]
+            bad = [(t + 1) % (cfg.vocab - 1) for t in cont[done + k:done + 15]]
+            return good + bad
+
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        tokens, st = dec.generate(first, n_generate, draft_override_fn=override)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        dec.close()
+        agree = sum(int(a == b) for a, b in zip(tokens, cont))
+        res["sweep"].append({
+            "forced_k": k, "accepted_tokens_per_s": (len(tokens) - 1) / dt, "steps": st["spec_steps"],
+            "mean_accept_len": st["accepted_drafts"] / max(st["spec_steps"], 1),
+            "mean_emitted_per_step": (len(tokens) - 1) / max(st["spec_steps"], 1),
+            "ms_per_step": dt * 1e3 / max(st["spec_steps"], 1),
+            "draft_ms": st["draft_ms"] / st["spec_steps"], "verify_ms": st["verify_ms"] / st["spec_steps"],
+            "accept_ms": st["accept_ms"] / st["spec_steps"], "append_ms": st["append_ms"] / st["spec_steps"],
+            "tokens_equal_serial_greedy": agree, "tokens": len(tokens)})
+        log(f"e2e: forced k={k}: {res['sweep'][-1]}")
+    return res
+
+
 def rocprof_summary(directory):
     """Text summary of a rocprofv3 CSV output directory: per-kernel durations from *_kernel_trace.csv and
     per-kernel counter averages from *_counter_collection.csv (whichever exist)."""
@@ -88,6 +160,8 @@ def main():
                     help="also run a plain 256 MiB device copy a few times (outside the timed region): the reference "
                          "dispatch for scaling FETCH_SIZE / WRITE_SIZE counter readings")
     ap.add_argument("--rocprof-summary", metavar="DIR", help="print a text summary of a rocprofv3 CSV output directory and exit")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end speculative decode measurement")
+    ap.add_argument("--e2e-tokens", type=int, default=1024)
     args = ap.parse_args()
     if args.rocprof_summary:
         rocprof_summary(args.rocprof_summary)
@@ -181,6 +255,16 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(SHAPES, weights, xs)
+    if not args.no_e2e:
+        del wd, xd, yd
+        try:
+            e2e = e2e_speculative(ctx, args.e2e_tokens, [7, 3, 15], lambda m: print(m, file=sys.stderr, flush=True))
+            out["e2e"] = e2e
+            out["accepted_tokens_per_s"] = e2e["sweep"][0]["accepted_tokens_per_s"]
+            out["config"]["e2e"] = ("35B-A3B-shaped MoE target (40 layers, 128 experts top-8, Q4_K experts, Q6_K attention, V 151936) "
+                                    "+ 5-layer drafter, prompt 2048, greedy accept, forced acceptance k=7 of 15 drafts")
+        except Exception as e:  # the GEMM line above stays valid
+            out["e2e_error"] = f"{type(e).__name__}: {e}"
     print(json.dumps(out))
 
 

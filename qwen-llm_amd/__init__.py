@@ -44,5 +44,7 @@ from .model import (  # noqa: F401,E402
     TargetModel,
     accept_greedy,
     synth_draft_weights,
+    synth_draft_weights_device,
+    synth_target_weights_device,
     synth_target_weights,
 )

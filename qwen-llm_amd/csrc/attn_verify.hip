@@ -44,7 +44,8 @@ template <int HD, typename TQ, int MAXW>
 __global__ void __launch_bounds__(64 * MAXW)
     attn_split_kernel(const TQ *__restrict__ q, const _Float16 *__restrict__ k_cache,
                       const _Float16 *__restrict__ vt_cache, float *__restrict__ part_o, float *__restrict__ part_ml,
-                      int64_t ctx_len, int n_rows, int n_q, int n_kv, int64_t vt_stride, int64_t chunk, float scale) {
+                      int64_t ctx_len, int n_rows, int n_q, int n_kv, int64_t vt_stride, int64_t chunk, float scale,
+                      int full_block, int64_t window) {
     constexpr int KS = HD / 32;  // k-steps of the score product
     constexpr int DT = HD / 16;  // 16-dim tiles of the output
     const int lane = threadIdx.x & 63;
@@ -79,7 +80,15 @@ __global__ void __launch_bounds__(64 * MAXW)
     for (int t = 0; t < DT; t++) acc[t] = float4_t{0, 0, 0, 0};
     float m_run = -INFINITY;  // running maximum of row n (base-2 logits), shared by its four lanes
     float l_run = 0.0f;       // this lane's share of the row sum
-    const int64_t row_limit = ctx_len + n;  // last visible key of row n
+    // visible keys of row n: [lo, hi].  Block-causal: everything up to the row's own position;
+    // full_block (drafter, non-causal): the whole block; a sliding window keeps |distance| < window.
+    const int64_t row_pos = ctx_len + n;
+    int64_t row_hi = full_block ? n_pos - 1 : row_pos;
+    int64_t row_lo = 0;
+    if (window > 0) {
+        row_lo = row_pos - window + 1;
+        row_hi = min(row_hi, row_pos + window - 1);
+    }
 
     const _Float16 *kbase = k_cache + static_cast<int64_t>(kvh) * HD + 8 * g;
     const _Float16 *vbase = vt_cache + static_cast<int64_t>(kvh) * HD * vt_stride;
@@ -101,14 +110,14 @@ __global__ void __launch_bounds__(64 * MAXW)
             }
             st[T] = s_acc;
         }
-        // mask: key visible to row n iff key <= ctx_len + n and key < c1
+        // mask: key visible to row n iff row_lo <= key <= row_hi and key < c1
         float p[8];
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const int64_t key = key0 + 8 * g + i;
             float v = (i < 4) ? st[0][i] : st[1][i - 4];
-            v = (key <= row_limit && key < c1) ? v : -INFINITY;
+            v = (key >= row_lo && key <= row_hi && key < c1) ? v : -INFINITY;
             p[i] = v;
             mx = fmaxf(mx, v);
         }
@@ -213,13 +222,15 @@ __global__ void __launch_bounds__(256) transpose_v_kernel(const _Float16 *__rest
 template <int HD, typename TQ>
 void launch_split(dim3 grid, int threads, hipStream_t st, const void *q, const _Float16 *k, const _Float16 *vt,
                   float *po, float *pml, int64_t ctx_len, int n_rows, int n_q, int n_kv, int64_t vt_stride,
-                  int64_t chunk, float scale) {
+                  int64_t chunk, float scale, int full_block, int64_t window) {
     if (threads <= 512)
         attn_split_kernel<HD, TQ, 8><<<grid, threads, 0, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, ctx_len,
-                                                               n_rows, n_q, n_kv, vt_stride, chunk, scale);
+                                                               n_rows, n_q, n_kv, vt_stride, chunk, scale, full_block,
+                                                               window);
     else
         attn_split_kernel<HD, TQ, 16><<<grid, threads, 0, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, ctx_len,
-                                                                n_rows, n_q, n_kv, vt_stride, chunk, scale);
+                                                                n_rows, n_q, n_kv, vt_stride, chunk, scale, full_block,
+                                                                window);
 }
 
 }  // namespace
@@ -228,6 +239,14 @@ extern "C" int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int3
                                             const void *v_cache, int32_t v_layout, int64_t ctx_len, int32_t n_rows,
                                             int32_t n_q, int32_t n_kv, int32_t head_dim, int64_t kv_capacity,
                                             float scale, float *out, dflash_stream_t stream) {
+    return dfl_attn_block(ctx, q, q_type, k_cache, v_cache, v_layout, ctx_len, n_rows, n_q, n_kv, head_dim, kv_capacity,
+                          scale, out, stream, 0, 0);
+}
+
+int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
+                       int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
+                       int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
+                       int64_t window) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!q || !k_cache || !v_cache || !out) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "attn_verify: null pointer");
     if (n_rows < 1 || n_rows > 16) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: n_rows %d outside 1..16", n_rows);
@@ -253,11 +272,11 @@ extern "C" int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int3
     const int64_t n_pos = ctx_len + n_rows;
 
     // KV splits: enough workgroups to cover the chip about twice, chunks a multiple of 32 keys
-    // and at least 256 keys long
+    // and at least 128 keys long (a split costs a partial tile per head and row)
     int64_t want = (2 * ctx->n_cu + n_kv - 1) / n_kv;
     int64_t chunk = (n_pos + want - 1) / want;
     chunk = (chunk + 31) / 32 * 32;
-    if (chunk < 256) chunk = 256;
+    if (chunk < 128) chunk = 128;
     const int n_splits = static_cast<int>((n_pos + chunk - 1) / chunk);
 
     size_t off = 0;
@@ -286,10 +305,10 @@ extern "C" int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int3
 #define DFL_ATTN(HD)                                                                                              \
     if (q_type == DFLASH_TYPE_F32)                                                                                \
         launch_split<HD, float>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, n_rows, n_q, n_kv, vt_stride, \
-                                chunk, scale);                                                                    \
+                                chunk, scale, full_block, window);                                                \
     else                                                                                                          \
         launch_split<HD, _Float16>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, n_rows, n_q, n_kv,      \
-                                   vt_stride, chunk, scale)
+                                   vt_stride, chunk, scale, full_block, window)
         if (head_dim == 64) {
             DFL_ATTN(64);
         } else if (head_dim == 128) {

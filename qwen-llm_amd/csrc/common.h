@@ -94,3 +94,10 @@ struct dfl_moe_scratch {
 // x_resid[n][hidden] += moe_ffn(cur[n][hidden]) for one layer; enqueue only.
 int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, const float *cur, int n,
                     const dfl_moe_scratch &scratch, float *x_resid, hipStream_t stream);
+
+// dflash_attn_verify_block with the drafter's masks: full_block != 0 lets every row see the whole
+// block (non-causal), window > 0 keeps only keys with |distance| < window.
+int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
+                       int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
+                       int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
+                       int64_t window);

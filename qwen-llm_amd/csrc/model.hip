@@ -160,6 +160,16 @@ __global__ void __launch_bounds__(64)
     for (int i = 0; i < per; i++) out[(static_cast<size_t>(row) * n_q + head) * hd + lane * per + i] = acc[i] / l;
 }
 
+// K/V rows f32 [m][kv_dim] -> f16 caches: K natural at row base + r, V transposed at column base + r
+__global__ void kv_to_f16_kernel(const float *__restrict__ k, const float *__restrict__ v, _Float16 *__restrict__ k16,
+                                 _Float16 *__restrict__ vt16, int kv_dim, int64_t cap16, int64_t base) {
+    const int row = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= kv_dim) return;
+    k16[(base + row) * kv_dim + e] = static_cast<_Float16>(k[static_cast<size_t>(row) * kv_dim + e]);
+    vt16[static_cast<size_t>(e) * cap16 + base + row] = static_cast<_Float16>(v[static_cast<size_t>(row) * kv_dim + e]);
+}
+
 template <typename T>
 bool dev_alloc(T **p, size_t count) {
     return hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T) + 256) == hipSuccess;
@@ -203,6 +213,11 @@ struct dflash_draft_session {
     float *ctx_raw = nullptr;  // [cap][n_taps*H] captured target hiddens
     float *ctx_h = nullptr;    // [cap][H]
     float *k_ctx = nullptr, *v_ctx = nullptr;  // [layer][cap][kv_dim]
+    // f16 mirror for the MFMA attention (used while the context positions are 0, 1, 2, ... and the
+    // block starts right behind them): K [layer][cap16][kv_dim], V transposed [layer][kv_dim][cap16]
+    _Float16 *k16 = nullptr, *vt16 = nullptr;
+    int64_t cap16 = 0;
+    bool contiguous = true;
     int32_t *pos_ctx = nullptr;                // [cap]
     float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
     float *g = nullptr, *u = nullptr, *logits = nullptr, *tmp = nullptr;
@@ -362,11 +377,14 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
     if (!s) return DFLASH_ERR_HIP;
     s->cfg = *cfg;
     s->capacity = ctx_capacity;
+    s->cap16 = (ctx_capacity + 16 + 31) / 32 * 32;
     s->vocab = vocab;
     const size_t H = cfg->hidden, kv_dim = static_cast<size_t>(cfg->n_kv) * cfg->head_dim,
                  q_dim = static_cast<size_t>(cfg->n_q) * cfg->head_dim, cap = ctx_capacity;
     bool ok = dev_alloc(&s->ctx_raw, cap * cfg->n_taps * H) && dev_alloc(&s->ctx_h, cap * H) &&
               dev_alloc(&s->k_ctx, cap * kv_dim * cfg->n_layers) && dev_alloc(&s->v_ctx, cap * kv_dim * cfg->n_layers) &&
+              dev_alloc(&s->k16, ((cap + 16 + 31) / 32 * 32) * kv_dim * cfg->n_layers) &&
+              dev_alloc(&s->vt16, ((cap + 16 + 31) / 32 * 32) * kv_dim * cfg->n_layers) &&
               dev_alloc(&s->pos_ctx, cap) && dev_alloc(&s->x, 16 * H) && dev_alloc(&s->cur, 16 * H) &&
               dev_alloc(&s->q, 16 * q_dim) && dev_alloc(&s->k, 16 * kv_dim) && dev_alloc(&s->v, 16 * kv_dim) &&
               dev_alloc(&s->attn, 16 * q_dim) && dev_alloc(&s->mix, 16 * H) && dev_alloc(&s->g, 16 * static_cast<size_t>(cfg->ffn)) &&
@@ -383,7 +401,7 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
 
 void dflash_draft_session_destroy(dflash_draft_session *s) {
     if (!s) return;
-    void *ptrs[] = {s->ctx_raw, s->ctx_h, s->k_ctx, s->v_ctx, s->pos_ctx, s->x, s->cur, s->q, s->k, s->v,
+    void *ptrs[] = {s->ctx_raw, s->ctx_h, s->k_ctx, s->v_ctx, s->k16, s->vt16, s->pos_ctx, s->x, s->cur, s->q, s->k, s->v,
                     s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -401,6 +419,8 @@ int32_t dflash_draft_append_ctx(dflash_ctx *ctx, dflash_draft_session *s, const 
         return dfl_fail(ctx, DFLASH_ERR_STATE, "append_ctx: %lld + %d columns exceed the context capacity %lld",
                         static_cast<long long>(s->ctx_len), n_cols, static_cast<long long>(s->capacity));
     if (n_cols == 0) return DFLASH_OK;
+    for (int i = 0; i < n_cols; i++)
+        if (positions[i] != s->ctx_len + i) s->contiguous = false;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const size_t feat = static_cast<size_t>(s->cfg.n_taps) * s->cfg.hidden;
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ctx_raw + s->ctx_len * feat, hidden_capture, n_cols * feat * sizeof(float),
@@ -427,6 +447,11 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
     const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
     const size_t feat = static_cast<size_t>(c.n_taps) * H;
     int32_t rc;
+    // MFMA attention over the f16 mirror when context column i sits at position i and the block
+    // starts at position ctx_len (the generation loop's case); else the general f32 kernel.  The
+    // mirror is only kept current while that holds, so leaving the fast path is final.
+    const bool fast = s->contiguous && noise_start == s->ctx_len && c.n_q / c.n_kv <= 16;
+    if (!fast) s->contiguous = false;
 
     // phase 1: fc + hidden_norm on the NEW context columns only (metal_dflash.rs:16045-16143)
     for (int64_t c0 = s->ctx_h_ready; c0 < s->ctx_len; c0 += 16) {
@@ -448,6 +473,8 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
         const dflash_draft_layer &L = head->layers[il];
         float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
         float *vc = s->v_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
+        _Float16 *k16 = s->k16 + il * static_cast<size_t>(s->cap16) * kv_dim;
+        _Float16 *vt16 = s->vt16 + il * static_cast<size_t>(s->cap16) * kv_dim;
         // context K/V for the delta only, normed and rotated at the columns' own positions
         for (int64_t c0 = s->kv_ready; c0 < s->ctx_len; c0 += 16) {
             const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
@@ -455,6 +482,9 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
             if ((rc = gemm(ctx, L.wv, s->ctx_h + c0 * H, vc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
             qk_norm_rope_kernel<<<dim3(c.n_kv, m), 64, 0, st>>>(nullptr, kc + c0 * kv_dim, nullptr, L.k_norm, nullptr,
                                                                s->pos_ctx + c0, 0, c.n_kv, hd, c.eps, c.rope_theta);
+            if (fast)
+                kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), m), 256, 0, st>>>(kc + c0 * kv_dim, vc + c0 * kv_dim, k16, vt16,
+                                                                              static_cast<int>(kv_dim), s->cap16, c0);
         }
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, L.attn_norm, s->cur, H, c.eps);
         if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, N, st))) return rc;
@@ -462,9 +492,19 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
         if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, N, st))) return rc;
         qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, nullptr, s->pos, c.n_q,
                                                                   c.n_kv, hd, c.eps, c.rope_theta);
-        draft_attn_kernel<<<dim3(c.n_q, N), 64, 0, st>>>(s->q, kc, vc, s->k, s->v, s->pos_ctx, static_cast<int>(s->ctx_len), N,
-                                                        c.n_q, c.n_kv, hd, static_cast<int>(noise_start), c.causal,
-                                                        L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
+        if (fast) {
+            // the block's own K/V go behind the context in the f16 mirror; one MFMA pass over both
+            kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), N), 256, 0, st>>>(s->k, s->v, k16, vt16, static_cast<int>(kv_dim),
+                                                                          s->cap16, s->ctx_len);
+            if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, k16, vt16, 1, s->ctx_len, N, c.n_q, c.n_kv, hd, s->cap16,
+                                     1.0f / sqrtf(static_cast<float>(hd)), s->attn, st, c.causal ? 0 : 1,
+                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0)))
+                return rc;
+        } else {
+            draft_attn_kernel<<<dim3(c.n_q, N), 64, 0, st>>>(s->q, kc, vc, s->k, s->v, s->pos_ctx, static_cast<int>(s->ctx_len),
+                                                            N, c.n_q, c.n_kv, hd, static_cast<int>(noise_start), c.causal,
+                                                            L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
+        }
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st))) return rc;
         add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, L.post_norm, s->cur, H, c.eps);

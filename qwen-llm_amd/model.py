@@ -187,6 +187,65 @@ def synth_draft_weights(cfg: DraftConfig, seed: int, wtype: int = synth.Q4_K, sw
     return w
 
 
+def _dev_mat(qtype, n_out, n_in, std, gen, device):
+    return (qtype, synth.random_blocks_device(qtype, n_out, n_in, std, gen, device))
+
+
+def synth_target_weights_device(cfg: ModelConfig, seed: int, device, wtype: int = synth.Q4_K, attn_type: int = synth.Q6_K,
+                                embd_type: int = synth.Q6_K):
+    """The same dictionary as synth_target_weights, but every matrix is generated on the device as random
+    quant blocks with scales chosen for N(0, 1/n_in)-like magnitudes (for timing large configurations: the host
+    quantiser would take minutes on tens of GB).  Not reproducible by the CPU checker's quantiser; use only where
+    results are compared between device paths."""
+    torch = _torch()
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    H, q_dim, kv_dim = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
+
+    def norm(n):
+        return 1.0 + 0.1 * torch.randn(n, generator=gen, device=device)
+
+    w = {"token_embd": _dev_mat(embd_type, cfg.vocab, H, 1.0, gen, device),
+         "output": _dev_mat(embd_type, cfg.vocab, H, H ** -0.5, gen, device), "output_norm": norm(H), "layers": []}
+    for _ in range(cfg.n_layers):
+        ffn = cfg.ffn_shared if cfg.n_expert else cfg.ffn
+        L = {"attn_norm": norm(H), "q_norm": norm(cfg.head_dim), "k_norm": norm(cfg.head_dim), "post_norm": norm(H),
+             "wq": _dev_mat(attn_type, q_dim, H, H ** -0.5, gen, device), "wk": _dev_mat(attn_type, kv_dim, H, H ** -0.5, gen, device),
+             "wv": _dev_mat(attn_type, kv_dim, H, H ** -0.5, gen, device), "wo": _dev_mat(attn_type, H, q_dim, q_dim ** -0.5, gen, device),
+             "gate": _dev_mat(wtype, ffn, H, H ** -0.5, gen, device), "up": _dev_mat(wtype, ffn, H, H ** -0.5, gen, device),
+             "down": _dev_mat(wtype, H, ffn, ffn ** -0.5, gen, device)}
+        if cfg.n_expert:
+            fe = cfg.ffn_expert
+            L["router"] = _dev_mat(synth.Q8_0, cfg.n_expert, H, H ** -0.5, gen, device)
+            L["shexp_gate"] = torch.randn(H, generator=gen, device=device) * H ** -0.5
+            L["gate_exps"] = _dev_mat(wtype, cfg.n_expert * fe, H, H ** -0.5, gen, device)
+            L["up_exps"] = _dev_mat(wtype, cfg.n_expert * fe, H, H ** -0.5, gen, device)
+            L["down_exps"] = _dev_mat(wtype, cfg.n_expert * H, fe, fe ** -0.5, gen, device)
+        w["layers"].append(L)
+    return w
+
+
+def synth_draft_weights_device(cfg: DraftConfig, seed: int, device, wtype: int = synth.Q4_K):
+    torch = _torch()
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed + 7919)
+    H, q_dim, kv_dim = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
+
+    def norm(n):
+        return 1.0 + 0.1 * torch.randn(n, generator=gen, device=device)
+
+    w = {"fc": _dev_mat(wtype, H, cfg.n_taps * H, (cfg.n_taps * H) ** -0.5, gen, device), "hidden_norm": norm(H),
+         "output_norm": norm(H), "layers": []}
+    for _ in range(cfg.n_layers):
+        w["layers"].append({
+            "attn_norm": norm(H), "q_norm": norm(cfg.head_dim), "k_norm": norm(cfg.head_dim), "post_norm": norm(H),
+            "wq": _dev_mat(wtype, q_dim, H, H ** -0.5, gen, device), "wk": _dev_mat(wtype, kv_dim, H, H ** -0.5, gen, device),
+            "wv": _dev_mat(wtype, kv_dim, H, H ** -0.5, gen, device), "wo": _dev_mat(wtype, H, q_dim, q_dim ** -0.5, gen, device),
+            "gate": _dev_mat(wtype, cfg.ffn, H, H ** -0.5, gen, device), "up": _dev_mat(wtype, cfg.ffn, H, H ** -0.5, gen, device),
+            "down": _dev_mat(wtype, H, cfg.ffn, cfg.ffn ** -0.5, gen, device), "is_swa": 0})
+    return w
+
+
 # ---- device-resident weights ----
 
 class _Uploader:
@@ -196,7 +255,10 @@ class _Uploader:
         self.keep = []
 
     def f32(self, a):
-        t = self.torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device)
+        if isinstance(a, self.torch.Tensor):
+            t = a.to(self.device, self.torch.float32).contiguous()
+        else:
+            t = self.torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device)
         self.keep.append(t)
         return t.data_ptr()
 
@@ -204,7 +266,10 @@ class _Uploader:
         if pair is None:
             return QTensorC(0, 0, None)
         qtype, blocks = pair
-        t = self.torch.from_numpy(np.ascontiguousarray(blocks)).to(self.device)
+        if isinstance(blocks, self.torch.Tensor):  # already resident (device-generated synthetic blocks)
+            t = blocks.to(self.device).contiguous()
+        else:
+            t = self.torch.from_numpy(np.ascontiguousarray(blocks)).to(self.device)
         self.keep.append(t)
         return QTensorC(int(qtype), 0, t.data_ptr())
 

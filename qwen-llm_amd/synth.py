@@ -153,3 +153,30 @@ def extreme_blocks(qtype: int, n_blocks: int, seed: int) -> np.ndarray:
         out[0::3, 2:] = 0x80
         out[1::3, 2:] = 0x7F
     return out
+
+
+def random_blocks_device(qtype: int, n_out: int, n_in: int, std: float, gen, device):
+    """[n_out, row_bytes] uint8 on `device`: random quant codes with super-block scales set so that the
+    dequantised weights have zero mean and roughly the standard deviation `std`.
+      Q4_K: codes uniform; w = d sc q - dmin m with dmin = 7.5 d  -> std(w) ~ 257 d
+      Q6_K: sub-block scales uniform in [-16, 16), q uniform      -> std(w) ~ 170 d
+      Q8_0: q uniform in [-128, 128)                              -> std(w) ~ 74 d"""
+    import torch
+
+    nblk = n_out * (n_in // BLOCK_ELEMS[qtype])
+    out = torch.randint(0, 256, (nblk, BLOCK_BYTES[qtype]), dtype=torch.uint8, device=device, generator=gen)
+
+    def f16_bytes(v):
+        return torch.tensor([v], dtype=torch.float16).view(torch.uint8).to(device)
+
+    if qtype == Q4_K:
+        d = std / 257.0
+        out[:, 0:2] = f16_bytes(d)
+        out[:, 2:4] = f16_bytes(7.5 * d)
+    elif qtype == Q6_K:
+        sc = torch.randint(-16, 16, (nblk, 16), dtype=torch.int8, device=device, generator=gen)
+        out[:, 192:208] = sc.view(torch.uint8)
+        out[:, 208:210] = f16_bytes(std / 170.0)
+    else:
+        out[:, 0:2] = f16_bytes(std / 74.0)
+    return out.view(n_out, -1)

@@ -198,3 +198,33 @@ def test_moe_verify_matches_oracle(ctx, oracle, name):
         close(out.logits.cpu().numpy(), lo, f"moe {name} logits n={n}")
         pos += n
     sess.close()
+
+
+def test_draft_block_general_positions(ctx, oracle, target):
+    """Context columns at arbitrary positions and a block that does not start right behind them: the
+    general f32 drafter attention (the MFMA path needs positions 0, 1, 2, ... and start == ctx_len)."""
+    model, (omodel, _keep) = target
+    dcfg = dfl.DraftConfig(**{**D1.as_dict(), "causal": 1, "swa_window": 12})
+    dw = dfl.synth_draft_weights(dcfg, seed=4, swa_layers=(0,))
+    head = dfl.DraftHead(ctx, dcfg, dw)
+    ohead, _k2 = oracle.build_draft_head(dcfg.as_dict(), dw)
+    rng = np.random.default_rng(41)
+    sess = dfl.Session(ctx, model, 64, TAPS)
+    ostate = oracle.TargetState(C1.as_dict(), 64)
+    dsess = dfl.DraftSession(ctx, head, model, 64)
+    toks = rng.integers(0, C1.vocab, 23).tolist()
+    hidden_o = []
+    for s in range(0, 23, 16):
+        blk = toks[s:s + 16]
+        out = sess.encode_packed_verify_layer_major(blk, s)
+        # every second column is given a position shifted by 3
+        dsess.append_target_ctx_columns(out.hidden_capture, [p + 3 * (p & 1) for p in range(s, s + len(blk))])
+        hidden_o.append(oracle.target_verify(omodel, ostate, blk, s, TAPS)[1])
+    pos_ctx = [p + 3 * (p & 1) for p in range(23)]
+    carry, start = 77, 29
+    argmax, logits, host = dsess.draft_block(carry, C1.vocab - 1, start, want_logits=True)
+    want = oracle.dflash_draft(omodel, ohead, [carry] + [C1.vocab - 1] * 15, np.concatenate(hidden_o).reshape(23, -1),
+                               pos_ctx, start)
+    close(logits.cpu().numpy(), want, "draft logits, general positions")
+    dsess.close()
+    sess.close()
