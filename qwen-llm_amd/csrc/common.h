@@ -85,8 +85,10 @@ struct dfl_moe_scratch {
     int32_t *sel_e = nullptr; // [16][n_used]
     float *sel_w = nullptr;   // [16][n_used]
     float *sg = nullptr;      // [16] shared-expert gate
-    float *act = nullptr;     // [16*n_used][ffn_expert]
-    float *eo = nullptr;      // [16*n_used][hidden]
+    float *act = nullptr;     // [16*n_used][ffn_expert]           (per-slot path)
+    float *eo = nullptr;      // [slots][16][hidden]; per-slot path: [16*n_used][hidden]
+    float *gate_out = nullptr, *up_out = nullptr;  // [slots][16][ffn_expert] (batched path)
+    int32_t *ids = nullptr, *n_distinct = nullptr, *slot_of = nullptr;  // distinct experts, their count, pick -> slot
     float *shared = nullptr;  // [16][hidden]
     float *g = nullptr, *u = nullptr;  // [16][ffn_shared]
 };
@@ -101,3 +103,12 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
                        int64_t window);
+
+// Few-row Q4_K GEMM over the matrices that the device-side list ids[0 .. *n_slots) picks out of a stack
+// (w_stack + id * w_stride_bytes): slot j reads activations x + j * x_stride (elements; 0 = shared) and
+// writes y + j * y_stride (floats) as [n_rows][n_out].  max_slots bounds *n_slots.  whole_groups != 0:
+// no split K (results independent of the other matrices in the batch).  Enqueue only.
+int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const int32_t *ids,
+                             const int32_t *n_slots, int max_slots, const void *x, int32_t x_type, size_t x_stride,
+                             float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
+                             int32_t whole_groups, dflash_stream_t stream);

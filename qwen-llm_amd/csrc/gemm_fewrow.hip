@@ -166,6 +166,23 @@ struct Q4KRange {
     int nb, n_wg, first_group;
 };
 
+// Batched mode (mixture-of-experts): the tile groups of several same-shaped matrices, picked out of
+// a stack by a device-side list, form one iteration space.  Global group index = slot *
+// groups_per_mat + local group; slot j uses matrix ids[j], activations x + j * x_stride and
+// output y + j * y_stride.  ids == nullptr: one matrix, one slot.
+struct Q4KBatch {
+    const int32_t *ids;      // [*n_slots] matrix index per slot
+    const int32_t *n_slots;  // device scalar
+    size_t w_stride;         // bytes between matrices of the stack
+    size_t x_stride;         // activation elements between slots (0: all slots share x)
+    size_t y_stride;         // output floats between slots
+    int groups_per_mat;
+    // Ranges are cut at tile-group boundaries only: no split K, so a (row, matrix) result does not
+    // depend on which other matrices take part (a verify block and a single-token pass then agree
+    // bit for bit), at the price of coarser load balance.
+    int whole_groups;
+};
+
 // Per-lane constants of the loads and of the activation write, set up once per kernel.
 template <int kWaves>
 struct Q4KLane {
@@ -343,18 +360,20 @@ constexpr int kWaitLds = 0xC07F;
 // Ends a tile group's segment: Y directly if this workgroup covered the group's whole K, else a
 // partial tile for the reduce kernel (slot 0: the range's first group, slot 1: its last).
 template <int kWaves>
-__device__ __forceinline__ void q4k_flush(const Q4KRange &rg, int group, float4_t &acc, float4_t &acc_min,
-                                          float *__restrict__ y, float *__restrict__ partials, int n_out, int n_rows,
-                                          int tid) {
+__device__ __forceinline__ void q4k_flush(const Q4KRange &rg, const Q4KBatch &bt, int group, float4_t &acc,
+                                          float4_t &acc_min, float *__restrict__ y, float *__restrict__ partials,
+                                          int n_out, int n_rows, int tid) {
     // rare path: an opaque copy of the thread index keeps its index arithmetic out of the stage loop
     asm volatile("" : "+v"(tid));
     const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
     float4_t res = acc - acc_min;
     acc = float4_t{0, 0, 0, 0};
     acc_min = float4_t{0, 0, 0, 0};
-    const int orow = (group * kWaves + wave) * 16 + n;
-    const int wg_first = q4k_wg_of(group * rg.nb, rg.total, rg.n_wg);
-    const int wg_last = q4k_wg_of((group + 1) * rg.nb - 1, rg.total, rg.n_wg);
+    const int slot_j = group / bt.groups_per_mat, lg = group - slot_j * bt.groups_per_mat;
+    y += static_cast<size_t>(slot_j) * bt.y_stride;
+    const int orow = (lg * kWaves + wave) * 16 + n;
+    const int wg_first = bt.whole_groups ? 0 : q4k_wg_of(group * rg.nb, rg.total, rg.n_wg);
+    const int wg_last = bt.whole_groups ? 0 : q4k_wg_of((group + 1) * rg.nb - 1, rg.total, rg.n_wg);
     if (wg_first == wg_last) {
         if (orow < n_out) {
 #pragma unroll
@@ -377,14 +396,19 @@ __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, int group, float4_
 template <int kWaves>
 __global__ void __launch_bounds__(256)
     q4k_reduce_kernel(const float *__restrict__ partials, float *__restrict__ y, int n_out, int nb, int n_rows,
-                      int n_groups, int n_wg) {
+                      int n_groups, int n_wg, Q4KBatch bt) {
     const int group = blockIdx.x / kWaves, wave = blockIdx.x % kWaves;
+    if (bt.ids) n_groups = bt.groups_per_mat * *bt.n_slots;
+    if (group >= n_groups) return;
+    if (n_wg > n_groups * nb) n_wg = n_groups * nb;
     const int total = n_groups * nb;
     const int wg_first = q4k_wg_of(group * nb, total, n_wg);
     const int wg_last = q4k_wg_of((group + 1) * nb - 1, total, n_wg);
     if (wg_first == wg_last) return;
     const int e = threadIdx.x, m = e >> 4, n = e & 15;
-    const int orow = (group * kWaves + wave) * 16 + n;
+    const int slot_j = group / bt.groups_per_mat, lg = group - slot_j * bt.groups_per_mat;
+    y += static_cast<size_t>(slot_j) * bt.y_stride;
+    const int orow = (lg * kWaves + wave) * 16 + n;
     if (m >= n_rows || orow >= n_out) return;
     // a contributor's partial sits in slot 0 if its range starts inside this group (true for all
     // but possibly the first contributor), else in slot 1
@@ -418,7 +442,7 @@ __device__ unsigned long long *g_trace = nullptr;  // [n_wg][16]
 template <int kWaves, typename XT>
 __global__ void __launch_bounds__(64 * kWaves)
     gemm_q4k_stream_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
-                           float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups) {
+                           float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt) {
     using G = Q4KGeom<kWaves>;
     extern __shared__ half8_t lds[];  // three buffers of kBufPieces
 
@@ -428,9 +452,19 @@ __global__ void __launch_bounds__(64 * kWaves)
     Q4KRange rg;
     rg.nb = nb;
     rg.n_wg = gridDim.x;
+    if (bt.ids) n_groups = bt.groups_per_mat * *bt.n_slots;  // how many matrices take part is decided on the device
     rg.total = n_groups * nb;
-    rg.it_begin = static_cast<int>(static_cast<uint32_t>(rg.total) * blockIdx.x / rg.n_wg);
-    rg.it_end = static_cast<int>(static_cast<uint32_t>(rg.total) * (blockIdx.x + 1) / rg.n_wg);
+    if (rg.n_wg > rg.total) rg.n_wg = rg.total;  // surplus workgroups leave
+    if (static_cast<int>(blockIdx.x) >= rg.n_wg) return;
+    if (bt.whole_groups) {
+        if (rg.n_wg > n_groups) rg.n_wg = n_groups;
+        if (static_cast<int>(blockIdx.x) >= rg.n_wg) return;
+        rg.it_begin = static_cast<int>(static_cast<uint32_t>(n_groups) * blockIdx.x / rg.n_wg) * nb;
+        rg.it_end = static_cast<int>(static_cast<uint32_t>(n_groups) * (blockIdx.x + 1) / rg.n_wg) * nb;
+    } else {
+        rg.it_begin = static_cast<int>(static_cast<uint32_t>(rg.total) * blockIdx.x / rg.n_wg);
+        rg.it_end = static_cast<int>(static_cast<uint32_t>(rg.total) * (blockIdx.x + 1) / rg.n_wg);
+    }
     if (rg.it_begin >= rg.it_end) return;
     rg.first_group = static_cast<int>(static_cast<uint32_t>(rg.it_begin) / static_cast<uint32_t>(nb));
     const int b0 = rg.it_begin - rg.first_group * nb;
@@ -440,8 +474,18 @@ __global__ void __launch_bounds__(64 * kWaves)
     const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(x);
     constexpr uint32_t kXBlockBytes = DFL_QK_K * sizeof(XT);
 
+    // first weight byte of a group's first row, its activations, and the local group index
+    auto group_w = [&](int group) {
+        const int j = group / bt.groups_per_mat, lg = group - j * bt.groups_per_mat;
+        const size_t mat = bt.ids ? static_cast<size_t>(bt.ids[j]) * bt.w_stride : 0;
+        return w + mat + static_cast<size_t>(lg) * group_bytes;
+    };
+    auto group_x = [&](int group) {
+        return xbytes + static_cast<size_t>(group / bt.groups_per_mat) * bt.x_stride * sizeof(XT);
+    };
+    auto group_local = [&](int group) { return group % bt.groups_per_mat; };
     Q4KLane<kWaves> L;
-    q4k_lane_w_offsets<kWaves>(L, tid, rg.first_group * G::kRows, n_out, row_bytes);
+    q4k_lane_w_offsets<kWaves>(L, tid, group_local(rg.first_group) * G::kRows, n_out, row_bytes);
     q4k_lane_x_offsets<kWaves, XT>(L, tid, n_rows, n_in);
     float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0};
     const Q4KMagic magic = q4k_magic();
@@ -449,19 +493,21 @@ __global__ void __launch_bounds__(64 * kWaves)
     // Cursors.  Weights: wstage = first byte of the next stage to load in its group's first row,
     // bw its super-block, gw its group, w_left the stages not loaded yet.  Activations run one
     // stage further ahead: xblock / bx / x_left.
-    const uint8_t *wstage = w + static_cast<size_t>(rg.first_group) * group_bytes + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
+    const uint8_t *wstage = group_w(rg.first_group) + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
     int bw = b0, gw = rg.first_group, w_left = rg.it_end - rg.it_begin;
-    const uint8_t *xblock = xbytes + static_cast<size_t>(b0) * kXBlockBytes;
-    int bx = b0, x_left = w_left;
+    const uint8_t *xblock = group_x(rg.first_group) + static_cast<size_t>(b0) * kXBlockBytes;
+    int bx = b0, gx = rg.first_group, x_left = w_left;
+    const bool ragged = bt.groups_per_mat * G::kRows > n_out;  // a matrix's last group has fewer rows
     auto advance_w = [&]() {
         wstage += DFL_Q4_K_BYTES;
         w_left--;
         if (++bw == nb) {
             bw = 0;
             gw++;
-            wstage += group_bytes - row_bytes;
-            if (w_left > 0 && (gw + 1) * G::kRows > n_out)  // ragged last group: re-clamp the rows
-                q4k_lane_w_offsets<kWaves>(L, tid, gw * G::kRows, n_out, row_bytes);
+            if (w_left > 0) {
+                wstage = group_w(gw);
+                if (ragged) q4k_lane_w_offsets<kWaves>(L, tid, group_local(gw) * G::kRows, n_out, row_bytes);
+            }
         }
     };
     auto advance_x = [&]() {
@@ -469,7 +515,8 @@ __global__ void __launch_bounds__(64 * kWaves)
         x_left--;
         if (++bx == nb) {
             bx = 0;
-            xblock = xbytes;
+            gx++;
+            if (x_left > 0) xblock = group_x(gx);
         }
     };
     auto issue_w_all = [&](half8_t *buf) {
@@ -551,7 +598,7 @@ __global__ void __launch_bounds__(64 * kWaves)
         done++;
         if (done <= 8) DFL_TR(1 + done);
         if (++bc == nb || n_left == 0) {
-            q4k_flush<kWaves>(rg, gc, acc, acc_min, y, partials, n_out, n_rows, tid);
+            q4k_flush<kWaves>(rg, bt, gc, acc, acc_min, y, partials, n_out, n_rows, tid);
             bc = 0;
             gc++;
         }
@@ -657,6 +704,87 @@ int env_int(const char *name, int fallback) {
 
 }  // namespace
 
+namespace {
+
+// Launches the streaming Q4_K kernel (and its split-K reduction): one matrix (batch == nullptr) or the
+// matrices a device-side list picks out of a stack (at most max_slots of them).
+int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in, int64_t n_out,
+                   int32_t n_rows, hipStream_t st, const Q4KBatch *batch, int max_slots) {
+    const int nb = static_cast<int>(n_in / DFL_QK_K);
+    const size_t row_bytes = static_cast<size_t>(nb) * DFL_Q4_K_BYTES;
+    const int tiles = static_cast<int>((n_out + 15) / 16);
+    if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
+    // 16-wave workgroups (256 weight rows per stage) when that still leaves every CU a few
+    // stages of work, else 8-wave ones
+    int waves = (static_cast<int64_t>((tiles + 15) / 16) * nb * max_slots >= 2ll * ctx->n_cu) ? 16 : 8;
+    waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
+    const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
+    const int groups = gpm * max_slots;           // upper bound in batched mode
+    int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
+    const int64_t total = static_cast<int64_t>(groups) * nb;
+    const int max_wgs = ctx->n_partial_wgs * 8 / waves;
+    if (n_wg > total) n_wg = static_cast<int>(total);
+    if (n_wg > max_wgs) n_wg = max_wgs;
+    if (n_wg < 1) n_wg = 1;
+    if (total * (n_wg + 1) >= (int64_t(1) << 31) || row_bytes * 256 >= (size_t(1) << 32))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: problem too large for 32-bit work indices");
+    float *partials = reinterpret_cast<float *>(ctx->tagged_partials);
+    // a single matrix whose ranges are whole tile groups needs no reduction; a batch always may
+    const bool split = batch ? !batch->whole_groups : groups % n_wg != 0;
+    Q4KBatch bt = {};
+    if (batch) bt = *batch;
+    bt.groups_per_mat = gpm;
+    const uint8_t *wb = static_cast<const uint8_t *>(w);
+    const int no = static_cast<int>(n_out);
+#define DFL_LAUNCH_Q4K(WAVES, XT)                                                                                      \
+    do {                                                                                                               \
+        const size_t lds = static_cast<size_t>(3 * Q4KGeom<WAVES>::kBufPieces) * sizeof(half8_t);                      \
+        if (lds > ctx->lds_bytes)                                                                                      \
+            return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: %zu bytes of LDS needed", lds);                 \
+        static bool attr = false;                                                                                      \
+        if (!attr) {                                                                                                   \
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<WAVES, XT>),  \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+            attr = true;                                                                                               \
+        }                                                                                                              \
+        {                                                                                                              \
+            dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                      \
+            gemm_q4k_stream_kernel<WAVES, XT><<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, \
+                                                                             no, nb, n_rows, groups, bt);              \
+        }                                                                                                              \
+        if (split) {                                                                                                   \
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                    \
+            q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);   \
+        }                                                                                                              \
+    } while (0)
+    if (waves == 16 && x_type == DFLASH_TYPE_F32)
+        DFL_LAUNCH_Q4K(16, float);
+    else if (waves == 16)
+        DFL_LAUNCH_Q4K(16, _Float16);
+    else if (x_type == DFLASH_TYPE_F32)
+        DFL_LAUNCH_Q4K(8, float);
+    else
+        DFL_LAUNCH_Q4K(8, _Float16);
+#undef DFL_LAUNCH_Q4K
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+}  // namespace
+
+int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const int32_t *ids,
+                             const int32_t *n_slots, int max_slots, const void *x, int32_t x_type, size_t x_stride,
+                             float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
+                             int32_t whole_groups, dflash_stream_t stream) {
+    if (n_in % DFL_QK_K || n_in <= 0 || n_out <= 0 || n_rows < 1 || n_rows > 16 || max_slots < 1)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_q4k_batched: bad shape");
+    if (reinterpret_cast<uintptr_t>(w_stack) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16)
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_q4k_batched: operand alignment");
+    Q4KBatch bt = {ids, n_slots, w_stride_bytes, x_stride, y_stride, 0, whole_groups};
+    return launch_q4k(ctx, w_stack, x, x_type, y, n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt, max_slots);
+}
+
 extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type,
                                       float *y, int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
@@ -691,56 +819,7 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
     const int target_waves = 8 * ctx->n_cu;
 
     if (w_type == DFLASH_TYPE_Q4_K) {
-        const int nb = static_cast<int>(n_in / DFL_QK_K);
-        if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
-            return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
-        // 16-wave workgroups (256 weight rows per stage) when that still leaves every CU a few
-        // stages of work, else 8-wave ones
-        int waves = (static_cast<int64_t>((tiles + 15) / 16) * nb >= 2ll * ctx->n_cu) ? 16 : 8;
-        waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
-        const int groups = (tiles + waves - 1) / waves;
-        int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
-        const int64_t total = static_cast<int64_t>(groups) * nb;
-        const int max_wgs = ctx->n_partial_wgs * 8 / waves;
-        if (n_wg > total) n_wg = static_cast<int>(total);
-        if (n_wg > max_wgs) n_wg = max_wgs;
-        if (n_wg < 1) n_wg = 1;
-        if (total * (n_wg + 1) >= (int64_t(1) << 31) || row_bytes * 256 >= (size_t(1) << 32))
-            return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: problem too large for 32-bit work indices");
-        float *partials = reinterpret_cast<float *>(ctx->tagged_partials);
-        const bool split = groups % n_wg != 0;  // else every range is a whole number of tile groups
-        const uint8_t *wb = static_cast<const uint8_t *>(w);
-        const int no = static_cast<int>(n_out);
-#define DFL_LAUNCH_Q4K(WAVES, XT)                                                                                      \
-    do {                                                                                                               \
-        const size_t lds = static_cast<size_t>(3 * Q4KGeom<WAVES>::kBufPieces) * sizeof(half8_t);                      \
-        if (lds > ctx->lds_bytes)                                                                                      \
-            return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: %zu bytes of LDS needed", lds);                 \
-        static bool attr = false;                                                                                      \
-        if (!attr) {                                                                                                   \
-            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<WAVES, XT>), \
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-            attr = true;                                                                                               \
-        }                                                                                                              \
-        {                                                                                                              \
-            dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                      \
-            gemm_q4k_stream_kernel<WAVES, XT>                                                                          \
-                <<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, no, nb, n_rows, groups);  \
-        }                                                                                                              \
-        if (split) {                                                                                                   \
-            dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                      \
-            q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg);       \
-        }                                                                                                              \
-    } while (0)
-        if (waves == 16 && x_type == DFLASH_TYPE_F32)
-            DFL_LAUNCH_Q4K(16, float);
-        else if (waves == 16)
-            DFL_LAUNCH_Q4K(16, _Float16);
-        else if (x_type == DFLASH_TYPE_F32)
-            DFL_LAUNCH_Q4K(8, float);
-        else
-            DFL_LAUNCH_Q4K(8, _Float16);
-#undef DFL_LAUNCH_Q4K
+        return launch_q4k(ctx, w, x, x_type, y, n_in, n_out, n_rows, st, nullptr, 1);
     } else {
         half8_t *xp = dfl_ws_take<half8_t>(ctx, &off, static_cast<size_t>(n_steps) * 64 * sizeof(half8_t));
         if (!xp) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");

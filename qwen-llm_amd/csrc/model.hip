@@ -252,7 +252,11 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
         const size_t used = std::min(cfg->n_expert_used, cfg->n_expert);
         ok = dev_alloc(&s->moe.probs, 16 * static_cast<size_t>(cfg->n_expert)) && dev_alloc(&s->moe.sel_e, 16 * used) &&
              dev_alloc(&s->moe.sel_w, 16 * used) && dev_alloc(&s->moe.sg, 16) &&
-             dev_alloc(&s->moe.act, 16 * used * cfg->ffn_expert) && dev_alloc(&s->moe.eo, 16 * used * cfg->hidden) &&
+             dev_alloc(&s->moe.act, 16 * used * cfg->ffn_expert) &&
+             dev_alloc(&s->moe.eo, 16 * std::min<size_t>(16 * used, cfg->n_expert) * cfg->hidden) &&
+             dev_alloc(&s->moe.gate_out, 16 * std::min<size_t>(16 * used, cfg->n_expert) * cfg->ffn_expert) &&
+             dev_alloc(&s->moe.up_out, 16 * std::min<size_t>(16 * used, cfg->n_expert) * cfg->ffn_expert) &&
+             dev_alloc(&s->moe.ids, cfg->n_expert) && dev_alloc(&s->moe.n_distinct, 1) && dev_alloc(&s->moe.slot_of, 16 * used) &&
              dev_alloc(&s->moe.shared, 16 * cfg->hidden);
         s->moe.g = s->g;
         s->moe.u = s->u;
@@ -270,7 +274,8 @@ void dflash_session_destroy(dflash_session *s) {
     if (!s) return;
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
                     s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax, s->hidden,
-                    s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared};
+                    s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared,
+                    s->moe.gate_out, s->moe.up_out, s->moe.ids, s->moe.n_distinct, s->moe.slot_of};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;

@@ -13,6 +13,8 @@
 #include "common.h"
 #include "device_quant.h"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr int kMaxSlots = 16;  // a row picks an expert at most once, and a block has at most 16 rows
@@ -169,6 +171,55 @@ __global__ void silu_mul_rows_kernel(float *__restrict__ g, const float *__restr
     }
 }
 
+// Distinct experts of the block, in ascending id order: ids[0 .. *n_distinct), and for every
+// (row, k) pick the index of its expert in that list.
+__global__ void __launch_bounds__(256)
+    moe_lists_kernel(const int32_t *__restrict__ sel_e, int n_picks, int n_expert, int32_t *__restrict__ ids,
+                     int32_t *__restrict__ n_distinct, int32_t *__restrict__ slot_of) {
+    extern __shared__ int32_t rank[];  // [n_expert]: 1 if picked, then its index in the list
+    for (int e = threadIdx.x; e < n_expert; e += blockDim.x) rank[e] = 0;
+    __syncthreads();
+    for (int s = threadIdx.x; s < n_picks; s += blockDim.x) rank[sel_e[s]] = 1;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int c = 0;
+        for (int e = 0; e < n_expert; e++) {
+            if (rank[e]) {
+                ids[c] = e;
+                rank[e] = c++;
+            }
+        }
+        *n_distinct = c;
+    }
+    __syncthreads();
+    for (int s = threadIdx.x; s < n_picks; s += blockDim.x) slot_of[s] = rank[sel_e[s]];
+}
+
+// g = silu(g) * u over the first *n_distinct slots of [slot][16][f]
+__global__ void silu_mul_slots_kernel(float *__restrict__ g, const float *__restrict__ u, const int32_t *__restrict__ n_distinct,
+                                      size_t per_slot) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= per_slot * static_cast<size_t>(*n_distinct)) return;
+    const float v = g[i];
+    g[i] = v / (1.0f + expf(-v)) * u[i];
+}
+
+// x[row] += sum_k w[row][k] * eo[slot_of[row][k]][row]  +  sg[row] * shared[row]
+__global__ void moe_combine_slots_kernel(const float *__restrict__ eo, const int32_t *__restrict__ slot_of,
+                                         const float *__restrict__ sel_w, const float *__restrict__ sg,
+                                         const float *__restrict__ shared, int n_used, int hidden, float *__restrict__ x) {
+    const int row = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= hidden) return;
+    float out = 0.0f;
+    for (int k = 0; k < n_used; k++) {
+        const size_t slot = slot_of[row * n_used + k];
+        out += sel_w[row * n_used + k] * eo[(slot * 16 + row) * hidden + i];
+    }
+    out += sg[row] * shared[static_cast<size_t>(row) * hidden + i];
+    x[static_cast<size_t>(row) * hidden + i] += out;
+}
+
 }  // namespace
 
 int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, const float *cur, int n,
@@ -191,32 +242,54 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     if (rc) return rc;
     moe_route_kernel<<<n, 64, E * sizeof(float), st>>>(s.probs, cur, L.shexp_gate, E, used, H, s.sel_e, s.sel_w, s.sg);
 
-    {
-        dim3 grid(1, E);  // x: 16 * (64 / LPR) output rows per workgroup
-        const int n_sub = H / 32;
-        if (n_sub <= 32) {
-            grid.x = (fe + 31) / 32;
-            moe_expert_kernel<true, 32><<<grid, 256, 0, st>>>(et, static_cast<const uint8_t *>(L.gate_exps.data),
-                                                             static_cast<const uint8_t *>(L.up_exps.data), rb_in, cur, s.sel_e,
-                                                             n_slots, used, H, fe, s.act);
-        } else {
-            grid.x = (fe + 15) / 16;
-            moe_expert_kernel<true, 64><<<grid, 256, 0, st>>>(et, static_cast<const uint8_t *>(L.gate_exps.data),
-                                                             static_cast<const uint8_t *>(L.up_exps.data), rb_in, cur, s.sel_e,
-                                                             n_slots, used, H, fe, s.act);
+    const bool batched = et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K && H % DFL_QK_K == 0 && fe % DFL_QK_K == 0 &&
+                         !getenv("DFLASH_MOE_PERSLOT");
+    if (batched) {
+        // the selected experts' matrices form one streaming GEMM each for gate, up and down: every
+        // distinct expert's weights are read once, with all block rows riding along on the MFMA;
+        // no split K, so a row's result is the same whichever other experts the block uses
+        const int max_slots = n_slots < E ? n_slots : E;
+        moe_lists_kernel<<<1, 256, E * sizeof(int32_t), st>>>(s.sel_e, n_slots, E, s.ids, s.n_distinct, s.slot_of);
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, static_cast<size_t>(fe) * rb_in, s.ids, s.n_distinct, max_slots, cur,
+                                       DFLASH_TYPE_F32, 0, s.gate_out, static_cast<size_t>(16) * fe, H, fe, n, 1, st)))
+            return rc;
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.up_exps.data, static_cast<size_t>(fe) * rb_in, s.ids, s.n_distinct, max_slots, cur,
+                                       DFLASH_TYPE_F32, 0, s.up_out, static_cast<size_t>(16) * fe, H, fe, n, 1, st)))
+            return rc;
+        const size_t per_slot = static_cast<size_t>(16) * fe;
+        silu_mul_slots_kernel<<<static_cast<unsigned>((per_slot * max_slots + 255) / 256), 256, 0, st>>>(s.gate_out, s.up_out,
+                                                                                                     s.n_distinct, per_slot);
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, static_cast<size_t>(H) * rb_dn, s.ids, s.n_distinct, max_slots,
+                                       s.gate_out, DFLASH_TYPE_F32, per_slot, s.eo, static_cast<size_t>(16) * H, fe, H, n, 1, st)))
+            return rc;
+    } else {
+        {
+            dim3 grid(1, E);  // x: 16 * (64 / LPR) output rows per workgroup
+            const int n_sub = H / 32;
+            if (n_sub <= 32) {
+                grid.x = (fe + 31) / 32;
+                moe_expert_kernel<true, 32><<<grid, 256, 0, st>>>(et, static_cast<const uint8_t *>(L.gate_exps.data),
+                                                                 static_cast<const uint8_t *>(L.up_exps.data), rb_in, cur, s.sel_e,
+                                                                 n_slots, used, H, fe, s.act);
+            } else {
+                grid.x = (fe + 15) / 16;
+                moe_expert_kernel<true, 64><<<grid, 256, 0, st>>>(et, static_cast<const uint8_t *>(L.gate_exps.data),
+                                                                 static_cast<const uint8_t *>(L.up_exps.data), rb_in, cur, s.sel_e,
+                                                                 n_slots, used, H, fe, s.act);
+            }
         }
-    }
-    {
-        dim3 grid(1, E);
-        const int n_sub = fe / 32;
-        if (n_sub <= 32) {
-            grid.x = (H + 31) / 32;
-            moe_expert_kernel<false, 32><<<grid, 256, 0, st>>>(dt, static_cast<const uint8_t *>(L.down_exps.data), nullptr, rb_dn,
-                                                              s.act, s.sel_e, n_slots, used, fe, H, s.eo);
-        } else {
-            grid.x = (H + 15) / 16;
-            moe_expert_kernel<false, 64><<<grid, 256, 0, st>>>(dt, static_cast<const uint8_t *>(L.down_exps.data), nullptr, rb_dn,
-                                                              s.act, s.sel_e, n_slots, used, fe, H, s.eo);
+        {
+            dim3 grid(1, E);
+            const int n_sub = fe / 32;
+            if (n_sub <= 32) {
+                grid.x = (H + 31) / 32;
+                moe_expert_kernel<false, 32><<<grid, 256, 0, st>>>(dt, static_cast<const uint8_t *>(L.down_exps.data), nullptr, rb_dn,
+                                                                  s.act, s.sel_e, n_slots, used, fe, H, s.eo);
+            } else {
+                grid.x = (H + 15) / 16;
+                moe_expert_kernel<false, 64><<<grid, 256, 0, st>>>(dt, static_cast<const uint8_t *>(L.down_exps.data), nullptr, rb_dn,
+                                                                  s.act, s.sel_e, n_slots, used, fe, H, s.eo);
+            }
         }
     }
     // shared expert: plain dense SwiGLU through the few-row GEMM
@@ -225,7 +298,11 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     const size_t nf = static_cast<size_t>(n) * fs;
     silu_mul_rows_kernel<<<static_cast<unsigned>((nf + 255) / 256), 256, 0, st>>>(s.g, s.u, nf);
     if ((rc = dflash_gemm_fewrow(ctx, L.down.type, L.down.data, s.g, DFLASH_TYPE_F32, s.shared, fs, H, n, st))) return rc;
-    moe_combine_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.sel_w, s.sg, s.shared, used, H, x_resid);
+    if (batched)
+        moe_combine_slots_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg, s.shared, used, H,
+                                                                         x_resid);
+    else
+        moe_combine_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.sel_w, s.sg, s.shared, used, H, x_resid);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

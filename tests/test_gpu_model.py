@@ -179,10 +179,14 @@ MOE_CASES = {
 }
 
 
-@pytest.mark.parametrize("name", list(MOE_CASES))
-def test_moe_verify_matches_oracle(ctx, oracle, name):
+@pytest.mark.parametrize("name,wtype", [("small", dfl.TYPE_Q4_K), ("wide", dfl.TYPE_Q4_K), ("small", dfl.TYPE_Q8_0)])
+def test_moe_verify_matches_oracle(ctx, oracle, name, wtype):
+    """Q4_K experts run as one batched streaming GEMM per projection; other types through the per-expert
+    f32 kernels.  Top-k routing is discontinuous: a row whose k-th and (k+1)-th expert probabilities are
+    closer than the activation error (1e-3) may pick a different expert than the f32 oracle, which
+    changes that whole row.  The seeds below have no such near tie in the rows compared."""
     cfg = MOE_CASES[name]
-    w = dfl.synth_target_weights(cfg, seed=23)
+    w = dfl.synth_target_weights(cfg, seed={"small": 23, "wide": 31}[name], wtype=wtype)
     model = dfl.TargetModel(ctx, cfg, w)
     omodel, _keep = oracle.build_model(cfg.as_dict(), w)
     taps = [0, 1]
