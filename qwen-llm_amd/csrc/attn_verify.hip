@@ -10,21 +10,24 @@
 //  * grid = (KV splits) x (KV heads); a workgroup owns one KV head and one contiguous chunk of
 //    key positions; each of its waves owns one query head of the GQA group, i.e. a 16-row tile
 //    (the block's rows are exactly the 16-wide side of v_mfma_f32_16x16x32_f16).
-//  * scores are computed transposed, S^T = K . Q^T: K rows are the A operand in their natural
-//    layout (a lane reads 16 contiguous bytes of a key), Q^T stays in registers for the whole
-//    kernel (pre-multiplied by scale*log2(e), rounded to f16 as the reference's decode kernel
-//    does, attn_v4.metal:20-31).  The result leaves every lane holding one query row and
-//    eight consecutive keys of a 32-key step, which is exactly the B operand of the second
-//    product O^T = V^T . P^T, so probabilities never move between lanes.
-//  * V is read through its transposed cache layout [kv head][dim][position]: the A operand of
-//    O^T wants 8 consecutive positions of one dim, 16 contiguous bytes there.
+//  * K and V stream HBM -> LDS once per workgroup in stages of 32 keys (direct-to-LDS loads into a
+//    ring of buffers, the next stages in flight while one is consumed), so the group's heads share
+//    one copy; the K tile is bank-swizzled on the way in so that MFMA operand reads are conflict-free.
+//  * scores are computed transposed, S^T = K . Q^T: K rows are the A operand, Q^T stays in
+//    registers for the whole kernel (pre-multiplied by scale*log2(e), rounded to f16 as the
+//    reference's decode kernel does, attn_v4.metal:20-31).  The result leaves every lane holding
+//    one query row and eight consecutive keys of the stage, which is exactly the B operand of the
+//    second product O^T = V^T . P^T, so probabilities never move between lanes.
+//  * V is cached transposed, [kv head][dim][position]: the A operand of O^T wants 8 consecutive
+//    positions of one dim, 16 contiguous bytes there.
 //  * online softmax in base 2 on the lanes' own values; the running maximum is shared by the
-//    four lanes of a row with two cross-lane exchanges per 32 keys, the accumulator rescale is
-//    skipped while no row's maximum moves.
+//    four lanes of a row with two cross-lane exchanges per stage, the accumulator rescale is
+//    skipped while no row's maximum moves, and stages every row sees in full skip the mask.
 //  * each workgroup writes (m, l, O) partials; a second small kernel merges the splits.
 #include "common.h"
 
 #include <cmath>
+#include <cstdlib>
 
 namespace {
 
@@ -39,164 +42,309 @@ __device__ __forceinline__ float xor_lane(float v, int mask) {
     return __shfl_xor(v, mask, 64);
 }
 
-// MAXW = most waves (query heads per KV head) a workgroup may have; it sets the register budget.
-template <int HD, typename TQ, int MAXW>
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+constexpr int kAttnBufs = 3;  // LDS ring: stages in flight + the one being consumed
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
+constexpr int attn_vmcnt(int n) { return ((n & 0xF) | ((n & 0x30) << 10)) | 0x0F70; }
+
+// bank swizzle of the K tile: 16-byte chunk j of key row r sits at chunk j ^ swz(r), so that the
+// eight key rows one MFMA operand read touches at a time land in eight different bank groups
+__device__ __forceinline__ int attn_swz(int r) { return (r & 3) | ((r >> 1) & 4); }
+
+// One workgroup = one KV head x one contiguous chunk of keys; wave w = query head w of the GQA
+// group.  Stage = 32 keys: the K tile [32 keys][HD] and the V^T tile [HD dims][32 keys] are copied
+// global -> LDS with direct-to-LDS loads into a ring of kAttnBufs buffers, so the whole group
+// shares one copy and the loads of the next stages are in flight while this one is consumed.
+// MAXW = most waves a workgroup may have; it sets the register budget.  HPW = query heads per wave:
+// with two, every K and V^T fragment read from LDS feeds two MFMAs (half the LDS traffic per head,
+// and two independent dependency chains per wave).
+template <int HD, typename TQ, int MAXW, int HPW>
 __global__ void __launch_bounds__(64 * MAXW)
     attn_split_kernel(const TQ *__restrict__ q, const _Float16 *__restrict__ k_cache,
                       const _Float16 *__restrict__ vt_cache, float *__restrict__ part_o, float *__restrict__ part_ml,
                       int64_t ctx_len, int n_rows, int n_q, int n_kv, int64_t vt_stride, int64_t chunk, float scale,
                       int full_block, int64_t window) {
-    constexpr int KS = HD / 32;  // k-steps of the score product
-    constexpr int DT = HD / 16;  // 16-dim tiles of the output
+    constexpr int KS = HD / 32;       // k-steps of the score product
+    constexpr int DT = HD / 16;       // 16-dim tiles of the output
+    constexpr int CH = HD / 8;        // 16-byte chunks per key row
+    constexpr int kKPieces = 32 * CH; // pieces of the K tile; the V^T tile has as many
+    constexpr int kWaveLoads = 2 * kKPieces / 64;
+    extern __shared__ half8_t lds[];  // kAttnBufs x (K tile, V^T tile)
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = blockDim.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int group = n_q / n_kv;
     const int kvh = blockIdx.y;
     const int split = blockIdx.x;
-    const int head = kvh * group + wave;
+    const int head0 = kvh * group + wave * HPW;  // this wave serves heads head0 .. head0 + HPW - 1
     const int64_t n_pos = ctx_len + n_rows;
     const int64_t c0 = split * chunk;
     const int64_t c1 = min(n_pos, c0 + chunk);
+    const int n_steps = static_cast<int>((c1 - c0 + 31) / 32);
     const int64_t kv_dim = static_cast<int64_t>(n_kv) * HD;
+    const int per_wave = (kWaveLoads + n_waves - 1) / n_waves;  // loads each wave issues per stage
+
+    const uint8_t *kbytes = reinterpret_cast<const uint8_t *>(k_cache + static_cast<int64_t>(kvh) * HD);
+    const uint8_t *vbytes = reinterpret_cast<const uint8_t *>(vt_cache + static_cast<int64_t>(kvh) * HD * vt_stride);
+    // Stage `st` (keys c0 + 32 st ..) into ring buffer st % kAttnBufs: wave-load qd covers LDS pieces
+    // 64 qd ..; this wave takes qd = j n_waves + wave, and loads past the end repeat earlier ones
+    // (same bytes to the same place) so that every wave issues per_wave loads.  Key rows at or past
+    // n_pos are never dereferenced: the last stage of the cache re-reads row n_pos - 1 instead (its
+    // scores are masked and its V columns zeroed below).
+    auto issue_stage = [&](int st) {
+        const int64_t key0 = c0 + 32ll * st;
+        half8_t *buf = lds + (st % kAttnBufs) * (2 * kKPieces);
+        for (int j = 0; j < per_wave; j++) {
+            const int qd = (j * n_waves + wave) % kWaveLoads;  // uniform
+            const int p = qd * 64 + lane;
+            const uint8_t *src;
+            if (qd * 64 < kKPieces) {
+                const int r = p / CH, jc = (p % CH) ^ attn_swz(r);
+                const int64_t key = min(key0 + r, n_pos - 1);
+                src = kbytes + key * kv_dim * 2 + jc * 16;
+            } else {
+                const int pv = p - kKPieces;
+                src = vbytes + ((static_cast<int64_t>(pv >> 2) * vt_stride + key0 + 8 * (pv & 3)) * 2);
+            }
+            __builtin_amdgcn_global_load_lds((gptr_t)(src), (lptr_t)(buf + qd * 64), 16, 0, 0);
+        }
+    };
+
+    // prologue: kAttnBufs - 1 stages in flight
+    int issued = 0;
+#pragma unroll
+    for (int st = 0; st < kAttnBufs - 1; st++) {
+        if (issued < n_steps) {
+            issue_stage(issued);
+            issued++;
+        }
+    }
 
     // Q^T fragments: lane (row n, g) holds Q[n][head][32 s + 8 g ..+8] * scale * log2(e)
-    half8_t qf[KS];
+    half8_t qf[HPW][KS];
     {
         const float mult = scale * kLog2e;
 #pragma unroll
-        for (int s = 0; s < KS; s++) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                float v = 0.0f;
-                if (n < n_rows) v = static_cast<float>(q[(static_cast<int64_t>(n) * n_q + head) * HD + 32 * s + 8 * g + i]);
-                qf[s][i] = static_cast<_Float16>(v * mult);
-            }
-        }
-    }
-
-    float4_t acc[DT];
-#pragma unroll
-    for (int t = 0; t < DT; t++) acc[t] = float4_t{0, 0, 0, 0};
-    float m_run = -INFINITY;  // running maximum of row n (base-2 logits), shared by its four lanes
-    float l_run = 0.0f;       // this lane's share of the row sum
-    // visible keys of row n: [lo, hi].  Block-causal: everything up to the row's own position;
-    // full_block (drafter, non-causal): the whole block; a sliding window keeps |distance| < window.
-    const int64_t row_pos = ctx_len + n;
-    int64_t row_hi = full_block ? n_pos - 1 : row_pos;
-    int64_t row_lo = 0;
-    if (window > 0) {
-        row_lo = row_pos - window + 1;
-        row_hi = min(row_hi, row_pos + window - 1);
-    }
-
-    const _Float16 *kbase = k_cache + static_cast<int64_t>(kvh) * HD + 8 * g;
-    const _Float16 *vbase = vt_cache + static_cast<int64_t>(kvh) * HD * vt_stride;
-
-    for (int64_t key0 = c0; key0 < c1; key0 += 32) {
-        // scores of 32 keys: tile T holds keys key0 + 8 (m / 4) + 4 T + (m % 4) in its row m, so
-        // that lane (n, g) ends up with keys key0 + 8 g .. + 7 (T = 0: first four, T = 1: last four)
-        float4_t st[2];
-#pragma unroll
-        for (int T = 0; T < 2; T++) {
-            int64_t key = key0 + 8 * (n >> 2) + 4 * T + (n & 3);
-            key = key < n_pos ? key : n_pos - 1;
-            const _Float16 *kp = kbase + key * kv_dim;
-            float4_t s_acc = {0, 0, 0, 0};
+        for (int h = 0; h < HPW; h++) {
 #pragma unroll
             for (int s = 0; s < KS; s++) {
-                half8_t kf = *reinterpret_cast<const half8_t *>(kp + 32 * s);
-                s_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[s], s_acc, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float v = 0.0f;
+                    if (n < n_rows)
+                        v = static_cast<float>(q[(static_cast<int64_t>(n) * n_q + head0 + h) * HD + 32 * s + 8 * g + i]);
+                    qf[h][s][i] = static_cast<_Float16>(v * mult);
+                }
             }
-            st[T] = s_acc;
         }
-        // mask: key visible to row n iff row_lo <= key <= row_hi and key < c1
-        float p[8];
-        float mx = -INFINITY;
+    }
+
+    float4_t acc[HPW][DT];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int64_t key = key0 + 8 * g + i;
-            float v = (i < 4) ? st[0][i] : st[1][i - 4];
-            v = (key >= row_lo && key <= row_hi && key < c1) ? v : -INFINITY;
-            p[i] = v;
-            mx = fmaxf(mx, v);
+    for (int h = 0; h < HPW; h++)
+#pragma unroll
+        for (int t = 0; t < DT; t++) acc[h][t] = float4_t{0, 0, 0, 0};
+    float m_run[HPW], l_run[HPW];  // running maximum of row n (base-2 logits, shared by its four lanes); this lane's share of the row sum
+#pragma unroll
+    for (int h = 0; h < HPW; h++) {
+        m_run[h] = -INFINITY;
+        l_run[h] = 0.0f;
+    }
+    // visible keys of row n, relative to c0: [lo, hi].  Block-causal: everything up to the row's own
+    // position; full_block (drafter, non-causal): the whole block; a window keeps |distance| < window.
+    const int64_t row_pos = ctx_len + n;
+    int64_t hi64 = full_block ? n_pos - 1 : row_pos;
+    int64_t lo64 = 0;
+    if (window > 0) {
+        lo64 = row_pos - window + 1;
+        hi64 = min(hi64, row_pos + window - 1);
+    }
+    hi64 = min(hi64, c1 - 1);
+    const int row_hi = static_cast<int>(max(min(hi64 - c0, static_cast<int64_t>(0x3fffffff)), static_cast<int64_t>(-1)));
+    const int row_lo = static_cast<int>(max(min(lo64 - c0, static_cast<int64_t>(0x3fffffff)), static_cast<int64_t>(0)));
+    // steps whose 32 keys are visible to every row need no masking: [all_lo, all_hi] in keys
+    int all_hi = row_hi, all_lo = row_lo;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        all_hi = min(all_hi, __shfl_xor(all_hi, off, 64));
+        all_lo = max(all_lo, __shfl_xor(all_lo, off, 64));
+    }
+    all_hi = __builtin_amdgcn_readfirstlane(all_hi);
+    all_lo = __builtin_amdgcn_readfirstlane(all_lo);
+
+    const int rk0 = 8 * (n >> 2) + (n & 3);  // key row of S^T tile 0 this lane's A operand reads
+    for (int st = 0; st < n_steps; st++) {
+        if (issued - st - 1 >= kAttnBufs - 2) {
+            // the loads of the kAttnBufs - 2 younger stages may still be in flight
+            switch (per_wave * (kAttnBufs - 2)) {
+                case 1: __builtin_amdgcn_s_waitcnt(attn_vmcnt(1)); break;
+                case 2: __builtin_amdgcn_s_waitcnt(attn_vmcnt(2)); break;
+                case 3: __builtin_amdgcn_s_waitcnt(attn_vmcnt(3)); break;
+                case 4: __builtin_amdgcn_s_waitcnt(attn_vmcnt(4)); break;
+                case 5: __builtin_amdgcn_s_waitcnt(attn_vmcnt(5)); break;
+                case 6: __builtin_amdgcn_s_waitcnt(attn_vmcnt(6)); break;
+                case 8: __builtin_amdgcn_s_waitcnt(attn_vmcnt(8)); break;
+                case 10: __builtin_amdgcn_s_waitcnt(attn_vmcnt(10)); break;
+                case 12: __builtin_amdgcn_s_waitcnt(attn_vmcnt(12)); break;
+                case 16: __builtin_amdgcn_s_waitcnt(attn_vmcnt(16)); break;
+                case 32: __builtin_amdgcn_s_waitcnt(attn_vmcnt(32)); break;
+                default: __builtin_amdgcn_s_waitcnt(attn_vmcnt(0)); break;
+            }
+        } else {
+            __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
         }
-        mx = fmaxf(mx, xor_lane(mx, 16));
-        mx = fmaxf(mx, xor_lane(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // all keys of this step masked for this row and nothing seen before: keep the state
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = exp2f(m_run - m_safe);  // 0 when m_run = -inf
-        float psum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            p[i] = exp2f(p[i] - m_safe);
-            psum += p[i];
+        __builtin_amdgcn_s_barrier();  // stage st is in LDS for everyone; buffer (st - 1) % kAttnBufs is free
+        if (issued < n_steps) {
+            issue_stage(issued);
+            issued++;
         }
-        l_run = l_run * alpha + psum;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        const half8_t *kt = lds + (st % kAttnBufs) * (2 * kKPieces);
+        const half8_t *vt = kt + kKPieces;
+        const int key0 = 32 * st;  // relative to c0
+
+        float4_t sc[HPW][2];
 #pragma unroll
-            for (int t = 0; t < DT; t++) acc[t] *= alpha;
+        for (int T = 0; T < 2; T++) {
+            const int r = rk0 + 4 * T;
+            const int sw = attn_swz(r);
+#pragma unroll
+            for (int h = 0; h < HPW; h++) sc[h][T] = float4_t{0, 0, 0, 0};
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const half8_t kf = kt[r * CH + ((4 * s + g) ^ sw)];
+#pragma unroll
+                for (int h = 0; h < HPW; h++) sc[h][T] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[h][s], sc[h][T], 0, 0, 0);
+            }
         }
-        m_run = m_new;
-        half8_t pf;
+        const bool masked = !(key0 >= all_lo && key0 + 31 <= all_hi);  // uniform: some key of this step is hidden from some row
+        half8_t pf[HPW];
 #pragma unroll
-        for (int i = 0; i < 8; i++) pf[i] = static_cast<_Float16>(p[i]);
-        // O^T tile t (dims 16 t ..): A = V^T[dim 16 t + n][keys key0 + 8 g ..+8]
-        const int64_t vkey = key0 + 8 * g;  // < vt_stride: the stride is a multiple of 32 and >= n_pos
-        // positions past the end of the cache hold whatever was there before (possibly NaN bit
-        // patterns), and 0 * NaN would poison the accumulator: zero them in the last step
-        const bool tail = key0 + 32 > n_pos;
+        for (int h = 0; h < HPW; h++) {
+            float p[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) p[i] = (i < 4) ? sc[h][0][i] : sc[h][1][i - 4];
+            if (masked) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int key = key0 + 8 * g + i;
+                    p[i] = (key >= row_lo && key <= row_hi) ? p[i] : -INFINITY;
+                }
+            }
+            float mx = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
+            mx = fmaxf(mx, xor_lane(mx, 16));
+            mx = fmaxf(mx, xor_lane(mx, 32));
+            const float m_new = fmaxf(m_run[h], mx);
+            // all keys of this step masked for this row and nothing seen before: keep the state
+            const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[h] - m_safe);  // 0 when m_run = -inf
+            float psum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                p[i] = __builtin_amdgcn_exp2f(p[i] - m_safe);
+                psum += p[i];
+            }
+            l_run[h] = l_run[h] * alpha + psum;
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+                for (int t = 0; t < DT; t++) acc[h][t] *= alpha;
+            }
+            m_run[h] = m_new;
+#pragma unroll
+            for (int i = 0; i < 8; i++) pf[h][i] = static_cast<_Float16>(p[i]);
+        }
+        // O^T tile t (dims 16 t ..): A = V^T[dim 16 t + n][keys key0 + 8 g ..+8].  Columns at or past
+        // n_pos hold whatever the cache held before (possibly NaN patterns; 0 * NaN would poison
+        // the accumulator): zero them in the last stage of the cache
+        const int64_t vkey = c0 + key0 + 8 * g;
+        const bool tail = c0 + key0 + 32 > n_pos;
 #pragma unroll
         for (int t = 0; t < DT; t++) {
-            half8_t vf = *reinterpret_cast<const half8_t *>(vbase + static_cast<int64_t>(16 * t + n) * vt_stride + vkey);
+            half8_t vf = vt[(16 * t + n) * 4 + g];
             if (tail) {
 #pragma unroll
                 for (int i = 0; i < 8; i++)
                     if (vkey + i >= n_pos) vf[i] = static_cast<_Float16>(0.0f);
             }
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, acc[t], 0, 0, 0);
+#pragma unroll
+            for (int h = 0; h < HPW; h++) acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[h], acc[h][t], 0, 0, 0);
         }
     }
 
-    // row sum over the four lanes of the row
-    l_run += xor_lane(l_run, 16);
-    l_run += xor_lane(l_run, 32);
-
-    // partials: O^T tile t, lane (row n, g) holds dims 16 t + 4 g + i
-    if (n < n_rows) {
-        const int64_t slot = (static_cast<int64_t>(split) * n_q + head) * 16 + n;
-        float *po = part_o + slot * HD;
+    // row sums over the four lanes of a row; partials: O^T tile t, lane (row n, g) holds dims 16 t + 4 g + i
 #pragma unroll
-        for (int t = 0; t < DT; t++) *reinterpret_cast<float4_t *>(po + 16 * t + 4 * g) = acc[t];
-        if (g == 0) {
-            part_ml[slot * 2] = m_run;
-            part_ml[slot * 2 + 1] = l_run;
+    for (int h = 0; h < HPW; h++) {
+        float l = l_run[h];
+        l += xor_lane(l, 16);
+        l += xor_lane(l, 32);
+        if (n < n_rows) {
+            const int64_t slot = (static_cast<int64_t>(split) * n_q + head0 + h) * 16 + n;
+            float *po = part_o + slot * HD;
+#pragma unroll
+            for (int t = 0; t < DT; t++) *reinterpret_cast<float4_t *>(po + 16 * t + 4 * g) = acc[h][t];
+            if (g == 0) {
+                part_ml[slot * 2] = m_run[h];
+                part_ml[slot * 2 + 1] = l;
+            }
         }
     }
 }
 
 // out[row][head][:] = sum_s 2^(m_s - m*) O_s / sum_s 2^(m_s - m*) l_s
+// One workgroup per (head, row): 256 threads = 8 split lanes x 32 dim lanes; a split lane adds up
+// every eighth split (float4 per dim lane, all loads independent), then the eight are summed in LDS.
 __global__ void __launch_bounds__(256)
     attn_combine_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml, float *__restrict__ out,
                         int n_rows, int n_q, int hd, int n_splits) {
+    __shared__ float wgt[1024];          // 2^(m_s - m*) per split (n_splits <= 1024)
+    __shared__ float red[8][256 + 4];    // partial outputs per split lane
+    __shared__ float red_l[8];
     const int head = blockIdx.x, row = blockIdx.y;
-    float m_star = -INFINITY;
-    for (int s = 0; s < n_splits; s++) {
-        const int64_t slot = (static_cast<int64_t>(s) * n_q + head) * 16 + row;
-        m_star = fmaxf(m_star, part_ml[slot * 2]);
+    const int tid = threadIdx.x;
+    const int64_t slot0 = static_cast<int64_t>(head) * 16 + row;
+    const int64_t slot_stride = static_cast<int64_t>(n_q) * 16;
+    // m* = max over splits
+    float m_loc = -INFINITY;
+    for (int s = tid; s < n_splits; s += 256) m_loc = fmaxf(m_loc, part_ml[(slot0 + s * slot_stride) * 2]);
+    for (int off = 32; off > 0; off >>= 1) m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off, 64));
+    if ((tid & 63) == 0) red_l[tid >> 6] = m_loc;
+    __syncthreads();
+    const float m_star = fmaxf(fmaxf(red_l[0], red_l[1]), fmaxf(red_l[2], red_l[3]));
+    __syncthreads();
+    for (int s = tid; s < n_splits; s += 256) {
+        const float m = part_ml[(slot0 + s * slot_stride) * 2];
+        wgt[s] = (m == -INFINITY) ? 0.0f : exp2f(m - m_star);
     }
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-        float o = 0.0f, l = 0.0f;
-        for (int s = 0; s < n_splits; s++) {
-            const int64_t slot = (static_cast<int64_t>(s) * n_q + head) * 16 + row;
-            const float m = part_ml[slot * 2];
-            if (m == -INFINITY) continue;
-            const float wgt = exp2f(m - m_star);
-            o += wgt * part_o[slot * hd + d];
-            l += wgt * part_ml[slot * 2 + 1];
-        }
-        out[(static_cast<int64_t>(row) * n_q + head) * hd + d] = o / l;
+    __syncthreads();
+    const int sl = tid >> 5, dl = tid & 31;  // split lane, dim lane
+    const int n_vec = hd / 4;                // float4 per row: 16, 32 or 64
+    float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+    float l = 0.0f;
+    for (int s = sl; s < n_splits; s += 8) {
+        const float w = wgt[s];
+        const float4_t *po = reinterpret_cast<const float4_t *>(part_o + (slot0 + s * slot_stride) * hd);
+        if (dl < n_vec) acc0 += w * po[dl];
+        if (dl + 32 < n_vec) acc1 += w * po[dl + 32];
+        if (dl == 0) l += w * part_ml[(slot0 + s * slot_stride) * 2 + 1];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        red[sl][4 * dl + i] = acc0[i];
+        red[sl][128 + 4 * dl + i] = acc1[i];
+    }
+    if (dl == 0) red_l[sl] = l;
+    __syncthreads();
+    float lsum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) lsum += red_l[k];
+    for (int d = tid; d < hd; d += 256) {
+        float o = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) o += red[k][d];
+        out[(static_cast<int64_t>(row) * n_q + head) * hd + d] = o / lsum;
     }
 }
 
@@ -223,14 +371,26 @@ template <int HD, typename TQ>
 void launch_split(dim3 grid, int threads, hipStream_t st, const void *q, const _Float16 *k, const _Float16 *vt,
                   float *po, float *pml, int64_t ctx_len, int n_rows, int n_q, int n_kv, int64_t vt_stride,
                   int64_t chunk, float scale, int full_block, int64_t window) {
+    const size_t lds = static_cast<size_t>(kAttnBufs) * 2 * (32 * HD / 8) * sizeof(half8_t);
+#define DFL_ATTN_LAUNCH(MAXW, HPW)                                                                                  \
+    do {                                                                                                            \
+        static bool attr = false;                                                                                   \
+        if (!attr) {                                                                                                \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_split_kernel<HD, TQ, MAXW, HPW>),         \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));          \
+            attr = true;                                                                                            \
+        }                                                                                                           \
+        attn_split_kernel<HD, TQ, MAXW, HPW><<<grid, threads / HPW, lds, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, \
+                                                                              ctx_len, n_rows, n_q, n_kv, vt_stride, \
+                                                                              chunk, scale, full_block, window);   \
+    } while (0)
+    // one head per wave: two (HPW = 2) halve the LDS reads per head but measured slower on MI355X
+    // (fewer waves to hide the per-stage dependency chain)
     if (threads <= 512)
-        attn_split_kernel<HD, TQ, 8><<<grid, threads, 0, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, ctx_len,
-                                                               n_rows, n_q, n_kv, vt_stride, chunk, scale, full_block,
-                                                               window);
+        DFL_ATTN_LAUNCH(8, 1);
     else
-        attn_split_kernel<HD, TQ, 16><<<grid, threads, 0, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, ctx_len,
-                                                                n_rows, n_q, n_kv, vt_stride, chunk, scale, full_block,
-                                                                window);
+        DFL_ATTN_LAUNCH(16, 1);
+#undef DFL_ATTN_LAUNCH
 }
 
 }  // namespace
@@ -271,9 +431,10 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     const int group = n_q / n_kv;
     const int64_t n_pos = ctx_len + n_rows;
 
-    // KV splits: enough workgroups to cover the chip about twice, chunks a multiple of 32 keys
+    // KV splits: enough workgroups to cover the chip once or twice, chunks a multiple of 32 keys
     // and at least 128 keys long (a split costs a partial tile per head and row)
-    int64_t want = (2 * ctx->n_cu + n_kv - 1) / n_kv;
+    const int per_cu = n_pos >= 16384 ? 2 : 1;  // short contexts: fewer splits, fewer partial tiles to merge
+    int64_t want = (static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv - 1) / n_kv;
     int64_t chunk = (n_pos + want - 1) / want;
     chunk = (chunk + 31) / 32 * 32;
     if (chunk < 128) chunk = 128;
@@ -318,8 +479,8 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
         }
 #undef DFL_ATTN
     }
-    attn_combine_kernel<<<dim3(n_q, n_rows), head_dim < 256 ? head_dim : 256, 0, st>>>(part_o, part_ml, out, n_rows, n_q,
-                                                                                   head_dim, n_splits);
+    if (n_splits > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: %d KV splits", n_splits);
+    attn_combine_kernel<<<dim3(n_q, n_rows), 256, 0, st>>>(part_o, part_ml, out, n_rows, n_q, head_dim, n_splits);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }
