@@ -164,7 +164,17 @@ __device__ __forceinline__ int q4k_wg_of(int it, int total, int n_wg) {
 struct Q4KRange {
     int total, it_begin, it_end;
     int nb, n_wg, first_group;
+    int wg;  // this workgroup's position in the range order (not its dispatch index)
 };
+
+// Range order.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2.
+// Consecutive ranges share weight rows (their boundary cache lines), activation blocks and
+// split-K partial tiles, so they are given to workgroups of the same XCD: dispatch index i
+// serves range (i mod 8) * (n / 8) + i / 8 when the count is a multiple of 8.
+__device__ __forceinline__ int q4k_range_index(int dispatch, int n_wg) {
+    if (n_wg % 8) return dispatch;
+    return (dispatch & 7) * (n_wg >> 3) + (dispatch >> 3);
+}
 
 // Batched mode (mixture-of-experts): the tile groups of several same-shaped matrices, picked out of
 // a stack by a device-side list, form one iteration space.  Global group index = slot *
@@ -383,7 +393,7 @@ __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, const Q4KBatch &bt
         return;
     }
     const int slot = (group == rg.first_group) ? 0 : 1;
-    float *p = partials + ((static_cast<size_t>(blockIdx.x) * 2 + slot) * kWaves + wave) * 256;
+    float *p = partials + ((static_cast<size_t>(rg.wg) * 2 + slot) * kWaves + wave) * 256;
 #pragma unroll
     for (int i = 0; i < 4; i++) p[(4 * g + i) * 16 + n] = res[i];
 }
@@ -459,11 +469,13 @@ __global__ void __launch_bounds__(64 * kWaves)
     if (bt.whole_groups) {
         if (rg.n_wg > n_groups) rg.n_wg = n_groups;
         if (static_cast<int>(blockIdx.x) >= rg.n_wg) return;
-        rg.it_begin = static_cast<int>(static_cast<uint32_t>(n_groups) * blockIdx.x / rg.n_wg) * nb;
-        rg.it_end = static_cast<int>(static_cast<uint32_t>(n_groups) * (blockIdx.x + 1) / rg.n_wg) * nb;
+        rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
+        rg.it_begin = static_cast<int>(static_cast<uint32_t>(n_groups) * rg.wg / rg.n_wg) * nb;
+        rg.it_end = static_cast<int>(static_cast<uint32_t>(n_groups) * (rg.wg + 1) / rg.n_wg) * nb;
     } else {
-        rg.it_begin = static_cast<int>(static_cast<uint32_t>(rg.total) * blockIdx.x / rg.n_wg);
-        rg.it_end = static_cast<int>(static_cast<uint32_t>(rg.total) * (blockIdx.x + 1) / rg.n_wg);
+        rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
+        rg.it_begin = static_cast<int>(static_cast<uint32_t>(rg.total) * rg.wg / rg.n_wg);
+        rg.it_end = static_cast<int>(static_cast<uint32_t>(rg.total) * (rg.wg + 1) / rg.n_wg);
     }
     if (rg.it_begin >= rg.it_end) return;
     rg.first_group = static_cast<int>(static_cast<uint32_t>(rg.it_begin) / static_cast<uint32_t>(nb));
