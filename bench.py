@@ -49,6 +49,72 @@ def cpu_baseline(shapes, weights, xs):
             "sample": f"first {int(rows_frac * 100)}% of the output rows of each of the 3 GEMMs, best of 3"}
 
 
+def attention_section(ctx):
+    """Block-causal verify attention, 16 query rows after L keys, 48 q / 8 kv heads of 128, f16 K/V resident in HBM
+    (V in the transposed cache layout): microseconds per call and KV-stream GB/s = (L + 16) * 8 * 128 * 2 * 2 B / time."""
+    import math
+
+    import torch
+
+    out = []
+    n_rows, n_q, n_kv, hd = 16, 48, 8, 128
+    for L in (4096, 32768, 131072):
+        cap = (L + n_rows + 31) // 32 * 32
+        g = torch.Generator(device="cuda")
+        g.manual_seed(10)
+        q = torch.randn((n_rows, n_q, hd), device="cuda", generator=g).half()
+        k = torch.randn((cap, n_kv, hd), device="cuda", generator=g).half()
+        vt = torch.randn((n_kv, hd, cap), device="cuda", generator=g).half()
+        o = torch.empty((n_rows, n_q, hd), device="cuda")
+        scale = 1.0 / math.sqrt(hd)
+        for _ in range(5):
+            ctx.attn_verify_block(q, k, vt, L, scale, v_transposed=True, out=o)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(30):
+            ctx.attn_verify_block(q, k, vt, L, scale, v_transposed=True, out=o)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / 30 * 1e3
+        kv_bytes = (L + n_rows) * n_kv * hd * 2 * 2
+        out.append({"context": L, "us_per_call": us, "kv_bytes": kv_bytes, "GBps": kv_bytes / (us * 1e-6) / 1e9,
+                    "frac_of_hbm_peak": kv_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS})
+        del q, k, vt, o
+    return out
+
+
+def acceptance_section(ctx):
+    """Stochastic acceptance of one block: vocabulary 151936, 15 drafts + bonus, target logits N(0,3), draft = target +
+    N(0,0.5), T 0.7 / top-p 0.95 / top-k 20, vocabulary-wide draft distribution (temperature 0.7), Philox stream.
+    Time per block (device kernels + the host-side decision read-back) and logits bytes / time."""
+    import torch
+
+    import qwen_llm_amd as dfl
+
+    vocab, n = 151936, 16
+    g = torch.Generator(device="cuda")
+    g.manual_seed(4)
+    target = torch.randn((n, vocab), device="cuda", generator=g) * 3.0
+    draft = target[: n - 1] + 0.5 * torch.randn((n - 1, vocab), device="cuda", generator=g)
+    toks = [int(t) for t in torch.argmax(target, dim=1).tolist()]
+    verified = [toks[0]] + [int(t) for t in torch.argmax(draft, dim=1).tolist()]
+    times, accepted = [], 0
+    for trial in range(24):
+        samp = dfl.Sampler(temperature=0.7, top_k=20, top_p=0.95, min_p=0.0, seed=trial, rng_kind=dfl.RNG_PHILOX)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        d = ctx.decide_dflash_accept_prefix(verified, target, vocab, None, samp, 1000, [], draft_logits=draft,
+                                            draft_temperature=0.7)
+        times.append(time.perf_counter() - t0)
+        accepted += len(d.accepted_drafts)
+    times = sorted(times[4:])
+    us = times[len(times) // 2] * 1e6
+    logits_bytes = (2 * n - 1) * vocab * 4
+    return {"vocab": vocab, "block": n, "us_per_block": us, "logits_bytes": logits_bytes,
+            "GBps": logits_bytes / (us * 1e-6) / 1e9, "mean_accepted": accepted / 24}
+
+
 def e2e_speculative(ctx, n_generate, sweep, log):
     """End-to-end DFlash speculative decode on the 35B-A3B-shaped synthetic MoE target (40 layers, hidden 2048,
     16 q / 2 kv heads of 256, 128 experts top-8 with F_exp 768 plus a shared expert; experts Q4_K, attention Q6_K,
@@ -255,8 +321,13 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(SHAPES, weights, xs)
+    del wd, xd, yd
+    try:
+        out["attention"] = attention_section(ctx)
+        out["acceptance"] = acceptance_section(ctx)
+    except Exception as e:  # the GEMM line above stays valid
+        out["sections_error"] = f"{type(e).__name__}: {e}"
     if not args.no_e2e:
-        del wd, xd, yd
         try:
             e2e = e2e_speculative(ctx, args.e2e_tokens, [7, 3, 15], lambda m: print(m, file=sys.stderr, flush=True))
             out["e2e"] = e2e
