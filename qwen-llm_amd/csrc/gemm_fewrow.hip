@@ -698,6 +698,102 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
     }
 }
 
+// ----------------------------------------------------------------------------
+// Q6_K kernel: half a super-block (128 weights of a row) per lane group and step
+// ----------------------------------------------------------------------------
+//
+// A wave owns a 16-row tile and a run of half super-blocks; lane (n, g) serves weight row n and, in
+// each of the half's four 32-element quarters, the eight weights 8 g .. 8 g + 7.  ggml's Q6_K packing
+// (ql[128], qh[64], int8 scales[16], f16 d; metal/tests/q6_k_f32_tile.rs:46-71) makes those 32 weights
+// come from just three 8-byte runs (two of ql, one of qh), eight scale bytes and d, so a lane issues
+// five loads per four MFMAs.  Blocks are 210 bytes, so these loads are only 2-byte aligned; gfx950
+// runs with unaligned vector memory access enabled and the compiler emits them as single loads.
+// Activations are read from the caller's matrix and rounded to f16 on the fly (all tiles read the
+// same rows: L2 hits).  Waves of a workgroup split K and add their tiles up in LDS in wave order.
+__device__ __forceinline__ uint64_t load_u64_unaligned(const uint8_t *p) {
+    uint64_t v;
+    __builtin_memcpy(&v, p, 8);
+    return v;
+}
+
+template <typename XT>
+__device__ __forceinline__ half8_t load_x8(const XT *p, bool live);
+template <>
+__device__ __forceinline__ half8_t load_x8<float>(const float *p, bool live) {
+    half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (live) {
+        const float4_t a = *reinterpret_cast<const float4_t *>(p), b = *reinterpret_cast<const float4_t *>(p + 4);
+        r = half8_t{static_cast<_Float16>(a[0]), static_cast<_Float16>(a[1]), static_cast<_Float16>(a[2]),
+                    static_cast<_Float16>(a[3]), static_cast<_Float16>(b[0]), static_cast<_Float16>(b[1]),
+                    static_cast<_Float16>(b[2]), static_cast<_Float16>(b[3])};
+    }
+    return r;
+}
+template <>
+__device__ __forceinline__ half8_t load_x8<_Float16>(const _Float16 *p, bool live) {
+    half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (live) r = *reinterpret_cast<const half8_t *>(p);
+    return r;
+}
+
+template <typename XT>
+__global__ void __launch_bounds__(64 * kMaxSplit)
+    gemm_q6k_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y, int n_out, int nb,
+                    size_t row_bytes, int n_rows, int n_split) {
+    extern __shared__ float red[];  // [n_split][256]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int row = min(n0 + n, n_out - 1);
+    const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
+    const int n_half = 2 * nb;
+    const int h0 = n_half * wave / n_split, h1 = n_half * (wave + 1) / n_split;
+    const bool x_live = n < n_rows;  // lane (m = n, g) of the A operand: activation row n
+    const XT *xrow = x + static_cast<size_t>(x_live ? n : 0) * (static_cast<size_t>(nb) * DFL_QK_K) + 8 * g;
+    float4_t acc = {0, 0, 0, 0};
+    for (int hb = h0; hb < h1; hb++) {
+        const uint8_t *blk = rowp + static_cast<size_t>(hb >> 1) * DFL_Q6_K_BYTES;
+        const int half = hb & 1;
+        const uint64_t qa = load_u64_unaligned(blk + 64 * half + 8 * g);
+        const uint64_t qb = load_u64_unaligned(blk + 64 * half + 32 + 8 * g);
+        const uint64_t qh = load_u64_unaligned(blk + 128 + 32 * half + 8 * g);
+        const uint64_t sc = load_u64_unaligned(blk + 192 + 8 * half);
+        const float d = half_at(blk + 208);
+        const XT *xk = xrow + static_cast<size_t>(hb) * 128;
+#pragma unroll
+        for (int kq = 0; kq < 4; kq++) {
+            const int is = (g >> 1) + 2 * kq;
+            const float ds = d * static_cast<float>(static_cast<int8_t>(sc >> (8 * is)));
+            const float off = -32.0f * ds;
+            const uint64_t src = (kq & 1) ? qb : qa;
+            const uint64_t lo = ((kq & 2) ? (src >> 4) : src) & 0x0F0F0F0F0F0F0F0Full;
+            const uint64_t hi = ((qh >> (2 * kq)) & 0x0303030303030303ull) << 4;
+            const uint64_t q = lo | hi;
+            const uint32_t q0 = static_cast<uint32_t>(q), q1 = static_cast<uint32_t>(q >> 32);
+            half8_t b;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                b[i] = static_cast<_Float16>(__builtin_fmaf(static_cast<float>((q0 >> (8 * i)) & 0xffu), ds, off));
+                b[4 + i] = static_cast<_Float16>(__builtin_fmaf(static_cast<float>((q1 >> (8 * i)) & 0xffu), ds, off));
+            }
+            const half8_t a = load_x8<XT>(xk + 32 * kq, x_live);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) red[wave * 256 + (4 * g + i) * 16 + n] = acc[i];
+    __syncthreads();
+    for (int e = threadIdx.x; e < 256; e += blockDim.x) {
+        int m = e >> 4, nn = e & 15;
+        if (m < n_rows && n0 + nn < n_out) {
+            float sum = 0.0f;
+            for (int ws = 0; ws < n_split; ws++) sum += red[ws * 256 + e];
+            y[static_cast<size_t>(m) * n_out + n0 + nn] = sum;
+        }
+    }
+}
+
 }  // namespace
 
 #ifdef DFLASH_TRACE
@@ -832,6 +928,24 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
 
     if (w_type == DFLASH_TYPE_Q4_K) {
         return launch_q4k(ctx, w, x, x_type, y, n_in, n_out, n_rows, st, nullptr, 1);
+    } else if (w_type == DFLASH_TYPE_Q6_K) {
+        if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
+            return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
+        const int nb = static_cast<int>(n_in / DFL_QK_K);
+        int split = (target_waves + tiles - 1) / tiles;
+        split = env_int("DFLASH_GEMM_NSPLIT", split);
+        if (split > 2 * nb) split = 2 * nb;
+        if (split > kMaxSplit) split = kMaxSplit;
+        if (split < 1) split = 1;
+        const size_t lds = static_cast<size_t>(split) * 256 * sizeof(float);
+        const uint8_t *wb = static_cast<const uint8_t *>(w);
+        dfl_timed timer(ctx, st, DFL_T_GEMM);
+        if (x_type == DFLASH_TYPE_F32)
+            gemm_q6k_kernel<float><<<tiles, 64 * split, lds, st>>>(wb, static_cast<const float *>(x), y, static_cast<int>(n_out),
+                                                                  nb, row_bytes, n_rows, split);
+        else
+            gemm_q6k_kernel<_Float16><<<tiles, 64 * split, lds, st>>>(wb, static_cast<const _Float16 *>(x), y,
+                                                                     static_cast<int>(n_out), nb, row_bytes, n_rows, split);
     } else {
         half8_t *xp = dfl_ws_take<half8_t>(ctx, &off, static_cast<size_t>(n_steps) * 64 * sizeof(half8_t));
         if (!xp) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");
@@ -850,12 +964,8 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
         size_t lds = static_cast<size_t>(split) * 256 * sizeof(float);
         const uint8_t *wb = static_cast<const uint8_t *>(w);
         dfl_timed timer(ctx, st, DFL_T_GEMM);
-        if (w_type == DFLASH_TYPE_Q6_K)
-            gemm_generic_kernel<DFLASH_TYPE_Q6_K>
-                <<<tiles, 64 * split, lds, st>>>(wb, xp, y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
-        else
-            gemm_generic_kernel<DFLASH_TYPE_Q8_0>
-                <<<tiles, 64 * split, lds, st>>>(wb, xp, y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
+        gemm_generic_kernel<DFLASH_TYPE_Q8_0>
+            <<<tiles, 64 * split, lds, st>>>(wb, xp, y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
     }
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
