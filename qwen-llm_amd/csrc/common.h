@@ -105,10 +105,11 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
                        int64_t window);
 
 // Few-row Q4_K GEMM over the matrices that the device-side list ids[0 .. *n_slots) picks out of a stack
-// (w_stack + id * w_stride_bytes): slot j reads activations x + j * x_stride (elements; 0 = shared) and
+// (w_stack + id * w_stride_bytes; id -1 = extra_w): slot j reads activations x + j * x_stride (elements; 0 = shared) and
 // writes y + j * y_stride (floats) as [n_rows][n_out].  max_slots bounds *n_slots.  whole_groups != 0:
 // no split K (results independent of the other matrices in the batch).  Enqueue only.
-int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const int32_t *ids,
-                             const int32_t *n_slots, int max_slots, const void *x, int32_t x_type, size_t x_stride,
+int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const void *extra_w,
+                             const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
+                             size_t x_stride,
                              float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
                              int32_t whole_groups, dflash_stream_t stream);

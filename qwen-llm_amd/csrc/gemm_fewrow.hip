@@ -181,7 +181,8 @@ __device__ __forceinline__ int q4k_range_index(int dispatch, int n_wg) {
 // groups_per_mat + local group; slot j uses matrix ids[j], activations x + j * x_stride and
 // output y + j * y_stride.  ids == nullptr: one matrix, one slot.
 struct Q4KBatch {
-    const int32_t *ids;      // [*n_slots] matrix index per slot
+    const int32_t *ids;      // [*n_slots] matrix index per slot; -1 = the extra matrix
+    const uint8_t *extra_w;  // a same-shaped matrix outside the stack (may be null if no id is -1)
     const int32_t *n_slots;  // device scalar
     size_t w_stride;         // bytes between matrices of the stack
     size_t x_stride;         // activation elements between slots (0: all slots share x)
@@ -489,8 +490,12 @@ __global__ void __launch_bounds__(64 * kWaves)
     // first weight byte of a group's first row, its activations, and the local group index
     auto group_w = [&](int group) {
         const int j = group / bt.groups_per_mat, lg = group - j * bt.groups_per_mat;
-        const size_t mat = bt.ids ? static_cast<size_t>(bt.ids[j]) * bt.w_stride : 0;
-        return w + mat + static_cast<size_t>(lg) * group_bytes;
+        const uint8_t *mat = w;
+        if (bt.ids) {
+            const int32_t id = bt.ids[j];
+            mat = id < 0 ? bt.extra_w : w + static_cast<size_t>(id) * bt.w_stride;
+        }
+        return mat + static_cast<size_t>(lg) * group_bytes;
     };
     auto group_x = [&](int group) {
         return xbytes + static_cast<size_t>(group / bt.groups_per_mat) * bt.x_stride * sizeof(XT);
@@ -881,15 +886,16 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
 
 }  // namespace
 
-int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const int32_t *ids,
-                             const int32_t *n_slots, int max_slots, const void *x, int32_t x_type, size_t x_stride,
+int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const void *extra_w,
+                             const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
+                             size_t x_stride,
                              float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
                              int32_t whole_groups, dflash_stream_t stream) {
     if (n_in % DFL_QK_K || n_in <= 0 || n_out <= 0 || n_rows < 1 || n_rows > 16 || max_slots < 1)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_q4k_batched: bad shape");
-    if (reinterpret_cast<uintptr_t>(w_stack) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16)
+    if (reinterpret_cast<uintptr_t>(w_stack) % 16 || reinterpret_cast<uintptr_t>(extra_w) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16)
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_q4k_batched: operand alignment");
-    Q4KBatch bt = {ids, n_slots, w_stride_bytes, x_stride, y_stride, 0, whole_groups};
+    Q4KBatch bt = {ids, static_cast<const uint8_t *>(extra_w), n_slots, w_stride_bytes, x_stride, y_stride, 0, whole_groups};
     return launch_q4k(ctx, w_stack, x, x_type, y, n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt, max_slots);
 }
 

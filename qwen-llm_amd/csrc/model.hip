@@ -253,10 +253,10 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
         ok = dev_alloc(&s->moe.probs, 16 * static_cast<size_t>(cfg->n_expert)) && dev_alloc(&s->moe.sel_e, 16 * used) &&
              dev_alloc(&s->moe.sel_w, 16 * used) && dev_alloc(&s->moe.sg, 16) &&
              dev_alloc(&s->moe.act, 16 * used * cfg->ffn_expert) &&
-             dev_alloc(&s->moe.eo, 16 * std::min<size_t>(16 * used, cfg->n_expert) * cfg->hidden) &&
-             dev_alloc(&s->moe.gate_out, 16 * std::min<size_t>(16 * used, cfg->n_expert) * cfg->ffn_expert) &&
-             dev_alloc(&s->moe.up_out, 16 * std::min<size_t>(16 * used, cfg->n_expert) * cfg->ffn_expert) &&
-             dev_alloc(&s->moe.ids, cfg->n_expert) && dev_alloc(&s->moe.n_distinct, 1) && dev_alloc(&s->moe.slot_of, 16 * used) &&
+             dev_alloc(&s->moe.eo, 16 * (std::min<size_t>(16 * used, cfg->n_expert) + 1) * cfg->hidden) &&
+             dev_alloc(&s->moe.gate_out, 16 * (std::min<size_t>(16 * used, cfg->n_expert) + 1) * cfg->ffn_expert) &&
+             dev_alloc(&s->moe.up_out, 16 * (std::min<size_t>(16 * used, cfg->n_expert) + 1) * cfg->ffn_expert) &&
+             dev_alloc(&s->moe.ids, cfg->n_expert + 1) && dev_alloc(&s->moe.n_distinct, 1) && dev_alloc(&s->moe.slot_of, 16 * used) &&
              dev_alloc(&s->moe.shared, 16 * cfg->hidden);
         s->moe.g = s->g;
         s->moe.u = s->u;

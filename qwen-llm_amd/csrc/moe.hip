@@ -19,62 +19,62 @@ namespace {
 
 constexpr int kMaxSlots = 16;  // a row picks an expert at most once, and a block has at most 16 rows
 
-// One wave per block row: softmax, top-k, renormalised weights, shared-expert gate.
-__global__ void __launch_bounds__(64)
+// One workgroup per block row, one thread per expert (n_expert <= 1024): softmax, top-k by rank
+// (an expert's rank = how many experts beat it: higher probability, or equal and lower id), the
+// renormalised weights in pick order, and the shared-expert gate.
+__global__ void __launch_bounds__(1024)
     moe_route_kernel(const float *__restrict__ logits, const float *__restrict__ x, const float *__restrict__ shexp_gate,
                      int n_expert, int n_used, int hidden, int32_t *__restrict__ sel_e, float *__restrict__ sel_w,
                      float *__restrict__ sg) {
     extern __shared__ float probs[];  // [n_expert]
+    __shared__ float red[16];
     __shared__ float pick_w[64];
-    const int row = blockIdx.x, lane = threadIdx.x;
-    const float *lr = logits + static_cast<size_t>(row) * n_expert;
-    float mx = -INFINITY;
-    for (int e = lane; e < n_expert; e += 64) mx = fmaxf(mx, lr[e]);
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
+    const float logit = tid < n_expert ? logits[static_cast<size_t>(row) * n_expert + tid] : -INFINITY;
+    float mx = logit;
     for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-    float sum = 0.0f;
-    for (int e = lane; e < n_expert; e += 64) {
-        const float p = expf(lr[e] - mx);
-        probs[e] = p;
-        sum += p;
-    }
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = red[0];
+    for (int w = 1; w < n_waves; w++) mx = fmaxf(mx, red[w]);
+    __syncthreads();
+    const float ex = tid < n_expert ? expf(logit - mx) : 0.0f;
+    float sum = ex;
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    const float inv = 1.0f / sum;
+    if (lane == 0) red[wave] = sum;
     __syncthreads();
-    for (int e = lane; e < n_expert; e += 64) probs[e] *= inv;
+    sum = 0.0f;
+    for (int w = 0; w < n_waves; w++) sum += red[w];
+    const float p = ex * (1.0f / sum);
+    if (tid < n_expert) probs[tid] = p;
     __syncthreads();
-    float wsum = 0.0f;
-    for (int k = 0; k < n_used; k++) {
-        float best = -1.0f;
-        int best_e = 0x7fffffff;
-        for (int e = lane; e < n_expert; e += 64) {
-            const float p = probs[e];
-            if (p > best) {  // ascending e per lane: strict > keeps the lower id
-                best = p;
-                best_e = e;
-            }
+    if (tid < n_expert) {
+        int rank = 0;
+        for (int e = 0; e < n_expert; e++) {
+            const float q = probs[e];
+            rank += (q > p || (q == p && e < tid)) ? 1 : 0;
         }
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ob = __shfl_xor(best, off, 64);
-            const int oe = __shfl_xor(best_e, off, 64);
-            if (ob > best || (ob == best && oe < best_e)) {
-                best = ob;
-                best_e = oe;
-            }
+        if (rank < n_used) {
+            sel_e[row * n_used + rank] = tid;
+            pick_w[rank] = p;
         }
-        if (lane == 0) {
-            sel_e[row * n_used + k] = best_e;
-            pick_w[k] = best;
-            probs[best_e] = -2.0f;  // taken
-        }
-        wsum += best;
-        __syncthreads();
     }
-    wsum = fmaxf(wsum, 6.103515625e-05f);  // 2^-14
-    if (lane < n_used) sel_w[row * n_used + lane] = pick_w[lane] / wsum;
+    // shared-expert gate: sigmoid(x . w)
     float dot = 0.0f;
-    for (int i = lane; i < hidden; i += 64) dot += x[static_cast<size_t>(row) * hidden + i] * shexp_gate[i];
+    for (int i = tid; i < hidden; i += blockDim.x) dot += x[static_cast<size_t>(row) * hidden + i] * shexp_gate[i];
     for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-    if (lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
+    __syncthreads();
+    if (lane == 0) red[wave] = dot;
+    __syncthreads();
+    if (tid == 0) {
+        float d = 0.0f;
+        for (int w = 0; w < n_waves; w++) d += red[w];
+        sg[row] = 1.0f / (1.0f + expf(-d));
+        float wsum = 0.0f;
+        for (int k = 0; k < n_used; k++) wsum += pick_w[k];  // in pick order, as the reference sums them
+        wsum = fmaxf(wsum, 6.103515625e-05f);               // 2^-14
+        for (int k = 0; k < n_used; k++) sel_w[row * n_used + k] = pick_w[k] / wsum;
+    }
 }
 
 // Collects the slots whose pick is `expert`; returns the count (uniform over the workgroup).
@@ -171,28 +171,39 @@ __global__ void silu_mul_rows_kernel(float *__restrict__ g, const float *__restr
     }
 }
 
-// Distinct experts of the block, in ascending id order: ids[0 .. *n_distinct), and for every
-// (row, k) pick the index of its expert in that list.
-__global__ void __launch_bounds__(256)
-    moe_lists_kernel(const int32_t *__restrict__ sel_e, int n_picks, int n_expert, int32_t *__restrict__ ids,
-                     int32_t *__restrict__ n_distinct, int32_t *__restrict__ slot_of) {
-    extern __shared__ int32_t rank[];  // [n_expert]: 1 if picked, then its index in the list
-    for (int e = threadIdx.x; e < n_expert; e += blockDim.x) rank[e] = 0;
+// Distinct experts of the block, in ascending id order: ids[0 .. n), then one slot with id -1 (the
+// shared expert, which every row uses) if with_shared; *n_slots = n (+ 1).  For every (row, k) pick,
+// slot_of = the index of its expert in that list.  One workgroup, one thread per expert.
+__global__ void __launch_bounds__(1024)
+    moe_lists_kernel(const int32_t *__restrict__ sel_e, int n_picks, int n_expert, int with_shared,
+                     int32_t *__restrict__ ids, int32_t *__restrict__ n_slots, int32_t *__restrict__ slot_of) {
+    extern __shared__ int32_t rank[];  // [n_expert]: picked flag, then the expert's index in the list
+    __shared__ int wave_count[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
+    if (tid < n_expert) rank[tid] = 0;
     __syncthreads();
-    for (int s = threadIdx.x; s < n_picks; s += blockDim.x) rank[sel_e[s]] = 1;
+    for (int s = tid; s < n_picks; s += blockDim.x) rank[sel_e[s]] = 1;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int c = 0;
-        for (int e = 0; e < n_expert; e++) {
-            if (rank[e]) {
-                ids[c] = e;
-                rank[e] = c++;
-            }
-        }
-        *n_distinct = c;
+    const bool picked = tid < n_expert && rank[tid] != 0;
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(picked);
+    if (lane == 0) wave_count[wave] = __popcll(mask);
+    __syncthreads();
+    int base = 0, total = 0;
+    for (int w = 0; w < n_waves; w++) {
+        if (w < wave) base += wave_count[w];
+        total += wave_count[w];
+    }
+    if (picked) {
+        const int idx = base + __popcll(mask & ((1ull << lane) - 1));
+        ids[idx] = tid;
+        rank[tid] = idx;
+    }
+    if (tid == 0) {
+        if (with_shared) ids[total] = -1;
+        *n_slots = total + (with_shared ? 1 : 0);
     }
     __syncthreads();
-    for (int s = threadIdx.x; s < n_picks; s += blockDim.x) slot_of[s] = rank[sel_e[s]];
+    for (int s = tid; s < n_picks; s += blockDim.x) slot_of[s] = rank[sel_e[s]];
 }
 
 // g = silu(g) * u over the first *n_distinct slots of [slot][16][f]
@@ -205,9 +216,11 @@ __global__ void silu_mul_slots_kernel(float *__restrict__ g, const float *__rest
 }
 
 // x[row] += sum_k w[row][k] * eo[slot_of[row][k]][row]  +  sg[row] * shared[row]
+// (shared == nullptr: the shared expert's output is the last slot of eo)
 __global__ void moe_combine_slots_kernel(const float *__restrict__ eo, const int32_t *__restrict__ slot_of,
                                          const float *__restrict__ sel_w, const float *__restrict__ sg,
-                                         const float *__restrict__ shared, int n_used, int hidden, float *__restrict__ x) {
+                                         const float *__restrict__ shared, const int32_t *__restrict__ n_slots, int n_used,
+                                         int hidden, float *__restrict__ x) {
     const int row = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= hidden) return;
@@ -216,7 +229,9 @@ __global__ void moe_combine_slots_kernel(const float *__restrict__ eo, const int
         const size_t slot = slot_of[row * n_used + k];
         out += sel_w[row * n_used + k] * eo[(slot * 16 + row) * hidden + i];
     }
-    out += sg[row] * shared[static_cast<size_t>(row) * hidden + i];
+    const float sh = shared ? shared[static_cast<size_t>(row) * hidden + i]
+                            : eo[((static_cast<size_t>(*n_slots) - 1) * 16 + row) * hidden + i];
+    out += sg[row] * sh;
     x[static_cast<size_t>(row) * hidden + i] += out;
 }
 
@@ -240,27 +255,36 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
 
     int32_t rc = dflash_gemm_fewrow(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
     if (rc) return rc;
-    moe_route_kernel<<<n, 64, E * sizeof(float), st>>>(s.probs, cur, L.shexp_gate, E, used, H, s.sel_e, s.sel_w, s.sg);
+    if (E > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: %d experts (at most 1024)", E);
+    const int route_threads = (E + 63) / 64 * 64;
+    moe_route_kernel<<<n, route_threads, E * sizeof(float), st>>>(s.probs, cur, L.shexp_gate, E, used, H, s.sel_e, s.sel_w, s.sg);
 
+    bool folded_shared = false;
     const bool batched = et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K && H % DFL_QK_K == 0 && fe % DFL_QK_K == 0 &&
                          !getenv("DFLASH_MOE_PERSLOT");
     if (batched) {
         // the selected experts' matrices form one streaming GEMM each for gate, up and down: every
         // distinct expert's weights are read once, with all block rows riding along on the MFMA;
         // no split K, so a row's result is the same whichever other experts the block uses
-        const int max_slots = n_slots < E ? n_slots : E;
-        moe_lists_kernel<<<1, 256, E * sizeof(int32_t), st>>>(s.sel_e, n_slots, E, s.ids, s.n_distinct, s.slot_of);
-        if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, static_cast<size_t>(fe) * rb_in, s.ids, s.n_distinct, max_slots, cur,
-                                       DFLASH_TYPE_F32, 0, s.gate_out, static_cast<size_t>(16) * fe, H, fe, n, 1, st)))
-            return rc;
-        if ((rc = dfl_gemm_q4k_batched(ctx, L.up_exps.data, static_cast<size_t>(fe) * rb_in, s.ids, s.n_distinct, max_slots, cur,
-                                       DFLASH_TYPE_F32, 0, s.up_out, static_cast<size_t>(16) * fe, H, fe, n, 1, st)))
-            return rc;
+        // the shared expert rides along as one more slot when it has the experts' shape
+        const bool fold = fs == fe && L.gate.type == DFLASH_TYPE_Q4_K && L.up.type == DFLASH_TYPE_Q4_K &&
+                          L.down.type == DFLASH_TYPE_Q4_K;
+        folded_shared = fold;
+        const int max_slots = (n_slots < E ? n_slots : E) + (fold ? 1 : 0);
+        moe_lists_kernel<<<1, route_threads, E * sizeof(int32_t), st>>>(s.sel_e, n_slots, E, fold ? 1 : 0, s.ids, s.n_distinct,
+                                                                       s.slot_of);
         const size_t per_slot = static_cast<size_t>(16) * fe;
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, static_cast<size_t>(fe) * rb_in, fold ? L.gate.data : nullptr, s.ids,
+                                       s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, per_slot, H, fe, n, 1, st)))
+            return rc;
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.up_exps.data, static_cast<size_t>(fe) * rb_in, fold ? L.up.data : nullptr, s.ids,
+                                       s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.up_out, per_slot, H, fe, n, 1, st)))
+            return rc;
         silu_mul_slots_kernel<<<static_cast<unsigned>((per_slot * max_slots + 255) / 256), 256, 0, st>>>(s.gate_out, s.up_out,
                                                                                                      s.n_distinct, per_slot);
-        if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, static_cast<size_t>(H) * rb_dn, s.ids, s.n_distinct, max_slots,
-                                       s.gate_out, DFLASH_TYPE_F32, per_slot, s.eo, static_cast<size_t>(16) * H, fe, H, n, 1, st)))
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, static_cast<size_t>(H) * rb_dn, fold ? L.down.data : nullptr, s.ids,
+                                       s.n_distinct, max_slots, s.gate_out, DFLASH_TYPE_F32, per_slot, s.eo,
+                                       static_cast<size_t>(16) * H, fe, H, n, 1, st)))
             return rc;
     } else {
         {
@@ -292,15 +316,17 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
             }
         }
     }
-    // shared expert: plain dense SwiGLU through the few-row GEMM
-    if ((rc = dflash_gemm_fewrow(ctx, L.gate.type, L.gate.data, cur, DFLASH_TYPE_F32, s.g, H, fs, n, st))) return rc;
-    if ((rc = dflash_gemm_fewrow(ctx, L.up.type, L.up.data, cur, DFLASH_TYPE_F32, s.u, H, fs, n, st))) return rc;
-    const size_t nf = static_cast<size_t>(n) * fs;
-    silu_mul_rows_kernel<<<static_cast<unsigned>((nf + 255) / 256), 256, 0, st>>>(s.g, s.u, nf);
-    if ((rc = dflash_gemm_fewrow(ctx, L.down.type, L.down.data, s.g, DFLASH_TYPE_F32, s.shared, fs, H, n, st))) return rc;
+    if (!folded_shared) {  // shared expert: plain dense SwiGLU through the few-row GEMM
+        if ((rc = dflash_gemm_fewrow(ctx, L.gate.type, L.gate.data, cur, DFLASH_TYPE_F32, s.g, H, fs, n, st))) return rc;
+        if ((rc = dflash_gemm_fewrow(ctx, L.up.type, L.up.data, cur, DFLASH_TYPE_F32, s.u, H, fs, n, st))) return rc;
+        const size_t nf = static_cast<size_t>(n) * fs;
+        silu_mul_rows_kernel<<<static_cast<unsigned>((nf + 255) / 256), 256, 0, st>>>(s.g, s.u, nf);
+        if ((rc = dflash_gemm_fewrow(ctx, L.down.type, L.down.data, s.g, DFLASH_TYPE_F32, s.shared, fs, H, n, st))) return rc;
+    }
     if (batched)
-        moe_combine_slots_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg, s.shared, used, H,
-                                                                         x_resid);
+        moe_combine_slots_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg,
+                                                                         folded_shared ? nullptr : s.shared, s.n_distinct, used,
+                                                                         H, x_resid);
     else
         moe_combine_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.sel_w, s.sg, s.shared, used, H, x_resid);
     DFL_HIP_CHECK(ctx, hipGetLastError());
