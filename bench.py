@@ -194,26 +194,30 @@ def rocprof_summary(directory):
     import csv
     import glob
 
+    def short(name):
+        name = name.replace("(anonymous namespace)::", "").replace("void ", "")
+        return name.split("(")[0]
+
     for path in sorted(glob.glob(os.path.join(directory, "**", "*_kernel_trace.csv"), recursive=True)):
         per = collections.defaultdict(list)
         for r in csv.DictReader(open(path)):
-            name = r["Kernel_Name"].split("(")[0]
+            name = short(r["Kernel_Name"])
             per[(name, r["Grid_Size_X"], r["Workgroup_Size_X"])].append(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
         print(f"# {os.path.basename(path)}: kernel, grid, workgroup, launches, avg / min / median / max duration (us)")
         for (name, grid, wg), d in sorted(per.items(), key=lambda kv: -sum(kv[1])):
             d.sort()
-            print(f"{name[-72:]:72s} grid {grid:>8s} wg {wg:>5s} n {len(d):5d}  avg {sum(d) / len(d) / 1e3:8.2f}  "
+            print(f"{name[:72]:72s} grid {grid:>8s} wg {wg:>5s} n {len(d):5d}  avg {sum(d) / len(d) / 1e3:8.2f}  "
                   f"min {d[0] / 1e3:8.2f}  med {d[len(d) // 2] / 1e3:8.2f}  max {d[-1] / 1e3:8.2f}")
     for path in sorted(glob.glob(os.path.join(directory, "**", "*_counter_collection.csv"), recursive=True)):
         per = collections.defaultdict(lambda: collections.defaultdict(list))
         for r in csv.DictReader(open(path)):
-            name = r["Kernel_Name"].split("(")[0]
+            name = short(r["Kernel_Name"])
             per[(name, r.get("Grid_Size", r.get("Grid_Size_X", "")))][r["Counter_Name"]].append(float(r["Counter_Value"]))
         print(f"# {os.path.basename(path)}: kernel, grid, dispatches, average counter value per dispatch")
         for (name, grid), ctrs in sorted(per.items()):
             vals = "  ".join(f"{c} {sum(v) / len(v):.1f}" for c, v in sorted(ctrs.items()))
             n = max(len(v) for v in ctrs.values())
-            print(f"{name[-72:]:72s} grid {grid:>8s} n {n:4d}  {vals}")
+            print(f"{name[:72]:72s} grid {grid:>8s} n {n:4d}  {vals}")
 
 
 def main():

@@ -15,12 +15,9 @@ struct dflash_ctx {
     char *workspace = nullptr;  // device scratch, owned
     size_t workspace_bytes = 0;
     int n_cu = 256;
-    int *counters = nullptr;  // zero-initialised arrival counters; every kernel leaves them zero
-    int n_counters = 0;
-    // split-K partial tiles of the Q4_K GEMM: {value, epoch tag} pairs, persistent across calls
-    void *tagged_partials = nullptr;
+    // split-K partial tiles of the Q4_K GEMM (written by the streaming kernel, added up by its reduce kernel)
+    void *partials = nullptr;
     int n_partial_wgs = 0;
-    uint32_t epoch = 0;
     size_t lds_bytes = 65536;  // LDS available to one workgroup
     char err[512] = {0};
     // per-kernel timers (off by default; when on, timed launches synchronise)

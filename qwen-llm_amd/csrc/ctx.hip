@@ -35,16 +35,11 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
         delete ctx;
         return DFLASH_ERR_HIP;
     }
-    ctx->n_counters = 1 << 16;
-    if (hipMalloc(reinterpret_cast<void **>(&ctx->counters), ctx->n_counters * sizeof(int)) != hipSuccess ||
-        hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(int)) != hipSuccess) {
-        dflash_ctx_destroy(ctx);
-        return DFLASH_ERR_HIP;
-    }
     ctx->n_partial_wgs = 1024;
     {
-        const size_t bytes = static_cast<size_t>(ctx->n_partial_wgs) * 2 * 8 * 256 * 8;
-        if (hipMalloc(&ctx->tagged_partials, bytes) != hipSuccess || hipMemset(ctx->tagged_partials, 0, bytes) != hipSuccess) {
+        // per workgroup: 2 partial tile sets of (8 waves x 256 floats); a 16-wave workgroup takes two entries
+        const size_t bytes = static_cast<size_t>(ctx->n_partial_wgs) * 2 * 8 * 256 * sizeof(float);
+        if (hipMalloc(&ctx->partials, bytes) != hipSuccess) {
             dflash_ctx_destroy(ctx);
             return DFLASH_ERR_HIP;
         }
@@ -60,8 +55,7 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
 void dflash_ctx_destroy(dflash_ctx *ctx) {
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
-    if (ctx->counters) (void)hipFree(ctx->counters);
-    if (ctx->tagged_partials) (void)hipFree(ctx->tagged_partials);
+    if (ctx->partials) (void)hipFree(ctx->partials);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     delete ctx;

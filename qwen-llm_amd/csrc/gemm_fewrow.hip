@@ -20,8 +20,8 @@
 //    way into the same ring.  See the comment on the kernel for the pipeline.
 //  * K is split where the ranges cut a tile group; partial tiles are added by a second
 //    small kernel in a fixed order, so results are run-to-run deterministic.
-//  * Q6_K / Q8_0 share a generic kernel: eight consecutive weights per lane are
-//    dequantised to f16 and fed to the same MFMA.
+//  * Q6_K has its own kernel (half a super-block per step, see there); Q8_0 uses a simple one:
+//    eight consecutive weights per lane are dequantised to f16 and fed to the same MFMA.
 #include "common.h"
 
 #include <cstdlib>
@@ -629,7 +629,7 @@ __global__ void __launch_bounds__(64 * kWaves)
 }
 
 // ----------------------------------------------------------------------------
-// Generic kernel (Q6_K, Q8_0): eight consecutive weights -> f16 -> MFMA
+// Generic kernel (Q8_0): eight consecutive weights -> f16 -> MFMA
 // ----------------------------------------------------------------------------
 
 __device__ __forceinline__ float half_at(const uint8_t *p) {
@@ -638,27 +638,6 @@ __device__ __forceinline__ float half_at(const uint8_t *p) {
 
 template <int TYPE>
 __device__ __forceinline__ half8_t dequant8(const uint8_t *row, int64_t k0);
-
-// Q6_K: y = d * scale[i/16] * (q - 32); ql/qh interleave as in ggml's dequantize_row_q6_K
-// (metal/tests/q6_k_f32_tile.rs:46-71).
-template <>
-__device__ __forceinline__ half8_t dequant8<DFLASH_TYPE_Q6_K>(const uint8_t *row, int64_t k0) {
-    const uint8_t *blk = row + (k0 >> 8) * DFL_Q6_K_BYTES;
-    int e = static_cast<int>(k0 & 255);
-    int half_idx = e >> 7, r = e & 127, kq = r >> 5, l0 = r & 31;
-    const uint8_t *ql = blk + 64 * half_idx + ((kq & 1) ? 32 : 0) + l0;
-    const uint8_t *qh = blk + 128 + 32 * half_idx + l0;
-    float ds = half_at(blk + 208) *
-               static_cast<float>(reinterpret_cast<const int8_t *>(blk + 192 + 8 * half_idx)[(l0 >> 4) + 2 * kq]);
-    half8_t v;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        int lo = (kq & 2) ? (ql[i] >> 4) : (ql[i] & 0x0f);
-        int hi = (qh[i] >> (2 * kq)) & 3;
-        v[i] = static_cast<_Float16>(ds * static_cast<float>((lo | (hi << 4)) - 32));
-    }
-    return v;
-}
 
 template <>
 __device__ __forceinline__ half8_t dequant8<DFLASH_TYPE_Q8_0>(const uint8_t *row, int64_t k0) {
@@ -842,7 +821,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     if (n_wg < 1) n_wg = 1;
     if (total * (n_wg + 1) >= (int64_t(1) << 31) || row_bytes * 256 >= (size_t(1) << 32))
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: problem too large for 32-bit work indices");
-    float *partials = reinterpret_cast<float *>(ctx->tagged_partials);
+    float *partials = reinterpret_cast<float *>(ctx->partials);
     // a single matrix whose ranges are whole tile groups needs no reduction; a batch always may
     const bool split = batch ? !batch->whole_groups : groups % n_wg != 0;
     Q4KBatch bt = {};
