@@ -20,7 +20,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, averaged over the three shapes of a step: FETCH_SIZE + WRITE_SIZE from
 # two rocprofv3 --pmc runs of this file, each scaled by what the same counter reads for a plain 256 MiB copy
 # (profiles/gemm_q4k_stream_kernel__hbm_traffic.txt).  A counter figure, not measured by this run.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 52.03e6
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 51.15e6
 
 
 def cpu_baseline(shapes, weights, xs):
