@@ -11,9 +11,10 @@
 //    of 1024.0 (low nibble) or 64.0 (high nibble, which sits four bits up), and one
 //    packed f16 fma per value pair, fma(1024+q, s, -1024*s), yields round(q*s) with a
 //    single rounding (s = d*sc_j in f16).  The per-sub-block minimum never touches the
-//    nibbles: sum_k dmin*m_j*x[k] = dmin*m_j * (sum of x over the sub-block), so the
-//    eight minima of a super-block meet eight pre-summed activations in one extra MFMA
-//    (two: the sums are carried as a high and a low f16 part).
+//    nibbles: each weight MFMA has a twin that multiplies the same activation fragment
+//    with dmin*m_j repeated eight times and accumulates into a second tile, subtracted
+//    at the end.  The matrix cores are nearly idle in this kernel and the vector ALU is
+//    not, so this is cheaper than pre-summing activations.
 //  * The kernel is a persistent stream: one workgroup per CU walks a contiguous range of
 //    (tile group x super-block) work, weights go HBM -> LDS with direct-to-LDS loads
 //    through a ring of buffers, activations are converted to f16 MFMA fragments on the
@@ -61,14 +62,11 @@ __global__ void __launch_bounds__(256) prep_x_natural_kernel(const T *__restrict
 // Q4_K kernel
 // ----------------------------------------------------------------------------
 
-// Activation fragments of one super-block b in LDS: kQ4KBlockFrags (= 640) half8 entries:
+// Activation fragments of one super-block b in LDS: kQ4KBlockFrags (= 512) half8 entries:
 //   [t*64 + lane], t = 0..7 : A fragment of MFMA t for lane (m = lane%16, g = lane/16),
 //        value i:  k = 256 b + 64 g + 8 t + perm[i],
-//        perm = {0,2,1,3,4,6,5,7}: the order in which the nibble unpack emits a lane's values;
-//   [512 + lane], [576 + lane] : A fragment of the minima MFMA for lane (m, g): values 0 and 1
-//        are the sums of row m's f16-rounded activations over sub-blocks 2g and 2g+1 (a high and
-//        a low f16 part in the two entries), values 2..7 stay zero.
-constexpr int kQ4KBlockFrags = 640;
+//        perm = {0,2,1,3,4,6,5,7}: the order in which the nibble unpack emits a lane's values.
+constexpr int kQ4KBlockFrags = 512;
 
 __device__ __forceinline__ half2_t as_half2(uint32_t bits) { return __builtin_bit_cast(half2_t, bits); }
 
@@ -125,9 +123,9 @@ __device__ __forceinline__ _Float16 byte_to_half(uint32_t v, int j) {
 // (only a uniform base moves), so a load costs no vector ALU work.  The stage's activations
 // (16 rows x 256 values, straight from the caller's f32 or f16 matrix, L2-resident) are loaded
 // into registers three stages ahead, rounded to f16, and written to LDS in MFMA fragment order
-// together with their sub-block sums one stage ahead.  Three LDS buffers rotate: while stage d
-// is computed out of one, the activations of d+1 are already in the second and the weights of
-// d+1 and d+2 are landing in the second and third.  The loads are issued between the MFMAs of
+// together with their sub-block sums one stage ahead.  Three weight buffers rotate (while stage d
+// is computed out of one, the weights of d+1 and d+2 are landing in the other two) and two
+// activation buffers alternate.  The loads are issued between the MFMAs of
 // the stage being computed (one weight load after every second MFMA, then the activations), in
 // the same order in every wave, which makes "everything but the youngest group of loads has
 // landed" a constant s_waitcnt at the top of a stage.  Waves then read their tile's quant bytes
@@ -146,14 +144,45 @@ struct Q4KGeom {
     static constexpr int kFull = kWaveLoads / kWaves;       // ... every wave issues this many,
     static constexpr int kExtra = kWaveLoads % kWaves;      // ... and waves below kExtra one more
     static constexpr int kXLoads = 16 / kWaves;             // activation loads per thread and stage
-    static constexpr int kBufPieces = kWPieces + kQ4KBlockFrags;
+    // LDS: a ring of three weight buffers, then two activation buffers (stage parity)
+    static constexpr int kLdsPieces = 3 * kWPieces + 2 * kQ4KBlockFrags;
     static_assert(kWPieces % 64 == 0, "whole wave-loads");
     static_assert(kFull + (kExtra ? 1 : 0) <= 4, "one weight load is issued after every second of a stage's 8 MFMAs");
     static_assert(kXLoads == 1 || kXLoads == 2, "8 or 16 waves");
 };
 
+// A workgroup-uniform pointer the compiler cannot prove uniform (it depends on a loaded matrix
+// index): moved to scalar registers so that stepping it and adding it to loads is scalar work.
+__device__ __forceinline__ const uint8_t *q4k_uniform(const uint8_t *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    return reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
+
+// Division of a 31-bit value by a divisor the host knows: n / d = (n * mul) >> (32 + shift), with
+// mul = floor(2^(31 + L) / d) + 1, shift = L - 1, L = ceil(log2 d) (mul == 0 stands for d == 1).
+// The kernel's work split is all uniform integer arithmetic, done by sixteen waves on one
+// scalar unit: a generic division there costs tens of instructions, this one two.
+struct Q4KDiv {
+    uint32_t mul, shift;
+};
+__host__ __device__ __forceinline__ uint32_t q4k_div(uint32_t n, Q4KDiv f) {
+#ifdef __HIP_DEVICE_COMPILE__
+    return f.mul ? (__umulhi(n, f.mul) >> f.shift) : n;
+#else
+    return f.mul ? static_cast<uint32_t>((static_cast<uint64_t>(n) * f.mul) >> (32 + f.shift)) : n;
+#endif
+}
+inline Q4KDiv q4k_make_div(uint32_t d) {
+    if (d <= 1) return {0, 0};
+    uint32_t L = 0;
+    while ((1ull << L) < d) L++;
+    return {static_cast<uint32_t>((1ull << (31 + L)) / d + 1), L - 1};
+}
 
 // index of the workgroup whose range contains flattened iteration `it`
 // (all of this index arithmetic fits 32 bits: the host checks total * n_wg < 2^31)
@@ -188,6 +217,7 @@ struct Q4KBatch {
     size_t x_stride;         // activation elements between slots (0: all slots share x)
     size_t y_stride;         // output floats between slots
     int groups_per_mat;
+    Q4KDiv by_gpm, by_nb, by_wg;  // dividers by groups_per_mat, super-blocks per row, workgroup count
     // Ranges are cut at tile-group boundaries only: no split K, so a (row, matrix) result does not
     // depend on which other matrices take part (a verify block and a single-token pass then agree
     // bit for bit), at the price of coarser load balance.
@@ -199,10 +229,8 @@ template <int kWaves>
 struct Q4KLane {
     uint32_t w_off[Q4KGeom<kWaves>::kFull + 1];  // weight piece: byte offset from (group's first row, super-block)
     uint32_t x_off[Q4KGeom<kWaves>::kXLoads];    // activation vector: byte offset from x[0][256 b]
-    uint32_t xw_off[Q4KGeom<kWaves>::kXLoads];   // its fragment half in LDS: byte offset from the buffer
-    uint32_t xs_off[Q4KGeom<kWaves>::kXLoads];   // its sums slot in LDS (lanes with sums_lane only)
+    uint32_t xw_off[Q4KGeom<kWaves>::kXLoads];   // its fragment half in LDS: byte offset from the activation buffer
     bool x_live[Q4KGeom<kWaves>::kXLoads];       // the row is below n_rows
-    bool sums_lane;
 };
 
 // Rows past n_out (ragged last group) re-read the last row; their results are never stored.
@@ -222,22 +250,19 @@ __device__ __forceinline__ void q4k_lane_w_offsets(Q4KLane<kWaves> &L, int tid, 
 
 // Activation item of (virtual wave vw = wave + kWaves r, lane l): row m = 8 (vw & 1) + (l & 7),
 // four values k = 4c .. 4c+3 with c = 8 (vw >> 1) + (l >> 3): a virtual wave is one sub-block of
-// eight rows, its global loads are eight 128-byte runs, its LDS writes are conflict-free, and a
-// sub-block sum is a reduction over lane bits 3..5.
+// eight rows, its global loads are eight 128-byte runs and its LDS writes are conflict-free.
 template <int kWaves, typename XT>
 __device__ __forceinline__ void q4k_lane_x_offsets(Q4KLane<kWaves> &L, int tid, int n_rows, uint32_t n_in) {
     using G = Q4KGeom<kWaves>;
     const int lane = tid & 63, wave = tid >> 6;
-    L.sums_lane = (lane >> 3) == 0;
 #pragma unroll
     for (int r = 0; r < G::kXLoads; r++) {
         const int vw = wave + kWaves * r;
         const int m = 8 * (vw & 1) + (lane & 7), c = 8 * (vw >> 1) + (lane >> 3);
-        const int g = c >> 4, c15 = c & 15, j = c >> 3;
+        const int g = c >> 4, c15 = c & 15;
         L.x_live[r] = m < n_rows;
         L.x_off[r] = (static_cast<uint32_t>(min(m, n_rows - 1)) * n_in + 4u * c) * static_cast<uint32_t>(sizeof(XT));
-        L.xw_off[r] = static_cast<uint32_t>((G::kWPieces + (c15 >> 1) * 64 + m + 16 * g) * 16 + 8 * (c15 & 1));
-        L.xs_off[r] = static_cast<uint32_t>((G::kWPieces + 512 + m + 16 * (j >> 1)) * 16 + 2 * (j & 1));
+        L.xw_off[r] = static_cast<uint32_t>(((c15 >> 1) * 64 + m + 16 * g) * 16 + 8 * (c15 & 1));
     }
 }
 
@@ -258,15 +283,34 @@ struct Q4KXRaw {
     typename Q4KXVec<XT>::type v[Q4KGeom<kWaves>::kXLoads];
 };
 
-template <int kWaves, typename XT>
-__device__ __forceinline__ void q4k_load_x(const uint8_t *xblock, const Q4KLane<kWaves> &L, Q4KXRaw<kWaves, XT> &raw) {
-    typedef typename Q4KXVec<XT>::type vec_t;
-#pragma unroll
-    for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) raw.v[r] = *reinterpret_cast<const vec_t *>(xblock + L.x_off[r]);
+// The activation loads are written as asm so that the compiler's own wait-count insertion does not
+// see them: it cannot know how many younger loads a stage has issued (that depends on how much of
+// the range is left) and would drain the whole load queue, weights in flight included, before the
+// first use of these registers.  The s_waitcnt at the top of each stage covers them instead: a
+// stage's activations are always older than the youngest group of loads.
+__device__ __forceinline__ void q4k_load_x_vec(const uint8_t *p, float4_t &v) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void q4k_load_x_vec(const uint8_t *p, half4_t &v) {
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
 }
 
-// Rounds a stage's raw activations to f16 and writes this thread's share of the fragments and
-// sub-block sums into the buffer at `buf`.
+// Placed after the s_waitcnt that covers a set of activation registers: their uses cannot be
+// scheduled above this point.
+template <int kWaves, typename XT>
+__device__ __forceinline__ void q4k_pin_x(Q4KXRaw<kWaves, XT> &raw) {
+#pragma unroll
+    for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) asm volatile("" : "+v"(raw.v[r]));
+}
+
+template <int kWaves, typename XT>
+__device__ __forceinline__ void q4k_load_x(const uint8_t *xblock, const Q4KLane<kWaves> &L, Q4KXRaw<kWaves, XT> &raw) {
+#pragma unroll
+    for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) q4k_load_x_vec(xblock + L.x_off[r], raw.v[r]);
+}
+
+// Rounds a stage's raw activations to f16 and writes this thread's share of the fragments into
+// the activation buffer at `buf`.
 template <int kWaves, typename XT>
 __device__ __forceinline__ void q4k_write_x(half8_t *buf, const Q4KLane<kWaves> &L, const Q4KXRaw<kWaves, XT> &raw,
                                             bool full_rows) {
@@ -282,15 +326,6 @@ __device__ __forceinline__ void q4k_write_x(half8_t *buf, const Q4KLane<kWaves> 
         }
         half4_t frag = {h[0], h[2], h[1], h[3]};
         *reinterpret_cast<half4_t *>(base + L.xw_off[r]) = frag;
-        float s = (static_cast<float>(h[0]) + static_cast<float>(h[1])) + (static_cast<float>(h[2]) + static_cast<float>(h[3]));
-        s += __shfl_xor(s, 8, 64);
-        s += __shfl_xor(s, 16, 64);
-        s += __shfl_xor(s, 32, 64);
-        if (L.sums_lane) {
-            const _Float16 hi = static_cast<_Float16>(s);
-            *reinterpret_cast<_Float16 *>(base + L.xs_off[r]) = hi;
-            *reinterpret_cast<_Float16 *>(base + L.xs_off[r] + 64 * 16) = static_cast<_Float16>(s - static_cast<float>(hi));
-        }
     }
 }
 
@@ -300,21 +335,21 @@ __device__ __forceinline__ void q4k_issue_w(const uint8_t *wstage, half8_t *buf,
     __builtin_amdgcn_global_load_lds((gptr_t)(wstage + L.w_off[j]), (lptr_t)(buf + (j * kWaves + wave) * 64), 16, 0, 0);
 }
 
-// One stage (one super-block) of this wave's tile out of the LDS buffer `buf`: 8 MFMAs plus 2 for
-// the minima.  hdr = {d|dmin, scales[0..3], [4..7], [8..11]}, q0/q1 = the lane's 32 quant bytes
+// One stage (one super-block) of this wave's tile out of the weight buffer `buf` and the activation
+// buffer `xcur`: 8 MFMAs for the scaled nibbles, 8 for the minima.  hdr = {d|dmin, scales[0..3], [4..7], [8..11]}, q0/q1 = the lane's 32 quant bytes
 // (chunk g: sub-blocks 2g in the low and 2g+1 in the high nibbles).  The loads of later stages
 // are issued in between: one weight load after every second MFMA (spread over the MFMAs, the
 // loads never queue up behind each other in the address unit), then the activations; the
 // activations of the next stage are converted and written to LDS half way through.
 template <int kWaves, typename XT>
-__device__ __forceinline__ void q4k_compute(const half8_t *buf, int lane, int wave, Q4KMagic magic, float4_t &acc,
+__device__ __forceinline__ void q4k_compute(const half8_t *buf, const half8_t *xcur, int lane, int wave, Q4KMagic magic, float4_t &acc,
                                             float4_t &acc_min, bool issue_w, const uint8_t *wstage, half8_t *wbuf,
                                             bool issue_x, const uint8_t *xblock, const Q4KLane<kWaves> &L,
                                             Q4KXRaw<kWaves, XT> &raw, bool write_x, half8_t *xbuf, bool full_rows) {
     using G = Q4KGeom<kWaves>;
     const int n = lane & 15, g = lane >> 4;
     const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(buf) + (wave * 16 + n) * 9;
-    const half8_t *a = buf + G::kWPieces + lane;
+    const half8_t *a = xcur + lane;
     const u32x4_t hdr = blk[0], q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
     // scales and minima of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles); the 6-bit codes of
     // sub-blocks 0..3 sit in one dword, those of 4..7 are split over two: select by bit mask,
@@ -330,11 +365,17 @@ __device__ __forceinline__ void q4k_compute(const half8_t *buf, int lane, int wa
     const _Float16 s_hi = byte_to_half(sc_sel, 1) * dm[0];
     const half2_t s2l = splat(s_lo), c2l = splat(s_lo * static_cast<_Float16>(-1024.0f));
     const half2_t s2h = splat(s_hi), c2h = splat(s_hi * static_cast<_Float16>(-64.0f));
+    // dmin*m of sub-blocks 2g and 2g+1, eight times each: the B operands of the minima MFMAs
+    const _Float16 m_lo = byte_to_half(mn_sel, 0) * dm[1], m_hi = byte_to_half(mn_sel, 1) * dm[1];
+    const half8_t bml = {m_lo, m_lo, m_lo, m_lo, m_lo, m_lo, m_lo, m_lo};
+    const half8_t bmh = {m_hi, m_hi, m_hi, m_hi, m_hi, m_hi, m_hi, m_hi};
     const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t * 64], bl, acc, 0, 0, 0);
+        const half8_t af = a[t * 64];
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bl, acc, 0, 0, 0);
+        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bml, acc_min, 0, 0, 0);
         if (t & 1) {
             const int j = t >> 1;
             if (issue_w && (j < G::kFull || (j == G::kFull && wave < G::kExtra))) q4k_issue_w<kWaves>(wstage, wbuf, L, j, wave);
@@ -347,7 +388,9 @@ __device__ __forceinline__ void q4k_compute(const half8_t *buf, int lane, int wa
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(4 + t) * 64], bh, acc, 0, 0, 0);
+        const half8_t af = a[(4 + t) * 64];
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bh, acc, 0, 0, 0);
+        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bmh, acc_min, 0, 0, 0);
         if (t & 1) {
             const int j = 2 + (t >> 1);
             if (issue_w && (j < G::kFull || (j == G::kFull && wave < G::kExtra))) q4k_issue_w<kWaves>(wstage, wbuf, L, j, wave);
@@ -355,11 +398,6 @@ __device__ __forceinline__ void q4k_compute(const half8_t *buf, int lane, int wa
         }
     }
     if (issue_x) q4k_load_x<kWaves, XT>(xblock, L, raw);
-    __builtin_amdgcn_sched_barrier(0);
-    // minima: lane (n, g) carries dmin*m of sub-blocks 2g and 2g+1 in values 0 and 1 of the B operand
-    const half8_t bm = {byte_to_half(mn_sel, 0) * dm[1], byte_to_half(mn_sel, 1) * dm[1], 0, 0, 0, 0, 0, 0};
-    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[512], bm, acc_min, 0, 0, 0);
-    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[576], bm, acc_min, 0, 0, 0);
 }
 
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt low bits [3:0],
@@ -380,12 +418,11 @@ __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, const Q4KBatch &bt
     float4_t res = acc - acc_min;
     acc = float4_t{0, 0, 0, 0};
     acc_min = float4_t{0, 0, 0, 0};
-    const int slot_j = group / bt.groups_per_mat, lg = group - slot_j * bt.groups_per_mat;
+    const int slot_j = bt.ids ? static_cast<int>(q4k_div(group, bt.by_gpm)) : 0, lg = group - slot_j * bt.groups_per_mat;
     y += static_cast<size_t>(slot_j) * bt.y_stride;
     const int orow = (lg * kWaves + wave) * 16 + n;
-    const int wg_first = bt.whole_groups ? 0 : q4k_wg_of(group * rg.nb, rg.total, rg.n_wg);
-    const int wg_last = bt.whole_groups ? 0 : q4k_wg_of((group + 1) * rg.nb - 1, rg.total, rg.n_wg);
-    if (wg_first == wg_last) {
+    // the group's whole K lies inside this workgroup's range: no other workgroup contributes
+    if (group * rg.nb >= rg.it_begin && (group + 1) * rg.nb <= rg.it_end) {
         if (orow < n_out) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
@@ -411,7 +448,6 @@ __global__ void __launch_bounds__(256)
     const int group = blockIdx.x / kWaves, wave = blockIdx.x % kWaves;
     if (bt.ids) n_groups = bt.groups_per_mat * *bt.n_slots;
     if (group >= n_groups) return;
-    if (n_wg > n_groups * nb) n_wg = n_groups * nb;
     const int total = n_groups * nb;
     const int wg_first = q4k_wg_of(group * nb, total, n_wg);
     const int wg_last = q4k_wg_of((group + 1) * nb - 1, total, n_wg);
@@ -444,6 +480,8 @@ __device__ unsigned long long *g_trace = nullptr;  // [n_wg][16]
     do {                                                                                   \
         if (threadIdx.x == 0 && g_trace) g_trace[blockIdx.x * 16 + (i)] = wall_clock64();  \
     } while (0)
+__device__ unsigned long long *g_trace2 = nullptr;  // [n_wg][16 waves][4]: cycles in load wait / barrier / compute, stages
+#define DFL_CYC() __builtin_readcyclecounter()
 #else
 #define DFL_TR(i) \
     do {          \
@@ -455,7 +493,7 @@ __global__ void __launch_bounds__(64 * kWaves)
     gemm_q4k_stream_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
                            float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt) {
     using G = Q4KGeom<kWaves>;
-    extern __shared__ half8_t lds[];  // three buffers of kBufPieces
+    extern __shared__ half8_t lds[];  // kLdsPieces
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -465,21 +503,16 @@ __global__ void __launch_bounds__(64 * kWaves)
     rg.n_wg = gridDim.x;
     if (bt.ids) n_groups = bt.groups_per_mat * *bt.n_slots;  // how many matrices take part is decided on the device
     rg.total = n_groups * nb;
-    if (rg.n_wg > rg.total) rg.n_wg = rg.total;  // surplus workgroups leave
-    if (static_cast<int>(blockIdx.x) >= rg.n_wg) return;
+    rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
     if (bt.whole_groups) {
-        if (rg.n_wg > n_groups) rg.n_wg = n_groups;
-        if (static_cast<int>(blockIdx.x) >= rg.n_wg) return;
-        rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
-        rg.it_begin = static_cast<int>(static_cast<uint32_t>(n_groups) * rg.wg / rg.n_wg) * nb;
-        rg.it_end = static_cast<int>(static_cast<uint32_t>(n_groups) * (rg.wg + 1) / rg.n_wg) * nb;
+        rg.it_begin = static_cast<int>(q4k_div(static_cast<uint32_t>(n_groups) * rg.wg, bt.by_wg)) * nb;
+        rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(n_groups) * (rg.wg + 1), bt.by_wg)) * nb;
     } else {
-        rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
-        rg.it_begin = static_cast<int>(static_cast<uint32_t>(rg.total) * rg.wg / rg.n_wg);
-        rg.it_end = static_cast<int>(static_cast<uint32_t>(rg.total) * (rg.wg + 1) / rg.n_wg);
+        rg.it_begin = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * rg.wg, bt.by_wg));
+        rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * (rg.wg + 1), bt.by_wg));
     }
-    if (rg.it_begin >= rg.it_end) return;
-    rg.first_group = static_cast<int>(static_cast<uint32_t>(rg.it_begin) / static_cast<uint32_t>(nb));
+    if (rg.it_begin >= rg.it_end) return;  // more workgroups than work
+    rg.first_group = static_cast<int>(q4k_div(rg.it_begin, bt.by_nb));
     const int b0 = rg.it_begin - rg.first_group * nb;
     const uint32_t row_bytes = static_cast<uint32_t>(nb) * DFL_Q4_K_BYTES;
     const uint32_t n_in = static_cast<uint32_t>(nb) * DFL_QK_K;
@@ -489,23 +522,23 @@ __global__ void __launch_bounds__(64 * kWaves)
 
     // first weight byte of a group's first row, its activations, and the local group index
     auto group_w = [&](int group) {
-        const int j = group / bt.groups_per_mat, lg = group - j * bt.groups_per_mat;
-        const uint8_t *mat = w;
-        if (bt.ids) {
-            const int32_t id = bt.ids[j];
-            mat = id < 0 ? bt.extra_w : w + static_cast<size_t>(id) * bt.w_stride;
-        }
-        return mat + static_cast<size_t>(lg) * group_bytes;
+        if (!bt.ids) return w + static_cast<size_t>(group) * group_bytes;
+        const int j = static_cast<int>(q4k_div(group, bt.by_gpm)), lg = group - j * bt.groups_per_mat;
+        const int32_t id = bt.ids[j];
+        const uint8_t *mat = id < 0 ? bt.extra_w : w + static_cast<size_t>(id) * bt.w_stride;
+        return q4k_uniform(mat + static_cast<size_t>(lg) * group_bytes);
     };
     auto group_x = [&](int group) {
-        return xbytes + static_cast<size_t>(group / bt.groups_per_mat) * bt.x_stride * sizeof(XT);
+        if (!bt.ids) return xbytes;
+        return xbytes + static_cast<size_t>(q4k_div(group, bt.by_gpm)) * bt.x_stride * sizeof(XT);
     };
-    auto group_local = [&](int group) { return group % bt.groups_per_mat; };
+    auto group_local = [&](int group) {
+        return bt.ids ? group - static_cast<int>(q4k_div(group, bt.by_gpm)) * bt.groups_per_mat : group;
+    };
+    DFL_TR(10);
     Q4KLane<kWaves> L;
     q4k_lane_w_offsets<kWaves>(L, tid, group_local(rg.first_group) * G::kRows, n_out, row_bytes);
-    q4k_lane_x_offsets<kWaves, XT>(L, tid, n_rows, n_in);
-    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0};
-    const Q4KMagic magic = q4k_magic();
+    DFL_TR(11);
 
     // Cursors.  Weights: wstage = first byte of the next stage to load in its group's first row,
     // bw its super-block, gw its group, w_left the stages not loaded yet.  Activations run one
@@ -541,12 +574,19 @@ __global__ void __launch_bounds__(64 * kWaves)
         for (int j = 0; j < G::kFull; j++) q4k_issue_w<kWaves>(wstage, buf, L, j, wave);
         if (wave < G::kExtra) q4k_issue_w<kWaves>(wstage, buf, L, G::kFull, wave);
     };
-    half8_t *buf_c = lds, *buf_n = lds + G::kBufPieces, *buf_f = lds + 2 * G::kBufPieces;
+    half8_t *buf_c = lds, *buf_n = lds + G::kWPieces, *buf_f = lds + 2 * G::kWPieces;
+    half8_t *x_c = lds + 3 * G::kWPieces, *x_n = x_c + kQ4KBlockFrags;
 
-    // Prologue, in this order: activations of stages 0 and 1, weights of stage 0 | weights of
-    // stage 1, activations of stage 2.  From then on stage d issues one group [weights of d+2,
-    // activations of d+3], and "all but the youngest group have landed" is what the top of each
-    // stage waits for; young_w / young_x say what the youngest group holds.
+    // Prologue, in this order: weights of stage 0 (first of all: everything else here hides behind
+    // their latency), activations of stages 0 and 1 | weights of stage 1, activations of stage 2.
+    // From then on stage d issues one group [weights of d+2, activations of d+3], and "all but the
+    // youngest group have landed" is what the top of each stage waits for; young_w / young_x say
+    // what the youngest group holds.
+    issue_w_all(buf_c);
+    advance_w();
+    q4k_lane_x_offsets<kWaves, XT>(L, tid, n_rows, n_in);
+    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0};
+    const Q4KMagic magic = q4k_magic();
     Q4KXRaw<kWaves, XT> raw_first, raw_a, raw_b;  // activations of stage 0 / odd stages / even stages >= 2
     bool young_w = false, young_x = false;
     q4k_load_x<kWaves, XT>(xblock, L, raw_first);
@@ -555,8 +595,6 @@ __global__ void __launch_bounds__(64 * kWaves)
         q4k_load_x<kWaves, XT>(xblock, L, raw_a);
         advance_x();
     }
-    issue_w_all(buf_c);
-    advance_w();
     if (w_left > 0) {
         issue_w_all(buf_n);
         advance_w();
@@ -567,19 +605,20 @@ __global__ void __launch_bounds__(64 * kWaves)
             young_x = true;
         }
     }
-    // the unused values of the minima fragments must be finite: zero them once (ordered before the
-    // first sums writes by a barrier that does not wait for the loads just issued)
-    for (int e = tid; e < 3 * 128; e += G::kThreads)
-        lds[(e >> 7) * G::kBufPieces + G::kWPieces + 512 + (e & 127)] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    __builtin_amdgcn_s_waitcnt(kWaitLds);
-    __builtin_amdgcn_s_barrier();
+    DFL_TR(12);
     DFL_TR(1);
     int gc = rg.first_group, bc = b0, n_left = rg.it_end - rg.it_begin;
     bool first = true;
     int done = 0;
     // One stage; `raw` holds the activations of the next stage and is refilled with those three ahead.
+#ifdef DFLASH_TRACE
+    unsigned long long cyc_wait = 0, cyc_bar = 0, cyc_comp = 0, cyc_n = 0;
+#endif
     auto stage = [&](Q4KXRaw<kWaves, XT> &raw) {
         constexpr int kW0 = G::kFull, kW1 = G::kFull + 1, kX = G::kXLoads;
+#ifdef DFLASH_TRACE
+        const unsigned long long c0 = DFL_CYC();
+#endif
         if (young_w && young_x) {
             if (wave < G::kExtra)
                 __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW1 + kX));
@@ -593,16 +632,35 @@ __global__ void __launch_bounds__(64 * kWaves)
         } else {
             __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
         }
-        if (first) q4k_write_x<kWaves, XT>(buf_c, L, raw_first, n_rows == 16);
+#ifdef DFLASH_TRACE
+        const unsigned long long c1 = DFL_CYC();
+#endif
+        q4k_pin_x<kWaves, XT>(raw);
+        if (first) {
+            q4k_pin_x<kWaves, XT>(raw_first);
+            q4k_write_x<kWaves, XT>(x_c, L, raw_first, n_rows == 16);
+        }
         first = false;
         __builtin_amdgcn_s_waitcnt(kWaitLds);
         // A bare barrier, not __syncthreads(): that one carries a workgroup-scope fence, which waits
         // for every load in flight and would undo the prefetch.  The waits above are the only
         // ordering this needs: each wave's own pieces have landed before it arrives here.
         __builtin_amdgcn_s_barrier();  // stage d is complete in buf_c; buf_f (stage d-1) is free
+#ifdef DFLASH_TRACE
+        const unsigned long long c2 = DFL_CYC();
+#endif
         const bool iw = w_left > 0, ix = x_left > 0;
-        q4k_compute<kWaves, XT>(buf_c, lane, wave, magic, acc, acc_min, iw, wstage, buf_f, ix, xblock, L, raw, n_left > 1,
-                                buf_n, n_rows == 16);
+        q4k_compute<kWaves, XT>(buf_c, x_c, lane, wave, magic, acc, acc_min, iw, wstage, buf_f, ix, xblock, L, raw, n_left > 1,
+                                x_n, n_rows == 16);
+#ifdef DFLASH_TRACE
+        {
+            const unsigned long long c3 = DFL_CYC();
+            cyc_wait += c1 - c0;
+            cyc_bar += c2 - c1;
+            cyc_comp += c3 - c2;
+            cyc_n++;
+        }
+#endif
         if (iw) advance_w();
         if (ix) advance_x();
         young_w = iw;
@@ -611,6 +669,9 @@ __global__ void __launch_bounds__(64 * kWaves)
         buf_c = buf_n;
         buf_n = buf_f;
         buf_f = t;
+        t = x_c;
+        x_c = x_n;
+        x_n = t;
         n_left--;
         done++;
         if (done <= 8) DFL_TR(1 + done);
@@ -626,6 +687,15 @@ __global__ void __launch_bounds__(64 * kWaves)
         stage(raw_b);
     }
     DFL_TR(13);
+#ifdef DFLASH_TRACE
+    if (lane == 0 && g_trace2) {
+        unsigned long long *t = g_trace2 + (static_cast<size_t>(blockIdx.x) * 16 + wave) * 4;
+        t[0] = cyc_wait;
+        t[1] = cyc_bar;
+        t[2] = cyc_comp;
+        t[3] = cyc_n;
+    }
+#endif
 }
 
 // ----------------------------------------------------------------------------
@@ -785,6 +855,10 @@ extern "C" void dflash_dbg_set_trace(uint64_t p) {
     unsigned long long *v = reinterpret_cast<unsigned long long *>(p);
     (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &v, sizeof(v));
 }
+extern "C" void dflash_dbg_set_trace2(uint64_t p) {
+    unsigned long long *v = reinterpret_cast<unsigned long long *>(p);
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace2), &v, sizeof(v));
+}
 #endif
 
 namespace {
@@ -827,11 +901,14 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     Q4KBatch bt = {};
     if (batch) bt = *batch;
     bt.groups_per_mat = gpm;
+    bt.by_gpm = q4k_make_div(static_cast<uint32_t>(gpm));
+    bt.by_nb = q4k_make_div(static_cast<uint32_t>(nb));
+    bt.by_wg = q4k_make_div(static_cast<uint32_t>(n_wg));
     const uint8_t *wb = static_cast<const uint8_t *>(w);
     const int no = static_cast<int>(n_out);
 #define DFL_LAUNCH_Q4K(WAVES, XT)                                                                                      \
     do {                                                                                                               \
-        const size_t lds = static_cast<size_t>(3 * Q4KGeom<WAVES>::kBufPieces) * sizeof(half8_t);                      \
+        const size_t lds = static_cast<size_t>(Q4KGeom<WAVES>::kLdsPieces) * sizeof(half8_t);                      \
         if (lds > ctx->lds_bytes)                                                                                      \
             return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: %zu bytes of LDS needed", lds);                 \
         static bool attr = false;                                                                                      \
@@ -874,7 +951,14 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_q4k_batched: bad shape");
     if (reinterpret_cast<uintptr_t>(w_stack) % 16 || reinterpret_cast<uintptr_t>(extra_w) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16)
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_q4k_batched: operand alignment");
-    Q4KBatch bt = {ids, static_cast<const uint8_t *>(extra_w), n_slots, w_stride_bytes, x_stride, y_stride, 0, whole_groups};
+    Q4KBatch bt = {};
+    bt.ids = ids;
+    bt.extra_w = static_cast<const uint8_t *>(extra_w);
+    bt.n_slots = n_slots;
+    bt.w_stride = w_stride_bytes;
+    bt.x_stride = x_stride;
+    bt.y_stride = y_stride;
+    bt.whole_groups = whole_groups;
     return launch_q4k(ctx, w_stack, x, x_type, y, n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt, max_slots);
 }
 
