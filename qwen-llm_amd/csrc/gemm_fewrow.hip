@@ -230,7 +230,7 @@ struct Q4KLane {
     uint32_t w_off[Q4KGeom<kWaves>::kFull + 1];  // weight piece: byte offset from (group's first row, super-block)
     uint32_t x_off[Q4KGeom<kWaves>::kXLoads];    // activation vector: byte offset from x[0][256 b]
     uint32_t xw_off[Q4KGeom<kWaves>::kXLoads];   // its fragment half in LDS: byte offset from the activation buffer
-    bool x_live[Q4KGeom<kWaves>::kXLoads];       // the row is below n_rows
+    uint32_t sc_sel;                             // byte selector of this lane's two scale codes (see q4k_compute)
 };
 
 // Rows past n_out (ragged last group) re-read the last row; their results are never stored.
@@ -255,12 +255,12 @@ template <int kWaves, typename XT>
 __device__ __forceinline__ void q4k_lane_x_offsets(Q4KLane<kWaves> &L, int tid, int n_rows, uint32_t n_in) {
     using G = Q4KGeom<kWaves>;
     const int lane = tid & 63, wave = tid >> 6;
+    L.sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
 #pragma unroll
     for (int r = 0; r < G::kXLoads; r++) {
         const int vw = wave + kWaves * r;
         const int m = 8 * (vw & 1) + (lane & 7), c = 8 * (vw >> 1) + (lane >> 3);
         const int g = c >> 4, c15 = c & 15;
-        L.x_live[r] = m < n_rows;
         L.x_off[r] = (static_cast<uint32_t>(min(m, n_rows - 1)) * n_in + 4u * c) * static_cast<uint32_t>(sizeof(XT));
         L.xw_off[r] = static_cast<uint32_t>(((c15 >> 1) * 64 + m + 16 * g) * 16 + 8 * (c15 & 1));
     }
@@ -288,11 +288,11 @@ struct Q4KXRaw {
 // the range is left) and would drain the whole load queue, weights in flight included, before the
 // first use of these registers.  The s_waitcnt at the top of each stage covers them instead: a
 // stage's activations are always older than the youngest group of loads.
-__device__ __forceinline__ void q4k_load_x_vec(const uint8_t *p, float4_t &v) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+__device__ __forceinline__ void q4k_load_x_vec(const uint8_t *base, uint32_t off, float4_t &v) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(off), "s"(base) : "memory");
 }
-__device__ __forceinline__ void q4k_load_x_vec(const uint8_t *p, half4_t &v) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+__device__ __forceinline__ void q4k_load_x_vec(const uint8_t *base, uint32_t off, half4_t &v) {
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(off), "s"(base) : "memory");
 }
 
 // Placed after the s_waitcnt that covers a set of activation registers: their uses cannot be
@@ -306,24 +306,20 @@ __device__ __forceinline__ void q4k_pin_x(Q4KXRaw<kWaves, XT> &raw) {
 template <int kWaves, typename XT>
 __device__ __forceinline__ void q4k_load_x(const uint8_t *xblock, const Q4KLane<kWaves> &L, Q4KXRaw<kWaves, XT> &raw) {
 #pragma unroll
-    for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) q4k_load_x_vec(xblock + L.x_off[r], raw.v[r]);
+    for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) q4k_load_x_vec(xblock, L.x_off[r], raw.v[r]);
 }
 
 // Rounds a stage's raw activations to f16 and writes this thread's share of the fragments into
-// the activation buffer at `buf`.
+// the activation buffer at `buf`.  Rows past n_rows repeat the last row: output rows depend on
+// their own activation row only, and those rows are never stored.
 template <int kWaves, typename XT>
-__device__ __forceinline__ void q4k_write_x(half8_t *buf, const Q4KLane<kWaves> &L, const Q4KXRaw<kWaves, XT> &raw,
-                                            bool full_rows) {
+__device__ __forceinline__ void q4k_write_x(half8_t *buf, const Q4KLane<kWaves> &L, const Q4KXRaw<kWaves, XT> &raw) {
     uint8_t *base = reinterpret_cast<uint8_t *>(buf);
 #pragma unroll
     for (int r = 0; r < Q4KGeom<kWaves>::kXLoads; r++) {
         _Float16 h[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) h[i] = static_cast<_Float16>(raw.v[r][i]);
-        if (!full_rows && !L.x_live[r]) {  // full_rows is uniform: a 16-row block never takes this
-#pragma unroll
-            for (int i = 0; i < 4; i++) h[i] = static_cast<_Float16>(0.0f);
-        }
         half4_t frag = {h[0], h[2], h[1], h[3]};
         *reinterpret_cast<half4_t *>(base + L.xw_off[r]) = frag;
     }
@@ -345,37 +341,48 @@ template <int kWaves, typename XT>
 __device__ __forceinline__ void q4k_compute(const half8_t *buf, const half8_t *xcur, int lane, int wave, Q4KMagic magic, float4_t &acc,
                                             float4_t &acc_min, bool issue_w, const uint8_t *wstage, half8_t *wbuf,
                                             bool issue_x, const uint8_t *xblock, const Q4KLane<kWaves> &L,
-                                            Q4KXRaw<kWaves, XT> &raw, bool write_x, half8_t *xbuf, bool full_rows) {
+                                            Q4KXRaw<kWaves, XT> &raw, bool write_x, half8_t *xbuf) {
     using G = Q4KGeom<kWaves>;
     const int n = lane & 15, g = lane >> 4;
     const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(buf) + (wave * 16 + n) * 9;
     const half8_t *a = xcur + lane;
     const u32x4_t hdr = blk[0], q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
+    // all eight activation fragments are fetched up front: their LDS latencies overlap each other
+    // and the scale decode instead of stalling every MFMA pair
+    half8_t af[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) af[t] = a[t * 64];
     // scales and minima of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles); the 6-bit codes of
     // sub-blocks 0..3 sit in one dword, those of 4..7 are split over two: select by bit mask,
     // not by branch
-    const int sh = 16 * (g & 1);
     const uint32_t upper = 0u - static_cast<uint32_t>(g >> 1);  // all ones for g = 2, 3
     const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
     const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu, mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
-    const uint32_t sc_sel = ((sc_hi & upper) | (sc_lo & ~upper)) >> sh;
-    const uint32_t mn_sel = ((mn_hi & upper) | (mn_lo & ~upper)) >> sh;
+    const uint32_t sc_word = (sc_hi & upper) | (sc_lo & ~upper), mn_word = (mn_hi & upper) | (mn_lo & ~upper);
+    // The two 6-bit codes of this lane sit in bytes (0,1) or (2,3) of those words.  A byte
+    // permute drops each into the mantissa of an f16 1024.0 (the lane's selector picks the byte
+    // pair), and one packed fma per pair, (1024 + code) * d - 1024 d, gives code * d rounded once:
+    // S = (s of sub-block 2g, s of 2g+1), M = (dmin*m of 2g, of 2g+1).
     const half2_t dm = __builtin_bit_cast(half2_t, hdr.x);
-    const _Float16 s_lo = byte_to_half(sc_sel, 0) * dm[0];
-    const _Float16 s_hi = byte_to_half(sc_sel, 1) * dm[0];
-    const half2_t s2l = splat(s_lo), c2l = splat(s_lo * static_cast<_Float16>(-1024.0f));
-    const half2_t s2h = splat(s_hi), c2h = splat(s_hi * static_cast<_Float16>(-64.0f));
+    const half2_t p_sc = as_half2(__builtin_amdgcn_perm(0x64646464u, sc_word, L.sc_sel));
+    const half2_t p_mn = as_half2(__builtin_amdgcn_perm(0x64646464u, mn_word, L.sc_sel));
+    const half2_t neg = dm * splat(static_cast<_Float16>(-1024.0f));
+    const half2_t S = __builtin_elementwise_fma(p_sc, splat(dm[0]), splat(neg[0]));
+    const half2_t M = __builtin_elementwise_fma(p_mn, splat(dm[1]), splat(neg[1]));
+    const half2_t unbias = {static_cast<_Float16>(-1024.0f), static_cast<_Float16>(-64.0f)};
+    const half2_t Cs = S * unbias;
+    const half2_t s2l = splat(S[0]), c2l = splat(Cs[0]);
+    const half2_t s2h = splat(S[1]), c2h = splat(Cs[1]);
     // dmin*m of sub-blocks 2g and 2g+1, eight times each: the B operands of the minima MFMAs
-    const _Float16 m_lo = byte_to_half(mn_sel, 0) * dm[1], m_hi = byte_to_half(mn_sel, 1) * dm[1];
+    const _Float16 m_lo = M[0], m_hi = M[1];
     const half8_t bml = {m_lo, m_lo, m_lo, m_lo, m_lo, m_lo, m_lo, m_lo};
     const half8_t bmh = {m_hi, m_hi, m_hi, m_hi, m_hi, m_hi, m_hi, m_hi};
     const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
-        const half8_t af = a[t * 64];
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bl, acc, 0, 0, 0);
-        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bml, acc_min, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
+        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bml, acc_min, 0, 0, 0);
         if (t & 1) {
             const int j = t >> 1;
             if (issue_w && (j < G::kFull || (j == G::kFull && wave < G::kExtra))) q4k_issue_w<kWaves>(wstage, wbuf, L, j, wave);
@@ -384,13 +391,12 @@ __device__ __forceinline__ void q4k_compute(const half8_t *buf, const half8_t *x
     }
     // the next stage's activations (in registers since the wait at the top of this stage) go to
     // LDS here, off the critical path between that wait and the barrier
-    if (write_x) q4k_write_x<kWaves, XT>(xbuf, L, raw, full_rows);
+    if (write_x) q4k_write_x<kWaves, XT>(xbuf, L, raw);
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
-        const half8_t af = a[(4 + t) * 64];
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bh, acc, 0, 0, 0);
-        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bmh, acc_min, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bh, acc, 0, 0, 0);
+        acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bmh, acc_min, 0, 0, 0);
         if (t & 1) {
             const int j = 2 + (t >> 1);
             if (issue_w && (j < G::kFull || (j == G::kFull && wave < G::kExtra))) q4k_issue_w<kWaves>(wstage, wbuf, L, j, wave);
@@ -638,7 +644,7 @@ __global__ void __launch_bounds__(64 * kWaves)
         q4k_pin_x<kWaves, XT>(raw);
         if (first) {
             q4k_pin_x<kWaves, XT>(raw_first);
-            q4k_write_x<kWaves, XT>(x_c, L, raw_first, n_rows == 16);
+            q4k_write_x<kWaves, XT>(x_c, L, raw_first);
         }
         first = false;
         __builtin_amdgcn_s_waitcnt(kWaitLds);
@@ -651,7 +657,7 @@ __global__ void __launch_bounds__(64 * kWaves)
 #endif
         const bool iw = w_left > 0, ix = x_left > 0;
         q4k_compute<kWaves, XT>(buf_c, x_c, lane, wave, magic, acc, acc_min, iw, wstage, buf_f, ix, xblock, L, raw, n_left > 1,
-                                x_n, n_rows == 16);
+                                x_n);
 #ifdef DFLASH_TRACE
         {
             const unsigned long long c3 = DFL_CYC();
