@@ -61,6 +61,35 @@ __device__ __forceinline__ int attn_swz(int r) { return (r & 3) | ((r >> 1) & 4)
 // MAXW = most waves a workgroup may have; it sets the register budget.  HPW = query heads per wave:
 // with two, every K and V^T fragment read from LDS feeds two MFMAs (half the LDS traffic per head,
 // and two independent dependency chains per wave).
+// eight consecutive query values (16-byte aligned) as floats
+__device__ __forceinline__ void attn_load8(const float *p, float v[8]) {
+    const float4_t a = *reinterpret_cast<const float4_t *>(p), b = *reinterpret_cast<const float4_t *>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        v[i] = a[i];
+        v[4 + i] = b[i];
+    }
+}
+__device__ __forceinline__ void attn_load8(const _Float16 *p, float v[8]) {
+    const half8_t a = *reinterpret_cast<const half8_t *>(p);
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = static_cast<float>(a[i]);
+}
+
+#ifdef DFLASH_TRACE
+// Debug build only: per-workgroup time stamps (100 MHz constant clock).
+__device__ unsigned long long *g_attn_trace = nullptr;  // [n_wg][16]
+#define ATT_TR(i)                                                                                                   \
+    do {                                                                                                            \
+        if (threadIdx.x == 0 && g_attn_trace)                                                                       \
+            g_attn_trace[(blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();                        \
+    } while (0)
+#else
+#define ATT_TR(i) \
+    do {          \
+    } while (0)
+#endif
+
 template <int HD, typename TQ, int MAXW, int HPW>
 __global__ void __launch_bounds__(64 * MAXW)
     attn_split_kernel(const TQ *__restrict__ q, const _Float16 *__restrict__ k_cache,
@@ -87,6 +116,7 @@ __global__ void __launch_bounds__(64 * MAXW)
     const int n_steps = static_cast<int>((c1 - c0 + 31) / 32);
     const int64_t kv_dim = static_cast<int64_t>(n_kv) * HD;
     const int per_wave = (kWaveLoads + n_waves - 1) / n_waves;  // loads each wave issues per stage
+    ATT_TR(0);
 
     const uint8_t *kbytes = reinterpret_cast<const uint8_t *>(k_cache + static_cast<int64_t>(kvh) * HD);
     const uint8_t *vbytes = reinterpret_cast<const uint8_t *>(vt_cache + static_cast<int64_t>(kvh) * HD * vt_stride);
@@ -124,25 +154,27 @@ __global__ void __launch_bounds__(64 * MAXW)
         }
     }
 
+    ATT_TR(1);
     // Q^T fragments: lane (row n, g) holds Q[n][head][32 s + 8 g ..+8] * scale * log2(e)
+    // (rows at or past n_rows repeat the last row: they are never stored)
     half8_t qf[HPW][KS];
     {
         const float mult = scale * kLog2e;
+        const int nq = min(n, n_rows - 1);
 #pragma unroll
         for (int h = 0; h < HPW; h++) {
+            const TQ *qrow = q + (static_cast<int64_t>(nq) * n_q + head0 + h) * HD + 8 * g;
 #pragma unroll
             for (int s = 0; s < KS; s++) {
+                float v[8];
+                attn_load8(qrow + 32 * s, v);
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    float v = 0.0f;
-                    if (n < n_rows)
-                        v = static_cast<float>(q[(static_cast<int64_t>(n) * n_q + head0 + h) * HD + 32 * s + 8 * g + i]);
-                    qf[h][s][i] = static_cast<_Float16>(v * mult);
-                }
+                for (int i = 0; i < 8; i++) qf[h][s][i] = static_cast<_Float16>(v[i] * mult);
             }
         }
     }
 
+    ATT_TR(2);
     float4_t acc[HPW][DT];
 #pragma unroll
     for (int h = 0; h < HPW; h++)
@@ -272,7 +304,9 @@ __global__ void __launch_bounds__(64 * MAXW)
 #pragma unroll
             for (int h = 0; h < HPW; h++) acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[h], acc[h][t], 0, 0, 0);
         }
+        if (st < 8) ATT_TR(3 + st);
     }
+    ATT_TR(12);
 
     // row sums over the four lanes of a row; partials: O^T tile t, lane (row n, g) holds dims 16 t + 4 g + i
 #pragma unroll
@@ -291,7 +325,17 @@ __global__ void __launch_bounds__(64 * MAXW)
             }
         }
     }
+    ATT_TR(13);
 }
+
+#ifdef DFLASH_TRACE
+}  // namespace
+extern "C" void dflash_dbg_set_attn_trace(uint64_t p) {
+    unsigned long long *v = reinterpret_cast<unsigned long long *>(p);
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(g_attn_trace), &v, sizeof(v));
+}
+namespace {
+#endif
 
 // out[row][head][:] = sum_s 2^(m_s - m*) O_s / sum_s 2^(m_s - m*) l_s
 // One workgroup per (head, row): 256 threads = 8 split lanes x 32 dim lanes; a split lane adds up
@@ -423,9 +467,9 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     if (v_layout != 0 && v_layout != 1) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "attn_verify: v_layout");
     if (v_layout == 1 && kv_capacity % 32)
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "attn_verify: transposed V needs a capacity that is a multiple of 32");
-    if (reinterpret_cast<uintptr_t>(k_cache) % 16 || reinterpret_cast<uintptr_t>(v_cache) % 16 ||
-        reinterpret_cast<uintptr_t>(out) % 16)
-        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "attn_verify: K, V and the output must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(k_cache) % 16 ||
+        reinterpret_cast<uintptr_t>(v_cache) % 16 || reinterpret_cast<uintptr_t>(out) % 16)
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "attn_verify: Q, K, V and the output must be 16-byte aligned");
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int group = n_q / n_kv;
@@ -433,11 +477,16 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 
     // KV splits: enough workgroups to cover the chip once or twice, chunks a multiple of 32 keys
     // and at least 128 keys long (a split costs a partial tile per head and row)
-    const int per_cu = n_pos >= 16384 ? 2 : 1;  // short contexts: fewer splits, fewer partial tiles to merge
+    int per_cu = n_pos >= 16384 ? 2 : 1;  // short contexts: fewer splits, fewer partial tiles to merge
+    int64_t min_chunk = 128;
+    if (const char *e = getenv("DFLASH_ATTN_PER_CU")) per_cu = atoi(e);  // tuning knobs
+    if (const char *e = getenv("DFLASH_ATTN_MIN_CHUNK")) min_chunk = atoi(e);
+    if (per_cu < 1) per_cu = 1;
+    if (min_chunk < 32) min_chunk = 32;
     int64_t want = (static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv - 1) / n_kv;
     int64_t chunk = (n_pos + want - 1) / want;
     chunk = (chunk + 31) / 32 * 32;
-    if (chunk < 128) chunk = 128;
+    if (chunk < min_chunk) chunk = min_chunk;
     const int n_splits = static_cast<int>((n_pos + chunk - 1) / chunk);
 
     size_t off = 0;
@@ -458,6 +507,9 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     }
     if (!part_o || !part_ml) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "attn_verify: workspace too small");
 
+#ifdef DFLASH_TRACE
+    if (const char *e = getenv("DFLASH_DBG_VT_STRIDE")) vt_stride = atoi(e);  // timing experiment only: wrong results
+#endif
     const dim3 grid(n_splits, n_kv);
     const int threads = 64 * group;
     const _Float16 *k = static_cast<const _Float16 *>(k_cache);
