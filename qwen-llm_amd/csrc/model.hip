@@ -37,17 +37,56 @@ __device__ float block_sum(float v, float *sh) {
     return r;
 }
 
-// kernel_rms_norm_batched_f32 (attn.metal:35-69): y = x * rsqrt(mean(x^2) + eps) * w, one row per workgroup
-__global__ void __launch_bounds__(256) rms_norm_kernel(const float *__restrict__ x, const float *__restrict__ w,
-                                                       float *__restrict__ y, int n, float eps) {
+// kernel_rms_norm_batched_f32 (attn.metal:35-69), optionally preceded by the residual add that
+// feeds it (kernel_add, elementwise.metal): x += add (add may be null), then
+// y = x * rsqrt(mean(x^2) + eps) * w.  One row per workgroup; a row of up to 4096 values (n a
+// multiple of 4) is read once and stays in registers between the two passes.
+__global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, const float *__restrict__ add,
+                                                       const float *__restrict__ w, float *__restrict__ y, int n,
+                                                       float eps) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
-    const float *xr = x + static_cast<size_t>(blockIdx.x) * n;
+    float *xr = x + static_cast<size_t>(blockIdx.x) * n;
+    const float *ar = add ? add + static_cast<size_t>(blockIdx.x) * n : nullptr;
     float *yr = y + static_cast<size_t>(blockIdx.x) * n;
+    const int tid = threadIdx.x;
+    if (n <= 4096 && n % 4 == 0) {
+        f4 v[4];
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = 4 * (tid + 256 * j);
+            v[j] = f4{0, 0, 0, 0};
+            if (i < n) {
+                v[j] = *reinterpret_cast<const f4 *>(xr + i);
+                if (ar) {
+                    v[j] += *reinterpret_cast<const f4 *>(ar + i);
+                    *reinterpret_cast<f4 *>(xr + i) = v[j];
+                }
+            }
+            s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
+        }
+        s = block_sum(s, sh);
+        const float scale = 1.0f / sqrtf(s / static_cast<float>(n) + eps);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = 4 * (tid + 256 * j);
+            if (i < n) *reinterpret_cast<f4 *>(yr + i) = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
+        }
+        return;
+    }
     float s = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) s += xr[i] * xr[i];
+    for (int i = tid; i < n; i += 256) {
+        float v = xr[i];
+        if (ar) {
+            v += ar[i];
+            xr[i] = v;
+        }
+        s += v * v;
+    }
     s = block_sum(s, sh);
     const float scale = 1.0f / sqrtf(s / static_cast<float>(n) + eps);
-    for (int i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * scale * w[i];
+    for (int i = tid; i < n; i += 256) yr[i] = xr[i] * scale * w[i];
 }
 
 // kernel_qk_rms_norm_rope_f32_packed_consecutive (attn.metal:137-196) + the f32 -> f16 KV scatter
@@ -55,11 +94,21 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(const float *__restrict__
 // NeoX RoPE over the full head (pairs (i, i + hd/2), angle = pos / theta^(2i/hd)).
 // Heads [0, n_q) are queries (rewritten in place, f32); heads [n_q, n_q+n_kv) are keys, written
 // as f16 into k_dst[pos][kv head][:] (k_dst == null: rewritten in place as f32 instead).
+// With vt_dst, n_kv more workgroups per row scatter the row's V heads, as f16, into column
+// pos[row] of the transposed cache [kv head][dim][capacity].
 __global__ void __launch_bounds__(64)
     qk_norm_rope_kernel(float *__restrict__ q, float *__restrict__ k, const float *__restrict__ q_w,
                         const float *__restrict__ k_w, _Float16 *__restrict__ k_dst, const int32_t *__restrict__ pos,
-                        int n_q, int n_kv, int hd, float eps, float theta) {
+                        int n_q, int n_kv, int hd, float eps, float theta, const float *__restrict__ v_src,
+                        _Float16 *__restrict__ vt_dst, int64_t capacity) {
     const int row = blockIdx.y, head = blockIdx.x, lane = threadIdx.x;
+    if (head >= n_q + n_kv) {
+        const int vh = head - n_q - n_kv;
+        const float *src = v_src + (static_cast<size_t>(row) * n_kv + vh) * hd;
+        _Float16 *dst = vt_dst + static_cast<size_t>(vh) * hd * capacity + pos[row];
+        for (int i = lane; i < hd; i += 64) dst[static_cast<size_t>(i) * capacity] = static_cast<_Float16>(src[i]);
+        return;
+    }
     const bool is_q = head < n_q;
     float *v = is_q ? q + (static_cast<size_t>(row) * n_q + head) * hd
                     : k + (static_cast<size_t>(row) * n_kv + (head - n_q)) * hd;
@@ -89,15 +138,6 @@ __global__ void __launch_bounds__(64)
             dst[i + half] = static_cast<_Float16>(rb);
         }
     }
-}
-
-// V rows f32 -> transposed f16 cache [kv head][dim][capacity] at column pos[row]
-__global__ void v_scatter_t_kernel(const float *__restrict__ v, _Float16 *__restrict__ vt, const int32_t *__restrict__ pos,
-                                   int kv_dim, int64_t capacity) {
-    const int row = blockIdx.y;
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= kv_dim) return;
-    vt[static_cast<size_t>(e) * capacity + pos[row]] = static_cast<_Float16>(v[static_cast<size_t>(row) * kv_dim + e]);
 }
 
 // kernel_silu_mul_f32 (elementwise.metal:193): g = silu(g) * u
@@ -320,19 +360,17 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_layer &L = model->layers[il];
         _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
-        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, L.attn_norm, s->cur, H, c.eps);
+        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
         if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, n, st))) return rc;
         if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, n, st))) return rc;
         if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, n, st))) return rc;
-        qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, n), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, kc, s->pos, c.n_q, c.n_kv,
-                                                                  hd, c.eps, c.rope_theta);
-        v_scatter_t_kernel<<<dim3(blocks_for(kv_dim), n), 256, 0, st>>>(s->v, vtc, s->pos, static_cast<int>(kv_dim), s->capacity);
+        qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, kc, s->pos, c.n_q, c.n_kv,
+                                                                      hd, c.eps, c.rope_theta, s->v, vtc, s->capacity);
         if ((rc = dflash_attn_verify_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity,
                                            scale, s->attn, st)))
             return rc;
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
-        add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
-        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, L.post_norm, s->cur, H, c.eps);
+        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps);  // x += mix first
         if (c.n_expert > 0) {
             if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, st))) return rc;
         } else {
@@ -346,7 +384,7 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
             if (tap_layers[t] == il)
                 capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
     }
-    rms_norm_kernel<<<n, 256, 0, st>>>(s->x, model->output_norm, s->cur, H, c.eps);
+    rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, model->output_norm, s->cur, H, c.eps);
     float *lg = logits ? logits : s->logits;
     if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
     int32_t *am = argmax ? argmax : s->argmax;
@@ -462,7 +500,7 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
     for (int64_t c0 = s->ctx_h_ready; c0 < s->ctx_len; c0 += 16) {
         const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
         if ((rc = gemm(ctx, head->fc, s->ctx_raw + c0 * feat, s->tmp, feat, H, m, st))) return rc;
-        rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps);
+        rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, nullptr, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps);
     }
     // phase 2: noise embedding
     int32_t ids_host[16], pos_host[16];
@@ -486,17 +524,17 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
             if ((rc = gemm(ctx, L.wk, s->ctx_h + c0 * H, kc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
             if ((rc = gemm(ctx, L.wv, s->ctx_h + c0 * H, vc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
             qk_norm_rope_kernel<<<dim3(c.n_kv, m), 64, 0, st>>>(nullptr, kc + c0 * kv_dim, nullptr, L.k_norm, nullptr,
-                                                               s->pos_ctx + c0, 0, c.n_kv, hd, c.eps, c.rope_theta);
+                                                               s->pos_ctx + c0, 0, c.n_kv, hd, c.eps, c.rope_theta, nullptr, nullptr, 0);
             if (fast)
                 kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), m), 256, 0, st>>>(kc + c0 * kv_dim, vc + c0 * kv_dim, k16, vt16,
                                                                               static_cast<int>(kv_dim), s->cap16, c0);
         }
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, L.attn_norm, s->cur, H, c.eps);
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
         if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, N, st))) return rc;
         if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, N, st))) return rc;
         if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, N, st))) return rc;
         qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, nullptr, s->pos, c.n_q,
-                                                                  c.n_kv, hd, c.eps, c.rope_theta);
+                                                                  c.n_kv, hd, c.eps, c.rope_theta, nullptr, nullptr, 0);
         if (fast) {
             // the block's own K/V go behind the context in the f16 mirror; one MFMA pass over both
             kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), N), 256, 0, st>>>(s->k, s->v, k16, vt16, static_cast<int>(kv_dim),
@@ -511,15 +549,14 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                                                             L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
         }
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st))) return rc;
-        add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, L.post_norm, s->cur, H, c.eps);
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps);  // x += mix first
         if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, N, st))) return rc;
         if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, N, st))) return rc;
         silu_mul_kernel<<<blocks_for(static_cast<size_t>(N) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(N) * c.ffn);
         if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st))) return rc;
         add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
     }
-    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, head->output_norm, s->cur, H, c.eps);
+    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, head->output_norm, s->cur, H, c.eps);
     float *lg = draft_logits ? draft_logits : s->logits;
     if ((rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st))) return rc;
     int32_t *am = draft_argmax ? draft_argmax : s->argmax;

@@ -19,62 +19,93 @@ namespace {
 
 constexpr int kMaxSlots = 16;  // a row picks an expert at most once, and a block has at most 16 rows
 
-// One workgroup per block row, one thread per expert (n_expert <= 1024): softmax, top-k by rank
-// (an expert's rank = how many experts beat it: higher probability, or equal and lower id), the
-// renormalised weights in pick order, and the shared-expert gate.
+// Routing of a whole block in one workgroup of sixteen waves (n_expert <= 1024, at most 16 rows).
+// Wave w serves block row w: softmax, top-k by rank (an expert's rank = how many experts beat it:
+// higher probability, or equal and lower id), the renormalised weights in pick order, and the
+// shared-expert gate; a row's arithmetic does not depend on how many rows the block has.  Then the
+// whole workgroup lists the block's distinct experts in ascending id order: ids[0 .. n), then one
+// slot with id -1 (the shared expert, which every row uses) if with_shared; *n_slots = n (+ 1); for
+// every (row, k) pick, slot_of = the index of its expert in that list.
 __global__ void __launch_bounds__(1024)
     moe_route_kernel(const float *__restrict__ logits, const float *__restrict__ x, const float *__restrict__ shexp_gate,
-                     int n_expert, int n_used, int hidden, int32_t *__restrict__ sel_e, float *__restrict__ sel_w,
-                     float *__restrict__ sg) {
-    extern __shared__ float probs[];  // [n_expert]
-    __shared__ float red[16];
-    __shared__ float pick_w[64];
-    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
-    const float logit = tid < n_expert ? logits[static_cast<size_t>(row) * n_expert + tid] : -INFINITY;
-    float mx = logit;
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-    if (lane == 0) red[wave] = mx;
-    __syncthreads();
-    mx = red[0];
-    for (int w = 1; w < n_waves; w++) mx = fmaxf(mx, red[w]);
-    __syncthreads();
-    const float ex = tid < n_expert ? expf(logit - mx) : 0.0f;
-    float sum = ex;
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    if (lane == 0) red[wave] = sum;
-    __syncthreads();
-    sum = 0.0f;
-    for (int w = 0; w < n_waves; w++) sum += red[w];
-    const float p = ex * (1.0f / sum);
-    if (tid < n_expert) probs[tid] = p;
-    __syncthreads();
-    if (tid < n_expert) {
-        int rank = 0;
-        for (int e = 0; e < n_expert; e++) {
-            const float q = probs[e];
-            rank += (q > p || (q == p && e < tid)) ? 1 : 0;
+                     int n_rows, int n_expert, int n_used, int hidden, int with_shared, int32_t *__restrict__ sel_e,
+                     float *__restrict__ sel_w, float *__restrict__ sg, int32_t *__restrict__ ids,
+                     int32_t *__restrict__ n_slots, int32_t *__restrict__ slot_of) {
+    extern __shared__ float probs[];  // [16][n_expert], then int32 rank[n_expert]
+    __shared__ float pick_w[16][64];
+    __shared__ int32_t pick_e[16][64];
+    __shared__ int wave_count[16];
+    int32_t *rank = reinterpret_cast<int32_t *>(probs + 16 * n_expert);
+    const int tid = threadIdx.x, lane = tid & 63, row = tid >> 6;
+    const bool live = row < n_rows;
+    float *pr = probs + row * n_expert;
+    if (live) {
+        const float *lg = logits + static_cast<size_t>(row) * n_expert;
+        float mx = -INFINITY;
+        for (int e = lane; e < n_expert; e += 64) mx = fmaxf(mx, lg[e]);
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        float sum = 0.0f;
+        for (int e = lane; e < n_expert; e += 64) {
+            const float ex = expf(lg[e] - mx);
+            pr[e] = ex;
+            sum += ex;
         }
-        if (rank < n_used) {
-            sel_e[row * n_used + rank] = tid;
-            pick_w[rank] = p;
-        }
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        const float inv = 1.0f / sum;
+        for (int e = lane; e < n_expert; e += 64) pr[e] *= inv;
     }
-    // shared-expert gate: sigmoid(x . w)
-    float dot = 0.0f;
-    for (int i = tid; i < hidden; i += blockDim.x) dot += x[static_cast<size_t>(row) * hidden + i] * shexp_gate[i];
-    for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+    if (tid < n_expert) rank[tid] = 0;
     __syncthreads();
-    if (lane == 0) red[wave] = dot;
+    if (live) {
+        for (int e = lane; e < n_expert; e += 64) {
+            const float p = pr[e];
+            int r = 0;
+            for (int o = 0; o < n_expert; o++) {
+                const float q = pr[o];
+                r += (q > p || (q == p && o < e)) ? 1 : 0;
+            }
+            if (r < n_used) {
+                sel_e[row * n_used + r] = e;
+                pick_e[row][r] = e;
+                pick_w[row][r] = p;
+                rank[e] = 1;  // picked by some row
+            }
+        }
+        // shared-expert gate: sigmoid(x . w)
+        const float *xr = x + static_cast<size_t>(row) * hidden;
+        float dot = 0.0f;
+        for (int i = lane; i < hidden; i += 64) dot += xr[i] * shexp_gate[i];
+        for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
+    }
     __syncthreads();
-    if (tid == 0) {
-        float d = 0.0f;
-        for (int w = 0; w < n_waves; w++) d += red[w];
-        sg[row] = 1.0f / (1.0f + expf(-d));
+    if (live && lane == 0) {
         float wsum = 0.0f;
-        for (int k = 0; k < n_used; k++) wsum += pick_w[k];  // in pick order, as the reference sums them
-        wsum = fmaxf(wsum, 6.103515625e-05f);               // 2^-14
-        for (int k = 0; k < n_used; k++) sel_w[row * n_used + k] = pick_w[k] / wsum;
+        for (int k = 0; k < n_used; k++) wsum += pick_w[row][k];  // in pick order, as the reference sums them
+        wsum = fmaxf(wsum, 6.103515625e-05f);                     // 2^-14
+        for (int k = 0; k < n_used; k++) sel_w[row * n_used + k] = pick_w[row][k] / wsum;
     }
+    // distinct experts of the block
+    const bool picked = tid < n_expert && rank[tid] != 0;
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(picked);
+    if (lane == 0) wave_count[row] = __popcll(mask);
+    __syncthreads();
+    int base = 0, total = 0;
+    for (int w = 0; w < 16; w++) {
+        if (w < row) base += wave_count[w];
+        total += wave_count[w];
+    }
+    if (picked) {
+        const int idx = base + __popcll(mask & ((1ull << lane) - 1));
+        ids[idx] = tid;
+        rank[tid] = idx;
+    }
+    if (tid == 0) {
+        if (with_shared) ids[total] = -1;
+        *n_slots = total + (with_shared ? 1 : 0);
+    }
+    __syncthreads();
+    if (live && lane < n_used) slot_of[row * n_used + lane] = rank[pick_e[row][lane]];
 }
 
 // Collects the slots whose pick is `expert`; returns the count (uniform over the workgroup).
@@ -171,41 +202,6 @@ __global__ void silu_mul_rows_kernel(float *__restrict__ g, const float *__restr
     }
 }
 
-// Distinct experts of the block, in ascending id order: ids[0 .. n), then one slot with id -1 (the
-// shared expert, which every row uses) if with_shared; *n_slots = n (+ 1).  For every (row, k) pick,
-// slot_of = the index of its expert in that list.  One workgroup, one thread per expert.
-__global__ void __launch_bounds__(1024)
-    moe_lists_kernel(const int32_t *__restrict__ sel_e, int n_picks, int n_expert, int with_shared,
-                     int32_t *__restrict__ ids, int32_t *__restrict__ n_slots, int32_t *__restrict__ slot_of) {
-    extern __shared__ int32_t rank[];  // [n_expert]: picked flag, then the expert's index in the list
-    __shared__ int wave_count[16];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
-    if (tid < n_expert) rank[tid] = 0;
-    __syncthreads();
-    for (int s = tid; s < n_picks; s += blockDim.x) rank[sel_e[s]] = 1;
-    __syncthreads();
-    const bool picked = tid < n_expert && rank[tid] != 0;
-    const unsigned long long mask = __builtin_amdgcn_ballot_w64(picked);
-    if (lane == 0) wave_count[wave] = __popcll(mask);
-    __syncthreads();
-    int base = 0, total = 0;
-    for (int w = 0; w < n_waves; w++) {
-        if (w < wave) base += wave_count[w];
-        total += wave_count[w];
-    }
-    if (picked) {
-        const int idx = base + __popcll(mask & ((1ull << lane) - 1));
-        ids[idx] = tid;
-        rank[tid] = idx;
-    }
-    if (tid == 0) {
-        if (with_shared) ids[total] = -1;
-        *n_slots = total + (with_shared ? 1 : 0);
-    }
-    __syncthreads();
-    for (int s = tid; s < n_picks; s += blockDim.x) slot_of[s] = rank[sel_e[s]];
-}
-
 // g = silu(g) * u over the first *n_distinct slots of [slot][16][f]
 __global__ void silu_mul_slots_kernel(float *__restrict__ g, const float *__restrict__ u, const int32_t *__restrict__ n_distinct,
                                       size_t per_slot) {
@@ -256,23 +252,28 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     int32_t rc = dflash_gemm_fewrow(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
     if (rc) return rc;
     if (E > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: %d experts (at most 1024)", E);
-    const int route_threads = (E + 63) / 64 * 64;
-    moe_route_kernel<<<n, route_threads, E * sizeof(float), st>>>(s.probs, cur, L.shexp_gate, E, used, H, s.sel_e, s.sel_w, s.sg);
-
-    bool folded_shared = false;
     const bool batched = et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K && H % DFL_QK_K == 0 && fe % DFL_QK_K == 0 &&
                          !getenv("DFLASH_MOE_PERSLOT");
+    // the shared expert rides along as one more slot of the batched GEMMs when it has the experts' shape
+    const bool folded_shared = batched && fs == fe && L.gate.type == DFLASH_TYPE_Q4_K && L.up.type == DFLASH_TYPE_Q4_K &&
+                               L.down.type == DFLASH_TYPE_Q4_K;
+    const size_t route_lds = static_cast<size_t>(17) * E * sizeof(float);
+    if (route_lds > 48 * 1024) {
+        static bool attr = false;
+        if (!attr) {
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(moe_route_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 1024 * sizeof(float)));
+            attr = true;
+        }
+    }
+    moe_route_kernel<<<1, 1024, route_lds, st>>>(s.probs, cur, L.shexp_gate, n, E, used, H, folded_shared ? 1 : 0,
+                                                                   s.sel_e, s.sel_w, s.sg, s.ids, s.n_distinct, s.slot_of);
     if (batched) {
         // the selected experts' matrices form one streaming GEMM each for gate, up and down: every
         // distinct expert's weights are read once, with all block rows riding along on the MFMA;
         // no split K, so a row's result is the same whichever other experts the block uses
-        // the shared expert rides along as one more slot when it has the experts' shape
-        const bool fold = fs == fe && L.gate.type == DFLASH_TYPE_Q4_K && L.up.type == DFLASH_TYPE_Q4_K &&
-                          L.down.type == DFLASH_TYPE_Q4_K;
-        folded_shared = fold;
+        const bool fold = folded_shared;
         const int max_slots = (n_slots < E ? n_slots : E) + (fold ? 1 : 0);
-        moe_lists_kernel<<<1, route_threads, E * sizeof(int32_t), st>>>(s.sel_e, n_slots, E, fold ? 1 : 0, s.ids, s.n_distinct,
-                                                                       s.slot_of);
         const size_t per_slot = static_cast<size_t>(16) * fe;
         if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, static_cast<size_t>(fe) * rb_in, fold ? L.gate.data : nullptr, s.ids,
                                        s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, per_slot, H, fe, n, 1, st)))
