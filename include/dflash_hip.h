@@ -75,6 +75,14 @@ void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable);
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms_host,
                                  int64_t *launches_host);
 
+/* Graph replay of the packed verify (the counterpart of the reference's one command buffer per
+ * verify block, encode_packed_verify_layer_major, metal_dflash.rs:10696-10719): a verify shape
+ * (model tensors, row count, taps, output pointers) is run launch by launch the first time,
+ * captured into a HIP graph the second time and replayed from then on, with the position read
+ * from device memory.  On by default (environment DFLASH_GRAPHS=0 turns it off); results are
+ * bit-identical either way.  Kernel timers switch it off while they are enabled. */
+void dflash_ctx_set_graphs(dflash_ctx *ctx, int32_t enable);
+
 /* ---- block dequantisation -------------------------------------------------------
  * codec::dequant_to_f32{,_into,_in_place} (codec.rs:256-302): ggml blocks -> f32,
  * bit-exact with ggml's dequantize_row_{q4_K,q6_K,q8_0}.  n_elems must be a multiple
@@ -241,6 +249,9 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
                               dflash_session **out);
 void dflash_session_destroy(dflash_session *s);
 int64_t dflash_session_kv_n_pos(const dflash_session *s);
+/* How many verify calls of this session were served by replaying a captured graph (see
+ * dflash_ctx_set_graphs); no counterpart in the reference, used by tests and benchmarks. */
+int64_t dflash_session_graph_replays(const dflash_session *session);
 
 /* encode_packed_verify_layer_major_inner(base, target_layer_ids, tokens, start_position, ...,
  * debug_logits_dst, n_eff_override) (metal_dflash.rs:10696-10719): forward of tokens[n] at

@@ -91,6 +91,8 @@ def _declare(L):
     L.dflash_version.restype = C.c_char_p
     L.dflash_ctx_set_kernel_timing.restype = None
     L.dflash_ctx_set_kernel_timing.argtypes = [vp, i32]
+    L.dflash_ctx_set_graphs.restype = None
+    L.dflash_ctx_set_graphs.argtypes = [vp, i32]
     L.dflash_ctx_kernel_timing.restype = i32
     L.dflash_ctx_kernel_timing.argtypes = [vp, i32, C.POINTER(C.c_double), C.POINTER(i64)]
     L.dflash_row_bytes.restype = sz
@@ -216,6 +218,10 @@ class Context:
 
     def set_kernel_timing(self, enable: bool):
         self._lib.dflash_ctx_set_kernel_timing(self._h, int(enable))
+
+    def set_graphs(self, enable: bool):
+        """Graph replay of the packed verify on or off (on by default; results are the same)."""
+        self._lib.dflash_ctx_set_graphs(self._h, int(enable))
 
     def kernel_timing(self, slot: int):
         ms, n = C.c_double(), C.c_int64()

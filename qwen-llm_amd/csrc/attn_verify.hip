@@ -27,6 +27,7 @@
 #include "common.h"
 
 #include <cmath>
+#include <algorithm>
 #include <cstdlib>
 
 namespace {
@@ -61,6 +62,16 @@ __device__ __forceinline__ int attn_swz(int r) { return (r & 3) | ((r >> 1) & 4)
 // MAXW = most waves a workgroup may have; it sets the register budget.  HPW = query heads per wave:
 // with two, every K and V^T fragment read from LDS feeds two MFMAs (half the LDS traffic per head,
 // and two independent dependency chains per wave).
+// Keys per KV split for n_pos visible positions: an even share of `want` splits, rounded up to
+// whole 32-key stages, at least min_chunk.  Host and kernels use the same rule, so a launch whose
+// context length is only known on the device (a captured graph) can size its grid for the largest
+// context and let surplus workgroups leave.
+__host__ __device__ __forceinline__ int64_t attn_chunk(int64_t n_pos, int64_t want, int64_t min_chunk) {
+    int64_t chunk = (n_pos + want - 1) / want;
+    chunk = (chunk + 31) / 32 * 32;
+    return chunk < min_chunk ? min_chunk : chunk;
+}
+
 // eight consecutive query values (16-byte aligned) as floats
 __device__ __forceinline__ void attn_load8(const float *p, float v[8]) {
     const float4_t a = *reinterpret_cast<const float4_t *>(p), b = *reinterpret_cast<const float4_t *>(p + 4);
@@ -94,8 +105,8 @@ template <int HD, typename TQ, int MAXW, int HPW>
 __global__ void __launch_bounds__(64 * MAXW)
     attn_split_kernel(const TQ *__restrict__ q, const _Float16 *__restrict__ k_cache,
                       const _Float16 *__restrict__ vt_cache, float *__restrict__ part_o, float *__restrict__ part_ml,
-                      int64_t ctx_len, int n_rows, int n_q, int n_kv, int64_t vt_stride, int64_t chunk, float scale,
-                      int full_block, int64_t window) {
+                      int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int n_rows, int n_q, int n_kv,
+                      int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window) {
     constexpr int KS = HD / 32;       // k-steps of the score product
     constexpr int DT = HD / 16;       // 16-dim tiles of the output
     constexpr int CH = HD / 8;        // 16-byte chunks per key row
@@ -110,7 +121,10 @@ __global__ void __launch_bounds__(64 * MAXW)
     const int kvh = blockIdx.y;
     const int split = blockIdx.x;
     const int head0 = kvh * group + wave * HPW;  // this wave serves heads head0 .. head0 + HPW - 1
+    if (ctx_len_dev) ctx_len = *ctx_len_dev;
     const int64_t n_pos = ctx_len + n_rows;
+    const int64_t chunk = attn_chunk(n_pos, want, min_chunk);
+    if (split * chunk >= n_pos) return;  // the grid is sized for the longest context
     const int64_t c0 = split * chunk;
     const int64_t c1 = min(n_pos, c0 + chunk);
     const int n_steps = static_cast<int>((c1 - c0 + 31) / 32);
@@ -342,7 +356,12 @@ namespace {
 // every eighth split (float4 per dim lane, all loads independent), then the eight are summed in LDS.
 __global__ void __launch_bounds__(256)
     attn_combine_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml, float *__restrict__ out,
-                        int n_rows, int n_q, int hd, int n_splits) {
+                        int n_rows, int n_q, int hd, int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int want,
+                        int min_chunk) {
+    if (ctx_len_dev) ctx_len = *ctx_len_dev;
+    const int64_t n_pos = ctx_len + n_rows;
+    const int64_t chunk = attn_chunk(n_pos, want, min_chunk);
+    const int n_splits = static_cast<int>((n_pos + chunk - 1) / chunk);
     __shared__ float wgt[1024];          // 2^(m_s - m*) per split (n_splits <= 1024)
     __shared__ float red[8][256 + 4];    // partial outputs per split lane
     __shared__ float red_l[8];
@@ -413,8 +432,8 @@ __global__ void __launch_bounds__(256) transpose_v_kernel(const _Float16 *__rest
 
 template <int HD, typename TQ>
 void launch_split(dim3 grid, int threads, hipStream_t st, const void *q, const _Float16 *k, const _Float16 *vt,
-                  float *po, float *pml, int64_t ctx_len, int n_rows, int n_q, int n_kv, int64_t vt_stride,
-                  int64_t chunk, float scale, int full_block, int64_t window) {
+                  float *po, float *pml, int64_t ctx_len, const int32_t *ctx_len_dev, int n_rows, int n_q, int n_kv,
+                  int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window) {
     const size_t lds = static_cast<size_t>(kAttnBufs) * 2 * (32 * HD / 8) * sizeof(half8_t);
 #define DFL_ATTN_LAUNCH(MAXW, HPW)                                                                                  \
     do {                                                                                                            \
@@ -425,8 +444,9 @@ void launch_split(dim3 grid, int threads, hipStream_t st, const void *q, const _
             attr = true;                                                                                            \
         }                                                                                                           \
         attn_split_kernel<HD, TQ, MAXW, HPW><<<grid, threads / HPW, lds, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, \
-                                                                              ctx_len, n_rows, n_q, n_kv, vt_stride, \
-                                                                              chunk, scale, full_block, window);   \
+                                                                              ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
+                                                                              vt_stride, want, min_chunk, scale,    \
+                                                                              full_block, window);                  \
     } while (0)
     // one head per wave: two (HPW = 2) halve the LDS reads per head but measured slower on MI355X
     // (fewer waves to hide the per-stage dependency chain)
@@ -444,13 +464,13 @@ extern "C" int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int3
                                             int32_t n_q, int32_t n_kv, int32_t head_dim, int64_t kv_capacity,
                                             float scale, float *out, dflash_stream_t stream) {
     return dfl_attn_block(ctx, q, q_type, k_cache, v_cache, v_layout, ctx_len, n_rows, n_q, n_kv, head_dim, kv_capacity,
-                          scale, out, stream, 0, 0);
+                          scale, out, stream, 0, 0, nullptr);
 }
 
 int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
-                       int64_t window) {
+                       int64_t window, const int32_t *ctx_len_dev) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!q || !k_cache || !v_cache || !out) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "attn_verify: null pointer");
     if (n_rows < 1 || n_rows > 16) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: n_rows %d outside 1..16", n_rows);
@@ -465,6 +485,8 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     if (q_type != DFLASH_TYPE_F32 && q_type != DFLASH_TYPE_F16)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: queries must be f32 or f16");
     if (v_layout != 0 && v_layout != 1) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "attn_verify: v_layout");
+    if (ctx_len_dev && v_layout != 1)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: a device-side context length needs the transposed V cache");
     if (v_layout == 1 && kv_capacity % 32)
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "attn_verify: transposed V needs a capacity that is a multiple of 32");
     if (reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(k_cache) % 16 ||
@@ -473,7 +495,9 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int group = n_q / n_kv;
-    const int64_t n_pos = ctx_len + n_rows;
+    // with ctx_len_dev the context length is read on the device (ctx_len is then only an upper
+    // bound): everything sized here is sized for the whole cache
+    const int64_t n_pos = ctx_len_dev ? kv_capacity : ctx_len + n_rows;
 
     // KV splits: enough workgroups to cover the chip once or twice, chunks a multiple of 32 keys
     // and at least 128 keys long (a split costs a partial tile per head and row)
@@ -483,11 +507,11 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     if (const char *e = getenv("DFLASH_ATTN_MIN_CHUNK")) min_chunk = atoi(e);
     if (per_cu < 1) per_cu = 1;
     if (min_chunk < 32) min_chunk = 32;
-    int64_t want = (static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv - 1) / n_kv;
-    int64_t chunk = (n_pos + want - 1) / want;
-    chunk = (chunk + 31) / 32 * 32;
-    if (chunk < min_chunk) chunk = min_chunk;
-    const int n_splits = static_cast<int>((n_pos + chunk - 1) / chunk);
+    const int want = static_cast<int>((static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv - 1) / n_kv);
+    // most splits any context up to n_pos can have
+    const int n_splits = ctx_len_dev
+                             ? static_cast<int>(std::min<int64_t>(want, (n_pos + min_chunk - 1) / min_chunk))
+                             : static_cast<int>((n_pos + attn_chunk(n_pos, want, min_chunk) - 1) / attn_chunk(n_pos, want, min_chunk));
 
     size_t off = 0;
     float *part_o = dfl_ws_take<float>(ctx, &off, static_cast<size_t>(n_splits) * n_q * 16 * head_dim * sizeof(float));
@@ -517,11 +541,11 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
         dfl_timed timer(ctx, st, DFL_T_ATTN);
 #define DFL_ATTN(HD)                                                                                              \
     if (q_type == DFLASH_TYPE_F32)                                                                                \
-        launch_split<HD, float>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, n_rows, n_q, n_kv, vt_stride, \
-                                chunk, scale, full_block, window);                                                \
+        launch_split<HD, float>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
+                                vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window);         \
     else                                                                                                          \
-        launch_split<HD, _Float16>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, n_rows, n_q, n_kv,      \
-                                   vt_stride, chunk, scale, full_block, window)
+        launch_split<HD, _Float16>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, \
+                                   n_kv, vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window)
         if (head_dim == 64) {
             DFL_ATTN(64);
         } else if (head_dim == 128) {
@@ -532,7 +556,8 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 #undef DFL_ATTN
     }
     if (n_splits > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: %d KV splits", n_splits);
-    attn_combine_kernel<<<dim3(n_q, n_rows), 256, 0, st>>>(part_o, part_ml, out, n_rows, n_q, head_dim, n_splits);
+    attn_combine_kernel<<<dim3(n_q, n_rows), 256, 0, st>>>(part_o, part_ml, out, n_rows, n_q, head_dim, ctx_len, ctx_len_dev, want,
+                                                          static_cast<int>(min_chunk));
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

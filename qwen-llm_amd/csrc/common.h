@@ -25,6 +25,12 @@ struct dflash_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     double timed_ms[8] = {0};
     int64_t timed_launches[8] = {0};
+    // captured-graph replay of the packed verify: a stream of the library's own to capture on and
+    // launch into (the caller's may be the legacy default stream, which cannot be captured) and
+    // the two events that order it against the caller's stream
+    bool graphs = true;
+    hipStream_t gstream = nullptr;
+    hipEvent_t g_in = nullptr, g_out = nullptr;
 };
 
 // Slots of the per-kernel timers.
@@ -95,11 +101,14 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_l
                     const dfl_moe_scratch &scratch, float *x_resid, hipStream_t stream);
 
 // dflash_attn_verify_block with the drafter's masks: full_block != 0 lets every row see the whole
-// block (non-causal), window > 0 keeps only keys with |distance| < window.
+// block (non-causal), window > 0 keeps only keys with |distance| < window.  ctx_len_dev != null:
+// the context length is read from that device word when the kernels run (ctx_len is then only
+// checked as an upper bound, launches are sized for the whole cache), so that the call can sit
+// in a captured graph that is replayed at other positions.
 int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
-                       int64_t window);
+                       int64_t window, const int32_t *ctx_len_dev);
 
 // Few-row Q4_K GEMM over the matrices that the device-side list ids[0 .. *n_slots) picks out of a stack
 // (w_stack + id * w_stride_bytes; id -1 = extra_w): slot j reads activations x + j * x_stride (elements; 0 = shared) and

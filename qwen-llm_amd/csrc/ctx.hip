@@ -1,6 +1,7 @@
 // Context lifetime, error reporting and block geometry of libdflash_hip.
 #include "common.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -44,10 +45,14 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
             return DFLASH_ERR_HIP;
         }
     }
-    if (hipEventCreate(&ctx->ev0) != hipSuccess || hipEventCreate(&ctx->ev1) != hipSuccess) {
+    if (hipEventCreate(&ctx->ev0) != hipSuccess || hipEventCreate(&ctx->ev1) != hipSuccess ||
+        hipStreamCreateWithFlags(&ctx->gstream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&ctx->g_in, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&ctx->g_out, hipEventDisableTiming) != hipSuccess) {
         dflash_ctx_destroy(ctx);
         return DFLASH_ERR_HIP;
     }
+    if (const char *e = getenv("DFLASH_GRAPHS")) ctx->graphs = atoi(e) != 0;
     *out = ctx;
     return DFLASH_OK;
 }
@@ -58,6 +63,9 @@ void dflash_ctx_destroy(dflash_ctx *ctx) {
     if (ctx->partials) (void)hipFree(ctx->partials);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    if (ctx->g_in) (void)hipEventDestroy(ctx->g_in);
+    if (ctx->g_out) (void)hipEventDestroy(ctx->g_out);
+    if (ctx->gstream) (void)hipStreamDestroy(ctx->gstream);
     delete ctx;
 }
 
@@ -68,6 +76,10 @@ void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable) {
         ctx->timed_ms[i] = 0.0;
         ctx->timed_launches[i] = 0;
     }
+}
+
+void dflash_ctx_set_graphs(dflash_ctx *ctx, int32_t enable) {
+    if (ctx) ctx->graphs = enable != 0;
 }
 
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms, int64_t *launches) {

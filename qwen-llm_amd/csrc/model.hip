@@ -10,6 +10,7 @@
 #include "device_quant.h"
 
 #include <algorithm>
+#include <map>
 #include <chrono>
 #include <cmath>
 #include <cstring>
@@ -243,6 +244,13 @@ struct dflash_session {
     float *hidden = nullptr;  // [16][n_taps][hidden] capture slots of the speculative step
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
     dfl_moe_scratch moe;
+    // Captured graphs of the packed verify, one per distinct call shape (a hash over the model's
+    // tensors, the row count, the taps and the output pointers).  A shape is run eagerly the first
+    // time, captured the second time and replayed from then on: everything position-dependent is
+    // read from device memory (pos[], written before each launch), nothing else changes.
+    std::map<uint64_t, hipGraphExec_t> graphs;
+    std::map<uint64_t, int> graph_seen;
+    int64_t graph_replays = 0;
 };
 
 struct dflash_draft_session {
@@ -312,6 +320,8 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
 
 void dflash_session_destroy(dflash_session *s) {
     if (!s) return;
+    for (auto &g : s->graphs)
+        if (g.second) (void)hipGraphExecDestroy(g.second);
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
                     s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax, s->hidden,
                     s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared,
@@ -322,6 +332,74 @@ void dflash_session_destroy(dflash_session *s) {
 }
 
 int64_t dflash_session_kv_n_pos(const dflash_session *s) { return s ? s->kv_n_pos : -1; }
+
+int64_t dflash_session_graph_replays(const dflash_session *s) { return s ? s->graph_replays : -1; }
+
+namespace {
+
+// 64-bit mix over a byte range (FNV-1a on 8-byte words, tail bytes one by one)
+uint64_t hash_bytes(const void *p, size_t n, uint64_t h) {
+    const uint8_t *b = static_cast<const uint8_t *>(p);
+    size_t i = 0;
+    for (; i + 8 <= n; i += 8) {
+        uint64_t w;
+        memcpy(&w, b + i, 8);
+        h = (h ^ w) * 0x100000001b3ull;
+        h ^= h >> 29;
+    }
+    for (; i < n; i++) h = (h ^ b[i]) * 0x100000001b3ull;
+    return h;
+}
+
+// Every launch of one packed verify, from the embedding rows to the argmax, on `st`: no host
+// reads, no synchronisation, nothing that depends on the position except through pos[] on the
+// device, so the sequence can be captured once and replayed.
+int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, int32_t n, int64_t start,
+                       const int32_t *tap_layers, int32_t n_taps, float *hidden_capture, float *lg, int32_t *am, float *gp,
+                       hipStream_t st) {
+    const dflash_model_cfg &c = model->cfg;
+    const int H = c.hidden, hd = c.head_dim;
+    const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
+    int32_t rc = embed_rows(ctx, model->token_embd, s->ids, n, H, s->x, st);
+    if (rc) return rc;
+    const float scale = 1.0f / sqrtf(static_cast<float>(hd));
+    const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
+    for (int il = 0; il < c.n_layers; il++) {
+        const dflash_layer &L = model->layers[il];
+        _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
+        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
+        if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, n, st))) return rc;
+        if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, n, st))) return rc;
+        if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, n, st))) return rc;
+        qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, kc, s->pos, c.n_q, c.n_kv,
+                                                                      hd, c.eps, c.rope_theta, s->v, vtc, s->capacity);
+        // the context length is read from pos[0] on the device: the same launches serve every position
+        if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity, scale,
+                                 s->attn, st, 0, 0, s->pos)))
+            return rc;
+        if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
+        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps);  // x += mix first
+        if (c.n_expert > 0) {
+            if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, st))) return rc;
+        } else {
+            if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, n, st))) return rc;
+            if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, n, st))) return rc;
+            silu_mul_kernel<<<blocks_for(static_cast<size_t>(n) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(n) * c.ffn);
+            if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
+            add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
+        }
+        for (int t = 0; t < n_taps; t++)
+            if (tap_layers[t] == il)
+                capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
+    }
+    rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, model->output_norm, s->cur, H, c.eps);
+    if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
+    if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gp, st))) return rc;
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+}  // namespace
 
 int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
                             int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps, int32_t *argmax,
@@ -347,49 +425,55 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
     if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "verify_block: session/model shape mismatch");
 
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int H = c.hidden, hd = c.head_dim;
-    const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
     int32_t pos_host[16];
     for (int i = 0; i < n; i++) pos_host[i] = static_cast<int32_t>(start + i);
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ids, tokens, n * sizeof(int32_t), hipMemcpyHostToDevice, st));
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos, pos_host, n * sizeof(int32_t), hipMemcpyHostToDevice, st));
-    int32_t rc = embed_rows(ctx, model->token_embd, s->ids, n, H, s->x, st);
-    if (rc) return rc;
-    const float scale = 1.0f / sqrtf(static_cast<float>(hd));
-    const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
-    for (int il = 0; il < c.n_layers; il++) {
-        const dflash_layer &L = model->layers[il];
-        _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
-        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
-        if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, n, st))) return rc;
-        if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, n, st))) return rc;
-        if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, n, st))) return rc;
-        qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, kc, s->pos, c.n_q, c.n_kv,
-                                                                      hd, c.eps, c.rope_theta, s->v, vtc, s->capacity);
-        if ((rc = dflash_attn_verify_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity,
-                                           scale, s->attn, st)))
-            return rc;
-        if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
-        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps);  // x += mix first
-        if (c.n_expert > 0) {
-            if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, st))) return rc;
-        } else {
-            if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, n, st))) return rc;
-            if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, n, st))) return rc;
-            silu_mul_kernel<<<blocks_for(static_cast<size_t>(n) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(n) * c.ffn);
-            if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
-            add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
-        }
-        for (int t = 0; t < n_taps; t++)
-            if (tap_layers[t] == il)
-                capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
-    }
-    rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, model->output_norm, s->cur, H, c.eps);
     float *lg = logits ? logits : s->logits;
-    if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
     int32_t *am = argmax ? argmax : s->argmax;
-    if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gap ? gap : s->gap, st))) return rc;
-    DFL_HIP_CHECK(ctx, hipGetLastError());
+    float *gp = gap ? gap : s->gap;
+    int32_t rc = DFLASH_OK;
+    const bool use_graph = ctx->graphs && !ctx->timing && ctx->gstream;
+    uint64_t key = 0;
+    if (use_graph) {
+        key = hash_bytes(model, sizeof(*model), 0x9e3779b97f4a7c15ull);
+        key = hash_bytes(model->layers, sizeof(dflash_layer) * c.n_layers, key);
+        const uintptr_t outs[4] = {reinterpret_cast<uintptr_t>(hidden_capture), reinterpret_cast<uintptr_t>(lg),
+                                   reinterpret_cast<uintptr_t>(am), reinterpret_cast<uintptr_t>(gp)};
+        key = hash_bytes(outs, sizeof(outs), key);
+        const int32_t shape[2] = {n, n_taps};
+        key = hash_bytes(shape, sizeof(shape), key);
+        if (n_taps > 0) key = hash_bytes(tap_layers, sizeof(int32_t) * n_taps, key);
+    }
+    auto exec_it = use_graph ? s->graphs.find(key) : s->graphs.end();
+    if (use_graph && exec_it == s->graphs.end() && s->graph_seen.size() > 256) s->graph_seen.clear();
+    if (use_graph && exec_it == s->graphs.end() && s->graphs.size() < 16 && s->graph_seen[key]++ >= 1) {
+        // second call of this shape: capture it
+        hipGraph_t graph = nullptr;
+        DFL_HIP_CHECK(ctx, hipStreamBeginCapture(ctx->gstream, hipStreamCaptureModeThreadLocal));
+        rc = verify_enqueue(ctx, model, s, n, start, tap_layers, n_taps, hidden_capture, lg, am, gp, ctx->gstream);
+        const hipError_t end = hipStreamEndCapture(ctx->gstream, &graph);
+        if (rc) {
+            if (graph) (void)hipGraphDestroy(graph);
+            return rc;
+        }
+        DFL_HIP_CHECK(ctx, end);
+        hipGraphExec_t exec = nullptr;
+        const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        DFL_HIP_CHECK(ctx, inst);
+        exec_it = s->graphs.emplace(key, exec).first;
+    }
+    if (exec_it != s->graphs.end()) {
+        DFL_HIP_CHECK(ctx, hipEventRecord(ctx->g_in, st));
+        DFL_HIP_CHECK(ctx, hipStreamWaitEvent(ctx->gstream, ctx->g_in, 0));
+        DFL_HIP_CHECK(ctx, hipGraphLaunch(exec_it->second, ctx->gstream));
+        s->graph_replays++;
+        DFL_HIP_CHECK(ctx, hipEventRecord(ctx->g_out, ctx->gstream));
+        DFL_HIP_CHECK(ctx, hipStreamWaitEvent(st, ctx->g_out, 0));
+    } else if ((rc = verify_enqueue(ctx, model, s, n, start, tap_layers, n_taps, hidden_capture, lg, am, gp, st))) {
+        return rc;
+    }
     s->kv_n_pos = start + n;
     if (argmax_host) {
         DFL_HIP_CHECK(ctx, hipMemcpyAsync(argmax_host, am, n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
@@ -541,7 +625,7 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                                                                           s->cap16, s->ctx_len);
             if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, k16, vt16, 1, s->ctx_len, N, c.n_q, c.n_kv, hd, s->cap16,
                                      1.0f / sqrtf(static_cast<float>(hd)), s->attn, st, c.causal ? 0 : 1,
-                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0)))
+                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, nullptr)))
                 return rc;
         } else {
             draft_attn_kernel<<<dim3(c.n_q, N), 64, 0, st>>>(s->q, kc, vc, s->k, s->v, s->pos_ctx, static_cast<int>(s->ctx_len),

@@ -109,6 +109,8 @@ def _lib():
         L.dflash_session_destroy.argtypes = [vp]
         L.dflash_session_kv_n_pos.restype = i64
         L.dflash_session_kv_n_pos.argtypes = [vp]
+        L.dflash_session_graph_replays.restype = i64
+        L.dflash_session_graph_replays.argtypes = [vp]
         L.dflash_verify_block.restype = i32
         L.dflash_verify_block.argtypes = [vp, C.POINTER(ModelC), vp, C.POINTER(i32), i32, i64, C.POINTER(i32), i32, vp,
                                           vp, vp, vp, C.POINTER(i32), vp]
@@ -349,6 +351,10 @@ class Session:
             gap.data_ptr(), hidden.data_ptr() if hidden is not None else None,
             logits.data_ptr() if logits is not None else None, host, _stream_ptr()))
         return VerifyOutput(argmax[:n], gap[:n], hidden, logits, list(host[:n]) if sync else None)
+
+    @property
+    def graph_replays(self) -> int:
+        return int(self._L.dflash_session_graph_replays(self._h))
 
     def encode_restore_after_partial_accept(self, start_position: int, n: int, n_keep: int):
         self.ctx._check(self._L.dflash_restore(self.ctx._h, self._h, start_position, n, n_keep))

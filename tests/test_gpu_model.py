@@ -232,3 +232,50 @@ def test_draft_block_general_positions(ctx, oracle, target):
     close(logits.cpu().numpy(), want, "draft logits, general positions")
     dsess.close()
     sess.close()
+
+
+def test_graph_replay_is_bit_identical_to_launch_by_launch(ctx, target):
+    """The packed verify replayed from a captured graph (second and later calls of a shape) against
+    the same calls made launch by launch: logits, hidden capture, argmax and gap bit for bit, at
+    moving positions, with a rollback and single-row calls in between and other GPU work and
+    synchronisations between the replays."""
+    import torch
+
+    model, _ = target
+    rng = np.random.default_rng(21)
+    cap = 320
+    blocks = [rng.integers(0, C1.vocab, 16).tolist() for _ in range(8)]
+    singles = rng.integers(0, C1.vocab, 8).tolist()
+
+    def run(graphs):
+        ctx.set_graphs(graphs)
+        sess = dfl.Session(ctx, model, cap, TAPS)
+        outs, pos = [], 0
+        scratch = torch.zeros(1 << 20, device="cuda")
+        for i, blk in enumerate(blocks):
+            o = sess.encode_packed_verify_layer_major(blk, pos, want_logits=True)
+            outs.append((o.logits.cpu().numpy(), o.hidden_capture.cpu().numpy(), o.argmax.cpu().numpy(), o.gap.cpu().numpy()))
+            del o
+            scratch += float(i)  # the program's own eager work between replays
+            torch.cuda.synchronize()
+            keep = 16 if i % 3 else 5  # partial accept: roll the cache back
+            sess.encode_restore_after_partial_accept(pos, 16, keep)
+            pos += keep
+            o = sess.encode_packed_verify_layer_major([singles[i]], pos, want_logits=True)
+            outs.append((o.logits.cpu().numpy(), o.hidden_capture.cpu().numpy(), o.argmax.cpu().numpy(), o.gap.cpu().numpy()))
+            del o
+            pos += 1
+        replays = sess.graph_replays
+        return outs, replays
+
+    try:
+        eager, r0 = run(False)
+        replay, r1 = run(True)
+    finally:
+        ctx.set_graphs(True)
+    assert r0 == 0
+    assert r1 >= 8, f"only {r1} of 16 calls were graph replays"
+    for i, (a, b) in enumerate(zip(eager, replay)):
+        for x, y, name in zip(a, b, ("logits", "hidden", "argmax", "gap")):
+            assert np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
+                                  y.view(np.uint32) if y.dtype == np.float32 else y), f"call {i}: {name} differs under graph replay"
