@@ -79,7 +79,8 @@ int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *to
  * verify block, encode_packed_verify_layer_major, metal_dflash.rs:10696-10719): a verify shape
  * (model tensors, row count, taps, output pointers) is run launch by launch the first time,
  * captured into a HIP graph the second time and replayed from then on, with the position read
- * from device memory.  On by default (environment DFLASH_GRAPHS=0 turns it off); results are
+ * from device memory.  Off by default (environment DFLASH_GRAPHS=1 or this call turn it on):
+ * on ROCm 7.2 a replay measured slightly slower than the launches it replaces; results are
  * bit-identical either way.  Kernel timers switch it off while they are enabled. */
 void dflash_ctx_set_graphs(dflash_ctx *ctx, int32_t enable);
 

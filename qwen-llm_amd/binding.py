@@ -220,7 +220,7 @@ class Context:
         self._lib.dflash_ctx_set_kernel_timing(self._h, int(enable))
 
     def set_graphs(self, enable: bool):
-        """Graph replay of the packed verify on or off (on by default; results are the same)."""
+        """Graph replay of the packed verify on or off (off by default; results are the same)."""
         self._lib.dflash_ctx_set_graphs(self._h, int(enable))
 
     def kernel_timing(self, slot: int):

@@ -28,7 +28,7 @@ struct dflash_ctx {
     // captured-graph replay of the packed verify: a stream of the library's own to capture on and
     // launch into (the caller's may be the legacy default stream, which cannot be captured) and
     // the two events that order it against the caller's stream
-    bool graphs = true;
+    bool graphs = false;
     hipStream_t gstream = nullptr;
     hipEvent_t g_in = nullptr, g_out = nullptr;
 };
@@ -109,6 +109,11 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
                        int64_t window, const int32_t *ctx_len_dev);
+
+// Few-row Q6_K GEMMs of up to three matrices over the same activations (a layer's q, k and v
+// projections) as one launch: y[m] = x . w[m]^T, [n_rows][n_out[m]] each.
+int32_t dfl_gemm_q6k_set(dflash_ctx *ctx, int n_mats, const void *const *w, float *const *y, const int64_t *n_out, const void *x,
+                         int32_t x_type, int64_t n_in, int32_t n_rows, dflash_stream_t stream);
 
 // Few-row Q4_K GEMM over the matrices that the device-side list ids[0 .. *n_slots) picks out of a stack
 // (w_stack + id * w_stride_bytes; id -1 = extra_w): slot j reads activations x + j * x_stride (elements; 0 = shared) and

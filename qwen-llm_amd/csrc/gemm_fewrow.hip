@@ -37,27 +37,6 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxSplit = 16;
 
-template <typename T>
-__device__ __forceinline__ _Float16 load_x(const T *x, int m, int n_rows, int64_t n_in, int64_t k) {
-    if (m >= n_rows) return static_cast<_Float16>(0.0f);
-    return static_cast<_Float16>(x[static_cast<int64_t>(m) * n_in + k]);
-}
-
-// Natural layout for the generic kernel: step s (32 k), lane (m, g), value i: k = 32 s + 8 g + i.
-template <typename T>
-__global__ void __launch_bounds__(256) prep_x_natural_kernel(const T *__restrict__ x, half8_t *__restrict__ xp,
-                                                             int n_rows, int64_t n_in, int64_t n_steps) {
-    int64_t item = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (item >= n_steps * 64) return;
-    int64_t s = item >> 6;
-    int lane = item & 63;
-    int m = lane & 15, g = lane >> 4;
-    half8_t v;
-#pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = load_x(x, m, n_rows, n_in, 32 * s + 8 * g + i);
-    xp[item] = v;
-}
-
 // ----------------------------------------------------------------------------
 // Q4_K kernel
 // ----------------------------------------------------------------------------
@@ -726,10 +705,13 @@ __device__ __forceinline__ half8_t dequant8<DFLASH_TYPE_Q8_0>(const uint8_t *row
     return v;
 }
 
-template <int TYPE>
+template <typename XT>
+__device__ __forceinline__ half8_t load_x8(const XT *p, bool live);
+
+template <int TYPE, typename XT>
 __global__ void __launch_bounds__(64 * kMaxSplit)
-    gemm_generic_kernel(const uint8_t *__restrict__ w, const half8_t *__restrict__ xp, float *__restrict__ y,
-                        int n_out, int64_t n_steps, size_t row_bytes, int n_rows, int n_split) {
+    gemm_generic_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y, int n_out,
+                        int64_t n_steps, size_t row_bytes, int n_rows, int n_split) {
     extern __shared__ float red[];  // [n_split][256]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -739,9 +721,11 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
     row = row < n_out ? row : n_out - 1;
     const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
     const int64_t s0 = n_steps * wave / n_split, s1 = n_steps * (wave + 1) / n_split;
+    const bool x_live = n < n_rows;  // lane (m = n, g) of the A operand: activation row n, straight from the caller's matrix
+    const XT *xrow = x + static_cast<size_t>(x_live ? n : 0) * (static_cast<size_t>(n_steps) * 32) + 8 * g;
     float4_t acc = {0, 0, 0, 0};
     for (int64_t s = s0; s < s1; s++) {
-        half8_t a = xp[s * 64 + lane];
+        half8_t a = load_x8<XT>(xrow + 32 * s, x_live);
         half8_t b = dequant8<TYPE>(rowp, 32 * s + 8 * g);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
     }
@@ -776,8 +760,6 @@ __device__ __forceinline__ uint64_t load_u64_unaligned(const uint8_t *p) {
     return v;
 }
 
-template <typename XT>
-__device__ __forceinline__ half8_t load_x8(const XT *p, bool live);
 template <>
 __device__ __forceinline__ half8_t load_x8<float>(const float *p, bool live) {
     half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -796,15 +778,30 @@ __device__ __forceinline__ half8_t load_x8<_Float16>(const _Float16 *p, bool liv
     return r;
 }
 
+// Up to three matrices that share the activations (the q, k and v projections of a layer) in one
+// launch: workgroup b serves tile b - tile_begin[m] of the matrix m whose tile range holds b.
+struct Q6KSet {
+    const uint8_t *w[3];
+    float *y[3];
+    int n_out[3];
+    int tile_begin[3];
+    int n_mats;
+};
+
 template <typename XT>
 __global__ void __launch_bounds__(64 * kMaxSplit)
-    gemm_q6k_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y, int n_out, int nb,
-                    size_t row_bytes, int n_rows, int n_split) {
+    gemm_q6k_kernel(Q6KSet set, const XT *__restrict__ x, int nb, size_t row_bytes, int n_rows, int n_split) {
     extern __shared__ float red[];  // [n_split][256]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    int mat = 0;
+    if (set.n_mats > 1 && static_cast<int>(blockIdx.x) >= set.tile_begin[1]) mat = 1;
+    if (set.n_mats > 2 && static_cast<int>(blockIdx.x) >= set.tile_begin[2]) mat = 2;
+    const uint8_t *__restrict__ w = set.w[mat];
+    float *__restrict__ y = set.y[mat];
+    const int n_out = set.n_out[mat];
+    const int n0 = (blockIdx.x - set.tile_begin[mat]) * 16;
     const int row = min(n0 + n, n_out - 1);
     const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
     const int n_half = 2 * nb;
@@ -874,7 +871,52 @@ int env_int(const char *name, int fallback) {
     return (v && *v) ? atoi(v) : fallback;
 }
 
+int32_t launch_q6k(dflash_ctx *ctx, Q6KSet set, const void *x, int32_t x_type, int64_t n_in, int32_t n_rows, hipStream_t st) {
+    if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
+    const int nb = static_cast<int>(n_in / DFL_QK_K);
+    const size_t row_bytes = static_cast<size_t>(nb) * DFL_Q6_K_BYTES;
+    int tiles = 0;
+    for (int m = 0; m < set.n_mats; m++) {
+        set.tile_begin[m] = tiles;
+        tiles += (set.n_out[m] + 15) / 16;
+    }
+    // waves of a workgroup split K: enough waves in total to fill the chip
+    const int target_waves = 8 * ctx->n_cu;
+    int split = (target_waves + tiles - 1) / tiles;
+    split = env_int("DFLASH_GEMM_NSPLIT", split);
+    if (split > 2 * nb) split = 2 * nb;
+    if (split > kMaxSplit) split = kMaxSplit;
+    if (split < 1) split = 1;
+    const size_t lds = static_cast<size_t>(split) * 256 * sizeof(float);
+    dfl_timed timer(ctx, st, DFL_T_GEMM);
+    if (x_type == DFLASH_TYPE_F32)
+        gemm_q6k_kernel<float><<<tiles, 64 * split, lds, st>>>(set, static_cast<const float *>(x), nb, row_bytes, n_rows, split);
+    else
+        gemm_q6k_kernel<_Float16><<<tiles, 64 * split, lds, st>>>(set, static_cast<const _Float16 *>(x), nb, row_bytes, n_rows, split);
+    return DFLASH_OK;
+}
+
 }  // namespace
+
+int32_t dfl_gemm_q6k_set(dflash_ctx *ctx, int n_mats, const void *const *w, float *const *y, const int64_t *n_out, const void *x,
+                         int32_t x_type, int64_t n_in, int32_t n_rows, dflash_stream_t stream) {
+    if (n_mats < 1 || n_mats > 3 || n_in <= 0 || n_in % DFL_QK_K || n_rows < 1 || n_rows > 16)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_q6k_set: bad shape");
+    Q6KSet set = {};
+    set.n_mats = n_mats;
+    for (int m = 0; m < n_mats; m++) {
+        if (!w[m] || !y[m] || n_out[m] <= 0 || n_out[m] > 0x7fffffffll || reinterpret_cast<uintptr_t>(w[m]) % 2)
+            return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "gemm_q6k_set: matrix %d", m);
+        set.w[m] = static_cast<const uint8_t *>(w[m]);
+        set.y[m] = y[m];
+        set.n_out[m] = static_cast<int>(n_out[m]);
+    }
+    const int32_t rc = launch_q6k(ctx, set, x, x_type, n_in, n_rows, static_cast<hipStream_t>(stream));
+    if (rc) return rc;
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
 
 namespace {
 
@@ -997,40 +1039,22 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t n_steps = n_in / 32;
-    size_t off = 0;
     const int tiles = static_cast<int>((n_out + 15) / 16);
     const int target_waves = 8 * ctx->n_cu;
 
     if (w_type == DFLASH_TYPE_Q4_K) {
         return launch_q4k(ctx, w, x, x_type, y, n_in, n_out, n_rows, st, nullptr, 1);
     } else if (w_type == DFLASH_TYPE_Q6_K) {
+        Q6KSet set = {};
+        set.n_mats = 1;
+        set.w[0] = static_cast<const uint8_t *>(w);
+        set.y[0] = y;
+        set.n_out[0] = static_cast<int>(n_out);
+        const int32_t rc = launch_q6k(ctx, set, x, x_type, n_in, n_rows, st);
+        if (rc) return rc;
+    } else {
         if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
             return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
-        const int nb = static_cast<int>(n_in / DFL_QK_K);
-        int split = (target_waves + tiles - 1) / tiles;
-        split = env_int("DFLASH_GEMM_NSPLIT", split);
-        if (split > 2 * nb) split = 2 * nb;
-        if (split > kMaxSplit) split = kMaxSplit;
-        if (split < 1) split = 1;
-        const size_t lds = static_cast<size_t>(split) * 256 * sizeof(float);
-        const uint8_t *wb = static_cast<const uint8_t *>(w);
-        dfl_timed timer(ctx, st, DFL_T_GEMM);
-        if (x_type == DFLASH_TYPE_F32)
-            gemm_q6k_kernel<float><<<tiles, 64 * split, lds, st>>>(wb, static_cast<const float *>(x), y, static_cast<int>(n_out),
-                                                                  nb, row_bytes, n_rows, split);
-        else
-            gemm_q6k_kernel<_Float16><<<tiles, 64 * split, lds, st>>>(wb, static_cast<const _Float16 *>(x), y,
-                                                                     static_cast<int>(n_out), nb, row_bytes, n_rows, split);
-    } else {
-        half8_t *xp = dfl_ws_take<half8_t>(ctx, &off, static_cast<size_t>(n_steps) * 64 * sizeof(half8_t));
-        if (!xp) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "gemm_fewrow: workspace too small");
-        unsigned prep_grid = static_cast<unsigned>((n_steps * 64 + 255) / 256);
-        if (x_type == DFLASH_TYPE_F32)
-            prep_x_natural_kernel<float><<<prep_grid, 256, 0, st>>>(static_cast<const float *>(x), xp, n_rows, n_in,
-                                                                    n_steps);
-        else
-            prep_x_natural_kernel<_Float16>
-                <<<prep_grid, 256, 0, st>>>(static_cast<const _Float16 *>(x), xp, n_rows, n_in, n_steps);
         int split = (target_waves + tiles - 1) / tiles;
         split = env_int("DFLASH_GEMM_NSPLIT", split);
         if (split > n_steps) split = static_cast<int>(n_steps);
@@ -1039,8 +1063,12 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
         size_t lds = static_cast<size_t>(split) * 256 * sizeof(float);
         const uint8_t *wb = static_cast<const uint8_t *>(w);
         dfl_timed timer(ctx, st, DFL_T_GEMM);
-        gemm_generic_kernel<DFLASH_TYPE_Q8_0>
-            <<<tiles, 64 * split, lds, st>>>(wb, xp, y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
+        if (x_type == DFLASH_TYPE_F32)
+            gemm_generic_kernel<DFLASH_TYPE_Q8_0, float><<<tiles, 64 * split, lds, st>>>(
+                wb, static_cast<const float *>(x), y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
+        else
+            gemm_generic_kernel<DFLASH_TYPE_Q8_0, _Float16><<<tiles, 64 * split, lds, st>>>(
+                wb, static_cast<const _Float16 *>(x), y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
     }
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;

@@ -223,6 +223,21 @@ int32_t gemm(dflash_ctx *ctx, const dflash_qtensor &w, const float *x, float *y,
     return dflash_gemm_fewrow(ctx, w.type, w.data, x, DFLASH_TYPE_F32, y, n_in, n_out, n, st);
 }
 
+// The q, k and v projections of a layer: one launch when all three are Q6_K, else three.
+int32_t gemm_qkv(dflash_ctx *ctx, const dflash_qtensor &wq, const dflash_qtensor &wk, const dflash_qtensor &wv, const float *x,
+                 float *q, float *k, float *v, int64_t n_in, int64_t q_dim, int64_t kv_dim, int n, hipStream_t st) {
+    if (wq.type == DFLASH_TYPE_Q6_K && wk.type == DFLASH_TYPE_Q6_K && wv.type == DFLASH_TYPE_Q6_K && n_in % DFL_QK_K == 0) {
+        const void *w[3] = {wq.data, wk.data, wv.data};
+        float *y[3] = {q, k, v};
+        const int64_t n_out[3] = {q_dim, kv_dim, kv_dim};
+        return dfl_gemm_q6k_set(ctx, 3, w, y, n_out, x, DFLASH_TYPE_F32, n_in, n, st);
+    }
+    int32_t rc;
+    if ((rc = gemm(ctx, wq, x, q, n_in, q_dim, n, st))) return rc;
+    if ((rc = gemm(ctx, wk, x, k, n_in, kv_dim, n, st))) return rc;
+    return gemm(ctx, wv, x, v, n_in, kv_dim, n, st);
+}
+
 int32_t embed_rows(dflash_ctx *ctx, const dflash_qtensor &t, const int32_t *ids_dev, int n, int hidden, float *out,
                    hipStream_t st) {
     size_t rb = dflash_row_bytes(t.type, hidden);
@@ -368,9 +383,7 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
         const dflash_layer &L = model->layers[il];
         _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
         rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
-        if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, n, st))) return rc;
-        if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, n, st))) return rc;
-        if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, n, st))) return rc;
+        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, H, q_dim, kv_dim, n, st))) return rc;
         qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, kc, s->pos, c.n_q, c.n_kv,
                                                                       hd, c.eps, c.rope_theta, s->v, vtc, s->capacity);
         // the context length is read from pos[0] on the device: the same launches serve every position
@@ -614,9 +627,7 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                                                                               static_cast<int>(kv_dim), s->cap16, c0);
         }
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
-        if ((rc = gemm(ctx, L.wq, s->cur, s->q, H, q_dim, N, st))) return rc;
-        if ((rc = gemm(ctx, L.wk, s->cur, s->k, H, kv_dim, N, st))) return rc;
-        if ((rc = gemm(ctx, L.wv, s->cur, s->v, H, kv_dim, N, st))) return rc;
+        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, H, q_dim, kv_dim, N, st))) return rc;
         qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, nullptr, s->pos, c.n_q,
                                                                   c.n_kv, hd, c.eps, c.rope_theta, nullptr, nullptr, 0);
         if (fast) {

@@ -272,7 +272,7 @@ def test_graph_replay_is_bit_identical_to_launch_by_launch(ctx, target):
         eager, r0 = run(False)
         replay, r1 = run(True)
     finally:
-        ctx.set_graphs(True)
+        ctx.set_graphs(False)
     assert r0 == 0
     assert r1 >= 8, f"only {r1} of 16 calls were graph replays"
     for i, (a, b) in enumerate(zip(eager, replay)):
