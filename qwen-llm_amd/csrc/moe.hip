@@ -19,9 +19,33 @@ namespace {
 
 constexpr int kMaxSlots = 16;  // a row picks an expert at most once, and a block has at most 16 rows
 
+// Maximum of a 64-bit key over the wave, in every lane: data-parallel-primitive moves within rows of
+// 16 lanes (shift right by 1, 2, 4, 8: lane 15 of a row then holds the row's maximum), then lane 15
+// of rows 0 and 2 broadcast into rows 1 and 3, then lane 31 into rows 2 and 3; lane 63 has the
+// result.  Lanes without a source read 0, the identity.  No LDS round trips, unlike a shuffle.
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#define DFL_MAX_STEP(ctrl, row_mask)                                                                            \
+    do {                                                                                                        \
+        const unsigned lo = __builtin_amdgcn_update_dpp(0u, static_cast<unsigned>(v), ctrl, row_mask, 0xf, false);      \
+        const unsigned hi = __builtin_amdgcn_update_dpp(0u, static_cast<unsigned>(v >> 32), ctrl, row_mask, 0xf, false); \
+        const unsigned long long o = (static_cast<unsigned long long>(hi) << 32) | lo;                          \
+        v = o > v ? o : v;                                                                                      \
+    } while (0)
+    DFL_MAX_STEP(0x111, 0xf);  // row_shr:1
+    DFL_MAX_STEP(0x112, 0xf);  // row_shr:2
+    DFL_MAX_STEP(0x114, 0xf);  // row_shr:4
+    DFL_MAX_STEP(0x118, 0xf);  // row_shr:8
+    DFL_MAX_STEP(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+    DFL_MAX_STEP(0x143, 0xc);  // row_bcast:31 into rows 2 and 3
+#undef DFL_MAX_STEP
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(v), 63);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(v >> 32), 63);
+    return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+
 // Routing of a whole block in one workgroup of sixteen waves (n_expert <= 1024, at most 16 rows).
-// Wave w serves block row w: softmax, top-k by rank (an expert's rank = how many experts beat it:
-// higher probability, or equal and lower id), the renormalised weights in pick order, and the
+// Wave w serves block row w: softmax, top-k (higher probability first, equal probabilities to the
+// lower id), the renormalised weights in pick order, and the
 // shared-expert gate; a row's arithmetic does not depend on how many rows the block has.  Then the
 // whole workgroup lists the block's distinct experts in ascending id order: ids[0 .. n), then one
 // slot with id -1 (the shared expert, which every row uses) if with_shared; *n_slots = n (+ 1); for
@@ -31,7 +55,8 @@ __global__ void __launch_bounds__(1024)
                      int n_rows, int n_expert, int n_used, int hidden, int with_shared, int32_t *__restrict__ sel_e,
                      float *__restrict__ sel_w, float *__restrict__ sg, int32_t *__restrict__ ids,
                      int32_t *__restrict__ n_slots, int32_t *__restrict__ slot_of) {
-    extern __shared__ float probs[];  // [16][n_expert], then int32 rank[n_expert]
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) float probs[];  // [16][n_expert], then int32 rank[n_expert]
     __shared__ float pick_w[16][64];
     __shared__ int32_t pick_e[16][64];
     __shared__ int wave_count[16];
@@ -57,24 +82,41 @@ __global__ void __launch_bounds__(1024)
     if (tid < n_expert) rank[tid] = 0;
     __syncthreads();
     if (live) {
-        for (int e = lane; e < n_expert; e += 64) {
-            const float p = pr[e];
-            int r = 0;
-            for (int o = 0; o < n_expert; o++) {
-                const float q = pr[o];
-                r += (q > p || (q == p && o < e)) ? 1 : 0;
+        // pick k = the best remaining expert: a wave-wide maximum over 64-bit keys (probability bits,
+        // then ~id, so that equal probabilities go to the lower id); the winner's probability is
+        // then marked taken (negative).  Same order as ranking every expert against all others, at
+        // n_used * n_expert / 64 steps instead of n_expert^2 / 64.
+        for (int k = 0; k < n_used; k++) {
+            unsigned long long best = 0;
+            for (int e = lane; e < n_expert; e += 64) {
+                const float p = pr[e];
+                const unsigned long long key = (static_cast<unsigned long long>(__float_as_uint(p)) << 32) | (0xffffffffu - static_cast<unsigned>(e));
+                if (p >= 0.0f && key > best) best = key;
             }
-            if (r < n_used) {
-                sel_e[row * n_used + r] = e;
-                pick_e[row][r] = e;
-                pick_w[row][r] = p;
-                rank[e] = 1;  // picked by some row
+            best = wave_max_u64(best);
+            int e_win = static_cast<int>(0xffffffffu - static_cast<unsigned>(best));
+            if (best == 0) e_win = k < n_expert ? k : n_expert - 1;  // nothing comparable left (NaN logits): stay in range
+            if (lane == 0) {
+                sel_e[row * n_used + k] = e_win;
+                pick_e[row][k] = e_win;
+                pick_w[row][k] = __uint_as_float(static_cast<unsigned>(best >> 32));
+                rank[e_win] = 1;  // picked by some row
+                pr[e_win] = -1.0f;
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
         // shared-expert gate: sigmoid(x . w)
         const float *xr = x + static_cast<size_t>(row) * hidden;
         float dot = 0.0f;
-        for (int i = lane; i < hidden; i += 64) dot += xr[i] * shexp_gate[i];
+        if (hidden % 4 == 0) {
+            for (int i = 4 * lane; i < hidden; i += 256) {
+                const f4 a = *reinterpret_cast<const f4 *>(xr + i), b = *reinterpret_cast<const f4 *>(shexp_gate + i);
+                dot += (a[0] * b[0] + a[1] * b[1]) + (a[2] * b[2] + a[3] * b[3]);
+            }
+        } else {
+            for (int i = lane; i < hidden; i += 64) dot += xr[i] * shexp_gate[i];
+        }
         for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
         if (lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
     }
