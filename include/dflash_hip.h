@@ -138,6 +138,39 @@ int32_t dflash_argmax_greedy(dflash_ctx *ctx, const float *logits, int32_t n_row
 int32_t dflash_top16(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64_t vocab, int64_t stride,
                      int32_t *ids, float *vals, dflash_stream_t stream);
 
+/* ---- DFlash-2 extras ---------------------------------------------------------------------
+ * dflash_dflash2_conv: kernel_dflash2_conv_f32 (kernels/dflash2.metal:40-69, encoder
+ *   metal/dflash.rs:98-111): y[t][c] = sum_tap (base[side][tap][c] + dyn[t][side][tap][c / group_size])
+ *   * x[t - tap][c], rows before the block read as zeros.  x, y [n_tokens][h] f32 (y must not alias
+ *   x); dyn [n_tokens][2 * kernel_size * h / group_size] f32, (group, tap, side) fastest to slowest;
+ *   base [2][kernel_size][h] f32.  Enqueue-only.
+ * dflash_select_draft_path: select_draft_path (metal_dflash.rs:17176-17251) with
+ *   DFlash2Codebook::dequant_row (:3275-3343), run on the device so that the top-16 and the
+ *   selector hidden never leave it: out[0] = topk_ids[0]; for every later position the candidate b
+ *   maximising topk_vals[pos][b] + sum_r (pred[r] * sel_h[pos][r]) * succ_b[r] (sums in rank order,
+ *   products and additions rounded separately; strict >, so the first maximum wins and candidate 0
+ *   when nothing compares greater; candidates below 0 or past the successor table are skipped);
+ *   the winner's predecessor row conditions the next position.  Codebooks are [n_rows][rank] rows
+ *   of F32, F16, Q8_0 or Q4_K in device memory; topk_ids/topk_vals [n][top_k], sel_h [n][rank] and
+ *   out_tokens [n] are device pointers; top_k <= 16, rank <= 1024, n <= 16.  With out_tokens_host
+ *   the call waits, copies the tokens and returns DFLASH_ERR_INVALID_TOKEN if a predecessor row was
+ *   out of range (the reference's BadDrafter("selector codebook row out of range")); without it the
+ *   call only enqueues. */
+typedef struct {
+    int32_t type; /* DFLASH_TYPE_F32 / F16 / Q8_0 / Q4_K */
+    int32_t pad;
+    int64_t n_rows;
+    const void *data; /* device */
+} dflash_codebook;
+
+int32_t dflash_dflash2_conv(dflash_ctx *ctx, const float *x, const float *dyn, const float *base, float *y,
+                            int32_t n_tokens, int32_t h, int32_t kernel_size, int32_t group_size, int32_t side,
+                            dflash_stream_t stream);
+int32_t dflash_select_draft_path(dflash_ctx *ctx, const dflash_codebook *predecessor, const dflash_codebook *successor,
+                                 int32_t rank, int32_t top_k, int32_t carry_token, int32_t n, const int32_t *topk_ids,
+                                 const float *topk_vals, const float *sel_h, int32_t *out_tokens,
+                                 int32_t *out_tokens_host, dflash_stream_t stream);
+
 /* ---- sampler state (host side) ------------------------------------------------------
  * SamplingConfig / Sampler (sampling.rs:18-145, 304-366): one request-local random stream.
  * rng_kind 0 = xoshiro256++ seeded by SplitMix64 (the reference's generator, sampling.rs:1621-1670),

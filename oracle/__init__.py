@@ -31,7 +31,7 @@ ERR = {
 
 def build(force: bool = False) -> str:
     """Compile liboracle.so with gcc (a few seconds)."""
-    srcs = [os.path.join(_DIR, f) for f in ("quant.c", "rng.c", "sampler.c", "forward.c", "dflash_oracle.h")]
+    srcs = [os.path.join(_DIR, f) for f in ("quant.c", "rng.c", "sampler.c", "forward.c", "dflash2.c", "dflash_oracle.h")]
     stale = force or not os.path.exists(_LIB_PATH) or any(
         os.path.getmtime(s) > os.path.getmtime(_LIB_PATH) for s in srcs)
     if stale:
@@ -50,6 +50,11 @@ class Sampler(C.Structure):
 
 class WeightedCandidate(C.Structure):
     _fields_ = [("token", C.c_int32), ("pad", C.c_int32), ("weight", C.c_double)]
+
+
+class Codebook(C.Structure):
+    _fields_ = [("type", C.c_int32), ("pad", C.c_int32), ("rank", C.c_size_t), ("n_rows", C.c_size_t),
+                ("data", C.c_void_p)]
 
 
 class AcceptDecision(C.Structure):
@@ -167,6 +172,10 @@ def _declare(L):
     L.orc_attn_draft.argtypes = [vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, C.c_uint32, C.c_int, C.c_uint32, vp]
     L.orc_target_verify.argtypes = [C.POINTER(Model), vp, sz, sz, vp, vp, sz, vp, vp, sz, vp]
     L.orc_dflash_draft.argtypes = [C.POINTER(Model), C.POINTER(DraftHead), vp, vp, sz, vp, C.c_uint32, vp]
+    L.orc_dflash2_conv.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, sz]
+    L.orc_dflash2_conv.restype = None
+    L.orc_codebook_row.argtypes = [C.POINTER(Codebook), sz, vp]
+    L.orc_select_draft_path.argtypes = [C.POINTER(Codebook), C.POINTER(Codebook), sz, sz, i32, sz, vp, vp, vp, vp, vp, vp]
 
 
 def _p(a: np.ndarray):
@@ -445,3 +454,47 @@ def dflash_draft(target: Model, head: DraftHead, noise_ids, ctx_stacked, pos_ctx
     if rc:
         raise RuntimeError(f"orc_dflash_draft failed: {rc}")
     return logits
+
+
+# ---- DFlash-2 extras ----
+F32, F16 = 0, 1
+
+
+def dflash2_conv(x, dyn, base, kernel_size: int, group_size: int, side: int) -> np.ndarray:
+    """x [n_tokens][h], dyn [n_tokens][2*kernel_size*h/group_size], base [2][kernel_size][h] -> y [n_tokens][h]."""
+    x = np.ascontiguousarray(x, np.float32)
+    dyn = np.ascontiguousarray(dyn, np.float32)
+    base = np.ascontiguousarray(base, np.float32)
+    n, h = x.shape
+    y = np.empty_like(x)
+    lib().orc_dflash2_conv(x.ctypes.data, dyn.ctypes.data, base.ctypes.data, y.ctypes.data, n, h, kernel_size, group_size, side)
+    return y
+
+
+def make_codebook(qtype: int, rows: np.ndarray, rank: int):
+    """rows: [n_rows][row bytes] uint8 (quantised types) or [n_rows][rank] float32/float16.  Returns (Codebook, keepalive)."""
+    rows = np.ascontiguousarray(rows)
+    return Codebook(qtype, 0, rank, rows.shape[0], rows.ctypes.data), rows
+
+
+def codebook_row(cb, row: int) -> np.ndarray:
+    out = np.empty(cb.rank, np.float32)
+    if lib().orc_codebook_row(C.byref(cb), row, out.ctypes.data):
+        raise ValueError("selector codebook row out of range")
+    return out
+
+
+def select_draft_path(pred_cb, succ_cb, top_k: int, rank: int, carry: int, n: int, ids, vals, sel_h):
+    """Returns (tokens [n], scores [n][top_k], valid [n][top_k]); raises ValueError on an invalid predecessor row."""
+    ids = np.ascontiguousarray(ids, np.int32)
+    vals = np.ascontiguousarray(vals, np.float32)
+    sel_h = np.ascontiguousarray(sel_h, np.float32)
+    out = np.zeros(n, np.int32)
+    scores = np.full((n, top_k), np.nan, np.float32)
+    valid = np.zeros((n, top_k), np.uint8)
+    rc = lib().orc_select_draft_path(C.byref(pred_cb), C.byref(succ_cb), top_k, rank, carry, n, ids.ctypes.data,
+                                     vals.ctypes.data, sel_h.ctypes.data, out.ctypes.data, scores.ctypes.data,
+                                     valid.ctypes.data)
+    if rc:
+        raise ValueError("selector codebook row out of range")
+    return out, scores, valid

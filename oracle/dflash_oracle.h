@@ -30,6 +30,10 @@
  *   - dense-proposal coupling (orc_couple_dense_proposal): the reference never
  *       builds a dense proposal; this function is pinned only through its
  *       reduction to the sparse coupling on small vocabularies.
+ *   - DFlash-2 conv ................... closed forms (one tap = a product, zero rows before the
+ *       block, side/group indexing against an independent numpy gather)
+ *   - DFlash-2 selector walk .......... the known-answer walks of metal_dflash/tests.rs:2978-3094
+ *       (scores, first-tie rule, sentinel and non-finite candidates, invalid predecessor)
  *   - f64 exp/ln are the host libm's, as the reference's are its platform's:
  *       last-ulp behaviour is parity unpinned (decisions compare against
  *       uniforms and are insensitive to it except with probability ~2^-50).
@@ -251,6 +255,29 @@ typedef struct {
 int orc_dflash_draft(const orc_model *target, const orc_draft_head *head, const int32_t *noise_ids,
                      const float *target_ctx_stacked, size_t ctx_len, const int32_t *pos_ctx,
                      uint32_t noise_start_pos, float *logits);
+
+/* ---- DFlash-2 extras (dflash2.c) ---- */
+enum { ORC_F32 = 0, ORC_F16 = 1 };
+
+/* kernels/dflash2.metal:40-69; x, y [n_tokens][h]; dyn [n_tokens][2*kernel_size*h/group_size]
+ * laid out (group, tap, side) fastest to slowest; base [2][kernel_size][h] */
+void orc_dflash2_conv(const float *x, const float *dyn, const float *base, float *y, size_t n_tokens, size_t h,
+                      size_t kernel_size, size_t group_size, size_t side);
+
+/* selector codebook: [n_rows][rank] rows of F32, F16, Q8_0 or Q4_K (metal_dflash.rs:3200-3343) */
+typedef struct {
+    int32_t type;
+    int32_t pad;
+    size_t rank, n_rows;
+    const void *data;
+} orc_codebook;
+
+int orc_codebook_row(const orc_codebook *cb, size_t row, float *out);
+
+/* metal_dflash.rs:17176-17251, 3473-3617 */
+int orc_select_draft_path(const orc_codebook *pred_cb, const orc_codebook *succ_cb, size_t top_k, size_t rank,
+                          int32_t carry, size_t n, const int32_t *ids, const float *vals, const float *sel_h,
+                          int32_t *out, float *scores, uint8_t *valid);
 
 #ifdef __cplusplus
 }

@@ -46,6 +46,10 @@ class WeightedCandidateC(C.Structure):
     _fields_ = [("token", C.c_int32), ("pad", C.c_int32), ("weight", C.c_double)]
 
 
+class CodebookC(C.Structure):
+    _fields_ = [("type", C.c_int32), ("pad", C.c_int32), ("n_rows", C.c_int64), ("data", C.c_void_p)]
+
+
 class AcceptDecisionC(C.Structure):
     _fields_ = [("n_accepted", C.c_int32), ("accepted_drafts", C.c_int32 * 16), ("carry_kind", C.c_int32),
                 ("carry_token", C.c_int32), ("stop_reason", C.c_int32), ("retain_input_count", C.c_int32),
@@ -91,6 +95,11 @@ def _declare(L):
     L.dflash_version.restype = C.c_char_p
     L.dflash_ctx_set_kernel_timing.restype = None
     L.dflash_ctx_set_kernel_timing.argtypes = [vp, i32]
+    L.dflash_dflash2_conv.restype = i32
+    L.dflash_dflash2_conv.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]
+    L.dflash_select_draft_path.restype = i32
+    L.dflash_select_draft_path.argtypes = [vp, C.POINTER(CodebookC), C.POINTER(CodebookC), i32, i32, i32, i32, vp, vp, vp,
+                                           vp, vp, vp]
     L.dflash_ctx_set_graphs.restype = None
     L.dflash_ctx_set_graphs.argtypes = [vp, i32]
     L.dflash_ctx_kernel_timing.restype = i32
@@ -303,6 +312,34 @@ class Context:
         self._check(self._lib.dflash_top16(self._h, logits.data_ptr(), n, v, stride, ids.data_ptr(), vals.data_ptr(),
                                            _stream_ptr()))
         return ids, vals
+
+    # ---- DFlash-2 extras (kernels/dflash2.metal:40-69; metal_dflash.rs:17176-17251)
+    def dflash2_conv(self, x, dyn, base, kernel_size: int, group_size: int, side: int):
+        """x [n_tokens, h], dyn [n_tokens, 2*kernel_size*h/group_size], base [2, kernel_size, h] (device f32) -> y."""
+        torch = _torch()
+        n, h = x.shape
+        y = torch.empty_like(x)
+        self._check(self._lib.dflash_dflash2_conv(self._h, x.data_ptr(), dyn.data_ptr(), base.data_ptr(), y.data_ptr(), n, h,
+                                                  kernel_size, group_size, side, _stream_ptr()))
+        return y
+
+    def select_draft_path(self, predecessor, successor, rank: int, carry_token: int, topk_ids, topk_vals, sel_h):
+        """predecessor / successor: (type, device tensor of rows); topk_ids/topk_vals [n, top_k], sel_h [n, rank]
+        on the device.  Returns the n tokens of the greedy selector walk (host list)."""
+        torch = _torch()
+        n, top_k = topk_ids.shape
+
+        def cb(pair):
+            qtype, rows = pair
+            return CodebookC(qtype, 0, rows.shape[0], rows.data_ptr())
+
+        pc, sc = cb(predecessor), cb(successor)
+        out = torch.empty(n, dtype=torch.int32, device=topk_ids.device)
+        host = (C.c_int32 * n)()
+        self._check(self._lib.dflash_select_draft_path(self._h, C.byref(pc), C.byref(sc), rank, top_k, carry_token, n,
+                                                       topk_ids.data_ptr(), topk_vals.data_ptr(), sel_h.data_ptr(),
+                                                       out.data_ptr(), host, _stream_ptr()))
+        return list(host)
 
     # ---- decide_dflash_accept_prefix (metal_dflash/accept.rs:76-84)
     def decide_dflash_accept_prefix(self, verified_tokens, target_logits, vocab, proposals, sampler: Sampler,

@@ -1,0 +1,196 @@
+// DFlash-2 extras of the block drafter: the two-tap dynamic depthwise convolution
+// (kernel_dflash2_conv_f32, kernels/dflash2.metal:40-69) and the greedy selector walk over the
+// predecessor / successor codebooks (select_draft_path, metal_dflash.rs:17176-17251; codebook rows
+// DFlash2Codebook::dequant_row, :3275-3343).  The per-row top-16 that feeds the walk is
+// dflash_top16.
+#include "common.h"
+#include "device_quant.h"
+
+namespace {
+
+// y[t][c] = sum_tap (base[side][tap][c] + dyn[t][side][tap][c / group_size]) * x[t - tap][c]; rows
+// before the block count as zeros; taps accumulate in order with a fused multiply-add, as the
+// reference kernel does.  One thread per element.
+__global__ void __launch_bounds__(256)
+    dflash2_conv_kernel(const float *__restrict__ x, const float *__restrict__ dyn, const float *__restrict__ base,
+                        float *__restrict__ y, int n_tokens, int h, int kernel_size, int group_size, int side) {
+    const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (gid >= static_cast<int64_t>(n_tokens) * h) return;
+    const int t = static_cast<int>(gid / h), c = static_cast<int>(gid % h);
+    const int n_groups = h / group_size, g = c / group_size;
+    const size_t dyn_row = static_cast<size_t>(t) * 2 * kernel_size * n_groups + static_cast<size_t>(side) * kernel_size * n_groups;
+    const size_t base_side = static_cast<size_t>(side) * kernel_size * h;
+    float acc = 0.0f;
+    for (int tap = 0; tap < kernel_size && tap <= t; tap++) {
+        const float b = base[base_side + static_cast<size_t>(tap) * h + c];
+        const float d = dyn[dyn_row + static_cast<size_t>(tap) * n_groups + g];
+        acc = __fmaf_rn(__fadd_rn(b, d), x[static_cast<size_t>(t - tap) * h + c], acc);
+    }
+    y[gid] = acc;
+}
+
+struct Codebook {
+    int type;
+    int rank;
+    int64_t n_rows;
+    const uint8_t *data;
+    size_t row_bytes;
+};
+
+// element r of row `row`
+__device__ __forceinline__ float codebook_elem(const Codebook &cb, int64_t row, int r) {
+    const uint8_t *p = cb.data + static_cast<size_t>(row) * cb.row_bytes;
+    if (cb.type == DFLASH_TYPE_F16) return __half2float(reinterpret_cast<const __half *>(p)[r]);
+    return dfl_dequant_elem(cb.type, p, r);
+}
+
+constexpr int kSelThreads = 256;
+constexpr int kSelMaxTopK = 16;
+constexpr int kSelMaxRank = 1024;
+
+// The walk, one workgroup.  Per position: all threads dequantise the candidates' successor rows and
+// form gate = pred * sel_h[pos] in LDS; thread b then scores candidate b with the reference's scalar
+// loop (products and additions rounded separately, rank order), thread 0 keeps the first strict
+// maximum, and all threads fetch the winner's predecessor row.  status: 0, or 1 when a predecessor
+// row is out of range (the walk stops there).
+__global__ void __launch_bounds__(kSelThreads)
+    dflash2_select_kernel(Codebook pred_cb, Codebook succ_cb, int top_k, int rank, int carry, int n,
+                          const int32_t *__restrict__ ids, const float *__restrict__ vals,
+                          const float *__restrict__ sel_h, int32_t *__restrict__ out, int32_t *__restrict__ status) {
+    extern __shared__ float lds[];  // pred[rank], gate[rank], succ[top_k][rank]
+    __shared__ float score[kSelMaxTopK];
+    __shared__ int chosen_s;
+    float *pred = lds, *gate = lds + rank, *succ = lds + 2 * rank;
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        out[0] = ids[0];
+        *status = 0;
+    }
+    if (n < 2) return;
+    if (carry < 0 || carry >= pred_cb.n_rows) {
+        if (tid == 0) *status = 1;
+        return;
+    }
+    for (int r = tid; r < rank; r += kSelThreads) pred[r] = codebook_elem(pred_cb, carry, r);
+    __syncthreads();
+    for (int pos = 1; pos < n; pos++) {
+        const float *hrow = sel_h + static_cast<size_t>(pos) * rank;
+        for (int r = tid; r < rank; r += kSelThreads) gate[r] = __fmul_rn(pred[r], hrow[r]);
+        for (int e = tid; e < top_k * rank; e += kSelThreads) {
+            const int b = e / rank, r = e - b * rank;
+            const int32_t cand = ids[pos * top_k + b];
+            if (cand >= 0 && cand < succ_cb.n_rows) succ[e] = codebook_elem(succ_cb, cand, r);
+        }
+        __syncthreads();
+        if (tid < top_k) {
+            const int32_t cand = ids[pos * top_k + tid];
+            float s = __builtin_nanf("");  // skipped candidates never compare greater
+            if (cand >= 0 && cand < succ_cb.n_rows) {
+                float dot = 0.0f;
+                const float *sr = succ + tid * rank;
+                for (int r = 0; r < rank; r++) dot = __fadd_rn(dot, __fmul_rn(gate[r], sr[r]));
+                s = __fadd_rn(vals[pos * top_k + tid], dot);
+            }
+            score[tid] = s;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int best_b = 0;
+            float best = -INFINITY;
+            for (int b = 0; b < top_k; b++) {
+                const int32_t cand = ids[pos * top_k + b];
+                if (cand < 0 || cand >= succ_cb.n_rows) continue;
+                if (score[b] > best) {
+                    best = score[b];
+                    best_b = b;
+                }
+            }
+            const int32_t chosen = ids[pos * top_k + best_b];
+            out[pos] = chosen;
+            chosen_s = chosen;
+            if (chosen < 0 || chosen >= pred_cb.n_rows) *status = 1;
+        }
+        __syncthreads();
+        const int chosen = chosen_s;
+        if (chosen < 0 || chosen >= pred_cb.n_rows) return;
+        for (int r = tid; r < rank; r += kSelThreads) pred[r] = codebook_elem(pred_cb, chosen, r);
+        __syncthreads();
+    }
+}
+
+int32_t check_codebook(dflash_ctx *ctx, const dflash_codebook *cb, int rank, Codebook *out, const char *what) {
+    if (!cb || !cb->data || cb->n_rows < 1) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "select_draft_path: %s codebook", what);
+    size_t rb = 0;
+    switch (cb->type) {
+    case DFLASH_TYPE_F32: rb = static_cast<size_t>(rank) * 4; break;
+    case DFLASH_TYPE_F16: rb = static_cast<size_t>(rank) * 2; break;
+    case DFLASH_TYPE_Q8_0:
+    case DFLASH_TYPE_Q4_K: rb = dflash_row_bytes(cb->type, rank); break;
+    default: break;
+    }
+    if (rb == 0)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "select_draft_path: %s codebook type %d with rank %d", what, cb->type, rank);
+    *out = Codebook{cb->type, rank, cb->n_rows, static_cast<const uint8_t *>(cb->data), rb};
+    return DFLASH_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t dflash_dflash2_conv(dflash_ctx *ctx, const float *x, const float *dyn, const float *base, float *y,
+                                       int32_t n_tokens, int32_t h, int32_t kernel_size, int32_t group_size, int32_t side,
+                                       dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!x || !dyn || !base || !y) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "dflash2_conv: null pointer");
+    if (n_tokens < 1 || h < 1 || kernel_size < 1 || group_size < 1 || h % group_size || (side != 0 && side != 1))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "dflash2_conv: n_tokens %d h %d kernel %d group %d side %d", n_tokens, h,
+                        kernel_size, group_size, side);
+    const size_t bytes = static_cast<size_t>(n_tokens) * h * sizeof(float);
+    if (dfl_ranges_overlap(y, bytes, x, bytes))
+        return dfl_fail(ctx, DFLASH_ERR_ALIAS, "dflash2_conv: y aliases x (taps read neighbouring rows)");
+    const int64_t total = static_cast<int64_t>(n_tokens) * h;
+    dflash2_conv_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        x, dyn, base, y, n_tokens, h, kernel_size, group_size, side);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+extern "C" int32_t dflash_select_draft_path(dflash_ctx *ctx, const dflash_codebook *predecessor,
+                                            const dflash_codebook *successor, int32_t rank, int32_t top_k, int32_t carry_token,
+                                            int32_t n, const int32_t *topk_ids, const float *topk_vals, const float *sel_h,
+                                            int32_t *out_tokens, int32_t *out_tokens_host, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!topk_ids || !topk_vals || !sel_h || !out_tokens)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "select_draft_path: null pointer");
+    if (n < 1 || n > 16 || top_k < 1 || top_k > kSelMaxTopK || rank < 1 || rank > kSelMaxRank)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "select_draft_path: n %d top_k %d rank %d", n, top_k, rank);
+    Codebook pc, sc;
+    int32_t rc;
+    if ((rc = check_codebook(ctx, predecessor, rank, &pc, "predecessor"))) return rc;
+    if ((rc = check_codebook(ctx, successor, rank, &sc, "successor"))) return rc;
+    size_t off = 0;
+    int32_t *status = dfl_ws_take<int32_t>(ctx, &off, sizeof(int32_t));
+    if (!status) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "select_draft_path: workspace too small");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t lds = static_cast<size_t>(2 + top_k) * rank * sizeof(float);
+    if (lds > 64 * 1024) {
+        static bool attr = false;
+        if (!attr) {
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(dflash2_select_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (2 + kSelMaxTopK) * kSelMaxRank * static_cast<int>(sizeof(float))));
+            attr = true;
+        }
+    }
+    dflash2_select_kernel<<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
+                                                       out_tokens, status);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    if (out_tokens_host) {
+        // the blocking form also reports an invalid predecessor row, as the reference's CPU walk does
+        int32_t status_host = 0;
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(out_tokens_host, out_tokens, n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(&status_host, status, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        if (status_host) return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "select_draft_path: selector codebook row out of range");
+    }
+    return DFLASH_OK;
+}

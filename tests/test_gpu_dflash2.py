@@ -1,0 +1,107 @@
+"""GPU parity of the DFlash-2 extras against the CPU oracle: the two-tap dynamic convolution
+(kernels/dflash2.metal:40-69) bit for bit, and the greedy selector walk (metal_dflash.rs:17176-17251)
+token for token: on the reference's own known-answer walks (metal_dflash/tests.rs:2978-3094) and on
+seeded random lattices with Q4_K, Q8_0, F16 and F32 codebooks at the released drafters' shape
+(rank 256, top-16, 8 and 16 positions), sentinels and out-of-range candidates included."""
+import numpy as np
+import pytest
+
+import qwen_llm_amd as dfl
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = dfl.Context(0)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("n,h,ks,gs", [(16, 2048, 2, 16), (8, 1024, 2, 16), (5, 96, 3, 8), (1, 64, 2, 16)])
+def test_conv_bit_exact(ctx, oracle, n, h, ks, gs):
+    import torch
+
+    rng = np.random.default_rng(n * 1000 + h)
+    x = rng.standard_normal((n, h)).astype(np.float32)
+    dyn = rng.standard_normal((n, 2 * ks * (h // gs))).astype(np.float32)
+    base = rng.standard_normal((2, ks, h)).astype(np.float32)
+    for side in (0, 1):
+        want = oracle.dflash2_conv(x, dyn, base, ks, gs, side)
+        got = ctx.dflash2_conv(torch.from_numpy(x).cuda(), torch.from_numpy(dyn).cuda(), torch.from_numpy(base).cuda(), ks, gs,
+                               side).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"side {side}"
+
+
+def test_conv_rejects_aliasing_and_bad_groups(ctx):
+    import torch
+
+    x = torch.zeros((4, 64), device="cuda")
+    dyn = torch.zeros((4, 2 * 2 * 4), device="cuda")
+    base = torch.zeros((2, 2, 64), device="cuda")
+    L = dfl.lib()
+    rc = L.dflash_dflash2_conv(ctx._h, x.data_ptr(), dyn.data_ptr(), base.data_ptr(), x.data_ptr(), 4, 64, 2, 16, 0, None)
+    L.dflash_status_name.restype = __import__("ctypes").c_char_p
+    assert L.dflash_status_name(rc) == b"Alias"
+    rc = L.dflash_dflash2_conv(ctx._h, x.data_ptr(), dyn.data_ptr(), base.data_ptr(), dyn.data_ptr(), 4, 64, 2, 24, 0, None)
+    assert rc != 0
+
+
+def walk_gpu(ctx, pred, succ, rank, carry, ids, vals, sel_h):
+    import torch
+
+    def dev(pair):
+        return pair[0], torch.from_numpy(np.ascontiguousarray(pair[1])).cuda()
+
+    return ctx.select_draft_path(dev(pred), dev(succ), rank, carry, torch.from_numpy(np.asarray(ids, np.int32)).cuda(),
+                                 torch.from_numpy(np.asarray(vals, np.float32)).cuda(),
+                                 torch.from_numpy(np.asarray(sel_h, np.float32)).cuda())
+
+
+def test_walk_reference_known_answers(ctx):
+    f32 = lambda rows: (dfl.TYPE_F32, np.asarray(rows, np.float32))
+    got = walk_gpu(ctx, f32([[1, 2], [2, 0], [0, 3], [1, 1]]), f32([[0, 0], [1, 1], [2, 0], [0, 1]]), 2, 0,
+                   np.array([0, 0, 1, 2, 3, 1]).reshape(3, 2), np.zeros((3, 2)), np.array([0, 0, 2, 0.5, 1, 2]).reshape(3, 2))
+    assert got == [0, 2, 3]
+    got = walk_gpu(ctx, f32([[1], [1]]), f32([[0], [1]]), 1, 0, np.array([0, 0, 0, 0, 1, 1, -1, 9]).reshape(2, 4),
+                   np.zeros((2, 4)), np.array([0, 1]).reshape(2, 1))
+    assert got == [0, 1]
+    got = walk_gpu(ctx, f32([[1], [1], [1]]), f32([[0], [0], [0]]), 1, 0, np.array([0, 0, 1, 2, 1, 2]).reshape(3, 2),
+                   np.array([0, 0, np.inf, 0, np.nan, -np.inf]).reshape(3, 2), np.array([0, 1, 1]).reshape(3, 1))
+    assert got == [0, 1, 1]
+    with pytest.raises(dfl.DFlashError):
+        walk_gpu(ctx, f32([[1], [1]]), f32([[0], [0], [1]]), 1, 0, np.array([0, 2]).reshape(2, 1), np.array([0.0, 1.0]).reshape(2, 1),
+                 np.array([0.0, 1.0]).reshape(2, 1))
+
+
+@pytest.mark.parametrize("kind", ["q4_k", "q8_0", "f16", "f32"])
+@pytest.mark.parametrize("n", [8, 16])
+def test_walk_matches_oracle_on_random_lattices(ctx, oracle, kind, n):
+    rank, top_k, vocab = 256, 16, 4096
+    for seed in range(6):
+        rng = np.random.default_rng(100 * seed + n)
+        if kind in ("q4_k", "q8_0"):
+            qt = dfl.synth.Q4_K if kind == "q4_k" else dfl.synth.Q8_0
+            tt = dfl.TYPE_Q4_K if kind == "q4_k" else dfl.TYPE_Q8_0
+            ot = oracle.Q4_K if kind == "q4_k" else oracle.Q8_0
+            pred_rows = dfl.synth.random_weight(qt, vocab, rank, seed=2 * seed)
+            succ_rows = dfl.synth.random_weight(qt, vocab, rank, seed=2 * seed + 1)
+        else:
+            dt = np.float16 if kind == "f16" else np.float32
+            tt = dfl.TYPE_F16 if kind == "f16" else dfl.TYPE_F32
+            ot = oracle.F16 if kind == "f16" else oracle.F32
+            pred_rows = (rng.standard_normal((vocab, rank)) * 0.05).astype(dt)
+            succ_rows = (rng.standard_normal((vocab, rank)) * 0.05).astype(dt)
+        ids = rng.integers(0, vocab, (n, top_k)).astype(np.int32)
+        ids[rng.random((n, top_k)) < 0.1] = -1           # unfilled top-k sentinels
+        ids[rng.random((n, top_k)) < 0.05] = vocab + 7   # past the table
+        ids[:, 0] = rng.integers(0, vocab, n)            # candidate 0 stays a valid predecessor
+        vals = np.sort(rng.standard_normal((n, top_k)).astype(np.float32), axis=1)[:, ::-1].copy()
+        vals[:, 1] = vals[:, 0]                          # a tie in the unary logits
+        sel_h = rng.standard_normal((n, rank)).astype(np.float32)
+        carry = int(rng.integers(0, vocab))
+        pc, k1 = oracle.make_codebook(ot, pred_rows, rank)
+        sc, k2 = oracle.make_codebook(ot, succ_rows, rank)
+        want, _, _ = oracle.select_draft_path(pc, sc, top_k, rank, carry, n, ids, vals, sel_h)
+        got = walk_gpu(ctx, (tt, pred_rows), (tt, succ_rows), rank, carry, ids, vals, sel_h)
+        assert got == want.tolist(), f"{kind} n={n} seed={seed}"
