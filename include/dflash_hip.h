@@ -241,6 +241,24 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified_tokens_hos
                              const int32_t *stop_ids_host, int32_t n_stop, dflash_accept_decision *out_host,
                              dflash_stream_t stream);
 
+/* draft_block_sampled (metal_dflash.rs:17268-17415): the selector walk of dflash_select_draft_path,
+ * but every position draws its token from softmax(score / T) over the top_k candidates with the
+ * proposal sampler (sample_with_distribution, sampling.rs:439-453: one draw per position; skipped
+ * candidates score -inf) and the sampled token conditions the next position.  The proposal sampler
+ * must use temperature only (temperature > 0, top_k 0, top_p 1, min_p 0), as the reference demands.
+ * Blocking; outputs on the host: out_tokens_host [n] (every slot pre-filled with the anchor's
+ * top-1, slots 1.. the sampled tokens), and for position p >= 1 the sparse proposal
+ * prop_cands_host[(p-1) * top_k ..][0 .. prop_counts_host[p-1]) = (token, weight) of the candidates
+ * with positive weight in distribution order: what decide / dflash_accept_prefix take as
+ * SparseProposal.  The sampler advances by the draws made; errors: DFLASH_ERR_INVALID_TOKEN (codebook
+ * row out of range) or the sampler's own codes (NaN score, no candidate with finite score). */
+int32_t dflash_select_draft_path_sampled(dflash_ctx *ctx, const dflash_codebook *predecessor,
+                                         const dflash_codebook *successor, int32_t rank, int32_t top_k,
+                                         int32_t carry_token, int32_t n, const int32_t *topk_ids, const float *topk_vals,
+                                         const float *sel_h, dflash_sampler *proposal_sampler, int32_t *out_tokens_host,
+                                         int32_t *prop_counts_host, dflash_weighted_candidate *prop_cands_host,
+                                         dflash_stream_t stream);
+
 /* ---- target model, session, packed verify -----------------------------------------------
  * Weights stay GGUF quant blocks used in place (crates/qwen-llm/src/lib.rs:17-18): a tensor is
  * a type tag and a device pointer to row-major [n_out][n_in/blk] blocks.  Norm weights are f32.

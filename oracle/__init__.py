@@ -176,6 +176,8 @@ def _declare(L):
     L.orc_dflash2_conv.restype = None
     L.orc_codebook_row.argtypes = [C.POINTER(Codebook), sz, vp]
     L.orc_select_draft_path.argtypes = [C.POINTER(Codebook), C.POINTER(Codebook), sz, sz, i32, sz, vp, vp, vp, vp, vp, vp]
+    L.orc_select_draft_path_sampled.argtypes = [C.POINTER(Codebook), C.POINTER(Codebook), sz, sz, i32, sz, vp, vp, vp,
+                                                C.POINTER(Sampler), vp, vp, C.POINTER(WeightedCandidate), C.POINTER(sz)]
 
 
 def _p(a: np.ndarray):
@@ -498,3 +500,19 @@ def select_draft_path(pred_cb, succ_cb, top_k: int, rank: int, carry: int, n: in
     if rc:
         raise ValueError("selector codebook row out of range")
     return out, scores, valid
+
+
+def select_draft_path_sampled(pred_cb, succ_cb, top_k: int, rank: int, carry: int, n: int, ids, vals, sel_h, proposal: Sampler):
+    """Returns (rc, tokens [n], proposals: one [(token, weight), ...] per position 1..n-1, err_pos); advances `proposal`."""
+    ids = np.ascontiguousarray(ids, np.int32)
+    vals = np.ascontiguousarray(vals, np.float32)
+    sel_h = np.ascontiguousarray(sel_h, np.float32)
+    out = np.zeros(n, np.int32)
+    counts = np.zeros(max(n - 1, 1), np.int32)
+    cands = (WeightedCandidate * (max(n - 1, 1) * top_k))()
+    err_pos = C.c_size_t(0)
+    rc = lib().orc_select_draft_path_sampled(C.byref(pred_cb), C.byref(succ_cb), top_k, rank, carry, n, ids.ctypes.data,
+                                             vals.ctypes.data, sel_h.ctypes.data, C.byref(proposal), out.ctypes.data,
+                                             counts.ctypes.data, cands, C.byref(err_pos))
+    props = [[(cands[p * top_k + i].token, cands[p * top_k + i].weight) for i in range(counts[p])] for p in range(n - 1)]
+    return rc, out, props, err_pos.value

@@ -109,3 +109,76 @@ done:
     free(pred);
     return rc;
 }
+
+/* draft_block_sampled (metal_dflash.rs:17268-17415): the walk above, but each position's token is
+ * drawn by sample_with_distribution (sampling.rs:439-453) over the top_k scores (skipped candidates
+ * score -inf) with the proposal sampler, one committed draw per position.  out[] is pre-filled with
+ * ids[0]; counts[pos-1] / cands[(pos-1)*top_k ..] receive the candidates with positive weight as
+ * (token id, weight) in distribution order.  Returns 0, -1 for a codebook row out of range, or the
+ * sampler's ORC_* code; *err_pos is the position of the error. */
+int orc_select_draft_path_sampled(const orc_codebook *pred_cb, const orc_codebook *succ_cb, size_t top_k, size_t rank,
+                                  int32_t carry, size_t n, const int32_t *ids, const float *vals, const float *sel_h,
+                                  orc_sampler *proposal, int32_t *out, int32_t *counts, orc_weighted_candidate *cands,
+                                  size_t *err_pos) {
+    float *pred = (float *)malloc(sizeof(float) * (rank * 3 + top_k));
+    orc_weighted_candidate *dc = (orc_weighted_candidate *)malloc(sizeof(orc_weighted_candidate) * top_k);
+    int rc = 0;
+    if (!pred || !dc) {
+        rc = -1;
+        goto done;
+    }
+    float *succ = pred + rank, *gate = succ + rank, *scores = gate + rank;
+    for (size_t p = 0; p < n; p++) out[p] = ids[0];
+    if (n == 0) goto done;
+    if (carry < 0 || orc_codebook_row(pred_cb, (size_t)carry, pred)) {
+        rc = -1;
+        if (err_pos) *err_pos = 0;
+        goto done;
+    }
+    for (size_t pos = 1; pos < n; pos++) {
+        if (err_pos) *err_pos = pos;
+        const float *hrow = sel_h + pos * rank;
+        for (size_t r = 0; r < rank; r++) gate[r] = pred[r] * hrow[r];
+        for (size_t b = 0; b < top_k; b++) {
+            scores[b] = -INFINITY;
+            const int32_t cand = ids[pos * top_k + b];
+            if (cand < 0 || (size_t)cand >= succ_cb->n_rows) continue;
+            if (orc_codebook_row(succ_cb, (size_t)cand, succ)) {
+                rc = -1;
+                goto done;
+            }
+            float dot = 0.0f;
+            for (size_t r = 0; r < rank; r++) dot += gate[r] * succ[r];
+            scores[b] = vals[pos * top_k + b] + dot;
+        }
+        orc_sampler next = *proposal;
+        const double u = orc_sampler_next_unit(&next);
+        size_t n_c = 0, idx = 0;
+        double total = 0.0;
+        int32_t tok = 0;
+        int64_t err_index = -1;
+        rc = orc_sampler_diagnose(proposal, scores, top_k, u, dc, top_k, &n_c, &total, &tok, &idx, &err_index);
+        if (rc) goto done;
+        next.draws = proposal->draws + 1;
+        *proposal = next;
+        const int32_t chosen = ids[pos * top_k + (size_t)tok];
+        int32_t cnt = 0;
+        for (size_t i = 0; i < n_c; i++) {
+            if (!(dc[i].weight > 0.0)) continue;
+            cands[(pos - 1) * top_k + cnt].token = ids[pos * top_k + (size_t)dc[i].token];
+            cands[(pos - 1) * top_k + cnt].pad = 0;
+            cands[(pos - 1) * top_k + cnt].weight = dc[i].weight;
+            cnt++;
+        }
+        counts[pos - 1] = cnt;
+        out[pos] = chosen;
+        if (chosen < 0 || orc_codebook_row(pred_cb, (size_t)chosen, pred)) {
+            rc = -1;
+            goto done;
+        }
+    }
+done:
+    free(pred);
+    free(dc);
+    return rc;
+}

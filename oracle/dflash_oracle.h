@@ -279,6 +279,12 @@ int orc_select_draft_path(const orc_codebook *pred_cb, const orc_codebook *succ_
                           int32_t carry, size_t n, const int32_t *ids, const float *vals, const float *sel_h,
                           int32_t *out, float *scores, uint8_t *valid);
 
+/* metal_dflash.rs:17268-17415 */
+int orc_select_draft_path_sampled(const orc_codebook *pred_cb, const orc_codebook *succ_cb, size_t top_k, size_t rank,
+                                  int32_t carry, size_t n, const int32_t *ids, const float *vals, const float *sel_h,
+                                  orc_sampler *proposal, int32_t *out, int32_t *counts, orc_weighted_candidate *cands,
+                                  size_t *err_pos);
+
 #ifdef __cplusplus
 }
 #endif

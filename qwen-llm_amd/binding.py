@@ -100,6 +100,9 @@ def _declare(L):
     L.dflash_select_draft_path.restype = i32
     L.dflash_select_draft_path.argtypes = [vp, C.POINTER(CodebookC), C.POINTER(CodebookC), i32, i32, i32, i32, vp, vp, vp,
                                            vp, vp, vp]
+    L.dflash_select_draft_path_sampled.restype = i32
+    L.dflash_select_draft_path_sampled.argtypes = [vp, C.POINTER(CodebookC), C.POINTER(CodebookC), i32, i32, i32, i32, vp, vp,
+                                                   vp, C.POINTER(SamplerC), vp, vp, C.POINTER(WeightedCandidateC), vp]
     L.dflash_ctx_set_graphs.restype = None
     L.dflash_ctx_set_graphs.argtypes = [vp, i32]
     L.dflash_ctx_kernel_timing.restype = i32
@@ -340,6 +343,29 @@ class Context:
                                                        topk_ids.data_ptr(), topk_vals.data_ptr(), sel_h.data_ptr(),
                                                        out.data_ptr(), host, _stream_ptr()))
         return list(host)
+
+    def select_draft_path_sampled(self, predecessor, successor, rank: int, carry_token: int, topk_ids, topk_vals, sel_h,
+                                  proposal_sampler: Sampler):
+        """The sampled selector walk (draft_block_sampled, metal_dflash.rs:17268-17415).  Returns (tokens, proposals):
+        tokens [n] on the host and, per position 1..n-1, (token, [(token, weight), ...]): the SparseProposal list that
+        decide_dflash_accept_prefix takes.  Advances the proposal sampler by one draw per position."""
+        torch = _torch()
+        n, top_k = topk_ids.shape
+
+        def cb(pair):
+            qtype, rows = pair
+            return CodebookC(qtype, 0, rows.shape[0], rows.data_ptr())
+
+        pc, sc = cb(predecessor), cb(successor)
+        toks = (C.c_int32 * n)()
+        counts = (C.c_int32 * max(n - 1, 1))()
+        cands = (WeightedCandidateC * (max(n - 1, 1) * top_k))()
+        self._check(self._lib.dflash_select_draft_path_sampled(self._h, C.byref(pc), C.byref(sc), rank, top_k, carry_token, n,
+                                                               topk_ids.data_ptr(), topk_vals.data_ptr(), sel_h.data_ptr(),
+                                                               C.byref(proposal_sampler.c), toks, counts, cands, _stream_ptr()))
+        props = [(toks[p + 1], [(cands[p * top_k + i].token, cands[p * top_k + i].weight) for i in range(counts[p])])
+                 for p in range(n - 1)]
+        return list(toks), props
 
     # ---- decide_dflash_accept_prefix (metal_dflash/accept.rs:76-84)
     def decide_dflash_accept_prefix(self, verified_tokens, target_logits, vocab, proposals, sampler: Sampler,

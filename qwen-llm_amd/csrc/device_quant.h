@@ -1,5 +1,8 @@
 // Element-wise device dequantisers, bit-exact with ggml's dequantize_row_{q4_K,q6_K,q8_0}
 // (y = (d*sc)*q - (dmin*m), y = (d*sc)*(q-32), y = d*q; every product rounded separately).
+// The compiler may fuse the last multiply into the subtraction; that changes nothing: d (f16, 11
+// bits) x a 6-8 bit code x a 4-6 bit quant is at most 24 bits and exact in f32, so the fused and
+// the separately rounded forms agree on every input.
 #pragma once
 
 #include "common.h"

@@ -1,10 +1,16 @@
 // DFlash-2 extras of the block drafter: the two-tap dynamic depthwise convolution
 // (kernel_dflash2_conv_f32, kernels/dflash2.metal:40-69) and the greedy selector walk over the
 // predecessor / successor codebooks (select_draft_path, metal_dflash.rs:17176-17251; codebook rows
-// DFlash2Codebook::dequant_row, :3275-3343).  The per-row top-16 that feeds the walk is
-// dflash_top16.
+// DFlash2Codebook::dequant_row, :3275-3343) with its sampled form (draft_block_sampled,
+// :17268-17415).  The per-row top-16 that feeds the walk is dflash_top16.
 #include "common.h"
 #include "device_quant.h"
+#include "sampler_chain.h"
+
+// The walk's scores follow the reference's scalar loop: every product and every addition is
+// rounded on its own: plain operators with contraction switched off (the __f*_rn intrinsics do not
+// stop the compiler from fusing them).
+#pragma clang fp contract(off)
 
 namespace {
 
@@ -24,7 +30,7 @@ __global__ void __launch_bounds__(256)
     for (int tap = 0; tap < kernel_size && tap <= t; tap++) {
         const float b = base[base_side + static_cast<size_t>(tap) * h + c];
         const float d = dyn[dyn_row + static_cast<size_t>(tap) * n_groups + g];
-        acc = __fmaf_rn(__fadd_rn(b, d), x[static_cast<size_t>(t - tap) * h + c], acc);
+        acc = __builtin_fmaf(b + d, x[static_cast<size_t>(t - tap) * h + c], acc);
     }
     y[gid] = acc;
 }
@@ -48,23 +54,43 @@ constexpr int kSelThreads = 256;
 constexpr int kSelMaxTopK = 16;
 constexpr int kSelMaxRank = 1024;
 
+// What the sampled walk reports besides the tokens.
+struct SampledOut {
+    int32_t status;      // 0, 1 = predecessor row out of range, else a DFLASH_ERR_* of the sampler
+    int32_t err_pos;     // position of that error
+    int32_t n_sampled;   // positions whose draw was made (the proposal sampler advances by this)
+    int32_t pad;
+    int32_t counts[16];                          // candidates with positive weight per position (index pos - 1)
+    dflash_weighted_candidate cands[15 * 16];    // [pos - 1][top_k], distribution order
+};
+
 // The walk, one workgroup.  Per position: all threads dequantise the candidates' successor rows and
 // form gate = pred * sel_h[pos] in LDS; thread b then scores candidate b with the reference's scalar
 // loop (products and additions rounded separately, rank order), thread 0 keeps the first strict
-// maximum, and all threads fetch the winner's predecessor row.  status: 0, or 1 when a predecessor
-// row is out of range (the walk stops there).
+// maximum (greedy) or samples from softmax(score / T) with the sampler chain and the position's
+// pre-drawn uniform (SAMPLED), and all threads fetch the winner's predecessor row.  status: 0, or 1
+// when a predecessor row is out of range (the walk stops there).
+template <bool SAMPLED>
 __global__ void __launch_bounds__(kSelThreads)
     dflash2_select_kernel(Codebook pred_cb, Codebook succ_cb, int top_k, int rank, int carry, int n,
                           const int32_t *__restrict__ ids, const float *__restrict__ vals,
-                          const float *__restrict__ sel_h, int32_t *__restrict__ out, int32_t *__restrict__ status) {
+                          const float *__restrict__ sel_h, int32_t *__restrict__ out, int32_t *__restrict__ status,
+                          float temperature, const double *__restrict__ uniforms, SampledOut *__restrict__ sampled) {
     extern __shared__ float lds[];  // pred[rank], gate[rank], succ[top_k][rank]
     __shared__ float score[kSelMaxTopK];
     __shared__ int chosen_s;
     float *pred = lds, *gate = lds + rank, *succ = lds + 2 * rank;
     const int tid = threadIdx.x;
+    __shared__ RowDist dist;
     if (tid == 0) {
         out[0] = ids[0];
         *status = 0;
+        if (SAMPLED) {
+            sampled->status = 0;
+            sampled->err_pos = 0;
+            sampled->n_sampled = 0;
+            for (int p = 1; p < n; p++) out[p] = ids[0];  // the reference pre-fills every slot with the anchor's top-1
+        }
     }
     if (n < 2) return;
     if (carry < 0 || carry >= pred_cb.n_rows) {
@@ -75,7 +101,7 @@ __global__ void __launch_bounds__(kSelThreads)
     __syncthreads();
     for (int pos = 1; pos < n; pos++) {
         const float *hrow = sel_h + static_cast<size_t>(pos) * rank;
-        for (int r = tid; r < rank; r += kSelThreads) gate[r] = __fmul_rn(pred[r], hrow[r]);
+        for (int r = tid; r < rank; r += kSelThreads) gate[r] = pred[r] * hrow[r];
         for (int e = tid; e < top_k * rank; e += kSelThreads) {
             const int b = e / rank, r = e - b * rank;
             const int32_t cand = ids[pos * top_k + b];
@@ -88,27 +114,84 @@ __global__ void __launch_bounds__(kSelThreads)
             if (cand >= 0 && cand < succ_cb.n_rows) {
                 float dot = 0.0f;
                 const float *sr = succ + tid * rank;
-                for (int r = 0; r < rank; r++) dot = __fadd_rn(dot, __fmul_rn(gate[r], sr[r]));
-                s = __fadd_rn(vals[pos * top_k + tid], dot);
+                for (int r = 0; r < rank; r++) dot += gate[r] * sr[r];  // two roundings each (contraction is off in this file)
+                s = vals[pos * top_k + tid] + dot;
             }
             score[tid] = s;
         }
         __syncthreads();
         if (tid == 0) {
             int best_b = 0;
-            float best = -INFINITY;
-            for (int b = 0; b < top_k; b++) {
-                const int32_t cand = ids[pos * top_k + b];
-                if (cand < 0 || cand >= succ_cb.n_rows) continue;
-                if (score[b] > best) {
-                    best = score[b];
-                    best_b = b;
+            if (!SAMPLED) {
+                float best = -INFINITY;
+                for (int b = 0; b < top_k; b++) {
+                    const int32_t cand = ids[pos * top_k + b];
+                    if (cand < 0 || cand >= succ_cb.n_rows) continue;
+                    if (score[b] > best) {
+                        best = score[b];
+                        best_b = b;
+                    }
+                }
+            } else {
+                // scores of skipped candidates are -inf; the "tokens" of the distribution are candidate indices
+                uint64_t keys[kSelMaxTopK];
+                int nan_at = -1;
+                for (int b = 0; b < top_k; b++) {
+                    const int32_t cand = ids[pos * top_k + b];
+                    const float sc = (cand < 0 || cand >= succ_cb.n_rows) ? -INFINITY : score[b];
+                    if (sc != sc && nan_at < 0) nan_at = b;
+                    const uint64_t key = cand_key(static_cast<uint32_t>(b), sc);
+                    int j = b;  // insertion sort, ascending keys = best first
+                    while (j > 0 && keys[j - 1] > key) {
+                        keys[j] = keys[j - 1];
+                        j--;
+                    }
+                    keys[j] = key;
+                }
+                dist.err = 0;
+                if (nan_at >= 0) {
+                    dist.err = DFLASH_ERR_NAN_LOGIT;
+                } else {
+                    ChainCfg cc = {};
+                    cc.temperature = temperature;
+                    cc.top_p = 1.0f;
+                    cc.min_p = 0.0f;
+                    cc.k = top_k;
+                    run_chain(keys, top_k, cc, &dist);
+                }
+                if (dist.err) {
+                    sampled->status = dist.err;
+                    sampled->err_pos = pos;
+                    *status = dist.err;
+                    chosen_s = -1;
+                } else {
+                    const int idx = pick_index(dist.weights, dist.n_keep, uniforms[pos - 1] * dist.total);
+                    best_b = dist.tokens[idx];
+                    sampled->n_sampled = pos;
+                    int cnt = 0;
+                    for (int i = 0; i < dist.n_keep; i++) {
+                        if (!(dist.weights[i] > 0.0)) continue;
+                        dflash_weighted_candidate &wc = sampled->cands[(pos - 1) * top_k + cnt++];
+                        wc.token = ids[pos * top_k + dist.tokens[i]];
+                        wc.weight = dist.weights[i];
+                    }
+                    sampled->counts[pos - 1] = cnt;
                 }
             }
+            if (SAMPLED && *status) {
+                // sampler error: stop the walk
+            } else {
             const int32_t chosen = ids[pos * top_k + best_b];
             out[pos] = chosen;
             chosen_s = chosen;
-            if (chosen < 0 || chosen >= pred_cb.n_rows) *status = 1;
+            if (chosen < 0 || chosen >= pred_cb.n_rows) {
+                *status = 1;
+                if (SAMPLED) {
+                    sampled->status = 1;
+                    sampled->err_pos = pos;
+                }
+            }
+            }
         }
         __syncthreads();
         const int chosen = chosen_s;
@@ -172,17 +255,17 @@ extern "C" int32_t dflash_select_draft_path(dflash_ctx *ctx, const dflash_codebo
     if (!status) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "select_draft_path: workspace too small");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const size_t lds = static_cast<size_t>(2 + top_k) * rank * sizeof(float);
-    if (lds > 64 * 1024) {
+    if (lds > 48 * 1024) {
         static bool attr = false;
         if (!attr) {
-            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(dflash2_select_kernel),
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(dflash2_select_kernel<false>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                                    (2 + kSelMaxTopK) * kSelMaxRank * static_cast<int>(sizeof(float))));
             attr = true;
         }
     }
-    dflash2_select_kernel<<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
-                                                       out_tokens, status);
+    dflash2_select_kernel<false><<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
+                                                              out_tokens, status, 0.0f, nullptr, nullptr);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     if (out_tokens_host) {
         // the blocking form also reports an invalid predecessor row, as the reference's CPU walk does
@@ -191,6 +274,68 @@ extern "C" int32_t dflash_select_draft_path(dflash_ctx *ctx, const dflash_codebo
         DFL_HIP_CHECK(ctx, hipMemcpyAsync(&status_host, status, sizeof(int32_t), hipMemcpyDeviceToHost, st));
         DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
         if (status_host) return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "select_draft_path: selector codebook row out of range");
+    }
+    return DFLASH_OK;
+}
+
+extern "C" int32_t dflash_select_draft_path_sampled(dflash_ctx *ctx, const dflash_codebook *predecessor,
+                                                    const dflash_codebook *successor, int32_t rank, int32_t top_k,
+                                                    int32_t carry_token, int32_t n, const int32_t *topk_ids,
+                                                    const float *topk_vals, const float *sel_h,
+                                                    dflash_sampler *proposal_sampler, int32_t *out_tokens_host,
+                                                    int32_t *prop_counts_host, dflash_weighted_candidate *prop_cands_host,
+                                                    dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!topk_ids || !topk_vals || !sel_h || !proposal_sampler || !out_tokens_host || !prop_counts_host || !prop_cands_host)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "select_draft_path_sampled: null pointer");
+    if (n < 1 || n > 16 || top_k < 1 || top_k > kSelMaxTopK || rank < 1 || rank > kSelMaxRank)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "select_draft_path_sampled: n %d top_k %d rank %d", n, top_k, rank);
+    const dflash_sampling_config &pc_cfg = proposal_sampler->cfg;
+    if (!(pc_cfg.temperature > 0.0f) || pc_cfg.top_k != 0 || pc_cfg.top_p != 1.0f || pc_cfg.min_p != 0.0f)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT,
+                        "select_draft_path_sampled: the proposal sampler must use temperature without target filters");
+    Codebook pc, sc;
+    int32_t rc;
+    if ((rc = check_codebook(ctx, predecessor, rank, &pc, "predecessor"))) return rc;
+    if ((rc = check_codebook(ctx, successor, rank, &sc, "successor"))) return rc;
+    size_t off = 0;
+    int32_t *status = dfl_ws_take<int32_t>(ctx, &off, sizeof(int32_t));
+    int32_t *out_dev = dfl_ws_take<int32_t>(ctx, &off, 16 * sizeof(int32_t));
+    double *uniforms = dfl_ws_take<double>(ctx, &off, 16 * sizeof(double));
+    SampledOut *sampled = dfl_ws_take<SampledOut>(ctx, &off, sizeof(SampledOut));
+    if (!status || !out_dev || !uniforms || !sampled)
+        return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "select_draft_path_sampled: workspace too small");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // one uniform per position, drawn ahead; the sampler is advanced afterwards by the draws actually made
+    double u_host[16] = {0};
+    if (n > 1) dflash_sampler_peek(proposal_sampler, n - 1, u_host);
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(uniforms, u_host, sizeof(u_host), hipMemcpyHostToDevice, st));
+    const size_t lds = static_cast<size_t>(2 + top_k) * rank * sizeof(float);
+    if (lds > 48 * 1024) {
+        static bool attr = false;
+        if (!attr) {
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(dflash2_select_kernel<true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (2 + kSelMaxTopK) * kSelMaxRank * static_cast<int>(sizeof(float))));
+            attr = true;
+        }
+    }
+    dflash2_select_kernel<true><<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
+                                                             out_dev, status, pc_cfg.temperature, uniforms, sampled);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    static SampledOut host;  // 4 KB; calls on one context are serial
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(&host, sampled, sizeof(host), hipMemcpyDeviceToHost, st));
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(out_tokens_host, out_dev, n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+    // every completed position consumed one draw, as each sample_with_distribution call commits its own
+    dflash_sampler_advance(proposal_sampler, static_cast<uint64_t>(host.n_sampled));
+    if (host.status == 1)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "select_draft_path_sampled: selector codebook row out of range at position %d",
+                        host.err_pos);
+    if (host.status) return dfl_fail(ctx, host.status, "select_draft_path_sampled: sampler error at position %d", host.err_pos);
+    for (int p = 0; p + 1 < n; p++) {
+        prop_counts_host[p] = host.counts[p];
+        for (int i = 0; i < host.counts[p]; i++) prop_cands_host[p * top_k + i] = host.cands[p * top_k + i];
     }
     return DFLASH_OK;
 }

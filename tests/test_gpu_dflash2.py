@@ -105,3 +105,61 @@ def test_walk_matches_oracle_on_random_lattices(ctx, oracle, kind, n):
         want, _, _ = oracle.select_draft_path(pc, sc, top_k, rank, carry, n, ids, vals, sel_h)
         got = walk_gpu(ctx, (tt, pred_rows), (tt, succ_rows), rank, carry, ids, vals, sel_h)
         assert got == want.tolist(), f"{kind} n={n} seed={seed}"
+
+
+@pytest.mark.parametrize("kind", ["q4_k", "f32"])
+def test_sampled_walk_matches_oracle(ctx, oracle, kind):
+    """draft_block_sampled (metal_dflash.rs:17268-17415): tokens, the sparse proposals (candidate token ids in
+    distribution order, weights to the last place of the f64 exponential) and the proposal sampler's stream position, against the oracle's
+    restatement (its sampler chain is pinned by tests/test_oracle_pins.py), over seeded lattices with sentinels."""
+    rank, top_k, vocab, n = 256, 16, 2048, 16
+    for seed in range(8):
+        rng = np.random.default_rng(7000 + seed)
+        if kind == "q4_k":
+            tt, ot = dfl.TYPE_Q4_K, oracle.Q4_K
+            pred_rows = dfl.synth.random_weight(dfl.synth.Q4_K, vocab, rank, seed=2 * seed)
+            succ_rows = dfl.synth.random_weight(dfl.synth.Q4_K, vocab, rank, seed=2 * seed + 1)
+        else:
+            tt, ot = dfl.TYPE_F32, oracle.F32
+            pred_rows = (rng.standard_normal((vocab, rank)) * 0.05).astype(np.float32)
+            succ_rows = (rng.standard_normal((vocab, rank)) * 0.05).astype(np.float32)
+        ids = np.stack([rng.permutation(vocab)[:top_k] for _ in range(n)]).astype(np.int32)
+        ids[rng.random((n, top_k)) < 0.1] = -1
+        ids[:, 0] = rng.integers(0, vocab, n)
+        vals = np.sort(rng.standard_normal((n, top_k)).astype(np.float32) * 2, axis=1)[:, ::-1].copy()
+        sel_h = rng.standard_normal((n, rank)).astype(np.float32)
+        carry = int(rng.integers(0, vocab))
+        temperature = [0.7, 1.0, 0.3][seed % 3]
+        osamp = oracle.make_sampler(temperature=temperature, top_k=0, top_p=1.0, min_p=0.0, seed=99 + seed)
+        pc, k1 = oracle.make_codebook(ot, pred_rows, rank)
+        sc, k2 = oracle.make_codebook(ot, succ_rows, rank)
+        rc, want_tokens, want_props, _ = oracle.select_draft_path_sampled(pc, sc, top_k, rank, carry, n, ids, vals, sel_h, osamp)
+        assert rc == 0
+        gsamp = dfl.Sampler(temperature=temperature, top_k=0, top_p=1.0, min_p=0.0, seed=99 + seed)
+        import torch
+
+        got_tokens, got_props = ctx.select_draft_path_sampled(
+            (tt, torch.from_numpy(pred_rows).cuda()), (tt, torch.from_numpy(succ_rows).cuda()), rank, carry,
+            torch.from_numpy(ids).cuda(), torch.from_numpy(vals).cuda(), torch.from_numpy(sel_h).cuda(), gsamp)
+        assert got_tokens == want_tokens.tolist(), f"{kind} seed {seed}"
+        assert gsamp.draws == int(osamp.draws) == n - 1
+        for p in range(n - 1):
+            tok, cands = got_props[p]
+            assert tok == want_tokens[p + 1]
+            assert [t for t, _ in cands] == [t for t, _ in want_props[p]], f"{kind} seed {seed} position {p + 1}"
+            # f64 exp on the device and in the host libm may differ in the last place
+            gw, ww = np.array([w for _, w in cands]), np.array([w for _, w in want_props[p]])
+            assert np.allclose(gw, ww, rtol=1e-12, atol=0.0), f"{kind} seed {seed} position {p + 1}: {np.max(np.abs(gw - ww) / ww)} {gw} {ww}"
+
+
+def test_sampled_walk_rejects_target_filters(ctx):
+    import torch
+
+    rows = torch.zeros((4, 32), device="cuda")
+    ids = torch.zeros((2, 2), dtype=torch.int32, device="cuda")
+    vals = torch.zeros((2, 2), device="cuda")
+    h = torch.zeros((2, 32), device="cuda")
+    for bad in (dict(temperature=0.0), dict(temperature=0.7, top_k=20), dict(temperature=0.7, top_p=0.9),
+                dict(temperature=0.7, min_p=0.1)):
+        with pytest.raises(dfl.DFlashError):
+            ctx.select_draft_path_sampled((dfl.TYPE_F32, rows), (dfl.TYPE_F32, rows), 32, 0, ids, vals, h, dfl.Sampler(seed=1, **bad))
