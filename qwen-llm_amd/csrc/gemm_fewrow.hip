@@ -684,6 +684,305 @@ __global__ void __launch_bounds__(64 * kWaves)
 }
 
 // ----------------------------------------------------------------------------
+// Q6_K streaming kernel
+// ----------------------------------------------------------------------------
+//
+// Same work split, activation path, flush and split-K reduction as the Q4_K stream above (one
+// workgroup per CU walks a contiguous range of (tile group x super-block), activations of a stage
+// are converted once per workgroup into MFMA fragments in LDS).  The weight path differs: a Q6_K
+// block is 210 bytes, so rows are only 2-byte aligned and are not copied straight into LDS.
+// Instead every wave stages its own 16 rows: the 13 16-byte pieces of each row's block (and its f16
+// d) are loaded into registers one stage ahead with wide unaligned loads - consecutive lanes take
+// consecutive pieces, so a row's 208 bytes are fetched as one run - and written to a private,
+// double-buffered LDS area at the top of the next stage.  Private areas need no barrier; the one
+// barrier per stage is for the shared activation fragments.
+//
+// Lane (n, g) of a wave serves weight row n, half h = g / 2 of the super-block and, in that half, the
+// quarters (g & 1) and 2 + (g & 1): the low and the high nibbles of the SAME 32 ql bytes, with the
+// bit pairs 2 (g & 1) and 4 + 2 (g & 1) of the half's 32 qh bytes.  MFMA t < 4 takes elements
+// 8 t .. 8 t + 7 of the low quarter, t >= 4 those of the high quarter.  A 6-bit value is assembled
+// in the mantissa of an f16 1024.0 (low nibble | qh bits << 4) or 64.0 (high nibble, sitting four
+// bits up, | qh bits << 8), and one packed fma per pair gives round(q * s), s = d * scale, exactly as
+// for Q4_K.  The format's offset, -32 s per weight, is not folded into that fma (-1056 s is not
+// exact in f16 and the error would be a quarter of a quant step on every weight of a sub-block):
+// like the Q4_K minima it goes through a twin MFMA, the same activation fragment times 32 s
+// repeated eight times, into a second accumulator that is subtracted at the end.
+constexpr int kQ6KRowStride = 240;  // bytes between a wave's staged rows in LDS (210 used)
+
+template <int kWaves>
+struct Q6KGeom {
+    static constexpr int kThreads = 64 * kWaves;
+    static constexpr int kRows = 16 * kWaves;
+    static constexpr int kWaveBytes = 16 * kQ6KRowStride;  // one staged block of a wave's 16 rows
+    static constexpr int kWBytes = 2 * kWaves * kWaveBytes;
+    static constexpr int kLdsBytes = kWBytes + 2 * kQ4KBlockFrags * 16;
+};
+
+// Activation item of a thread for the Q6_K lane assignment (see q4k_lane_x_offsets for the thread
+// -> (row, four values) map): values k = 4 c .. 4 c + 3 of the super-block belong to half c / 32,
+// quarter (c / 8) % 4, elements 4 (c % 8) ..
+template <int kWaves, typename XT>
+__device__ __forceinline__ void q6k_lane_x_offsets(Q4KLane<kWaves> &L, int tid, int n_rows, uint32_t n_in) {
+    using G = Q4KGeom<kWaves>;
+    const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+    for (int r = 0; r < G::kXLoads; r++) {
+        const int vw = wave + kWaves * r;
+        const int m = 8 * (vw & 1) + (lane & 7), c = 8 * (vw >> 1) + (lane >> 3);
+        const int h = c >> 5, quarter = (c >> 3) & 3, l4 = c & 7;
+        const int g = 2 * h + (quarter & 1), t = 4 * (quarter >> 1) + (l4 >> 1);
+        L.x_off[r] = (static_cast<uint32_t>(min(m, n_rows - 1)) * n_in + 4u * c) * static_cast<uint32_t>(sizeof(XT));
+        L.xw_off[r] = static_cast<uint32_t>((t * 64 + m + 16 * g) * 16 + 8 * (l4 & 1));
+    }
+}
+
+// A wave's weight registers for one stage: 208 16-byte pieces (16 rows x 13) over 64 lanes, and d.
+struct Q6KRegs {
+    u32x4_t p[4];
+    uint32_t d;
+};
+
+struct Q6KLane {
+    uint32_t g_off[4];  // global byte offset of piece j from (group's first row, super-block)
+    uint32_t l_off[4];  // its LDS byte offset in the wave's area
+    uint32_t gd_off;    // d of row (lane % 16)
+    bool live3;         // the fourth piece exists (lane + 192 < 208); other lanes re-load piece 207 and drop it
+};
+
+__device__ __forceinline__ void q6k_lane_w_offsets(Q6KLane &W, int lane, int wave, int row0, int n_out, uint32_t row_bytes) {
+    const int last = n_out - 1 - row0;  // rows past n_out (ragged last group) re-read the last row
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int i = min(lane + 64 * j, 207);
+        const int r = i / 13, piece = i % 13;
+        W.g_off[j] = static_cast<uint32_t>(min(wave * 16 + r, last)) * row_bytes + 16u * piece;
+        W.l_off[j] = static_cast<uint32_t>(r * kQ6KRowStride + 16 * piece);
+    }
+    W.live3 = lane + 192 < 208;
+    W.gd_off = static_cast<uint32_t>(min(wave * 16 + (lane & 15), last)) * row_bytes + 208u;
+}
+
+// Five loads per wave and stage (four 16-byte pieces and d), written as asm like the activation
+// loads and for the same reason: the kernel's own s_waitcnt at the top of a stage covers them, and
+// the compiler must not drain younger loads on their account.  The addresses are only 2-byte
+// aligned; gfx950 runs with unaligned vector memory access enabled.
+constexpr int kQ6KLoads = 5;
+__device__ __forceinline__ void q6k_load_w(const uint8_t *wstage, const Q6KLane &W, Q6KRegs &R) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(R.p[j]) : "v"(W.g_off[j]), "s"(wstage) : "memory");
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(R.d) : "v"(W.gd_off), "s"(wstage) : "memory");
+}
+
+// after the s_waitcnt that covers R: its uses cannot be scheduled above this point
+__device__ __forceinline__ void q6k_pin_w(Q6KRegs &R) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) asm volatile("" : "+v"(R.p[j]));
+    asm volatile("" : "+v"(R.d));
+}
+
+__device__ __forceinline__ void q6k_store_w(uint8_t *area, const Q6KLane &W, const Q6KRegs &R, int lane) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        if (j < 3 || W.live3) *reinterpret_cast<u32x4_t *>(area + W.l_off[j]) = R.p[j];
+    if (lane < 16) *reinterpret_cast<uint16_t *>(area + lane * kQ6KRowStride + 208) = static_cast<uint16_t>(R.d);
+}
+
+// Eight f16 weights of one MFMA: q = nibble | (two qh bits << 4), value round(q s).
+//   HIGH = false: low nibbles, bits pre-shifted to 0..1:   1024 + q via magic 0x6400, c = -1024 s
+//   HIGH = true : high nibbles (four bits up), qh bits go eight bits up: 64 + q via 0x5400, c = -64 s
+template <bool HIGH>
+__device__ __forceinline__ half8_t unpack6(uint32_t w0, uint32_t w1, uint32_t h0, uint32_t h1, half2_t s2, half2_t c2,
+                                           uint32_t magic) {
+    constexpr uint32_t mask = HIGH ? 0x00F000F0u : 0x000F000Fu;
+    constexpr int up = HIGH ? 8 : 4;
+    auto one = [&](uint32_t w, uint32_t h) {
+        const uint32_t bits = ((w & mask) | magic) | ((h & 0x00030003u) << up);
+        return __builtin_elementwise_fma(as_half2(bits), s2, c2);
+    };
+    const half2_t p0 = one(w0, h0), p1 = one(w0 >> 8, h0 >> 8), p2 = one(w1, h1), p3 = one(w1 >> 8, h1 >> 8);
+    half8_t r = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+    return r;
+}
+
+template <int kWaves, typename XT>
+__global__ void __launch_bounds__(64 * kWaves)
+    gemm_q6k_stream_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
+                           float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt) {
+    using G6 = Q6KGeom<kWaves>;
+    using G = Q4KGeom<kWaves>;
+    extern __shared__ half8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    Q4KRange rg;
+    rg.nb = nb;
+    rg.n_wg = gridDim.x;
+    rg.total = n_groups * nb;
+    rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
+    rg.it_begin = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * rg.wg, bt.by_wg));
+    rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * (rg.wg + 1), bt.by_wg));
+    if (rg.it_begin >= rg.it_end) return;
+    rg.first_group = static_cast<int>(q4k_div(rg.it_begin, bt.by_nb));
+    const int b0 = rg.it_begin - rg.first_group * nb;
+    const uint32_t row_bytes = static_cast<uint32_t>(nb) * DFL_Q6_K_BYTES;
+    const uint32_t n_in = static_cast<uint32_t>(nb) * DFL_QK_K;
+    const size_t group_bytes = static_cast<size_t>(G6::kRows) * row_bytes;
+    constexpr uint32_t kXBlockBytes = DFL_QK_K * sizeof(XT);
+    const bool ragged = n_groups * G6::kRows > n_out;
+
+    Q6KLane W;
+    q6k_lane_w_offsets(W, lane, wave, rg.first_group * G6::kRows, n_out, row_bytes);
+    // cursors: weights (next stage to load), activations (next to load), compute
+    const uint8_t *wstage = q4k_uniform(w + static_cast<size_t>(rg.first_group) * group_bytes + static_cast<size_t>(b0) * DFL_Q6_K_BYTES);
+    int bw = b0, gw = rg.first_group, w_left = rg.it_end - rg.it_begin;
+    const uint8_t *xblock = q4k_uniform(reinterpret_cast<const uint8_t *>(x) + static_cast<size_t>(b0) * kXBlockBytes);
+    int bx = b0, x_left = w_left;
+    auto advance_w = [&]() {
+        wstage += DFL_Q6_K_BYTES;
+        w_left--;
+        if (++bw == nb) {
+            bw = 0;
+            gw++;
+            if (w_left > 0) {
+                wstage = q4k_uniform(w + static_cast<size_t>(gw) * group_bytes);
+                if (ragged) q6k_lane_w_offsets(W, lane, wave, gw * G6::kRows, n_out, row_bytes);
+            }
+        }
+    };
+    auto advance_x = [&]() {
+        xblock += kXBlockBytes;
+        x_left--;
+        if (++bx == nb) {
+            bx = 0;
+            if (x_left > 0) xblock = reinterpret_cast<const uint8_t *>(x);
+        }
+    };
+    uint8_t *area = reinterpret_cast<uint8_t *>(lds) + wave * (2 * G6::kWaveBytes);  // this wave's two weight buffers
+    half8_t *x_c = reinterpret_cast<half8_t *>(reinterpret_cast<uint8_t *>(lds) + G6::kWBytes), *x_n = x_c + kQ4KBlockFrags;
+
+    // prologue: weights of stage 0 into LDS, those of stage 1 into registers; activations of stages 0..2.
+    // Load order from here on: ... W(d+1) at the top of stage d-1 | X(d+2) at its end | W(d+2) at the top
+    // of stage d ...; the wait at the top of stage d leaves only the youngest activation loads in flight.
+    Q6KRegs R;
+    q6k_load_w(wstage, W, R);
+    advance_w();
+    Q4KLane<kWaves> L;
+    q6k_lane_x_offsets<kWaves, XT>(L, tid, n_rows, n_in);
+    Q4KXRaw<kWaves, XT> raw_first, raw_a, raw_b;
+    q4k_load_x<kWaves, XT>(xblock, L, raw_first);
+    advance_x();
+    if (x_left > 0) {
+        q4k_load_x<kWaves, XT>(xblock, L, raw_a);
+        advance_x();
+    }
+    __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+    q6k_pin_w(R);
+    q4k_pin_x<kWaves, XT>(raw_first);
+    q4k_pin_x<kWaves, XT>(raw_a);
+    q6k_store_w(area, W, R, lane);
+    if (w_left > 0) {
+        q6k_load_w(wstage, W, R);
+        advance_w();
+    }
+    bool young_x = false;
+    if (x_left > 0) {
+        q4k_load_x<kWaves, XT>(xblock, L, raw_b);
+        advance_x();
+        young_x = true;
+    }
+
+    const int n = lane & 15, g = lane >> 4;
+    const int h = g >> 1, odd = g & 1;
+    const uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+    float4_t acc = {0, 0, 0, 0}, acc_off = {0, 0, 0, 0};
+    int gc = rg.first_group, bc = b0, n_left = rg.it_end - rg.it_begin;
+    int cur = 0;  // weight buffer of the stage being computed
+    bool first = true;
+    auto stage = [&](Q4KXRaw<kWaves, XT> &raw) {
+        // everything but the activation loads issued at the end of the previous stage has landed:
+        // the next stage's weights (in R) and the next stage's activations (in raw)
+        if (young_x)
+            __builtin_amdgcn_s_waitcnt(q4k_vmcnt(G::kXLoads));
+        else
+            __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+        q6k_pin_w(R);
+        q4k_pin_x<kWaves, XT>(raw);
+        // the next stage's weights go into the other buffer, the ones after that into the registers
+        if (n_left > 1) q6k_store_w(area + (cur ^ 1) * G6::kWaveBytes, W, R, lane);
+        if (w_left > 0) {
+            q6k_load_w(wstage, W, R);
+            advance_w();
+        }
+        if (first) q4k_write_x<kWaves, XT>(x_c, L, raw_first);
+        first = false;
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        __builtin_amdgcn_s_barrier();  // the stage's activation fragments are complete; the other fragment buffer is free
+        const uint8_t *rowp = area + cur * G6::kWaveBytes + n * kQ6KRowStride;
+        const u32x4_t qa = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd);
+        const u32x4_t qb = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd + 16);
+        u32x4_t ha = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h);
+        u32x4_t hb = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h + 16);
+        // scales of the half: bytes 2 q + (0, 1) belong to quarter q
+        const uint32_t sc4 = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h) >> (16 * odd)) & 0xffffu;       // low quarter
+        const uint32_t sc4h = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h + 4) >> (16 * odd)) & 0xffffu;  // high quarter
+        const float d = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(rowp + 208)));
+        const half8_t *a = x_c + lane;
+        half8_t af[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) af[t] = a[t * 64];
+        // this lane's qh bit pairs start at bit 2 odd (low quarter) and 4 + 2 odd (high quarter)
+        const int hs = 2 * odd;
+        const uint32_t hq[8] = {ha.x >> hs, ha.y >> hs, ha.z >> hs, ha.w >> hs, hb.x >> hs, hb.y >> hs, hb.z >> hs, hb.w >> hs};
+        const uint32_t ql[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        auto scale = [&](uint32_t pair, int j) {
+            return static_cast<_Float16>(d * static_cast<float>(static_cast<int8_t>(pair >> (8 * j))));
+        };
+        const _Float16 s_l0 = scale(sc4, 0), s_l1 = scale(sc4, 1), s_h0 = scale(sc4h, 0), s_h1 = scale(sc4h, 1);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const _Float16 sl = (t >> 1) ? s_l1 : s_l0;
+            half8_t bl = unpack6<false>(ql[2 * t], ql[2 * t + 1], hq[2 * t], hq[2 * t + 1], splat(sl),
+                                        splat(sl * static_cast<_Float16>(-1024.0f)), magic_lo);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
+            const _Float16 o = sl * static_cast<_Float16>(32.0f);
+            const half8_t bo = {o, o, o, o, o, o, o, o};
+            acc_off = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bo, acc_off, 0, 0, 0);
+        }
+        if (n_left > 1) q4k_write_x<kWaves, XT>(x_n, L, raw);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const _Float16 sh = (t >> 1) ? s_h1 : s_h0;
+            half8_t bh = unpack6<true>(ql[2 * t], ql[2 * t + 1], hq[2 * t] >> 4, hq[2 * t + 1] >> 4, splat(sh),
+                                       splat(sh * static_cast<_Float16>(-64.0f)), magic_hi);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bh, acc, 0, 0, 0);
+            const _Float16 o = sh * static_cast<_Float16>(32.0f);
+            const half8_t bo = {o, o, o, o, o, o, o, o};
+            acc_off = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bo, acc_off, 0, 0, 0);
+        }
+        young_x = x_left > 0;
+        if (young_x) {
+            q4k_load_x<kWaves, XT>(xblock, L, raw);
+            advance_x();
+        }
+        cur ^= 1;
+        half8_t *tx = x_c;
+        x_c = x_n;
+        x_n = tx;
+        n_left--;
+        if (++bc == nb || n_left == 0) {
+            q4k_flush<kWaves>(rg, bt, gc, acc, acc_off, y, partials, n_out, n_rows, tid);
+            bc = 0;
+            gc++;
+        }
+    };
+    while (n_left > 0) {
+        stage(raw_a);
+        if (n_left == 0) break;
+        stage(raw_b);
+    }
+}
+
+// ----------------------------------------------------------------------------
 // Generic kernel (Q8_0): eight consecutive weights -> f16 -> MFMA
 // ----------------------------------------------------------------------------
 
@@ -990,6 +1289,71 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
 
 }  // namespace
 
+namespace {
+
+// The streaming Q6_K kernel (and its split-K reduction) on one matrix.
+int32_t launch_q6k_stream(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in,
+                          int64_t n_out, int32_t n_rows, hipStream_t st) {
+    const int nb = static_cast<int>(n_in / DFL_QK_K);
+    const size_t row_bytes = static_cast<size_t>(nb) * DFL_Q6_K_BYTES;
+    const int tiles = static_cast<int>((n_out + 15) / 16);
+    if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
+    int waves = (static_cast<int64_t>((tiles + 15) / 16) * nb >= 2ll * ctx->n_cu) ? 16 : 8;
+    waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
+    const int groups = (tiles + waves - 1) / waves;
+    int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
+    const int64_t total = static_cast<int64_t>(groups) * nb;
+    const int max_wgs = ctx->n_partial_wgs * 8 / waves;
+    if (n_wg > total) n_wg = static_cast<int>(total);
+    if (n_wg > max_wgs) n_wg = max_wgs;
+    if (n_wg < 1) n_wg = 1;
+    if (total * (n_wg + 1) >= (int64_t(1) << 31) || row_bytes * 256 >= (size_t(1) << 32))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: problem too large for 32-bit work indices");
+    float *partials = reinterpret_cast<float *>(ctx->partials);
+    const bool split = groups % n_wg != 0;
+    Q4KBatch bt = {};
+    bt.groups_per_mat = groups;
+    bt.by_gpm = q4k_make_div(static_cast<uint32_t>(groups));
+    bt.by_nb = q4k_make_div(static_cast<uint32_t>(nb));
+    bt.by_wg = q4k_make_div(static_cast<uint32_t>(n_wg));
+    const uint8_t *wb = static_cast<const uint8_t *>(w);
+    const int no = static_cast<int>(n_out);
+#define DFL_LAUNCH_Q6K(WAVES, XT)                                                                                      \
+    do {                                                                                                               \
+        const size_t lds = Q6KGeom<WAVES>::kLdsBytes;                                                                  \
+        if (lds > ctx->lds_bytes)                                                                                      \
+            return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: %zu bytes of LDS needed", lds);                 \
+        static bool attr = false;                                                                                      \
+        if (!attr) {                                                                                                   \
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q6k_stream_kernel<WAVES, XT>),  \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+            attr = true;                                                                                               \
+        }                                                                                                              \
+        {                                                                                                              \
+            dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                      \
+            gemm_q6k_stream_kernel<WAVES, XT><<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, \
+                                                                             no, nb, n_rows, groups, bt);              \
+        }                                                                                                              \
+        if (split) {                                                                                                   \
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                    \
+            q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);   \
+        }                                                                                                              \
+    } while (0)
+    if (waves == 16 && x_type == DFLASH_TYPE_F32)
+        DFL_LAUNCH_Q6K(16, float);
+    else if (waves == 16)
+        DFL_LAUNCH_Q6K(16, _Float16);
+    else if (x_type == DFLASH_TYPE_F32)
+        DFL_LAUNCH_Q6K(8, float);
+    else
+        DFL_LAUNCH_Q6K(8, _Float16);
+#undef DFL_LAUNCH_Q6K
+    return DFLASH_OK;
+}
+
+}  // namespace
+
 int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const void *extra_w,
                              const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
                              size_t x_stride,
@@ -1044,6 +1408,9 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
 
     if (w_type == DFLASH_TYPE_Q4_K) {
         return launch_q4k(ctx, w, x, x_type, y, n_in, n_out, n_rows, st, nullptr, 1);
+    } else if (w_type == DFLASH_TYPE_Q6_K && env_int("DFLASH_Q6K_STREAM", 1)) {
+        const int32_t rc = launch_q6k_stream(ctx, w, x, x_type, y, n_in, n_out, n_rows, st);
+        if (rc) return rc;
     } else if (w_type == DFLASH_TYPE_Q6_K) {
         Q6KSet set = {};
         set.n_mats = 1;
