@@ -20,7 +20,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, averaged over the three shapes of a step: FETCH_SIZE + WRITE_SIZE from
 # two rocprofv3 --pmc runs of this file, each scaled by what the same counter reads for a plain 256 MiB copy
 # (profiles/gemm_q4k_stream_kernel__hbm_traffic.txt).  A counter figure, not measured by this run.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 51.15e6
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 51.02e6
 
 
 def cpu_baseline(shapes, weights, xs):
@@ -81,6 +81,41 @@ def attention_section(ctx):
         out.append({"context": L, "us_per_call": us, "kv_bytes": kv_bytes, "GBps": kv_bytes / (us * 1e-6) / 1e9,
                     "frac_of_hbm_peak": kv_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS})
         del q, k, vt, o
+    return out
+
+
+def q6k_section(ctx):
+    """Few-row Q6_K GEMM, M=16, f32 activations: the output head of the end-to-end model (2048 -> 151936, 255 MB)
+    and a 5120 -> 5120 projection (21.5 MB); weights rotate over enough copies to stay out of the memory-side cache.
+    Microseconds per call (split-K reduction included) and weight GB/s."""
+    import torch
+
+    import qwen_llm_amd as dfl
+
+    out = []
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    for n_in, n_out in ((2048, 151936), (5120, 5120)):
+        nbytes = n_in * n_out * 210 // 256
+        n_sets = min(24, max(2, int(400e6 // nbytes) + 1))
+        ws = [dfl.synth.random_blocks_device(dfl.synth.Q6_K, n_out, n_in, 0.02, g, "cuda") for _ in range(n_sets)]
+        x = torch.randn((16, n_in), device="cuda", generator=g)
+        y = torch.empty((16, n_out), device="cuda")
+        for w in ws:
+            ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q6_K, x, y, n_in, n_out, 16)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 3
+        e0.record()
+        for _ in range(reps):
+            for w in ws:
+                ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q6_K, x, y, n_in, n_out, 16)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / (reps * n_sets) * 1e3
+        out.append({"n_in": n_in, "n_out": n_out, "weight_bytes": nbytes, "us_per_call": us,
+                    "GBps": nbytes / (us * 1e-6) / 1e9, "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS})
+        del ws, x, y
     return out
 
 
@@ -227,8 +262,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain 256 MiB device copy a few times (outside the timed region): the reference "
-                         "dispatch for scaling FETCH_SIZE / WRITE_SIZE counter readings")
+                    help="also run a plain 256 MiB read + 256 MiB write kernel (an int32 add) a few times, outside the timed "
+                         "region: the reference dispatch for scaling FETCH_SIZE / WRITE_SIZE counter readings")
     ap.add_argument("--rocprof-summary", metavar="DIR", help="print a text summary of a rocprofv3 CSV output directory and exit")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end speculative decode measurement")
     ap.add_argument("--e2e-tokens", type=int, default=1024)
@@ -274,10 +309,12 @@ def main():
             ctx.encode_mat_mat_dispatch_dflash_verify(w[k], dfl.TYPE_Q4_K, x, y, n_in, n_out, 16)
 
     if args.calibrate_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        # a plain streaming kernel of known traffic: reads 256 MiB, writes 256 MiB (an int32 add, so that its name
+        # differs from the device copies that made the weight sets)
+        src = torch.ones(64 << 20, dtype=torch.int32, device="cuda")
         dst = torch.empty_like(src)
         for _ in range(5):
-            dst.copy_(src)
+            torch.add(src, 1, out=dst)
         torch.cuda.synchronize()
         del src, dst
     for _ in range(args.warmup):
@@ -343,6 +380,7 @@ def main():
     del wd, xd, yd
     if not args.gemm_only:
         try:
+            out["gemm_q6k"] = q6k_section(ctx)
             out["attention"] = attention_section(ctx)
             out["acceptance"] = acceptance_section(ctx)
         except Exception as e:  # the GEMM line above stays valid
