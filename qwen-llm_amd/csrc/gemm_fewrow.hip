@@ -990,22 +990,71 @@ __device__ __forceinline__ float half_at(const uint8_t *p) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(p[0] | (p[1] << 8))));
 }
 
+// Eight weights of a row, in two halves so that the loads of several steps can be in flight before
+// the first conversion: the raw bytes, then the f16 fragment.
 template <int TYPE>
-__device__ __forceinline__ half8_t dequant8(const uint8_t *row, int64_t k0);
+struct Raw8;
 
 template <>
-__device__ __forceinline__ half8_t dequant8<DFLASH_TYPE_Q8_0>(const uint8_t *row, int64_t k0) {
-    const uint8_t *blk = row + (k0 >> 5) * DFL_Q8_0_BYTES;
-    float d = half_at(blk);
-    const int8_t *q = reinterpret_cast<const int8_t *>(blk + 2 + (k0 & 31));
-    half8_t v;
-#pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = static_cast<_Float16>(d * static_cast<float>(q[i]));
+struct Raw8<DFLASH_TYPE_Q8_0> {
+    uint64_t q;  // eight int8 quants
+    float d;
+};
+
+__device__ __forceinline__ uint64_t load_u64_unaligned(const uint8_t *p) {
+    uint64_t v;
+    __builtin_memcpy(&v, p, 8);
     return v;
 }
 
+template <int TYPE>
+__device__ __forceinline__ Raw8<TYPE> load_raw8(const uint8_t *row, int64_t k0);
+template <int TYPE>
+__device__ __forceinline__ half8_t convert_raw8(const Raw8<TYPE> &r);
+
+// Blocks are 34 bytes, so the quants are only 2-byte aligned; gfx950 runs with unaligned vector
+// memory access enabled and the copy below becomes one 8-byte load.
+template <>
+__device__ __forceinline__ Raw8<DFLASH_TYPE_Q8_0> load_raw8<DFLASH_TYPE_Q8_0>(const uint8_t *row, int64_t k0) {
+    const uint8_t *blk = row + (k0 >> 5) * DFL_Q8_0_BYTES;
+    Raw8<DFLASH_TYPE_Q8_0> r;
+    r.d = half_at(blk);
+    r.q = load_u64_unaligned(blk + 2 + (k0 & 31));
+    return r;
+}
+
+template <>
+__device__ __forceinline__ half8_t convert_raw8<DFLASH_TYPE_Q8_0>(const Raw8<DFLASH_TYPE_Q8_0> &r) {
+    half8_t v;
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = static_cast<_Float16>(r.d * static_cast<float>(static_cast<int8_t>(r.q >> (8 * i))));
+    return v;
+}
+
+// Eight consecutive activations (16-byte aligned) in two halves as well: the raw load, then the f16
+// fragment.
 template <typename XT>
-__device__ __forceinline__ half8_t load_x8(const XT *p, bool live);
+struct RawX8;
+template <>
+struct RawX8<float> {
+    float4_t a, b;
+};
+template <>
+struct RawX8<_Float16> {
+    half8_t v;
+};
+__device__ __forceinline__ RawX8<float> load_rawx8(const float *p) {
+    return RawX8<float>{*reinterpret_cast<const float4_t *>(p), *reinterpret_cast<const float4_t *>(p + 4)};
+}
+__device__ __forceinline__ RawX8<_Float16> load_rawx8(const _Float16 *p) {
+    return RawX8<_Float16>{*reinterpret_cast<const half8_t *>(p)};
+}
+__device__ __forceinline__ half8_t convert_rawx8(const RawX8<float> &r) {
+    return half8_t{static_cast<_Float16>(r.a[0]), static_cast<_Float16>(r.a[1]), static_cast<_Float16>(r.a[2]),
+                   static_cast<_Float16>(r.a[3]), static_cast<_Float16>(r.b[0]), static_cast<_Float16>(r.b[1]),
+                   static_cast<_Float16>(r.b[2]), static_cast<_Float16>(r.b[3])};
+}
+__device__ __forceinline__ half8_t convert_rawx8(const RawX8<_Float16> &r) { return r.v; }
 
 template <int TYPE, typename XT>
 __global__ void __launch_bounds__(64 * kMaxSplit)
@@ -1020,13 +1069,15 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
     row = row < n_out ? row : n_out - 1;
     const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
     const int64_t s0 = n_steps * wave / n_split, s1 = n_steps * (wave + 1) / n_split;
-    const bool x_live = n < n_rows;  // lane (m = n, g) of the A operand: activation row n, straight from the caller's matrix
-    const XT *xrow = x + static_cast<size_t>(x_live ? n : 0) * (static_cast<size_t>(n_steps) * 32) + 8 * g;
+    // lane (m = n, g) of the A operand: activation row n, straight from the caller's matrix.  Lanes
+    // past n_rows repeat the last row (a row of A only reaches the same row of the product, which is
+    // never stored for them): no branch around the loads, so the loads of all steps can be in flight
+    const XT *xrow = x + static_cast<size_t>(n < n_rows ? n : n_rows - 1) * (static_cast<size_t>(n_steps) * 32) + 8 * g;
     float4_t acc = {0, 0, 0, 0};
     for (int64_t s = s0; s < s1; s++) {
-        half8_t a = load_x8<XT>(xrow + 32 * s, x_live);
-        half8_t b = dequant8<TYPE>(rowp, 32 * s + 8 * g);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+        const RawX8<XT> a = load_rawx8(xrow + 32 * s);
+        const Raw8<TYPE> r = load_raw8<TYPE>(rowp, 32 * s + 8 * g);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(convert_rawx8(a), convert_raw8<TYPE>(r), acc, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) red[wave * 256 + (4 * g + i) * 16 + n] = acc[i];
@@ -1036,6 +1087,84 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
         if (m < n_rows && n0 + nn < n_out) {
             float sum = 0.0f;
             for (int ws = 0; ws < n_split; ws++) sum += red[ws * 256 + e];
+            y[static_cast<size_t>(m) * n_out + n0 + nn] = sum;
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------
+// Q8_0, staged: the same product with both operands brought in through LDS
+// ----------------------------------------------------------------------------
+//
+// The kernel above reads MFMA operands straight from memory: each 16-lane group of a load touches 16
+// different rows, i.e. 16 cache lines for 256 bytes, and the texture path (one line per clock) bounds
+// the kernel, not latency or bandwidth (measured: 10.5 us for a 128 x 2048 router, 6 us of it the
+// address path; issuing all loads at once changed nothing).  Here a workgroup copies its 16 weight
+// rows and the activations in row-contiguous 16-byte pieces (a wave-load = 8 full lines), converts
+// the activations to f16 once, and every wave then takes its fragments from LDS:
+//   X  [step][k-group][row] half8 pieces, a step's four groups 17 pieces apart (the writes, which
+//      walk along a row, and the fragment reads, which walk along the rows, are both conflict-free);
+//   W  the raw rows, 16 bytes of padding between rows (16 rows land in 16 different banks).
+// K is walked in chunks of 2048; waves split a chunk's 64 steps and add up in LDS in wave order, so
+// for n_in <= 2048 the result is bit-identical to the kernel above.  Needs n_in % 256 == 0 (rows of
+// 34-byte blocks are then 16-byte multiples).
+constexpr int kQ8ChunkSteps = 64;                                  // 2048 weights of a row
+constexpr int kQ8XPieces = kQ8ChunkSteps * 68;                     // padded: 4 groups x 17 pieces per step
+constexpr int kQ8WRowStride = kQ8ChunkSteps * DFL_Q8_0_BYTES + 16; // bytes
+constexpr size_t kQ8StagedLds = static_cast<size_t>(kMaxSplit) * 256 * sizeof(float) + static_cast<size_t>(kQ8XPieces) * 16 +
+                                16 * static_cast<size_t>(kQ8WRowStride);
+
+template <typename XT>
+__global__ void __launch_bounds__(64 * kMaxSplit)
+    gemm_q8_0_staged_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y, int n_out,
+                            int n_steps, size_t row_bytes, int n_rows, int n_split) {
+    extern __shared__ __attribute__((aligned(16))) float red[];  // [kMaxSplit][256], then X pieces, then W rows
+    half8_t *xs = reinterpret_cast<half8_t *>(red + kMaxSplit * 256);
+    uint8_t *ws = reinterpret_cast<uint8_t *>(xs + kQ8XPieces);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    float4_t acc = {0, 0, 0, 0};
+    for (int c0 = 0; c0 < n_steps; c0 += kQ8ChunkSteps) {
+        const int cs = min(kQ8ChunkSteps, n_steps - c0);  // steps of this chunk (a multiple of 8)
+        if (c0) __syncthreads();                          // the previous chunk's fragments have been read
+        // weights: cs * 34 / 16 pieces per row
+        const int wp_row = cs * DFL_Q8_0_BYTES / 16;
+        for (int p = tid; p < 16 * wp_row; p += blockDim.x) {
+            const int r = p / wp_row, c = p - r * wp_row;
+            const int row = min(n0 + r, n_out - 1);
+            *reinterpret_cast<u32x4_t *>(ws + r * kQ8WRowStride + 16 * c) = *reinterpret_cast<const u32x4_t *>(
+                w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(c0) * DFL_Q8_0_BYTES + 16 * c);
+        }
+        // activations: 4 cs pieces of eight per row; rows past n_rows repeat the last one
+        const int xp_row = 4 * cs;
+        for (int p = tid; p < 16 * xp_row; p += blockDim.x) {
+            const int r = p / xp_row, c = p - r * xp_row;
+            const XT *src = x + static_cast<size_t>(min(r, n_rows - 1)) * (static_cast<size_t>(n_steps) * 32) +
+                            static_cast<size_t>(c0) * 32 + 8 * c;
+            xs[(c >> 2) * 68 + (c & 3) * 17 + r] = convert_rawx8(load_rawx8(src));
+        }
+        __syncthreads();
+        const int s0 = cs * wave / n_split, s1 = cs * (wave + 1) / n_split;
+        const uint8_t *rowp = ws + n * kQ8WRowStride;
+        for (int s = s0; s < s1; s++) {
+            const uint8_t *blk = rowp + s * DFL_Q8_0_BYTES;  // 2-byte aligned
+            const uint16_t *q16 = reinterpret_cast<const uint16_t *>(blk + 2 + 8 * g);
+            Raw8<DFLASH_TYPE_Q8_0> r;
+            r.d = static_cast<float>(__builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t *>(blk)));
+            r.q = static_cast<uint64_t>(q16[0]) | (static_cast<uint64_t>(q16[1]) << 16) | (static_cast<uint64_t>(q16[2]) << 32) |
+                  (static_cast<uint64_t>(q16[3]) << 48);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xs[s * 68 + g * 17 + n], convert_raw8<DFLASH_TYPE_Q8_0>(r), acc, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) red[wave * 256 + (4 * g + i) * 16 + n] = acc[i];
+    __syncthreads();
+    for (int e = tid; e < 256; e += blockDim.x) {
+        const int m = e >> 4, nn = e & 15;
+        if (m < n_rows && n0 + nn < n_out) {
+            float sum = 0.0f;
+            for (int wv = 0; wv < n_split; wv++) sum += red[wv * 256 + e];
             y[static_cast<size_t>(m) * n_out + n0 + nn] = sum;
         }
     }
@@ -1053,30 +1182,6 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
 // runs with unaligned vector memory access enabled and the compiler emits them as single loads.
 // Activations are read from the caller's matrix and rounded to f16 on the fly (all tiles read the
 // same rows: L2 hits).  Waves of a workgroup split K and add their tiles up in LDS in wave order.
-__device__ __forceinline__ uint64_t load_u64_unaligned(const uint8_t *p) {
-    uint64_t v;
-    __builtin_memcpy(&v, p, 8);
-    return v;
-}
-
-template <>
-__device__ __forceinline__ half8_t load_x8<float>(const float *p, bool live) {
-    half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (live) {
-        const float4_t a = *reinterpret_cast<const float4_t *>(p), b = *reinterpret_cast<const float4_t *>(p + 4);
-        r = half8_t{static_cast<_Float16>(a[0]), static_cast<_Float16>(a[1]), static_cast<_Float16>(a[2]),
-                    static_cast<_Float16>(a[3]), static_cast<_Float16>(b[0]), static_cast<_Float16>(b[1]),
-                    static_cast<_Float16>(b[2]), static_cast<_Float16>(b[3])};
-    }
-    return r;
-}
-template <>
-__device__ __forceinline__ half8_t load_x8<_Float16>(const _Float16 *p, bool live) {
-    half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (live) r = *reinterpret_cast<const half8_t *>(p);
-    return r;
-}
-
 // Up to three matrices that share the activations (the q, k and v projections of a layer) in one
 // launch: workgroup b serves tile b - tile_begin[m] of the matrix m whose tile range holds b.
 struct Q6KSet {
@@ -1105,8 +1210,9 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
     const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
     const int n_half = 2 * nb;
     const int h0 = n_half * wave / n_split, h1 = n_half * (wave + 1) / n_split;
-    const bool x_live = n < n_rows;  // lane (m = n, g) of the A operand: activation row n
-    const XT *xrow = x + static_cast<size_t>(x_live ? n : 0) * (static_cast<size_t>(nb) * DFL_QK_K) + 8 * g;
+    // lane (m = n, g) of the A operand: activation row n (lanes past n_rows repeat the last row: a
+    // row of A only reaches the same row of the product, which is never stored for them)
+    const XT *xrow = x + static_cast<size_t>(n < n_rows ? n : n_rows - 1) * (static_cast<size_t>(nb) * DFL_QK_K) + 8 * g;
     float4_t acc = {0, 0, 0, 0};
     for (int hb = h0; hb < h1; hb++) {
         const uint8_t *blk = rowp + static_cast<size_t>(hb >> 1) * DFL_Q6_K_BYTES;
@@ -1133,8 +1239,7 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
                 b[i] = static_cast<_Float16>(__builtin_fmaf(static_cast<float>((q0 >> (8 * i)) & 0xffu), ds, off));
                 b[4 + i] = static_cast<_Float16>(__builtin_fmaf(static_cast<float>((q1 >> (8 * i)) & 0xffu), ds, off));
             }
-            const half8_t a = load_x8<XT>(xk + 32 * kq, x_live);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(convert_rawx8(load_rawx8(xk + 32 * kq)), b, acc, 0, 0, 0);
         }
     }
 #pragma unroll
@@ -1430,7 +1535,26 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
         size_t lds = static_cast<size_t>(split) * 256 * sizeof(float);
         const uint8_t *wb = static_cast<const uint8_t *>(w);
         dfl_timed timer(ctx, st, DFL_T_GEMM);
-        if (x_type == DFLASH_TYPE_F32)
+        if (n_in % 256 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+            env_int("DFLASH_Q8_STAGED", 1)) {
+            static bool attr = false;
+            if (!attr) {
+                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_staged_kernel<float>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kQ8StagedLds)));
+                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_staged_kernel<_Float16>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kQ8StagedLds)));
+                attr = true;
+            }
+            // the waves of a workgroup split a 64-step chunk
+            if (split > kQ8ChunkSteps) split = kQ8ChunkSteps;
+            if (x_type == DFLASH_TYPE_F32)
+                gemm_q8_0_staged_kernel<float><<<tiles, 64 * split, kQ8StagedLds, st>>>(
+                    wb, static_cast<const float *>(x), y, static_cast<int>(n_out), static_cast<int>(n_steps), row_bytes, n_rows, split);
+            else
+                gemm_q8_0_staged_kernel<_Float16><<<tiles, 64 * split, kQ8StagedLds, st>>>(
+                    wb, static_cast<const _Float16 *>(x), y, static_cast<int>(n_out), static_cast<int>(n_steps), row_bytes, n_rows,
+                    split);
+        } else if (x_type == DFLASH_TYPE_F32)
             gemm_generic_kernel<DFLASH_TYPE_Q8_0, float><<<tiles, 64 * split, lds, st>>>(
                 wb, static_cast<const float *>(x), y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
         else

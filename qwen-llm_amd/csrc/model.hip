@@ -98,21 +98,26 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
 // With vt_dst, n_kv more workgroups per row scatter the row's V heads, as f16, into column
 // pos[row] of the transposed cache [kv head][dim][capacity].
 __global__ void __launch_bounds__(64)
-    qk_norm_rope_kernel(float *__restrict__ q, float *__restrict__ k, const float *__restrict__ q_w,
-                        const float *__restrict__ k_w, _Float16 *__restrict__ k_dst, const int32_t *__restrict__ pos,
-                        int n_q, int n_kv, int hd, float eps, float theta, const float *__restrict__ v_src,
-                        _Float16 *__restrict__ vt_dst, int64_t capacity) {
+    qk_norm_rope_kernel(const float *q_in, int64_t q_ld, const float *k_in, int64_t k_ld, float *q_out, float *k_out,
+                        const float *__restrict__ q_w, const float *__restrict__ k_w, _Float16 *__restrict__ k_dst,
+                        const int32_t *__restrict__ pos, int n_q, int n_kv, int hd, float eps, float theta,
+                        const float *__restrict__ v_src, int64_t v_ld, _Float16 *__restrict__ vt_dst, int64_t capacity) {
     const int row = blockIdx.y, head = blockIdx.x, lane = threadIdx.x;
     if (head >= n_q + n_kv) {
         const int vh = head - n_q - n_kv;
-        const float *src = v_src + (static_cast<size_t>(row) * n_kv + vh) * hd;
+        const float *src = v_src + static_cast<size_t>(row) * v_ld + static_cast<size_t>(vh) * hd;
         _Float16 *dst = vt_dst + static_cast<size_t>(vh) * hd * capacity + pos[row];
         for (int i = lane; i < hd; i += 64) dst[static_cast<size_t>(i) * capacity] = static_cast<_Float16>(src[i]);
         return;
     }
     const bool is_q = head < n_q;
-    float *v = is_q ? q + (static_cast<size_t>(row) * n_q + head) * hd
-                    : k + (static_cast<size_t>(row) * n_kv + (head - n_q)) * hd;
+    // input rows may be slices of a wider matrix (row strides q_ld, k_ld); outputs are dense.  In
+    // place (q_out == q_in with a dense q_ld) is fine: a lane reads its two elements before it
+    // writes them.
+    const float *v = is_q ? q_in + static_cast<size_t>(row) * q_ld + static_cast<size_t>(head) * hd
+                          : k_in + static_cast<size_t>(row) * k_ld + static_cast<size_t>(head - n_q) * hd;
+    float *o = is_q ? q_out + (static_cast<size_t>(row) * n_q + head) * hd
+                    : (k_dst ? nullptr : k_out + (static_cast<size_t>(row) * n_kv + (head - n_q)) * hd);
     const float *w = is_q ? q_w : k_w;
     const int half = hd / 2;
     float s = 0.0f;
@@ -130,9 +135,9 @@ __global__ void __launch_bounds__(64)
         float sn, cs;
         sincosf(freq, &sn, &cs);
         const float ra = a * cs - b * sn, rb = a * sn + b * cs;
-        if (is_q || !k_dst) {
-            v[i] = ra;
-            v[i + half] = rb;
+        if (o) {
+            o[i] = ra;
+            o[i + half] = rb;
         } else {
             _Float16 *dst = k_dst + (static_cast<size_t>(pos[row]) * n_kv + (head - n_q)) * hd;
             dst[i] = static_cast<_Float16>(ra);
@@ -147,6 +152,18 @@ __global__ void silu_mul_kernel(float *__restrict__ g, const float *__restrict__
     if (i < n) {
         float x = g[i];
         g[i] = x / (1.0f + expf(-x)) * u[i];
+    }
+}
+
+// The same over two column slices of one wider matrix (gate and up projected in one GEMM):
+// out[row][i] = silu(g[row * ld + i]) * u[row * ld + i], out dense [rows][n].
+__global__ void silu_mul_ld_kernel(const float *__restrict__ g, const float *__restrict__ u, int64_t ld,
+                                   float *__restrict__ out, int n) {
+    const int row = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float x = g[static_cast<size_t>(row) * ld + i];
+        out[static_cast<size_t>(row) * n + i] = x / (1.0f + expf(-x)) * u[static_cast<size_t>(row) * ld + i];
     }
 }
 
@@ -202,13 +219,16 @@ __global__ void __launch_bounds__(64)
 }
 
 // K/V rows f32 [m][kv_dim] -> f16 caches: K natural at row base + r, V transposed at column base + r
-__global__ void kv_to_f16_kernel(const float *__restrict__ k, const float *__restrict__ v, _Float16 *__restrict__ k16,
-                                 _Float16 *__restrict__ vt16, int kv_dim, int64_t cap16, int64_t base) {
+__global__ void kv_to_f16_kernel(const float *__restrict__ k, const float *__restrict__ v, int64_t v_ld,
+                                 _Float16 *__restrict__ k16, _Float16 *__restrict__ vt16, int kv_dim, int64_t cap16,
+                                 int64_t base, float *__restrict__ v_copy) {
     const int row = blockIdx.y;
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= kv_dim) return;
+    const float vv = v[static_cast<size_t>(row) * v_ld + e];
     k16[(base + row) * kv_dim + e] = static_cast<_Float16>(k[static_cast<size_t>(row) * kv_dim + e]);
-    vt16[static_cast<size_t>(e) * cap16 + base + row] = static_cast<_Float16>(v[static_cast<size_t>(row) * kv_dim + e]);
+    vt16[static_cast<size_t>(e) * cap16 + base + row] = static_cast<_Float16>(vv);
+    if (v_copy) v_copy[static_cast<size_t>(row) * kv_dim + e] = vv;  // dense f32 copy of a V slice
 }
 
 template <typename T>
@@ -223,9 +243,22 @@ int32_t gemm(dflash_ctx *ctx, const dflash_qtensor &w, const float *x, float *y,
     return dflash_gemm_fewrow(ctx, w.type, w.data, x, DFLASH_TYPE_F32, y, n_in, n_out, n, st);
 }
 
-// The q, k and v projections of a layer: one launch when all three are Q6_K, else three.
+// True if b's rows follow a's rows_a rows directly in memory and both have the same type: the two
+// are then one matrix of more rows, and one GEMM serves both (its output rows hold a's columns, then
+// b's).  Loaders that place a layer's wq, wk, wv (and gate, up) back to back get this for free.
+bool adjacent(const dflash_qtensor &a, int64_t rows_a, const dflash_qtensor &b, int64_t n_in) {
+    const size_t rb = dflash_row_bytes(a.type, n_in);
+    return a.type == b.type && rb != 0 &&
+           static_cast<const uint8_t *>(b.data) == static_cast<const uint8_t *>(a.data) + static_cast<size_t>(rows_a) * rb;
+}
+
+// The q, k and v projections of a layer.  Returns in *packed whether they went out as one GEMM into
+// pk[n][q_dim + 2 kv_dim] (adjacent weights) or as separate ones into q, k, v.
 int32_t gemm_qkv(dflash_ctx *ctx, const dflash_qtensor &wq, const dflash_qtensor &wk, const dflash_qtensor &wv, const float *x,
-                 float *q, float *k, float *v, int64_t n_in, int64_t q_dim, int64_t kv_dim, int n, hipStream_t st) {
+                 float *q, float *k, float *v, float *pk, bool allow_packed, bool *packed, int64_t n_in, int64_t q_dim,
+                 int64_t kv_dim, int n, hipStream_t st) {
+    *packed = allow_packed && pk && adjacent(wq, q_dim, wk, n_in) && adjacent(wk, kv_dim, wv, n_in);
+    if (*packed) return gemm(ctx, wq, x, pk, n_in, q_dim + 2 * kv_dim, n, st);
     if (wq.type == DFLASH_TYPE_Q6_K && wk.type == DFLASH_TYPE_Q6_K && wv.type == DFLASH_TYPE_Q6_K && n_in % DFL_QK_K == 0) {
         const void *w[3] = {wq.data, wk.data, wv.data};
         float *y[3] = {q, k, v};
@@ -236,6 +269,21 @@ int32_t gemm_qkv(dflash_ctx *ctx, const dflash_qtensor &wq, const dflash_qtensor
     if ((rc = gemm(ctx, wq, x, q, n_in, q_dim, n, st))) return rc;
     if ((rc = gemm(ctx, wk, x, k, n_in, kv_dim, n, st))) return rc;
     return gemm(ctx, wv, x, v, n_in, kv_dim, n, st);
+}
+
+// Dense SwiGLU input: g = silu(x Wg^T) * (x Wu^T), one GEMM when gate and up are adjacent.
+int32_t gemm_gate_up(dflash_ctx *ctx, const dflash_qtensor &gate, const dflash_qtensor &up, const float *x, float *g, float *u,
+                     float *pk, int64_t n_in, int64_t ffn, int n, hipStream_t st) {
+    int32_t rc;
+    if (pk && adjacent(gate, ffn, up, n_in)) {
+        if ((rc = gemm(ctx, gate, x, pk, n_in, 2 * ffn, n, st))) return rc;
+        silu_mul_ld_kernel<<<dim3(blocks_for(static_cast<size_t>(ffn)), n), 256, 0, st>>>(pk, pk + ffn, 2 * ffn, g, static_cast<int>(ffn));
+        return DFLASH_OK;
+    }
+    if ((rc = gemm(ctx, gate, x, g, n_in, ffn, n, st))) return rc;
+    if ((rc = gemm(ctx, up, x, u, n_in, ffn, n, st))) return rc;
+    silu_mul_kernel<<<blocks_for(static_cast<size_t>(n) * ffn), 256, 0, st>>>(g, u, static_cast<size_t>(n) * ffn);
+    return DFLASH_OK;
 }
 
 int32_t embed_rows(dflash_ctx *ctx, const dflash_qtensor &t, const int32_t *ids_dev, int n, int hidden, float *out,
@@ -256,6 +304,7 @@ struct dflash_session {
     _Float16 *k_cache = nullptr, *vt_cache = nullptr;
     float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
     float *g = nullptr, *u = nullptr, *logits = nullptr, *gap = nullptr;
+    float *pk = nullptr;  // [16][max(q_dim + 2 kv_dim, 2 ffn)]: output of a fused q/k/v or gate/up GEMM
     float *hidden = nullptr;  // [16][n_taps][hidden] capture slots of the speculative step
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
     dfl_moe_scratch moe;
@@ -284,6 +333,7 @@ struct dflash_draft_session {
     int32_t *pos_ctx = nullptr;                // [cap]
     float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
     float *g = nullptr, *u = nullptr, *logits = nullptr, *tmp = nullptr;
+    float *pk = nullptr;  // [16][max(q_dim + 2 kv_dim, 2 ffn)]: output of a fused q/k/v or gate/up GEMM
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
 };
 
@@ -308,6 +358,7 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
               dev_alloc(&s->x, 16 * cfg->hidden) && dev_alloc(&s->cur, 16 * cfg->hidden) && dev_alloc(&s->q, 16 * q_dim) &&
               dev_alloc(&s->k, 16 * kv_dim) && dev_alloc(&s->v, 16 * kv_dim) && dev_alloc(&s->attn, 16 * q_dim) &&
               dev_alloc(&s->mix, 16 * cfg->hidden) && dev_alloc(&s->g, 16 * f) && dev_alloc(&s->u, 16 * f) &&
+              dev_alloc(&s->pk, 16 * std::max(q_dim + 2 * kv_dim, 2 * f)) &&
               dev_alloc(&s->logits, 16 * static_cast<size_t>(cfg->vocab)) && dev_alloc(&s->gap, 16) &&
               dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) && dev_alloc(&s->argmax, 16) &&
               dev_alloc(&s->hidden, 16 * static_cast<size_t>(std::max(n_taps, 1)) * cfg->hidden);
@@ -340,7 +391,7 @@ void dflash_session_destroy(dflash_session *s) {
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
                     s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax, s->hidden,
                     s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared,
-                    s->moe.gate_out, s->moe.up_out, s->moe.ids, s->moe.n_distinct, s->moe.slot_of};
+                    s->moe.gate_out, s->moe.up_out, s->moe.ids, s->moe.n_distinct, s->moe.slot_of, s->pk};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;
@@ -383,9 +434,13 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
         const dflash_layer &L = model->layers[il];
         _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
         rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
-        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, H, q_dim, kv_dim, n, st))) return rc;
-        qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, kc, s->pos, c.n_q, c.n_kv,
-                                                                      hd, c.eps, c.rope_theta, s->v, vtc, s->capacity);
+        bool packed;
+        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, true, &packed, H, q_dim, kv_dim, n, st))) return rc;
+        const int64_t tot = q_dim + 2 * kv_dim;
+        qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(
+            packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
+            L.k_norm, kc, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, packed ? s->pk + q_dim + kv_dim : s->v,
+            packed ? tot : kv_dim, vtc, s->capacity);
         // the context length is read from pos[0] on the device: the same launches serve every position
         if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity, scale,
                                  s->attn, st, 0, 0, s->pos)))
@@ -395,9 +450,7 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
         if (c.n_expert > 0) {
             if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, st))) return rc;
         } else {
-            if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, n, st))) return rc;
-            if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, n, st))) return rc;
-            silu_mul_kernel<<<blocks_for(static_cast<size_t>(n) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(n) * c.ffn);
+            if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, n, st))) return rc;
             if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
             add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
         }
@@ -529,6 +582,7 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
               dev_alloc(&s->q, 16 * q_dim) && dev_alloc(&s->k, 16 * kv_dim) && dev_alloc(&s->v, 16 * kv_dim) &&
               dev_alloc(&s->attn, 16 * q_dim) && dev_alloc(&s->mix, 16 * H) && dev_alloc(&s->g, 16 * static_cast<size_t>(cfg->ffn)) &&
               dev_alloc(&s->u, 16 * static_cast<size_t>(cfg->ffn)) && dev_alloc(&s->logits, 16 * static_cast<size_t>(vocab)) &&
+              dev_alloc(&s->pk, 16 * std::max(q_dim + 2 * kv_dim, 2 * static_cast<size_t>(cfg->ffn))) &&
               dev_alloc(&s->tmp, 16 * std::max(H, kv_dim)) && dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) &&
               dev_alloc(&s->argmax, 16);
     if (!ok) {
@@ -542,7 +596,7 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
 void dflash_draft_session_destroy(dflash_draft_session *s) {
     if (!s) return;
     void *ptrs[] = {s->ctx_raw, s->ctx_h, s->k_ctx, s->v_ctx, s->k16, s->vt16, s->pos_ctx, s->x, s->cur, s->q, s->k, s->v,
-                    s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax};
+                    s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax, s->pk};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;
@@ -618,22 +672,36 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
         // context K/V for the delta only, normed and rotated at the columns' own positions
         for (int64_t c0 = s->kv_ready; c0 < s->ctx_len; c0 += 16) {
             const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
-            if ((rc = gemm(ctx, L.wk, s->ctx_h + c0 * H, kc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
-            if ((rc = gemm(ctx, L.wv, s->ctx_h + c0 * H, vc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
-            qk_norm_rope_kernel<<<dim3(c.n_kv, m), 64, 0, st>>>(nullptr, kc + c0 * kv_dim, nullptr, L.k_norm, nullptr,
-                                                               s->pos_ctx + c0, 0, c.n_kv, hd, c.eps, c.rope_theta, nullptr, nullptr, 0);
+            // wk and wv adjacent: one GEMM into pk[m][2 kv_dim]; K is rotated out of it into the context
+            // cache, V is copied out of it by the mirror kernel
+            const bool kv_packed = fast && adjacent(L.wk, kv_dim, L.wv, H);
+            if (kv_packed) {
+                if ((rc = gemm(ctx, L.wk, s->ctx_h + c0 * H, s->pk, H, 2 * kv_dim, m, st))) return rc;
+            } else {
+                if ((rc = gemm(ctx, L.wk, s->ctx_h + c0 * H, kc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
+                if ((rc = gemm(ctx, L.wv, s->ctx_h + c0 * H, vc + c0 * kv_dim, H, kv_dim, m, st))) return rc;
+            }
+            qk_norm_rope_kernel<<<dim3(c.n_kv, m), 64, 0, st>>>(nullptr, 0, kv_packed ? s->pk : kc + c0 * kv_dim,
+                                                               kv_packed ? 2 * kv_dim : kv_dim, nullptr, kc + c0 * kv_dim, nullptr,
+                                                               L.k_norm, nullptr, s->pos_ctx + c0, 0, c.n_kv, hd, c.eps,
+                                                               c.rope_theta, nullptr, 0, nullptr, 0);
             if (fast)
-                kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), m), 256, 0, st>>>(kc + c0 * kv_dim, vc + c0 * kv_dim, k16, vt16,
-                                                                              static_cast<int>(kv_dim), s->cap16, c0);
+                kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), m), 256, 0, st>>>(
+                    kc + c0 * kv_dim, kv_packed ? s->pk + kv_dim : vc + c0 * kv_dim, kv_packed ? 2 * kv_dim : kv_dim, k16, vt16,
+                    static_cast<int>(kv_dim), s->cap16, c0, kv_packed ? vc + c0 * kv_dim : nullptr);
         }
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
-        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, H, q_dim, kv_dim, N, st))) return rc;
-        qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, s->k, L.q_norm, L.k_norm, nullptr, s->pos, c.n_q,
-                                                                  c.n_kv, hd, c.eps, c.rope_theta, nullptr, nullptr, 0);
+        bool packed;  // only on the fast path: the general attention kernel reads V dense
+        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st))) return rc;
+        const int64_t tot = q_dim + 2 * kv_dim;
+        qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(
+            packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
+            L.k_norm, nullptr, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, nullptr, 0, nullptr, 0);
         if (fast) {
             // the block's own K/V go behind the context in the f16 mirror; one MFMA pass over both
-            kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), N), 256, 0, st>>>(s->k, s->v, k16, vt16, static_cast<int>(kv_dim),
-                                                                          s->cap16, s->ctx_len);
+            kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), N), 256, 0, st>>>(s->k, packed ? s->pk + q_dim + kv_dim : s->v,
+                                                                          packed ? tot : kv_dim, k16, vt16, static_cast<int>(kv_dim),
+                                                                          s->cap16, s->ctx_len, nullptr);
             if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, k16, vt16, 1, s->ctx_len, N, c.n_q, c.n_kv, hd, s->cap16,
                                      1.0f / sqrtf(static_cast<float>(hd)), s->attn, st, c.causal ? 0 : 1,
                                      L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, nullptr)))
@@ -645,9 +713,7 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
         }
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st))) return rc;
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps);  // x += mix first
-        if ((rc = gemm(ctx, L.gate, s->cur, s->g, H, c.ffn, N, st))) return rc;
-        if ((rc = gemm(ctx, L.up, s->cur, s->u, H, c.ffn, N, st))) return rc;
-        silu_mul_kernel<<<blocks_for(static_cast<size_t>(N) * c.ffn), 256, 0, st>>>(s->g, s->u, static_cast<size_t>(N) * c.ffn);
+        if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, N, st))) return rc;
         if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st))) return rc;
         add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
     }

@@ -65,12 +65,53 @@ __global__ void __launch_bounds__(1024)
     const bool live = row < n_rows;
     float *pr = probs + row * n_expert;
     if (live) {
+        // Everything this row reads from memory is requested before anything waits for it: its first
+        // 256 router logits and (2048 elements at a time) the operands of the shared-expert gate
+        // sigmoid(x . w); one memory latency instead of one per phase.
         const float *lg = logits + static_cast<size_t>(row) * n_expert;
+        float lgv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
+        const float *xr = x + static_cast<size_t>(row) * hidden;
+        float dot = 0.0f;
+        if (hidden % 4 == 0) {
+            for (int base = 0; base < hidden; base += 2048) {
+                f4 xa[8], gb[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int i = base + 4 * lane + 256 * j;
+                    xa[j] = gb[j] = f4{0, 0, 0, 0};
+                    if (i < hidden) {
+                        xa[j] = *reinterpret_cast<const f4 *>(xr + i);
+                        gb[j] = *reinterpret_cast<const f4 *>(shexp_gate + i);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (base + 4 * lane + 256 * j < hidden)
+                        dot += (xa[j][0] * gb[j][0] + xa[j][1] * gb[j][1]) + (xa[j][2] * gb[j][2] + xa[j][3] * gb[j][3]);
+            }
+        } else {
+            for (int i = lane; i < hidden; i += 64) dot += xr[i] * shexp_gate[i];
+        }
+        for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
+
         float mx = -INFINITY;
-        for (int e = lane; e < n_expert; e += 64) mx = fmaxf(mx, lg[e]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) mx = fmaxf(mx, lgv[j]);
+        for (int e = lane + 256; e < n_expert; e += 64) mx = fmaxf(mx, lg[e]);
         for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
         float sum = 0.0f;
-        for (int e = lane; e < n_expert; e += 64) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (lane + 64 * j < n_expert) {
+                const float ex = expf(lgv[j] - mx);
+                pr[lane + 64 * j] = ex;
+                sum += ex;
+            }
+        }
+        for (int e = lane + 256; e < n_expert; e += 64) {
             const float ex = expf(lg[e] - mx);
             pr[e] = ex;
             sum += ex;
@@ -106,19 +147,6 @@ __global__ void __launch_bounds__(1024)
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
         }
-        // shared-expert gate: sigmoid(x . w)
-        const float *xr = x + static_cast<size_t>(row) * hidden;
-        float dot = 0.0f;
-        if (hidden % 4 == 0) {
-            for (int i = 4 * lane; i < hidden; i += 256) {
-                const f4 a = *reinterpret_cast<const f4 *>(xr + i), b = *reinterpret_cast<const f4 *>(shexp_gate + i);
-                dot += (a[0] * b[0] + a[1] * b[1]) + (a[2] * b[2] + a[3] * b[3]);
-            }
-        } else {
-            for (int i = lane; i < hidden; i += 64) dot += xr[i] * shexp_gate[i];
-        }
-        for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-        if (lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
     }
     __syncthreads();
     if (live && lane == 0) {

@@ -275,11 +275,33 @@ class _Uploader:
         self.keep.append(t)
         return QTensorC(int(qtype), 0, t.data_ptr())
 
+    def q_adjacent(self, pairs):
+        """Uploads matrices of one type and one row length back to back in a single allocation (rows of the
+        first, then the second, ...): the library then runs a layer's wq/wk/wv (or gate/up) as ONE GEMM.
+        Falls back to separate uploads when the types differ."""
+        if any(p is None for p in pairs) or len({int(p[0]) for p in pairs}) != 1:
+            return [self.q(p) for p in pairs]
+        torch = self.torch
+        flats = []
+        for _, blocks in pairs:
+            if isinstance(blocks, torch.Tensor):
+                flats.append(blocks.to(self.device).contiguous().view(torch.uint8).reshape(-1))
+            else:
+                flats.append(torch.from_numpy(np.ascontiguousarray(blocks).view(np.uint8).reshape(-1)).to(self.device))
+        whole = torch.cat(flats)
+        self.keep.append(whole)
+        out, off = [], 0
+        for (qtype, _), f in zip(pairs, flats):
+            out.append(QTensorC(int(qtype), 0, whole.data_ptr() + off))
+            off += f.numel()
+        return out
+
 
 class TargetModel:
     """Device copy of a weight dictionary plus the ``dflash_model`` descriptor."""
 
-    def __init__(self, ctx: Context, cfg: ModelConfig, weights: dict):
+    def __init__(self, ctx: Context, cfg: ModelConfig, weights: dict, adjacent: bool = True):
+        """``adjacent``: place each layer's wq/wk/wv and gate/up back to back in device memory (one GEMM each)."""
         self.ctx, self.cfg = ctx, cfg
         up = _Uploader(f"cuda:{ctx.device}")
         self._up = up
@@ -288,8 +310,14 @@ class TargetModel:
             L = self._layers[il]
             for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
                 setattr(L, k, up.f32(Lw[k]))
+            grouped = ()
+            if adjacent:
+                grouped = ("wq", "wk", "wv", "gate", "up")
+                L.wq, L.wk, L.wv = up.q_adjacent([Lw.get("wq"), Lw.get("wk"), Lw.get("wv")])
+                L.gate, L.up = up.q_adjacent([Lw.get("gate"), Lw.get("up")])
             for k in ("wq", "wk", "wv", "wo", "gate", "up", "down", "router", "gate_exps", "up_exps", "down_exps"):
-                setattr(L, k, up.q(Lw.get(k)))
+                if k not in grouped:
+                    setattr(L, k, up.q(Lw.get(k)))
             L.shexp_gate = up.f32(Lw["shexp_gate"]) if "shexp_gate" in Lw else None
         self.c = ModelC(ModelCfgC(**cfg.as_dict()), self._layers, up.q(weights["token_embd"]), up.q(weights["output"]),
                         up.f32(weights["output_norm"]))
@@ -361,7 +389,7 @@ class Session:
 
 
 class DraftHead:
-    def __init__(self, ctx: Context, cfg: DraftConfig, weights: dict):
+    def __init__(self, ctx: Context, cfg: DraftConfig, weights: dict, adjacent: bool = True):
         self.ctx, self.cfg = ctx, cfg
         up = _Uploader(f"cuda:{ctx.device}")
         self._up = up
@@ -370,8 +398,14 @@ class DraftHead:
             L = self._layers[il]
             for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
                 setattr(L, k, up.f32(Lw[k]))
+            grouped = ()
+            if adjacent:
+                grouped = ("wq", "wk", "wv", "gate", "up")
+                L.wq, L.wk, L.wv = up.q_adjacent([Lw["wq"], Lw["wk"], Lw["wv"]])
+                L.gate, L.up = up.q_adjacent([Lw["gate"], Lw["up"]])
             for k in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
-                setattr(L, k, up.q(Lw[k]))
+                if k not in grouped:
+                    setattr(L, k, up.q(Lw[k]))
             L.is_swa = int(Lw.get("is_swa", 0))
         self.c = DraftHeadC(DraftCfgC(**cfg.as_dict()), self._layers, up.q(weights["fc"]), up.f32(weights["hidden_norm"]),
                             up.f32(weights["output_norm"]))

@@ -170,6 +170,55 @@ def test_draft_block_matches_oracle(ctx, oracle, target, causal, swa):
     sess.close()
 
 
+def test_separate_and_adjacent_weight_layouts_agree(ctx, oracle, target):
+    """A layer's wq/wk/wv and gate/up uploaded back to back run as one GEMM each (the default of the
+    mirror); uploaded separately they run as three and two.  Both layouts must match the oracle, and each
+    other to GEMM tolerance (the split-K boundaries differ, so not bit for bit)."""
+    model_adj, (omodel, _keep) = target
+    w = dfl.synth_target_weights(C1, seed=11)
+    model_sep = dfl.TargetModel(ctx, C1, w, adjacent=False)
+    L0a, L0s = model_adj.c.layers[0], model_sep.c.layers[0]
+    rb = 1024 // 256 * 144
+    assert L0a.wk.data == L0a.wq.data + 16 * 128 * rb and L0a.wv.data == L0a.wk.data + 8 * 128 * rb
+    assert L0a.up.data == L0a.gate.data + 3072 * rb
+    assert L0s.wk.data != L0s.wq.data + 16 * 128 * rb or L0s.wv.data != L0s.wk.data + 8 * 128 * rb
+    dw = dfl.synth_draft_weights(D1, seed=3)
+    ohead, _k2 = oracle.build_draft_head(D1.as_dict(), dw)
+    rng = np.random.default_rng(23)
+    cap = 64
+    toks = rng.integers(0, C1.vocab, 32).tolist()
+    carry = int(rng.integers(0, C1.vocab))
+    outs = {}
+    for name, model, adjacent in (("adjacent", model_adj, True), ("separate", model_sep, False)):
+        head = dfl.DraftHead(ctx, D1, dw, adjacent=adjacent)
+        sess = dfl.Session(ctx, model, cap, TAPS)
+        dsess = dfl.DraftSession(ctx, head, model, cap)
+        logits, hidden = [], []
+        for s in range(0, 32, 16):
+            out = sess.encode_packed_verify_layer_major(toks[s:s + 16], s, want_logits=True)
+            dsess.append_target_ctx_columns(out.hidden_capture, list(range(s, s + 16)))
+            logits.append(out.logits.cpu().numpy())
+            hidden.append(out.hidden_capture.cpu().numpy())
+        _, dl, _ = dsess.draft_block(carry, C1.vocab - 1, 32, want_logits=True)
+        outs[name] = (np.concatenate(logits), np.concatenate(hidden), dl.cpu().numpy())
+        dsess.close()
+        sess.close()
+    ostate = oracle.TargetState(C1.as_dict(), cap)
+    lo, ho = [], []
+    for s in range(0, 32, 16):
+        l, h = oracle.target_verify(omodel, ostate, toks[s:s + 16], s, TAPS)
+        lo.append(l)
+        ho.append(h)
+    lo, ho = np.concatenate(lo), np.concatenate(ho)
+    want_d = oracle.dflash_draft(omodel, ohead, [carry] + [C1.vocab - 1] * 15, ho.reshape(32, -1), list(range(32)), 32)
+    for name, (lg, hid, dl) in outs.items():
+        close(lg, lo, f"{name}: verify logits")
+        close(hid, ho, f"{name}: hidden")
+        close(dl, want_d, f"{name}: draft logits")
+    close(outs["adjacent"][0], outs["separate"][0], "adjacent vs separate verify logits")
+    close(outs["adjacent"][2], outs["separate"][2], "adjacent vs separate draft logits")
+
+
 MOE_CASES = {
     # hidden 512: 16 sub-blocks per row (half-wave rows); hidden 2048 / F_exp 768: the end-to-end shape's widths
     "small": dfl.ModelConfig(n_layers=2, hidden=512, n_q=8, n_kv=2, head_dim=64, ffn=0, vocab=4096, n_expert=16,
