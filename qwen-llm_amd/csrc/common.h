@@ -96,9 +96,13 @@ struct dfl_moe_scratch {
     float *g = nullptr, *u = nullptr;  // [16][ffn_shared]
 };
 
-// x_resid[n][hidden] += moe_ffn(cur[n][hidden]) for one layer; enqueue only.
+// x_resid[n][hidden] += moe_ffn(cur[n][hidden]) for one layer; enqueue only.  gate_done: scratch.sg
+// already holds sigmoid(cur . shexp_gate) per row (the norm kernel that wrote cur computed it).
+// next_norm_w / next_cur / next_done (all or none): the RMSNorm that reads x_resid next may be done
+// in the same pass, next_cur = rms_norm(x_resid) * next_norm_w; *next_done says whether it was.
 int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, const float *cur, int n,
-                    const dfl_moe_scratch &scratch, float *x_resid, hipStream_t stream);
+                    const dfl_moe_scratch &scratch, float *x_resid, bool gate_done, const float *next_norm_w,
+                    float *next_cur, bool *next_done, hipStream_t stream);
 
 // dflash_attn_verify_block with the drafter's masks: full_block != 0 lets every row see the whole
 // block (non-causal), window > 0 keeps only keys with |distance| < window.  ctx_len_dev != null:

@@ -41,10 +41,13 @@ __device__ float block_sum(float v, float *sh) {
 // kernel_rms_norm_batched_f32 (attn.metal:35-69), optionally preceded by the residual add that
 // feeds it (kernel_add, elementwise.metal): x += add (add may be null), then
 // y = x * rsqrt(mean(x^2) + eps) * w.  One row per workgroup; a row of up to 4096 values (n a
-// multiple of 4) is read once and stays in registers between the two passes.
+// multiple of 4) is read once and stays in registers between the two passes.  With gate_w, the row's
+// sigmoid(y . gate_w) also goes to gate_out[row] (the shared-expert gate of a mixture-of-experts
+// layer, forward.rs:749-824: the normalised row is at hand here, in registers).
 __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, const float *__restrict__ add,
                                                        const float *__restrict__ w, float *__restrict__ y, int n,
-                                                       float eps) {
+                                                       float eps, const float *__restrict__ gate_w,
+                                                       float *__restrict__ gate_out) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
     float *xr = x + static_cast<size_t>(blockIdx.x) * n;
@@ -69,10 +72,22 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
         }
         s = block_sum(s, sh);
         const float scale = 1.0f / sqrtf(s / static_cast<float>(n) + eps);
+        float dot = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int i = 4 * (tid + 256 * j);
-            if (i < n) *reinterpret_cast<f4 *>(yr + i) = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
+            if (i < n) {
+                const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
+                *reinterpret_cast<f4 *>(yr + i) = o;
+                if (gate_w) {
+                    const f4 gw = *reinterpret_cast<const f4 *>(gate_w + i);
+                    dot += (o[0] * gw[0] + o[1] * gw[1]) + (o[2] * gw[2] + o[3] * gw[3]);
+                }
+            }
+        }
+        if (gate_w) {
+            dot = block_sum(dot, sh);
+            if (tid == 0) gate_out[blockIdx.x] = 1.0f / (1.0f + expf(-dot));
         }
         return;
     }
@@ -87,7 +102,16 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
     }
     s = block_sum(s, sh);
     const float scale = 1.0f / sqrtf(s / static_cast<float>(n) + eps);
-    for (int i = tid; i < n; i += 256) yr[i] = xr[i] * scale * w[i];
+    float dot = 0.0f;
+    for (int i = tid; i < n; i += 256) {
+        const float o = xr[i] * scale * w[i];
+        yr[i] = o;
+        if (gate_w) dot += o * gate_w[i];
+    }
+    if (gate_w) {
+        dot = block_sum(dot, sh);
+        if (tid == 0) gate_out[blockIdx.x] = 1.0f / (1.0f + expf(-dot));
+    }
 }
 
 // kernel_qk_rms_norm_rope_f32_packed_consecutive (attn.metal:137-196) + the f32 -> f16 KV scatter
@@ -430,10 +454,13 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
     if (rc) return rc;
     const float scale = 1.0f / sqrtf(static_cast<float>(hd));
     const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
+    bool cur_ready = false;  // s->cur already holds this layer's normalised input
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_layer &L = model->layers[il];
         _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
-        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
+        // (a mixture-of-experts layer leaves the next layer's normalised input behind)
+        if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
+        cur_ready = false;
         bool packed;
         if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, true, &packed, H, q_dim, kv_dim, n, st))) return rc;
         const int64_t tot = q_dim + 2 * kv_dim;
@@ -446,9 +473,14 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
                                  s->attn, st, 0, 0, s->pos)))
             return rc;
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
-        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps);  // x += mix first
-        if (c.n_expert > 0) {
-            if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, st))) return rc;
+        // x += mix first; a mixture-of-experts layer also gets its shared-expert gate from here
+        const bool moe = c.n_expert > 0;
+        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps, moe ? L.shexp_gate : nullptr,
+                                           moe ? s->moe.sg : nullptr);
+        if (moe) {
+            const float *next_w = il + 1 < c.n_layers ? model->layers[il + 1].attn_norm : model->output_norm;
+            if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, L.shexp_gate != nullptr, next_w, s->cur, &cur_ready, st)))
+                return rc;
         } else {
             if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, n, st))) return rc;
             if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
@@ -458,7 +490,7 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
             if (tap_layers[t] == il)
                 capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
     }
-    rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, model->output_norm, s->cur, H, c.eps);
+    if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, model->output_norm, s->cur, H, c.eps, nullptr, nullptr);
     if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
     if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gp, st))) return rc;
     DFL_HIP_CHECK(ctx, hipGetLastError());
@@ -651,7 +683,7 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
     for (int64_t c0 = s->ctx_h_ready; c0 < s->ctx_len; c0 += 16) {
         const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
         if ((rc = gemm(ctx, head->fc, s->ctx_raw + c0 * feat, s->tmp, feat, H, m, st))) return rc;
-        rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, nullptr, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps);
+        rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, nullptr, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps, nullptr, nullptr);
     }
     // phase 2: noise embedding
     int32_t ids_host[16], pos_host[16];
@@ -690,7 +722,7 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                     kc + c0 * kv_dim, kv_packed ? s->pk + kv_dim : vc + c0 * kv_dim, kv_packed ? 2 * kv_dim : kv_dim, k16, vt16,
                     static_cast<int>(kv_dim), s->cap16, c0, kv_packed ? vc + c0 * kv_dim : nullptr);
         }
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps);
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
         bool packed;  // only on the fast path: the general attention kernel reads V dense
         if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st))) return rc;
         const int64_t tot = q_dim + 2 * kv_dim;
@@ -712,12 +744,12 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                                                             L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
         }
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st))) return rc;
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps);  // x += mix first
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps, nullptr, nullptr);  // x += mix first
         if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, N, st))) return rc;
         if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st))) return rc;
         add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
     }
-    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, head->output_norm, s->cur, H, c.eps);
+    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, head->output_norm, s->cur, H, c.eps, nullptr, nullptr);
     float *lg = draft_logits ? draft_logits : s->logits;
     if ((rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st))) return rc;
     int32_t *am = draft_argmax ? draft_argmax : s->argmax;

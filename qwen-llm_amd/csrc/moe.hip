@@ -43,6 +43,21 @@ __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
     return (static_cast<unsigned long long>(hi) << 32) | lo;
 }
 
+// The same for a float maximum (NaN operands are ignored, as v_max_f32 does); lanes without a source
+// keep their own value.
+__device__ __forceinline__ float wave_max_f32(float v) {
+#define DFL_FMAX_STEP(ctrl, row_mask)                                                                              \
+    v = fmaxf(v, __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(v), __float_as_uint(v), ctrl, row_mask, 0xf, false)))
+    DFL_FMAX_STEP(0x111, 0xf);
+    DFL_FMAX_STEP(0x112, 0xf);
+    DFL_FMAX_STEP(0x114, 0xf);
+    DFL_FMAX_STEP(0x118, 0xf);
+    DFL_FMAX_STEP(0x142, 0xa);
+    DFL_FMAX_STEP(0x143, 0xc);
+#undef DFL_FMAX_STEP
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
+}
+
 // Routing of a whole block in one workgroup of sixteen waves (n_expert <= 1024, at most 16 rows).
 // Wave w serves block row w: softmax, top-k (higher probability first, equal probabilities to the
 // lower id), the renormalised weights in pick order, and the
@@ -74,7 +89,9 @@ __global__ void __launch_bounds__(1024)
         for (int j = 0; j < 4; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
         const float *xr = x + static_cast<size_t>(row) * hidden;
         float dot = 0.0f;
-        if (hidden % 4 == 0) {
+        if (!shexp_gate) {
+            // the gate was computed by the kernel that wrote x
+        } else if (hidden % 4 == 0) {
             for (int base = 0; base < hidden; base += 2048) {
                 f4 xa[8], gb[8];
 #pragma unroll
@@ -95,7 +112,7 @@ __global__ void __launch_bounds__(1024)
             for (int i = lane; i < hidden; i += 64) dot += xr[i] * shexp_gate[i];
         }
         for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-        if (lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
+        if (shexp_gate && lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
 
         float mx = -INFINITY;
 #pragma unroll
@@ -176,6 +193,131 @@ __global__ void __launch_bounds__(1024)
     }
     __syncthreads();
     if (live && lane < n_used) slot_of[row * n_used + lane] = rank[pick_e[row][lane]];
+}
+
+// The same routing for n_expert <= 256, n_used <= 64, with a row's probabilities held in registers
+// (four per lane) and one workgroup barrier in all: a row's picks stay in its wave (lane k keeps pick
+// k), the row's picked experts go out as a 256-bit mask, and after the barrier every thread derives
+// the block's ascending expert list and the slot of each pick from the union of the sixteen masks by
+// population counts.  Same arithmetic, in the same order, as moe_route_kernel.
+__global__ void __launch_bounds__(1024)
+    moe_route_small_kernel(const float *__restrict__ logits, const float *__restrict__ x, const float *__restrict__ shexp_gate,
+                           int n_rows, int n_expert, int n_used, int hidden, int with_shared, int32_t *__restrict__ sel_e,
+                           float *__restrict__ sel_w, float *__restrict__ sg, int32_t *__restrict__ ids,
+                           int32_t *__restrict__ n_slots, int32_t *__restrict__ slot_of) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ unsigned long long row_mask[16][4];
+    const int tid = threadIdx.x, lane = tid & 63, row = tid >> 6;
+    const bool live = row < n_rows;
+    int my_e = 0;
+    unsigned long long m[4] = {0, 0, 0, 0};
+    if (live) {
+        const float *lg = logits + static_cast<size_t>(row) * n_expert;
+        float lgv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
+        const float *xr = x + static_cast<size_t>(row) * hidden;
+        float dot = 0.0f;
+        if (!shexp_gate) {
+            // the gate was computed by the kernel that wrote x
+        } else if (hidden % 4 == 0) {
+            for (int base = 0; base < hidden; base += 2048) {
+                f4 xa[8], gb[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int i = base + 4 * lane + 256 * j;
+                    xa[j] = gb[j] = f4{0, 0, 0, 0};
+                    if (i < hidden) {
+                        xa[j] = *reinterpret_cast<const f4 *>(xr + i);
+                        gb[j] = *reinterpret_cast<const f4 *>(shexp_gate + i);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (base + 4 * lane + 256 * j < hidden)
+                        dot += (xa[j][0] * gb[j][0] + xa[j][1] * gb[j][1]) + (xa[j][2] * gb[j][2] + xa[j][3] * gb[j][3]);
+            }
+        } else {
+            for (int i = lane; i < hidden; i += 64) dot += xr[i] * shexp_gate[i];
+        }
+        for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (shexp_gate && lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
+
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 4; j++) mx = fmaxf(mx, lgv[j]);
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        float pv[4];
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            pv[j] = 0.0f;
+            if (lane + 64 * j < n_expert) {
+                pv[j] = expf(lgv[j] - mx);
+                sum += pv[j];
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int j = 0; j < 4; j++) pv[j] = lane + 64 * j < n_expert ? pv[j] * inv : -1.0f;  // no such expert: never picked
+
+        // pick k = the highest remaining probability, equal probabilities to the lower id: a wave-wide
+        // float maximum (one DPP instruction per step), then the first lane / register that holds it,
+        // found with compares into scalar masks.  Taken and missing experts are -1, NaN never compares
+        // equal: if nothing is left (NaN logits) the pick falls back to an index in range.
+        float my_p = 0.0f;
+        for (int k = 0; k < n_used; k++) {
+            const float pmax = wave_max_f32(fmaxf(fmaxf(pv[0], pv[1]), fmaxf(pv[2], pv[3])));
+            int e_win = -1;
+#pragma unroll
+            for (int j = 3; j >= 0; j--) {
+                const unsigned long long hit = __builtin_amdgcn_ballot_w64(pv[j] == pmax);
+                if (hit) e_win = 64 * j + __builtin_ctzll(hit);
+            }
+            const bool none = !(pmax >= 0.0f) || e_win < 0;
+            if (none) e_win = k < n_expert ? k : n_expert - 1;
+            if (lane == k) {
+                my_e = e_win;
+                my_p = none ? 0.0f : pmax;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (lane + 64 * j == e_win) pv[j] = -1.0f;  // taken
+                if ((e_win >> 6) == j) m[j] |= 1ull << (e_win & 63);
+            }
+        }
+        float wsum = 0.0f;
+        for (int k = 0; k < n_used; k++) wsum += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_p), k));  // in pick order
+        wsum = fmaxf(wsum, 6.103515625e-05f);  // 2^-14
+        if (lane < n_used) {
+            sel_e[row * n_used + lane] = my_e;
+            sel_w[row * n_used + lane] = my_p / wsum;
+        }
+    }
+    if (lane < 4) row_mask[row][lane] = m[lane & 3];
+    __syncthreads();
+    unsigned long long un[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) un[j] |= row_mask[r][j];
+    auto slot = [&](int e) {  // experts below e in the union
+        int below = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (j < (e >> 6)) below += __popcll(un[j]);
+            if (j == (e >> 6)) below += __popcll(un[j] & ((1ull << (e & 63)) - 1));
+        }
+        return below;
+    };
+    if (tid < n_expert && ((un[tid >> 6] >> (tid & 63)) & 1)) ids[slot(tid)] = tid;
+    if (tid == 0) {
+        const int total = __popcll(un[0]) + __popcll(un[1]) + __popcll(un[2]) + __popcll(un[3]);
+        if (with_shared) ids[total] = -1;
+        *n_slots = total + (with_shared ? 1 : 0);
+    }
+    if (live && lane < n_used) slot_of[row * n_used + lane] = slot(my_e);
 }
 
 // Collects the slots whose pick is `expert`; returns the count (uniform over the workgroup).
@@ -301,10 +443,64 @@ __global__ void moe_combine_slots_kernel(const float *__restrict__ eo, const int
     x[static_cast<size_t>(row) * hidden + i] += out;
 }
 
+// The same, followed in the same pass by the RMSNorm that consumes x next (the following layer's
+// attention norm or the output norm): y = x * rsqrt(mean(x^2) + eps) * norm_w.  One workgroup per
+// row, the row (hidden <= 4096, a multiple of 4) in registers; element sums and the sum of squares
+// are taken in the order of moe_combine_slots_kernel followed by the norm kernel.
+__global__ void __launch_bounds__(256)
+    moe_combine_norm_kernel(const float *__restrict__ eo, const int32_t *__restrict__ slot_of, const float *__restrict__ sel_w,
+                            const float *__restrict__ sg, const float *__restrict__ shared, const int32_t *__restrict__ n_slots,
+                            int n_used, int hidden, float *__restrict__ x, const float *__restrict__ norm_w,
+                            float *__restrict__ y, float eps) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ float sh[4];
+    __shared__ float w_k[64];
+    __shared__ int32_t slot_k[64];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    if (tid < n_used) {
+        w_k[tid] = sel_w[row * n_used + tid];
+        slot_k[tid] = slot_of[row * n_used + tid];
+    }
+    __syncthreads();
+    const float gate = sg[row];
+    const size_t last = static_cast<size_t>(*n_slots) - 1;
+    f4 v[4];
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int i = 4 * (tid + 256 * j);
+        v[j] = f4{0, 0, 0, 0};
+        if (i < hidden) {
+            f4 out = {0, 0, 0, 0};
+            for (int k = 0; k < n_used; k++)
+                out += w_k[k] * *reinterpret_cast<const f4 *>(eo + (static_cast<size_t>(slot_k[k]) * 16 + row) * hidden + i);
+            const f4 shv = shared ? *reinterpret_cast<const f4 *>(shared + static_cast<size_t>(row) * hidden + i)
+                                  : *reinterpret_cast<const f4 *>(eo + (last * 16 + row) * hidden + i);
+            out += gate * shv;
+            v[j] = *reinterpret_cast<const f4 *>(x + static_cast<size_t>(row) * hidden + i) + out;
+            *reinterpret_cast<f4 *>(x + static_cast<size_t>(row) * hidden + i) = v[j];
+        }
+        s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
+    }
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if ((tid & 63) == 0) sh[tid >> 6] = s;
+    __syncthreads();
+    s = ((sh[0] + sh[1]) + sh[2]) + sh[3];
+    const float scale = 1.0f / sqrtf(s / static_cast<float>(hidden) + eps);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int i = 4 * (tid + 256 * j);
+        if (i < hidden)
+            *reinterpret_cast<f4 *>(y + static_cast<size_t>(row) * hidden + i) = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
+    }
+}
+
 }  // namespace
 
 int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, const float *cur, int n,
-                    const dfl_moe_scratch &s, float *x_resid, hipStream_t st) {
+                    const dfl_moe_scratch &s, float *x_resid, bool gate_done, const float *next_norm_w, float *next_cur,
+                    bool *next_done, hipStream_t st) {
+    if (next_done) *next_done = false;
     const int E = c.n_expert, used = c.n_expert_used < E ? c.n_expert_used : E;
     const int H = c.hidden, fe = c.ffn_expert, fs = c.ffn_shared;
     const int n_slots = n * used;
@@ -336,8 +532,13 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
             attr = true;
         }
     }
-    moe_route_kernel<<<1, 1024, route_lds, st>>>(s.probs, cur, L.shexp_gate, n, E, used, H, folded_shared ? 1 : 0,
-                                                                   s.sel_e, s.sel_w, s.sg, s.ids, s.n_distinct, s.slot_of);
+    const float *gate_w = gate_done ? nullptr : L.shexp_gate;  // null: sg is already there
+    if (E <= 256)
+        moe_route_small_kernel<<<1, 1024, 0, st>>>(s.probs, cur, gate_w, n, E, used, H, folded_shared ? 1 : 0, s.sel_e,
+                                                   s.sel_w, s.sg, s.ids, s.n_distinct, s.slot_of);
+    else
+        moe_route_kernel<<<1, 1024, route_lds, st>>>(s.probs, cur, gate_w, n, E, used, H, folded_shared ? 1 : 0,
+                                                     s.sel_e, s.sel_w, s.sg, s.ids, s.n_distinct, s.slot_of);
     if (batched) {
         // the selected experts' matrices form one streaming GEMM each for gate, up and down: every
         // distinct expert's weights are read once, with all block rows riding along on the MFMA;
@@ -394,7 +595,11 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         silu_mul_rows_kernel<<<static_cast<unsigned>((nf + 255) / 256), 256, 0, st>>>(s.g, s.u, nf);
         if ((rc = dflash_gemm_fewrow(ctx, L.down.type, L.down.data, s.g, DFLASH_TYPE_F32, s.shared, fs, H, n, st))) return rc;
     }
-    if (batched)
+    if (batched && next_norm_w && next_cur && next_done && H <= 4096 && H % 4 == 0) {
+        moe_combine_norm_kernel<<<n, 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg, folded_shared ? nullptr : s.shared, s.n_distinct,
+                                                   used, H, x_resid, next_norm_w, next_cur, c.eps);
+        *next_done = true;
+    } else if (batched)
         moe_combine_slots_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg,
                                                                          folded_shared ? nullptr : s.shared, s.n_distinct, used,
                                                                          H, x_resid);
