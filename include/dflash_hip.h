@@ -359,6 +359,14 @@ int64_t dflash_draft_session_ctx_len(const dflash_draft_session *s);
 int32_t dflash_draft_append_ctx(dflash_ctx *ctx, dflash_draft_session *s, const float *hidden_capture, int32_t n_cols,
                                 const int32_t *positions_host, dflash_stream_t stream);
 
+/* The first phases of draft_block_inner alone (metal_dflash.rs:16045-16143 and the context K/V
+ * projections that follow): fc + hidden_norm and every layer's K/V for the context columns appended
+ * since they were last brought up to date.  dflash_draft_block does this itself for whatever is
+ * pending; calling it after a prompt's columns were appended moves that work (one pass over the
+ * whole prompt) out of the first speculative step.  Enqueue-only. */
+int32_t dflash_draft_prepare_ctx(dflash_ctx *ctx, const dflash_draft_head *head, dflash_draft_session *s,
+                                 dflash_stream_t stream);
+
 /* MetalDFlashDraftDecoder::draft_block / draft_block_with_logits (metal_dflash.rs:17257-17513;
  * CPU oracle Forward::dflash_draft, forward.rs:380-662): noise ids [carry, mask x (block-1)] at
  * positions noise_start_pos.., attention over ctx || noise, shared embedding and lm_head of the

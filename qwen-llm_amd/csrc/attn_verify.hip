@@ -503,8 +503,11 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     // and at least 128 keys long (a split costs a partial tile per head and row)
     int per_cu = n_pos >= 16384 ? 2 : 1;  // short contexts: fewer splits, fewer partial tiles to merge
     int64_t min_chunk = 128;
-    if (const char *e = getenv("DFLASH_ATTN_PER_CU")) per_cu = atoi(e);  // tuning knobs
-    if (const char *e = getenv("DFLASH_ATTN_MIN_CHUNK")) min_chunk = atoi(e);
+    // tuning knobs, read once per process
+    static const int env_per_cu = [] { const char *e = getenv("DFLASH_ATTN_PER_CU"); return e ? atoi(e) : 0; }();
+    static const int env_min_chunk = [] { const char *e = getenv("DFLASH_ATTN_MIN_CHUNK"); return e ? atoi(e) : 0; }();
+    if (env_per_cu > 0) per_cu = env_per_cu;
+    if (env_min_chunk > 0) min_chunk = env_min_chunk;
     if (per_cu < 1) per_cu = 1;
     if (min_chunk < 32) min_chunk = 32;
     const int want = static_cast<int>((static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv - 1) / n_kv);

@@ -1270,10 +1270,19 @@ extern "C" void dflash_dbg_set_trace2(uint64_t p) {
 
 namespace {
 
-int env_int(const char *name, int fallback) {
-    const char *v = getenv(name);
-    return (v && *v) ? atoi(v) : fallback;
-}
+// Tuning knobs from the environment, each read once per process (getenv walks the whole environment,
+// and a launch-bound caller pays for that on every launch).
+struct EnvInt {
+    bool set;
+    int value;
+    explicit EnvInt(const char *name) {
+        const char *v = getenv(name);
+        set = v && *v;
+        value = set ? atoi(v) : 0;
+    }
+    int get(int fallback) const { return set ? value : fallback; }
+};
+#define env_int(name, fallback) ([]() -> const EnvInt & { static const EnvInt e(name); return e; }().get(fallback))
 
 int32_t launch_q6k(dflash_ctx *ctx, Q6KSet set, const void *x, int32_t x_type, int64_t n_in, int32_t n_rows, hipStream_t st) {
     if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))

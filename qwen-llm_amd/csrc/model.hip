@@ -191,6 +191,21 @@ __global__ void silu_mul_ld_kernel(const float *__restrict__ g, const float *__r
     }
 }
 
+// Up to sixteen host integers reach the device as a kernel argument (by value, in the dispatch
+// packet) instead of through a pageable host-to-device copy, which costs tens of microseconds of
+// idle GPU at every phase boundary of a speculative step.  ids may be null (positions only).
+struct Int16Args {
+    int32_t v[16];
+};
+__global__ void set_ids_pos_kernel(Int16Args ids, Int16Args pos, int n, int32_t *__restrict__ ids_dst,
+                                   int32_t *__restrict__ pos_dst) {
+    const int i = threadIdx.x;
+    if (i < n) {
+        if (ids_dst) ids_dst[i] = ids.v[i];
+        pos_dst[i] = pos.v[i];
+    }
+}
+
 // kernel_add_inplace_f32 (elementwise.metal:89)
 __global__ void add_kernel(float *__restrict__ x, const float *__restrict__ y, size_t n) {
     size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -523,10 +538,12 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
     if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "verify_block: session/model shape mismatch");
 
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int32_t pos_host[16];
-    for (int i = 0; i < n; i++) pos_host[i] = static_cast<int32_t>(start + i);
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ids, tokens, n * sizeof(int32_t), hipMemcpyHostToDevice, st));
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos, pos_host, n * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    Int16Args ids_arg = {}, pos_arg = {};
+    for (int i = 0; i < n; i++) {
+        ids_arg.v[i] = tokens[i];
+        pos_arg.v[i] = static_cast<int32_t>(start + i);
+    }
+    set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, n, s->ids, s->pos);
     float *lg = logits ? logits : s->logits;
     int32_t *am = argmax ? argmax : s->argmax;
     float *gp = gap ? gap : s->gap;
@@ -651,50 +668,36 @@ int32_t dflash_draft_append_ctx(dflash_ctx *ctx, dflash_draft_session *s, const 
     const size_t feat = static_cast<size_t>(s->cfg.n_taps) * s->cfg.hidden;
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ctx_raw + s->ctx_len * feat, hidden_capture, n_cols * feat * sizeof(float),
                                       hipMemcpyDeviceToDevice, st));
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos_ctx + s->ctx_len, positions, n_cols * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    if (n_cols <= 16) {
+        Int16Args none = {}, pos_arg = {};
+        for (int i = 0; i < n_cols; i++) pos_arg.v[i] = positions[i];
+        set_ids_pos_kernel<<<1, 64, 0, st>>>(none, pos_arg, n_cols, nullptr, s->pos_ctx + s->ctx_len);
+    } else {
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos_ctx + s->ctx_len, positions, n_cols * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    }
     s->ctx_len += n_cols;
     return DFLASH_OK;
 }
 
-int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
-                           dflash_draft_session *s, int32_t carry, int32_t mask_token, int64_t noise_start,
-                           int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream) {
-    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
-    if (!target || !head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_block: null argument");
-    const dflash_draft_cfg &c = head->cfg;
-    if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_block: session/head shape mismatch");
-    if (c.hidden != target->cfg.hidden) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "draft_block: drafter and target hidden sizes differ");
-    const int V = target->cfg.vocab;
-    if (V != s->vocab) return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_block: vocabulary mismatch");
-    if (carry < 0 || carry >= V || mask_token < 0 || mask_token >= V)
-        return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "draft_block: carry %d / mask %d outside vocabulary %d", carry, mask_token, V);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const int N = c.block_size, H = c.hidden, hd = c.head_dim;
-    const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
-    const size_t feat = static_cast<size_t>(c.n_taps) * H;
-    int32_t rc;
-    // MFMA attention over the f16 mirror when context column i sits at position i and the block
-    // starts at position ctx_len (the generation loop's case); else the general f32 kernel.  The
-    // mirror is only kept current while that holds, so leaving the fast path is final.
-    const bool fast = s->contiguous && noise_start == s->ctx_len && c.n_q / c.n_kv <= 16;
-    if (!fast) s->contiguous = false;
+namespace {
 
-    // phase 1: fc + hidden_norm on the NEW context columns only (metal_dflash.rs:16045-16143)
+// Phase 1 of the drafter (metal_dflash.rs:16045-16143) and the per-layer context K/V, for the
+// context columns appended since the last call: fc + hidden_norm, then each layer's K (normed and
+// rotated at the column's own position) and V, and the f16 mirror while it is kept (mirror).
+// The watermarks advance once everything was enqueued without error.
+int32_t draft_prepare(dflash_ctx *ctx, const dflash_draft_head *head, dflash_draft_session *s, bool mirror, hipStream_t st) {
+    const dflash_draft_cfg &c = head->cfg;
+    const int H = c.hidden, hd = c.head_dim;
+    const size_t kv_dim = static_cast<size_t>(c.n_kv) * hd;
+    const size_t feat = static_cast<size_t>(c.n_taps) * H;
+    const bool fast = mirror;
+    int32_t rc;
+    if (s->ctx_h_ready >= s->ctx_len && s->kv_ready >= s->ctx_len) return DFLASH_OK;
     for (int64_t c0 = s->ctx_h_ready; c0 < s->ctx_len; c0 += 16) {
         const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
         if ((rc = gemm(ctx, head->fc, s->ctx_raw + c0 * feat, s->tmp, feat, H, m, st))) return rc;
         rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, nullptr, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps, nullptr, nullptr);
     }
-    // phase 2: noise embedding
-    int32_t ids_host[16], pos_host[16];
-    for (int i = 0; i < N; i++) {
-        ids_host[i] = i == 0 ? carry : mask_token;
-        pos_host[i] = static_cast<int32_t>(noise_start + i);
-    }
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->ids, ids_host, N * sizeof(int32_t), hipMemcpyHostToDevice, st));
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos, pos_host, N * sizeof(int32_t), hipMemcpyHostToDevice, st));
-    if ((rc = embed_rows(ctx, target->token_embd, s->ids, N, H, s->x, st))) return rc;
-
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_draft_layer &L = head->layers[il];
         float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
@@ -722,6 +725,63 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                     kc + c0 * kv_dim, kv_packed ? s->pk + kv_dim : vc + c0 * kv_dim, kv_packed ? 2 * kv_dim : kv_dim, k16, vt16,
                     static_cast<int>(kv_dim), s->cap16, c0, kv_packed ? vc + c0 * kv_dim : nullptr);
         }
+    }
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    s->ctx_h_ready = s->ctx_len;
+    s->kv_ready = s->ctx_len;
+    return DFLASH_OK;
+}
+
+}  // namespace
+
+int32_t dflash_draft_prepare_ctx(dflash_ctx *ctx, const dflash_draft_head *head, dflash_draft_session *s, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_prepare_ctx: null argument");
+    if (memcmp(&head->cfg, &s->cfg, sizeof(head->cfg)) != 0)
+        return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_prepare_ctx: session/head shape mismatch");
+    return draft_prepare(ctx, head, s, s->contiguous && head->cfg.n_q / head->cfg.n_kv <= 16, static_cast<hipStream_t>(stream));
+}
+
+int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
+                           dflash_draft_session *s, int32_t carry, int32_t mask_token, int64_t noise_start,
+                           int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!target || !head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_block: null argument");
+    const dflash_draft_cfg &c = head->cfg;
+    if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_block: session/head shape mismatch");
+    if (c.hidden != target->cfg.hidden) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "draft_block: drafter and target hidden sizes differ");
+    const int V = target->cfg.vocab;
+    if (V != s->vocab) return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_block: vocabulary mismatch");
+    if (carry < 0 || carry >= V || mask_token < 0 || mask_token >= V)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "draft_block: carry %d / mask %d outside vocabulary %d", carry, mask_token, V);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int N = c.block_size, H = c.hidden, hd = c.head_dim;
+    const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
+    const size_t feat = static_cast<size_t>(c.n_taps) * H;
+    int32_t rc;
+    // MFMA attention over the f16 mirror when context column i sits at position i and the block
+    // starts at position ctx_len (the generation loop's case); else the general f32 kernel.  The
+    // mirror is only kept current while that holds, so leaving the fast path is final.
+    const bool fast = s->contiguous && noise_start == s->ctx_len && c.n_q / c.n_kv <= 16;
+    if (!fast) s->contiguous = false;
+
+    // phase 1 and the context K/V of the new columns (a no-op if dflash_draft_prepare_ctx ran)
+    if ((rc = draft_prepare(ctx, head, s, fast, st))) return rc;
+    // phase 2: noise embedding
+    Int16Args ids_arg = {}, pos_arg = {};
+    for (int i = 0; i < N; i++) {
+        ids_arg.v[i] = i == 0 ? carry : mask_token;
+        pos_arg.v[i] = static_cast<int32_t>(noise_start + i);
+    }
+    set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, N, s->ids, s->pos);
+    if ((rc = embed_rows(ctx, target->token_embd, s->ids, N, H, s->x, st))) return rc;
+
+    for (int il = 0; il < c.n_layers; il++) {
+        const dflash_draft_layer &L = head->layers[il];
+        float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
+        float *vc = s->v_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
+        _Float16 *k16 = s->k16 + il * static_cast<size_t>(s->cap16) * kv_dim;
+        _Float16 *vt16 = s->vt16 + il * static_cast<size_t>(s->cap16) * kv_dim;
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
         bool packed;  // only on the fast path: the general attention kernel reads V dense
         if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st))) return rc;

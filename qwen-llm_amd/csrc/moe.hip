@@ -518,8 +518,9 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     int32_t rc = dflash_gemm_fewrow(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
     if (rc) return rc;
     if (E > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: %d experts (at most 1024)", E);
+    static const bool per_slot_forced = getenv("DFLASH_MOE_PERSLOT") != nullptr;  // read once per process
     const bool batched = et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K && H % DFL_QK_K == 0 && fe % DFL_QK_K == 0 &&
-                         !getenv("DFLASH_MOE_PERSLOT");
+                         !per_slot_forced;
     // the shared expert rides along as one more slot of the batched GEMMs when it has the experts' shape
     const bool folded_shared = batched && fs == fe && L.gate.type == DFLASH_TYPE_Q4_K && L.up.type == DFLASH_TYPE_Q4_K &&
                                L.down.type == DFLASH_TYPE_Q4_K;

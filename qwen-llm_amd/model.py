@@ -122,6 +122,8 @@ def _lib():
         L.dflash_draft_session_destroy.argtypes = [vp]
         L.dflash_draft_session_ctx_len.restype = i64
         L.dflash_draft_session_ctx_len.argtypes = [vp]
+        L.dflash_draft_prepare_ctx.restype = i32
+        L.dflash_draft_prepare_ctx.argtypes = [vp, vp, vp, vp]
         L.dflash_draft_append_ctx.restype = i32
         L.dflash_draft_append_ctx.argtypes = [vp, vp, vp, i32, C.POINTER(i32), vp]
         L.dflash_draft_block.restype = i32
@@ -450,6 +452,11 @@ class DraftSession:
         self.ctx._check(self._L.dflash_draft_append_ctx(self.ctx._h, self._h, hc.data_ptr() if n else None, n, pos,
                                                         _stream_ptr()))
 
+    def prepare_ctx(self):
+        """Bring fc + hidden_norm and the per-layer context K/V up to date for the columns appended so far
+        (draft_block does it lazily otherwise)."""
+        self.ctx._check(self._L.dflash_draft_prepare_ctx(self.ctx._h, C.byref(self.head.c), self._h, _stream_ptr()))
+
     def draft_block(self, carry_token: int, mask_token: int, noise_start_pos: int, want_logits=False, sync=True):
         torch = _torch()
         dev = f"cuda:{self.ctx.device}"
@@ -536,6 +543,9 @@ class SpeculativeDecoder:
             out = self.session.encode_packed_verify_layer_major(blk, s)
             self.draft_session.append_target_ctx_columns(out.hidden_capture, list(range(s, s + len(blk))))
             last = out
+        # the drafter's pass over the prompt's columns belongs to the prefill, not to the first step
+        self.draft_session.prepare_ctx()
+        _torch().cuda.synchronize()
         self.position = len(prompt)
         return last.argmax_host[-1]
 

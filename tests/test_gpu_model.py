@@ -170,19 +170,22 @@ def test_draft_block_matches_oracle(ctx, oracle, target, causal, swa):
     sess.close()
 
 
-def test_separate_and_adjacent_weight_layouts_agree(ctx, oracle, target):
+@pytest.mark.parametrize("wtype", [dfl.TYPE_Q4_K, dfl.TYPE_Q6_K])
+def test_separate_and_adjacent_weight_layouts_agree(ctx, oracle, wtype):
     """A layer's wq/wk/wv and gate/up uploaded back to back run as one GEMM each (the default of the
-    mirror); uploaded separately they run as three and two.  Both layouts must match the oracle, and each
-    other to GEMM tolerance (the split-K boundaries differ, so not bit for bit)."""
-    model_adj, (omodel, _keep) = target
-    w = dfl.synth_target_weights(C1, seed=11)
+    mirror); uploaded separately they run as three and two (Q6_K: the three projections in one launch of
+    the set kernel).  Both layouts must match the oracle, and each other to GEMM tolerance (the split-K
+    boundaries differ, so not bit for bit)."""
+    w = dfl.synth_target_weights(C1, seed=11, wtype=wtype)
+    omodel, _keep = oracle.build_model(C1.as_dict(), w)
+    model_adj = dfl.TargetModel(ctx, C1, w)
     model_sep = dfl.TargetModel(ctx, C1, w, adjacent=False)
     L0a, L0s = model_adj.c.layers[0], model_sep.c.layers[0]
-    rb = 1024 // 256 * 144
+    rb = 1024 // 256 * (144 if wtype == dfl.TYPE_Q4_K else 210)
     assert L0a.wk.data == L0a.wq.data + 16 * 128 * rb and L0a.wv.data == L0a.wk.data + 8 * 128 * rb
     assert L0a.up.data == L0a.gate.data + 3072 * rb
     assert L0s.wk.data != L0s.wq.data + 16 * 128 * rb or L0s.wv.data != L0s.wk.data + 8 * 128 * rb
-    dw = dfl.synth_draft_weights(D1, seed=3)
+    dw = dfl.synth_draft_weights(D1, seed=3, wtype=wtype)
     ohead, _k2 = oracle.build_draft_head(D1.as_dict(), dw)
     rng = np.random.default_rng(23)
     cap = 64
