@@ -201,6 +201,13 @@ struct Q4KBatch {
     // depend on which other matrices take part (a verify block and a single-token pass then agree
     // bit for bit), at the price of coarser load balance.
     int whole_groups;
+    // SwiGLU pair mode (needs whole_groups): slot j stands for TWO matrices, ids[j] of this stack
+    // (gate) and ids[j] of a second stack w2 / extra_w2 (up), and y gets silu(x . gate^T) * (x . up^T).
+    // In the kernel's iteration space every tile group appears twice in a row (virtual group 2 g is
+    // the gate half, 2 g + 1 the up half of real group g); ranges are cut between pairs, the gate
+    // tile waits in registers while the up tile is computed.
+    int pair;
+    const uint8_t *w2, *extra_w2;
 };
 
 // Per-lane constants of the loads and of the activation write, set up once per kernel.
@@ -395,19 +402,29 @@ constexpr int kWaitLds = 0xC07F;
 // partial tile for the reduce kernel (slot 0: the range's first group, slot 1: its last).
 template <int kWaves>
 __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, const Q4KBatch &bt, int group, float4_t &acc,
-                                          float4_t &acc_min, float *__restrict__ y, float *__restrict__ partials,
-                                          int n_out, int n_rows, int tid) {
+                                          float4_t &acc_min, float4_t &stash, float *__restrict__ y,
+                                          float *__restrict__ partials, int n_out, int n_rows, int tid) {
     // rare path: an opaque copy of the thread index keeps its index arithmetic out of the stage loop
     asm volatile("" : "+v"(tid));
     const int lane = tid & 63, wave = tid >> 6, n = lane & 15, g = lane >> 4;
     float4_t res = acc - acc_min;
     acc = float4_t{0, 0, 0, 0};
     acc_min = float4_t{0, 0, 0, 0};
+    // the group's whole K lies inside this workgroup's range: no other workgroup contributes
+    const bool whole = group * rg.nb >= rg.it_begin && (group + 1) * rg.nb <= rg.it_end;
+    if (bt.pair) {
+        if ((group & 1) == 0) {  // gate half: keep the tile for the up half that follows
+            stash = res;
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) res[i] = stash[i] / (1.0f + expf(-stash[i])) * res[i];  // silu(gate) * up
+        group >>= 1;
+    }
     const int slot_j = bt.ids ? static_cast<int>(q4k_div(group, bt.by_gpm)) : 0, lg = group - slot_j * bt.groups_per_mat;
     y += static_cast<size_t>(slot_j) * bt.y_stride;
     const int orow = (lg * kWaves + wave) * 16 + n;
-    // the group's whole K lies inside this workgroup's range: no other workgroup contributes
-    if (group * rg.nb >= rg.it_begin && (group + 1) * rg.nb <= rg.it_end) {
+    if (whole) {
         if (orow < n_out) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
@@ -486,12 +503,15 @@ __global__ void __launch_bounds__(64 * kWaves)
     Q4KRange rg;
     rg.nb = nb;
     rg.n_wg = gridDim.x;
-    if (bt.ids) n_groups = bt.groups_per_mat * *bt.n_slots;  // how many matrices take part is decided on the device
+    const int vshift = bt.pair ? 1 : 0;  // virtual groups per real group, as a shift
+    if (bt.ids) n_groups = (bt.groups_per_mat * *bt.n_slots) << vshift;  // how many matrices take part is decided on the device
     rg.total = n_groups * nb;
     rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
     if (bt.whole_groups) {
-        rg.it_begin = static_cast<int>(q4k_div(static_cast<uint32_t>(n_groups) * rg.wg, bt.by_wg)) * nb;
-        rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(n_groups) * (rg.wg + 1), bt.by_wg)) * nb;
+        // cut between real groups (pair mode: between pairs of virtual groups)
+        const uint32_t units = static_cast<uint32_t>(n_groups) >> vshift;
+        rg.it_begin = (static_cast<int>(q4k_div(units * rg.wg, bt.by_wg)) << vshift) * nb;
+        rg.it_end = (static_cast<int>(q4k_div(units * (rg.wg + 1), bt.by_wg)) << vshift) * nb;
     } else {
         rg.it_begin = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * rg.wg, bt.by_wg));
         rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * (rg.wg + 1), bt.by_wg));
@@ -508,16 +528,19 @@ __global__ void __launch_bounds__(64 * kWaves)
     // first weight byte of a group's first row, its activations, and the local group index
     auto group_w = [&](int group) {
         if (!bt.ids) return w + static_cast<size_t>(group) * group_bytes;
+        const bool up = bt.pair && (group & 1);
+        group >>= vshift;
         const int j = static_cast<int>(q4k_div(group, bt.by_gpm)), lg = group - j * bt.groups_per_mat;
         const int32_t id = bt.ids[j];
-        const uint8_t *mat = id < 0 ? bt.extra_w : w + static_cast<size_t>(id) * bt.w_stride;
+        const uint8_t *mat = id < 0 ? (up ? bt.extra_w2 : bt.extra_w) : (up ? bt.w2 : w) + static_cast<size_t>(id) * bt.w_stride;
         return q4k_uniform(mat + static_cast<size_t>(lg) * group_bytes);
     };
     auto group_x = [&](int group) {
         if (!bt.ids) return xbytes;
-        return xbytes + static_cast<size_t>(q4k_div(group, bt.by_gpm)) * bt.x_stride * sizeof(XT);
+        return xbytes + static_cast<size_t>(q4k_div(group >> vshift, bt.by_gpm)) * bt.x_stride * sizeof(XT);
     };
     auto group_local = [&](int group) {
+        group >>= vshift;
         return bt.ids ? group - static_cast<int>(q4k_div(group, bt.by_gpm)) * bt.groups_per_mat : group;
     };
     DFL_TR(10);
@@ -570,7 +593,7 @@ __global__ void __launch_bounds__(64 * kWaves)
     issue_w_all(buf_c);
     advance_w();
     q4k_lane_x_offsets<kWaves, XT>(L, tid, n_rows, n_in);
-    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0};
+    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0}, stash = {0, 0, 0, 0};
     const Q4KMagic magic = q4k_magic();
     Q4KXRaw<kWaves, XT> raw_first, raw_a, raw_b;  // activations of stage 0 / odd stages / even stages >= 2
     bool young_w = false, young_x = false;
@@ -661,7 +684,7 @@ __global__ void __launch_bounds__(64 * kWaves)
         done++;
         if (done <= 8) DFL_TR(1 + done);
         if (++bc == nb || n_left == 0) {
-            q4k_flush<kWaves>(rg, bt, gc, acc, acc_min, y, partials, n_out, n_rows, tid);
+            q4k_flush<kWaves>(rg, bt, gc, acc, acc_min, stash, y, partials, n_out, n_rows, tid);
             bc = 0;
             gc++;
         }
@@ -894,7 +917,7 @@ __global__ void __launch_bounds__(64 * kWaves)
     const int n = lane & 15, g = lane >> 4;
     const int h = g >> 1, odd = g & 1;
     const uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
-    float4_t acc = {0, 0, 0, 0}, acc_off = {0, 0, 0, 0};
+    float4_t acc = {0, 0, 0, 0}, acc_off = {0, 0, 0, 0}, stash = {0, 0, 0, 0};  // stash: unused here (no pair mode)
     int gc = rg.first_group, bc = b0, n_left = rg.it_end - rg.it_begin;
     int cur = 0;  // weight buffer of the stage being computed
     bool first = true;
@@ -970,7 +993,7 @@ __global__ void __launch_bounds__(64 * kWaves)
         x_n = tx;
         n_left--;
         if (++bc == nb || n_left == 0) {
-            q4k_flush<kWaves>(rg, bt, gc, acc, acc_off, y, partials, n_out, n_rows, tid);
+            q4k_flush<kWaves>(rg, bt, gc, acc, acc_off, stash, y, partials, n_out, n_rows, tid);
             bc = 0;
             gc++;
         }
@@ -1347,7 +1370,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     int waves = (static_cast<int64_t>((tiles + 15) / 16) * nb * max_slots >= 2ll * ctx->n_cu) ? 16 : 8;
     waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
     const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
-    const int groups = gpm * max_slots;           // upper bound in batched mode
+    const int groups = gpm * max_slots * ((batch && batch->pair) ? 2 : 1);  // upper bound in batched mode (pair mode: virtual groups)
     int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
     const int64_t total = static_cast<int64_t>(groups) * nb;
     const int max_wgs = ctx->n_partial_wgs * 8 / waves;
@@ -1472,12 +1495,18 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
                              const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
                              size_t x_stride,
                              float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
-                             int32_t whole_groups, dflash_stream_t stream) {
+                             int32_t whole_groups, const void *w_stack_up, const void *extra_w_up, dflash_stream_t stream) {
     if (n_in % DFL_QK_K || n_in <= 0 || n_out <= 0 || n_rows < 1 || n_rows > 16 || max_slots < 1)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_q4k_batched: bad shape");
-    if (reinterpret_cast<uintptr_t>(w_stack) % 16 || reinterpret_cast<uintptr_t>(extra_w) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16)
+    if (reinterpret_cast<uintptr_t>(w_stack) % 16 || reinterpret_cast<uintptr_t>(extra_w) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16 ||
+        reinterpret_cast<uintptr_t>(w_stack_up) % 16 || reinterpret_cast<uintptr_t>(extra_w_up) % 16)
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_q4k_batched: operand alignment");
+    if (w_stack_up && (!whole_groups || (extra_w != nullptr) != (extra_w_up != nullptr)))
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "gemm_q4k_batched: the gate/up pair needs whole groups and both or neither extra matrix");
     Q4KBatch bt = {};
+    bt.pair = w_stack_up ? 1 : 0;
+    bt.w2 = static_cast<const uint8_t *>(w_stack_up);
+    bt.extra_w2 = static_cast<const uint8_t *>(extra_w_up);
     bt.ids = ids;
     bt.extra_w = static_cast<const uint8_t *>(extra_w);
     bt.n_slots = n_slots;

@@ -414,15 +414,6 @@ __global__ void silu_mul_rows_kernel(float *__restrict__ g, const float *__restr
     }
 }
 
-// g = silu(g) * u over the first *n_distinct slots of [slot][16][f]
-__global__ void silu_mul_slots_kernel(float *__restrict__ g, const float *__restrict__ u, const int32_t *__restrict__ n_distinct,
-                                      size_t per_slot) {
-    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i >= per_slot * static_cast<size_t>(*n_distinct)) return;
-    const float v = g[i];
-    g[i] = v / (1.0f + expf(-v)) * u[i];
-}
-
 // x[row] += sum_k w[row][k] * eo[slot_of[row][k]][row]  +  sg[row] * shared[row]
 // (shared == nullptr: the shared expert's output is the last slot of eo)
 __global__ void moe_combine_slots_kernel(const float *__restrict__ eo, const int32_t *__restrict__ slot_of,
@@ -547,17 +538,15 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         const bool fold = folded_shared;
         const int max_slots = (n_slots < E ? n_slots : E) + (fold ? 1 : 0);
         const size_t per_slot = static_cast<size_t>(16) * fe;
+        // gate and up of every selected expert in one launch, silu(gate) * up applied to the tiles
+        // while they are still in registers
         if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, static_cast<size_t>(fe) * rb_in, fold ? L.gate.data : nullptr, s.ids,
-                                       s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, per_slot, H, fe, n, 1, st)))
+                                       s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, per_slot, H, fe, n, 1,
+                                       L.up_exps.data, fold ? L.up.data : nullptr, st)))
             return rc;
-        if ((rc = dfl_gemm_q4k_batched(ctx, L.up_exps.data, static_cast<size_t>(fe) * rb_in, fold ? L.up.data : nullptr, s.ids,
-                                       s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.up_out, per_slot, H, fe, n, 1, st)))
-            return rc;
-        silu_mul_slots_kernel<<<static_cast<unsigned>((per_slot * max_slots + 255) / 256), 256, 0, st>>>(s.gate_out, s.up_out,
-                                                                                                     s.n_distinct, per_slot);
         if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, static_cast<size_t>(H) * rb_dn, fold ? L.down.data : nullptr, s.ids,
                                        s.n_distinct, max_slots, s.gate_out, DFLASH_TYPE_F32, per_slot, s.eo,
-                                       static_cast<size_t>(16) * H, fe, H, n, 1, st)))
+                                       static_cast<size_t>(16) * H, fe, H, n, 1, nullptr, nullptr, st)))
             return rc;
     } else {
         {
