@@ -90,7 +90,7 @@ struct dfl_moe_scratch {
     float *sg = nullptr;      // [16] shared-expert gate
     float *act = nullptr;     // [16*n_used][ffn_expert]           (per-slot path)
     float *eo = nullptr;      // [slots][16][hidden]; per-slot path: [16*n_used][hidden]
-    float *gate_out = nullptr, *up_out = nullptr;  // [slots][16][ffn_expert] (batched path)
+    float *gate_out = nullptr;  // [slots][16][ffn_expert]: silu(gate) * up of every slot (batched path)
     int32_t *ids = nullptr, *n_distinct = nullptr, *slot_of = nullptr;  // distinct experts, their count, pick -> slot
     float *shared = nullptr;  // [16][hidden]
     float *g = nullptr, *u = nullptr;  // [16][ffn_shared]

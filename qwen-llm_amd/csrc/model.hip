@@ -408,7 +408,6 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
              dev_alloc(&s->moe.act, 16 * used * cfg->ffn_expert) &&
              dev_alloc(&s->moe.eo, 16 * (std::min<size_t>(16 * used, cfg->n_expert) + 1) * cfg->hidden) &&
              dev_alloc(&s->moe.gate_out, 16 * (std::min<size_t>(16 * used, cfg->n_expert) + 1) * cfg->ffn_expert) &&
-             dev_alloc(&s->moe.up_out, 16 * (std::min<size_t>(16 * used, cfg->n_expert) + 1) * cfg->ffn_expert) &&
              dev_alloc(&s->moe.ids, cfg->n_expert + 1) && dev_alloc(&s->moe.n_distinct, 1) && dev_alloc(&s->moe.slot_of, 16 * used) &&
              dev_alloc(&s->moe.shared, 16 * cfg->hidden);
         s->moe.g = s->g;
@@ -430,7 +429,7 @@ void dflash_session_destroy(dflash_session *s) {
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
                     s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax, s->hidden,
                     s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared,
-                    s->moe.gate_out, s->moe.up_out, s->moe.ids, s->moe.n_distinct, s->moe.slot_of, s->pk};
+                    s->moe.gate_out, s->moe.ids, s->moe.n_distinct, s->moe.slot_of, s->pk};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;

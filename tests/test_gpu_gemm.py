@@ -137,6 +137,28 @@ def test_gemm_deterministic_and_linear(ctx):
     assert (ys - (y1 + y2)).abs().max().item() <= 4e-3 * scale
 
 
+@pytest.mark.parametrize("qtype", [dfl.synth.Q4_K, dfl.synth.Q6_K])
+@pytest.mark.parametrize("n_in,n_out", [(2048, 5120), (4096, 2048), (2048, 12288), (6144, 2048)])
+def test_gemm_small_split_k_repeats(ctx, oracle, qtype, n_in, n_out):
+    """Products of a few MB (the projections of a decoder layer) are split over K across workgroups, their
+    partial tiles living in a scratch buffer that every launch shares.  Forty launches in a row, alternating
+    with another shape: every result bit-identical to the first and within the GEMM bar of the f64 reference."""
+    import torch
+
+    w = dev(dfl.synth.random_weight(qtype, n_out, n_in, seed=5))
+    w2 = dev(dfl.synth.random_weight(qtype, 1024, 2048, seed=6))
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn((16, n_in), device="cuda", generator=g, dtype=torch.float32)
+    x2 = torch.randn((16, 2048), device="cuda", generator=g, dtype=torch.float32)
+    first = ctx.gemm_fewrow(w, qtype, x, n_in, n_out).clone()
+    other = ctx.gemm_fewrow(w2, qtype, x2, 2048, 1024).clone()
+    for _ in range(20):
+        assert torch.equal(ctx.gemm_fewrow(w, qtype, x, n_in, n_out), first)
+        assert torch.equal(ctx.gemm_fewrow(w2, qtype, x2, 2048, 1024), other)
+    ref = f64_reference(oracle, qtype, w.cpu().numpy(), x.cpu().numpy(), n_in, n_out)
+    check_gemm(first.cpu().numpy(), ref, f"split-K {n_in}x{n_out}")
+
+
 @pytest.mark.parametrize("n_in,n_out", [(5120, 17408), (17408, 5120), (5120, 6144)])
 def test_gemm_fewrow_full_size_q4k(ctx, oracle, n_in, n_out):
     """the three production shapes, X f16 N(0,1), W = Q4_K(N(0,0.02)), seed 1; checked on a
