@@ -332,6 +332,10 @@ typedef struct {
     int32_t causal;
     uint32_t swa_window; /* 0 = full */
     float eps, rope_theta;
+    /* DFlash-2 (loader.rs:367-376, 1030-1056); all zero for a DFlash-1 drafter.  conv_kernel_size > 0:
+     * every layer carries the two convolution pairs; selector_rank > 0: the head carries the
+     * selector (selector_top_k must then be 16, the width of the top-16 kernel). */
+    int32_t conv_kernel_size, conv_group_size, selector_rank, selector_top_k;
 } dflash_draft_cfg;
 
 typedef struct {
@@ -339,6 +343,10 @@ typedef struct {
     dflash_qtensor wq, wk, wv, wo, gate, up, down;
     int32_t is_swa;
     int32_t pad;
+    /* DFlashConvTensors (loader.rs:305-323): blk.N.{attn,ffn}_conv_proj.weight
+     * [hidden -> 2 * kernel * hidden / group] and blk.N.{attn,ffn}_conv_base, f32 [2][kernel][hidden] */
+    dflash_qtensor conv_attn_proj, conv_ffn_proj;
+    const float *conv_attn_base, *conv_ffn_base;
 } dflash_draft_layer;
 
 typedef struct {
@@ -346,6 +354,10 @@ typedef struct {
     const dflash_draft_layer *layers; /* host array */
     dflash_qtensor fc;                /* [n_taps*hidden -> hidden] */
     const float *hidden_norm, *output_norm;
+    /* DFlashSelectorTensors (loader.rs:325-340): selector_hidden.weight [hidden -> rank] and the
+     * per-token predecessor / successor tables, [vocab][rank] */
+    dflash_qtensor selector_hidden;
+    dflash_codebook selector_predecessor, selector_successor;
 } dflash_draft_head;
 
 typedef struct dflash_draft_session dflash_draft_session;
@@ -371,7 +383,11 @@ int32_t dflash_draft_prepare_ctx(dflash_ctx *ctx, const dflash_draft_head *head,
  * CPU oracle Forward::dflash_draft, forward.rs:380-662): noise ids [carry, mask x (block-1)] at
  * positions noise_start_pos.., attention over ctx || noise, shared embedding and lm_head of the
  * target.  Outputs (device, may be NULL): draft_argmax[block] i32 (slot 0 unused by callers),
- * draft_logits[block][vocab].  If argmax_host is non-NULL the call waits and copies. */
+ * draft_logits[block][vocab].  If argmax_host is non-NULL the call waits and copies.
+ * A DFlash-2 head (cfg.conv_kernel_size / cfg.selector_rank) adds the per-layer convolutions
+ * (metal_dflash.rs:16210-16262, 16795-16820, 16836-16885, 17003-17022) and replaces the argmax by
+ * the top-16 + selector gate + lattice walk of :17098-17130 and select_draft_path (:17176-17251):
+ * draft_argmax then holds the walk's tokens. */
 int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
                            dflash_draft_session *s, int32_t carry_token, int32_t mask_token, int64_t noise_start_pos,
                            int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream);

@@ -109,6 +109,13 @@ class DraftHead(C.Structure):
                 ("output_norm", C.c_void_p)]
 
 
+class DFlash2Ext(C.Structure):
+    _fields_ = [("conv_kernel_size", C.c_int32), ("conv_group_size", C.c_int32), ("selector_rank", C.c_int32),
+                ("pad", C.c_int32), ("conv_attn_proj", C.POINTER(QTensor)), ("conv_ffn_proj", C.POINTER(QTensor)),
+                ("conv_attn_base", C.POINTER(C.c_void_p)), ("conv_ffn_base", C.POINTER(C.c_void_p)),
+                ("selector_hidden", QTensor)]
+
+
 _lib = None
 
 
@@ -172,6 +179,9 @@ def _declare(L):
     L.orc_attn_draft.argtypes = [vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, C.c_uint32, C.c_int, C.c_uint32, vp]
     L.orc_target_verify.argtypes = [C.POINTER(Model), vp, sz, sz, vp, vp, sz, vp, vp, sz, vp]
     L.orc_dflash_draft.argtypes = [C.POINTER(Model), C.POINTER(DraftHead), vp, vp, sz, vp, C.c_uint32, vp]
+    L.orc_dflash_draft_ex.restype = C.c_int
+    L.orc_dflash_draft_ex.argtypes = [C.POINTER(Model), C.POINTER(DraftHead), C.POINTER(DFlash2Ext), vp, vp, sz, vp,
+                                      C.c_uint32, vp, vp]
     L.orc_dflash2_conv.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, sz]
     L.orc_dflash2_conv.restype = None
     L.orc_codebook_row.argtypes = [C.POINTER(Codebook), sz, vp]
@@ -414,10 +424,43 @@ def build_draft_head(cfg: dict, weights: dict):
         for k in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
             setattr(L, k, keep.q(Lw[k]))
         L.is_swa = int(Lw.get("is_swa", 0))
-    h = DraftHead(DraftCfg(**cfg), layers, keep.q(weights["fc"]), keep.f32(weights["hidden_norm"]),
-                  keep.f32(weights["output_norm"]))
+    known = {n for n, _ in DraftCfg._fields_}
+    h = DraftHead(DraftCfg(**{k: v for k, v in cfg.items() if k in known}), layers, keep.q(weights["fc"]),
+                  keep.f32(weights["hidden_norm"]), keep.f32(weights["output_norm"]))
     keep.bufs.append(layers)
     return h, keep
+
+
+def build_dflash2_ext(cfg: dict, weights: dict):
+    """The DFlash-2 additions of a drafter: cfg carries conv_kernel_size / conv_group_size / selector_rank, every
+    layer 'conv_attn_proj', 'conv_ffn_proj' ((type, blocks), [2*kernel*H/group rows][H]) and 'conv_attn_base',
+    'conv_ffn_base' (f32 [2][kernel][H]); the head 'selector_hidden' ((type, blocks), [rank rows][H]).
+    Returns (DFlash2Ext, keepalive)."""
+    keep = _Keep()
+    n = cfg["n_layers"]
+    ap, fp = (QTensor * n)(), (QTensor * n)()
+    ab, fb = (C.c_void_p * n)(), (C.c_void_p * n)()
+    for il, Lw in enumerate(weights["layers"]):
+        ap[il], fp[il] = keep.q(Lw["conv_attn_proj"]), keep.q(Lw["conv_ffn_proj"])
+        ab[il], fb[il] = keep.f32(Lw["conv_attn_base"]), keep.f32(Lw["conv_ffn_base"])
+    ext = DFlash2Ext(cfg["conv_kernel_size"], cfg["conv_group_size"], cfg["selector_rank"], 0, ap, fp, ab, fb,
+                     keep.q(weights["selector_hidden"]))
+    keep.bufs += [ap, fp, ab, fb]
+    return ext, keep
+
+
+def dflash_draft_ex(target: Model, head: DraftHead, ext: DFlash2Ext, noise_ids, ctx_stacked, pos_ctx, noise_start_pos: int):
+    """The DFlash-2 drafter forward: returns (logits [block, V], sel_h [block, selector_rank])."""
+    ids = np.asarray(noise_ids, np.int32)
+    ctx_stacked = np.ascontiguousarray(ctx_stacked, dtype=np.float32)
+    pos = np.asarray(pos_ctx if len(pos_ctx) else [0], np.int32)
+    logits = np.zeros((head.cfg.block_size, target.cfg.vocab), np.float32)
+    sel_h = np.zeros((head.cfg.block_size, max(ext.selector_rank, 1)), np.float32)
+    rc = lib().orc_dflash_draft_ex(C.byref(target), C.byref(head), C.byref(ext), _p(ids), _p(ctx_stacked), len(pos_ctx),
+                                   _p(pos), noise_start_pos, _p(logits), _p(sel_h))
+    if rc:
+        raise RuntimeError(f"orc_dflash_draft_ex failed: {rc}")
+    return logits, sel_h
 
 
 class TargetState:

@@ -34,6 +34,13 @@
  *       block, side/group indexing against an independent numpy gather)
  *   - DFlash-2 selector walk .......... the known-answer walks of metal_dflash/tests.rs:2978-3094
  *       (scores, first-tie rule, sentinel and non-finite candidates, invalid predecessor)
+ *   - DFlash-2 drafter forward (orc_dflash_draft_ex): the reference has no CPU form of it.  Pinned
+ *       by reduction to the DFlash-1 forward, bit for bit: identity convolutions (zero coefficient
+ *       projections, identity base kernels) reproduce it; a per-channel power-of-two scaling on side 1
+ *       equals the DFlash-1 forward with the matching rows of attn_output / ffn_down scaled (so side 1
+ *       sits on the sublayer outputs, side 0 on their inputs).  Which coefficient tensor feeds which
+ *       convolution (attention pair / FFN pair) follows metal_dflash.rs:16210-16262, 16836-16885 by
+ *       reading only: for that part parity unpinned.
  *   - f64 exp/ln are the host libm's, as the reference's are its platform's:
  *       last-ulp behaviour is parity unpinned (decisions compare against
  *       uniforms and are insensitive to it except with probability ~2^-50).
@@ -284,6 +291,25 @@ int orc_select_draft_path_sampled(const orc_codebook *pred_cb, const orc_codeboo
                                   int32_t carry, size_t n, const int32_t *ids, const float *vals, const float *sel_h,
                                   orc_sampler *proposal, int32_t *out, int32_t *counts, orc_weighted_candidate *cands,
                                   size_t *err_pos);
+
+/* DFlash-2 drafter forward (draft_block_inner with layer.conv and head.selector present,
+ * metal_dflash.rs:16195-16275, 16795-16900, 17003-17030, 17098-17130): per layer, the dynamic
+ * coefficients dyn = conv_proj . (normed sublayer input) serve both sides of a sublayer; side 0
+ * convolves the normed input that q/k/v (gate/up) read, side 1 convolves the sublayer's output
+ * (attn_output / ffn_down) before the residual add.  The tail also returns the selector gate
+ * sel_h = selector_hidden . (output-normed hidden), [block][selector_rank].  ext == NULL is
+ * orc_dflash_draft. */
+typedef struct {
+    int32_t conv_kernel_size, conv_group_size, selector_rank, pad;
+    const orc_qtensor *conv_attn_proj, *conv_ffn_proj; /* [n_layers], each [H -> 2*kernel*H/group] */
+    const float *const *conv_attn_base;                /* [n_layers] -> [2][kernel][H] */
+    const float *const *conv_ffn_base;
+    orc_qtensor selector_hidden;                       /* [H -> rank] */
+} orc_dflash2_ext;
+
+int orc_dflash_draft_ex(const orc_model *target, const orc_draft_head *head, const orc_dflash2_ext *ext,
+                        const int32_t *noise_ids, const float *target_ctx_stacked, size_t ctx_len,
+                        const int32_t *pos_ctx, uint32_t noise_start_pos, float *logits, float *sel_h);
 
 #ifdef __cplusplus
 }

@@ -343,7 +343,18 @@ int orc_target_verify(const orc_model *m, const int32_t *tokens, size_t n, size_
 int orc_dflash_draft(const orc_model *target, const orc_draft_head *head, const int32_t *noise_ids,
                      const float *target_ctx_stacked, size_t ctx_len, const int32_t *pos_ctx,
                      uint32_t noise_start_pos, float *logits) {
+    return orc_dflash_draft_ex(target, head, NULL, noise_ids, target_ctx_stacked, ctx_len, pos_ctx, noise_start_pos, logits,
+                               NULL);
+}
+
+/* forward.rs:380-662, with the DFlash-2 convolutions and selector gate of draft_block_inner
+ * (metal_dflash.rs:16195-16275, 16795-16900, 17003-17030, 17098-17130) when ext is given */
+int orc_dflash_draft_ex(const orc_model *target, const orc_draft_head *head, const orc_dflash2_ext *ext,
+                        const int32_t *noise_ids, const float *target_ctx_stacked, size_t ctx_len,
+                        const int32_t *pos_ctx, uint32_t noise_start_pos, float *logits, float *sel_h) {
     const orc_draft_cfg *c = &head->cfg;
+    const int conv = ext && ext->conv_kernel_size > 0;
+    const size_t ck = conv ? (size_t)ext->conv_kernel_size : 0, cg = conv ? (size_t)ext->conv_group_size : 1;
     size_t n = (size_t)c->block_size, h = (size_t)c->hidden, f = (size_t)c->ffn, hd = (size_t)c->head_dim;
     size_t nq = (size_t)c->n_q, nkv = (size_t)c->n_kv, q_dim = nq * hd, kv_dim = nkv * hd;
     size_t feat = (size_t)c->n_taps * h, V = (size_t)target->cfg.vocab;
@@ -370,11 +381,19 @@ int orc_dflash_draft(const orc_model *target, const orc_draft_head *head, const 
         float *vc = (float *)malloc((ctx_len ? ctx_len : 1) * kv_dim * sizeof(float));
         float *ao = (float *)malloc(n * q_dim * sizeof(float)), *proj = (float *)malloc(n * h * sizeof(float));
         float *g = (float *)malloc(n * f * sizeof(float)), *u = (float *)malloc(n * f * sizeof(float));
+        const size_t dyn_dim = conv ? 2 * ck * (h / cg) : 1;
+        float *dyn = (float *)malloc(n * dyn_dim * sizeof(float)), *cv = (float *)malloc(n * h * sizeof(float));
         for (size_t il = 0; il < (size_t)c->n_layers; il++) {
             const orc_draft_layer *L = &head->layers[il];
             for (size_t i = 0; i < n; i++) orc_rms_norm(x + i * h, L->attn_norm, h, c->eps, nn + i * h);
-            rc |= qmat(&L->wq, nn, q, h, q_dim, n) | qmat(&L->wk, nn, kn, h, kv_dim, n) |
-                  qmat(&L->wv, nn, vn, h, kv_dim, n);
+            const float *src = nn;  /* what q/k/v read */
+            if (conv) {
+                rc |= qmat(&ext->conv_attn_proj[il], nn, dyn, h, dyn_dim, n);
+                orc_dflash2_conv(nn, dyn, ext->conv_attn_base[il], cv, n, h, ck, cg, 0);
+                src = cv;
+            }
+            rc |= qmat(&L->wq, src, q, h, q_dim, n) | qmat(&L->wk, src, kn, h, kv_dim, n) |
+                  qmat(&L->wv, src, vn, h, kv_dim, n);
             if (ctx_len)
                 rc |= qmat(&L->wk, ctx_h, kc, h, kv_dim, ctx_len) | qmat(&L->wv, ctx_h, vc, h, kv_dim, ctx_len);
             for (size_t i = 0; i < n; i++)
@@ -402,15 +421,34 @@ int orc_dflash_draft(const orc_model *target, const orc_draft_head *head, const 
             orc_attn_draft(q, kc, vc, kn, vn, pos_ctx, ctx_len, n, nq, nkv, hd, noise_start_pos, c->causal,
                            L->is_swa ? c->swa_window : 0u, ao);
             rc |= qmat(&L->wo, ao, proj, q_dim, h, n);
-            for (size_t i = 0; i < n * h; i++) x[i] += proj[i];
+            if (conv) {  /* side 1 between attn_output and the residual; same coefficients */
+                orc_dflash2_conv(proj, dyn, ext->conv_attn_base[il], cv, n, h, ck, cg, 1);
+                for (size_t i = 0; i < n * h; i++) x[i] += cv[i];
+            } else {
+                for (size_t i = 0; i < n * h; i++) x[i] += proj[i];
+            }
             for (size_t i = 0; i < n; i++) orc_rms_norm(x + i * h, L->post_norm, h, c->eps, nn + i * h);
-            rc |= qmat(&L->gate, nn, g, h, f, n) | qmat(&L->up, nn, u, h, f, n);
+            src = nn;  /* what gate/up read */
+            if (conv) {
+                rc |= qmat(&ext->conv_ffn_proj[il], nn, dyn, h, dyn_dim, n);
+                orc_dflash2_conv(nn, dyn, ext->conv_ffn_base[il], cv, n, h, ck, cg, 0);
+                src = cv;
+            }
+            rc |= qmat(&L->gate, src, g, h, f, n) | qmat(&L->up, src, u, h, f, n);
             for (size_t i = 0; i < n * f; i++) g[i] = orc_silu(g[i]) * u[i];
             rc |= qmat(&L->down, g, proj, f, h, n);
-            for (size_t i = 0; i < n * h; i++) x[i] += proj[i];
+            if (conv) {
+                orc_dflash2_conv(proj, dyn, ext->conv_ffn_base[il], cv, n, h, ck, cg, 1);
+                for (size_t i = 0; i < n * h; i++) x[i] += cv[i];
+            } else {
+                for (size_t i = 0; i < n * h; i++) x[i] += proj[i];
+            }
         }
         for (size_t i = 0; i < n; i++) orc_rms_norm(x + i * h, head->output_norm, h, c->eps, nn + i * h);
         rc |= qmat(&target->output, nn, logits, h, V, n);
+        if (ext && sel_h && ext->selector_rank > 0) rc |= qmat(&ext->selector_hidden, nn, sel_h, h, (size_t)ext->selector_rank, n);
+        free(dyn);
+        free(cv);
         free(q);
         free(kn);
         free(vn);

@@ -374,6 +374,12 @@ struct dflash_draft_session {
     float *g = nullptr, *u = nullptr, *logits = nullptr, *tmp = nullptr;
     float *pk = nullptr;  // [16][max(q_dim + 2 kv_dim, 2 ffn)]: output of a fused q/k/v or gate/up GEMM
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
+    // DFlash-2 (MetalDFlashSession conv_buf / conv_dyn_* / topk_* / sel_h, metal_dflash.rs:5144-5155)
+    float *conv_buf = nullptr;   // [16][H]
+    float *conv_dyn = nullptr;   // [16][2 * kernel * H / group]: one sublayer's coefficients at a time
+    int32_t *topk_ids = nullptr; // [16][16]
+    float *topk_vals = nullptr;  // [16][16]
+    float *sel_h = nullptr;      // [16][selector_rank]
 };
 
 extern "C" {
@@ -614,6 +620,12 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
     if (cfg->n_layers < 1 || cfg->block_size < 1 || cfg->block_size > 16 || cfg->n_q % cfg->n_kv ||
         (cfg->head_dim != 64 && cfg->head_dim != 128 && cfg->head_dim != 256) || cfg->n_taps < 1 || ctx_capacity < 1)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "draft_session_create: unsupported drafter shape");
+    // DFlash-2 walls (loader.rs:1047-1057; the selector reads the top-16 kernel's output, so top_k = 16)
+    if (cfg->conv_kernel_size < 0 || cfg->conv_kernel_size > 8 || cfg->selector_rank < 0 || cfg->selector_rank > 1024 ||
+        (cfg->conv_kernel_size > 0 && (cfg->conv_group_size < 1 || cfg->hidden % cfg->conv_group_size)) ||
+        (cfg->selector_rank > 0 && cfg->selector_top_k != 16))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "draft_session_create: unsupported DFlash-2 shape (kernel %d group %d rank %d top_k %d)",
+                        cfg->conv_kernel_size, cfg->conv_group_size, cfg->selector_rank, cfg->selector_top_k);
     dflash_draft_session *s = new (std::nothrow) dflash_draft_session();
     if (!s) return DFLASH_ERR_HIP;
     s->cfg = *cfg;
@@ -633,6 +645,12 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
               dev_alloc(&s->pk, 16 * std::max(q_dim + 2 * kv_dim, 2 * static_cast<size_t>(cfg->ffn))) &&
               dev_alloc(&s->tmp, 16 * std::max(H, kv_dim)) && dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) &&
               dev_alloc(&s->argmax, 16);
+    if (ok && cfg->conv_kernel_size > 0)
+        ok = dev_alloc(&s->conv_buf, 16 * H) &&
+             dev_alloc(&s->conv_dyn, 16 * static_cast<size_t>(2) * cfg->conv_kernel_size * (H / cfg->conv_group_size));
+    if (ok && cfg->selector_rank > 0)
+        ok = dev_alloc(&s->topk_ids, 16 * 16) && dev_alloc(&s->topk_vals, 16 * 16) &&
+             dev_alloc(&s->sel_h, 16 * static_cast<size_t>(cfg->selector_rank));
     if (!ok) {
         dflash_draft_session_destroy(s);
         return dfl_fail(ctx, DFLASH_ERR_HIP, "draft_session_create: out of device memory");
@@ -644,7 +662,8 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
 void dflash_draft_session_destroy(dflash_draft_session *s) {
     if (!s) return;
     void *ptrs[] = {s->ctx_raw, s->ctx_h, s->k_ctx, s->v_ctx, s->k16, s->vt16, s->pos_ctx, s->x, s->cur, s->q, s->k, s->v,
-                    s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax, s->pk};
+                    s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax, s->pk,
+                    s->conv_buf, s->conv_dyn, s->topk_ids, s->topk_vals, s->sel_h};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;
@@ -763,6 +782,15 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
     // mirror is only kept current while that holds, so leaving the fast path is final.
     const bool fast = s->contiguous && noise_start == s->ctx_len && c.n_q / c.n_kv <= 16;
     if (!fast) s->contiguous = false;
+    const bool conv = c.conv_kernel_size > 0;
+    const int64_t conv_dyn_dim = conv ? static_cast<int64_t>(2) * c.conv_kernel_size * (H / c.conv_group_size) : 0;
+    if (conv)
+        for (int il = 0; il < c.n_layers; il++)
+            if (!head->layers[il].conv_attn_proj.data || !head->layers[il].conv_ffn_proj.data || !head->layers[il].conv_attn_base ||
+                !head->layers[il].conv_ffn_base)
+                return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_block: layer %d lacks its convolution tensors", il);
+    if (c.selector_rank > 0 && (!head->selector_hidden.data || !head->selector_predecessor.data || !head->selector_successor.data))
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_block: the head lacks its selector tensors");
 
     // phase 1 and the context K/V of the new columns (a no-op if dflash_draft_prepare_ctx ran)
     if ((rc = draft_prepare(ctx, head, s, fast, st))) return rc;
@@ -782,8 +810,18 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
         _Float16 *k16 = s->k16 + il * static_cast<size_t>(s->cap16) * kv_dim;
         _Float16 *vt16 = s->vt16 + il * static_cast<size_t>(s->cap16) * kv_dim;
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
+        // DFlash-2 attention convolution (metal_dflash.rs:16210-16262): the dynamic coefficients come
+        // from the normed input and serve both sides; q/k/v read the side-0 result
+        const float *attn_src = s->cur;
+        if (conv) {
+            if ((rc = gemm(ctx, L.conv_attn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st))) return rc;
+            if ((rc = dflash_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_attn_base, s->conv_buf, N, H, c.conv_kernel_size,
+                                          c.conv_group_size, 0, st)))
+                return rc;
+            attn_src = s->conv_buf;
+        }
         bool packed;  // only on the fast path: the general attention kernel reads V dense
-        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st))) return rc;
+        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, attn_src, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st))) return rc;
         const int64_t tot = q_dim + 2 * kv_dim;
         qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(
             packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
@@ -803,16 +841,51 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                                                             L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
         }
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st))) return rc;
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps, nullptr, nullptr);  // x += mix first
-        if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, N, st))) return rc;
+        // residual 1 (x += attn_output; DFlash-2: its side-1 convolution, same coefficients, :16795-16820),
+        // folded into the norm that follows
+        const float *resid = s->mix;
+        if (conv) {
+            if ((rc = dflash_dflash2_conv(ctx, s->mix, s->conv_dyn, L.conv_attn_base, s->conv_buf, N, H, c.conv_kernel_size,
+                                          c.conv_group_size, 1, st)))
+                return rc;
+            resid = s->conv_buf;
+        }
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, resid, L.post_norm, s->cur, H, c.eps, nullptr, nullptr);
+        const float *ffn_src = s->cur;
+        if (conv) {  // the FFN pair (:16836-16885, 17003-17022)
+            if ((rc = gemm(ctx, L.conv_ffn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st))) return rc;
+            if ((rc = dflash_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_ffn_base, s->conv_buf, N, H, c.conv_kernel_size,
+                                          c.conv_group_size, 0, st)))
+                return rc;
+            ffn_src = s->conv_buf;
+        }
+        if ((rc = gemm_gate_up(ctx, L.gate, L.up, ffn_src, s->g, s->u, s->pk, H, c.ffn, N, st))) return rc;
         if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st))) return rc;
-        add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(N) * H);
+        resid = s->mix;
+        if (conv) {
+            if ((rc = dflash_dflash2_conv(ctx, s->mix, s->conv_dyn, L.conv_ffn_base, s->conv_buf, N, H, c.conv_kernel_size,
+                                          c.conv_group_size, 1, st)))
+                return rc;
+            resid = s->conv_buf;
+        }
+        add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, resid, static_cast<size_t>(N) * H);
     }
     rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, head->output_norm, s->cur, H, c.eps, nullptr, nullptr);
     float *lg = draft_logits ? draft_logits : s->logits;
     if ((rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st))) return rc;
     int32_t *am = draft_argmax ? draft_argmax : s->argmax;
-    if ((rc = dflash_argmax_greedy(ctx, lg, N, V, V, am, st))) return rc;
+    if (c.selector_rank > 0) {
+        // DFlash-2 tail (:17098-17130, select_draft_path :17176-17251): the 16 best candidates of every
+        // row, the selector gate W_h . h of the output-normed hidden, and the predecessor-conditioned
+        // walk, all on the device
+        if ((rc = dflash_top16(ctx, lg, N, V, V, s->topk_ids, s->topk_vals, st))) return rc;
+        if ((rc = gemm(ctx, head->selector_hidden, s->cur, s->sel_h, H, c.selector_rank, N, st))) return rc;
+        if ((rc = dflash_select_draft_path(ctx, &head->selector_predecessor, &head->selector_successor, c.selector_rank,
+                                           c.selector_top_k, carry, N, s->topk_ids, s->topk_vals, s->sel_h, am, nullptr, st)))
+            return rc;
+    } else if ((rc = dflash_argmax_greedy(ctx, lg, N, V, V, am, st))) {
+        return rc;
+    }
     DFL_HIP_CHECK(ctx, hipGetLastError());
     // watermarks advance only once everything was enqueued without error (metal_dflash.rs:17143-17150)
     s->ctx_h_ready = s->ctx_len;

@@ -14,7 +14,7 @@ from dataclasses import asdict, dataclass
 import numpy as np
 
 from . import synth
-from .binding import Context, DFlashError, _stream_ptr, _torch, lib
+from .binding import CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
 
 
 @dataclass
@@ -51,6 +51,11 @@ class DraftConfig:
     swa_window: int = 0
     eps: float = 1e-6
     rope_theta: float = 1e6
+    # DFlash-2 (loader.rs:367-376): all zero for a DFlash-1 drafter
+    conv_kernel_size: int = 0
+    conv_group_size: int = 0
+    selector_rank: int = 0
+    selector_top_k: int = 0
 
     def as_dict(self):
         return asdict(self)
@@ -81,18 +86,22 @@ class ModelC(C.Structure):
 class DraftCfgC(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "n_q", "n_kv", "head_dim", "ffn", "block_size", "n_taps",
                                           "causal")] + \
-               [("swa_window", C.c_uint32), ("eps", C.c_float), ("rope_theta", C.c_float)]
+               [("swa_window", C.c_uint32), ("eps", C.c_float), ("rope_theta", C.c_float)] + \
+               [(n, C.c_int32) for n in ("conv_kernel_size", "conv_group_size", "selector_rank", "selector_top_k")]
 
 
 class DraftLayerC(C.Structure):
     _fields_ = [("attn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("post_norm", C.c_void_p),
                 ("wq", QTensorC), ("wk", QTensorC), ("wv", QTensorC), ("wo", QTensorC), ("gate", QTensorC),
-                ("up", QTensorC), ("down", QTensorC), ("is_swa", C.c_int32), ("pad", C.c_int32)]
+                ("up", QTensorC), ("down", QTensorC), ("is_swa", C.c_int32), ("pad", C.c_int32),
+                ("conv_attn_proj", QTensorC), ("conv_ffn_proj", QTensorC), ("conv_attn_base", C.c_void_p),
+                ("conv_ffn_base", C.c_void_p)]
 
 
 class DraftHeadC(C.Structure):
     _fields_ = [("cfg", DraftCfgC), ("layers", C.POINTER(DraftLayerC)), ("fc", QTensorC), ("hidden_norm", C.c_void_p),
-                ("output_norm", C.c_void_p)]
+                ("output_norm", C.c_void_p), ("selector_hidden", QTensorC), ("selector_predecessor", CodebookC),
+                ("selector_successor", CodebookC)]
 
 
 _declared = False
@@ -173,7 +182,8 @@ def synth_target_weights(cfg: ModelConfig, seed: int, wtype: int = synth.Q4_K, e
     return w
 
 
-def synth_draft_weights(cfg: DraftConfig, seed: int, wtype: int = synth.Q4_K, swa_layers=()):
+def synth_draft_weights(cfg: DraftConfig, seed: int, wtype: int = synth.Q4_K, swa_layers=(), vocab=None,
+                        codebook_type: int = synth.Q4_K):
     rng = np.random.default_rng(seed + 7919)
     q_dim, kv_dim = cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
     s = seed * 1000003 + 500000
@@ -188,6 +198,23 @@ def synth_draft_weights(cfg: DraftConfig, seed: int, wtype: int = synth.Q4_K, sw
             "wv": _mat(wtype, kv_dim, cfg.hidden, b + 3), "wo": _mat(wtype, cfg.hidden, q_dim, b + 4),
             "gate": _mat(wtype, cfg.ffn, cfg.hidden, b + 5), "up": _mat(wtype, cfg.ffn, cfg.hidden, b + 6),
             "down": _mat(wtype, cfg.hidden, cfg.ffn, b + 7), "is_swa": int(il in swa_layers)})
+        if cfg.conv_kernel_size:
+            dyn_dim = 2 * cfg.conv_kernel_size * (cfg.hidden // cfg.conv_group_size)
+            L = w["layers"][-1]
+            L["conv_attn_proj"] = _mat(wtype, dyn_dim, cfg.hidden, b + 8)
+            L["conv_ffn_proj"] = _mat(wtype, dyn_dim, cfg.hidden, b + 9)
+            # base kernels near the identity tap (tap 0 about 1, the others small), f32 [2][kernel][hidden]
+            for name in ("conv_attn_base", "conv_ffn_base"):
+                base = (0.1 * rng.standard_normal((2, cfg.conv_kernel_size, cfg.hidden))).astype(np.float32)
+                base[:, 0, :] += 1.0
+                L[name] = base
+    if cfg.selector_rank:
+        if vocab is None:
+            raise ValueError("a DFlash-2 selector needs the target vocabulary size")
+        w["selector_hidden"] = _mat(wtype, cfg.selector_rank, cfg.hidden, s + 2)
+        # per-token predecessor / successor tables [vocab][rank]
+        w["selector_predecessor"] = (codebook_type, synth.random_weight(codebook_type, vocab, cfg.selector_rank, s + 3, std=1.0))
+        w["selector_successor"] = (codebook_type, synth.random_weight(codebook_type, vocab, cfg.selector_rank, s + 4, std=1.0))
     return w
 
 
@@ -409,8 +436,17 @@ class DraftHead:
                 if k not in grouped:
                     setattr(L, k, up.q(Lw[k]))
             L.is_swa = int(Lw.get("is_swa", 0))
+            if cfg.conv_kernel_size:
+                L.conv_attn_proj, L.conv_ffn_proj = up.q(Lw["conv_attn_proj"]), up.q(Lw["conv_ffn_proj"])
+                L.conv_attn_base, L.conv_ffn_base = up.f32(Lw["conv_attn_base"]), up.f32(Lw["conv_ffn_base"])
         self.c = DraftHeadC(DraftCfgC(**cfg.as_dict()), self._layers, up.q(weights["fc"]), up.f32(weights["hidden_norm"]),
                             up.f32(weights["output_norm"]))
+        if cfg.selector_rank:
+            self.c.selector_hidden = up.q(weights["selector_hidden"])
+            for name in ("selector_predecessor", "selector_successor"):
+                qtype, rows = weights[name]
+                t = up.q((qtype, rows))
+                setattr(self.c, name, CodebookC(int(qtype), 0, int(rows.shape[0]), t.data))
 
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self._up.keep)

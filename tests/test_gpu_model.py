@@ -222,6 +222,94 @@ def test_separate_and_adjacent_weight_layouts_agree(ctx, oracle, wtype):
     close(outs["adjacent"][2], outs["separate"][2], "adjacent vs separate draft logits")
 
 
+@pytest.mark.parametrize("codebook_type", [dfl.TYPE_Q4_K, dfl.TYPE_Q8_0])
+def test_dflash2_draft_block_matches_oracle(ctx, oracle, target, codebook_type):
+    """A DFlash-2 head (two-tap dynamic convolutions around both sublayers, block of 8, selector of rank
+    256 over the top-16 candidates; metal_dflash.rs:16210-16262, 16795-16885, 17003-17022, 17098-17251)
+    against the oracle's restatement: logits to the stack tolerance; the tokens of the device-side walk
+    are checked along the DEVICE's own path (each pick conditions the next): every pick is one of that
+    row's top-16 and its score, recomputed from the oracle's selector gate and codebook rows, is the best
+    of the row up to the logit error."""
+    model, (omodel, _keep) = target
+    dcfg = dfl.DraftConfig(**{**D1.as_dict(), "block_size": 8, "conv_kernel_size": 2, "conv_group_size": 64,
+                              "selector_rank": 256, "selector_top_k": 16})
+    dw = dfl.synth_draft_weights(dcfg, seed=9, vocab=C1.vocab, codebook_type=codebook_type)
+    head = dfl.DraftHead(ctx, dcfg, dw)
+    ohead, _k2 = oracle.build_draft_head(dcfg.as_dict(), dw)
+    ext, _k3 = oracle.build_dflash2_ext(dcfg.as_dict(), dw)
+    pred_cb, _k4 = oracle.make_codebook(codebook_type, dw["selector_predecessor"][1], 256)
+    succ_cb, _k5 = oracle.make_codebook(codebook_type, dw["selector_successor"][1], 256)
+    rng = np.random.default_rng(31)
+    cap = 64
+    sess = dfl.Session(ctx, model, cap, TAPS)
+    ostate = oracle.TargetState(C1.as_dict(), cap)
+    dsess = dfl.DraftSession(ctx, head, model, cap)
+    mask_token = C1.vocab - 1
+    hidden_o, pos = [], 0
+    for n_new in (24, 5):
+        toks = rng.integers(0, C1.vocab, n_new).tolist()
+        for s0 in range(0, n_new, 16):
+            blk = toks[s0:s0 + 16]
+            out = sess.encode_packed_verify_layer_major(blk, pos)
+            dsess.append_target_ctx_columns(out.hidden_capture, list(range(pos, pos + len(blk))))
+            hidden_o.append(oracle.target_verify(omodel, ostate, blk, pos, TAPS)[1])
+            pos += len(blk)
+        carry = int(rng.integers(0, C1.vocab))
+        tokens_dev, logits, host = dsess.draft_block(carry, mask_token, pos, want_logits=True)
+        ctx_o = np.concatenate(hidden_o).reshape(pos, -1)
+        want, sel_h = oracle.dflash_draft_ex(omodel, ohead, ext, [carry] + [mask_token] * 7, ctx_o, list(range(pos)), pos)
+        lg = logits.cpu().numpy()
+        # two more f16-operand GEMMs per sublayer (the coefficient projections) whose outputs multiply the
+        # activations: the stack bound is widened accordingly (DFlash-1 on this shape: l2 about 3e-3)
+        close(lg, want, f"dflash2 draft logits ctx={pos}", tol=5e-2, l2_tol=8e-3)
+        assert host == tokens_dev.cpu().tolist()
+        ids_d, vals_d = ctx.top16(logits)
+        ids_d, vals_d = ids_d.cpu().numpy(), vals_d.cpu().numpy()
+        assert host[0] == ids_d[0][0]
+        rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+        prev = carry
+        for p in range(1, 8):
+            gate = oracle.codebook_row(pred_cb, prev).astype(np.float64) * sel_h[p].astype(np.float64)
+            scores = np.array([vals_d[p][b] + float(gate @ oracle.codebook_row(succ_cb, int(ids_d[p][b])).astype(np.float64))
+                               for b in range(16)])
+            assert host[p] in ids_d[p].tolist(), f"position {p}: pick {host[p]} is not a top-16 candidate"
+            mine = scores[ids_d[p].tolist().index(host[p])]
+            assert mine >= scores.max() - 4e-2 * rms, f"position {p}: pick scores {mine}, best {scores.max()}"
+            prev = host[p]
+    dsess.close()
+    sess.close()
+
+
+def test_dflash2_identity_convolutions_equal_dflash1_on_the_device(ctx, target):
+    """With zero coefficient projections and identity base kernels every convolution returns its input bit
+    for bit, so the DFlash-2 launches must reproduce the DFlash-1 drafter's logits exactly: the convolutions
+    sit where the reference puts them and touch nothing else."""
+    model, _ = target
+    d1 = dfl.DraftConfig(**{**D1.as_dict(), "block_size": 8})
+    d2 = dfl.DraftConfig(**{**d1.as_dict(), "conv_kernel_size": 2, "conv_group_size": 64})
+    dw = dfl.synth_draft_weights(d2, seed=9)
+    ident = {**dw, "layers": []}
+    for L in dw["layers"]:
+        base = np.zeros((2, 2, d2.hidden), np.float32)
+        base[:, 0, :] = 1.0
+        zero = (L["conv_attn_proj"][0], np.zeros_like(L["conv_attn_proj"][1]))
+        ident["layers"].append({**L, "conv_attn_proj": zero, "conv_ffn_proj": zero, "conv_attn_base": base, "conv_ffn_base": base})
+    rng = np.random.default_rng(2)
+    toks = rng.integers(0, C1.vocab, 16).tolist()
+    got = []
+    for cfg, w in ((d1, dw), (d2, ident)):
+        head = dfl.DraftHead(ctx, cfg, w)
+        sess = dfl.Session(ctx, model, 64, TAPS)
+        dsess = dfl.DraftSession(ctx, head, model, 64)
+        out = sess.encode_packed_verify_layer_major(toks, 0)
+        dsess.append_target_ctx_columns(out.hidden_capture, list(range(16)))
+        _, logits, _ = dsess.draft_block(11, C1.vocab - 1, 16, want_logits=True)
+        got.append(logits.cpu().numpy())
+        dsess.close()
+        sess.close()
+    assert np.array_equal(got[0].view(np.uint32), got[1].view(np.uint32))
+
+
 MOE_CASES = {
     # hidden 512: 16 sub-blocks per row (half-wave rows); hidden 2048 / F_exp 768: the end-to-end shape's widths
     "small": dfl.ModelConfig(n_layers=2, hidden=512, n_q=8, n_kv=2, head_dim=64, ffn=0, vocab=4096, n_expert=16,

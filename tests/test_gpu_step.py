@@ -111,6 +111,29 @@ def test_generate_greedy_equals_serial_greedy(ctx, world, margin, partial):
     dec.close()
 
 
+def test_generate_with_a_dflash2_head_equals_serial_greedy(ctx, world):
+    """The step loop with a DFlash-2 drafter (blocks of 8, convolutions, selector walk on the device): whatever
+    the selector proposes, the emitted tokens are the target's serial greedy decode."""
+    cont = world["cont"]
+    undecided = np.flatnonzero(~world["decided"])
+    n_tok = int(min(40, undecided[0] if len(undecided) else 40))
+    d2 = dfl.DraftConfig(**{**D1.as_dict(), "block_size": 8, "conv_kernel_size": 2, "conv_group_size": 64,
+                            "selector_rank": 64, "selector_top_k": 16})
+    head = dfl.DraftHead(ctx, d2, dfl.synth_draft_weights(d2, seed=5, vocab=C1.vocab, codebook_type=dfl.TYPE_Q8_0))
+    dec = dfl.SpeculativeDecoder(ctx, world["model"], head, TAPS, 256, MASK)
+    first = dec.prefill(world["prompt"])
+
+    def override(tokens, position):  # the block has 7 drafts
+        done = len(tokens)
+        if (position // 3) % 2 == 0:
+            return cont[done:done + 4] + [-1] * 3
+        return None
+    tokens, stats = dec.generate(first, n_tok, draft_override_fn=override)
+    assert tokens == cont[:n_tok]
+    assert stats["accepted_drafts"] > 0 and stats["spec_steps"] >= n_tok // 8
+    dec.close()
+
+
 def test_generate_sampled_equals_serial_sampler(ctx, world, oracle):
     """Deterministic-proposal coupling == serial sampling with the same stream (sampling.rs:2837-2865).
     The serial stream is the CPU oracle's sampler applied to the logits of a token-by-token pass through
