@@ -392,6 +392,13 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
                            dflash_draft_session *s, int32_t carry_token, int32_t mask_token, int64_t noise_start_pos,
                            int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream);
 
+/* The selector inputs the last draft block of a DFlash-2 head left in the session
+ * (MetalDFlashSession::topk_ids / topk_vals / sel_h, metal_dflash.rs:5150-5155), copied to the
+ * caller's device buffers: [block][16] i32, [block][16] f32, [block][selector_rank] f32 (any may be
+ * NULL).  Enqueue-only.  DFLASH_ERR_STATE for a DFlash-1 session. */
+int32_t dflash_draft_session_selector_inputs(dflash_ctx *ctx, const dflash_draft_session *s, int32_t *topk_ids,
+                                             float *topk_vals, float *sel_h, dflash_stream_t stream);
+
 /* ---- one speculative transition -----------------------------------------------------------
  * The body of the generation loop of crates/qwen-cli/src/qwen/dflash.rs:700-1241: draft a block
  * from `carry` at `position`, verify [carry, drafts...] in one packed pass, accept a prefix,
@@ -407,8 +414,12 @@ int32_t dflash_accept_greedy(const int32_t *verify_input_host, const int32_t *ve
 
 typedef struct {
     int32_t mask_token;
-    int32_t sampled_mode;           /* 0: greedy argmax accept; 1: sampler-coupled accept of the drafter's argmax
-                                       (couple_deterministic_proposal), logits stay on the device */
+    int32_t sampled_mode;           /* 0: greedy argmax accept; 1: sampler-coupled accept of the drafter's greedy
+                                       tokens (couple_deterministic_proposal), logits stay on the device; 2: a
+                                       DFlash-2 head drafts by the sampled selector walk (draft_block_sampled,
+                                       metal_dflash.rs:17268-17415) with proposal_sampler and the target's sampler
+                                       is coupled to the walk's candidate distributions (couple_sparse_proposal;
+                                       qwen/dflash.rs:508-519, 706-716) */
     float fallback_margin;          /* greedy only: replay when a committed row's packed top-2 gap is below this
                                        (DFLASH_VERIFY_FALLBACK_MARGIN_DEFAULT = 0.1); <= 0 disables */
     int32_t fallback_partial;       /* 1: keep rows before the first flagged row (QWEN_DFLASH_VERIFY_FALLBACK_PARTIAL) */
@@ -427,13 +438,15 @@ typedef struct {
 
 /* draft_override_host (may be NULL): block_size-1 token ids replacing the drafter's proposals for slots
  * 1.. (entries < 0 keep the drafter's token): the loop's prefix-replay drafts (qwen/dflash.rs:700-712).
- * sampler is required when sampled_mode != 0.  Blocking. */
+ * sampler is required when sampled_mode != 0, proposal_sampler (temperature only, its seed the
+ * target's ^ 0x4446_4c41_5348_3251 in the reference) when sampled_mode == 2, which takes no override.
+ * Blocking. */
 int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
                          dflash_session *session, dflash_draft_session *draft_session,
                          const int32_t *tap_layers_host, int32_t n_taps, int32_t carry_token, int64_t position,
-                         const dflash_step_cfg *cfg, dflash_sampler *sampler, int64_t remaining_output_budget,
-                         const int32_t *stop_ids_host, int32_t n_stop, const int32_t *draft_override_host,
-                         dflash_step_result *out_host, dflash_stream_t stream);
+                         const dflash_step_cfg *cfg, dflash_sampler *sampler, dflash_sampler *proposal_sampler,
+                         int64_t remaining_output_budget, const int32_t *stop_ids_host, int32_t n_stop,
+                         const int32_t *draft_override_host, dflash_step_result *out_host, dflash_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -752,6 +752,20 @@ int32_t draft_prepare(dflash_ctx *ctx, const dflash_draft_head *head, dflash_dra
 
 }  // namespace
 
+int32_t dflash_draft_session_selector_inputs(dflash_ctx *ctx, const dflash_draft_session *s, int32_t *topk_ids,
+                                             float *topk_vals, float *sel_h, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "selector_inputs: null session");
+    if (!s->sel_h) return dfl_fail(ctx, DFLASH_ERR_STATE, "selector_inputs: the session's drafter has no selector");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t n = s->cfg.block_size;
+    if (topk_ids) DFL_HIP_CHECK(ctx, hipMemcpyAsync(topk_ids, s->topk_ids, n * 16 * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+    if (topk_vals) DFL_HIP_CHECK(ctx, hipMemcpyAsync(topk_vals, s->topk_vals, n * 16 * sizeof(float), hipMemcpyDeviceToDevice, st));
+    if (sel_h)
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(sel_h, s->sel_h, n * s->cfg.selector_rank * sizeof(float), hipMemcpyDeviceToDevice, st));
+    return DFLASH_OK;
+}
+
 int32_t dflash_draft_prepare_ctx(dflash_ctx *ctx, const dflash_draft_head *head, dflash_draft_session *s, dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_prepare_ctx: null argument");
@@ -760,9 +774,26 @@ int32_t dflash_draft_prepare_ctx(dflash_ctx *ctx, const dflash_draft_head *head,
     return draft_prepare(ctx, head, s, s->contiguous && head->cfg.n_q / head->cfg.n_kv <= 16, static_cast<hipStream_t>(stream));
 }
 
+namespace {
+int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head, dflash_draft_session *s,
+                         int32_t carry, int32_t mask_token, int64_t noise_start, int32_t *draft_argmax, float *draft_logits,
+                         int32_t *argmax_host, dflash_stream_t stream, bool skip_selector_walk);
+}
+
 int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
                            dflash_draft_session *s, int32_t carry, int32_t mask_token, int64_t noise_start,
                            int32_t *draft_argmax, float *draft_logits, int32_t *argmax_host, dflash_stream_t stream) {
+    return draft_block_impl(ctx, target, head, s, carry, mask_token, noise_start, draft_argmax, draft_logits, argmax_host, stream,
+                            false);
+}
+
+namespace {
+
+// skip_selector_walk (DFlash-2 heads): stop after the top-16 candidates and the selector gate are in
+// the session's buffers; the caller walks the lattice itself (the sampled walk of a speculative step).
+int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head, dflash_draft_session *s,
+                         int32_t carry, int32_t mask_token, int64_t noise_start, int32_t *draft_argmax, float *draft_logits,
+                         int32_t *argmax_host, dflash_stream_t stream, bool skip_selector_walk) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!target || !head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_block: null argument");
     const dflash_draft_cfg &c = head->cfg;
@@ -880,7 +911,8 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
         // walk, all on the device
         if ((rc = dflash_top16(ctx, lg, N, V, V, s->topk_ids, s->topk_vals, st))) return rc;
         if ((rc = gemm(ctx, head->selector_hidden, s->cur, s->sel_h, H, c.selector_rank, N, st))) return rc;
-        if ((rc = dflash_select_draft_path(ctx, &head->selector_predecessor, &head->selector_successor, c.selector_rank,
+        if (!skip_selector_walk &&
+            (rc = dflash_select_draft_path(ctx, &head->selector_predecessor, &head->selector_successor, c.selector_rank,
                                            c.selector_top_k, carry, N, s->topk_ids, s->topk_vals, s->sel_h, am, nullptr, st)))
             return rc;
     } else if ((rc = dflash_argmax_greedy(ctx, lg, N, V, V, am, st))) {
@@ -896,6 +928,8 @@ int32_t dflash_draft_block(dflash_ctx *ctx, const dflash_model *target, const df
     }
     return DFLASH_OK;
 }
+
+}  // namespace
 
 int32_t dflash_accept_greedy(const int32_t *verify_input, const int32_t *verify_argmax, int32_t n, int64_t budget,
                              const int32_t *stop_ids, int32_t n_stop, dflash_accept_decision *out) {
@@ -1050,12 +1084,17 @@ int32_t margin_fallback(dflash_ctx *ctx, const dflash_model *target, dflash_sess
 
 int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head, dflash_session *sess,
                          dflash_draft_session *dsess, const int32_t *taps, int32_t n_taps, int32_t carry, int64_t position,
-                         const dflash_step_cfg *cfg, dflash_sampler *sampler, int64_t budget, const int32_t *stop_ids,
-                         int32_t n_stop, const int32_t *draft_override, dflash_step_result *res, dflash_stream_t stream) {
+                         const dflash_step_cfg *cfg, dflash_sampler *sampler, dflash_sampler *proposal_sampler, int64_t budget,
+                         const int32_t *stop_ids, int32_t n_stop, const int32_t *draft_override, dflash_step_result *res,
+                         dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!target || !head || !sess || !dsess || !cfg || !res || (n_stop > 0 && !stop_ids) || budget < 0)
         return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "spec_step: null or invalid argument");
     if (cfg->sampled_mode != 0 && !sampler) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "spec_step: sampled mode needs a sampler");
+    const bool sampled_drafts = cfg->sampled_mode == 2;
+    if (sampled_drafts && (!proposal_sampler || head->cfg.selector_rank <= 0 || draft_override))
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT,
+                        "spec_step: sampled drafting needs a selector head and a proposal sampler, and takes no draft override");
     if (n_taps != head->cfg.n_taps || n_taps > sess->n_taps || !taps)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "spec_step: %d tapped layers, the drafter expects %d", n_taps, head->cfg.n_taps);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1065,9 +1104,22 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
     int32_t rc;
 
     auto t0 = std::chrono::steady_clock::now();
-    if ((rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, nullptr, nullptr,
-                                 res->draft_tokens, st)))
+    int32_t prop_counts[16] = {0};
+    dflash_weighted_candidate prop_cands[16 * 16];
+    if (sampled_drafts) {
+        // draft_block_sampled (metal_dflash.rs:17268-17415): the drafter up to its top-16 and selector gate,
+        // then the walk that draws every position from softmax(score / T) with the proposal sampler
+        if ((rc = draft_block_impl(ctx, target, head, dsess, carry, cfg->mask_token, position, nullptr, nullptr, nullptr, st, true)))
+            return rc;
+        if ((rc = dflash_select_draft_path_sampled(ctx, &head->selector_predecessor, &head->selector_successor,
+                                                   head->cfg.selector_rank, head->cfg.selector_top_k, carry, N, dsess->topk_ids,
+                                                   dsess->topk_vals, dsess->sel_h, proposal_sampler, res->draft_tokens, prop_counts,
+                                                   prop_cands, st)))
+            return rc;
+    } else if ((rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, nullptr, nullptr,
+                                        res->draft_tokens, st))) {
         return rc;
+    }
     res->draft_ms = ms_since(t0);
     res->draft_tokens[0] = carry;
     if (draft_override)
@@ -1083,7 +1135,15 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
     res->verify_ms = ms_since(t0);
 
     t0 = std::chrono::steady_clock::now();
-    if (cfg->sampled_mode != 0) {
+    if (sampled_drafts) {  // couple_sparse_proposal with the walk's candidate distributions
+        // the walk leaves row r's candidates at r * top_k; the decision takes the rows back to back
+        const int top_k = head->cfg.selector_top_k;
+        int n_packed = 0;
+        for (int r = 0; r < N - 1; r++)
+            for (int i = 0; i < prop_counts[r]; i++) prop_cands[n_packed++] = prop_cands[r * top_k + i];
+        rc = dflash_accept_prefix(ctx, verify_input, N, sess->logits, target->cfg.vocab, 1, N - 1, verify_input + 1, prop_counts,
+                                  prop_cands, nullptr, 0.0f, sampler, budget, stop_ids, n_stop, &res->decision, st);
+    } else if (cfg->sampled_mode != 0) {
         rc = dflash_accept_prefix(ctx, verify_input, N, sess->logits, target->cfg.vocab, 0, 0, nullptr, nullptr, nullptr,
                                   nullptr, 0.0f, sampler, budget, stop_ids, n_stop, &res->decision, st);
     } else {

@@ -488,6 +488,22 @@ class DraftSession:
         self.ctx._check(self._L.dflash_draft_append_ctx(self.ctx._h, self._h, hc.data_ptr() if n else None, n, pos,
                                                         _stream_ptr()))
 
+    def selector_inputs(self):
+        """(topk_ids [block, 16] i32, topk_vals [block, 16] f32, sel_h [block, rank] f32) of the last draft block of a
+        DFlash-2 head, copied off the session's buffers."""
+        torch = _torch()
+        L = self._L
+        L.dflash_draft_session_selector_inputs.restype = C.c_int32
+        L.dflash_draft_session_selector_inputs.argtypes = [C.c_void_p] * 6
+        n, rank = self.head.cfg.block_size, self.head.cfg.selector_rank
+        dev = f"cuda:{self.ctx.device}"
+        ids = torch.empty((n, 16), dtype=torch.int32, device=dev)
+        vals = torch.empty((n, 16), dtype=torch.float32, device=dev)
+        sel_h = torch.empty((n, max(rank, 1)), dtype=torch.float32, device=dev)
+        self.ctx._check(L.dflash_draft_session_selector_inputs(self.ctx._h, self._h, ids.data_ptr(), vals.data_ptr(),
+                                                               sel_h.data_ptr(), _stream_ptr()))
+        return ids, vals, sel_h
+
     def prepare_ctx(self):
         """Bring fc + hidden_norm and the per-layer context K/V up to date for the columns appended so far
         (draft_block does it lazily otherwise)."""
@@ -548,20 +564,25 @@ class SpeculativeDecoder:
 
     def __init__(self, ctx: Context, target: TargetModel, head: DraftHead, tap_layers, kv_capacity: int,
                  mask_token: int, sampler: Sampler | None = None, fallback_margin: float = 0.0,
-                 fallback_partial: bool = True, stop_ids=()):
+                 fallback_partial: bool = True, stop_ids=(), proposal_sampler: Sampler | None = None):
+        """``proposal_sampler`` (with ``sampler`` and a DFlash-2 head): the drafter samples its tokens along the
+        selector walk and the target's sampler is coupled to the walk's candidate distributions
+        (qwen/dflash.rs:508-519: temperature of the target's sampler only, seed ^ 0x4446_4c41_5348_3251)."""
         self.ctx, self.target, self.head = ctx, target, head
         self.tap_layers = list(tap_layers)
         self.session = Session(ctx, target, kv_capacity, self.tap_layers)
         self.draft_session = DraftSession(ctx, head, target, kv_capacity)
         self.sampler = sampler
+        self.proposal_sampler = proposal_sampler
         self.stop_ids = list(stop_ids)
-        self.cfg = StepCfgC(mask_token, int(sampler is not None), fallback_margin, int(fallback_partial),
+        mode = 0 if sampler is None else (2 if proposal_sampler is not None else 1)
+        self.cfg = StepCfgC(mask_token, mode, fallback_margin, int(fallback_partial),
                             DFLASH_VERIFY_FALLBACK_PARTIAL_MIN_GAP)
         self._L = _lib()
         self._L.dflash_spec_step.restype = C.c_int32
         self._L.dflash_spec_step.argtypes = [
             C.c_void_p, C.POINTER(ModelC), C.POINTER(DraftHeadC), C.c_void_p, C.c_void_p, C.POINTER(C.c_int32),
-            C.c_int32, C.c_int32, C.c_int64, C.POINTER(StepCfgC), C.POINTER(SamplerC), C.c_int64,
+            C.c_int32, C.c_int32, C.c_int64, C.POINTER(StepCfgC), C.POINTER(SamplerC), C.POINTER(SamplerC), C.c_int64,
             C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_int32), C.POINTER(StepResultC), C.c_void_p]
         self.position = 0
 
@@ -596,7 +617,9 @@ class SpeculativeDecoder:
         self.ctx._check(self._L.dflash_spec_step(
             self.ctx._h, C.byref(self.target.c), C.byref(self.head.c), self.session._h, self.draft_session._h, taps,
             len(self.tap_layers), carry, self.position, C.byref(self.cfg),
-            C.byref(self.sampler.c) if self.sampler is not None else None, budget, stops, len(self.stop_ids), ov,
+            C.byref(self.sampler.c) if self.sampler is not None else None,
+            C.byref(self.proposal_sampler.c) if self.proposal_sampler is not None else None, budget, stops,
+            len(self.stop_ids), ov,
             C.byref(res), _stream_ptr()))
         self.position += res.decision.retain_input_count
         return res

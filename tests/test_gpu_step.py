@@ -134,6 +134,64 @@ def test_generate_with_a_dflash2_head_equals_serial_greedy(ctx, world):
     dec.close()
 
 
+def test_sampled_dflash2_step_equals_its_parts(ctx, world, oracle):
+    """sampled_mode 2 (draft_block_sampled + couple_sparse_proposal, qwen/dflash.rs:508-519, 706-716;
+    metal_dflash.rs:17268-17415): a speculative step with a DFlash-2 head, a proposal sampler and the target's
+    sampler must decide exactly what the parts decide when composed by hand on an identical second pair of
+    sessions: the oracle's sampled walk over the drafter's selector inputs, a packed verify of those tokens,
+    and the oracle's accept-prefix over the verify logits with the walk's sparse proposals.  Samplers advance
+    identically.  Three consecutive steps, each continuing from the previous decision."""
+    d2 = dfl.DraftConfig(**{**D1.as_dict(), "block_size": 8, "conv_kernel_size": 2, "conv_group_size": 64,
+                            "selector_rank": 64, "selector_top_k": 16})
+    dw = dfl.synth_draft_weights(d2, seed=5, vocab=C1.vocab, codebook_type=dfl.TYPE_Q8_0)
+    head = dfl.DraftHead(ctx, d2, dw)
+    pred_cb, _k1 = oracle.make_codebook(dfl.TYPE_Q8_0, dw["selector_predecessor"][1], 64)
+    succ_cb, _k2 = oracle.make_codebook(dfl.TYPE_Q8_0, dw["selector_successor"][1], 64)
+    tkw = dict(temperature=0.9, top_k=20, top_p=0.95, min_p=0.0, seed=77)
+    pkw = dict(temperature=0.9, top_k=0, top_p=1.0, min_p=0.0, seed=77 ^ 0x4446_4c41_5348_3251)
+    dec = dfl.SpeculativeDecoder(ctx, world["model"], head, TAPS, 256, MASK, sampler=dfl.Sampler(**tkw),
+                                 proposal_sampler=dfl.Sampler(**pkw))
+    first = dec.prefill(world["prompt"])
+    # the by-hand twin
+    sess = dfl.Session(ctx, world["model"], 256, TAPS)
+    dsess = dfl.DraftSession(ctx, head, world["model"], 256)
+    for s0 in range(0, PROMPT_LEN, 16):
+        blk = world["prompt"][s0:s0 + 16]
+        out = sess.encode_packed_verify_layer_major(blk, s0)
+        dsess.append_target_ctx_columns(out.hidden_capture, list(range(s0, s0 + len(blk))))
+    otarget, oprop = oracle.make_sampler(**tkw), oracle.make_sampler(**pkw)
+    carry, pos = first, PROMPT_LEN
+    for _ in range(3):
+        res = dec.step(carry, 1000)
+        got = dfl.AcceptDecision(res.decision)
+        # by hand
+        dsess.draft_block(carry, MASK, pos)
+        ids, vals, sel_h = (t.cpu().numpy() for t in dsess.selector_inputs())
+        rc, toks, props, _err = oracle.select_draft_path_sampled(pred_cb, succ_cb, 16, 64, carry, 8, ids, vals, sel_h, oprop)
+        assert rc == 0
+        block = [carry] + [int(t) for t in toks[1:]]
+        assert list(res.draft_tokens[:8]) == block
+        out = sess.encode_packed_verify_layer_major(block, pos, want_logits=True)
+        proposals = [(block[r + 1], props[r]) for r in range(7)]
+        rc, want = oracle.decide_accept_prefix(block, out.logits.cpu().numpy(), C1.vocab, proposals, otarget, 1000, [])
+        assert rc == 0
+        assert got.key() == want.key()
+        assert dec.sampler.draws == oracle.sampler_state(otarget)[1]
+        assert dec.proposal_sampler.draws == oracle.sampler_state(oprop)[1]
+        n_keep = want.retain_input_count
+        sess.encode_restore_after_partial_accept(pos, 8, n_keep)
+        dsess.append_target_ctx_columns(out.hidden_capture[:n_keep], list(range(pos, pos + n_keep)))
+        pos += n_keep
+        carry = want.carry_token
+        assert dec.position == pos
+    # a draft override has no meaning when the drafts carry their proposal distributions
+    with pytest.raises(dfl.DFlashError):
+        dec.step(carry, 1000, draft_override=[1, 2, 3])
+    dsess.close()
+    sess.close()
+    dec.close()
+
+
 def test_generate_sampled_equals_serial_sampler(ctx, world, oracle):
     """Deterministic-proposal coupling == serial sampling with the same stream (sampling.rs:2837-2865).
     The serial stream is the CPU oracle's sampler applied to the logits of a token-by-token pass through
