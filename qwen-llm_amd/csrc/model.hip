@@ -197,11 +197,21 @@ __global__ void silu_mul_ld_kernel(const float *__restrict__ g, const float *__r
 struct Int16Args {
     int32_t v[16];
 };
+// dev_ids (may be null): where ids.v[i] is negative, the id comes from dev_ids[i] instead, clamped
+// into [0, vocab) (the host checks the copied-back values and reports an invalid token; the clamp only
+// keeps the embedding gather inside its table meanwhile).
 __global__ void set_ids_pos_kernel(Int16Args ids, Int16Args pos, int n, int32_t *__restrict__ ids_dst,
-                                   int32_t *__restrict__ pos_dst) {
+                                   int32_t *__restrict__ pos_dst, const int32_t *__restrict__ dev_ids, int vocab) {
     const int i = threadIdx.x;
     if (i < n) {
-        if (ids_dst) ids_dst[i] = ids.v[i];
+        if (ids_dst) {
+            int32_t id = ids.v[i];
+            if (dev_ids && id < 0) {
+                id = dev_ids[i];
+                if (id < 0 || id >= vocab) id = 0;
+            }
+            ids_dst[i] = id;
+        }
         pos_dst[i] = pos.v[i];
     }
 }
@@ -519,10 +529,30 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
 
 }  // namespace
 
+namespace {
+int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
+                          const int32_t *dev_tokens, int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps,
+                          int32_t *argmax, float *gap, float *hidden_capture, float *logits, int32_t *argmax_host,
+                          dflash_stream_t stream);
+}
+
 int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
                             int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps, int32_t *argmax,
                             float *gap, float *hidden_capture, float *logits, int32_t *argmax_host,
                             dflash_stream_t stream) {
+    return verify_block_impl(ctx, model, s, tokens, nullptr, n, start, tap_layers, n_taps, argmax, gap, hidden_capture, logits,
+                             argmax_host, stream);
+}
+
+namespace {
+
+// dev_tokens (may be null): device ids that stand in wherever tokens[i] is negative (the drafter's
+// output, still on the device: a speculative step then needs no host round trip between drafting and
+// verifying).
+int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
+                          const int32_t *dev_tokens, int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps,
+                          int32_t *argmax, float *gap, float *hidden_capture, float *logits, int32_t *argmax_host,
+                          dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!model || !s || !tokens) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "verify_block: null argument");
     const dflash_model_cfg &c = model->cfg;
@@ -535,7 +565,7 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
         return dfl_fail(ctx, DFLASH_ERR_STATE, "verify_block: positions %lld..%lld exceed the KV capacity %lld",
                         static_cast<long long>(start), static_cast<long long>(start + n), static_cast<long long>(s->capacity));
     for (int i = 0; i < n; i++)
-        if (tokens[i] < 0 || tokens[i] >= c.vocab)
+        if ((tokens[i] < 0 && !dev_tokens) || tokens[i] >= c.vocab)
             return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "verify_block: token %d at index %d outside vocabulary %d",
                             tokens[i], i, c.vocab);
     if (n_taps < 0 || n_taps > s->n_taps || (n_taps > 0 && (!tap_layers || !hidden_capture)))
@@ -548,7 +578,7 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
         ids_arg.v[i] = tokens[i];
         pos_arg.v[i] = static_cast<int32_t>(start + i);
     }
-    set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, n, s->ids, s->pos);
+    set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, n, s->ids, s->pos, dev_tokens, c.vocab);
     float *lg = logits ? logits : s->logits;
     int32_t *am = argmax ? argmax : s->argmax;
     float *gp = gap ? gap : s->gap;
@@ -601,6 +631,8 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
     }
     return DFLASH_OK;
 }
+
+}  // namespace
 
 int32_t dflash_restore(dflash_ctx *ctx, dflash_session *s, int64_t start, int32_t n, int32_t n_keep) {
     if (!ctx || !s) return DFLASH_ERR_INVALID_INPUT;
@@ -689,7 +721,7 @@ int32_t dflash_draft_append_ctx(dflash_ctx *ctx, dflash_draft_session *s, const 
     if (n_cols <= 16) {
         Int16Args none = {}, pos_arg = {};
         for (int i = 0; i < n_cols; i++) pos_arg.v[i] = positions[i];
-        set_ids_pos_kernel<<<1, 64, 0, st>>>(none, pos_arg, n_cols, nullptr, s->pos_ctx + s->ctx_len);
+        set_ids_pos_kernel<<<1, 64, 0, st>>>(none, pos_arg, n_cols, nullptr, s->pos_ctx + s->ctx_len, nullptr, 0);
     } else {
         DFL_HIP_CHECK(ctx, hipMemcpyAsync(s->pos_ctx + s->ctx_len, positions, n_cols * sizeof(int32_t), hipMemcpyHostToDevice, st));
     }
@@ -831,7 +863,7 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         ids_arg.v[i] = i == 0 ? carry : mask_token;
         pos_arg.v[i] = static_cast<int32_t>(noise_start + i);
     }
-    set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, N, s->ids, s->pos);
+    set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, N, s->ids, s->pos, nullptr, 0);
     if ((rc = embed_rows(ctx, target->token_embd, s->ids, N, H, s->x, st))) return rc;
 
     for (int il = 0; il < c.n_layers; il++) {
@@ -1116,23 +1148,59 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
                                                    dsess->topk_vals, dsess->sel_h, proposal_sampler, res->draft_tokens, prop_counts,
                                                    prop_cands, st)))
             return rc;
-    } else if ((rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, nullptr, nullptr,
-                                        res->draft_tokens, st))) {
-        return rc;
+    } else {
+        // The drafter's tokens stay on the device and the verify is enqueued right behind the drafter:
+        // no host round trip between the two phases, and the GPU does not wait for the host to start
+        // launching the verify.  The phases are timed by events on the stream.
+        if ((rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, dsess->argmax, nullptr, nullptr, st)))
+            return rc;
     }
-    res->draft_ms = ms_since(t0);
-    res->draft_tokens[0] = carry;
-    if (draft_override)
-        for (int i = 1; i < N; i++)
-            if (draft_override[i - 1] >= 0) res->draft_tokens[i] = draft_override[i - 1];
-
-    t0 = std::chrono::steady_clock::now();
     const int32_t *verify_input = res->draft_tokens;
-    if ((rc = dflash_verify_block(ctx, target, sess, verify_input, N, position, taps, n_taps, nullptr, nullptr, sess->hidden,
-                                  nullptr, res->verify_argmax, st)))
-        return rc;
-    DFL_HIP_CHECK(ctx, hipMemcpy(res->verify_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost));
-    res->verify_ms = ms_since(t0);
+    if (sampled_drafts) {
+        res->draft_ms = ms_since(t0);
+        res->draft_tokens[0] = carry;
+        t0 = std::chrono::steady_clock::now();
+        if ((rc = dflash_verify_block(ctx, target, sess, verify_input, N, position, taps, n_taps, nullptr, nullptr, sess->hidden,
+                                      nullptr, res->verify_argmax, st)))
+            return rc;
+        DFL_HIP_CHECK(ctx, hipMemcpy(res->verify_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost));
+        res->verify_ms = ms_since(t0);
+    } else {
+        const bool timed = !ctx->timing;  // the per-kernel timers use the same events
+        if (timed) DFL_HIP_CHECK(ctx, hipEventRecord(ctx->ev0, st));
+        int32_t tokens_in[16];
+        tokens_in[0] = carry;
+        for (int i = 1; i < N; i++) tokens_in[i] = (draft_override && draft_override[i - 1] >= 0) ? draft_override[i - 1] : -1;
+        const double enqueue_draft_ms = ms_since(t0);
+        t0 = std::chrono::steady_clock::now();
+        if ((rc = verify_block_impl(ctx, target, sess, tokens_in, dsess->argmax, N, position, taps, n_taps, nullptr, nullptr,
+                                    sess->hidden, nullptr, nullptr, st)))
+            return rc;
+        if (timed) DFL_HIP_CHECK(ctx, hipEventRecord(ctx->ev1, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(res->verify_argmax, sess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(res->verify_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(res->draft_tokens, dsess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        const double wall_ms = enqueue_draft_ms + ms_since(t0);
+        // the wall time of the two phases, split by the GPU time of the verify
+        float verify_gpu_ms = 0.0f;
+        if (timed && hipEventElapsedTime(&verify_gpu_ms, ctx->ev0, ctx->ev1) == hipSuccess && verify_gpu_ms < wall_ms) {
+            res->verify_ms = verify_gpu_ms;
+            res->draft_ms = wall_ms - verify_gpu_ms;
+        } else {
+            res->draft_ms = enqueue_draft_ms;
+            res->verify_ms = wall_ms - enqueue_draft_ms;
+        }
+        for (int i = 1; i < N; i++) {
+            if (tokens_in[i] >= 0) res->draft_tokens[i] = tokens_in[i];
+            if (res->draft_tokens[i] < 0 || res->draft_tokens[i] >= target->cfg.vocab) {
+                (void)dflash_restore(ctx, sess, position, N, 0);  // nothing is committed
+                return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "spec_step: the drafter produced token %d at slot %d (vocabulary %d)",
+                                res->draft_tokens[i], i, target->cfg.vocab);
+            }
+        }
+        res->draft_tokens[0] = carry;
+    }
 
     t0 = std::chrono::steady_clock::now();
     if (sampled_drafts) {  // couple_sparse_proposal with the walk's candidate distributions
