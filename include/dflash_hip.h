@@ -448,6 +448,46 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
                          int64_t remaining_output_budget, const int32_t *stop_ids_host, int32_t n_stop,
                          const int32_t *draft_override_host, dflash_step_result *out_host, dflash_stream_t stream);
 
+/* ---- adaptive speculation policy (host logic only) ------------------------------------------
+ * DflashAdaptiveState, dflash_speculation_enabled, dflash_prefix_replay_*, verify_fallback_margin
+ * (crates/qwen-cli/src/qwen/dflash.rs:5-376): when the loop speculates, when it takes an exact
+ * single-token step instead, and when it probes again.  The thresholds are the reference's own
+ * (calibrated on its hardware).  A caller's loop: prepare_mode, backoff_active / probe_due ->
+ * dflash_speculation_enabled; off step: record_off_step; speculative step: begin_spec_step before,
+ * record_spec_step after. */
+enum { DFLASH_BACKOFF_NONE = 0, DFLASH_BACKOFF_ACCEPTANCE = 1, DFLASH_BACKOFF_FALLBACK = 2 };
+#define DFLASH_OFF_CTX_DEFAULT 16384 /* hard stop of speculation past the calibrated range */
+
+typedef struct {
+    int32_t alpha_window[16];   /* accepted drafts of the last speculative steps */
+    int32_t n_alpha;
+    uint8_t fallback_window[8]; /* whether the exact fallback ran (long-context lane) */
+    int32_t n_fallback;
+    int32_t reentry_accepts[2]; /* accepted drafts of the last probes (long-context lane) */
+    int32_t n_reentry;
+    int32_t reason;             /* DFLASH_BACKOFF_* */
+    int32_t long_mode;
+    int64_t off_steps_since_probe;
+} dflash_adaptive_state;
+
+void dflash_adaptive_init(dflash_adaptive_state *s);
+void dflash_adaptive_prepare_mode(dflash_adaptive_state *s, int32_t long_mode);
+int32_t dflash_adaptive_backoff_active(const dflash_adaptive_state *s);
+int32_t dflash_adaptive_probe_due(const dflash_adaptive_state *s, int32_t sampled_mode, int32_t long_mode);
+void dflash_adaptive_record_off_step(dflash_adaptive_state *s);
+void dflash_adaptive_begin_spec_step(dflash_adaptive_state *s);
+void dflash_adaptive_record_spec_step(dflash_adaptive_state *s, int32_t n_accepted, int32_t fallback_ran, int32_t was_probe,
+                                      int32_t reentry_eligible, int32_t sampled_mode, int32_t long_mode, int64_t position);
+int32_t dflash_speculation_enabled(int32_t spec_disabled, int64_t position, int64_t off_ctx, int64_t remaining_context_tokens,
+                                   int32_t block_size, int32_t backoff_active, int32_t backoff_probe_due);
+int32_t dflash_prefix_replay_allowed(int32_t spec_disabled, int64_t position, int64_t off_ctx, int64_t remaining_context_tokens,
+                                     int32_t block_size, int32_t long_mode, int32_t backoff_active, int32_t backoff_probe_due);
+/* 1 and *drafts = history + n_emitted if emitted is a prefix of history with draft_tokens more behind it, else 0 */
+int32_t dflash_prefix_replay_drafts(const int32_t *history, int64_t n_history, const int32_t *emitted, int64_t n_emitted,
+                                    int64_t draft_tokens, const int32_t **drafts);
+/* verify_fallback_margin (qwen/dflash.rs:126-136): 0.1, or 0.75 at positions >= DFLASH_OFF_CTX_DEFAULT */
+float dflash_verify_fallback_margin(int64_t n_pos);
+
 #ifdef __cplusplus
 }
 #endif

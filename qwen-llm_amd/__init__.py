@@ -40,7 +40,9 @@ from .model import (  # noqa: F401,E402
     DraftSession,
     ModelConfig,
     Session,
+    AdaptiveStateC,
     SpeculativeDecoder,
+    adaptive_lib,
     TargetModel,
     accept_greedy,
     synth_draft_weights,

@@ -366,6 +366,7 @@ class Session:
     def __init__(self, ctx: Context, model: TargetModel, kv_capacity: int, tap_layers=()):
         self.ctx, self.model = ctx, model
         self.tap_layers = list(tap_layers)
+        self.capacity = int(kv_capacity)
         self._L = _lib()
         h = C.c_void_p()
         cfgc = ModelCfgC(**model.cfg.as_dict())
@@ -522,6 +523,39 @@ class DraftSession:
         return argmax, logits, (list(host) if sync else None)
 
 
+# ---- adaptive speculation policy (qwen/dflash.rs:5-376): host logic of the library ----
+
+class AdaptiveStateC(C.Structure):
+    _fields_ = [("alpha_window", C.c_int32 * 16), ("n_alpha", C.c_int32), ("fallback_window", C.c_uint8 * 8),
+                ("n_fallback", C.c_int32), ("reentry_accepts", C.c_int32 * 2), ("n_reentry", C.c_int32),
+                ("reason", C.c_int32), ("long_mode", C.c_int32), ("off_steps_since_probe", C.c_int64)]
+
+
+_adaptive_declared = False
+
+
+def adaptive_lib():
+    """The library with the policy functions' signatures declared (they run on the host; no GPU needed)."""
+    global _adaptive_declared
+    L = lib()
+    if not _adaptive_declared:
+        i32, i64, sp = C.c_int32, C.c_int64, C.POINTER(AdaptiveStateC)
+        for name, res, args in (
+                ("dflash_adaptive_init", None, [sp]), ("dflash_adaptive_prepare_mode", None, [sp, i32]),
+                ("dflash_adaptive_backoff_active", i32, [sp]), ("dflash_adaptive_probe_due", i32, [sp, i32, i32]),
+                ("dflash_adaptive_record_off_step", None, [sp]), ("dflash_adaptive_begin_spec_step", None, [sp]),
+                ("dflash_adaptive_record_spec_step", None, [sp, i32, i32, i32, i32, i32, i32, i64]),
+                ("dflash_speculation_enabled", i32, [i32, i64, i64, i64, i32, i32, i32]),
+                ("dflash_prefix_replay_allowed", i32, [i32, i64, i64, i64, i32, i32, i32, i32]),
+                ("dflash_prefix_replay_drafts", i32, [C.POINTER(i32), i64, C.POINTER(i32), i64, i64,
+                                                      C.POINTER(C.POINTER(i32))]),
+                ("dflash_verify_fallback_margin", C.c_float, [i64])):
+            f = getattr(L, name)
+            f.restype, f.argtypes = res, args
+        _adaptive_declared = True
+    return L
+
+
 # ---- one speculative transition and the generation loop (qwen/dflash.rs:700-1241) ----
 
 from .binding import AcceptDecision, AcceptDecisionC, Sampler, SamplerC  # noqa: E402
@@ -624,13 +658,37 @@ class SpeculativeDecoder:
         self.position += res.decision.retain_input_count
         return res
 
-    def generate(self, first_carry: int, max_tokens: int, on_step=None, draft_override_fn=None):
-        """Emit up to max_tokens tokens starting with first_carry.  Returns (tokens, stats)."""
+    def _off_step(self, carry: int, append_ctx: bool) -> int:
+        """One exact single-token step with hidden capture (the loop's off step, qwen/dflash.rs:617-690): the KV and
+        the drafter context stay current; returns the next token (argmax, or a draw of the target's sampler)."""
+        sampled = self.sampler is not None
+        out = self.session.encode_packed_verify_layer_major([carry], self.position, want_logits=sampled)
+        if append_ctx:
+            self.draft_session.append_target_ctx_columns(out.hidden_capture, [self.position])
+        self.position += 1
+        if not sampled:
+            return out.argmax_host[0]
+        d = self.ctx.decide_dflash_accept_prefix([carry], out.logits, self.target.cfg.vocab, None, self.sampler, 1 << 30, [])
+        return d.carry_token
+
+    def generate(self, first_carry: int, max_tokens: int, on_step=None, draft_override_fn=None, adaptive: bool = False,
+                 off_ctx: int = 16384):
+        """Emit up to max_tokens tokens starting with first_carry.  Returns (tokens, stats).
+        ``adaptive``: run the reference loop's back-off policy (qwen/dflash.rs:566-612, 1218-1231): speculation turns
+        off while the trailing acceptance window is below break-even (exact single-token steps keep the caches
+        current), probes again every few off steps, and stops for good at ``off_ctx`` or when a block no longer fits."""
         tokens = [first_carry]
         stats = {"spec_steps": 0, "accepted_drafts": 0, "drafts_scored": 0, "fallback_calls": 0, "draft_ms": 0.0,
                  "verify_ms": 0.0, "accept_ms": 0.0, "fallback_ms": 0.0, "append_ms": 0.0, "restore_ms": 0.0,
-                 "stop_reason": None}
+                 "stop_reason": None, "off_steps": 0, "backoff_probe_steps": 0, "backoff_reason": 0}
         carry = first_carry
+        L = adaptive_lib() if adaptive else None
+        state = AdaptiveStateC()
+        if adaptive:
+            L.dflash_adaptive_init(C.byref(state))
+        spec_disabled = False
+        sampled = int(self.sampler is not None)
+        n_block = self.head.cfg.block_size
         while True:
             if carry in self.stop_ids:
                 stats["stop_reason"] = "eos"
@@ -638,6 +696,24 @@ class SpeculativeDecoder:
             if len(tokens) >= max_tokens:
                 stats["stop_reason"] = "token_limit"
                 break
+            was_probe, long_mode = False, False
+            if adaptive:
+                long_mode = off_ctx > 16384 and self.position >= 16384
+                L.dflash_adaptive_prepare_mode(C.byref(state), int(long_mode))
+                active = L.dflash_adaptive_backoff_active(C.byref(state))
+                due = L.dflash_adaptive_probe_due(C.byref(state), sampled, int(long_mode))
+                remaining = self.session.capacity - self.position
+                if not L.dflash_speculation_enabled(int(spec_disabled), self.position, off_ctx, remaining, n_block, active, due):
+                    if self.position >= off_ctx or remaining < n_block:
+                        spec_disabled = True  # terminal: the drafter context is no longer fed
+                    stats["off_steps"] += 1
+                    L.dflash_adaptive_record_off_step(C.byref(state))
+                    carry = self._off_step(carry, not spec_disabled)
+                    tokens.append(carry)
+                    continue
+                was_probe = bool(active and due)
+                stats["backoff_probe_steps"] += int(was_probe)
+                L.dflash_adaptive_begin_spec_step(C.byref(state))
             ov = draft_override_fn(tokens, self.position) if draft_override_fn else None
             res = self.step(carry, max_tokens - len(tokens), ov)
             d = res.decision
@@ -653,6 +729,10 @@ class SpeculativeDecoder:
             if d.stop_reason:
                 stats["stop_reason"] = "eos" if d.stop_reason == 1 else "token_limit"
                 break
+            if adaptive:
+                L.dflash_adaptive_record_spec_step(C.byref(state), d.n_accepted, res.fallback_ran, int(was_probe), int(ov is None),
+                                                   sampled, int(long_mode), self.position)
+                stats["backoff_reason"] = state.reason
             carry = d.carry_token
             tokens.append(carry)
         return tokens, stats

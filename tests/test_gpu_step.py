@@ -217,3 +217,64 @@ def test_generate_sampled_equals_serial_sampler(ctx, world, oracle):
     assert stats["accepted_drafts"] > 0
     assert dec.sampler.draws == n_tok - 1 == oracle.sampler_state(osamp)[1]
     dec.close()
+
+
+def test_adaptive_generate_backs_off_probes_and_stays_exact(ctx, world):
+    """The loop under the back-off policy (qwen/dflash.rs:566-690, 1218-1231): a drafter that never hits fills the
+    acceptance window, speculation turns off, exact single-token steps carry on (the drafter context stays fed, so
+    probes can run), and the emitted tokens are still the target's serial greedy decode."""
+    cont = world["cont"]
+    undecided = np.flatnonzero(~world["decided"])
+    n_tok = int(min(70, undecided[0] if len(undecided) else 70))
+    assert n_tok >= 40
+    dec, first = new_decoder(ctx, world)
+    seen = []
+    tokens, stats = dec.generate(first, n_tok, adaptive=True, on_step=lambda r: seen.append(r.decision.n_accepted))
+    assert tokens == cont[:n_tok]
+    # 16 speculative steps fill the window (random drafter: almost nothing accepted), then off steps with a probe
+    # after every 8 of them
+    assert stats["spec_steps"] >= 16 and stats["off_steps"] >= 16
+    assert stats["backoff_probe_steps"] >= 1 and stats["backoff_reason"] == 1
+    assert stats["spec_steps"] + stats["off_steps"] + stats["accepted_drafts"] in (n_tok - 1, n_tok)
+    assert dec.session.kv_n_pos == PROMPT_LEN + n_tok - 1 == dec.draft_session.ctx_len
+    dec.close()
+
+
+def test_adaptive_generate_stops_speculating_at_off_ctx_and_near_capacity(ctx, world):
+    """Past off_ctx (or with less than a block of room) every step is an exact single-token step and the drafter
+    context is no longer appended (qwen/dflash.rs:617-624)."""
+    cont = world["cont"]
+    undecided = np.flatnonzero(~world["decided"])
+    n_tok = int(min(40, undecided[0] if len(undecided) else 40))
+    dec, first = new_decoder(ctx, world)
+    off_ctx = PROMPT_LEN + 12
+    tokens, stats = dec.generate(first, n_tok, adaptive=True, off_ctx=off_ctx,
+                                 draft_override_fn=lambda t, p: cont[len(t):len(t) + 3] + [-1] * 12)
+    assert tokens == cont[:n_tok]
+    assert stats["spec_steps"] == 3 and stats["accepted_drafts"] == 9  # positions 40, 44, 48; 52 >= off_ctx
+    assert stats["off_steps"] == n_tok - 1 - 12
+    assert dec.draft_session.ctx_len == off_ctx and dec.session.kv_n_pos == PROMPT_LEN + n_tok - 1
+    dec.close()
+
+
+def test_adaptive_generate_sampled_equals_serial_sampler(ctx, world, oracle):
+    """Off steps draw from the same sampler stream as speculative steps, so the emitted stream is the serial one."""
+    n_tok = 48
+    kw = dict(temperature=0.8, top_k=20, top_p=0.95, min_p=0.0, seed=77)
+    osamp = oracle.make_sampler(**kw)
+    serial = dfl.Session(ctx, world["model"], 256, TAPS)
+    out = None
+    for s in range(0, PROMPT_LEN, 16):
+        out = serial.encode_packed_verify_layer_major(world["prompt"][s:s + 16], s)
+    want = [out.argmax_host[-1]]
+    while len(want) < n_tok:
+        out = serial.encode_packed_verify_layer_major([want[-1]], PROMPT_LEN + len(want) - 1, want_logits=True)
+        rc, tok, _idx, _err = oracle.sample(osamp, out.logits.cpu().numpy()[0])
+        assert rc == 0
+        want.append(tok)
+    serial.close()
+    dec, first = new_decoder(ctx, world, sampler=dfl.Sampler(**kw))
+    tokens, stats = dec.generate(first, n_tok, adaptive=True)
+    assert tokens == want
+    assert stats["off_steps"] > 0 and dec.sampler.draws == n_tok - 1
+    dec.close()
