@@ -40,6 +40,9 @@ enum {
     DFLASH_ERR_INVALID_TOKEN = 8,   /* DFlashAcceptError::InvalidToken / ForwardError::BadToken */
     DFLASH_ERR_PROPOSAL_MISMATCH = 9,
     DFLASH_ERR_STATE = 10,          /* kv_n_pos != start_position and similar guard walls */
+    DFLASH_ERR_IO = 11,             /* GgufError::Io: open / stat / mmap failed */
+    DFLASH_ERR_FORMAT = 12,         /* GgufError::BadMagic / Decode: not a well-formed GGUF v3 file */
+    DFLASH_ERR_METADATA = 13,       /* LoadError::BadMetadata / Missing / Shape / UnsupportedArch */
     /* sampling errors, numbered 32 + the sampler's own code */
     DFLASH_ERR_EMPTY_LOGITS = 33,
     DFLASH_ERR_INVALID_TEMPERATURE = 34,
@@ -97,8 +100,9 @@ size_t dflash_row_bytes(int32_t type, size_t n_in);
  * (metal_forward/dispatch.rs:365-378; kernel kernels/mat_mat_fewrow_gen.metal:374-474).
  *   Y[n_rows][n_out] = X[n_rows][n_in] . W^T,  W = quant blocks, row-major [n_out][n_in/blk]
  * x_type: DFLASH_TYPE_F32 (the reference's activations) or DFLASH_TYPE_F16; Y is f32.
- * 1 <= n_rows <= 16; n_in % 256 == 0 (Q4_K, Q6_K) or % 32 == 0 (Q8_0); W 16-byte aligned
- * (2-byte for Q8_0); Y must not alias X or W.  Enqueue-only. */
+ * 1 <= n_rows <= 16; n_in % 256 == 0 (Q4_K, Q6_K) or % 32 == 0 (Q8_0, and plain F32 / F16 matrices
+ * such as a router stored unquantised); W 16-byte aligned (2-byte for Q8_0 and Q6_K); Y must not
+ * alias X or W.  Enqueue-only. */
 int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
                            int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream);
 
@@ -487,6 +491,82 @@ int32_t dflash_prefix_replay_drafts(const int32_t *history, int64_t n_history, c
                                     int64_t draft_tokens, const int32_t **drafts);
 /* verify_fallback_margin (qwen/dflash.rs:126-136): 0.1, or 0.75 at positions >= DFLASH_OFF_CTX_DEFAULT */
 float dflash_verify_fallback_margin(int64_t n_pos);
+
+/* ---- GGUF reader and drafter loader (host only) -----------------------------------------------
+ * GgufFile (crates/qwen-llm/src/gguf.rs:129-740, layout :1320-1480): a read-only mapping of one
+ * little-endian GGUF v3 file with its metadata and tensor table validated up front: counts and
+ * lengths capped (:1303-1316), keys and tensor names unique, 1..4 dimensions, no zero or oversized
+ * dimension, offsets aligned to general.alignment (default 32, at most 65536), every tensor inside
+ * the file, no two tensors overlapping (:840-940).  Tensor bytes are NOT copied: data_host points
+ * into the mapping and stays valid until dflash_gguf_close.  Split (multi-shard) files are not
+ * read.  A failed call leaves its message in dflash_gguf_last_error (for open: in `err`). */
+typedef struct dflash_gguf dflash_gguf;
+
+typedef struct {
+    int32_t type;          /* ggml type id; DFLASH_TYPE_* for the types the kernels take */
+    int32_t n_dims;        /* after dropping trailing 1s (gguf.rs:840-846) */
+    uint64_t shape[4];     /* shape[0] = the fastest dimension (a matrix is [n_in, n_out]) */
+    uint64_t n_bytes;      /* 0 = tensor absent (optional members of the structs below) */
+    const void *data_host;
+} dflash_gguf_tensor;
+
+int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *err, size_t err_cap); /* GgufFile::open */
+void dflash_gguf_close(dflash_gguf *g);
+const char *dflash_gguf_last_error(const dflash_gguf *g);
+int64_t dflash_gguf_tensor_count(const dflash_gguf *g);
+int64_t dflash_gguf_kv_count(const dflash_gguf *g);
+uint64_t dflash_gguf_alignment(const dflash_gguf *g);
+uint64_t dflash_gguf_data_start(const dflash_gguf *g); /* file offset of the tensor data */
+/* i-th tensor in file order; *name points into the handle */
+int32_t dflash_gguf_tensor_at(const dflash_gguf *g, int64_t i, const char **name, dflash_gguf_tensor *out);
+/* GgufFile::find (:474): 1 = found, 0 = no such tensor */
+int32_t dflash_gguf_find(const dflash_gguf *g, const char *name, dflash_gguf_tensor *out);
+/* Scalar getters (:514-545, :697): 1 = present with a usable type, 0 = absent or another type.
+ * get_u64 takes any integer type with a non-negative value; get_f64 takes f32 / f64. */
+int32_t dflash_gguf_get_u64(const dflash_gguf *g, const char *key, uint64_t *out);
+int32_t dflash_gguf_get_f64(const dflash_gguf *g, const char *key, double *out);
+int32_t dflash_gguf_get_bool(const dflash_gguf *g, const char *key, int32_t *out);
+int32_t dflash_gguf_get_str(const dflash_gguf *g, const char *key, const char **out, uint64_t *len); /* not 0-terminated */
+/* Array getters (:546-696): the array's length, or -1 if the key is absent, or -2 if it is not an
+ * array of that kind (u64: any integer type, no negative element; bool; f64: f32 / f64); up to
+ * `cap` elements are written to out (which may be NULL with cap 0). */
+int64_t dflash_gguf_get_u64_array(const dflash_gguf *g, const char *key, uint64_t *out, int64_t cap);
+int64_t dflash_gguf_get_bool_array(const dflash_gguf *g, const char *key, uint8_t *out, int64_t cap);
+int64_t dflash_gguf_get_f64_array(const dflash_gguf *g, const char *key, double *out, int64_t cap);
+
+/* open_dflash_drafter_for_target (crates/qwen-llm/src/loader.rs:832-1290): reads a drafter file of
+ * either convention (arch "dflash-draft": keys dflash-draft.*, tensors dflash_fc / dflash_hidden_norm
+ * / blk.N.post_attention_norm; arch "dflash": keys dflash.*, tensors fc / enc.output_norm /
+ * blk.N.ffn_norm, target layers stored as layer-input indices and turned into post-block ids by
+ * subtracting 1, :1010-1023), validates it against the target (hidden sizes equal, mask token inside
+ * the vocabulary, tapped layers inside the target, n_target_features == taps * hidden, pattern length
+ * == block_count, sliding-window layers need a window) and binds every tensor with its shape checked.
+ * selector_hidden.weight present = DFlash-2: the four conv / selector keys and all conv and selector
+ * tensors become mandatory (:1029-1056).  Norms and conv bases must be F32. */
+typedef struct {
+    uint32_t hidden_size, vocab_size, n_layer; /* DFlashTargetShape (loader.rs:849-856) */
+} dflash_target_shape;
+
+typedef struct {
+    dflash_gguf_tensor attn_norm, wq, wk, wv, wo, q_norm, k_norm, post_norm, gate, up, down;
+    dflash_gguf_tensor conv_attn_base, conv_attn_proj, conv_ffn_base, conv_ffn_proj; /* DFlash-2 only */
+    int32_t is_swa, pad;
+} dflash_gguf_draft_layer;
+
+enum { DFLASH_GGUF_MAX_TAPS = 64 };
+typedef struct {
+    dflash_draft_cfg cfg;
+    int32_t mask_token_id;
+    int32_t convention;       /* 1 = "dflash-draft", 2 = "dflash" */
+    int32_t n_target_layers;  /* == cfg.n_taps */
+    int32_t target_layer_ids[DFLASH_GGUF_MAX_TAPS]; /* post-block layer ids of the target */
+    dflash_gguf_tensor fc, hidden_norm, output_norm;
+    dflash_gguf_tensor selector_hidden, selector_predecessor, selector_successor; /* DFlash-2 only */
+} dflash_gguf_draft_head;
+
+/* layers: caller's array of layer_cap entries; cfg.n_layers of them are filled. */
+int32_t dflash_gguf_open_drafter(dflash_gguf *g, const dflash_target_shape *target, dflash_gguf_draft_head *out,
+                                 dflash_gguf_draft_layer *layers, int32_t layer_cap);
 
 #ifdef __cplusplus
 }

@@ -154,6 +154,15 @@ int orc_dequant(int type, const uint8_t *blocks, size_t n_elems, float *out) {
     case ORC_Q4_K: return orc_dequant_q4_k(blocks, n_elems, out);
     case ORC_Q6_K: return orc_dequant_q6_k(blocks, n_elems, out);
     case ORC_Q8_0: return orc_dequant_q8_0(blocks, n_elems, out);
+    /* unquantised tensors (tensor.rs:164-208): F32 as stored, F16 widened exactly */
+    case ORC_F32: memcpy(out, blocks, n_elems * 4); return 0;
+    case ORC_F16:
+        for (size_t i = 0; i < n_elems; i++) {
+            uint16_t bits;
+            memcpy(&bits, blocks + 2 * i, 2);
+            out[i] = orc_f16_to_f32(bits);
+        }
+        return 0;
     default: return -1;
     }
 }
@@ -164,6 +173,8 @@ size_t orc_row_bytes(int type, size_t n_in) {
     case ORC_Q4_K: return n_in / ORC_QK_K * ORC_Q4_K_BYTES;
     case ORC_Q6_K: return n_in / ORC_QK_K * ORC_Q6_K_BYTES;
     case ORC_Q8_0: return n_in / ORC_QK8_0 * ORC_Q8_0_BYTES;
+    case ORC_F32: return n_in * 4;
+    case ORC_F16: return n_in * 2;
     default: return 0;
     }
 }

@@ -17,7 +17,7 @@ TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q6_K = 0, 1, 8, 12, 14
 
 STATUS = {
     0: "Ok", 1: "BadShape", 2: "Unsupported", 3: "Alias", 4: "Alignment", 5: "Workspace", 6: "Hip",
-    7: "InvalidInput", 8: "InvalidToken", 9: "ProposalMismatch", 10: "State", 33: "EmptyLogits",
+    7: "InvalidInput", 8: "InvalidToken", 9: "ProposalMismatch", 10: "State", 11: "Io", 12: "Format", 13: "Metadata", 33: "EmptyLogits",
     34: "InvalidTemperature", 35: "InvalidTopP", 36: "InvalidMinP", 37: "NanLogit", 38: "VocabularyTooLarge",
     39: "NoCandidates", 40: "ProposalTokenOutOfRange", 41: "InvalidProposalWeight", 42: "MissingProposalToken",
 }

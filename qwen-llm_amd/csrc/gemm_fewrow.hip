@@ -1054,6 +1054,36 @@ __device__ __forceinline__ half8_t convert_raw8<DFLASH_TYPE_Q8_0>(const Raw8<DFL
     return v;
 }
 
+// Unquantised matrices (a router or a small projection stored as F32 / F16): rows are 16-byte multiples
+// because n_in is a multiple of 32.
+template <>
+struct Raw8<DFLASH_TYPE_F32> {
+    float4_t a, b;
+};
+template <>
+struct Raw8<DFLASH_TYPE_F16> {
+    half8_t v;
+};
+template <>
+__device__ __forceinline__ Raw8<DFLASH_TYPE_F32> load_raw8<DFLASH_TYPE_F32>(const uint8_t *row, int64_t k0) {
+    const float *p = reinterpret_cast<const float *>(row) + k0;
+    return Raw8<DFLASH_TYPE_F32>{*reinterpret_cast<const float4_t *>(p), *reinterpret_cast<const float4_t *>(p + 4)};
+}
+template <>
+__device__ __forceinline__ half8_t convert_raw8<DFLASH_TYPE_F32>(const Raw8<DFLASH_TYPE_F32> &r) {
+    return half8_t{static_cast<_Float16>(r.a[0]), static_cast<_Float16>(r.a[1]), static_cast<_Float16>(r.a[2]),
+                   static_cast<_Float16>(r.a[3]), static_cast<_Float16>(r.b[0]), static_cast<_Float16>(r.b[1]),
+                   static_cast<_Float16>(r.b[2]), static_cast<_Float16>(r.b[3])};
+}
+template <>
+__device__ __forceinline__ Raw8<DFLASH_TYPE_F16> load_raw8<DFLASH_TYPE_F16>(const uint8_t *row, int64_t k0) {
+    return Raw8<DFLASH_TYPE_F16>{*reinterpret_cast<const half8_t *>(reinterpret_cast<const _Float16 *>(row) + k0)};
+}
+template <>
+__device__ __forceinline__ half8_t convert_raw8<DFLASH_TYPE_F16>(const Raw8<DFLASH_TYPE_F16> &r) {
+    return r.v;
+}
+
 // Eight consecutive activations (16-byte aligned) in two halves as well: the raw load, then the f16
 // fragment.
 template <typename XT>
@@ -1528,9 +1558,10 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
                         static_cast<long long>(n_in), static_cast<long long>(n_out));
     if (x_type != DFLASH_TYPE_F32 && x_type != DFLASH_TYPE_F16)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: activations must be f32 or f16");
-    if (w_type != DFLASH_TYPE_Q4_K && w_type != DFLASH_TYPE_Q6_K && w_type != DFLASH_TYPE_Q8_0)
+    const bool plain = w_type == DFLASH_TYPE_F32 || w_type == DFLASH_TYPE_F16;
+    if (w_type != DFLASH_TYPE_Q4_K && w_type != DFLASH_TYPE_Q6_K && w_type != DFLASH_TYPE_Q8_0 && !plain)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: weight type %d has no few-row kernel", w_type);
-    const int64_t blk = (w_type == DFLASH_TYPE_Q8_0) ? DFL_QK8_0 : DFL_QK_K;
+    const int64_t blk = (w_type == DFLASH_TYPE_Q8_0 || plain) ? DFL_QK8_0 : DFL_QK_K;
     if (n_in % blk)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: n_in %lld is not a multiple of %lld",
                         static_cast<long long>(n_in), static_cast<long long>(blk));
@@ -1538,7 +1569,7 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
     const size_t w_bytes = row_bytes * static_cast<size_t>(n_out);
     const size_t x_bytes = static_cast<size_t>(n_rows) * n_in * (x_type == DFLASH_TYPE_F32 ? 4 : 2);
     const size_t y_bytes = static_cast<size_t>(n_rows) * n_out * 4;
-    if (reinterpret_cast<uintptr_t>(w) % (w_type == DFLASH_TYPE_Q4_K ? 16 : 2) ||
+    if (reinterpret_cast<uintptr_t>(w) % ((w_type == DFLASH_TYPE_Q4_K || plain) ? 16 : 2) ||
         reinterpret_cast<uintptr_t>(x) % 4 || reinterpret_cast<uintptr_t>(y) % 4)
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: operand alignment");
     if (dfl_ranges_overlap(y, y_bytes, x, x_bytes) || dfl_ranges_overlap(y, y_bytes, w, w_bytes))
@@ -1573,7 +1604,20 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
         size_t lds = static_cast<size_t>(split) * 256 * sizeof(float);
         const uint8_t *wb = static_cast<const uint8_t *>(w);
         dfl_timed timer(ctx, st, DFL_T_GEMM);
-        if (n_in % 256 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+#define DFL_LAUNCH_GENERIC(TYPE)                                                                                         \
+    do {                                                                                                                 \
+        if (x_type == DFLASH_TYPE_F32)                                                                                   \
+            gemm_generic_kernel<TYPE, float><<<tiles, 64 * split, lds, st>>>(                                            \
+                wb, static_cast<const float *>(x), y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);       \
+        else                                                                                                             \
+            gemm_generic_kernel<TYPE, _Float16><<<tiles, 64 * split, lds, st>>>(                                         \
+                wb, static_cast<const _Float16 *>(x), y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);    \
+    } while (0)
+        if (w_type == DFLASH_TYPE_F32)
+            DFL_LAUNCH_GENERIC(DFLASH_TYPE_F32);
+        else if (w_type == DFLASH_TYPE_F16)
+            DFL_LAUNCH_GENERIC(DFLASH_TYPE_F16);
+        else if (n_in % 256 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
             env_int("DFLASH_Q8_STAGED", 1)) {
             static bool attr = false;
             if (!attr) {
@@ -1592,12 +1636,9 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
                 gemm_q8_0_staged_kernel<_Float16><<<tiles, 64 * split, kQ8StagedLds, st>>>(
                     wb, static_cast<const _Float16 *>(x), y, static_cast<int>(n_out), static_cast<int>(n_steps), row_bytes, n_rows,
                     split);
-        } else if (x_type == DFLASH_TYPE_F32)
-            gemm_generic_kernel<DFLASH_TYPE_Q8_0, float><<<tiles, 64 * split, lds, st>>>(
-                wb, static_cast<const float *>(x), y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
-        else
-            gemm_generic_kernel<DFLASH_TYPE_Q8_0, _Float16><<<tiles, 64 * split, lds, st>>>(
-                wb, static_cast<const _Float16 *>(x), y, static_cast<int>(n_out), n_steps, row_bytes, n_rows, split);
+        } else
+            DFL_LAUNCH_GENERIC(DFLASH_TYPE_Q8_0);
+#undef DFL_LAUNCH_GENERIC
     }
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;

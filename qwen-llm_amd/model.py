@@ -285,11 +285,20 @@ class _Uploader:
         self.device = device
         self.keep = []
 
+    def _from_numpy(self, a):
+        """torch view of a host array; read-only arrays (views into a mapped GGUF file) are only ever copied from."""
+        if a.flags.writeable:
+            return self.torch.from_numpy(a)
+        import warnings
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            return self.torch.from_numpy(a)
+
     def f32(self, a):
         if isinstance(a, self.torch.Tensor):
             t = a.to(self.device, self.torch.float32).contiguous()
         else:
-            t = self.torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device)
+            t = self._from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device)
         self.keep.append(t)
         return t.data_ptr()
 
@@ -300,7 +309,7 @@ class _Uploader:
         if isinstance(blocks, self.torch.Tensor):  # already resident (device-generated synthetic blocks)
             t = blocks.to(self.device).contiguous()
         else:
-            t = self.torch.from_numpy(np.ascontiguousarray(blocks)).to(self.device)
+            t = self._from_numpy(np.ascontiguousarray(blocks)).to(self.device)
         self.keep.append(t)
         return QTensorC(int(qtype), 0, t.data_ptr())
 
@@ -316,7 +325,7 @@ class _Uploader:
             if isinstance(blocks, torch.Tensor):
                 flats.append(blocks.to(self.device).contiguous().view(torch.uint8).reshape(-1))
             else:
-                flats.append(torch.from_numpy(np.ascontiguousarray(blocks).view(np.uint8).reshape(-1)).to(self.device))
+                flats.append(self._from_numpy(np.ascontiguousarray(blocks).view(np.uint8).reshape(-1)).to(self.device))
         whole = torch.cat(flats)
         self.keep.append(whole)
         out, off = [], 0
