@@ -1152,7 +1152,12 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         // The drafter's tokens stay on the device and the verify is enqueued right behind the drafter:
         // no host round trip between the two phases, and the GPU does not wait for the host to start
         // launching the verify.  The phases are timed by events on the stream.
-        if ((rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, dsess->argmax, nullptr, nullptr, st)))
+        // A caller that supplies every draft (prefix replay, qwen/dflash.rs:700-712) skips the drafter, as the
+        // reference does; the context columns it leaves pending are taken up by the next draft.
+        bool all_given = draft_override != nullptr;
+        for (int i = 0; all_given && i < N - 1; i++) all_given = draft_override[i] >= 0;
+        if (!all_given &&
+            (rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, dsess->argmax, nullptr, nullptr, st)))
             return rc;
     }
     const int32_t *verify_input = res->draft_tokens;

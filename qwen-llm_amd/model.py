@@ -681,15 +681,21 @@ class SpeculativeDecoder:
         return d.carry_token
 
     def generate(self, first_carry: int, max_tokens: int, on_step=None, draft_override_fn=None, adaptive: bool = False,
-                 off_ctx: int = 16384):
+                 off_ctx: int = 16384, prefix_replay=None, position_margin: bool = False):
         """Emit up to max_tokens tokens starting with first_carry.  Returns (tokens, stats).
         ``adaptive``: run the reference loop's back-off policy (qwen/dflash.rs:566-612, 1218-1231): speculation turns
         off while the trailing acceptance window is below break-even (exact single-token steps keep the caches
-        current), probes again every few off steps, and stops for good at ``off_ctx`` or when a block no longer fits."""
+        current), probes again every few off steps, and stops for good at ``off_ctx`` or when a block no longer fits.
+        ``prefix_replay`` (with ``adaptive``, greedy only): a previous generation's tokens; while the emitted tokens
+        are a prefix of it, its continuation replaces the drafter's tokens, also through back-off (:594-612, 700-712),
+        and such steps do not count as re-entry evidence.  ``position_margin``: the greedy fallback margin follows the
+        position (verify_fallback_margin, :126-136) instead of the constructor's value."""
         tokens = [first_carry]
+        history = [int(t) for t in prefix_replay] if prefix_replay is not None else None
+        hist_c = (C.c_int32 * max(len(history), 1))(*history) if history else None
         stats = {"spec_steps": 0, "accepted_drafts": 0, "drafts_scored": 0, "fallback_calls": 0, "draft_ms": 0.0,
                  "verify_ms": 0.0, "accept_ms": 0.0, "fallback_ms": 0.0, "append_ms": 0.0, "restore_ms": 0.0,
-                 "stop_reason": None, "off_steps": 0, "backoff_probe_steps": 0, "backoff_reason": 0}
+                 "stop_reason": None, "off_steps": 0, "backoff_probe_steps": 0, "backoff_reason": 0, "prefix_replay_steps": 0}
         carry = first_carry
         L = adaptive_lib() if adaptive else None
         state = AdaptiveStateC()
@@ -705,14 +711,23 @@ class SpeculativeDecoder:
             if len(tokens) >= max_tokens:
                 stats["stop_reason"] = "token_limit"
                 break
-            was_probe, long_mode = False, False
+            was_probe, long_mode, replay = False, False, None
+            if position_margin:
+                self.cfg.fallback_margin = adaptive_lib().dflash_verify_fallback_margin(self.position)
             if adaptive:
                 long_mode = off_ctx > 16384 and self.position >= 16384
                 L.dflash_adaptive_prepare_mode(C.byref(state), int(long_mode))
                 active = L.dflash_adaptive_backoff_active(C.byref(state))
                 due = L.dflash_adaptive_probe_due(C.byref(state), sampled, int(long_mode))
                 remaining = self.session.capacity - self.position
-                if not L.dflash_speculation_enabled(int(spec_disabled), self.position, off_ctx, remaining, n_block, active, due):
+                if history and not sampled and L.dflash_prefix_replay_allowed(
+                        int(spec_disabled), self.position, off_ctx, remaining, n_block, int(long_mode), active, due):
+                    emitted = (C.c_int32 * len(tokens))(*tokens)
+                    drafts = C.POINTER(C.c_int32)()
+                    if L.dflash_prefix_replay_drafts(hist_c, len(history), emitted, len(tokens), n_block - 1, C.byref(drafts)):
+                        replay = [drafts[i] for i in range(n_block - 1)]
+                if replay is None and not L.dflash_speculation_enabled(int(spec_disabled), self.position, off_ctx, remaining,
+                                                                       n_block, active, due):
                     if self.position >= off_ctx or remaining < n_block:
                         spec_disabled = True  # terminal: the drafter context is no longer fed
                     stats["off_steps"] += 1
@@ -723,7 +738,8 @@ class SpeculativeDecoder:
                 was_probe = bool(active and due)
                 stats["backoff_probe_steps"] += int(was_probe)
                 L.dflash_adaptive_begin_spec_step(C.byref(state))
-            ov = draft_override_fn(tokens, self.position) if draft_override_fn else None
+            ov = replay if replay is not None else (draft_override_fn(tokens, self.position) if draft_override_fn else None)
+            stats["prefix_replay_steps"] += int(replay is not None)
             res = self.step(carry, max_tokens - len(tokens), ov)
             d = res.decision
             stats["spec_steps"] += 1
@@ -739,8 +755,8 @@ class SpeculativeDecoder:
                 stats["stop_reason"] = "eos" if d.stop_reason == 1 else "token_limit"
                 break
             if adaptive:
-                L.dflash_adaptive_record_spec_step(C.byref(state), d.n_accepted, res.fallback_ran, int(was_probe), int(ov is None),
-                                                   sampled, int(long_mode), self.position)
+                L.dflash_adaptive_record_spec_step(C.byref(state), d.n_accepted, res.fallback_ran, int(was_probe),
+                                                   int(replay is None), sampled, int(long_mode), self.position)
                 stats["backoff_reason"] = state.reason
             carry = d.carry_token
             tokens.append(carry)

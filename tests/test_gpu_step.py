@@ -291,3 +291,37 @@ def test_adaptive_generate_sampled_equals_serial_sampler(ctx, world, oracle):
     assert tokens == want
     assert stats["off_steps"] > 0 and dec.sampler.draws == n_tok - 1
     dec.close()
+
+
+def test_prefix_replay_feeds_a_previous_generation_and_skips_the_drafter(ctx, world):
+    """Prefix replay (qwen/dflash.rs:594-612, 700-712): with a previous generation as history, every step's drafts
+    are its continuation (all accepted: 15 drafts + the bonus per step), the drafter is not run (no draft time is
+    recorded for a step whose drafts are all given), and when the history runs out the loop drafts again."""
+    cont = world["cont"]
+    undecided = np.flatnonzero(~world["decided"])
+    n_tok = int(min(60, undecided[0] if len(undecided) else 60))
+    history = cont[:36]
+    dec, first = new_decoder(ctx, world)
+    seen = []
+    tokens, stats = dec.generate(first, n_tok, adaptive=True, prefix_replay=history,
+                                 on_step=lambda r: seen.append((r.decision.n_accepted, r.draft_ms)))
+    assert tokens == cont[:n_tok]
+    # 1 + 16 + 16 = 33 tokens after two replay steps; 36 - 33 = 3 < 15 drafts left: replay ends
+    assert stats["prefix_replay_steps"] == 2 and [a for a, _ in seen[:2]] == [15, 15]
+    assert stats["spec_steps"] > 2 and dec.draft_session.ctx_len == dec.session.kv_n_pos == PROMPT_LEN + n_tok - 1
+    # a history that disagrees with what was emitted is never replayed
+    dec2, first2 = new_decoder(ctx, world)
+    wrong = [cont[0] + 1] + cont[1:40]
+    tokens2, stats2 = dec2.generate(first2, 30, adaptive=True, prefix_replay=wrong)
+    assert tokens2 == cont[:30] and stats2["prefix_replay_steps"] == 0
+    dec.close()
+    dec2.close()
+
+
+def test_position_margin_follows_the_reference_rule(ctx, world):
+    cont = world["cont"]
+    dec, first = new_decoder(ctx, world, fallback_partial=True)
+    tokens, stats = dec.generate(first, 24, position_margin=True)
+    assert tokens == cont[:24]
+    assert abs(dec.cfg.fallback_margin - 0.1) < 1e-7  # below 16384 positions (qwen/dflash.rs:126-136)
+    dec.close()
