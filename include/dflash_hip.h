@@ -428,6 +428,9 @@ typedef struct {
                                        (DFLASH_VERIFY_FALLBACK_MARGIN_DEFAULT = 0.1); <= 0 disables */
     int32_t fallback_partial;       /* 1: keep rows before the first flagged row (QWEN_DFLASH_VERIFY_FALLBACK_PARTIAL) */
     float fallback_partial_min_gap; /* a partially replayed row below this gap escalates to a whole-block replay (0.15) */
+    int32_t replay_only;            /* 1: a prefix-replay step (qwen/dflash.rs:700-712): draft_override_host supplies
+                                       every draft and the drafter is not run (the context columns it leaves pending
+                                       are taken up by the next draft); a missing entry is DFLASH_ERR_INVALID_INPUT */
 } dflash_step_cfg;
 
 typedef struct {

@@ -1152,11 +1152,14 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         // The drafter's tokens stay on the device and the verify is enqueued right behind the drafter:
         // no host round trip between the two phases, and the GPU does not wait for the host to start
         // launching the verify.  The phases are timed by events on the stream.
-        // A caller that supplies every draft (prefix replay, qwen/dflash.rs:700-712) skips the drafter, as the
+        // A prefix-replay step (qwen/dflash.rs:700-712) supplies every draft and skips the drafter, as the
         // reference does; the context columns it leaves pending are taken up by the next draft.
-        bool all_given = draft_override != nullptr;
-        for (int i = 0; all_given && i < N - 1; i++) all_given = draft_override[i] >= 0;
-        if (!all_given &&
+        if (cfg->replay_only) {
+            for (int i = 0; i < N - 1; i++)
+                if (!draft_override || draft_override[i] < 0)
+                    return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "spec_step: a replay-only step needs all %d drafts", N - 1);
+        }
+        if (!cfg->replay_only &&
             (rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, dsess->argmax, nullptr, nullptr, st)))
             return rc;
     }

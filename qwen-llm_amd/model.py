@@ -572,7 +572,7 @@ from .binding import AcceptDecision, AcceptDecisionC, Sampler, SamplerC  # noqa:
 
 class StepCfgC(C.Structure):
     _fields_ = [("mask_token", C.c_int32), ("sampled_mode", C.c_int32), ("fallback_margin", C.c_float),
-                ("fallback_partial", C.c_int32), ("fallback_partial_min_gap", C.c_float)]
+                ("fallback_partial", C.c_int32), ("fallback_partial_min_gap", C.c_float), ("replay_only", C.c_int32)]
 
 
 class StepResultC(C.Structure):
@@ -649,8 +649,11 @@ class SpeculativeDecoder:
         self.position = len(prompt)
         return last.argmax_host[-1]
 
-    def step(self, carry: int, budget: int, draft_override=None) -> StepResultC:
+    def step(self, carry: int, budget: int, draft_override=None, replay_only: bool = False) -> StepResultC:
+        """One speculative transition.  ``replay_only``: a prefix-replay step, ``draft_override`` holds every draft
+        and the drafter is not run."""
         res = StepResultC()
+        self.cfg.replay_only = int(replay_only)
         n = self.head.cfg.block_size
         ov = None
         if draft_override is not None:
@@ -740,7 +743,7 @@ class SpeculativeDecoder:
                 L.dflash_adaptive_begin_spec_step(C.byref(state))
             ov = replay if replay is not None else (draft_override_fn(tokens, self.position) if draft_override_fn else None)
             stats["prefix_replay_steps"] += int(replay is not None)
-            res = self.step(carry, max_tokens - len(tokens), ov)
+            res = self.step(carry, max_tokens - len(tokens), ov, replay_only=replay is not None)
             d = res.decision
             stats["spec_steps"] += 1
             stats["accepted_drafts"] += d.n_accepted
