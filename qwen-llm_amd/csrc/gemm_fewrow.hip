@@ -1395,10 +1395,12 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     const int tiles = static_cast<int>((n_out + 15) / 16);
     if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
-    // 8-wave workgroups (128 weight rows per stage): measured equal to 16-wave ones on large single
-    // matrices and faster wherever granularity counts (batches cut at tile-group boundaries, small
-    // matrices); the 16-wave instantiation stays selectable
-    const int waves = env_int("DFLASH_GEMM_WAVES", 8) == 16 ? 16 : 8;
+    // A single matrix: 16-wave workgroups (256 weight rows per stage) when that still leaves every CU
+    // a few stages of work, else 8-wave ones.  A batch is cut at tile-group boundaries only, so the
+    // finer 8-wave groups balance it better (measured: the two expert launches of a 35B-A3B-shaped
+    // layer take 50 us instead of 56 us).
+    int waves = (!batch && static_cast<int64_t>((tiles + 15) / 16) * nb >= 2ll * ctx->n_cu) ? 16 : 8;
+    waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
     const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
     const int groups = gpm * max_slots * ((batch && batch->pair) ? 2 : 1);  // upper bound in batched mode (pair mode: virtual groups)
     int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
@@ -1466,7 +1468,8 @@ int32_t launch_q6k_stream(dflash_ctx *ctx, const void *w, const void *x, int32_t
     const int tiles = static_cast<int>((n_out + 15) / 16);
     if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
-    const int waves = env_int("DFLASH_GEMM_WAVES", 8) == 16 ? 16 : 8;  // as for Q4_K: 8-wave workgroups measured best
+    int waves = (static_cast<int64_t>((tiles + 15) / 16) * nb >= 2ll * ctx->n_cu) ? 16 : 8;
+    waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
     const int groups = (tiles + waves - 1) / waves;
     int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
     const int64_t total = static_cast<int64_t>(groups) * nb;
