@@ -15,6 +15,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <exception>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -273,7 +274,7 @@ int32_t parse(dflash_gguf *g) {
         uint64_t offset;
     };
     std::vector<Raw> raw;
-    g->tensors.reserve(n_tensors);
+    g->tensors.reserve(std::min<uint64_t>(n_tensors, g->size / 33));  // a table entry is at least 33 bytes
     for (uint64_t i = 0; i < n_tensors; i++) {
         const uint64_t nlen = r.get<uint64_t>();
         if (!r.ok) return DFLASH_ERR_FORMAT;
@@ -384,7 +385,12 @@ extern "C" int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *e
         }
         g->map = static_cast<const uint8_t *>(m);
     }
-    const int32_t rc = parse(g);
+    int32_t rc;
+    try {
+        rc = parse(g);
+    } catch (const std::exception &e) {  // allocation failure: nothing may cross the C boundary
+        rc = fail(g, DFLASH_ERR_IO, "out of memory while reading the header (%s)", e.what());
+    }
     if (rc) {
         say(g->err);
         dflash_gguf_close(g);
@@ -568,8 +574,8 @@ struct Loader {
 
 }  // namespace
 
-extern "C" int32_t dflash_gguf_open_drafter(dflash_gguf *g, const dflash_target_shape *target, dflash_gguf_draft_head *out,
-                                            dflash_gguf_draft_layer *layers, int32_t layer_cap) {
+static int32_t open_drafter_impl(dflash_gguf *g, const dflash_target_shape *target, dflash_gguf_draft_head *out,
+                                 dflash_gguf_draft_layer *layers, int32_t layer_cap) {
     if (!g) return DFLASH_ERR_INVALID_INPUT;
     if (!target || !out || !layers) return fail(g, DFLASH_ERR_INVALID_INPUT, "open_drafter: null argument");
     if (target->hidden_size == 0 || target->vocab_size == 0 || target->n_layer == 0)
@@ -731,4 +737,13 @@ extern "C" int32_t dflash_gguf_open_drafter(dflash_gguf *g, const dflash_target_
         Y.is_swa = pattern[i] != 0;
     }
     return L.rc;
+}
+
+extern "C" int32_t dflash_gguf_open_drafter(dflash_gguf *g, const dflash_target_shape *target, dflash_gguf_draft_head *out,
+                                            dflash_gguf_draft_layer *layers, int32_t layer_cap) {
+    try {
+        return open_drafter_impl(g, target, out, layers, layer_cap);
+    } catch (const std::exception &e) {  // nothing may cross the C boundary
+        return g ? fail(g, DFLASH_ERR_IO, "open_drafter: %s", e.what()) : DFLASH_ERR_IO;
+    }
 }
