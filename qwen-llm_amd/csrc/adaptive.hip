@@ -110,7 +110,7 @@ void dflash_adaptive_record_spec_step(dflash_adaptive_state *s, int32_t n_accept
         for (int i = 0; i < s->n_fallback; i++) ran += s->fallback_window[i];
         const bool fallback_losing = s->n_fallback == kLongFallbackWindow && ran >= kLongFallbackLimit;
         bool early_fallback_losing = false;
-        if (s->n_fallback >= kLongFallbackEarlyWindow) {
+        if (s->n_fallback >= kLongFallbackEarlyWindow && s->n_alpha >= kLongFallbackEarlyWindow) {
             int early = 0;
             int64_t acc = 0;
             for (int i = s->n_fallback - kLongFallbackEarlyWindow; i < s->n_fallback; i++) early += s->fallback_window[i];
