@@ -226,6 +226,42 @@ def e2e_speculative(ctx, n_generate, sweep, log):
             "accept_ms": st["accept_ms"] / st["spec_steps"], "append_ms": st["append_ms"] / st["spec_steps"],
             "tokens_equal_serial_greedy": agree, "tokens": len(tokens)})
         log(f"e2e: forced k={k}: {res['sweep'][-1]}")
+
+    # Stochastic acceptance (sampler coupled to deterministic drafts), forced the same way: the serial sampler's own
+    # stream (temperature 0.7, top-k 20, top-p 0.95, one draw per token, through the same kernels) supplies the first
+    # k drafts of every block.  Shorter run: the serial stream costs one full decode step per token.
+    n_s, k = min(n_generate, 256), 7
+    kw = dict(temperature=0.7, top_k=20, top_p=0.95, min_p=0.0, seed=1)
+    samp = dfl.Sampler(**kw)
+    serial = dfl.Session(ctx, target, cap, taps)
+    for s0 in range(0, prompt_len, 16):
+        out = serial.encode_packed_verify_layer_major(prompt[s0:s0 + 16], s0, want_hidden=False)
+    stream = [out.argmax_host[-1]]
+    while len(stream) < n_s + 16:
+        out = serial.encode_packed_verify_layer_major([stream[-1]], prompt_len + len(stream) - 1, want_logits=True,
+                                                       want_hidden=False)
+        stream.append(ctx.decide_dflash_accept_prefix([stream[-1]], out.logits, cfg.vocab, None, samp, 1 << 30, []).carry_token)
+    serial.close()
+    dec = dfl.SpeculativeDecoder(ctx, target, head, taps, cap, mask, sampler=dfl.Sampler(**kw))
+    first = dec.prefill(prompt)
+
+    def override_s(tokens, position):
+        done = len(tokens)
+        return stream[done:done + k] + [(t + 1) % (cfg.vocab - 1) for t in stream[done + k:done + 15]]
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    tokens, st = dec.generate(first, n_s, draft_override_fn=override_s)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    dec.close()
+    res["sampled"] = {
+        "forced_k": k, "sampling": kw, "accepted_tokens_per_s": (len(tokens) - 1) / dt, "steps": st["spec_steps"],
+        "mean_accept_len": st["accepted_drafts"] / max(st["spec_steps"], 1), "ms_per_step": dt * 1e3 / max(st["spec_steps"], 1),
+        "draft_ms": st["draft_ms"] / st["spec_steps"], "verify_ms": st["verify_ms"] / st["spec_steps"],
+        "accept_ms": st["accept_ms"] / st["spec_steps"],
+        "tokens_equal_serial_sampler": sum(int(a == b) for a, b in zip(tokens, stream)), "tokens": len(tokens)}
+    log(f"e2e: sampled, forced k={k}: {res['sampled']}")
     return res
 
 
