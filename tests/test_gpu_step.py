@@ -325,3 +325,29 @@ def test_position_margin_follows_the_reference_rule(ctx, world):
     assert tokens == cont[:24]
     assert abs(dec.cfg.fallback_margin - 0.1) < 1e-7  # below 16384 positions (qwen/dflash.rs:126-136)
     dec.close()
+
+
+@pytest.mark.parametrize("k", [0, 5, 15])
+def test_baseline_plumbing_case_prefix_512(ctx, world, k):
+    """The first BASELINE configuration at its own sizes: 4-layer decoder, a prefix of 512 uniform-random tokens
+    (seed 0) prefilled into the f16 KV cache, one 16-token block whose first k drafts are copied from the target's
+    own continuation: the accepted prefix is exactly k and the next token is the target's.  The expectation is the
+    token-by-token decode through the same kernels (the CPU oracle pins those on the short prompt above)."""
+    prompt = np.random.default_rng(0).integers(0, C1.vocab - 1, 512).tolist()
+    serial = dfl.Session(ctx, world["model"], 640, TAPS)
+    out = None
+    for s in range(0, 512, 16):
+        out = serial.encode_packed_verify_layer_major(prompt[s:s + 16], s)
+    cont = [out.argmax_host[-1]]
+    while len(cont) < 17:
+        cont.append(serial.encode_packed_verify_layer_major([cont[-1]], 512 + len(cont) - 1).argmax_host[0])
+    serial.close()
+    dec = dfl.SpeculativeDecoder(ctx, world["model"], world["head"], TAPS, 640, MASK)
+    first = dec.prefill(prompt)
+    assert first == cont[0] and dec.session.kv_n_pos == 512 == dec.draft_session.ctx_len
+    wrong = [(t + 1) % (C1.vocab - 1) for t in cont[1:16]]
+    res = dec.step(first, budget=1000, draft_override=cont[1:1 + k] + wrong[k:])
+    d = res.decision
+    assert d.n_accepted == k and list(d.accepted_drafts[:k]) == cont[1:1 + k] and d.carry_token == cont[k + 1]
+    assert dec.session.kv_n_pos == 512 + k + 1 == dec.position == dec.draft_session.ctx_len
+    dec.close()
