@@ -328,9 +328,137 @@ __device__ bool in_list(const int32_t *ids, int n, int32_t v) {
     return false;
 }
 
-// accept.rs:147-183 with the couplings of sampling.rs:692-790; one thread.
+// What one row of the walk comes to, given that every row before it accepted.
+struct RowOutcome {
+    int32_t acc;         // the draft is accepted (draft rows only)
+    int32_t token;       // correction token (rejected draft row) or bonus token (last row)
+    int32_t draws;       // random draws this row consumes
+    int32_t err;         // DFLASH_ERR_* of this row, 0 if none
+    int64_t err_index;
+};
+
+// One row of accept.rs:147-183 with the couplings of sampling.rs:692-790.  A row that is reached has seen only
+// accepting rows before it, and an accepting row consumes exactly one draw (none when greedy): row r therefore
+// starts at draw r whatever the rows before it held, which is what lets every row be evaluated at once.
+__device__ RowOutcome decide_row(const DecideArgs &a, int row, const double *p_total) {
+    RowOutcome o = {0, 0, 0, 0, -1};
+    const int n_drafts = a.n_tokens - 1;
+    const bool greedy = a.temperature == 0.0f;
+    const RowDist &rd = a.rows[row];
+    int draws = greedy ? 0 : row;
+    const int draws0 = draws;
+    if (row == n_drafts) {  // bonus = sample(last reached row)
+        if (rd.err) {
+            o.err = rd.err;
+            o.err_index = rd.err_index;
+            return o;
+        }
+        int idx = 0;
+        if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
+        o.token = rd.tokens[idx];
+        o.draws = draws - draws0;
+        return o;
+    }
+    const int32_t draft = a.verified[row + 1];
+    if (a.mode == 0) {  // deterministic coupling: draw the target token, accept iff it is the draft
+        if (rd.err) {
+            o.err = rd.err;
+            o.err_index = rd.err_index;
+            return o;
+        }
+        int idx = 0;
+        if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
+        o.token = rd.tokens[idx];
+        o.acc = o.token == draft;
+        o.draws = draws - draws0;
+        return o;
+    }
+    // proposal probability q(draft) and, per target candidate, q(candidate)
+    double prop_total = 0.0, prop_tok_w = 0.0;
+    const dflash_weighted_candidate *pc = nullptr;
+    int n_pc = 0;
+    if (a.mode == 1) {
+        pc = a.prop_cands + a.prop_offsets[row];
+        n_pc = a.prop_counts[row];
+        if (n_pc == 0) o.err = DFLASH_ERR_NO_CANDIDATES;
+        for (int j = 0; j < n_pc && !o.err; j++) {
+            if (!isfinite(pc[j].weight) || pc[j].weight < 0.0) {
+                o.err = DFLASH_ERR_INVALID_PROPOSAL_WEIGHT;
+                o.err_index = pc[j].token;
+                break;
+            }
+            prop_total += pc[j].weight;
+            if (pc[j].token == draft) prop_tok_w += pc[j].weight;
+        }
+        if (!o.err && !(isfinite(prop_total) && prop_total > 0.0)) o.err = DFLASH_ERR_NO_CANDIDATES;
+        if (!o.err && !(isfinite(prop_tok_w) && prop_tok_w > 0.0)) {
+            o.err = DFLASH_ERR_MISSING_PROPOSAL_TOKEN;
+            o.err_index = draft;
+        }
+    } else {
+        if (rd.d_err) {
+            o.err = rd.d_err;
+            o.err_index = rd.d_err_index;
+        }
+        prop_total = p_total[row];
+        if (!o.err && !(isfinite(prop_total) && prop_total > 0.0)) o.err = DFLASH_ERR_NO_CANDIDATES;
+        if (!o.err) {
+            prop_tok_w = exp(static_cast<double>(a.draft[row * a.draft_stride + draft]) / static_cast<double>(a.draft_temperature) -
+                             rd.d_max_scaled);
+            if (!(isfinite(prop_tok_w) && prop_tok_w > 0.0)) {
+                o.err = DFLASH_ERR_MISSING_PROPOSAL_TOKEN;
+                o.err_index = draft;
+            }
+        }
+    }
+    if (!o.err && rd.err) {
+        o.err = rd.err;
+        o.err_index = rd.err_index;
+    }
+    if (o.err) return o;
+    double tp = -0.0;
+    for (int i = 0; i < rd.n_keep; i++)
+        if (rd.tokens[i] == draft) tp += rd.weights[i];
+    const double target_probability = tp / rd.total;
+    const double proposal_probability = prop_tok_w / prop_total;
+    const double acceptance = fmin(target_probability / proposal_probability, 1.0);
+    if (a.uniforms[draws++] < acceptance) {
+        o.acc = 1;
+    } else {
+        double residual[kMaxK];
+        double residual_total = 0.0;
+        for (int i = 0; i < rd.n_keep; i++) {
+            const double p = rd.weights[i] / rd.total;
+            double q;
+            if (a.mode == 1) {
+                double qs = -0.0;
+                for (int j = 0; j < n_pc; j++)
+                    if (pc[j].token == rd.tokens[i]) qs += pc[j].weight;
+                q = qs / prop_total;
+            } else {
+                q = exp(static_cast<double>(a.draft[row * a.draft_stride + rd.tokens[i]]) / static_cast<double>(a.draft_temperature) -
+                        rd.d_max_scaled) /
+                    prop_total;
+            }
+            const double wgt = fmax(p - q, 0.0);
+            residual_total += wgt;
+            residual[i] = wgt;
+        }
+        if (!(isfinite(residual_total) && residual_total > 0.0)) {
+            o.err = DFLASH_ERR_NO_CANDIDATES;
+            return o;
+        }
+        o.token = rd.tokens[pick_index(residual, rd.n_keep, a.uniforms[draws++] * residual_total)];
+    }
+    o.draws = draws - draws0;
+    return o;
+}
+
+// Thread r evaluates row r (all rows at once); thread 0 then walks the outcomes in order exactly as the serial
+// loop of accept.rs:147-183 does: rows behind the first rejection, stop or error are never looked at.
 __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__ out) {
     __shared__ double p_total[kMaxRows];
+    __shared__ RowOutcome outcome[kMaxRows + 1];
     const int n_drafts = a.n_tokens - 1;
     if (a.mode == 2 && static_cast<int>(threadIdx.x) < n_drafts) {
         // P = sequential sum of the tile sums, tile order
@@ -339,6 +467,8 @@ __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__
         p_total[threadIdx.x] = P;
     }
     __syncthreads();
+    if (static_cast<int>(threadIdx.x) <= n_drafts) outcome[threadIdx.x] = decide_row(a, threadIdx.x, p_total);
+    __syncthreads();
     if (threadIdx.x != 0) return;
     dflash_accept_decision d;
     memset(&d, 0, sizeof(d));
@@ -346,128 +476,27 @@ __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__
     d.err_index = -1;
     int accepted = 0, draws = 0, carry_kind = DFLASH_CARRY_NONE, stop = DFLASH_STOP_NONE, carry_token = 0;
     int err = 0;
-    const bool greedy = a.temperature == 0.0f;
     for (;;) {
         const int row = accepted;
-        const RowDist &rd = a.rows[row];
-        if (row == n_drafts) {  // bonus = sample(last reached row)
-            if (rd.err) {
-                err = rd.err;
-                d.err_index = rd.err_index;
-                d.err_row = row;
-                break;
-            }
-            int idx = 0;
-            if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
+        const RowOutcome &o = outcome[row];
+        if (o.err) {
+            err = o.err;
+            d.err_index = o.err_index;
+            d.err_row = row;
+            break;
+        }
+        draws += o.draws;
+        if (row == n_drafts) {
             carry_kind = DFLASH_CARRY_BONUS;
-            carry_token = rd.tokens[idx];
+            carry_token = o.token;
+            break;
+        }
+        if (!o.acc) {
+            carry_kind = DFLASH_CARRY_CORRECTION;
+            carry_token = o.token;
             break;
         }
         const int32_t draft = a.verified[row + 1];
-        bool acc = false;
-        int32_t correction = 0;
-        if (a.mode == 0) {  // deterministic coupling: draw the target token, accept iff it is the draft
-            if (rd.err) {
-                err = rd.err;
-                d.err_index = rd.err_index;
-                d.err_row = row;
-                break;
-            }
-            int idx = 0;
-            if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
-            correction = rd.tokens[idx];
-            acc = correction == draft;
-        } else {
-            // proposal probability q(draft) and, per target candidate, q(candidate)
-            double prop_total = 0.0, prop_tok_w = 0.0;
-            const dflash_weighted_candidate *pc = nullptr;
-            int n_pc = 0;
-            if (a.mode == 1) {
-                pc = a.prop_cands + a.prop_offsets[row];
-                n_pc = a.prop_counts[row];
-                if (n_pc == 0) err = DFLASH_ERR_NO_CANDIDATES;
-                for (int j = 0; j < n_pc && !err; j++) {
-                    if (!isfinite(pc[j].weight) || pc[j].weight < 0.0) {
-                        err = DFLASH_ERR_INVALID_PROPOSAL_WEIGHT;
-                        d.err_index = pc[j].token;
-                        break;
-                    }
-                    prop_total += pc[j].weight;
-                    if (pc[j].token == draft) prop_tok_w += pc[j].weight;
-                }
-                if (!err && !(isfinite(prop_total) && prop_total > 0.0)) err = DFLASH_ERR_NO_CANDIDATES;
-                if (!err && !(isfinite(prop_tok_w) && prop_tok_w > 0.0)) {
-                    err = DFLASH_ERR_MISSING_PROPOSAL_TOKEN;
-                    d.err_index = draft;
-                }
-            } else {
-                if (rd.d_err) {
-                    err = rd.d_err;
-                    d.err_index = rd.d_err_index;
-                }
-                prop_total = p_total[row];
-                if (!err && !(isfinite(prop_total) && prop_total > 0.0)) err = DFLASH_ERR_NO_CANDIDATES;
-                if (!err) {
-                    prop_tok_w = exp(static_cast<double>(a.draft[row * a.draft_stride + draft]) /
-                                         static_cast<double>(a.draft_temperature) -
-                                     rd.d_max_scaled);
-                    if (!(isfinite(prop_tok_w) && prop_tok_w > 0.0)) {
-                        err = DFLASH_ERR_MISSING_PROPOSAL_TOKEN;
-                        d.err_index = draft;
-                    }
-                }
-            }
-            if (!err && rd.err) {
-                err = rd.err;
-                d.err_index = rd.err_index;
-            }
-            if (err) {
-                d.err_row = row;
-                break;
-            }
-            double tp = -0.0;
-            for (int i = 0; i < rd.n_keep; i++)
-                if (rd.tokens[i] == draft) tp += rd.weights[i];
-            const double target_probability = tp / rd.total;
-            const double proposal_probability = prop_tok_w / prop_total;
-            const double acceptance = fmin(target_probability / proposal_probability, 1.0);
-            if (a.uniforms[draws++] < acceptance) {
-                acc = true;
-            } else {
-                double residual[kMaxK];
-                double residual_total = 0.0;
-                for (int i = 0; i < rd.n_keep; i++) {
-                    const double p = rd.weights[i] / rd.total;
-                    double q;
-                    if (a.mode == 1) {
-                        double qs = -0.0;
-                        for (int j = 0; j < n_pc; j++)
-                            if (pc[j].token == rd.tokens[i]) qs += pc[j].weight;
-                        q = qs / prop_total;
-                    } else {
-                        q = exp(static_cast<double>(a.draft[row * a.draft_stride + rd.tokens[i]]) /
-                                    static_cast<double>(a.draft_temperature) -
-                                rd.d_max_scaled) /
-                            prop_total;
-                    }
-                    const double wgt = fmax(p - q, 0.0);
-                    residual_total += wgt;
-                    residual[i] = wgt;
-                }
-                if (!(isfinite(residual_total) && residual_total > 0.0)) {
-                    err = DFLASH_ERR_NO_CANDIDATES;
-                    d.err_row = row;
-                    draws--;  // reported only; nothing is committed on an error
-                    break;
-                }
-                correction = rd.tokens[pick_index(residual, rd.n_keep, a.uniforms[draws++] * residual_total)];
-            }
-        }
-        if (!acc) {
-            carry_kind = DFLASH_CARRY_CORRECTION;
-            carry_token = correction;
-            break;
-        }
         d.accepted_drafts[accepted++] = draft;
         if (in_list(a.stop_ids, a.n_stop, draft)) {
             stop = DFLASH_STOP_EOS;
