@@ -460,11 +460,23 @@ __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__
     __shared__ double p_total[kMaxRows];
     __shared__ RowOutcome outcome[kMaxRows + 1];
     const int n_drafts = a.n_tokens - 1;
-    if (a.mode == 2 && static_cast<int>(threadIdx.x) < n_drafts) {
-        // P = sequential sum of the tile sums, tile order
+    if (a.mode == 2) {
+        // P = sequential sum of a row's tile sums, in tile order.  The sums come through LDS 64 tiles at a time
+        // (all threads load, coalesced and independent), so that the ordered additions of thread r do not each
+        // wait for a load from memory.
+        __shared__ double staged[kMaxRows][64];
         double P = 0.0;
-        for (int t = 0; t < a.n_tiles; t++) P += a.tile_sums[threadIdx.x * a.n_tiles + t];
-        p_total[threadIdx.x] = P;
+        for (int t0 = 0; t0 < a.n_tiles; t0 += 64) {
+            const int t = t0 + static_cast<int>(threadIdx.x);
+            for (int r = 0; r < n_drafts; r++) staged[r][threadIdx.x] = t < a.n_tiles ? a.tile_sums[r * a.n_tiles + t] : 0.0;
+            __syncthreads();
+            if (static_cast<int>(threadIdx.x) < n_drafts) {
+                const int n = min(64, a.n_tiles - t0);
+                for (int i = 0; i < n; i++) P += staged[threadIdx.x][i];
+            }
+            __syncthreads();
+        }
+        if (static_cast<int>(threadIdx.x) < n_drafts) p_total[threadIdx.x] = P;
     }
     __syncthreads();
     if (static_cast<int>(threadIdx.x) <= n_drafts) outcome[threadIdx.x] = decide_row(a, threadIdx.x, p_total);
