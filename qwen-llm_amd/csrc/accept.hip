@@ -202,6 +202,8 @@ __global__ void __launch_bounds__(kSelThreads)
     row_merge_kernel(const ChunkOut *__restrict__ chunks, int n_chunks, const ChunkOut *__restrict__ draft_chunks,
                      ChainCfg cfg, RowDist *__restrict__ rows, int32_t *__restrict__ greedy_out) {
     __shared__ uint64_t sk[2 * kSelThreads];
+    __shared__ double chain_l[kMaxK], chain_w[kMaxK];
+    __shared__ int chain_tok[kMaxK];
     const int row = blockIdx.x, tid = threadIdx.x;
     const int k = cfg.k;
     const int n_in = n_chunks * k;  // <= 2048, checked on the host
@@ -239,7 +241,7 @@ __global__ void __launch_bounds__(kSelThreads)
     } else {
         int len = 0;
         while (len < k && sk[len] != kNoKey) len++;
-        run_chain(sk, len, cfg, d);
+        run_chain(sk, len, cfg, d, ChainScratch{chain_l, chain_w, chain_tok});
     }
     if (draft_chunks) {
         uint64_t best = kNoKey;
@@ -340,11 +342,11 @@ struct RowOutcome {
 // One row of accept.rs:147-183 with the couplings of sampling.rs:692-790.  A row that is reached has seen only
 // accepting rows before it, and an accepting row consumes exactly one draw (none when greedy): row r therefore
 // starts at draw r whatever the rows before it held, which is what lets every row be evaluated at once.
-__device__ RowOutcome decide_row(const DecideArgs &a, int row, const double *p_total) {
+__device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int row, const double *p_total) {
     RowOutcome o = {0, 0, 0, 0, -1};
     const int n_drafts = a.n_tokens - 1;
     const bool greedy = a.temperature == 0.0f;
-    const RowDist &rd = a.rows[row];
+    const RowDist &rd = rows[row];
     int draws = greedy ? 0 : row;
     const int draws0 = draws;
     if (row == n_drafts) {  // bonus = sample(last reached row)
@@ -459,6 +461,15 @@ __device__ RowOutcome decide_row(const DecideArgs &a, int row, const double *p_t
 __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__ out) {
     __shared__ double p_total[kMaxRows];
     __shared__ RowOutcome outcome[kMaxRows + 1];
+    // the rows' distributions are walked element by element: they are copied to LDS once, coalesced
+    __shared__ RowDist rows_sh[kMaxRows];
+    static_assert(sizeof(RowDist) % 4 == 0, "copied as words");
+    {
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(a.rows);
+        uint32_t *dst = reinterpret_cast<uint32_t *>(rows_sh);
+        const int n_words = a.n_tokens * static_cast<int>(sizeof(RowDist) / 4);
+        for (int i = threadIdx.x; i < n_words; i += blockDim.x) dst[i] = src[i];
+    }
     const int n_drafts = a.n_tokens - 1;
     if (a.mode == 2) {
         // P = sequential sum of a row's tile sums, in tile order.  The sums come through LDS 64 tiles at a time
@@ -479,7 +490,7 @@ __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__
         if (static_cast<int>(threadIdx.x) < n_drafts) p_total[threadIdx.x] = P;
     }
     __syncthreads();
-    if (static_cast<int>(threadIdx.x) <= n_drafts) outcome[threadIdx.x] = decide_row(a, threadIdx.x, p_total);
+    if (static_cast<int>(threadIdx.x) <= n_drafts) outcome[threadIdx.x] = decide_row(a, rows_sh, threadIdx.x, p_total);
     __syncthreads();
     if (threadIdx.x != 0) return;
     dflash_accept_decision d;

@@ -59,9 +59,16 @@ struct ChainCfg {
 };
 
 // sampling.rs:1541-1615 on the ordered candidates of one row (keys ascending = best first)
-__device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowDist *d) {
-    double l[kMaxK];
-    int tok[kMaxK];
+// Work arrays of the chain (kMaxK entries each): a caller that runs the chain on one thread of a workgroup
+// keeps them in LDS; private arrays of this size live in scratch memory, where every access is a trip to memory.
+struct ChainScratch {
+    double *l, *w;
+    int *tok;
+};
+
+__device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowDist *d, const ChainScratch &scratch) {
+    double *l = scratch.l;
+    int *tok = scratch.tok;
     for (int i = 0; i < len; i++) {
         l[i] = static_cast<double>(key_logit(keys[i]));
         tok[i] = key_token(keys[i]);
@@ -96,7 +103,7 @@ __device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowD
     }
     const double temperature = static_cast<double>(c.temperature);
     for (int i = 0; i < len; i++) l[i] /= temperature;
-    double w[kMaxK];
+    double *w = scratch.w;
     int n_inf = 0;
     for (int i = 0; i < len; i++) n_inf += (l[i] == INFINITY);
     if (n_inf > 0) {
@@ -142,6 +149,13 @@ __device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowD
         d->tokens[i] = tok[i];
         d->weights[i] = w[i];
     }
+}
+
+// the same with private work arrays
+__device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowDist *d) {
+    double l[kMaxK], w[kMaxK];
+    int tok[kMaxK];
+    run_chain(keys, len, c, d, ChainScratch{l, w, tok});
 }
 
 // first candidate whose running sum exceeds x, else the last (sampling.rs:1587-1596)
