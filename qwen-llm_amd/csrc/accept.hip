@@ -309,12 +309,13 @@ __global__ void __launch_bounds__(256) dense_tile_sum_kernel(const float *__rest
 struct DecideArgs {
     int32_t n_tokens, n_stop, mode, vocab;
     int64_t budget;
-    const int32_t *verified;   // [n_tokens]
+    // The block's small host inputs travel by value, in the kernel arguments: a pageable host-to-device copy
+    // of a few bytes costs several microseconds of idle GPU each.
+    int32_t verified[kMaxRows];      // [n_tokens]
+    double uniforms[kMaxRows + 2];   // [n_tokens + 1]
+    int32_t prop_offsets[kMaxRows], prop_counts[kMaxRows];  // sparse proposals: row r's candidates in prop_cands
     const int32_t *stop_ids;   // [n_stop]
-    const double *uniforms;    // [n_tokens + 1]
     const RowDist *rows;
-    // sparse proposals
-    const int32_t *prop_tokens, *prop_offsets, *prop_counts;
     const dflash_weighted_candidate *prop_cands;
     // dense proposals
     const float *draft;
@@ -794,29 +795,22 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
     ChunkOut *dchunks = dfl_ws_take<ChunkOut>(ctx, &off, sizeof(ChunkOut) * n_tokens * n_chunks);
     RowDist *rows = dfl_ws_take<RowDist>(ctx, &off, sizeof(RowDist) * n_tokens);
     double *tile_sums = dfl_ws_take<double>(ctx, &off, sizeof(double) * n_tokens * n_tiles);
-    double *d_uniforms = dfl_ws_take<double>(ctx, &off, sizeof(double) * (kMaxRows + 2));
-    int32_t *d_small = dfl_ws_take<int32_t>(ctx, &off, sizeof(int32_t) * (4 * kMaxRows + n_stop + 8));
+    int32_t *d_stop = dfl_ws_take<int32_t>(ctx, &off, sizeof(int32_t) * (n_stop + 8));
     dflash_weighted_candidate *d_cands =
         dfl_ws_take<dflash_weighted_candidate>(ctx, &off, sizeof(dflash_weighted_candidate) * (n_cands + 1));
     dflash_accept_decision *d_out = dfl_ws_take<dflash_accept_decision>(ctx, &off, sizeof(dflash_accept_decision));
-    if (!chunks || !dchunks || !rows || !tile_sums || !d_uniforms || !d_small || !d_cands || !d_out)
+    if (!chunks || !dchunks || !rows || !tile_sums || !d_stop || !d_cands || !d_out)
         return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "accept_prefix: workspace too small");
 
-    // small host inputs -> device
-    double uniforms[kMaxRows + 2];
-    dflash_sampler_peek(sampler, n_tokens + 1, uniforms);
-    int32_t small[4 * kMaxRows + 8];
-    int32_t *h_verified = small, *h_ptok = small + kMaxRows, *h_poff = small + 2 * kMaxRows, *h_pcnt = small + 3 * kMaxRows;
-    memset(small, 0, sizeof(small));
-    for (int i = 0; i < n_tokens; i++) h_verified[i] = verified[i];
+    // small host inputs: by value in the decision kernel's arguments; only the variable-length lists are copied
+    DecideArgs a;
+    memset(&a, 0, sizeof(a));
+    dflash_sampler_peek(sampler, n_tokens + 1, a.uniforms);
+    for (int i = 0; i < n_tokens; i++) a.verified[i] = verified[i];
     for (int r = 0; r < n_drafts && mode == 1; r++) {
-        h_ptok[r] = prop_tokens[r];
-        h_poff[r] = prop_offsets[r];
-        h_pcnt[r] = prop_counts[r];
+        a.prop_offsets[r] = prop_offsets[r];
+        a.prop_counts[r] = prop_counts[r];
     }
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(d_uniforms, uniforms, sizeof(double) * (n_tokens + 1), hipMemcpyHostToDevice, st));
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(d_small, small, sizeof(int32_t) * 4 * kMaxRows, hipMemcpyHostToDevice, st));
-    int32_t *d_stop = d_small + 4 * kMaxRows;
     if (n_stop > 0)
         DFL_HIP_CHECK(ctx, hipMemcpyAsync(d_stop, stop_ids, sizeof(int32_t) * n_stop, hipMemcpyHostToDevice, st));
     if (n_cands > 0)
@@ -840,19 +834,13 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
                                                           cfg, rows, nullptr);
         if (mode == 2 && n_drafts > 0)
             dense_tile_sum_kernel<<<dim3(n_tiles, n_drafts), 256, 0, st>>>(draft_logits, vocab, vocab, draft_temperature, rows, tile_sums);
-        DecideArgs a;
         a.n_tokens = n_tokens;
         a.n_stop = n_stop;
         a.mode = mode;
         a.vocab = static_cast<int32_t>(vocab);
         a.budget = budget;
-        a.verified = d_small;
         a.stop_ids = d_stop;
-        a.uniforms = d_uniforms;
         a.rows = rows;
-        a.prop_tokens = d_small + kMaxRows;
-        a.prop_offsets = d_small + 2 * kMaxRows;
-        a.prop_counts = d_small + 3 * kMaxRows;
         a.prop_cands = d_cands;
         a.draft = draft_logits;
         a.draft_stride = vocab;
