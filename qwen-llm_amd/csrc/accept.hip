@@ -851,8 +851,10 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
         decide_kernel<<<1, 64, 0, st>>>(a, d_out);
     }
     DFL_HIP_CHECK(ctx, hipGetLastError());
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(out, d_out, sizeof(*out), hipMemcpyDeviceToHost, st));
+    static_assert(sizeof(dflash_accept_decision) <= DFL_PINNED_BYTES, "the decision is read back through the pinned page");
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(ctx->pinned, d_out, sizeof(*out), hipMemcpyDeviceToHost, st));
     DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+    memcpy(out, ctx->pinned, sizeof(*out));
     if (out->err_code) {
         int32_t code = out->err_code;
         return dfl_fail(ctx, code, "DFlash target row %d: %s (index %lld)", out->err_row, dflash_status_name(code),

@@ -31,7 +31,11 @@ struct dflash_ctx {
     bool graphs = false;
     hipStream_t gstream = nullptr;
     hipEvent_t g_in = nullptr, g_out = nullptr;
+    // pinned host staging for the few words a blocking call reads back (a device-to-host copy into pageable
+    // memory is staged by the runtime and costs several microseconds each); one page, owned
+    void *pinned = nullptr;
 };
+enum { DFL_PINNED_BYTES = 4096 };
 
 // Slots of the per-kernel timers.
 enum { DFL_T_GEMM = 0, DFL_T_ATTN = 1, DFL_T_ACCEPT = 2, DFL_T_ARGMAX = 3, DFL_T_REDUCE = 4 };

@@ -52,6 +52,11 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
         dflash_ctx_destroy(ctx);
         return DFLASH_ERR_HIP;
     }
+    if (hipHostMalloc(&ctx->pinned, DFL_PINNED_BYTES, hipHostMallocDefault) != hipSuccess) {
+        ctx->pinned = nullptr;
+        dflash_ctx_destroy(ctx);
+        return DFLASH_ERR_HIP;
+    }
     if (const char *e = getenv("DFLASH_GRAPHS")) ctx->graphs = atoi(e) != 0;
     *out = ctx;
     return DFLASH_OK;
@@ -66,6 +71,7 @@ void dflash_ctx_destroy(dflash_ctx *ctx) {
     if (ctx->g_in) (void)hipEventDestroy(ctx->g_in);
     if (ctx->g_out) (void)hipEventDestroy(ctx->g_out);
     if (ctx->gstream) (void)hipStreamDestroy(ctx->gstream);
+    if (ctx->pinned) (void)hipHostFree(ctx->pinned);
     delete ctx;
 }
 

@@ -1185,10 +1185,16 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
                                     sess->hidden, nullptr, nullptr, st)))
             return rc;
         if (timed) DFL_HIP_CHECK(ctx, hipEventRecord(ctx->ev1, st));
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(res->verify_argmax, sess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(res->verify_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost, st));
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(res->draft_tokens, dsess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        // read back through the context's pinned page: three truly asynchronous copies, one wait
+        int32_t *pin_argmax = static_cast<int32_t *>(ctx->pinned), *pin_draft = pin_argmax + 16;
+        float *pin_gap = reinterpret_cast<float *>(pin_argmax + 32);
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(pin_argmax, sess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(pin_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(pin_draft, dsess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
         DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        memcpy(res->verify_argmax, pin_argmax, N * sizeof(int32_t));
+        memcpy(res->verify_gap, pin_gap, N * sizeof(float));
+        memcpy(res->draft_tokens, pin_draft, N * sizeof(int32_t));
         const double wall_ms = enqueue_draft_ms + ms_since(t0);
         // the wall time of the two phases, split by the GPU time of the verify
         float verify_gpu_ms = 0.0f;
