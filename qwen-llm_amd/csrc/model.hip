@@ -626,8 +626,9 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
     }
     s->kv_n_pos = start + n;
     if (argmax_host) {
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(argmax_host, am, n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(ctx->pinned, am, n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
         DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        memcpy(argmax_host, ctx->pinned, n * sizeof(int32_t));
     }
     return DFLASH_OK;
 }
@@ -955,8 +956,9 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
     s->ctx_h_ready = s->ctx_len;
     s->kv_ready = s->ctx_len;
     if (argmax_host) {
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(argmax_host, am, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        DFL_HIP_CHECK(ctx, hipMemcpyAsync(ctx->pinned, am, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
         DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        memcpy(argmax_host, ctx->pinned, N * sizeof(int32_t));
     }
     return DFLASH_OK;
 }
