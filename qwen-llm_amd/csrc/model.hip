@@ -749,6 +749,7 @@ int32_t draft_prepare(dflash_ctx *ctx, const dflash_draft_head *head, dflash_dra
         if ((rc = gemm(ctx, head->fc, s->ctx_raw + c0 * feat, s->tmp, feat, H, m, st))) return rc;
         rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, nullptr, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps, nullptr, nullptr);
     }
+    const float *pending_resid = nullptr;
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_draft_layer &L = head->layers[il];
         float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
@@ -867,13 +868,15 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
     set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, N, s->ids, s->pos, nullptr, 0);
     if ((rc = embed_rows(ctx, target->token_embd, s->ids, N, H, s->x, st))) return rc;
 
+    const float *pending_resid = nullptr;
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_draft_layer &L = head->layers[il];
         float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
         float *vc = s->v_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
         _Float16 *k16 = s->k16 + il * static_cast<size_t>(s->cap16) * kv_dim;
         _Float16 *vt16 = s->vt16 + il * static_cast<size_t>(s->cap16) * kv_dim;
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
+        // the previous layer's second residual (x += ffn output) is folded into this norm
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
         // DFlash-2 attention convolution (metal_dflash.rs:16210-16262): the dynamic coefficients come
         // from the normed input and serve both sides; q/k/v read the side-0 result
         const float *attn_src = s->cur;
@@ -887,19 +890,21 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         bool packed;  // only on the fast path: the general attention kernel reads V dense
         if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, attn_src, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st))) return rc;
         const int64_t tot = q_dim + 2 * kv_dim;
-        qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(
-            packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
-            L.k_norm, nullptr, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, nullptr, 0, nullptr, 0);
         if (fast) {
-            // the block's own K/V go behind the context in the f16 mirror; one MFMA pass over both
-            kv_to_f16_kernel<<<dim3(blocks_for(kv_dim), N), 256, 0, st>>>(s->k, packed ? s->pk + q_dim + kv_dim : s->v,
-                                                                          packed ? tot : kv_dim, k16, vt16, static_cast<int>(kv_dim),
-                                                                          s->cap16, s->ctx_len, nullptr);
+            // the block's own K (normed, rotated) and V go behind the context in the f16 mirror, written by the
+            // same kernel (positions pos[i] = ctx_len + i on this path); one MFMA pass over context and block
+            qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, N), 64, 0, st>>>(
+                packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k,
+                L.q_norm, L.k_norm, k16, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, packed ? s->pk + q_dim + kv_dim : s->v,
+                packed ? tot : kv_dim, vt16, s->cap16);
             if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, k16, vt16, 1, s->ctx_len, N, c.n_q, c.n_kv, hd, s->cap16,
                                      1.0f / sqrtf(static_cast<float>(hd)), s->attn, st, c.causal ? 0 : 1,
                                      L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, nullptr)))
                 return rc;
         } else {
+            qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, q_dim, s->k, kv_dim, s->q, s->k, L.q_norm, L.k_norm,
+                                                                     nullptr, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta,
+                                                                     nullptr, 0, nullptr, 0);
             draft_attn_kernel<<<dim3(c.n_q, N), 64, 0, st>>>(s->q, kc, vc, s->k, s->v, s->pos_ctx, static_cast<int>(s->ctx_len),
                                                             N, c.n_q, c.n_kv, hd, static_cast<int>(noise_start), c.causal,
                                                             L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
@@ -932,9 +937,9 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                 return rc;
             resid = s->conv_buf;
         }
-        add_kernel<<<blocks_for(static_cast<size_t>(N) * H), 256, 0, st>>>(s->x, resid, static_cast<size_t>(N) * H);
+        pending_resid = resid;  // residual 2: added by the norm that reads x next (same x + r, one launch fewer)
     }
-    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, nullptr, head->output_norm, s->cur, H, c.eps, nullptr, nullptr);
+    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, head->output_norm, s->cur, H, c.eps, nullptr, nullptr);
     float *lg = draft_logits ? draft_logits : s->logits;
     if ((rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st))) return rc;
     int32_t *am = draft_argmax ? draft_argmax : s->argmax;
