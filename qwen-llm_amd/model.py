@@ -658,8 +658,13 @@ class SpeculativeDecoder:
         ov = None
         if draft_override is not None:
             ov = (C.c_int32 * (n - 1))(*(list(draft_override) + [-1] * (n - 1))[: n - 1])
-        taps = (C.c_int32 * len(self.tap_layers))(*self.tap_layers)
-        stops = (C.c_int32 * max(len(self.stop_ids), 1))(*self.stop_ids)
+        # the constant argument arrays are built once (rebuilt if the lists change)
+        key = (tuple(self.tap_layers), tuple(self.stop_ids))
+        if getattr(self, "_arg_key", None) != key:
+            self._arg_key = key
+            self._taps_c = (C.c_int32 * len(self.tap_layers))(*self.tap_layers)
+            self._stops_c = (C.c_int32 * max(len(self.stop_ids), 1))(*self.stop_ids)
+        taps, stops = self._taps_c, self._stops_c
         self.ctx._check(self._L.dflash_spec_step(
             self.ctx._h, C.byref(self.target.c), C.byref(self.head.c), self.session._h, self.draft_session._h, taps,
             len(self.tap_layers), carry, self.position, C.byref(self.cfg),
