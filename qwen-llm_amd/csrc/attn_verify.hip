@@ -431,18 +431,14 @@ __global__ void __launch_bounds__(256) transpose_v_kernel(const _Float16 *__rest
 }
 
 template <int HD, typename TQ>
-void launch_split(dim3 grid, int threads, hipStream_t st, const void *q, const _Float16 *k, const _Float16 *vt,
+int32_t launch_split(dflash_ctx *ctx, dim3 grid, int threads, hipStream_t st, const void *q, const _Float16 *k, const _Float16 *vt,
                   float *po, float *pml, int64_t ctx_len, const int32_t *ctx_len_dev, int n_rows, int n_q, int n_kv,
                   int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window) {
     const size_t lds = static_cast<size_t>(kAttnBufs) * 2 * (32 * HD / 8) * sizeof(half8_t);
 #define DFL_ATTN_LAUNCH(MAXW, HPW)                                                                                  \
     do {                                                                                                            \
-        static bool attr = false;                                                                                   \
-        if (!attr) {                                                                                                \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_split_kernel<HD, TQ, MAXW, HPW>),         \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));          \
-            attr = true;                                                                                            \
-        }                                                                                                           \
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(attn_split_kernel<HD, TQ, MAXW, HPW>), lds)) \
+            return rc_;                                                                                             \
         attn_split_kernel<HD, TQ, MAXW, HPW><<<grid, threads / HPW, lds, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, \
                                                                               ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
                                                                               vt_stride, want, min_chunk, scale,    \
@@ -455,6 +451,7 @@ void launch_split(dim3 grid, int threads, hipStream_t st, const void *q, const _
     else
         DFL_ATTN_LAUNCH(16, 1);
 #undef DFL_ATTN_LAUNCH
+    return DFLASH_OK;
 }
 
 }  // namespace
@@ -537,18 +534,20 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 #ifdef DFLASH_TRACE
     if (const char *e = getenv("DFLASH_DBG_VT_STRIDE")) vt_stride = atoi(e);  // timing experiment only: wrong results
 #endif
+    if (n_splits > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: %d KV splits", n_splits);
     const dim3 grid(n_splits, n_kv);
     const int threads = 64 * group;
     const _Float16 *k = static_cast<const _Float16 *>(k_cache);
+    int32_t rc = DFLASH_OK;
     {
         dfl_timed timer(ctx, st, DFL_T_ATTN);
 #define DFL_ATTN(HD)                                                                                              \
     if (q_type == DFLASH_TYPE_F32)                                                                                \
-        launch_split<HD, float>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
-                                vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window);         \
+        rc = launch_split<HD, float>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
+                                     vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window);    \
     else                                                                                                          \
-        launch_split<HD, _Float16>(grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, \
-                                   n_kv, vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window)
+        rc = launch_split<HD, _Float16>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, \
+                                        n_kv, vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window)
         if (head_dim == 64) {
             DFL_ATTN(64);
         } else if (head_dim == 128) {
@@ -558,7 +557,7 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
         }
 #undef DFL_ATTN
     }
-    if (n_splits > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: %d KV splits", n_splits);
+    if (rc) return rc;
     attn_combine_kernel<<<dim3(n_q, n_rows), 256, 0, st>>>(part_o, part_ml, out, n_rows, n_q, head_dim, ctx_len, ctx_len_dev, want,
                                                           static_cast<int>(min_chunk));
     DFL_HIP_CHECK(ctx, hipGetLastError());

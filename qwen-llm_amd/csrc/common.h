@@ -34,8 +34,13 @@ struct dflash_ctx {
     // pinned host staging for the few words a blocking call reads back (a device-to-host copy into pageable
     // memory is staged by the runtime and costs several microseconds each); one page, owned
     void *pinned = nullptr;
+    // kernels whose dynamic-LDS limit has already been raised for this context (the attribute is kept per
+    // device by the runtime, so the record lives with the context, not in process-wide flags)
+    const void *lds_attr_fn[96] = {nullptr};
+    size_t lds_attr_bytes[96] = {0};
+    int n_lds_attr = 0;
 };
-enum { DFL_PINNED_BYTES = 4096 };
+enum { DFL_PINNED_BYTES = 8192 };
 
 // Slots of the per-kernel timers.
 enum { DFL_T_GEMM = 0, DFL_T_ATTN = 1, DFL_T_ACCEPT = 2, DFL_T_ARGMAX = 3, DFL_T_REDUCE = 4 };
@@ -69,6 +74,10 @@ int32_t dfl_fail(dflash_ctx *ctx, int32_t status, const char *fmt, ...);
         if (e_ != hipSuccess)                                                             \
             return dfl_fail((ctx), DFLASH_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
     } while (0)
+
+// Makes sure kernel `fn` may be launched with `bytes` of dynamic LDS on the context's device
+// (hipFuncAttributeMaxDynamicSharedMemorySize), calling the runtime only the first time.
+int32_t dfl_raise_lds_limit(dflash_ctx *ctx, const void *fn, size_t bytes);
 
 // Carves `bytes` (256-aligned) out of the context workspace starting at *offset.
 template <typename T>

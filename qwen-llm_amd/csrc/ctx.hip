@@ -15,6 +15,23 @@ int32_t dfl_fail(dflash_ctx *ctx, int32_t status, const char *fmt, ...) {
     return status;
 }
 
+int32_t dfl_raise_lds_limit(dflash_ctx *ctx, const void *fn, size_t bytes) {
+    constexpr int kCap = static_cast<int>(sizeof(ctx->lds_attr_fn) / sizeof(ctx->lds_attr_fn[0]));
+    for (int i = 0; i < ctx->n_lds_attr; i++)
+        if (ctx->lds_attr_fn[i] == fn) {
+            if (ctx->lds_attr_bytes[i] >= bytes) return DFLASH_OK;
+            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+            ctx->lds_attr_bytes[i] = bytes;
+            return DFLASH_OK;
+        }
+    DFL_HIP_CHECK(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    if (ctx->n_lds_attr < kCap) {  // a full table only costs the repeated runtime call
+        ctx->lds_attr_fn[ctx->n_lds_attr] = fn;
+        ctx->lds_attr_bytes[ctx->n_lds_attr++] = bytes;
+    }
+    return DFLASH_OK;
+}
+
 extern "C" {
 
 int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **out) {

@@ -256,13 +256,9 @@ extern "C" int32_t dflash_select_draft_path(dflash_ctx *ctx, const dflash_codebo
     hipStream_t st = static_cast<hipStream_t>(stream);
     const size_t lds = static_cast<size_t>(2 + top_k) * rank * sizeof(float);
     if (lds > 48 * 1024) {
-        static bool attr = false;
-        if (!attr) {
-            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(dflash2_select_kernel<false>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (2 + kSelMaxTopK) * kSelMaxRank * static_cast<int>(sizeof(float))));
-            attr = true;
-        }
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(dflash2_select_kernel<false>),
+                                                    (2 + kSelMaxTopK) * kSelMaxRank * sizeof(float)))
+            return rc_;
     }
     dflash2_select_kernel<false><<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
                                                               out_tokens, status, 0.0f, nullptr, nullptr);
@@ -312,19 +308,16 @@ extern "C" int32_t dflash_select_draft_path_sampled(dflash_ctx *ctx, const dflas
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(uniforms, u_host, sizeof(u_host), hipMemcpyHostToDevice, st));
     const size_t lds = static_cast<size_t>(2 + top_k) * rank * sizeof(float);
     if (lds > 48 * 1024) {
-        static bool attr = false;
-        if (!attr) {
-            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(dflash2_select_kernel<true>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (2 + kSelMaxTopK) * kSelMaxRank * static_cast<int>(sizeof(float))));
-            attr = true;
-        }
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(dflash2_select_kernel<true>),
+                                                    (2 + kSelMaxTopK) * kSelMaxRank * sizeof(float)))
+            return rc_;
     }
     dflash2_select_kernel<true><<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
                                                              out_dev, status, pc_cfg.temperature, uniforms, sampled);
     DFL_HIP_CHECK(ctx, hipGetLastError());
-    static SampledOut host;  // 4 KB; calls on one context are serial
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(&host, sampled, sizeof(host), hipMemcpyDeviceToHost, st));
+    static_assert(sizeof(SampledOut) <= DFL_PINNED_BYTES, "the walk's result is read back through the context's pinned page");
+    const SampledOut &host = *static_cast<const SampledOut *>(ctx->pinned);
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(ctx->pinned, sampled, sizeof(SampledOut), hipMemcpyDeviceToHost, st));
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(out_tokens_host, out_dev, n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
     DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
     // every completed position consumed one draw, as each sample_with_distribution call commits its own

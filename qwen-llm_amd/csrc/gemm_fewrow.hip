@@ -1427,12 +1427,8 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         const size_t lds = static_cast<size_t>(Q4KGeom<WAVES>::kLdsPieces) * sizeof(half8_t);                      \
         if (lds > ctx->lds_bytes)                                                                                      \
             return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: %zu bytes of LDS needed", lds);                 \
-        static bool attr = false;                                                                                      \
-        if (!attr) {                                                                                                   \
-            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_stream_kernel<WAVES, XT>),  \
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-            attr = true;                                                                                               \
-        }                                                                                                              \
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(gemm_q4k_stream_kernel<WAVES, XT>), lds)) \
+            return rc_;                                                                                                \
         {                                                                                                              \
             dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                      \
             gemm_q4k_stream_kernel<WAVES, XT><<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, \
@@ -1493,12 +1489,8 @@ int32_t launch_q6k_stream(dflash_ctx *ctx, const void *w, const void *x, int32_t
         const size_t lds = Q6KGeom<WAVES>::kLdsBytes;                                                                  \
         if (lds > ctx->lds_bytes)                                                                                      \
             return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: %zu bytes of LDS needed", lds);                 \
-        static bool attr = false;                                                                                      \
-        if (!attr) {                                                                                                   \
-            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q6k_stream_kernel<WAVES, XT>),  \
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-            attr = true;                                                                                               \
-        }                                                                                                              \
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(gemm_q6k_stream_kernel<WAVES, XT>), lds)) \
+            return rc_;                                                                                                \
         {                                                                                                              \
             dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                      \
             gemm_q6k_stream_kernel<WAVES, XT><<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, \
@@ -1549,9 +1541,21 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
     return launch_q4k(ctx, w_stack, x, x_type, y, n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt, max_slots);
 }
 
+namespace {
+int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in,
+                         int64_t n_out, int32_t n_rows, dflash_stream_t stream);
+}
+
 extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type,
                                       float *y, int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    return gemm_fewrow_impl(ctx, w_type, w, x, x_type, y, n_in, n_out, n_rows, stream);
+}
+
+namespace {
+
+int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in,
+                         int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
     if (!w || !x || !y) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "gemm_fewrow: null pointer");
     if (n_rows < 1 || n_rows > 16)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: n_rows %d outside 1..16", n_rows);
@@ -1621,14 +1625,11 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
             DFL_LAUNCH_GENERIC(DFLASH_TYPE_F16);
         else if (n_in % 256 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
             env_int("DFLASH_Q8_STAGED", 1)) {
-            static bool attr = false;
-            if (!attr) {
-                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_staged_kernel<float>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kQ8StagedLds)));
-                DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_staged_kernel<_Float16>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kQ8StagedLds)));
-                attr = true;
-            }
+            if (const int32_t rc_ = dfl_raise_lds_limit(ctx, x_type == DFLASH_TYPE_F32
+                                                                 ? reinterpret_cast<const void *>(gemm_q8_0_staged_kernel<float>)
+                                                                 : reinterpret_cast<const void *>(gemm_q8_0_staged_kernel<_Float16>),
+                                                        kQ8StagedLds))
+                return rc_;
             // the waves of a workgroup split a 64-step chunk
             if (split > kQ8ChunkSteps) split = kQ8ChunkSteps;
             if (x_type == DFLASH_TYPE_F32)
@@ -1645,3 +1646,5 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }
+
+}  // namespace

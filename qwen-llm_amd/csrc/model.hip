@@ -471,6 +471,45 @@ uint64_t hash_bytes(const void *p, size_t n, uint64_t h) {
     return h;
 }
 
+// Key of a model for the captured-graph cache: the fields a launch depends on (shape, tensor types and device
+// pointers), one by one, so that padding bytes a caller left uninitialised never split the cache.
+uint64_t hash_model(const dflash_model *m) {
+    uint64_t h = 0x9e3779b97f4a7c15ull;
+    auto word = [&](uint64_t w) {
+        h = (h ^ w) * 0x100000001b3ull;
+        h ^= h >> 29;
+    };
+    auto ptr = [&](const void *p) { word(reinterpret_cast<uintptr_t>(p)); };
+    auto qt = [&](const dflash_qtensor &t) {
+        word(static_cast<uint32_t>(t.type));
+        ptr(t.data);
+    };
+    const dflash_model_cfg &c = m->cfg;
+    const int32_t ints[11] = {c.n_layers, c.hidden, c.n_q, c.n_kv, c.head_dim, c.ffn, c.vocab, c.n_expert, c.n_expert_used,
+                              c.ffn_expert, c.ffn_shared};
+    for (int32_t v : ints) word(static_cast<uint32_t>(v));
+    uint32_t fb[2];
+    memcpy(fb, &c.eps, 4);
+    memcpy(fb + 1, &c.rope_theta, 4);
+    word(fb[0]);
+    word(fb[1]);
+    qt(m->token_embd);
+    qt(m->output);
+    ptr(m->output_norm);
+    for (int il = 0; il < c.n_layers; il++) {
+        const dflash_layer &L = m->layers[il];
+        ptr(L.attn_norm);
+        ptr(L.q_norm);
+        ptr(L.k_norm);
+        ptr(L.post_norm);
+        for (const dflash_qtensor *t : {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down, &L.router, &L.gate_exps, &L.up_exps,
+                                        &L.down_exps})
+            qt(*t);
+        ptr(L.shexp_gate);
+    }
+    return h;
+}
+
 // Every launch of one packed verify, from the embedding rows to the argmax, on `st`: no host
 // reads, no synchronisation, nothing that depends on the position except through pos[] on the
 // device, so the sequence can be captured once and replayed.
@@ -586,8 +625,7 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
     const bool use_graph = ctx->graphs && !ctx->timing && ctx->gstream;
     uint64_t key = 0;
     if (use_graph) {
-        key = hash_bytes(model, sizeof(*model), 0x9e3779b97f4a7c15ull);
-        key = hash_bytes(model->layers, sizeof(dflash_layer) * c.n_layers, key);
+        key = hash_model(model);
         const uintptr_t outs[4] = {reinterpret_cast<uintptr_t>(hidden_capture), reinterpret_cast<uintptr_t>(lg),
                                    reinterpret_cast<uintptr_t>(am), reinterpret_cast<uintptr_t>(gp)};
         key = hash_bytes(outs, sizeof(outs), key);
@@ -1141,6 +1179,23 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
     const int N = head->cfg.block_size;
     res->n_block = N;
     int32_t rc;
+    // A failed step commits nothing: whatever phase fails, the target's KV position goes back to where the block
+    // started and both samplers to their state on entry, so that the caller can retry (or fall back to a serial
+    // step) on the same random stream.  The message of the failing call is kept.
+    const dflash_sampler sampler_in = sampler ? *sampler : dflash_sampler{};
+    const dflash_sampler proposal_in = proposal_sampler ? *proposal_sampler : dflash_sampler{};
+    const int64_t kv_in = sess->kv_n_pos;
+#define STEP_HIP(expr)                                                                                        \
+    do {                                                                                                      \
+        const hipError_t e_ = (expr);                                                                         \
+        if (e_ != hipSuccess) return undo(dfl_fail(ctx, DFLASH_ERR_HIP, "spec_step: %s", hipGetErrorString(e_))); \
+    } while (0)
+    auto undo = [&](int32_t status) {
+        if (sampler) *sampler = sampler_in;
+        if (proposal_sampler) *proposal_sampler = proposal_in;
+        sess->kv_n_pos = kv_in;  // stale rows stay in place; the next verify overwrites them
+        return status;
+    };
 
     auto t0 = std::chrono::steady_clock::now();
     int32_t prop_counts[16] = {0};
@@ -1149,12 +1204,12 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         // draft_block_sampled (metal_dflash.rs:17268-17415): the drafter up to its top-16 and selector gate,
         // then the walk that draws every position from softmax(score / T) with the proposal sampler
         if ((rc = draft_block_impl(ctx, target, head, dsess, carry, cfg->mask_token, position, nullptr, nullptr, nullptr, st, true)))
-            return rc;
+            return undo(rc);
         if ((rc = dflash_select_draft_path_sampled(ctx, &head->selector_predecessor, &head->selector_successor,
                                                    head->cfg.selector_rank, head->cfg.selector_top_k, carry, N, dsess->topk_ids,
                                                    dsess->topk_vals, dsess->sel_h, proposal_sampler, res->draft_tokens, prop_counts,
                                                    prop_cands, st)))
-            return rc;
+            return undo(rc);
     } else {
         // The drafter's tokens stay on the device and the verify is enqueued right behind the drafter:
         // no host round trip between the two phases, and the GPU does not wait for the host to start
@@ -1168,7 +1223,7 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         }
         if (!cfg->replay_only &&
             (rc = dflash_draft_block(ctx, target, head, dsess, carry, cfg->mask_token, position, dsess->argmax, nullptr, nullptr, st)))
-            return rc;
+            return undo(rc);
     }
     const int32_t *verify_input = res->draft_tokens;
     if (sampled_drafts) {
@@ -1177,12 +1232,12 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         t0 = std::chrono::steady_clock::now();
         if ((rc = dflash_verify_block(ctx, target, sess, verify_input, N, position, taps, n_taps, nullptr, nullptr, sess->hidden,
                                       nullptr, res->verify_argmax, st)))
-            return rc;
-        DFL_HIP_CHECK(ctx, hipMemcpy(res->verify_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost));
+            return undo(rc);
+        STEP_HIP(hipMemcpy(res->verify_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost));
         res->verify_ms = ms_since(t0);
     } else {
         const bool timed = !ctx->timing;  // the per-kernel timers use the same events
-        if (timed) DFL_HIP_CHECK(ctx, hipEventRecord(ctx->ev0, st));
+        if (timed) STEP_HIP(hipEventRecord(ctx->ev0, st));
         int32_t tokens_in[16];
         tokens_in[0] = carry;
         for (int i = 1; i < N; i++) tokens_in[i] = (draft_override && draft_override[i - 1] >= 0) ? draft_override[i - 1] : -1;
@@ -1190,15 +1245,15 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         t0 = std::chrono::steady_clock::now();
         if ((rc = verify_block_impl(ctx, target, sess, tokens_in, dsess->argmax, N, position, taps, n_taps, nullptr, nullptr,
                                     sess->hidden, nullptr, nullptr, st)))
-            return rc;
-        if (timed) DFL_HIP_CHECK(ctx, hipEventRecord(ctx->ev1, st));
+            return undo(rc);
+        if (timed) STEP_HIP(hipEventRecord(ctx->ev1, st));
         // read back through the context's pinned page: three truly asynchronous copies, one wait
         int32_t *pin_argmax = static_cast<int32_t *>(ctx->pinned), *pin_draft = pin_argmax + 16;
         float *pin_gap = reinterpret_cast<float *>(pin_argmax + 32);
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(pin_argmax, sess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(pin_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost, st));
-        DFL_HIP_CHECK(ctx, hipMemcpyAsync(pin_draft, dsess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-        DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        STEP_HIP(hipMemcpyAsync(pin_argmax, sess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        STEP_HIP(hipMemcpyAsync(pin_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost, st));
+        STEP_HIP(hipMemcpyAsync(pin_draft, dsess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        STEP_HIP(hipStreamSynchronize(st));
         memcpy(res->verify_argmax, pin_argmax, N * sizeof(int32_t));
         memcpy(res->verify_gap, pin_gap, N * sizeof(float));
         memcpy(res->draft_tokens, pin_draft, N * sizeof(int32_t));
@@ -1215,9 +1270,8 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         for (int i = 1; i < N; i++) {
             if (tokens_in[i] >= 0) res->draft_tokens[i] = tokens_in[i];
             if (res->draft_tokens[i] < 0 || res->draft_tokens[i] >= target->cfg.vocab) {
-                (void)dflash_restore(ctx, sess, position, N, 0);  // nothing is committed
-                return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "spec_step: the drafter produced token %d at slot %d (vocabulary %d)",
-                                res->draft_tokens[i], i, target->cfg.vocab);
+                return undo(dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "spec_step: the drafter produced token %d at slot %d (vocabulary %d)",
+                                res->draft_tokens[i], i, target->cfg.vocab));
             }
         }
         res->draft_tokens[0] = carry;
@@ -1239,16 +1293,13 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         rc = dflash_accept_greedy(verify_input, res->verify_argmax, N, budget, stop_ids, n_stop, &res->decision);
         if (rc) dfl_fail(ctx, rc, "spec_step: greedy accept rejected its input");
     }
-    if (rc) {  // nothing is committed: put the KV back where the block started
-        (void)dflash_restore(ctx, sess, position, N, 0);
-        return rc;
-    }
+    if (rc) return undo(rc);
     res->accept_ms = ms_since(t0);
 
     if (cfg->sampled_mode == 0 && cfg->fallback_margin > 0.0f) {
         t0 = std::chrono::steady_clock::now();
         if ((rc = margin_fallback(ctx, target, sess, taps, n_taps, verify_input, N, position, cfg, budget, stop_ids, n_stop, res, st)))
-            return rc;
+            return undo(rc);
         if (res->fallback_ran) res->fallback_ms = ms_since(t0);
     }
 
@@ -1257,16 +1308,18 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
         t0 = std::chrono::steady_clock::now();
         int32_t positions[16];
         for (int i = 0; i < n_keep; i++) positions[i] = static_cast<int32_t>(position + i);
-        if ((rc = dflash_draft_append_ctx(ctx, dsess, sess->hidden, n_keep, positions, st))) return rc;
-        DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+        if ((rc = dflash_draft_append_ctx(ctx, dsess, sess->hidden, n_keep, positions, st))) return undo(rc);
+        STEP_HIP(hipStreamSynchronize(st));
         res->append_ms = ms_since(t0);
     }
     if (!res->fallback_ran && n_keep < N) {
         t0 = std::chrono::steady_clock::now();
-        if ((rc = dflash_restore(ctx, sess, position, N, n_keep))) return rc;
+        if ((rc = dflash_restore(ctx, sess, position, N, n_keep))) return undo(rc);
         res->restore_ms = ms_since(t0);
     }
     return DFLASH_OK;
 }
+
+#undef STEP_HIP
 
 }  // extern "C"

@@ -497,6 +497,10 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     const int n_slots = n * used;
     if (used < 1 || used > 64 || E > 8192 || fe % 32 || H % 32)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: n_expert %d / n_expert_used %d / ffn_expert %d unsupported", E, used, fe);
+    if (!L.router.data || !L.gate_exps.data || !L.up_exps.data || !L.down_exps.data || !L.shexp_gate || !L.gate.data ||
+        !L.up.data || !L.down.data)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT,
+                        "moe: a mixture-of-experts layer needs router, gate/up/down_exps, shexp_gate and the shared expert's gate/up/down");
     const int et = L.gate_exps.type;
     if (et != L.up_exps.type || (et != DFLASH_TYPE_Q4_K && et != DFLASH_TYPE_Q6_K && et != DFLASH_TYPE_Q8_0))
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: expert weight type %d", et);
@@ -517,12 +521,8 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
                                L.down.type == DFLASH_TYPE_Q4_K;
     const size_t route_lds = static_cast<size_t>(17) * E * sizeof(float);
     if (route_lds > 48 * 1024) {
-        static bool attr = false;
-        if (!attr) {
-            DFL_HIP_CHECK(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(moe_route_kernel),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 1024 * sizeof(float)));
-            attr = true;
-        }
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(moe_route_kernel), 17 * 1024 * sizeof(float)))
+            return rc_;
     }
     const float *gate_w = gate_done ? nullptr : L.shexp_gate;  // null: sg is already there
     if (E <= 256)

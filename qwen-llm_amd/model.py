@@ -721,7 +721,7 @@ class SpeculativeDecoder:
                 break
             was_probe, long_mode, replay = False, False, None
             if position_margin:
-                self.cfg.fallback_margin = adaptive_lib().dflash_verify_fallback_margin(self.position)
+                self.cfg.fallback_margin = adaptive_lib().dflash_verify_fallback_margin(self.position + n_block)
             if adaptive:
                 long_mode = off_ctx > 16384 and self.position >= 16384
                 L.dflash_adaptive_prepare_mode(C.byref(state), int(long_mode))
