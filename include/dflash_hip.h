@@ -106,6 +106,22 @@ size_t dflash_row_bytes(int32_t type, size_t n_in);
 int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
                            int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream);
 
+/* The same product for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  It takes no context and calls no
+ * hipMalloc / hipFree or any allocating routine: the split-K partial tiles that dflash_gemm_fewrow keeps in
+ * its context's buffer live in a fixed 8 MiB array of the library's device image (one copy per GPU, held until
+ * the process ends).  Same arguments, guards, kernels and results (bit for bit) as dflash_gemm_fewrow on a
+ * GPU of up to 256 compute units; the launch never uses more workgroups than the array has partial-tile
+ * sets for.  Shapes beyond DFLASH_NOALLOC_MAX_N_IN / DFLASH_NOALLOC_MAX_N_OUT are refused with
+ * DFLASH_ERR_BAD_SHAPE.  Runs on the current device.  All calls on one GPU share that GPU's array: calls
+ * on one stream are ordered; calls that overlap in time on the same GPU (several streams or threads) race.
+ * Enqueue-only.  dflash_gemm_fewrow_noalloc_error() returns the calling thread's last message. */
+#define DFLASH_NOALLOC_MAX_N_IN 262144
+#define DFLASH_NOALLOC_MAX_N_OUT 1048576
+int32_t dflash_gemm_fewrow_noalloc(int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
+                                   int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream);
+const char *dflash_gemm_fewrow_noalloc_error(void);
+
 /* ---- block-causal verify attention ------------------------------------------------
  * The reference verifies a block with a per-row loop: encode_scatter_offset_f32_to_f16_kv +
  * encode_attn_decode_v4_f32 / encode_attn_decode_f16kv_f32, once per row

@@ -113,6 +113,10 @@ def _declare(L):
     L.dflash_dequant.argtypes = [vp, i32, vp, sz, vp, vp]
     L.dflash_gemm_fewrow.restype = i32
     L.dflash_gemm_fewrow.argtypes = [vp, i32, vp, vp, i32, vp, i64, i64, i32, vp]
+    L.dflash_gemm_fewrow_noalloc.restype = i32
+    L.dflash_gemm_fewrow_noalloc.argtypes = [i32, vp, vp, i32, vp, i64, i64, i32, vp]
+    L.dflash_gemm_fewrow_noalloc_error.restype = C.c_char_p
+    L.dflash_gemm_fewrow_noalloc_error.argtypes = []
     for name in ("dflash_argmax_top2", "dflash_top16"):
         getattr(L, name).restype = i32
         getattr(L, name).argtypes = [vp, vp, i32, i64, i64, vp, vp, vp]

@@ -26,6 +26,8 @@
 #include "common.h"
 
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
 
 namespace {
 
@@ -1648,3 +1650,93 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
 }
 
 }  // namespace
+
+// ----------------------------------------------------------------------------
+// The same product for callers that may not allocate
+// ----------------------------------------------------------------------------
+//
+// The streaming kernels keep split-K partial tiles in device memory between the GEMM kernel and its
+// reduction.  dflash_gemm_fewrow takes that buffer from the context, which allocated it.  The entry
+// below takes it from a fixed array in the library's device image instead and needs no context, so
+// nothing on its path allocates: no hipMalloc / hipFree, no workspace, no stream or event creation.
+// The array is sized for kNoAllocEntries partial-tile sets (one per 8-wave workgroup, two per 16-wave
+// workgroup): launches are clamped to that many workgroups, which covers every CU of an MI355X.
+// Every call on a GPU uses that GPU's one copy of the array: calls that overlap in time on the same
+// GPU (two streams, two threads) race on it; calls on one stream are ordered and safe.  Nothing in
+// the array has to start at zero: the reduction reads only the tiles the same launch wrote.
+namespace {
+constexpr int kNoAllocEntries = 512;
+constexpr size_t kNoAllocScratchBytes = static_cast<size_t>(kNoAllocEntries) * 2 * 8 * 256 * sizeof(float);  // 8 MiB
+constexpr int kNoAllocMaxDevices = 64;
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+
+struct NoAllocDevice {
+    void *ptr = nullptr;  // this device's copy of `scratch` (hipGetSymbolAddress, once per device)
+    int n_cu = 0;
+    size_t lds_bytes = 0;
+    // the context fields that remember per-device kernel attributes, carried from call to call
+    const void *lds_attr_fn[96] = {nullptr};
+    size_t lds_attr_bytes[96] = {0};
+    int n_lds_attr = 0;
+};
+NoAllocDevice g_noalloc[kNoAllocMaxDevices];
+std::mutex g_noalloc_mutex;  // guards the table above (the enqueue itself is short)
+thread_local char g_noalloc_err[512] = "";
+
+int32_t noalloc_fail(int32_t status, const char *msg) {
+    snprintf(g_noalloc_err, sizeof(g_noalloc_err), "%s", msg);
+    return status;
+}
+
+}  // namespace
+
+extern "C" const char *dflash_gemm_fewrow_noalloc_error(void) { return g_noalloc_err; }
+
+extern "C" int32_t dflash_gemm_fewrow_noalloc(int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
+                                              int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
+    g_noalloc_err[0] = 0;
+    if (n_in > DFLASH_NOALLOC_MAX_N_IN || n_out > DFLASH_NOALLOC_MAX_N_OUT)
+        return noalloc_fail(DFLASH_ERR_BAD_SHAPE, "gemm_fewrow_noalloc: n_in / n_out beyond DFLASH_NOALLOC_MAX_N_IN / _N_OUT");
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0) return noalloc_fail(DFLASH_ERR_HIP, "gemm_fewrow_noalloc: no current device");
+    if (device >= kNoAllocMaxDevices) return noalloc_fail(DFLASH_ERR_UNSUPPORTED, "gemm_fewrow_noalloc: device index beyond 63");
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    NoAllocDevice &dev = g_noalloc[device];
+    if (!dev.ptr) {
+        // first call on this device, which is the current one: its own address of the array, and its shape
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr)
+            return noalloc_fail(DFLASH_ERR_HIP, "gemm_fewrow_noalloc: hipGetSymbolAddress(scratch) failed");
+        int n_cu = 0, lds = 0;
+        if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess || n_cu < 1)
+            return noalloc_fail(DFLASH_ERR_HIP, "gemm_fewrow_noalloc: device attributes unavailable");
+        dev.n_cu = n_cu;
+        dev.lds_bytes = static_cast<size_t>(lds);
+        dev.ptr = ptr;
+    }
+    // a context on the stack that owns nothing: the launch code reads its shape fields and the partial-tile buffer
+    dflash_ctx local;
+    local.device = device;
+    local.n_cu = dev.n_cu;
+    local.lds_bytes = dev.lds_bytes;
+    local.partials = dev.ptr;
+    local.n_partial_wgs = kNoAllocEntries;
+    memcpy(local.lds_attr_fn, dev.lds_attr_fn, sizeof(dev.lds_attr_fn));
+    memcpy(local.lds_attr_bytes, dev.lds_attr_bytes, sizeof(dev.lds_attr_bytes));
+    local.n_lds_attr = dev.n_lds_attr;
+    int32_t rc;
+    if (!w || !x || !y)
+        rc = dfl_fail(&local, DFLASH_ERR_INVALID_INPUT, "gemm_fewrow_noalloc: null pointer");
+    else
+        rc = gemm_fewrow_impl(&local, w_type, w, x, x_type, y, n_in, n_out, n_rows, stream);
+    memcpy(dev.lds_attr_fn, local.lds_attr_fn, sizeof(dev.lds_attr_fn));
+    memcpy(dev.lds_attr_bytes, local.lds_attr_bytes, sizeof(dev.lds_attr_bytes));
+    dev.n_lds_attr = local.n_lds_attr;
+    if (rc) snprintf(g_noalloc_err, sizeof(g_noalloc_err), "%s", local.err);
+    return rc;
+}
