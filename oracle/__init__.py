@@ -168,6 +168,10 @@ def _declare(L):
                                            vp, sz, C.POINTER(AcceptDecision)]
     L.orc_decide_accept_prefix_dense.argtypes = [vp, sz, vp, vp, sz, f32, C.POINTER(Sampler), sz, vp, sz,
                                                  C.POINTER(AcceptDecision)]
+    L.orc_decide_accept_prefix_batch.restype = None
+    L.orc_decide_accept_prefix_batch.argtypes = [sz, vp, sz, vp, vp, sz, f32, vp, sz, vp, vp]
+    L.orc_router_margin_take.restype = f32
+    L.orc_router_margin_take.argtypes = []
     L.orc_rms_norm.argtypes = [vp, vp, sz, f32, vp]
     L.orc_silu.restype = f32
     L.orc_silu.argtypes = [f32]
@@ -374,6 +378,23 @@ def decide_accept_prefix_dense(verified_tokens, target_logits, draft_logits, voc
     return rc, out
 
 
+def decide_accept_prefix_batch(verified_tokens, target_logits, draft_logits, draft_temperature, samplers, budget):
+    """verified_tokens [trials, n]; target_logits [trials, n, vocab]; draft_logits [trials, n-1, vocab] or None;
+    samplers: list of Sampler (advanced in place).  Returns (status list, list of AcceptDecision)."""
+    toks = np.ascontiguousarray(verified_tokens, dtype=np.int32)
+    t = np.ascontiguousarray(target_logits, dtype=np.float32)
+    d = None if draft_logits is None else np.ascontiguousarray(draft_logits, dtype=np.float32)
+    n_trials, n = toks.shape
+    arr = (Sampler * n_trials)(*samplers)
+    outs = (AcceptDecision * n_trials)()
+    status = np.zeros(n_trials, np.int32)
+    lib().orc_decide_accept_prefix_batch(n_trials, _p(toks), n, _p(t), _p(d) if d is not None else None, t.shape[2],
+                                         draft_temperature, arr, budget, outs, _p(status))
+    for i in range(n_trials):
+        C.memmove(C.byref(samplers[i]), C.byref(arr[i]), C.sizeof(Sampler))
+    return status.tolist(), list(outs)
+
+
 # ---- synthetic decoder / drafter (plain dictionaries of numpy arrays in, numpy out) ----
 
 class _Keep:
@@ -486,6 +507,12 @@ def target_verify(model: Model, state: TargetState, tokens, start_pos: int, tap_
     if rc:
         raise RuntimeError(f"orc_target_verify failed: {rc}")
     return logits, hidden[:, :len(tap_layers)]
+
+
+def router_margin_take() -> float:
+    """Smallest relative gap between the last expert picked and the best one left out over every routing decision
+    since the previous call (inf if there was none)."""
+    return float(lib().orc_router_margin_take())
 
 
 def dflash_draft(target: Model, head: DraftHead, noise_ids, ctx_stacked, pos_ctx, noise_start_pos: int):

@@ -179,6 +179,17 @@ int orc_decide_accept_prefix_dense(const int32_t *verified_tokens, size_t n_toke
                                    size_t remaining_output_budget, const int32_t *stop_ids, size_t n_stop,
                                    orc_accept_decision *out);
 
+/* n_trials independent block decisions (dense proposals when draft_logits != NULL, deterministic drafts otherwise),
+ * OpenMP across trials; trial t uses samplers[t], verified_tokens[t][n_tokens], target_logits[t][n_tokens][vocab],
+ * draft_logits[t][n_tokens-1][vocab] and writes out[t], status[t] */
+void orc_decide_accept_prefix_batch(size_t n_trials, const int32_t *verified_tokens, size_t n_tokens,
+                                    const float *target_logits, const float *draft_logits, size_t vocab,
+                                    float draft_temperature, orc_sampler *samplers, size_t remaining_output_budget,
+                                    orc_accept_decision *out, int32_t *status);
+
+/* smallest relative router gap (last pick vs best expert left out) since the previous call; +inf if none */
+float orc_router_margin_take(void);
+
 /* ---- f32 forward primitives (forward.rs:1244-1371) ---- */
 void orc_rms_norm(const float *x, const float *w, size_t n, float eps, float *out);
 float orc_silu(float x);

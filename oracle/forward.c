@@ -193,6 +193,16 @@ static int ffn_dense(const orc_layer *L, const float *x, size_t h, size_t f, flo
     return rc;
 }
 
+/* Smallest relative gap between the last expert picked and the best one left out, over every routing decision since
+ * the last orc_router_margin_take(): lets a test tell a wrong pick from a near tie that an f16-operand router may
+ * break the other way.  Test scaffolding; not part of the reference. */
+static float g_router_margin = INFINITY;
+float orc_router_margin_take(void) {
+    float m = g_router_margin;
+    g_router_margin = INFINITY;
+    return m;
+}
+
 /* forward.rs:749-824 */
 static int ffn_moe(const orc_model_cfg *c, const orc_layer *L, const float *x, float *out) {
     size_t h = (size_t)c->hidden, ne = (size_t)c->n_expert;
@@ -212,6 +222,14 @@ static int ffn_moe(const orc_model_cfg *c, const orc_layer *L, const float *x, f
         }
         taken[best] = 1;
         pick[k] = best;
+    }
+    if (used < ne) {
+        float runner_up = 0.0f;
+        for (size_t e = 0; e < ne; e++)
+            if (!taken[e] && probs[e] > runner_up) runner_up = probs[e];
+        float last = probs[pick[used - 1]];
+        float rel = last > 0.0f ? (last - runner_up) / last : 0.0f;
+        if (rel < g_router_margin) g_router_margin = rel;
     }
     float weight_sum = 0.0f;
     for (size_t k = 0; k < used; k++) weight_sum += probs[pick[k]];

@@ -767,3 +767,24 @@ int orc_decide_accept_prefix_dense(const int32_t *verified_tokens, size_t n_toke
     return decide(verified_tokens, n_tokens, target_logits, n_tokens * vocab, vocab, 2, 0, NULL, NULL, NULL, NULL,
                   draft_logits, draft_temperature, sampler, remaining_output_budget, stop_ids, n_stop, out);
 }
+
+/* Many independent block decisions at once, one per sampler, OpenMP across trials: each trial is exactly
+ * orc_decide_accept_prefix_dense (draft_logits != NULL) or orc_decide_accept_prefix without proposals
+ * (draft_logits == NULL) on its own slice.  For checking long seeded runs in bounded wall time; no counterpart
+ * in the reference (its accept decision is per block). */
+void orc_decide_accept_prefix_batch(size_t n_trials, const int32_t *verified_tokens, size_t n_tokens,
+                                    const float *target_logits, const float *draft_logits, size_t vocab,
+                                    float draft_temperature, orc_sampler *samplers, size_t remaining_output_budget,
+                                    orc_accept_decision *out, int32_t *status) {
+#pragma omp parallel for schedule(dynamic, 1)
+    for (long t = 0; t < (long)n_trials; t++) {
+        const int32_t *tok = verified_tokens + (size_t)t * n_tokens;
+        const float *tl = target_logits + (size_t)t * n_tokens * vocab;
+        if (draft_logits)
+            status[t] = orc_decide_accept_prefix_dense(tok, n_tokens, tl, draft_logits + (size_t)t * (n_tokens - 1) * vocab, vocab,
+                                                       draft_temperature, &samplers[t], remaining_output_budget, NULL, 0, &out[t]);
+        else
+            status[t] = orc_decide_accept_prefix(tok, n_tokens, tl, n_tokens * vocab, vocab, 0, 0, NULL, NULL, NULL, NULL,
+                                                 &samplers[t], remaining_output_budget, NULL, 0, &out[t]);
+    }
+}

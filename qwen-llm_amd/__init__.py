@@ -49,6 +49,7 @@ from .model import (  # noqa: F401,E402
     synth_draft_weights_device,
     synth_target_weights_device,
     synth_target_weights,
+    synth_target_weights_blocks,
 )
 from . import gguf  # noqa: F401,E402
 from .gguf import GgufFile, open_dflash_drafter, open_target, write_gguf  # noqa: F401,E402

@@ -18,6 +18,7 @@
 //    the rows of the block.
 #include "common.h"
 #include "sampler_chain.h"
+#include "accept_wide.h"
 
 #include <cmath>
 #include <cstring>
@@ -197,14 +198,39 @@ __global__ void __launch_bounds__(kSelThreads)
     if (tid == 0) o->nan_first = nan_sh;
 }
 
+// The dense proposal's side of a row: its largest draft logit (scaled) and NaN / no-candidate errors.
+__device__ void merge_draft_side(const ChunkOut *__restrict__ draft_chunks, int n_chunks, int row, const ChainCfg &cfg, RowDist *d) {
+    uint64_t best = kNoKey;
+    int dn = kNoNan;
+    for (int c = 0; c < n_chunks; c++) {
+        const ChunkOut &dc = draft_chunks[row * n_chunks + c];
+        best = dc.keys[0] < best ? dc.keys[0] : best;
+        dn = dc.nan_first < dn ? dc.nan_first : dn;
+    }
+    d->d_err = 0;
+    d->d_err_index = -1;
+    d->d_max_scaled = static_cast<double>(key_logit(best)) / static_cast<double>(cfg.draft_temperature);
+    if (dn != kNoNan) {
+        d->d_err = DFLASH_ERR_NAN_LOGIT;
+        d->d_err_index = dn;
+    } else if (!isfinite(d->d_max_scaled)) {
+        d->d_err = DFLASH_ERR_NO_CANDIDATES;
+    }
+}
+
 // One workgroup per row: merge the chunk lists, order the best k, run the chain.
 __global__ void __launch_bounds__(kSelThreads)
     row_merge_kernel(const ChunkOut *__restrict__ chunks, int n_chunks, const ChunkOut *__restrict__ draft_chunks,
-                     ChainCfg cfg, RowDist *__restrict__ rows, int32_t *__restrict__ greedy_out) {
+                     ChainCfg cfg, RowDist *__restrict__ rows, int32_t *__restrict__ greedy_out, bool draft_only) {
     __shared__ uint64_t sk[2 * kSelThreads];
     __shared__ double chain_l[kMaxK], chain_w[kMaxK];
     __shared__ int chain_tok[kMaxK];
     const int row = blockIdx.x, tid = threadIdx.x;
+    RowDist *d = rows + row;
+    if (draft_only) {  // the target side of these rows was filled by the wide chain
+        if (tid == 0) merge_draft_side(draft_chunks, n_chunks, row, cfg, d);
+        return;
+    }
     const int k = cfg.k;
     const int n_in = n_chunks * k;  // <= 2048, checked on the host
     int n_sort = 2;
@@ -216,7 +242,6 @@ __global__ void __launch_bounds__(kSelThreads)
     }
     bitonic_sort(sk, n_sort);
     if (tid != 0) return;
-    RowDist *d = rows + row;
     d->n_keep = 0;
     d->err = 0;
     d->err_index = -1;
@@ -243,22 +268,7 @@ __global__ void __launch_bounds__(kSelThreads)
         while (len < k && sk[len] != kNoKey) len++;
         run_chain(sk, len, cfg, d, ChainScratch{chain_l, chain_w, chain_tok});
     }
-    if (draft_chunks) {
-        uint64_t best = kNoKey;
-        int dn = kNoNan;
-        for (int c = 0; c < n_chunks; c++) {
-            const ChunkOut &dc = draft_chunks[row * n_chunks + c];
-            best = dc.keys[0] < best ? dc.keys[0] : best;
-            dn = dc.nan_first < dn ? dc.nan_first : dn;
-        }
-        d->d_max_scaled = static_cast<double>(key_logit(best)) / static_cast<double>(cfg.draft_temperature);
-        if (dn != kNoNan) {
-            d->d_err = DFLASH_ERR_NAN_LOGIT;
-            d->d_err_index = dn;
-        } else if (!isfinite(d->d_max_scaled)) {
-            d->d_err = DFLASH_ERR_NO_CANDIDATES;
-        }
-    }
+    if (draft_chunks) merge_draft_side(draft_chunks, n_chunks, row, cfg, d);
 }
 
 // top-16 output from the merged order
@@ -323,7 +333,31 @@ struct DecideArgs {
     const double *tile_sums;
     int32_t n_tiles;
     float temperature, draft_temperature;
+    // wide candidate sets (effective top-k above kMaxK): row r's kept candidates are the first n_keep sorted keys
+    // / weights at r * wide_stride of these arrays instead of the arrays inside RowDist; null otherwise
+    const uint64_t *wide_keys;
+    const double *wide_w;
+    int64_t wide_stride;
 };
+
+// A row's kept candidates, wherever they live.
+struct DistView {
+    const RowDist *rd;
+    const uint64_t *keys;  // null: inline arrays of rd
+    const double *w;
+    __device__ int32_t token(int i) const { return keys ? static_cast<int32_t>(keys[i] & kWideTokenMask) : rd->tokens[i]; }
+    __device__ double weight(int i) const { return w ? w[i] : rd->weights[i]; }
+};
+
+// first candidate whose running sum exceeds x, else the last (sampling.rs:1587-1596)
+__device__ int pick_index_view(const DistView &v, int n, double x) {
+    double cumulative = 0.0;
+    for (int i = 0; i < n; i++) {
+        cumulative += v.weight(i);
+        if (x < cumulative) return i;
+    }
+    return n - 1;
+}
 
 __device__ bool in_list(const int32_t *ids, int n, int32_t v) {
     for (int i = 0; i < n; i++)
@@ -348,6 +382,8 @@ __device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int r
     const int n_drafts = a.n_tokens - 1;
     const bool greedy = a.temperature == 0.0f;
     const RowDist &rd = rows[row];
+    const DistView dv = {&rd, a.wide_keys ? a.wide_keys + row * a.wide_stride : nullptr,
+                         a.wide_w ? a.wide_w + row * a.wide_stride : nullptr};
     int draws = greedy ? 0 : row;
     const int draws0 = draws;
     if (row == n_drafts) {  // bonus = sample(last reached row)
@@ -357,8 +393,8 @@ __device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int r
             return o;
         }
         int idx = 0;
-        if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
-        o.token = rd.tokens[idx];
+        if (!greedy) idx = pick_index_view(dv, rd.n_keep, a.uniforms[draws++] * rd.total);
+        o.token = dv.token(idx);
         o.draws = draws - draws0;
         return o;
     }
@@ -370,8 +406,8 @@ __device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int r
             return o;
         }
         int idx = 0;
-        if (!greedy) idx = pick_index(rd.weights, rd.n_keep, a.uniforms[draws++] * rd.total);
-        o.token = rd.tokens[idx];
+        if (!greedy) idx = pick_index_view(dv, rd.n_keep, a.uniforms[draws++] * rd.total);
+        o.token = dv.token(idx);
         o.acc = o.token == draft;
         o.draws = draws - draws0;
         return o;
@@ -421,37 +457,48 @@ __device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int r
     if (o.err) return o;
     double tp = -0.0;
     for (int i = 0; i < rd.n_keep; i++)
-        if (rd.tokens[i] == draft) tp += rd.weights[i];
+        if (dv.token(i) == draft) tp += dv.weight(i);
     const double target_probability = tp / rd.total;
     const double proposal_probability = prop_tok_w / prop_total;
     const double acceptance = fmin(target_probability / proposal_probability, 1.0);
     if (a.uniforms[draws++] < acceptance) {
         o.acc = 1;
     } else {
-        double residual[kMaxK];
-        double residual_total = 0.0;
-        for (int i = 0; i < rd.n_keep; i++) {
-            const double p = rd.weights[i] / rd.total;
+        // residual weights max(p_i - q_i, 0) in the target's order (sampling.rs:752-790): summed first, then walked
+        // again for the pick; the second pass recomputes the same values, so no per-candidate array is needed
+        auto residual_at = [&](int i) {
+            const double p = dv.weight(i) / rd.total;
             double q;
             if (a.mode == 1) {
+                const int32_t ti = dv.token(i);
                 double qs = -0.0;
                 for (int j = 0; j < n_pc; j++)
-                    if (pc[j].token == rd.tokens[i]) qs += pc[j].weight;
+                    if (pc[j].token == ti) qs += pc[j].weight;
                 q = qs / prop_total;
             } else {
-                q = exp(static_cast<double>(a.draft[row * a.draft_stride + rd.tokens[i]]) / static_cast<double>(a.draft_temperature) -
+                q = exp(static_cast<double>(a.draft[row * a.draft_stride + dv.token(i)]) / static_cast<double>(a.draft_temperature) -
                         rd.d_max_scaled) /
                     prop_total;
             }
-            const double wgt = fmax(p - q, 0.0);
-            residual_total += wgt;
-            residual[i] = wgt;
-        }
+            return fmax(p - q, 0.0);
+        };
+        double residual_total = 0.0;
+        for (int i = 0; i < rd.n_keep; i++) residual_total += residual_at(i);
         if (!(isfinite(residual_total) && residual_total > 0.0)) {
             o.err = DFLASH_ERR_NO_CANDIDATES;
             return o;
         }
-        o.token = rd.tokens[pick_index(residual, rd.n_keep, a.uniforms[draws++] * residual_total)];
+        const double x = a.uniforms[draws++] * residual_total;
+        int pick = rd.n_keep - 1;
+        double cumulative = 0.0;
+        for (int i = 0; i < rd.n_keep; i++) {
+            cumulative += residual_at(i);
+            if (x < cumulative) {
+                pick = i;
+                break;
+            }
+        }
+        o.token = dv.token(pick);
     }
     o.draws = draws - draws0;
     return o;
@@ -653,7 +700,7 @@ int32_t dflash_argmax_greedy(dflash_ctx *ctx, const float *logits, int32_t n_row
     cfg.k = 1;
     dfl_timed timer(ctx, st, DFL_T_ARGMAX);
     select_chunk_kernel<<<dim3(n_chunks, n_rows), kSelThreads, 0, st>>>(logits, vocab, stride, 1, chunks, false);
-    row_merge_kernel<<<n_rows, kSelThreads, 0, st>>>(chunks, n_chunks, nullptr, cfg, rows, idx);
+    row_merge_kernel<<<n_rows, kSelThreads, 0, st>>>(chunks, n_chunks, nullptr, cfg, rows, idx, false);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }
@@ -781,11 +828,9 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
     }
     const dflash_sampling_config &sc = sampler->cfg;
     int64_t k_eff = (sc.temperature == 0.0f) ? 1 : ((sc.top_k == 0 || static_cast<int64_t>(sc.top_k) >= vocab) ? vocab : static_cast<int64_t>(sc.top_k));
-    if (k_eff > kMaxK)
-        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "accept_prefix: top_k %lld candidates (1..%d supported on the GPU)",
-                        static_cast<long long>(k_eff), kMaxK);
+    const bool wide = k_eff > kMaxK;  // top_k = 0 or a large top_k: full order by radix sort (accept_wide.hip)
     const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
-    if (n_chunks * k_eff > 2 * kSelThreads)
+    if (!wide && n_chunks * k_eff > 2 * kSelThreads)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "accept_prefix: vocabulary %lld x top_k %lld too large", static_cast<long long>(vocab), static_cast<long long>(k_eff));
 
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -827,11 +872,24 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
     cfg.mode = mode;
     {
         dfl_timed timer(ctx, st, DFL_T_ACCEPT);
-        select_chunk_kernel<<<dim3(n_chunks, n_tokens), kSelThreads, 0, st>>>(target_logits, vocab, vocab, cfg.k, chunks, false);
-        if (mode == 2 && n_drafts > 0)
+        const bool dense = mode == 2 && n_drafts > 0;
+        const uint64_t *wide_keys = nullptr;
+        const double *wide_w = nullptr;
+        if (wide) {
+            if (const int32_t rc_ = dfl_accept_wide_rows(ctx, target_logits, n_tokens, vocab, vocab, cfg, rows, &off, &wide_keys, &wide_w, st))
+                return rc_;
+        } else {
+            select_chunk_kernel<<<dim3(n_chunks, n_tokens), kSelThreads, 0, st>>>(target_logits, vocab, vocab, cfg.k, chunks, false);
+        }
+        if (dense)
             select_chunk_kernel<<<dim3(n_chunks, n_drafts), kSelThreads, 0, st>>>(draft_logits, vocab, vocab, 1, dchunks, false);
-        row_merge_kernel<<<n_tokens, kSelThreads, 0, st>>>(chunks, n_chunks, (mode == 2 && n_drafts > 0) ? dchunks : nullptr,
-                                                          cfg, rows, nullptr);
+        if (!wide)
+            row_merge_kernel<<<n_tokens, kSelThreads, 0, st>>>(chunks, n_chunks, dense ? dchunks : nullptr, cfg, rows, nullptr, false);
+        else if (dense)
+            row_merge_kernel<<<n_drafts, kSelThreads, 0, st>>>(chunks, n_chunks, dchunks, cfg, rows, nullptr, true);
+        a.wide_keys = wide_keys;
+        a.wide_w = wide_w;
+        a.wide_stride = vocab;
         if (mode == 2 && n_drafts > 0)
             dense_tile_sum_kernel<<<dim3(n_tiles, n_drafts), 256, 0, st>>>(draft_logits, vocab, vocab, draft_temperature, rows, tile_sums);
         a.n_tokens = n_tokens;

@@ -12,9 +12,35 @@
 // operations: no fused multiply-adds from here on in the including file.
 #pragma clang fp contract(off)
 
-namespace {
+constexpr int kMaxK = 64;  // most candidates a row keeps inline (wider sets live in device arrays, accept_wide.hip)
 
-constexpr int kMaxK = 64;  // largest supported top-k
+// ------------------------------------------------------------------------------------------
+// per-row results
+// ------------------------------------------------------------------------------------------
+struct RowDist {
+    int32_t n_keep;     // candidates after every filter (above kMaxK: tokens / weights are in the wide arrays instead)
+    int32_t err;        // DFLASH_ERR_* or 0
+    int64_t err_index;  // NaN index etc.
+    double total;       // sum of the kept weights (sequential)
+    int32_t tokens[kMaxK];
+    double weights[kMaxK];
+    // dense proposal side
+    int32_t d_err;
+    int32_t d_pad;
+    int64_t d_err_index;
+    double d_max_scaled;  // f64(max draft logit) / T
+    double d_total;       // P
+};
+
+struct ChainCfg {
+    float temperature, top_p, min_p;
+    int32_t k;          // effective top-k
+    double ln_min_p;    // ln(f64(min_p)), computed on the host
+    float draft_temperature;
+    int32_t mode;       // proposal mode
+};
+
+namespace {
 
 // sampling.rs:1206-1220: a u32 whose ascending order is descending f32 total order
 __device__ __host__ __forceinline__ uint32_t desc_bits(uint32_t bits) {
@@ -31,32 +57,6 @@ __device__ __forceinline__ float key_logit(uint64_t key) {
     return __uint_as_float(bits);
 }
 __device__ __forceinline__ int32_t key_token(uint64_t key) { return static_cast<int32_t>(static_cast<uint32_t>(key)); }
-
-// ------------------------------------------------------------------------------------------
-// per-row results
-// ------------------------------------------------------------------------------------------
-struct RowDist {
-    int32_t n_keep;     // candidates after every filter
-    int32_t err;        // DFLASH_ERR_* or 0
-    int64_t err_index;  // NaN index etc.
-    double total;       // sum of the kept weights (sequential)
-    int32_t tokens[kMaxK];
-    double weights[kMaxK];
-    // dense proposal side
-    int32_t d_err;
-    int32_t d_pad;
-    int64_t d_err_index;
-    double d_max_scaled;  // f64(max draft logit) / T
-    double d_total;       // P
-};
-
-struct ChainCfg {
-    float temperature, top_p, min_p;
-    int32_t k;          // effective top-k (<= kMaxK)
-    double ln_min_p;    // ln(f64(min_p)), computed on the host
-    float draft_temperature;
-    int32_t mode;       // proposal mode
-};
 
 // sampling.rs:1541-1615 on the ordered candidates of one row (keys ascending = best first)
 // Work arrays of the chain (kMaxK entries each): a caller that runs the chain on one thread of a workgroup

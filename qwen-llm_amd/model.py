@@ -182,6 +182,36 @@ def synth_target_weights(cfg: ModelConfig, seed: int, wtype: int = synth.Q4_K, e
     return w
 
 
+def synth_target_weights_blocks(cfg: ModelConfig, seed: int, wtype: int = synth.Q4_K, attn_type: int = synth.Q6_K,
+                                embd_type: int = synth.Q6_K):
+    """The dictionary of synth_target_weights with every matrix made of random quant blocks at N(0, 1/n_in)-like
+    magnitudes (synth.random_blocks_scaled) instead of quantised Gaussians: seconds instead of minutes for the
+    128-expert shape, on the host, so that the same bytes feed the CPU checker."""
+    rng = np.random.default_rng(seed)
+    H, q_dim, kv_dim = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
+
+    def mat(qtype, n_out, n_in, std=None):
+        return (qtype, synth.random_blocks_scaled(qtype, n_out, n_in, std if std is not None else n_in ** -0.5, rng))
+
+    w = {"token_embd": mat(embd_type, cfg.vocab, H, 1.0), "output": mat(embd_type, cfg.vocab, H),
+         "output_norm": _norm_w(rng, H), "layers": []}
+    for _ in range(cfg.n_layers):
+        ffn = cfg.ffn_shared if cfg.n_expert else cfg.ffn
+        L = {"attn_norm": _norm_w(rng, H), "q_norm": _norm_w(rng, cfg.head_dim), "k_norm": _norm_w(rng, cfg.head_dim),
+             "post_norm": _norm_w(rng, H), "wq": mat(attn_type, q_dim, H), "wk": mat(attn_type, kv_dim, H),
+             "wv": mat(attn_type, kv_dim, H), "wo": mat(attn_type, H, q_dim), "gate": mat(wtype, ffn, H),
+             "up": mat(wtype, ffn, H), "down": mat(wtype, H, ffn)}
+        if cfg.n_expert:
+            fe = cfg.ffn_expert
+            L["router"] = mat(synth.Q8_0, cfg.n_expert, H)
+            L["shexp_gate"] = (rng.standard_normal(H) * H ** -0.5).astype(np.float32)
+            L["gate_exps"] = mat(wtype, cfg.n_expert * fe, H)
+            L["up_exps"] = mat(wtype, cfg.n_expert * fe, H)
+            L["down_exps"] = mat(wtype, cfg.n_expert * H, fe)
+        w["layers"].append(L)
+    return w
+
+
 def synth_draft_weights(cfg: DraftConfig, seed: int, wtype: int = synth.Q4_K, swa_layers=(), vocab=None,
                         codebook_type: int = synth.Q4_K):
     rng = np.random.default_rng(seed + 7919)

@@ -155,6 +155,24 @@ def extreme_blocks(qtype: int, n_blocks: int, seed: int) -> np.ndarray:
     return out
 
 
+def random_blocks_scaled(qtype: int, n_out: int, n_in: int, std: float, rng) -> np.ndarray:
+    """[n_out, row_bytes] uint8 on the host: random quant codes with super-block scales chosen so that the dequantised
+    weights have zero mean and roughly the standard deviation `std` (the host twin of random_blocks_device, for
+    shapes too large for the quantisers; both the HIP kernels and the CPU checker consume the bytes as they are)."""
+    nblk = n_out * (n_in // BLOCK_ELEMS[qtype])
+    out = rng.integers(0, 256, (nblk, BLOCK_BYTES[qtype]), dtype=np.uint8)
+    if qtype == Q4_K:
+        d = std / 257.0
+        out[:, 0:2] = _f16_bytes(np.full(1, d, np.float32))
+        out[:, 2:4] = _f16_bytes(np.full(1, 7.5 * d, np.float32))
+    elif qtype == Q6_K:
+        out[:, 192:208] = rng.integers(-16, 16, (nblk, 16)).astype(np.int8).view(np.uint8)
+        out[:, 208:210] = _f16_bytes(np.full(1, std / 170.0, np.float32))
+    else:
+        out[:, 0:2] = _f16_bytes(np.full(1, std / 74.0, np.float32))
+    return out.reshape(n_out, -1)
+
+
 def random_blocks_device(qtype: int, n_out: int, n_in: int, std: float, gen, device):
     """[n_out, row_bytes] uint8 on `device`: random quant codes with super-block scales set so that the
     dequantised weights have zero mean and roughly the standard deviation `std`.

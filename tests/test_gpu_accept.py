@@ -307,27 +307,40 @@ def test_seeded_trials_small_vocab(ctx, oracle, mode, kind):
     assert lengths[0] > 0 and lengths[1:].sum() > 0  # both outcomes exercised
 
 
-def test_seeded_trials_full_vocab_dense(ctx, oracle):
-    """vocab 151936, block 16, draft = target + N(0, 0.5), Philox stream: 200 seeded trials"""
+@pytest.mark.parametrize("kind,n_trials", [(dfl.RNG_PHILOX, 10000), (dfl.RNG_XOSHIRO, 2000)])
+def test_seeded_trials_full_vocab_dense(ctx, oracle, kind, n_trials):
+    """Stochastic acceptance at its benchmark size: vocabulary 151936, block 16, target logits N(0, 3), draft = target +
+    N(0, 0.5), temperature 0.7 / top-p 0.95 / top-k 20, vocabulary-wide draft distribution; seeds 0 .. n_trials - 1:
+    10000 trials on the Philox stream, 2000 on xoshiro256++.  Accepted length, tokens, carry, stop reason and
+    draws used equal the oracle's in every trial.  Logits are generated on the device a batch at a time and copied
+    to the host, where the oracle decides the batch's trials in parallel."""
     import torch
 
-    vocab, n, T = 151936, 16, 0.7
+    vocab, n, T, batch = 151936, 16, 0.7, 32
     g = torch.Generator(device="cuda")
-    acc_total = 0
-    for seed in range(200):
-        g.manual_seed(seed)
-        tl = torch.randn((n, vocab), device="cuda", generator=g) * 3
-        dl = tl[: n - 1] + torch.randn((n - 1, vocab), device="cuda", generator=g) * 0.5
-        drafts = torch.multinomial(torch.softmax(dl.double() / T, dim=1), 1, generator=g).flatten().tolist()
-        toks = [seed % vocab] + drafts
-        gs = dfl.Sampler(T, top_k=20, top_p=0.95, seed=seed, rng_kind=dfl.RNG_PHILOX)
-        os_ = oracle.make_sampler(T, 20, 0.95, 0.0, seed, dfl.RNG_PHILOX)
-        gd = ctx.decide_dflash_accept_prefix(toks, tl, vocab, None, gs, 100, [], draft_logits=dl, draft_temperature=T)
-        rc, od = oracle.decide_accept_prefix_dense(toks, tl.cpu().numpy(), dl.cpu().numpy(), vocab, T, os_, 100, [])
-        assert rc == 0 and gd.key() == od.key(), f"trial {seed}"
-        assert gs.state() == oracle.sampler_state(os_)
-        acc_total += len(gd.accepted_drafts)
-    assert acc_total > 0
+    acc_hist = np.zeros(n, np.int64)
+    for b0 in range(0, n_trials, batch):
+        nb = min(batch, n_trials - b0)
+        g.manual_seed(1_000_003 * (kind + 1) + b0)
+        tl = torch.randn((nb, n, vocab), device="cuda", generator=g) * 3
+        dl = tl[:, : n - 1] + torch.randn((nb, n - 1, vocab), device="cuda", generator=g) * 0.5
+        drafts = torch.multinomial(torch.softmax(dl.reshape(-1, vocab).double() / T, dim=1), 1, generator=g).reshape(nb, n - 1)
+        toks = torch.cat([torch.arange(b0, b0 + nb, device="cuda").reshape(nb, 1) % vocab, drafts], dim=1).to(torch.int32).cpu().numpy()
+        gpu = []
+        for t in range(nb):
+            gs = dfl.Sampler(T, top_k=20, top_p=0.95, seed=b0 + t, rng_kind=kind)
+            gd = ctx.decide_dflash_accept_prefix(toks[t].tolist(), tl[t], vocab, None, gs, 100, [], draft_logits=dl[t],
+                                                 draft_temperature=T)
+            gpu.append((gd, gs))
+        samplers = [oracle.make_sampler(T, 20, 0.95, 0.0, b0 + t, kind) for t in range(nb)]
+        status, outs = oracle.decide_accept_prefix_batch(toks, tl.cpu().numpy(), dl.cpu().numpy(), T, samplers, 100)
+        for t in range(nb):
+            gd, gs = gpu[t]
+            assert status[t] == 0 and gd.key() == outs[t].key(), f"trial {b0 + t}"
+            assert gs.state() == oracle.sampler_state(samplers[t]), f"trial {b0 + t}"
+            acc_hist[len(gd.accepted_drafts)] += 1
+        del tl, dl
+    assert acc_hist.sum() == n_trials and acc_hist[0] > 0 and acc_hist[1:].sum() > 0  # rejections at row 0 and later
 
 
 def test_greedy_longest_prefix_full_vocab(ctx, oracle):
@@ -345,8 +358,108 @@ def test_greedy_longest_prefix_full_vocab(ctx, oracle):
         assert (r[1].carry_kind, r[1].carry_token) == (want_kind, int(am[k]))
 
 
-def test_unsupported_top_k_declines(ctx):
-    s = dfl.Sampler(1.0, top_k=0, seed=1)
-    with pytest.raises(dfl.DFlashError) as e:
-        ctx.decide_dflash_accept_prefix([0, 1], dev(np.zeros((2, 4096), np.float32)), 4096, None, s, 4, [])
-    assert e.value.kind == "Unsupported" and s.draws == 0
+QWEN_CHAT = dict(temperature=0.7, top_k=200, top_p=1.0, min_p=0.05)  # SamplingConfig::qwen_chat, sampling.rs:47-56
+
+
+def _wide_block(rng, vocab, n, spread=3.0):
+    tl = (rng.standard_normal((n, vocab)) * spread).astype(np.float32)
+    dl = (tl[: n - 1] + rng.standard_normal((n - 1, vocab)).astype(np.float32) * 0.5).astype(np.float32)
+    return tl, dl
+
+
+@pytest.mark.parametrize("top_k", [0, 64, 65, 200, 5000])
+@pytest.mark.parametrize("filters", [dict(top_p=1.0, min_p=0.0), dict(top_p=0.9, min_p=0.0), dict(top_p=1.0, min_p=0.05),
+                                     dict(top_p=0.97, min_p=0.02)])
+def test_wide_top_k_matches_oracle(ctx, oracle, top_k, filters):
+    """top_k = 0 (whole vocabulary, sampling.rs:1198-1214), the kMaxK boundary (64 inline, 65 through the sorted
+    arrays), the reference's chat value 200 and top_k = vocabulary, with every filter combination, for the three
+    couplings: decisions, tokens, draws and sampler state equal the oracle's."""
+    vocab, n = 5000, 6
+    rng = np.random.default_rng(1000 + top_k)
+    for trial in range(12):
+        tl, dl = _wide_block(rng, vocab, n)
+        T = 0.7
+        for mode in ("deterministic", "sparse", "dense"):
+            if mode == "deterministic":
+                drafts = [int(np.argmax(tl[r])) if rng.random() < 0.7 else int(rng.integers(vocab)) for r in range(n - 1)]
+            else:
+                drafts = sample_drafts(dl, T, rng)
+            toks = [int(rng.integers(vocab))] + drafts
+            skw = dict(temperature=T, top_k=top_k, seed=trial, **filters)
+            props = None
+            if mode == "sparse":
+                props = []
+                for r in range(n - 1):
+                    top = np.argsort(-dl[r])[:16]
+                    if drafts[r] not in top:
+                        top[-1] = drafts[r]
+                    z = dl[r][top].astype(np.float64) / T
+                    props.append((drafts[r], [(int(a), float(b)) for a, b in zip(top, np.exp(z - z.max()))]))
+            r = both(ctx, oracle, toks, tl, vocab, props, 100, [], draft=dl if mode == "dense" else None, draft_T=T, **skw)
+            assert r[2] == 0
+            assert_same(oracle, *r)
+
+
+def test_wide_top_k_edge_rows(ctx, oracle):
+    """NaN, +inf ties, all -inf but one, equal logits (ties go to the lower token id) and a -0.0 / +0.0 pair through
+    the sorted path."""
+    vocab = 3000
+    rng = np.random.default_rng(7)
+    base = (rng.standard_normal((2, vocab)) * 2).astype(np.float32)
+    cases = []
+    a = base.copy(); a[0, 1234] = np.nan; cases.append(a)
+    a = base.copy(); a[0, [5, 2500]] = np.inf; cases.append(a)
+    a = np.full((2, vocab), -np.inf, np.float32); a[:, 77] = 1.0; cases.append(a)
+    a = np.zeros((2, vocab), np.float32); cases.append(a)
+    a = base.copy(); a[0, 10] = -0.0; a[0, 11] = 0.0; a[0, 12:40] = 0.0; cases.append(a)
+    a = np.full((2, vocab), -np.inf, np.float32); cases.append(a)
+    for rows in cases:
+        for seed in range(4):
+            r = both(ctx, oracle, [1, int(np.nanargmax(np.where(np.isfinite(rows[0]), rows[0], -1e30)))], rows, vocab, None, 10, [],
+                     temperature=0.9, top_k=0, top_p=0.95, min_p=0.01, seed=seed)
+            assert_same(oracle, *r)
+
+
+def test_qwen_chat_preset_full_vocabulary(ctx, oracle):
+    """The reference's default chat sampler (temperature 0.7, top_k 200, min_p 0.05) at vocabulary 151936, block 16, both
+    random streams, coupled to drafts sampled from the vocabulary-wide draft distribution and to deterministic drafts."""
+    import torch
+
+    vocab, n, T = 151936, 16, 0.7
+    g = torch.Generator(device="cuda")
+    for kind in (dfl.RNG_XOSHIRO, dfl.RNG_PHILOX):
+        for seed in range(6):
+            g.manual_seed(100 + seed)
+            tl = torch.randn((n, vocab), device="cuda", generator=g) * 3
+            dl = tl[: n - 1] + torch.randn((n - 1, vocab), device="cuda", generator=g) * 0.5
+            drafts = torch.multinomial(torch.softmax(dl.double() / T, dim=1), 1, generator=g).flatten().tolist()
+            toks = [seed] + drafts
+            for dense in (True, False):
+                gs = dfl.Sampler(seed=seed, rng_kind=kind, **QWEN_CHAT)
+                os_ = oracle.make_sampler(QWEN_CHAT["temperature"], QWEN_CHAT["top_k"], QWEN_CHAT["top_p"], QWEN_CHAT["min_p"], seed, kind)
+                if dense:
+                    gd = ctx.decide_dflash_accept_prefix(toks, tl, vocab, None, gs, 100, [], draft_logits=dl, draft_temperature=T)
+                    rc, od = oracle.decide_accept_prefix_dense(toks, tl.cpu().numpy(), dl.cpu().numpy(), vocab, T, os_, 100, [])
+                else:
+                    gd = ctx.decide_dflash_accept_prefix(toks, tl, vocab, None, gs, 100, [])
+                    rc, od = oracle.decide_accept_prefix(toks, tl.cpu().numpy(), vocab, None, os_, 100, [])
+                assert rc == 0 and gd.key() == od.key(), (kind, seed, dense)
+                assert gs.state() == oracle.sampler_state(os_)
+
+
+def test_full_vocabulary_order_top_k_zero(ctx, oracle):
+    """top_k = 0 at vocabulary 151936 with top_p: the chain walks all 151936 ordered candidates."""
+    import torch
+
+    vocab, n = 151936, 4
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    tl = torch.randn((n, vocab), device="cuda", generator=g) * 2
+    for seed in range(4):
+        toks = [3] + [int(t) for t in torch.argmax(tl[: n - 1], dim=1).tolist()]
+        gs = dfl.Sampler(1.0, top_k=0, top_p=0.9, seed=seed)
+        os_ = oracle.make_sampler(1.0, 0, 0.9, 0.0, seed, 0)
+        gd = ctx.decide_dflash_accept_prefix(toks, tl, vocab, None, gs, 100, [])
+        rc, od = oracle.decide_accept_prefix(toks, tl.cpu().numpy(), vocab, None, os_, 100, [])
+        assert rc == 0 and gd.key() == od.key(), seed
+        assert gs.state() == oracle.sampler_state(os_)

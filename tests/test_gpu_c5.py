@@ -1,0 +1,110 @@
+"""GPU parity at the end-to-end configuration's own widths, at reduced depth: a 35B-A3B-shaped mixture-of-experts
+target (hidden 2048, 16 q / 2 kv heads of 256, 128 experts top-8 with F_exp 768 plus a shared expert, Q4_K experts,
+Q6_K attention, vocabulary 151936; 2 layers instead of 40) and a 5-layer-shaped drafter (2 layers here) in one
+generation loop.  The 128-expert routing kernel, the batched expert GEMMs at their real expert count and the
+151936-wide output head are compared with the CPU oracle; the loop is compared with the serial greedy decode.
+
+Weights are random quant blocks (synth.random_blocks_scaled): the quantisers would take minutes at this size, and
+both sides consume the same bytes.  Top-8-of-128 routing is discontinuous: the seeds are chosen so that no routing
+decision of the compared rows is a near tie (the oracle reports its smallest relative gap; asserted below)."""
+import numpy as np
+import pytest
+
+import qwen_llm_amd as dfl
+
+pytestmark = pytest.mark.gpu
+
+C5 = dfl.ModelConfig(n_layers=2, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=151936, n_expert=128,
+                     n_expert_used=8, ffn_expert=768, ffn_shared=768)
+D5 = dfl.DraftConfig(n_layers=2, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=6144, block_size=16, n_taps=2)
+TAPS = [0, 1]
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = dfl.Context(0, workspace_bytes=256 << 20)
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def weights():
+    return dfl.synth_target_weights_blocks(C5, 41)
+
+
+def close(got, want, label, tol=3e-2, l2_tol=5e-3):
+    got, want = np.asarray(got, np.float32), np.asarray(want, np.float32)
+    assert got.shape == want.shape and np.all(np.isfinite(got)), label
+    rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    err = np.max(np.abs(got - want) / np.maximum(np.abs(want), rms))
+    l2 = np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want.astype(np.float64))
+    print(f"{label}: max err {err:.3e} l2 {l2:.3e}")
+    assert err <= tol and l2 <= l2_tol, f"{label}: max err {err:.3e}, rel l2 {l2:.3e}"
+
+
+def test_moe_128_experts_verify_matches_oracle(ctx, oracle, weights):
+    model = dfl.TargetModel(ctx, C5, weights)
+    omodel, _keep = oracle.build_model(C5.as_dict(), weights)
+    sess = dfl.Session(ctx, model, 64, TAPS)
+    ostate = oracle.TargetState(C5.as_dict(), 64)
+    rng = np.random.default_rng(52)
+    pos = 0
+    oracle.router_margin_take()
+    for n in (16, 3):
+        blk = rng.integers(0, C5.vocab, n).tolist()
+        out = sess.encode_packed_verify_layer_major(blk, pos, want_logits=True)
+        lo, hid = oracle.target_verify(omodel, ostate, blk, pos, TAPS)
+        margin = oracle.router_margin_take()
+        assert margin > 5e-3, f"seed no longer decisive: smallest relative router gap {margin:.2e}"
+        close(out.hidden_capture.cpu().numpy(), hid, f"C5-shape hidden n={n}")
+        close(out.logits.cpu().numpy(), lo, f"C5-shape logits n={n}")
+        top = np.sort(lo, axis=1)
+        decided = (top[:, -1] - top[:, -2]) > 2e-2 * lo.std()
+        assert np.array_equal(np.asarray(out.argmax_host)[decided], lo.argmax(axis=1)[decided])
+        pos += n
+    sess.close()
+
+
+def test_generate_on_the_moe_shape_equals_serial_greedy(ctx, weights):
+    """MoE target + drafter in one loop at the end-to-end widths: every emitted token is the target's serial greedy
+    decode through the same kernels, through full accepts, partial accepts and rollbacks."""
+    model = dfl.TargetModel(ctx, C5, weights)
+    rng = np.random.default_rng(7)
+
+    def mat(n_out, n_in):
+        return (dfl.synth.Q4_K, dfl.synth.random_blocks_scaled(dfl.synth.Q4_K, n_out, n_in, n_in ** -0.5, rng))
+
+    def norm(n):
+        return (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+
+    H, qd, kvd = D5.hidden, D5.n_q * D5.head_dim, D5.n_kv * D5.head_dim
+    dw = {"fc": mat(H, D5.n_taps * H), "hidden_norm": norm(H), "output_norm": norm(H), "layers": []}
+    for _ in range(D5.n_layers):
+        dw["layers"].append({"attn_norm": norm(H), "q_norm": norm(D5.head_dim), "k_norm": norm(D5.head_dim), "post_norm": norm(H),
+                             "wq": mat(qd, H), "wk": mat(kvd, H), "wv": mat(kvd, H), "wo": mat(H, qd), "gate": mat(D5.ffn, H),
+                             "up": mat(D5.ffn, H), "down": mat(H, D5.ffn), "is_swa": 0})
+    head = dfl.DraftHead(ctx, D5, dw)
+    prompt = rng.integers(0, C5.vocab - 1, 37).tolist()
+    n_tok = 30
+    serial = dfl.Session(ctx, model, 128, TAPS)
+    out = None
+    for s in range(0, len(prompt), 16):
+        out = serial.encode_packed_verify_layer_major(prompt[s:s + 16], s)
+    want = [out.argmax_host[-1]]
+    while len(want) < n_tok + 16:
+        want.append(serial.encode_packed_verify_layer_major([want[-1]], len(prompt) + len(want) - 1).argmax_host[0])
+    serial.close()
+    dec = dfl.SpeculativeDecoder(ctx, model, head, TAPS, 128, C5.vocab - 1)
+    first = dec.prefill(prompt)
+    assert first == want[0]
+
+    def override(tokens, position):
+        done = len(tokens)
+        k = (0, 15, 3, 7)[(position // 2) % 4]
+        return want[done:done + k] + [-1] * (15 - k)
+
+    tokens, stats = dec.generate(first, n_tok, draft_override_fn=override)
+    assert tokens == want[:n_tok], f"diverged at {next(i for i, (a, b) in enumerate(zip(tokens, want)) if a != b)}"
+    assert stats["accepted_drafts"] > 0 and stats["spec_steps"] >= 2
+    assert dec.session.kv_n_pos == len(prompt) + n_tok - 1
+    dec.close()

@@ -192,13 +192,17 @@ def test_sampled_dflash2_step_equals_its_parts(ctx, world, oracle):
     dec.close()
 
 
-def test_generate_sampled_equals_serial_sampler(ctx, world, oracle):
+@pytest.mark.parametrize("kw", [
+    dict(temperature=0.8, top_k=20, top_p=0.95, min_p=0.0, seed=1234),
+    dict(temperature=0.7, top_k=200, top_p=1.0, min_p=0.05, seed=5),   # SamplingConfig::qwen_chat (sampling.rs:47-56)
+    dict(temperature=1.0, top_k=0, top_p=0.9, min_p=0.0, seed=6),      # whole-vocabulary order
+], ids=["top20", "qwen_chat", "top_k_off"])
+def test_generate_sampled_equals_serial_sampler(ctx, world, oracle, kw):
     """Deterministic-proposal coupling == serial sampling with the same stream (sampling.rs:2837-2865).
     The serial stream is the CPU oracle's sampler applied to the logits of a token-by-token pass through
     the same device kernels: with random-init weights the top-20 logits are near ties, so a stream
     drawn from the oracle's own logits (1e-3 away) is not a usable expectation."""
     n_tok = 40
-    kw = dict(temperature=0.8, top_k=20, top_p=0.95, min_p=0.0, seed=1234)
     osamp = oracle.make_sampler(**kw)
     serial = dfl.Session(ctx, world["model"], 256, TAPS)
     out = None

@@ -226,3 +226,25 @@ def test_dense_block_decision_equals_rowwise_couplings(oracle):
             carry = (oracle.CARRY_BONUS, oracle.sample(b, tl[n - 1])[1])
         assert (d.accepted(), d.carry_kind, d.carry_token) == (acc, carry[0], carry[1])
         same_rng(oracle, a, b)
+
+
+def test_batched_decisions_equal_single_calls(oracle):
+    """The OpenMP batch entry used by the long GPU runs is the per-block decision, trial by trial."""
+    rng = np.random.default_rng(12)
+    V, n, T, B = 3000, 6, 0.7, 9
+    tl = (rng.standard_normal((B, n, V)) * 3).astype(np.float32)
+    dl = tl[:, : n - 1] + rng.standard_normal((B, n - 1, V)).astype(np.float32) * 0.5
+    toks = rng.integers(0, V, (B, n)).astype(np.int32)
+    toks[:, 1:] = dl.argmax(axis=2)
+    for dense in (True, False):
+        for kind in (0, 1):
+            a = [oracle.make_sampler(T, 20, 0.95, 0.0, 100 + b, kind) for b in range(B)]
+            b_ = [oracle.make_sampler(T, 20, 0.95, 0.0, 100 + b, kind) for b in range(B)]
+            status, outs = oracle.decide_accept_prefix_batch(toks, tl, dl if dense else None, T, a, 50)
+            for t in range(B):
+                if dense:
+                    rc, od = oracle.decide_accept_prefix_dense(toks[t].tolist(), tl[t], dl[t], V, T, b_[t], 50, [])
+                else:
+                    rc, od = oracle.decide_accept_prefix(toks[t].tolist(), tl[t], V, None, b_[t], 50, [])
+                assert rc == status[t] == 0 and od.key() == outs[t].key()
+                assert oracle.sampler_state(a[t]) == oracle.sampler_state(b_[t])
