@@ -25,6 +25,7 @@
 //    eight consecutive weights per lane are dequantised to f16 and fed to the same MFMA.
 #include "common.h"
 
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -444,7 +445,12 @@ __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, const Q4KBatch &bt
 // split over several workgroups of the streaming kernel; adds the partial tiles in workgroup
 // order (so sums are run-to-run deterministic) and writes Y.  Spreading this over the chip
 // instead of leaving it to the group's last contributor matters when K is long: a group then
-// has a dozen partial tiles.
+// has a dozen partial tiles.  (Measured on MI355X: a last-arriver reduction inside the streaming
+// kernel, with device-scope stores, one atomic arrival count per tile and device-scope loads, is slower
+// than this second launch, 22.7 / 27.9 / 16.3 us per call against 21.8 / 20.7 / 12.8 us on the three
+// M = 16 projection shapes: the contributors sit on different XCDs, so the chain store -> count -> load
+// crosses to memory three times at the tail of the kernel; with device-scope fences instead, each of which
+// writes back and invalidates an XCD's whole L2, it is nine times slower.)
 template <int kWaves>
 __global__ void __launch_bounds__(256)
     q4k_reduce_kernel(const float *__restrict__ partials, float *__restrict__ y, int n_out, int nb, int n_rows,
@@ -706,6 +712,215 @@ __global__ void __launch_bounds__(64 * kWaves)
         t[3] = cyc_n;
     }
 #endif
+}
+
+// ----------------------------------------------------------------------------
+// Q4_K slab kernel: the streaming kernel for a single matrix whose ranges are short
+// ----------------------------------------------------------------------------
+//
+// Same work split, output flush and split-K reduction as gemm_q4k_stream_kernel (16-wave tile groups,
+// one contiguous range of (tile group x super-block) stages per workgroup), for the common case that a
+// workgroup's range is at most kSlabStages stages long: every C2-shaped projection on a 256-CU chip.
+// What differs is what the waves of a workgroup share:
+//   * the activations of ALL the range's stages are converted to f16 MFMA fragments once, at the start,
+//     into a resident slab in LDS (8 KB per stage), together with each stage's sub-block sums;
+//   * every wave then streams its own 16 weight rows through a private ring of three LDS buffers
+//     (direct-to-LDS loads of 144 row-contiguous 16-byte pieces per stage) and never meets the other
+//     waves again: no barrier per stage, no per-stage activation work, and a wave starts computing as
+//     soon as ITS first 2.3 KB have landed instead of when the whole 37 KB stage has.
+// The sub-block minima cost one MFMA per stage instead of eight: sum_k x[m][k] * (dmin m_j)[n] over a
+// sub-block j is (sum_k x[m][k]) * (dmin m_j)[n], so the stage's 16 x 8 sub-block sums of the (f16-rounded)
+// activations, split into f16 high and low parts, form one A fragment (k-slots: high and low part of
+// sub-blocks 2g and 2g+1 for lane group g, four slots zero) against B = the lane's two minima twice.
+constexpr int kSlabStages = 6;
+constexpr int kSlabWaves = 16;
+constexpr int kSlabRing = 3;
+constexpr int kSlabWavePieces = 144;                          // 16 rows x 9 pieces of 16 bytes
+constexpr int kSlabStageBytes = kQ4KBlockFrags * 16 + 64 * 8; // 512 A fragments + 64 x (4 f16) sub-block sums
+constexpr int kSlabWaveLoads = 3;                             // 64 + 64 + 16 lanes
+constexpr size_t kSlabLdsBytes = static_cast<size_t>(kSlabStages) * kSlabStageBytes +
+                                 static_cast<size_t>(kSlabWaves) * kSlabRing * kSlabWavePieces * 16;
+static_assert(kSlabLdsBytes <= 160 * 1024, "one workgroup per CU, all of its LDS");
+
+// One stage of a wave's tile: 8 MFMAs for the scaled nibbles, one for the minima.
+__device__ __forceinline__ void q4k_slab_compute(const u32x4_t *blk, const half8_t *a, const half4_t *twin, int g, uint32_t sc_sel,
+                                                 Q4KMagic magic, float4_t &acc, float4_t &acc_min) {
+    const u32x4_t hdr = blk[0], q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
+    half8_t af[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) af[t] = a[t * 64];
+    const half4_t tw = *twin;
+    // scales and minima of sub-blocks 2g and 2g+1 (see q4k_compute)
+    const uint32_t upper = 0u - static_cast<uint32_t>(g >> 1);
+    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu, mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t sc_word = (sc_hi & upper) | (sc_lo & ~upper), mn_word = (mn_hi & upper) | (mn_lo & ~upper);
+    const half2_t dm = __builtin_bit_cast(half2_t, hdr.x);
+    const half2_t p_sc = as_half2(__builtin_amdgcn_perm(0x64646464u, sc_word, sc_sel));
+    const half2_t p_mn = as_half2(__builtin_amdgcn_perm(0x64646464u, mn_word, sc_sel));
+    const half2_t neg = dm * splat(static_cast<_Float16>(-1024.0f));
+    const half2_t S = __builtin_elementwise_fma(p_sc, splat(dm[0]), splat(neg[0]));
+    const half2_t M = __builtin_elementwise_fma(p_mn, splat(dm[1]), splat(neg[1]));
+    const half2_t unbias = {static_cast<_Float16>(-1024.0f), static_cast<_Float16>(-64.0f)};
+    const half2_t Cs = S * unbias;
+    const half2_t s2l = splat(S[0]), c2l = splat(Cs[0]);
+    const half2_t s2h = splat(S[1]), c2h = splat(Cs[1]);
+    const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const _Float16 zero = static_cast<_Float16>(0.0f);
+    const half8_t a_min = {tw[0], tw[1], tw[2], tw[3], zero, zero, zero, zero};
+    const half8_t b_min = {M[0], M[1], M[0], M[1], zero, zero, zero, zero};
+    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_min, b_min, acc_min, 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bh, acc, 0, 0, 0);
+    }
+}
+
+// s_waitcnt vmcnt(3 n): at most n load groups (three instructions each) still in flight, n uniform
+__device__ __forceinline__ void q4k_slab_wait_groups(int n) {
+    if (n <= 0)
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+    else if (n == 1)
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(3));
+    else if (n == 2)
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(6));
+    else if (n == 3)
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(9));
+    else if (n == 4)
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(12));
+    else if (n == 5)
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(15));
+    else
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(18));
+}
+
+template <typename XT>
+__global__ void __launch_bounds__(64 * kSlabWaves)
+    gemm_q4k_slab_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
+                         float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt) {
+    constexpr int kW = kSlabWaves;
+    extern __shared__ half8_t lds[];
+    uint8_t *slab = reinterpret_cast<uint8_t *>(lds);                                   // [kSlabStages][kSlabStageBytes]
+    half8_t *ring = reinterpret_cast<half8_t *>(slab + kSlabStages * kSlabStageBytes);  // [wave][kSlabRing][144]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    Q4KRange rg;
+    rg.nb = nb;
+    rg.n_wg = gridDim.x;
+    rg.total = n_groups * nb;
+    rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
+    rg.it_begin = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * rg.wg, bt.by_wg));
+    rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * (rg.wg + 1), bt.by_wg));
+    const int len = rg.it_end - rg.it_begin;  // <= kSlabStages (host)
+    if (len <= 0) return;
+    rg.first_group = static_cast<int>(q4k_div(rg.it_begin, bt.by_nb));
+    const int b0 = rg.it_begin - rg.first_group * nb;
+    const uint32_t row_bytes = static_cast<uint32_t>(nb) * DFL_Q4_K_BYTES;
+    const uint32_t n_in = static_cast<uint32_t>(nb) * DFL_QK_K;
+    const size_t group_bytes = static_cast<size_t>(16 * kW) * row_bytes;
+
+    // ---- this wave's weight loads: piece p = 64 j + lane of its 16 rows x 9 pieces (j = 2: 16 lanes) ----
+    half8_t *my_ring = ring + wave * (kSlabRing * kSlabWavePieces);
+    uint32_t w_off[kSlabWaveLoads];
+    auto set_w_offsets = [&](int group) {  // rows past n_out (ragged last group) re-read the last row
+        const int last = n_out - 1 - (group * kW + wave) * 16;
+#pragma unroll
+        for (int j = 0; j < kSlabWaveLoads; j++) {
+            const int p = min(64 * j + lane, kSlabWavePieces - 1);
+            const int r = max(min(p / 9, last), -(wave * 16));  // a wave wholly past n_out stays inside the group
+            w_off[j] = static_cast<uint32_t>(wave * 16 + r) * row_bytes + static_cast<uint32_t>(p % 9) * 16u;
+        }
+    };
+    const bool ragged = n_groups * 16 * kW > n_out;
+    set_w_offsets(rg.first_group);
+    const uint8_t *wstage = w + static_cast<size_t>(rg.first_group) * group_bytes + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
+    int bw = b0, gw = rg.first_group, w_issued = 0;
+    auto issue_w = [&]() {  // the next stage's 144 pieces into ring buffer (w_issued % 3)
+        half8_t *buf = my_ring + (w_issued % kSlabRing) * kSlabWavePieces;
+        __builtin_amdgcn_global_load_lds((gptr_t)(wstage + w_off[0]), (lptr_t)(buf), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(wstage + w_off[1]), (lptr_t)(buf + 64), 16, 0, 0);
+        if (lane < 16) __builtin_amdgcn_global_load_lds((gptr_t)(wstage + w_off[2]), (lptr_t)(buf + 128), 16, 0, 0);
+        w_issued++;
+        wstage += DFL_Q4_K_BYTES;
+        if (++bw == nb) {
+            bw = 0;
+            gw++;
+            if (w_issued < len) {
+                wstage = w + static_cast<size_t>(gw) * group_bytes;
+                if (ragged) set_w_offsets(gw);
+            }
+        }
+    };
+
+    // ---- activations of every stage of the range: loads first (they come from L2 and are needed first) ----
+    // thread -> (row m, four values k = 4c .. 4c+3): wave = sub-block pair half, see q4k_lane_x_offsets
+    const int xm = 8 * (wave & 1) + (lane & 7), xc = 8 * (wave >> 1) + (lane >> 3);
+    const uint32_t x_off = (static_cast<uint32_t>(min(xm, n_rows - 1)) * n_in + 4u * xc) * static_cast<uint32_t>(sizeof(XT));
+    const uint32_t xw_off = static_cast<uint32_t>((((xc & 15) >> 1) * 64 + xm + 16 * (xc >> 4)) * 16 + 8 * (xc & 1));
+    const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(x);
+    typename Q4KXVec<XT>::type raw[kSlabStages];
+    {
+        int b = b0;
+#pragma unroll
+        for (int t = 0; t < kSlabStages; t++) {
+            if (t < len) q4k_load_x_vec(xbytes + static_cast<size_t>(b) * (DFL_QK_K * sizeof(XT)), x_off, raw[t]);
+            if (++b == nb) b = 0;
+        }
+    }
+    issue_w();
+    if (len > 1) issue_w();
+    q4k_slab_wait_groups(w_issued);  // the activations (older than every weight load) are in registers
+#pragma unroll
+    for (int t = 0; t < kSlabStages; t++) {
+        if (t < len) {
+            asm volatile("" : "+v"(raw[t]));
+            uint8_t *stage = slab + t * kSlabStageBytes;
+            _Float16 h[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) h[i] = static_cast<_Float16>(raw[t][i]);
+            const half4_t frag = {h[0], h[2], h[1], h[3]};
+            *reinterpret_cast<half4_t *>(stage + xw_off) = frag;
+            // sub-block sum of the rounded values over the eight lanes that share this row
+            float sum = (static_cast<float>(h[0]) + static_cast<float>(h[1])) + (static_cast<float>(h[2]) + static_cast<float>(h[3]));
+            sum += __shfl_xor(sum, 8, 64);
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            if (lane < 8) {
+                const int j = wave >> 1;  // this wave's sub-block
+                const _Float16 hi = static_cast<_Float16>(sum), lo = static_cast<_Float16>(sum - static_cast<float>(hi));
+                _Float16 *tw = reinterpret_cast<_Float16 *>(stage + kQ4KBlockFrags * 16) + (xm + 16 * (j >> 1)) * 4 + (j & 1);
+                tw[0] = hi;
+                tw[2] = lo;
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitLds);
+    __builtin_amdgcn_s_barrier();  // the slab is complete; from here on the waves run independently
+
+    const int n = lane & 15, g = lane >> 4;
+    const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
+    const Q4KMagic magic = q4k_magic();
+    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0}, stash = {0, 0, 0, 0};
+    int gc = rg.first_group, bc = b0;
+    for (int t = 0; t < len; t++) {
+        q4k_slab_wait_groups(w_issued - 1 - t);  // loads land in order: stage t has when only later ones are in flight
+        if (w_issued < len) issue_w();           // stage t+2 into the buffer stage t-1 has been read out of
+        const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(my_ring + (t % kSlabRing) * kSlabWavePieces) + n * 9;
+        const uint8_t *stage = slab + t * kSlabStageBytes;
+        q4k_slab_compute(blk, reinterpret_cast<const half8_t *>(stage) + lane,
+                         reinterpret_cast<const half4_t *>(stage + kQ4KBlockFrags * 16) + lane, g, sc_sel, magic, acc, acc_min);
+        if (++bc == nb || t + 1 == len) {
+            q4k_flush<kW>(rg, bt, gc, acc, acc_min, stash, y, partials, n_out, n_rows, tid);
+            bc = 0;
+            gc++;
+        }
+    }
 }
 
 // ----------------------------------------------------------------------------
@@ -1403,6 +1618,16 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     // layer take 50 us instead of 56 us).
     int waves = (!batch && static_cast<int64_t>((tiles + 15) / 16) * nb >= 2ll * ctx->n_cu) ? 16 : 8;
     waves = env_int("DFLASH_GEMM_WAVES", waves) == 16 ? 16 : 8;
+    // A single matrix whose per-workgroup range is at most kSlabStages stages long takes the slab kernel (16-wave
+    // groups): resident activation slab, wave-private weight rings, no per-stage barrier.
+    bool slab = false;
+    if (!batch && env_int("DFLASH_Q4K_SLAB", 1) && kSlabLdsBytes <= ctx->lds_bytes) {
+        const int64_t total16 = static_cast<int64_t>((tiles + 15) / 16) * nb;
+        const int64_t wgs = std::min<int64_t>(std::min<int64_t>(env_int("DFLASH_GEMM_WGS", ctx->n_cu), total16), ctx->n_partial_wgs / 2);
+        // the longest range is ceil(total / wgs) stages
+        slab = wgs >= 1 && (total16 + wgs - 1) / wgs <= kSlabStages;
+        if (slab) waves = 16;
+    }
     const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
     const int groups = gpm * max_slots * ((batch && batch->pair) ? 2 : 1);  // upper bound in batched mode (pair mode: virtual groups)
     int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
@@ -1441,7 +1666,24 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
             q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);   \
         }                                                                                                              \
     } while (0)
-    if (waves == 16 && x_type == DFLASH_TYPE_F32)
+    if (slab) {
+        const void *fn = x_type == DFLASH_TYPE_F32 ? reinterpret_cast<const void *>(gemm_q4k_slab_kernel<float>)
+                                                   : reinterpret_cast<const void *>(gemm_q4k_slab_kernel<_Float16>);
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, fn, kSlabLdsBytes)) return rc_;
+        {
+            dfl_timed timer(ctx, st, DFL_T_GEMM);
+            if (x_type == DFLASH_TYPE_F32)
+                gemm_q4k_slab_kernel<float><<<n_wg, 64 * kSlabWaves, kSlabLdsBytes, st>>>(wb, static_cast<const float *>(x), y, partials, no,
+                                                                                         nb, n_rows, groups, bt);
+            else
+                gemm_q4k_slab_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kSlabLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
+                                                                                            partials, no, nb, n_rows, groups, bt);
+        }
+        if (split) {
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);
+            q4k_reduce_kernel<16><<<groups * 16, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);
+        }
+    } else if (waves == 16 && x_type == DFLASH_TYPE_F32)
         DFL_LAUNCH_Q4K(16, float);
     else if (waves == 16)
         DFL_LAUNCH_Q4K(16, _Float16);
