@@ -58,6 +58,8 @@ enum {
 
 /* ggml tensor type tags (crates/qwen-llm/src/tensor.rs:164-208) */
 enum { DFLASH_TYPE_F32 = 0, DFLASH_TYPE_F16 = 1, DFLASH_TYPE_Q8_0 = 8, DFLASH_TYPE_Q4_K = 12, DFLASH_TYPE_Q6_K = 14 };
+/* Not a ggml type: Q4_K blocks in this library's tiled order (dflash_repack_q4k_tiled). */
+enum { DFLASH_TYPE_Q4_K_TILED = 1012 };
 
 /* ---- context ------------------------------------------------------------------
  * Replaces MetalContext + the per-call scratch the reference keeps in
@@ -94,6 +96,17 @@ void dflash_ctx_set_graphs(dflash_ctx *ctx, int32_t enable);
 int32_t dflash_dequant(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_elems, float *out_f32,
                        dflash_stream_t stream);
 size_t dflash_row_bytes(int32_t type, size_t n_in);
+
+/* ---- Q4_K weights in tiled order -------------------------------------------------
+ * No counterpart in the reference (it streams GGUF row order, loader.rs tensors as mapped): a one-time
+ * permutation of whole 144-byte blocks, done when a matrix is uploaded, into the order the M <= 16 GEMM reads it in:
+ *   [tile group of 256 rows][super-block][tile 0..15][row 0..15][block],  last group padded with zero blocks.
+ * dflash_q4k_tiled_bytes: size of the tiled matrix (0 for a bad shape).  dflash_repack_q4k_tiled: W in GGUF row
+ * order (16-byte aligned) -> w_tiled (128-byte aligned, dflash_q4k_tiled_bytes long, not overlapping W).  The
+ * result is passed to dflash_gemm_fewrow as w_type DFLASH_TYPE_Q4_K_TILED and gives bit-identical Y.  Enqueue-only. */
+size_t dflash_q4k_tiled_bytes(int64_t n_in, int64_t n_out);
+int32_t dflash_repack_q4k_tiled(dflash_ctx *ctx, const void *w, void *w_tiled, int64_t n_in, int64_t n_out,
+                                dflash_stream_t stream);
 
 /* ---- few-row quantised GEMM ---------------------------------------------------
  * encode_mat_mat_dispatch_dflash_verify(ctx, enc, weight, x, y, n_in, n_out, n_query)

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libdflash_hip.so")
 HEADER_PATH = os.path.join(PKG_DIR, "..", "include", "dflash_hip.h")
 
 TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q6_K = 0, 1, 8, 12, 14
+TYPE_Q4_K_TILED = 1012  # Q4_K blocks in the library's tiled order (Context.repack_q4k_tiled)
 
 STATUS = {
     0: "Ok", 1: "BadShape", 2: "Unsupported", 3: "Alias", 4: "Alignment", 5: "Workspace", 6: "Hip",
@@ -113,6 +114,10 @@ def _declare(L):
     L.dflash_dequant.argtypes = [vp, i32, vp, sz, vp, vp]
     L.dflash_gemm_fewrow.restype = i32
     L.dflash_gemm_fewrow.argtypes = [vp, i32, vp, vp, i32, vp, i64, i64, i32, vp]
+    L.dflash_q4k_tiled_bytes.restype = sz
+    L.dflash_q4k_tiled_bytes.argtypes = [i64, i64]
+    L.dflash_repack_q4k_tiled.restype = i32
+    L.dflash_repack_q4k_tiled.argtypes = [vp, vp, vp, i64, i64, vp]
     L.dflash_gemm_fewrow_noalloc.restype = i32
     L.dflash_gemm_fewrow_noalloc.argtypes = [i32, vp, vp, i32, vp, i64, i64, i32, vp]
     L.dflash_gemm_fewrow_noalloc_error.restype = C.c_char_p
@@ -266,6 +271,17 @@ class Context:
         self._check(self._lib.dflash_gemm_fewrow(self._h, w_type, weight.data_ptr(), x.data_ptr(), x_type,
                                                  y.data_ptr(), n_in, n_out, n_query, _stream_ptr()))
         return y
+
+    def repack_q4k_tiled(self, weight, n_in: int, n_out: int):
+        """Q4_K blocks in GGUF row order -> a new tensor in tiled order (w_type TYPE_Q4_K_TILED): a one-time
+        permutation of whole blocks at upload; the few-row GEMM on it gives bit-identical results."""
+        torch = _torch()
+        nbytes = self._lib.dflash_q4k_tiled_bytes(n_in, n_out)
+        if nbytes == 0:
+            raise DFlashError(2, f"bad Q4_K shape {n_out} x {n_in}")
+        out = torch.empty(nbytes, dtype=torch.uint8, device=weight.device)
+        self._check(self._lib.dflash_repack_q4k_tiled(self._h, weight.data_ptr(), out.data_ptr(), n_in, n_out, _stream_ptr()))
+        return out
 
     def gemm_fewrow(self, weight, w_type: int, x, n_in: int, n_out: int):
         torch = _torch()

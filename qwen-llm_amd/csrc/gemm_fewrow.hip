@@ -213,6 +213,10 @@ struct Q4KBatch {
     const uint8_t *w2, *extra_w2;
 };
 
+// Tiled order (see gemm_q4k_tiled_kernel): one wave's 16 rows of a stage, and a whole 256-row stage, in bytes.
+constexpr int kTiledTileBytes = 16 * DFL_Q4_K_BYTES;    // 2304
+constexpr int kTiledStageBytes = 16 * kTiledTileBytes;  // 36864
+
 // Per-lane constants of the loads and of the activation write, set up once per kernel.
 template <int kWaves>
 struct Q4KLane {
@@ -225,7 +229,7 @@ struct Q4KLane {
 // Rows past n_out (ragged last group) re-read the last row; their results are never stored.
 template <int kWaves>
 __device__ __forceinline__ void q4k_lane_w_offsets(Q4KLane<kWaves> &L, int tid, int row0, int n_out,
-                                                   uint32_t row_bytes) {
+                                                   uint32_t row_bytes, bool tiled = false) {
     using G = Q4KGeom<kWaves>;
     const int lane = tid & 63, wave = tid >> 6;
     const int last = n_out - 1 - row0;
@@ -233,7 +237,8 @@ __device__ __forceinline__ void q4k_lane_w_offsets(Q4KLane<kWaves> &L, int tid, 
     for (int j = 0; j <= G::kFull; j++) {
         const int p = min((j * kWaves + wave) * 64 + lane, G::kWPieces - 1);
         const int r = min(p / 9, last);
-        L.w_off[j] = static_cast<uint32_t>(r) * row_bytes + static_cast<uint32_t>(p % 9) * 16u;
+        // tiled order: a stage is its LDS image, 256 rows x 144 bytes in one piece (padding rows exist)
+        L.w_off[j] = tiled ? static_cast<uint32_t>(p) * 16u : static_cast<uint32_t>(r) * row_bytes + static_cast<uint32_t>(p % 9) * 16u;
     }
 }
 
@@ -492,7 +497,14 @@ __device__ unsigned long long *g_trace = nullptr;  // [n_wg][16]
     } while (0)
 __device__ unsigned long long *g_trace2 = nullptr;  // [n_wg][16 waves][4]: cycles in load wait / barrier / compute, stages
 #define DFL_CYC() __builtin_readcyclecounter()
+#define DFL_TRW(i)                                                                                          \
+    do {                                                                                                    \
+        if ((threadIdx.x & 63) == 0 && g_trace2) g_trace2[(blockIdx.x * 16 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); \
+    } while (0)
 #else
+#define DFL_TRW(i) \
+    do {           \
+    } while (0)
 #define DFL_TR(i) \
     do {          \
     } while (0)
@@ -501,7 +513,7 @@ __device__ unsigned long long *g_trace2 = nullptr;  // [n_wg][16 waves][4]: cycl
 template <int kWaves, typename XT>
 __global__ void __launch_bounds__(64 * kWaves)
     gemm_q4k_stream_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
-                           float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt) {
+                           float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt, int tiled) {
     using G = Q4KGeom<kWaves>;
     extern __shared__ half8_t lds[];  // kLdsPieces
 
@@ -553,24 +565,26 @@ __global__ void __launch_bounds__(64 * kWaves)
     };
     DFL_TR(10);
     Q4KLane<kWaves> L;
-    q4k_lane_w_offsets<kWaves>(L, tid, group_local(rg.first_group) * G::kRows, n_out, row_bytes);
+    q4k_lane_w_offsets<kWaves>(L, tid, group_local(rg.first_group) * G::kRows, n_out, row_bytes, tiled);
     DFL_TR(11);
 
     // Cursors.  Weights: wstage = first byte of the next stage to load in its group's first row,
     // bw its super-block, gw its group, w_left the stages not loaded yet.  Activations run one
     // stage further ahead: xblock / bx / x_left.
-    const uint8_t *wstage = group_w(rg.first_group) + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
+    // (tiled order, single matrix with 16 waves only: stage it of the iteration space is the it-th 36 864-byte piece)
+    const uint8_t *wstage = tiled ? w + static_cast<size_t>(rg.it_begin) * kTiledStageBytes
+                                  : group_w(rg.first_group) + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
     int bw = b0, gw = rg.first_group, w_left = rg.it_end - rg.it_begin;
     const uint8_t *xblock = group_x(rg.first_group) + static_cast<size_t>(b0) * kXBlockBytes;
     int bx = b0, gx = rg.first_group, x_left = w_left;
     const bool ragged = bt.groups_per_mat * G::kRows > n_out;  // a matrix's last group has fewer rows
     auto advance_w = [&]() {
-        wstage += DFL_Q4_K_BYTES;
+        wstage += tiled ? kTiledStageBytes : DFL_Q4_K_BYTES;
         w_left--;
         if (++bw == nb) {
             bw = 0;
             gw++;
-            if (w_left > 0) {
+            if (w_left > 0 && !tiled) {
                 wstage = group_w(gw);
                 if (ragged) q4k_lane_w_offsets<kWaves>(L, tid, group_local(gw) * G::kRows, n_out, row_bytes);
             }
@@ -819,6 +833,7 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * (rg.wg + 1), bt.by_wg));
     const int len = rg.it_end - rg.it_begin;  // <= kSlabStages (host)
     if (len <= 0) return;
+    DFL_TR(0);
     rg.first_group = static_cast<int>(q4k_div(rg.it_begin, bt.by_nb));
     const int b0 = rg.it_begin - rg.first_group * nb;
     const uint32_t row_bytes = static_cast<uint32_t>(nb) * DFL_Q4_K_BYTES;
@@ -876,6 +891,8 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     issue_w();
     if (len > 1) issue_w();
     q4k_slab_wait_groups(w_issued);  // the activations (older than every weight load) are in registers
+    DFL_TR(1);
+    DFL_TRW(0);
 #pragma unroll
     for (int t = 0; t < kSlabStages; t++) {
         if (t < len) {
@@ -901,7 +918,10 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
         }
     }
     __builtin_amdgcn_s_waitcnt(kWaitLds);
+    DFL_TRW(1);
     __builtin_amdgcn_s_barrier();  // the slab is complete; from here on the waves run independently
+    DFL_TR(2);
+    DFL_TRW(2);
 
     const int n = lane & 15, g = lane >> 4;
     const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
@@ -910,7 +930,12 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     int gc = rg.first_group, bc = b0;
     for (int t = 0; t < len; t++) {
         q4k_slab_wait_groups(w_issued - 1 - t);  // loads land in order: stage t has when only later ones are in flight
+        if (t == 0) DFL_TRW(4);
+        if (t == 1) DFL_TRW(5);
+        if (t == 2) DFL_TRW(6);
+        if (t == 3) DFL_TRW(7);
         if (w_issued < len) issue_w();           // stage t+2 into the buffer stage t-1 has been read out of
+        DFL_TR(3 + t);
         const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(my_ring + (t % kSlabRing) * kSlabWavePieces) + n * 9;
         const uint8_t *stage = slab + t * kSlabStageBytes;
         q4k_slab_compute(blk, reinterpret_cast<const half8_t *>(stage) + lane,
@@ -921,6 +946,254 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
             gc++;
         }
     }
+    DFL_TR(9);
+    DFL_TRW(3);
+}
+
+// ----------------------------------------------------------------------------
+// Q4_K in tiled order: the slab kernel on weights repacked once, at load time
+// ----------------------------------------------------------------------------
+//
+// In ggml order a matrix is [row][super-block] of 144-byte blocks, so the 16 rows x 1 super-block a wave needs per
+// stage are sixteen 144-byte runs a row stride apart.  Measured on MI355X (50 MB matrix, counters of the slab kernel
+// against a plain copy of the same bytes): L2 misses 496 k lines instead of 392 k (blocks straddle 128-byte lines and
+// the two halves of a line are asked for at different times), 1.8x the L2 requests, and HBM delivering 5 TB/s of
+// traffic where the copy gets 7.3 TB/s: the kernel's time is its memory traffic, not its arithmetic.
+// The tiled order removes all three: the matrix is cut into tile groups of 256 rows (the last one padded with zero
+// blocks) and stored as
+//     [tile group][super-block][tile 0..15][row 0..15][144-byte block],
+// i.e. stage (group, super-block) of the streaming kernels is one contiguous 36 864-byte piece, a wave's share of it
+// (one tile) one contiguous, 128-byte aligned 2304-byte piece, and a workgroup's range of stages one contiguous run.
+// Blocks are unchanged (same 144 bytes, same values): dflash_repack_q4k_tiled is a permutation of whole blocks.
+
+__global__ void __launch_bounds__(256)
+    q4k_repack_tiled_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int n_out, int nb, int64_t n_pieces) {
+    const int64_t p = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;  // 16-byte piece of the tiled matrix
+    if (p >= n_pieces) return;
+    const int piece = static_cast<int>(p % 9);
+    const int64_t blk = p / 9;                       // block index in tiled order
+    const int row_in_group = static_cast<int>(blk % 256);
+    const int64_t stage = blk / 256;                 // group * nb + sb
+    const int sb = static_cast<int>(stage % nb);
+    const int64_t row = (stage / nb) * 256 + row_in_group;
+    u32x4_t v = {0, 0, 0, 0};
+    if (row < n_out) v = *reinterpret_cast<const u32x4_t *>(src + (row * nb + sb) * DFL_Q4_K_BYTES + piece * 16);
+    *reinterpret_cast<u32x4_t *>(dst + p * 16) = v;
+}
+
+__device__ __forceinline__ void q4k_load_x8(const uint8_t *base, uint32_t off, float4_t &a, float4_t &b) {
+    asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:16" : "=&v"(a), "=&v"(b) : "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void q4k_load_x8(const uint8_t *base, uint32_t off, half8_t &a, half8_t &) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(a) : "v"(off), "s"(base) : "memory");
+}
+template <typename XT>
+struct Q4KX8;
+template <>
+struct Q4KX8<float> {
+    typedef float4_t type;
+    static constexpr int kLoads = 2;
+};
+template <>
+struct Q4KX8<_Float16> {
+    typedef half8_t type;
+    static constexpr int kLoads = 1;
+};
+__device__ __forceinline__ void q4k_x8_to_half(const float4_t &a, const float4_t &b, _Float16 *h) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        h[i] = static_cast<_Float16>(a[i]);
+        h[4 + i] = static_cast<_Float16>(b[i]);
+    }
+}
+__device__ __forceinline__ void q4k_x8_to_half(const half8_t &a, const half8_t &, _Float16 *h) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) h[i] = a[i];
+}
+
+// sum over the four lanes of a quad (every lane gets it), without a trip through LDS
+__device__ __forceinline__ float q4k_quad_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+    return v;
+}
+
+// A stage's activation fragments in the tiled kernel: the eight 1 KB fragment sets (one per MFMA) sit 1040 bytes
+// apart, so that the eight lanes that convert one row's 64 values (same slot in eight different sets) write to
+// different banks; then the sub-block sums.
+constexpr int kTiledFragStride = 1024 + 16;
+constexpr int kTiledStageX = 8 * kTiledFragStride + 64 * 8;
+constexpr size_t kTiledLdsBytes = static_cast<size_t>(kSlabStages) * kTiledStageX +
+                                  static_cast<size_t>(kSlabWaves) * kSlabRing * kSlabWavePieces * 16;
+static_assert(kTiledLdsBytes <= 160 * 1024, "one workgroup per CU, all of its LDS");
+
+// q4k_slab_compute with the fragment sets kTiledFragStride apart
+__device__ __forceinline__ void q4k_tiled_compute(const u32x4_t *blk, const uint8_t *stage, int lane, int g, uint32_t sc_sel,
+                                                  Q4KMagic magic, float4_t &acc, float4_t &acc_min) {
+    const u32x4_t hdr = blk[0], q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
+    half8_t af[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) af[t] = *reinterpret_cast<const half8_t *>(stage + t * kTiledFragStride + lane * 16);
+    const half4_t tw = *reinterpret_cast<const half4_t *>(stage + 8 * kTiledFragStride + lane * 8);
+    const uint32_t upper = 0u - static_cast<uint32_t>(g >> 1);
+    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu, mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t sc_word = (sc_hi & upper) | (sc_lo & ~upper), mn_word = (mn_hi & upper) | (mn_lo & ~upper);
+    const half2_t dm = __builtin_bit_cast(half2_t, hdr.x);
+    const half2_t p_sc = as_half2(__builtin_amdgcn_perm(0x64646464u, sc_word, sc_sel));
+    const half2_t p_mn = as_half2(__builtin_amdgcn_perm(0x64646464u, mn_word, sc_sel));
+    const half2_t neg = dm * splat(static_cast<_Float16>(-1024.0f));
+    const half2_t S = __builtin_elementwise_fma(p_sc, splat(dm[0]), splat(neg[0]));
+    const half2_t M = __builtin_elementwise_fma(p_mn, splat(dm[1]), splat(neg[1]));
+    const half2_t unbias = {static_cast<_Float16>(-1024.0f), static_cast<_Float16>(-64.0f)};
+    const half2_t Cs = S * unbias;
+    const half2_t s2l = splat(S[0]), c2l = splat(Cs[0]);
+    const half2_t s2h = splat(S[1]), c2h = splat(Cs[1]);
+    const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const _Float16 zero = static_cast<_Float16>(0.0f);
+    const half8_t a_min = {tw[0], tw[1], tw[2], tw[3], zero, zero, zero, zero};
+    const half8_t b_min = {M[0], M[1], M[0], M[1], zero, zero, zero, zero};
+    acc_min = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_min, b_min, acc_min, 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bh, acc, 0, 0, 0);
+    }
+}
+
+// The tiled kernel.  Same work split, flush and reduction as the slab kernel.  Order of the prologue: the
+// activation loads alone, then (once they are back and converted) the first three weight stages into the wave's
+// ring; see the measurements at the issue points.
+template <typename XT>
+__global__ void __launch_bounds__(64 * kSlabWaves)
+    gemm_q4k_tiled_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
+                          float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt) {
+    constexpr int kW = kSlabWaves;
+    constexpr int kPre = 2;  // weight stages issued ahead of the wait for the activations
+    extern __shared__ half8_t lds[];
+    uint8_t *slab = reinterpret_cast<uint8_t *>(lds);                                // [kSlabStages][kTiledStageX]
+    half8_t *ring = reinterpret_cast<half8_t *>(slab + kSlabStages * kTiledStageX);  // [wave][kSlabRing][144]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    Q4KRange rg;
+    rg.nb = nb;
+    rg.n_wg = gridDim.x;
+    rg.total = n_groups * nb;
+    rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
+    rg.it_begin = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * rg.wg, bt.by_wg));
+    rg.it_end = static_cast<int>(q4k_div(static_cast<uint32_t>(rg.total) * (rg.wg + 1), bt.by_wg));
+    const int len = rg.it_end - rg.it_begin;  // <= kSlabStages (host)
+    if (len <= 0) return;
+    DFL_TR(0);
+    rg.first_group = static_cast<int>(q4k_div(rg.it_begin, bt.by_nb));
+    const int b0 = rg.it_begin - rg.first_group * nb;
+    const uint32_t n_in = static_cast<uint32_t>(nb) * DFL_QK_K;
+
+    // ---- activations of every stage of the range ----
+    // item (stage s, row m, eight values k = 8c .. 8c+7): virtual wave v = wave + 16 r covers stage v / 8, rows
+    // 8 ((v >> 2) & 1) + (lane >> 3), chunks 8 (v & 3) + (lane & 7): eight lanes read one row's 128 (f16) or 256 (f32)
+    // contiguous bytes, and the four lanes of a quad hold one sub-block of one row
+    constexpr int kItems = (kSlabStages * 8 + kW - 1) / kW;  // 3
+    typename Q4KX8<XT>::type raw_a[kItems], raw_b[kItems];
+    const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(x);
+#pragma unroll
+    for (int r = 0; r < kItems; r++) {
+        const int v = wave + kW * r, s = v >> 3;
+        if (s < len) {
+            const int m = 8 * ((v >> 2) & 1) + (lane >> 3), c = 8 * (v & 3) + (lane & 7);
+            int b = b0 + s;
+            while (b >= nb) b -= nb;
+            const uint32_t off = (static_cast<uint32_t>(min(m, n_rows - 1)) * n_in + 8u * c) * static_cast<uint32_t>(sizeof(XT));
+            q4k_load_x8(xbytes + static_cast<size_t>(b) * (DFL_QK_K * sizeof(XT)), off, raw_a[r], raw_b[r]);
+        }
+    }
+
+    // ---- this wave's weight tiles: 144 contiguous 16-byte pieces per stage, piece 64 j + lane in load j ----
+    half8_t *my_ring = ring + wave * (kSlabRing * kSlabWavePieces);
+    const uint8_t *wlane = w + static_cast<size_t>(rg.it_begin) * kTiledStageBytes + static_cast<size_t>(wave) * kTiledTileBytes +
+                           static_cast<size_t>(lane) * 16;
+    int w_issued = 0;
+    auto issue_w = [&]() {  // the next stage's 144 pieces into ring buffer (w_issued % 3)
+        half8_t *buf = my_ring + (w_issued % kSlabRing) * kSlabWavePieces;
+        __builtin_amdgcn_global_load_lds((gptr_t)(wlane), (lptr_t)(buf), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(wlane + 1024), (lptr_t)(buf + 64), 16, 0, 0);
+        if (lane < 16) __builtin_amdgcn_global_load_lds((gptr_t)(wlane + 2048), (lptr_t)(buf + 128), 16, 0, 0);
+        w_issued++;
+        wlane += kTiledStageBytes;
+    };
+    // Two stages go out ahead of the wait for the activations, the third after the slab barrier.  Measured (50 MB
+    // matrix, kernel time): 15.6 / 15.2 / 14.6 / 14.8 us with 0 / 1 / 2 / 3 stages ahead.  A CU's memory pipeline
+    // takes new loads only as fast as data returns (27 KB/us, its share of HBM), so a wave that issues more stalls
+    // at the issue and reaches the barrier late; with none ahead the activations are back after 1.2 us instead of
+    // 3.5, but the weights start 2 us later.
+    for (int t = 0; t < kPre; t++)
+        if (t < len) issue_w();
+    q4k_slab_wait_groups(w_issued);  // the activations (older than every weight load) are in registers
+    DFL_TR(1);
+    DFL_TRW(0);
+#pragma unroll
+    for (int r = 0; r < kItems; r++) {
+        const int v = wave + kW * r, s = v >> 3;
+        if (s < len) {
+            asm volatile("" : "+v"(raw_a[r]));
+            if (Q4KX8<XT>::kLoads == 2) asm volatile("" : "+v"(raw_b[r]));
+            const int m = 8 * ((v >> 2) & 1) + (lane >> 3), c = 8 * (v & 3) + (lane & 7);
+            const int j = c >> 2, quarter = c & 3;  // sub-block, eight-value unit in it
+            uint8_t *stage = slab + s * kTiledStageX;
+            _Float16 h[8];
+            q4k_x8_to_half(raw_a[r], raw_b[r], h);
+            // fragment slot of MFMA t = 4 (j & 1) + quarter, lane (m, g = j >> 1); element order of the unpack
+            const half8_t frag = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+            *reinterpret_cast<half8_t *>(stage + (4 * (j & 1) + quarter) * kTiledFragStride + (16 * (j >> 1) + m) * 16) = frag;
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) sum += static_cast<float>(h[i]);
+            sum = q4k_quad_sum(sum);  // the sub-block's sum of the rounded values
+            if (quarter == 0) {
+                const _Float16 hi = static_cast<_Float16>(sum), lo = static_cast<_Float16>(sum - static_cast<float>(hi));
+                _Float16 *tw = reinterpret_cast<_Float16 *>(stage + 8 * kTiledFragStride) + (m + 16 * (j >> 1)) * 4 + (j & 1);
+                tw[0] = hi;
+                tw[2] = lo;
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitLds);
+    DFL_TRW(1);
+    __builtin_amdgcn_s_barrier();  // the slab is complete; from here on the waves run independently
+    DFL_TR(2);
+    DFL_TRW(2);
+    for (int t = kPre; t < kSlabRing; t++)
+        if (t < len) issue_w();
+
+    const int n = lane & 15, g = lane >> 4;
+    const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
+    const Q4KMagic magic = q4k_magic();
+    float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0}, stash = {0, 0, 0, 0};
+    int gc = rg.first_group, bc = b0;
+    for (int t = 0; t < len; t++) {
+        q4k_slab_wait_groups(w_issued - 1 - t);  // loads land in order: stage t has when only later ones are in flight
+        if (t == 0) DFL_TRW(4);
+        if (t == 1) DFL_TRW(5);
+        if (t == 2) DFL_TRW(6);
+        if (t == 3) DFL_TRW(7);
+        DFL_TR(3 + t);
+        const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(my_ring + (t % kSlabRing) * kSlabWavePieces) + n * 9;
+        q4k_tiled_compute(blk, slab + t * kTiledStageX, lane, g, sc_sel, magic, acc, acc_min);
+        // stage t+3 into the buffer this stage has just been read out of (its reads are complete: the MFMAs above used them)
+        if (w_issued < len) issue_w();
+        if (++bc == nb || t + 1 == len) {
+            q4k_flush<kW>(rg, bt, gc, acc, acc_min, stash, y, partials, n_out, n_rows, tid);
+            bc = 0;
+            gc++;
+        }
+    }
+    DFL_TR(9);
+    DFL_TRW(3);
 }
 
 // ----------------------------------------------------------------------------
@@ -1606,7 +1879,7 @@ namespace {
 // Launches the streaming Q4_K kernel (and its split-K reduction): one matrix (batch == nullptr) or the
 // matrices a device-side list picks out of a stack (at most max_slots of them).
 int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in, int64_t n_out,
-                   int32_t n_rows, hipStream_t st, const Q4KBatch *batch, int max_slots) {
+                   int32_t n_rows, hipStream_t st, const Q4KBatch *batch, int max_slots, bool tiled = false) {
     const int nb = static_cast<int>(n_in / DFL_QK_K);
     const size_t row_bytes = static_cast<size_t>(nb) * DFL_Q4_K_BYTES;
     const int tiles = static_cast<int>((n_out + 15) / 16);
@@ -1621,13 +1894,15 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     // A single matrix whose per-workgroup range is at most kSlabStages stages long takes the slab kernel (16-wave
     // groups): resident activation slab, wave-private weight rings, no per-stage barrier.
     bool slab = false;
-    if (!batch && env_int("DFLASH_Q4K_SLAB", 1) && kSlabLdsBytes <= ctx->lds_bytes) {
+    if (!batch && (tiled || env_int("DFLASH_Q4K_SLAB", 1)) && kSlabLdsBytes <= ctx->lds_bytes) {
         const int64_t total16 = static_cast<int64_t>((tiles + 15) / 16) * nb;
         const int64_t wgs = std::min<int64_t>(std::min<int64_t>(env_int("DFLASH_GEMM_WGS", ctx->n_cu), total16), ctx->n_partial_wgs / 2);
         // the longest range is ceil(total / wgs) stages
         slab = wgs >= 1 && (total16 + wgs - 1) / wgs <= kSlabStages;
         if (slab) waves = 16;
     }
+    if (tiled && batch) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: tiled Q4_K is for single matrices");
+    if (tiled) waves = 16;  // the tiled order is cut in 256-row groups
     const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
     const int groups = gpm * max_slots * ((batch && batch->pair) ? 2 : 1);  // upper bound in batched mode (pair mode: virtual groups)
     int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
@@ -1659,14 +1934,31 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         {                                                                                                              \
             dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                      \
             gemm_q4k_stream_kernel<WAVES, XT><<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, \
-                                                                             no, nb, n_rows, groups, bt);              \
+                                                                             no, nb, n_rows, groups, bt, tiled ? 1 : 0); \
         }                                                                                                              \
         if (split) {                                                                                                   \
             dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                    \
             q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);   \
         }                                                                                                              \
     } while (0)
-    if (slab) {
+    if (slab && tiled) {
+        const void *fn = x_type == DFLASH_TYPE_F32 ? reinterpret_cast<const void *>(gemm_q4k_tiled_kernel<float>)
+                                                   : reinterpret_cast<const void *>(gemm_q4k_tiled_kernel<_Float16>);
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, fn, kTiledLdsBytes)) return rc_;
+        {
+            dfl_timed timer(ctx, st, DFL_T_GEMM);
+            if (x_type == DFLASH_TYPE_F32)
+                gemm_q4k_tiled_kernel<float><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const float *>(x), y, partials, no,
+                                                                                           nb, n_rows, groups, bt);
+            else
+                gemm_q4k_tiled_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
+                                                                                              partials, no, nb, n_rows, groups, bt);
+        }
+        if (split) {
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);
+            q4k_reduce_kernel<16><<<groups * 16, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);
+        }
+    } else if (slab) {
         const void *fn = x_type == DFLASH_TYPE_F32 ? reinterpret_cast<const void *>(gemm_q4k_slab_kernel<float>)
                                                    : reinterpret_cast<const void *>(gemm_q4k_slab_kernel<_Float16>);
         if (const int32_t rc_ = dfl_raise_lds_limit(ctx, fn, kSlabLdsBytes)) return rc_;
@@ -1790,6 +2082,33 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
                          int64_t n_out, int32_t n_rows, dflash_stream_t stream);
 }
 
+extern "C" size_t dflash_q4k_tiled_bytes(int64_t n_in, int64_t n_out) {
+    if (n_in <= 0 || n_out <= 0 || n_in % DFL_QK_K) return 0;
+    const size_t groups = (static_cast<size_t>(n_out) + 255) / 256;
+    return groups * static_cast<size_t>(n_in / DFL_QK_K) * kTiledStageBytes;
+}
+
+extern "C" int32_t dflash_repack_q4k_tiled(dflash_ctx *ctx, const void *w, void *w_tiled, int64_t n_in, int64_t n_out,
+                                           dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!w || !w_tiled) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "repack_q4k_tiled: null pointer");
+    if (n_in <= 0 || n_out <= 0 || n_in % DFL_QK_K || n_in > 0x7fffffffll || n_out > 0x7fffffffll)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "repack_q4k_tiled: n_in %lld / n_out %lld", static_cast<long long>(n_in),
+                        static_cast<long long>(n_out));
+    if (reinterpret_cast<uintptr_t>(w) % 16 || reinterpret_cast<uintptr_t>(w_tiled) % 128)
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "repack_q4k_tiled: source must be 16-byte, destination 128-byte aligned");
+    const size_t out_bytes = dflash_q4k_tiled_bytes(n_in, n_out);
+    const size_t in_bytes = static_cast<size_t>(n_out) * (n_in / DFL_QK_K) * DFL_Q4_K_BYTES;
+    if (dfl_ranges_overlap(w_tiled, out_bytes, w, in_bytes)) return dfl_fail(ctx, DFLASH_ERR_ALIAS, "repack_q4k_tiled: buffers overlap");
+    const int64_t n_pieces = static_cast<int64_t>(out_bytes / 16);
+    const int64_t blocks = (n_pieces + 255) / 256;
+    if (blocks > 0x7fffffffll) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "repack_q4k_tiled: matrix too large");
+    q4k_repack_tiled_kernel<<<static_cast<unsigned>(blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint8_t *>(w), static_cast<uint8_t *>(w_tiled), static_cast<int>(n_out), static_cast<int>(n_in / DFL_QK_K), n_pieces);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
 extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type,
                                       float *y, int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
@@ -1809,6 +2128,8 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
     if (x_type != DFLASH_TYPE_F32 && x_type != DFLASH_TYPE_F16)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: activations must be f32 or f16");
     const bool plain = w_type == DFLASH_TYPE_F32 || w_type == DFLASH_TYPE_F16;
+    const bool tiled = w_type == DFLASH_TYPE_Q4_K_TILED;
+    if (tiled) w_type = DFLASH_TYPE_Q4_K;
     if (w_type != DFLASH_TYPE_Q4_K && w_type != DFLASH_TYPE_Q6_K && w_type != DFLASH_TYPE_Q8_0 && !plain)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: weight type %d has no few-row kernel", w_type);
     const int64_t blk = (w_type == DFLASH_TYPE_Q8_0 || plain) ? DFL_QK8_0 : DFL_QK_K;
@@ -1816,7 +2137,7 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: n_in %lld is not a multiple of %lld",
                         static_cast<long long>(n_in), static_cast<long long>(blk));
     const size_t row_bytes = dflash_row_bytes(w_type, static_cast<size_t>(n_in));
-    const size_t w_bytes = row_bytes * static_cast<size_t>(n_out);
+    const size_t w_bytes = tiled ? dflash_q4k_tiled_bytes(n_in, n_out) : row_bytes * static_cast<size_t>(n_out);
     const size_t x_bytes = static_cast<size_t>(n_rows) * n_in * (x_type == DFLASH_TYPE_F32 ? 4 : 2);
     const size_t y_bytes = static_cast<size_t>(n_rows) * n_out * 4;
     if (reinterpret_cast<uintptr_t>(w) % ((w_type == DFLASH_TYPE_Q4_K || plain) ? 16 : 2) ||
@@ -1831,7 +2152,9 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
     const int target_waves = 8 * ctx->n_cu;
 
     if (w_type == DFLASH_TYPE_Q4_K) {
-        return launch_q4k(ctx, w, x, x_type, y, n_in, n_out, n_rows, st, nullptr, 1);
+        if (tiled && reinterpret_cast<uintptr_t>(w) % 128)
+            return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: tiled Q4_K weights must be 128-byte aligned");
+        return launch_q4k(ctx, w, x, x_type, y, n_in, n_out, n_rows, st, nullptr, 1, tiled);
     } else if (w_type == DFLASH_TYPE_Q6_K && env_int("DFLASH_Q6K_STREAM", 1)) {
         const int32_t rc = launch_q6k_stream(ctx, w, x, x_type, y, n_in, n_out, n_rows, st);
         if (rc) return rc;

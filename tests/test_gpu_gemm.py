@@ -192,3 +192,58 @@ def test_gemm_guards(ctx):
     with pytest.raises(dfl.DFlashError) as e:
         ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q4_K, xy, xy, 256, 16, 4)
     assert e.value.kind == "Alias"
+
+
+TILED_SHAPES = [(256, 16, 16), (256, 250, 3), (768, 257, 16), (1024, 4096, 7), (1280, 1000, 16), (2048, 5120, 1),
+                (5120, 6144, 16), (5120, 17408, 16), (17408, 5120, 16),
+                (2048, 50000, 16), (8192, 16384, 5)]  # the last two: ranges longer than six stages (the per-stage-barrier kernel)
+
+
+@pytest.mark.parametrize("n_in,n_out,n_rows", TILED_SHAPES)
+@pytest.mark.parametrize("x_dtype", ["f32", "f16"])
+def test_gemm_q4k_tiled_order_is_bit_identical(ctx, n_in, n_out, n_rows, x_dtype):
+    """The one-time repack into tiled order permutes whole blocks: the GEMM on it must give the very bits the GEMM on
+    GGUF row order gives (ragged n_out, ranges that wrap over tile groups, every row count), and the padding rows of
+    the last tile group must leave the output alone (guard bands around Y)."""
+    import torch
+    rng = np.random.default_rng(n_in + n_out + n_rows)
+    w = dfl.synth.random_blocks(dfl.synth.Q4_K, n_out * n_in // 256, n_in + n_out)
+    x = rng.standard_normal((n_rows, n_in)).astype(np.float32 if x_dtype == "f32" else np.float16)
+    wd, xd = dev(w), dev(x)
+    want = ctx.gemm_fewrow(wd, dfl.TYPE_Q4_K, xd, n_in, n_out)
+    wt = ctx.repack_q4k_tiled(wd, n_in, n_out)
+    guard = 64
+    buf = torch.full((n_rows * n_out + 2 * guard,), float("nan"), dtype=torch.float32, device="cuda")
+    y = buf[guard:guard + n_rows * n_out].view(n_rows, n_out)
+    ctx.encode_mat_mat_dispatch_dflash_verify(wt, dfl.TYPE_Q4_K_TILED, xd, y, n_in, n_out, n_rows)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int32), want.view(torch.int32))
+    assert torch.isnan(buf[:guard]).all() and torch.isnan(buf[-guard:]).all()
+
+
+def test_q4k_tiled_repack_layout(ctx):
+    """Block (row r, super-block b) of the row-order matrix sits at [r // 256][b][r % 256] of the tiled one; rows
+    past n_out are zero blocks."""
+    n_in, n_out = 768, 300
+    nb = n_in // 256
+    w = dfl.synth.random_blocks(dfl.synth.Q4_K, n_out * nb, 5)
+    wt = ctx.repack_q4k_tiled(dev(w), n_in, n_out).cpu().numpy()
+    groups = (n_out + 255) // 256
+    assert wt.size == groups * nb * 256 * 144
+    src = np.zeros((groups * 256, nb, 144), np.uint8)
+    src[:n_out] = np.asarray(w).reshape(n_out, nb, 144)
+    want = src.reshape(groups, 256, nb, 144).transpose(0, 2, 1, 3)
+    assert np.array_equal(wt.reshape(groups, nb, 256, 144), want)
+
+
+def test_q4k_tiled_guards(ctx):
+    import torch
+    n_in, n_out = 512, 64
+    w = dev(dfl.synth.random_blocks(dfl.synth.Q4_K, n_out * n_in // 256, 1))
+    with pytest.raises(dfl.DFlashError):
+        ctx.repack_q4k_tiled(w, 500, n_out)
+    wt = ctx.repack_q4k_tiled(w, n_in, n_out)
+    x = torch.zeros((4, n_in), dtype=torch.float32, device="cuda")
+    y = torch.empty((4, n_out), dtype=torch.float32, device="cuda")
+    with pytest.raises(dfl.DFlashError):  # misaligned tiled weights
+        ctx.encode_mat_mat_dispatch_dflash_verify(wt[16:], dfl.TYPE_Q4_K_TILED, x, y, n_in, n_out, 4)
