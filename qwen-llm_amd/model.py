@@ -14,7 +14,7 @@ from dataclasses import asdict, dataclass
 import numpy as np
 
 from . import synth
-from .binding import CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
+from .binding import TYPE_Q4_K, TYPE_Q4_K_TILED, CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
 
 
 @dataclass
@@ -310,9 +310,11 @@ def synth_draft_weights_device(cfg: DraftConfig, seed: int, device, wtype: int =
 # ---- device-resident weights ----
 
 class _Uploader:
-    def __init__(self, device):
+    def __init__(self, device, ctx=None):
+        """``ctx``: when given, Q4_K matrices uploaded with a tile shape are repacked into the tiled order."""
         self.torch = _torch()
         self.device = device
+        self.ctx = ctx
         self.keep = []
 
     def _from_numpy(self, a):
@@ -332,7 +334,9 @@ class _Uploader:
         self.keep.append(t)
         return t.data_ptr()
 
-    def q(self, pair):
+    def q(self, pair, tile_shape=None):
+        """``tile_shape`` = (n_out, n_in): a Q4_K matrix that only the few-row GEMM reads is repacked into the
+        library's tiled order (a permutation of whole blocks, bit-identical products, faster streaming)."""
         if pair is None:
             return QTensorC(0, 0, None)
         qtype, blocks = pair
@@ -340,15 +344,20 @@ class _Uploader:
             t = blocks.to(self.device).contiguous()
         else:
             t = self._from_numpy(np.ascontiguousarray(blocks)).to(self.device)
+        if tile_shape is not None and self.ctx is not None and int(qtype) == TYPE_Q4_K:
+            t = self.ctx.repack_q4k_tiled(t, tile_shape[1], tile_shape[0])
+            qtype = TYPE_Q4_K_TILED
         self.keep.append(t)
         return QTensorC(int(qtype), 0, t.data_ptr())
 
-    def q_adjacent(self, pairs):
+    def q_adjacent(self, pairs, tile_shapes=None):
         """Uploads matrices of one type and one row length back to back in a single allocation (rows of the
         first, then the second, ...): the library then runs a layer's wq/wk/wv (or gate/up) as ONE GEMM.
-        Falls back to separate uploads when the types differ."""
+        Falls back to separate uploads when the types differ.  ``tile_shapes`` = [(n_out, n_in), ...]: Q4_K sets
+        whose row counts are all multiples of 256 are repacked as one tiled matrix (tile groups are 256 rows, so
+        every member still starts where its row-order address arithmetic says)."""
         if any(p is None for p in pairs) or len({int(p[0]) for p in pairs}) != 1:
-            return [self.q(p) for p in pairs]
+            return [self.q(p, ts) for p, ts in zip(pairs, tile_shapes or [None] * len(pairs))]
         torch = self.torch
         flats = []
         for _, blocks in pairs:
@@ -357,10 +366,15 @@ class _Uploader:
             else:
                 flats.append(self._from_numpy(np.ascontiguousarray(blocks).view(np.uint8).reshape(-1)).to(self.device))
         whole = torch.cat(flats)
+        qtype = int(pairs[0][0])
+        if (tile_shapes is not None and self.ctx is not None and qtype == TYPE_Q4_K
+                and all(ts is not None and ts[0] % 256 == 0 for ts in tile_shapes)):
+            whole = self.ctx.repack_q4k_tiled(whole, tile_shapes[0][1], sum(ts[0] for ts in tile_shapes))
+            qtype = TYPE_Q4_K_TILED
         self.keep.append(whole)
         out, off = [], 0
-        for (qtype, _), f in zip(pairs, flats):
-            out.append(QTensorC(int(qtype), 0, whole.data_ptr() + off))
+        for f in flats:
+            out.append(QTensorC(qtype, 0, whole.data_ptr() + off))
             off += f.numel()
         return out
 
@@ -368,12 +382,20 @@ class _Uploader:
 class TargetModel:
     """Device copy of a weight dictionary plus the ``dflash_model`` descriptor."""
 
-    def __init__(self, ctx: Context, cfg: ModelConfig, weights: dict, adjacent: bool = True):
-        """``adjacent``: place each layer's wq/wk/wv and gate/up back to back in device memory (one GEMM each)."""
+    def __init__(self, ctx: Context, cfg: ModelConfig, weights: dict, adjacent: bool = True, tiled: bool = True):
+        """``adjacent``: place each layer's wq/wk/wv and gate/up back to back in device memory (one GEMM each).
+        ``tiled``: repack the Q4_K matrices that only the few-row GEMM reads (attention projections, a dense layer's
+        FFN, the output head) into the library's tiled order at upload; expert stacks, a mixture layer's shared
+        expert (the batched expert kernel reads it in row order) and the embedding table stay in GGUF row order."""
         self.ctx, self.cfg = ctx, cfg
-        up = _Uploader(f"cuda:{ctx.device}")
+        up = _Uploader(f"cuda:{ctx.device}", ctx if tiled else None)
         self._up = up
         self._layers = (LayerC * cfg.n_layers)()
+        H, qd, kvd = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
+        dense = cfg.n_expert == 0
+        shape = {"wq": (qd, H), "wk": (kvd, H), "wv": (kvd, H), "wo": (H, qd)}
+        if dense:
+            shape.update({"gate": (cfg.ffn, H), "up": (cfg.ffn, H), "down": (H, cfg.ffn)})
         for il, Lw in enumerate(weights["layers"]):
             L = self._layers[il]
             for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
@@ -381,14 +403,14 @@ class TargetModel:
             grouped = ()
             if adjacent:
                 grouped = ("wq", "wk", "wv", "gate", "up")
-                L.wq, L.wk, L.wv = up.q_adjacent([Lw.get("wq"), Lw.get("wk"), Lw.get("wv")])
-                L.gate, L.up = up.q_adjacent([Lw.get("gate"), Lw.get("up")])
+                L.wq, L.wk, L.wv = up.q_adjacent([Lw.get("wq"), Lw.get("wk"), Lw.get("wv")], [shape["wq"], shape["wk"], shape["wv"]])
+                L.gate, L.up = up.q_adjacent([Lw.get("gate"), Lw.get("up")], [shape.get("gate"), shape.get("up")])
             for k in ("wq", "wk", "wv", "wo", "gate", "up", "down", "router", "gate_exps", "up_exps", "down_exps"):
                 if k not in grouped:
-                    setattr(L, k, up.q(Lw.get(k)))
+                    setattr(L, k, up.q(Lw.get(k), shape.get(k)))
             L.shexp_gate = up.f32(Lw["shexp_gate"]) if "shexp_gate" in Lw else None
-        self.c = ModelC(ModelCfgC(**cfg.as_dict()), self._layers, up.q(weights["token_embd"]), up.q(weights["output"]),
-                        up.f32(weights["output_norm"]))
+        self.c = ModelC(ModelCfgC(**cfg.as_dict()), self._layers, up.q(weights["token_embd"]),
+                        up.q(weights["output"], (cfg.vocab, H)), up.f32(weights["output_norm"]))
 
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self._up.keep)
@@ -458,11 +480,15 @@ class Session:
 
 
 class DraftHead:
-    def __init__(self, ctx: Context, cfg: DraftConfig, weights: dict, adjacent: bool = True):
+    def __init__(self, ctx: Context, cfg: DraftConfig, weights: dict, adjacent: bool = True, tiled: bool = True):
+        """``adjacent`` / ``tiled``: as for TargetModel."""
         self.ctx, self.cfg = ctx, cfg
-        up = _Uploader(f"cuda:{ctx.device}")
+        up = _Uploader(f"cuda:{ctx.device}", ctx if tiled else None)
         self._up = up
         self._layers = (DraftLayerC * cfg.n_layers)()
+        H, qd, kvd = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
+        shape = {"wq": (qd, H), "wk": (kvd, H), "wv": (kvd, H), "wo": (H, qd), "gate": (cfg.ffn, H), "up": (cfg.ffn, H),
+                 "down": (H, cfg.ffn)}
         for il, Lw in enumerate(weights["layers"]):
             L = self._layers[il]
             for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
@@ -470,16 +496,16 @@ class DraftHead:
             grouped = ()
             if adjacent:
                 grouped = ("wq", "wk", "wv", "gate", "up")
-                L.wq, L.wk, L.wv = up.q_adjacent([Lw["wq"], Lw["wk"], Lw["wv"]])
-                L.gate, L.up = up.q_adjacent([Lw["gate"], Lw["up"]])
+                L.wq, L.wk, L.wv = up.q_adjacent([Lw["wq"], Lw["wk"], Lw["wv"]], [shape["wq"], shape["wk"], shape["wv"]])
+                L.gate, L.up = up.q_adjacent([Lw["gate"], Lw["up"]], [shape["gate"], shape["up"]])
             for k in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
                 if k not in grouped:
-                    setattr(L, k, up.q(Lw[k]))
+                    setattr(L, k, up.q(Lw[k], shape[k]))
             L.is_swa = int(Lw.get("is_swa", 0))
             if cfg.conv_kernel_size:
                 L.conv_attn_proj, L.conv_ffn_proj = up.q(Lw["conv_attn_proj"]), up.q(Lw["conv_ffn_proj"])
                 L.conv_attn_base, L.conv_ffn_base = up.f32(Lw["conv_attn_base"]), up.f32(Lw["conv_ffn_base"])
-        self.c = DraftHeadC(DraftCfgC(**cfg.as_dict()), self._layers, up.q(weights["fc"]), up.f32(weights["hidden_norm"]),
+        self.c = DraftHeadC(DraftCfgC(**cfg.as_dict()), self._layers, up.q(weights["fc"], (H, cfg.n_taps * H)), up.f32(weights["hidden_norm"]),
                             up.f32(weights["output_norm"]))
         if cfg.selector_rank:
             self.c.selector_hidden = up.q(weights["selector_hidden"])
