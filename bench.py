@@ -18,9 +18,20 @@ METRIC = "accepted tokens/s @ batch1 block16; verify Q4_K GEMM HBM GB/s (% of pe
 SHAPES = [(5120, 17408), (17408, 5120), (5120, 6144)]  # (n_in, n_out)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, averaged over the three shapes of a step: FETCH_SIZE + WRITE_SIZE from
-# two rocprofv3 --pmc runs of this file, each scaled by what the same counter reads for a plain 256 MiB copy
-# (profiles/gemm_q4k_stream_kernel__hbm_traffic.txt).  A counter figure, not measured by this run.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 51.02e6
+# two rocprofv3 --pmc runs of this file, each scaled by what the same counter reads for a plain 256 MiB copy.  A
+# counter figure, not measured by this run: read from the line "traffic_bytes_per_launch: N" of the summary below.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_q4k_tiled_kernel__hbm_traffic.txt")
+
+
+def measured_traffic():
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1])
+    except OSError:
+        pass
+    return None
 
 
 def cpu_baseline(shapes, weights, xs):
@@ -332,24 +343,44 @@ def main():
     ctx = dfl.Context(0)
     rng = np.random.default_rng(1)
     weights, xs, wd, xd, yd = [], [], [], [], []
+    # The weights are uploaded the way a model's are: Q4_K blocks repacked once into the library's tiled order
+    # (a permutation of whole 144-byte blocks; same bytes streamed, bit-identical products).  One copy of each matrix
+    # stays in GGUF row order so that the same kernel family can be timed on it beside the headline.
+    wrow = []
     for n_in, n_out in SHAPES:
         w = dfl.synth.random_weight(dfl.synth.Q4_K, n_out, n_in, seed=1)
         x = rng.standard_normal((16, n_in)).astype(np.float16)
         weights.append(w)
         xs.append(x)
         w0 = torch.from_numpy(w).cuda()
-        wd.append([w0] + [w0.clone() for _ in range(max(1, args.weight_sets) - 1)])
+        wrow.append(w0)
+        t0 = ctx.repack_q4k_tiled(w0, n_in, n_out)
+        wd.append([t0] + [t0.clone() for _ in range(max(1, args.weight_sets) - 1)])
         xd.append(torch.from_numpy(x).cuda())
         yd.append(torch.empty((16, n_out), dtype=torch.float32, device="cuda"))
     w_bytes = [int(w.size) for w in weights]
+    w_type = dfl.TYPE_Q4_K_TILED
 
     n_sets = len(wd[0])
     turn = [0]
 
+    # the launches go straight through the C ABI with arguments marshalled once: a call then costs the host about a
+    # microsecond, well under the kernels' time, so the GPU never waits for Python
+    from qwen_llm_amd.binding import _stream_ptr
+    gemm_c = ctx._lib.dflash_gemm_fewrow
+
+    def bound_call(w, wt, i):
+        n_in, n_out = SHAPES[i]
+        a = (ctx._h, wt, w.data_ptr(), xd[i].data_ptr(), dfl.TYPE_F16, yd[i].data_ptr(), n_in, n_out, 16, _stream_ptr())
+        return a
+
+    step_args = [[bound_call(wd[i][k], w_type, i) for i in range(len(SHAPES))] for k in range(n_sets)]
+
     def step():
         k = turn[0] = (turn[0] + 1) % n_sets
-        for (n_in, n_out), w, x, y in zip(SHAPES, wd, xd, yd):
-            ctx.encode_mat_mat_dispatch_dflash_verify(w[k], dfl.TYPE_Q4_K, x, y, n_in, n_out, 16)
+        for a in step_args[k]:
+            if gemm_c(*a):
+                raise RuntimeError(ctx._lib.dflash_last_error(ctx._h).decode())
 
     if args.calibrate_copy:
         # a plain streaming kernel of known traffic: reads 256 MiB, writes 256 MiB (an int32 add, so that its name
@@ -373,25 +404,59 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = e0.elapsed_time(e1) / args.steps
 
-    # dominant kernel alone: events inside the library around gemm_q4k_stream_kernel, on its stream; whole steps
+    # dominant kernel alone: events inside the library around the GEMM kernel, on its stream; whole steps
     # (all three shapes, rotating weight sets) so that no launch finds its weights in a cache
     reps = max(20, args.steps // 4)
-    acc_ms, acc_n = [0.0] * len(SHAPES), [0] * len(SHAPES)
-    for _ in range(reps):
-        k = turn[0] = (turn[0] + 1) % n_sets
-        for i, ((n_in, n_out), w, x, y) in enumerate(zip(SHAPES, wd, xd, yd)):
-            ctx.set_kernel_timing(True)  # restarts the accumulators
-            ctx.encode_mat_mat_dispatch_dflash_verify(w[k], dfl.TYPE_Q4_K, x, y, n_in, n_out, 16)
-            ms, n = ctx.kernel_timing(ctx.T_GEMM)
-            acc_ms[i] += ms
-            acc_n[i] += n
-    ctx.set_kernel_timing(False)
-    per_shape = [{"n_in": n_in, "n_out": n_out, "weight_bytes": nbytes, "kernel_us": ms / n * 1e3,
-                  "GBps": nbytes / (ms / n * 1e-3) / 1e9}
-                 for (n_in, n_out), nbytes, ms, n in zip(SHAPES, w_bytes, acc_ms, acc_n)]
+
+    def kernel_times(sets, wt):
+        """Average launch duration of the streaming kernel alone: back-to-back launches between two events on the
+        stream they run on, the split-K reduction launch switched off meanwhile (an event pair around every single
+        launch would add the dispatch latency, about 2.5 us, to each)."""
+        ctx.set_stream_kernel_only(True)
+        out = []
+        try:
+            for i, w in enumerate(sets):
+                calls = [bound_call(wk, wt, i) for wk in w]
+                for a in calls:
+                    gemm_c(*a)
+                torch.cuda.synchronize()
+                k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                n = reps * len(w)
+                k0.record()
+                for k in range(n):
+                    gemm_c(*calls[k % len(calls)])
+                k1.record()
+                torch.cuda.synchronize()
+                out.append(k0.elapsed_time(k1) / n * 1e3)
+        finally:
+            ctx.set_stream_kernel_only(False)
+        return out
+
+    tiled_us = kernel_times(wd, w_type)
+    # the same launches on GGUF row order, rotating over as many copies
+    row_sets = [[w] + [w.clone() for _ in range(n_sets - 1)] for w in wrow]
+    row_us = kernel_times(row_sets, dfl.TYPE_Q4_K)
+    del row_sets
+    # a read-only stream over the same buffers with the same launch shape: the practical ceiling of such a kernel
+    probe_out = torch.zeros(1024, dtype=torch.int32, device="cuda")
+    probe_us = []
+    for i in range(len(SHAPES)):
+        ctx.hbm_read_probe(wd[i], n_sets, probe_out)
+        torch.cuda.synchronize()
+        p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n_probe = 8 * n_sets
+        p0.record()
+        ctx.hbm_read_probe(wd[i], n_probe, probe_out)
+        p1.record()
+        torch.cuda.synchronize()
+        probe_us.append(p0.elapsed_time(p1) / n_probe * 1e3)
+    per_shape = [{"n_in": n_in, "n_out": n_out, "weight_bytes": nbytes, "kernel_us": us, "GBps": nbytes / (us * 1e-6) / 1e9,
+                  "row_order_kernel_us": rus, "read_probe_us": pus}
+                 for (n_in, n_out), nbytes, us, rus, pus in zip(SHAPES, w_bytes, tiled_us, row_us, probe_us)]
     k_bytes = sum(p["weight_bytes"] for p in per_shape) / len(per_shape)
     k_us = sum(p["kernel_us"] for p in per_shape) / len(per_shape)
     achieved = k_bytes / (k_us * 1e-6) / 1e9
+    ceiling = sum(w_bytes) / (sum(probe_us) * 1e-6) / 1e9
 
     out = {
         "metric": METRIC,
@@ -407,12 +472,14 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "few-row Q4_K dequant GEMM, M=16, (K,N) in {(5120,17408),(17408,5120),(5120,6144)}, "
-                               "X f16 N(0,1), W Q4_K from N(0,0.02) seed 1, f32 accumulation",
+                               "X f16 N(0,1), W Q4_K from N(0,0.02) seed 1 (blocks in the library's tiled order, "
+                               "repacked once at upload), f32 accumulation",
                    "weight_bytes_per_step": sum(w_bytes), "block": 16, "batch": 1, "weight_sets": n_sets,
                    "weight_footprint_bytes": n_sets * sum(w_bytes)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "gemm_q4k_stream_kernel", "bytes_per_launch": k_bytes, "us_per_launch": k_us},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(),
+                     "kernel": "gemm_q4k_tiled_kernel", "bytes_per_launch": k_bytes, "us_per_launch": k_us,
+                     "read_probe_GBps": ceiling, "frac_of_read_probe": achieved / ceiling},
         "shapes": per_shape,
         "pct_of_hbm_peak": 100.0 * sum(w_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "accepted_tokens_per_s": None,
@@ -420,7 +487,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(SHAPES, weights, xs)
-    del wd, xd, yd
+    del wd, xd, yd, wrow
     if not args.gemm_only:
         try:
             out["gemm_q6k"] = q6k_section(ctx)

@@ -79,6 +79,11 @@ const char *dflash_version(void);
 void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable);
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms_host,
                                  int64_t *launches_host);
+/* Measurement aid (no counterpart in the reference): while on, a split-K Q4_K GEMM call launches its streaming
+ * kernel only and leaves Y without the reduction, so that back-to-back launches of that one kernel can be timed
+ * between two events of the caller's (an event pair around a single launch adds the dispatch latency, about 2.5 us,
+ * to a 15 us kernel).  Results are wrong while it is on. */
+void dflash_ctx_set_stream_kernel_only(dflash_ctx *ctx, int32_t enable);
 
 /* Graph replay of the packed verify (the counterpart of the reference's one command buffer per
  * verify block, encode_packed_verify_layer_major, metal_dflash.rs:10696-10719): a verify shape
@@ -96,6 +101,14 @@ void dflash_ctx_set_graphs(dflash_ctx *ctx, int32_t enable);
 int32_t dflash_dequant(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_elems, float *out_f32,
                        dflash_stream_t stream);
 size_t dflash_row_bytes(int32_t type, size_t n_in);
+
+/* ---- measurement aid: streaming-read probe ------------------------------------------
+ * No counterpart in the reference.  n_launches launches of a kernel that reads `bytes` (multiple of 16) of
+ * bufs[k % n_bufs] (16-byte aligned) once with a grid-stride loop of 16-byte loads and stores a word per
+ * workgroup into out_words[n_cu].  bench.py times it over the GEMM's own weight buffers (rotating, so that
+ * nothing is found in a cache) as the practical ceiling of a read-only stream.  Enqueue-only. */
+int32_t dflash_hbm_read_probe(dflash_ctx *ctx, const void *const *bufs, int32_t n_bufs, size_t bytes, int32_t n_launches,
+                              void *out_words, dflash_stream_t stream);
 
 /* ---- Q4_K weights in tiled order -------------------------------------------------
  * No counterpart in the reference (it streams GGUF row order, loader.rs tensors as mapped): a one-time

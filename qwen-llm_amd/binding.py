@@ -104,6 +104,8 @@ def _declare(L):
     L.dflash_select_draft_path_sampled.restype = i32
     L.dflash_select_draft_path_sampled.argtypes = [vp, C.POINTER(CodebookC), C.POINTER(CodebookC), i32, i32, i32, i32, vp, vp,
                                                    vp, C.POINTER(SamplerC), vp, vp, C.POINTER(WeightedCandidateC), vp]
+    L.dflash_ctx_set_stream_kernel_only.restype = None
+    L.dflash_ctx_set_stream_kernel_only.argtypes = [vp, i32]
     L.dflash_ctx_set_graphs.restype = None
     L.dflash_ctx_set_graphs.argtypes = [vp, i32]
     L.dflash_ctx_kernel_timing.restype = i32
@@ -114,6 +116,8 @@ def _declare(L):
     L.dflash_dequant.argtypes = [vp, i32, vp, sz, vp, vp]
     L.dflash_gemm_fewrow.restype = i32
     L.dflash_gemm_fewrow.argtypes = [vp, i32, vp, vp, i32, vp, i64, i64, i32, vp]
+    L.dflash_hbm_read_probe.restype = i32
+    L.dflash_hbm_read_probe.argtypes = [vp, C.POINTER(vp), i32, sz, i32, vp, vp]
     L.dflash_q4k_tiled_bytes.restype = sz
     L.dflash_q4k_tiled_bytes.argtypes = [i64, i64]
     L.dflash_repack_q4k_tiled.restype = i32
@@ -240,6 +244,10 @@ class Context:
     def set_kernel_timing(self, enable: bool):
         self._lib.dflash_ctx_set_kernel_timing(self._h, int(enable))
 
+    def set_stream_kernel_only(self, enable: bool):
+        """Measurement aid: split-K GEMM calls launch their streaming kernel only (Y incomplete while on)."""
+        self._lib.dflash_ctx_set_stream_kernel_only(self._h, int(enable))
+
     def set_graphs(self, enable: bool):
         """Graph replay of the packed verify on or off (off by default; results are the same)."""
         self._lib.dflash_ctx_set_graphs(self._h, int(enable))
@@ -271,6 +279,13 @@ class Context:
         self._check(self._lib.dflash_gemm_fewrow(self._h, w_type, weight.data_ptr(), x.data_ptr(), x_type,
                                                  y.data_ptr(), n_in, n_out, n_query, _stream_ptr()))
         return y
+
+    def hbm_read_probe(self, bufs, n_launches: int, scratch):
+        """``n_launches`` launches of a read-only streaming kernel over the equally sized uint8 tensors ``bufs``
+        (in turn); ``scratch``: int32[n_cu]."""
+        ptrs = (C.c_void_p * len(bufs))(*[b.data_ptr() for b in bufs])
+        nbytes = bufs[0].numel() * bufs[0].element_size()
+        self._check(self._lib.dflash_hbm_read_probe(self._h, ptrs, len(bufs), nbytes, n_launches, scratch.data_ptr(), _stream_ptr()))
 
     def repack_q4k_tiled(self, weight, n_in: int, n_out: int):
         """Q4_K blocks in GGUF row order -> a new tensor in tiled order (w_type TYPE_Q4_K_TILED): a one-time

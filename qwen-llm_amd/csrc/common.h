@@ -22,6 +22,9 @@ struct dflash_ctx {
     char err[512] = {0};
     // per-kernel timers (off by default; when on, timed launches synchronise)
     bool timing = false;
+    // measurement aid: split-K GEMM calls launch their streaming kernel only (Y is left without its reduction), so
+    // that back-to-back launches of that one kernel can be timed between two events
+    bool stream_kernel_only = false;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     double timed_ms[8] = {0};
     int64_t timed_launches[8] = {0};

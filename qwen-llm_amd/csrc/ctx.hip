@@ -105,6 +105,10 @@ void dflash_ctx_set_graphs(dflash_ctx *ctx, int32_t enable) {
     if (ctx) ctx->graphs = enable != 0;
 }
 
+void dflash_ctx_set_stream_kernel_only(dflash_ctx *ctx, int32_t enable) {
+    if (ctx) ctx->stream_kernel_only = enable != 0;
+}
+
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms, int64_t *launches) {
     if (!ctx || slot < 0 || slot >= 8 || !total_ms || !launches) return DFLASH_ERR_INVALID_INPUT;
     *total_ms = ctx->timed_ms[slot];

@@ -96,3 +96,40 @@ extern "C" int32_t dflash_dequant(dflash_ctx *ctx, int32_t type, const void *blo
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }
+
+// ---- streaming-read probe ----------------------------------------------------------------------
+// Reads `bytes` of device memory once (a grid-stride loop of 16-byte loads, 8 workgroups of 256 threads per CU) and
+// stores one word per workgroup: the rate a plain read-only stream reaches on this device, to set beside the rates
+// of the kernels that stream weights.
+namespace {
+constexpr int kProbeThreads = 256;
+__global__ void __launch_bounds__(kProbeThreads) read_probe_kernel(const uint4 *__restrict__ p, size_t n_pieces, uint32_t *__restrict__ out,
+                                                                    int n_out_words) {
+    uint4 a = {0, 0, 0, 0};
+    for (size_t i = blockIdx.x * static_cast<size_t>(kProbeThreads) + threadIdx.x; i < n_pieces; i += static_cast<size_t>(gridDim.x) * kProbeThreads) {
+        const uint4 v = p[i];
+        a.x ^= v.x;
+        a.y ^= v.y;
+        a.z ^= v.z;
+        a.w ^= v.w;
+    }
+    uint32_t acc = a.x ^ a.y ^ a.z ^ a.w;
+    for (int off = 32; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, 64);
+    if (threadIdx.x == 0) out[blockIdx.x % n_out_words] = acc;  // (a plain store: the words are a sink, not a checksum anyone reads)
+}
+}  // namespace
+
+extern "C" int32_t dflash_hbm_read_probe(dflash_ctx *ctx, const void *const *bufs, int32_t n_bufs, size_t bytes, int32_t n_launches,
+                                         void *out_words, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!bufs || n_bufs < 1 || n_launches < 1 || !out_words || bytes % 16)
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "hbm_read_probe: buffers of a multiple of 16 bytes and %d output words", ctx->n_cu);
+    for (int i = 0; i < n_bufs; i++)
+        if (!bufs[i] || reinterpret_cast<uintptr_t>(bufs[i]) % 16)
+            return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "hbm_read_probe: buffer %d is null or not 16-byte aligned", i);
+    for (int k = 0; k < n_launches; k++)
+        read_probe_kernel<<<ctx->n_cu * 8, kProbeThreads, 0, static_cast<hipStream_t>(stream)>>>(
+            static_cast<const uint4 *>(bufs[k % n_bufs]), bytes / 16, static_cast<uint32_t *>(out_words), ctx->n_cu);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}

@@ -1915,7 +1915,8 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: problem too large for 32-bit work indices");
     float *partials = reinterpret_cast<float *>(ctx->partials);
     // a single matrix whose ranges are whole tile groups needs no reduction; a batch always may
-    const bool split = batch ? !batch->whole_groups : groups % n_wg != 0;
+    const bool split = (batch ? !batch->whole_groups : groups % n_wg != 0);
+    const bool reduce = split && !ctx->stream_kernel_only;
     Q4KBatch bt = {};
     if (batch) bt = *batch;
     bt.groups_per_mat = gpm;
@@ -1936,7 +1937,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
             gemm_q4k_stream_kernel<WAVES, XT><<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, \
                                                                              no, nb, n_rows, groups, bt, tiled ? 1 : 0); \
         }                                                                                                              \
-        if (split) {                                                                                                   \
+        if (reduce) {                                                                                                  \
             dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                    \
             q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);   \
         }                                                                                                              \
@@ -1954,7 +1955,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
                 gemm_q4k_tiled_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
                                                                                               partials, no, nb, n_rows, groups, bt);
         }
-        if (split) {
+        if (reduce) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);
             q4k_reduce_kernel<16><<<groups * 16, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);
         }
@@ -1971,7 +1972,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
                 gemm_q4k_slab_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kSlabLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
                                                                                             partials, no, nb, n_rows, groups, bt);
         }
-        if (split) {
+        if (reduce) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);
             q4k_reduce_kernel<16><<<groups * 16, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);
         }
