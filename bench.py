@@ -325,6 +325,8 @@ def main():
                     help="copies of the three weight matrices the timed loops rotate over; 3 x 118 MB exceeds the 256 MB "
                          "memory-side cache, so weights come from HBM as they do in a real model (1 = cache-resident)")
     ap.add_argument("--gemm-only", action="store_true", help="skip the attention, acceptance and end-to-end sections")
+    ap.add_argument("--shapes", default="0,1,2", help="which of the three GEMM shapes take part (for per-shape profiles; the "
+                                                      "metric is defined on all three)")
     args = ap.parse_args()
     if args.rocprof_summary:
         rocprof_summary(args.rocprof_summary)
@@ -339,6 +341,8 @@ def main():
 
     import qwen_llm_amd as dfl
 
+    global SHAPES
+    SHAPES = [SHAPES[int(i)] for i in args.shapes.split(",")]
     torch.cuda.set_device(0)
     ctx = dfl.Context(0)
     rng = np.random.default_rng(1)
@@ -474,6 +478,7 @@ def main():
         "config": {"workload": "few-row Q4_K dequant GEMM, M=16, (K,N) in {(5120,17408),(17408,5120),(5120,6144)}, "
                                "X f16 N(0,1), W Q4_K from N(0,0.02) seed 1 (blocks in the library's tiled order, "
                                "repacked once at upload), f32 accumulation",
+                   "shapes_in_this_run": args.shapes,
                    "weight_bytes_per_step": sum(w_bytes), "block": 16, "batch": 1, "weight_sets": n_sets,
                    "weight_footprint_bytes": n_sets * sum(w_bytes)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
