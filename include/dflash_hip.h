@@ -102,6 +102,20 @@ int32_t dflash_dequant(dflash_ctx *ctx, int32_t type, const void *blocks, size_t
                        dflash_stream_t stream);
 size_t dflash_row_bytes(int32_t type, size_t n_in);
 
+/* ---- scale range of a quantised tensor (load-time guard) ----------------------------------
+ * No counterpart in the reference (its kernels scale in f32 after the MMA, mat_mat_fewrow_gen.metal:437-444).  The few-row
+ * Q4_K / Q6_K kernels here apply d * scale in f16 before the MFMA, which is finite only while
+ *   Q4_K: |d| <= DFLASH_Q4_K_MAX_D and |dmin| <= DFLASH_Q4_K_MAX_DMIN,   Q6_K: |d| <= DFLASH_Q6_K_MAX_D
+ * (weight scales of real checkpoints are 1e-4 .. 1e-1).  Call this once per tensor when it is uploaded: it scans the
+ * super-block headers on the device, returns the maxima in max_abs_host[2] (|d|, |dmin|; may be NULL) and
+ * DFLASH_ERR_UNSUPPORTED with a message for a tensor out of range or with a NaN / infinite scale, DFLASH_OK otherwise
+ * (and for types whose kernels have no such limit).  Blocking. */
+#define DFLASH_Q4_K_MAX_D 1.0f
+#define DFLASH_Q4_K_MAX_DMIN 32.0f
+#define DFLASH_Q6_K_MAX_D 0.25f
+int32_t dflash_check_scale_range(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_blocks, float *max_abs_host,
+                                 dflash_stream_t stream);
+
 /* ---- measurement aid: streaming-read probe ------------------------------------------
  * No counterpart in the reference.  n_launches launches of a kernel that reads `bytes` (multiple of 16) of
  * bufs[k % n_bufs] (16-byte aligned) once with a grid-stride loop of 16-byte loads and stores a word per

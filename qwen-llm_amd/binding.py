@@ -116,6 +116,8 @@ def _declare(L):
     L.dflash_dequant.argtypes = [vp, i32, vp, sz, vp, vp]
     L.dflash_gemm_fewrow.restype = i32
     L.dflash_gemm_fewrow.argtypes = [vp, i32, vp, vp, i32, vp, i64, i64, i32, vp]
+    L.dflash_check_scale_range.restype = i32
+    L.dflash_check_scale_range.argtypes = [vp, i32, vp, sz, C.POINTER(f32), vp]
     L.dflash_hbm_read_probe.restype = i32
     L.dflash_hbm_read_probe.argtypes = [vp, C.POINTER(vp), i32, sz, i32, vp, vp]
     L.dflash_q4k_tiled_bytes.restype = sz
@@ -203,6 +205,12 @@ def _torch():
     return torch
 
 
+def _empty(*args, **kwargs):
+    """Every output tensor the host mirror allocates comes from here (tests swap it for an allocator that puts guard
+    bands around the tensor)."""
+    return _torch().empty(*args, **kwargs)
+
+
 def _stream_ptr():
     torch = _torch()
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -261,7 +269,7 @@ class Context:
     def dequant_to_f32(self, qtype: int, blocks, n_elems: int, out=None):
         torch = _torch()
         if out is None:
-            out = torch.empty(n_elems, dtype=torch.float32, device=blocks.device)
+            out = _empty(n_elems, dtype=torch.float32, device=blocks.device)
         self._check(self._lib.dflash_dequant(self._h, qtype, blocks.data_ptr(), n_elems, out.data_ptr(),
                                              _stream_ptr()))
         return out
@@ -280,6 +288,13 @@ class Context:
                                                  y.data_ptr(), n_in, n_out, n_query, _stream_ptr()))
         return y
 
+    def check_scale_range(self, qtype: int, blocks, n_blocks: int):
+        """Load-time guard: raises DFlashError (UNSUPPORTED) for a Q4_K / Q6_K tensor whose super-block scales are
+        outside the few-row kernels' f16 range; returns (max |d|, max |dmin|)."""
+        out = (C.c_float * 2)()
+        self._check(self._lib.dflash_check_scale_range(self._h, int(qtype), blocks.data_ptr(), int(n_blocks), out, _stream_ptr()))
+        return float(out[0]), float(out[1])
+
     def hbm_read_probe(self, bufs, n_launches: int, scratch):
         """``n_launches`` launches of a read-only streaming kernel over the equally sized uint8 tensors ``bufs``
         (in turn); ``scratch``: int32[n_cu]."""
@@ -294,13 +309,13 @@ class Context:
         nbytes = self._lib.dflash_q4k_tiled_bytes(n_in, n_out)
         if nbytes == 0:
             raise DFlashError(2, f"bad Q4_K shape {n_out} x {n_in}")
-        out = torch.empty(nbytes, dtype=torch.uint8, device=weight.device)
+        out = _empty(nbytes, dtype=torch.uint8, device=weight.device)
         self._check(self._lib.dflash_repack_q4k_tiled(self._h, weight.data_ptr(), out.data_ptr(), n_in, n_out, _stream_ptr()))
         return out
 
     def gemm_fewrow(self, weight, w_type: int, x, n_in: int, n_out: int):
         torch = _torch()
-        y = torch.empty((x.shape[0], n_out), dtype=torch.float32, device=x.device)
+        y = _empty((x.shape[0], n_out), dtype=torch.float32, device=x.device)
         return self.encode_mat_mat_dispatch_dflash_verify(weight, w_type, x, y, n_in, n_out, x.shape[0])
 
     # ---- per-row scatter + decode attention loop of packed verify (metal_dflash.rs:9963-10062)
@@ -313,7 +328,7 @@ class Context:
         cap, n_kv = k_cache.shape[0], k_cache.shape[1]
         q_type = TYPE_F32 if q.dtype == torch.float32 else TYPE_F16
         if out is None:
-            out = torch.empty((n_rows, n_q, hd), dtype=torch.float32, device=q.device)
+            out = _empty((n_rows, n_q, hd), dtype=torch.float32, device=q.device)
         self._check(self._lib.dflash_attn_verify_block(self._h, q.data_ptr(), q_type, k_cache.data_ptr(),
                                                        v_cache.data_ptr(), 1 if v_transposed else 0, ctx_len, n_rows,
                                                        n_q, n_kv, hd, cap, scale, out.data_ptr(), _stream_ptr()))
@@ -328,8 +343,8 @@ class Context:
     def argmax_top2(self, logits):
         torch = _torch()
         logits, n, v, stride = self._rows(logits)
-        idx = torch.empty(n, dtype=torch.int32, device=logits.device)
-        gap = torch.empty(n, dtype=torch.float32, device=logits.device)
+        idx = _empty(n, dtype=torch.int32, device=logits.device)
+        gap = _empty(n, dtype=torch.float32, device=logits.device)
         self._check(self._lib.dflash_argmax_top2(self._h, logits.data_ptr(), n, v, stride, idx.data_ptr(),
                                                  gap.data_ptr(), _stream_ptr()))
         return idx, gap
@@ -337,7 +352,7 @@ class Context:
     def argmax_greedy(self, logits):
         torch = _torch()
         logits, n, v, stride = self._rows(logits)
-        idx = torch.empty(n, dtype=torch.int32, device=logits.device)
+        idx = _empty(n, dtype=torch.int32, device=logits.device)
         self._check(self._lib.dflash_argmax_greedy(self._h, logits.data_ptr(), n, v, stride, idx.data_ptr(),
                                                    _stream_ptr()))
         return idx
@@ -345,8 +360,8 @@ class Context:
     def top16(self, logits):
         torch = _torch()
         logits, n, v, stride = self._rows(logits)
-        ids = torch.empty((n, 16), dtype=torch.int32, device=logits.device)
-        vals = torch.empty((n, 16), dtype=torch.float32, device=logits.device)
+        ids = _empty((n, 16), dtype=torch.int32, device=logits.device)
+        vals = _empty((n, 16), dtype=torch.float32, device=logits.device)
         self._check(self._lib.dflash_top16(self._h, logits.data_ptr(), n, v, stride, ids.data_ptr(), vals.data_ptr(),
                                            _stream_ptr()))
         return ids, vals
@@ -372,7 +387,7 @@ class Context:
             return CodebookC(qtype, 0, rows.shape[0], rows.data_ptr())
 
         pc, sc = cb(predecessor), cb(successor)
-        out = torch.empty(n, dtype=torch.int32, device=topk_ids.device)
+        out = _empty(n, dtype=torch.int32, device=topk_ids.device)
         host = (C.c_int32 * n)()
         self._check(self._lib.dflash_select_draft_path(self._h, C.byref(pc), C.byref(sc), rank, top_k, carry_token, n,
                                                        topk_ids.data_ptr(), topk_vals.data_ptr(), sel_h.data_ptr(),

@@ -5,6 +5,8 @@
 // multiply-add, so __fmul_rn / __fsub_rn are used throughout.
 #include "common.h"
 
+#include <cstring>
+
 namespace {
 
 __device__ __forceinline__ float h2f(const uint8_t *p) {
@@ -131,5 +133,77 @@ extern "C" int32_t dflash_hbm_read_probe(dflash_ctx *ctx, const void *const *buf
         read_probe_kernel<<<ctx->n_cu * 8, kProbeThreads, 0, static_cast<hipStream_t>(stream)>>>(
             static_cast<const uint4 *>(bufs[k % n_bufs]), bytes / 16, static_cast<uint32_t *>(out_words), ctx->n_cu);
     DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+// ---- super-block scale range of a quantised tensor ------------------------------------------------
+// The few-row Q4_K / Q6_K kernels form (1024 + code) * (d * scale) in f16 on the way to the MFMA: exact and fast,
+// and finite only while |d| (and |dmin|) stay in the range below.  Real checkpoints are orders of magnitude inside
+// it (d is a weight scale, about 1e-4 .. 1e-1); a tensor outside it is declined at load time instead of silently
+// producing infinities.
+namespace {
+__global__ void __launch_bounds__(256) scale_range_kernel(const uint8_t *__restrict__ blocks, size_t n_blocks, int block_bytes, int d_off,
+                                                          int dmin_off, uint32_t *__restrict__ out) {
+    // out[0] = max |d| as f32 bits, out[1] = max |dmin|, out[2] = 1 if any is NaN or infinite
+    uint32_t md = 0, mm = 0, bad = 0;
+    for (size_t b = blockIdx.x * static_cast<size_t>(256) + threadIdx.x; b < n_blocks; b += static_cast<size_t>(gridDim.x) * 256) {
+        const uint8_t *p = blocks + b * block_bytes;
+        const __half d = *reinterpret_cast<const __half *>(p + d_off);
+        const float fd = fabsf(__half2float(d));
+        if (!(fd <= 65504.0f)) bad = 1;
+        md = max(md, __float_as_uint(fd));
+        if (dmin_off >= 0) {
+            const float fm = fabsf(__half2float(*reinterpret_cast<const __half *>(p + dmin_off)));
+            if (!(fm <= 65504.0f)) bad = 1;
+            mm = max(mm, __float_as_uint(fm));
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        md = max(md, static_cast<uint32_t>(__shfl_xor(static_cast<int>(md), off, 64)));
+        mm = max(mm, static_cast<uint32_t>(__shfl_xor(static_cast<int>(mm), off, 64)));
+        bad |= static_cast<uint32_t>(__shfl_xor(static_cast<int>(bad), off, 64));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        atomicMax(out, md);  // non-negative floats order like their bit patterns
+        atomicMax(out + 1, mm);
+        if (bad) atomicOr(out + 2, 1u);
+    }
+}
+}  // namespace
+
+extern "C" int32_t dflash_check_scale_range(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_blocks, float *max_abs_host,
+                                            dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!blocks || n_blocks == 0) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "check_scale_range: no blocks");
+    int block_bytes, d_off, dmin_off;
+    float lim_d, lim_dmin;
+    if (type == DFLASH_TYPE_Q4_K || type == DFLASH_TYPE_Q4_K_TILED) {
+        block_bytes = DFL_Q4_K_BYTES, d_off = 0, dmin_off = 2, lim_d = DFLASH_Q4_K_MAX_D, lim_dmin = DFLASH_Q4_K_MAX_DMIN;
+    } else if (type == DFLASH_TYPE_Q6_K) {
+        block_bytes = DFL_Q6_K_BYTES, d_off = 208, dmin_off = -1, lim_d = DFLASH_Q6_K_MAX_D, lim_dmin = 0.0f;
+    } else {
+        if (max_abs_host) max_abs_host[0] = max_abs_host[1] = 0.0f;
+        return DFLASH_OK;  // the other types' kernels scale in f32
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    size_t ws_off = 0;
+    uint32_t *out = dfl_ws_take<uint32_t>(ctx, &ws_off, 4 * sizeof(uint32_t));
+    if (!out) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "check_scale_range: no workspace");
+    DFL_HIP_CHECK(ctx, hipMemsetAsync(out, 0, 4 * sizeof(uint32_t), st));
+    const size_t want = (n_blocks + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(want < static_cast<size_t>(ctx->n_cu) * 8 ? want : static_cast<size_t>(ctx->n_cu) * 8);
+    scale_range_kernel<<<grid, 256, 0, st>>>(static_cast<const uint8_t *>(blocks), n_blocks, block_bytes, d_off, dmin_off, out);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    uint32_t *host = static_cast<uint32_t *>(ctx->pinned);
+    DFL_HIP_CHECK(ctx, hipMemcpyAsync(host, out, 4 * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
+    float md, mm;
+    memcpy(&md, host, 4);
+    memcpy(&mm, host + 1, 4);
+    if (max_abs_host) max_abs_host[0] = md, max_abs_host[1] = mm;
+    if (host[2] || md > lim_d || (dmin_off >= 0 && mm > lim_dmin))
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED,
+                        "tensor declined: super-block scales out of the few-row kernels' f16 range (max |d| %g, limit %g; max |dmin| %g, limit %g%s)",
+                        md, lim_d, mm, lim_dmin, host[2] ? "; NaN or infinite scale" : "");
     return DFLASH_OK;
 }

@@ -14,6 +14,7 @@ from dataclasses import asdict, dataclass
 import numpy as np
 
 from . import synth
+from . import binding as _binding
 from .binding import TYPE_Q4_K, TYPE_Q4_K_TILED, CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
 
 
@@ -310,12 +311,22 @@ def synth_draft_weights_device(cfg: DraftConfig, seed: int, device, wtype: int =
 # ---- device-resident weights ----
 
 class _Uploader:
-    def __init__(self, device, ctx=None):
-        """``ctx``: when given, Q4_K matrices uploaded with a tile shape are repacked into the tiled order."""
+    def __init__(self, device, ctx=None, tiled=True):
+        """``ctx``: when given, every Q4_K / Q6_K tensor's super-block scales are range-checked on upload (a tensor the
+        few-row kernels cannot take is declined with DFlashError) and, with ``tiled``, Q4_K matrices uploaded with a
+        tile shape are repacked into the tiled order."""
         self.torch = _torch()
         self.device = device
         self.ctx = ctx
+        self.tiled = tiled and ctx is not None
         self.keep = []
+
+    _BLOCK_BYTES = {12: 144, 14: 210}
+
+    def _guard(self, qtype, t):
+        bb = self._BLOCK_BYTES.get(int(qtype))
+        if self.ctx is not None and bb:
+            self.ctx.check_scale_range(int(qtype), t, t.numel() * t.element_size() // bb)
 
     def _from_numpy(self, a):
         """torch view of a host array; read-only arrays (views into a mapped GGUF file) are only ever copied from."""
@@ -344,7 +355,8 @@ class _Uploader:
             t = blocks.to(self.device).contiguous()
         else:
             t = self._from_numpy(np.ascontiguousarray(blocks)).to(self.device)
-        if tile_shape is not None and self.ctx is not None and int(qtype) == TYPE_Q4_K:
+        self._guard(qtype, t)
+        if tile_shape is not None and self.tiled and int(qtype) == TYPE_Q4_K:
             t = self.ctx.repack_q4k_tiled(t, tile_shape[1], tile_shape[0])
             qtype = TYPE_Q4_K_TILED
         self.keep.append(t)
@@ -367,7 +379,8 @@ class _Uploader:
                 flats.append(self._from_numpy(np.ascontiguousarray(blocks).view(np.uint8).reshape(-1)).to(self.device))
         whole = torch.cat(flats)
         qtype = int(pairs[0][0])
-        if (tile_shapes is not None and self.ctx is not None and qtype == TYPE_Q4_K
+        self._guard(qtype, whole)
+        if (tile_shapes is not None and self.tiled and qtype == TYPE_Q4_K
                 and all(ts is not None and ts[0] % 256 == 0 for ts in tile_shapes)):
             whole = self.ctx.repack_q4k_tiled(whole, tile_shapes[0][1], sum(ts[0] for ts in tile_shapes))
             qtype = TYPE_Q4_K_TILED
@@ -388,7 +401,7 @@ class TargetModel:
         FFN, the output head) into the library's tiled order at upload; expert stacks, a mixture layer's shared
         expert (the batched expert kernel reads it in row order) and the embedding table stay in GGUF row order."""
         self.ctx, self.cfg = ctx, cfg
-        up = _Uploader(f"cuda:{ctx.device}", ctx if tiled else None)
+        up = _Uploader(f"cuda:{ctx.device}", ctx, tiled)
         self._up = up
         self._layers = (LayerC * cfg.n_layers)()
         H, qd, kvd = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
@@ -460,10 +473,10 @@ class Session:
         toks = (C.c_int32 * max(n, 1))(*[int(t) for t in tokens])
         n_taps = len(self.tap_layers) if want_hidden else 0
         taps = (C.c_int32 * max(n_taps, 1))(*self.tap_layers[:n_taps])
-        argmax = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
-        gap = torch.empty(max(n, 1), dtype=torch.float32, device=dev)
-        hidden = torch.empty((n, n_taps, cfg.hidden), dtype=torch.float32, device=dev) if n_taps else None
-        logits = torch.empty((n, cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
+        argmax = _binding._empty(max(n, 1), dtype=torch.int32, device=dev)
+        gap = _binding._empty(max(n, 1), dtype=torch.float32, device=dev)
+        hidden = _binding._empty((n, n_taps, cfg.hidden), dtype=torch.float32, device=dev) if n_taps else None
+        logits = _binding._empty((n, cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
         host = (C.c_int32 * max(n, 1))() if sync else None
         self.ctx._check(self._L.dflash_verify_block(
             self.ctx._h, C.byref(self.model.c), self._h, toks, n, start_position, taps, n_taps, argmax.data_ptr(),
@@ -483,7 +496,7 @@ class DraftHead:
     def __init__(self, ctx: Context, cfg: DraftConfig, weights: dict, adjacent: bool = True, tiled: bool = True):
         """``adjacent`` / ``tiled``: as for TargetModel."""
         self.ctx, self.cfg = ctx, cfg
-        up = _Uploader(f"cuda:{ctx.device}", ctx if tiled else None)
+        up = _Uploader(f"cuda:{ctx.device}", ctx, tiled)
         self._up = up
         self._layers = (DraftLayerC * cfg.n_layers)()
         H, qd, kvd = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
@@ -563,9 +576,9 @@ class DraftSession:
         L.dflash_draft_session_selector_inputs.argtypes = [C.c_void_p] * 6
         n, rank = self.head.cfg.block_size, self.head.cfg.selector_rank
         dev = f"cuda:{self.ctx.device}"
-        ids = torch.empty((n, 16), dtype=torch.int32, device=dev)
-        vals = torch.empty((n, 16), dtype=torch.float32, device=dev)
-        sel_h = torch.empty((n, max(rank, 1)), dtype=torch.float32, device=dev)
+        ids = _binding._empty((n, 16), dtype=torch.int32, device=dev)
+        vals = _binding._empty((n, 16), dtype=torch.float32, device=dev)
+        sel_h = _binding._empty((n, max(rank, 1)), dtype=torch.float32, device=dev)
         self.ctx._check(L.dflash_draft_session_selector_inputs(self.ctx._h, self._h, ids.data_ptr(), vals.data_ptr(),
                                                                sel_h.data_ptr(), _stream_ptr()))
         return ids, vals, sel_h
@@ -579,8 +592,8 @@ class DraftSession:
         torch = _torch()
         dev = f"cuda:{self.ctx.device}"
         N = self.head.cfg.block_size
-        argmax = torch.empty(N, dtype=torch.int32, device=dev)
-        logits = torch.empty((N, self.target.cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
+        argmax = _binding._empty(N, dtype=torch.int32, device=dev)
+        logits = _binding._empty((N, self.target.cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
         host = (C.c_int32 * N)() if sync else None
         self.ctx._check(self._L.dflash_draft_block(
             self.ctx._h, C.byref(self.target.c), C.byref(self.head.c), self._h, carry_token, mask_token, noise_start_pos,

@@ -133,11 +133,13 @@ def extreme_blocks(qtype: int, n_blocks: int, seed: int) -> np.ndarray:
     super-block scales across many binades (including negative ones)."""
     rng = np.random.default_rng(seed)
     out = rng.integers(0, 256, (n_blocks, BLOCK_BYTES[qtype]), dtype=np.uint8)
-    # |d * sc| stays below 64: the Q4_K few-row kernel forms 1024 * d * sc in f16
-    scales = (rng.choice([1.0, -1.0], n_blocks) * 2.0 ** rng.integers(-12, -3, n_blocks)).astype(np.float32)
+    # up to the limits the few-row kernels accept (dflash_check_scale_range): Q4_K |d| <= 1 and |dmin| <= 32, Q6_K
+    # |d| <= 0.25; the reference's own extreme blocks (d = 0.001, dmin = 5, metal/mat_mat.rs:4228-4265) are inside
+    top = {Q4_K: 0, Q6_K: -2}.get(qtype, 0)
+    scales = (rng.choice([1.0, -1.0], n_blocks) * 2.0 ** rng.integers(-12, top + 1, n_blocks)).astype(np.float32)
     if qtype == Q4_K:
         out[:, 0:2] = _f16_bytes(scales)
-        out[:, 2:4] = _f16_bytes((rng.choice([1.0, -1.0], n_blocks) * 2.0 ** rng.integers(-12, 3, n_blocks)))
+        out[:, 2:4] = _f16_bytes((rng.choice([1.0, -1.0], n_blocks) * 2.0 ** rng.integers(-12, 6, n_blocks)))
         out[0::7, 4:16] = 0xFF
         out[1::7, 4:16] = 0x00
         out[2::7, 16:] = 0xFF
@@ -152,6 +154,26 @@ def extreme_blocks(qtype: int, n_blocks: int, seed: int) -> np.ndarray:
         out[:, 0:2] = _f16_bytes(scales)
         out[0::3, 2:] = 0x80
         out[1::3, 2:] = 0x7F
+    return out
+
+
+def reference_extreme_blocks(qtype: int, n_blocks: int) -> np.ndarray:
+    """The reference's extreme few-row blocks (metal/mat_mat.rs:4228-4265): d = 0.001 (Q4_K: dmin = 5), every other
+    byte 0x00 / 0xFF (Q6_K scales and Q8_0 quants 0x80 / 0x7F), the pattern shifted by one from block to block."""
+    bb = BLOCK_BYTES[qtype]
+    i = np.arange(bb)[None, :] + np.arange(n_blocks)[:, None]
+    even = (i % 2 == 0)
+    out = np.where(even, 0x00, 0xFF).astype(np.uint8)
+    d = _f16_bytes(np.full(1, 0.001, np.float32))
+    if qtype == Q4_K:
+        out[:, 0:2] = d
+        out[:, 2:4] = _f16_bytes(np.full(1, 5.0, np.float32))
+    elif qtype == Q6_K:
+        out[:, 192:208] = np.where(even[:, 192:208], 0x80, 0x7F)
+        out[:, 208:210] = d
+    else:
+        out[:, 2:] = np.where(even[:, 2:], 0x80, 0x7F)
+        out[:, 0:2] = d
     return out
 
 

@@ -79,7 +79,7 @@ def test_argmax_greedy_total_order_and_nan(ctx, oracle):
     assert oracle.greedy_token(row)[2] == 123
 
 
-def test_top16_matches_oracle(ctx, oracle):
+def test_top16_matches_oracle(ctx, oracle, canaries):
     for row in special_rows():
         ids, vals = ctx.top16(dev(row))
         wi, wv = oracle.top16(row)

@@ -54,7 +54,7 @@ CASES = [
 @pytest.mark.parametrize("L,n_rows,n_q,n_kv,hd", CASES)
 @pytest.mark.parametrize("transposed", [False, True])
 @pytest.mark.parametrize("q_f16", [False, True])
-def test_attn_matches_oracle(ctx, oracle, L, n_rows, n_q, n_kv, hd, transposed, q_f16):
+def test_attn_matches_oracle(ctx, oracle, L, n_rows, n_q, n_kv, hd, transposed, q_f16, canaries):
     q, k, v, cap = make_case(L * 7 + n_q, L, n_rows, n_q, n_kv, hd)
     scale = 1.0 / math.sqrt(hd)
     if q_f16:
@@ -66,7 +66,7 @@ def test_attn_matches_oracle(ctx, oracle, L, n_rows, n_q, n_kv, hd, transposed, 
     check(got, want, f"L={L} rows={n_rows} q={n_q} kv={n_kv} hd={hd}")
 
 
-def test_block_causality_and_prefix_visibility(ctx):
+def test_block_causality_and_prefix_visibility(ctx, canaries):
     """row i must not see block rows > i, and must see the whole prefix: perturbing a later block
     row leaves earlier rows bit-identical; perturbing prefix position 0 changes every row"""
     L, n_rows, n_q, n_kv, hd = 200, 16, 8, 4, 128
@@ -84,7 +84,7 @@ def test_block_causality_and_prefix_visibility(ctx):
     assert np.all(np.any(pert != base, axis=(1, 2)))
 
 
-def test_equals_sixteen_single_query_attentions(ctx):
+def test_equals_sixteen_single_query_attentions(ctx, canaries):
     """the packed call == n_rows separate one-row calls over growing prefixes (the reference's loop)"""
     L, n_q, n_kv, hd = 333, 12, 4, 128
     q, k, v, cap = make_case(5, L, 16, n_q, n_kv, hd)
@@ -97,7 +97,7 @@ def test_equals_sixteen_single_query_attentions(ctx):
 
 
 @pytest.mark.parametrize("L", [32768, 131072])
-def test_attn_long_context(ctx, oracle, L):
+def test_attn_long_context(ctx, oracle, L, canaries):
     """production shape: 48 q / 8 kv heads, hd 128; checked on a few heads against the oracle
     (the oracle is O(L) per row and head) and through linearity in V over all heads"""
     import torch
@@ -124,7 +124,7 @@ def test_attn_long_context(ctx, oracle, L):
     assert (out1 - 0.75).abs().max().item() < 2e-3
 
 
-def test_attn_guards(ctx):
+def test_attn_guards(ctx, canaries):
     import torch
 
     q = torch.zeros((17, 4, 128), device="cuda")

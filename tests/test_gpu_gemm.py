@@ -82,7 +82,7 @@ SHAPES = [(256, 16, 16), (256, 1, 1), (512, 17, 3), (1024, 33, 16), (2560, 100, 
 @pytest.mark.parametrize("qtype", QTYPES)
 @pytest.mark.parametrize("n_in,n_out,n_rows", SHAPES)
 @pytest.mark.parametrize("x_dtype", ["f32", "f16"])
-def test_gemm_fewrow_small_shapes(ctx, oracle, qtype, n_in, n_out, n_rows, x_dtype):
+def test_gemm_fewrow_small_shapes(ctx, oracle, qtype, n_in, n_out, n_rows, x_dtype, canaries):
     """tile edges, ragged n_out, every row count class, random + extreme blocks"""
     rng = np.random.default_rng(n_in * 31 + n_out * 7 + n_rows)
     nblk = n_in // dfl.synth.BLOCK_ELEMS[qtype] * n_out
@@ -96,7 +96,7 @@ def test_gemm_fewrow_small_shapes(ctx, oracle, qtype, n_in, n_out, n_rows, x_dty
 
 
 @pytest.mark.parametrize("qtype", QTYPES)
-def test_gemm_fewrow_extreme_blocks(ctx, oracle, qtype):
+def test_gemm_fewrow_extreme_blocks(ctx, oracle, qtype, canaries):
     """metal/mat_mat.rs:4228-4265: large minima / saturated codes must stay finite and accurate"""
     n_in, n_out, n_rows = 1024, 48, 16
     nblk = n_in // dfl.synth.BLOCK_ELEMS[qtype] * n_out
@@ -139,7 +139,7 @@ def test_gemm_deterministic_and_linear(ctx):
 
 @pytest.mark.parametrize("qtype", [dfl.synth.Q4_K, dfl.synth.Q6_K])
 @pytest.mark.parametrize("n_in,n_out", [(2048, 5120), (4096, 2048), (2048, 12288), (6144, 2048)])
-def test_gemm_small_split_k_repeats(ctx, oracle, qtype, n_in, n_out):
+def test_gemm_small_split_k_repeats(ctx, oracle, qtype, n_in, n_out, canaries):
     """Products of a few MB (the projections of a decoder layer) are split over K across workgroups, their
     partial tiles living in a scratch buffer that every launch shares.  Forty launches in a row, alternating
     with another shape: every result bit-identical to the first and within the GEMM bar of the f64 reference."""
@@ -201,7 +201,7 @@ TILED_SHAPES = [(256, 16, 16), (256, 250, 3), (768, 257, 16), (1024, 4096, 7), (
 
 @pytest.mark.parametrize("n_in,n_out,n_rows", TILED_SHAPES)
 @pytest.mark.parametrize("x_dtype", ["f32", "f16"])
-def test_gemm_q4k_tiled_order_is_bit_identical(ctx, n_in, n_out, n_rows, x_dtype):
+def test_gemm_q4k_tiled_order_is_bit_identical(ctx, n_in, n_out, n_rows, x_dtype, canaries):
     """The one-time repack into tiled order permutes whole blocks: the GEMM on it must give the very bits the GEMM on
     GGUF row order gives (ragged n_out, ranges that wrap over tile groups, every row count), and the padding rows of
     the last tile group must leave the output alone (guard bands around Y)."""
@@ -247,3 +247,71 @@ def test_q4k_tiled_guards(ctx):
     y = torch.empty((4, n_out), dtype=torch.float32, device="cuda")
     with pytest.raises(dfl.DFlashError):  # misaligned tiled weights
         ctx.encode_mat_mat_dispatch_dflash_verify(wt[16:], dfl.TYPE_Q4_K_TILED, x, y, n_in, n_out, 4)
+
+
+@pytest.mark.parametrize("qtype", QTYPES)
+def test_gemm_fewrow_reference_extreme_blocks(ctx, oracle, qtype, canaries):
+    """The reference's own extreme blocks (metal/mat_mat.rs:4228-4265: d = 0.001, Q4_K dmin = 5, alternating 0x00 / 0xFF
+    bytes, the pattern shifted from block to block) at a ragged shape, against the f64 product."""
+    n_in, n_out, n_rows = 1024, 45, 13
+    nblk = n_in // dfl.synth.BLOCK_ELEMS[qtype] * n_out
+    w = dfl.synth.reference_extreme_blocks(qtype, nblk)
+    x = np.random.default_rng(9).standard_normal((n_rows, n_in)).astype(np.float32)
+    ref = f64_reference(oracle, qtype, w, x, n_in, n_out)
+    y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+    check_gemm(y, ref, f"reference extreme q{qtype}")
+
+
+def _with_scales(qtype, n_blocks, d, dmin=None):
+    w = dfl.synth.random_blocks(qtype, n_blocks, 3).copy()
+    off = {dfl.synth.Q4_K: 0, dfl.synth.Q6_K: 208}[qtype]
+    w[:, off:off + 2] = np.full(1, d, np.float16).view(np.uint8)
+    if dmin is not None:
+        w[:, 2:4] = np.full(1, dmin, np.float16).view(np.uint8)
+    return w
+
+
+def test_scale_range_guard(ctx, oracle):
+    """A tensor whose super-block scales leave the f16 range of the few-row kernels is declined when it is uploaded
+    (never computed to infinities); at the limits the product is still right."""
+    n_in, n_out = 512, 32
+    nblk = n_in // 256 * n_out
+    x = np.random.default_rng(2).standard_normal((16, n_in)).astype(np.float32)
+    # at the documented limits: accepted and accurate
+    for qtype, d, dmin in ((dfl.synth.Q4_K, 1.0, 32.0), (dfl.synth.Q4_K, -1.0, -32.0), (dfl.synth.Q6_K, 0.25, None)):
+        w = _with_scales(qtype, nblk, d, dmin)
+        md, mm = ctx.check_scale_range(qtype, dev(w), nblk)
+        assert md == abs(d) and (dmin is None or mm == abs(dmin))
+        y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+        assert np.all(np.isfinite(y))
+        check_gemm(y, f64_reference(oracle, qtype, w, x, n_in, n_out), f"limit q{qtype} d={d}")
+    # beyond them: declined with a message that names the figure
+    for qtype, d, dmin in ((dfl.synth.Q4_K, 128.0, 0.5), (dfl.synth.Q4_K, 0.01, 64.0), (dfl.synth.Q6_K, 128.0, None),
+                           (dfl.synth.Q4_K, np.inf, 0.5), (dfl.synth.Q4_K, np.nan, 0.5)):
+        w = _with_scales(qtype, nblk, d, dmin)
+        with pytest.raises(dfl.DFlashError) as e:
+            ctx.check_scale_range(qtype, dev(w), nblk)
+        assert e.value.status == 2 and "declined" in str(e.value)
+    # one bad block among many is found
+    w = _with_scales(dfl.synth.Q4_K, 4096, 0.01, 0.02)
+    w[3071, 0:2] = np.full(1, 128.0, np.float16).view(np.uint8)
+    with pytest.raises(dfl.DFlashError):
+        ctx.check_scale_range(dfl.synth.Q4_K, dev(w), 4096)
+    # types without the limit pass
+    assert ctx.check_scale_range(dfl.synth.Q8_0, dev(dfl.synth.random_blocks(dfl.synth.Q8_0, 64, 1)), 64) == (0.0, 0.0)
+
+
+def test_model_upload_declines_out_of_range_tensor(ctx):
+    """The guard sits in the upload path of the host mirror: a model with one |d| = 128 block does not load."""
+    cfg = dfl.ModelConfig(n_layers=1, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, vocab=512)
+    w = dfl.synth_target_weights(cfg, seed=3)
+    qtype, blocks = w["layers"][0]["wo"]
+    blocks = np.array(blocks, copy=True)
+    flat = blocks.reshape(-1, dfl.synth.BLOCK_BYTES[qtype])
+    off = {dfl.synth.Q4_K: 0, dfl.synth.Q6_K: 208, dfl.synth.Q8_0: 0}[qtype]
+    flat[5, off:off + 2] = np.full(1, 128.0, np.float16).view(np.uint8)
+    w["layers"][0]["wo"] = (qtype, blocks)
+    if qtype == dfl.synth.Q8_0:
+        pytest.skip("synthetic wo is Q8_0: no f16-range limit")
+    with pytest.raises(dfl.DFlashError):
+        dfl.TargetModel(ctx, cfg, w)
