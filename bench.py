@@ -60,9 +60,10 @@ def cpu_baseline(shapes, weights, xs):
             "sample": f"first {int(rows_frac * 100)}% of the output rows of each of the 3 GEMMs, best of 3"}
 
 
-def attention_section(ctx):
+def attention_section(ctx, with_cpu=True):
     """Block-causal verify attention, 16 query rows after L keys, 48 q / 8 kv heads of 128, f16 K/V resident in HBM
-    (V in the transposed cache layout): microseconds per call and KV-stream GB/s = (L + 16) * 8 * 128 * 2 * 2 B / time."""
+    (V in the transposed cache layout): microseconds per call and KV-stream GB/s = (L + 16) * 8 * 128 * 2 * 2 B / time.
+    cpu_baseline: the oracle's per-(row, head) f32 attention (OpenMP) on the same tensors at the shortest context."""
     import math
 
     import torch
@@ -91,6 +92,20 @@ def attention_section(ctx):
         kv_bytes = (L + n_rows) * n_kv * hd * 2 * 2
         out.append({"context": L, "us_per_call": us, "kv_bytes": kv_bytes, "GBps": kv_bytes / (us * 1e-6) / 1e9,
                     "frac_of_hbm_peak": kv_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS})
+        if with_cpu and L == 4096:
+            import oracle
+            qn = q.float().cpu().numpy()
+            kn = k[:L + n_rows].float().cpu().numpy()
+            vn = vt[:, :, :L + n_rows].permute(2, 0, 1).contiguous().float().cpu().numpy()
+            oracle.attn_verify_block(qn, kn, vn, L, scale)
+            best = 1e30
+            for _ in range(3):
+                t0 = time.perf_counter()
+                oracle.attn_verify_block(qn, kn, vn, L, scale)
+                best = min(best, time.perf_counter() - t0)
+            out[-1]["cpu_baseline"] = {"value": kv_bytes / best / 1e9, "unit": "GB/s", "us_per_call": best * 1e6,
+                                       "cores": min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))),
+                                       "kind": "port", "sample": "the context-4096 call, best of 3 (f32 K/V on the host)"}
         del q, k, vt, o
     return out
 
@@ -130,7 +145,7 @@ def q6k_section(ctx):
     return out
 
 
-def acceptance_section(ctx):
+def acceptance_section(ctx, with_cpu=True):
     """Stochastic acceptance of one block: vocabulary 151936, 15 drafts + bonus, target logits N(0,3), draft = target +
     N(0,0.5), T 0.7 / top-p 0.95 / top-k 20, vocabulary-wide draft distribution (temperature 0.7), Philox stream.
     Time per block (device kernels + the host-side decision read-back) and logits bytes / time."""
@@ -157,8 +172,101 @@ def acceptance_section(ctx):
     times = sorted(times[4:])
     us = times[len(times) // 2] * 1e6
     logits_bytes = (2 * n - 1) * vocab * 4
-    return {"vocab": vocab, "block": n, "us_per_block": us, "logits_bytes": logits_bytes,
-            "GBps": logits_bytes / (us * 1e-6) / 1e9, "mean_accepted": accepted / 24}
+    res = {"vocab": vocab, "block": n, "us_per_block": us, "logits_bytes": logits_bytes,
+           "GBps": logits_bytes / (us * 1e-6) / 1e9, "mean_accepted": accepted / 24}
+    if with_cpu:
+        # the oracle's restatement of decide_dflash_accept_prefix + Sampler (one thread per block, as the reference's
+        # host code runs it) on the same logits, same samplers
+        import oracle
+        tn, dn = target.cpu().numpy(), draft.cpu().numpy()
+        cpu_times, cpu_accepted = [], 0
+        for trial in range(8):
+            so = oracle.make_sampler(temperature=0.7, top_k=20, top_p=0.95, min_p=0.0, seed=trial, rng_kind=oracle.RNG_PHILOX)
+            t0 = time.perf_counter()
+            rc, d = oracle.decide_accept_prefix_dense(verified, tn, dn, vocab, 0.7, so, 1000, [])
+            cpu_times.append(time.perf_counter() - t0)
+            cpu_accepted += int(d.n_accepted) if hasattr(d, "n_accepted") else 0
+        cpu_times.sort()
+        cpu_us = cpu_times[len(cpu_times) // 2] * 1e6
+        res["cpu_baseline"] = {"value": logits_bytes / (cpu_us * 1e-6) / 1e9, "unit": "GB/s", "us_per_block": cpu_us, "cores": 1,
+                               "kind": "port", "sample": "8 of the 24 blocks, median"}
+    return res
+
+
+def c1_section(ctx, with_cpu=True):
+    """The CPU-runnable plumbing case: greedy verify of one 16-token draft block on a 4-layer dense decoder (hidden 1024,
+    16 q / 8 kv heads of 128, SwiGLU 3072, vocabulary 32000; Q4_K projections, Q6_K embedding and output head, random
+    blocks) after a 512-token prefix; the first 7 drafts are the target's own greedy continuation, so the accepted
+    prefix is known.  GPU: verify + greedy accept + rollback per block.  cpu_baseline: the oracle's forward (OpenMP)
+    and acceptance on the same weights and tokens, the one verify block timed after an untimed prefill."""
+    import numpy as np
+    import torch
+
+    import qwen_llm_amd as dfl
+
+    cfg = dfl.ModelConfig(n_layers=4, hidden=1024, n_q=16, n_kv=8, head_dim=128, ffn=3072, vocab=32000)
+    weights = dfl.synth_target_weights_blocks(cfg, 0, attn_type=dfl.synth.Q4_K)
+    model = dfl.TargetModel(ctx, cfg, weights)
+    prompt = np.random.default_rng(0).integers(0, cfg.vocab, 512).tolist()
+    sess = dfl.Session(ctx, model, 640, [])
+    for s0 in range(0, 512, 16):
+        out = sess.encode_packed_verify_layer_major(prompt[s0:s0 + 16], s0, want_hidden=False)
+    cont = [out.argmax_host[-1]]
+    for i in range(8):
+        cont.append(sess.encode_packed_verify_layer_major([cont[-1]], 512 + i, want_hidden=False).argmax_host[0])
+    sess.encode_restore_after_partial_accept(512, 8, 0)
+    k = 7
+    rng = np.random.default_rng(1)
+    block = cont[:1 + k] + [int((cont[1 + k] + 1 + rng.integers(0, 100)) % cfg.vocab)] + rng.integers(0, cfg.vocab, 15 - k - 1).tolist()
+
+    def one():
+        o = sess.encode_packed_verify_layer_major(block, 512, want_hidden=False)
+        acc = 0
+        while acc < 15 and block[1 + acc] == o.argmax_host[acc]:
+            acc += 1
+        sess.encode_restore_after_partial_accept(512, 16, 0)
+        return acc, o.argmax_host[acc]
+
+    for _ in range(3):
+        acc, bonus = one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 20
+    for _ in range(reps):
+        one()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / reps * 1e3
+    sess.close()
+    res = {"config": "4 layers, hidden 1024, 16q/8kv x 128, ffn 3072, vocab 32000, prefix 512, block 16, forced k=7",
+           "ms_per_verify_block": ms, "accepted_drafts": acc, "bonus_token": int(bonus),
+           "blocks_per_s": 1e3 / ms, "accepted_tokens_per_s": (acc + 1) * 1e3 / ms}
+    if with_cpu:
+        import oracle
+        omodel, _keep = oracle.build_model(cfg.as_dict(), weights)
+        ostate = oracle.TargetState(cfg.as_dict(), 640)
+        for s0 in range(0, 512, 16):
+            oracle.target_verify(omodel, ostate, prompt[s0:s0 + 16], s0, [])
+        t0 = time.perf_counter()
+        lo, _ = oracle.target_verify(omodel, ostate, block, 512, [])
+        am = lo.argmax(axis=1)
+        oacc = 0
+        while oacc < 15 and block[1 + oacc] == int(am[oacc]):
+            oacc += 1
+        cpu_ms = (time.perf_counter() - t0) * 1e3
+        res["cpu_baseline"] = {"value": 1e3 / cpu_ms, "unit": "blocks/s", "ms_per_verify_block": cpu_ms,
+                               "cores": min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))), "kind": "port",
+                               "sample": "the one 16-token verify block after an untimed 512-token prefill, single run",
+                               "accepted_drafts": oacc, "bonus_token": int(am[oacc])}
+        res["matches_cpu"] = bool(oacc == acc and int(am[oacc]) == int(bonus))
+    return res
+
+
+def acceptance_table(hist):
+    """Per-position acceptance of the draft block from the histogram of accepted lengths: position i (1-based) is
+    accepted in the steps that accepted at least i drafts.  alpha_pos1 is the first position's rate."""
+    steps = max(sum(hist), 1)
+    at_least = [sum(hist[i:]) / steps for i in range(1, 16)]
+    return {"alpha_pos1": at_least[0], "per_position_acceptance": at_least, "accept_len_hist": list(hist)}
 
 
 def e2e_speculative(ctx, n_generate, sweep, log):
@@ -236,6 +344,7 @@ def e2e_speculative(ctx, n_generate, sweep, log):
             "draft_ms": st["draft_ms"] / st["spec_steps"], "verify_ms": st["verify_ms"] / st["spec_steps"],
             "accept_ms": st["accept_ms"] / st["spec_steps"], "append_ms": st["append_ms"] / st["spec_steps"],
             "tokens_equal_serial_greedy": agree, "tokens": len(tokens)})
+        res["sweep"][-1].update(acceptance_table(st.get("accept_len_hist", [0] * 16)))
         log(f"e2e: forced k={k}: {res['sweep'][-1]}")
 
     # Stochastic acceptance (sampler coupled to deterministic drafts), forced the same way: the serial sampler's own
@@ -272,6 +381,7 @@ def e2e_speculative(ctx, n_generate, sweep, log):
         "draft_ms": st["draft_ms"] / st["spec_steps"], "verify_ms": st["verify_ms"] / st["spec_steps"],
         "accept_ms": st["accept_ms"] / st["spec_steps"],
         "tokens_equal_serial_sampler": sum(int(a == b) for a, b in zip(tokens, stream)), "tokens": len(tokens)}
+    res["sampled"].update(acceptance_table(st.get("accept_len_hist", [0] * 16)))
     log(f"e2e: sampled, forced k={k}: {res['sampled']}")
     return res
 
@@ -495,9 +605,11 @@ def main():
     del wd, xd, yd, wrow
     if not args.gemm_only:
         try:
+            with_cpu = not args.no_cpu_baseline
             out["gemm_q6k"] = q6k_section(ctx)
-            out["attention"] = attention_section(ctx)
-            out["acceptance"] = acceptance_section(ctx)
+            out["attention"] = attention_section(ctx, with_cpu)
+            out["acceptance"] = acceptance_section(ctx, with_cpu)
+            out["c1_verify"] = c1_section(ctx, with_cpu)
         except Exception as e:  # the GEMM line above stays valid
             out["sections_error"] = f"{type(e).__name__}: {e}"
     if not args.no_e2e and not args.gemm_only:

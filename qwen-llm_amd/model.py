@@ -821,6 +821,8 @@ class SpeculativeDecoder:
             d = res.decision
             stats["spec_steps"] += 1
             stats["accepted_drafts"] += d.n_accepted
+            hist = stats.setdefault("accept_len_hist", [0] * 16)  # steps by number of accepted drafts (0..15)
+            hist[min(d.n_accepted, 15)] += 1
             stats["drafts_scored"] += res.n_block - 1
             stats["fallback_calls"] += res.fallback_ran
             for k in ("draft_ms", "verify_ms", "accept_ms", "fallback_ms", "append_ms", "restore_ms"):
