@@ -269,8 +269,11 @@ void dflash_sampler_advance(dflash_sampler *s, uint64_t draws);
  *                    (sum order: 1024-token tiles, 256 four-element slots, halving tree, tiles
  *                    added in order)
  * The whole block is validated before anything is drawn; the sampler advances by the draws
- * actually consumed and only on DFLASH_OK.  top_k must be in 1..64 (or vocab <= 64) when
- * temperature > 0.  Synchronises: the decision is returned on the host. */
+ * actually consumed and only on DFLASH_OK.  Any top_k (sampling.rs:1198-1214, 1273-1296): up to 64
+ * candidates per row stay on the streaming selection kernels; top_k = 0 (the whole vocabulary) and
+ * top_k > 64 order the block's rows with one device-wide sort and need about 3 * 8 bytes per
+ * (row, token) of context workspace (DFLASH_ERR_WORKSPACE names the figure).  Synchronises: the
+ * decision is returned on the host. */
 enum { DFLASH_CARRY_NONE = 0, DFLASH_CARRY_CORRECTION = 1, DFLASH_CARRY_BONUS = 2 };
 enum { DFLASH_STOP_NONE = 0, DFLASH_STOP_EOS = 1, DFLASH_STOP_TOKEN_LIMIT = 2 };
 
@@ -503,7 +506,9 @@ typedef struct {
  * 1.. (entries < 0 keep the drafter's token): the loop's prefix-replay drafts (qwen/dflash.rs:700-712).
  * sampler is required when sampled_mode != 0, proposal_sampler (temperature only, its seed the
  * target's ^ 0x4446_4c41_5348_3251 in the reference) when sampled_mode == 2, which takes no override.
- * Blocking. */
+ * On ANY error nothing is committed: both samplers and the session's kv_n_pos are put back to what
+ * they were on entry (the drafter session's watermarks only advance after a whole block), so the
+ * caller may retry the step or fall back to a plain decode step at `position`.  Blocking. */
 int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dflash_draft_head *head,
                          dflash_session *session, dflash_draft_session *draft_session,
                          const int32_t *tap_layers_host, int32_t n_taps, int32_t carry_token, int64_t position,
