@@ -106,6 +106,8 @@ def _declare(L):
                                                    vp, C.POINTER(SamplerC), vp, vp, C.POINTER(WeightedCandidateC), vp]
     L.dflash_ctx_set_stream_kernel_only.restype = None
     L.dflash_ctx_set_stream_kernel_only.argtypes = [vp, i32]
+    L.dflash_ctx_set_draft_graphs.restype = None
+    L.dflash_ctx_set_draft_graphs.argtypes = [vp, i32]
     L.dflash_ctx_set_graphs.restype = None
     L.dflash_ctx_set_graphs.argtypes = [vp, i32]
     L.dflash_ctx_kernel_timing.restype = i32
@@ -251,6 +253,10 @@ class Context:
 
     def set_kernel_timing(self, enable: bool):
         self._lib.dflash_ctx_set_kernel_timing(self._h, int(enable))
+
+    def set_draft_graphs(self, enable: bool):
+        """Graph replay of the drafter's block forward on or off (off by default; results are the same)."""
+        self._lib.dflash_ctx_set_draft_graphs(self._h, int(enable))
 
     def set_stream_kernel_only(self, enable: bool):
         """Measurement aid: split-K GEMM calls launch their streaming kernel only (Y incomplete while on)."""

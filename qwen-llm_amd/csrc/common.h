@@ -32,6 +32,7 @@ struct dflash_ctx {
     // launch into (the caller's may be the legacy default stream, which cannot be captured) and
     // the two events that order it against the caller's stream
     bool graphs = false;
+    bool draft_graphs = false;  // graph replay of the drafter's block forward (measured: no faster than direct launches)
     hipStream_t gstream = nullptr;
     hipEvent_t g_in = nullptr, g_out = nullptr;
     // pinned host staging for the few words a blocking call reads back (a device-to-host copy into pageable

@@ -75,6 +75,7 @@ int32_t dflash_ctx_create(int32_t device, size_t workspace_bytes, dflash_ctx **o
         return DFLASH_ERR_HIP;
     }
     if (const char *e = getenv("DFLASH_GRAPHS")) ctx->graphs = atoi(e) != 0;
+    if (const char *e = getenv("DFLASH_DRAFT_GRAPH")) ctx->draft_graphs = atoi(e) != 0;
     *out = ctx;
     return DFLASH_OK;
 }
@@ -103,6 +104,10 @@ void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable) {
 
 void dflash_ctx_set_graphs(dflash_ctx *ctx, int32_t enable) {
     if (ctx) ctx->graphs = enable != 0;
+}
+
+void dflash_ctx_set_draft_graphs(dflash_ctx *ctx, int32_t enable) {
+    if (ctx) ctx->draft_graphs = enable != 0;
 }
 
 void dflash_ctx_set_stream_kernel_only(dflash_ctx *ctx, int32_t enable) {

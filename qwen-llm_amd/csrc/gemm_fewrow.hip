@@ -1072,9 +1072,8 @@ __device__ __forceinline__ void q4k_tiled_compute(const u32x4_t *blk, const uint
 template <typename XT>
 __global__ void __launch_bounds__(64 * kSlabWaves)
     gemm_q4k_tiled_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y,
-                          float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt) {
+                          float *__restrict__ partials, int n_out, int nb, int n_rows, int n_groups, Q4KBatch bt, int kPre) {
     constexpr int kW = kSlabWaves;
-    constexpr int kPre = 2;  // weight stages issued ahead of the wait for the activations
     extern __shared__ half8_t lds[];
     uint8_t *slab = reinterpret_cast<uint8_t *>(lds);                                // [kSlabStages][kTiledStageX]
     half8_t *ring = reinterpret_cast<half8_t *>(slab + kSlabStages * kTiledStageX);  // [wave][kSlabRing][144]
@@ -1126,8 +1125,9 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
         w_issued++;
         wlane += kTiledStageBytes;
     };
-    // Two stages go out ahead of the wait for the activations, the third after the slab barrier.  Measured (50 MB
-    // matrix, kernel time): 15.6 / 15.2 / 14.6 / 14.8 us with 0 / 1 / 2 / 3 stages ahead.  A CU's memory pipeline
+    // kPre (host: two, or one for ranges of at most two stages) stages go out ahead of the wait for the activations,
+    // the rest of the first three after the slab barrier.  Measured (50 MB matrix, kernel time): 15.6 / 15.2 / 14.6 /
+    // 14.8 us with 0 / 1 / 2 / 3 stages ahead.  A CU's memory pipeline
     // takes new loads only as fast as data returns (27 KB/us, its share of HBM), so a wave that issues more stalls
     // at the issue and reaches the barrier late; with none ahead the activations are back after 1.2 us instead of
     // 3.5, but the weights start 2 us later.
@@ -1946,14 +1946,17 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         const void *fn = x_type == DFLASH_TYPE_F32 ? reinterpret_cast<const void *>(gemm_q4k_tiled_kernel<float>)
                                                    : reinterpret_cast<const void *>(gemm_q4k_tiled_kernel<_Float16>);
         if (const int32_t rc_ = dfl_raise_lds_limit(ctx, fn, kTiledLdsBytes)) return rc_;
+        // weight stages issued ahead of the wait for the activations: two, or one when no range is longer than two
+        // stages (measured on the 17.7 MB shape: 11.2 against 12.0 us per call; on the 50 MB shapes 19.1 against 18.7)
+        const int k_pre = env_int("DFLASH_Q4K_PRE", (total + n_wg - 1) / n_wg <= 2 ? 1 : 2);
         {
             dfl_timed timer(ctx, st, DFL_T_GEMM);
             if (x_type == DFLASH_TYPE_F32)
                 gemm_q4k_tiled_kernel<float><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const float *>(x), y, partials, no,
-                                                                                           nb, n_rows, groups, bt);
+                                                                                           nb, n_rows, groups, bt, k_pre);
             else
                 gemm_q4k_tiled_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
-                                                                                              partials, no, nb, n_rows, groups, bt);
+                                                                                              partials, no, nb, n_rows, groups, bt, k_pre);
         }
         if (reduce) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);

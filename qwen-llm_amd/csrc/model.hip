@@ -390,6 +390,11 @@ struct dflash_draft_session {
     int32_t *topk_ids = nullptr; // [16][16]
     float *topk_vals = nullptr;  // [16][16]
     float *sel_h = nullptr;      // [16][selector_rank]
+    // captured graphs of the block forward (everything after the context preparation), one per distinct
+    // (head, target, outputs) key; see draft_block_impl
+    std::map<uint64_t, hipGraphExec_t> graphs;
+    std::map<uint64_t, int> graph_seen;
+    int64_t graph_replays = 0;
 };
 
 extern "C" {
@@ -737,8 +742,12 @@ void dflash_draft_session_destroy(dflash_draft_session *s) {
                     s->conv_buf, s->conv_dyn, s->topk_ids, s->topk_vals, s->sel_h};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
+    for (auto &g : s->graphs)
+        if (g.second) (void)hipGraphExecDestroy(g.second);
     delete s;
 }
+
+int64_t dflash_draft_session_graph_replays(const dflash_draft_session *s) { return s ? s->graph_replays : -1; }
 
 int64_t dflash_draft_session_ctx_len(const dflash_draft_session *s) { return s ? s->ctx_len : -1; }
 
@@ -904,6 +913,13 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         pos_arg.v[i] = static_cast<int32_t>(noise_start + i);
     }
     set_ids_pos_kernel<<<1, 64, 0, st>>>(ids_arg, pos_arg, N, s->ids, s->pos, nullptr, 0);
+    float *lg = draft_logits ? draft_logits : s->logits;
+    int32_t *am = draft_argmax ? draft_argmax : s->argmax;
+    // Everything from the noise embedding to the argmax, on stream `st`: the launches depend on the call only through
+    // device memory (ids, pos; the attention reads the context length from pos[0]) - except the DFlash-2 selector
+    // walk, which takes the carry by value - so they can be captured once and replayed.
+    auto enqueue = [&](hipStream_t st) -> int32_t {
+    int32_t rc;
     if ((rc = embed_rows(ctx, target->token_embd, s->ids, N, H, s->x, st))) return rc;
 
     const float *pending_resid = nullptr;
@@ -935,9 +951,11 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                 packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k,
                 L.q_norm, L.k_norm, k16, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, packed ? s->pk + q_dim + kv_dim : s->v,
                 packed ? tot : kv_dim, vt16, s->cap16);
+            // (context length = pos[0], read on the device: the launch does not depend on it, so a captured graph
+            // of the block stays valid as the context grows; chunking, and so the result, is the same either way)
             if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, k16, vt16, 1, s->ctx_len, N, c.n_q, c.n_kv, hd, s->cap16,
                                      1.0f / sqrtf(static_cast<float>(hd)), s->attn, st, c.causal ? 0 : 1,
-                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, nullptr)))
+                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, s->pos)))
                 return rc;
         } else {
             qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, q_dim, s->k, kv_dim, s->q, s->k, L.q_norm, L.k_norm,
@@ -978,9 +996,7 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         pending_resid = resid;  // residual 2: added by the norm that reads x next (same x + r, one launch fewer)
     }
     rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, head->output_norm, s->cur, H, c.eps, nullptr, nullptr);
-    float *lg = draft_logits ? draft_logits : s->logits;
     if ((rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st))) return rc;
-    int32_t *am = draft_argmax ? draft_argmax : s->argmax;
     if (c.selector_rank > 0) {
         // DFlash-2 tail (:17098-17130, select_draft_path :17176-17251): the 16 best candidates of every
         // row, the selector gate W_h . h of the output-normed hidden, and the predecessor-conditioned
@@ -992,6 +1008,62 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                                            c.selector_top_k, carry, N, s->topk_ids, s->topk_vals, s->sel_h, am, nullptr, st)))
             return rc;
     } else if ((rc = dflash_argmax_greedy(ctx, lg, N, V, V, am, st))) {
+        return rc;
+    }
+    return DFLASH_OK;
+    };  // enqueue
+
+    // Graph replay (off by default; DFLASH_DRAFT_GRAPH=1 or dflash_ctx_set_draft_graphs(ctx, 1) turn it on): a block is
+    // about 80 launches of 4..8 us kernels.  Second call with the same key captures, later ones replay.  Measured on
+    // the 5-layer drafter of the end-to-end configuration: 0.79 ms per block replayed against 0.77 ms launched one by
+    // one - the block is bound by the kernels' own dependent-launch latency on the GPU, not by the host's enqueueing -
+    // so it stays off, like the verify's.  Not for a walk that takes the carry by value, not on the
+    // general-attention path (its launches depend on the context length), not under kernel timers.
+    const bool walk_by_value = c.selector_rank > 0 && !skip_selector_walk;
+    const bool use_graph = ctx->draft_graphs && fast && !walk_by_value && !ctx->timing && ctx->gstream;
+    uint64_t key = 0;
+    if (use_graph) {
+        key = hash_model(target);
+        const uintptr_t ptrs[6] = {reinterpret_cast<uintptr_t>(head->layers), reinterpret_cast<uintptr_t>(head->fc.data),
+                                   reinterpret_cast<uintptr_t>(head->output_norm), reinterpret_cast<uintptr_t>(lg),
+                                   reinterpret_cast<uintptr_t>(am), static_cast<uintptr_t>(skip_selector_walk)};
+        key = hash_bytes(ptrs, sizeof(ptrs), key);
+        for (int il = 0; il < c.n_layers; il++) {
+            const dflash_draft_layer &L = head->layers[il];
+            const uintptr_t lp[9] = {reinterpret_cast<uintptr_t>(L.wq.data), reinterpret_cast<uintptr_t>(L.wk.data),
+                                     reinterpret_cast<uintptr_t>(L.wv.data), reinterpret_cast<uintptr_t>(L.wo.data),
+                                     reinterpret_cast<uintptr_t>(L.gate.data), reinterpret_cast<uintptr_t>(L.up.data),
+                                     reinterpret_cast<uintptr_t>(L.down.data), static_cast<uintptr_t>(L.wq.type),
+                                     static_cast<uintptr_t>(L.is_swa)};
+            key = hash_bytes(lp, sizeof(lp), key);
+        }
+    }
+    auto exec_it = use_graph ? s->graphs.find(key) : s->graphs.end();
+    if (use_graph && exec_it == s->graphs.end() && s->graph_seen.size() > 64) s->graph_seen.clear();
+    if (use_graph && exec_it == s->graphs.end() && s->graphs.size() < 8 && s->graph_seen[key]++ >= 1) {
+        hipGraph_t graph = nullptr;
+        DFL_HIP_CHECK(ctx, hipStreamBeginCapture(ctx->gstream, hipStreamCaptureModeThreadLocal));
+        rc = enqueue(ctx->gstream);
+        const hipError_t end = hipStreamEndCapture(ctx->gstream, &graph);
+        if (rc) {
+            if (graph) (void)hipGraphDestroy(graph);
+            return rc;
+        }
+        DFL_HIP_CHECK(ctx, end);
+        hipGraphExec_t exec = nullptr;
+        const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        DFL_HIP_CHECK(ctx, inst);
+        exec_it = s->graphs.emplace(key, exec).first;
+    }
+    if (exec_it != s->graphs.end()) {
+        DFL_HIP_CHECK(ctx, hipEventRecord(ctx->g_in, st));
+        DFL_HIP_CHECK(ctx, hipStreamWaitEvent(ctx->gstream, ctx->g_in, 0));
+        DFL_HIP_CHECK(ctx, hipGraphLaunch(exec_it->second, ctx->gstream));
+        s->graph_replays++;
+        DFL_HIP_CHECK(ctx, hipEventRecord(ctx->g_out, ctx->gstream));
+        DFL_HIP_CHECK(ctx, hipStreamWaitEvent(st, ctx->g_out, 0));
+    } else if ((rc = enqueue(st))) {
         return rc;
     }
     DFL_HIP_CHECK(ctx, hipGetLastError());

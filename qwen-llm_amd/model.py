@@ -132,6 +132,8 @@ def _lib():
         L.dflash_draft_session_destroy.argtypes = [vp]
         L.dflash_draft_session_ctx_len.restype = i64
         L.dflash_draft_session_ctx_len.argtypes = [vp]
+        L.dflash_draft_session_graph_replays.restype = i64
+        L.dflash_draft_session_graph_replays.argtypes = [vp]
         L.dflash_draft_prepare_ctx.restype = i32
         L.dflash_draft_prepare_ctx.argtypes = [vp, vp, vp, vp]
         L.dflash_draft_append_ctx.restype = i32
@@ -557,6 +559,10 @@ class DraftSession:
     def ctx_len(self) -> int:
         return self._L.dflash_draft_session_ctx_len(self._h)
 
+    @property
+    def graph_replays(self) -> int:
+        return int(self._L.dflash_draft_session_graph_replays(self._h))
+
     def append_target_ctx_columns(self, hidden_capture, positions):
         """hidden_capture: device f32 [n_cols][n_taps][hidden]; positions: their token positions."""
         n = len(positions)
@@ -588,12 +594,17 @@ class DraftSession:
         (draft_block does it lazily otherwise)."""
         self.ctx._check(self._L.dflash_draft_prepare_ctx(self.ctx._h, C.byref(self.head.c), self._h, _stream_ptr()))
 
-    def draft_block(self, carry_token: int, mask_token: int, noise_start_pos: int, want_logits=False, sync=True):
+    def draft_block(self, carry_token: int, mask_token: int, noise_start_pos: int, want_logits=False, sync=True, out=None):
+        """``out`` = (argmax, logits) tensors to write into (the same output pointers from call to call let the
+        library replay its captured graph of the block); fresh tensors otherwise."""
         torch = _torch()
         dev = f"cuda:{self.ctx.device}"
         N = self.head.cfg.block_size
-        argmax = _binding._empty(N, dtype=torch.int32, device=dev)
-        logits = _binding._empty((N, self.target.cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
+        if out is not None:
+            argmax, logits = out
+        else:
+            argmax = _binding._empty(N, dtype=torch.int32, device=dev)
+            logits = _binding._empty((N, self.target.cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
         host = (C.c_int32 * N)() if sync else None
         self.ctx._check(self._L.dflash_draft_block(
             self.ctx._h, C.byref(self.target.c), C.byref(self.head.c), self._h, carry_token, mask_token, noise_start_pos,

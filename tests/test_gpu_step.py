@@ -355,3 +355,57 @@ def test_baseline_plumbing_case_prefix_512(ctx, world, k):
     assert d.n_accepted == k and list(d.accepted_drafts[:k]) == cont[1:1 + k] and d.carry_token == cont[k + 1]
     assert dec.session.kv_n_pos == 512 + k + 1 == dec.position == dec.draft_session.ctx_len
     dec.close()
+
+
+def test_draft_graph_replays_equal_eager_blocks(ctx, world):
+    """The drafter's block forward replayed from its captured graph gives the very logits the launches give one by one:
+    eight consecutive blocks on two sessions (graph on / off) as the context grows by a ragged number of columns per
+    step, with eager work (verify, context append, read-backs) and synchronisations between the replays; then a whole
+    generation with the graph on equals the one with it off."""
+    import torch
+    head = dfl.DraftHead(ctx, D1, dfl.synth_draft_weights(D1, seed=4))
+    model = world["model"]
+    sess = dfl.Session(ctx, model, 256, TAPS)
+    ds = {True: dfl.DraftSession(ctx, head, model, 256), False: dfl.DraftSession(ctx, head, model, 256)}
+    outs = {g: (torch.empty(D1.block_size, dtype=torch.int32, device="cuda"),
+                torch.empty((D1.block_size, C1.vocab), dtype=torch.float32, device="cuda")) for g in ds}
+    for s0 in range(0, PROMPT_LEN, 16):
+        blk = world["prompt"][s0:s0 + 16]
+        out = sess.encode_packed_verify_layer_major(blk, s0)
+        for d in ds.values():
+            d.append_target_ctx_columns(out.hidden_capture, list(range(s0, s0 + len(blk))))
+    pos, carry = PROMPT_LEN, int(out.argmax_host[-1])
+    rng = np.random.default_rng(3)
+    try:
+        for step in range(8):
+            got = {}
+            for g, d in ds.items():
+                ctx.set_draft_graphs(g)
+                d.draft_block(carry, MASK, pos, want_logits=True, out=outs[g])
+                got[g] = (outs[g][0].cpu().numpy().copy(), outs[g][1].cpu().numpy().copy())
+            assert np.array_equal(got[True][0], got[False][0]), f"step {step}: draft tokens differ"
+            assert np.array_equal(got[True][1].view(np.uint32), got[False][1].view(np.uint32)), f"step {step}: logits differ"
+            # eager work between replays: verify a block, keep a ragged prefix, append its columns to both drafters
+            keep = int(rng.integers(1, 9))
+            block = [carry] + [int(t) for t in got[True][0][1:]]
+            v = sess.encode_packed_verify_layer_major(block, pos)
+            sess.encode_restore_after_partial_accept(pos, len(block), keep)
+            for d in ds.values():
+                d.append_target_ctx_columns(v.hidden_capture[:keep], list(range(pos, pos + keep)))
+            carry, pos = int(v.argmax_host[keep - 1]), pos + keep
+        assert ds[True].graph_replays >= 6 and ds[False].graph_replays == 0
+        results = {}
+        for g in (True, False):
+            ctx.set_draft_graphs(g)
+            dec = dfl.SpeculativeDecoder(ctx, model, head, TAPS, 256, MASK)
+            first = dec.prefill(world["prompt"])
+            results[g] = dec.generate(first, 40)[0]
+            if g:
+                assert dec.draft_session.graph_replays > 0
+            dec.close()
+        assert results[True] == results[False]
+    finally:
+        ctx.set_draft_graphs(False)
+        sess.close()
+        for d in ds.values():
+            d.close()
