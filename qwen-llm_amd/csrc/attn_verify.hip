@@ -46,7 +46,7 @@ __device__ __forceinline__ float xor_lane(float v, int mask) {
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-constexpr int kAttnBufs = 3;  // LDS ring: stages in flight + the one being consumed
+constexpr int kAttnBufs = 3;  // LDS ring: stages in flight + the one being consumed (a fourth buffer measured the same)
 
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 constexpr int attn_vmcnt(int n) { return ((n & 0xF) | ((n & 0x30) << 10)) | 0x0F70; }
