@@ -545,14 +545,24 @@ __global__ void __launch_bounds__(64 * kWaves)
     const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(x);
     constexpr uint32_t kXBlockBytes = DFL_QK_K * sizeof(XT);
 
-    // first weight byte of a group's first row, its activations, and the local group index
+    // first weight byte of a group's first row, its activations, and the local group index.  Tiled order: a
+    // matrix is cut in 256-row tile groups stored [group][super-block][256 rows x 144 bytes]; an 8-wave workgroup
+    // owns the lower or the upper 128 rows of one, i.e. the first or second half of each of its stages.
+    constexpr int kPerTiled = 16 / kWaves;  // this kernel's groups per tile group of the tiled order
     auto group_w = [&](int group) {
-        if (!bt.ids) return w + static_cast<size_t>(group) * group_bytes;
-        const bool up = bt.pair && (group & 1);
-        group >>= vshift;
-        const int j = static_cast<int>(q4k_div(group, bt.by_gpm)), lg = group - j * bt.groups_per_mat;
-        const int32_t id = bt.ids[j];
-        const uint8_t *mat = id < 0 ? (up ? bt.extra_w2 : bt.extra_w) : (up ? bt.w2 : w) + static_cast<size_t>(id) * bt.w_stride;
+        const uint8_t *mat = w;
+        int lg = group;
+        if (bt.ids) {
+            const bool up = bt.pair && (group & 1);
+            const int g = group >> vshift;
+            const int j = static_cast<int>(q4k_div(g, bt.by_gpm));
+            lg = g - j * bt.groups_per_mat;
+            const int32_t id = bt.ids[j];
+            mat = id < 0 ? (up ? bt.extra_w2 : bt.extra_w) : (up ? bt.w2 : w) + static_cast<size_t>(id) * bt.w_stride;
+        }
+        if (tiled)
+            return q4k_uniform(mat + static_cast<size_t>(lg / kPerTiled) * nb * kTiledStageBytes +
+                               static_cast<size_t>(lg % kPerTiled) * (G::kRows * DFL_Q4_K_BYTES));
         return q4k_uniform(mat + static_cast<size_t>(lg) * group_bytes);
     };
     auto group_x = [&](int group) {
@@ -571,9 +581,7 @@ __global__ void __launch_bounds__(64 * kWaves)
     // Cursors.  Weights: wstage = first byte of the next stage to load in its group's first row,
     // bw its super-block, gw its group, w_left the stages not loaded yet.  Activations run one
     // stage further ahead: xblock / bx / x_left.
-    // (tiled order, single matrix with 16 waves only: stage it of the iteration space is the it-th 36 864-byte piece)
-    const uint8_t *wstage = tiled ? w + static_cast<size_t>(rg.it_begin) * kTiledStageBytes
-                                  : group_w(rg.first_group) + static_cast<size_t>(b0) * DFL_Q4_K_BYTES;
+    const uint8_t *wstage = group_w(rg.first_group) + static_cast<size_t>(b0) * (tiled ? kTiledStageBytes : DFL_Q4_K_BYTES);
     int bw = b0, gw = rg.first_group, w_left = rg.it_end - rg.it_begin;
     const uint8_t *xblock = group_x(rg.first_group) + static_cast<size_t>(b0) * kXBlockBytes;
     int bx = b0, gx = rg.first_group, x_left = w_left;
@@ -584,9 +592,9 @@ __global__ void __launch_bounds__(64 * kWaves)
         if (++bw == nb) {
             bw = 0;
             gw++;
-            if (w_left > 0 && !tiled) {
+            if (w_left > 0) {
                 wstage = group_w(gw);
-                if (ragged) q4k_lane_w_offsets<kWaves>(L, tid, group_local(gw) * G::kRows, n_out, row_bytes);
+                if (ragged && !tiled) q4k_lane_w_offsets<kWaves>(L, tid, group_local(gw) * G::kRows, n_out, row_bytes);
             }
         }
     };
@@ -1902,8 +1910,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         slab = wgs >= 1 && (total16 + wgs - 1) / wgs <= kSlabStages;
         if (slab) waves = 16;
     }
-    if (tiled && batch) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: tiled Q4_K is for single matrices");
-    if (tiled) waves = 16;  // the tiled order is cut in 256-row groups
+    if (tiled && !batch) waves = 16;  // a single tiled matrix: whole 256-row tile groups (a batch may use their halves)
     const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
     const int groups = gpm * max_slots * ((batch && batch->pair) ? 2 : 1);  // upper bound in batched mode (pair mode: virtual groups)
     int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
@@ -2060,7 +2067,8 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
                              const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
                              size_t x_stride,
                              float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
-                             int32_t whole_groups, const void *w_stack_up, const void *extra_w_up, dflash_stream_t stream) {
+                             int32_t whole_groups, const void *w_stack_up, const void *extra_w_up, int32_t tiled,
+                             dflash_stream_t stream) {
     if (n_in % DFL_QK_K || n_in <= 0 || n_out <= 0 || n_rows < 1 || n_rows > 16 || max_slots < 1)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_q4k_batched: bad shape");
     if (reinterpret_cast<uintptr_t>(w_stack) % 16 || reinterpret_cast<uintptr_t>(extra_w) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16 ||
@@ -2079,7 +2087,7 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
     bt.x_stride = x_stride;
     bt.y_stride = y_stride;
     bt.whole_groups = whole_groups;
-    return launch_q4k(ctx, w_stack, x, x_type, y, n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt, max_slots);
+    return launch_q4k(ctx, w_stack, x, x_type, y, n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt, max_slots, tiled != 0);
 }
 
 namespace {

@@ -502,11 +502,13 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT,
                         "moe: a mixture-of-experts layer needs router, gate/up/down_exps, shexp_gate and the shared expert's gate/up/down");
     const int et = L.gate_exps.type;
-    if (et != L.up_exps.type || (et != DFLASH_TYPE_Q4_K && et != DFLASH_TYPE_Q6_K && et != DFLASH_TYPE_Q8_0))
+    const bool tiled = et == DFLASH_TYPE_Q4_K_TILED;  // every expert matrix repacked on its own (stack stride = tiled size)
+    if (et != L.up_exps.type || (et != DFLASH_TYPE_Q4_K && et != DFLASH_TYPE_Q6_K && et != DFLASH_TYPE_Q8_0 && !tiled))
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: expert weight type %d", et);
     const int dt = L.down_exps.type;
-    if (dt != DFLASH_TYPE_Q4_K && dt != DFLASH_TYPE_Q6_K && dt != DFLASH_TYPE_Q8_0)
-        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: expert weight type %d", dt);
+    if ((dt != DFLASH_TYPE_Q4_K && dt != DFLASH_TYPE_Q6_K && dt != DFLASH_TYPE_Q8_0 && dt != DFLASH_TYPE_Q4_K_TILED) ||
+        (dt == DFLASH_TYPE_Q4_K_TILED) != tiled)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: expert weight types %d / %d (tiled stacks go together)", et, dt);
     const size_t rb_in = dflash_row_bytes(et, H), rb_dn = dflash_row_bytes(dt, fe);
     if (rb_in == 0 || rb_dn == 0) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "moe: row sizes do not fit the block size");
 
@@ -514,11 +516,13 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     if (rc) return rc;
     if (E > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: %d experts (at most 1024)", E);
     static const bool per_slot_forced = getenv("DFLASH_MOE_PERSLOT") != nullptr;  // read once per process
-    const bool batched = et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K && H % DFL_QK_K == 0 && fe % DFL_QK_K == 0 &&
+    const bool batched = (tiled || (et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K)) && H % DFL_QK_K == 0 && fe % DFL_QK_K == 0 &&
                          !per_slot_forced;
-    // the shared expert rides along as one more slot of the batched GEMMs when it has the experts' shape
-    const bool folded_shared = batched && fs == fe && L.gate.type == DFLASH_TYPE_Q4_K && L.up.type == DFLASH_TYPE_Q4_K &&
-                               L.down.type == DFLASH_TYPE_Q4_K;
+    if (tiled && !batched) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: tiled expert stacks need the batched path");
+    // the shared expert rides along as one more slot of the batched GEMMs when it has the experts' shape (and order)
+    const bool folded_shared = batched && fs == fe && L.gate.type == et && L.up.type == et && L.down.type == et;
+    const size_t stride_in = tiled ? dflash_q4k_tiled_bytes(H, fe) : static_cast<size_t>(fe) * rb_in;
+    const size_t stride_dn = tiled ? dflash_q4k_tiled_bytes(fe, H) : static_cast<size_t>(H) * rb_dn;
     const size_t route_lds = static_cast<size_t>(17) * E * sizeof(float);
     if (route_lds > 48 * 1024) {
         if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(moe_route_kernel), 17 * 1024 * sizeof(float)))
@@ -540,13 +544,13 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         const size_t per_slot = static_cast<size_t>(16) * fe;
         // gate and up of every selected expert in one launch, silu(gate) * up applied to the tiles
         // while they are still in registers
-        if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, static_cast<size_t>(fe) * rb_in, fold ? L.gate.data : nullptr, s.ids,
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, stride_in, fold ? L.gate.data : nullptr, s.ids,
                                        s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, per_slot, H, fe, n, 1,
-                                       L.up_exps.data, fold ? L.up.data : nullptr, st)))
+                                       L.up_exps.data, fold ? L.up.data : nullptr, tiled ? 1 : 0, st)))
             return rc;
-        if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, static_cast<size_t>(H) * rb_dn, fold ? L.down.data : nullptr, s.ids,
+        if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, stride_dn, fold ? L.down.data : nullptr, s.ids,
                                        s.n_distinct, max_slots, s.gate_out, DFLASH_TYPE_F32, per_slot, s.eo,
-                                       static_cast<size_t>(16) * H, fe, H, n, 1, nullptr, nullptr, st)))
+                                       static_cast<size_t>(16) * H, fe, H, n, 1, nullptr, nullptr, tiled ? 1 : 0, st)))
             return rc;
     } else {
         {

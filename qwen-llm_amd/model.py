@@ -9,6 +9,7 @@ numpy arrays (GGUF quant blocks as uint8 rows), uploaded once and used in place.
 from __future__ import annotations
 
 import ctypes as C
+import os
 from dataclasses import asdict, dataclass
 
 import numpy as np
@@ -320,7 +321,7 @@ class _Uploader:
         self.torch = _torch()
         self.device = device
         self.ctx = ctx
-        self.tiled = tiled and ctx is not None
+        self.tiled = tiled and ctx is not None and not os.environ.get("DFLASH_NO_TILED")  # (the variable: for A/B runs)
         self.keep = []
 
     _BLOCK_BYTES = {12: 144, 14: 210}
@@ -400,8 +401,9 @@ class TargetModel:
     def __init__(self, ctx: Context, cfg: ModelConfig, weights: dict, adjacent: bool = True, tiled: bool = True):
         """``adjacent``: place each layer's wq/wk/wv and gate/up back to back in device memory (one GEMM each).
         ``tiled``: repack the Q4_K matrices that only the few-row GEMM reads (attention projections, a dense layer's
-        FFN, the output head) into the library's tiled order at upload; expert stacks, a mixture layer's shared
-        expert (the batched expert kernel reads it in row order) and the embedding table stay in GGUF row order."""
+        FFN, the output head; a mixture layer's expert stacks and shared expert when they are all Q4_K with row counts
+        that are multiples of 256) into the library's tiled order at upload; the embedding table and the router stay
+        in GGUF row order."""
         self.ctx, self.cfg = ctx, cfg
         up = _Uploader(f"cuda:{ctx.device}", ctx, tiled)
         self._up = up
@@ -411,6 +413,15 @@ class TargetModel:
         shape = {"wq": (qd, H), "wk": (kvd, H), "wv": (kvd, H), "wo": (H, qd)}
         if dense:
             shape.update({"gate": (cfg.ffn, H), "up": (cfg.ffn, H), "down": (H, cfg.ffn)})
+        elif cfg.ffn_expert % 256 == 0 and H % 256 == 0 and cfg.ffn_shared % 256 == 0:
+            # a stack whose members have a multiple of 256 rows tiles as ONE matrix (tile groups never straddle
+            # experts); the three stacks and the shared expert go together, or the batched kernel declines
+            E, fe, fs = cfg.n_expert, cfg.ffn_expert, cfg.ffn_shared
+            moe_shape = {"gate_exps": (E * fe, H), "up_exps": (E * fe, H), "down_exps": (E * H, fe),
+                         "gate": (fs, H), "up": (fs, H), "down": (H, fs)}
+            first = weights["layers"][0] if weights["layers"] else {}
+            if all(first.get(k) is not None and int(first[k][0]) == TYPE_Q4_K for k in moe_shape):
+                shape.update(moe_shape)
         for il, Lw in enumerate(weights["layers"]):
             L = self._layers[il]
             for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
