@@ -323,6 +323,7 @@ class _Uploader:
         self.ctx = ctx
         self.tiled = tiled and ctx is not None and not os.environ.get("DFLASH_NO_TILED")  # (the variable: for A/B runs)
         self.keep = []
+        self.n_tiled = 0  # uploads that went into the tiled order
 
     _BLOCK_BYTES = {12: 144, 14: 210}
 
@@ -362,6 +363,7 @@ class _Uploader:
         if tile_shape is not None and self.tiled and int(qtype) == TYPE_Q4_K:
             t = self.ctx.repack_q4k_tiled(t, tile_shape[1], tile_shape[0])
             qtype = TYPE_Q4_K_TILED
+            self.n_tiled += 1
         self.keep.append(t)
         return QTensorC(int(qtype), 0, t.data_ptr())
 
@@ -387,6 +389,7 @@ class _Uploader:
                 and all(ts is not None and ts[0] % 256 == 0 for ts in tile_shapes)):
             whole = self.ctx.repack_q4k_tiled(whole, tile_shapes[0][1], sum(ts[0] for ts in tile_shapes))
             qtype = TYPE_Q4_K_TILED
+            self.n_tiled += 1
         self.keep.append(whole)
         out, off = [], 0
         for f in flats:
@@ -440,6 +443,11 @@ class TargetModel:
 
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self._up.keep)
+
+    @property
+    def tiled_tensors(self) -> int:
+        """Number of uploads (single matrices, fused sets, expert stacks) held in the tiled order."""
+        return self._up.n_tiled
 
 
 class VerifyOutput:

@@ -65,6 +65,27 @@ def test_moe_128_experts_verify_matches_oracle(ctx, oracle, weights):
     sess.close()
 
 
+def test_tiled_expert_stacks_are_bit_identical_to_row_order(ctx, weights):
+    """The expert stacks and the shared expert of this shape (768 and 2048 rows per expert: multiples of 256) are
+    uploaded in the tiled order; that is a permutation of whole blocks read by the same kernel with the same split
+    of work, so every output bit equals the row-order upload's, for a full block and for a ragged one."""
+    tiled = dfl.TargetModel(ctx, C5, weights)
+    rows = dfl.TargetModel(ctx, C5, weights, tiled=False)
+    assert tiled.tiled_tensors > 0 and rows.tiled_tensors == 0
+    rng = np.random.default_rng(3)
+    s_t, s_r = dfl.Session(ctx, tiled, 64, TAPS), dfl.Session(ctx, rows, 64, TAPS)
+    pos = 0
+    for n in (16, 5, 1):
+        blk = rng.integers(0, C5.vocab, n).tolist()
+        a = s_t.encode_packed_verify_layer_major(blk, pos, want_logits=True)
+        b = s_r.encode_packed_verify_layer_major(blk, pos, want_logits=True)
+        assert np.array_equal(a.hidden_capture.cpu().numpy(), b.hidden_capture.cpu().numpy()), f"hidden n={n}"
+        assert np.array_equal(a.logits.cpu().numpy(), b.logits.cpu().numpy()), f"logits n={n}"
+        pos += n
+    s_t.close()
+    s_r.close()
+
+
 def test_generate_on_the_moe_shape_equals_serial_greedy(ctx, weights):
     """MoE target + drafter in one loop at the end-to-end widths: every emitted token is the target's serial greedy
     decode through the same kernels, through full accepts, partial accepts and rollbacks."""
