@@ -106,7 +106,8 @@ __global__ void __launch_bounds__(64 * MAXW)
     attn_split_kernel(const TQ *__restrict__ q, const _Float16 *__restrict__ k_cache,
                       const _Float16 *__restrict__ vt_cache, float *__restrict__ part_o, float *__restrict__ part_ml,
                       int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int n_rows, int n_q, int n_kv,
-                      int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window) {
+                      int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window,
+                      int split_stride) {
     constexpr int KS = HD / 32;       // k-steps of the score product
     constexpr int DT = HD / 16;       // 16-dim tiles of the output
     constexpr int CH = HD / 8;        // 16-byte chunks per key row
@@ -119,8 +120,10 @@ __global__ void __launch_bounds__(64 * MAXW)
     const int n = lane & 15, g = lane >> 4;
     const int group = n_q / n_kv;
     const int kvh = blockIdx.y;
-    const int split = blockIdx.x;
-    const int head0 = kvh * group + wave * HPW;  // this wave serves heads head0 .. head0 + HPW - 1
+    // blockIdx.x = split + split_stride * (part of the GQA group this workgroup serves); split_stride is a multiple
+    // of 8, so the workgroups that read one chunk of keys are dispatched to the same XCD and share its L2 copy
+    const int split = blockIdx.x % split_stride;
+    const int head0 = kvh * group + ((blockIdx.x / split_stride) * n_waves + wave) * HPW;  // this wave serves heads head0 .. head0 + HPW - 1
     if (ctx_len_dev) ctx_len = *ctx_len_dev;
     const int64_t n_pos = ctx_len + n_rows;
     const int64_t chunk = attn_chunk(n_pos, want, min_chunk);
@@ -433,7 +436,7 @@ __global__ void __launch_bounds__(256) transpose_v_kernel(const _Float16 *__rest
 template <int HD, typename TQ>
 int32_t launch_split(dflash_ctx *ctx, dim3 grid, int threads, hipStream_t st, const void *q, const _Float16 *k, const _Float16 *vt,
                   float *po, float *pml, int64_t ctx_len, const int32_t *ctx_len_dev, int n_rows, int n_q, int n_kv,
-                  int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window) {
+                  int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window, int split_stride) {
     const size_t lds = static_cast<size_t>(kAttnBufs) * 2 * (32 * HD / 8) * sizeof(half8_t);
 #define DFL_ATTN_LAUNCH(MAXW, HPW)                                                                                  \
     do {                                                                                                            \
@@ -442,7 +445,7 @@ int32_t launch_split(dflash_ctx *ctx, dim3 grid, int threads, hipStream_t st, co
         attn_split_kernel<HD, TQ, MAXW, HPW><<<grid, threads / HPW, lds, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, \
                                                                               ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
                                                                               vt_stride, want, min_chunk, scale,    \
-                                                                              full_block, window);                  \
+                                                                              full_block, window, split_stride);    \
     } while (0)
     // one head per wave: two (HPW = 2) halve the LDS reads per head but measured slower on MI355X
     // (fewer waves to hide the per-stage dependency chain)
@@ -492,22 +495,33 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int group = n_q / n_kv;
-    // with ctx_len_dev the context length is read on the device (ctx_len is then only an upper
-    // bound): everything sized here is sized for the whole cache
-    const int64_t n_pos = ctx_len_dev ? kv_capacity : ctx_len + n_rows;
+    // with ctx_len_dev the context length is read on the device: everything sized here is then sized for the
+    // largest context of the bucket
+    const int64_t bucket = dfl_attn_bucket(ctx_len + n_rows);
+    const int64_t n_pos = ctx_len_dev ? std::min<int64_t>(kv_capacity, 2 * bucket - 1) : ctx_len + n_rows;
 
-    // KV splits: enough workgroups to cover the chip once or twice, chunks a multiple of 32 keys
-    // and at least 128 keys long (a split costs a partial tile per head and row)
-    int per_cu = n_pos >= 16384 ? 2 : 1;  // short contexts: fewer splits, fewer partial tiles to merge
-    int64_t min_chunk = 128;
+    // KV splits: enough workgroups to cover the chip once or twice, chunks a multiple of 32 keys and at least
+    // min_chunk keys long (a split costs a partial tile per head and row).  The policy is a function of the
+    // bucket alone.
+    int per_cu = bucket >= 16384 ? 2 : 1;  // short contexts: fewer splits, fewer partial tiles to merge
+    int64_t min_chunk = bucket >= 8192 ? 128 : 64;
+    // A workgroup serves hw heads of a GQA group (one wave each).  What a workgroup moves is its chunk of K and V,
+    // its heads' queries and their partial outputs, and one CU takes in only 20-30 KB per microsecond: at short
+    // contexts, where whole groups would leave most CUs without a workgroup, the group is divided until the chip
+    // is covered (the chunk is then read by group / hw workgroups, of one XCD).
+    int hw = group;
+    while (hw % 2 == 0 && static_cast<int64_t>(n_kv) * (group / hw) * ((bucket + min_chunk - 1) / min_chunk) < ctx->n_cu) hw /= 2;
     // tuning knobs, read once per process
     static const int env_per_cu = [] { const char *e = getenv("DFLASH_ATTN_PER_CU"); return e ? atoi(e) : 0; }();
     static const int env_min_chunk = [] { const char *e = getenv("DFLASH_ATTN_MIN_CHUNK"); return e ? atoi(e) : 0; }();
+    static const int env_hw = [] { const char *e = getenv("DFLASH_ATTN_HW"); return e ? atoi(e) : 0; }();
     if (env_per_cu > 0) per_cu = env_per_cu;
     if (env_min_chunk > 0) min_chunk = env_min_chunk;
+    if (env_hw > 0 && group % env_hw == 0) hw = env_hw;
     if (per_cu < 1) per_cu = 1;
     if (min_chunk < 32) min_chunk = 32;
-    const int want = static_cast<int>((static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv - 1) / n_kv);
+    const int n_parts = group / hw;  // workgroups per (chunk, KV head)
+    const int want = static_cast<int>((static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv * n_parts - 1) / (n_kv * n_parts));
     // most splits any context up to n_pos can have
     const int n_splits = ctx_len_dev
                              ? static_cast<int>(std::min<int64_t>(want, (n_pos + min_chunk - 1) / min_chunk))
@@ -535,8 +549,9 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     if (const char *e = getenv("DFLASH_DBG_VT_STRIDE")) vt_stride = atoi(e);  // timing experiment only: wrong results
 #endif
     if (n_splits > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: %d KV splits", n_splits);
-    const dim3 grid(n_splits, n_kv);
-    const int threads = 64 * group;
+    const int split_stride = (n_splits + 7) / 8 * 8;
+    const dim3 grid(split_stride * n_parts, n_kv);
+    const int threads = 64 * hw;
     const _Float16 *k = static_cast<const _Float16 *>(k_cache);
     int32_t rc = DFLASH_OK;
     {
@@ -544,10 +559,12 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 #define DFL_ATTN(HD)                                                                                              \
     if (q_type == DFLASH_TYPE_F32)                                                                                \
         rc = launch_split<HD, float>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
-                                     vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window);    \
+                                     vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window,     \
+                                     split_stride);                                                               \
     else                                                                                                          \
         rc = launch_split<HD, _Float16>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, \
-                                        n_kv, vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window)
+                                        n_kv, vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window, \
+                                        split_stride)
         if (head_dim == 64) {
             DFL_ATTN(64);
         } else if (head_dim == 128) {

@@ -32,6 +32,7 @@ struct dflash_ctx {
     // launch into (the caller's may be the legacy default stream, which cannot be captured) and
     // the two events that order it against the caller's stream
     bool graphs = false;
+    bool capturing = false;     // the launches being enqueued go into a graph: position-dependent values come from device memory
     bool draft_graphs = false;  // graph replay of the drafter's block forward (measured: no faster than direct launches)
     hipStream_t gstream = nullptr;
     hipEvent_t g_in = nullptr, g_out = nullptr;
@@ -123,9 +124,18 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_l
 
 // dflash_attn_verify_block with the drafter's masks: full_block != 0 lets every row see the whole
 // block (non-causal), window > 0 keeps only keys with |distance| < window.  ctx_len_dev != null:
-// the context length is read from that device word when the kernels run (ctx_len is then only
-// checked as an upper bound, launches are sized for the whole cache), so that the call can sit
-// in a captured graph that is replayed at other positions.
+// the context length is read from that device word when the kernels run, so that the call can sit
+// in a captured graph that is replayed at other positions.  How the keys are cut into chunks and
+// the heads into workgroups depends on dfl_attn_bucket(ctx_len + n_rows) only, and with ctx_len_dev
+// the launches are sized for the largest context of that bucket: a captured call stays valid, and
+// bit-identical to a direct one, at every context of the bucket it was captured in (a graph key
+// must therefore include the bucket).
+// Lower bound of the power-of-two range [b, 2 b) that holds n_pos visible positions (at least 256).
+inline int64_t dfl_attn_bucket(int64_t n_pos) {
+    int64_t b = 256;
+    while (2 * b <= n_pos) b *= 2;
+    return b;
+}
 int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,

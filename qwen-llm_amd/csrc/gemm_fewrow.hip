@@ -455,7 +455,12 @@ __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, const Q4KBatch &bt
 // than this second launch, 22.7 / 27.9 / 16.3 us per call against 21.8 / 20.7 / 12.8 us on the three
 // M = 16 projection shapes: the contributors sit on different XCDs, so the chain store -> count -> load
 // crosses to memory three times at the tail of the kernel; with device-scope fences instead, each of which
-// writes back and invalidates an XCD's whole L2, it is nine times slower.)
+// writes back and invalidates an XCD's whole L2, it is nine times slower.  Leaving the sum to the kernel that
+// reads Y inside the model (the q/k norm + RoPE kernel adding seven or eight partial tiles per element as it
+// loads, the residual + RMSNorm kernel sixteen) is slower as well: 7.8 us instead of 5.0 + 4.0 for the former
+// with its 320 waves, 11.7 instead of 5.4 + 3.9 for the latter with its 16 workgroups (a CU takes in only
+// 20-30 KB per microsecond, so a narrow kernel that reads 8-16 times the data loses more than the launch it
+// saves); a 40-layer verify took 4.77 ms instead of 4.70 ms with the first alone.)
 template <int kWaves>
 __global__ void __launch_bounds__(256)
     q4k_reduce_kernel(const float *__restrict__ partials, float *__restrict__ y, int n_out, int nb, int n_rows,

@@ -542,9 +542,10 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
             packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
             L.k_norm, kc, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, packed ? s->pk + q_dim + kv_dim : s->v,
             packed ? tot : kv_dim, vtc, s->capacity);
-        // the context length is read from pos[0] on the device: the same launches serve every position
+        // under capture the context length is read from pos[0] on the device: the same launches then serve every
+        // position of the bucket
         if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity, scale,
-                                 s->attn, st, 0, 0, s->pos)))
+                                 s->attn, st, 0, 0, ctx->capturing ? s->pos : nullptr)))
             return rc;
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
         // x += mix first; a mixture-of-experts layer also gets its shared-expert gate from here
@@ -634,7 +635,8 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
         const uintptr_t outs[4] = {reinterpret_cast<uintptr_t>(hidden_capture), reinterpret_cast<uintptr_t>(lg),
                                    reinterpret_cast<uintptr_t>(am), reinterpret_cast<uintptr_t>(gp)};
         key = hash_bytes(outs, sizeof(outs), key);
-        const int32_t shape[2] = {n, n_taps};
+        // (the attention launches are cut by the bucket of the context length: see dfl_attn_block)
+        const int64_t shape[3] = {n, n_taps, dfl_attn_bucket(start + n)};
         key = hash_bytes(shape, sizeof(shape), key);
         if (n_taps > 0) key = hash_bytes(tap_layers, sizeof(int32_t) * n_taps, key);
     }
@@ -644,7 +646,9 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
         // second call of this shape: capture it
         hipGraph_t graph = nullptr;
         DFL_HIP_CHECK(ctx, hipStreamBeginCapture(ctx->gstream, hipStreamCaptureModeThreadLocal));
+        ctx->capturing = true;
         rc = verify_enqueue(ctx, model, s, n, start, tap_layers, n_taps, hidden_capture, lg, am, gp, ctx->gstream);
+        ctx->capturing = false;
         const hipError_t end = hipStreamEndCapture(ctx->gstream, &graph);
         if (rc) {
             if (graph) (void)hipGraphDestroy(graph);
@@ -951,11 +955,11 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                 packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k,
                 L.q_norm, L.k_norm, k16, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, packed ? s->pk + q_dim + kv_dim : s->v,
                 packed ? tot : kv_dim, vt16, s->cap16);
-            // (context length = pos[0], read on the device: the launch does not depend on it, so a captured graph
-            // of the block stays valid as the context grows; chunking, and so the result, is the same either way)
+            // (under capture the context length is pos[0], read on the device: the launches then serve every context
+            // of the bucket; chunking, and so the result, is the same either way)
             if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, k16, vt16, 1, s->ctx_len, N, c.n_q, c.n_kv, hd, s->cap16,
                                      1.0f / sqrtf(static_cast<float>(hd)), s->attn, st, c.causal ? 0 : 1,
-                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, s->pos)))
+                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, ctx->capturing ? s->pos : nullptr)))
                 return rc;
         } else {
             qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, q_dim, s->k, kv_dim, s->q, s->k, L.q_norm, L.k_norm,
@@ -1028,6 +1032,8 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                                    reinterpret_cast<uintptr_t>(head->output_norm), reinterpret_cast<uintptr_t>(lg),
                                    reinterpret_cast<uintptr_t>(am), static_cast<uintptr_t>(skip_selector_walk)};
         key = hash_bytes(ptrs, sizeof(ptrs), key);
+        const int64_t bucket = dfl_attn_bucket(s->ctx_len + c.block_size);  // (see dfl_attn_block)
+        key = hash_bytes(&bucket, sizeof(bucket), key);
         for (int il = 0; il < c.n_layers; il++) {
             const dflash_draft_layer &L = head->layers[il];
             const uintptr_t lp[9] = {reinterpret_cast<uintptr_t>(L.wq.data), reinterpret_cast<uintptr_t>(L.wk.data),
@@ -1043,7 +1049,9 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
     if (use_graph && exec_it == s->graphs.end() && s->graphs.size() < 8 && s->graph_seen[key]++ >= 1) {
         hipGraph_t graph = nullptr;
         DFL_HIP_CHECK(ctx, hipStreamBeginCapture(ctx->gstream, hipStreamCaptureModeThreadLocal));
+        ctx->capturing = true;
         rc = enqueue(ctx->gstream);
+        ctx->capturing = false;
         const hipError_t end = hipStreamEndCapture(ctx->gstream, &graph);
         if (rc) {
             if (graph) (void)hipGraphDestroy(graph);

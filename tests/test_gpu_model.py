@@ -378,14 +378,16 @@ def test_graph_replay_is_bit_identical_to_launch_by_launch(ctx, target):
     """The packed verify replayed from a captured graph (second and later calls of a shape) against
     the same calls made launch by launch: logits, hidden capture, argmax and gap bit for bit, at
     moving positions, with a rollback and single-row calls in between and other GPU work and
-    synchronisations between the replays."""
+    synchronisations between the replays.  The context grows past 256 positions on the way: the attention launches
+    are cut by the power-of-two range of the context length, so a graph serves one such range and the next range
+    captures its own."""
     import torch
 
     model, _ = target
     rng = np.random.default_rng(21)
-    cap = 320
-    blocks = [rng.integers(0, C1.vocab, 16).tolist() for _ in range(8)]
-    singles = rng.integers(0, C1.vocab, 8).tolist()
+    cap = 448
+    blocks = [rng.integers(0, C1.vocab, 16).tolist() for _ in range(24)]
+    singles = rng.integers(0, C1.vocab, 24).tolist()
 
     def run(graphs):
         ctx.set_graphs(graphs)
@@ -405,6 +407,7 @@ def test_graph_replay_is_bit_identical_to_launch_by_launch(ctx, target):
             outs.append((o.logits.cpu().numpy(), o.hidden_capture.cpu().numpy(), o.argmax.cpu().numpy(), o.gap.cpu().numpy()))
             del o
             pos += 1
+        assert pos > 288
         replays = sess.graph_replays
         return outs, replays
 
@@ -414,7 +417,7 @@ def test_graph_replay_is_bit_identical_to_launch_by_launch(ctx, target):
     finally:
         ctx.set_graphs(False)
     assert r0 == 0
-    assert r1 >= 8, f"only {r1} of 16 calls were graph replays"
+    assert r1 >= 36, f"only {r1} of 48 calls were graph replays"
     for i, (a, b) in enumerate(zip(eager, replay)):
         for x, y, name in zip(a, b, ("logits", "hidden", "argmax", "gap")):
             assert np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
