@@ -6,16 +6,20 @@
 // :1206-1235, RNG :1621-1670), crates/qwen-llm/src/metal_dflash/accept.rs:76-183 (block decision,
 // CPU-only in the reference).
 //
-// Everything here is HBM-bound streaming over [rows][vocab] f32 plus O(top_k) arithmetic:
-//  * a row is cut into chunks of 8192 tokens so that rows x chunks workgroups cover the chip;
-//    each workgroup streams its chunk once with coalesced loads;
+// Everything here is HBM-bound streaming over [rows][vocab] f32 plus O(top_k) arithmetic, and, at one block per
+// call, a chain of latencies (a dependent launch, a trip to memory for what another XCD wrote, an LDS read) rather
+// than a volume of work:
+//  * a row is cut into chunks (8192 tokens for the argmax, 16384 for the top-k selection) so that rows x chunks
+//    workgroups cover the chip in one round; each workgroup streams its chunk once with coalesced loads;
 //  * order decisions use the reference's integer keys (descending f32 total order above ascending
 //    token id), so the selected candidates and their order are exact, not approximately sorted;
-//  * top-k of a chunk: the k-th best of the 1024 per-thread bests bounds every winner, so only
-//    the <= 8k elements of the k winning threads are sorted (bitonic, in LDS);
-//  * everything that feeds a comparison with a uniform draw is f64 and sequential, in the order
-//    of the reference's loops: one thread walks the <= 64 candidates of a row, one thread walks
-//    the rows of the block.
+//  * top-k of a chunk: the k-th best of the 1024 per-thread bests bounds every winner, so only the elements of the
+//    k winning threads are ranked; ranks come from counting (keys are distinct), not from sorting networks in LDS,
+//    whose every step is a workgroup barrier;
+//  * everything that feeds a comparison with a uniform draw is f64 and added in the order of the reference's
+//    loops; what is independent per candidate (conversions, exponentials) is done a candidate per lane;
+//  * a block with dense draft proposals is three launches: selection of both logit tensors, the rows' chains
+//    together with the draft rows' tile sums, the decision (written straight to pinned host memory).
 #include "common.h"
 #include "sampler_chain.h"
 #include "accept_wide.h"
@@ -25,7 +29,11 @@
 
 namespace {
 
-constexpr int kChunk = 8192;       // tokens per workgroup
+constexpr int kChunk = 8192;       // tokens per workgroup of the argmax / top-2 kernel
+// Tokens per workgroup of the top-k selection.  A 16-row block with dense draft proposals is 31 rows: at 8192 tokens
+// per workgroup that is 589 workgroups of 1024 threads, more than the chip holds at once (two per CU), and the kernel
+// takes two rounds of a workgroup whose time is mostly latency; at 16384 it is 310 and one round.
+constexpr int kSelChunk = 16384;
 constexpr int kSelThreads = 1024;  // 8 tokens per thread
 constexpr int kMaxRows = 16;
 constexpr uint64_t kNoKey = ~0ull;
@@ -135,17 +143,113 @@ __device__ uint64_t block_min_u64(uint64_t v, uint64_t *sh) {
     return r;
 }
 
+// Ascending sort of one key per lane over the wave (bitonic network of 21 compare-exchange steps between lanes: no
+// LDS arrays, no barriers).
+__device__ __forceinline__ uint64_t wave_sort_u64(uint64_t v) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int size = 2; size <= 64; size <<= 1) {
+#pragma unroll
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            const uint32_t lo = __shfl_xor(static_cast<uint32_t>(v), stride, 64), hi = __shfl_xor(static_cast<uint32_t>(v >> 32), stride, 64);
+            const uint64_t o = (static_cast<uint64_t>(hi) << 32) | lo;
+            const bool lower = (lane & stride) == 0, ascending = (lane & size) == 0;
+            const uint64_t mn = v < o ? v : o, mx = v < o ? o : v;
+            v = (lower == ascending) ? mn : mx;
+        }
+    }
+    return v;
+}
+
+// Minimum of a key over the wave, in every lane: data-parallel-primitive moves within rows of 16 lanes (shift right
+// by 1, 2, 4, 8: lane 15 of a row then holds the row's minimum), then lane 15 of rows 0 and 2 into rows 1 and 3, then
+// lane 31 into rows 2 and 3; lane 63 has the result.  Lanes without a source read the identity.  No LDS round trips.
+__device__ __forceinline__ uint64_t wave_min_u64(uint64_t v) {
+#define DFL_MIN_STEP(ctrl, row_mask)                                                                                     \
+    do {                                                                                                                 \
+        const unsigned lo = __builtin_amdgcn_update_dpp(0xffffffffu, static_cast<unsigned>(v), ctrl, row_mask, 0xf, false);       \
+        const unsigned hi = __builtin_amdgcn_update_dpp(0xffffffffu, static_cast<unsigned>(v >> 32), ctrl, row_mask, 0xf, false); \
+        const uint64_t o = (static_cast<uint64_t>(hi) << 32) | lo;                                                       \
+        v = o < v ? o : v;                                                                                               \
+    } while (0)
+    DFL_MIN_STEP(0x111, 0xf);  // row_shr:1
+    DFL_MIN_STEP(0x112, 0xf);  // row_shr:2
+    DFL_MIN_STEP(0x114, 0xf);  // row_shr:4
+    DFL_MIN_STEP(0x118, 0xf);  // row_shr:8
+    DFL_MIN_STEP(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+    DFL_MIN_STEP(0x143, 0xc);  // row_bcast:31 into rows 2 and 3
+#undef DFL_MIN_STEP
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(v), 63);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(v >> 32), 63);
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+// The k smallest keys, in order, of n_lists <= 64 ascending lists of k keys each (list l at base + l * stride; missing
+// keys are kNoKey, at the end), by ONE wave: lane l holds the head of list l, a step takes the minimum of the heads
+// and advances the list it came from (keys are distinct).  Returns the k-th; with `out`, out[0 .. k) gets them all.
+// (Measured in the selection kernel, k = 20: 3.3 us; every published key searching the sixteen lists instead, spread
+// over all 1024 threads, 5.7 us: the waves of a workgroup share four instruction issuers, and the index arithmetic
+// of 5120 searches costs more than twenty dependent steps of one wave.)
+__device__ __forceinline__ uint64_t wave_merge_lists(const uint64_t *base, int n_lists, int stride, int k, uint64_t *out) {
+    const int lane = threadIdx.x & 63;
+    const bool own = lane < n_lists;
+    const uint64_t *list = base + (own ? lane : 0) * stride;
+    int pos = 0;
+    uint64_t head = own ? list[0] : kNoKey;
+    uint64_t next = (own && k > 1) ? list[1] : kNoKey;  // fetched one step ahead of its use
+    uint64_t m = kNoKey;
+    for (int step = 0; step < k; step++) {
+        m = wave_min_u64(head);
+        if (out && lane == 0) out[step] = m;
+        if (own && head == m && m != kNoKey) {
+            head = next;
+            pos++;
+            next = pos + 1 < k ? list[pos + 1] : kNoKey;
+        }
+    }
+    return m;
+}
+
+// below[j] = number of keys below x[j] in the ascending list of 1 <= n <= kMaxK keys at base + off[j], four binary
+// searches in lockstep: a probe is an LDS read the next one depends on, and a thread that runs its searches one
+// after the other spends its time waiting for them.  step0 = the largest power of two <= n.
+__device__ __forceinline__ void count_below4(const uint64_t *base, const int (&off)[4], int n, int step0, const uint64_t (&x)[4],
+                                             int (&below)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) below[j] = 0;
+    for (int step = step0; step >= 1; step >>= 1) {
+        uint64_t v[4];
+        int probe[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            probe[j] = below[j] + step;
+            v[j] = base[off[j] + (probe[j] <= n ? probe[j] : n) - 1];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) below[j] = (probe[j] <= n && v[j] < x[j]) ? probe[j] : below[j];
+    }
+}
+
 // K == 1 fast path is the greedy / draft-max case: only the minimum key is needed.
-__global__ void __launch_bounds__(kSelThreads)
-    select_chunk_kernel(const float *__restrict__ logits, int64_t vocab, int64_t stride, int k,
-                        ChunkOut *__restrict__ out, bool nan_is_candidate) {
-    __shared__ uint64_t sk[kSelThreads];
-    __shared__ uint64_t cand[8 * kMaxK];
+//
+// K > 1, without a sort over the workgroup (a bitonic network in LDS is one workgroup barrier per step, 91 steps
+// here): every wave sorts its 64 per-thread bests between its lanes and publishes the first k; the k-th best of all
+// 1024 per-thread bests (it bounds every winner of the chunk) is the k-th key of the merge of the sixteen published
+// lists, which wave 0 runs; the at most 16 k elements at or below that bound are then ranked by counting the
+// candidates below each, and a candidate of rank r < k is output r.  Keys are distinct (the token id is in the low
+// bits), so ranks are too.
+__device__ __forceinline__ void select_chunk_body(const float *__restrict__ logits, int64_t vocab, int64_t stride, int k,
+                                                  ChunkOut *__restrict__ out, bool nan_is_candidate, int row) {
+    __shared__ uint64_t sk[kSelThreads];  // k == 1: scratch of the minimum; else [16 waves][kMaxK] published bests
+    __shared__ uint64_t cand[(kSelChunk / kSelThreads) * kMaxK];
+    __shared__ uint64_t outk[kMaxK];
+    __shared__ uint64_t tau_sh;
+    __shared__ int rank_sh[kSelThreads];  // [16 waves][kMaxK] published bests, then the candidates (at most as many)
     __shared__ int cnt;
     __shared__ int nan_sh;
-    const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    const int chunk = blockIdx.x, tid = threadIdx.x;
     const float *x = logits + row * stride;
-    uint64_t keys[kChunk / kSelThreads];
+    uint64_t keys[kSelChunk / kSelThreads];
     uint64_t best = kNoKey;
     int nan_first = kNoNan;
     if (tid == 0) {
@@ -153,8 +257,8 @@ __global__ void __launch_bounds__(kSelThreads)
         nan_sh = kNoNan;
     }
 #pragma unroll
-    for (int j = 0; j < kChunk / kSelThreads; j++) {
-        int64_t i = static_cast<int64_t>(chunk) * kChunk + j * kSelThreads + tid;
+    for (int j = 0; j < kSelChunk / kSelThreads; j++) {
+        int64_t i = static_cast<int64_t>(chunk) * kSelChunk + j * kSelThreads + tid;
         uint64_t key = kNoKey;
         if (i < vocab) {
             float v = x[i];
@@ -180,22 +284,60 @@ __global__ void __launch_bounds__(kSelThreads)
         return;
     }
     // k-th best of the per-thread bests bounds every winner of the chunk
-    sk[tid] = best;
-    bitonic_sort(sk, kSelThreads);
-    const uint64_t tau = sk[k - 1];
+    const int lane = tid & 63, wave = tid >> 6;
+    const uint64_t sorted = wave_sort_u64(best);
+    if (lane < k) sk[wave * kMaxK + lane] = sorted;
+    if (tid < kMaxK) outk[tid] = kNoKey;
+    rank_sh[tid] = 0;
+    __syncthreads();
+    // the k-th best of the sixteen published lists: wave 0 merges them (fewer than k keys in all: kNoKey, and every
+    // key of the chunk is a candidate)
+    if (wave == 0) {
+        const uint64_t kth = wave_merge_lists(sk, kSelThreads / 64, kMaxK, k, nullptr);
+        if (lane == 0) tau_sh = kth;
+    }
+    __syncthreads();
+    const uint64_t tau = tau_sh;
     if (best <= tau && best != kNoKey) {
 #pragma unroll
-        for (int j = 0; j < kChunk / kSelThreads; j++)
+        for (int j = 0; j < kSelChunk / kSelThreads; j++)
             if (keys[j] <= tau && keys[j] != kNoKey) cand[atomicAdd(&cnt, 1)] = keys[j];
     }
     __syncthreads();
-    const int n_cand = cnt;  // <= 8 k
-    int n_sort = 2;
-    while (n_sort < n_cand) n_sort <<= 1;
-    for (int i = n_cand + tid; i < n_sort; i += kSelThreads) cand[i] = kNoKey;
-    bitonic_sort(cand, n_sort);
-    if (tid < k) o->keys[tid] = tid < n_sort ? cand[tid] : kNoKey;
+    const int n_cand = cnt;  // <= 16 k <= kSelThreads
+    if (n_cand > 0) {
+        // candidate i = tid % n_cand counts the candidates below it in slice tid / n_cand of the list
+        const int slices = kSelThreads / n_cand, i = tid % n_cand, sl = tid / n_cand;
+        if (sl < slices) {
+            const int per = (n_cand + slices - 1) / slices, j0 = sl * per, j1 = min(n_cand, j0 + per);
+            const uint64_t key = cand[i];
+            int c = 0;
+            for (int j = j0; j < j1; j++) c += cand[j] < key;
+            if (c) atomicAdd(&rank_sh[i], c);
+        }
+    }
+    __syncthreads();
+    if (tid < n_cand && rank_sh[tid] < k) outk[rank_sh[tid]] = cand[tid];
+    __syncthreads();
+    if (tid < k) o->keys[tid] = outk[tid];
     if (tid == 0) o->nan_first = nan_sh;
+}
+
+__global__ void __launch_bounds__(kSelThreads)
+    select_chunk_kernel(const float *__restrict__ logits, int64_t vocab, int64_t stride, int k,
+                        ChunkOut *__restrict__ out, bool nan_is_candidate) {
+    select_chunk_body(logits, vocab, stride, k, out, nan_is_candidate, blockIdx.y);
+}
+
+// Two row sets in one launch: rows [0, n_a) of a (best k_a keys of every chunk), then the rows of b (best key).
+__global__ void __launch_bounds__(kSelThreads)
+    select_pair_kernel(const float *__restrict__ a, int n_a, int k_a, ChunkOut *__restrict__ out_a, const float *__restrict__ b,
+                       ChunkOut *__restrict__ out_b, int64_t vocab, int64_t stride) {
+    const int row = blockIdx.y;
+    if (row < n_a)
+        select_chunk_body(a, vocab, stride, k_a, out_a, false, row);
+    else
+        select_chunk_body(b, vocab, stride, 1, out_b, false, row - n_a);
 }
 
 // The dense proposal's side of a row: its largest draft logit (scaled) and NaN / no-candidate errors.
@@ -218,57 +360,109 @@ __device__ void merge_draft_side(const ChunkOut *__restrict__ draft_chunks, int 
     }
 }
 
-// One workgroup per row: merge the chunk lists, order the best k, run the chain.
-__global__ void __launch_bounds__(kSelThreads)
-    row_merge_kernel(const ChunkOut *__restrict__ chunks, int n_chunks, const ChunkOut *__restrict__ draft_chunks,
-                     ChainCfg cfg, RowDist *__restrict__ rows, int32_t *__restrict__ greedy_out, bool draft_only) {
+// One workgroup per row: merge the chunk lists, order the best k, run the chain (wave 0, a candidate per lane).
+__device__ __forceinline__ void row_merge_body(const ChunkOut *__restrict__ chunks, int n_chunks,
+                                               const ChunkOut *__restrict__ draft_chunks, const ChainCfg &cfg,
+                                               RowDist *__restrict__ rows, int32_t *__restrict__ greedy_out, bool draft_only,
+                                               int row) {
     __shared__ uint64_t sk[2 * kSelThreads];
-    __shared__ double chain_l[kMaxK], chain_w[kMaxK];
-    __shared__ int chain_tok[kMaxK];
-    const int row = blockIdx.x, tid = threadIdx.x;
+    const int tid = threadIdx.x;
     RowDist *d = rows + row;
     if (draft_only) {  // the target side of these rows was filled by the wide chain
         if (tid == 0) merge_draft_side(draft_chunks, n_chunks, row, cfg, d);
         return;
     }
+    // The chunks' lists are ascending: the rank of a key among all of them is the sum, over the lists, of the keys
+    // below it (binary searches); the keys of rank < k, in rank order, are the row's candidates, best first.
     const int k = cfg.k;
     const int n_in = n_chunks * k;  // <= 2048, checked on the host
-    int n_sort = 2;
-    while (n_sort < n_in) n_sort <<= 1;
-    for (int i = tid; i < n_sort; i += kSelThreads) {
-        uint64_t key = kNoKey;
-        if (i < n_in) key = chunks[row * n_chunks + i / k].keys[i % k];
-        sk[i] = key;
+    __shared__ uint64_t lists[2 * kSelThreads];
+    __shared__ int rank_sh[2 * kSelThreads];
+    __shared__ uint64_t red[kSelThreads / 64];
+    if (tid < kMaxK) sk[tid] = kNoKey;
+    uint64_t mine = kNoKey;
+    for (int i = tid; i < n_in; i += kSelThreads) {
+        const uint64_t key = chunks[row * n_chunks + i / k].keys[i % k];
+        lists[i] = key;
+        rank_sh[i] = 0;
+        mine = key < mine ? key : mine;
     }
-    bitonic_sort(sk, n_sort);
-    if (tid != 0) return;
-    d->n_keep = 0;
-    d->err = 0;
-    d->err_index = -1;
-    d->total = 0.0;
-    d->d_err = 0;
-    d->d_err_index = -1;
+    if (k == 1) {
+        mine = block_min_u64(mine, red);
+        if (tid == 0) sk[0] = mine;
+    } else {
+        __syncthreads();
+        // (key, list) pairs over all threads: a thread's searches are independent of each other
+        // (consecutive threads: consecutive keys against the same list, so that a wave's probes fall on different
+        // banks and its additions on different counters)
+        const int step0 = 1 << (31 - __clz(k));
+        for (int p0 = tid; p0 < n_in * n_chunks; p0 += 4 * kSelThreads) {
+            int off[4], slot[4], below[4];
+            uint64_t key[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int p = p0 + j * kSelThreads;
+                const bool live = p < n_in * n_chunks;
+                const int c = live ? p / n_in : 0;
+                slot[j] = live ? p - c * n_in : 0;
+                off[j] = c * k;
+                key[j] = live ? lists[slot[j]] : 0;  // (nothing is below key 0)
+            }
+            count_below4(lists, off, k, step0, key, below);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (below[j] && key[j] != kNoKey) atomicAdd(&rank_sh[slot[j]], below[j]);
+        }
+        __syncthreads();
+        for (int i = tid; i < n_in; i += kSelThreads)
+            if (lists[i] != kNoKey && rank_sh[i] < k) sk[rank_sh[i]] = lists[i];
+    }
+    __syncthreads();
+    if (tid >= 64) {
+        // the dense proposal's side is independent of the target's: the first lane of the second wave takes it
+        if (tid == 64 && draft_chunks) merge_draft_side(draft_chunks, n_chunks, row, cfg, d);
+        return;
+    }
     int nan_first = kNoNan;
-    for (int c = 0; c < n_chunks; c++) {
+    for (int c = tid; c < n_chunks; c += 64) {
         int nf = chunks[row * n_chunks + c].nan_first;
         nan_first = nf < nan_first ? nf : nan_first;
     }
-    if (greedy_out) greedy_out[row] = nan_first != kNoNan ? ~nan_first : key_token(sk[0]);
+    for (int off = 32; off > 0; off >>= 1) nan_first = min(nan_first, __shfl_xor(nan_first, off, 64));
+    if (tid == 0) {
+        d->n_keep = 0;
+        d->err = 0;
+        d->err_index = -1;
+        d->total = 0.0;
+        if (!draft_chunks) {
+            d->d_err = 0;
+            d->d_err_index = -1;
+        }
+        if (greedy_out) greedy_out[row] = nan_first != kNoNan ? ~nan_first : key_token(sk[0]);
+    }
     if (nan_first != kNoNan) {
-        d->err = DFLASH_ERR_NAN_LOGIT;
-        d->err_index = nan_first;
+        if (tid == 0) {
+            d->err = DFLASH_ERR_NAN_LOGIT;
+            d->err_index = nan_first;
+        }
     } else if (cfg.temperature == 0.0f) {
         // greedy target: one-hot on the total-order argmax (sampling.rs:391-400)
-        d->n_keep = 1;
-        d->total = 1.0;
-        d->tokens[0] = key_token(sk[0]);
-        d->weights[0] = 1.0;
+        if (tid == 0) {
+            d->n_keep = 1;
+            d->total = 1.0;
+            d->tokens[0] = key_token(sk[0]);
+            d->weights[0] = 1.0;
+        }
     } else {
-        int len = 0;
-        while (len < k && sk[len] != kNoKey) len++;
-        run_chain(sk, len, cfg, d, ChainScratch{chain_l, chain_w, chain_tok});
+        const int len = __popcll(__builtin_amdgcn_ballot_w64(tid < k && sk[tid < k ? tid : 0] != kNoKey));  // (missing keys sort last)
+        run_chain_wave(sk, len, cfg, d);
     }
-    if (draft_chunks) merge_draft_side(draft_chunks, n_chunks, row, cfg, d);
+}
+
+__global__ void __launch_bounds__(kSelThreads)
+    row_merge_kernel(const ChunkOut *__restrict__ chunks, int n_chunks, const ChunkOut *__restrict__ draft_chunks,
+                     ChainCfg cfg, RowDist *__restrict__ rows, int32_t *__restrict__ greedy_out, bool draft_only) {
+    row_merge_body(chunks, n_chunks, draft_chunks, cfg, rows, greedy_out, draft_only, blockIdx.x);
 }
 
 // top-16 output from the merged order
@@ -289,31 +483,51 @@ __global__ void __launch_bounds__(kSelThreads)
     }
 }
 
-// Dense proposal: tile sums of exp(d/T - max/T) in the fixed shape: 1024-token tiles, slot t
-// holds ((e[4t]+e[4t+1])+e[4t+2])+e[4t+3], then a halving tree over the 256 slots.
-__global__ void __launch_bounds__(256) dense_tile_sum_kernel(const float *__restrict__ draft, int64_t vocab,
-                                                             int64_t stride, float temperature,
-                                                             const RowDist *__restrict__ rows,
-                                                             double *__restrict__ tile_sums) {
-    __shared__ double slot[256];
-    const int row = blockIdx.y, tile = blockIdx.x, t = threadIdx.x;
-    const double T = static_cast<double>(temperature);
-    const double mx = rows[row].d_max_scaled;
+// The rows' chains and the dense proposal's tile sums in one launch (neither needs the other; both need only the
+// chunk selection): workgroups [0, n_rows) are row_merge_kernel's, the rest take eight 1024-token tiles each of draft
+// row (workgroup - n_rows) / blocks_per_row.  A tile sum is the sum of exp(d/T - max/T) in a fixed shape: slot t of
+// a tile holds ((e[4t]+e[4t+1])+e[4t+2])+e[4t+3], then a halving tree over the 256 slots; max is the row's largest
+// draft logit, which every tile workgroup takes from the chunk minima itself.
+__global__ void __launch_bounds__(kSelThreads)
+    rows_and_tiles_kernel(const ChunkOut *__restrict__ chunks, int n_chunks, const ChunkOut *__restrict__ draft_chunks, ChainCfg cfg,
+                          RowDist *__restrict__ rows, int n_rows, bool draft_only, const float *__restrict__ draft, int64_t vocab,
+                          int64_t stride, int n_tiles, int blocks_per_row, double *__restrict__ tile_sums) {
+    if (static_cast<int>(blockIdx.x) < n_rows) {
+        row_merge_body(chunks, n_chunks, draft_chunks, cfg, rows, nullptr, draft_only, blockIdx.x);
+        return;
+    }
+    __shared__ double slot[4][256];
+    __shared__ uint64_t red[kSelThreads / 64];
+    const int b = blockIdx.x - n_rows, row = b / blocks_per_row, q = threadIdx.x >> 8, t = threadIdx.x & 255;
+    uint64_t best = kNoKey;
+    for (int c = threadIdx.x; c < n_chunks; c += kSelThreads) {
+        const uint64_t key = draft_chunks[row * n_chunks + c].keys[0];
+        best = key < best ? key : best;
+    }
+    best = block_min_u64(best, red);
+    const double T = static_cast<double>(cfg.draft_temperature);
+    const double mx = static_cast<double>(key_logit(best)) / T;  // merge_draft_side's d_max_scaled
     const float *x = draft + row * stride;
-    const int64_t base = static_cast<int64_t>(tile) * 1024 + 4 * t;
-    double acc = 0.0;
+    // (eight tiles per workgroup, two per quarter: with four, a 15-row block is more workgroups than the chip holds
+    // at once)
+    for (int half = 0; half < 2; half++) {
+        const int tile = (b - row * blocks_per_row) * 8 + 4 * half + q;
+        const int64_t base = static_cast<int64_t>(tile) * 1024 + 4 * t;
+        double acc = 0.0;
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-        int64_t i = base + e;
-        double v = (i < vocab) ? exp(static_cast<double>(x[i]) / T - mx) : 0.0;
-        acc = (e == 0) ? v : acc + v;
+        for (int e = 0; e < 4; e++) {
+            int64_t i = base + e;
+            double v = (tile < n_tiles && i < vocab) ? exp(static_cast<double>(x[i]) / T - mx) : 0.0;
+            acc = (e == 0) ? v : acc + v;
+        }
+        __syncthreads();  // (the previous half's sums have been read)
+        slot[q][t] = acc;
+        for (int s = 128; s >= 1; s >>= 1) {
+            __syncthreads();
+            if (t < s) slot[q][t] += slot[q][t + s];
+        }
+        if (t == 0 && tile < n_tiles) tile_sums[row * n_tiles + tile] = slot[q][0];
     }
-    slot[t] = acc;
-    for (int s = 128; s >= 1; s >>= 1) {
-        __syncthreads();
-        if (t < s) slot[t] += slot[t + s];
-    }
-    if (t == 0) tile_sums[row * gridDim.x + tile] = slot[0];
 }
 
 struct DecideArgs {
@@ -372,13 +586,19 @@ struct RowOutcome {
     int32_t draws;       // random draws this row consumes
     int32_t err;         // DFLASH_ERR_* of this row, 0 if none
     int64_t err_index;
+    // a rejected row under a stochastic proposal: its correction token is still to be drawn from the residual
+    // distribution (residual_pick, by the whole wave, for the one row the walk stops at)
+    int32_t need_residual;
+    int32_t residual_draw;  // index of the uniform draw the pick uses
+    double prop_total;
 };
 
 // One row of accept.rs:147-183 with the couplings of sampling.rs:692-790.  A row that is reached has seen only
 // accepting rows before it, and an accepting row consumes exactly one draw (none when greedy): row r therefore
 // starts at draw r whatever the rows before it held, which is what lets every row be evaluated at once.
-__device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int row, const double *p_total) {
-    RowOutcome o = {0, 0, 0, 0, -1};
+__device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int row, const double *p_total,
+                                 const float *draft_tok_logit) {
+    RowOutcome o = {0, 0, 0, 0, -1, 0, 0, 0.0};
     const int n_drafts = a.n_tokens - 1;
     const bool greedy = a.temperature == 0.0f;
     const RowDist &rd = rows[row];
@@ -442,8 +662,8 @@ __device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int r
         prop_total = p_total[row];
         if (!o.err && !(isfinite(prop_total) && prop_total > 0.0)) o.err = DFLASH_ERR_NO_CANDIDATES;
         if (!o.err) {
-            prop_tok_w = exp(static_cast<double>(a.draft[row * a.draft_stride + draft]) / static_cast<double>(a.draft_temperature) -
-                             rd.d_max_scaled);
+            // (draft_tok_logit[row] = a.draft[row][draft], fetched ahead)
+            prop_tok_w = exp(static_cast<double>(draft_tok_logit[row]) / static_cast<double>(a.draft_temperature) - rd.d_max_scaled);
             if (!(isfinite(prop_tok_w) && prop_tok_w > 0.0)) {
                 o.err = DFLASH_ERR_MISSING_PROPOSAL_TOKEN;
                 o.err_index = draft;
@@ -464,96 +684,175 @@ __device__ RowOutcome decide_row(const DecideArgs &a, const RowDist *rows, int r
     if (a.uniforms[draws++] < acceptance) {
         o.acc = 1;
     } else {
-        // residual weights max(p_i - q_i, 0) in the target's order (sampling.rs:752-790): summed first, then walked
-        // again for the pick; the second pass recomputes the same values, so no per-candidate array is needed
-        auto residual_at = [&](int i) {
-            const double p = dv.weight(i) / rd.total;
-            double q;
-            if (a.mode == 1) {
-                const int32_t ti = dv.token(i);
-                double qs = -0.0;
-                for (int j = 0; j < n_pc; j++)
-                    if (pc[j].token == ti) qs += pc[j].weight;
-                q = qs / prop_total;
-            } else {
-                q = exp(static_cast<double>(a.draft[row * a.draft_stride + dv.token(i)]) / static_cast<double>(a.draft_temperature) -
-                        rd.d_max_scaled) /
-                    prop_total;
-            }
-            return fmax(p - q, 0.0);
-        };
-        double residual_total = 0.0;
-        for (int i = 0; i < rd.n_keep; i++) residual_total += residual_at(i);
-        if (!(isfinite(residual_total) && residual_total > 0.0)) {
-            o.err = DFLASH_ERR_NO_CANDIDATES;
-            return o;
-        }
-        const double x = a.uniforms[draws++] * residual_total;
-        int pick = rd.n_keep - 1;
-        double cumulative = 0.0;
-        for (int i = 0; i < rd.n_keep; i++) {
-            cumulative += residual_at(i);
-            if (x < cumulative) {
-                pick = i;
-                break;
-            }
-        }
-        o.token = dv.token(pick);
+        // the correction token comes from the residual distribution: one more draw
+        o.need_residual = 1;
+        o.residual_draw = draws++;
+        o.prop_total = prop_total;
     }
     o.draws = draws - draws0;
     return o;
 }
 
+// The correction token of rejected row `row`: residual weights max(p_i - q_i, 0) in the target's order
+// (sampling.rs:752-790), summed first, then walked again for the pick; the second pass recomputes the same values,
+// so no per-candidate array is needed.  By the whole wave: lane j computes the weight of candidate base + j (one f64
+// exponential each under a dense proposal, the expensive part), and the sums add those values in candidate order,
+// one addition after the other.
+__device__ void residual_pick(const DecideArgs &a, const RowDist *rows, int row, RowOutcome &o, const float *draft_logit_of) {
+    const int lane = threadIdx.x & 63;
+    const RowDist &rd = rows[row];
+    const DistView dv = {&rd, a.wide_keys ? a.wide_keys + row * a.wide_stride : nullptr,
+                         a.wide_w ? a.wide_w + row * a.wide_stride : nullptr};
+    const dflash_weighted_candidate *pc = a.mode == 1 ? a.prop_cands + a.prop_offsets[row] : nullptr;
+    const int n_pc = a.mode == 1 ? a.prop_counts[row] : 0;
+    const double prop_total = o.prop_total;
+    auto residual_at = [&](int i) {
+        const double p = dv.weight(i) / rd.total;
+        double q;
+        if (a.mode == 1) {
+            const int32_t ti = dv.token(i);
+            double qs = -0.0;
+            for (int j = 0; j < n_pc; j++)
+                if (pc[j].token == ti) qs += pc[j].weight;
+            q = qs / prop_total;
+        } else {
+            // (draft_logit_of: the row's candidates' draft logits, fetched ahead; else they are read here)
+            const float dl = draft_logit_of ? draft_logit_of[i] : a.draft[row * a.draft_stride + dv.token(i)];
+            q = exp(static_cast<double>(dl) / static_cast<double>(a.draft_temperature) - rd.d_max_scaled) / prop_total;
+        }
+        return fmax(p - q, 0.0);
+    };
+    const int n_keep = rd.n_keep;
+    double residual_total = 0.0;
+    for (int base = 0; base < n_keep; base += 64) {
+        const double r = base + lane < n_keep ? residual_at(base + lane) : 0.0;
+        const int m = min(64, n_keep - base);
+        for (int j = 0; j < m; j++) residual_total += chain_bcast(r, j);
+    }
+    if (!(isfinite(residual_total) && residual_total > 0.0)) {
+        o.err = DFLASH_ERR_NO_CANDIDATES;
+        return;
+    }
+    const double x = a.uniforms[o.residual_draw] * residual_total;
+    int pick = n_keep - 1;
+    double cumulative = 0.0;
+    bool found = false;
+    for (int base = 0; base < n_keep && !found; base += 64) {
+        const double r = base + lane < n_keep ? residual_at(base + lane) : 0.0;
+        const int m = min(64, n_keep - base);
+        for (int j = 0; j < m; j++) {
+            cumulative += chain_bcast(r, j);
+            if (x < cumulative) {
+                pick = base + j;
+                found = true;
+                break;
+            }
+        }
+    }
+    o.token = dv.token(pick);
+}
+
 // Thread r evaluates row r (all rows at once); thread 0 then walks the outcomes in order exactly as the serial
 // loop of accept.rs:147-183 does: rows behind the first rejection, stop or error are never looked at.
-__global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__ out) {
+__global__ void __launch_bounds__(64) decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__ out) {
+    constexpr int kStage = 256;  // tile sums per row and round
     __shared__ double p_total[kMaxRows];
     __shared__ RowOutcome outcome[kMaxRows + 1];
     // the rows' distributions are walked element by element: they are copied to LDS once, coalesced
     __shared__ RowDist rows_sh[kMaxRows];
-    static_assert(sizeof(RowDist) % 4 == 0, "copied as words");
-    {
-        const uint32_t *src = reinterpret_cast<const uint32_t *>(a.rows);
-        uint32_t *dst = reinterpret_cast<uint32_t *>(rows_sh);
-        const int n_words = a.n_tokens * static_cast<int>(sizeof(RowDist) / 4);
-        for (int i = threadIdx.x; i < n_words; i += blockDim.x) dst[i] = src[i];
-    }
+    __shared__ double staged[kMaxRows][kStage];
+    __shared__ float draft_tok_logit[kMaxRows];
+    __shared__ float resid_logit[kMaxRows][kMaxK];
+    static_assert(sizeof(RowDist) % 8 == 0, "copied as double words");
+    const int tid = threadIdx.x;
     const int n_drafts = a.n_tokens - 1;
-    if (a.mode == 2) {
-        // P = sequential sum of a row's tile sums, in tile order.  The sums come through LDS 64 tiles at a time
-        // (all threads load, coalesced and independent), so that the ordered additions of thread r do not each
-        // wait for a load from memory.
-        __shared__ double staged[kMaxRows][64];
-        double P = 0.0;
-        for (int t0 = 0; t0 < a.n_tiles; t0 += 64) {
-            const int t = t0 + static_cast<int>(threadIdx.x);
-            for (int r = 0; r < n_drafts; r++) staged[r][threadIdx.x] = t < a.n_tiles ? a.tile_sums[r * a.n_tiles + t] : 0.0;
-            __syncthreads();
-            if (static_cast<int>(threadIdx.x) < n_drafts) {
-                const int n = min(64, a.n_tiles - t0);
-                for (int i = 0; i < n; i++) P += staged[threadIdx.x][i];
+    const bool dense = a.mode == 2;
+    // What the kernel reads from memory is written by other XCDs and comes from memory at about two microseconds a
+    // trip: everything whose address is known is requested before anything is waited for (the first round of tile
+    // sums, each draft row's logit of its own draft token, the rows), the candidates' draft logits as soon as the
+    // rows are there, and the arithmetic runs on LDS copies.
+    double tsum[kMaxRows - 1][kStage / 64];
+    float my_logit = 0.0f;
+    if (dense) {
+#pragma unroll
+        for (int r = 0; r < kMaxRows - 1; r++)
+#pragma unroll
+            for (int u = 0; u < kStage / 64; u++) {
+                const int t = u * 64 + tid;
+                tsum[r][u] = (r < n_drafts && t < a.n_tiles) ? a.tile_sums[r * a.n_tiles + t] : 0.0;
             }
-            __syncthreads();
+        if (tid < n_drafts) my_logit = a.draft[tid * a.draft_stride + a.verified[tid + 1]];
+    }
+    {
+        const uint64_t *src = reinterpret_cast<const uint64_t *>(a.rows);
+        uint64_t *dst = reinterpret_cast<uint64_t *>(rows_sh);
+        const int n_words = a.n_tokens * static_cast<int>(sizeof(RowDist) / 8);
+        for (int base = 0; base < n_words; base += 64 * 8) {
+            uint64_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = base + u * 64 + tid < n_words ? src[base + u * 64 + tid] : 0;
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (base + u * 64 + tid < n_words) dst[base + u * 64 + tid] = v[u];
         }
-        if (static_cast<int>(threadIdx.x) < n_drafts) p_total[threadIdx.x] = P;
+    }
+    if (dense) {
+#pragma unroll
+        for (int r = 0; r < kMaxRows - 1; r++)
+#pragma unroll
+            for (int u = 0; u < kStage / 64; u++) staged[r][u * 64 + tid] = tsum[r][u];
+        if (tid < n_drafts) draft_tok_logit[tid] = my_logit;
     }
     __syncthreads();
-    if (static_cast<int>(threadIdx.x) <= n_drafts) outcome[threadIdx.x] = decide_row(a, rows_sh, threadIdx.x, p_total);
+    const bool prefetched = dense && !a.wide_keys;
+    if (prefetched) {
+        float v[kMaxRows - 1];
+#pragma unroll
+        for (int r = 0; r < kMaxRows - 1; r++)
+            v[r] = (r < n_drafts && tid < rows_sh[r].n_keep) ? a.draft[r * a.draft_stride + rows_sh[r].tokens[tid]] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < kMaxRows - 1; r++) resid_logit[r][tid] = v[r];
+    }
+    if (dense) {
+        // P = sequential sum of a row's tile sums, in tile order, by thread r from the LDS copies
+        double P = 0.0;
+        for (int t0 = 0; t0 < a.n_tiles; t0 += kStage) {
+            if (t0 > 0) {  // further rounds (vocabularies above 262144 tokens)
+                __syncthreads();
+                for (int r = 0; r < n_drafts; r++)
+                    for (int u = 0; u < kStage / 64; u++) {
+                        const int t = t0 + u * 64 + tid;
+                        staged[r][u * 64 + tid] = t < a.n_tiles ? a.tile_sums[r * a.n_tiles + t] : 0.0;
+                    }
+                __syncthreads();
+            }
+            if (tid < n_drafts) {
+                const int n = min(kStage, a.n_tiles - t0);
+                for (int i = 0; i < n; i++) P += staged[tid][i];
+            }
+        }
+        if (tid < n_drafts) p_total[tid] = P;
+    }
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    dflash_accept_decision d;
-    memset(&d, 0, sizeof(d));
-    d.err_row = -1;
-    d.err_index = -1;
+    if (tid <= n_drafts) outcome[tid] = decide_row(a, rows_sh, tid, p_total, draft_tok_logit);
+    __syncthreads();
+    // The walk, by every lane alike (the workgroup is one wave; everything it reads is uniform): at the row it stops
+    // at, a rejected draft's correction token is drawn by the whole wave.  The decision is put together in LDS and
+    // leaves as one coalesced store: `out` may be host memory, where every separate store is a transaction over the
+    // bus.
+    __shared__ dflash_accept_decision d_sh;
+    static_assert(sizeof(dflash_accept_decision) % 4 == 0, "copied as words");
     int accepted = 0, draws = 0, carry_kind = DFLASH_CARRY_NONE, stop = DFLASH_STOP_NONE, carry_token = 0;
-    int err = 0;
+    int err = 0, err_row = -1;
+    int64_t err_index = -1;
     for (;;) {
         const int row = accepted;
-        const RowOutcome &o = outcome[row];
+        RowOutcome o = outcome[row];
+        if (!o.err && o.need_residual) residual_pick(a, rows_sh, row, o, prefetched ? resid_logit[row] : nullptr);
         if (o.err) {
             err = o.err;
-            d.err_index = o.err_index;
-            d.err_row = row;
+            err_index = o.err_index;
+            err_row = row;
             break;
         }
         draws += o.draws;
@@ -568,7 +867,7 @@ __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__
             break;
         }
         const int32_t draft = a.verified[row + 1];
-        d.accepted_drafts[accepted++] = draft;
+        accepted++;
         if (in_list(a.stop_ids, a.n_stop, draft)) {
             stop = DFLASH_STOP_EOS;
             break;
@@ -578,22 +877,29 @@ __global__ void decide_kernel(DecideArgs a, dflash_accept_decision *__restrict__
             break;
         }
     }
-    if (err) {
-        const int er = d.err_row;
-        const int64_t ei = d.err_index;
+    if (threadIdx.x == 0) {
+        dflash_accept_decision &d = d_sh;
         memset(&d, 0, sizeof(d));
-        d.err_row = er;
-        d.err_index = ei;
-        d.err_code = err;
-    } else {
-        d.n_accepted = accepted;
-        d.carry_kind = carry_kind;
-        d.carry_token = carry_token;
-        d.stop_reason = stop;
-        d.retain_input_count = 1 + accepted - (stop != DFLASH_STOP_NONE ? 1 : 0);
-        d.draws_used = draws;
+        d.err_row = err_row;
+        d.err_index = err_index;
+        if (err) {
+            d.err_code = err;
+        } else {
+            for (int i = 0; i < accepted; i++) d.accepted_drafts[i] = a.verified[i + 1];
+            d.n_accepted = accepted;
+            d.carry_kind = carry_kind;
+            d.carry_token = carry_token;
+            d.stop_reason = stop;
+            d.retain_input_count = 1 + accepted - (stop != DFLASH_STOP_NONE ? 1 : 0);
+            d.draws_used = draws;
+        }
     }
-    *out = d;
+    __syncthreads();
+    {
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(&d_sh);
+        uint32_t *dst = reinterpret_cast<uint32_t *>(out);
+        for (int i = threadIdx.x; i < static_cast<int>(sizeof(dflash_accept_decision) / 4); i += blockDim.x) dst[i] = src[i];
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -690,7 +996,7 @@ int32_t dflash_argmax_greedy(dflash_ctx *ctx, const float *logits, int32_t n_row
     if (rc) return rc;
     if (!idx) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "argmax_greedy: null output");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
+    const int n_chunks = static_cast<int>((vocab + kSelChunk - 1) / kSelChunk);
     if (n_chunks > 2 * kSelThreads) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "argmax_greedy: vocabulary too large");
     size_t off = 0;
     ChunkOut *chunks = dfl_ws_take<ChunkOut>(ctx, &off, sizeof(ChunkOut) * n_rows * n_chunks);
@@ -712,7 +1018,7 @@ int32_t dflash_top16(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64
     if (rc) return rc;
     if (!ids || !vals) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "top16: null output");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
+    const int n_chunks = static_cast<int>((vocab + kSelChunk - 1) / kSelChunk);
     if (n_chunks * 16 > 2 * kSelThreads) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "top16: vocabulary too large");
     size_t off = 0;
     ChunkOut *chunks = dfl_ws_take<ChunkOut>(ctx, &off, sizeof(ChunkOut) * n_rows * n_chunks);
@@ -829,7 +1135,7 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
     const dflash_sampling_config &sc = sampler->cfg;
     int64_t k_eff = (sc.temperature == 0.0f) ? 1 : ((sc.top_k == 0 || static_cast<int64_t>(sc.top_k) >= vocab) ? vocab : static_cast<int64_t>(sc.top_k));
     const bool wide = k_eff > kMaxK;  // top_k = 0 or a large top_k: full order by radix sort (accept_wide.hip)
-    const int n_chunks = static_cast<int>((vocab + kChunk - 1) / kChunk);
+    const int n_chunks = static_cast<int>((vocab + kSelChunk - 1) / kSelChunk);
     if (!wide && n_chunks * k_eff > 2 * kSelThreads)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "accept_prefix: vocabulary %lld x top_k %lld too large", static_cast<long long>(vocab), static_cast<long long>(k_eff));
 
@@ -878,20 +1184,25 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
         if (wide) {
             if (const int32_t rc_ = dfl_accept_wide_rows(ctx, target_logits, n_tokens, vocab, vocab, cfg, rows, &off, &wide_keys, &wide_w, st))
                 return rc_;
+            if (dense) select_chunk_kernel<<<dim3(n_chunks, n_drafts), kSelThreads, 0, st>>>(draft_logits, vocab, vocab, 1, dchunks, false);
+        } else if (dense) {
+            select_pair_kernel<<<dim3(n_chunks, n_tokens + n_drafts), kSelThreads, 0, st>>>(target_logits, n_tokens, cfg.k, chunks,
+                                                                                         draft_logits, dchunks, vocab, vocab);
         } else {
             select_chunk_kernel<<<dim3(n_chunks, n_tokens), kSelThreads, 0, st>>>(target_logits, vocab, vocab, cfg.k, chunks, false);
         }
-        if (dense)
-            select_chunk_kernel<<<dim3(n_chunks, n_drafts), kSelThreads, 0, st>>>(draft_logits, vocab, vocab, 1, dchunks, false);
-        if (!wide)
-            row_merge_kernel<<<n_tokens, kSelThreads, 0, st>>>(chunks, n_chunks, dense ? dchunks : nullptr, cfg, rows, nullptr, false);
-        else if (dense)
-            row_merge_kernel<<<n_drafts, kSelThreads, 0, st>>>(chunks, n_chunks, dchunks, cfg, rows, nullptr, true);
+        // the rows' chains and, for dense proposals, the tile sums of the draft rows: one launch
+        if (dense) {
+            const int blocks_per_row = (n_tiles + 7) / 8;
+            const int n_row_wgs = wide ? n_drafts : n_tokens;  // (wide: the chain has run; only the draft side is merged)
+            rows_and_tiles_kernel<<<n_row_wgs + n_drafts * blocks_per_row, kSelThreads, 0, st>>>(
+                chunks, n_chunks, dchunks, cfg, rows, n_row_wgs, wide, draft_logits, vocab, vocab, n_tiles, blocks_per_row, tile_sums);
+        } else if (!wide) {
+            row_merge_kernel<<<n_tokens, kSelThreads, 0, st>>>(chunks, n_chunks, nullptr, cfg, rows, nullptr, false);
+        }
         a.wide_keys = wide_keys;
         a.wide_w = wide_w;
         a.wide_stride = vocab;
-        if (mode == 2 && n_drafts > 0)
-            dense_tile_sum_kernel<<<dim3(n_tiles, n_drafts), 256, 0, st>>>(draft_logits, vocab, vocab, draft_temperature, rows, tile_sums);
         a.n_tokens = n_tokens;
         a.n_stop = n_stop;
         a.mode = mode;
@@ -906,11 +1217,16 @@ int32_t dflash_accept_prefix(dflash_ctx *ctx, const int32_t *verified, int32_t n
         a.n_tiles = n_tiles;
         a.temperature = sc.temperature;
         a.draft_temperature = draft_temperature;
-        decide_kernel<<<1, 64, 0, st>>>(a, d_out);
+        // the decision goes straight to the context's pinned page when the device can address it (one copy less
+        // between the last kernel and the host)
+        static_assert(sizeof(dflash_accept_decision) <= DFL_PINNED_BYTES, "the decision is read back through the pinned page");
+        void *pinned_dev = nullptr;
+        const bool direct = ctx->pinned && hipHostGetDevicePointer(&pinned_dev, ctx->pinned, 0) == hipSuccess && pinned_dev;
+        if (!direct) (void)hipGetLastError();
+        decide_kernel<<<1, 64, 0, st>>>(a, direct ? static_cast<dflash_accept_decision *>(pinned_dev) : d_out);
+        DFL_HIP_CHECK(ctx, hipGetLastError());
+        if (!direct) DFL_HIP_CHECK(ctx, hipMemcpyAsync(ctx->pinned, d_out, sizeof(*out), hipMemcpyDeviceToHost, st));
     }
-    DFL_HIP_CHECK(ctx, hipGetLastError());
-    static_assert(sizeof(dflash_accept_decision) <= DFL_PINNED_BYTES, "the decision is read back through the pinned page");
-    DFL_HIP_CHECK(ctx, hipMemcpyAsync(ctx->pinned, d_out, sizeof(*out), hipMemcpyDeviceToHost, st));
     DFL_HIP_CHECK(ctx, hipStreamSynchronize(st));
     memcpy(out, ctx->pinned, sizeof(*out));
     if (out->err_code) {

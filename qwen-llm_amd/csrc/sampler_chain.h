@@ -151,6 +151,73 @@ __device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowD
     }
 }
 
+// A lane's double in every lane (src uniform).
+__device__ __forceinline__ double chain_bcast(double v, int src) {
+    const unsigned long long b = static_cast<unsigned long long>(__double_as_longlong(v));
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(b), src);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(b >> 32), src);
+    return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
+
+// run_chain by one whole wave (len <= 64): lane i holds candidate i.  What the reference does element by element
+// without carrying anything from one element to the next (the conversions, the division by the temperature, the
+// exponentials, the filters' comparisons) is done by all lanes at once; every sum that is compared with something is
+// still added in candidate order, one addition after the other, on values that are the same bits as run_chain's.
+// The candidates are in descending logit order, so what min-p and the +inf rule keep is a prefix: its length is a
+// population count.
+__device__ void run_chain_wave(const uint64_t *keys, int len, const ChainCfg &c, RowDist *d) {
+    const int lane = threadIdx.x & 63;
+    double l = lane < len ? static_cast<double>(key_logit(keys[lane])) : 0.0;
+    const int tok = lane < len ? key_token(keys[lane]) : 0;
+    auto fail = [&]() {
+        if (lane == 0) d->err = DFLASH_ERR_NO_CANDIDATES;
+    };
+    if (c.min_p > 0.0f && len > 0) {
+        const double max_logit = chain_bcast(l, 0);
+        if (isfinite(max_logit)) {
+            const double threshold = max_logit + c.ln_min_p;
+            len = __popcll(__builtin_amdgcn_ballot_w64(lane < len && l >= threshold));
+        }
+    }
+    if (len == 0) return fail();
+    if (chain_bcast(l, 0) == INFINITY) len = __popcll(__builtin_amdgcn_ballot_w64(lane < len && l == INFINITY));
+    l = l / static_cast<double>(c.temperature);
+    const int n_inf = __popcll(__builtin_amdgcn_ballot_w64(lane < len && l == INFINITY));
+    double w;
+    if (n_inf > 0) {
+        w = (l == INFINITY) ? 1.0 : 0.0;
+    } else {
+        const double max_logit = chain_bcast(l, 0);
+        if (max_logit == -INFINITY) return fail();
+        w = lane < len ? exp(l - max_logit) : 0.0;
+        if (__builtin_amdgcn_ballot_w64(lane < len && !isfinite(w)) != 0) return fail();
+    }
+    if (c.top_p < 1.0f) {
+        double total = -0.0;
+        for (int i = 0; i < len; i++) total += chain_bcast(w, i);
+        const double target = total * static_cast<double>(c.top_p);
+        double cumulative = 0.0;
+        int keep = 0;
+        for (int i = 0; i < len; i++) {
+            cumulative += chain_bcast(w, i);
+            keep++;
+            if (cumulative >= target) break;
+        }
+        len = keep < 1 ? 1 : keep;
+    }
+    double total_weight = -0.0;
+    for (int i = 0; i < len; i++) total_weight += chain_bcast(w, i);
+    if (!(isfinite(total_weight) && total_weight > 0.0)) return fail();
+    if (lane == 0) {
+        d->n_keep = len;
+        d->total = total_weight;
+    }
+    if (lane < len) {
+        d->tokens[lane] = tok;
+        d->weights[lane] = w;
+    }
+}
+
 // the same with private work arrays
 __device__ void run_chain(const uint64_t *keys, int len, const ChainCfg &c, RowDist *d) {
     double l[kMaxK], w[kMaxK];
