@@ -307,6 +307,45 @@ def test_seeded_trials_small_vocab(ctx, oracle, mode, kind):
     assert lengths[0] > 0 and lengths[1:].sum() > 0  # both outcomes exercised
 
 
+@pytest.mark.parametrize("vocab", [16384 + 5, 2 * 16384 + 63, 3 * 16384])
+@pytest.mark.parametrize("top_k", [2, 20, 64])
+def test_selection_at_chunk_boundaries(ctx, oracle, vocab, top_k):
+    """The top-k selection cuts a row into 16384-token chunks.  Vocabularies whose last chunk holds fewer tokens than
+    k (every one of them is then a candidate of its chunk), exactly fills, or ends one short of a wave; rows whose
+    winners all sit in one chunk, straddle a boundary, or are -inf but for a handful: decisions and sampler state
+    equal the oracle's, dense and deterministic drafts, 40 seeds each."""
+    n, T = 16, 0.7
+    rng = np.random.default_rng(vocab * 131 + top_k)
+    tl, dl = block_inputs(rng, vocab, n)
+    tl[1, :] = -np.inf
+    tl[1, rng.integers(0, vocab, 5)] = rng.standard_normal(5).astype(np.float32)      # fewer finite logits than k
+    tl[2, 16384 - 3:16384 + 3] += 30.0                                                  # winners on both sides of a cut
+    tl[3, vocab - 4:] += 30.0                                                           # winners at the ragged end
+    tl[4, :16384] -= 50.0                                                               # one chunk out of the running
+    dl = (tl[: n - 1] + rng.standard_normal((n - 1, vocab)) * 0.5).astype(np.float32)
+    dl[~np.isfinite(dl)] = -30.0
+    tl_dev, dl_dev = dev(tl), dev(dl)
+    lengths = set()
+    for seed in range(40):
+        r2 = np.random.default_rng(seed)
+        drafts = [int(np.argmax(tl[r])) if r2.random() < 0.8 else int(r2.integers(vocab)) for r in range(n - 1)]
+        toks = [int(r2.integers(vocab))] + drafts
+        for dense in (False, True):
+            gs = dfl.Sampler(temperature=T, top_k=top_k, top_p=0.95, seed=seed, rng_kind=dfl.RNG_PHILOX)
+            os_ = oracle.make_sampler(T, top_k, 0.95, 0.0, seed, dfl.RNG_PHILOX)
+            if dense:
+                rc, od = oracle.decide_accept_prefix_dense(toks, tl, dl, vocab, T, os_, 100, [])
+                gd = ctx.decide_dflash_accept_prefix(toks, tl_dev, vocab, None, gs, 100, [], draft_logits=dl_dev, draft_temperature=T)
+            else:
+                rc, od = oracle.decide_accept_prefix(toks, tl, vocab, None, os_, 100, [])
+                gd = ctx.decide_dflash_accept_prefix(toks, tl_dev, vocab, None, gs, 100, [])
+            assert rc == 0
+            assert gd.key() == od.key(), f"seed {seed} dense {dense}"
+            assert gs.state() == oracle.sampler_state(os_), f"seed {seed} dense {dense}"
+            lengths.add(len(gd.accepted_drafts))
+    assert len(lengths) > 1
+
+
 @pytest.mark.parametrize("kind,n_trials", [(dfl.RNG_PHILOX, 10000), (dfl.RNG_XOSHIRO, 2000)])
 def test_seeded_trials_full_vocab_dense(ctx, oracle, kind, n_trials):
     """Stochastic acceptance at its benchmark size: vocabulary 151936, block 16, target logits N(0, 3), draft = target +
