@@ -174,6 +174,16 @@ def acceptance_section(ctx, with_cpu=True):
     logits_bytes = (2 * n - 1) * vocab * 4
     res = {"vocab": vocab, "block": n, "us_per_block": us, "logits_bytes": logits_bytes,
            "GBps": logits_bytes / (us * 1e-6) / 1e9, "mean_accepted": accepted / 24}
+    # the same block between two HIP events around its kernels (the library's own timer slot for acceptance): without
+    # the launch from an idle GPU and the host's wait for the decision
+    ctx.set_kernel_timing(True)
+    for trial in range(8):
+        samp = dfl.Sampler(temperature=0.7, top_k=20, top_p=0.95, min_p=0.0, seed=100 + trial, rng_kind=dfl.RNG_PHILOX)
+        ctx.decide_dflash_accept_prefix(verified, target, vocab, None, samp, 1000, [], draft_logits=draft, draft_temperature=0.7)
+    ms, count = ctx.kernel_timing(2)
+    ctx.set_kernel_timing(False)
+    if count:
+        res["us_between_events"] = ms * 1e3 / count
     if with_cpu:
         # the oracle's restatement of decide_dflash_accept_prefix + Sampler (one thread per block, as the reference's
         # host code runs it) on the same logits, same samplers
