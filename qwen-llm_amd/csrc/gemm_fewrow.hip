@@ -2009,7 +2009,11 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
 
 namespace {
 
-// The streaming Q6_K kernel (and its split-K reduction) on one matrix.
+// The streaming Q6_K kernel (and its split-K reduction) on one matrix.  (Measured and not kept: for the few-MB
+// attention projections, workgroups of two waves that take the whole K of their 32 rows, as many as there are row
+// groups (160 for a 5120-row q/k/v product, 64 for a 2048-row output projection): no partial tiles and no reduce
+// launch, every test green, but a 40-layer verify took 4.88 instead of 4.71 ms: 8 or 16 dependent stages of one
+// small workgroup are a longer chain than one or two stages on every CU plus the reduce launch.)
 int32_t launch_q6k_stream(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in,
                           int64_t n_out, int32_t n_rows, hipStream_t st) {
     const int nb = static_cast<int>(n_in / DFL_QK_K);
