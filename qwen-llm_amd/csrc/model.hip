@@ -280,6 +280,58 @@ __global__ void kv_to_f16_kernel(const float *__restrict__ k, const float *__res
     if (v_copy) v_copy[static_cast<size_t>(row) * kv_dim + e] = vv;  // dense f32 copy of a V slice
 }
 
+// The drafter's context K/V of up to 16 new columns, every layer in one launch, out of the batched projection
+// pk[layer][col][k heads | v heads]: what qk_norm_rope_kernel (key heads, same arithmetic) and kv_to_f16_kernel do
+// per layer.  blockIdx = (head: keys then values, column, layer); one wave per head.
+struct CtxKvNorms {
+    const float *k_norm[16];  // per layer (may be null)
+};
+__global__ void __launch_bounds__(64)
+    ctx_kv_finish_kernel(const float *__restrict__ pk, int kv_dim, CtxKvNorms norms, float *__restrict__ k_ctx,
+                         float *__restrict__ v_ctx, size_t ctx_layer_stride, _Float16 *__restrict__ k16, _Float16 *__restrict__ vt16,
+                         size_t f16_layer_stride, int64_t cap16, const int32_t *__restrict__ pos, int64_t c0, int n_kv, int hd,
+                         float eps, float theta) {
+    const int head = blockIdx.x, col = blockIdx.y, il = blockIdx.z, lane = threadIdx.x;
+    const float *row = pk + (static_cast<size_t>(il) * 16 + col) * 2 * kv_dim;
+    float *kc = k_ctx + il * ctx_layer_stride + (c0 + col) * kv_dim;
+    float *vc = v_ctx + il * ctx_layer_stride + (c0 + col) * kv_dim;
+    _Float16 *k16l = k16 + il * f16_layer_stride, *vt16l = vt16 + il * f16_layer_stride;
+    if (head >= n_kv) {  // a value head: f32 copy, and the f16 mirror's transposed column
+        const int vh = head - n_kv;
+        for (int i = lane; i < hd; i += 64) {
+            const int e = vh * hd + i;
+            const float vv = row[kv_dim + e];
+            vc[e] = vv;
+            vt16l[static_cast<size_t>(e) * cap16 + c0 + col] = static_cast<_Float16>(vv);
+        }
+        return;
+    }
+    const float *v = row + static_cast<size_t>(head) * hd;
+    const float *w = norms.k_norm[il];
+    const int half = hd / 2;
+    float s = 0.0f;
+    for (int i = lane; i < hd; i += 64) s += v[i] * v[i];
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    const float scale = 1.0f / sqrtf(s / static_cast<float>(hd) + eps);
+    const float p = static_cast<float>(pos[col]);
+    for (int i = lane; i < half; i += 64) {
+        float a = v[i] * scale, b = v[i + half] * scale;
+        if (w) {
+            a *= w[i];
+            b *= w[i + half];
+        }
+        const float freq = p / powf(theta, static_cast<float>(2 * i) / static_cast<float>(hd));
+        float sn, cs;
+        sincosf(freq, &sn, &cs);
+        const float ra = a * cs - b * sn, rb = a * sn + b * cs;
+        const int e = head * hd + i;
+        kc[e] = ra;
+        kc[e + half] = rb;
+        k16l[(c0 + col) * kv_dim + e] = static_cast<_Float16>(ra);
+        k16l[(c0 + col) * kv_dim + e + half] = static_cast<_Float16>(rb);
+    }
+}
+
 template <typename T>
 bool dev_alloc(T **p, size_t count) {
     return hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T) + 256) == hipSuccess;
@@ -384,6 +436,10 @@ struct dflash_draft_session {
     float *g = nullptr, *u = nullptr, *logits = nullptr, *tmp = nullptr;
     float *pk = nullptr;  // [16][max(q_dim + 2 kv_dim, 2 ffn)]: output of a fused q/k/v or gate/up GEMM
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
+    // every layer's context K/V projection as ONE batched GEMM (draft_prepare): its output [layer][16][2 kv_dim],
+    // the list 0 .. n_layers - 1 and its length for the batched kernel
+    float *pk_layers = nullptr;
+    int32_t *layer_ids = nullptr, *n_layers_dev = nullptr;
     // DFlash-2 (MetalDFlashSession conv_buf / conv_dyn_* / topk_* / sel_h, metal_dflash.rs:5144-5155)
     float *conv_buf = nullptr;   // [16][H]
     float *conv_dyn = nullptr;   // [16][2 * kernel * H / group]: one sublayer's coefficients at a time
@@ -724,7 +780,15 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
               dev_alloc(&s->u, 16 * static_cast<size_t>(cfg->ffn)) && dev_alloc(&s->logits, 16 * static_cast<size_t>(vocab)) &&
               dev_alloc(&s->pk, 16 * std::max(q_dim + 2 * kv_dim, 2 * static_cast<size_t>(cfg->ffn))) &&
               dev_alloc(&s->tmp, 16 * std::max(H, kv_dim)) && dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) &&
-              dev_alloc(&s->argmax, 16);
+              dev_alloc(&s->argmax, 16) && dev_alloc(&s->pk_layers, static_cast<size_t>(cfg->n_layers) * 16 * 2 * kv_dim) &&
+              dev_alloc(&s->layer_ids, static_cast<size_t>(cfg->n_layers)) && dev_alloc(&s->n_layers_dev, 1);
+    if (ok) {
+        std::vector<int32_t> ids(static_cast<size_t>(cfg->n_layers));
+        for (int i = 0; i < cfg->n_layers; i++) ids[i] = i;
+        const int32_t n = cfg->n_layers;
+        ok = hipMemcpy(s->layer_ids, ids.data(), ids.size() * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess &&
+             hipMemcpy(s->n_layers_dev, &n, sizeof(n), hipMemcpyHostToDevice) == hipSuccess;
+    }
     if (ok && cfg->conv_kernel_size > 0)
         ok = dev_alloc(&s->conv_buf, 16 * H) &&
              dev_alloc(&s->conv_dyn, 16 * static_cast<size_t>(2) * cfg->conv_kernel_size * (H / cfg->conv_group_size));
@@ -742,7 +806,8 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
 void dflash_draft_session_destroy(dflash_draft_session *s) {
     if (!s) return;
     void *ptrs[] = {s->ctx_raw, s->ctx_h, s->k_ctx, s->v_ctx, s->k16, s->vt16, s->pos_ctx, s->x, s->cur, s->q, s->k, s->v,
-                    s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax, s->pk,
+                    s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax, s->pk, s->pk_layers,
+                    s->layer_ids, s->n_layers_dev,
                     s->conv_buf, s->conv_dyn, s->topk_ids, s->topk_vals, s->sel_h};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -800,8 +865,41 @@ int32_t draft_prepare(dflash_ctx *ctx, const dflash_draft_head *head, dflash_dra
         if ((rc = gemm(ctx, head->fc, s->ctx_raw + c0 * feat, s->tmp, feat, H, m, st))) return rc;
         rms_norm_kernel<<<m, 256, 0, st>>>(s->tmp, nullptr, head->hidden_norm, s->ctx_h + c0 * H, H, c.eps, nullptr, nullptr);
     }
+    // Every layer's K/V projection reads the same rows (ctx_h): when the layers' [wk; wv] pairs are Q4_K matrices
+    // an equal distance apart (the loader put all layers' q/k/v in one allocation), they run as ONE batched GEMM,
+    // whole K per workgroup, and one kernel norms, rotates and scatters all layers' results: 2 launches per 16
+    // columns instead of 4 per layer.
+    bool layers_batched = fast && c.n_layers >= 2 && c.n_layers <= 16 && H % DFL_QK_K == 0 && s->pk_layers;
+    size_t w_stride = 0;
+    if (layers_batched) {
+        const dflash_draft_layer &L0 = head->layers[0];
+        const bool tiled0 = L0.wk.type == DFLASH_TYPE_Q4_K_TILED;
+        layers_batched = (L0.wk.type == DFLASH_TYPE_Q4_K || tiled0) && (!tiled0 || (2 * kv_dim) % 256 == 0);
+        w_stride = static_cast<size_t>(static_cast<const uint8_t *>(head->layers[1].wk.data) - static_cast<const uint8_t *>(L0.wk.data));
+        for (int il = 0; il < c.n_layers && layers_batched; il++) {
+            const dflash_draft_layer &L = head->layers[il];
+            layers_batched = L.wk.type == L0.wk.type && adjacent(L.wk, kv_dim, L.wv, H) && head->layers[1].wk.data > L0.wk.data &&
+                             static_cast<const uint8_t *>(L.wk.data) == static_cast<const uint8_t *>(L0.wk.data) + il * w_stride;
+        }
+        layers_batched = layers_batched && w_stride % 16 == 0;
+    }
+    if (layers_batched) {
+        CtxKvNorms norms = {};
+        for (int il = 0; il < c.n_layers; il++) norms.k_norm[il] = head->layers[il].k_norm;
+        const bool tiled = head->layers[0].wk.type == DFLASH_TYPE_Q4_K_TILED;
+        for (int64_t c0 = s->kv_ready; c0 < s->ctx_len; c0 += 16) {
+            const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
+            if ((rc = dfl_gemm_q4k_batched(ctx, head->layers[0].wk.data, w_stride, nullptr, s->layer_ids, s->n_layers_dev, c.n_layers,
+                                           s->ctx_h + c0 * H, DFLASH_TYPE_F32, 0, s->pk_layers, static_cast<size_t>(16) * 2 * kv_dim, H,
+                                           2 * static_cast<int64_t>(kv_dim), m, 1, nullptr, nullptr, tiled ? 1 : 0, st)))
+                return rc;
+            ctx_kv_finish_kernel<<<dim3(2 * c.n_kv, m, c.n_layers), 64, 0, st>>>(
+                s->pk_layers, static_cast<int>(kv_dim), norms, s->k_ctx, s->v_ctx, static_cast<size_t>(s->capacity) * kv_dim, s->k16,
+                s->vt16, static_cast<size_t>(s->cap16) * kv_dim, s->cap16, s->pos_ctx + c0, c0, c.n_kv, hd, c.eps, c.rope_theta);
+        }
+    }
     const float *pending_resid = nullptr;
-    for (int il = 0; il < c.n_layers; il++) {
+    for (int il = 0; il < c.n_layers && !layers_batched; il++) {
         const dflash_draft_layer &L = head->layers[il];
         float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
         float *vc = s->v_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;

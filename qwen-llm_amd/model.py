@@ -523,6 +523,14 @@ class DraftHead:
         H, qd, kvd = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
         shape = {"wq": (qd, H), "wk": (kvd, H), "wv": (kvd, H), "wo": (H, qd), "gate": (cfg.ffn, H), "up": (cfg.ffn, H),
                  "down": (H, cfg.ffn)}
+        # every layer's wq / wk / wv in ONE allocation, layer after layer (same types throughout): each layer's three
+        # are then adjacent (one GEMM for the block's q/k/v) and the layers' [wk; wv] pairs are an equal distance apart,
+        # which lets the library project the context columns' K/V of all layers with one batched GEMM
+        qkv_all = None
+        lw = weights["layers"]
+        if adjacent and len(lw) > 1 and len({int(Lw[k][0]) for Lw in lw for k in ("wq", "wk", "wv")}) == 1:
+            qkv_all = up.q_adjacent([Lw[k] for Lw in lw for k in ("wq", "wk", "wv")],
+                                    [shape[k] for _ in lw for k in ("wq", "wk", "wv")])
         for il, Lw in enumerate(weights["layers"]):
             L = self._layers[il]
             for k in ("attn_norm", "q_norm", "k_norm", "post_norm"):
@@ -530,7 +538,10 @@ class DraftHead:
             grouped = ()
             if adjacent:
                 grouped = ("wq", "wk", "wv", "gate", "up")
-                L.wq, L.wk, L.wv = up.q_adjacent([Lw["wq"], Lw["wk"], Lw["wv"]], [shape["wq"], shape["wk"], shape["wv"]])
+                if qkv_all is not None:
+                    L.wq, L.wk, L.wv = qkv_all[3 * il:3 * il + 3]
+                else:
+                    L.wq, L.wk, L.wv = up.q_adjacent([Lw["wq"], Lw["wk"], Lw["wv"]], [shape["wq"], shape["wk"], shape["wv"]])
                 L.gate, L.up = up.q_adjacent([Lw["gate"], Lw["up"]], [shape["gate"], shape["up"]])
             for k in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
                 if k not in grouped:
