@@ -332,6 +332,18 @@ __global__ void __launch_bounds__(64)
     }
 }
 
+// The few words a speculative step hands back to the host (the verify's argmax and top-2 gaps, the drafter's
+// tokens), written by one small kernel straight into the context's pinned page: [16] argmax, [16] drafts, [16] gaps.
+__global__ void step_readback_kernel(const int32_t *__restrict__ argmax, const float *__restrict__ gap,
+                                     const int32_t *__restrict__ draft, int n, int32_t *__restrict__ out) {
+    const int i = threadIdx.x;
+    if (i < n) {
+        out[i] = argmax[i];
+        out[16 + i] = draft[i];
+        out[32 + i] = __float_as_int(gap[i]);
+    }
+}
+
 template <typename T>
 bool dev_alloc(T **p, size_t count) {
     return hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T) + 256) == hipSuccess;
@@ -1425,12 +1437,20 @@ int32_t dflash_spec_step(dflash_ctx *ctx, const dflash_model *target, const dfla
                                     sess->hidden, nullptr, nullptr, st)))
             return undo(rc);
         if (timed) STEP_HIP(hipEventRecord(ctx->ev1, st));
-        // read back through the context's pinned page: three truly asynchronous copies, one wait
+        // read back through the context's pinned page, one wait
         int32_t *pin_argmax = static_cast<int32_t *>(ctx->pinned), *pin_draft = pin_argmax + 16;
         float *pin_gap = reinterpret_cast<float *>(pin_argmax + 32);
-        STEP_HIP(hipMemcpyAsync(pin_argmax, sess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-        STEP_HIP(hipMemcpyAsync(pin_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost, st));
-        STEP_HIP(hipMemcpyAsync(pin_draft, dsess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        void *pinned_dev = nullptr;
+        if (hipHostGetDevicePointer(&pinned_dev, ctx->pinned, 0) == hipSuccess && pinned_dev) {
+            // (one launch that writes the pinned page directly instead of three copy commands)
+            step_readback_kernel<<<1, 64, 0, st>>>(sess->argmax, sess->gap, dsess->argmax, N, static_cast<int32_t *>(pinned_dev));
+            STEP_HIP(hipGetLastError());
+        } else {
+            (void)hipGetLastError();
+            STEP_HIP(hipMemcpyAsync(pin_argmax, sess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+            STEP_HIP(hipMemcpyAsync(pin_gap, sess->gap, N * sizeof(float), hipMemcpyDeviceToHost, st));
+            STEP_HIP(hipMemcpyAsync(pin_draft, dsess->argmax, N * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        }
         STEP_HIP(hipStreamSynchronize(st));
         memcpy(res->verify_argmax, pin_argmax, N * sizeof(int32_t));
         memcpy(res->verify_gap, pin_gap, N * sizeof(float));
