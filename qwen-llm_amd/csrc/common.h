@@ -25,6 +25,12 @@ struct dflash_ctx {
     // measurement aid: split-K GEMM calls launch their streaming kernel only (Y is left without its reduction), so
     // that back-to-back launches of that one kernel can be timed between two events
     bool stream_kernel_only = false;
+    // Set by a caller inside the library for the duration of one few-row GEMM call on a fused gate | up matrix
+    // (2 ffn output rows, ffn a multiple of 16): if the call is split over K, its reduction writes
+    // silu(gate) * up to swiglu_out[n_rows][ffn] instead of the sums to Y and sets swiglu_done; if it is not (Y is
+    // complete), swiglu_done stays false and the caller applies the activation itself.
+    float *swiglu_out = nullptr;
+    bool swiglu_done = false;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     double timed_ms[8] = {0};
     int64_t timed_launches[8] = {0};

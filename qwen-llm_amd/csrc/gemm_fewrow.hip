@@ -461,6 +461,48 @@ __device__ __forceinline__ void q4k_flush(const Q4KRange &rg, const Q4KBatch &bt
 // with its 320 waves, 11.7 instead of 5.4 + 3.9 for the latter with its 16 workgroups (a CU takes in only
 // 20-30 KB per microsecond, so a narrow kernel that reads 8-16 times the data loses more than the launch it
 // saves); a 40-layer verify took 4.77 ms instead of 4.70 ms with the first alone.)
+// Element e = 16 m + n of output tile (group, wave) of a split group: the sum of its partial tiles in workgroup order.
+template <int kWaves>
+__device__ __forceinline__ float q4k_partial_sum(const float *__restrict__ partials, int group, int wave, int e, int nb, int total,
+                                                 int n_wg, int wg_first, int wg_last) {
+    // a contributor's partial sits in slot 0 if its range starts inside this group (true for all
+    // but possibly the first contributor), else in slot 1
+    const int first_begin = static_cast<int>(static_cast<uint32_t>(total) * wg_first / n_wg);
+    const int first_slot = first_begin >= group * nb ? 0 : 1;
+    const size_t stride = static_cast<size_t>(2) * kWaves * 256;  // floats per workgroup
+    const float *p = partials + static_cast<size_t>(wave) * 256 + e;
+    float sum = p[wg_first * stride + static_cast<size_t>(first_slot) * kWaves * 256];
+    int wg = wg_first + 1;
+    for (; wg + 3 <= wg_last; wg += 4) {
+        const float a0 = p[wg * stride], a1 = p[(wg + 1) * stride], a2 = p[(wg + 2) * stride], a3 = p[(wg + 3) * stride];
+        sum = (((sum + a0) + a1) + a2) + a3;
+    }
+    for (; wg <= wg_last; wg++) sum += p[wg * stride];
+    return sum;
+}
+
+// The reduction of a fused gate | up product (one matrix of 2 ffn rows: the gate's, then the up's) with the SwiGLU
+// that follows it: out[m][c] = silu(gate[m][c]) * up[m][c], one workgroup per 16 gate columns, each value either the
+// sum of its partial tiles (same order as q4k_reduce_kernel) or, for a group one workgroup covered alone, what the
+// streaming kernel stored in y.  One launch instead of the reduction and the activation kernel; same bits.
+template <int kWaves>
+__global__ void __launch_bounds__(256)
+    q4k_reduce_swiglu_kernel(const float *__restrict__ partials, const float *__restrict__ y, float *__restrict__ out, int ffn, int nb,
+                             int n_rows, int n_groups, int n_wg) {
+    const int e = threadIdx.x, m = e >> 4, n = e & 15;
+    const int col = blockIdx.x * 16 + n;
+    if (m >= n_rows || col >= ffn) return;
+    const int total = n_groups * nb, n_out = 2 * ffn;
+    auto value = [&](int c) {
+        const int tile = c >> 4, group = tile / kWaves, wave = tile - group * kWaves;
+        const int wg_first = q4k_wg_of(group * nb, total, n_wg), wg_last = q4k_wg_of((group + 1) * nb - 1, total, n_wg);
+        if (wg_first == wg_last) return y[static_cast<size_t>(m) * n_out + c];
+        return q4k_partial_sum<kWaves>(partials, group, wave, e, nb, total, n_wg, wg_first, wg_last);
+    };
+    const float g = value(col), u = value(col + ffn);  // (ffn is a multiple of 16: the same n in both tiles)
+    out[static_cast<size_t>(m) * ffn + col] = g / (1.0f + expf(-g)) * u;
+}
+
 template <int kWaves>
 __global__ void __launch_bounds__(256)
     q4k_reduce_kernel(const float *__restrict__ partials, float *__restrict__ y, int n_out, int nb, int n_rows,
@@ -477,20 +519,7 @@ __global__ void __launch_bounds__(256)
     y += static_cast<size_t>(slot_j) * bt.y_stride;
     const int orow = (lg * kWaves + wave) * 16 + n;
     if (m >= n_rows || orow >= n_out) return;
-    // a contributor's partial sits in slot 0 if its range starts inside this group (true for all
-    // but possibly the first contributor), else in slot 1
-    const int first_begin = static_cast<int>(static_cast<uint32_t>(total) * wg_first / n_wg);
-    const int first_slot = first_begin >= group * nb ? 0 : 1;
-    const size_t stride = static_cast<size_t>(2) * kWaves * 256;  // floats per workgroup
-    const float *p = partials + static_cast<size_t>(wave) * 256 + e;
-    float sum = p[wg_first * stride + static_cast<size_t>(first_slot) * kWaves * 256];
-    int wg = wg_first + 1;
-    for (; wg + 3 <= wg_last; wg += 4) {
-        const float a0 = p[wg * stride], a1 = p[(wg + 1) * stride], a2 = p[(wg + 2) * stride], a3 = p[(wg + 3) * stride];
-        sum = (((sum + a0) + a1) + a2) + a3;
-    }
-    for (; wg <= wg_last; wg++) sum += p[wg * stride];
-    y[static_cast<size_t>(m) * n_out + orow] = sum;
+    y[static_cast<size_t>(m) * n_out + orow] = q4k_partial_sum<kWaves>(partials, group, wave, e, nb, total, n_wg, wg_first, wg_last);
 }
 
 #ifdef DFLASH_TRACE
@@ -1930,6 +1959,9 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     // a single matrix whose ranges are whole tile groups needs no reduction; a batch always may
     const bool split = (batch ? !batch->whole_groups : groups % n_wg != 0);
     const bool reduce = split && !ctx->stream_kernel_only;
+    // a caller inside the library may ask for the SwiGLU of a fused gate | up product in place of the plain reduction
+    float *swiglu_out = batch ? nullptr : ctx->swiglu_out;
+    if (swiglu_out) ctx->swiglu_done = false;
     Q4KBatch bt = {};
     if (batch) bt = *batch;
     bt.groups_per_mat = gpm;
@@ -1950,7 +1982,11 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
             gemm_q4k_stream_kernel<WAVES, XT><<<n_wg, 64 * WAVES, lds, st>>>(wb, static_cast<const XT *>(x), y, partials, \
                                                                              no, nb, n_rows, groups, bt, tiled ? 1 : 0); \
         }                                                                                                              \
-        if (reduce) {                                                                                                  \
+        if (reduce && swiglu_out) {                                                                                    \
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                    \
+            q4k_reduce_swiglu_kernel<WAVES><<<no / 32, 256, 0, st>>>(partials, y, swiglu_out, no / 2, nb, n_rows, groups, n_wg); \
+            ctx->swiglu_done = true;                                                                                   \
+        } else if (reduce) {                                                                                           \
             dfl_timed timer(ctx, st, DFL_T_REDUCE);                                                                    \
             q4k_reduce_kernel<WAVES><<<groups * WAVES, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);   \
         }                                                                                                              \
@@ -1971,7 +2007,11 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
                 gemm_q4k_tiled_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
                                                                                               partials, no, nb, n_rows, groups, bt, k_pre);
         }
-        if (reduce) {
+        if (reduce && swiglu_out) {
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);
+            q4k_reduce_swiglu_kernel<16><<<no / 32, 256, 0, st>>>(partials, y, swiglu_out, no / 2, nb, n_rows, groups, n_wg);
+            ctx->swiglu_done = true;
+        } else if (reduce) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);
             q4k_reduce_kernel<16><<<groups * 16, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);
         }
@@ -1988,7 +2028,11 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
                 gemm_q4k_slab_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kSlabLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
                                                                                             partials, no, nb, n_rows, groups, bt);
         }
-        if (reduce) {
+        if (reduce && swiglu_out) {
+            dfl_timed timer(ctx, st, DFL_T_REDUCE);
+            q4k_reduce_swiglu_kernel<16><<<no / 32, 256, 0, st>>>(partials, y, swiglu_out, no / 2, nb, n_rows, groups, n_wg);
+            ctx->swiglu_done = true;
+        } else if (reduce) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);
             q4k_reduce_kernel<16><<<groups * 16, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);
         }

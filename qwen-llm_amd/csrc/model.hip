@@ -389,8 +389,16 @@ int32_t gemm_gate_up(dflash_ctx *ctx, const dflash_qtensor &gate, const dflash_q
                      float *pk, int64_t n_in, int64_t ffn, int n, hipStream_t st) {
     int32_t rc;
     if (pk && adjacent(gate, ffn, up, n_in)) {
-        if ((rc = gemm(ctx, gate, x, pk, n_in, 2 * ffn, n, st))) return rc;
-        silu_mul_ld_kernel<<<dim3(blocks_for(static_cast<size_t>(ffn)), n), 256, 0, st>>>(pk, pk + ffn, 2 * ffn, g, static_cast<int>(ffn));
+        // (a product split over K applies the activation in its reduction: one launch less)
+        ctx->swiglu_out = ffn % 16 == 0 ? g : nullptr;
+        ctx->swiglu_done = false;
+        rc = gemm(ctx, gate, x, pk, n_in, 2 * ffn, n, st);
+        const bool done = ctx->swiglu_done;
+        ctx->swiglu_out = nullptr;
+        ctx->swiglu_done = false;
+        if (rc) return rc;
+        if (!done)
+            silu_mul_ld_kernel<<<dim3(blocks_for(static_cast<size_t>(ffn)), n), 256, 0, st>>>(pk, pk + ffn, 2 * ffn, g, static_cast<int>(ffn));
         return DFLASH_OK;
     }
     if ((rc = gemm(ctx, gate, x, g, n_in, ffn, n, st))) return rc;
@@ -597,11 +605,14 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
     const float scale = 1.0f / sqrtf(static_cast<float>(hd));
     const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
     bool cur_ready = false;  // s->cur already holds this layer's normalised input
+    const float *pending_resid = nullptr;  // a dense layer's FFN output still to be added to s->x
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_layer &L = model->layers[il];
         _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
         // (a mixture-of-experts layer leaves the next layer's normalised input behind)
-        if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
+        // (a dense layer leaves its FFN output in s->mix: the residual add is folded into this norm)
+        if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
+        pending_resid = nullptr;
         cur_ready = false;
         bool packed;
         if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, true, &packed, H, q_dim, kv_dim, n, st))) return rc;
@@ -627,13 +638,19 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
         } else {
             if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, n, st))) return rc;
             if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
-            add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
+            // x += mix: by the next norm, unless this layer's residual is captured first
+            bool tapped = false;
+            for (int t = 0; t < n_taps; t++) tapped = tapped || tap_layers[t] == il;
+            if (tapped)
+                add_kernel<<<blocks_for(static_cast<size_t>(n) * H), 256, 0, st>>>(s->x, s->mix, static_cast<size_t>(n) * H);
+            else
+                pending_resid = s->mix;
         }
         for (int t = 0; t < n_taps; t++)
             if (tap_layers[t] == il)
                 capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
     }
-    if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, nullptr, model->output_norm, s->cur, H, c.eps, nullptr, nullptr);
+    if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, model->output_norm, s->cur, H, c.eps, nullptr, nullptr);
     if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
     if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gp, st))) return rc;
     DFL_HIP_CHECK(ctx, hipGetLastError());
