@@ -159,10 +159,12 @@ int32_t dfl_gemm_q6k_set(dflash_ctx *ctx, int n_mats, const void *const *w, floa
 // whole_groups): SwiGLU pair, y = silu(x . gate^T) * (x . up^T) with the gate matrices from w_stack /
 // extra_w and the up matrices, same ids, from w_stack_up / extra_w_up.  tiled != 0: every matrix (the stacks'
 // members, the extras) is in the tiled order of dflash_repack_q4k_tiled and w_stride_bytes is the tiled size.
-// Enqueue only.
+// y_type: DFLASH_TYPE_F32, or DFLASH_TYPE_F16 (y then points to f16 and y_stride counts f16 elements) where
+// dfl_q4k_batched_f16_out() says the path that will run can write it.  Enqueue only.
+bool dfl_q4k_batched_f16_out(const dflash_ctx *ctx, int32_t tiled, int32_t whole_groups, int64_t n_out);
 int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const void *extra_w,
                              const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
                              size_t x_stride,
-                             float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
+                             void *y, int32_t y_type, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
                              int32_t whole_groups, const void *w_stack_up, const void *extra_w_up, int32_t tiled,
                              dflash_stream_t stream);

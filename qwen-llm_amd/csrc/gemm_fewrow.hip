@@ -126,8 +126,18 @@ struct Q4KGeom {
     static constexpr int kFull = kWaveLoads / kWaves;       // ... every wave issues this many,
     static constexpr int kExtra = kWaveLoads % kWaves;      // ... and waves below kExtra one more
     static constexpr int kXLoads = 16 / kWaves;             // activation loads per thread and stage
-    // LDS: a ring of three weight buffers, then two activation buffers (stage parity)
-    static constexpr int kLdsPieces = 3 * kWPieces + 2 * kQ4KBlockFrags;
+    // Weight stages in flight ahead of the one being computed.  A workgroup streams only as fast as
+    // (bytes in flight) / (memory latency): with two 18 KB stages in flight an 8-wave group gets
+    // ~14 KB/us whatever the rest of the chip does, so it keeps more of them in flight; a 16-wave
+    // group's stages are twice the size and LDS holds no more than three of them.
+#ifndef DFLASH_Q4K_AHEAD8
+#define DFLASH_Q4K_AHEAD8 4
+#endif
+    static constexpr int kAhead = kWaves == 8 ? DFLASH_Q4K_AHEAD8 : 2;
+    static constexpr int kRing = kAhead + 1;
+    // LDS: a ring of kRing weight buffers, then two activation buffers (stage parity)
+    static constexpr int kLdsPieces = kRing * kWPieces + 2 * kQ4KBlockFrags;
+    static_assert(kLdsPieces * 16 <= 160 * 1024, "fits one CU's LDS");
     static_assert(kWPieces % 64 == 0, "whole wave-loads");
     static_assert(kFull + (kExtra ? 1 : 0) <= 4, "one weight load is issued after every second of a stage's 8 MFMAs");
     static_assert(kXLoads == 1 || kXLoads == 2, "8 or 16 waves");
@@ -211,6 +221,7 @@ struct Q4KBatch {
     // tile waits in registers while the up tile is computed.
     int pair;
     const uint8_t *w2, *extra_w2;
+    int y_f16;  // the output is f16 (gemm_q4k_experts_kernel only)
 };
 
 // Tiled order (see gemm_q4k_tiled_kernel): one wave's 16 rows of a stage, and a whole 256-row stage, in bytes.
@@ -405,6 +416,25 @@ __device__ __forceinline__ void q4k_compute(const half8_t *buf, const half8_t *x
 constexpr int q4k_vmcnt(int n) { return ((n & 0xF) | ((n & 0x30) << 10)) | 0x0F70; }
 // s_waitcnt lgkmcnt(0) alone
 constexpr int kWaitLds = 0xC07F;
+// s_waitcnt vmcnt(v) for a wave-uniform run-time v (the instruction takes an immediate); anything
+// past the table waits for every load, which is always sufficient
+__device__ __forceinline__ void q4k_wait_vm(int v) {
+    switch (v) {
+#define DFL_VM(n)                                      \
+    case n:                                            \
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(n));      \
+        break;
+        DFL_VM(1) DFL_VM(2) DFL_VM(3) DFL_VM(4) DFL_VM(5) DFL_VM(6) DFL_VM(7) DFL_VM(8) DFL_VM(9) DFL_VM(10) DFL_VM(11) DFL_VM(12)
+        DFL_VM(13) DFL_VM(14) DFL_VM(15) DFL_VM(16) DFL_VM(17) DFL_VM(18) DFL_VM(19) DFL_VM(20) DFL_VM(21) DFL_VM(22) DFL_VM(23) DFL_VM(24)
+        DFL_VM(25) DFL_VM(26) DFL_VM(27) DFL_VM(28) DFL_VM(29) DFL_VM(30) DFL_VM(31) DFL_VM(32) DFL_VM(33) DFL_VM(34) DFL_VM(35) DFL_VM(36)
+        DFL_VM(37) DFL_VM(38) DFL_VM(39) DFL_VM(40) DFL_VM(41) DFL_VM(42) DFL_VM(43) DFL_VM(44) DFL_VM(45) DFL_VM(46) DFL_VM(47) DFL_VM(48)
+        DFL_VM(49) DFL_VM(50) DFL_VM(51) DFL_VM(52) DFL_VM(53) DFL_VM(54) DFL_VM(55) DFL_VM(56) DFL_VM(57) DFL_VM(58) DFL_VM(59) DFL_VM(60)
+        DFL_VM(61) DFL_VM(62)
+#undef DFL_VM
+    default:
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+    }
+}
 
 // Ends a tile group's segment: Y directly if this workgroup covered the group's whole K, else a
 // partial tile for the reduce kernel (slot 0: the range's first group, slot 1: its last).
@@ -535,7 +565,15 @@ __device__ unsigned long long *g_trace2 = nullptr;  // [n_wg][16 waves][4]: cycl
     do {                                                                                                    \
         if ((threadIdx.x & 63) == 0 && g_trace2) g_trace2[(blockIdx.x * 16 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); \
     } while (0)
+// the streaming kernel's stamps: a gate/up pair launch writes 1024 workgroups further on than a plain one
+#define DFL_TRS(i)                                                                                              \
+    do {                                                                                                        \
+        if (threadIdx.x == 0 && g_trace) g_trace[(blockIdx.x + (bt.pair ? 1024 : 0)) * 16 + (i)] = wall_clock64(); \
+    } while (0)
 #else
+#define DFL_TRS(i) \
+    do {           \
+    } while (0)
 #define DFL_TRW(i) \
     do {           \
     } while (0)
@@ -553,12 +591,13 @@ __global__ void __launch_bounds__(64 * kWaves)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    DFL_TR(0);
+    DFL_TRS(0);
     Q4KRange rg;
     rg.nb = nb;
     rg.n_wg = gridDim.x;
     const int vshift = bt.pair ? 1 : 0;  // virtual groups per real group, as a shift
-    if (bt.ids) n_groups = (bt.groups_per_mat * *bt.n_slots) << vshift;  // how many matrices take part is decided on the device
+    const int n_slots = bt.ids ? *bt.n_slots : 1;
+    if (bt.ids) n_groups = (bt.groups_per_mat * n_slots) << vshift;  // how many matrices take part is decided on the device
     rg.total = n_groups * nb;
     rg.wg = q4k_range_index(blockIdx.x, rg.n_wg);
     if (bt.whole_groups) {
@@ -583,6 +622,21 @@ __global__ void __launch_bounds__(64 * kWaves)
     // matrix is cut in 256-row tile groups stored [group][super-block][256 rows x 144 bytes]; an 8-wave workgroup
     // owns the lower or the upper 128 rows of one, i.e. the first or second half of each of its stages.
     constexpr int kPerTiled = 16 / kWaves;  // this kernel's groups per tile group of the tiled order
+    // The matrix index of a slot comes out of a register window over the list (lane l holds the id of slot
+    // slot_base + l), read with one vector load per 64 slots.  A load of ids[j] at every change of matrix would be
+    // a vector load too (the compiler cannot prove the list is not written), and the wait for it is a wait for
+    // every weight stage in flight: the prefetch would start from nothing at every tile group.
+    int slot_base = -64;  // no window yet: the first use (before any weight load is issued) reads it
+    int32_t ids_window = 0;
+    auto slot_id = [&](int j) {
+        if (j < slot_base || j >= slot_base + 64) {
+            slot_base = j;
+            ids_window = bt.ids[min(j + lane, n_slots - 1)];
+            __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+            asm volatile("" : "+v"(ids_window));
+        }
+        return __builtin_amdgcn_readlane(ids_window, j - slot_base);
+    };
     auto group_w = [&](int group) {
         const uint8_t *mat = w;
         int lg = group;
@@ -591,7 +645,7 @@ __global__ void __launch_bounds__(64 * kWaves)
             const int g = group >> vshift;
             const int j = static_cast<int>(q4k_div(g, bt.by_gpm));
             lg = g - j * bt.groups_per_mat;
-            const int32_t id = bt.ids[j];
+            const int32_t id = slot_id(j);
             mat = id < 0 ? (up ? bt.extra_w2 : bt.extra_w) : (up ? bt.w2 : w) + static_cast<size_t>(id) * bt.w_stride;
         }
         if (tiled)
@@ -607,10 +661,10 @@ __global__ void __launch_bounds__(64 * kWaves)
         group >>= vshift;
         return bt.ids ? group - static_cast<int>(q4k_div(group, bt.by_gpm)) * bt.groups_per_mat : group;
     };
-    DFL_TR(10);
+    DFL_TRS(10);
     Q4KLane<kWaves> L;
     q4k_lane_w_offsets<kWaves>(L, tid, group_local(rg.first_group) * G::kRows, n_out, row_bytes, tiled);
-    DFL_TR(11);
+    DFL_TRS(11);
 
     // Cursors.  Weights: wstage = first byte of the next stage to load in its group's first row,
     // bw its super-block, gw its group, w_left the stages not loaded yet.  Activations run one
@@ -646,39 +700,44 @@ __global__ void __launch_bounds__(64 * kWaves)
         for (int j = 0; j < G::kFull; j++) q4k_issue_w<kWaves>(wstage, buf, L, j, wave);
         if (wave < G::kExtra) q4k_issue_w<kWaves>(wstage, buf, L, G::kFull, wave);
     };
-    half8_t *buf_c = lds, *buf_n = lds + G::kWPieces, *buf_f = lds + 2 * G::kWPieces;
-    half8_t *x_c = lds + 3 * G::kWPieces, *x_n = x_c + kQ4KBlockFrags;
+    constexpr int kAhead = G::kAhead, kRing = G::kRing;
+    // weight ring: slot_c holds the stage being computed, slot_i takes the next stage to be loaded
+    int slot_c = 0, slot_i = 0;
+    auto ring = [&](int slot) { return lds + slot * G::kWPieces; };
+    half8_t *x_c = lds + kRing * G::kWPieces, *x_n = x_c + kQ4KBlockFrags;
 
-    // Prologue, in this order: weights of stage 0 (first of all: everything else here hides behind
-    // their latency), activations of stages 0 and 1 | weights of stage 1, activations of stage 2.
-    // From then on stage d issues one group [weights of d+2, activations of d+3], and "all but the
-    // youngest group have landed" is what the top of each stage waits for; young_w / young_x say
-    // what the youngest group holds.
-    issue_w_all(buf_c);
+    // Loads are issued, and return, in groups: group 0 = [weights of stage 0 (first of all: everything
+    // else here hides behind their latency), activations of stages 0 and 1], group p = [weights of
+    // stage p, activations of stage p + 1].  The prologue issues groups 0 .. kAhead-1, stage d issues
+    // group d + kAhead, and the top of stage d waits until group d has landed, i.e. until no more
+    // loads are outstanding than the (up to kAhead - 1) younger groups hold.
+    issue_w_all(ring(0));
     advance_w();
+    slot_i = 1;
     q4k_lane_x_offsets<kWaves, XT>(L, tid, n_rows, n_in);
     float4_t acc = {0, 0, 0, 0}, acc_min = {0, 0, 0, 0}, stash = {0, 0, 0, 0};
     const Q4KMagic magic = q4k_magic();
-    Q4KXRaw<kWaves, XT> raw_first, raw_a, raw_b;  // activations of stage 0 / odd stages / even stages >= 2
-    bool young_w = false, young_x = false;
+    Q4KXRaw<kWaves, XT> raw_first, raws[kAhead];  // activations of stage 0; raws[d % kAhead]: those of stage d + 1
     q4k_load_x<kWaves, XT>(xblock, L, raw_first);
     advance_x();
     if (x_left > 0) {
-        q4k_load_x<kWaves, XT>(xblock, L, raw_a);
+        q4k_load_x<kWaves, XT>(xblock, L, raws[0]);
         advance_x();
     }
-    if (w_left > 0) {
-        issue_w_all(buf_n);
-        advance_w();
-        young_w = true;
-        if (x_left > 0) {
-            q4k_load_x<kWaves, XT>(xblock, L, raw_b);
-            advance_x();
-            young_x = true;
+#pragma unroll
+    for (int p = 1; p < kAhead; p++) {
+        if (w_left > 0) {
+            issue_w_all(ring(p));
+            advance_w();
+            slot_i = p + 1;
+            if (x_left > 0) {
+                q4k_load_x<kWaves, XT>(xblock, L, raws[p]);
+                advance_x();
+            }
         }
     }
-    DFL_TR(12);
-    DFL_TR(1);
+    DFL_TRS(12);
+    DFL_TRS(1);
     int gc = rg.first_group, bc = b0, n_left = rg.it_end - rg.it_begin;
     bool first = true;
     int done = 0;
@@ -691,18 +750,15 @@ __global__ void __launch_bounds__(64 * kWaves)
 #ifdef DFLASH_TRACE
         const unsigned long long c0 = DFL_CYC();
 #endif
-        if (young_w && young_x) {
+        if (n_left > kAhead) {  // every younger group exists and is whole
             if (wave < G::kExtra)
-                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW1 + kX));
+                __builtin_amdgcn_s_waitcnt(q4k_vmcnt((kAhead - 1) * (kW1 + kX)));
             else
-                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW0 + kX));
-        } else if (young_w) {
-            if (wave < G::kExtra)
-                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW1));
-            else
-                __builtin_amdgcn_s_waitcnt(q4k_vmcnt(kW0));
+                __builtin_amdgcn_s_waitcnt(q4k_vmcnt((kAhead - 1) * (kW0 + kX)));
         } else {
-            __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+            // the range ends within reach: n_left - 1 younger weight stages, the last of them without activations
+            const int ow = n_left - 1, ox = n_left >= 2 ? n_left - 2 : 0;
+            q4k_wait_vm(ow * (wave < G::kExtra ? kW1 : kW0) + ox * kX);
         }
 #ifdef DFLASH_TRACE
         const unsigned long long c1 = DFL_CYC();
@@ -717,13 +773,13 @@ __global__ void __launch_bounds__(64 * kWaves)
         // A bare barrier, not __syncthreads(): that one carries a workgroup-scope fence, which waits
         // for every load in flight and would undo the prefetch.  The waits above are the only
         // ordering this needs: each wave's own pieces have landed before it arrives here.
-        __builtin_amdgcn_s_barrier();  // stage d is complete in buf_c; buf_f (stage d-1) is free
+        __builtin_amdgcn_s_barrier();  // stage d is complete in its ring slot; the slot of stage d-1 is free
 #ifdef DFLASH_TRACE
         const unsigned long long c2 = DFL_CYC();
 #endif
         const bool iw = w_left > 0, ix = x_left > 0;
-        q4k_compute<kWaves, XT>(buf_c, x_c, lane, wave, magic, acc, acc_min, iw, wstage, buf_f, ix, xblock, L, raw, n_left > 1,
-                                x_n);
+        q4k_compute<kWaves, XT>(ring(slot_c), x_c, lane, wave, magic, acc, acc_min, iw, wstage, ring(slot_i), ix, xblock, L, raw,
+                                n_left > 1, x_n);
 #ifdef DFLASH_TRACE
         {
             const unsigned long long c3 = DFL_CYC();
@@ -735,18 +791,14 @@ __global__ void __launch_bounds__(64 * kWaves)
 #endif
         if (iw) advance_w();
         if (ix) advance_x();
-        young_w = iw;
-        young_x = ix;
-        half8_t *t = buf_c;
-        buf_c = buf_n;
-        buf_n = buf_f;
-        buf_f = t;
-        t = x_c;
+        slot_c = slot_c + 1 == kRing ? 0 : slot_c + 1;
+        if (iw) slot_i = slot_i + 1 == kRing ? 0 : slot_i + 1;
+        half8_t *t = x_c;
         x_c = x_n;
         x_n = t;
         n_left--;
         done++;
-        if (done <= 8) DFL_TR(1 + done);
+        if (done <= 8) DFL_TRS(1 + done);
         if (++bc == nb || n_left == 0) {
             q4k_flush<kWaves>(rg, bt, gc, acc, acc_min, stash, y, partials, n_out, n_rows, tid);
             bc = 0;
@@ -754,14 +806,14 @@ __global__ void __launch_bounds__(64 * kWaves)
         }
     };
     while (n_left > 0) {
-        stage(raw_a);
-        if (n_left == 0) break;
-        stage(raw_b);
+#pragma unroll
+        for (int u = 0; u < kAhead; u++)
+            if (n_left > 0) stage(raws[u]);
     }
-    DFL_TR(13);
+    DFL_TRS(13);
 #ifdef DFLASH_TRACE
     if (lane == 0 && g_trace2) {
-        unsigned long long *t = g_trace2 + (static_cast<size_t>(blockIdx.x) * 16 + wave) * 4;
+        unsigned long long *t = g_trace2 + (static_cast<size_t>(blockIdx.x + (bt.pair ? 1024 : 0)) * 16 + wave) * 4;
         t[0] = cyc_wait;
         t[1] = cyc_bar;
         t[2] = cyc_comp;
@@ -1237,6 +1289,325 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     }
     DFL_TR(9);
     DFL_TRW(3);
+}
+
+// ----------------------------------------------------------------------------
+// Q4_K expert kernel: the matrices a device-side list picks out of a stack, tiled order
+// ----------------------------------------------------------------------------
+//
+// The batched mode of gemm_q4k_stream_kernel is bound by its own instructions (sixteen MFMAs and a workgroup barrier
+// per stage, two waves per SIMD to hide them: a CU streams 15 KB/us where the single-matrix tiled kernel takes in
+// 20) and by its coarse work unit (a 128-row group over the whole K: 186 units for 31 experts' gate/up on 256 CUs).
+// This kernel gives the tiled kernel's structure to a batch: a wave owns one 16-row tile over the matrix's whole K
+// (gate and up of the same tile in pair mode) and streams it through its private ring of three LDS buffers with
+// direct-to-LDS loads, meeting the other waves only where the shared activations change.  The activations of four
+// stages at a time sit in LDS as MFMA fragments with their sub-block sums (so the minima cost one MFMA per stage):
+//   * x shared by every slot (gate/up, a drafter's per-layer projections of the same columns): a workgroup takes a
+//     contiguous run of (slot, tile) units, sixteen per round, one per wave; the slab is refilled only when K is
+//     longer than four stages (twice per round for K = 2048);
+//   * x per slot (down: every expert has its own SwiGLU rows): a unit is (slot, sixteen tiles) and the slab is
+//     refilled when the slot changes.
+// A (row, matrix) result never depends on which other matrices take part: whole K per wave, fixed order.
+constexpr int kExpChunk = 4;  // stages of activations in LDS at a time
+constexpr size_t kExpRingEnd = static_cast<size_t>(kExpChunk) * kTiledStageX +
+                               static_cast<size_t>(kSlabWaves) * kSlabRing * kSlabWavePieces * 16;
+constexpr size_t kExpLdsBytes = kExpRingEnd + (kSlabWaves / 2) * 64 * sizeof(float4_t);  // + the up tiles of split pairs
+static_assert(kExpLdsBytes <= 160 * 1024, "one workgroup per CU, all of its LDS");
+
+// q4k_tiled_compute for the expert kernel, which carries more state per lane (activations on their way for the next
+// refill, a second accumulator in pair mode) inside the 128 registers sixteen waves leave each other: the minima
+// product is subtracted in the same accumulator (B operand negated) and the activation fragments are fetched four at
+// a time.
+__device__ __forceinline__ void q4k_experts_compute(const u32x4_t *blk, const uint8_t *stage, int lane, int g, uint32_t sc_sel,
+                                                    Q4KMagic magic, float4_t &acc) {
+    const u32x4_t hdr = blk[0], q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
+    half8_t af[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) af[t] = *reinterpret_cast<const half8_t *>(stage + t * kTiledFragStride + lane * 16);
+    const half4_t tw = *reinterpret_cast<const half4_t *>(stage + 8 * kTiledFragStride + lane * 8);
+    const uint32_t upper = 0u - static_cast<uint32_t>(g >> 1);
+    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu, mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t sc_word = (sc_hi & upper) | (sc_lo & ~upper), mn_word = (mn_hi & upper) | (mn_lo & ~upper);
+    const half2_t dm = __builtin_bit_cast(half2_t, hdr.x);
+    const half2_t p_sc = as_half2(__builtin_amdgcn_perm(0x64646464u, sc_word, sc_sel));
+    const half2_t p_mn = as_half2(__builtin_amdgcn_perm(0x64646464u, mn_word, sc_sel));
+    const half2_t neg = dm * splat(static_cast<_Float16>(-1024.0f));
+    const half2_t S = __builtin_elementwise_fma(p_sc, splat(dm[0]), splat(neg[0]));
+    // -(dmin * m): (1024 + code) * (-dmin) + 1024 dmin, rounded once like its positive twin
+    const half2_t M = __builtin_elementwise_fma(p_mn, splat(-dm[1]), splat(-neg[1]));
+    const half2_t unbias = {static_cast<_Float16>(-1024.0f), static_cast<_Float16>(-64.0f)};
+    const half2_t Cs = S * unbias;
+    const half2_t s2l = splat(S[0]), c2l = splat(Cs[0]);
+    const half2_t s2h = splat(S[1]), c2h = splat(Cs[1]);
+    const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const _Float16 zero = static_cast<_Float16>(0.0f);
+    const half8_t a_min = {tw[0], tw[1], tw[2], tw[3], zero, zero, zero, zero};
+    const half8_t b_min = {M[0], M[1], M[0], M[1], zero, zero, zero, zero};
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_min, b_min, acc, 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) af[t] = *reinterpret_cast<const half8_t *>(stage + (4 + t) * kTiledFragStride + lane * 16);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bh, acc, 0, 0, 0);
+    }
+}
+
+template <typename XT, typename YT>
+__global__ void __launch_bounds__(64 * kSlabWaves)
+    gemm_q4k_experts_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, YT *__restrict__ y, int n_out, int nb,
+                            int n_rows, Q4KBatch bt, int upm, Q4KDiv by_upm, int max_slots) {
+    constexpr int kW = kSlabWaves;
+    constexpr int kItems = kExpChunk * 8 / kW;  // activation items (eight values of one row) per thread and refill: 2
+    constexpr int kXInstr = kItems * Q4KX8<XT>::kLoads;
+    extern __shared__ half8_t lds[];
+    uint8_t *slab = reinterpret_cast<uint8_t *>(lds);                              // [kExpChunk][kTiledStageX]
+    half8_t *ring = reinterpret_cast<half8_t *>(slab + kExpChunk * kTiledStageX);  // [wave][kSlabRing][144]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool per_slot_x = bt.x_stride != 0;
+    // ---- activations: items as in gemm_q4k_tiled_kernel (virtual wave v = wave + 16 r: stage v / 8 of the chunk) ----
+    typename Q4KX8<XT>::type raw_a[kItems], raw_b[kItems];
+    const uint32_t n_in = static_cast<uint32_t>(nb) * DFL_QK_K;
+    const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(x);
+    uint32_t x_off[kItems];
+#pragma unroll
+    for (int r = 0; r < kItems; r++) {
+        const int v = wave + kW * r;
+        const int m = 8 * ((v >> 2) & 1) + (lane >> 3), c = 8 * (v & 3) + (lane & 7);
+        x_off[r] = (static_cast<uint32_t>(min(m, n_rows - 1)) * n_in + 8u * c) * static_cast<uint32_t>(sizeof(XT));
+    }
+    auto chunk_len = [&](int c) { return min(kExpChunk, nb - c * kExpChunk); };
+    auto load_x = [&](int xslot, int c) {  // stages past the chunk's end re-read its last stage (never converted)
+        const uint8_t *xb = q4k_uniform(xbytes + static_cast<size_t>(xslot) * bt.x_stride * sizeof(XT));
+        const int last = chunk_len(c) - 1;
+#pragma unroll
+        for (int r = 0; r < kItems; r++) {
+            const int sb = c * kExpChunk + min((wave + kW * r) >> 3, last);
+            q4k_load_x8(xb + static_cast<size_t>(sb) * (DFL_QK_K * sizeof(XT)), x_off[r], raw_a[r], raw_b[r]);
+        }
+    };
+    const int n_slots = min(*bt.n_slots, max_slots);  // (the bound the host sized the buffers for)
+    const int tiles = (n_out + 15) >> 4;
+    const int halves = bt.pair ? 2 : 1;
+    const int n_chunks = (nb + kExpChunk - 1) / kExpChunk;
+    // units: (slot, tile) with shared x, (slot, group of sixteen tiles) with x per slot; upm = units per matrix
+    const uint32_t units = static_cast<uint32_t>(n_slots) * static_cast<uint32_t>(upm);
+    const int wg = q4k_range_index(blockIdx.x, gridDim.x);
+    const int u0 = static_cast<int>(q4k_div(units * wg, bt.by_wg)), u1 = static_cast<int>(q4k_div(units * (wg + 1), bt.by_wg));
+    if (u0 >= u1) return;  // more workgroups than work (the whole workgroup leaves: no barrier is missed)
+    // Pair mode with at most eight units for this workgroup: gate and up of a unit go to two waves (w and w + 8)
+    // instead of one after the other on the same wave.  A lightly loaded wave is bound by its own chain of dependent
+    // instructions (~0.7 us per stage with nothing else on its SIMD), so halving the chain is what shortens the
+    // kernel; every product is still one wave's whole-K sum in the same order, so the bits do not depend on the mode.
+    const bool hsplit = bt.pair && !per_slot_x && u1 - u0 <= kW / 2;
+    const int n_rounds = per_slot_x ? u1 - u0 : (hsplit ? 1 : (u1 - u0 + kW - 1) / kW);
+    const int h_begin = hsplit ? wave >> 3 : 0, h_end = hsplit ? h_begin + 1 : halves;
+
+    // matrix index of a slot: a register window over the list (see gemm_q4k_stream_kernel)
+    // (Measured and not kept: the first window, the slot count and shared activations all loaded at the very top of
+    // the kernel - 1.2-1.5 us slower per launch than this order.)
+    int slot_base = -64;  // no window yet: the first use (before any weight load is issued) reads it
+    int32_t ids_window = 0;
+    auto slot_id = [&](int j) {
+        if (j < slot_base || j >= slot_base + 64) {
+            slot_base = j;
+            ids_window = bt.ids[min(j + lane, n_slots - 1)];
+            __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+            asm volatile("" : "+v"(ids_window));
+        }
+        return __builtin_amdgcn_readlane(ids_window, j - slot_base);
+    };
+    // this wave's unit in round r
+    auto unit_of = [&](int r, int &slot, int &tile) {
+        if (per_slot_x) {
+            const int g = u0 + r;
+            slot = static_cast<int>(q4k_div(g, by_upm));
+            tile = (g - slot * upm) * kW + wave;
+            return tile < tiles;
+        }
+        const int u = hsplit ? u0 + (wave & 7) : u0 + r * kW + wave;
+        slot = static_cast<int>(q4k_div(min(u, u1 - 1), by_upm));
+        tile = u - slot * upm;
+        return u < u1;
+    };
+    // whose activations round r needs (uniform over the workgroup)
+    auto xslot_of = [&](int r) { return per_slot_x ? static_cast<int>(q4k_div(u0 + r, by_upm)) : 0; };
+    auto tile_base = [&](int slot, int tile, int half) {
+        const int32_t id = slot_id(slot);
+        const uint8_t *mat = id < 0 ? (half ? bt.extra_w2 : bt.extra_w) : (half ? bt.w2 : w) + static_cast<size_t>(id) * bt.w_stride;
+        return q4k_uniform(mat + static_cast<size_t>(tile >> 4) * nb * kTiledStageBytes + static_cast<size_t>(tile & 15) * kTiledTileBytes);
+    };
+
+    auto convert = [&](int c) {
+        const int clen = chunk_len(c);
+        int cl = lane;  // (opaque copy: the slab addresses are not worth registers across the stage loop)
+        asm volatile("" : "+v"(cl));
+#pragma unroll
+        for (int r = 0; r < kItems; r++) {
+            asm volatile("" : "+v"(raw_a[r]));
+            if (Q4KX8<XT>::kLoads == 2) asm volatile("" : "+v"(raw_b[r]));
+            const int v = wave + kW * r, s = v >> 3;
+            if (s < clen) {
+                const int m = 8 * ((v >> 2) & 1) + (cl >> 3), c8 = 8 * (v & 3) + (cl & 7);
+                const int j = c8 >> 2, quarter = c8 & 3;  // sub-block, eight-value unit in it
+                uint8_t *stage = slab + s * kTiledStageX;
+                _Float16 h[8];
+                q4k_x8_to_half(raw_a[r], raw_b[r], h);
+                const half8_t frag = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+                *reinterpret_cast<half8_t *>(stage + (4 * (j & 1) + quarter) * kTiledFragStride + (16 * (j >> 1) + m) * 16) = frag;
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) sum += static_cast<float>(h[i]);
+                sum = q4k_quad_sum(sum);
+                if (quarter == 0) {
+                    const _Float16 hi = static_cast<_Float16>(sum), lo = static_cast<_Float16>(sum - static_cast<float>(hi));
+                    _Float16 *tw = reinterpret_cast<_Float16 *>(stage + 8 * kTiledFragStride) + (m + 16 * (j >> 1)) * 4 + (j & 1);
+                    tw[0] = hi;
+                    tw[2] = lo;
+                }
+            }
+        }
+    };
+
+    // ---- this wave's weight stream: for every round it takes part in, chunk by chunk, gate then up, stage by stage ----
+    // (Measured and not kept: a workgroup with k < 16 units letting its k waves divide the ring area among them, rings
+    // up to 48 / k stages deep, filled at once or one extra stage per stage computed: 21.6 -> 22.9 us for 31 experts'
+    // gate/up.  A lightly loaded wave is not waiting for memory but for its own stage, ~0.7 us of dependent LDS reads,
+    // unpacking and MFMAs with nothing else on its SIMD to overlap.)
+    constexpr int depth = kSlabRing;
+    half8_t *my_ring = ring + wave * (depth * kSlabWavePieces);
+    int it_r = 0, it_c = 0, it_h = h_begin, it_s = 0;
+    bool it_valid = false;
+    const uint8_t *it_base0 = nullptr, *it_base1 = nullptr;
+    auto it_seek = [&]() {  // the first round at or after it_r with a unit for this wave
+        int slot = 0, tile = 0;
+        while (it_r < n_rounds && !unit_of(it_r, slot, tile)) it_r++;
+        it_valid = it_r < n_rounds;
+        if (it_valid) {
+            it_base0 = tile_base(slot, tile, 0);
+            if (bt.pair) it_base1 = tile_base(slot, tile, 1);
+        }
+    };
+    int w_issued = 0, w_done = 0, ring_i = 0, ring_c = 0;
+    auto issue = [&]() {  // the stream's next stage (144 pieces) into the ring
+        const uint8_t *src = (it_h ? it_base1 : it_base0) + static_cast<size_t>(it_c * kExpChunk + it_s) * kTiledStageBytes +
+                             static_cast<size_t>(lane) * 16;
+        half8_t *buf = my_ring + ring_i * kSlabWavePieces;
+        __builtin_amdgcn_global_load_lds((gptr_t)(src), (lptr_t)(buf), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(src + 1024), (lptr_t)(buf + 64), 16, 0, 0);
+        if (lane < 16) __builtin_amdgcn_global_load_lds((gptr_t)(src + 2048), (lptr_t)(buf + 128), 16, 0, 0);
+        w_issued++;
+        ring_i = ring_i + 1 == depth ? 0 : ring_i + 1;
+        if (++it_s < chunk_len(it_c)) return;
+        it_s = 0;
+        if (++it_h < h_end) return;
+        it_h = h_begin;
+        if (++it_c < n_chunks) return;
+        it_c = 0;
+        it_r++;
+        it_seek();
+    };
+
+    // ---- prologue: the first activations (oldest loads), two weight stages, then the slab ----
+    int slab_slot = xslot_of(0), slab_chunk = 0;
+    load_x(slab_slot, 0);
+    it_seek();
+    for (int t = 0; t < 2; t++)
+        if (it_valid) issue();
+    q4k_wait_vm(3 * w_issued);  // the activations are older than every weight load
+    convert(0);
+    __builtin_amdgcn_s_waitcnt(kWaitLds);
+    __builtin_amdgcn_s_barrier();
+    bool x_pending = false;  // activations of the next refill are on their way (issued when w_issued was x_pos)
+    int x_pos = 0;
+
+    const int n = lane & 15, g = lane >> 4;
+    const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
+    const Q4KMagic magic = q4k_magic();
+    for (int r = 0; r < n_rounds; r++) {
+        int slot = 0, tile = 0;
+        const bool active = unit_of(r, slot, tile);
+        const int xslot = xslot_of(r);
+        float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+        for (int c = 0; c < n_chunks; c++) {
+            if (xslot != slab_slot || c != slab_chunk) {
+                __builtin_amdgcn_s_barrier();  // every wave has read what it needed of the old slab
+                if (x_pending) q4k_wait_vm(3 * min(w_issued - x_pos, w_issued - w_done));
+                x_pending = false;
+                convert(c);
+                __builtin_amdgcn_s_waitcnt(kWaitLds);
+                __builtin_amdgcn_s_barrier();
+                slab_slot = xslot;
+                slab_chunk = c;
+            }
+            // the activations of the step after this one, if they differ, start now
+            {
+                int nslot = -1, nc = 0;
+                if (c + 1 < n_chunks) {
+                    nslot = xslot;
+                    nc = c + 1;
+                } else if (r + 1 < n_rounds) {
+                    nslot = xslot_of(r + 1);
+                }
+                if (nslot >= 0 && (nslot != slab_slot || nc != slab_chunk)) {
+                    load_x(nslot, nc);
+                    x_pending = true;
+                    x_pos = w_issued;
+                }
+            }
+            while (w_issued - w_done < depth && it_valid) issue();  // (fills the ring once, after the prologue)
+            if (!active) continue;
+            const int clen = chunk_len(c);
+            for (int h = h_begin; h < h_end; h++) {
+                for (int s = 0; s < clen; s++) {
+                    // stage w_done has landed when only younger loads are in flight
+                    const bool x_younger = x_pending && x_pos > w_done;
+                    q4k_wait_vm(3 * (w_issued - 1 - w_done) + (x_younger ? kXInstr : 0));
+                    if (!x_younger) x_pending = false;
+                    const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(my_ring + ring_c * kSlabWavePieces) + n * 9;
+                    if (h == 0)
+                        q4k_experts_compute(blk, slab + s * kTiledStageX, lane, g, sc_sel, magic, acc0);
+                    else
+                        q4k_experts_compute(blk, slab + s * kTiledStageX, lane, g, sc_sel, magic, acc1);
+                    w_done++;
+                    ring_c = ring_c + 1 == depth ? 0 : ring_c + 1;
+                    if (it_valid) issue();  // the next stage into the buffer this one has just been read out of
+                }
+            }
+        }
+        if (hsplit) {  // the up tile crosses to the wave that holds the gate tile
+            float4_t *xchg = reinterpret_cast<float4_t *>(reinterpret_cast<uint8_t *>(lds) + kExpRingEnd) + (wave & 7) * 64 + lane;
+            if (active && wave >= kW / 2) *xchg = acc1;
+            __builtin_amdgcn_s_waitcnt(kWaitLds);
+            __builtin_amdgcn_s_barrier();
+            if (active && wave < kW / 2) acc1 = *xchg;
+        }
+        if (active && !(hsplit && wave >= kW / 2)) {
+            float4_t res = acc0;
+            if (bt.pair) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) res[i] = res[i] / (1.0f + expf(-res[i])) * acc1[i];  // silu(gate) * up
+            }
+            // (rare path: an opaque copy of the lane index keeps its address arithmetic out of the stage loop's registers)
+            int ol = lane;
+            asm volatile("" : "+v"(ol));
+            const int on = ol & 15, og = ol >> 4;
+            YT *yo = y + static_cast<size_t>(slot) * bt.y_stride;
+            const int orow = tile * 16 + on;
+            if (orow < n_out) {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (4 * og + i < n_rows) yo[static_cast<size_t>(4 * og + i) * n_out + orow] = static_cast<YT>(res[i]);
+            }
+        }
+    }
 }
 
 // ----------------------------------------------------------------------------
@@ -1928,6 +2299,42 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     const int tiles = static_cast<int>((n_out + 15) / 16);
     if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
+    if (batch && dfl_q4k_batched_f16_out(ctx, tiled, batch->whole_groups, n_out)) {
+        // whole-K batch over tiled matrices: one 16-row tile per wave (gemm_q4k_experts_kernel)
+        if (reinterpret_cast<uintptr_t>(x) % 16)
+            return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_q4k_batched: activations must be 16-byte aligned");
+        const bool per_slot_x = batch->x_stride != 0;
+        const int upm = per_slot_x ? (tiles + 15) / 16 : tiles;  // units per matrix
+        int n_wg = env_int("DFLASH_MOE_WGS", ctx->n_cu);
+        if (n_wg < 1) n_wg = 1;
+        if (static_cast<int64_t>(max_slots) * upm * (n_wg + 1) >= (int64_t(1) << 31) || nb > 4096)
+            return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: batch too large for 32-bit work indices");
+        Q4KBatch bt = *batch;
+        bt.by_wg = q4k_make_div(static_cast<uint32_t>(n_wg));
+        const Q4KDiv by_upm = q4k_make_div(static_cast<uint32_t>(upm));
+        const uint8_t *wb = static_cast<const uint8_t *>(w);
+        const int no = static_cast<int>(n_out);
+#define DFL_LAUNCH_EXPERTS(XT, YT)                                                                                          \
+    do {                                                                                                                    \
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(gemm_q4k_experts_kernel<XT, YT>), kExpLdsBytes)) \
+            return rc_;                                                                                                     \
+        dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                               \
+        gemm_q4k_experts_kernel<XT, YT><<<n_wg, 64 * kSlabWaves, kExpLdsBytes, st>>>(wb, static_cast<const XT *>(x), reinterpret_cast<YT *>(y), \
+                                                                                    no, nb, n_rows, bt, upm, by_upm, max_slots); \
+    } while (0)
+        if (x_type == DFLASH_TYPE_F32 && !bt.y_f16)
+            DFL_LAUNCH_EXPERTS(float, float);
+        else if (x_type == DFLASH_TYPE_F32)
+            DFL_LAUNCH_EXPERTS(float, _Float16);
+        else if (!bt.y_f16)
+            DFL_LAUNCH_EXPERTS(_Float16, float);
+        else
+            DFL_LAUNCH_EXPERTS(_Float16, _Float16);
+#undef DFL_LAUNCH_EXPERTS
+        DFL_HIP_CHECK(ctx, hipGetLastError());
+        return DFLASH_OK;
+    }
+    if (batch && batch->y_f16) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_q4k_batched: f16 output needs the tiled whole-K path");
     // A single matrix: 16-wave workgroups (256 weight rows per stage) when that still leaves every CU
     // a few stages of work, else 8-wave ones.  A batch is cut at tile-group boundaries only, so the
     // finer 8-wave groups balance it better (measured: the two expert launches of a 35B-A3B-shaped
@@ -1947,7 +2354,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     if (tiled && !batch) waves = 16;  // a single tiled matrix: whole 256-row tile groups (a batch may use their halves)
     const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
     const int groups = gpm * max_slots * ((batch && batch->pair) ? 2 : 1);  // upper bound in batched mode (pair mode: virtual groups)
-    int n_wg = env_int("DFLASH_GEMM_WGS", ctx->n_cu);
+    int n_wg = batch ? env_int("DFLASH_MOE_WGS", ctx->n_cu) : env_int("DFLASH_GEMM_WGS", ctx->n_cu);
     const int64_t total = static_cast<int64_t>(groups) * nb;
     const int max_wgs = ctx->n_partial_wgs * 8 / waves;
     if (n_wg > total) n_wg = static_cast<int>(total);
@@ -2116,12 +2523,18 @@ int32_t launch_q6k_stream(dflash_ctx *ctx, const void *w, const void *x, int32_t
 
 }  // namespace
 
+bool dfl_q4k_batched_f16_out(const dflash_ctx *ctx, int32_t tiled, int32_t whole_groups, int64_t n_out) {
+    return tiled && whole_groups && n_out % 16 == 0 && kExpLdsBytes <= ctx->lds_bytes && env_int("DFLASH_MOE_EXPERTS_KERNEL", 1);
+}
+
 int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const void *extra_w,
                              const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
                              size_t x_stride,
-                             float *y, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
+                             void *y, int32_t y_type, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
                              int32_t whole_groups, const void *w_stack_up, const void *extra_w_up, int32_t tiled,
                              dflash_stream_t stream) {
+    if (y_type != DFLASH_TYPE_F32 && y_type != DFLASH_TYPE_F16)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_q4k_batched: output type %d", y_type);
     if (n_in % DFL_QK_K || n_in <= 0 || n_out <= 0 || n_rows < 1 || n_rows > 16 || max_slots < 1)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_q4k_batched: bad shape");
     if (reinterpret_cast<uintptr_t>(w_stack) % 16 || reinterpret_cast<uintptr_t>(extra_w) % 16 || w_stride_bytes % 16 || (x_stride * (x_type == DFLASH_TYPE_F32 ? 4 : 2)) % 16 ||
@@ -2140,7 +2553,9 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
     bt.x_stride = x_stride;
     bt.y_stride = y_stride;
     bt.whole_groups = whole_groups;
-    return launch_q4k(ctx, w_stack, x, x_type, y, n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt, max_slots, tiled != 0);
+    bt.y_f16 = y_type == DFLASH_TYPE_F16;
+    return launch_q4k(ctx, w_stack, x, x_type, static_cast<float *>(y), n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt,
+                      max_slots, tiled != 0);
 }
 
 namespace {

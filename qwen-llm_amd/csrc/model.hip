@@ -919,7 +919,7 @@ int32_t draft_prepare(dflash_ctx *ctx, const dflash_draft_head *head, dflash_dra
         for (int64_t c0 = s->kv_ready; c0 < s->ctx_len; c0 += 16) {
             const int m = static_cast<int>(std::min<int64_t>(16, s->ctx_len - c0));
             if ((rc = dfl_gemm_q4k_batched(ctx, head->layers[0].wk.data, w_stride, nullptr, s->layer_ids, s->n_layers_dev, c.n_layers,
-                                           s->ctx_h + c0 * H, DFLASH_TYPE_F32, 0, s->pk_layers, static_cast<size_t>(16) * 2 * kv_dim, H,
+                                           s->ctx_h + c0 * H, DFLASH_TYPE_F32, 0, s->pk_layers, DFLASH_TYPE_F32, static_cast<size_t>(16) * 2 * kv_dim, H,
                                            2 * static_cast<int64_t>(kv_dim), m, 1, nullptr, nullptr, tiled ? 1 : 0, st)))
                 return rc;
             ctx_kv_finish_kernel<<<dim3(2 * c.n_kv, m, c.n_layers), 64, 0, st>>>(
@@ -927,7 +927,6 @@ int32_t draft_prepare(dflash_ctx *ctx, const dflash_draft_head *head, dflash_dra
                 s->vt16, static_cast<size_t>(s->cap16) * kv_dim, s->cap16, s->pos_ctx + c0, c0, c.n_kv, hd, c.eps, c.rope_theta);
         }
     }
-    const float *pending_resid = nullptr;
     for (int il = 0; il < c.n_layers && !layers_batched; il++) {
         const dflash_draft_layer &L = head->layers[il];
         float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;

@@ -544,12 +544,15 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         const size_t per_slot = static_cast<size_t>(16) * fe;
         // gate and up of every selected expert in one launch, silu(gate) * up applied to the tiles
         // while they are still in registers
+        // (handed to the down product as f16 where the path writes it: the down kernel rounds its activations to f16
+        // as it loads them, so the bits it computes with are the same and the hand-off is half the size)
+        const int32_t mid_type = dfl_q4k_batched_f16_out(ctx, tiled ? 1 : 0, 1, fe) ? DFLASH_TYPE_F16 : DFLASH_TYPE_F32;
         if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, stride_in, fold ? L.gate.data : nullptr, s.ids,
-                                       s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, per_slot, H, fe, n, 1,
+                                       s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, mid_type, per_slot, H, fe, n, 1,
                                        L.up_exps.data, fold ? L.up.data : nullptr, tiled ? 1 : 0, st)))
             return rc;
         if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, stride_dn, fold ? L.down.data : nullptr, s.ids,
-                                       s.n_distinct, max_slots, s.gate_out, DFLASH_TYPE_F32, per_slot, s.eo,
+                                       s.n_distinct, max_slots, s.gate_out, mid_type, per_slot, s.eo, DFLASH_TYPE_F32,
                                        static_cast<size_t>(16) * H, fe, H, n, 1, nullptr, nullptr, tiled ? 1 : 0, st)))
             return rc;
     } else {

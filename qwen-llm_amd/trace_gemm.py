@@ -31,13 +31,18 @@ def build():
     objs, procs = [], []
     for src in b.sources():
         obj = os.path.join(TRACE_DIR, os.path.basename(src)[:-4] + ".o")
-        cmd = [b.HIPCC] + [f for f in b.FLAGS if f != "-shared"] + ["-DDFLASH_TRACE", "-c", src, "-o", obj]
+        cmd = [b.HIPCC] + [f for f in b.FLAGS if f != "-shared"] + [b.RESOURCE_FLAG, "-DDFLASH_TRACE", "-c", src, "-o", obj]
         procs.append(subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
         objs.append(obj)
     for p in procs:
         out, _ = p.communicate()
         if p.returncode:
-            sys.exit(out)
+            sys.exit(b.strip_remarks(out))
+        # the stamps cost registers: a kernel that starts to spill with them may save a register an asm load is still
+        # filling (see build.py), so such a build is refused, not run
+        bad = b.check_no_scratch(out)
+        if bad:
+            sys.exit("the trace build spills in kernels that keep loads in flight; not usable:\n  " + "\n  ".join(bad))
     subprocess.check_call([b.HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", TRACE_LIB] + objs)
     for o in objs:
         os.remove(o)

@@ -65,10 +65,12 @@ def test_moe_128_experts_verify_matches_oracle(ctx, oracle, weights):
     sess.close()
 
 
-def test_tiled_expert_stacks_are_bit_identical_to_row_order(ctx, weights):
+def test_tiled_expert_stacks_agree_with_row_order(ctx, weights):
     """The expert stacks and the shared expert of this shape (768 and 2048 rows per expert: multiples of 256) are
-    uploaded in the tiled order; that is a permutation of whole blocks read by the same kernel with the same split
-    of work, so every output bit equals the row-order upload's, for a full block and for a ragged one."""
+    uploaded in the tiled order and run through the expert kernel (one 16-row tile per wave, minima through the
+    activations' sub-block sums); the row-order upload of the same bytes runs the streaming kernel's batched mode.
+    Same weights, same f16 rounding of the activations, different order of the f32 sums: the two agree far inside the
+    tolerance either has against the CPU restatement, for a full block and for ragged ones."""
     tiled = dfl.TargetModel(ctx, C5, weights)
     rows = dfl.TargetModel(ctx, C5, weights, tiled=False)
     assert tiled.tiled_tensors > 0 and rows.tiled_tensors == 0
@@ -79,11 +81,30 @@ def test_tiled_expert_stacks_are_bit_identical_to_row_order(ctx, weights):
         blk = rng.integers(0, C5.vocab, n).tolist()
         a = s_t.encode_packed_verify_layer_major(blk, pos, want_logits=True)
         b = s_r.encode_packed_verify_layer_major(blk, pos, want_logits=True)
-        assert np.array_equal(a.hidden_capture.cpu().numpy(), b.hidden_capture.cpu().numpy()), f"hidden n={n}"
-        assert np.array_equal(a.logits.cpu().numpy(), b.logits.cpu().numpy()), f"logits n={n}"
+        close(a.hidden_capture.cpu().numpy(), b.hidden_capture.cpu().numpy(), f"tiled vs row order, hidden n={n}", tol=5e-3, l2_tol=1e-3)
+        close(a.logits.cpu().numpy(), b.logits.cpu().numpy(), f"tiled vs row order, logits n={n}", tol=5e-3, l2_tol=1e-3)
         pos += n
     s_t.close()
     s_r.close()
+
+
+def test_expert_kernel_rows_do_not_depend_on_the_rest_of_the_block(ctx, weights):
+    """A row verified alone and the same row at the head of a 16-row block (other rows, so other experts, around it)
+    give the same result: every (row, expert) product of the expert kernel is one wave's whole-K sum in a fixed order,
+    and rows past the block's end are never stored.  (Compared to 1e-4: the attention kernel splits the keys by the
+    block's last position, so its f32 sums are not ordered identically in the two calls.)"""
+    model = dfl.TargetModel(ctx, C5, weights)
+    rng = np.random.default_rng(11)
+    blk = rng.integers(0, C5.vocab, 16).tolist()
+    s_blk, s_one = dfl.Session(ctx, model, 64, TAPS), dfl.Session(ctx, model, 64, TAPS)
+    a = s_blk.encode_packed_verify_layer_major(blk, 0, want_logits=True)
+    hid, lo = a.hidden_capture.cpu().numpy(), a.logits.cpu().numpy()
+    b = s_one.encode_packed_verify_layer_major(blk[:1], 0, want_logits=True)
+    close(b.hidden_capture.cpu().numpy()[:1], hid[:1], "row alone vs in a block, hidden", tol=1e-4, l2_tol=1e-5)
+    close(b.logits.cpu().numpy()[:1], lo[:1], "row alone vs in a block, logits", tol=1e-4, l2_tol=1e-5)
+    assert b.argmax_host[0] == a.argmax_host[0]
+    s_blk.close()
+    s_one.close()
 
 
 def test_generate_on_the_moe_shape_equals_serial_greedy(ctx, weights):
