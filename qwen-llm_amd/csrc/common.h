@@ -162,9 +162,21 @@ int32_t dfl_gemm_q6k_set(dflash_ctx *ctx, int n_mats, const void *const *w, floa
 // y_type: DFLASH_TYPE_F32, or DFLASH_TYPE_F16 (y then points to f16 and y_stride counts f16 elements) where
 // dfl_q4k_batched_f16_out() says the path that will run can write it.  Enqueue only.
 bool dfl_q4k_batched_f16_out(const dflash_ctx *ctx, int32_t tiled, int32_t whole_groups, int64_t n_out);
+// Routing folded into the launch (route != null; where dfl_q4k_batched_can_route() allows it): ids and n_slots are
+// then OUTPUTS.  Every workgroup derives the block's expert list from the router logits itself (the arithmetic of
+// the stand-alone routing kernel, n_expert <= 256), workgroup 0 writes ids, *n_slots, sel_e, sel_w and slot_of for
+// the launches that follow; the shared-expert gate is not computed here.
+struct dfl_route_args {
+    const float *logits;  // [n_rows][n_expert]
+    int32_t n_expert, n_used, with_shared;
+    int32_t *sel_e;   // [n_rows][n_used]
+    float *sel_w;     // [n_rows][n_used]
+    int32_t *slot_of; // [n_rows][n_used]
+};
+bool dfl_q4k_batched_can_route(const dflash_ctx *ctx, int32_t tiled, int64_t n_out, int32_t n_expert, int32_t n_used);
 int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stride_bytes, const void *extra_w,
                              const int32_t *ids, const int32_t *n_slots, int max_slots, const void *x, int32_t x_type,
                              size_t x_stride,
                              void *y, int32_t y_type, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
                              int32_t whole_groups, const void *w_stack_up, const void *extra_w_up, int32_t tiled,
-                             dflash_stream_t stream);
+                             dflash_stream_t stream, const dfl_route_args *route = nullptr);

@@ -24,6 +24,7 @@
 //  * Q6_K has its own kernel (half a super-block per step, see there); Q8_0 uses a simple one:
 //    eight consecutive weights per lane are dequantised to f16 and fed to the same MFMA.
 #include "common.h"
+#include "moe_route.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -222,6 +223,11 @@ struct Q4KBatch {
     int pair;
     const uint8_t *w2, *extra_w2;
     int y_f16;  // the output is f16 (gemm_q4k_experts_kernel only)
+    // routing folded into gemm_q4k_experts_kernel (route_logits != null): ids / n_slots are written, not read
+    const float *route_logits;
+    int route_experts, route_used, route_shared;
+    int32_t *route_sel_e, *route_slot_of;
+    float *route_sel_w;
 };
 
 // Tiled order (see gemm_q4k_tiled_kernel): one wave's 16 rows of a stage, and a whole 256-row stage, in bytes.
@@ -1311,7 +1317,9 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
 constexpr int kExpChunk = 4;  // stages of activations in LDS at a time
 constexpr size_t kExpRingEnd = static_cast<size_t>(kExpChunk) * kTiledStageX +
                                static_cast<size_t>(kSlabWaves) * kSlabRing * kSlabWavePieces * 16;
-constexpr size_t kExpLdsBytes = kExpRingEnd + (kSlabWaves / 2) * 64 * sizeof(float4_t);  // + the up tiles of split pairs
+constexpr size_t kExpXchgEnd = kExpRingEnd + (kSlabWaves / 2) * 64 * sizeof(float4_t);  // + the up tiles of split pairs
+constexpr int kExpRouteIds = 264;  // expert list of a routed launch: at most 256 experts + the shared one
+constexpr size_t kExpLdsBytes = kExpXchgEnd + 16 * 4 * sizeof(unsigned long long) + kExpRouteIds * sizeof(int32_t);
 static_assert(kExpLdsBytes <= 160 * 1024, "one workgroup per CU, all of its LDS");
 
 // q4k_tiled_compute for the expert kernel, which carries more state per lane (activations on their way for the next
@@ -1359,7 +1367,7 @@ __device__ __forceinline__ void q4k_experts_compute(const u32x4_t *blk, const ui
     }
 }
 
-template <typename XT, typename YT>
+template <typename XT, typename YT, bool kRoute>
 __global__ void __launch_bounds__(64 * kSlabWaves)
     gemm_q4k_experts_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, YT *__restrict__ y, int n_out, int nb,
                             int n_rows, Q4KBatch bt, int upm, Q4KDiv by_upm, int max_slots) {
@@ -1393,7 +1401,52 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
             q4k_load_x8(xb + static_cast<size_t>(sb) * (DFL_QK_K * sizeof(XT)), x_off[r], raw_a[r], raw_b[r]);
         }
     };
-    const int n_slots = min(*bt.n_slots, max_slots);  // (the bound the host sized the buffers for)
+    int32_t *ids_lds = reinterpret_cast<int32_t *>(reinterpret_cast<uint8_t *>(lds) + kExpXchgEnd + 16 * 4 * sizeof(unsigned long long));
+    int n_slots;
+    if constexpr (kRoute) {
+        // The block's routing, by every workgroup for itself: wave w takes row w (dfl_route::route_row, the arithmetic
+        // of the stand-alone kernel), the union of the rows' masks gives the ascending expert list, kept in LDS.
+        // The shared activations are on their way meanwhile.
+        load_x(0, 0);
+        unsigned long long *row_mask = reinterpret_cast<unsigned long long *>(reinterpret_cast<uint8_t *>(lds) + kExpXchgEnd);
+        const int E = bt.route_experts, used = bt.route_used;
+        dfl_route::RowPicks pk;
+        pk.my_e = 0;
+        pk.my_w = 0.0f;
+        pk.m[0] = pk.m[1] = pk.m[2] = pk.m[3] = 0;
+        if (wave < n_rows) pk = dfl_route::route_row(bt.route_logits + static_cast<size_t>(wave) * E, E, used, lane);
+        if (lane < 4) row_mask[wave * 4 + lane] = dfl_route::pick4(pk.m, lane);
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        __builtin_amdgcn_s_barrier();
+        unsigned long long un[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) un[j] |= row_mask[r * 4 + j];
+        const int total = __popcll(un[0]) + __popcll(un[1]) + __popcll(un[2]) + __popcll(un[3]);
+        n_slots = min(total + (bt.route_shared ? 1 : 0), max_slots);
+        const bool listed = tid < E && ((dfl_route::pick4(un, tid >> 6) >> (tid & 63)) & 1);
+        const int my_slot = listed ? dfl_route::slot_below(un, tid) : 0;
+        if (listed) ids_lds[my_slot] = tid;
+        if (tid == 0 && bt.route_shared) ids_lds[total] = -1;
+        if (blockIdx.x == 0) {  // one copy for the launches that follow
+            int32_t *ids_out = const_cast<int32_t *>(bt.ids);
+            if (listed) ids_out[my_slot] = tid;
+            if (tid == 0) {
+                if (bt.route_shared) ids_out[total] = -1;
+                *const_cast<int32_t *>(bt.n_slots) = n_slots;
+            }
+            if (wave < n_rows && lane < used) {
+                bt.route_sel_e[wave * used + lane] = pk.my_e;
+                bt.route_sel_w[wave * used + lane] = pk.my_w;
+                bt.route_slot_of[wave * used + lane] = dfl_route::slot_below(un, pk.my_e);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        __builtin_amdgcn_s_barrier();
+    } else {
+        n_slots = min(*bt.n_slots, max_slots);  // (the bound the host sized the buffers for)
+    }
     const int tiles = (n_out + 15) >> 4;
     const int halves = bt.pair ? 2 : 1;
     const int n_chunks = (nb + kExpChunk - 1) / kExpChunk;
@@ -1416,6 +1469,10 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     int slot_base = -64;  // no window yet: the first use (before any weight load is issued) reads it
     int32_t ids_window = 0;
     auto slot_id = [&](int j) {
+        if constexpr (kRoute) {  // the list is in LDS; whatever it holds, the index stays inside the stack
+            const int32_t id = __builtin_amdgcn_readfirstlane(ids_lds[min(max(j, 0), kExpRouteIds - 1)]);
+            return min(max(id, -1), bt.route_experts - 1);
+        }
         if (j < slot_base || j >= slot_base + 64) {
             slot_base = j;
             ids_window = bt.ids[min(j + lane, n_slots - 1)];
@@ -1517,7 +1574,7 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
 
     // ---- prologue: the first activations (oldest loads), two weight stages, then the slab ----
     int slab_slot = xslot_of(0), slab_chunk = 0;
-    load_x(slab_slot, 0);
+    if (!kRoute) load_x(slab_slot, 0);
     it_seek();
     for (int t = 0; t < 2; t++)
         if (it_valid) issue();
@@ -2299,8 +2356,12 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     const int tiles = static_cast<int>((n_out + 15) / 16);
     if (reinterpret_cast<uintptr_t>(x) % (x_type == DFLASH_TYPE_F32 ? 16 : 8))
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: activations must be 16-byte (f32) / 8-byte (f16) aligned");
-    if (batch && dfl_q4k_batched_f16_out(ctx, tiled, batch->whole_groups, n_out)) {
-        // whole-K batch over tiled matrices: one 16-row tile per wave (gemm_q4k_experts_kernel)
+    // whole-K batch over tiled matrices: one 16-row tile per wave (gemm_q4k_experts_kernel).  A plain product over a
+    // shared x with less than two tiles per wave-slot of the chip (a drafter's five [wk; wv] pairs: 320 tiles) stays
+    // with the streaming kernel: every workgroup of the expert kernel converts all of x for one or two tiles
+    // (14.2 against 11.4 us for that launch).
+    if (batch && dfl_q4k_batched_f16_out(ctx, tiled, batch->whole_groups, n_out) &&
+        (batch->pair || batch->x_stride != 0 || batch->y_f16 || batch->route_logits || static_cast<int64_t>(max_slots) * tiles >= 2ll * ctx->n_cu)) {
         if (reinterpret_cast<uintptr_t>(x) % 16)
             return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_q4k_batched: activations must be 16-byte aligned");
         const bool per_slot_x = batch->x_stride != 0;
@@ -2314,27 +2375,36 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         const Q4KDiv by_upm = q4k_make_div(static_cast<uint32_t>(upm));
         const uint8_t *wb = static_cast<const uint8_t *>(w);
         const int no = static_cast<int>(n_out);
-#define DFL_LAUNCH_EXPERTS(XT, YT)                                                                                          \
+#define DFL_LAUNCH_EXPERTS(XT, YT, ROUTE)                                                                                   \
     do {                                                                                                                    \
-        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(gemm_q4k_experts_kernel<XT, YT>), kExpLdsBytes)) \
+        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(gemm_q4k_experts_kernel<XT, YT, ROUTE>), kExpLdsBytes)) \
             return rc_;                                                                                                     \
         dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                               \
-        gemm_q4k_experts_kernel<XT, YT><<<n_wg, 64 * kSlabWaves, kExpLdsBytes, st>>>(wb, static_cast<const XT *>(x), reinterpret_cast<YT *>(y), \
-                                                                                    no, nb, n_rows, bt, upm, by_upm, max_slots); \
+        gemm_q4k_experts_kernel<XT, YT, ROUTE><<<n_wg, 64 * kSlabWaves, kExpLdsBytes, st>>>(wb, static_cast<const XT *>(x), reinterpret_cast<YT *>(y), \
+                                                                                           no, nb, n_rows, bt, upm, by_upm, max_slots); \
     } while (0)
-        if (x_type == DFLASH_TYPE_F32 && !bt.y_f16)
-            DFL_LAUNCH_EXPERTS(float, float);
+        if (bt.route_logits) {
+            if (x_type != DFLASH_TYPE_F32 || per_slot_x || bt.route_experts > 256 || bt.route_experts < 1 || bt.route_used < 1 ||
+                bt.route_used > 64 || bt.route_used > bt.route_experts || max_slots + 0 > kExpRouteIds - 1)
+                return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_q4k_batched: routing inside the launch needs f32 shared activations and at most 256 experts");
+            if (bt.y_f16)
+                DFL_LAUNCH_EXPERTS(float, _Float16, true);
+            else
+                DFL_LAUNCH_EXPERTS(float, float, true);
+        } else if (x_type == DFLASH_TYPE_F32 && !bt.y_f16)
+            DFL_LAUNCH_EXPERTS(float, float, false);
         else if (x_type == DFLASH_TYPE_F32)
-            DFL_LAUNCH_EXPERTS(float, _Float16);
+            DFL_LAUNCH_EXPERTS(float, _Float16, false);
         else if (!bt.y_f16)
-            DFL_LAUNCH_EXPERTS(_Float16, float);
+            DFL_LAUNCH_EXPERTS(_Float16, float, false);
         else
-            DFL_LAUNCH_EXPERTS(_Float16, _Float16);
+            DFL_LAUNCH_EXPERTS(_Float16, _Float16, false);
 #undef DFL_LAUNCH_EXPERTS
         DFL_HIP_CHECK(ctx, hipGetLastError());
         return DFLASH_OK;
     }
-    if (batch && batch->y_f16) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_q4k_batched: f16 output needs the tiled whole-K path");
+    if (batch && (batch->y_f16 || batch->route_logits))
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_q4k_batched: f16 output and routing inside the launch need the tiled whole-K path");
     // A single matrix: 16-wave workgroups (256 weight rows per stage) when that still leaves every CU
     // a few stages of work, else 8-wave ones.  A batch is cut at tile-group boundaries only, so the
     // finer 8-wave groups balance it better (measured: the two expert launches of a 35B-A3B-shaped
@@ -2523,6 +2593,11 @@ int32_t launch_q6k_stream(dflash_ctx *ctx, const void *w, const void *x, int32_t
 
 }  // namespace
 
+bool dfl_q4k_batched_can_route(const dflash_ctx *ctx, int32_t tiled, int64_t n_out, int32_t n_expert, int32_t n_used) {
+    return dfl_q4k_batched_f16_out(ctx, tiled, 1, n_out) && n_expert >= 1 && n_expert <= 256 && n_used >= 1 && n_used <= 64 &&
+           n_used <= n_expert && env_int("DFLASH_MOE_FUSED_ROUTE", 1);
+}
+
 bool dfl_q4k_batched_f16_out(const dflash_ctx *ctx, int32_t tiled, int32_t whole_groups, int64_t n_out) {
     return tiled && whole_groups && n_out % 16 == 0 && kExpLdsBytes <= ctx->lds_bytes && env_int("DFLASH_MOE_EXPERTS_KERNEL", 1);
 }
@@ -2532,7 +2607,7 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
                              size_t x_stride,
                              void *y, int32_t y_type, size_t y_stride, int64_t n_in, int64_t n_out, int32_t n_rows,
                              int32_t whole_groups, const void *w_stack_up, const void *extra_w_up, int32_t tiled,
-                             dflash_stream_t stream) {
+                             dflash_stream_t stream, const dfl_route_args *route) {
     if (y_type != DFLASH_TYPE_F32 && y_type != DFLASH_TYPE_F16)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_q4k_batched: output type %d", y_type);
     if (n_in % DFL_QK_K || n_in <= 0 || n_out <= 0 || n_rows < 1 || n_rows > 16 || max_slots < 1)
@@ -2554,6 +2629,17 @@ int32_t dfl_gemm_q4k_batched(dflash_ctx *ctx, const void *w_stack, size_t w_stri
     bt.y_stride = y_stride;
     bt.whole_groups = whole_groups;
     bt.y_f16 = y_type == DFLASH_TYPE_F16;
+    if (route) {
+        if (!route->logits || !route->sel_e || !route->sel_w || !route->slot_of || x_stride != 0)
+            return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "gemm_q4k_batched: routing inside the launch needs its buffers and shared activations");
+        bt.route_logits = route->logits;
+        bt.route_experts = route->n_expert;
+        bt.route_used = route->n_used;
+        bt.route_shared = route->with_shared;
+        bt.route_sel_e = route->sel_e;
+        bt.route_sel_w = route->sel_w;
+        bt.route_slot_of = route->slot_of;
+    }
     return launch_q4k(ctx, w_stack, x, x_type, static_cast<float *>(y), n_in, n_out, n_rows, static_cast<hipStream_t>(stream), &bt,
                       max_slots, tiled != 0);
 }

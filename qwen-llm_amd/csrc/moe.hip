@@ -12,6 +12,7 @@
 // if there are none, so HBM traffic is the distinct experts of the block, not rows x k.
 #include "common.h"
 #include "device_quant.h"
+#include "moe_route.h"
 
 #include <cstdlib>
 
@@ -41,21 +42,6 @@ __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
     const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(v), 63);
     const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(v >> 32), 63);
     return (static_cast<unsigned long long>(hi) << 32) | lo;
-}
-
-// The same for a float maximum (NaN operands are ignored, as v_max_f32 does); lanes without a source
-// keep their own value.
-__device__ __forceinline__ float wave_max_f32(float v) {
-#define DFL_FMAX_STEP(ctrl, row_mask)                                                                              \
-    v = fmaxf(v, __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(v), __float_as_uint(v), ctrl, row_mask, 0xf, false)))
-    DFL_FMAX_STEP(0x111, 0xf);
-    DFL_FMAX_STEP(0x112, 0xf);
-    DFL_FMAX_STEP(0x114, 0xf);
-    DFL_FMAX_STEP(0x118, 0xf);
-    DFL_FMAX_STEP(0x142, 0xa);
-    DFL_FMAX_STEP(0x143, 0xc);
-#undef DFL_FMAX_STEP
-    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
 }
 
 // Routing of a whole block in one workgroup of sixteen waves (n_expert <= 1024, at most 16 rows).
@@ -213,9 +199,6 @@ __global__ void __launch_bounds__(1024)
     unsigned long long m[4] = {0, 0, 0, 0};
     if (live) {
         const float *lg = logits + static_cast<size_t>(row) * n_expert;
-        float lgv[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
         const float *xr = x + static_cast<size_t>(row) * hidden;
         float dot = 0.0f;
         if (!shexp_gate) {
@@ -243,56 +226,13 @@ __global__ void __launch_bounds__(1024)
         for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
         if (shexp_gate && lane == 0) sg[row] = 1.0f / (1.0f + expf(-dot));
 
-        float mx = -INFINITY;
+        const dfl_route::RowPicks pk = dfl_route::route_row(lg, n_expert, n_used, lane);
+        my_e = pk.my_e;
 #pragma unroll
-        for (int j = 0; j < 4; j++) mx = fmaxf(mx, lgv[j]);
-        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-        float pv[4];
-        float sum = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            pv[j] = 0.0f;
-            if (lane + 64 * j < n_expert) {
-                pv[j] = expf(lgv[j] - mx);
-                sum += pv[j];
-            }
-        }
-        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-        const float inv = 1.0f / sum;
-#pragma unroll
-        for (int j = 0; j < 4; j++) pv[j] = lane + 64 * j < n_expert ? pv[j] * inv : -1.0f;  // no such expert: never picked
-
-        // pick k = the highest remaining probability, equal probabilities to the lower id: a wave-wide
-        // float maximum (one DPP instruction per step), then the first lane / register that holds it,
-        // found with compares into scalar masks.  Taken and missing experts are -1, NaN never compares
-        // equal: if nothing is left (NaN logits) the pick falls back to an index in range.
-        float my_p = 0.0f;
-        for (int k = 0; k < n_used; k++) {
-            const float pmax = wave_max_f32(fmaxf(fmaxf(pv[0], pv[1]), fmaxf(pv[2], pv[3])));
-            int e_win = -1;
-#pragma unroll
-            for (int j = 3; j >= 0; j--) {
-                const unsigned long long hit = __builtin_amdgcn_ballot_w64(pv[j] == pmax);
-                if (hit) e_win = 64 * j + __builtin_ctzll(hit);
-            }
-            const bool none = !(pmax >= 0.0f) || e_win < 0;
-            if (none) e_win = k < n_expert ? k : n_expert - 1;
-            if (lane == k) {
-                my_e = e_win;
-                my_p = none ? 0.0f : pmax;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (lane + 64 * j == e_win) pv[j] = -1.0f;  // taken
-                if ((e_win >> 6) == j) m[j] |= 1ull << (e_win & 63);
-            }
-        }
-        float wsum = 0.0f;
-        for (int k = 0; k < n_used; k++) wsum += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_p), k));  // in pick order
-        wsum = fmaxf(wsum, 6.103515625e-05f);  // 2^-14
+        for (int j = 0; j < 4; j++) m[j] = pk.m[j];
         if (lane < n_used) {
             sel_e[row * n_used + lane] = my_e;
-            sel_w[row * n_used + lane] = my_p / wsum;
+            sel_w[row * n_used + lane] = pk.my_w;
         }
     }
     if (lane < 4) row_mask[row][lane] = m[lane & 3];
@@ -302,15 +242,7 @@ __global__ void __launch_bounds__(1024)
     for (int r = 0; r < 16; r++)
 #pragma unroll
         for (int j = 0; j < 4; j++) un[j] |= row_mask[r][j];
-    auto slot = [&](int e) {  // experts below e in the union
-        int below = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            if (j < (e >> 6)) below += __popcll(un[j]);
-            if (j == (e >> 6)) below += __popcll(un[j] & ((1ull << (e & 63)) - 1));
-        }
-        return below;
-    };
+    auto slot = [&](int e) { return dfl_route::slot_below(un, e); };  // experts below e in the union
     if (tid < n_expert && ((un[tid >> 6] >> (tid & 63)) & 1)) ids[slot(tid)] = tid;
     if (tid == 0) {
         const int total = __popcll(un[0]) + __popcll(un[1]) + __popcll(un[2]) + __popcll(un[3]);
@@ -529,7 +461,12 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
             return rc_;
     }
     const float *gate_w = gate_done ? nullptr : L.shexp_gate;  // null: sg is already there
-    if (E <= 256)
+    // the routing can ride in the gate/up launch (every workgroup derives the expert list itself): one launch fewer
+    const bool route_inside = batched && tiled && !gate_w && n <= 16 &&
+                              dfl_q4k_batched_can_route(ctx, 1, fe, E, used);
+    if (route_inside) {
+        // nothing to launch here
+    } else if (E <= 256)
         moe_route_small_kernel<<<1, 1024, 0, st>>>(s.probs, cur, gate_w, n, E, used, H, folded_shared ? 1 : 0, s.sel_e,
                                                    s.sel_w, s.sg, s.ids, s.n_distinct, s.slot_of);
     else
@@ -547,9 +484,10 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         // (handed to the down product as f16 where the path writes it: the down kernel rounds its activations to f16
         // as it loads them, so the bits it computes with are the same and the hand-off is half the size)
         const int32_t mid_type = dfl_q4k_batched_f16_out(ctx, tiled ? 1 : 0, 1, fe) ? DFLASH_TYPE_F16 : DFLASH_TYPE_F32;
+        const dfl_route_args route = {s.probs, E, used, folded_shared ? 1 : 0, s.sel_e, s.sel_w, s.slot_of};
         if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, stride_in, fold ? L.gate.data : nullptr, s.ids,
                                        s.n_distinct, max_slots, cur, DFLASH_TYPE_F32, 0, s.gate_out, mid_type, per_slot, H, fe, n, 1,
-                                       L.up_exps.data, fold ? L.up.data : nullptr, tiled ? 1 : 0, st)))
+                                       L.up_exps.data, fold ? L.up.data : nullptr, tiled ? 1 : 0, st, route_inside ? &route : nullptr)))
             return rc;
         if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, stride_dn, fold ? L.down.data : nullptr, s.ids,
                                        s.n_distinct, max_slots, s.gate_out, mid_type, per_slot, s.eo, DFLASH_TYPE_F32,

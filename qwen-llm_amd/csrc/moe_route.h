@@ -1,0 +1,113 @@
+// Routing of one block row by one wave, for n_expert <= 256 and n_used <= 64: softmax over the router logits, top-k
+// (higher probability first, equal probabilities to the lower expert id), renormalised weights in pick order (the
+// reference's packed route, metal_dflash.rs:10184-10403; CPU form ffn_moe, forward.rs:749-824), and the row's picked
+// experts as a 256-bit mask.  Shared by the stand-alone routing kernel (moe.hip) and the expert GEMM kernel that
+// derives the block's expert list itself (gemm_fewrow.hip): same instructions, same order, same bits.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace dfl_route {
+
+// Maximum of a float over the wave, in every lane: data-parallel-primitive moves within rows of 16 lanes (shift right
+// by 1, 2, 4, 8: lane 15 of a row then holds the row's maximum), then lane 15 of rows 0 and 2 broadcast into rows 1
+// and 3, then lane 31 into rows 2 and 3; lane 63 has the result.  NaN operands are ignored, as v_max_f32 does; lanes
+// without a source keep their own value.  No LDS round trips, unlike a shuffle.
+__device__ __forceinline__ float wave_max_f32(float v) {
+#define DFL_FMAX_STEP(ctrl, row_mask)                                                                              \
+    v = fmaxf(v, __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(v), __float_as_uint(v), ctrl, row_mask, 0xf, false)))
+    DFL_FMAX_STEP(0x111, 0xf);
+    DFL_FMAX_STEP(0x112, 0xf);
+    DFL_FMAX_STEP(0x114, 0xf);
+    DFL_FMAX_STEP(0x118, 0xf);
+    DFL_FMAX_STEP(0x142, 0xa);
+    DFL_FMAX_STEP(0x143, 0xc);
+#undef DFL_FMAX_STEP
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
+}
+
+struct RowPicks {
+    int my_e;                  // lane k < n_used: the expert of pick k
+    float my_w;                // lane k < n_used: its renormalised weight
+    unsigned long long m[4];   // the row's picked experts (every lane)
+};
+
+// lg: the row's n_expert router logits.  Called by all 64 lanes of a wave.
+__device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int n_expert, int n_used, int lane) {
+    RowPicks r;
+    r.my_e = 0;
+    r.m[0] = r.m[1] = r.m[2] = r.m[3] = 0;
+    float lgv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; j++) mx = fmaxf(mx, lgv[j]);
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float pv[4];
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        pv[j] = 0.0f;
+        if (lane + 64 * j < n_expert) {
+            pv[j] = expf(lgv[j] - mx);
+            sum += pv[j];
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int j = 0; j < 4; j++) pv[j] = lane + 64 * j < n_expert ? pv[j] * inv : -1.0f;  // no such expert: never picked
+
+    // pick k = the highest remaining probability, equal probabilities to the lower id: a wave-wide float maximum
+    // (one DPP instruction per step), then the first lane / register that holds it, found with compares into scalar
+    // masks.  Taken and missing experts are -1, NaN never compares equal: if nothing is left (NaN logits) the pick
+    // falls back to an index in range.
+    float my_p = 0.0f;
+    for (int k = 0; k < n_used; k++) {
+        const float pmax = wave_max_f32(fmaxf(fmaxf(pv[0], pv[1]), fmaxf(pv[2], pv[3])));
+        int e_win = -1;
+#pragma unroll
+        for (int j = 3; j >= 0; j--) {
+            const unsigned long long hit = __builtin_amdgcn_ballot_w64(pv[j] == pmax);
+            if (hit) e_win = 64 * j + __builtin_ctzll(hit);
+        }
+        const bool none = !(pmax >= 0.0f) || e_win < 0;
+        if (none) e_win = k < n_expert ? k : n_expert - 1;
+        if (lane == k) {
+            r.my_e = e_win;
+            my_p = none ? 0.0f : pmax;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (lane + 64 * j == e_win) pv[j] = -1.0f;  // taken
+            if ((e_win >> 6) == j) r.m[j] |= 1ull << (e_win & 63);
+        }
+    }
+    float wsum = 0.0f;
+    for (int k = 0; k < n_used; k++) wsum += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_p), k));  // in pick order
+    wsum = fmaxf(wsum, 6.103515625e-05f);  // 2^-14
+    r.my_w = my_p / wsum;
+    return r;
+}
+
+// v[i & 3] without indexing the array by a run-time value (which would move it from registers to scratch memory)
+__device__ __forceinline__ unsigned long long pick4(const unsigned long long v[4], int i) {
+    i &= 3;
+    return i == 0 ? v[0] : i == 1 ? v[1] : i == 2 ? v[2] : v[3];
+}
+
+// experts below e in the union of the rows' masks = e's slot in the block's ascending expert list
+__device__ __forceinline__ int slot_below(const unsigned long long un[4], int e) {
+    int below = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if (j < (e >> 6)) below += __popcll(un[j]);
+        if (j == (e >> 6)) below += __popcll(un[j] & ((1ull << (e & 63)) - 1));
+    }
+    return below;
+}
+
+}  // namespace dfl_route
