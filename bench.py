@@ -396,6 +396,44 @@ def e2e_speculative(ctx, n_generate, sweep, log):
     return res
 
 
+def moe_layer_probe(distinct_list, blocks=40):
+    """Verify blocks on a 4-layer 35B-A3B-shaped mixture-of-experts target (random quant blocks) whose 16 tokens are
+    drawn from `nd` distinct ones: 16 distinct random tokens touch about 80 of the 128 experts per layer, 4 about 30,
+    1 exactly 8 (+ the shared expert).  Meant to run under `rocprofv3 --kernel-trace --stats`: the expert launches
+    show up per kernel instance (gate/up: f32 in, f16 out; down: f16 in, f32 out).  Prints wall-clock per block."""
+    import numpy as np
+    import torch
+
+    import qwen_llm_amd as dfl
+
+    cfg = dfl.ModelConfig(n_layers=4, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=32000, n_expert=128,
+                          n_expert_used=8, ffn_expert=768, ffn_shared=768)
+    ctx = dfl.Context(0, workspace_bytes=256 << 20)
+    model = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_blocks(cfg, 41))
+    sess = dfl.Session(ctx, model, 4096, [0, 1])
+    rng = np.random.default_rng(5)
+    pos = 0
+    for _ in range(128):  # a 2048-token context
+        sess.encode_packed_verify_layer_major(rng.integers(0, cfg.vocab, 16).tolist(), pos)
+        pos += 16
+    out = []
+    for nd in distinct_list:
+        def block():
+            base = rng.integers(0, cfg.vocab, nd)
+            sess.encode_packed_verify_layer_major([int(base[i % nd]) for i in range(16)], pos)
+            sess.encode_restore_after_partial_accept(pos, 16, 0)
+        for _ in range(10):
+            block()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(blocks):
+            block()
+        torch.cuda.synchronize()
+        out.append({"distinct_tokens": nd, "ms_per_4_layer_verify": (time.perf_counter() - t0) / blocks * 1e3})
+    sess.close()
+    print(json.dumps({"moe_layer_probe": out}))
+
+
 def rocprof_summary(directory):
     """Text summary of a rocprofv3 CSV output directory: per-kernel durations from *_kernel_trace.csv and
     per-kernel counter averages from *_counter_collection.csv (whichever exist)."""
@@ -445,6 +483,8 @@ def main():
                     help="copies of the three weight matrices the timed loops rotate over; 3 x 118 MB exceeds the 256 MB "
                          "memory-side cache, so weights come from HBM as they do in a real model (1 = cache-resident)")
     ap.add_argument("--gemm-only", action="store_true", help="skip the attention, acceptance and end-to-end sections")
+    ap.add_argument("--moe-layer", metavar="N[,N...]", help="only run the mixture-of-experts layer probe with blocks of N "
+                                                             "distinct tokens (e.g. 16,4,1) and exit; for kernel traces")
     ap.add_argument("--shapes", default="0,1,2", help="which of the three GEMM shapes take part (for per-shape profiles; the "
                                                       "metric is defined on all three)")
     args = ap.parse_args()
@@ -455,6 +495,10 @@ def main():
         print("bench.py measures one GPU: the DFlash step is batch-1 and this build has no multi-GPU path; "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.moe_layer:
+        moe_layer_probe([int(v) for v in args.moe_layer.split(",")])
+        return
 
     import numpy as np
     import torch

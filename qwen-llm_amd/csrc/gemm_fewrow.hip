@@ -1418,11 +1418,8 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
         if (lane < 4) row_mask[wave * 4 + lane] = dfl_route::pick4(pk.m, lane);
         __builtin_amdgcn_s_waitcnt(kWaitLds);
         __builtin_amdgcn_s_barrier();
-        unsigned long long un[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) un[j] |= row_mask[r * 4 + j];
+        unsigned long long un[4];
+        dfl_route::union_of_rows(row_mask, lane, un);
         const int total = __popcll(un[0]) + __popcll(un[1]) + __popcll(un[2]) + __popcll(un[3]);
         n_slots = min(total + (bt.route_shared ? 1 : 0), max_slots);
         const bool listed = tid < E && ((dfl_route::pick4(un, tid >> 6) >> (tid & 63)) & 1);

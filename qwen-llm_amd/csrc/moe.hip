@@ -237,11 +237,8 @@ __global__ void __launch_bounds__(1024)
     }
     if (lane < 4) row_mask[row][lane] = m[lane & 3];
     __syncthreads();
-    unsigned long long un[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int r = 0; r < 16; r++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) un[j] |= row_mask[r][j];
+    unsigned long long un[4];
+    dfl_route::union_of_rows(&row_mask[0][0], lane, un);
     auto slot = [&](int e) { return dfl_route::slot_below(un, e); };  // experts below e in the union
     if (tid < n_expert && ((un[tid >> 6] >> (tid & 63)) & 1)) ids[slot(tid)] = tid;
     if (tid == 0) {

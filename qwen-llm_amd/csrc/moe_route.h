@@ -28,6 +28,21 @@ __device__ __forceinline__ float wave_max_f32(float v) {
     return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
 }
 
+// The sum over the wave by the same moves (lanes without a source add 0): lane 63 ends with
+// ((row 0 + row 1) + (row 2 + row 3)), each row summed lane 0 upwards in a tree of shifts; every lane gets that value.
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#define DFL_FADD_STEP(ctrl, row_mask) \
+    v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), ctrl, row_mask, 0xf, false))
+    DFL_FADD_STEP(0x111, 0xf);
+    DFL_FADD_STEP(0x112, 0xf);
+    DFL_FADD_STEP(0x114, 0xf);
+    DFL_FADD_STEP(0x118, 0xf);
+    DFL_FADD_STEP(0x142, 0xa);
+    DFL_FADD_STEP(0x143, 0xc);
+#undef DFL_FADD_STEP
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
+}
+
 struct RowPicks {
     int my_e;                  // lane k < n_used: the expert of pick k
     float my_w;                // lane k < n_used: its renormalised weight
@@ -45,7 +60,7 @@ __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int 
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 4; j++) mx = fmaxf(mx, lgv[j]);
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = wave_max_f32(mx);
     float pv[4];
     float sum = 0.0f;
 #pragma unroll
@@ -56,7 +71,7 @@ __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int 
             sum += pv[j];
         }
     }
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    sum = wave_sum_f32(sum);
     const float inv = 1.0f / sum;
 #pragma unroll
     for (int j = 0; j < 4; j++) pv[j] = lane + 64 * j < n_expert ? pv[j] * inv : -1.0f;  // no such expert: never picked
@@ -97,6 +112,23 @@ __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int 
 __device__ __forceinline__ unsigned long long pick4(const unsigned long long v[4], int i) {
     i &= 3;
     return i == 0 ? v[0] : i == 1 ? v[1] : i == 2 ? v[2] : v[3];
+}
+
+// The union of the sixteen rows' masks (row_mask[row * 4 + j] in LDS, complete): lane l reads word l, four xor-shuffle
+// steps OR the rows together, and words 0..3 are read back out of lanes 0..3.  Called by a whole wave.
+__device__ __forceinline__ void union_of_rows(const unsigned long long *row_mask, int lane, unsigned long long un[4]) {
+    unsigned long long v = row_mask[lane];
+    for (int off = 4; off < 64; off <<= 1) {
+        const unsigned lo = __shfl_xor(static_cast<unsigned>(v), off, 64), hi = __shfl_xor(static_cast<unsigned>(v >> 32), off, 64);
+        v |= (static_cast<unsigned long long>(hi) << 32) | lo;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        // (readlane returns int: through unsigned, or a low word with bit 31 set would smear over the high word)
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<unsigned>(v), j));
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<unsigned>(v >> 32), j));
+        un[j] = (static_cast<unsigned long long>(hi) << 32) | lo;
+    }
 }
 
 // experts below e in the union of the rows' masks = e's slot in the block's ascending expert list
