@@ -396,10 +396,11 @@ def e2e_speculative(ctx, n_generate, sweep, log):
     return res
 
 
-def moe_layer_probe(distinct_list, blocks=40):
+def moe_layer_probe(nd, blocks=60):
     """Verify blocks on a 4-layer 35B-A3B-shaped mixture-of-experts target (random quant blocks) whose 16 tokens are
     drawn from `nd` distinct ones: 16 distinct random tokens touch about 80 of the 128 experts per layer, 4 about 30,
-    1 exactly 8 (+ the shared expert).  Meant to run under `rocprofv3 --kernel-trace --stats`: the expert launches
+    1 exactly 8 (+ the shared expert).  Every block of the run (the 2048-token context included) is drawn that way,
+    so under `rocprofv3 --kernel-trace --stats` the per-kernel averages are those of one load: the expert launches
     show up per kernel instance (gate/up: f32 in, f16 out; down: f16 in, f32 out).  Prints wall-clock per block."""
     import numpy as np
     import torch
@@ -412,26 +413,25 @@ def moe_layer_probe(distinct_list, blocks=40):
     model = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_blocks(cfg, 41))
     sess = dfl.Session(ctx, model, 4096, [0, 1])
     rng = np.random.default_rng(5)
+
+    def draw():
+        base = rng.integers(0, cfg.vocab, nd)
+        return [int(base[i % nd]) for i in range(16)]
+
     pos = 0
     for _ in range(128):  # a 2048-token context
-        sess.encode_packed_verify_layer_major(rng.integers(0, cfg.vocab, 16).tolist(), pos)
+        sess.encode_packed_verify_layer_major(draw(), pos)
         pos += 16
-    out = []
-    for nd in distinct_list:
-        def block():
-            base = rng.integers(0, cfg.vocab, nd)
-            sess.encode_packed_verify_layer_major([int(base[i % nd]) for i in range(16)], pos)
-            sess.encode_restore_after_partial_accept(pos, 16, 0)
-        for _ in range(10):
-            block()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(blocks):
-            block()
-        torch.cuda.synchronize()
-        out.append({"distinct_tokens": nd, "ms_per_4_layer_verify": (time.perf_counter() - t0) / blocks * 1e3})
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(blocks):
+        sess.encode_packed_verify_layer_major(draw(), pos)
+        sess.encode_restore_after_partial_accept(pos, 16, 0)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / blocks * 1e3
     sess.close()
-    print(json.dumps({"moe_layer_probe": out}))
+    print(json.dumps({"moe_layer_probe": {"distinct_tokens": nd, "layers": cfg.n_layers, "blocks": 128 + blocks,
+                                          "ms_per_block_from_the_host": ms}}))
 
 
 def rocprof_summary(directory):
@@ -483,8 +483,8 @@ def main():
                     help="copies of the three weight matrices the timed loops rotate over; 3 x 118 MB exceeds the 256 MB "
                          "memory-side cache, so weights come from HBM as they do in a real model (1 = cache-resident)")
     ap.add_argument("--gemm-only", action="store_true", help="skip the attention, acceptance and end-to-end sections")
-    ap.add_argument("--moe-layer", metavar="N[,N...]", help="only run the mixture-of-experts layer probe with blocks of N "
-                                                             "distinct tokens (e.g. 16,4,1) and exit; for kernel traces")
+    ap.add_argument("--moe-layer", metavar="N", type=int, help="only run the mixture-of-experts layer probe with blocks of N "
+                                                               "distinct tokens (16, 4, 1 ...) and exit; for kernel traces")
     ap.add_argument("--shapes", default="0,1,2", help="which of the three GEMM shapes take part (for per-shape profiles; the "
                                                       "metric is defined on all three)")
     args = ap.parse_args()
@@ -497,7 +497,7 @@ def main():
         sys.exit(2)
 
     if args.moe_layer:
-        moe_layer_probe([int(v) for v in args.moe_layer.split(",")])
+        moe_layer_probe(max(1, min(16, args.moe_layer)))
         return
 
     import numpy as np
