@@ -65,6 +65,32 @@ def test_moe_128_experts_verify_matches_oracle(ctx, oracle, weights):
     sess.close()
 
 
+def test_more_slots_than_one_round_of_the_expert_kernel(ctx, oracle):
+    """Top-12 routing over 128 experts: a 16-row block then touches about 99 distinct experts (128 (1 - e^-1.5); more
+    than 85 with near certainty), i.e. more than 4096 (slot, tile) units for the gate/up launch, so its workgroups
+    run two rounds of sixteen units (slab refilled four times, ring streaming across the round boundary), and the
+    expert list is longer than one 64-entry window for the down launch.  Compared with the CPU oracle like the top-8
+    shape."""
+    cfg = dfl.ModelConfig(n_layers=2, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=8192, n_expert=128,
+                          n_expert_used=12, ffn_expert=768, ffn_shared=768)
+    w = dfl.synth_target_weights_blocks(cfg, 43)
+    model = dfl.TargetModel(ctx, cfg, w)
+    assert model.tiled_tensors > 0
+    omodel, _keep = oracle.build_model(cfg.as_dict(), w)
+    sess = dfl.Session(ctx, model, 64, TAPS)
+    ostate = oracle.TargetState(cfg.as_dict(), 64)
+    rng = np.random.default_rng(128)  # (of seeds 100..159 the one whose 384 routing decisions are furthest from a tie)
+    oracle.router_margin_take()
+    blk = rng.integers(0, cfg.vocab, 16).tolist()
+    out = sess.encode_packed_verify_layer_major(blk, 0, want_logits=True)
+    lo, hid = oracle.target_verify(omodel, ostate, blk, 0, TAPS)
+    margin = oracle.router_margin_take()
+    assert margin > 5e-3, f"seed no longer decisive: smallest relative router gap {margin:.2e}"
+    close(out.hidden_capture.cpu().numpy(), hid, "top-12 hidden")
+    close(out.logits.cpu().numpy(), lo, "top-12 logits")
+    sess.close()
+
+
 def test_tiled_expert_stacks_agree_with_row_order(ctx, weights):
     """The expert stacks and the shared expert of this shape (768 and 2048 rows per expert: multiples of 256) are
     uploaded in the tiled order and run through the expert kernel (one 16-row tile per wave, minima through the
