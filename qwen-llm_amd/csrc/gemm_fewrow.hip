@@ -1826,7 +1826,14 @@ __global__ void __launch_bounds__(64 * kWaves)
             gw++;
             if (w_left > 0) {
                 wstage = q4k_uniform(w + static_cast<size_t>(gw) * group_bytes);
-                if (ragged) q6k_lane_w_offsets(W, lane, wave, gw * G6::kRows, n_out, row_bytes);
+                // only the matrix's last group has rows to clamp (every other group's offsets are the same); the
+                // lane index goes in through an opaque copy so that nothing of this rare path is kept in registers
+                // (or spilled) across the stage loop
+                if (ragged && gw == n_groups - 1) {
+                    int ol = lane;
+                    asm volatile("" : "+v"(ol));
+                    q6k_lane_w_offsets(W, ol, wave, gw * G6::kRows, n_out, row_bytes);
+                }
             }
         }
     };
