@@ -133,6 +133,48 @@ def test_expert_kernel_rows_do_not_depend_on_the_rest_of_the_block(ctx, weights)
     s_one.close()
 
 
+_ROUTE_PROBE = r"""
+import sys
+import numpy as np
+import qwen_llm_amd as dfl
+cfg = dfl.ModelConfig(n_layers=2, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=8192, n_expert=128,
+                      n_expert_used=8, ffn_expert=768, ffn_shared=768)
+ctx = dfl.Context(0, workspace_bytes=64 << 20)
+model = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_blocks(cfg, 47))
+sess = dfl.Session(ctx, model, 64, [0, 1])
+rng = np.random.default_rng(9)
+outs = []
+pos = 0
+for n in (16, 4, 1):
+    out = sess.encode_packed_verify_layer_major(rng.integers(0, cfg.vocab, n).tolist(), pos, want_logits=True)
+    outs.append(out.logits.cpu().numpy())
+    pos += n
+np.save(sys.argv[1], np.concatenate(outs, axis=0))
+"""
+
+
+def test_routing_inside_the_expert_launch_equals_the_routing_kernel(tmp_path):
+    """The expert list, the weights and the slots come out of the same row arithmetic (moe_route.h) whether the
+    gate/up launch derives them in its prologue or moe_route_small_kernel does in a launch of its own: the logits of
+    three blocks (16, 4 and 1 rows) are equal bit for bit.  The switch is read once per process, so each setting runs
+    in a process of its own (two short-lived ones, one after the other)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    got = {}
+    for flag in ("1", "0"):
+        path = str(tmp_path / f"logits_{flag}.npy")
+        env = dict(os.environ, DFLASH_MOE_FUSED_ROUTE=flag, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+        r = subprocess.run([sys.executable, "-c", _ROUTE_PROBE, path], env=env, cwd=root, capture_output=True, text=True, timeout=240)
+        assert r.returncode == 0, r.stderr[-2000:]
+        got[flag] = np.load(path)
+    assert got["1"].shape == got["0"].shape == (21, 8192)
+    assert np.all(np.isfinite(got["1"]))
+    assert np.array_equal(got["1"], got["0"])
+
+
 def test_generate_on_the_moe_shape_equals_serial_greedy(ctx, weights):
     """MoE target + drafter in one loop at the end-to-end widths: every emitted token is the target's serial greedy
     decode through the same kernels, through full accepts, partial accepts and rollbacks."""
