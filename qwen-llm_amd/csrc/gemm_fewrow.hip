@@ -1370,7 +1370,7 @@ __device__ __forceinline__ void q4k_experts_compute(const u32x4_t *blk, const ui
 template <typename XT, typename YT, bool kRoute>
 __global__ void __launch_bounds__(64 * kSlabWaves)
     gemm_q4k_experts_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, YT *__restrict__ y, int n_out, int nb,
-                            int n_rows, Q4KBatch bt, int upm, Q4KDiv by_upm, int max_slots) {
+                            int n_rows, Q4KBatch bt, int upm, Q4KDiv by_upm, int max_slots, int early_ids) {
     constexpr int kW = kSlabWaves;
     constexpr int kItems = kExpChunk * 8 / kW;  // activation items (eight values of one row) per thread and refill: 2
     constexpr int kXInstr = kItems * Q4KX8<XT>::kLoads;
@@ -1402,6 +1402,8 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
         }
     };
     int32_t *ids_lds = reinterpret_cast<int32_t *>(reinterpret_cast<uint8_t *>(lds) + kExpXchgEnd + 16 * 4 * sizeof(unsigned long long));
+    int slot_base = -64;  // no window of the list yet: the first use (before any weight load is issued) reads it
+    int32_t ids_window = 0;
     int n_slots;
     if constexpr (kRoute) {
         // The block's routing, by every workgroup for itself: wave w takes row w (dfl_route::route_row, the arithmetic
@@ -1442,7 +1444,14 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
         __builtin_amdgcn_s_waitcnt(kWaitLds);
         __builtin_amdgcn_s_barrier();
     } else {
+        if (early_ids) {  // the first window of the list travels with the slot count: one trip to memory instead of two
+            ids_window = bt.ids[min(lane, max_slots - 1)];
+            slot_base = 0;
+        }
         n_slots = min(*bt.n_slots, max_slots);  // (the bound the host sized the buffers for)
+        // one wait for both, stated here on every path so that none is implied at the window's later uses
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+        asm volatile("" : "+v"(ids_window));
     }
     const int tiles = (n_out + 15) >> 4;
     const int halves = bt.pair ? 2 : 1;
@@ -1461,10 +1470,8 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     const int h_begin = hsplit ? wave >> 3 : 0, h_end = hsplit ? h_begin + 1 : halves;
 
     // matrix index of a slot: a register window over the list (see gemm_q4k_stream_kernel)
-    // (Measured and not kept: the first window, the slot count and shared activations all loaded at the very top of
-    // the kernel - 1.2-1.5 us slower per launch than this order.)
-    int slot_base = -64;  // no window yet: the first use (before any weight load is issued) reads it
-    int32_t ids_window = 0;
+    // (Measured and not kept: shared activations loaded at the very top of the kernel as well, ahead of the slot
+    // count - 1.2-1.5 us slower per launch than this order.)
     auto slot_id = [&](int j) {
         if constexpr (kRoute) {  // the list is in LDS; whatever it holds, the index stays inside the stack
             const int32_t id = __builtin_amdgcn_readfirstlane(ids_lds[min(max(j, 0), kExpRouteIds - 1)]);
@@ -2377,6 +2384,8 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         Q4KBatch bt = *batch;
         bt.by_wg = q4k_make_div(static_cast<uint32_t>(n_wg));
         const Q4KDiv by_upm = q4k_make_div(static_cast<uint32_t>(upm));
+        // the first 64 list entries are loaded together with the slot count (0.5 us per down launch at light load)
+        const int early_ids = env_int("DFLASH_EXP_EARLY_IDS", 1);
         const uint8_t *wb = static_cast<const uint8_t *>(w);
         const int no = static_cast<int>(n_out);
 #define DFL_LAUNCH_EXPERTS(XT, YT, ROUTE)                                                                                   \
@@ -2385,7 +2394,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
             return rc_;                                                                                                     \
         dfl_timed timer(ctx, st, DFL_T_GEMM);                                                                               \
         gemm_q4k_experts_kernel<XT, YT, ROUTE><<<n_wg, 64 * kSlabWaves, kExpLdsBytes, st>>>(wb, static_cast<const XT *>(x), reinterpret_cast<YT *>(y), \
-                                                                                           no, nb, n_rows, bt, upm, by_upm, max_slots); \
+                                                                                           no, nb, n_rows, bt, upm, by_upm, max_slots, early_ids); \
     } while (0)
         if (bt.route_logits) {
             if (x_type != DFLASH_TYPE_F32 || per_slot_x || bt.route_experts > 256 || bt.route_experts < 1 || bt.route_used < 1 ||
