@@ -383,7 +383,9 @@ int64_t dflash_session_graph_replays(const dflash_session *session);
  * Outputs (device, may be NULL): argmax[n] i32 and gap[n] f32 (argmax_top2 of each row),
  * hidden_capture[n][n_taps][hidden] f32 (residual stream after the tapped layers, :10535-10551),
  * logits[n][vocab] f32.  If argmax_host is non-NULL the call waits and copies the n indices
- * there (the reference returns Vec<i32>).  1 <= n <= 16. */
+ * there (the reference returns Vec<i32>).  With argmax, gap, logits and argmax_host all NULL the
+ * output head (final norm, vocabulary projection, argmax) is not run: a prefill block, of which
+ * only the K/V rows and the tapped hidden rows are wanted.  1 <= n <= 16. */
 int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,
                             const int32_t *tokens_host, int32_t n, int64_t start_position,
                             const int32_t *tap_layers_host, int32_t n_taps, int32_t *argmax, float *gap,

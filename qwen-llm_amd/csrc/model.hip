@@ -596,7 +596,7 @@ uint64_t hash_model(const dflash_model *m) {
 // device, so the sequence can be captured once and replayed.
 int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, int32_t n, int64_t start,
                        const int32_t *tap_layers, int32_t n_taps, float *hidden_capture, float *lg, int32_t *am, float *gp,
-                       hipStream_t st) {
+                       hipStream_t st, bool want_head = true) {
     const dflash_model_cfg &c = model->cfg;
     const int H = c.hidden, hd = c.head_dim;
     const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
@@ -650,9 +650,11 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
             if (tap_layers[t] == il)
                 capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
     }
-    if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, model->output_norm, s->cur, H, c.eps, nullptr, nullptr);
-    if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
-    if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gp, st))) return rc;
+    if (want_head) {  // (not for a caller that asked for no output of it: a prefill block wants K/V and the taps only)
+        if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, model->output_norm, s->cur, H, c.eps, nullptr, nullptr);
+        if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
+        if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gp, st))) return rc;
+    }
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }
@@ -663,15 +665,17 @@ namespace {
 int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
                           const int32_t *dev_tokens, int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps,
                           int32_t *argmax, float *gap, float *hidden_capture, float *logits, int32_t *argmax_host,
-                          dflash_stream_t stream);
+                          dflash_stream_t stream, bool want_head = true);
 }
 
 int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
                             int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps, int32_t *argmax,
                             float *gap, float *hidden_capture, float *logits, int32_t *argmax_host,
                             dflash_stream_t stream) {
+    // no output of the head asked for: it is not run (inside the library a null output means the session's own buffer)
+    const bool want_head = argmax || gap || logits || argmax_host;
     return verify_block_impl(ctx, model, s, tokens, nullptr, n, start, tap_layers, n_taps, argmax, gap, hidden_capture, logits,
-                             argmax_host, stream);
+                             argmax_host, stream, want_head);
 }
 
 namespace {
@@ -682,7 +686,7 @@ namespace {
 int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
                           const int32_t *dev_tokens, int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps,
                           int32_t *argmax, float *gap, float *hidden_capture, float *logits, int32_t *argmax_host,
-                          dflash_stream_t stream) {
+                          dflash_stream_t stream, bool want_head) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!model || !s || !tokens) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "verify_block: null argument");
     const dflash_model_cfg &c = model->cfg;
@@ -721,7 +725,7 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
                                    reinterpret_cast<uintptr_t>(am), reinterpret_cast<uintptr_t>(gp)};
         key = hash_bytes(outs, sizeof(outs), key);
         // (the attention launches are cut by the bucket of the context length: see dfl_attn_block)
-        const int64_t shape[3] = {n, n_taps, dfl_attn_bucket(start + n)};
+        const int64_t shape[4] = {n, n_taps, dfl_attn_bucket(start + n), want_head ? 1 : 0};
         key = hash_bytes(shape, sizeof(shape), key);
         if (n_taps > 0) key = hash_bytes(tap_layers, sizeof(int32_t) * n_taps, key);
     }
@@ -732,7 +736,7 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
         hipGraph_t graph = nullptr;
         DFL_HIP_CHECK(ctx, hipStreamBeginCapture(ctx->gstream, hipStreamCaptureModeThreadLocal));
         ctx->capturing = true;
-        rc = verify_enqueue(ctx, model, s, n, start, tap_layers, n_taps, hidden_capture, lg, am, gp, ctx->gstream);
+        rc = verify_enqueue(ctx, model, s, n, start, tap_layers, n_taps, hidden_capture, lg, am, gp, ctx->gstream, want_head);
         ctx->capturing = false;
         const hipError_t end = hipStreamEndCapture(ctx->gstream, &graph);
         if (rc) {
@@ -753,7 +757,7 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
         s->graph_replays++;
         DFL_HIP_CHECK(ctx, hipEventRecord(ctx->g_out, ctx->gstream));
         DFL_HIP_CHECK(ctx, hipStreamWaitEvent(st, ctx->g_out, 0));
-    } else if ((rc = verify_enqueue(ctx, model, s, n, start, tap_layers, n_taps, hidden_capture, lg, am, gp, st))) {
+    } else if ((rc = verify_enqueue(ctx, model, s, n, start, tap_layers, n_taps, hidden_capture, lg, am, gp, st, want_head))) {
         return rc;
     }
     s->kv_n_pos = start + n;

@@ -484,9 +484,11 @@ class Session:
         return self._L.dflash_session_kv_n_pos(self._h)
 
     def encode_packed_verify_layer_major(self, tokens, start_position: int, want_logits=False, want_hidden=True,
-                                         sync=True) -> VerifyOutput:
+                                         sync=True, want_head=True) -> VerifyOutput:
         """Forward of ``tokens`` at positions start_position.. ; appends K/V; returns argmax, top-2
-        gap, the tapped hidden rows [n][n_taps][hidden] and (optionally) the logits."""
+        gap, the tapped hidden rows [n][n_taps][hidden] and (optionally) the logits.  ``want_head=False`` (with
+        ``want_logits=False``): no output of the head is asked for and the library does not run it (prefill blocks);
+        argmax, gap and argmax_host of the result are then None."""
         torch = _torch()
         cfg = self.model.cfg
         n = len(tokens)
@@ -494,16 +496,20 @@ class Session:
         toks = (C.c_int32 * max(n, 1))(*[int(t) for t in tokens])
         n_taps = len(self.tap_layers) if want_hidden else 0
         taps = (C.c_int32 * max(n_taps, 1))(*self.tap_layers[:n_taps])
-        argmax = _binding._empty(max(n, 1), dtype=torch.int32, device=dev)
-        gap = _binding._empty(max(n, 1), dtype=torch.float32, device=dev)
+        want_head = want_head or want_logits
+        argmax = _binding._empty(max(n, 1), dtype=torch.int32, device=dev) if want_head else None
+        gap = _binding._empty(max(n, 1), dtype=torch.float32, device=dev) if want_head else None
         hidden = _binding._empty((n, n_taps, cfg.hidden), dtype=torch.float32, device=dev) if n_taps else None
         logits = _binding._empty((n, cfg.vocab), dtype=torch.float32, device=dev) if want_logits else None
+        sync = sync and want_head
         host = (C.c_int32 * max(n, 1))() if sync else None
         self.ctx._check(self._L.dflash_verify_block(
-            self.ctx._h, C.byref(self.model.c), self._h, toks, n, start_position, taps, n_taps, argmax.data_ptr(),
-            gap.data_ptr(), hidden.data_ptr() if hidden is not None else None,
+            self.ctx._h, C.byref(self.model.c), self._h, toks, n, start_position, taps, n_taps,
+            argmax.data_ptr() if want_head else None, gap.data_ptr() if want_head else None,
+            hidden.data_ptr() if hidden is not None else None,
             logits.data_ptr() if logits is not None else None, host, _stream_ptr()))
-        return VerifyOutput(argmax[:n], gap[:n], hidden, logits, list(host[:n]) if sync else None)
+        return VerifyOutput(argmax[:n] if want_head else None, gap[:n] if want_head else None, hidden, logits,
+                            list(host[:n]) if sync else None)
 
     @property
     def graph_replays(self) -> int:
@@ -750,7 +756,8 @@ class SpeculativeDecoder:
         last = None
         for s in range(0, len(prompt), 16):
             blk = list(prompt[s:s + 16])
-            out = self.session.encode_packed_verify_layer_major(blk, s)
+            # only the last block's head is wanted; the others leave K/V and the tapped rows (and do not wait)
+            out = self.session.encode_packed_verify_layer_major(blk, s, want_head=s + 16 >= len(prompt))
             self.draft_session.append_target_ctx_columns(out.hidden_capture, list(range(s, s + len(blk))))
             last = out
         # the drafter's pass over the prompt's columns belongs to the prefill, not to the first step
