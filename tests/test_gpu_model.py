@@ -99,6 +99,33 @@ def test_verify_block_matches_oracle_and_restore(ctx, oracle, target):
     sess.close()
 
 
+def test_a_block_without_head_outputs_leaves_the_same_state(ctx, target):
+    """A verify block whose caller asks for none of the head's outputs (a prefill block) does not run the head; its K/V
+    rows and tapped hidden rows are those of the same block run in full: the next block's logits are equal bit for
+    bit, for a 16-row and a ragged block, and the guards still hold."""
+    model, _ = target
+    rng = np.random.default_rng(77)
+    blocks = [rng.integers(0, C1.vocab, n).tolist() for n in (16, 5, 16)]
+    full, lean = dfl.Session(ctx, model, 64, TAPS), dfl.Session(ctx, model, 64, TAPS)
+    pos = 0
+    for blk in blocks[:2]:
+        a = full.encode_packed_verify_layer_major(blk, pos)
+        b = lean.encode_packed_verify_layer_major(blk, pos, want_head=False)
+        assert b.argmax is None and b.gap is None and b.argmax_host is None and b.logits is None
+        assert np.array_equal(a.hidden_capture.cpu().numpy(), b.hidden_capture.cpu().numpy())
+        pos += len(blk)
+    assert lean.kv_n_pos == full.kv_n_pos == pos
+    a = full.encode_packed_verify_layer_major(blocks[2], pos, want_logits=True)
+    b = lean.encode_packed_verify_layer_major(blocks[2], pos, want_logits=True)
+    assert np.array_equal(a.logits.cpu().numpy(), b.logits.cpu().numpy())
+    assert a.argmax_host == b.argmax_host
+    with pytest.raises(dfl.DFlashError) as e:
+        lean.encode_packed_verify_layer_major([1, 2], 3, want_head=False)
+    assert e.value.status == 10
+    full.close()
+    lean.close()
+
+
 def test_verify_guard_walls(ctx, target):
     model, _ = target
     sess = dfl.Session(ctx, model, 64, TAPS)
