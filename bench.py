@@ -310,9 +310,10 @@ def e2e_speculative(ctx, n_generate, sweep, log):
     # the target's serial greedy continuation (token by token through the same kernels)
     serial = dfl.Session(ctx, target, cap, taps)
     t0 = time.perf_counter()
-    for s0 in range(0, prompt_len, 16):
-        # (only the last block's head output is wanted; the others leave their K/V rows and are not waited for)
-        out = serial.encode_packed_verify_layer_major(prompt[s0:s0 + 16], s0, want_hidden=False, want_head=s0 + 16 >= prompt_len)
+    # every block but the last without the output head, two blocks in flight (dflash_prefill_blocks); the last with it
+    body = (prompt_len - 1) // 16 * 16
+    serial.prefill_blocks(prompt[:body], 0, want_hidden=False)
+    out = serial.encode_packed_verify_layer_major(prompt[body:], body, want_hidden=False)
     prefill_s = time.perf_counter() - t0
     cont = [out.argmax_host[-1]]
     t0 = time.perf_counter()

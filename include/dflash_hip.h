@@ -397,6 +397,32 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
  * state (encode_restore_to_pre_block, :15789-15905). */
 int32_t dflash_restore(dflash_ctx *ctx, dflash_session *session, int64_t start_position, int32_t n, int32_t n_keep);
 
+/* The packed prefill with hidden capture (metal_dflash.rs:10779-15648; the reference walks the prompt in chunks of
+ * layer_scratch.n rows, :10770-10778): tokens_host[n_tokens] at positions start_position .., in blocks of 16 rows
+ * through the same layers as dflash_verify_block, without the output head; K/V rows are appended, the tapped hidden
+ * rows go to hidden_capture[n_tokens][n_taps][hidden] (device; may be NULL with n_taps = 0).  Consecutive blocks run
+ * on two streams one layer apart (the second stream, a second set of scratch buffers and a second context's
+ * workspace belong to the session and are made on the first call), ordered by events where a block reads the
+ * previous block's K/V rows; the caller's stream continues behind both.  Results equal those of the same blocks
+ * through dflash_verify_block bit for bit.  Guards as dflash_verify_block; on an error kv_n_pos is unchanged. */
+int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,
+                              const int32_t *tokens_host, int32_t n_tokens, int64_t start_position,
+                              const int32_t *tap_layers_host, int32_t n_taps, float *hidden_capture,
+                              dflash_stream_t stream);
+
+/* The packed prefill with hidden capture (metal_dflash.rs:10779-15648; the reference walks the prompt in chunks of
+ * layer_scratch.n rows, :10770-10778): tokens_host[n_tokens] at positions start_position .., in blocks of 16 rows
+ * through the same layers as dflash_verify_block, without the output head; K/V rows are appended, the tapped hidden
+ * rows go to hidden_capture[n_tokens][n_taps][hidden] (device; may be NULL with n_taps = 0).  Consecutive blocks run
+ * on two streams one layer apart (the second stream, a second set of scratch buffers and a second context's
+ * workspace belong to the session and are made on the first call), ordered by events where a block reads the
+ * previous block's K/V rows; the caller's stream continues behind both.  Results equal those of the same blocks
+ * through dflash_verify_block bit for bit.  Guards as dflash_verify_block; on an error kv_n_pos is unchanged. */
+int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,
+                              const int32_t *tokens_host, int32_t n_tokens, int64_t start_position,
+                              const int32_t *tap_layers_host, int32_t n_taps, float *hidden_capture,
+                              dflash_stream_t stream);
+
 /* ---- block drafter ----------------------------------------------------------------------
  * DFlashConfig / DFlashHead / DFlashLayer (loader.rs:342-399), MetalDFlashSession
  * (metal_dflash.rs:5053-5191). */

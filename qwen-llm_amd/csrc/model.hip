@@ -436,6 +436,28 @@ struct dflash_session {
     std::map<uint64_t, hipGraphExec_t> graphs;
     std::map<uint64_t, int> graph_seen;
     int64_t graph_replays = 0;
+    struct PrefillPipe *pipe = nullptr;  // second lane of dflash_prefill_blocks, made on first use
+};
+
+// Second lane of a pipelined prefill.  A 16-row block's layers are a chain of small dependent launches that leave most
+// of the GPU idle; two consecutive blocks, one layer apart, fill each other's gaps.  The lane has its own context
+// (split-K partial tiles, attention workspace: what two concurrent launches of one kind must not share), its own
+// scratch (a session of capacity 16 whose K/V pointers are redirected to the owner's cache) and its own stream.
+// Block b needs block b-1's K/V rows of a layer before its attention in that layer: one event per (lane, layer),
+// recorded behind the launch that writes the rows, waited for by the other lane.
+struct PrefillPipe {
+    dflash_ctx *ctx2 = nullptr;
+    dflash_session *shadow = nullptr;
+    _Float16 *own_k = nullptr, *own_vt = nullptr;  // the shadow session's own (unused) cache, put back before it is destroyed
+    int64_t own_capacity = 0;
+    hipStream_t stream2 = nullptr;
+    std::vector<hipEvent_t> kv_done[2];
+    hipEvent_t fork = nullptr, join = nullptr;
+};
+// what verify_enqueue is told when it runs as one lane of the pipeline
+struct PrefillLane {
+    const hipEvent_t *mine, *other;
+    bool wait_other;  // there is a previous block on the other lane
 };
 
 struct dflash_draft_session {
@@ -521,6 +543,24 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
 
 void dflash_session_destroy(dflash_session *s) {
     if (!s) return;
+    if (PrefillPipe *p = s->pipe) {
+        if (p->stream2) (void)hipStreamSynchronize(p->stream2);
+        for (auto &v : p->kv_done)
+            for (hipEvent_t e : v)
+                if (e) (void)hipEventDestroy(e);
+        if (p->fork) (void)hipEventDestroy(p->fork);
+        if (p->join) (void)hipEventDestroy(p->join);
+        if (p->shadow) {  // give it back its own cache before it frees what it owns
+            p->shadow->k_cache = p->own_k;
+            p->shadow->vt_cache = p->own_vt;
+            p->shadow->capacity = p->own_capacity;
+            dflash_session_destroy(p->shadow);
+        }
+        if (p->stream2) (void)hipStreamDestroy(p->stream2);
+        if (p->ctx2) dflash_ctx_destroy(p->ctx2);
+        delete p;
+        s->pipe = nullptr;
+    }
     for (auto &g : s->graphs)
         if (g.second) (void)hipGraphExecDestroy(g.second);
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
@@ -596,7 +636,7 @@ uint64_t hash_model(const dflash_model *m) {
 // device, so the sequence can be captured once and replayed.
 int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, int32_t n, int64_t start,
                        const int32_t *tap_layers, int32_t n_taps, float *hidden_capture, float *lg, int32_t *am, float *gp,
-                       hipStream_t st, bool want_head = true) {
+                       hipStream_t st, bool want_head = true, const PrefillLane *lane = nullptr) {
     const dflash_model_cfg &c = model->cfg;
     const int H = c.hidden, hd = c.head_dim;
     const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
@@ -621,6 +661,10 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
             packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
             L.k_norm, kc, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, packed ? s->pk + q_dim + kv_dim : s->v,
             packed ? tot : kv_dim, vtc, s->capacity);
+        if (lane) {  // this block's K/V rows of the layer are written; the previous block's must be before the attention reads them
+            DFL_HIP_CHECK(ctx, hipEventRecord(lane->mine[il], st));
+            if (lane->wait_other) DFL_HIP_CHECK(ctx, hipStreamWaitEvent(st, lane->other[il], 0));
+        }
         // under capture the context length is read from pos[0] on the device: the same launches then serve every
         // position of the bucket
         if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity, scale,
@@ -779,6 +823,91 @@ int32_t dflash_restore(dflash_ctx *ctx, dflash_session *s, int64_t start, int32_
         return dfl_fail(ctx, DFLASH_ERR_STATE, "restore: kv_n_pos %lld != start %lld + n %d (must follow the matching verify)",
                         static_cast<long long>(s->kv_n_pos), static_cast<long long>(start), n);
     s->kv_n_pos = start + n_keep;  // stale rows stay in place; the next verify overwrites them
+    return DFLASH_OK;
+}
+
+namespace {
+int32_t prefill_pipe_create(dflash_ctx *ctx, dflash_session *s) {
+    PrefillPipe *p = new (std::nothrow) PrefillPipe();
+    if (!p) return dfl_fail(ctx, DFLASH_ERR_HIP, "prefill_blocks: out of host memory");
+    s->pipe = p;  // (whatever has been made so far is taken down with the session)
+    int32_t rc = dflash_ctx_create(ctx->device, ctx->workspace_bytes, &p->ctx2);
+    if (rc) return dfl_fail(ctx, rc, "prefill_blocks: second context");
+    if ((rc = dflash_session_create(p->ctx2, &s->cfg, 16, s->n_taps, &p->shadow))) return dfl_fail(ctx, rc, "prefill_blocks: second scratch set");
+    p->own_k = p->shadow->k_cache;
+    p->own_vt = p->shadow->vt_cache;
+    p->own_capacity = p->shadow->capacity;
+    p->shadow->k_cache = s->k_cache;
+    p->shadow->vt_cache = s->vt_cache;
+    p->shadow->capacity = s->capacity;
+    DFL_HIP_CHECK(ctx, hipStreamCreateWithFlags(&p->stream2, hipStreamNonBlocking));
+    for (auto &v : p->kv_done) {
+        v.assign(s->cfg.n_layers, nullptr);
+        for (hipEvent_t &e : v) DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    }
+    DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&p->fork, hipEventDisableTiming));
+    DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&p->join, hipEventDisableTiming));
+    return DFLASH_OK;
+}
+}  // namespace
+
+int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
+                              int32_t n_tokens, int64_t start, const int32_t *tap_layers, int32_t n_taps,
+                              float *hidden_capture, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!model || !s || !tokens) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "prefill_blocks: null argument");
+    const dflash_model_cfg &c = model->cfg;
+    if (n_tokens < 1) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "prefill_blocks: n_tokens %d", n_tokens);
+    if (s->kv_n_pos != start)
+        return dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_blocks: kv_n_pos %lld != start_position %lld",
+                        static_cast<long long>(s->kv_n_pos), static_cast<long long>(start));
+    if (start < 0 || start + n_tokens > s->capacity)
+        return dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_blocks: positions %lld..%lld exceed the KV capacity %lld",
+                        static_cast<long long>(start), static_cast<long long>(start + n_tokens), static_cast<long long>(s->capacity));
+    for (int i = 0; i < n_tokens; i++)
+        if (tokens[i] < 0 || tokens[i] >= c.vocab)
+            return dfl_fail(ctx, DFLASH_ERR_INVALID_TOKEN, "prefill_blocks: token %d at index %d outside vocabulary %d", tokens[i], i, c.vocab);
+    if (n_taps < 0 || n_taps > s->n_taps || (n_taps > 0 && (!tap_layers || !hidden_capture)))
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "prefill_blocks: hidden capture arguments");
+    if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_blocks: session/model shape mismatch");
+    int32_t rc = DFLASH_OK;
+    if (!s->pipe && (rc = prefill_pipe_create(ctx, s))) return rc;
+    PrefillPipe *p = s->pipe;
+    if (!p->shadow || !p->stream2 || !p->join) return dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_blocks: the second lane could not be set up earlier");
+    hipStream_t lanes_st[2] = {static_cast<hipStream_t>(stream), p->stream2};
+    dflash_ctx *lanes_ctx[2] = {ctx, p->ctx2};
+    dflash_session *lanes_s[2] = {s, p->shadow};
+    // the second lane starts behind whatever the caller's stream holds (earlier blocks' K/V rows among it)
+    DFL_HIP_CHECK(ctx, hipEventRecord(p->fork, lanes_st[0]));
+    DFL_HIP_CHECK(ctx, hipStreamWaitEvent(lanes_st[1], p->fork, 0));
+    const size_t cap_row = static_cast<size_t>(std::max(n_taps, 0)) * c.hidden;
+    int block = 0;
+    for (int32_t t0 = 0; t0 < n_tokens && !rc; t0 += 16, block++) {
+        const int lane_i = block & 1;
+        const int32_t n = std::min<int32_t>(16, n_tokens - t0);
+        dflash_session *ls = lanes_s[lane_i];
+        Int16Args ids_arg = {}, pos_arg = {};
+        for (int i = 0; i < n; i++) {
+            ids_arg.v[i] = tokens[t0 + i];
+            pos_arg.v[i] = static_cast<int32_t>(start + t0 + i);
+        }
+        set_ids_pos_kernel<<<1, 64, 0, lanes_st[lane_i]>>>(ids_arg, pos_arg, n, ls->ids, ls->pos, nullptr, c.vocab);
+        const PrefillLane lane = {p->kv_done[lane_i].data(), p->kv_done[lane_i ^ 1].data(), block > 0};
+        rc = verify_enqueue(lanes_ctx[lane_i], model, ls, n, start + t0, tap_layers, n_taps,
+                            hidden_capture ? hidden_capture + static_cast<size_t>(t0) * cap_row : nullptr, ls->logits, ls->argmax, ls->gap,
+                            lanes_st[lane_i], false, &lane);
+        if (rc && lane_i == 1) rc = dfl_fail(ctx, rc, "prefill_blocks: %s", dflash_last_error(p->ctx2));
+    }
+    // the caller's stream continues behind both lanes
+    const hipError_t e1 = hipEventRecord(p->join, lanes_st[1]);
+    const hipError_t e2 = e1 == hipSuccess ? hipStreamWaitEvent(lanes_st[0], p->join, 0) : e1;
+    if (rc) {
+        (void)hipStreamSynchronize(lanes_st[1]);
+        (void)hipStreamSynchronize(lanes_st[0]);
+        return rc;  // (kv_n_pos unchanged: rows written past it are overwritten by the next block)
+    }
+    DFL_HIP_CHECK(ctx, e2);
+    s->kv_n_pos = start + n_tokens;
     return DFLASH_OK;
 }
 

@@ -511,6 +511,25 @@ class Session:
         return VerifyOutput(argmax[:n] if want_head else None, gap[:n] if want_head else None, hidden, logits,
                             list(host[:n]) if sync else None)
 
+    def prefill_blocks(self, tokens, start_position: int, want_hidden=True):
+        """The prompt's blocks without the output head, two blocks in flight (dflash_prefill_blocks); returns the tapped
+        hidden rows [n_tokens][n_taps][hidden] (or None).  Enqueue only."""
+        torch = _torch()
+        cfg = self.model.cfg
+        n = len(tokens)
+        L = self._L
+        L.dflash_prefill_blocks.restype = C.c_int32
+        L.dflash_prefill_blocks.argtypes = [C.c_void_p, C.POINTER(ModelC), C.c_void_p, C.POINTER(C.c_int32), C.c_int32, C.c_int64,
+                                            C.POINTER(C.c_int32), C.c_int32, C.c_void_p, C.c_void_p]
+        toks = (C.c_int32 * max(n, 1))(*[int(t) for t in tokens])
+        n_taps = len(self.tap_layers) if want_hidden else 0
+        taps = (C.c_int32 * max(n_taps, 1))(*self.tap_layers[:n_taps])
+        hidden = (_binding._empty((n, n_taps, cfg.hidden), dtype=torch.float32, device=f"cuda:{self.ctx.device}")
+                  if n_taps else None)
+        self.ctx._check(L.dflash_prefill_blocks(self.ctx._h, C.byref(self.model.c), self._h, toks, n, start_position, taps, n_taps,
+                                                hidden.data_ptr() if hidden is not None else None, _stream_ptr()))
+        return hidden
+
     @property
     def graph_replays(self) -> int:
         return int(self._L.dflash_session_graph_replays(self._h))
@@ -753,13 +772,15 @@ class SpeculativeDecoder:
         """Run the prompt through the packed verify in blocks of 16, feed the tapped hidden rows to
         the drafter context, and return the argmax after the last prompt token."""
         assert len(prompt) > 0 and self.position == 0
-        last = None
-        for s in range(0, len(prompt), 16):
-            blk = list(prompt[s:s + 16])
-            # only the last block's head is wanted; the others leave K/V and the tapped rows (and do not wait)
-            out = self.session.encode_packed_verify_layer_major(blk, s, want_head=s + 16 >= len(prompt))
-            self.draft_session.append_target_ctx_columns(out.hidden_capture, list(range(s, s + len(blk))))
-            last = out
+        # every block but the last: K/V and the tapped rows only, two blocks in flight; the last one with its head
+        body = (len(prompt) - 1) // 16 * 16
+        if body:
+            hidden = self.session.prefill_blocks(list(prompt[:body]), 0)
+            for s in range(0, body, 16):
+                self.draft_session.append_target_ctx_columns(hidden[s:s + 16], list(range(s, s + 16)))
+        blk = list(prompt[body:])
+        last = self.session.encode_packed_verify_layer_major(blk, body)
+        self.draft_session.append_target_ctx_columns(last.hidden_capture, list(range(body, body + len(blk))))
         # the drafter's pass over the prompt's columns belongs to the prefill, not to the first step
         self.draft_session.prepare_ctx()
         _torch().cuda.synchronize()

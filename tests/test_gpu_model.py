@@ -126,6 +126,41 @@ def test_a_block_without_head_outputs_leaves_the_same_state(ctx, target):
     lean.close()
 
 
+def test_pipelined_prefill_equals_block_by_block(ctx, target):
+    """dflash_prefill_blocks (two blocks in flight on two streams, ordered by per-layer events) leaves the K/V rows and
+    the tapped hidden rows of the same blocks run one by one through dflash_verify_block: the captured rows and the
+    next block's logits are equal bit for bit, over a ragged token count, twice in a row on one session (the second
+    lane's scratch and events are reused), and its guards hold."""
+    model, _ = target
+    rng = np.random.default_rng(78)
+    first = rng.integers(0, C1.vocab, 16 * 5 + 7).tolist()   # five full blocks and a ragged one
+    second = rng.integers(0, C1.vocab, 16 * 3).tolist()
+    probe = rng.integers(0, C1.vocab, 9).tolist()
+    ref, pipe = dfl.Session(ctx, model, 256, TAPS), dfl.Session(ctx, model, 256, TAPS)
+    pos = 0
+    for chunk in (first, second):
+        got = pipe.prefill_blocks(chunk, pos)
+        want = []
+        for s0 in range(0, len(chunk), 16):
+            out = ref.encode_packed_verify_layer_major(chunk[s0:s0 + 16], pos + s0, want_head=False)
+            want.append(out.hidden_capture.cpu().numpy())
+        assert np.array_equal(got.cpu().numpy(), np.concatenate(want, axis=0))
+        pos += len(chunk)
+        assert pipe.kv_n_pos == ref.kv_n_pos == pos
+    a = ref.encode_packed_verify_layer_major(probe, pos, want_logits=True)
+    b = pipe.encode_packed_verify_layer_major(probe, pos, want_logits=True)
+    assert np.array_equal(a.logits.cpu().numpy(), b.logits.cpu().numpy())
+    assert a.argmax_host == b.argmax_host
+    with pytest.raises(dfl.DFlashError) as e:
+        pipe.prefill_blocks([1, 2, 3], 0)
+    assert e.value.status == 10
+    with pytest.raises(dfl.DFlashError) as e:
+        pipe.prefill_blocks([1, C1.vocab], pipe.kv_n_pos)
+    assert e.value.status == 8
+    ref.close()
+    pipe.close()
+
+
 def test_verify_guard_walls(ctx, target):
     model, _ = target
     sess = dfl.Session(ctx, model, 64, TAPS)
