@@ -309,8 +309,10 @@ def e2e_speculative(ctx, n_generate, sweep, log):
 
     # the target's serial greedy continuation (token by token through the same kernels)
     serial = dfl.Session(ctx, target, cap, taps)
+    serial.prepare_prefill()
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    # every block but the last without the output head, two blocks in flight (dflash_prefill_blocks); the last with it
+    # every block but the last without the output head, four blocks in flight (dflash_prefill_blocks); the last with it
     body = (prompt_len - 1) // 16 * 16
     serial.prefill_blocks(prompt[:body], 0, want_hidden=False)
     out = serial.encode_packed_verify_layer_major(prompt[body:], body, want_hidden=False)

@@ -400,24 +400,15 @@ int32_t dflash_restore(dflash_ctx *ctx, dflash_session *session, int64_t start_p
 /* The packed prefill with hidden capture (metal_dflash.rs:10779-15648; the reference walks the prompt in chunks of
  * layer_scratch.n rows, :10770-10778): tokens_host[n_tokens] at positions start_position .., in blocks of 16 rows
  * through the same layers as dflash_verify_block, without the output head; K/V rows are appended, the tapped hidden
- * rows go to hidden_capture[n_tokens][n_taps][hidden] (device; may be NULL with n_taps = 0).  Consecutive blocks run
- * on two streams one layer apart (the second stream, a second set of scratch buffers and a second context's
- * workspace belong to the session and are made on the first call), ordered by events where a block reads the
- * previous block's K/V rows; the caller's stream continues behind both.  Results equal those of the same blocks
- * through dflash_verify_block bit for bit.  Guards as dflash_verify_block; on an error kv_n_pos is unchanged. */
-int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,
-                              const int32_t *tokens_host, int32_t n_tokens, int64_t start_position,
-                              const int32_t *tap_layers_host, int32_t n_taps, float *hidden_capture,
-                              dflash_stream_t stream);
-
-/* The packed prefill with hidden capture (metal_dflash.rs:10779-15648; the reference walks the prompt in chunks of
- * layer_scratch.n rows, :10770-10778): tokens_host[n_tokens] at positions start_position .., in blocks of 16 rows
- * through the same layers as dflash_verify_block, without the output head; K/V rows are appended, the tapped hidden
- * rows go to hidden_capture[n_tokens][n_taps][hidden] (device; may be NULL with n_taps = 0).  Consecutive blocks run
- * on two streams one layer apart (the second stream, a second set of scratch buffers and a second context's
- * workspace belong to the session and are made on the first call), ordered by events where a block reads the
- * previous block's K/V rows; the caller's stream continues behind both.  Results equal those of the same blocks
- * through dflash_verify_block bit for bit.  Guards as dflash_verify_block; on an error kv_n_pos is unchanged. */
+ * rows go to hidden_capture[n_tokens][n_taps][hidden] (device; may be NULL with n_taps = 0).  Up to four consecutive
+ * blocks are in flight on as many streams (DFLASH_PREFILL_LANES, 1..8; the extra streams, scratch sets and
+ * contexts' workspaces belong to the session and are made on the first call), ordered by per-layer events where a
+ * block reads the earlier blocks' K/V rows; the caller's stream continues behind all of them.  Results equal those
+ * of the same blocks through dflash_verify_block bit for bit.  Guards as dflash_verify_block; on an error kv_n_pos
+ * is unchanged. */
+/* Makes the extra streams, scratch sets and contexts of dflash_prefill_blocks ahead of its first call (which makes
+ * them otherwise): the allocations then stay out of the first prompt's latency.  No counterpart in the reference. */
+int32_t dflash_prefill_prepare(dflash_ctx *ctx, dflash_session *session);
 int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,
                               const int32_t *tokens_host, int32_t n_tokens, int64_t start_position,
                               const int32_t *tap_layers_host, int32_t n_taps, float *hidden_capture,

@@ -439,20 +439,26 @@ struct dflash_session {
     struct PrefillPipe *pipe = nullptr;  // second lane of dflash_prefill_blocks, made on first use
 };
 
-// Second lane of a pipelined prefill.  A 16-row block's layers are a chain of small dependent launches that leave most
-// of the GPU idle; two consecutive blocks, one layer apart, fill each other's gaps.  The lane has its own context
+// Extra lanes of a pipelined prefill.  A 16-row block's layers are a chain of small dependent launches that leave most
+// of the GPU idle; consecutive blocks, a layer or so apart, fill each other's gaps.  An extra lane has its own context
 // (split-K partial tiles, attention workspace: what two concurrent launches of one kind must not share), its own
 // scratch (a session of capacity 16 whose K/V pointers are redirected to the owner's cache) and its own stream.
-// Block b needs block b-1's K/V rows of a layer before its attention in that layer: one event per (lane, layer),
-// recorded behind the launch that writes the rows, waited for by the other lane.
+// Block b needs the earlier blocks' K/V rows of a layer before its attention in that layer: one event per (lane,
+// layer), recorded behind the launch that writes the rows and behind the wait for the previous block's event.
+constexpr int kMaxPrefillLanes = 8;
 struct PrefillPipe {
-    dflash_ctx *ctx2 = nullptr;
-    dflash_session *shadow = nullptr;
-    _Float16 *own_k = nullptr, *own_vt = nullptr;  // the shadow session's own (unused) cache, put back before it is destroyed
-    int64_t own_capacity = 0;
-    hipStream_t stream2 = nullptr;
-    std::vector<hipEvent_t> kv_done[2];
-    hipEvent_t fork = nullptr, join = nullptr;
+    int n_lanes = 4;  // blocks in flight: lane 0 is the owner itself (its context, its scratch, the caller's stream)
+    struct Extra {
+        dflash_ctx *ctx = nullptr;
+        dflash_session *shadow = nullptr;
+        _Float16 *own_k = nullptr, *own_vt = nullptr;  // the shadow session's own (unused) cache, put back before it is destroyed
+        int64_t own_capacity = 0;
+        hipStream_t stream = nullptr;
+        hipEvent_t join = nullptr;
+    } extra[kMaxPrefillLanes - 1];
+    std::vector<hipEvent_t> kv_done[kMaxPrefillLanes];
+    hipEvent_t fork = nullptr;
+    bool ready = false;
 };
 // what verify_enqueue is told when it runs as one lane of the pipeline
 struct PrefillLane {
@@ -544,20 +550,22 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
 void dflash_session_destroy(dflash_session *s) {
     if (!s) return;
     if (PrefillPipe *p = s->pipe) {
-        if (p->stream2) (void)hipStreamSynchronize(p->stream2);
+        for (auto &x : p->extra)
+            if (x.stream) (void)hipStreamSynchronize(x.stream);
         for (auto &v : p->kv_done)
             for (hipEvent_t e : v)
                 if (e) (void)hipEventDestroy(e);
         if (p->fork) (void)hipEventDestroy(p->fork);
-        if (p->join) (void)hipEventDestroy(p->join);
-        if (p->shadow) {  // give it back its own cache before it frees what it owns
-            p->shadow->k_cache = p->own_k;
-            p->shadow->vt_cache = p->own_vt;
-            p->shadow->capacity = p->own_capacity;
-            dflash_session_destroy(p->shadow);
+        for (auto &x : p->extra) {
+            if (x.join) (void)hipEventDestroy(x.join);
+            if (x.shadow) {  // give it back its own cache before it frees what it owns
+                x.shadow->k_cache = x.own_k;
+                x.shadow->vt_cache = x.own_vt;
+                x.shadow->capacity = x.own_capacity;
+                dflash_session_destroy(x.shadow);
+            }
+            if (x.ctx) dflash_ctx_destroy(x.ctx);  // (the stream belongs to the process-wide pool)
         }
-        if (p->stream2) (void)hipStreamDestroy(p->stream2);
-        if (p->ctx2) dflash_ctx_destroy(p->ctx2);
         delete p;
         s->pipe = nullptr;
     }
@@ -661,9 +669,12 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
             packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
             L.k_norm, kc, s->pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta, packed ? s->pk + q_dim + kv_dim : s->v,
             packed ? tot : kv_dim, vtc, s->capacity);
-        if (lane) {  // this block's K/V rows of the layer are written; the previous block's must be before the attention reads them
-            DFL_HIP_CHECK(ctx, hipEventRecord(lane->mine[il], st));
+        if (lane) {
+            // This block's K/V rows of the layer are written; the earlier blocks' must be before the attention reads
+            // them.  The wait for the previous block comes first and the record behind it: the event then stands for
+            // "rows of this block AND of every block before it", whichever lanes those ran on.
             if (lane->wait_other) DFL_HIP_CHECK(ctx, hipStreamWaitEvent(st, lane->other[il], 0));
+            DFL_HIP_CHECK(ctx, hipEventRecord(lane->mine[il], st));
         }
         // under capture the context length is read from pos[0] on the device: the same launches then serve every
         // position of the bucket
@@ -831,25 +842,48 @@ int32_t prefill_pipe_create(dflash_ctx *ctx, dflash_session *s) {
     PrefillPipe *p = new (std::nothrow) PrefillPipe();
     if (!p) return dfl_fail(ctx, DFLASH_ERR_HIP, "prefill_blocks: out of host memory");
     s->pipe = p;  // (whatever has been made so far is taken down with the session)
-    int32_t rc = dflash_ctx_create(ctx->device, ctx->workspace_bytes, &p->ctx2);
-    if (rc) return dfl_fail(ctx, rc, "prefill_blocks: second context");
-    if ((rc = dflash_session_create(p->ctx2, &s->cfg, 16, s->n_taps, &p->shadow))) return dfl_fail(ctx, rc, "prefill_blocks: second scratch set");
-    p->own_k = p->shadow->k_cache;
-    p->own_vt = p->shadow->vt_cache;
-    p->own_capacity = p->shadow->capacity;
-    p->shadow->k_cache = s->k_cache;
-    p->shadow->vt_cache = s->vt_cache;
-    p->shadow->capacity = s->capacity;
-    DFL_HIP_CHECK(ctx, hipStreamCreateWithFlags(&p->stream2, hipStreamNonBlocking));
-    for (auto &v : p->kv_done) {
-        v.assign(s->cfg.n_layers, nullptr);
-        for (hipEvent_t &e : v) DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    static const int lanes_env = [] {
+        const char *v = getenv("DFLASH_PREFILL_LANES");
+        return v && *v ? atoi(v) : 4;  // measured on the 35B-A3B shape: 3290 / 4530 / 5160 / 5650 / 5150 / 4870 prompt tokens/s with
+    }();                               // 1 / 2 / 3 / 4 / 6 / 8 blocks in flight (a process has four hardware queues)
+    p->n_lanes = std::max(1, std::min(kMaxPrefillLanes, lanes_env));
+    for (int i = 0; i + 1 < p->n_lanes; i++) {
+        PrefillPipe::Extra &x = p->extra[i];
+        int32_t rc = dflash_ctx_create(ctx->device, ctx->workspace_bytes, &x.ctx);
+        if (rc) return dfl_fail(ctx, rc, "prefill_blocks: context of lane %d", i + 1);
+        if ((rc = dflash_session_create(x.ctx, &s->cfg, 16, s->n_taps, &x.shadow)))
+            return dfl_fail(ctx, rc, "prefill_blocks: scratch set of lane %d", i + 1);
+        x.own_k = x.shadow->k_cache;
+        x.own_vt = x.shadow->vt_cache;
+        x.own_capacity = x.shadow->capacity;
+        x.shadow->k_cache = s->k_cache;
+        x.shadow->vt_cache = s->vt_cache;
+        x.shadow->capacity = s->capacity;
+        // The lane streams are made once per process and device and shared by every session.  Streams made afresh
+        // for a second session (after the first one's were destroyed) landed on fewer hardware queues: its prefill
+        // ran at the pace of two lanes (448 against 348 ms for 2048 tokens).
+        static hipStream_t pool[16][kMaxPrefillLanes - 1] = {};
+        const int dev = ctx->device >= 0 && ctx->device < 16 ? ctx->device : 0;
+        if (!pool[dev][i]) DFL_HIP_CHECK(ctx, hipStreamCreateWithFlags(&pool[dev][i], hipStreamNonBlocking));
+        x.stream = pool[dev][i];
+        DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&x.join, hipEventDisableTiming));
+    }
+    for (int i = 0; i < p->n_lanes; i++) {
+        p->kv_done[i].assign(s->cfg.n_layers, nullptr);
+        for (hipEvent_t &e : p->kv_done[i]) DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
     }
     DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&p->fork, hipEventDisableTiming));
-    DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&p->join, hipEventDisableTiming));
+    p->ready = true;
     return DFLASH_OK;
 }
 }  // namespace
+
+int32_t dflash_prefill_prepare(dflash_ctx *ctx, dflash_session *s) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "prefill_prepare: null session");
+    if (s->pipe) return s->pipe->ready ? DFLASH_OK : dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_prepare: the extra lanes could not be set up earlier");
+    return prefill_pipe_create(ctx, s);
+}
 
 int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
                               int32_t n_tokens, int64_t start, const int32_t *tap_layers, int32_t n_taps,
@@ -873,17 +907,23 @@ int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash
     int32_t rc = DFLASH_OK;
     if (!s->pipe && (rc = prefill_pipe_create(ctx, s))) return rc;
     PrefillPipe *p = s->pipe;
-    if (!p->shadow || !p->stream2 || !p->join) return dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_blocks: the second lane could not be set up earlier");
-    hipStream_t lanes_st[2] = {static_cast<hipStream_t>(stream), p->stream2};
-    dflash_ctx *lanes_ctx[2] = {ctx, p->ctx2};
-    dflash_session *lanes_s[2] = {s, p->shadow};
-    // the second lane starts behind whatever the caller's stream holds (earlier blocks' K/V rows among it)
+    if (!p->ready) return dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_blocks: the extra lanes could not be set up earlier");
+    const int n_lanes = p->n_lanes;
+    hipStream_t lanes_st[kMaxPrefillLanes] = {static_cast<hipStream_t>(stream)};
+    dflash_ctx *lanes_ctx[kMaxPrefillLanes] = {ctx};
+    dflash_session *lanes_s[kMaxPrefillLanes] = {s};
+    // the extra lanes start behind whatever the caller's stream holds (earlier blocks' K/V rows among it)
     DFL_HIP_CHECK(ctx, hipEventRecord(p->fork, lanes_st[0]));
-    DFL_HIP_CHECK(ctx, hipStreamWaitEvent(lanes_st[1], p->fork, 0));
+    for (int i = 1; i < n_lanes; i++) {
+        lanes_st[i] = p->extra[i - 1].stream;
+        lanes_ctx[i] = p->extra[i - 1].ctx;
+        lanes_s[i] = p->extra[i - 1].shadow;
+        DFL_HIP_CHECK(ctx, hipStreamWaitEvent(lanes_st[i], p->fork, 0));
+    }
     const size_t cap_row = static_cast<size_t>(std::max(n_taps, 0)) * c.hidden;
     int block = 0;
     for (int32_t t0 = 0; t0 < n_tokens && !rc; t0 += 16, block++) {
-        const int lane_i = block & 1;
+        const int lane_i = block % n_lanes, prev_i = (block + n_lanes - 1) % n_lanes;
         const int32_t n = std::min<int32_t>(16, n_tokens - t0);
         dflash_session *ls = lanes_s[lane_i];
         Int16Args ids_arg = {}, pos_arg = {};
@@ -892,21 +932,23 @@ int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash
             pos_arg.v[i] = static_cast<int32_t>(start + t0 + i);
         }
         set_ids_pos_kernel<<<1, 64, 0, lanes_st[lane_i]>>>(ids_arg, pos_arg, n, ls->ids, ls->pos, nullptr, c.vocab);
-        const PrefillLane lane = {p->kv_done[lane_i].data(), p->kv_done[lane_i ^ 1].data(), block > 0};
+        const PrefillLane lane = {p->kv_done[lane_i].data(), p->kv_done[prev_i].data(), block > 0 && n_lanes > 1};
         rc = verify_enqueue(lanes_ctx[lane_i], model, ls, n, start + t0, tap_layers, n_taps,
                             hidden_capture ? hidden_capture + static_cast<size_t>(t0) * cap_row : nullptr, ls->logits, ls->argmax, ls->gap,
                             lanes_st[lane_i], false, &lane);
-        if (rc && lane_i == 1) rc = dfl_fail(ctx, rc, "prefill_blocks: %s", dflash_last_error(p->ctx2));
+        if (rc && lane_i > 0) rc = dfl_fail(ctx, rc, "prefill_blocks: %s", dflash_last_error(lanes_ctx[lane_i]));
     }
-    // the caller's stream continues behind both lanes
-    const hipError_t e1 = hipEventRecord(p->join, lanes_st[1]);
-    const hipError_t e2 = e1 == hipSuccess ? hipStreamWaitEvent(lanes_st[0], p->join, 0) : e1;
+    // the caller's stream continues behind every lane
+    hipError_t err = hipSuccess;
+    for (int i = 1; i < n_lanes && err == hipSuccess; i++) {
+        err = hipEventRecord(p->extra[i - 1].join, lanes_st[i]);
+        if (err == hipSuccess) err = hipStreamWaitEvent(lanes_st[0], p->extra[i - 1].join, 0);
+    }
     if (rc) {
-        (void)hipStreamSynchronize(lanes_st[1]);
-        (void)hipStreamSynchronize(lanes_st[0]);
+        for (int i = n_lanes - 1; i >= 0; i--) (void)hipStreamSynchronize(lanes_st[i]);
         return rc;  // (kv_n_pos unchanged: rows written past it are overwritten by the next block)
     }
-    DFL_HIP_CHECK(ctx, e2);
+    DFL_HIP_CHECK(ctx, err);
     s->kv_n_pos = start + n_tokens;
     return DFLASH_OK;
 }

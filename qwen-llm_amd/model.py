@@ -511,6 +511,12 @@ class Session:
         return VerifyOutput(argmax[:n] if want_head else None, gap[:n] if want_head else None, hidden, logits,
                             list(host[:n]) if sync else None)
 
+    def prepare_prefill(self):
+        """Makes the extra lanes of prefill_blocks now instead of inside its first call."""
+        self._L.dflash_prefill_prepare.restype = C.c_int32
+        self._L.dflash_prefill_prepare.argtypes = [C.c_void_p, C.c_void_p]
+        self.ctx._check(self._L.dflash_prefill_prepare(self.ctx._h, self._h))
+
     def prefill_blocks(self, tokens, start_position: int, want_hidden=True):
         """The prompt's blocks without the output head, two blocks in flight (dflash_prefill_blocks); returns the tapped
         hidden rows [n_tokens][n_taps][hidden] (or None).  Enqueue only."""
@@ -749,6 +755,7 @@ class SpeculativeDecoder:
         self.ctx, self.target, self.head = ctx, target, head
         self.tap_layers = list(tap_layers)
         self.session = Session(ctx, target, kv_capacity, self.tap_layers)
+        self.session.prepare_prefill()  # (the prompt's lanes are made with the decoder, not inside its first prefill)
         self.draft_session = DraftSession(ctx, head, target, kv_capacity)
         self.sampler = sampler
         self.proposal_sampler = proposal_sampler
@@ -772,7 +779,7 @@ class SpeculativeDecoder:
         """Run the prompt through the packed verify in blocks of 16, feed the tapped hidden rows to
         the drafter context, and return the argmax after the last prompt token."""
         assert len(prompt) > 0 and self.position == 0
-        # every block but the last: K/V and the tapped rows only, two blocks in flight; the last one with its head
+        # every block but the last: K/V and the tapped rows only, four blocks in flight; the last one with its head
         body = (len(prompt) - 1) // 16 * 16
         if body:
             hidden = self.session.prefill_blocks(list(prompt[:body]), 0)
