@@ -133,6 +133,26 @@ def test_expert_kernel_rows_do_not_depend_on_the_rest_of_the_block(ctx, weights)
     s_one.close()
 
 
+def test_pipelined_prefill_on_the_moe_shape_equals_block_by_block(ctx, weights):
+    """Four blocks in flight through the mixture-of-experts layers (each lane routes and runs its experts in its own
+    scratch and context): captured rows and the following block's logits equal block-by-block execution bit for bit."""
+    model = dfl.TargetModel(ctx, C5, weights)
+    rng = np.random.default_rng(21)
+    toks = rng.integers(0, C5.vocab, 16 * 6 + 3).tolist()
+    probe = rng.integers(0, C5.vocab, 16).tolist()
+    ref, pipe = dfl.Session(ctx, model, 256, TAPS), dfl.Session(ctx, model, 256, TAPS)
+    got = pipe.prefill_blocks(toks, 0)
+    want = []
+    for s0 in range(0, len(toks), 16):
+        want.append(ref.encode_packed_verify_layer_major(toks[s0:s0 + 16], s0, want_head=False).hidden_capture.cpu().numpy())
+    assert np.array_equal(got.cpu().numpy(), np.concatenate(want, axis=0))
+    a = ref.encode_packed_verify_layer_major(probe, len(toks), want_logits=True)
+    b = pipe.encode_packed_verify_layer_major(probe, len(toks), want_logits=True)
+    assert np.array_equal(a.logits.cpu().numpy(), b.logits.cpu().numpy())
+    ref.close()
+    pipe.close()
+
+
 _ROUTE_PROBE = r"""
 import sys
 import numpy as np
