@@ -124,9 +124,26 @@ struct dfl_moe_scratch {
 // already holds sigmoid(cur . shexp_gate) per row (the norm kernel that wrote cur computed it).
 // next_norm_w / next_cur / next_done (all or none): the RMSNorm that reads x_resid next may be done
 // in the same pass, next_cur = rms_norm(x_resid) * next_norm_w; *next_done says whether it was.
-int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, const float *cur, int n,
+// pre_add / pre_norm_w (both or neither; only where dfl_moe_norm_fusable() holds): the layer's input has not been
+// normalised yet, x_resid still lacks pre_add (the attention's output projection), and `cur` is where the normalised rows
+// go: cur = rms_norm(x_resid + pre_add) * pre_norm_w, computed inside the router's launch with the shared-expert gate
+// (gate_done is then implied); x_resid += pre_add happens where the experts' sum is added.
+int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, float *cur, int n,
                     const dfl_moe_scratch &scratch, float *x_resid, bool gate_done, const float *next_norm_w,
-                    float *next_cur, bool *next_done, hipStream_t stream);
+                    float *next_cur, bool *next_done, hipStream_t stream, const float *pre_add = nullptr,
+                    const float *pre_norm_w = nullptr);
+bool dfl_moe_norm_fusable(const dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, int n);
+
+// Residual add + RMSNorm + shared-expert gate + Q8_0 router product of a mixture-of-experts layer as one launch:
+// cur[n_rows][hidden] = rms_norm(x + add) * norm_w, gate_out[r] = sigmoid(cur[r] . gate_w),
+// logits[n_rows][n_expert] = cur . router_w^T, bit-identical to the norm kernel followed by the few-row GEMM.
+// x is left as it is.  dfl_router_norm_fits: whether the shape is one the kernel takes (hidden a multiple of 256, at
+// most 2048; 1..16 rows); switched off by DFLASH_MOE_FUSED_NORM=0.  Enqueue only.
+bool dfl_router_norm_fits(const dflash_ctx *ctx, int32_t router_type, const void *router_w, int64_t hidden, int32_t n_expert,
+                          int32_t n_rows);
+int32_t dfl_router_norm(dflash_ctx *ctx, const void *router_w, const float *x, const float *add, const float *norm_w,
+                        const float *gate_w, float eps, float *cur, float *gate_out, float *logits, int64_t hidden,
+                        int32_t n_expert, int32_t n_rows, hipStream_t stream);
 
 // dflash_attn_verify_block with the drafter's masks: full_block != 0 lets every row see the whole
 // block (non-causal), window > 0 keeps only keys with |distance| < window.  ctx_len_dev != null:

@@ -10,7 +10,9 @@
 #include "device_quant.h"
 
 #include <algorithm>
+#include <array>
 #include <map>
+#include <mutex>
 #include <chrono>
 #include <cmath>
 #include <cstring>
@@ -436,7 +438,7 @@ struct dflash_session {
     std::map<uint64_t, hipGraphExec_t> graphs;
     std::map<uint64_t, int> graph_seen;
     int64_t graph_replays = 0;
-    struct PrefillPipe *pipe = nullptr;  // second lane of dflash_prefill_blocks, made on first use
+    struct PrefillPipe *pipe = nullptr;  // extra lanes of dflash_prefill_blocks (dflash_prefill_prepare, else made on first use)
 };
 
 // Extra lanes of a pipelined prefill.  A 16-row block's layers are a chain of small dependent launches that leave most
@@ -684,11 +686,16 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
         if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
         // x += mix first; a mixture-of-experts layer also gets its shared-expert gate from here
         const bool moe = c.n_expert > 0;
-        rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps, moe ? L.shexp_gate : nullptr,
-                                           moe ? s->moe.sg : nullptr);
+        // (where the router's launch can take the add and the norm along, they are left to it; s->x then gets its
+        // s->mix together with the experts' sum)
+        const bool norm_in_router = moe && dfl_moe_norm_fusable(ctx, c, L, n);
+        if (!norm_in_router)
+            rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps, moe ? L.shexp_gate : nullptr,
+                                               moe ? s->moe.sg : nullptr);
         if (moe) {
             const float *next_w = il + 1 < c.n_layers ? model->layers[il + 1].attn_norm : model->output_norm;
-            if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, L.shexp_gate != nullptr, next_w, s->cur, &cur_ready, st)))
+            if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, L.shexp_gate != nullptr, next_w, s->cur, &cur_ready, st,
+                                  norm_in_router ? s->mix : nullptr, norm_in_router ? L.post_norm : nullptr)))
                 return rc;
         } else {
             if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, n, st))) return rc;
@@ -862,10 +869,14 @@ int32_t prefill_pipe_create(dflash_ctx *ctx, dflash_session *s) {
         // The lane streams are made once per process and device and shared by every session.  Streams made afresh
         // for a second session (after the first one's were destroyed) landed on fewer hardware queues: its prefill
         // ran at the pace of two lanes (448 against 348 ms for 2048 tokens).
-        static hipStream_t pool[16][kMaxPrefillLanes - 1] = {};
-        const int dev = ctx->device >= 0 && ctx->device < 16 ? ctx->device : 0;
-        if (!pool[dev][i]) DFL_HIP_CHECK(ctx, hipStreamCreateWithFlags(&pool[dev][i], hipStreamNonBlocking));
-        x.stream = pool[dev][i];
+        {
+            static std::mutex pool_mutex;
+            static std::map<int, std::array<hipStream_t, kMaxPrefillLanes - 1>> pool;  // by device ordinal
+            std::lock_guard<std::mutex> lock(pool_mutex);
+            hipStream_t &slot = pool[ctx->device][i];  // (a new entry starts as null pointers)
+            if (!slot) DFL_HIP_CHECK(ctx, hipStreamCreateWithFlags(&slot, hipStreamNonBlocking));
+            x.stream = slot;
+        }
         DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&x.join, hipEventDisableTiming));
     }
     for (int i = 0; i < p->n_lanes; i++) {

@@ -371,7 +371,7 @@ __global__ void __launch_bounds__(256)
     moe_combine_norm_kernel(const float *__restrict__ eo, const int32_t *__restrict__ slot_of, const float *__restrict__ sel_w,
                             const float *__restrict__ sg, const float *__restrict__ shared, const int32_t *__restrict__ n_slots,
                             int n_used, int hidden, float *__restrict__ x, const float *__restrict__ norm_w,
-                            float *__restrict__ y, float eps) {
+                            float *__restrict__ y, float eps, const float *__restrict__ pre_add) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
     __shared__ float w_k[64];
@@ -397,7 +397,10 @@ __global__ void __launch_bounds__(256)
             const f4 shv = shared ? *reinterpret_cast<const f4 *>(shared + static_cast<size_t>(row) * hidden + i)
                                   : *reinterpret_cast<const f4 *>(eo + (last * 16 + row) * hidden + i);
             out += gate * shv;
-            v[j] = *reinterpret_cast<const f4 *>(x + static_cast<size_t>(row) * hidden + i) + out;
+            v[j] = *reinterpret_cast<const f4 *>(x + static_cast<size_t>(row) * hidden + i);
+            // (a residual term the norm before this layer's experts left out: it goes in first, as it would have there)
+            if (pre_add) v[j] += *reinterpret_cast<const f4 *>(pre_add + static_cast<size_t>(row) * hidden + i);
+            v[j] += out;
             *reinterpret_cast<f4 *>(x + static_cast<size_t>(row) * hidden + i) = v[j];
         }
         s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
@@ -417,10 +420,30 @@ __global__ void __launch_bounds__(256)
 
 }  // namespace
 
-int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, const float *cur, int n,
+namespace {
+// whether the layer's expert stacks take the batched launches (one streaming GEMM per projection over the distinct experts)
+bool moe_batched(const dflash_model_cfg &c, const dflash_layer &L) {
+    static const bool per_slot_forced = getenv("DFLASH_MOE_PERSLOT") != nullptr;  // read once per process
+    const int et = L.gate_exps.type, dt = L.down_exps.type;
+    const bool tiled = et == DFLASH_TYPE_Q4_K_TILED;
+    return (tiled || (et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K)) && c.hidden % DFL_QK_K == 0 && c.ffn_expert % DFL_QK_K == 0 &&
+           !per_slot_forced;
+}
+}  // namespace
+
+bool dfl_moe_norm_fusable(const dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, int n) {
+    // the residual term is added back by moe_combine_norm_kernel, which the batched path ends with
+    return c.n_expert > 0 && L.shexp_gate && L.router.data && L.gate_exps.data && L.down_exps.data && moe_batched(c, L) &&
+           c.hidden <= 4096 && c.hidden % 4 == 0 && dfl_router_norm_fits(ctx, L.router.type, L.router.data, c.hidden, c.n_expert, n);
+}
+
+int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, float *cur, int n,
                     const dfl_moe_scratch &s, float *x_resid, bool gate_done, const float *next_norm_w, float *next_cur,
-                    bool *next_done, hipStream_t st) {
+                    bool *next_done, hipStream_t st, const float *pre_add, const float *pre_norm_w) {
     if (next_done) *next_done = false;
+    if ((pre_add != nullptr) != (pre_norm_w != nullptr) ||
+        (pre_add && !(next_norm_w && next_cur && next_done && dfl_moe_norm_fusable(ctx, c, L, n))))
+        return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "moe: the norm can ride in the router's launch only where dfl_moe_norm_fusable() holds");
     const int E = c.n_expert, used = c.n_expert_used < E ? c.n_expert_used : E;
     const int H = c.hidden, fe = c.ffn_expert, fs = c.ffn_shared;
     const int n_slots = n * used;
@@ -441,12 +464,16 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     const size_t rb_in = dflash_row_bytes(et, H), rb_dn = dflash_row_bytes(dt, fe);
     if (rb_in == 0 || rb_dn == 0) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "moe: row sizes do not fit the block size");
 
-    int32_t rc = dflash_gemm_fewrow(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
+    int32_t rc;
+    if (pre_add) {
+        rc = dfl_router_norm(ctx, L.router.data, x_resid, pre_add, pre_norm_w, L.shexp_gate, c.eps, cur, s.sg, s.probs, H, E, n, st);
+        gate_done = true;
+    } else {
+        rc = dflash_gemm_fewrow(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
+    }
     if (rc) return rc;
     if (E > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: %d experts (at most 1024)", E);
-    static const bool per_slot_forced = getenv("DFLASH_MOE_PERSLOT") != nullptr;  // read once per process
-    const bool batched = (tiled || (et == DFLASH_TYPE_Q4_K && dt == DFLASH_TYPE_Q4_K)) && H % DFL_QK_K == 0 && fe % DFL_QK_K == 0 &&
-                         !per_slot_forced;
+    const bool batched = moe_batched(c, L);
     if (tiled && !batched) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: tiled expert stacks need the batched path");
     // the shared expert rides along as one more slot of the batched GEMMs when it has the experts' shape (and order)
     const bool folded_shared = batched && fs == fe && L.gate.type == et && L.up.type == et && L.down.type == et;
@@ -529,7 +556,7 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     }
     if (batched && next_norm_w && next_cur && next_done && H <= 4096 && H % 4 == 0) {
         moe_combine_norm_kernel<<<n, 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg, folded_shared ? nullptr : s.shared, s.n_distinct,
-                                                   used, H, x_resid, next_norm_w, next_cur, c.eps);
+                                                   used, H, x_resid, next_norm_w, next_cur, c.eps, pre_add);
         *next_done = true;
     } else if (batched)
         moe_combine_slots_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg,

@@ -167,17 +167,16 @@ outs = []
 pos = 0
 for n in (16, 4, 1):
     out = sess.encode_packed_verify_layer_major(rng.integers(0, cfg.vocab, n).tolist(), pos, want_logits=True)
-    outs.append(out.logits.cpu().numpy())
+    outs.append(np.concatenate([out.logits.cpu().numpy(), out.hidden_capture.cpu().numpy().reshape(n, -1)], axis=1))
     pos += n
 np.save(sys.argv[1], np.concatenate(outs, axis=0))
 """
 
 
-def test_routing_inside_the_expert_launch_equals_the_routing_kernel(tmp_path):
-    """The expert list, the weights and the slots come out of the same row arithmetic (moe_route.h) whether the
-    gate/up launch derives them in its prologue or moe_route_small_kernel does in a launch of its own: the logits of
-    three blocks (16, 4 and 1 rows) are equal bit for bit.  The switch is read once per process, so each setting runs
-    in a process of its own (two short-lived ones, one after the other)."""
+def _probe_under(tmp_path, knob):
+    """Logits and captured rows of three blocks (16, 4 and 1 rows) with the environment switch `knob` at 1 and at 0.  The
+    switches are read once per process, so each setting runs in a process of its own (two short-lived ones, one after
+    the other)."""
     import os
     import subprocess
     import sys
@@ -185,14 +184,31 @@ def test_routing_inside_the_expert_launch_equals_the_routing_kernel(tmp_path):
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     got = {}
     for flag in ("1", "0"):
-        path = str(tmp_path / f"logits_{flag}.npy")
-        env = dict(os.environ, DFLASH_MOE_FUSED_ROUTE=flag, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+        path = str(tmp_path / f"out_{flag}.npy")
+        env = dict(os.environ, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+        env[knob] = flag
         r = subprocess.run([sys.executable, "-c", _ROUTE_PROBE, path], env=env, cwd=root, capture_output=True, text=True, timeout=240)
         assert r.returncode == 0, r.stderr[-2000:]
         got[flag] = np.load(path)
-    assert got["1"].shape == got["0"].shape == (21, 8192)
+    assert got["1"].shape == got["0"].shape == (21, 8192 + 2 * 2048)
     assert np.all(np.isfinite(got["1"]))
-    assert np.array_equal(got["1"], got["0"])
+    return got["1"], got["0"]
+
+
+def test_routing_inside_the_expert_launch_equals_the_routing_kernel(tmp_path):
+    """The expert list, the weights and the slots come out of the same row arithmetic (moe_route.h) whether the
+    gate/up launch derives them in its prologue or moe_route_small_kernel does in a launch of its own: logits and
+    captured rows are equal bit for bit."""
+    on, off = _probe_under(tmp_path, "DFLASH_MOE_FUSED_ROUTE")
+    assert np.array_equal(on, off)
+
+
+def test_norm_inside_the_router_launch_equals_the_norm_kernel(tmp_path):
+    """Residual add, RMSNorm and shared-expert gate computed by every workgroup of the router's launch (the residual
+    term added to x later, with the experts' sum) against rms_norm_kernel followed by the Q8_0 product: the sums are
+    taken in the same order, so logits and captured rows are equal bit for bit."""
+    on, off = _probe_under(tmp_path, "DFLASH_MOE_FUSED_NORM")
+    assert np.array_equal(on, off)
 
 
 def test_generate_on_the_moe_shape_equals_serial_greedy(ctx, weights):
