@@ -2205,10 +2205,10 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
 // with the norm of all 16 rows inside each of the 8 workgroups, 290 KB each: slower than the two launches.)  The
 // workgroups of tile 0 write the row's f32 copy (cur, read by the expert products) and its gate.  x itself is NOT
 // updated (other workgroups are still reading the row): the caller adds `add` again where it next updates the
-// residual.  Sums are taken in rms_norm_kernel's order and the product in the order of the kernel above with 16
-// waves (each of the four waves here plays four of them, one after the other), so cur, gate_out and y have the bits
-// of the two separate launches.  One 64-step chunk: hidden <= 2048.
-__global__ void __launch_bounds__(256)
+// residual.  Sums are taken in rms_norm_kernel's order (the first four waves do the norm) and the product in the order
+// of the kernel above with 16 waves, so cur, gate_out and y have the bits of the two separate launches.  One 64-step
+// chunk: hidden <= 2048.
+__global__ void __launch_bounds__(64 * kMaxSplit)
     q8_0_norm_router_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, const float *__restrict__ add,
                             const float *__restrict__ norm_w, const float *__restrict__ gate_w, float eps,
                             float *__restrict__ cur, float *__restrict__ gate_out, float *__restrict__ y, int n_out,
@@ -2224,50 +2224,58 @@ __global__ void __launch_bounds__(256)
     const int n0 = blockIdx.x * 16, r = blockIdx.y;
     const int hidden = 32 * n_steps;
     const bool first_tile = blockIdx.x == 0;
+    const bool norm_wave = wave < 4;  // the norm is the work of 256 threads, as in rms_norm_kernel; the row's loads go out first
+    f4 v[2] = {f4{0, 0, 0, 0}, f4{0, 0, 0, 0}};
+    if (norm_wave) {
+        const float *xr = x + static_cast<size_t>(r) * hidden, *ar = add + static_cast<size_t>(r) * hidden;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int i = 4 * (tid + 256 * j);
+            if (i < hidden) v[j] = *reinterpret_cast<const f4 *>(xr + i) + *reinterpret_cast<const f4 *>(ar + i);
+        }
+    }
     const int wp_row = n_steps * DFL_Q8_0_BYTES / 16;
-    for (int p = tid; p < 16 * wp_row; p += 256) {
+    for (int p = tid; p < 16 * wp_row; p += 64 * kMaxSplit) {
         const int wr = p / wp_row, c = p - wr * wp_row;
         const int row = min(n0 + wr, n_out - 1);
         *reinterpret_cast<u32x4_t *>(ws + wr * kQ8WRowStride + 16 * c) =
             *reinterpret_cast<const u32x4_t *>(w + static_cast<size_t>(row) * row_bytes + 16 * c);
     }
-    const float *xr = x + static_cast<size_t>(r) * hidden, *ar = add + static_cast<size_t>(r) * hidden;
-    f4 v[2];
-    float s = 0.0f;
+    if (norm_wave) {
+        float s = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int i = 4 * (tid + 256 * j);
-        v[j] = f4{0, 0, 0, 0};
-        if (i < hidden) v[j] = *reinterpret_cast<const f4 *>(xr + i) + *reinterpret_cast<const f4 *>(ar + i);
-        s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
+        for (int j = 0; j < 2; j++)
+            s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
+        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        if (lane == 0) sq_part[wave] = s;
     }
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-    if (lane == 0) sq_part[wave] = s;
     __syncthreads();
-    float tot = 0.0f;
+    if (norm_wave) {
+        float tot = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 4; k++) tot += sq_part[k];
-    const float scale = 1.0f / sqrtf(tot / static_cast<float>(hidden) + eps);
-    float dot = 0.0f;
+        for (int k = 0; k < 4; k++) tot += sq_part[k];
+        const float scale = 1.0f / sqrtf(tot / static_cast<float>(hidden) + eps);
+        float dot = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int i = 4 * (tid + 256 * j);
-        if (i < hidden) {
-            const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
-            if (first_tile) {
-                *reinterpret_cast<f4 *>(cur + static_cast<size_t>(r) * hidden + i) = o;
-                const f4 gw = *reinterpret_cast<const f4 *>(gate_w + i);
-                dot += (o[0] * gw[0] + o[1] * gw[1]) + (o[2] * gw[2] + o[3] * gw[3]);
+        for (int j = 0; j < 2; j++) {
+            const int i = 4 * (tid + 256 * j);
+            if (i < hidden) {
+                const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
+                if (first_tile) {
+                    *reinterpret_cast<f4 *>(cur + static_cast<size_t>(r) * hidden + i) = o;
+                    const f4 gw = *reinterpret_cast<const f4 *>(gate_w + i);
+                    dot += (o[0] * gw[0] + o[1] * gw[1]) + (o[2] * gw[2] + o[3] * gw[3]);
+                }
+                // values 8 c .. 8 c + 7 are piece c = 4 step + k-group; this thread's four are its lower or upper half
+                h4 *piece = reinterpret_cast<h4 *>(&xrow[i >> 3]);
+                piece[(i >> 2) & 1] = h4{static_cast<_Float16>(o[0]), static_cast<_Float16>(o[1]), static_cast<_Float16>(o[2]),
+                                         static_cast<_Float16>(o[3])};
             }
-            // values 8 c .. 8 c + 7 are piece c = 4 step + k-group; this thread's four are its lower or upper half
-            h4 *piece = reinterpret_cast<h4 *>(&xrow[i >> 3]);
-            piece[(i >> 2) & 1] = h4{static_cast<_Float16>(o[0]), static_cast<_Float16>(o[1]), static_cast<_Float16>(o[2]),
-                                     static_cast<_Float16>(o[3])};
         }
-    }
-    if (first_tile) {  // (the same for the whole workgroup)
-        for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-        if (lane == 0) dot_part[wave] = dot;
+        if (first_tile) {  // (the same for the whole workgroup)
+            for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+            if (lane == 0) dot_part[wave] = dot;
+        }
     }
     __syncthreads();  // the row, the weight rows and the gate's partial sums are in LDS
     if (first_tile && tid == 0) {
@@ -2277,25 +2285,22 @@ __global__ void __launch_bounds__(256)
     }
     const uint8_t *rowp = ws + n * kQ8WRowStride;
     const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    const int ri = r & 3;
-    for (int k = 0; k < 4; k++) {
-        const int vw = 4 * wave + k;  // the wave of the 16-wave kernel whose steps these are
-        const int s0 = n_steps * vw / kMaxSplit, s1 = n_steps * (vw + 1) / kMaxSplit;
-        float4_t acc = {0, 0, 0, 0};
-        for (int st = s0; st < s1; st++) {
-            const uint8_t *blk = rowp + st * DFL_Q8_0_BYTES;  // 2-byte aligned
-            const uint16_t *q16 = reinterpret_cast<const uint16_t *>(blk + 2 + 8 * g);
-            Raw8<DFLASH_TYPE_Q8_0> rw;
-            rw.d = static_cast<float>(__builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t *>(blk)));
-            rw.q = static_cast<uint64_t>(q16[0]) | (static_cast<uint64_t>(q16[1]) << 16) | (static_cast<uint64_t>(q16[2]) << 32) |
-                   (static_cast<uint64_t>(q16[3]) << 48);
-            const half8_t piece = xrow[4 * st + g];
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(n == r ? piece : zero, convert_raw8<DFLASH_TYPE_Q8_0>(rw), acc, 0, 0, 0);
-        }
-        // output row r sits in lane group r / 4, element r % 4
-        const float mine = ri == 0 ? acc[0] : ri == 1 ? acc[1] : ri == 2 ? acc[2] : acc[3];
-        if (g == (r >> 2)) red[vw][n] = mine;
+    const int s0 = n_steps * wave / kMaxSplit, s1 = n_steps * (wave + 1) / kMaxSplit;
+    float4_t acc = {0, 0, 0, 0};
+    for (int st = s0; st < s1; st++) {
+        const uint8_t *blk = rowp + st * DFL_Q8_0_BYTES;  // 2-byte aligned
+        const uint16_t *q16 = reinterpret_cast<const uint16_t *>(blk + 2 + 8 * g);
+        Raw8<DFLASH_TYPE_Q8_0> rw;
+        rw.d = static_cast<float>(__builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t *>(blk)));
+        rw.q = static_cast<uint64_t>(q16[0]) | (static_cast<uint64_t>(q16[1]) << 16) | (static_cast<uint64_t>(q16[2]) << 32) |
+               (static_cast<uint64_t>(q16[3]) << 48);
+        const half8_t piece = xrow[4 * st + g];
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(n == r ? piece : zero, convert_raw8<DFLASH_TYPE_Q8_0>(rw), acc, 0, 0, 0);
     }
+    // output row r sits in lane group r / 4, element r % 4
+    const int ri = r & 3;
+    const float mine = ri == 0 ? acc[0] : ri == 1 ? acc[1] : ri == 2 ? acc[2] : acc[3];
+    if (g == (r >> 2)) red[wave][n] = mine;
     __syncthreads();
     if (tid < 16 && n0 + tid < n_out) {
         float sum = 0.0f;
@@ -2739,7 +2744,7 @@ int32_t dfl_router_norm(dflash_ctx *ctx, const void *router_w, const float *x, c
     const int n_steps = static_cast<int>(hidden / DFL_QK8_0);
     const int tiles = (n_expert + 15) / 16;
     dfl_timed timer(ctx, st, DFL_T_GEMM);
-    q8_0_norm_router_kernel<<<dim3(tiles, n_rows), 256, 0, st>>>(static_cast<const uint8_t *>(router_w), x, add, norm_w, gate_w, eps, cur,
+    q8_0_norm_router_kernel<<<dim3(tiles, n_rows), 64 * kMaxSplit, 0, st>>>(static_cast<const uint8_t *>(router_w), x, add, norm_w, gate_w, eps, cur,
                                                                  gate_out, logits, n_expert, n_steps,
                                                                  static_cast<size_t>(n_steps) * DFL_Q8_0_BYTES);
     DFL_HIP_CHECK(ctx, hipGetLastError());
