@@ -18,6 +18,10 @@ struct dflash_ctx {
     // split-K partial tiles of the Q4_K GEMM (written by the streaming kernel, added up by its reduce kernel)
     void *partials = nullptr;
     int n_partial_wgs = 0;
+    // workgroups of a batched (expert) launch; 0 = one per CU.  The pipelined prefill sets it on its lanes' contexts for
+    // the duration of a call: an expert workgroup fills a CU's LDS, so launches of different lanes cannot share a CU,
+    // and with half the CUs each two of them run side by side, one's start-up and tail under the other's streaming.
+    int batch_wgs = 0;
     size_t lds_bytes = 65536;  // LDS available to one workgroup
     char err[512] = {0};
     // per-kernel timers (off by default; when on, timed launches synchronise)

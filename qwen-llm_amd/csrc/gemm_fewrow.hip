@@ -2491,7 +2491,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
             return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_q4k_batched: activations must be 16-byte aligned");
         const bool per_slot_x = batch->x_stride != 0;
         const int upm = per_slot_x ? (tiles + 15) / 16 : tiles;  // units per matrix
-        int n_wg = env_int("DFLASH_MOE_WGS", ctx->n_cu);
+        int n_wg = env_int("DFLASH_MOE_WGS", ctx->batch_wgs > 0 ? ctx->batch_wgs : ctx->n_cu);
         if (n_wg < 1) n_wg = 1;
         if (static_cast<int64_t>(max_slots) * upm * (n_wg + 1) >= (int64_t(1) << 31) || nb > 4096)
             return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_fewrow: batch too large for 32-bit work indices");
@@ -2551,7 +2551,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     if (tiled && !batch) waves = 16;  // a single tiled matrix: whole 256-row tile groups (a batch may use their halves)
     const int gpm = (tiles + waves - 1) / waves;  // tile groups per matrix
     const int groups = gpm * max_slots * ((batch && batch->pair) ? 2 : 1);  // upper bound in batched mode (pair mode: virtual groups)
-    int n_wg = batch ? env_int("DFLASH_MOE_WGS", ctx->n_cu) : env_int("DFLASH_GEMM_WGS", ctx->n_cu);
+    int n_wg = batch ? env_int("DFLASH_MOE_WGS", ctx->batch_wgs > 0 ? ctx->batch_wgs : ctx->n_cu) : env_int("DFLASH_GEMM_WGS", ctx->n_cu);
     const int64_t total = static_cast<int64_t>(groups) * nb;
     const int max_wgs = ctx->n_partial_wgs * 8 / waves;
     if (n_wg > total) n_wg = static_cast<int>(total);
