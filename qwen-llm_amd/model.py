@@ -518,8 +518,8 @@ class Session:
         self.ctx._check(self._L.dflash_prefill_prepare(self.ctx._h, self._h))
 
     def prefill_blocks(self, tokens, start_position: int, want_hidden=True):
-        """The prompt's blocks without the output head, two blocks in flight (dflash_prefill_blocks); returns the tapped
-        hidden rows [n_tokens][n_taps][hidden] (or None).  Enqueue only."""
+        """The prompt's blocks without the output head, several blocks in flight on the library's lane streams
+        (dflash_prefill_blocks); returns the tapped hidden rows [n_tokens][n_taps][hidden] (or None).  Enqueue only."""
         torch = _torch()
         cfg = self.model.cfg
         n = len(tokens)
