@@ -940,7 +940,7 @@ int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash
         return v && *v ? atoi(v) : 0;
     }();
     const int owner_wgs = ctx->batch_wgs;
-    if (n_lanes > 1)
+    if (n_lanes > 1 && n_tokens > 16)  // (a lone block keeps the whole chip)
         for (int i = 0; i < n_lanes; i++) lanes_ctx[i]->batch_wgs = lane_wgs_env > 0 ? lane_wgs_env : std::max(1, ctx->n_cu / 2);
     int block = 0;
     for (int32_t t0 = 0; t0 < n_tokens && !rc; t0 += 16, block++) {
@@ -959,7 +959,8 @@ int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash
                             lanes_st[lane_i], false, &lane);
         if (rc && lane_i > 0) rc = dfl_fail(ctx, rc, "prefill_blocks: %s", dflash_last_error(lanes_ctx[lane_i]));
     }
-    ctx->batch_wgs = owner_wgs;  // (the extra lanes' contexts serve nothing else)
+    ctx->batch_wgs = owner_wgs;
+    for (int i = 1; i < n_lanes; i++) lanes_ctx[i]->batch_wgs = 0;
     // the caller's stream continues behind every lane
     hipError_t err = hipSuccess;
     for (int i = 1; i < n_lanes && err == hipSuccess; i++) {
