@@ -385,7 +385,8 @@ int64_t dflash_session_graph_replays(const dflash_session *session);
  * logits[n][vocab] f32.  If argmax_host is non-NULL the call waits and copies the n indices
  * there (the reference returns Vec<i32>).  With argmax, gap, logits and argmax_host all NULL the
  * output head (final norm, vocabulary projection, argmax) is not run: a prefill block, of which
- * only the K/V rows and the tapped hidden rows are wanted.  1 <= n <= 16. */
+ * only the K/V rows and the tapped hidden rows are wanted (the last layer then stops behind its
+ * K/V rows unless its residual is tapped).  1 <= n <= 16. */
 int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,
                             const int32_t *tokens_host, int32_t n, int64_t start_position,
                             const int32_t *tap_layers_host, int32_t n_taps, int32_t *argmax, float *gap,

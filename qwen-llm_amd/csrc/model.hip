@@ -678,6 +678,13 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
             if (lane->wait_other) DFL_HIP_CHECK(ctx, hipStreamWaitEvent(st, lane->other[il], 0));
             DFL_HIP_CHECK(ctx, hipEventRecord(lane->mine[il], st));
         }
+        // A block nobody asked head outputs of needs nothing of the last layer beyond its K/V rows, unless that layer's
+        // residual is tapped: its attention, output projection and FFN would only feed the head.
+        if (!want_head && il == c.n_layers - 1) {
+            bool tapped_last = false;
+            for (int t = 0; t < n_taps; t++) tapped_last = tapped_last || tap_layers[t] == il;
+            if (!tapped_last) break;
+        }
         // under capture the context length is read from pos[0] on the device: the same launches then serve every
         // position of the bucket
         if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity, scale,

@@ -99,14 +99,16 @@ def test_verify_block_matches_oracle_and_restore(ctx, oracle, target):
     sess.close()
 
 
-def test_a_block_without_head_outputs_leaves_the_same_state(ctx, target):
-    """A verify block whose caller asks for none of the head's outputs (a prefill block) does not run the head; its K/V
-    rows and tapped hidden rows are those of the same block run in full: the next block's logits are equal bit for
-    bit, for a 16-row and a ragged block, and the guards still hold."""
+@pytest.mark.parametrize("taps", [TAPS, [0, 2]], ids=["last-layer-tapped", "last-layer-untapped"])
+def test_a_block_without_head_outputs_leaves_the_same_state(ctx, target, taps):
+    """A verify block whose caller asks for none of the head's outputs (a prefill block) does not run the head (nor,
+    when the last layer's residual is not tapped, anything of that layer behind its K/V rows); its K/V rows and
+    tapped hidden rows are those of the same block run in full: the next block's logits are equal bit for bit, for a
+    16-row and a ragged block, and the guards still hold."""
     model, _ = target
     rng = np.random.default_rng(77)
     blocks = [rng.integers(0, C1.vocab, n).tolist() for n in (16, 5, 16)]
-    full, lean = dfl.Session(ctx, model, 64, TAPS), dfl.Session(ctx, model, 64, TAPS)
+    full, lean = dfl.Session(ctx, model, 64, taps), dfl.Session(ctx, model, 64, taps)
     pos = 0
     for blk in blocks[:2]:
         a = full.encode_packed_verify_layer_major(blk, pos)
@@ -127,7 +129,7 @@ def test_a_block_without_head_outputs_leaves_the_same_state(ctx, target):
 
 
 def test_pipelined_prefill_equals_block_by_block(ctx, target):
-    """dflash_prefill_blocks (two blocks in flight on two streams, ordered by per-layer events) leaves the K/V rows and
+    """dflash_prefill_blocks (several blocks in flight on the lane streams, ordered by per-layer events) leaves the K/V rows and
     the tapped hidden rows of the same blocks run one by one through dflash_verify_block: the captured rows and the
     next block's logits are equal bit for bit, over a ragged token count, twice in a row on one session (the second
     lane's scratch and events are reused), and its guards hold."""
