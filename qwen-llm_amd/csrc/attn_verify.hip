@@ -372,19 +372,25 @@ __global__ void __launch_bounds__(256)
     const int tid = threadIdx.x;
     const int64_t slot0 = static_cast<int64_t>(head) * 16 + row;
     const int64_t slot_stride = static_cast<int64_t>(n_q) * 16;
-    // m* = max over splits
+    // m* = max over splits (a thread keeps the maxima it loaded: n_splits <= 1024 = 4 per thread)
     float m_loc = -INFINITY;
-    for (int s = tid; s < n_splits; s += 256) m_loc = fmaxf(m_loc, part_ml[(slot0 + s * slot_stride) * 2]);
+    float m_own[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int s = tid + 256 * j;
+        m_own[j] = s < n_splits ? part_ml[(slot0 + s * slot_stride) * 2] : -INFINITY;
+        m_loc = fmaxf(m_loc, m_own[j]);
+    }
     for (int off = 32; off > 0; off >>= 1) m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off, 64));
     if ((tid & 63) == 0) red_l[tid >> 6] = m_loc;
     __syncthreads();
     const float m_star = fmaxf(fmaxf(red_l[0], red_l[1]), fmaxf(red_l[2], red_l[3]));
-    __syncthreads();
-    for (int s = tid; s < n_splits; s += 256) {
-        const float m = part_ml[(slot0 + s * slot_stride) * 2];
-        wgt[s] = (m == -INFINITY) ? 0.0f : exp2f(m - m_star);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int s = tid + 256 * j;
+        if (s < n_splits) wgt[s] = (m_own[j] == -INFINITY) ? 0.0f : exp2f(m_own[j] - m_star);
     }
-    __syncthreads();
+    __syncthreads();  // (also: every thread has read red_l before the split lanes write their sums into it)
     const int sl = tid >> 5, dl = tid & 31;  // split lane, dim lane
     const int n_vec = hd / 4;                // float4 per row: 16, 32 or 64
     float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
