@@ -279,7 +279,7 @@ def acceptance_table(hist):
     return {"alpha_pos1": at_least[0], "per_position_acceptance": at_least, "accept_len_hist": list(hist)}
 
 
-def e2e_speculative(ctx, n_generate, sweep, log):
+def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048):
     """End-to-end DFlash speculative decode on the 35B-A3B-shaped synthetic MoE target (40 layers, hidden 2048,
     16 q / 2 kv heads of 256, 128 experts top-8 with F_exp 768 plus a shared expert; experts Q4_K, attention Q6_K,
     vocabulary 151936) with a 5-layer drafter fed by 3 tapped layers, batch 1, block 16, prompt 2048, greedy accept.
@@ -297,7 +297,7 @@ def e2e_speculative(ctx, n_generate, sweep, log):
                           n_expert_used=8, ffn_expert=768, ffn_shared=768)
     dcfg = dfl.DraftConfig(n_layers=5, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=6144, block_size=16, n_taps=3)
     taps = [1, 19, 38]
-    prompt_len, cap = 2048, 2048 + n_generate + 64
+    cap = prompt_len + n_generate + 64
     t0 = time.perf_counter()
     target = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_device(cfg, 0, "cuda"))
     head = dfl.DraftHead(ctx, dcfg, dfl.synth_draft_weights_device(dcfg, 0, "cuda"))
@@ -483,6 +483,7 @@ def main():
     ap.add_argument("--rocprof-summary", metavar="DIR", help="print a text summary of a rocprofv3 CSV output directory and exit")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end speculative decode measurement")
     ap.add_argument("--e2e-tokens", type=int, default=1024)
+    ap.add_argument("--e2e-prompt", type=int, default=2048, help="prompt length of the end-to-end section (the headline uses 2048)")
     ap.add_argument("--weight-sets", type=int, default=3,
                     help="copies of the three weight matrices the timed loops rotate over; 3 x 118 MB exceeds the 256 MB "
                          "memory-side cache, so weights come from HBM as they do in a real model (1 = cache-resident)")
@@ -672,7 +673,8 @@ def main():
             out["sections_error"] = f"{type(e).__name__}: {e}"
     if not args.no_e2e and not args.gemm_only:
         try:
-            e2e = e2e_speculative(ctx, args.e2e_tokens, [7, 3, 15], lambda m: print(m, file=sys.stderr, flush=True))
+            e2e = e2e_speculative(ctx, args.e2e_tokens, [7, 3, 15], lambda m: print(m, file=sys.stderr, flush=True),
+                                  prompt_len=args.e2e_prompt)
             out["e2e"] = e2e
             out["accepted_tokens_per_s"] = e2e["sweep"][0]["accepted_tokens_per_s"]
             out["config"]["e2e"] = ("35B-A3B-shaped MoE target (40 layers, 128 experts top-8, Q4_K experts, Q6_K attention, V 151936) "

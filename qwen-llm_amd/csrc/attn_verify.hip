@@ -515,8 +515,14 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     // its heads' queries and their partial outputs, and one CU takes in only 20-30 KB per microsecond: at short
     // contexts, where whole groups would leave most CUs without a workgroup, the group is divided until the chip
     // is covered (the chunk is then read by group / hw workgroups, of one XCD).
+    // (Measured on the 16 q / 2 kv head shape of 256, 40-layer verify: covering half the chip is enough - 4 heads per
+    // workgroup at 2 k of context, 2 at 1 k: 4.19 against 4.24 ms and 4.35 against 4.57 ms - but eight waves on one chunk
+    // are too many - at 4-8 k, 4 heads per workgroup: 4.75 against 4.81 ms, 4.20 against 4.28 ms.)
+    static const int env_cover_div = [] { const char *e = getenv("DFLASH_ATTN_COVER_DIV"); return e ? atoi(e) : 0; }();
+    const int cover_div = env_cover_div > 0 ? env_cover_div : 2;
     int hw = group;
-    while (hw % 2 == 0 && static_cast<int64_t>(n_kv) * (group / hw) * ((bucket + min_chunk - 1) / min_chunk) < ctx->n_cu) hw /= 2;
+    if (cover_div > 1 && group % 4 == 0 && group > 4 && bucket < 16384) hw = 4;
+    while (hw % 2 == 0 && static_cast<int64_t>(n_kv) * (group / hw) * ((bucket + min_chunk - 1) / min_chunk) < ctx->n_cu / cover_div) hw /= 2;
     // tuning knobs, read once per process
     static const int env_per_cu = [] { const char *e = getenv("DFLASH_ATTN_PER_CU"); return e ? atoi(e) : 0; }();
     static const int env_min_chunk = [] { const char *e = getenv("DFLASH_ATTN_MIN_CHUNK"); return e ? atoi(e) : 0; }();
