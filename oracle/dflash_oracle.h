@@ -34,13 +34,18 @@
  *       block, side/group indexing against an independent numpy gather)
  *   - DFlash-2 selector walk .......... the known-answer walks of metal_dflash/tests.rs:2978-3094
  *       (scores, first-tie rule, sentinel and non-finite candidates, invalid predecessor)
- *   - DFlash-2 drafter forward (orc_dflash_draft_ex): the reference has no CPU form of it.  Pinned
- *       by reduction to the DFlash-1 forward, bit for bit: identity convolutions (zero coefficient
- *       projections, identity base kernels) reproduce it; a per-channel power-of-two scaling on side 1
- *       equals the DFlash-1 forward with the matching rows of attn_output / ffn_down scaled (so side 1
- *       sits on the sublayer outputs, side 0 on their inputs).  Which coefficient tensor feeds which
- *       convolution (attention pair / FFN pair) follows metal_dflash.rs:16210-16262, 16836-16885 by
- *       reading only: for that part parity unpinned.
+ *   - DFlash-2 drafter forward (orc_dflash_draft_ex): the reference has no CPU form of it and its
+ *       model-witness tests need checkpoint files, so it is pinned by what the formula fixes.
+ *       Static part, by reduction to the DFlash-1 forward bit for bit: identity convolutions (zero
+ *       coefficient projections, identity base kernels) reproduce it; a per-channel power-of-two scaling
+ *       on side 1 equals the DFlash-1 forward with the matching rows of attn_output / ffn_down scaled (so
+ *       side 1 sits on the sublayer outputs, side 0 on their inputs).  Dynamic coefficients, always with
+ *       non-zero projections (metal_dflash.rs:16210-16262, 16795-16885, 17003-17022): an independent
+ *       float64 model of the whole layer; a projection that makes the coefficients a constant c equals
+ *       the static forward with base + c on both sides, for the attention pair and for the FFN pair
+ *       separately while the other pair keeps its own random projection (each pair reads ONE coefficient
+ *       vector, of its own projection); a norm doubled with the projection halved leaves every bit
+ *       unchanged (coefficients come from the normed, pre-convolution input).
  *   - f64 exp/ln are the host libm's, as the reference's are its platform's:
  *       last-ulp behaviour is parity unpinned (decisions compare against
  *       uniforms and are insensitive to it except with probability ~2^-50).
