@@ -170,6 +170,31 @@ int32_t dflash_gemm_fewrow_noalloc(int32_t w_type, const void *w, const void *x,
                                    int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream);
 const char *dflash_gemm_fewrow_noalloc_error(void);
 
+/* ---- few-row GEMM over activations in fragment order -----------------------------------------
+ * No counterpart in the reference (its kernels read row-major f32 activations, dispatch.rs:365-378).  The small
+ * projections of a layer (a few MB: the q/k/v, output and drafter matrices of a 2048-wide model) are bound by launch
+ * latency and by a split-K sum through memory, not by bytes.  Where the kernel that produces the 16 activation rows
+ * can write them as f16 in the order the MFMA operands are read ("XF": per 256 values of K, 512 slots of 16 bytes;
+ * slot (t, lane = 16 g + row) holds eight consecutive values of the row, the octet given by the consumer's type),
+ * one launch computes the whole product with every output tile's K inside one workgroup: no partial tiles, no
+ * second launch.  dflash_verify_block / dflash_draft_block use this hand-off between their own kernels; these three
+ * calls expose it.
+ *   dflash_xf_bytes: size of an XF buffer for n_in values per row (n_in % 256 == 0; 0 otherwise).
+ *   dflash_gemm_fewrow_xf_kind: the XF kind (DFLASH_XF_Q4K / DFLASH_XF_Q6K) this (type, shape) reads, or
+ *     DFLASH_XF_NONE where it is not taken: w_type must be DFLASH_TYPE_Q4_K_TILED or DFLASH_TYPE_Q6_K, n_in at most
+ *     8192, and the matrix at most one round of the chip (about 320 workgroups of 16 or 32 rows).
+ *   dflash_pack_xf: row-major x[n_rows][n_in] (f32 or f16) -> xf, rounding to f16 as every few-row kernel does.
+ *   dflash_gemm_fewrow_xf: Y[n_rows][n_out] = X . W^T; same guards as dflash_gemm_fewrow; DFLASH_ERR_UNSUPPORTED
+ *     where the kind is DFLASH_XF_NONE.  A (row, column) result depends on that activation row and weight row only.
+ * All enqueue-only. */
+enum { DFLASH_XF_NONE = 0, DFLASH_XF_Q4K = 1, DFLASH_XF_Q6K = 2 };
+size_t dflash_xf_bytes(int64_t n_in);
+int32_t dflash_gemm_fewrow_xf_kind(dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out);
+int32_t dflash_pack_xf(dflash_ctx *ctx, const void *x, int32_t x_type, int32_t n_rows, int64_t n_in, int32_t kind, void *xf,
+                       dflash_stream_t stream);
+int32_t dflash_gemm_fewrow_xf(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in,
+                              int64_t n_out, int32_t n_rows, dflash_stream_t stream);
+
 /* ---- block-causal verify attention ------------------------------------------------
  * The reference verifies a block with a per-row loop: encode_scatter_offset_f32_to_f16_kv +
  * encode_attn_decode_v4_f32 / encode_attn_decode_f16kv_f32, once per row

@@ -15,6 +15,7 @@ HEADER_PATH = os.path.join(PKG_DIR, "..", "include", "dflash_hip.h")
 
 TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q6_K = 0, 1, 8, 12, 14
 TYPE_Q4_K_TILED = 1012  # Q4_K blocks in the library's tiled order (Context.repack_q4k_tiled)
+XF_NONE, XF_Q4K, XF_Q6K = 0, 1, 2  # fragment orders of Context.pack_xf
 
 STATUS = {
     0: "Ok", 1: "BadShape", 2: "Unsupported", 3: "Alias", 4: "Alignment", 5: "Workspace", 6: "Hip",
@@ -126,6 +127,14 @@ def _declare(L):
     L.dflash_q4k_tiled_bytes.argtypes = [i64, i64]
     L.dflash_repack_q4k_tiled.restype = i32
     L.dflash_repack_q4k_tiled.argtypes = [vp, vp, vp, i64, i64, vp]
+    L.dflash_xf_bytes.restype = sz
+    L.dflash_xf_bytes.argtypes = [i64]
+    L.dflash_gemm_fewrow_xf_kind.restype = i32
+    L.dflash_gemm_fewrow_xf_kind.argtypes = [vp, i32, i64, i64]
+    L.dflash_pack_xf.restype = i32
+    L.dflash_pack_xf.argtypes = [vp, vp, i32, i32, i64, i32, vp, vp]
+    L.dflash_gemm_fewrow_xf.restype = i32
+    L.dflash_gemm_fewrow_xf.argtypes = [vp, i32, vp, vp, vp, i64, i64, i32, vp]
     L.dflash_gemm_fewrow_noalloc.restype = i32
     L.dflash_gemm_fewrow_noalloc.argtypes = [i32, vp, vp, i32, vp, i64, i64, i32, vp]
     L.dflash_gemm_fewrow_noalloc_error.restype = C.c_char_p
@@ -323,6 +332,31 @@ class Context:
         torch = _torch()
         y = _empty((x.shape[0], n_out), dtype=torch.float32, device=x.device)
         return self.encode_mat_mat_dispatch_dflash_verify(weight, w_type, x, y, n_in, n_out, x.shape[0])
+
+    # ---- the same product over activations handed over in MFMA fragment order (no counterpart in the reference)
+    def xf_kind(self, w_type: int, n_in: int, n_out: int) -> int:
+        """XF kind the whole-K kernel reads for this matrix (XF_Q4K / XF_Q6K), or XF_NONE where it does not take it."""
+        return int(self._lib.dflash_gemm_fewrow_xf_kind(self._h, int(w_type), n_in, n_out))
+
+    def pack_xf(self, x, kind: int):
+        """x [n_rows, n_in] f32 / f16 -> a uint8 tensor holding the rows as f16 in fragment order `kind`."""
+        torch = _torch()
+        n_rows, n_in = x.shape
+        nbytes = self._lib.dflash_xf_bytes(n_in)
+        if nbytes == 0:
+            raise DFlashError(1, f"n_in {n_in} is not a multiple of 256")
+        xf = _empty(nbytes, dtype=torch.uint8, device=x.device)
+        x_type = TYPE_F32 if x.dtype == torch.float32 else TYPE_F16
+        self._check(self._lib.dflash_pack_xf(self._h, x.data_ptr(), x_type, n_rows, n_in, int(kind), xf.data_ptr(), _stream_ptr()))
+        return xf
+
+    def gemm_fewrow_xf(self, weight, w_type: int, xf, n_rows: int, n_in: int, n_out: int, y=None):
+        torch = _torch()
+        if y is None:
+            y = _empty((n_rows, n_out), dtype=torch.float32, device=xf.device)
+        self._check(self._lib.dflash_gemm_fewrow_xf(self._h, int(w_type), weight.data_ptr(), xf.data_ptr(), y.data_ptr(), n_in,
+                                                     n_out, n_rows, _stream_ptr()))
+        return y
 
     # ---- per-row scatter + decode attention loop of packed verify (metal_dflash.rs:9963-10062)
     def attn_verify_block(self, q, k_cache, v_cache, ctx_len: int, scale: float, v_transposed: bool = False,

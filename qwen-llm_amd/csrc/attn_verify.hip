@@ -360,7 +360,7 @@ namespace {
 __global__ void __launch_bounds__(256)
     attn_combine_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml, float *__restrict__ out,
                         int n_rows, int n_q, int hd, int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int want,
-                        int min_chunk) {
+                        int min_chunk, void *__restrict__ out_xf, int out_xf_kind) {
     if (ctx_len_dev) ctx_len = *ctx_len_dev;
     const int64_t n_pos = ctx_len + n_rows;
     const int64_t chunk = attn_chunk(n_pos, want, min_chunk);
@@ -416,7 +416,15 @@ __global__ void __launch_bounds__(256)
         float o = 0.0f;
 #pragma unroll
         for (int k = 0; k < 8; k++) o += red[k][d];
-        out[(static_cast<int64_t>(row) * n_q + head) * hd + d] = o / lsum;
+        o /= lsum;
+        out[(static_cast<int64_t>(row) * n_q + head) * hd + d] = o;
+        if (out_xf) {
+            // eight consecutive dims sit in eight consecutive lanes of one wave (hd is a multiple of 64)
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = __shfl_down(o, i, 64);
+            if ((d & 7) == 0) dfl_xf_store(out_xf, out_xf_kind, row, head * hd + d, v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
+        }
     }
 }
 
@@ -476,8 +484,11 @@ extern "C" int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int3
 int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
-                       int64_t window, const int32_t *ctx_len_dev) {
+                       int64_t window, const int32_t *ctx_len_dev, void *out_xf, int out_xf_kind) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (out_xf && ((n_q * head_dim) % DFL_QK_K || reinterpret_cast<uintptr_t>(out_xf) % 16 ||
+                   (out_xf_kind != DFL_XF_Q4K && out_xf_kind != DFL_XF_Q6K)))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: fragment-order output needs n_q * head_dim %% 256 == 0 and a kind");
     if (!q || !k_cache || !v_cache || !out) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "attn_verify: null pointer");
     if (n_rows < 1 || n_rows > 16) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: n_rows %d outside 1..16", n_rows);
     if (n_q < 1 || n_kv < 1 || n_q % n_kv || n_q / n_kv > 16)
@@ -557,9 +568,6 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     }
     if (!part_o || !part_ml) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "attn_verify: workspace too small");
 
-#ifdef DFLASH_TRACE
-    if (const char *e = getenv("DFLASH_DBG_VT_STRIDE")) vt_stride = atoi(e);  // timing experiment only: wrong results
-#endif
     if (n_splits > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: %d KV splits", n_splits);
     const int split_stride = (n_splits + 7) / 8 * 8;
     const dim3 grid(split_stride * n_parts, n_kv);
@@ -588,7 +596,7 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     }
     if (rc) return rc;
     attn_combine_kernel<<<dim3(n_q, n_rows), 256, 0, st>>>(part_o, part_ml, out, n_rows, n_q, head_dim, ctx_len, ctx_len_dev, want,
-                                                          static_cast<int>(min_chunk));
+                                                          static_cast<int>(min_chunk), out_xf, out_xf_kind);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

@@ -110,6 +110,62 @@ static inline bool dfl_ranges_overlap(const void *a, size_t na, const void *b, s
 
 enum { DFL_QK_K = 256, DFL_Q4_K_BYTES = 144, DFL_Q6_K_BYTES = 210, DFL_Q8_0_BYTES = 34, DFL_QK8_0 = 32 };
 
+// ---- activations in MFMA fragment order ("XF") -----------------------------------------------------------------
+// The hand-off format between a kernel that produces the 16 activation rows of a few-row GEMM and the whole-K GEMM
+// kernels (gemm_whole.hip) that consume them: f16, already in the order the consumer's MFMA A operands are read in,
+// so that a wave loads a stage's eight fragments with eight coalesced 16-byte loads and no trip through LDS.
+// Per super-block b (256 values of K) 512 slots of 16 bytes: slot (t, lane) at byte ((b * 8 + t) * 64 + lane) * 16,
+// lane = 16 g + m (m = row), holds row m's eight consecutive values k = 256 b + 8 o + {0,2,1,3,4,6,5,7}[i] (the order
+// in which the nibble unpack emits a lane's weights), with octet o = 8 g + t for a Q4_K consumer and
+// o = 16 (g >> 1) + 8 (t >> 2) + 4 (g & 1) + (t & 3) for a Q6_K consumer (its quarters interleave).  Rows a producer
+// does not write keep whatever the buffer held: a row of the product depends on its own activation row only.
+enum { DFL_XF_NONE = 0, DFL_XF_Q4K = 1, DFL_XF_Q6K = 2 };
+static inline size_t dfl_xf_bytes(int64_t n_in) { return static_cast<size_t>(n_in / 256) * 8192; }
+#ifdef __HIPCC__
+// byte offset of the slot of row m's values k0 .. k0 + 7 (k0 a multiple of 8)
+__host__ __device__ static inline uint32_t dfl_xf_slot(int kind, int m, int k0) {
+    const int b = k0 >> 8, o = (k0 >> 3) & 31;
+    int g, t;
+    if (kind == DFL_XF_Q6K) {
+        const int h = o >> 4, quarter = (o >> 2) & 3;
+        g = 2 * h + (quarter & 1);
+        t = 4 * (quarter >> 1) + (o & 3);
+    } else {
+        g = o >> 3;
+        t = o & 7;
+    }
+    return static_cast<uint32_t>(((b * 8 + t) * 64 + 16 * g + m) * 16);
+}
+__device__ static inline void dfl_xf_store(void *xf, int kind, int m, int k0, float v0, float v1, float v2, float v3, float v4,
+                                           float v5, float v6, float v7) {
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    const h8 frag = {static_cast<_Float16>(v0), static_cast<_Float16>(v2), static_cast<_Float16>(v1), static_cast<_Float16>(v3),
+                     static_cast<_Float16>(v4), static_cast<_Float16>(v6), static_cast<_Float16>(v5), static_cast<_Float16>(v7)};
+    *reinterpret_cast<h8 *>(static_cast<uint8_t *>(xf) + dfl_xf_slot(kind, m, k0)) = frag;
+}
+// Lanes (2 p, 2 p + 1) of a wave hold values i .. i + 3 and i + 4 .. i + 7 of row m (i a multiple of 8 on the even lane):
+// the even lane stores the octet.  Every lane of the wave must call it.
+__device__ static inline void dfl_xf_store_pair(void *xf, int kind, int m, int i, float a, float b, float c, float d) {
+    const float e = __shfl_down(a, 1, 64), f = __shfl_down(b, 1, 64), g = __shfl_down(c, 1, 64), h = __shfl_down(d, 1, 64);
+    if ((threadIdx.x & 1) == 0) dfl_xf_store(xf, kind, m, i, a, b, c, d, e, f, g, h);
+}
+#endif
+
+// Whole-K few-row GEMM over activations in XF order (gemm_whole.hip): y[n_rows][n_out] = x . w^T with every output tile's
+// whole K inside one workgroup (its waves split K and add up in LDS in a fixed order): no partial tiles, no second launch.
+// dfl_whole_kind: the XF kind a producer must write for this matrix (DFL_XF_NONE: the shape or type does not take
+// this path: more than two stages per wave, or more tiles than one round of the chip).  pair_ffn > 0: w is a fused
+// gate | up matrix of 2 * pair_ffn rows and the output is silu(gate) * up, [n_rows][pair_ffn]: as f32 in y (may be null)
+// and / or as XF of kind y_xf_kind in y_xf (may be null), the activations of the down projection that follows.
+int dfl_whole_kind(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out, int64_t pair_ffn);
+int32_t dfl_gemm_whole(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in, int64_t n_out,
+                       int32_t n_rows, int64_t pair_ffn, void *y_xf, int y_xf_kind, hipStream_t stream);
+
+// dflash_dflash2_conv whose result also goes to y_xf in fragment order (XF; h a multiple of 256), for the whole-K
+// projection that reads it.
+int32_t dfl_dflash2_conv(dflash_ctx *ctx, const float *x, const float *dyn, const float *base, float *y, int32_t n_tokens, int32_t h,
+                         int32_t kernel_size, int32_t group_size, int32_t side, dflash_stream_t stream, void *y_xf, int y_xf_kind);
+
 // Device scratch of the mixture-of-experts FFN (owned by the target session).
 struct dfl_moe_scratch {
     float *probs = nullptr;   // [16][n_expert] router logits
@@ -128,6 +184,7 @@ struct dfl_moe_scratch {
 // already holds sigmoid(cur . shexp_gate) per row (the norm kernel that wrote cur computed it).
 // next_norm_w / next_cur / next_done (all or none): the RMSNorm that reads x_resid next may be done
 // in the same pass, next_cur = rms_norm(x_resid) * next_norm_w; *next_done says whether it was.
+// next_xf / next_xf_kind: where that norm is done here, its rows also go to next_xf in fragment order (XF).
 // pre_add / pre_norm_w (both or neither; only where dfl_moe_norm_fusable() holds): the layer's input has not been
 // normalised yet, x_resid still lacks pre_add (the attention's output projection), and `cur` is where the normalised rows
 // go: cur = rms_norm(x_resid + pre_add) * pre_norm_w, computed inside the router's launch with the shared-expert gate
@@ -135,7 +192,7 @@ struct dfl_moe_scratch {
 int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, float *cur, int n,
                     const dfl_moe_scratch &scratch, float *x_resid, bool gate_done, const float *next_norm_w,
                     float *next_cur, bool *next_done, hipStream_t stream, const float *pre_add = nullptr,
-                    const float *pre_norm_w = nullptr);
+                    const float *pre_norm_w = nullptr, void *next_xf = nullptr, int next_xf_kind = 0);
 bool dfl_moe_norm_fusable(const dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, int n);
 
 // Residual add + RMSNorm + shared-expert gate + Q8_0 router product of a mixture-of-experts layer as one launch:
@@ -156,7 +213,8 @@ int32_t dfl_router_norm(dflash_ctx *ctx, const void *router_w, const float *x, c
 // the heads into workgroups depends on dfl_attn_bucket(ctx_len + n_rows) only, and with ctx_len_dev
 // the launches are sized for the largest context of that bucket: a captured call stays valid, and
 // bit-identical to a direct one, at every context of the bucket it was captured in (a graph key
-// must therefore include the bucket).
+// must therefore include the bucket).  out_xf / out_xf_kind: the rows [n_rows][n_q * head_dim] also go to out_xf in
+// fragment order (XF), for the output projection that reads them.
 // Lower bound of the power-of-two range [b, 2 b) that holds n_pos visible positions (at least 256).
 inline int64_t dfl_attn_bucket(int64_t n_pos) {
     int64_t b = 256;
@@ -166,7 +224,7 @@ inline int64_t dfl_attn_bucket(int64_t n_pos) {
 int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
-                       int64_t window, const int32_t *ctx_len_dev);
+                       int64_t window, const int32_t *ctx_len_dev, void *out_xf = nullptr, int out_xf_kind = 0);
 
 // Few-row Q6_K GEMMs of up to three matrices over the same activations (a layer's q, k and v
 // projections) as one launch: y[m] = x . w[m]^T, [n_rows][n_out[m]] each.

@@ -19,7 +19,8 @@ namespace {
 // reference kernel does.  One thread per element.
 __global__ void __launch_bounds__(256)
     dflash2_conv_kernel(const float *__restrict__ x, const float *__restrict__ dyn, const float *__restrict__ base,
-                        float *__restrict__ y, int n_tokens, int h, int kernel_size, int group_size, int side) {
+                        float *__restrict__ y, int n_tokens, int h, int kernel_size, int group_size, int side,
+                        void *__restrict__ y_xf, int y_xf_kind) {
     const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (gid >= static_cast<int64_t>(n_tokens) * h) return;
     const int t = static_cast<int>(gid / h), c = static_cast<int>(gid % h);
@@ -33,6 +34,13 @@ __global__ void __launch_bounds__(256)
         acc = __builtin_fmaf(b + d, x[static_cast<size_t>(t - tap) * h + c], acc);
     }
     y[gid] = acc;
+    if (y_xf) {
+        // (h a multiple of 256: the grid has no ragged end and eight consecutive lanes hold eight consecutive channels of a row)
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = __shfl_down(acc, i, 64);
+        if ((c & 7) == 0) dfl_xf_store(y_xf, y_xf_kind, t, c, v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
+    }
 }
 
 struct Codebook {
@@ -222,7 +230,14 @@ int32_t check_codebook(dflash_ctx *ctx, const dflash_codebook *cb, int rank, Cod
 extern "C" int32_t dflash_dflash2_conv(dflash_ctx *ctx, const float *x, const float *dyn, const float *base, float *y,
                                        int32_t n_tokens, int32_t h, int32_t kernel_size, int32_t group_size, int32_t side,
                                        dflash_stream_t stream) {
+    return dfl_dflash2_conv(ctx, x, dyn, base, y, n_tokens, h, kernel_size, group_size, side, stream, nullptr, DFL_XF_NONE);
+}
+
+int32_t dfl_dflash2_conv(dflash_ctx *ctx, const float *x, const float *dyn, const float *base, float *y, int32_t n_tokens, int32_t h,
+                         int32_t kernel_size, int32_t group_size, int32_t side, dflash_stream_t stream, void *y_xf, int y_xf_kind) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (y_xf && (h % DFL_QK_K || n_tokens > 16 || (y_xf_kind != DFL_XF_Q4K && y_xf_kind != DFL_XF_Q6K)))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "dflash2_conv: fragment-order output needs h %% 256 == 0, at most 16 rows and a kind");
     if (!x || !dyn || !base || !y) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "dflash2_conv: null pointer");
     if (n_tokens < 1 || h < 1 || kernel_size < 1 || group_size < 1 || h % group_size || (side != 0 && side != 1))
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "dflash2_conv: n_tokens %d h %d kernel %d group %d side %d", n_tokens, h,
@@ -232,7 +247,7 @@ extern "C" int32_t dflash_dflash2_conv(dflash_ctx *ctx, const float *x, const fl
         return dfl_fail(ctx, DFLASH_ERR_ALIAS, "dflash2_conv: y aliases x (taps read neighbouring rows)");
     const int64_t total = static_cast<int64_t>(n_tokens) * h;
     dflash2_conv_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
-        x, dyn, base, y, n_tokens, h, kernel_size, group_size, side);
+        x, dyn, base, y, n_tokens, h, kernel_size, group_size, side, y_xf, y_xf_kind);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

@@ -1,0 +1,389 @@
+// Whole-K few-row GEMM for the small matrices of a verify or draft layer (a few MB each):
+//   Y[n_rows][n_out] = X[n_rows][n_in] . W^T,  X handed over in MFMA fragment order (common.h, "XF").
+// Same contraction as encode_mat_mat_dispatch_dflash_verify (metal_forward/dispatch.rs:365-378, kernel
+// kernels/mat_mat_fewrow_gen.metal:374-474); used inside the layer loops where the kernel that produces X can
+// write it in fragment order.
+//
+// Why a second kernel family.  The streaming kernels (gemm_fewrow.hip) give every CU a contiguous run of
+// (tile group x super-block) stages; where a run cuts a tile group the K sum is split over workgroups and a second
+// launch adds the partial tiles.  For a 50 MB matrix that is the right shape.  For the 6-9 MB projections of a
+// 2048-wide model it is two dependent launches of 7-10 us + 4 us in which every wave sees one or two stages: the
+// time is launch latency, the trip for the first bytes, and a reduction through memory.  Here every (tile, stage)
+// of the matrix is one wave-slot of ONE round of the chip:
+//   * a workgroup owns `tl` output units over the whole K; wave = (tile lane, K slice), a slice is one or two
+//     super-blocks; every load of a wave (weights straight into registers, the stage's eight activation fragments
+//     with eight coalesced 16-byte loads from the XF buffer, which sits in L2) is issued before anything is waited for;
+//   * the slices' partial tiles are added in LDS in slice order (deterministic), by the wave of slice 0, which writes Y.
+// No partial tiles in memory, no second launch, no loop.  A (row, column) result depends on nothing but its own
+// activation row and weight row, so a 16-row block and a single row give the same bits.
+//
+// Arithmetic: that of the streaming kernels (exact f16 integers from the quant bits, one packed fma with
+// s = d * scale, f32 accumulation on v_mfma_f32_16x16x32_f16; the Q4_K minima and the Q6_K offset through a twin MFMA
+// of the same activation fragment into a second accumulator that is subtracted at the end).
+#include "common.h"
+#include "mfma_unpack.h"
+
+#include <cstdlib>
+
+namespace {
+
+struct WholeArgs {
+    const uint8_t *w;
+    const uint8_t *xf;
+    float *y;
+    uint8_t *y_xf;
+    int y_xf_kind;
+    int n_out;   // rows of w (pair mode: 2 * ffn)
+    int nb;      // super-blocks per row
+    int n_rows;
+    int ksplit;  // K slices per unit; waves per workgroup = ksplit * tl
+    int tl;      // units per workgroup
+    int n_units; // plain: ceil(tiles / R) units of R consecutive tiles; pair: ffn / 16 units of (gate tile, up tile)
+    int pair_off;  // pair mode: tiles between a gate tile and its up tile; 0 = plain
+    uint32_t row_bytes;  // Q6_K (GGUF row order): bytes per weight row
+};
+
+// ---- Q4_K, tiled order: [tile group of 256 rows][super-block][tile][row][144-byte block] ----
+struct Q4W {
+    u32x4_t hdr, q0, q1;
+};
+__device__ __forceinline__ void load_w(Q4W &r, const WholeArgs &a, int tile, int b, int n, int g) {
+    const uint8_t *p = a.w + ((static_cast<size_t>(tile >> 4) * a.nb + b) * 16 + (tile & 15)) * (16 * DFL_Q4_K_BYTES) +
+                       n * DFL_Q4_K_BYTES;
+    r.hdr = *reinterpret_cast<const u32x4_t *>(p);
+    r.q0 = *reinterpret_cast<const u32x4_t *>(p + 16 + 32 * g);
+    r.q1 = *reinterpret_cast<const u32x4_t *>(p + 32 + 32 * g);
+}
+// One super-block of one tile: lane (n = weight row, g = 64-value chunk) against the eight activation fragments.
+__device__ __forceinline__ void compute(const Q4W &r, const half8_t (&af)[8], int g, uint32_t sc_sel, Q4KMagic magic,
+                                        float4_t &acc, float4_t &acc_sub) {
+    const u32x4_t hdr = r.hdr;
+    const uint32_t upper = 0u - static_cast<uint32_t>(g >> 1);
+    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu, mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t sc_word = (sc_hi & upper) | (sc_lo & ~upper), mn_word = (mn_hi & upper) | (mn_lo & ~upper);
+    const half2_t dm = __builtin_bit_cast(half2_t, hdr.x);
+    const half2_t p_sc = as_half2(__builtin_amdgcn_perm(0x64646464u, sc_word, sc_sel));
+    const half2_t p_mn = as_half2(__builtin_amdgcn_perm(0x64646464u, mn_word, sc_sel));
+    const half2_t neg = dm * splat(static_cast<_Float16>(-1024.0f));
+    const half2_t S = __builtin_elementwise_fma(p_sc, splat(dm[0]), splat(neg[0]));
+    const half2_t M = __builtin_elementwise_fma(p_mn, splat(dm[1]), splat(neg[1]));
+    const half2_t unbias = {static_cast<_Float16>(-1024.0f), static_cast<_Float16>(-64.0f)};
+    const half2_t Cs = S * unbias;
+    const half2_t s2l = splat(S[0]), c2l = splat(Cs[0]);
+    const half2_t s2h = splat(S[1]), c2h = splat(Cs[1]);
+    const _Float16 m_lo = M[0], m_hi = M[1];
+    const half8_t bml = {m_lo, m_lo, m_lo, m_lo, m_lo, m_lo, m_lo, m_lo};
+    const half8_t bmh = {m_hi, m_hi, m_hi, m_hi, m_hi, m_hi, m_hi, m_hi};
+    const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bl = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
+        acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bml, acc_sub, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const half8_t bh = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bh, acc, 0, 0, 0);
+        acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bmh, acc_sub, 0, 0, 0);
+    }
+}
+
+// ---- Q6_K, GGUF row order: 210-byte blocks (ql[128], qh[64], scales[16], d), rows 2-byte aligned ----
+typedef u32x4_t u32x4_unaligned_t __attribute__((aligned(2)));
+typedef uint32_t u32_unaligned_t __attribute__((aligned(2)));
+struct Q6W {
+    u32x4_t qa, qb, ha, hb;
+    uint32_t sc_l, sc_h, d;
+};
+__device__ __forceinline__ void load_w(Q6W &r, const WholeArgs &a, int tile, int b, int n, int g) {
+    const int row = min(tile * 16 + n, a.n_out - 1);  // rows past the matrix re-read its last row; never stored
+    const uint8_t *p = a.w + static_cast<size_t>(row) * a.row_bytes + static_cast<size_t>(b) * DFL_Q6_K_BYTES;
+    const int h = g >> 1, odd = g & 1;
+    // unaligned vector loads (gfx950 runs with unaligned access enabled)
+    r.qa = *reinterpret_cast<const u32x4_unaligned_t *>(p + 64 * h + 32 * odd);
+    r.qb = *reinterpret_cast<const u32x4_unaligned_t *>(p + 64 * h + 32 * odd + 16);
+    r.ha = *reinterpret_cast<const u32x4_unaligned_t *>(p + 128 + 32 * h);
+    r.hb = *reinterpret_cast<const u32x4_unaligned_t *>(p + 128 + 32 * h + 16);
+    r.sc_l = *reinterpret_cast<const u32_unaligned_t *>(p + 192 + 8 * h);
+    r.sc_h = *reinterpret_cast<const u32_unaligned_t *>(p + 192 + 8 * h + 4);
+    r.d = *reinterpret_cast<const uint16_t *>(p + 208);
+}
+__device__ __forceinline__ void compute(const Q6W &r, const half8_t (&af)[8], int g, uint32_t, Q4KMagic magic, float4_t &acc,
+                                        float4_t &acc_sub) {
+    const int odd = g & 1;
+    const uint32_t sc4 = (r.sc_l >> (16 * odd)) & 0xffffu, sc4h = (r.sc_h >> (16 * odd)) & 0xffffu;
+    const float d = __half2float(__ushort_as_half(static_cast<unsigned short>(r.d)));
+    const int hs = 2 * odd;
+    const uint32_t hq[8] = {r.ha.x >> hs, r.ha.y >> hs, r.ha.z >> hs, r.ha.w >> hs, r.hb.x >> hs, r.hb.y >> hs, r.hb.z >> hs, r.hb.w >> hs};
+    const uint32_t ql[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+    auto scale = [&](uint32_t pair, int j) { return static_cast<_Float16>(d * static_cast<float>(static_cast<int8_t>(pair >> (8 * j)))); };
+    const _Float16 s_l0 = scale(sc4, 0), s_l1 = scale(sc4, 1), s_h0 = scale(sc4h, 0), s_h1 = scale(sc4h, 1);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const _Float16 sl = (t >> 1) ? s_l1 : s_l0;
+        const half8_t bl = unpack6<false>(ql[2 * t], ql[2 * t + 1], hq[2 * t], hq[2 * t + 1], splat(sl),
+                                          splat(sl * static_cast<_Float16>(-1024.0f)), magic.lo);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
+        const _Float16 o = sl * static_cast<_Float16>(32.0f);
+        const half8_t bo = {o, o, o, o, o, o, o, o};
+        acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bo, acc_sub, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const _Float16 sh = (t >> 1) ? s_h1 : s_h0;
+        const half8_t bh = unpack6<true>(ql[2 * t], ql[2 * t + 1], hq[2 * t] >> 4, hq[2 * t + 1] >> 4, splat(sh),
+                                         splat(sh * static_cast<_Float16>(-64.0f)), magic.hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bh, acc, 0, 0, 0);
+        const _Float16 o = sh * static_cast<_Float16>(32.0f);
+        const half8_t bo = {o, o, o, o, o, o, o, o};
+        acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bo, acc_sub, 0, 0, 0);
+    }
+}
+
+__device__ __forceinline__ void load_xf(half8_t (&af)[8], const uint8_t *xf, int b, int lane) {
+    const half8_t *p = reinterpret_cast<const half8_t *>(xf) + static_cast<size_t>(b) * 512 + lane;
+#pragma unroll
+    for (int t = 0; t < 8; t++) af[t] = p[t * 64];
+}
+
+// W: Q4W or Q6W.  R: tiles per wave and stage (they share the stage's activation fragments).
+template <typename W, int R>
+__global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
+    __shared__ float4_t red[16 * R * 64];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tlane = wave / a.ksplit, kslice = wave - tlane * a.ksplit;
+    const int unit = blockIdx.x * a.tl + tlane;
+    const bool active = unit < a.n_units;
+    const int n = lane & 15, g = lane >> 4;
+    const int b0 = a.nb * kslice / a.ksplit, b1 = a.nb * (kslice + 1) / a.ksplit;  // one or two stages (host)
+    const bool two = b1 - b0 > 1;
+    const int n_tiles = (a.n_out + 15) >> 4;
+    int tile[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) tile[r] = min(a.pair_off ? unit + r * a.pair_off : unit * R + r, n_tiles - 1);
+    float4_t acc[R], acc_sub[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = acc_sub[r] = float4_t{0, 0, 0, 0};
+    if (active) {
+        const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
+        const Q4KMagic magic = q4k_magic();
+        W w0[R], w1[R];
+        half8_t af[8];
+        // the weights come from HBM, the activations from L2: weights first
+#pragma unroll
+        for (int r = 0; r < R; r++) load_w(w0[r], a, tile[r], b0, n, g);
+        // (both stages' weights in flight together where the registers hold them)
+        constexpr bool kEarly = sizeof(W) * R <= 96;
+        if (kEarly && two) {
+#pragma unroll
+            for (int r = 0; r < R; r++) load_w(w1[r], a, tile[r], b0 + 1, n, g);
+        }
+        load_xf(af, a.xf, b0, lane);
+#pragma unroll
+        for (int r = 0; r < R; r++) compute(w0[r], af, g, sc_sel, magic, acc[r], acc_sub[r]);
+        if (two) {
+            if (!kEarly) {
+#pragma unroll
+                for (int r = 0; r < R; r++) load_w(w1[r], a, tile[r], b0 + 1, n, g);
+            }
+            load_xf(af, a.xf, b0 + 1, lane);
+#pragma unroll
+            for (int r = 0; r < R; r++) compute(w1[r], af, g, sc_sel, magic, acc[r], acc_sub[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) red[(wave * R + r) * 64 + lane] = acc[r] - acc_sub[r];
+    __syncthreads();
+    if (kslice != 0 || !active) return;
+    float4_t sum[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        sum[r] = red[(wave * R + r) * 64 + lane];
+        for (int s = 1; s < a.ksplit; s++) sum[r] += red[((wave + s) * R + r) * 64 + lane];
+    }
+    if (!a.pair_off) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int col = (unit * R + r) * 16 + n;
+            if (col < a.n_out) {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (4 * g + i < a.n_rows) a.y[static_cast<size_t>(4 * g + i) * a.n_out + col] = sum[r][i];
+            }
+        }
+        return;
+    }
+    if constexpr (R == 2) {
+        // SwiGLU of the (gate tile, up tile) pair: out[m][16 unit + n] = silu(gate) * up
+        const int ffn = a.n_out >> 1;
+        float4_t out;
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = sum[0][i] / (1.0f + expf(-sum[0][i])) * sum[1][i];
+        const int col = unit * 16 + n;
+        if (a.y && col < ffn) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (4 * g + i < a.n_rows) a.y[static_cast<size_t>(4 * g + i) * ffn + col] = out[i];
+        }
+        if (a.y_xf) {
+            // the tile through this wave's own LDS slot: lane (m, octet) then holds eight consecutive columns of a row
+            float *f = reinterpret_cast<float *>(&red[wave * R * 64]);
+            red[wave * R * 64 + lane] = out;
+            __builtin_amdgcn_wave_barrier();
+            if (lane < 32) {
+                const int m = lane >> 1, oct = lane & 1;
+                float v[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = f[((8 * oct + i) + 16 * (m >> 2)) * 4 + (m & 3)];
+                dfl_xf_store(a.y_xf, a.y_xf_kind, m, unit * 16 + 8 * oct, v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
+            }
+        }
+    }
+}
+
+// Row-major activations -> XF: one thread per (row, eight consecutive values).
+template <typename XT>
+__global__ void __launch_bounds__(256) pack_xf_kernel(const XT *__restrict__ x, int n_rows, int n_in, int kind, uint8_t *__restrict__ xf) {
+    const int oct = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+    if (8 * oct >= n_in || m >= n_rows) return;
+    const XT *p = x + static_cast<size_t>(m) * n_in + 8 * oct;
+    dfl_xf_store(xf, kind, m, 8 * oct, static_cast<float>(p[0]), static_cast<float>(p[1]), static_cast<float>(p[2]), static_cast<float>(p[3]),
+                 static_cast<float>(p[4]), static_cast<float>(p[5]), static_cast<float>(p[6]), static_cast<float>(p[7]));
+}
+
+struct EnvInt {
+    const char *name;
+    bool set;
+    int value;
+    explicit EnvInt(const char *n) : name(n), set(false), value(0) {
+        if (const char *e = getenv(n)) {
+            set = true;
+            value = atoi(e);
+        }
+    }
+    int get(int fallback) const { return set ? value : fallback; }
+};
+#define env_int(name, fallback) ([]() -> const EnvInt & { static const EnvInt e(name); return e; }().get(fallback))
+
+struct WholePlan {
+    int kind, ksplit, tl, R, n_units, n_wg;
+};
+
+// The split of a matrix over waves, or kind == DFL_XF_NONE where this path does not take it.
+WholePlan whole_plan(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out, int64_t pair_ffn) {
+    WholePlan p = {DFL_XF_NONE, 0, 0, 0, 0, 0};
+    if (!env_int("DFLASH_GEMM_WHOLE", 1)) return p;
+    const int kind = w_type == DFLASH_TYPE_Q4_K_TILED ? DFL_XF_Q4K : w_type == DFLASH_TYPE_Q6_K ? DFL_XF_Q6K : DFL_XF_NONE;
+    if (kind == DFL_XF_NONE || n_in <= 0 || n_in % DFL_QK_K || n_out <= 0 || n_out >= (1 << 24)) return p;
+    const int nb = static_cast<int>(n_in / DFL_QK_K);
+    if (nb > 32) return p;  // more than two stages per wave
+    if (pair_ffn && (n_out != 2 * pair_ffn || pair_ffn % 16)) return p;
+    const int ksplit = nb < 16 ? nb : 16, tl = 16 / ksplit;
+    const int tiles = static_cast<int>((n_out + 15) / 16);
+    int R = pair_ffn ? 2 : 1;
+    int n_units = pair_ffn ? static_cast<int>(pair_ffn / 16) : tiles;
+    // one round of the chip: at most one workgroup per CU (a wave's registers leave room for one), a quarter more tolerated
+    const int max_wg = ctx->n_cu + ctx->n_cu / 4;
+    if (!pair_ffn && (n_units + tl - 1) / tl > max_wg) {
+        R = 2;
+        n_units = (tiles + 1) / 2;
+    }
+    const int n_wg = (n_units + tl - 1) / tl;
+    if (n_wg > max_wg) return p;
+    p = {kind, ksplit, tl, R, n_units, n_wg};
+    return p;
+}
+
+}  // namespace
+
+int dfl_whole_kind(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out, int64_t pair_ffn) {
+    return whole_plan(ctx, w_type, n_in, n_out, pair_ffn).kind;
+}
+
+int32_t dfl_gemm_whole(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in, int64_t n_out,
+                       int32_t n_rows, int64_t pair_ffn, void *y_xf, int y_xf_kind, hipStream_t st) {
+    const WholePlan p = whole_plan(ctx, w_type, n_in, n_out, pair_ffn);
+    if (p.kind == DFL_XF_NONE) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: type %d, %lld -> %lld not taken", w_type,
+                                               static_cast<long long>(n_in), static_cast<long long>(n_out));
+    if (!w || !xf || n_rows < 1 || n_rows > 16 || (!y && !(pair_ffn && y_xf)))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_whole: null operand or n_rows %d", n_rows);
+    if (reinterpret_cast<uintptr_t>(xf) % 16 || reinterpret_cast<uintptr_t>(w) % (p.kind == DFL_XF_Q4K ? 16 : 2) ||
+        (y_xf && reinterpret_cast<uintptr_t>(y_xf) % 16))
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_whole: operand alignment");
+    if (y_xf && (!pair_ffn || (y_xf_kind != DFL_XF_Q4K && y_xf_kind != DFL_XF_Q6K)))
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: fragment-order output needs the SwiGLU pair mode and a kind");
+    WholeArgs a;
+    a.w = static_cast<const uint8_t *>(w);
+    a.xf = static_cast<const uint8_t *>(xf);
+    a.y = y;
+    a.y_xf = static_cast<uint8_t *>(y_xf);
+    a.y_xf_kind = y_xf_kind;
+    a.n_out = static_cast<int>(n_out);
+    a.nb = static_cast<int>(n_in / DFL_QK_K);
+    a.n_rows = n_rows;
+    a.ksplit = p.ksplit;
+    a.tl = p.tl;
+    a.n_units = p.n_units;
+    a.pair_off = pair_ffn ? static_cast<int>(pair_ffn / 16) : 0;
+    a.row_bytes = static_cast<uint32_t>(a.nb) * DFL_Q6_K_BYTES;
+    const int threads = 64 * p.ksplit * p.tl;
+    dfl_timed timer(ctx, st, DFL_T_GEMM);
+    if (p.kind == DFL_XF_Q4K) {
+        if (p.R == 2)
+            gemm_whole_kernel<Q4W, 2><<<p.n_wg, threads, 0, st>>>(a);
+        else
+            gemm_whole_kernel<Q4W, 1><<<p.n_wg, threads, 0, st>>>(a);
+    } else {
+        if (p.R == 2)
+            gemm_whole_kernel<Q6W, 2><<<p.n_wg, threads, 0, st>>>(a);
+        else
+            gemm_whole_kernel<Q6W, 1><<<p.n_wg, threads, 0, st>>>(a);
+    }
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+extern "C" size_t dflash_xf_bytes(int64_t n_in) { return n_in > 0 && n_in % DFL_QK_K == 0 ? dfl_xf_bytes(n_in) : 0; }
+
+extern "C" int32_t dflash_gemm_fewrow_xf_kind(dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out) {
+    return ctx ? dfl_whole_kind(ctx, w_type, n_in, n_out, 0) : DFL_XF_NONE;
+}
+
+extern "C" int32_t dflash_pack_xf(dflash_ctx *ctx, const void *x, int32_t x_type, int32_t n_rows, int64_t n_in, int32_t kind,
+                                  void *xf, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!x || !xf || n_rows < 1 || n_rows > 16 || n_in <= 0 || n_in % DFL_QK_K || n_in > (1 << 24))
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "pack_xf: n_rows %d, n_in %lld", n_rows, static_cast<long long>(n_in));
+    if (kind != DFL_XF_Q4K && kind != DFL_XF_Q6K) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "pack_xf: kind %d", kind);
+    if (x_type != DFLASH_TYPE_F32 && x_type != DFLASH_TYPE_F16) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "pack_xf: x_type %d", x_type);
+    if (reinterpret_cast<uintptr_t>(xf) % 16) return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "pack_xf: xf must be 16-byte aligned");
+    const size_t x_bytes = static_cast<size_t>(n_rows) * n_in * (x_type == DFLASH_TYPE_F32 ? 4 : 2);
+    if (dfl_ranges_overlap(x, x_bytes, xf, dfl_xf_bytes(n_in))) return dfl_fail(ctx, DFLASH_ERR_ALIAS, "pack_xf: xf overlaps x");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid(static_cast<unsigned>((n_in / 8 + 255) / 256), n_rows);
+    if (x_type == DFLASH_TYPE_F32)
+        pack_xf_kernel<float><<<grid, 256, 0, st>>>(static_cast<const float *>(x), n_rows, static_cast<int>(n_in), kind, static_cast<uint8_t *>(xf));
+    else
+        pack_xf_kernel<_Float16><<<grid, 256, 0, st>>>(static_cast<const _Float16 *>(x), n_rows, static_cast<int>(n_in), kind,
+                                                     static_cast<uint8_t *>(xf));
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+extern "C" int32_t dflash_gemm_fewrow_xf(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in,
+                                         int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (dfl_whole_kind(ctx, w_type, n_in, n_out, 0) == DFL_XF_NONE)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow_xf: type %d, %lld -> %lld is not taken by the whole-K kernels", w_type,
+                        static_cast<long long>(n_in), static_cast<long long>(n_out));
+    if (n_in > 0 && n_out > 0 && y && xf && w) {
+        const size_t wb = w_type == DFLASH_TYPE_Q4_K_TILED ? dflash_q4k_tiled_bytes(n_in, n_out) : dflash_row_bytes(w_type, n_in) * n_out;
+        const size_t yb = static_cast<size_t>(n_rows > 0 ? n_rows : 1) * n_out * sizeof(float);
+        if (dfl_ranges_overlap(y, yb, xf, dfl_xf_bytes(n_in)) || dfl_ranges_overlap(y, yb, w, wb))
+            return dfl_fail(ctx, DFLASH_ERR_ALIAS, "gemm_fewrow_xf: y aliases an input");
+    }
+    return dfl_gemm_whole(ctx, w_type, w, xf, y, n_in, n_out, n_rows, 0, nullptr, DFL_XF_NONE, static_cast<hipStream_t>(stream));
+}

@@ -45,11 +45,13 @@ __device__ float block_sum(float v, float *sh) {
 // y = x * rsqrt(mean(x^2) + eps) * w.  One row per workgroup; a row of up to 4096 values (n a
 // multiple of 4) is read once and stays in registers between the two passes.  With gate_w, the row's
 // sigmoid(y . gate_w) also goes to gate_out[row] (the shared-expert gate of a mixture-of-experts
-// layer, forward.rs:749-824: the normalised row is at hand here, in registers).
+// layer, forward.rs:749-824: the normalised row is at hand here, in registers).  With y_xf (n a multiple of 256, at most
+// 4096), y also goes there as f16 in the fragment order a whole-K GEMM reads (common.h, "XF").
 __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, const float *__restrict__ add,
                                                        const float *__restrict__ w, float *__restrict__ y, int n,
                                                        float eps, const float *__restrict__ gate_w,
-                                                       float *__restrict__ gate_out) {
+                                                       float *__restrict__ gate_out, void *__restrict__ y_xf = nullptr,
+                                                       int y_xf_kind = 0) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
     float *xr = x + static_cast<size_t>(blockIdx.x) * n;
@@ -81,6 +83,8 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
             if (i < n) {
                 const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
                 *reinterpret_cast<f4 *>(yr + i) = o;
+                // (the host passes y_xf only for n a multiple of 256: whole waves are inside or outside the row)
+                if (y_xf) dfl_xf_store_pair(y_xf, y_xf_kind, blockIdx.x, i & ~7, o[0], o[1], o[2], o[3]);
                 if (gate_w) {
                     const f4 gw = *reinterpret_cast<const f4 *>(gate_w + i);
                     dot += (o[0] * gw[0] + o[1] * gw[1]) + (o[2] * gw[2] + o[3] * gw[3]);
@@ -367,12 +371,35 @@ bool adjacent(const dflash_qtensor &a, int64_t rows_a, const dflash_qtensor &b, 
            static_cast<const uint8_t *>(b.data) == static_cast<const uint8_t *>(a.data) + static_cast<size_t>(rows_a) * rb;
 }
 
+// Which of a layer's projections take the whole-K kernel over activations in fragment order (gemm_whole.hip), and the
+// XF kind each of them reads; DFL_XF_NONE: the projection stays with the streaming kernels and row-major activations.
+// The kernel that PRODUCES a projection's input rows is told to write them in that order as well.
+struct LayerXf {
+    int qkv = DFL_XF_NONE, wo = DFL_XF_NONE, gate_up = DFL_XF_NONE, down = DFL_XF_NONE;
+};
+template <typename LayerT>
+LayerXf layer_xf(const dflash_ctx *ctx, const LayerT &L, bool packed_qkv_allowed, int64_t H, int64_t q_dim, int64_t kv_dim,
+                 int64_t ffn, bool dense_ffn) {
+    LayerXf k;
+    if (packed_qkv_allowed && adjacent(L.wq, q_dim, L.wk, H) && adjacent(L.wk, kv_dim, L.wv, H))
+        k.qkv = dfl_whole_kind(ctx, L.wq.type, H, q_dim + 2 * kv_dim, 0);
+    k.wo = dfl_whole_kind(ctx, L.wo.type, q_dim, H, 0);
+    if (dense_ffn && ffn > 0) {
+        if (adjacent(L.gate, ffn, L.up, H)) k.gate_up = dfl_whole_kind(ctx, L.gate.type, H, 2 * ffn, ffn);
+        k.down = dfl_whole_kind(ctx, L.down.type, ffn, H, 0);
+    }
+    return k;
+}
+
 // The q, k and v projections of a layer.  Returns in *packed whether they went out as one GEMM into
-// pk[n][q_dim + 2 kv_dim] (adjacent weights) or as separate ones into q, k, v.
+// pk[n][q_dim + 2 kv_dim] (adjacent weights) or as separate ones into q, k, v.  xf_kind != DFL_XF_NONE (from
+// layer_xf: implies adjacent weights): the rows are in x_xf in fragment order and the whole-K kernel takes them.
 int32_t gemm_qkv(dflash_ctx *ctx, const dflash_qtensor &wq, const dflash_qtensor &wk, const dflash_qtensor &wv, const float *x,
                  float *q, float *k, float *v, float *pk, bool allow_packed, bool *packed, int64_t n_in, int64_t q_dim,
-                 int64_t kv_dim, int n, hipStream_t st) {
+                 int64_t kv_dim, int n, hipStream_t st, const void *x_xf = nullptr, int xf_kind = DFL_XF_NONE) {
     *packed = allow_packed && pk && adjacent(wq, q_dim, wk, n_in) && adjacent(wk, kv_dim, wv, n_in);
+    if (*packed && xf_kind != DFL_XF_NONE && x_xf)
+        return dfl_gemm_whole(ctx, wq.type, wq.data, x_xf, pk, n_in, q_dim + 2 * kv_dim, n, 0, nullptr, DFL_XF_NONE, st);
     if (*packed) return gemm(ctx, wq, x, pk, n_in, q_dim + 2 * kv_dim, n, st);
     if (wq.type == DFLASH_TYPE_Q6_K && wk.type == DFLASH_TYPE_Q6_K && wv.type == DFLASH_TYPE_Q6_K && n_in % DFL_QK_K == 0) {
         const void *w[3] = {wq.data, wk.data, wv.data};
@@ -386,10 +413,16 @@ int32_t gemm_qkv(dflash_ctx *ctx, const dflash_qtensor &wq, const dflash_qtensor
     return gemm(ctx, wv, x, v, n_in, kv_dim, n, st);
 }
 
-// Dense SwiGLU input: g = silu(x Wg^T) * (x Wu^T), one GEMM when gate and up are adjacent.
+// Dense SwiGLU input: g = silu(x Wg^T) * (x Wu^T), one GEMM when gate and up are adjacent.  xf_kind != DFL_XF_NONE
+// (from layer_xf): the rows are in x_xf in fragment order and the whole-K kernel computes the pair with the
+// activation in its epilogue; g_xf / g_xf_kind: the result also goes there in the order the down projection reads.
 int32_t gemm_gate_up(dflash_ctx *ctx, const dflash_qtensor &gate, const dflash_qtensor &up, const float *x, float *g, float *u,
-                     float *pk, int64_t n_in, int64_t ffn, int n, hipStream_t st) {
+                     float *pk, int64_t n_in, int64_t ffn, int n, hipStream_t st, const void *x_xf = nullptr,
+                     int xf_kind = DFL_XF_NONE, void *g_xf = nullptr, int g_xf_kind = DFL_XF_NONE) {
     int32_t rc;
+    if (xf_kind != DFL_XF_NONE && x_xf)
+        return dfl_gemm_whole(ctx, gate.type, gate.data, x_xf, g, n_in, 2 * ffn, n, ffn, g_xf_kind != DFL_XF_NONE ? g_xf : nullptr,
+                              g_xf_kind, st);
     if (pk && adjacent(gate, ffn, up, n_in)) {
         // (a product split over K applies the activation in its reduction: one launch less)
         ctx->swiglu_out = ffn % 16 == 0 ? g : nullptr;
@@ -428,6 +461,8 @@ struct dflash_session {
     float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
     float *g = nullptr, *u = nullptr, *logits = nullptr, *gap = nullptr;
     float *pk = nullptr;  // [16][max(q_dim + 2 kv_dim, 2 ffn)]: output of a fused q/k/v or gate/up GEMM
+    // cur and attn once more, as f16 in MFMA fragment order, for the projections that take the whole-K kernel
+    uint8_t *xf_cur = nullptr, *xf_attn = nullptr, *xf_g = nullptr;
     float *hidden = nullptr;  // [16][n_taps][hidden] capture slots of the speculative step
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
     dfl_moe_scratch moe;
@@ -485,6 +520,8 @@ struct dflash_draft_session {
     float *x = nullptr, *cur = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *mix = nullptr;
     float *g = nullptr, *u = nullptr, *logits = nullptr, *tmp = nullptr;
     float *pk = nullptr;  // [16][max(q_dim + 2 kv_dim, 2 ffn)]: output of a fused q/k/v or gate/up GEMM
+    // cur, attn and g once more, as f16 in MFMA fragment order, for the projections that take the whole-K kernel
+    uint8_t *xf_cur = nullptr, *xf_attn = nullptr, *xf_g = nullptr;
     int32_t *ids = nullptr, *pos = nullptr, *argmax = nullptr;
     // every layer's context K/V projection as ONE batched GEMM (draft_prepare): its output [layer][16][2 kv_dim],
     // the list 0 .. n_layers - 1 and its length for the batched kernel
@@ -525,6 +562,9 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
               dev_alloc(&s->k, 16 * kv_dim) && dev_alloc(&s->v, 16 * kv_dim) && dev_alloc(&s->attn, 16 * q_dim) &&
               dev_alloc(&s->mix, 16 * cfg->hidden) && dev_alloc(&s->g, 16 * f) && dev_alloc(&s->u, 16 * f) &&
               dev_alloc(&s->pk, 16 * std::max(q_dim + 2 * kv_dim, 2 * f)) &&
+              dev_alloc(&s->xf_cur, dfl_xf_bytes((cfg->hidden + 255) / 256 * 256)) &&
+              dev_alloc(&s->xf_attn, dfl_xf_bytes((static_cast<int64_t>(q_dim) + 255) / 256 * 256)) &&
+              dev_alloc(&s->xf_g, dfl_xf_bytes((static_cast<int64_t>(f) + 255) / 256 * 256)) &&
               dev_alloc(&s->logits, 16 * static_cast<size_t>(cfg->vocab)) && dev_alloc(&s->gap, 16) &&
               dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) && dev_alloc(&s->argmax, 16) &&
               dev_alloc(&s->hidden, 16 * static_cast<size_t>(std::max(n_taps, 1)) * cfg->hidden);
@@ -576,7 +616,7 @@ void dflash_session_destroy(dflash_session *s) {
     void *ptrs[] = {s->k_cache, s->vt_cache, s->x, s->cur, s->q, s->k, s->v, s->attn, s->mix,
                     s->g, s->u, s->logits, s->gap, s->ids, s->pos, s->argmax, s->hidden,
                     s->moe.probs, s->moe.sel_e, s->moe.sel_w, s->moe.sg, s->moe.act, s->moe.eo, s->moe.shared,
-                    s->moe.gate_out, s->moe.ids, s->moe.n_distinct, s->moe.slot_of, s->pk};
+                    s->moe.gate_out, s->moe.ids, s->moe.n_distinct, s->moe.slot_of, s->pk, s->xf_cur, s->xf_attn, s->xf_g};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;
@@ -656,16 +696,27 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
     const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
     bool cur_ready = false;  // s->cur already holds this layer's normalised input
     const float *pending_resid = nullptr;  // a dense layer's FFN output still to be added to s->x
+    // which projections of a layer read their rows in fragment order (past the last layer: none, the head streams)
+    auto layer_kinds = [&](int il) {
+        return il < c.n_layers ? layer_xf(ctx, model->layers[il], s->pk != nullptr, H, static_cast<int64_t>(q_dim),
+                                          static_cast<int64_t>(kv_dim), c.ffn, c.n_expert == 0)
+                               : LayerXf();
+    };
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_layer &L = model->layers[il];
         _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
         // (a mixture-of-experts layer leaves the next layer's normalised input behind)
         // (a dense layer leaves its FFN output in s->mix: the residual add is folded into this norm)
-        if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
+        const bool moe = c.n_expert > 0;
+        const LayerXf xk = layer_kinds(il);
+        if (!cur_ready)
+            rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr,
+                                               xk.qkv ? s->xf_cur : nullptr, xk.qkv);
         pending_resid = nullptr;
         cur_ready = false;
         bool packed;
-        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, true, &packed, H, q_dim, kv_dim, n, st))) return rc;
+        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, s->cur, s->q, s->k, s->v, s->pk, true, &packed, H, q_dim, kv_dim, n, st, s->xf_cur, xk.qkv)))
+            return rc;
         const int64_t tot = q_dim + 2 * kv_dim;
         qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(
             packed ? s->pk : s->q, packed ? tot : q_dim, packed ? s->pk + q_dim : s->k, packed ? tot : kv_dim, s->q, s->k, L.q_norm,
@@ -688,25 +739,37 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
         // under capture the context length is read from pos[0] on the device: the same launches then serve every
         // position of the bucket
         if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, kc, vtc, 1, start, n, c.n_q, c.n_kv, hd, s->capacity, scale,
-                                 s->attn, st, 0, 0, ctx->capturing ? s->pos : nullptr)))
+                                 s->attn, st, 0, 0, ctx->capturing ? s->pos : nullptr, xk.wo ? s->xf_attn : nullptr, xk.wo)))
             return rc;
-        if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st))) return rc;
+        if (xk.wo)
+            rc = dfl_gemm_whole(ctx, L.wo.type, L.wo.data, s->xf_attn, s->mix, static_cast<int64_t>(q_dim), H, n, 0, nullptr, DFL_XF_NONE, st);
+        else
+            rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, n, st);
+        if (rc) return rc;
         // x += mix first; a mixture-of-experts layer also gets its shared-expert gate from here
-        const bool moe = c.n_expert > 0;
         // (where the router's launch can take the add and the norm along, they are left to it; s->x then gets its
         // s->mix together with the experts' sum)
         const bool norm_in_router = moe && dfl_moe_norm_fusable(ctx, c, L, n);
         if (!norm_in_router)
             rms_norm_kernel<<<n, 256, 0, st>>>(s->x, s->mix, L.post_norm, s->cur, H, c.eps, moe ? L.shexp_gate : nullptr,
-                                               moe ? s->moe.sg : nullptr);
+                                               moe ? s->moe.sg : nullptr, xk.gate_up ? s->xf_cur : nullptr, xk.gate_up);
         if (moe) {
             const float *next_w = il + 1 < c.n_layers ? model->layers[il + 1].attn_norm : model->output_norm;
+            const int next_kind = layer_kinds(il + 1).qkv;  // (the next layer's q/k/v read what this layer's last kernel normalises)
             if ((rc = dfl_moe_ffn(ctx, c, L, s->cur, n, s->moe, s->x, L.shexp_gate != nullptr, next_w, s->cur, &cur_ready, st,
-                                  norm_in_router ? s->mix : nullptr, norm_in_router ? L.post_norm : nullptr)))
+                                  norm_in_router ? s->mix : nullptr, norm_in_router ? L.post_norm : nullptr,
+                                  next_kind ? s->xf_cur : nullptr, next_kind)))
                 return rc;
         } else {
-            if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, n, st))) return rc;
-            if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st))) return rc;
+            // the down projection reads fragment-order rows only where the gate/up launch can write them
+            const int down_kind = xk.gate_up ? xk.down : DFL_XF_NONE;
+            if ((rc = gemm_gate_up(ctx, L.gate, L.up, s->cur, s->g, s->u, s->pk, H, c.ffn, n, st, s->xf_cur, xk.gate_up, s->xf_g, down_kind)))
+                return rc;
+            if (down_kind)
+                rc = dfl_gemm_whole(ctx, L.down.type, L.down.data, s->xf_g, s->mix, c.ffn, H, n, 0, nullptr, DFL_XF_NONE, st);
+            else
+                rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, n, st);
+            if (rc) return rc;
             // x += mix: by the next norm, unless this layer's residual is captured first
             bool tapped = false;
             for (int t = 0; t < n_taps; t++) tapped = tapped || tap_layers[t] == il;
@@ -1015,7 +1078,10 @@ int32_t dflash_draft_session_create(dflash_ctx *ctx, const dflash_draft_cfg *cfg
               dev_alloc(&s->pk, 16 * std::max(q_dim + 2 * kv_dim, 2 * static_cast<size_t>(cfg->ffn))) &&
               dev_alloc(&s->tmp, 16 * std::max(H, kv_dim)) && dev_alloc(&s->ids, 16) && dev_alloc(&s->pos, 16) &&
               dev_alloc(&s->argmax, 16) && dev_alloc(&s->pk_layers, static_cast<size_t>(cfg->n_layers) * 16 * 2 * kv_dim) &&
-              dev_alloc(&s->layer_ids, static_cast<size_t>(cfg->n_layers)) && dev_alloc(&s->n_layers_dev, 1);
+              dev_alloc(&s->layer_ids, static_cast<size_t>(cfg->n_layers)) && dev_alloc(&s->n_layers_dev, 1) &&
+              dev_alloc(&s->xf_cur, dfl_xf_bytes((static_cast<int64_t>(H) + 255) / 256 * 256)) &&
+              dev_alloc(&s->xf_attn, dfl_xf_bytes((static_cast<int64_t>(q_dim) + 255) / 256 * 256)) &&
+              dev_alloc(&s->xf_g, dfl_xf_bytes((static_cast<int64_t>(cfg->ffn) + 255) / 256 * 256));
     if (ok) {
         std::vector<int32_t> ids(static_cast<size_t>(cfg->n_layers));
         for (int i = 0; i < cfg->n_layers; i++) ids[i] = i;
@@ -1041,7 +1107,7 @@ void dflash_draft_session_destroy(dflash_draft_session *s) {
     if (!s) return;
     void *ptrs[] = {s->ctx_raw, s->ctx_h, s->k_ctx, s->v_ctx, s->k16, s->vt16, s->pos_ctx, s->x, s->cur, s->q, s->k, s->v,
                     s->attn, s->mix, s->g, s->u, s->logits, s->tmp, s->ids, s->pos, s->argmax, s->pk, s->pk_layers,
-                    s->layer_ids, s->n_layers_dev,
+                    s->layer_ids, s->n_layers_dev, s->xf_cur, s->xf_attn, s->xf_g,
                     s->conv_buf, s->conv_dyn, s->topk_ids, s->topk_vals, s->sel_h};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -1265,19 +1331,23 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         _Float16 *k16 = s->k16 + il * static_cast<size_t>(s->cap16) * kv_dim;
         _Float16 *vt16 = s->vt16 + il * static_cast<size_t>(s->cap16) * kv_dim;
         // the previous layer's second residual (x += ffn output) is folded into this norm
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr);
+        // (in a DFlash-2 layer the side-0 convolution sits between the norm and the projection: it writes the fragment-order rows)
+        const LayerXf xk = layer_xf(ctx, L, fast && s->pk != nullptr, H, static_cast<int64_t>(q_dim), static_cast<int64_t>(kv_dim), c.ffn, true);
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr,
+                                           xk.qkv && !conv ? s->xf_cur : nullptr, xk.qkv);
         // DFlash-2 attention convolution (metal_dflash.rs:16210-16262): the dynamic coefficients come
         // from the normed input and serve both sides; q/k/v read the side-0 result
         const float *attn_src = s->cur;
         if (conv) {
             if ((rc = gemm(ctx, L.conv_attn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st))) return rc;
-            if ((rc = dflash_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_attn_base, s->conv_buf, N, H, c.conv_kernel_size,
-                                          c.conv_group_size, 0, st)))
+            if ((rc = dfl_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_attn_base, s->conv_buf, N, H, c.conv_kernel_size,
+                                       c.conv_group_size, 0, st, xk.qkv ? s->xf_cur : nullptr, xk.qkv)))
                 return rc;
             attn_src = s->conv_buf;
         }
         bool packed;  // only on the fast path: the general attention kernel reads V dense
-        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, attn_src, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st))) return rc;
+        if ((rc = gemm_qkv(ctx, L.wq, L.wk, L.wv, attn_src, s->q, s->k, s->v, s->pk, fast, &packed, H, q_dim, kv_dim, N, st, s->xf_cur, xk.qkv)))
+            return rc;
         const int64_t tot = q_dim + 2 * kv_dim;
         if (fast) {
             // the block's own K (normed, rotated) and V go behind the context in the f16 mirror, written by the
@@ -1290,7 +1360,8 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
             // of the bucket; chunking, and so the result, is the same either way)
             if ((rc = dfl_attn_block(ctx, s->q, DFLASH_TYPE_F32, k16, vt16, 1, s->ctx_len, N, c.n_q, c.n_kv, hd, s->cap16,
                                      1.0f / sqrtf(static_cast<float>(hd)), s->attn, st, c.causal ? 0 : 1,
-                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, ctx->capturing ? s->pos : nullptr)))
+                                     L.is_swa ? static_cast<int64_t>(c.swa_window) : 0, ctx->capturing ? s->pos : nullptr,
+                                     xk.wo ? s->xf_attn : nullptr, xk.wo)))
                 return rc;
         } else {
             qk_norm_rope_kernel<<<dim3(c.n_q + c.n_kv, N), 64, 0, st>>>(s->q, q_dim, s->k, kv_dim, s->q, s->k, L.q_norm, L.k_norm,
@@ -1300,7 +1371,11 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                                                             N, c.n_q, c.n_kv, hd, static_cast<int>(noise_start), c.causal,
                                                             L.is_swa ? static_cast<int>(c.swa_window) : 0, s->attn);
         }
-        if ((rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st))) return rc;
+        if (fast && xk.wo)  // (only the MFMA attention writes its rows in fragment order)
+            rc = dfl_gemm_whole(ctx, L.wo.type, L.wo.data, s->xf_attn, s->mix, static_cast<int64_t>(q_dim), H, N, 0, nullptr, DFL_XF_NONE, st);
+        else
+            rc = gemm(ctx, L.wo, s->attn, s->mix, q_dim, H, N, st);
+        if (rc) return rc;
         // residual 1 (x += attn_output; DFlash-2: its side-1 convolution, same coefficients, :16795-16820),
         // folded into the norm that follows
         const float *resid = s->mix;
@@ -1310,17 +1385,24 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                 return rc;
             resid = s->conv_buf;
         }
-        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, resid, L.post_norm, s->cur, H, c.eps, nullptr, nullptr);
+        rms_norm_kernel<<<N, 256, 0, st>>>(s->x, resid, L.post_norm, s->cur, H, c.eps, nullptr, nullptr,
+                                           xk.gate_up && !conv ? s->xf_cur : nullptr, xk.gate_up);
         const float *ffn_src = s->cur;
         if (conv) {  // the FFN pair (:16836-16885, 17003-17022)
             if ((rc = gemm(ctx, L.conv_ffn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st))) return rc;
-            if ((rc = dflash_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_ffn_base, s->conv_buf, N, H, c.conv_kernel_size,
-                                          c.conv_group_size, 0, st)))
+            if ((rc = dfl_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_ffn_base, s->conv_buf, N, H, c.conv_kernel_size,
+                                       c.conv_group_size, 0, st, xk.gate_up ? s->xf_cur : nullptr, xk.gate_up)))
                 return rc;
             ffn_src = s->conv_buf;
         }
-        if ((rc = gemm_gate_up(ctx, L.gate, L.up, ffn_src, s->g, s->u, s->pk, H, c.ffn, N, st))) return rc;
-        if ((rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st))) return rc;
+        const int down_kind = xk.gate_up ? xk.down : DFL_XF_NONE;  // fragment-order rows only from the gate/up launch's epilogue
+        if ((rc = gemm_gate_up(ctx, L.gate, L.up, ffn_src, s->g, s->u, s->pk, H, c.ffn, N, st, s->xf_cur, xk.gate_up, s->xf_g, down_kind)))
+            return rc;
+        if (down_kind)
+            rc = dfl_gemm_whole(ctx, L.down.type, L.down.data, s->xf_g, s->mix, c.ffn, H, N, 0, nullptr, DFL_XF_NONE, st);
+        else
+            rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st);
+        if (rc) return rc;
         resid = s->mix;
         if (conv) {
             if ((rc = dflash_dflash2_conv(ctx, s->mix, s->conv_dyn, L.conv_ffn_base, s->conv_buf, N, H, c.conv_kernel_size,

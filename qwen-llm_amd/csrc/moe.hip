@@ -371,7 +371,8 @@ __global__ void __launch_bounds__(256)
     moe_combine_norm_kernel(const float *__restrict__ eo, const int32_t *__restrict__ slot_of, const float *__restrict__ sel_w,
                             const float *__restrict__ sg, const float *__restrict__ shared, const int32_t *__restrict__ n_slots,
                             int n_used, int hidden, float *__restrict__ x, const float *__restrict__ norm_w,
-                            float *__restrict__ y, float eps, const float *__restrict__ pre_add) {
+                            float *__restrict__ y, float eps, const float *__restrict__ pre_add, void *__restrict__ y_xf,
+                            int y_xf_kind) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
     __shared__ float w_k[64];
@@ -413,8 +414,12 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int i = 4 * (tid + 256 * j);
-        if (i < hidden)
-            *reinterpret_cast<f4 *>(y + static_cast<size_t>(row) * hidden + i) = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
+        if (i < hidden) {
+            const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
+            *reinterpret_cast<f4 *>(y + static_cast<size_t>(row) * hidden + i) = o;
+            // (hidden a multiple of 256 here: whole waves are inside or outside the row)
+            if (y_xf) dfl_xf_store_pair(y_xf, y_xf_kind, row, i & ~7, o[0], o[1], o[2], o[3]);
+        }
     }
 }
 
@@ -439,7 +444,7 @@ bool dfl_moe_norm_fusable(const dflash_ctx *ctx, const dflash_model_cfg &c, cons
 
 int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, float *cur, int n,
                     const dfl_moe_scratch &s, float *x_resid, bool gate_done, const float *next_norm_w, float *next_cur,
-                    bool *next_done, hipStream_t st, const float *pre_add, const float *pre_norm_w) {
+                    bool *next_done, hipStream_t st, const float *pre_add, const float *pre_norm_w, void *next_xf, int next_xf_kind) {
     if (next_done) *next_done = false;
     if ((pre_add != nullptr) != (pre_norm_w != nullptr) ||
         (pre_add && !(next_norm_w && next_cur && next_done && dfl_moe_norm_fusable(ctx, c, L, n))))
@@ -556,7 +561,8 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
     }
     if (batched && next_norm_w && next_cur && next_done && H <= 4096 && H % 4 == 0) {
         moe_combine_norm_kernel<<<n, 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg, folded_shared ? nullptr : s.shared, s.n_distinct,
-                                                   used, H, x_resid, next_norm_w, next_cur, c.eps, pre_add);
+                                                   used, H, x_resid, next_norm_w, next_cur, c.eps, pre_add,
+                                                   H % DFL_QK_K == 0 ? next_xf : nullptr, next_xf_kind);
         *next_done = true;
     } else if (batched)
         moe_combine_slots_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg,

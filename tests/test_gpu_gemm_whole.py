@@ -1,0 +1,112 @@
+"""GPU parity of the whole-K few-row GEMM over activations in fragment order (dflash_pack_xf,
+dflash_gemm_fewrow_xf): against float64 of the oracle's dequant (<= 1e-2 relative, f32 accumulation), and
+against dflash_gemm_fewrow on the same weights (same operands rounded the same way: the two may differ only in
+the order of the f32 sums)."""
+import numpy as np
+import pytest
+
+import qwen_llm_amd as dfl
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = dfl.Context(0)
+    yield c
+    c.close()
+
+
+def dev(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def check(y, ref, label):
+    y = y.astype(np.float64)
+    assert np.all(np.isfinite(y)), f"{label}: non-finite output"
+    rel_l2 = np.linalg.norm(y - ref) / max(np.linalg.norm(ref), 1e-30)
+    rms = np.sqrt(np.mean(ref ** 2))
+    elem = np.max(np.abs(y - ref) / np.maximum(np.abs(ref), rms))
+    assert rel_l2 <= 2e-3 and elem <= 1e-2, f"{label}: rel_l2 {rel_l2:.3e} elem {elem:.3e}"
+
+
+# (n_in, n_out, rows): one stage per wave (n_in <= 4096), two (up to 8192), ragged tile and row counts, two tiles per wave
+SHAPES = [(256, 16, 16), (256, 40, 1), (1024, 272, 16), (2048, 5120, 16), (2048, 1000, 7), (4096, 2048, 16), (6144, 2048, 16),
+          (5120, 6144, 16), (2048, 12288, 16), (3072, 100, 3), (8192, 48, 16)]
+
+
+def upload(ctx, qtype, n_in, n_out, seed, extreme=False):
+    """(device weight, type tag for the GEMM, host blocks in GGUF row order)."""
+    if extreme:
+        blocks = dfl.synth.extreme_blocks(qtype, n_out * n_in // 256, seed=seed).reshape(n_out, -1)
+    else:
+        blocks = dfl.synth.random_weight(qtype, n_out, n_in, seed=seed)
+    wd = dev(blocks)
+    if qtype == dfl.synth.Q4_K:
+        return ctx.repack_q4k_tiled(wd, n_in, n_out), dfl.TYPE_Q4_K_TILED, blocks, wd
+    return wd, dfl.TYPE_Q6_K, blocks, wd
+
+
+@pytest.mark.parametrize("qtype", [dfl.synth.Q4_K, dfl.synth.Q6_K])
+@pytest.mark.parametrize("n_in,n_out,rows", SHAPES)
+@pytest.mark.parametrize("x_dtype", [np.float32, np.float16])
+def test_whole_k_gemm_matches_oracle_and_streaming_kernels(ctx, oracle, canaries, qtype, n_in, n_out, rows, x_dtype):
+    w, w_type, blocks, w_rows = upload(ctx, qtype, n_in, n_out, seed=n_in + n_out)
+    kind = ctx.xf_kind(w_type, n_in, n_out)
+    assert kind == (dfl.XF_Q4K if qtype == dfl.synth.Q4_K else dfl.XF_Q6K)
+    x = np.random.default_rng(rows).standard_normal((rows, n_in)).astype(x_dtype)
+    xd = dev(x)
+    xf = ctx.pack_xf(xd, kind)
+    y = ctx.gemm_fewrow_xf(w, w_type, xf, rows, n_in, n_out).cpu().numpy()
+    canaries.check()
+    wf = oracle.dequant(qtype, blocks, n_in * n_out).reshape(n_out, n_in).astype(np.float64)
+    ref = x.astype(np.float16).astype(np.float64) @ wf.T  # every few-row kernel rounds its activations to f16
+    check(y, ref, f"{n_in}->{n_out} x{rows}")
+    # the streaming kernels on the same operands: same products, other order of the f32 sums
+    y2 = ctx.gemm_fewrow(w, w_type, xd, n_in, n_out).cpu().numpy()
+    assert np.max(np.abs(y - y2)) <= 2e-5 * max(np.max(np.abs(ref)), 1.0) + 1e-4 * np.sqrt(np.mean(ref ** 2))
+
+
+@pytest.mark.parametrize("qtype", [dfl.synth.Q4_K, dfl.synth.Q6_K])
+def test_whole_k_gemm_extreme_blocks(ctx, oracle, qtype):
+    """The reference's extreme blocks (metal/mat_mat.rs:4228-4265: largest scales and codes) within the kernels' range."""
+    n_in, n_out, rows = 2048, 320, 16
+    w, w_type, blocks, _ = upload(ctx, qtype, n_in, n_out, seed=5, extreme=True)
+    x = np.random.default_rng(6).standard_normal((rows, n_in)).astype(np.float32)
+    xf = ctx.pack_xf(dev(x), ctx.xf_kind(w_type, n_in, n_out))
+    y = ctx.gemm_fewrow_xf(w, w_type, xf, rows, n_in, n_out).cpu().numpy()
+    wf = oracle.dequant(qtype, blocks, n_in * n_out).reshape(n_out, n_in).astype(np.float64)
+    check(y, x.astype(np.float16).astype(np.float64) @ wf.T, "extreme")
+
+
+def test_rows_are_independent(ctx):
+    """A row of the product depends on its own activation row only: a 16-row block and each row alone agree bit for
+    bit (what makes a packed verify equal to token-by-token decoding through the same kernel)."""
+    n_in, n_out = 2048, 5120
+    for qtype in (dfl.synth.Q4_K, dfl.synth.Q6_K):
+        w, w_type, _, _ = upload(ctx, qtype, n_in, n_out, seed=9)
+        kind = ctx.xf_kind(w_type, n_in, n_out)
+        x = dev(np.random.default_rng(3).standard_normal((16, n_in)).astype(np.float32))
+        y = ctx.gemm_fewrow_xf(w, w_type, ctx.pack_xf(x, kind), 16, n_in, n_out).cpu().numpy()
+        for r in (0, 7, 15):
+            y1 = ctx.gemm_fewrow_xf(w, w_type, ctx.pack_xf(x[r:r + 1].contiguous(), kind), 1, n_in, n_out).cpu().numpy()
+            assert np.array_equal(y1[0].view(np.uint32), y[r].view(np.uint32))
+
+
+def test_shapes_outside_the_path_are_declined(ctx):
+    import torch
+
+    assert ctx.xf_kind(dfl.TYPE_Q4_K_TILED, 17408, 5120) == dfl.XF_NONE      # more than two stages per wave
+    assert ctx.xf_kind(dfl.TYPE_Q6_K, 2048, 151936) == dfl.XF_NONE           # more than one round of the chip
+    assert ctx.xf_kind(dfl.TYPE_Q4_K, 2048, 2048) == dfl.XF_NONE             # GGUF row order Q4_K: streaming kernels only
+    assert ctx.xf_kind(dfl.TYPE_Q8_0, 2048, 2048) == dfl.XF_NONE
+    buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    y = torch.zeros((16, 5120), dtype=torch.float32, device="cuda")
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.gemm_fewrow_xf(buf, dfl.TYPE_Q4_K_TILED, buf, 16, 17408, 5120, y=y)
+    assert e.value.kind == "Unsupported"
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.pack_xf(torch.zeros((16, 300), device="cuda"), dfl.XF_Q4K)
+    assert e.value.kind == "BadShape"
