@@ -127,15 +127,16 @@ def q6k_section(ctx):
         ws = [dfl.synth.random_blocks_device(dfl.synth.Q6_K, n_out, n_in, 0.02, g, "cuda") for _ in range(n_sets)]
         x = torch.randn((16, n_in), device="cuda", generator=g)
         y = torch.empty((16, n_out), device="cuda")
+        tag = ctx.checked_type(dfl.TYPE_Q6_K, ws[0])  # (every set comes from the same generator: one range check speaks for all)
         for w in ws:
-            ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q6_K, x, y, n_in, n_out, 16)
+            ctx.encode_mat_mat_dispatch_dflash_verify(w, tag, x, y, n_in, n_out, 16)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         reps = 3
         e0.record()
         for _ in range(reps):
             for w in ws:
-                ctx.encode_mat_mat_dispatch_dflash_verify(w, dfl.TYPE_Q6_K, x, y, n_in, n_out, 16)
+                ctx.encode_mat_mat_dispatch_dflash_verify(w, tag, x, y, n_in, n_out, 16)
         e1.record()
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) / (reps * n_sets) * 1e3
@@ -608,7 +609,7 @@ def main():
     tiled_us = kernel_times(wd, w_type)
     # the same launches on GGUF row order, rotating over as many copies
     row_sets = [[w] + [w.clone() for _ in range(n_sets - 1)] for w in wrow]
-    row_us = kernel_times(row_sets, dfl.TYPE_Q4_K)
+    row_us = kernel_times(row_sets, dfl.TYPE_Q4_K | dfl.TYPE_RANGE_CHECKED)  # (the same blocks the repack range-checked)
     del row_sets
     # a read-only stream over the same buffers with the same launch shape: the practical ceiling of such a kernel
     probe_out = torch.zeros(1024, dtype=torch.int32, device="cuda")

@@ -110,17 +110,32 @@ int32_t dflash_dequant(dflash_ctx *ctx, int32_t type, const void *blocks, size_t
                        dflash_stream_t stream);
 size_t dflash_row_bytes(int32_t type, size_t n_in);
 
-/* ---- scale range of a quantised tensor (load-time guard) ----------------------------------
- * No counterpart in the reference (its kernels scale in f32 after the MMA, mat_mat_fewrow_gen.metal:437-444).  The few-row
- * Q4_K / Q6_K kernels here apply d * scale in f16 before the MFMA, which is finite only while
+/* ---- scale range of a quantised tensor: the precondition of the fast kernels ------------------------
+ * No counterpart in the reference: its kernels scale in f32 after the MMA (mat_mat_fewrow_gen.metal:437-444) and take
+ * any ggml block.  The fast few-row Q4_K / Q6_K kernels here apply d * scale in f16 before the MFMA, which is finite
+ * only while
  *   Q4_K: |d| <= DFLASH_Q4_K_MAX_D and |dmin| <= DFLASH_Q4_K_MAX_DMIN,   Q6_K: |d| <= DFLASH_Q6_K_MAX_D
- * (weight scales of real checkpoints are 1e-4 .. 1e-1).  Call this once per tensor when it is uploaded: it scans the
- * super-block headers on the device, returns the maxima in max_abs_host[2] (|d|, |dmin|; may be NULL) and
- * DFLASH_ERR_UNSUPPORTED with a message for a tensor out of range or with a NaN / infinite scale, DFLASH_OK otherwise
- * (and for types whose kernels have no such limit).  Blocking. */
+ * (weight scales of real checkpoints are 1e-4 .. 1e-1).  The precondition is part of the tensor's tag:
+ *   - dflash_check_scale_range scans a tensor's super-block headers on the device (once, when it is uploaded),
+ *     returns the maxima in max_abs_host[2] (|d|, |dmin|; may be NULL) and DFLASH_ERR_UNSUPPORTED with a message for
+ *     a tensor out of range or with a NaN / infinite scale, DFLASH_OK otherwise (and for types whose kernels have
+ *     no such limit).  Blocking.
+ *   - Only a tensor that passed may be tagged as checked: w_type | DFLASH_TYPE_RANGE_CHECKED where a call takes the
+ *     type as an argument, flags = DFLASH_QT_RANGE_CHECKED in a dflash_qtensor.  dflash_repack_q4k_tiled runs the
+ *     scan itself, so DFLASH_TYPE_Q4_K_TILED is checked by construction.
+ *   - dflash_gemm_fewrow / dflash_gemm_fewrow_noalloc on an UNTAGGED Q4_K / Q6_K tensor run a kernel that dequantises
+ *     in f32 exactly as ggml does and accumulates in f32: correct for every block a GGUF file can hold (what the
+ *     reference's seam promises), about two orders of magnitude slower.  The model-level calls
+ *     (dflash_verify_block, dflash_prefill_blocks, dflash_draft_block, dflash_draft_prepare_ctx, dflash_spec_step)
+ *     decline a model that holds an untagged Q4_K / Q6_K tensor with DFLASH_ERR_UNSUPPORTED, naming it.
+ * A result is therefore either correct or declined: never an infinity with status 0. */
 #define DFLASH_Q4_K_MAX_D 1.0f
 #define DFLASH_Q4_K_MAX_DMIN 32.0f
 #define DFLASH_Q6_K_MAX_D 0.25f
+enum {
+    DFLASH_TYPE_RANGE_CHECKED = 65536, /* 0x10000, OR-ed into a w_type argument */
+    DFLASH_QT_RANGE_CHECKED = 1        /* dflash_qtensor.flags */
+};
 int32_t dflash_check_scale_range(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_blocks, float *max_abs_host,
                                  dflash_stream_t stream);
 
@@ -138,7 +153,9 @@ int32_t dflash_hbm_read_probe(dflash_ctx *ctx, const void *const *bufs, int32_t 
  *   [tile group of 256 rows][super-block][tile 0..15][row 0..15][block],  last group padded with zero blocks.
  * dflash_q4k_tiled_bytes: size of the tiled matrix (0 for a bad shape).  dflash_repack_q4k_tiled: W in GGUF row
  * order (16-byte aligned) -> w_tiled (128-byte aligned, dflash_q4k_tiled_bytes long, not overlapping W).  The
- * result is passed to dflash_gemm_fewrow as w_type DFLASH_TYPE_Q4_K_TILED and gives bit-identical Y.  Enqueue-only. */
+ * result is passed to dflash_gemm_fewrow as w_type DFLASH_TYPE_Q4_K_TILED and gives bit-identical Y.  The source is
+ * range-checked first (dflash_check_scale_range; DFLASH_ERR_UNSUPPORTED for a tensor out of range, nothing is written
+ * then), so a tiled tensor is always one the fast kernels take.  Blocking. */
 size_t dflash_q4k_tiled_bytes(int64_t n_in, int64_t n_out);
 int32_t dflash_repack_q4k_tiled(dflash_ctx *ctx, const void *w, void *w_tiled, int64_t n_in, int64_t n_out,
                                 dflash_stream_t stream);
@@ -148,6 +165,8 @@ int32_t dflash_repack_q4k_tiled(dflash_ctx *ctx, const void *w, void *w_tiled, i
  * (metal_forward/dispatch.rs:365-378; kernel kernels/mat_mat_fewrow_gen.metal:374-474).
  *   Y[n_rows][n_out] = X[n_rows][n_in] . W^T,  W = quant blocks, row-major [n_out][n_in/blk]
  * x_type: DFLASH_TYPE_F32 (the reference's activations) or DFLASH_TYPE_F16; Y is f32.
+ * w_type: a ggml tag (any block of that type is computed correctly), or tag | DFLASH_TYPE_RANGE_CHECKED /
+ * DFLASH_TYPE_Q4_K_TILED for a tensor that passed dflash_check_scale_range (the fast kernels).
  * 1 <= n_rows <= 16; n_in % 256 == 0 (Q4_K, Q6_K) or % 32 == 0 (Q8_0, and plain F32 / F16 matrices
  * such as a router stored unquantised); W 16-byte aligned (2-byte for Q8_0 and Q6_K); Y must not
  * alias X or W.  Enqueue-only. */
@@ -181,8 +200,9 @@ const char *dflash_gemm_fewrow_noalloc_error(void);
  * calls expose it.
  *   dflash_xf_bytes: size of an XF buffer for n_in values per row (n_in % 256 == 0; 0 otherwise).
  *   dflash_gemm_fewrow_xf_kind: the XF kind (DFLASH_XF_Q4K / DFLASH_XF_Q6K) this (type, shape) reads, or
- *     DFLASH_XF_NONE where it is not taken: w_type must be DFLASH_TYPE_Q4_K_TILED or DFLASH_TYPE_Q6_K, n_in at most
- *     8192, and the matrix at most one round of the chip (about 320 workgroups of 16 or 32 rows).
+ *     DFLASH_XF_NONE where it is not taken: w_type must be DFLASH_TYPE_Q4_K_TILED or DFLASH_TYPE_Q6_K |
+ *     DFLASH_TYPE_RANGE_CHECKED (these kernels scale in f16: a range-checked tensor only), n_in at most 8192, and
+ *     the matrix at most one round of the chip (about 320 workgroups of 16 or 32 rows).
  *   dflash_pack_xf: row-major x[n_rows][n_in] (f32 or f16) -> xf, rounding to f16 as every few-row kernel does.
  *   dflash_gemm_fewrow_xf: Y[n_rows][n_out] = X . W^T; same guards as dflash_gemm_fewrow; DFLASH_ERR_UNSUPPORTED
  *     where the kind is DFLASH_XF_NONE.  A (row, column) result depends on that activation row and weight row only.
@@ -363,7 +383,7 @@ int32_t dflash_select_draft_path_sampled(dflash_ctx *ctx, const dflash_codebook 
  * Gated-DeltaNet layers of the hybrid target, which the synthetic configurations do not have). */
 typedef struct {
     int32_t type;
-    int32_t pad;
+    int32_t flags; /* DFLASH_QT_RANGE_CHECKED: the tensor passed dflash_check_scale_range (Q4_K / Q6_K; see there) */
     const void *data; /* device */
 } dflash_qtensor;
 

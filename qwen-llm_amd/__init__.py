@@ -21,6 +21,8 @@ from .binding import (  # noqa: F401
     TYPE_Q4_K_TILED,
     TYPE_Q6_K,
     TYPE_Q8_0,
+    TYPE_RANGE_CHECKED,
+    QT_RANGE_CHECKED,
     XF_NONE,
     XF_Q4K,
     XF_Q6K,

@@ -16,6 +16,8 @@ HEADER_PATH = os.path.join(PKG_DIR, "..", "include", "dflash_hip.h")
 TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q6_K = 0, 1, 8, 12, 14
 TYPE_Q4_K_TILED = 1012  # Q4_K blocks in the library's tiled order (Context.repack_q4k_tiled)
 XF_NONE, XF_Q4K, XF_Q6K = 0, 1, 2  # fragment orders of Context.pack_xf
+TYPE_RANGE_CHECKED = 0x10000  # OR-ed into a w_type: the tensor passed Context.check_scale_range (fast Q4_K / Q6_K kernels)
+QT_RANGE_CHECKED = 1  # the same fact in a dflash_qtensor's flags
 
 STATUS = {
     0: "Ok", 1: "BadShape", 2: "Unsupported", 3: "Alias", 4: "Alignment", 5: "Workspace", 6: "Hip",
@@ -302,6 +304,15 @@ class Context:
         self._check(self._lib.dflash_gemm_fewrow(self._h, w_type, weight.data_ptr(), x.data_ptr(), x_type,
                                                  y.data_ptr(), n_in, n_out, n_query, _stream_ptr()))
         return y
+
+    def checked_type(self, qtype: int, blocks) -> int:
+        """Range-checks a Q4_K / Q6_K tensor (raises DFlashError where the fast kernels cannot take it) and returns the
+        type tag that selects them: ``qtype | TYPE_RANGE_CHECKED``.  Other types come back unchanged."""
+        bb = {TYPE_Q4_K: 144, TYPE_Q6_K: 210}.get(int(qtype))
+        if bb is None:
+            return int(qtype)
+        self.check_scale_range(int(qtype), blocks, blocks.numel() * blocks.element_size() // bb)
+        return int(qtype) | TYPE_RANGE_CHECKED
 
     def check_scale_range(self, qtype: int, blocks, n_blocks: int):
         """Load-time guard: raises DFlashError (UNSUPPORTED) for a Q4_K / Q6_K tensor whose super-block scales are

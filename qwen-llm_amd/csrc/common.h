@@ -226,6 +226,10 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
                        int64_t window, const int32_t *ctx_len_dev, void *out_xf = nullptr, int out_xf_kind = 0);
 
+// dflash_gemm_fewrow for a tensor of a model that passed dfl_model_tensors_checked (the fast kernels).
+int32_t dfl_gemm_fewrow_checked(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
+                                int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream);
+
 // Few-row Q6_K GEMMs of up to three matrices over the same activations (a layer's q, k and v
 // projections) as one launch: y[m] = x . w[m]^T, [n_rows][n_out[m]] each.
 int32_t dfl_gemm_q6k_set(dflash_ctx *ctx, int n_mats, const void *const *w, float *const *y, const int64_t *n_out, const void *x,

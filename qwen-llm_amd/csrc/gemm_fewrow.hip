@@ -24,6 +24,7 @@
 //  * Q6_K has its own kernel (half a super-block per step, see there); Q8_0 uses a simple one:
 //    eight consecutive weights per lane are dequantised to f16 and fed to the same MFMA.
 #include "common.h"
+#include "device_quant.h"
 #include "mfma_unpack.h"
 #include "moe_route.h"
 
@@ -2415,6 +2416,34 @@ int32_t dfl_gemm_q6k_set(dflash_ctx *ctx, int n_mats, const void *const *w, floa
 
 namespace {
 
+// The product for a Q4_K / Q6_K tensor that was not range-checked: every weight dequantised in f32 exactly as ggml does
+// (dfl_dequant_elem), f32 activations (f16 ones widened), f32 sums.  Correct for every block the format can hold - the
+// contract of the reference's seam, whose kernels scale in f32 after the MMA (mat_mat_fewrow_gen.metal:437-444) - and slow:
+// one wave per weight row, no matrix cores.  Lanes stride over K, sixteen row sums per lane, a butterfly at the end.
+template <typename XT>
+__global__ void __launch_bounds__(256)
+    gemm_safe_kernel(int type, const uint8_t *__restrict__ w, size_t row_bytes, const XT *__restrict__ x, float *__restrict__ y, int n_in,
+                     int n_out, int n_rows) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= n_out) return;
+    const uint8_t *wr = w + static_cast<size_t>(row) * row_bytes;
+    float acc[16];
+#pragma unroll
+    for (int m = 0; m < 16; m++) acc[m] = 0.0f;
+    for (int k = lane; k < n_in; k += 64) {
+        const float wv = dfl_dequant_elem(type, wr, k);
+#pragma unroll
+        for (int m = 0; m < 16; m++)
+            if (m < n_rows) acc[m] += wv * static_cast<float>(x[static_cast<size_t>(m) * n_in + k]);
+    }
+#pragma unroll
+    for (int m = 0; m < 16; m++) {
+        float v = acc[m];
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+        if (lane == 0 && m < n_rows) y[static_cast<size_t>(m) * n_out + row] = v;
+    }
+}
+
 // Launches the streaming Q4_K kernel (and its split-K reduction): one matrix (batch == nullptr) or the
 // matrices a device-side list picks out of a stack (at most max_slots of them).
 int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in, int64_t n_out,
@@ -2768,6 +2797,8 @@ extern "C" int32_t dflash_repack_q4k_tiled(dflash_ctx *ctx, const void *w, void 
     const size_t out_bytes = dflash_q4k_tiled_bytes(n_in, n_out);
     const size_t in_bytes = static_cast<size_t>(n_out) * (n_in / DFL_QK_K) * DFL_Q4_K_BYTES;
     if (dfl_ranges_overlap(w_tiled, out_bytes, w, in_bytes)) return dfl_fail(ctx, DFLASH_ERR_ALIAS, "repack_q4k_tiled: buffers overlap");
+    // a tiled tensor goes to the fast kernels unconditionally: it must be one they can take
+    if (const int32_t rc = dflash_check_scale_range(ctx, DFLASH_TYPE_Q4_K, w, in_bytes / DFL_Q4_K_BYTES, nullptr, stream)) return rc;
     const int64_t n_pieces = static_cast<int64_t>(out_bytes / 16);
     const int64_t blocks = (n_pieces + 255) / 256;
     if (blocks > 0x7fffffffll) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "repack_q4k_tiled: matrix too large");
@@ -2783,6 +2814,11 @@ extern "C" int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const voi
     return gemm_fewrow_impl(ctx, w_type, w, x, x_type, y, n_in, n_out, n_rows, stream);
 }
 
+int32_t dfl_gemm_fewrow_checked(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,
+                                int64_t n_in, int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
+    return gemm_fewrow_impl(ctx, w_type | DFLASH_TYPE_RANGE_CHECKED, w, x, x_type, y, n_in, n_out, n_rows, stream);
+}
+
 namespace {
 
 int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y, int64_t n_in,
@@ -2795,6 +2831,9 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
                         static_cast<long long>(n_in), static_cast<long long>(n_out));
     if (x_type != DFLASH_TYPE_F32 && x_type != DFLASH_TYPE_F16)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: activations must be f32 or f16");
+    // the fast Q4_K / Q6_K kernels scale in f16: only for a tensor tagged as range-checked (the tiled order is, by construction)
+    const bool checked = (w_type & DFLASH_TYPE_RANGE_CHECKED) != 0 || w_type == DFLASH_TYPE_Q4_K_TILED;
+    w_type &= ~DFLASH_TYPE_RANGE_CHECKED;
     const bool plain = w_type == DFLASH_TYPE_F32 || w_type == DFLASH_TYPE_F16;
     const bool tiled = w_type == DFLASH_TYPE_Q4_K_TILED;
     if (tiled) w_type = DFLASH_TYPE_Q4_K;
@@ -2819,7 +2858,18 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
     const int tiles = static_cast<int>((n_out + 15) / 16);
     const int target_waves = 8 * ctx->n_cu;
 
-    if (w_type == DFLASH_TYPE_Q4_K) {
+    if ((w_type == DFLASH_TYPE_Q4_K || w_type == DFLASH_TYPE_Q6_K) && !checked) {
+        // any block the format can hold: ggml's f32 dequantisation and f32 sums (gemm_safe_kernel)
+        dfl_timed timer(ctx, st, DFL_T_GEMM);
+        const unsigned grid = static_cast<unsigned>((n_out + 3) / 4);
+        if (x_type == DFLASH_TYPE_F32)
+            gemm_safe_kernel<float><<<grid, 256, 0, st>>>(w_type, static_cast<const uint8_t *>(w), row_bytes, static_cast<const float *>(x), y,
+                                                       static_cast<int>(n_in), static_cast<int>(n_out), n_rows);
+        else
+            gemm_safe_kernel<_Float16><<<grid, 256, 0, st>>>(w_type, static_cast<const uint8_t *>(w), row_bytes,
+                                                          static_cast<const _Float16 *>(x), y, static_cast<int>(n_in),
+                                                          static_cast<int>(n_out), n_rows);
+    } else if (w_type == DFLASH_TYPE_Q4_K) {
         if (tiled && reinterpret_cast<uintptr_t>(w) % 128)
             return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_fewrow: tiled Q4_K weights must be 128-byte aligned");
         return launch_q4k(ctx, w, x, x_type, y, n_in, n_out, n_rows, st, nullptr, 1, tiled);

@@ -387,8 +387,19 @@ int32_t dfl_gemm_whole(dflash_ctx *ctx, int32_t w_type, const void *w, const voi
 
 extern "C" size_t dflash_xf_bytes(int64_t n_in) { return n_in > 0 && n_in % DFL_QK_K == 0 ? dfl_xf_bytes(n_in) : 0; }
 
+namespace {
+// The public entries take a range-checked tensor only (there is no f32 kernel behind them): the tiled order, or
+// DFLASH_TYPE_Q6_K | DFLASH_TYPE_RANGE_CHECKED.  Returns the bare type, or -1.
+int32_t xf_public_type(int32_t w_type) {
+    if (w_type == DFLASH_TYPE_Q4_K_TILED) return w_type;
+    if (w_type == (DFLASH_TYPE_Q6_K | DFLASH_TYPE_RANGE_CHECKED)) return DFLASH_TYPE_Q6_K;
+    return -1;
+}
+}  // namespace
+
 extern "C" int32_t dflash_gemm_fewrow_xf_kind(dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out) {
-    return ctx ? dfl_whole_kind(ctx, w_type, n_in, n_out, 0) : DFL_XF_NONE;
+    const int32_t t = xf_public_type(w_type);
+    return ctx && t >= 0 ? dfl_whole_kind(ctx, t, n_in, n_out, 0) : DFL_XF_NONE;
 }
 
 extern "C" int32_t dflash_pack_xf(dflash_ctx *ctx, const void *x, int32_t x_type, int32_t n_rows, int64_t n_in, int32_t kind,
@@ -415,6 +426,13 @@ extern "C" int32_t dflash_pack_xf(dflash_ctx *ctx, const void *x, int32_t x_type
 extern "C" int32_t dflash_gemm_fewrow_xf(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in,
                                          int64_t n_out, int32_t n_rows, dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    const int32_t tagged = w_type;
+    w_type = xf_public_type(tagged);
+    if (w_type < 0)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED,
+                        "gemm_fewrow_xf: type tag %d: only DFLASH_TYPE_Q4_K_TILED and DFLASH_TYPE_Q6_K | DFLASH_TYPE_RANGE_CHECKED "
+                        "(a tensor that passed dflash_check_scale_range) are taken",
+                        tagged);
     if (dfl_whole_kind(ctx, w_type, n_in, n_out, 0) == DFL_XF_NONE)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow_xf: type %d, %lld -> %lld is not taken by the whole-K kernels", w_type,
                         static_cast<long long>(n_in), static_cast<long long>(n_out));

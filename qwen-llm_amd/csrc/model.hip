@@ -359,7 +359,7 @@ inline unsigned blocks_for(size_t n, int threads = 256) { return static_cast<uns
 
 int32_t gemm(dflash_ctx *ctx, const dflash_qtensor &w, const float *x, float *y, int64_t n_in, int64_t n_out, int n,
              hipStream_t st) {
-    return dflash_gemm_fewrow(ctx, w.type, w.data, x, DFLASH_TYPE_F32, y, n_in, n_out, n, st);
+    return dfl_gemm_fewrow_checked(ctx, w.type, w.data, x, DFLASH_TYPE_F32, y, n_in, n_out, n, st);
 }
 
 // True if b's rows follow a's rows_a rows directly in memory and both have the same type: the two
@@ -369,6 +369,41 @@ bool adjacent(const dflash_qtensor &a, int64_t rows_a, const dflash_qtensor &b, 
     const size_t rb = dflash_row_bytes(a.type, n_in);
     return a.type == b.type && rb != 0 &&
            static_cast<const uint8_t *>(b.data) == static_cast<const uint8_t *>(a.data) + static_cast<size_t>(rows_a) * rb;
+}
+
+// The fast kernels take a Q4_K / Q6_K tensor only if it was range-checked (dflash_check_scale_range); the model-level
+// calls use nothing else, so they decline a model that holds an untagged one.  (The tiled order is checked when it is made.)
+bool tensor_checked(const dflash_qtensor &t) {
+    return !t.data || (t.type != DFLASH_TYPE_Q4_K && t.type != DFLASH_TYPE_Q6_K) || (t.flags & DFLASH_QT_RANGE_CHECKED);
+}
+int32_t unchecked(dflash_ctx *ctx, const char *what, int layer) {
+    return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED,
+                    "%s (layer %d) is a Q4_K / Q6_K tensor without DFLASH_QT_RANGE_CHECKED: run dflash_check_scale_range on it when it is uploaded",
+                    what, layer);
+}
+int32_t model_tensors_checked(dflash_ctx *ctx, const dflash_model *m) {
+    if (!tensor_checked(m->token_embd)) return unchecked(ctx, "token_embd", -1);
+    if (!tensor_checked(m->output)) return unchecked(ctx, "output", -1);
+    for (int il = 0; il < m->cfg.n_layers; il++) {
+        const dflash_layer &L = m->layers[il];
+        const dflash_qtensor *ts[] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down, &L.router, &L.gate_exps, &L.up_exps, &L.down_exps};
+        const char *names[] = {"wq", "wk", "wv", "wo", "gate", "up", "down", "router", "gate_exps", "up_exps", "down_exps"};
+        for (int i = 0; i < 11; i++)
+            if (!tensor_checked(*ts[i])) return unchecked(ctx, names[i], il);
+    }
+    return DFLASH_OK;
+}
+int32_t head_tensors_checked(dflash_ctx *ctx, const dflash_draft_head *h) {
+    if (!tensor_checked(h->fc)) return unchecked(ctx, "fc", -1);
+    if (!tensor_checked(h->selector_hidden)) return unchecked(ctx, "selector_hidden", -1);
+    for (int il = 0; il < h->cfg.n_layers; il++) {
+        const dflash_draft_layer &L = h->layers[il];
+        const dflash_qtensor *ts[] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down, &L.conv_attn_proj, &L.conv_ffn_proj};
+        const char *names[] = {"wq", "wk", "wv", "wo", "gate", "up", "down", "conv_attn_proj", "conv_ffn_proj"};
+        for (int i = 0; i < 9; i++)
+            if (!tensor_checked(*ts[i])) return unchecked(ctx, names[i], il);
+    }
+    return DFLASH_OK;
 }
 
 // Which of a layer's projections take the whole-K kernel over activations in fragment order (gemm_whole.hip), and the
@@ -821,6 +856,7 @@ int32_t verify_block_impl(dflash_ctx *ctx, const dflash_model *model, dflash_ses
                           dflash_stream_t stream, bool want_head) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!model || !s || !tokens) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "verify_block: null argument");
+    if (const int32_t rc_ = model_tensors_checked(ctx, model)) return rc_;
     const dflash_model_cfg &c = model->cfg;
     // guard walls (metal_dflash.rs:9080-9186)
     if (n < 1 || n > 16) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "verify_block: n %d outside 1..16", n);
@@ -971,6 +1007,7 @@ int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash
                               float *hidden_capture, dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!model || !s || !tokens) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "prefill_blocks: null argument");
+    if (const int32_t rc_ = model_tensors_checked(ctx, model)) return rc_;
     const dflash_model_cfg &c = model->cfg;
     if (n_tokens < 1) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "prefill_blocks: n_tokens %d", n_tokens);
     if (s->kv_n_pos != start)
@@ -1251,6 +1288,7 @@ int32_t dflash_draft_session_selector_inputs(dflash_ctx *ctx, const dflash_draft
 int32_t dflash_draft_prepare_ctx(dflash_ctx *ctx, const dflash_draft_head *head, dflash_draft_session *s, dflash_stream_t stream) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_prepare_ctx: null argument");
+    if (const int32_t rc_ = head_tensors_checked(ctx, head)) return rc_;
     if (memcmp(&head->cfg, &s->cfg, sizeof(head->cfg)) != 0)
         return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_prepare_ctx: session/head shape mismatch");
     return draft_prepare(ctx, head, s, s->contiguous && head->cfg.n_q / head->cfg.n_kv <= 16, static_cast<hipStream_t>(stream));
@@ -1278,6 +1316,8 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
                          int32_t *argmax_host, dflash_stream_t stream, bool skip_selector_walk) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
     if (!target || !head || !s) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "draft_block: null argument");
+    if (const int32_t rc_ = model_tensors_checked(ctx, target)) return rc_;
+    if (const int32_t rc_ = head_tensors_checked(ctx, head)) return rc_;
     const dflash_draft_cfg &c = head->cfg;
     if (memcmp(&c, &s->cfg, sizeof(c)) != 0) return dfl_fail(ctx, DFLASH_ERR_STATE, "draft_block: session/head shape mismatch");
     if (c.hidden != target->cfg.hidden) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "draft_block: drafter and target hidden sizes differ");

@@ -474,7 +474,7 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         rc = dfl_router_norm(ctx, L.router.data, x_resid, pre_add, pre_norm_w, L.shexp_gate, c.eps, cur, s.sg, s.probs, H, E, n, st);
         gate_done = true;
     } else {
-        rc = dflash_gemm_fewrow(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
+        rc = dfl_gemm_fewrow_checked(ctx, L.router.type, L.router.data, cur, DFLASH_TYPE_F32, s.probs, H, E, n, st);
     }
     if (rc) return rc;
     if (E > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe: %d experts (at most 1024)", E);
@@ -553,11 +553,11 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
         }
     }
     if (!folded_shared) {  // shared expert: plain dense SwiGLU through the few-row GEMM
-        if ((rc = dflash_gemm_fewrow(ctx, L.gate.type, L.gate.data, cur, DFLASH_TYPE_F32, s.g, H, fs, n, st))) return rc;
-        if ((rc = dflash_gemm_fewrow(ctx, L.up.type, L.up.data, cur, DFLASH_TYPE_F32, s.u, H, fs, n, st))) return rc;
+        if ((rc = dfl_gemm_fewrow_checked(ctx, L.gate.type, L.gate.data, cur, DFLASH_TYPE_F32, s.g, H, fs, n, st))) return rc;
+        if ((rc = dfl_gemm_fewrow_checked(ctx, L.up.type, L.up.data, cur, DFLASH_TYPE_F32, s.u, H, fs, n, st))) return rc;
         const size_t nf = static_cast<size_t>(n) * fs;
         silu_mul_rows_kernel<<<static_cast<unsigned>((nf + 255) / 256), 256, 0, st>>>(s.g, s.u, nf);
-        if ((rc = dflash_gemm_fewrow(ctx, L.down.type, L.down.data, s.g, DFLASH_TYPE_F32, s.shared, fs, H, n, st))) return rc;
+        if ((rc = dfl_gemm_fewrow_checked(ctx, L.down.type, L.down.data, s.g, DFLASH_TYPE_F32, s.shared, fs, H, n, st))) return rc;
     }
     if (batched && next_norm_w && next_cur && next_done && H <= 4096 && H % 4 == 0) {
         moe_combine_norm_kernel<<<n, 256, 0, st>>>(s.eo, s.slot_of, s.sel_w, s.sg, folded_shared ? nullptr : s.shared, s.n_distinct,

@@ -16,7 +16,7 @@ import numpy as np
 
 from . import synth
 from . import binding as _binding
-from .binding import TYPE_Q4_K, TYPE_Q4_K_TILED, CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
+from .binding import QT_RANGE_CHECKED, TYPE_Q4_K, TYPE_Q4_K_TILED, CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
 
 
 @dataclass
@@ -64,7 +64,7 @@ class DraftConfig:
 
 
 class QTensorC(C.Structure):
-    _fields_ = [("type", C.c_int32), ("pad", C.c_int32), ("data", C.c_void_p)]
+    _fields_ = [("type", C.c_int32), ("flags", C.c_int32), ("data", C.c_void_p)]
 
 
 class ModelCfgC(C.Structure):
@@ -327,10 +327,13 @@ class _Uploader:
 
     _BLOCK_BYTES = {12: 144, 14: 210}
 
-    def _guard(self, qtype, t):
+    def _guard(self, qtype, t) -> int:
+        """Range check of a Q4_K / Q6_K tensor; returns the dflash_qtensor flags it has earned."""
         bb = self._BLOCK_BYTES.get(int(qtype))
         if self.ctx is not None and bb:
             self.ctx.check_scale_range(int(qtype), t, t.numel() * t.element_size() // bb)
+            return QT_RANGE_CHECKED
+        return 0
 
     def _from_numpy(self, a):
         """torch view of a host array; read-only arrays (views into a mapped GGUF file) are only ever copied from."""
@@ -359,13 +362,13 @@ class _Uploader:
             t = blocks.to(self.device).contiguous()
         else:
             t = self._from_numpy(np.ascontiguousarray(blocks)).to(self.device)
-        self._guard(qtype, t)
+        flags = self._guard(qtype, t)
         if tile_shape is not None and self.tiled and int(qtype) == TYPE_Q4_K:
             t = self.ctx.repack_q4k_tiled(t, tile_shape[1], tile_shape[0])
             qtype = TYPE_Q4_K_TILED
             self.n_tiled += 1
         self.keep.append(t)
-        return QTensorC(int(qtype), 0, t.data_ptr())
+        return QTensorC(int(qtype), flags, t.data_ptr())
 
     def q_adjacent(self, pairs, tile_shapes=None):
         """Uploads matrices of one type and one row length back to back in a single allocation (rows of the
@@ -384,7 +387,7 @@ class _Uploader:
                 flats.append(self._from_numpy(np.ascontiguousarray(blocks).view(np.uint8).reshape(-1)).to(self.device))
         whole = torch.cat(flats)
         qtype = int(pairs[0][0])
-        self._guard(qtype, whole)
+        flags = self._guard(qtype, whole)
         if (tile_shapes is not None and self.tiled and qtype == TYPE_Q4_K
                 and all(ts is not None and ts[0] % 256 == 0 for ts in tile_shapes)):
             whole = self.ctx.repack_q4k_tiled(whole, tile_shapes[0][1], sum(ts[0] for ts in tile_shapes))
@@ -393,7 +396,7 @@ class _Uploader:
         self.keep.append(whole)
         out, off = [], 0
         for f in flats:
-            out.append(QTensorC(qtype, 0, whole.data_ptr() + off))
+            out.append(QTensorC(qtype, flags, whole.data_ptr() + off))
             off += f.numel()
         return out
 

@@ -312,6 +312,8 @@ impl<'a> DFlashDecoder<'a> {
 /// metal_forward/dispatch.rs:365-378: the verifier's few-row mat-mat seam.  `Declined` keeps the caller on its
 /// incumbent kernel, as the Metal route selection does.
 #[allow(clippy::too_many_arguments)]
+/// `weight_type`: the ggml tag of a tensor nobody checked (any block is computed correctly, by the f32 kernel), or
+/// `tag | DFLASH_TYPE_RANGE_CHECKED` / `DFLASH_TYPE_Q4_K_TILED` for one `prepare_weight` accepted (the fast kernels).
 pub fn encode_mat_mat_dispatch_dflash_verify(base: &HipForward, weight_type: i32, weight: *const c_void, x: *const c_void,
                                              x_type: i32, y: *mut f32, n_in: usize, n_out: usize, n_query: u32)
                                              -> Result<(), DFlashError> {
@@ -322,16 +324,19 @@ pub fn encode_mat_mat_dispatch_dflash_verify(base: &HipForward, weight_type: i32
 }
 
 /// Loader step for one quantised tensor already in device memory: range guard, then (Q4_K matrices the few-row GEMM
-/// alone reads) the one-time repack into tiled order.  Returns the type tag to store in the tensor descriptor.
+/// alone reads) the one-time repack into tiled order.  Returns the descriptor to store in the model: the type tag and,
+/// for a Q4_K / Q6_K tensor that passed the guard, `flags = DFLASH_QT_RANGE_CHECKED`, without which the model-level
+/// calls decline the model and `dflash_gemm_fewrow` takes its slow f32 kernel.
 pub fn prepare_weight(base: &HipForward, type_: i32, blocks: *const c_void, n_blocks: usize, tiled_dst: Option<*mut c_void>,
-                      n_in: i64, n_out: i64) -> Result<i32, DFlashError> {
+                      n_in: i64, n_out: i64) -> Result<sys::dflash_qtensor, DFlashError> {
     let rc = unsafe { sys::dflash_check_scale_range(base.ctx, type_, blocks, n_blocks, ptr::null_mut(), base.stream) };
     check(base.ctx, rc, -1)?;
+    let flags = if type_ == 12 || type_ == 14 { sys::DFLASH_QT_RANGE_CHECKED } else { 0 };
     if let (12, Some(dst)) = (type_, tiled_dst) {
         debug_assert!(unsafe { sys::dflash_q4k_tiled_bytes(n_in, n_out) } > 0);
         let rc = unsafe { sys::dflash_repack_q4k_tiled(base.ctx, blocks, dst, n_in, n_out, base.stream) };
         check(base.ctx, rc, -1)?;
-        return Ok(sys::DFLASH_TYPE_Q4_K_TILED);
+        return Ok(sys::dflash_qtensor { type_: sys::DFLASH_TYPE_Q4_K_TILED, flags, data: dst as *const c_void });
     }
-    Ok(type_)
+    Ok(sys::dflash_qtensor { type_, flags, data: blocks })
 }

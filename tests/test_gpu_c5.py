@@ -254,3 +254,55 @@ def test_generate_on_the_moe_shape_equals_serial_greedy(ctx, weights):
     assert stats["accepted_drafts"] > 0 and stats["spec_steps"] >= 2
     assert dec.session.kv_n_pos == len(prompt) + n_tok - 1
     dec.close()
+
+
+def test_full_depth_generation_equals_serial_greedy(ctx):
+    """The end-to-end configuration at its own size: all 40 layers (15 GB of Q4_K / Q6_K weights generated on the
+    device), the 5-layer drafter fed by three tapped layers, a prompt of 2048 seeded tokens through the pipelined
+    prefill, then 256 tokens by speculative steps with greedy acceptance.  Random-init models never agree, so the
+    number of accepted drafts is forced block by block on the schedule 7, 3, 15, 0, 1 (the target's own serial
+    continuation supplies the first k drafts, wrong tokens the rest; the drafter runs all the same).  Property, which
+    does not depend on the size: every emitted token equals the serial greedy decode through the same kernels, the
+    accept lengths are the forced ones."""
+    import torch
+
+    cfg = dfl.ModelConfig(n_layers=40, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=151936, n_expert=128,
+                          n_expert_used=8, ffn_expert=768, ffn_shared=768)
+    dcfg = dfl.DraftConfig(n_layers=5, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=6144, block_size=16, n_taps=3)
+    taps, prompt_len, n_generate = [1, 19, 38], 2048, 256
+    cap = prompt_len + n_generate + 64
+    target = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_device(cfg, 0, "cuda"))
+    head = dfl.DraftHead(ctx, dcfg, dfl.synth_draft_weights_device(dcfg, 0, "cuda"))
+    prompt = np.random.default_rng(0).integers(0, cfg.vocab - 1, prompt_len).tolist()
+    serial = dfl.Session(ctx, target, cap, taps)
+    body = (prompt_len - 1) // 16 * 16
+    serial.prefill_blocks(prompt[:body], 0, want_hidden=False)
+    out = serial.encode_packed_verify_layer_major(prompt[body:], body, want_hidden=False)
+    cont = [out.argmax_host[-1]]
+    while len(cont) < n_generate + 16:
+        out = serial.encode_packed_verify_layer_major([cont[-1]], prompt_len + len(cont) - 1, want_hidden=False)
+        cont.append(out.argmax_host[0])
+    serial.close()
+
+    schedule, forced = [7, 3, 15, 0, 1], []
+    dec = dfl.SpeculativeDecoder(ctx, target, head, taps, cap, cfg.vocab - 1)
+    first = dec.prefill(prompt)
+    assert first == cont[0]
+
+    def override(tokens, position):
+        k = schedule[len(forced) % len(schedule)]
+        forced.append(k)
+        done = len(tokens)
+        return cont[done:done + k] + [(t + 1) % (cfg.vocab - 1) for t in cont[done + k:done + 15]]
+
+    tokens, st = dec.generate(first, n_generate, draft_override_fn=override)
+    torch.cuda.synchronize()
+    assert n_generate - 16 <= len(tokens) <= n_generate + 16 and tokens == cont[:len(tokens)]
+    # a block accepts exactly its forced drafts (a wrong draft is the target's token + 1, never the target's token),
+    # except the last one, which the token budget may cut short
+    hist = st["accept_len_hist"]
+    want = [0] * 16
+    for k in forced[:-1]:
+        want[k] += 1
+    assert all(h >= w for h, w in zip(hist, want)) and sum(hist) == len(forced)
+    dec.close()

@@ -23,6 +23,11 @@ def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
+def gemm_fast(ctx, w, qtype, x, n_in, n_out):
+    """The few-row GEMM through the fast kernels: the tensor is range-checked first, as a loader must, and tagged."""
+    return ctx.gemm_fewrow(w, ctx.checked_type(qtype, w), x, n_in, n_out)
+
+
 @pytest.mark.parametrize("qtype", QTYPES)
 @pytest.mark.parametrize("kind", ["random", "extreme", "quantised"])
 def test_dequant_bit_exact(ctx, oracle, qtype, kind):
@@ -91,7 +96,7 @@ def test_gemm_fewrow_small_shapes(ctx, oracle, qtype, n_in, n_out, n_rows, x_dty
     if x_dtype == "f16":
         x = x.astype(np.float16)
     ref = f64_reference(oracle, qtype, w, x.astype(np.float32), n_in, n_out)
-    y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+    y = gemm_fast(ctx, dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
     check_gemm(y, ref, f"q{qtype} {n_in}x{n_out}x{n_rows} {x_dtype}")
 
 
@@ -103,7 +108,7 @@ def test_gemm_fewrow_extreme_blocks(ctx, oracle, qtype, canaries):
     w = dfl.synth.extreme_blocks(qtype, nblk, seed=5)
     x = np.random.default_rng(5).standard_normal((n_rows, n_in)).astype(np.float32)
     ref = f64_reference(oracle, qtype, w, x, n_in, n_out)
-    y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+    y = gemm_fast(ctx, dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
     check_gemm(y, ref, f"extreme q{qtype}")
 
 
@@ -113,7 +118,7 @@ def test_gemm_matches_oracle_f32_path(ctx, oracle):
     w = dfl.synth.random_weight(dfl.synth.Q4_K, n_out, n_in, seed=1)
     x = np.random.default_rng(1).standard_normal((n_rows, n_in)).astype(np.float32)
     want = oracle.gemm_fewrow(dfl.synth.Q4_K, w, x, n_in, n_out)
-    got = ctx.gemm_fewrow(dev(w), dfl.synth.Q4_K, dev(x), n_in, n_out).cpu().numpy()
+    got = gemm_fast(ctx, dev(w), dfl.synth.Q4_K, dev(x), n_in, n_out).cpu().numpy()
     rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
     assert np.max(np.abs(got - want) / np.maximum(np.abs(want), rms)) <= 1e-2
 
@@ -127,12 +132,12 @@ def test_gemm_deterministic_and_linear(ctx):
     g = torch.Generator(device="cuda").manual_seed(1)
     x1 = torch.randn((16, n_in), device="cuda", generator=g, dtype=torch.float32).half()
     x2 = torch.randn((16, n_in), device="cuda", generator=g, dtype=torch.float32).half()
-    y1 = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, x1, n_in, n_out)
-    y1b = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, x1, n_in, n_out)
+    y1 = gemm_fast(ctx, w, dfl.TYPE_Q4_K, x1, n_in, n_out)
+    y1b = gemm_fast(ctx, w, dfl.TYPE_Q4_K, x1, n_in, n_out)
     assert torch.equal(y1, y1b)
-    y2 = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, x2, n_in, n_out)
+    y2 = gemm_fast(ctx, w, dfl.TYPE_Q4_K, x2, n_in, n_out)
     xs = (x1.float() + x2.float())
-    ys = ctx.gemm_fewrow(w, dfl.TYPE_Q4_K, xs, n_in, n_out)
+    ys = gemm_fast(ctx, w, dfl.TYPE_Q4_K, xs, n_in, n_out)
     scale = ys.abs().max().item()
     assert (ys - (y1 + y2)).abs().max().item() <= 4e-3 * scale
 
@@ -150,11 +155,11 @@ def test_gemm_small_split_k_repeats(ctx, oracle, qtype, n_in, n_out, canaries):
     g = torch.Generator(device="cuda").manual_seed(2)
     x = torch.randn((16, n_in), device="cuda", generator=g, dtype=torch.float32)
     x2 = torch.randn((16, 2048), device="cuda", generator=g, dtype=torch.float32)
-    first = ctx.gemm_fewrow(w, qtype, x, n_in, n_out).clone()
-    other = ctx.gemm_fewrow(w2, qtype, x2, 2048, 1024).clone()
+    first = gemm_fast(ctx, w, qtype, x, n_in, n_out).clone()
+    other = gemm_fast(ctx, w2, qtype, x2, 2048, 1024).clone()
     for _ in range(20):
-        assert torch.equal(ctx.gemm_fewrow(w, qtype, x, n_in, n_out), first)
-        assert torch.equal(ctx.gemm_fewrow(w2, qtype, x2, 2048, 1024), other)
+        assert torch.equal(gemm_fast(ctx, w, qtype, x, n_in, n_out), first)
+        assert torch.equal(gemm_fast(ctx, w2, qtype, x2, 2048, 1024), other)
     ref = f64_reference(oracle, qtype, w.cpu().numpy(), x.cpu().numpy(), n_in, n_out)
     check_gemm(first.cpu().numpy(), ref, f"split-K {n_in}x{n_out}")
 
@@ -165,7 +170,7 @@ def test_gemm_fewrow_full_size_q4k(ctx, oracle, n_in, n_out):
     sample of output columns against the f64 reference (the oracle takes seconds per 256 rows)"""
     w = dfl.synth.random_weight(dfl.synth.Q4_K, n_out, n_in, seed=1)
     x = np.random.default_rng(1).standard_normal((16, n_in)).astype(np.float16)
-    y = ctx.gemm_fewrow(dev(w), dfl.synth.Q4_K, dev(x), n_in, n_out).cpu().numpy()
+    y = gemm_fast(ctx, dev(w), dfl.synth.Q4_K, dev(x), n_in, n_out).cpu().numpy()
     rows = np.unique(np.concatenate([np.arange(0, 64), np.arange(n_out - 64, n_out),
                                      np.random.default_rng(2).integers(0, n_out, 384)]))
     ref = f64_reference(oracle, dfl.synth.Q4_K, w[rows], x.astype(np.float32), n_in, len(rows))
@@ -210,7 +215,7 @@ def test_gemm_q4k_tiled_order_is_bit_identical(ctx, n_in, n_out, n_rows, x_dtype
     w = dfl.synth.random_blocks(dfl.synth.Q4_K, n_out * n_in // 256, n_in + n_out)
     x = rng.standard_normal((n_rows, n_in)).astype(np.float32 if x_dtype == "f32" else np.float16)
     wd, xd = dev(w), dev(x)
-    want = ctx.gemm_fewrow(wd, dfl.TYPE_Q4_K, xd, n_in, n_out)
+    want = gemm_fast(ctx, wd, dfl.TYPE_Q4_K, xd, n_in, n_out)
     wt = ctx.repack_q4k_tiled(wd, n_in, n_out)
     guard = 64
     buf = torch.full((n_rows * n_out + 2 * guard,), float("nan"), dtype=torch.float32, device="cuda")
@@ -258,7 +263,7 @@ def test_gemm_fewrow_reference_extreme_blocks(ctx, oracle, qtype, canaries):
     w = dfl.synth.reference_extreme_blocks(qtype, nblk)
     x = np.random.default_rng(9).standard_normal((n_rows, n_in)).astype(np.float32)
     ref = f64_reference(oracle, qtype, w, x, n_in, n_out)
-    y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+    y = gemm_fast(ctx, dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
     check_gemm(y, ref, f"reference extreme q{qtype}")
 
 
@@ -282,7 +287,7 @@ def test_scale_range_guard(ctx, oracle):
         w = _with_scales(qtype, nblk, d, dmin)
         md, mm = ctx.check_scale_range(qtype, dev(w), nblk)
         assert md == abs(d) and (dmin is None or mm == abs(dmin))
-        y = ctx.gemm_fewrow(dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
+        y = gemm_fast(ctx, dev(w), qtype, dev(x), n_in, n_out).cpu().numpy()
         assert np.all(np.isfinite(y))
         check_gemm(y, f64_reference(oracle, qtype, w, x, n_in, n_out), f"limit q{qtype} d={d}")
     # beyond them: declined with a message that names the figure
@@ -315,3 +320,64 @@ def test_model_upload_declines_out_of_range_tensor(ctx):
         pytest.skip("synthetic wo is Q8_0: no f16-range limit")
     with pytest.raises(dfl.DFlashError):
         dfl.TargetModel(ctx, cfg, w)
+
+
+def test_model_with_an_untagged_tensor_is_declined(ctx):
+    """The model-level calls use the fast kernels only, so a Q4_K / Q6_K tensor whose descriptor lacks the
+    range-checked flag (a loader that skipped dflash_check_scale_range) is declined by name, before any launch."""
+    cfg = dfl.ModelConfig(n_layers=2, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, vocab=512)
+    model = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights(cfg, seed=3), tiled=False)
+    sess = dfl.Session(ctx, model, 64, [0])
+    try:
+        sess.encode_packed_verify_layer_major([1, 2, 3], 0)  # as uploaded: fine
+        sess.encode_restore_after_partial_accept(0, 3, 0)
+        down = model._layers[1].down
+        if down.type not in (dfl.TYPE_Q4_K, dfl.TYPE_Q6_K):
+            pytest.skip("the synthetic down projection went into the tiled order (checked by construction)")
+        down.flags = 0
+        with pytest.raises(dfl.DFlashError) as e:
+            sess.encode_packed_verify_layer_major([1, 2, 3], 0)
+        assert e.value.kind == "Unsupported" and "down (layer 1)" in str(e.value)
+    finally:
+        sess.close()
+
+
+@pytest.mark.parametrize("qtype", [dfl.synth.Q4_K, dfl.synth.Q6_K])
+@pytest.mark.parametrize("x_dtype", [np.float32, np.float16])
+def test_untagged_tensor_takes_the_f32_kernel_and_any_block(ctx, oracle, qtype, x_dtype, canaries):
+    """The seam's contract (dispatch.rs:365-378; the reference scales in f32 after the MMA,
+    mat_mat_fewrow_gen.metal:437-444): a tensor that nobody range-checked is computed correctly whatever its blocks
+    hold - here super-block scales of +-128 and +-60000, far outside the fast kernels' f16 range - by ggml's f32
+    dequantisation and f32 sums; never infinities with status OK."""
+    n_in, n_out, n_rows = 1024, 77, 13
+    nblk = n_in // 256 * n_out
+    w = dfl.synth.random_blocks(qtype, nblk, 11).copy()
+    off = {dfl.synth.Q4_K: 0, dfl.synth.Q6_K: 208}[qtype]
+    d = np.where(np.arange(nblk) % 3 == 0, 128.0, np.where(np.arange(nblk) % 3 == 1, -60000.0, 0.03)).astype(np.float16)
+    w[:, off:off + 2] = d.view(np.uint8).reshape(nblk, 2)
+    if qtype == dfl.synth.Q4_K:
+        w[:, 2:4] = np.full(nblk, 200.0, np.float16).view(np.uint8).reshape(nblk, 2)
+    wd = dev(w)
+    with pytest.raises(dfl.DFlashError):  # a loader that asks is told; the tag cannot be earned
+        ctx.checked_type(qtype, wd)
+    x = np.random.default_rng(4).standard_normal((n_rows, n_in)).astype(x_dtype)
+    y = ctx.gemm_fewrow(wd, qtype, dev(x), n_in, n_out).cpu().numpy()
+    canaries.check()
+    ref = f64_reference(oracle, qtype, w, x.astype(np.float32), n_in, n_out)
+    assert np.all(np.isfinite(y))
+    assert np.max(np.abs(y - ref)) <= 2e-5 * np.max(np.abs(ref))
+    # and on an ordinary tensor the two paths agree to the fast kernels' f16-operand tolerance
+    w2 = dfl.synth.random_weight(qtype, n_out, n_in, seed=12)
+    w2d = dev(w2)
+    y_safe = ctx.gemm_fewrow(w2d, qtype, dev(x), n_in, n_out).cpu().numpy()
+    y_fast = gemm_fast(ctx, w2d, qtype, dev(x), n_in, n_out).cpu().numpy()
+    check_gemm(y_fast, y_safe.astype(np.float64), "fast against f32 kernel")
+
+
+def test_repack_declines_a_tensor_out_of_range(ctx):
+    """The tiled order goes to the fast kernels unconditionally, so the repack checks the range itself."""
+    n_in, n_out = 512, 256
+    w = _with_scales(dfl.synth.Q4_K, n_in // 256 * n_out, 128.0, 0.5)
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.repack_q4k_tiled(dev(w), n_in, n_out)
+    assert e.value.status == 2

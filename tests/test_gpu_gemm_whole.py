@@ -46,7 +46,7 @@ def upload(ctx, qtype, n_in, n_out, seed, extreme=False):
     wd = dev(blocks)
     if qtype == dfl.synth.Q4_K:
         return ctx.repack_q4k_tiled(wd, n_in, n_out), dfl.TYPE_Q4_K_TILED, blocks, wd
-    return wd, dfl.TYPE_Q6_K, blocks, wd
+    return wd, ctx.checked_type(dfl.TYPE_Q6_K, wd), blocks, wd
 
 
 @pytest.mark.parametrize("qtype", [dfl.synth.Q4_K, dfl.synth.Q6_K])
@@ -99,7 +99,9 @@ def test_shapes_outside_the_path_are_declined(ctx):
     import torch
 
     assert ctx.xf_kind(dfl.TYPE_Q4_K_TILED, 17408, 5120) == dfl.XF_NONE      # more than two stages per wave
-    assert ctx.xf_kind(dfl.TYPE_Q6_K, 2048, 151936) == dfl.XF_NONE           # more than one round of the chip
+    assert ctx.xf_kind(dfl.TYPE_Q6_K | dfl.TYPE_RANGE_CHECKED, 2048, 151936) == dfl.XF_NONE  # more than one round of the chip
+    assert ctx.xf_kind(dfl.TYPE_Q6_K | dfl.TYPE_RANGE_CHECKED, 2048, 2048) == dfl.XF_Q6K
+    assert ctx.xf_kind(dfl.TYPE_Q6_K, 2048, 2048) == dfl.XF_NONE             # not range-checked: these kernels scale in f16
     assert ctx.xf_kind(dfl.TYPE_Q4_K, 2048, 2048) == dfl.XF_NONE             # GGUF row order Q4_K: streaming kernels only
     assert ctx.xf_kind(dfl.TYPE_Q8_0, 2048, 2048) == dfl.XF_NONE
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")

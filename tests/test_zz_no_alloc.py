@@ -18,6 +18,7 @@ def _run_pair(ctx, L, qtype, n_in, n_out, n_rows, seed, x_f16):
     if x_f16:
         x = x.half()
     x_type = dfl.TYPE_F16 if x_f16 else dfl.TYPE_F32
+    qtype = ctx.checked_type(qtype, w)  # the tag of a range-checked tensor: both entry points then take the fast kernels
     want = ctx.gemm_fewrow(w, qtype, x, n_in, n_out)
     got = torch.full((n_rows, n_out), float("nan"), dtype=torch.float32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
