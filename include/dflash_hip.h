@@ -79,12 +79,6 @@ const char *dflash_version(void);
 void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable);
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms_host,
                                  int64_t *launches_host);
-/* Measurement aid (no counterpart in the reference): while on, a split-K Q4_K GEMM call launches its streaming
- * kernel only and leaves Y without the reduction, so that back-to-back launches of that one kernel can be timed
- * between two events of the caller's (an event pair around a single launch adds the dispatch latency, about 2.5 us,
- * to a 15 us kernel).  Results are wrong while it is on. */
-void dflash_ctx_set_stream_kernel_only(dflash_ctx *ctx, int32_t enable);
-
 /* Graph replay of the packed verify (the counterpart of the reference's one command buffer per
  * verify block, encode_packed_verify_layer_major, metal_dflash.rs:10696-10719): a verify shape
  * (model tensors, row count, taps, output pointers) is run launch by launch the first time,
@@ -139,14 +133,6 @@ enum {
 int32_t dflash_check_scale_range(dflash_ctx *ctx, int32_t type, const void *blocks, size_t n_blocks, float *max_abs_host,
                                  dflash_stream_t stream);
 
-/* ---- measurement aid: streaming-read probe ------------------------------------------
- * No counterpart in the reference.  n_launches launches of a kernel that reads `bytes` (multiple of 16) of
- * bufs[k % n_bufs] (16-byte aligned) once with a grid-stride loop of 16-byte loads and stores a word per
- * workgroup into out_words[n_cu].  bench.py times it over the GEMM's own weight buffers (rotating, so that
- * nothing is found in a cache) as the practical ceiling of a read-only stream.  Enqueue-only. */
-int32_t dflash_hbm_read_probe(dflash_ctx *ctx, const void *const *bufs, int32_t n_bufs, size_t bytes, int32_t n_launches,
-                              void *out_words, dflash_stream_t stream);
-
 /* ---- Q4_K weights in tiled order -------------------------------------------------
  * No counterpart in the reference (it streams GGUF row order, loader.rs tensors as mapped): a one-time
  * permutation of whole 144-byte blocks, done when a matrix is uploaded, into the order the M <= 16 GEMM reads it in:
@@ -180,7 +166,11 @@ int32_t dflash_gemm_fewrow(dflash_ctx *ctx, int32_t w_type, const void *w, const
  * the process ends).  Same arguments, guards, kernels and results (bit for bit) as dflash_gemm_fewrow on a
  * GPU of up to 256 compute units; the launch never uses more workgroups than the array has partial-tile
  * sets for.  Shapes beyond DFLASH_NOALLOC_MAX_N_IN / DFLASH_NOALLOC_MAX_N_OUT are refused with
- * DFLASH_ERR_BAD_SHAPE.  Runs on the current device.  All calls on one GPU share that GPU's array: calls
+ * DFLASH_ERR_BAD_SHAPE.  Runs on the CURRENT device (hipSetDevice): `stream` must belong to it, and the scratch
+ * array and compute-unit count used are that device's.  Bit-identity with dflash_gemm_fewrow holds while both use the
+ * same number of workgroups, i.e. with the environment knob DFLASH_GEMM_WGS unset (a debugging aid; the two entry
+ * points cap it differently).  A type tag without DFLASH_TYPE_RANGE_CHECKED takes the f32 kernel, as in
+ * dflash_gemm_fewrow.  All calls on one GPU share that GPU's array: calls
  * on one stream are ordered; calls that overlap in time on the same GPU (several streams or threads) race.
  * Enqueue-only.  dflash_gemm_fewrow_noalloc_error() returns the calling thread's last message. */
 #define DFLASH_NOALLOC_MAX_N_IN 262144
@@ -705,6 +695,25 @@ typedef struct {
 /* layers: caller's array of layer_cap entries; cfg.n_layers of them are filled. */
 int32_t dflash_gguf_open_drafter(dflash_gguf *g, const dflash_target_shape *target, dflash_gguf_draft_head *out,
                                  dflash_gguf_draft_layer *layers, int32_t layer_cap);
+
+/* =====================================================================================================
+ * MEASUREMENT AIDS - not part of the drop-in surface.  No reference seam corresponds to them and no caller of the
+ * engine needs them; bench.py uses them to time one kernel in isolation.  An integration can leave them unbound.
+ * ===================================================================================================== */
+/* While on, a split-K Q4_K GEMM call launches its streaming
+ * kernel only and leaves Y without the reduction, so that back-to-back launches of that one kernel can be timed
+ * between two events of the caller's (an event pair around a single launch adds the dispatch latency, about 2.5 us,
+ * to a 15 us kernel).  Results are wrong while it is on. */
+void dflash_ctx_set_stream_kernel_only(dflash_ctx *ctx, int32_t enable);
+
+
+/* Streaming-read probe: n_launches launches of a kernel that reads `bytes` (multiple of 16) of
+ * bufs[k % n_bufs] (16-byte aligned) once with a grid-stride loop of 16-byte loads and stores a word per
+ * workgroup into out_words[n_cu].  bench.py times it over the GEMM's own weight buffers (rotating, so that
+ * nothing is found in a cache) as the practical ceiling of a read-only stream.  Enqueue-only. */
+int32_t dflash_hbm_read_probe(dflash_ctx *ctx, const void *const *bufs, int32_t n_bufs, size_t bytes, int32_t n_launches,
+                              void *out_words, dflash_stream_t stream);
+
 
 #ifdef __cplusplus
 }

@@ -32,19 +32,30 @@ INSPECTED_SPILLS = {}
 RESOURCE_FLAG = "-Rpass-analysis=kernel-resource-usage"
 
 
-def check_no_scratch(compiler_output: str) -> list:
-    """Names of guarded kernels that the resource-usage remarks report with scratch or spilled VGPRs."""
-    bad, name = [], None
+def check_no_scratch(compiler_output: str, expect=NO_SCRATCH_KERNELS) -> list:
+    """Complaints about the guarded kernels in one compiler run: a kernel that spills VGPRs or has a scratch frame, and
+    - so that the guard cannot pass vacuously when the remark format changes or the flag is dropped - a guarded kernel
+    (of ``expect``) that the resource-usage remarks do not report at all.  The guard covers spills only: a plain
+    register copy of an asm load's output ahead of the hand-placed wait would be the same hazard without a spill, and
+    is what the bit-exact GEMM tests are the backstop for."""
+    bad, name, seen = [], None, set()
     for line in compiler_output.splitlines():
         m = re.search(r"remark: Function Name: (\S+)", line)
         if m:
             name = m.group(1)
+            seen.update(k for k in NO_SCRATCH_KERNELS if k in name)
             continue
+        guarded = name and any(k in name for k in NO_SCRATCH_KERNELS)
         m = re.search(r"remark:\s+VGPRs Spill: (\d+)", line)
-        if m and name and any(k in name for k in NO_SCRATCH_KERNELS):
+        if m and guarded:
             allowed = next((n for frag, n in INSPECTED_SPILLS.items() if frag in name), 0)
             if int(m.group(1)) != allowed:
                 bad.append(f"{name}: {m.group(1)} VGPRs spilled (inspected: {allowed})")
+        m = re.search(r"remark:\s+ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and guarded and int(m.group(1)) != 0 and not any(frag in name for frag in INSPECTED_SPILLS):
+            bad.append(f"{name}: {m.group(1)} bytes of scratch per lane")
+    bad += [f"{k}: no resource-usage remark found (is {RESOURCE_FLAG} still passed, has the remark format changed?)"
+            for k in expect if k not in seen]
     return bad
 
 
@@ -94,7 +105,8 @@ def build(verbose: bool = False) -> str:
             failed = True
             sys.stderr.write(f"hipcc failed for {src}:\n{out}\n")
             continue
-        bad = check_no_scratch(raw)
+        # (the guarded kernels all live in gemm_fewrow.hip: only there is their absence from the remarks a failure)
+        bad = check_no_scratch(raw, NO_SCRATCH_KERNELS if os.path.basename(src) == "gemm_fewrow.hip" else ())
         if bad:
             failed = True
             sys.stderr.write(f"{src}: kernels with loads in flight must not use scratch:\n  " + "\n  ".join(bad) + "\n")

@@ -951,10 +951,47 @@ int32_t dflash_restore(dflash_ctx *ctx, dflash_session *s, int64_t start, int32_
 }
 
 namespace {
+void prefill_pipe_destroy_extras(PrefillPipe *p) {
+    for (auto &x : p->extra) {
+        if (x.join) (void)hipEventDestroy(x.join);
+        if (x.shadow) {  // give it back its own cache before it frees what it owns
+            x.shadow->k_cache = x.own_k;
+            x.shadow->vt_cache = x.own_vt;
+            x.shadow->capacity = x.own_capacity;
+            dflash_session_destroy(x.shadow);
+        }
+        if (x.ctx) dflash_ctx_destroy(x.ctx);  // (the stream belongs to the process-wide pool)
+        x = PrefillPipe::Extra();
+    }
+}
+
+int32_t prefill_pipe_create_lanes(dflash_ctx *ctx, dflash_session *s, PrefillPipe *p);
+
+// The extra lanes of the pipelined prefill.  If one of them cannot be made (device memory), what was made is taken down
+// again and the prefill runs with the owner's lane alone: slower, never failing for that reason.
 int32_t prefill_pipe_create(dflash_ctx *ctx, dflash_session *s) {
     PrefillPipe *p = new (std::nothrow) PrefillPipe();
     if (!p) return dfl_fail(ctx, DFLASH_ERR_HIP, "prefill_blocks: out of host memory");
     s->pipe = p;  // (whatever has been made so far is taken down with the session)
+    if (prefill_pipe_create_lanes(ctx, s, p) != DFLASH_OK) {
+        for (auto &v : p->kv_done) {
+            for (hipEvent_t e : v)
+                if (e) (void)hipEventDestroy(e);
+            v.clear();
+        }
+        if (p->fork) (void)hipEventDestroy(p->fork);
+        p->fork = nullptr;
+        prefill_pipe_destroy_extras(p);
+        p->n_lanes = 1;
+        p->kv_done[0].assign(s->cfg.n_layers, nullptr);
+        for (hipEvent_t &e : p->kv_done[0]) DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        DFL_HIP_CHECK(ctx, hipEventCreateWithFlags(&p->fork, hipEventDisableTiming));
+        p->ready = true;
+    }
+    return DFLASH_OK;
+}
+
+int32_t prefill_pipe_create_lanes(dflash_ctx *ctx, dflash_session *s, PrefillPipe *p) {
     static const int lanes_env = [] {
         const char *v = getenv("DFLASH_PREFILL_LANES");
         return v && *v ? atoi(v) : 4;  // measured on the 35B-A3B shape: 3290 / 4530 / 5160 / 5650 / 5150 / 4870 prompt tokens/s with
@@ -962,7 +999,9 @@ int32_t prefill_pipe_create(dflash_ctx *ctx, dflash_session *s) {
     p->n_lanes = std::max(1, std::min(kMaxPrefillLanes, lanes_env));
     for (int i = 0; i + 1 < p->n_lanes; i++) {
         PrefillPipe::Extra &x = p->extra[i];
-        int32_t rc = dflash_ctx_create(ctx->device, ctx->workspace_bytes, &x.ctx);
+        // A lane's context serves verify blocks only (attention partials, split-K tiles): the default workspace, not the
+        // owner's, which may have been sized for the wide sampler.
+        int32_t rc = dflash_ctx_create(ctx->device, std::min<size_t>(ctx->workspace_bytes, size_t(128) << 20), &x.ctx);
         if (rc) return dfl_fail(ctx, rc, "prefill_blocks: context of lane %d", i + 1);
         if ((rc = dflash_session_create(x.ctx, &s->cfg, 16, s->n_taps, &x.shadow)))
             return dfl_fail(ctx, rc, "prefill_blocks: scratch set of lane %d", i + 1);

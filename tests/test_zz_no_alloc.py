@@ -2,6 +2,8 @@
 through the C ABI with caller-owned buffers only, its output must equal dflash_gemm_fewrow's bit for bit
 (same kernels, same launch shape, same order of the split-K sums), on two calls in a row, the second with
 a smaller input (the fixed scratch array then still holds the first call's partial tiles)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -34,7 +36,22 @@ def test_noalloc_gemm_equals_context_gemm_twice_in_a_row():
     torch.cuda.set_device(0)
     ctx = dfl.Context(0)
     L = dfl.lib()
+    assert "DFLASH_GEMM_WGS" not in os.environ, "bit-identity of the two entry points holds with the workgroup knob unset"
     try:
+        # nothing may be allocated by the entry point itself: a first call (symbol look-up, module load) aside, free
+        # device memory must read the same before and after a call through the C ABI with caller-owned buffers
+        w = torch.from_numpy(dfl.synth.random_weight(dfl.TYPE_Q4_K, 272, 1024, seed=9)).cuda()
+        tag = ctx.checked_type(dfl.TYPE_Q4_K, w)
+        x = torch.zeros((5, 1024), dtype=torch.float32, device="cuda")
+        y = torch.empty((5, 272), dtype=torch.float32, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+        assert L.dflash_gemm_fewrow_noalloc(tag, w.data_ptr(), x.data_ptr(), dfl.TYPE_F32, y.data_ptr(), 1024, 272, 5, stream) == 0
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info(0)[0]
+        for _ in range(3):
+            assert L.dflash_gemm_fewrow_noalloc(tag, w.data_ptr(), x.data_ptr(), dfl.TYPE_F32, y.data_ptr(), 1024, 272, 5, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info(0)[0] == free_before, "the no-allocation entry point allocated device memory"
         # split-K shapes (partial tiles go through the scratch array), larger then smaller, for both streaming kernels
         _run_pair(ctx, L, dfl.TYPE_Q4_K, 5120, 6144, 16, 1, True)
         _run_pair(ctx, L, dfl.TYPE_Q4_K, 1024, 272, 5, 2, False)
