@@ -599,34 +599,36 @@ def main():
         n = max(len(base), int(kernel_footprint // nbytes) + 1)
         return list(base) + [base[0].clone() for _ in range(n - len(base))]
 
-    def kernel_times(sets, wt, kernel_only):
-        """Average time per call over back-to-back calls between two events on the stream they run on (an event pair
-        around every single launch would add the dispatch latency, about 2.5 us, to each).  kernel_only: the split-K
-        reduction launch is switched off meanwhile, so the figure is the streaming kernel alone (Y incomplete); else
-        the whole call, streaming kernel + reduction."""
-        ctx.set_stream_kernel_only(kernel_only)
-        out = []
-        try:
-            for i, w in enumerate(sets):
-                calls = [bound_call(wk, wt, i) for wk in w]
-                for a in calls:
-                    gemm_c(*a)
-                torch.cuda.synchronize()
-                k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                n = max(reps, 3) * len(w)
-                k0.record()
-                for k in range(n):
-                    gemm_c(*calls[k % len(calls)])
-                k1.record()
-                torch.cuda.synchronize()
-                out.append(k0.elapsed_time(k1) / n * 1e3)
-        finally:
-            ctx.set_stream_kernel_only(False)
-        return out
+    n_per_shape = 8 * max(reps, 3)  # the same number of launches for every shape: a trace's average then weighs them equally
+
+    def kernel_times(sets, wt):
+        """Per shape: (the streaming kernel's own duration, the whole call's time), both in microseconds.
+        Kernel: the library's timer slot 5, i.e. the start / stop stamps of that one dispatch (what a kernel trace reports
+        as its duration; an event pair recorded around a launch would add the dispatch latency, about 2.5 us).  Whole
+        call (streaming kernel + split-K reduction): back-to-back calls between two events on the stream they run on."""
+        kern, call = [], []
+        for i, w in enumerate(sets):
+            calls = [bound_call(wk, wt, i) for wk in w]
+            for a in calls:
+                gemm_c(*a)
+            torch.cuda.synchronize()
+            ctx.set_kernel_timing(2)  # stamps on the dispatches; the launches still follow each other without a wait
+            for k in range(n_per_shape):
+                gemm_c(*calls[k % len(calls)])
+            ms, count = ctx.kernel_timing(5)
+            ctx.set_kernel_timing(0)
+            kern.append(ms / max(count, 1) * 1e3)
+            k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            k0.record()
+            for k in range(n_per_shape):
+                gemm_c(*calls[k % len(calls)])
+            k1.record()
+            torch.cuda.synchronize()
+            call.append(k0.elapsed_time(k1) / n_per_shape * 1e3)
+        return kern, call
 
     big = [copies(wd[i], w_bytes[i]) for i in range(len(SHAPES))]
-    tiled_us = kernel_times(big, w_type, True)
-    call_us = kernel_times(big, w_type, False)
+    tiled_us, call_us = kernel_times(big, w_type)
     # a read-only stream over the same buffers with the same launch shape: the practical ceiling of such a kernel
     probe_out = torch.zeros(1024, dtype=torch.int32, device="cuda")
     probe_us = []
@@ -644,7 +646,7 @@ def main():
     del big
     # the same launches on GGUF row order, rotating over as many copies (the same blocks the repack range-checked)
     row_sets = [copies([w], nb_) for w, nb_ in zip(wrow, w_bytes)]
-    row_us = kernel_times(row_sets, dfl.TYPE_Q4_K | dfl.TYPE_RANGE_CHECKED, True)
+    row_us, _ = kernel_times(row_sets, dfl.TYPE_Q4_K | dfl.TYPE_RANGE_CHECKED)
     del row_sets
     per_shape = [{"n_in": n_in, "n_out": n_out, "weight_bytes": nbytes, "kernel_us": us, "GBps": nbytes / (us * 1e-6) / 1e9,
                   "call_us_with_reduction": cus, "row_order_kernel_us": rus, "read_probe_us": pus, "rotating_copies": nk}
@@ -678,9 +680,10 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(),
                      "kernel": "gemm_q4k_tiled_kernel", "bytes_per_launch": k_bytes, "us_per_launch": k_us,
                      "read_probe_GBps": ceiling, "frac_of_read_probe": achieved / ceiling,
-                     "note": "streaming kernel alone, its split-K reduction launch excluded (Y incomplete while timed); every "
-                             "launch streams from HBM (each shape rotates over more than 256 MB of copies); the whole "
-                             "call is shapes[].call_us_with_reduction, the whole step is `value`",
+                     "note": "the streaming kernel's own duration (start / stop stamps of the dispatch, as a kernel trace reports "
+                             "it), mean over the three shapes; its split-K reduction is another kernel; every launch streams "
+                             "from HBM (each shape rotates over more than 256 MB of copies); the whole call is "
+                             "shapes[].call_us_with_reduction, the whole step is `value`",
                      "whole_call_frac": k_bytes / (sum(call_us) / len(call_us) * 1e-6) / 1e9 / HBM_PEAK_GBS},
         "shapes": per_shape,
         "pct_of_hbm_peak": 100.0 * sum(w_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,

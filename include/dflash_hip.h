@@ -75,7 +75,11 @@ const char *dflash_version(void);
 /* Per-kernel GPU timers: enable_phase_timers / maybe_record (metal_dflash.rs:5181-5190, 5622).
  * While enabled, each call brackets its dominant kernel with events on the call's stream and
  * waits for it, accumulating into a slot: 0 few-row GEMM, 1 verify attention, 2 acceptance,
- * 3 argmax/top-k, 4 split-K reduction of the few-row GEMM.  Enabling or disabling clears the slots. */
+ * 3 argmax/top-k, 4 split-K reduction of the few-row GEMM.  enable == 2 instead: nothing waits; the single-matrix
+ * Q4_K streaming kernel (slot 5) and its reduction (slot 6) are dispatched with start / stop stamps of their own - the
+ * duration a kernel trace reports, without the dispatch latency an event pair around a launch includes, and with the
+ * kernels still running back to back - which dflash_ctx_kernel_timing waits for and adds up when it is called.
+ * Changing the mode clears the slots. */
 void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable);
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms_host,
                                  int64_t *launches_host);
@@ -697,16 +701,9 @@ int32_t dflash_gguf_open_drafter(dflash_gguf *g, const dflash_target_shape *targ
                                  dflash_gguf_draft_layer *layers, int32_t layer_cap);
 
 /* =====================================================================================================
- * MEASUREMENT AIDS - not part of the drop-in surface.  No reference seam corresponds to them and no caller of the
- * engine needs them; bench.py uses them to time one kernel in isolation.  An integration can leave them unbound.
+ * MEASUREMENT AID - not part of the drop-in surface.  No reference seam corresponds to it and no caller of the
+ * engine needs them; bench.py uses it to find the ceiling of a read-only stream.  An integration can leave it unbound.
  * ===================================================================================================== */
-/* While on, a split-K Q4_K GEMM call launches its streaming
- * kernel only and leaves Y without the reduction, so that back-to-back launches of that one kernel can be timed
- * between two events of the caller's (an event pair around a single launch adds the dispatch latency, about 2.5 us,
- * to a 15 us kernel).  Results are wrong while it is on. */
-void dflash_ctx_set_stream_kernel_only(dflash_ctx *ctx, int32_t enable);
-
-
 /* Streaming-read probe: n_launches launches of a kernel that reads `bytes` (multiple of 16) of
  * bufs[k % n_bufs] (16-byte aligned) once with a grid-stride loop of 16-byte loads and stores a word per
  * workgroup into out_words[n_cu].  bench.py times it over the GEMM's own weight buffers (rotating, so that

@@ -107,8 +107,6 @@ def _declare(L):
     L.dflash_select_draft_path_sampled.restype = i32
     L.dflash_select_draft_path_sampled.argtypes = [vp, C.POINTER(CodebookC), C.POINTER(CodebookC), i32, i32, i32, i32, vp, vp,
                                                    vp, C.POINTER(SamplerC), vp, vp, C.POINTER(WeightedCandidateC), vp]
-    L.dflash_ctx_set_stream_kernel_only.restype = None
-    L.dflash_ctx_set_stream_kernel_only.argtypes = [vp, i32]
     L.dflash_ctx_set_draft_graphs.restype = None
     L.dflash_ctx_set_draft_graphs.argtypes = [vp, i32]
     L.dflash_ctx_set_graphs.restype = None
@@ -262,16 +260,14 @@ class Context:
     # ---- enable_phase_timers (metal_dflash.rs:5181-5190)
     T_GEMM, T_ATTN, T_ACCEPT, T_ARGMAX, T_REDUCE = 0, 1, 2, 3, 4
 
-    def set_kernel_timing(self, enable: bool):
+    def set_kernel_timing(self, enable):
+        """False / 0: off; True / 1: event pairs around the dominant kernels (each timed launch waits); 2: dispatch stamps
+        of the Q4_K streaming kernel and its reduction (slots 5 and 6), read when kernel_timing() is called."""
         self._lib.dflash_ctx_set_kernel_timing(self._h, int(enable))
 
     def set_draft_graphs(self, enable: bool):
         """Graph replay of the drafter's block forward on or off (off by default; results are the same)."""
         self._lib.dflash_ctx_set_draft_graphs(self._h, int(enable))
-
-    def set_stream_kernel_only(self, enable: bool):
-        """Measurement aid: split-K GEMM calls launch their streaming kernel only (Y incomplete while on)."""
-        self._lib.dflash_ctx_set_stream_kernel_only(self._h, int(enable))
 
     def set_graphs(self, enable: bool):
         """Graph replay of the packed verify on or off (off by default; results are the same)."""

@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <vector>
 
 #include "../../include/dflash_hip.h"
 
@@ -26,9 +27,6 @@ struct dflash_ctx {
     char err[512] = {0};
     // per-kernel timers (off by default; when on, timed launches synchronise)
     bool timing = false;
-    // measurement aid: split-K GEMM calls launch their streaming kernel only (Y is left without its reduction), so
-    // that back-to-back launches of that one kernel can be timed between two events
-    bool stream_kernel_only = false;
     // Set by a caller inside the library for the duration of one few-row GEMM call on a fused gate | up matrix
     // (2 ffn output rows, ffn a multiple of 16): if the call is split over K, its reduction writes
     // silu(gate) * up to swiglu_out[n_rows][ffn] instead of the sums to Y and sets swiglu_done; if it is not (Y is
@@ -36,6 +34,12 @@ struct dflash_ctx {
     float *swiglu_out = nullptr;
     bool swiglu_done = false;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // start / stop stamps of single dispatches (hipExtLaunchKernelGGL), see DFL_T_KERNEL_*: while `stamping` is on, a stamped
+    // launch takes the next event pair of the pool and does not wait; the pairs are read when the timers are queried
+    bool stamping = false;
+    std::vector<hipEvent_t> stamp_events;  // pairs
+    std::vector<int> stamp_slot;           // slot of pair i
+    size_t stamps_used = 0;
     double timed_ms[8] = {0};
     int64_t timed_launches[8] = {0};
     // captured-graph replay of the packed verify: a stream of the library's own to capture on and
@@ -58,9 +62,31 @@ struct dflash_ctx {
 enum { DFL_PINNED_BYTES = 8192 };
 
 // Slots of the per-kernel timers.
-enum { DFL_T_GEMM = 0, DFL_T_ATTN = 1, DFL_T_ACCEPT = 2, DFL_T_ARGMAX = 3, DFL_T_REDUCE = 4 };
+enum { DFL_T_GEMM = 0, DFL_T_ATTN = 1, DFL_T_ACCEPT = 2, DFL_T_ARGMAX = 3, DFL_T_REDUCE = 4,
+       // the tiled Q4_K streaming kernel and its reduction by the device's own start / stop stamps of that one dispatch (what a
+       // kernel trace reports as its duration), not by events recorded around the launch (which add the dispatch latency)
+       DFL_T_KERNEL_Q4K_TILED = 5, DFL_T_KERNEL_Q4K_REDUCE = 6 };
 
 // Brackets the dominant kernel of a call with events on its stream when timing is on.
+// The event pair a stamped launch passes to hipExtLaunchKernelGGL: null pointers while stamping is off.
+struct dfl_stamp {
+    hipEvent_t start = nullptr, stop = nullptr;
+    dfl_stamp(dflash_ctx *ctx, int slot) {
+        if (!ctx->stamping) return;
+        if (ctx->stamps_used * 2 + 2 > ctx->stamp_events.size()) {
+            hipEvent_t a = nullptr, b = nullptr;
+            if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return;
+            ctx->stamp_events.push_back(a);
+            ctx->stamp_events.push_back(b);
+            ctx->stamp_slot.push_back(slot);
+        }
+        start = ctx->stamp_events[2 * ctx->stamps_used];
+        stop = ctx->stamp_events[2 * ctx->stamps_used + 1];
+        ctx->stamp_slot[ctx->stamps_used] = slot;
+        ctx->stamps_used++;
+    }
+};
+
 struct dfl_timed {
     dflash_ctx *ctx;
     hipStream_t st;

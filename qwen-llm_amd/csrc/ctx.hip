@@ -86,6 +86,7 @@ void dflash_ctx_destroy(dflash_ctx *ctx) {
     if (ctx->partials) (void)hipFree(ctx->partials);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    for (hipEvent_t e : ctx->stamp_events) (void)hipEventDestroy(e);
     if (ctx->g_in) (void)hipEventDestroy(ctx->g_in);
     if (ctx->g_out) (void)hipEventDestroy(ctx->g_out);
     if (ctx->gstream) (void)hipStreamDestroy(ctx->gstream);
@@ -95,7 +96,9 @@ void dflash_ctx_destroy(dflash_ctx *ctx) {
 
 void dflash_ctx_set_kernel_timing(dflash_ctx *ctx, int32_t enable) {
     if (!ctx) return;
-    ctx->timing = enable != 0;
+    ctx->timing = enable == 1;
+    ctx->stamping = enable == 2;
+    ctx->stamps_used = 0;
     for (int i = 0; i < 8; i++) {
         ctx->timed_ms[i] = 0.0;
         ctx->timed_launches[i] = 0;
@@ -110,12 +113,20 @@ void dflash_ctx_set_draft_graphs(dflash_ctx *ctx, int32_t enable) {
     if (ctx) ctx->draft_graphs = enable != 0;
 }
 
-void dflash_ctx_set_stream_kernel_only(dflash_ctx *ctx, int32_t enable) {
-    if (ctx) ctx->stream_kernel_only = enable != 0;
-}
-
 int32_t dflash_ctx_kernel_timing(const dflash_ctx *ctx, int32_t slot, double *total_ms, int64_t *launches) {
     if (!ctx || slot < 0 || slot >= 8 || !total_ms || !launches) return DFLASH_ERR_INVALID_INPUT;
+    if (ctx->stamps_used) {  // the stamped dispatches since the last query: wait for them and add their durations up
+        dflash_ctx *c = const_cast<dflash_ctx *>(ctx);
+        (void)hipDeviceSynchronize();
+        for (size_t i = 0; i < c->stamps_used; i++) {
+            float ms = 0.0f;
+            if (hipEventElapsedTime(&ms, c->stamp_events[2 * i], c->stamp_events[2 * i + 1]) == hipSuccess) {
+                c->timed_ms[c->stamp_slot[i]] += ms;
+                c->timed_launches[c->stamp_slot[i]] += 1;
+            }
+        }
+        c->stamps_used = 0;
+    }
     *total_ms = ctx->timed_ms[slot];
     *launches = ctx->timed_launches[slot];
     return DFLASH_OK;

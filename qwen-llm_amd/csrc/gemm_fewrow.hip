@@ -28,6 +28,8 @@
 #include "mfma_unpack.h"
 #include "moe_route.h"
 
+#include <hip/hip_ext.h>
+
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
@@ -2534,7 +2536,7 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
     float *partials = reinterpret_cast<float *>(ctx->partials);
     // a single matrix whose ranges are whole tile groups needs no reduction; a batch always may
     const bool split = (batch ? !batch->whole_groups : groups % n_wg != 0);
-    const bool reduce = split && !ctx->stream_kernel_only;
+    const bool reduce = split;
     // a caller inside the library may ask for the SwiGLU of a fused gate | up product in place of the plain reduction
     float *swiglu_out = batch ? nullptr : ctx->swiglu_out;
     if (swiglu_out) ctx->swiglu_done = false;
@@ -2574,14 +2576,16 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         // weight stages issued ahead of the wait for the activations: two, or one when no range is longer than two
         // stages (measured on the 17.7 MB shape: 11.2 against 12.0 us per call; on the 50 MB shapes 19.1 against 18.7)
         const int k_pre = env_int("DFLASH_Q4K_PRE", (total + n_wg - 1) / n_wg <= 2 ? 1 : 2);
+        // (while stamping is on, a dispatch carries start / stop stamps of its own: the kernel's duration as a trace reports it)
         {
             dfl_timed timer(ctx, st, DFL_T_GEMM);
+            const dfl_stamp sp(ctx, DFL_T_KERNEL_Q4K_TILED);
             if (x_type == DFLASH_TYPE_F32)
-                gemm_q4k_tiled_kernel<float><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const float *>(x), y, partials, no,
-                                                                                           nb, n_rows, groups, bt, k_pre);
+                hipExtLaunchKernelGGL(gemm_q4k_tiled_kernel<float>, dim3(n_wg), dim3(64 * kSlabWaves), kTiledLdsBytes, st, sp.start, sp.stop, 0,
+                                      wb, static_cast<const float *>(x), y, partials, no, nb, n_rows, groups, bt, k_pre);
             else
-                gemm_q4k_tiled_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kTiledLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
-                                                                                              partials, no, nb, n_rows, groups, bt, k_pre);
+                hipExtLaunchKernelGGL(gemm_q4k_tiled_kernel<_Float16>, dim3(n_wg), dim3(64 * kSlabWaves), kTiledLdsBytes, st, sp.start, sp.stop, 0,
+                                      wb, static_cast<const _Float16 *>(x), y, partials, no, nb, n_rows, groups, bt, k_pre);
         }
         if (reduce && swiglu_out) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);
@@ -2589,7 +2593,9 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
             ctx->swiglu_done = true;
         } else if (reduce) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);
-            q4k_reduce_kernel<16><<<groups * 16, 256, 0, st>>>(partials, y, no, nb, n_rows, groups, n_wg, bt);
+            const dfl_stamp sp(ctx, DFL_T_KERNEL_Q4K_REDUCE);
+            hipExtLaunchKernelGGL(q4k_reduce_kernel<16>, dim3(groups * 16), dim3(256), 0, st, sp.start, sp.stop, 0, partials, y, no, nb, n_rows,
+                                  groups, n_wg, bt);
         }
     } else if (slab) {
         const void *fn = x_type == DFLASH_TYPE_F32 ? reinterpret_cast<const void *>(gemm_q4k_slab_kernel<float>)
@@ -2597,12 +2603,13 @@ int32_t launch_q4k(dflash_ctx *ctx, const void *w, const void *x, int32_t x_type
         if (const int32_t rc_ = dfl_raise_lds_limit(ctx, fn, kSlabLdsBytes)) return rc_;
         {
             dfl_timed timer(ctx, st, DFL_T_GEMM);
+            const dfl_stamp sp(ctx, DFL_T_KERNEL_Q4K_TILED);  // (the same slot as the tiled kernel: one of the two runs)
             if (x_type == DFLASH_TYPE_F32)
-                gemm_q4k_slab_kernel<float><<<n_wg, 64 * kSlabWaves, kSlabLdsBytes, st>>>(wb, static_cast<const float *>(x), y, partials, no,
-                                                                                         nb, n_rows, groups, bt);
+                hipExtLaunchKernelGGL(gemm_q4k_slab_kernel<float>, dim3(n_wg), dim3(64 * kSlabWaves), kSlabLdsBytes, st, sp.start, sp.stop, 0, wb,
+                                      static_cast<const float *>(x), y, partials, no, nb, n_rows, groups, bt);
             else
-                gemm_q4k_slab_kernel<_Float16><<<n_wg, 64 * kSlabWaves, kSlabLdsBytes, st>>>(wb, static_cast<const _Float16 *>(x), y,
-                                                                                            partials, no, nb, n_rows, groups, bt);
+                hipExtLaunchKernelGGL(gemm_q4k_slab_kernel<_Float16>, dim3(n_wg), dim3(64 * kSlabWaves), kSlabLdsBytes, st, sp.start, sp.stop, 0, wb,
+                                      static_cast<const _Float16 *>(x), y, partials, no, nb, n_rows, groups, bt);
         }
         if (reduce && swiglu_out) {
             dfl_timed timer(ctx, st, DFL_T_REDUCE);
