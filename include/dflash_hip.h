@@ -630,8 +630,15 @@ float dflash_verify_fallback_margin(int64_t n_pos);
  * lengths capped (:1303-1316), keys and tensor names unique, 1..4 dimensions, no zero or oversized
  * dimension, offsets aligned to general.alignment (default 32, at most 65536), every tensor inside
  * the file, no two tensors overlapping (:840-940).  Tensor bytes are NOT copied: data_host points
- * into the mapping and stays valid until dflash_gguf_close.  Split (multi-shard) files are not
- * read.  A failed call leaves its message in dflash_gguf_last_error (for open: in `err`). */
+ * into the mapping and stays valid until dflash_gguf_close.  A failed call leaves its message in
+ * dflash_gguf_last_error (for open: in `err`).
+ * Split models (GgufFile::open, gguf.rs:154-228, :954-1095): a file whose split.count exceeds 1 must be
+ * shard 0 (split.no = 0), carry split.tensors.count, and be named <prefix>-00001-of-<count, 5 digits>.gguf;
+ * its siblings <prefix>-0000N-of-... are opened beside it (at most 1024), each checked for its own
+ * split.no, the same split.count and, when present, the same split.tensors.count.  The handle then
+ * holds the first shard's metadata and the tensors of all shards in shard order; a name may appear in
+ * one shard only and the merged table must hold exactly the declared number of tensors.
+ * dflash_gguf_alignment / dflash_gguf_data_start describe the first shard. */
 typedef struct dflash_gguf dflash_gguf;
 
 typedef struct {
@@ -646,6 +653,7 @@ int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *err, size_t 
 void dflash_gguf_close(dflash_gguf *g);
 const char *dflash_gguf_last_error(const dflash_gguf *g);
 int64_t dflash_gguf_tensor_count(const dflash_gguf *g);
+int64_t dflash_gguf_shard_count(const dflash_gguf *g); /* GgufFile::shard_count: 1 for a single file */
 int64_t dflash_gguf_kv_count(const dflash_gguf *g);
 uint64_t dflash_gguf_alignment(const dflash_gguf *g);
 uint64_t dflash_gguf_data_start(const dflash_gguf *g); /* file offset of the tensor data */

@@ -1,9 +1,10 @@
 // GGUF v3 reader and DFlash drafter loader (host only; no device code in this file).
 //
-// Follows GgufFile (crates/qwen-llm/src/gguf.rs:129-740, layout and validation :790-940, :1303-1600)
-// and open_dflash_drafter_for_target (crates/qwen-llm/src/loader.rs:832-1290).  The file is mapped
-// read-only; every read of the header is bounds-checked against the mapping; tensor bytes are never
-// copied (callers upload straight from the mapping).
+// Follows GgufFile (crates/qwen-llm/src/gguf.rs:129-740, layout and validation :790-940, :1303-1600,
+// split files :154-228 and :954-1095) and open_dflash_drafter_for_target
+// (crates/qwen-llm/src/loader.rs:832-1290).  Each file is mapped read-only; every read of a header is
+// bounds-checked against its mapping; tensor bytes are never copied (callers upload straight from the
+// mapping).  A split model is one handle: the first shard's metadata, the tensors of every shard.
 #include <fcntl.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -29,6 +30,7 @@ constexpr uint64_t kDefaultAlignment = 32, kMaxAlignment = 65536;
 constexpr uint64_t kMaxTensors = 1000000, kMaxKv = 1000000, kMaxKeyLen = 1024, kMaxTensorNameLen = 64;
 constexpr uint64_t kMaxStringLen = 100ull << 20, kMaxArrayLen = 10000000, kMaxDimension = 1ull << 30;
 constexpr uint64_t kMaxElements = 1ull << 40;
+constexpr uint64_t kMaxSplits = 1024;  // gguf.rs:42
 // loader caps (loader.rs:104-107)
 constexpr uint32_t kMaxArchLayers = 4096, kMaxArchDim = 1u << 20, kMaxBlockSize = 4096;
 constexpr uint64_t kMaxKernelDim = 1ull << 20;
@@ -80,6 +82,7 @@ struct dflash_gguf {
     std::unordered_map<std::string, Value> kv;
     std::vector<Tensor> tensors;
     std::unordered_map<std::string, size_t> by_name;
+    std::vector<dflash_gguf *> more;  // shards 1.. of a split model (their tensors are merged into `tensors`)
     mutable std::string err;
 };
 
@@ -357,20 +360,15 @@ const Value *find_kv(const dflash_gguf *g, const char *key) {
 
 }  // namespace
 
-extern "C" int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *err, size_t err_cap) {
-    auto say = [&](const std::string &m) {
-        if (err && err_cap) snprintf(err, err_cap, "%s", m.c_str());
-    };
-    if (out) *out = nullptr;
-    if (!path || !out) {
-        say("null argument");
-        return DFLASH_ERR_INVALID_INPUT;
-    }
+namespace {
+
+// Maps and parses one file.  On failure the message is in *msg and nothing stays open.
+int32_t open_one(const char *path, dflash_gguf **out, std::string *msg) {
     dflash_gguf *g = new dflash_gguf();
     g->fd = open(path, O_RDONLY | O_CLOEXEC);
     struct stat st;
     if (g->fd < 0 || fstat(g->fd, &st) != 0 || !S_ISREG(st.st_mode)) {
-        say(std::string("cannot open ") + path + ": " + (g->fd < 0 ? strerror(errno) : "not a regular file"));
+        *msg = std::string("cannot open ") + path + ": " + (g->fd < 0 ? strerror(errno) : "not a regular file");
         dflash_gguf_close(g);
         return DFLASH_ERR_IO;
     }
@@ -378,7 +376,7 @@ extern "C" int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *e
     if (g->size) {
         void *m = mmap(nullptr, g->size, PROT_READ, MAP_PRIVATE, g->fd, 0);
         if (m == MAP_FAILED) {
-            say(std::string("mmap failed: ") + strerror(errno));
+            *msg = std::string("mmap failed: ") + strerror(errno);
             g->map = nullptr;
             dflash_gguf_close(g);
             return DFLASH_ERR_IO;
@@ -388,11 +386,110 @@ extern "C" int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *e
     int32_t rc;
     try {
         rc = parse(g);
-    } catch (const std::exception &e) {  // allocation failure: nothing may cross the C boundary
+    } catch (const std::exception &e) {  // allocation failure while building the tables
         rc = fail(g, DFLASH_ERR_IO, "out of memory while reading the header (%s)", e.what());
     }
     if (rc) {
-        say(g->err);
+        *msg = g->err;
+        dflash_gguf_close(g);
+        return rc;
+    }
+    *out = g;
+    return DFLASH_OK;
+}
+
+bool kv_u64(const dflash_gguf *g, const char *key, uint64_t *out) {
+    const Value *v = find_kv(g, key);
+    return v && int_as_u64(g, v->type, v->at, out);
+}
+
+std::string split_suffix(uint64_t no, uint64_t count) {  // gguf.rs:985: shard numbers in names are 1-based
+    char buf[64];
+    snprintf(buf, sizeof(buf), "-%05llu-of-%05llu.gguf", static_cast<unsigned long long>(no + 1), static_cast<unsigned long long>(count));
+    return buf;
+}
+
+std::string fmt(const char *f, ...) {
+    char buf[768];
+    va_list ap;
+    va_start(ap, f);
+    vsnprintf(buf, sizeof(buf), f, ap);
+    va_end(ap);
+    return buf;
+}
+
+// The rest of a split model, `first` being its shard 0 (GgufFile::open, gguf.rs:154-228): the siblings are named
+// by the first file's own suffix; each must carry its own number, the same count and (when present) the same
+// total; tensors are appended shard by shard, never past the declared total, and a name may appear once.
+int32_t open_split(dflash_gguf *first, const char *path, uint64_t count, std::string *msg) {
+    using ull = unsigned long long;
+    if (count > kMaxSplits) return *msg = fmt("split.count %llu in %s exceeds cap %llu", (ull)count, path, (ull)kMaxSplits), DFLASH_ERR_FORMAT;
+    uint64_t no = 0, total = 0;
+    if (!kv_u64(first, "split.no", &no)) return *msg = fmt("missing \"split.no\" in split GGUF %s", path), DFLASH_ERR_FORMAT;
+    if (no != 0)
+        return *msg = fmt("illegal split file idx %llu (file: %s), model must be loaded with the first split", (ull)no, path), DFLASH_ERR_FORMAT;
+    if (!kv_u64(first, "split.tensors.count", &total))
+        return *msg = fmt("missing \"split.tensors.count\" in split GGUF %s", path), DFLASH_ERR_FORMAT;
+    if (total > kMaxTensors) return *msg = fmt("split.tensors.count %llu in %s exceeds cap %llu", (ull)total, path, (ull)kMaxTensors), DFLASH_ERR_FORMAT;
+    const std::string p(path), suffix = split_suffix(0, count);
+    if (p.size() < suffix.size() || p.compare(p.size() - suffix.size(), suffix.size(), suffix) != 0)
+        return *msg = fmt("invalid split file name: %s (expected suffix \"%s\")", path, suffix.c_str()), DFLASH_ERR_FORMAT;
+    const std::string prefix = p.substr(0, p.size() - suffix.size());
+    if (prefix.empty()) return *msg = fmt("invalid split file: %s", path), DFLASH_ERR_FORMAT;
+    if (first->tensors.size() > total)
+        return *msg = fmt("split shards declare %llu tensors but at least %zu were found", (ull)total, first->tensors.size()), DFLASH_ERR_FORMAT;
+    for (uint64_t idx = 1; idx < count; idx++) {
+        const std::string sp = prefix + split_suffix(idx, count);
+        dflash_gguf *s = nullptr;
+        if (const int32_t rc = open_one(sp.c_str(), &s, msg)) return rc;
+        first->more.push_back(s);  // owned from here on: closed with `first`
+        uint64_t got = 0;
+        if (!kv_u64(s, "split.no", &got)) return *msg = fmt("missing \"split.no\" in GGUF split %s", sp.c_str()), DFLASH_ERR_FORMAT;
+        if (got != idx) return *msg = fmt("invalid split file idx: %llu (file: %s), expected %llu", (ull)got, sp.c_str(), (ull)idx), DFLASH_ERR_FORMAT;
+        if (!kv_u64(s, "split.count", &got)) return *msg = fmt("missing \"split.count\" in GGUF split %s", sp.c_str()), DFLASH_ERR_FORMAT;
+        if (got > kMaxSplits) return *msg = fmt("split.count %llu in %s exceeds cap %llu", (ull)got, sp.c_str(), (ull)kMaxSplits), DFLASH_ERR_FORMAT;
+        if (got != count) return *msg = fmt("invalid split count: %llu (file: %s), expected %llu", (ull)got, sp.c_str(), (ull)count), DFLASH_ERR_FORMAT;
+        if (find_kv(s, "split.tensors.count") && kv_u64(s, "split.tensors.count", &got)) {
+            if (got > kMaxTensors) return *msg = fmt("split.tensors.count %llu in %s exceeds cap %llu", (ull)got, sp.c_str(), (ull)kMaxTensors), DFLASH_ERR_FORMAT;
+            if (got != total) return *msg = fmt("invalid split tensor count: %llu (file: %s), expected %llu", (ull)got, sp.c_str(), (ull)total), DFLASH_ERR_FORMAT;
+        }
+        if (first->tensors.size() + s->tensors.size() > total)
+            return *msg = fmt("split shards declare %llu tensors but at least %zu were found", (ull)total, first->tensors.size() + s->tensors.size()), DFLASH_ERR_FORMAT;
+        for (const Tensor &t : s->tensors) {
+            if (!first->by_name.emplace(t.name, first->tensors.size()).second)
+                return *msg = fmt("invalid model: tensor \"%s\" is duplicated across GGUF splits", t.name.c_str()), DFLASH_ERR_FORMAT;
+            first->tensors.push_back(t);  // data_host points into the sibling's mapping, which lives as long as `first`
+        }
+    }
+    if (first->tensors.size() != total)
+        return *msg = fmt("corrupted split model: %llu tensors expected but %zu found", (ull)total, first->tensors.size()), DFLASH_ERR_FORMAT;
+    return DFLASH_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *err, size_t err_cap) {
+    auto say = [&](const std::string &m) {
+        if (err && err_cap) snprintf(err, err_cap, "%s", m.c_str());
+    };
+    if (out) *out = nullptr;
+    if (!path || !out) {
+        say("null argument");
+        return DFLASH_ERR_INVALID_INPUT;
+    }
+    dflash_gguf *g = nullptr;
+    std::string msg;
+    int32_t rc;
+    try {
+        rc = open_one(path, &g, &msg);
+        uint64_t count = 0;
+        if (!rc && kv_u64(g, "split.count", &count) && count > 1) rc = open_split(g, path, count, &msg);
+    } catch (const std::exception &e) {  // allocation failure: nothing may cross the C boundary
+        rc = DFLASH_ERR_IO;
+        msg = std::string("out of memory while reading the header (") + e.what() + ")";
+    }
+    if (rc) {
+        say(msg);
         dflash_gguf_close(g);
         return rc;
     }
@@ -402,11 +499,13 @@ extern "C" int32_t dflash_gguf_open(const char *path, dflash_gguf **out, char *e
 
 extern "C" void dflash_gguf_close(dflash_gguf *g) {
     if (!g) return;
+    for (dflash_gguf *s : g->more) dflash_gguf_close(s);
     if (g->map) munmap(const_cast<uint8_t *>(g->map), g->size);
     if (g->fd >= 0) close(g->fd);
     delete g;
 }
 
+extern "C" int64_t dflash_gguf_shard_count(const dflash_gguf *g) { return g ? static_cast<int64_t>(1 + g->more.size()) : 0; }
 extern "C" const char *dflash_gguf_last_error(const dflash_gguf *g) { return g ? g->err.c_str() : "null handle"; }
 extern "C" int64_t dflash_gguf_tensor_count(const dflash_gguf *g) { return g ? static_cast<int64_t>(g->tensors.size()) : 0; }
 extern "C" int64_t dflash_gguf_kv_count(const dflash_gguf *g) { return g ? static_cast<int64_t>(g->kv.size()) : 0; }

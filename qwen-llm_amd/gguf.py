@@ -62,6 +62,7 @@ def gguf_lib():
         for name, res, args in (
                 ("dflash_gguf_open", i32, [cp, C.POINTER(vp), cp, C.c_size_t]), ("dflash_gguf_close", None, [vp]),
                 ("dflash_gguf_last_error", cp, [vp]), ("dflash_gguf_tensor_count", i64, [vp]),
+                ("dflash_gguf_shard_count", i64, [vp]),
                 ("dflash_gguf_kv_count", i64, [vp]), ("dflash_gguf_alignment", u64, [vp]),
                 ("dflash_gguf_data_start", u64, [vp]),
                 ("dflash_gguf_tensor_at", i32, [vp, i64, C.POINTER(cp), tp]), ("dflash_gguf_find", i32, [vp, cp, tp]),
@@ -104,7 +105,8 @@ class GgufTensor:
 
 
 class GgufFile:
-    """GgufFile::open (gguf.rs:154): a validated read-only mapping of one GGUF v3 file."""
+    """GgufFile::open (gguf.rs:154): a validated read-only mapping of one GGUF v3 file, or of all shards of a split
+    model opened by its first shard (the metadata is the first shard's, the tensor table every shard's)."""
 
     def __init__(self, path: str):
         self._L = gguf_lib()
@@ -136,6 +138,10 @@ class GgufFile:
     @property
     def tensor_count(self) -> int:
         return int(self._L.dflash_gguf_tensor_count(self._h))
+
+    @property
+    def shard_count(self) -> int:
+        return int(self._L.dflash_gguf_shard_count(self._h))
 
     @property
     def kv_count(self) -> int:
@@ -411,6 +417,25 @@ def write_gguf(path, metadata: dict, tensors: dict, alignment: int = 32, version
             end = start + off
             f.seek(0, 2)
             f.write(b"\0" * (end - f.tell()))
+
+
+def split_path(prefix, no: int, count: int) -> str:
+    """File name of shard ``no`` (0-based) of ``count`` (split_suffix, gguf.rs:985: numbers in names start at 1)."""
+    return f"{prefix}-{no + 1:05d}-of-{count:05d}.gguf"
+
+
+def write_split_gguf(prefix, metadata: dict, shards: list, alignment: int = 32) -> list:
+    """Writes a split model: ``shards`` is one tensor dictionary per file.  Every shard carries split.no (u16),
+    split.count (u16) and split.tensors.count (i32) as converters write them; the model's own metadata goes into
+    the first shard only.  Returns the paths, first shard first."""
+    total = sum(len(t) for t in shards)
+    paths = []
+    for no, tensors in enumerate(shards):
+        md = dict(metadata) if no == 0 else {}
+        md.update({"split.no": (_U16, no), "split.count": (_U16, len(shards)), "split.tensors.count": (_I32, total)})
+        paths.append(split_path(prefix, no, len(shards)))
+        write_gguf(paths[-1], md, tensors, alignment=alignment)
+    return paths
 
 
 def _mat_entry(pair, n_in, rows_shape):

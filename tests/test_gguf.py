@@ -300,3 +300,150 @@ def test_target_file_round_trip_dense_and_moe(tmp_path):
         with pytest.raises(dfl.DFlashError) as e:
             dfl.open_target(g)
         assert "unsupported architecture" in str(e.value)
+
+
+# ---- split (multi-shard) models: the cases of the reference's own tests (gguf.rs:2223-2640) ----
+
+def split_shard(path, no, count, total, tensors, extra=None):
+    md = dict(extra or {})
+    md.update({"split.no": (G._U16, no), "split.count": (G._U16, count), "split.tensors.count": (G._I32, total)})
+    G.write_gguf(path, md, tensors)
+
+
+def one(v):
+    return np.full(1, v, np.float32)
+
+
+def expect_split_error(path, status, fragment):
+    with pytest.raises(dfl.DFlashError) as e:
+        dfl.GgufFile(path)
+    assert e.value.status == status and fragment in str(e.value), str(e.value)
+
+
+def test_split_model_opens_from_its_first_shard(tmp_path):
+    """opens_split_gguf_from_first_shard (gguf.rs:2223): two shards, one tensor each at the same shard-local offset."""
+    first, second = tmp_path / "model-00001-of-00002.gguf", tmp_path / "model-00002-of-00002.gguf"
+    split_shard(first, 0, 2, 2, {"a": one(1.0)}, {"general.architecture": "qwen35"})
+    split_shard(second, 1, 2, 2, {"b": one(2.0)}, {"general.architecture": "other"})
+    with dfl.GgufFile(first) as g:
+        assert g.shard_count == 2 and g.tensor_count == 2
+        assert [t.name for t in g.tensors()] == ["a", "b"]            # shard order
+        assert g.find("a").f32()[0] == 1.0 and g.find("b").f32()[0] == 2.0
+        assert g.architecture() == "qwen35"                             # the first shard's metadata is the model's
+
+
+def test_write_split_gguf_round_trip(tmp_path):
+    rng = np.random.default_rng(0)
+    shards = [{"a": rng.standard_normal((3, 8)).astype(np.float32)}, {},
+              {"b": rng.standard_normal(64).astype(np.float32), "c": one(7.0)}]
+    paths = G.write_split_gguf(tmp_path / "m", {"general.architecture": "qwen35moe", "k": 5}, shards)
+    assert [p.rsplit("/", 1)[1] for p in paths] == ["m-00001-of-00003.gguf", "m-00002-of-00003.gguf", "m-00003-of-00003.gguf"]
+    with dfl.GgufFile(paths[0]) as g:
+        assert g.shard_count == 3 and g.tensor_count == 3 and g.get_u64("k") == 5
+        for sh in shards:
+            for name, a in sh.items():
+                assert np.array_equal(g.find(name).f32(), a)
+    # a single file reports one shard
+    G.write_gguf(tmp_path / "single.gguf", {"split.count": (G._U16, 1)}, {"a": one(1.0)})
+    with dfl.GgufFile(tmp_path / "single.gguf") as g:
+        assert g.shard_count == 1 and g.tensor_count == 1
+
+
+def test_split_model_with_unpadded_empty_first_shard(tmp_path):
+    """opens_split_gguf_with_unpadded_empty_first_shard (gguf.rs:2323): a metadata-only first shard may end at its header."""
+    first, second = tmp_path / "model-00001-of-00002.gguf", tmp_path / "model-00002-of-00002.gguf"
+    kv = (s(b"split.no") + struct.pack("<IH", 2, 0) + s(b"split.count") + struct.pack("<IH", 2, 2) +
+          s(b"split.tensors.count") + struct.pack("<Ii", 5, 1))
+    first.write_bytes(header(0, 3) + kv)
+    split_shard(second, 1, 2, 1, {"only": one(3.0)})
+    with dfl.GgufFile(first) as g:
+        assert g.shard_count == 2 and g.tensor_count == 1 and g.find("only").f32()[0] == 3.0
+
+
+def test_split_model_rejections(tmp_path, monkeypatch):
+    a, b = {"a": one(1.0)}, {"b": one(2.0)}
+
+    def pair(name):
+        d = tmp_path / name
+        d.mkdir()
+        return d / "model-00001-of-00002.gguf", d / "model-00002-of-00002.gguf"
+
+    # rejects_opening_nonfirst_split (:2375)
+    first, second = pair("nonfirst")
+    split_shard(second, 1, 2, 2, b)
+    expect_split_error(second, 12, "must be loaded with the first split")
+    # rejects_missing_split_sibling (:2395): an I/O error, not a format error
+    first, second = pair("missing")
+    split_shard(first, 0, 2, 2, a)
+    expect_split_error(first, 11, "cannot open")
+    # rejects_bad_split_suffix (:2415)
+    split_shard(tmp_path / "model.gguf", 0, 2, 1, a)
+    expect_split_error(tmp_path / "model.gguf", 12, "invalid split file name")
+    split_shard(tmp_path / "-00001-of-00002.gguf", 0, 2, 1, a)   # a suffix and nothing before it
+    monkeypatch.chdir(tmp_path)
+    expect_split_error("-00001-of-00002.gguf", 12, "invalid split file: ")
+    # rejects_wrong_split_no (:2435)
+    first, second = pair("wrong_no")
+    split_shard(first, 0, 2, 2, a)
+    split_shard(second, 0, 2, 2, b)
+    expect_split_error(first, 12, "invalid split file idx: 0")
+    # rejects_wrong_split_count (:2468)
+    first, second = pair("wrong_count")
+    split_shard(first, 0, 2, 2, a)
+    split_shard(second, 1, 3, 2, b)
+    expect_split_error(first, 12, "invalid split count: 3")
+    # a sibling with another total
+    first, second = pair("wrong_total")
+    split_shard(first, 0, 2, 2, a)
+    split_shard(second, 1, 2, 3, b)
+    expect_split_error(first, 12, "invalid split tensor count: 3")
+    # rejects_duplicate_tensor_names_across_splits (:2501)
+    first, second = pair("dup")
+    split_shard(first, 0, 2, 2, a)
+    split_shard(second, 1, 2, 2, a)
+    expect_split_error(first, 12, "duplicated across GGUF splits")
+    # rejects_split_tensor_count_mismatch (:2534): fewer tensors than declared
+    first, second = pair("short")
+    split_shard(first, 0, 2, 3, a)
+    split_shard(second, 1, 2, 3, b)
+    expect_split_error(first, 12, "3 tensors expected but 2 found")
+    # rejects_split_tensor_count_overrun_while_merging (:2567): more than declared, caught before the merge
+    first, second = pair("over")
+    split_shard(first, 0, 2, 1, a)
+    split_shard(second, 1, 2, 1, b)
+    expect_split_error(first, 12, "declare 1 tensors but at least 2")
+    # rejects_absurd_split_count_before_allocating_paths (:2600)
+    G.write_gguf(tmp_path / "absurd-00001-of-02000.gguf", {"split.no": (G._U16, 0), "split.count": (G._U16, 2000),
+                                                          "split.tensors.count": (G._I32, 1)}, a)
+    expect_split_error(tmp_path / "absurd-00001-of-02000.gguf", 12, "exceeds cap 1024")
+    # rejects_absurd_split_tensor_count_before_allocating_table (:2617)
+    G.write_gguf(tmp_path / "big-00001-of-00002.gguf", {"split.no": (G._U16, 0), "split.count": (G._U16, 2),
+                                                       "split.tensors.count": (G._U64, 10 ** 9)}, a)
+    expect_split_error(tmp_path / "big-00001-of-00002.gguf", 12, "split.tensors.count 1000000000")
+    # the first shard without its number or its total
+    G.write_gguf(tmp_path / "nono-00001-of-00002.gguf", {"split.count": (G._U16, 2), "split.tensors.count": (G._I32, 1)}, a)
+    expect_split_error(tmp_path / "nono-00001-of-00002.gguf", 12, 'missing "split.no"')
+    G.write_gguf(tmp_path / "nototal-00001-of-00002.gguf", {"split.count": (G._U16, 2), "split.no": (G._U16, 0)}, a)
+    expect_split_error(tmp_path / "nototal-00001-of-00002.gguf", 12, 'missing "split.tensors.count"')
+
+
+def test_drafter_loads_from_a_split_model(tmp_path):
+    """The loader sees one tensor table whichever shard holds a tensor: a drafter written over three shards reads
+    back the same configuration and weights as from one file."""
+    w = write_drafter(tmp_path / "one.gguf", D2, 2)
+    md = G.draft_head_metadata(D2, IDS, mask_token_id=511, swa_pattern=(False,) * D2.n_layers, convention=2)
+    t = G.draft_head_tensors(D2, w, 2)
+    names = list(t)
+    paths = G.write_split_gguf(tmp_path / "drafter", md, [{n: t[n] for n in names[i::3]} for i in range(3)])
+    with dfl.GgufFile(paths[0]) as g:
+        assert g.shard_count == 3 and g.tensor_count == len(names)
+    cfg1, w1, ids1, mask1 = load(tmp_path / "one.gguf")
+    cfg3, w3, ids3, mask3 = load(paths[0])
+    assert same_cfg(cfg1, cfg3) and ids1 == ids3 and mask1 == mask3
+    for k in w1:
+        if k == "layers":
+            for La, Lb in zip(w1[k], w3[k]):
+                for kk in La:
+                    assert same_weights(La[kk], Lb[kk]), kk
+        else:
+            assert same_weights(w1[k], w3[k]), k
