@@ -105,9 +105,15 @@ template <int HD, typename TQ, int MAXW, int HPW>
 __global__ void __launch_bounds__(64 * MAXW)
     attn_split_kernel(const TQ *__restrict__ q, const _Float16 *__restrict__ k_cache,
                       const _Float16 *__restrict__ vt_cache, float *__restrict__ part_o, float *__restrict__ part_ml,
-                      int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int n_rows, int n_q, int n_kv,
+                      int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int n_rows_total, int n_q, int n_kv,
                       int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window,
-                      int split_stride) {
+                      int split_stride, int64_t part_slots) {
+    // blockIdx.z: which block of sixteen query rows (a prefill group hands over many: block b's rows follow block
+    // b - 1's in q and in the cache, its partial tiles sit part_slots slots further on)
+    const int n_rows = min(16, n_rows_total - 16 * static_cast<int>(blockIdx.z));
+    q += static_cast<int64_t>(blockIdx.z) * 16 * n_q * HD;
+    part_o += static_cast<int64_t>(blockIdx.z) * part_slots * HD;
+    part_ml += static_cast<int64_t>(blockIdx.z) * part_slots * 2;
     constexpr int KS = HD / 32;       // k-steps of the score product
     constexpr int DT = HD / 16;       // 16-dim tiles of the output
     constexpr int CH = HD / 8;        // 16-byte chunks per key row
@@ -125,6 +131,7 @@ __global__ void __launch_bounds__(64 * MAXW)
     const int split = blockIdx.x % split_stride;
     const int head0 = kvh * group + ((blockIdx.x / split_stride) * n_waves + wave) * HPW;  // this wave serves heads head0 .. head0 + HPW - 1
     if (ctx_len_dev) ctx_len = *ctx_len_dev;
+    ctx_len += 16 * static_cast<int64_t>(blockIdx.z);
     const int64_t n_pos = ctx_len + n_rows;
     const int64_t chunk = attn_chunk(n_pos, want, min_chunk);
     if (split * chunk >= n_pos) return;  // the grid is sized for the longest context
@@ -359,9 +366,17 @@ namespace {
 // every eighth split (float4 per dim lane, all loads independent), then the eight are summed in LDS.
 __global__ void __launch_bounds__(256)
     attn_combine_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml, float *__restrict__ out,
-                        int n_rows, int n_q, int hd, int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int want,
-                        int min_chunk, void *__restrict__ out_xf, int out_xf_kind) {
+                        int n_rows_total, int n_q, int hd, int64_t ctx_len, const int32_t *__restrict__ ctx_len_dev, int want,
+                        int min_chunk, void *__restrict__ out_xf, int out_xf_kind, int64_t part_slots, size_t xf_stride) {
+    // blockIdx.z: which block of sixteen rows (see attn_split_kernel); rows past a short last block leave
+    const int n_rows = min(16, n_rows_total - 16 * static_cast<int>(blockIdx.z));
+    if (static_cast<int>(blockIdx.y) >= n_rows) return;
+    part_o += static_cast<int64_t>(blockIdx.z) * part_slots * hd;
+    part_ml += static_cast<int64_t>(blockIdx.z) * part_slots * 2;
+    out += static_cast<int64_t>(blockIdx.z) * 16 * n_q * hd;
+    if (out_xf) out_xf = static_cast<uint8_t *>(out_xf) + blockIdx.z * xf_stride;
     if (ctx_len_dev) ctx_len = *ctx_len_dev;
+    ctx_len += 16 * static_cast<int64_t>(blockIdx.z);
     const int64_t n_pos = ctx_len + n_rows;
     const int64_t chunk = attn_chunk(n_pos, want, min_chunk);
     const int n_splits = static_cast<int>((n_pos + chunk - 1) / chunk);
@@ -450,7 +465,8 @@ __global__ void __launch_bounds__(256) transpose_v_kernel(const _Float16 *__rest
 template <int HD, typename TQ>
 int32_t launch_split(dflash_ctx *ctx, dim3 grid, int threads, hipStream_t st, const void *q, const _Float16 *k, const _Float16 *vt,
                   float *po, float *pml, int64_t ctx_len, const int32_t *ctx_len_dev, int n_rows, int n_q, int n_kv,
-                  int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window, int split_stride) {
+                  int64_t vt_stride, int want, int min_chunk, float scale, int full_block, int64_t window, int split_stride,
+                  int64_t part_slots) {
     const size_t lds = static_cast<size_t>(kAttnBufs) * 2 * (32 * HD / 8) * sizeof(half8_t);
 #define DFL_ATTN_LAUNCH(MAXW, HPW)                                                                                  \
     do {                                                                                                            \
@@ -459,7 +475,7 @@ int32_t launch_split(dflash_ctx *ctx, dim3 grid, int threads, hipStream_t st, co
         attn_split_kernel<HD, TQ, MAXW, HPW><<<grid, threads / HPW, lds, st>>>(static_cast<const TQ *>(q), k, vt, po, pml, \
                                                                               ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
                                                                               vt_stride, want, min_chunk, scale,    \
-                                                                              full_block, window, split_stride);    \
+                                                                              full_block, window, split_stride, part_slots); \
     } while (0)
     // one head per wave: two (HPW = 2) halve the LDS reads per head but measured slower on MI355X
     // (fewer waves to hide the per-stage dependency chain)
@@ -481,24 +497,72 @@ extern "C" int32_t dflash_attn_verify_block(dflash_ctx *ctx, const void *q, int3
                           scale, out, stream, 0, 0, nullptr);
 }
 
+// n_rows_total rows, sixteen to a block (every block in the same bucket of context lengths: the caller's business);
+// max_blocks_out: how many blocks the workspace holds partial tiles for (the caller launches the rest in further runs).
+static int32_t attn_rows(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
+                         int32_t v_layout, int64_t ctx_len, int32_t n_rows_total, int32_t n_q, int32_t n_kv, int32_t head_dim,
+                         int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
+                         int64_t window, const int32_t *ctx_len_dev, void *out_xf, int out_xf_kind, int32_t *blocks_done);
+
 int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
                        int64_t window, const int32_t *ctx_len_dev, void *out_xf, int out_xf_kind) {
     if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (n_rows < 1 || n_rows > 16) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: n_rows %d outside 1..16", n_rows);
+    return attn_rows(ctx, q, q_type, k_cache, v_cache, v_layout, ctx_len, n_rows, n_q, n_kv, head_dim, kv_capacity, scale, out, stream,
+                     full_block, window, ctx_len_dev, out_xf, out_xf_kind, nullptr);
+}
+
+int32_t dfl_attn_blocks(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *vt_cache, int64_t ctx_len,
+                        int32_t n_rows_total, int32_t n_q, int32_t n_kv, int32_t head_dim, int64_t kv_capacity, float scale,
+                        float *out, dflash_stream_t stream, void *out_xf, int out_xf_kind) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (n_rows_total < 1) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: %d rows", n_rows_total);
+    const size_t q_block = static_cast<size_t>(16) * n_q * head_dim;
+    const size_t xf_block = dfl_xf_bytes(static_cast<int64_t>(n_q) * head_dim);
+    const size_t q_el = q_type == DFLASH_TYPE_F16 ? 2 : 4;
+    int32_t done = 0;
+    const int32_t n_blocks = (n_rows_total + 15) / 16;
+    while (done < n_blocks) {
+        // a run: the blocks from `done` on that share its bucket (the split policy is a function of the bucket)
+        const int64_t len0 = ctx_len + 16ll * done;
+        const int64_t bucket = dfl_attn_bucket(len0 + std::min(16, n_rows_total - 16 * done));
+        int32_t run = 1;
+        while (done + run < n_blocks &&
+               dfl_attn_bucket(ctx_len + 16ll * (done + run) + std::min(16, n_rows_total - 16 * (done + run))) == bucket)
+            run++;
+        const int32_t rows = std::min(n_rows_total - 16 * done, 16 * run);
+        int32_t taken = 0;
+        const int32_t rc = attn_rows(ctx, static_cast<const uint8_t *>(q) + done * q_block * q_el, q_type, k_cache, vt_cache, 1, len0, rows,
+                                     n_q, n_kv, head_dim, kv_capacity, scale, out + done * q_block, stream, 0, 0, nullptr,
+                                     out_xf ? static_cast<uint8_t *>(out_xf) + done * xf_block : nullptr, out_xf_kind, &taken);
+        if (rc) return rc;
+        done += taken;
+    }
+    return DFLASH_OK;
+}
+
+static int32_t attn_rows(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *v_cache,
+                         int32_t v_layout, int64_t ctx_len, int32_t n_rows_total, int32_t n_q, int32_t n_kv, int32_t head_dim,
+                         int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
+                         int64_t window, const int32_t *ctx_len_dev, void *out_xf, int out_xf_kind, int32_t *blocks_done) {
+    int32_t n_blocks = (n_rows_total + 15) / 16;
+    const int32_t n_rows = std::min(16, n_rows_total);  // rows of the first block: what the split policy looks at
+    if (n_blocks > 1 && (v_layout != 1 || ctx_len_dev))
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: several blocks need the transposed V cache and a host-side context length");
     if (out_xf && ((n_q * head_dim) % DFL_QK_K || reinterpret_cast<uintptr_t>(out_xf) % 16 ||
                    (out_xf_kind != DFL_XF_Q4K && out_xf_kind != DFL_XF_Q6K)))
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: fragment-order output needs n_q * head_dim %% 256 == 0 and a kind");
     if (!q || !k_cache || !v_cache || !out) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "attn_verify: null pointer");
-    if (n_rows < 1 || n_rows > 16) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: n_rows %d outside 1..16", n_rows);
     if (n_q < 1 || n_kv < 1 || n_q % n_kv || n_q / n_kv > 16)
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "attn_verify: %d query heads over %d KV heads (group must be 1..16)",
                         n_q, n_kv);
     if (head_dim != 64 && head_dim != 128 && head_dim != 256)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: head_dim %d (64, 128, 256 supported)", head_dim);
-    if (ctx_len < 0 || ctx_len + n_rows > kv_capacity)
+    if (ctx_len < 0 || ctx_len + n_rows_total > kv_capacity)
         return dfl_fail(ctx, DFLASH_ERR_STATE, "attn_verify: context %lld + %d rows exceeds the cache capacity %lld",
-                        static_cast<long long>(ctx_len), n_rows, static_cast<long long>(kv_capacity));
+                        static_cast<long long>(ctx_len), n_rows_total, static_cast<long long>(kv_capacity));
     if (q_type != DFLASH_TYPE_F32 && q_type != DFLASH_TYPE_F16)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: queries must be f32 or f16");
     if (v_layout != 0 && v_layout != 1) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "attn_verify: v_layout");
@@ -515,7 +579,8 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     // with ctx_len_dev the context length is read on the device: everything sized here is then sized for the
     // largest context of the bucket
     const int64_t bucket = dfl_attn_bucket(ctx_len + n_rows);
-    const int64_t n_pos = ctx_len_dev ? std::min<int64_t>(kv_capacity, 2 * bucket - 1) : ctx_len + n_rows;
+    // (several blocks: sized for the last one, which sees the most keys)
+    int64_t n_pos = ctx_len_dev ? std::min<int64_t>(kv_capacity, 2 * bucket - 1) : ctx_len + n_rows_total;
 
     // KV splits: enough workgroups to cover the chip once or twice, chunks a multiple of 32 keys and at least
     // min_chunk keys long (a split costs a partial tile per head and row).  The policy is a function of the
@@ -546,13 +611,28 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
     const int n_parts = group / hw;  // workgroups per (chunk, KV head)
     const int want = static_cast<int>((static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv * n_parts - 1) / (n_kv * n_parts));
     // most splits any context up to n_pos can have
-    const int n_splits = ctx_len_dev
-                             ? static_cast<int>(std::min<int64_t>(want, (n_pos + min_chunk - 1) / min_chunk))
-                             : static_cast<int>((n_pos + attn_chunk(n_pos, want, min_chunk) - 1) / attn_chunk(n_pos, want, min_chunk));
+    auto splits_for = [&](int64_t np) {
+        return ctx_len_dev ? static_cast<int>(std::min<int64_t>(want, (np + min_chunk - 1) / min_chunk))
+                           : static_cast<int>((np + attn_chunk(np, want, min_chunk) - 1) / attn_chunk(np, want, min_chunk));
+    };
+    int n_splits = splits_for(n_pos);
+    // several blocks: as many as the workspace has room for partial tiles of (the caller comes back for the rest)
+    const size_t slot_bytes = static_cast<size_t>(n_q) * 16 * (head_dim + 2) * sizeof(float);
+    if (n_blocks > 1) {
+        const size_t room = ctx->workspace_bytes > 4096 ? ctx->workspace_bytes - 4096 : 0;
+        while (n_blocks > 1 && static_cast<size_t>(n_blocks) * n_splits * slot_bytes > room) {
+            n_blocks--;
+            n_rows_total = 16 * n_blocks;
+            n_pos = ctx_len + n_rows_total;
+            n_splits = splits_for(n_pos);
+        }
+    }
+    if (blocks_done) *blocks_done = n_blocks;
+    const int64_t part_slots = static_cast<int64_t>(n_splits) * n_q * 16;
 
     size_t off = 0;
-    float *part_o = dfl_ws_take<float>(ctx, &off, static_cast<size_t>(n_splits) * n_q * 16 * head_dim * sizeof(float));
-    float *part_ml = dfl_ws_take<float>(ctx, &off, static_cast<size_t>(n_splits) * n_q * 16 * 2 * sizeof(float));
+    float *part_o = dfl_ws_take<float>(ctx, &off, static_cast<size_t>(n_blocks) * part_slots * head_dim * sizeof(float));
+    float *part_ml = dfl_ws_take<float>(ctx, &off, static_cast<size_t>(n_blocks) * part_slots * 2 * sizeof(float));
     const _Float16 *vt = static_cast<const _Float16 *>(v_cache);
     int64_t vt_stride = kv_capacity;
     if (v_layout == 0) {
@@ -570,7 +650,7 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 
     if (n_splits > 1024) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "attn_verify: %d KV splits", n_splits);
     const int split_stride = (n_splits + 7) / 8 * 8;
-    const dim3 grid(split_stride * n_parts, n_kv);
+    const dim3 grid(split_stride * n_parts, n_kv, n_blocks);
     const int threads = 64 * hw;
     const _Float16 *k = static_cast<const _Float16 *>(k_cache);
     int32_t rc = DFLASH_OK;
@@ -578,13 +658,13 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
         dfl_timed timer(ctx, st, DFL_T_ATTN);
 #define DFL_ATTN(HD)                                                                                              \
     if (q_type == DFLASH_TYPE_F32)                                                                                \
-        rc = launch_split<HD, float>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, n_kv, \
+        rc = launch_split<HD, float>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows_total, n_q, n_kv, \
                                      vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window,     \
-                                     split_stride);                                                               \
+                                     split_stride, part_slots);                                                   \
     else                                                                                                          \
-        rc = launch_split<HD, _Float16>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows, n_q, \
+        rc = launch_split<HD, _Float16>(ctx, grid, threads, st, q, k, vt, part_o, part_ml, ctx_len, ctx_len_dev, n_rows_total, n_q, \
                                         n_kv, vt_stride, want, static_cast<int>(min_chunk), scale, full_block, window, \
-                                        split_stride)
+                                        split_stride, part_slots)
         if (head_dim == 64) {
             DFL_ATTN(64);
         } else if (head_dim == 128) {
@@ -595,8 +675,9 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
 #undef DFL_ATTN
     }
     if (rc) return rc;
-    attn_combine_kernel<<<dim3(n_q, n_rows), 256, 0, st>>>(part_o, part_ml, out, n_rows, n_q, head_dim, ctx_len, ctx_len_dev, want,
-                                                          static_cast<int>(min_chunk), out_xf, out_xf_kind);
+    attn_combine_kernel<<<dim3(n_q, n_rows, n_blocks), 256, 0, st>>>(part_o, part_ml, out, n_rows_total, n_q, head_dim, ctx_len, ctx_len_dev,
+                                                                    want, static_cast<int>(min_chunk), out_xf, out_xf_kind, part_slots,
+                                                                    dfl_xf_bytes(static_cast<int64_t>(n_q) * head_dim));
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

@@ -186,6 +186,11 @@ __device__ static inline void dfl_xf_store_pair(void *xf, int kind, int m, int i
 int dfl_whole_kind(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out, int64_t pair_ffn);
 int32_t dfl_gemm_whole(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in, int64_t n_out,
                        int32_t n_rows, int64_t pair_ffn, void *y_xf, int y_xf_kind, hipStream_t stream);
+// The same for n_rows_total rows, sixteen to a block (the last one may be shorter): block i's rows are in XF order at
+// xf + i * dfl_xf_bytes(n_in), its result at y + i * 16 * n_out (pair mode: 16 * pair_ffn; y_xf + i * dfl_xf_bytes(pair_ffn)).
+// The weights are read once and stay in registers while the blocks pass; a row's bits are those of dfl_gemm_whole.
+int32_t dfl_gemm_whole_blocks(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in, int64_t n_out,
+                              int32_t n_rows_total, int64_t pair_ffn, void *y_xf, int y_xf_kind, hipStream_t stream);
 
 // dflash_dflash2_conv whose result also goes to y_xf in fragment order (XF; h a multiple of 256), for the whole-K
 // projection that reads it.
@@ -221,13 +226,44 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_l
                     const float *pre_norm_w = nullptr, void *next_xf = nullptr, int next_xf_kind = 0);
 bool dfl_moe_norm_fusable(const dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, int n);
 
+// The same FFN for the rows of several consecutive 16-row blocks at once (a prompt's prefill): the rows are regrouped
+// by expert, so a pass reads every touched expert about once however many blocks there are.  cur holds the layer's
+// normalised input and scratch.sg the rows' shared-expert gates (the norm kernel's work); x_resid += experts(cur),
+// then cur = rms_norm(x_resid) * next_norm_w, also to next_xf (block b of sixteen rows at
+// next_xf + b * next_xf_stride bytes) where next_xf_kind says so.  Every row gets the bits dfl_moe_ffn gives it inside
+// its own block.  Takes layers with tiled Q4_K expert stacks and a shared expert of the experts' shape
+// (dfl_moe_group_fits); scratch of dfl_moe_group_max_slots(cfg, n_rows) slots.  Enqueue only.
+struct dfl_moe_group_scratch {
+    float *logits = nullptr;      // [rows][n_expert]
+    float *sg = nullptr;          // [rows]
+    int32_t *sel_e = nullptr;     // [rows][n_used]
+    float *sel_w = nullptr;       // [rows][n_used]
+    int32_t *pick_pos = nullptr;  // [rows][n_used]: row of eo that holds the pick's output
+    int32_t *ids = nullptr;       // [max_slots]
+    int32_t *n_slots = nullptr;
+    int32_t *slot_rows = nullptr; // [max_slots][16]
+    _Float16 *xg = nullptr;       // [max_slots][16][hidden]
+    _Float16 *act = nullptr;      // [max_slots][16][ffn_expert]
+    float *eo = nullptr;          // [max_slots][16][hidden]
+    int max_slots = 0;
+};
+int dfl_moe_group_max_slots(const dflash_model_cfg &cfg, int n_rows);
+bool dfl_moe_group_fits(const dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, int n_rows);
+int32_t dfl_moe_ffn_group(dflash_ctx *ctx, const dflash_model_cfg &cfg, const dflash_layer &layer, float *x_resid,
+                          float *cur, int n_rows, const dfl_moe_group_scratch &scratch, const float *next_norm_w, void *next_xf,
+                          int next_xf_kind, size_t next_xf_stride, hipStream_t stream);
+
 // Residual add + RMSNorm + shared-expert gate + Q8_0 router product of a mixture-of-experts layer as one launch:
 // cur[n_rows][hidden] = rms_norm(x + add) * norm_w, gate_out[r] = sigmoid(cur[r] . gate_w),
 // logits[n_rows][n_expert] = cur . router_w^T, bit-identical to the norm kernel followed by the few-row GEMM.
 // x is left as it is.  dfl_router_norm_fits: whether the shape is one the kernel takes (hidden a multiple of 256, at
-// most 2048; 1..16 rows); switched off by DFLASH_MOE_FUSED_NORM=0.  Enqueue only.
+// most 2048; every row is a workgroup column of its own, 1..4096 of them); switched off by DFLASH_MOE_FUSED_NORM=0.  Enqueue only.
 bool dfl_router_norm_fits(const dflash_ctx *ctx, int32_t router_type, const void *router_w, int64_t hidden, int32_t n_expert,
                           int32_t n_rows);
+// The router product alone for any number of rows, sixteen to a workgroup row: logits[n_rows][n_expert] = cur . router_w^T
+// with the bits dfl_router_norm (and the few-row GEMM of a Q8_0 router) gives each row.  Same shapes as dfl_router_norm_fits.
+int32_t dfl_router_rows(dflash_ctx *ctx, const void *router_w, const float *cur, float *logits, int64_t hidden, int32_t n_expert,
+                        int32_t n_rows, hipStream_t stream);
 int32_t dfl_router_norm(dflash_ctx *ctx, const void *router_w, const float *x, const float *add, const float *norm_w,
                         const float *gate_w, float eps, float *cur, float *gate_out, float *logits, int64_t hidden,
                         int32_t n_expert, int32_t n_rows, hipStream_t stream);
@@ -251,6 +287,15 @@ int32_t dfl_attn_block(dflash_ctx *ctx, const void *q, int32_t q_type, const voi
                        int32_t v_layout, int64_t ctx_len, int32_t n_rows, int32_t n_q, int32_t n_kv, int32_t head_dim,
                        int64_t kv_capacity, float scale, float *out, dflash_stream_t stream, int32_t full_block,
                        int64_t window, const int32_t *ctx_len_dev, void *out_xf = nullptr, int out_xf_kind = 0);
+
+// Block-causal attention of n_rows_total consecutive query rows, sixteen to a block, each block exactly as
+// dfl_attn_block would run it alone at its own context length (ctx_len + 16 b): the same split of the keys, so the same
+// bits.  Blocks whose context lengths fall in the same bucket go out as one launch pair (as many of them as the
+// workspace has room for partial tiles of).  Transposed V cache; block b's rows at q + 16 b rows, out likewise,
+// out_xf + b * dfl_xf_bytes(n_q * head_dim).  The K/V rows of all the blocks are in the cache already.
+int32_t dfl_attn_blocks(dflash_ctx *ctx, const void *q, int32_t q_type, const void *k_cache, const void *vt_cache, int64_t ctx_len,
+                        int32_t n_rows_total, int32_t n_q, int32_t n_kv, int32_t head_dim, int64_t kv_capacity, float scale,
+                        float *out, dflash_stream_t stream, void *out_xf, int out_xf_kind);
 
 // dflash_gemm_fewrow for a tensor of a model that passed dfl_model_tensors_checked (the fast kernels).
 int32_t dfl_gemm_fewrow_checked(dflash_ctx *ctx, int32_t w_type, const void *w, const void *x, int32_t x_type, float *y,

@@ -539,7 +539,27 @@ __device__ unsigned long long *g_trace2 = nullptr;  // [n_wg][16 waves][4]: cycl
     do {                                                                                                        \
         if (threadIdx.x == 0 && g_trace) g_trace[(blockIdx.x + (bt.pair ? 1024 : 0)) * 16 + (i)] = wall_clock64(); \
     } while (0)
+// the expert kernel's stamps, per wave, kept in scalar registers and written at the end: a gate/up pair launch writes
+// 256 workgroups further on than a down launch
+#define DFL_TRE_DECL unsigned long long tre_[7] = {0, 0, 0, 0, 0, 0, 0}
+#define DFL_TRE(i) tre_[i] = wall_clock64()
+#define DFL_TRE_FLUSH                                                                                                \
+    do {                                                                                                             \
+        if ((threadIdx.x & 63) == 0 && g_trace2) {                                                                   \
+            unsigned long long *o_ = g_trace2 + ((blockIdx.x + (bt.pair ? 256 : 0)) * 16 + (threadIdx.x >> 6)) * 8;   \
+            for (int i_ = 0; i_ < 7; i_++) o_[i_] = tre_[i_];                                                        \
+        }                                                                                                            \
+    } while (0)
 #else
+#define DFL_TRE_DECL \
+    do {             \
+    } while (0)
+#define DFL_TRE_FLUSH \
+    do {              \
+    } while (0)
+#define DFL_TRE(i) \
+    do {           \
+    } while (0)
 #define DFL_TRS(i) \
     do {           \
     } while (0)
@@ -1343,6 +1363,8 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool per_slot_x = bt.x_stride != 0;
+    DFL_TRE_DECL;
+    DFL_TRE(0);
     // ---- activations: items as in gemm_q4k_tiled_kernel (virtual wave v = wave + 16 r: stage v / 8 of the chunk) ----
     typename Q4KX8<XT>::type raw_a[kItems], raw_b[kItems];
     const uint32_t n_in = static_cast<uint32_t>(nb) * DFL_QK_K;
@@ -1416,6 +1438,7 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
         __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
         asm volatile("" : "+v"(ids_window));
     }
+    DFL_TRE(1);
     const int tiles = (n_out + 15) >> 4;
     const int halves = bt.pair ? 2 : 1;
     const int n_chunks = (nb + kExpChunk - 1) / kExpChunk;
@@ -1545,10 +1568,12 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     it_seek();
     for (int t = 0; t < 2; t++)
         if (it_valid) issue();
+    DFL_TRE(2);
     q4k_wait_vm(3 * w_issued);  // the activations are older than every weight load
     convert(0);
     __builtin_amdgcn_s_waitcnt(kWaitLds);
     __builtin_amdgcn_s_barrier();
+    DFL_TRE(3);
     bool x_pending = false;  // activations of the next refill are on their way (issued when w_issued was x_pos)
     int x_pos = 0;
 
@@ -1595,6 +1620,7 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
                     const bool x_younger = x_pending && x_pos > w_done;
                     q4k_wait_vm(3 * (w_issued - 1 - w_done) + (x_younger ? kXInstr : 0));
                     if (!x_younger) x_pending = false;
+                    if (w_done == 0) DFL_TRE(4);
                     const u32x4_t *blk = reinterpret_cast<const u32x4_t *>(my_ring + ring_c * kSlabWavePieces) + n * 9;
                     if (h == 0)
                         q4k_experts_compute(blk, slab + s * kTiledStageX, lane, g, sc_sel, magic, acc0);
@@ -1606,6 +1632,7 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
                 }
             }
         }
+        if (r + 1 == n_rounds) DFL_TRE(5);
         if (hsplit) {  // the up tile crosses to the wave that holds the gate tile
             float4_t *xchg = reinterpret_cast<float4_t *>(reinterpret_cast<uint8_t *>(lds) + kExpRingEnd) + (wave & 7) * 64 + lane;
             if (active && wave >= kW / 2) *xchg = acc1;
@@ -1632,6 +1659,8 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
             }
         }
     }
+    DFL_TRE(6);
+    DFL_TRE_FLUSH;
 }
 
 // ----------------------------------------------------------------------------
@@ -2088,7 +2117,11 @@ constexpr size_t kQ8StagedLds = static_cast<size_t>(kMaxSplit) * 256 * sizeof(fl
 template <typename XT>
 __global__ void __launch_bounds__(64 * kMaxSplit)
     gemm_q8_0_staged_kernel(const uint8_t *__restrict__ w, const XT *__restrict__ x, float *__restrict__ y, int n_out,
-                            int n_steps, size_t row_bytes, int n_rows, int n_split) {
+                            int n_steps, size_t row_bytes, int n_rows_total, int n_split) {
+    // blockIdx.y: which block of sixteen rows (a prefill group hands over many)
+    const int n_rows = min(16, n_rows_total - 16 * static_cast<int>(blockIdx.y));
+    x += static_cast<size_t>(blockIdx.y) * 16 * (static_cast<size_t>(n_steps) * 32);
+    y += static_cast<size_t>(blockIdx.y) * 16 * n_out;
     extern __shared__ __attribute__((aligned(16))) float red[];  // [kMaxSplit][256], then X pieces, then W rows
     half8_t *xs = reinterpret_cast<half8_t *>(red + kMaxSplit * 256);
     uint8_t *ws = reinterpret_cast<uint8_t *>(xs + kQ8XPieces);
@@ -2241,12 +2274,12 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
         rw.q = static_cast<uint64_t>(q16[0]) | (static_cast<uint64_t>(q16[1]) << 16) | (static_cast<uint64_t>(q16[2]) << 32) |
                (static_cast<uint64_t>(q16[3]) << 48);
         const half8_t piece = xrow[4 * st + g];
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(n == r ? piece : zero, convert_raw8<DFLASH_TYPE_Q8_0>(rw), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(n == (r & 15) ? piece : zero, convert_raw8<DFLASH_TYPE_Q8_0>(rw), acc, 0, 0, 0);
     }
-    // output row r sits in lane group r / 4, element r % 4
+    // the row rides in MFMA row r % 16 (any one would do: the other fifteen are zeros): lane group (r % 16) / 4, element r % 4
     const int ri = r & 3;
     const float mine = ri == 0 ? acc[0] : ri == 1 ? acc[1] : ri == 2 ? acc[2] : acc[3];
-    if (g == (r >> 2)) red[wave][n] = mine;
+    if (g == ((r & 15) >> 2)) red[wave][n] = mine;
     __syncthreads();
     if (tid < 16 && n0 + tid < n_out) {
         float sum = 0.0f;
@@ -2704,7 +2737,7 @@ bool dfl_router_norm_fits(const dflash_ctx *ctx, int32_t router_type, const void
     static const bool on = env_int("DFLASH_MOE_FUSED_NORM", 1) != 0;  // read once per process
     // (up to 128 tiles the separate router product runs 16 waves per workgroup as well: same bits)
     return on && router_type == DFLASH_TYPE_Q8_0 && hidden >= 256 && hidden % 256 == 0 && hidden <= 32 * kQ8ChunkSteps &&
-           n_expert >= 1 && (n_expert + 15) / 16 <= 128 && n_rows >= 1 && n_rows <= 16 &&
+           n_expert >= 1 && (n_expert + 15) / 16 <= 128 && n_rows >= 1 && n_rows <= 4096 &&
            reinterpret_cast<uintptr_t>(router_w) % 16 == 0 && ctx->lds_bytes >= 48 * 1024;
 }
 
@@ -2726,6 +2759,22 @@ int32_t dfl_router_norm(dflash_ctx *ctx, const void *router_w, const float *x, c
     q8_0_norm_router_kernel<<<dim3(tiles, n_rows), 64 * kMaxSplit, 0, st>>>(static_cast<const uint8_t *>(router_w), x, add, norm_w, gate_w, eps, cur,
                                                                  gate_out, logits, n_expert, n_steps,
                                                                  static_cast<size_t>(n_steps) * DFL_Q8_0_BYTES);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+int32_t dfl_router_rows(dflash_ctx *ctx, const void *router_w, const float *cur, float *logits, int64_t hidden, int32_t n_expert,
+                        int32_t n_rows, hipStream_t st) {
+    if (!router_w || !cur || !logits || n_rows < 1 || !dfl_router_norm_fits(ctx, DFLASH_TYPE_Q8_0, router_w, hidden, n_expert, 16) ||
+        reinterpret_cast<uintptr_t>(cur) % 16)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "router_rows: hidden %lld / %d experts / %d rows", static_cast<long long>(hidden), n_expert,
+                        n_rows);
+    if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(gemm_q8_0_staged_kernel<float>), kQ8StagedLds)) return rc_;
+    const int n_steps = static_cast<int>(hidden / DFL_QK8_0);
+    dfl_timed timer(ctx, st, DFL_T_GEMM);
+    // sixteen waves split the 64 steps of a row, as the few-row product of a router does for one block
+    gemm_q8_0_staged_kernel<float><<<dim3((n_expert + 15) / 16, (n_rows + 15) / 16), 64 * kMaxSplit, kQ8StagedLds, st>>>(
+        static_cast<const uint8_t *>(router_w), cur, logits, n_expert, n_steps, static_cast<size_t>(n_steps) * DFL_Q8_0_BYTES, n_rows, kMaxSplit);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

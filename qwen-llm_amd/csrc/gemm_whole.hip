@@ -41,6 +41,11 @@ struct WholeArgs {
     int n_units; // plain: ceil(tiles / R) units of R consecutive tiles; pair: ffn / 16 units of (gate tile, up tile)
     int pair_off;  // pair mode: tiles between a gate tile and its up tile; 0 = plain
     uint32_t row_bytes;  // Q6_K (GGUF row order): bytes per weight row
+    // several 16-row blocks against the same weights (a prefill): block i reads xf + i * xf_stride bytes and writes
+    // y + i * y_stride floats (y_xf + i * y_xf_stride bytes); the last block has rows_last rows, the others 16
+    int n_blocks, rows_last;
+    uint32_t xf_stride, y_xf_stride;
+    size_t y_stride;
 };
 
 // ---- Q4_K, tiled order: [tile group of 256 rows][super-block][tile][row][144-byte block] ----
@@ -169,7 +174,8 @@ __device__ __forceinline__ void load_xf(half8_t (&af)[8], const uint8_t *xf, int
 }
 
 // W: Q4W or Q6W.  R: tiles per wave and stage (they share the stage's activation fragments).
-template <typename W, int R>
+// kMulti: several 16-row blocks per launch (a.n_blocks); the single-block instances keep the registers of a kernel without the loop.
+template <typename W, int R, bool kMulti>
 __global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
     // [16 waves][R] partial tiles; Q6_K: then a staging area per wave
     extern __shared__ float4_t red[];
@@ -186,89 +192,103 @@ __global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
 #pragma unroll
     for (int r = 0; r < R; r++) tile[r] = min(a.pair_off ? unit + r * a.pair_off : unit * R + r, n_tiles - 1);
     float4_t acc[R], acc_sub[R];
+    const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
+    const Q4KMagic magic = q4k_magic();
+    uint8_t *area = reinterpret_cast<uint8_t *>(red + 16 * R * 64) + wave * kQ6AreaBytes;
+    // (every load in flight together where the registers hold them; else one tile at a time)
+    constexpr bool kEarly = sizeof(W) * R <= 96;
+    W w0[kEarly ? R : 1], w1[kEarly ? R : 1];
+    if (kEarly && active) {
+        // the weights come from HBM, the activations from L2: weights first; they stay in registers for every block
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = acc_sub[r] = float4_t{0, 0, 0, 0};
-    if (active) {
-        const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
-        const Q4KMagic magic = q4k_magic();
-        uint8_t *area = reinterpret_cast<uint8_t *>(red + 16 * R * 64) + wave * kQ6AreaBytes;
-        half8_t af[8];
-        // (every load in flight together where the registers hold them; else one tile at a time)
-        constexpr bool kEarly = sizeof(W) * R <= 96;
-        if constexpr (kEarly) {
-            W w0[R], w1[R];
-            // the weights come from HBM, the activations from L2: weights first
+        for (int r = 0; r < (kEarly ? R : 1); r++) load_w(w0[r], a, tile[r], b0, lane);
+        if (two) {
 #pragma unroll
-            for (int r = 0; r < R; r++) load_w(w0[r], a, tile[r], b0, lane);
-            if (two) {
+            for (int r = 0; r < (kEarly ? R : 1); r++) load_w(w1[r], a, tile[r], b0 + 1, lane);
+        }
+    }
+    const int n_blocks = kMulti ? a.n_blocks : 1;
+    half8_t af[8];
+    if (kEarly && active) load_xf(af, a.xf, b0, lane);
+    for (int blk = 0; blk < n_blocks; blk++) {
+        const uint8_t *xf = a.xf + static_cast<size_t>(blk) * a.xf_stride;
+        const int n_rows = blk + 1 == n_blocks ? a.rows_last : 16;
 #pragma unroll
-                for (int r = 0; r < R; r++) load_w(w1[r], a, tile[r], b0 + 1, lane);
-            }
-            load_xf(af, a.xf, b0, lane);
+        for (int r = 0; r < R; r++) acc[r] = acc_sub[r] = float4_t{0, 0, 0, 0};
+        if (active) {
+            if constexpr (kEarly) {
+                // (af holds this block's first stage: loaded above, or behind the previous block's products)
 #pragma unroll
-            for (int r = 0; r < R; r++) compute(w0[r], af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
-            if (two) {
-                load_xf(af, a.xf, b0 + 1, lane);
+                for (int r = 0; r < R; r++) compute(w0[r], af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
+                if (two) {
+                    load_xf(af, xf, b0 + 1, lane);
 #pragma unroll
-                for (int r = 0; r < R; r++) compute(w1[r], af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
-            }
-        } else {
-            for (int b = b0; b < b1; b++) {
-                load_xf(af, a.xf, b, lane);
+                    for (int r = 0; r < R; r++) compute(w1[r], af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
+                }
+                // the next block's fragments travel while this block's partial tiles are summed and written
+                if (kMulti && blk + 1 < n_blocks) load_xf(af, xf + a.xf_stride, b0, lane);
+            } else {
+                for (int b = b0; b < b1; b++) {
+                    load_xf(af, xf, b, lane);
 #pragma unroll
-                for (int r = 0; r < R; r++) {
-                    W w;
-                    load_w(w, a, tile[r], b, lane);
-                    compute(w, af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
+                    for (int r = 0; r < R; r++) {
+                        W w;
+                        load_w(w, a, tile[r], b, lane);
+                        compute(w, af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
+                    }
                 }
             }
         }
-    }
+        if (blk) __syncthreads();  // the previous block's partial tiles have been summed
 #pragma unroll
-    for (int r = 0; r < R; r++) red[(wave * R + r) * 64 + lane] = acc[r] - acc_sub[r];
-    __syncthreads();
-    if (kslice != 0 || !active) return;
-    float4_t sum[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        sum[r] = red[(wave * R + r) * 64 + lane];
-        for (int s = 1; s < a.ksplit; s++) sum[r] += red[((wave + s) * R + r) * 64 + lane];
-    }
-    if (!a.pair_off) {
+        for (int r = 0; r < R; r++) red[(wave * R + r) * 64 + lane] = acc[r] - acc_sub[r];
+        __syncthreads();
+        if (kslice != 0 || !active) continue;
+        float4_t sum[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int col = (unit * R + r) * 16 + n;
-            if (col < a.n_out) {
+            sum[r] = red[(wave * R + r) * 64 + lane];
+            for (int s = 1; s < a.ksplit; s++) sum[r] += red[((wave + s) * R + r) * 64 + lane];
+        }
+        float *y = a.y ? a.y + static_cast<size_t>(blk) * a.y_stride : nullptr;
+        if (!a.pair_off) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int col = (unit * R + r) * 16 + n;
+                if (col < a.n_out) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (4 * g + i < n_rows) y[static_cast<size_t>(4 * g + i) * a.n_out + col] = sum[r][i];
+                }
+            }
+            continue;
+        }
+        if constexpr (R == 2) {
+            // SwiGLU of the (gate tile, up tile) pair: out[m][16 unit + n] = silu(gate) * up
+            const int ffn = a.n_out >> 1;
+            float4_t out;
+#pragma unroll
+            for (int i = 0; i < 4; i++) out[i] = sum[0][i] / (1.0f + expf(-sum[0][i])) * sum[1][i];
+            const int col = unit * 16 + n;
+            if (y && col < ffn) {
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    if (4 * g + i < a.n_rows) a.y[static_cast<size_t>(4 * g + i) * a.n_out + col] = sum[r][i];
+                    if (4 * g + i < n_rows) y[static_cast<size_t>(4 * g + i) * ffn + col] = out[i];
             }
-        }
-        return;
-    }
-    if constexpr (R == 2) {
-        // SwiGLU of the (gate tile, up tile) pair: out[m][16 unit + n] = silu(gate) * up
-        const int ffn = a.n_out >> 1;
-        float4_t out;
+            if (a.y_xf) {
+                // the tile through this wave's own LDS slot: lane (m, octet) then holds eight consecutive columns of a row
+                // (the slot's partial tile has been read: by this wave, above)
+                float *f = reinterpret_cast<float *>(&red[wave * R * 64]);
+                red[wave * R * 64 + lane] = out;
+                __builtin_amdgcn_wave_barrier();
+                if (lane < 32) {
+                    const int m = lane >> 1, oct = lane & 1;
+                    float v[8];
 #pragma unroll
-        for (int i = 0; i < 4; i++) out[i] = sum[0][i] / (1.0f + expf(-sum[0][i])) * sum[1][i];
-        const int col = unit * 16 + n;
-        if (a.y && col < ffn) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (4 * g + i < a.n_rows) a.y[static_cast<size_t>(4 * g + i) * ffn + col] = out[i];
-        }
-        if (a.y_xf) {
-            // the tile through this wave's own LDS slot: lane (m, octet) then holds eight consecutive columns of a row
-            float *f = reinterpret_cast<float *>(&red[wave * R * 64]);
-            red[wave * R * 64 + lane] = out;
-            __builtin_amdgcn_wave_barrier();
-            if (lane < 32) {
-                const int m = lane >> 1, oct = lane & 1;
-                float v[8];
-#pragma unroll
-                for (int i = 0; i < 8; i++) v[i] = f[((8 * oct + i) + 16 * (m >> 2)) * 4 + (m & 3)];
-                dfl_xf_store(a.y_xf, a.y_xf_kind, m, unit * 16 + 8 * oct, v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
+                    for (int i = 0; i < 8; i++) v[i] = f[((8 * oct + i) + 16 * (m >> 2)) * 4 + (m & 3)];
+                    dfl_xf_store(a.y_xf + static_cast<size_t>(blk) * a.y_xf_stride, a.y_xf_kind, m, unit * 16 + 8 * oct, v[0], v[1], v[2],
+                                 v[3], v[4], v[5], v[6], v[7]);
+                }
             }
         }
     }
@@ -335,6 +355,14 @@ int dfl_whole_kind(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t 
 
 int32_t dfl_gemm_whole(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in, int64_t n_out,
                        int32_t n_rows, int64_t pair_ffn, void *y_xf, int y_xf_kind, hipStream_t st) {
+    return dfl_gemm_whole_blocks(ctx, w_type, w, xf, y, n_in, n_out, n_rows, pair_ffn, y_xf, y_xf_kind, st);
+}
+
+int32_t dfl_gemm_whole_blocks(dflash_ctx *ctx, int32_t w_type, const void *w, const void *xf, float *y, int64_t n_in, int64_t n_out,
+                              int32_t n_rows_total, int64_t pair_ffn, void *y_xf, int y_xf_kind, hipStream_t st) {
+    const int32_t n_blocks = (n_rows_total + 15) / 16;
+    const int32_t n_rows = n_rows_total - 16 * (n_blocks - 1);  // rows of the last block
+    if (n_rows_total < 1 || n_blocks > 4096) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_whole: %d rows", n_rows_total);
     const WholePlan p = whole_plan(ctx, w_type, n_in, n_out, pair_ffn);
     if (p.kind == DFL_XF_NONE) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: type %d, %lld -> %lld not taken", w_type,
                                                static_cast<long long>(n_in), static_cast<long long>(n_out));
@@ -359,28 +387,25 @@ int32_t dfl_gemm_whole(dflash_ctx *ctx, int32_t w_type, const void *w, const voi
     a.n_units = p.n_units;
     a.pair_off = pair_ffn ? static_cast<int>(pair_ffn / 16) : 0;
     a.row_bytes = static_cast<uint32_t>(a.nb) * DFL_Q6_K_BYTES;
+    a.n_blocks = n_blocks;
+    a.rows_last = n_rows;
+    a.xf_stride = static_cast<uint32_t>(dfl_xf_bytes(n_in));
+    a.y_xf_stride = static_cast<uint32_t>(dfl_xf_bytes(pair_ffn ? pair_ffn : 256));
+    a.y_stride = static_cast<size_t>(16) * (pair_ffn ? pair_ffn : n_out);
     const int threads = 64 * p.ksplit * p.tl;
     const size_t red_bytes = static_cast<size_t>(16) * p.R * 64 * sizeof(float4_t);
     const size_t lds = red_bytes + (p.kind == DFL_XF_Q6K ? static_cast<size_t>(16) * kQ6AreaBytes : 0);
-    const void *fn = p.kind == DFL_XF_Q4K ? (p.R == 2 ? reinterpret_cast<const void *>(gemm_whole_kernel<Q4W, 2>)
-                                                      : reinterpret_cast<const void *>(gemm_whole_kernel<Q4W, 1>))
-                                          : (p.R == 2 ? reinterpret_cast<const void *>(gemm_whole_kernel<Q6W, 2>)
-                                                      : reinterpret_cast<const void *>(gemm_whole_kernel<Q6W, 1>));
+    typedef void (*kernel_t)(WholeArgs);
+    const bool multi = n_blocks > 1;
+    const kernel_t fn = p.kind == DFL_XF_Q4K ? (p.R == 2 ? (multi ? gemm_whole_kernel<Q4W, 2, true> : gemm_whole_kernel<Q4W, 2, false>)
+                                                         : (multi ? gemm_whole_kernel<Q4W, 1, true> : gemm_whole_kernel<Q4W, 1, false>))
+                                             : (p.R == 2 ? (multi ? gemm_whole_kernel<Q6W, 2, true> : gemm_whole_kernel<Q6W, 2, false>)
+                                                         : (multi ? gemm_whole_kernel<Q6W, 1, true> : gemm_whole_kernel<Q6W, 1, false>));
     if (lds > ctx->lds_bytes) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: %zu bytes of LDS needed", lds);
     if (lds > 48 * 1024)
-        if (const int32_t rc = dfl_raise_lds_limit(ctx, fn, lds)) return rc;
+        if (const int32_t rc = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(fn), lds)) return rc;
     dfl_timed timer(ctx, st, DFL_T_GEMM);
-    if (p.kind == DFL_XF_Q4K) {
-        if (p.R == 2)
-            gemm_whole_kernel<Q4W, 2><<<p.n_wg, threads, lds, st>>>(a);
-        else
-            gemm_whole_kernel<Q4W, 1><<<p.n_wg, threads, lds, st>>>(a);
-    } else {
-        if (p.R == 2)
-            gemm_whole_kernel<Q6W, 2><<<p.n_wg, threads, lds, st>>>(a);
-        else
-            gemm_whole_kernel<Q6W, 1><<<p.n_wg, threads, lds, st>>>(a);
-    }
+    fn<<<p.n_wg, threads, lds, st>>>(a);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

@@ -51,7 +51,7 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
                                                        const float *__restrict__ w, float *__restrict__ y, int n,
                                                        float eps, const float *__restrict__ gate_w,
                                                        float *__restrict__ gate_out, void *__restrict__ y_xf = nullptr,
-                                                       int y_xf_kind = 0) {
+                                                       int y_xf_kind = 0, size_t xf_stride = 0) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
     float *xr = x + static_cast<size_t>(blockIdx.x) * n;
@@ -84,7 +84,10 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
                 const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
                 *reinterpret_cast<f4 *>(yr + i) = o;
                 // (the host passes y_xf only for n a multiple of 256: whole waves are inside or outside the row)
-                if (y_xf) dfl_xf_store_pair(y_xf, y_xf_kind, blockIdx.x, i & ~7, o[0], o[1], o[2], o[3]);
+                // (more than sixteen rows: block b of sixteen at y_xf + b * xf_stride bytes)
+                if (y_xf)
+                    dfl_xf_store_pair(static_cast<uint8_t *>(y_xf) + (blockIdx.x >> 4) * xf_stride, y_xf_kind, blockIdx.x & 15, i & ~7, o[0],
+                                      o[1], o[2], o[3]);
                 if (gate_w) {
                     const f4 gw = *reinterpret_cast<const f4 *>(gate_w + i);
                     dot += (o[0] * gw[0] + o[1] * gw[1]) + (o[2] * gw[2] + o[3] * gw[3]);
@@ -219,6 +222,19 @@ __global__ void set_ids_pos_kernel(Int16Args ids, Int16Args pos, int n, int32_t 
             ids_dst[i] = id;
         }
         pos_dst[i] = pos.v[i];
+    }
+}
+
+// The same for the rows of a prefill group: up to 512 token ids by value, positions start, start + 1, ...
+constexpr int kMaxGroupRows = 512;
+struct IntGroupArgs {
+    int32_t v[kMaxGroupRows];
+};
+__global__ void set_group_ids_pos_kernel(IntGroupArgs ids, int start, int n, int32_t *__restrict__ ids_dst, int32_t *__restrict__ pos_dst) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        ids_dst[i] = ids.v[i];
+        pos_dst[i] = start + i;
     }
 }
 
@@ -518,7 +534,19 @@ struct dflash_session {
 // Block b needs the earlier blocks' K/V rows of a layer before its attention in that layer: one event per (lane,
 // layer), recorded behind the launch that writes the rows and behind the wait for the previous block's event.
 constexpr int kMaxPrefillLanes = 8;
+// Scratch of the grouped prefill of a mixture-of-experts target: the rows of up to `rows / 16` consecutive blocks pass
+// through a layer together (one launch per operator, the weights of a projection read once for all of them, the
+// experts regrouped by dfl_moe_ffn_group), attention alone block by block.  Null pointers: not set up (a dense
+// target, or no device memory for it), and the lanes below serve instead.
+struct PrefillGroup {
+    int rows = 0;
+    float *x = nullptr, *cur = nullptr, *mix = nullptr, *pk = nullptr, *q = nullptr, *attn = nullptr;
+    uint8_t *xf_cur = nullptr, *xf_attn = nullptr;
+    int32_t *ids = nullptr, *pos = nullptr;
+    dfl_moe_group_scratch moe;
+};
 struct PrefillPipe {
+    PrefillGroup group;
     int n_lanes = 4;  // blocks in flight: lane 0 is the owner itself (its context, its scratch, the caller's stream)
     struct Extra {
         dflash_ctx *ctx = nullptr;
@@ -624,6 +652,59 @@ int32_t dflash_session_create(dflash_ctx *ctx, const dflash_model_cfg *cfg, int6
     return DFLASH_OK;
 }
 
+namespace {
+void prefill_group_free(PrefillGroup *g) {
+    void *ptrs[] = {g->x, g->cur, g->mix, g->pk, g->q, g->attn, g->xf_cur, g->xf_attn, g->ids, g->pos, g->moe.logits, g->moe.sg,
+                    g->moe.sel_e, g->moe.sel_w, g->moe.pick_pos, g->moe.ids, g->moe.n_slots, g->moe.slot_rows, g->moe.xg, g->moe.act,
+                    g->moe.eo};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    *g = PrefillGroup();
+}
+
+// Blocks per pass of the grouped prefill (DFLASH_PREFILL_GROUP; 0 or 1 switches it off).  Measured on the 35B-A3B
+// shape, 2048-token prompt: see the prefill section of the bench.
+int prefill_group_blocks() {
+    static const int v = [] {
+        const char *e = getenv("DFLASH_PREFILL_GROUP");
+        return e && *e ? atoi(e) : 16;
+    }();
+    return std::max(0, std::min(kMaxGroupRows / 16, v));
+}
+
+// Sets the group scratch up for a mixture-of-experts shape; leaves it empty (no error) where the shape is not one the
+// grouped path takes or the memory is not there.
+void prefill_group_alloc(dflash_session *s, PrefillGroup *g) {
+    const dflash_model_cfg &c = s->cfg;
+    const int blocks = prefill_group_blocks();
+    const int used = c.n_expert_used < c.n_expert ? c.n_expert_used : c.n_expert;
+    if (blocks < 2 || c.n_expert < 1 || c.n_expert > 256 || used < 1 || c.hidden % DFL_QK_K || c.ffn_expert % DFL_QK_K) return;
+    int rows = 16 * blocks;
+    while (rows > 16 && rows * used > 4096) rows -= 16;
+    if (static_cast<int64_t>(rows) > s->capacity) rows = static_cast<int>((s->capacity + 15) / 16 * 16);
+    if (rows < 32) return;
+    const size_t H = c.hidden, q_dim = static_cast<size_t>(c.n_q) * c.head_dim, kv_dim = static_cast<size_t>(c.n_kv) * c.head_dim;
+    const size_t R = rows, nb = rows / 16;
+    const int max_slots = dfl_moe_group_max_slots(c, rows);
+    const size_t S = max_slots;
+    const bool ok = dev_alloc(&g->x, R * H) && dev_alloc(&g->cur, R * H) && dev_alloc(&g->mix, R * H) &&
+                    dev_alloc(&g->pk, R * (q_dim + 2 * kv_dim)) && dev_alloc(&g->q, R * q_dim) && dev_alloc(&g->attn, R * q_dim) &&
+                    dev_alloc(&g->xf_cur, nb * dfl_xf_bytes(H)) && dev_alloc(&g->xf_attn, nb * dfl_xf_bytes(q_dim)) &&
+                    dev_alloc(&g->ids, R) && dev_alloc(&g->pos, R) && dev_alloc(&g->moe.logits, R * c.n_expert) &&
+                    dev_alloc(&g->moe.sg, R) && dev_alloc(&g->moe.sel_e, R * used) && dev_alloc(&g->moe.sel_w, R * used) &&
+                    dev_alloc(&g->moe.pick_pos, R * used) && dev_alloc(&g->moe.ids, S) && dev_alloc(&g->moe.n_slots, 1) &&
+                    dev_alloc(&g->moe.slot_rows, S * 16) && dev_alloc(&g->moe.xg, S * 16 * H) &&
+                    dev_alloc(&g->moe.act, S * 16 * c.ffn_expert) && dev_alloc(&g->moe.eo, S * 16 * H);
+    if (!ok) {
+        (void)hipGetLastError();  // (an allocation that failed leaves its error behind)
+        prefill_group_free(g);
+        return;
+    }
+    g->moe.max_slots = max_slots;
+    g->rows = rows;
+}
+}  // namespace
+
 void dflash_session_destroy(dflash_session *s) {
     if (!s) return;
     if (PrefillPipe *p = s->pipe) {
@@ -643,6 +724,7 @@ void dflash_session_destroy(dflash_session *s) {
             }
             if (x.ctx) dflash_ctx_destroy(x.ctx);  // (the stream belongs to the process-wide pool)
         }
+        prefill_group_free(&p->group);
         delete p;
         s->pipe = nullptr;
     }
@@ -973,6 +1055,7 @@ int32_t prefill_pipe_create(dflash_ctx *ctx, dflash_session *s) {
     PrefillPipe *p = new (std::nothrow) PrefillPipe();
     if (!p) return dfl_fail(ctx, DFLASH_ERR_HIP, "prefill_blocks: out of host memory");
     s->pipe = p;  // (whatever has been made so far is taken down with the session)
+    prefill_group_alloc(s, &p->group);
     if (prefill_pipe_create_lanes(ctx, s, p) != DFLASH_OK) {
         for (auto &v : p->kv_done) {
             for (hipEvent_t e : v)
@@ -1041,6 +1124,82 @@ int32_t dflash_prefill_prepare(dflash_ctx *ctx, dflash_session *s) {
     return prefill_pipe_create(ctx, s);
 }
 
+namespace {
+
+// Whether every layer of the model is one the grouped prefill takes: q/k/v adjacent and, like the output projection,
+// a whole-K product over fragment-order rows; the experts as dfl_moe_ffn_group wants them.
+bool prefill_group_takes(const dflash_ctx *ctx, const dflash_model *model, const PrefillGroup &g) {
+    const dflash_model_cfg &c = model->cfg;
+    if (!g.rows || c.n_expert < 1) return false;
+    const int64_t H = c.hidden, q_dim = static_cast<int64_t>(c.n_q) * c.head_dim, kv_dim = static_cast<int64_t>(c.n_kv) * c.head_dim;
+    for (int il = 0; il < c.n_layers; il++) {
+        const dflash_layer &L = model->layers[il];
+        const LayerXf k = layer_xf(ctx, L, true, H, q_dim, kv_dim, c.ffn, false);
+        if (k.qkv == DFL_XF_NONE || k.wo == DFL_XF_NONE || !dfl_moe_group_fits(ctx, c, L, g.rows)) return false;
+    }
+    return true;
+}
+
+// One group of n rows (positions start .. start + n - 1) through every layer, on `st`: K/V rows into the session's
+// cache, tapped residuals into hidden_capture.  A row gets the bits verify_enqueue gives it in its own 16-row block:
+// every operator here is that block's operator over more rows (or the block's own launch: attention).
+int32_t prefill_group_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, PrefillGroup &g, const int32_t *tokens,
+                              int32_t n, int64_t start, const int32_t *tap_layers, int32_t n_taps, float *hidden_capture,
+                              hipStream_t st) {
+    const dflash_model_cfg &c = model->cfg;
+    const int H = c.hidden, hd = c.head_dim;
+    const size_t q_dim = static_cast<size_t>(c.n_q) * hd, kv_dim = static_cast<size_t>(c.n_kv) * hd;
+    const int64_t tot = static_cast<int64_t>(q_dim + 2 * kv_dim);
+    const size_t xf_h = dfl_xf_bytes(H), xf_q = dfl_xf_bytes(static_cast<int64_t>(q_dim));
+    IntGroupArgs ids_arg = {};
+    for (int i = 0; i < n; i++) ids_arg.v[i] = tokens[i];
+    set_group_ids_pos_kernel<<<(n + 255) / 256, 256, 0, st>>>(ids_arg, static_cast<int>(start), n, g.ids, g.pos);
+    int32_t rc = embed_rows(ctx, model->token_embd, g.ids, n, H, g.x, st);
+    if (rc) return rc;
+    const float scale = 1.0f / sqrtf(static_cast<float>(hd));
+    const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
+    auto qkv_kind = [&](int il) {
+        return il < c.n_layers ? layer_xf(ctx, model->layers[il], true, H, static_cast<int64_t>(q_dim), static_cast<int64_t>(kv_dim), c.ffn, false).qkv
+                               : DFL_XF_NONE;
+    };
+    for (int il = 0; il < c.n_layers; il++) {
+        const dflash_layer &L = model->layers[il];
+        _Float16 *kc = s->k_cache + il * per_layer, *vtc = s->vt_cache + il * per_layer;
+        const LayerXf xk = layer_xf(ctx, L, true, H, static_cast<int64_t>(q_dim), static_cast<int64_t>(kv_dim), c.ffn, false);
+        if (il == 0)  // (later layers: the experts' last kernel has normalised their input)
+            rms_norm_kernel<<<n, 256, 0, st>>>(g.x, nullptr, L.attn_norm, g.cur, H, c.eps, nullptr, nullptr, g.xf_cur, xk.qkv, xf_h);
+        if ((rc = dfl_gemm_whole_blocks(ctx, L.wq.type, L.wq.data, g.xf_cur, g.pk, H, tot, n, 0, nullptr, DFL_XF_NONE, st))) return rc;
+        qk_norm_rope_kernel<<<dim3(c.n_q + 2 * c.n_kv, n), 64, 0, st>>>(g.pk, tot, g.pk + q_dim, tot, g.q, nullptr, L.q_norm, L.k_norm, kc,
+                                                                      g.pos, c.n_q, c.n_kv, hd, c.eps, c.rope_theta,
+                                                                      g.pk + q_dim + kv_dim, tot, vtc, s->capacity);
+        // nothing of the last layer beyond its K/V rows is needed unless its residual is tapped (as in verify_enqueue)
+        if (il == c.n_layers - 1) {
+            bool tapped_last = false;
+            for (int t = 0; t < n_taps; t++) tapped_last = tapped_last || tap_layers[t] == il;
+            if (!tapped_last) break;
+        }
+        if ((rc = dfl_attn_blocks(ctx, g.q, DFLASH_TYPE_F32, kc, vtc, start, n, c.n_q, c.n_kv, hd, s->capacity, scale, g.attn, st, g.xf_attn,
+                                  xk.wo)))
+            return rc;
+        if ((rc = dfl_gemm_whole_blocks(ctx, L.wo.type, L.wo.data, g.xf_attn, g.mix, static_cast<int64_t>(q_dim), H, n, 0, nullptr,
+                                        DFL_XF_NONE, st)))
+            return rc;
+        const float *next_w = il + 1 < c.n_layers ? model->layers[il + 1].attn_norm : model->output_norm;
+        const int next_kind = qkv_kind(il + 1);
+        // x += mix, the experts' norm and the shared-expert gates: the block path's norm kernel over all the rows
+        rms_norm_kernel<<<n, 256, 0, st>>>(g.x, g.mix, L.post_norm, g.cur, H, c.eps, L.shexp_gate, g.moe.sg);
+        if ((rc = dfl_moe_ffn_group(ctx, c, L, g.x, g.cur, n, g.moe, next_w, next_kind ? g.xf_cur : nullptr, next_kind, xf_h, st)))
+            return rc;
+        for (int t = 0; t < n_taps; t++)
+            if (tap_layers[t] == il)
+                capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(g.x, hidden_capture, H, n_taps, t);
+    }
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+}  // namespace
+
 int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *s, const int32_t *tokens,
                               int32_t n_tokens, int64_t start, const int32_t *tap_layers, int32_t n_taps,
                               float *hidden_capture, dflash_stream_t stream) {
@@ -1065,6 +1224,21 @@ int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash
     if (!s->pipe && (rc = prefill_pipe_create(ctx, s))) return rc;
     PrefillPipe *p = s->pipe;
     if (!p->ready) return dfl_fail(ctx, DFLASH_ERR_STATE, "prefill_blocks: the extra lanes could not be set up earlier");
+    if (n_tokens > 16 && start + n_tokens <= 0x7fffffffll && prefill_group_takes(ctx, model, p->group)) {
+        // rows of many blocks per pass (see PrefillGroup); the caller's stream alone
+        const size_t cap_row = static_cast<size_t>(std::max(n_taps, 0)) * c.hidden;
+        for (int32_t t0 = 0; t0 < n_tokens; t0 += p->group.rows) {
+            const int32_t n = std::min<int32_t>(p->group.rows, n_tokens - t0);
+            if ((rc = prefill_group_enqueue(ctx, model, s, p->group, tokens + t0, n, start + t0, tap_layers, n_taps,
+                                            hidden_capture ? hidden_capture + static_cast<size_t>(t0) * cap_row : nullptr,
+                                            static_cast<hipStream_t>(stream)))) {
+                (void)hipStreamSynchronize(static_cast<hipStream_t>(stream));
+                return rc;  // (kv_n_pos unchanged: rows written past it are overwritten by the next block)
+            }
+        }
+        s->kv_n_pos = start + n_tokens;
+        return DFLASH_OK;
+    }
     const int n_lanes = p->n_lanes;
     hipStream_t lanes_st[kMaxPrefillLanes] = {static_cast<hipStream_t>(stream)};
     dflash_ctx *lanes_ctx[kMaxPrefillLanes] = {ctx};

@@ -372,19 +372,22 @@ __global__ void __launch_bounds__(256)
                             const float *__restrict__ sg, const float *__restrict__ shared, const int32_t *__restrict__ n_slots,
                             int n_used, int hidden, float *__restrict__ x, const float *__restrict__ norm_w,
                             float *__restrict__ y, float eps, const float *__restrict__ pre_add, void *__restrict__ y_xf,
-                            int y_xf_kind) {
+                            int y_xf_kind, int grouped = 0, size_t xf_stride = 0) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
     __shared__ float w_k[64];
-    __shared__ int32_t slot_k[64];
+    __shared__ int32_t slot_k[64];  // row of eo that holds pick k of this row
     const int row = blockIdx.x, tid = threadIdx.x;
+    // grouped (rows of several 16-row blocks, moe_group_slots_kernel): slot_of is the eo row of a pick itself, and the
+    // shared expert's slots are the last gridDim.x / 16 (rounded up) of the list, one per block of rows
     if (tid < n_used) {
         w_k[tid] = sel_w[row * n_used + tid];
-        slot_k[tid] = slot_of[row * n_used + tid];
+        slot_k[tid] = grouped ? slot_of[row * n_used + tid] : slot_of[row * n_used + tid] * 16 + row;
     }
     __syncthreads();
     const float gate = sg[row];
-    const size_t last = static_cast<size_t>(*n_slots) - 1;
+    const size_t last = grouped ? (static_cast<size_t>(*n_slots) - (gridDim.x + 15) / 16 + (row >> 4)) * 16 + (row & 15)
+                                : (static_cast<size_t>(*n_slots) - 1) * 16 + row;
     f4 v[4];
     float s = 0.0f;
 #pragma unroll
@@ -394,9 +397,9 @@ __global__ void __launch_bounds__(256)
         if (i < hidden) {
             f4 out = {0, 0, 0, 0};
             for (int k = 0; k < n_used; k++)
-                out += w_k[k] * *reinterpret_cast<const f4 *>(eo + (static_cast<size_t>(slot_k[k]) * 16 + row) * hidden + i);
+                out += w_k[k] * *reinterpret_cast<const f4 *>(eo + static_cast<size_t>(slot_k[k]) * hidden + i);
             const f4 shv = shared ? *reinterpret_cast<const f4 *>(shared + static_cast<size_t>(row) * hidden + i)
-                                  : *reinterpret_cast<const f4 *>(eo + (last * 16 + row) * hidden + i);
+                                  : *reinterpret_cast<const f4 *>(eo + last * hidden + i);
             out += gate * shv;
             v[j] = *reinterpret_cast<const f4 *>(x + static_cast<size_t>(row) * hidden + i);
             // (a residual term the norm before this layer's experts left out: it goes in first, as it would have there)
@@ -418,9 +421,108 @@ __global__ void __launch_bounds__(256)
             const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
             *reinterpret_cast<f4 *>(y + static_cast<size_t>(row) * hidden + i) = o;
             // (hidden a multiple of 256 here: whole waves are inside or outside the row)
-            if (y_xf) dfl_xf_store_pair(y_xf, y_xf_kind, row, i & ~7, o[0], o[1], o[2], o[3]);
+            if (y_xf)
+                dfl_xf_store_pair(static_cast<uint8_t *>(y_xf) + (row >> 4) * xf_stride, y_xf_kind, row & 15, i & ~7, o[0], o[1], o[2], o[3]);
         }
     }
+}
+
+// ---- rows of several 16-row blocks through one pass over the experts (prefill) ----
+//
+// A block of 16 rows touches 60-80 of 128 experts, so block after block re-reads most of a layer's expert weights;
+// 256 rows touch all of them about once.  The rows are therefore regrouped by expert: a slot is (expert, up to sixteen
+// of the rows that picked it), the expert kernels run their per-slot-activations mode over gathered copies of those
+// rows, and every row then sums its picks' outputs in pick order.  A (row, expert) product is one wave's whole-K sum
+// over the row's own activations, so it has the bits it has when the row's block runs alone.
+
+// Picks of every row: wave w of workgroup b routes row 16 b + w (dfl_route::route_row, as in the block kernels).
+__global__ void __launch_bounds__(1024)
+    moe_group_route_kernel(const float *__restrict__ logits, int n_rows, int n_expert, int n_used, int32_t *__restrict__ sel_e,
+                           float *__restrict__ sel_w) {
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 16 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const dfl_route::RowPicks pk = dfl_route::route_row(logits + static_cast<size_t>(row) * n_expert, n_expert, n_used, lane);
+    if (lane < n_used) {
+        sel_e[row * n_used + lane] = pk.my_e;
+        sel_w[row * n_used + lane] = pk.my_w;
+    }
+}
+
+// The slot list of a group of rows.  Expert e with c picks gets ceil(c / 16) consecutive slots, experts in ascending
+// order; behind them one slot per block of sixteen rows for the shared expert (id -1, rows 16 b .. 16 b + 15).
+//   ids[slot], *n_slots;  slot_rows[slot][16]: the rows whose activations the slot multiplies (unused places repeat
+//   row 0: computed, never read);  pick_pos[row][k] = 16 slot + place of the pick's output row.
+// Places inside an expert's slots are handed out by an atomic counter, so they vary from run to run; no sum does.
+// One workgroup; n_rows * n_used <= 4096, n_expert <= 256.
+constexpr int kGroupPicksPerThread = 4;
+__global__ void __launch_bounds__(1024)
+    moe_group_slots_kernel(const int32_t *__restrict__ sel_e, int n_rows, int n_used, int n_expert, int32_t *__restrict__ ids,
+                           int32_t *__restrict__ n_slots, int32_t *__restrict__ slot_rows, int32_t *__restrict__ pick_pos,
+                           int max_slots) {
+    __shared__ int cnt[256], base[257];
+    const int tid = threadIdx.x;
+    if (tid < 256) cnt[tid] = 0;
+    __syncthreads();
+    const int n_picks = n_rows * n_used;
+    int my_e[kGroupPicksPerThread], my_place[kGroupPicksPerThread];
+#pragma unroll
+    for (int j = 0; j < kGroupPicksPerThread; j++) {
+        const int p = tid + 1024 * j;
+        my_e[j] = -1;
+        my_place[j] = 0;
+        if (p < n_picks) {
+            my_e[j] = min(max(sel_e[p], 0), n_expert - 1);
+            my_place[j] = atomicAdd(&cnt[my_e[j]], 1);
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int b = 0;
+        for (int e = 0; e < n_expert; e++) {
+            base[e] = b;
+            b += (cnt[e] + 15) >> 4;
+        }
+        base[n_expert] = b;
+    }
+    __syncthreads();
+    const int total = base[n_expert], n_blocks = (n_rows + 15) >> 4;
+    if (tid == 0) *n_slots = min(total + n_blocks, max_slots);  // (the host sizes max_slots for the worst case)
+    if (tid < n_expert) {
+        const int c = cnt[tid], b = base[tid];
+        for (int t = 0; t < ((c + 15) >> 4); t++) ids[b + t] = tid;
+        if (c & 15)
+            for (int m = c & 15; m < 16; m++) slot_rows[(b + (c >> 4)) * 16 + m] = 0;
+    }
+    for (int r = tid; r < 16 * n_blocks; r += 1024) {
+        slot_rows[total * 16 + r] = min(r, n_rows - 1);
+        if ((r & 15) == 0) ids[total + (r >> 4)] = -1;
+    }
+#pragma unroll
+    for (int j = 0; j < kGroupPicksPerThread; j++) {
+        const int p = tid + 1024 * j;
+        if (p < n_picks) {
+            const int at = (base[my_e[j]] + (my_place[j] >> 4)) * 16 + (my_place[j] & 15);
+            slot_rows[at] = p / n_used;
+            pick_pos[p] = at;
+        }
+    }
+}
+
+// xg[slot][place][:] = f16(cur[slot_rows[slot][place]][:]): what the expert kernel would round the row to as it loads it.
+__global__ void __launch_bounds__(256)
+    moe_group_gather_kernel(const float *__restrict__ cur, const int32_t *__restrict__ slot_rows, const int32_t *__restrict__ n_slots,
+                            int hidden, _Float16 *__restrict__ xg) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    const int at = blockIdx.y;
+    if ((at >> 4) >= *n_slots) return;
+    const int i = 8 * (blockIdx.x * 256 + threadIdx.x);
+    if (i >= hidden) return;
+    const float *src = cur + static_cast<size_t>(slot_rows[at]) * hidden + i;
+    const f4 a = *reinterpret_cast<const f4 *>(src), b = *reinterpret_cast<const f4 *>(src + 4);
+    const h8 o = {static_cast<_Float16>(a[0]), static_cast<_Float16>(a[1]), static_cast<_Float16>(a[2]), static_cast<_Float16>(a[3]),
+                  static_cast<_Float16>(b[0]), static_cast<_Float16>(b[1]), static_cast<_Float16>(b[2]), static_cast<_Float16>(b[3])};
+    *reinterpret_cast<h8 *>(xg + static_cast<size_t>(at) * hidden + i) = o;
 }
 
 }  // namespace
@@ -570,6 +672,53 @@ int32_t dfl_moe_ffn(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_lay
                                                                          H, x_resid);
     else
         moe_combine_kernel<<<dim3((H + 255) / 256, n), 256, 0, st>>>(s.eo, s.sel_w, s.sg, s.shared, used, H, x_resid);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
+int dfl_moe_group_max_slots(const dflash_model_cfg &c, int n_rows) {
+    const int used = c.n_expert_used < c.n_expert ? c.n_expert_used : c.n_expert;
+    const int picks = n_rows * used;
+    // sum over experts of ceil(count / 16) <= distinct experts + picks / 16, and one shared-expert slot per block
+    return (picks < c.n_expert ? picks : c.n_expert) + picks / 16 + (n_rows + 15) / 16;
+}
+
+bool dfl_moe_group_fits(const dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, int n_rows) {
+    const int E = c.n_expert, used = c.n_expert_used < E ? c.n_expert_used : E;
+    const bool tiled = L.gate_exps.type == DFLASH_TYPE_Q4_K_TILED && L.up_exps.type == DFLASH_TYPE_Q4_K_TILED &&
+                       L.down_exps.type == DFLASH_TYPE_Q4_K_TILED;
+    const bool folded = c.ffn_shared == c.ffn_expert && L.gate.type == DFLASH_TYPE_Q4_K_TILED && L.up.type == DFLASH_TYPE_Q4_K_TILED &&
+                        L.down.type == DFLASH_TYPE_Q4_K_TILED;
+    return E >= 1 && E <= 256 && used >= 1 && used <= 64 && n_rows >= 1 && n_rows * used <= 1024 * kGroupPicksPerThread && tiled && folded &&
+           c.hidden % DFL_QK_K == 0 && c.ffn_expert % DFL_QK_K == 0 && c.hidden <= 4096 && L.shexp_gate && L.router.data &&
+           dfl_router_norm_fits(ctx, L.router.type, L.router.data, c.hidden, E, 16) &&
+           dfl_q4k_batched_f16_out(ctx, 1, 1, c.ffn_expert);
+}
+
+int32_t dfl_moe_ffn_group(dflash_ctx *ctx, const dflash_model_cfg &c, const dflash_layer &L, float *x_resid,
+                          float *cur, int n_rows, const dfl_moe_group_scratch &s, const float *next_norm_w, void *next_xf,
+                          int next_xf_kind, size_t next_xf_stride, hipStream_t st) {
+    if (!dfl_moe_group_fits(ctx, c, L, n_rows) || !x_resid || !cur || !next_norm_w)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "moe group: layer or row count (%d) not taken", n_rows);
+    const int E = c.n_expert, used = c.n_expert_used < E ? c.n_expert_used : E, H = c.hidden, fe = c.ffn_expert;
+    const int max_slots = dfl_moe_group_max_slots(c, n_rows);
+    if (max_slots > s.max_slots) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "moe group: scratch sized for %d slots, %d needed", s.max_slots, max_slots);
+    int32_t rc;
+    if ((rc = dfl_router_rows(ctx, L.router.data, cur, s.logits, H, E, n_rows, st))) return rc;
+    moe_group_route_kernel<<<(n_rows + 15) / 16, 1024, 0, st>>>(s.logits, n_rows, E, used, s.sel_e, s.sel_w);
+    moe_group_slots_kernel<<<1, 1024, 0, st>>>(s.sel_e, n_rows, used, E, s.ids, s.n_slots, s.slot_rows, s.pick_pos, max_slots);
+    moe_group_gather_kernel<<<dim3((H / 8 + 255) / 256, max_slots * 16), 256, 0, st>>>(cur, s.slot_rows, s.n_slots, H, s.xg);
+    const size_t stride_in = dflash_q4k_tiled_bytes(H, fe), stride_dn = dflash_q4k_tiled_bytes(fe, H);
+    if ((rc = dfl_gemm_q4k_batched(ctx, L.gate_exps.data, stride_in, L.gate.data, s.ids, s.n_slots, max_slots, s.xg, DFLASH_TYPE_F16,
+                                   static_cast<size_t>(16) * H, s.act, DFLASH_TYPE_F16, static_cast<size_t>(16) * fe, H, fe, 16, 1,
+                                   L.up_exps.data, L.up.data, 1, st, nullptr)))
+        return rc;
+    if ((rc = dfl_gemm_q4k_batched(ctx, L.down_exps.data, stride_dn, L.down.data, s.ids, s.n_slots, max_slots, s.act, DFLASH_TYPE_F16,
+                                   static_cast<size_t>(16) * fe, s.eo, DFLASH_TYPE_F32, static_cast<size_t>(16) * H, fe, H, 16, 1, nullptr,
+                                   nullptr, 1, st, nullptr)))
+        return rc;
+    moe_combine_norm_kernel<<<n_rows, 256, 0, st>>>(s.eo, s.pick_pos, s.sel_w, s.sg, nullptr, s.n_slots, used, H, x_resid, next_norm_w,
+                                                    cur, c.eps, nullptr, next_xf, next_xf_kind, 1, next_xf_stride);
     DFL_HIP_CHECK(ctx, hipGetLastError());
     return DFLASH_OK;
 }

@@ -153,6 +153,33 @@ def test_pipelined_prefill_on_the_moe_shape_equals_block_by_block(ctx, weights):
     pipe.close()
 
 
+def test_grouped_prefill_over_several_groups_equals_block_by_block(ctx, weights):
+    """A prompt longer than one group of the grouped prefill (256 rows a pass: every projection once for all of them, the
+    experts regrouped by expert) with a ragged tail, started at a position that is not a multiple of 16: captured rows,
+    and the logits of a block that follows (which read every K/V row written), equal block-by-block execution bit for bit."""
+    model = dfl.TargetModel(ctx, C5, weights)
+    rng = np.random.default_rng(23)
+    head = rng.integers(0, C5.vocab, 5).tolist()
+    toks = rng.integers(0, C5.vocab, 256 + 16 * 2 + 5).tolist()
+    probe = rng.integers(0, C5.vocab, 16).tolist()
+    ref, pipe = dfl.Session(ctx, model, 512, TAPS), dfl.Session(ctx, model, 512, TAPS)
+    for s in (ref, pipe):
+        s.encode_packed_verify_layer_major(head, 0, want_head=False)
+    got = pipe.prefill_blocks(toks, len(head))
+    want = []
+    for s0 in range(0, len(toks), 16):
+        want.append(ref.encode_packed_verify_layer_major(toks[s0:s0 + 16], len(head) + s0, want_head=False).hidden_capture.cpu().numpy())
+    want = np.concatenate(want, axis=0)
+    got = got.cpu().numpy()
+    bad = np.flatnonzero(np.any(got.reshape(len(toks), -1) != want.reshape(len(toks), -1), axis=1))
+    assert bad.size == 0, f"rows that differ: {bad[:16].tolist()} of {len(toks)}"
+    a = ref.encode_packed_verify_layer_major(probe, len(head) + len(toks), want_logits=True)
+    b = pipe.encode_packed_verify_layer_major(probe, len(head) + len(toks), want_logits=True)
+    assert np.array_equal(a.logits.cpu().numpy(), b.logits.cpu().numpy())
+    ref.close()
+    pipe.close()
+
+
 _ROUTE_PROBE = r"""
 import sys
 import numpy as np
