@@ -608,8 +608,16 @@ static int32_t attn_rows(dflash_ctx *ctx, const void *q, int32_t q_type, const v
     if (env_hw > 0 && group % env_hw == 0) hw = env_hw;
     if (per_cu < 1) per_cu = 1;
     if (min_chunk < 32) min_chunk = 32;
-    const int n_parts = group / hw;  // workgroups per (chunk, KV head)
+    int n_parts = group / hw;  // workgroups per (chunk, KV head)
     const int want = static_cast<int>((static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv * n_parts - 1) / (n_kv * n_parts));
+    // Several blocks in one launch cover the chip between them: a workgroup then serves the whole GQA group, so a chunk
+    // of keys is staged once instead of group / hw times (a workgroup's LDS ring leaves no room for a second one on
+    // its CU, whatever its size).  The split of the keys (want, min_chunk) stays the single block's, and a head is one
+    // wave's work either way: the same bits.
+    if (n_blocks > 1) {
+        hw = group;
+        n_parts = 1;
+    }
     // most splits any context up to n_pos can have
     auto splits_for = [&](int64_t np) {
         return ctx_len_dev ? static_cast<int>(std::min<int64_t>(want, (np + min_chunk - 1) / min_chunk))

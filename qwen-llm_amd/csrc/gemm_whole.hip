@@ -97,6 +97,48 @@ __device__ __forceinline__ void compute(const Q4W &r, const half8_t (&af)[8], in
     }
 }
 
+// The same in two steps, for a launch that multiplies many row blocks with one set of weights: the B operands of a
+// super-block's eight MFMAs once (unpack), then only the MFMAs per row block (mma), in compute()'s order.
+struct Q4F {
+    half8_t b[8];
+    _Float16 m_lo, m_hi;
+};
+__device__ __forceinline__ void unpack(const Q4W &r, int lane, uint8_t *, uint32_t sc_sel, Q4KMagic magic, Q4F &f) {
+    const int g = lane >> 4;
+    const u32x4_t hdr = r.hdr;
+    const uint32_t upper = 0u - static_cast<uint32_t>(g >> 1);
+    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu, mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t sc_word = (sc_hi & upper) | (sc_lo & ~upper), mn_word = (mn_hi & upper) | (mn_lo & ~upper);
+    const half2_t dm = __builtin_bit_cast(half2_t, hdr.x);
+    const half2_t p_sc = as_half2(__builtin_amdgcn_perm(0x64646464u, sc_word, sc_sel));
+    const half2_t p_mn = as_half2(__builtin_amdgcn_perm(0x64646464u, mn_word, sc_sel));
+    const half2_t neg = dm * splat(static_cast<_Float16>(-1024.0f));
+    const half2_t S = __builtin_elementwise_fma(p_sc, splat(dm[0]), splat(neg[0]));
+    const half2_t M = __builtin_elementwise_fma(p_mn, splat(dm[1]), splat(neg[1]));
+    const half2_t unbias = {static_cast<_Float16>(-1024.0f), static_cast<_Float16>(-64.0f)};
+    const half2_t Cs = S * unbias;
+    const half2_t s2l = splat(S[0]), c2l = splat(Cs[0]);
+    const half2_t s2h = splat(S[1]), c2h = splat(Cs[1]);
+    f.m_lo = M[0];
+    f.m_hi = M[1];
+    const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        f.b[t] = unpack_scale<false>(qw[2 * t], qw[2 * t + 1], s2l, c2l, magic.lo);
+        f.b[4 + t] = unpack_scale<true>(qw[2 * t], qw[2 * t + 1], s2h, c2h, magic.hi);
+    }
+}
+__device__ __forceinline__ void mma(const Q4F &f, const half8_t (&af)[8], float4_t &acc, float4_t &acc_sub) {
+    const half8_t bml = {f.m_lo, f.m_lo, f.m_lo, f.m_lo, f.m_lo, f.m_lo, f.m_lo, f.m_lo};
+    const half8_t bmh = {f.m_hi, f.m_hi, f.m_hi, f.m_hi, f.m_hi, f.m_hi, f.m_hi, f.m_hi};
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], f.b[t], acc, 0, 0, 0);
+        acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], t < 4 ? bml : bmh, acc_sub, 0, 0, 0);
+    }
+}
+
 // ---- Q6_K, GGUF row order: 210-byte blocks (ql[128], qh[64], scales[16], d), rows 2-byte aligned ----
 // A tile's stage is 16 runs of 210 bytes a row stride apart.  They are loaded as 208 pieces of 16 bytes (13 per row,
 // consecutive lanes taking consecutive pieces: row-contiguous requests) plus d, and pass through a wave-private LDS
@@ -167,6 +209,67 @@ __device__ __forceinline__ void compute(const Q6W &r, const half8_t (&af)[8], in
     }
 }
 
+struct Q6F {
+    half8_t b[8];
+    _Float16 o[4];  // 32 s of the four scale pairs: low quarter's two, high quarter's two
+};
+__device__ __forceinline__ void unpack(const Q6W &r, int lane, uint8_t *area, uint32_t, Q4KMagic magic, Q6F &f) {
+    const int n = lane & 15, g = lane >> 4, h = g >> 1, odd = g & 1;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int i = lane + 64 * j;
+        if (i < 208) *reinterpret_cast<u32x4_t *>(area + (i / 13) * kQ6RowStride + 16 * (i % 13)) = r.p[j];
+    }
+    if (lane < 16) *reinterpret_cast<uint16_t *>(area + lane * kQ6RowStride + 208) = static_cast<uint16_t>(r.d);
+    __builtin_amdgcn_wave_barrier();
+    const uint8_t *rowp = area + n * kQ6RowStride;
+    const u32x4_t qa = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd);
+    const u32x4_t qb = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd + 16);
+    const u32x4_t ha = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h);
+    const u32x4_t hb = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h + 16);
+    const uint32_t sc4 = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h) >> (16 * odd)) & 0xffffu;
+    const uint32_t sc4h = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h + 4) >> (16 * odd)) & 0xffffu;
+    const float d = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(rowp + 208)));
+    __builtin_amdgcn_wave_barrier();
+    const int hs = 2 * odd;
+    const uint32_t hq[8] = {ha.x >> hs, ha.y >> hs, ha.z >> hs, ha.w >> hs, hb.x >> hs, hb.y >> hs, hb.z >> hs, hb.w >> hs};
+    const uint32_t ql[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+    auto scale = [&](uint32_t pair, int j) { return static_cast<_Float16>(d * static_cast<float>(static_cast<int8_t>(pair >> (8 * j)))); };
+    const _Float16 s_l0 = scale(sc4, 0), s_l1 = scale(sc4, 1), s_h0 = scale(sc4h, 0), s_h1 = scale(sc4h, 1);
+    const _Float16 k32 = static_cast<_Float16>(32.0f);
+    f.o[0] = s_l0 * k32;
+    f.o[1] = s_l1 * k32;
+    f.o[2] = s_h0 * k32;
+    f.o[3] = s_h1 * k32;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const _Float16 sl = (t >> 1) ? s_l1 : s_l0, sh = (t >> 1) ? s_h1 : s_h0;
+        f.b[t] = unpack6<false>(ql[2 * t], ql[2 * t + 1], hq[2 * t], hq[2 * t + 1], splat(sl), splat(sl * static_cast<_Float16>(-1024.0f)),
+                                magic.lo);
+        f.b[4 + t] = unpack6<true>(ql[2 * t], ql[2 * t + 1], hq[2 * t] >> 4, hq[2 * t + 1] >> 4, splat(sh),
+                                   splat(sh * static_cast<_Float16>(-64.0f)), magic.hi);
+    }
+}
+__device__ __forceinline__ void mma(const Q6F &f, const half8_t (&af)[8], float4_t &acc, float4_t &acc_sub) {
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], f.b[t], acc, 0, 0, 0);
+        const _Float16 o = f.o[t >> 1];
+        const half8_t bo = {o, o, o, o, o, o, o, o};
+        acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bo, acc_sub, 0, 0, 0);
+    }
+}
+template <typename W>
+struct FragsOf;
+template <>
+struct FragsOf<Q4W> {
+    typedef Q4F type;
+};
+template <>
+struct FragsOf<Q6W> {
+    typedef Q6F type;
+};
+
 __device__ __forceinline__ void load_xf(half8_t (&af)[8], const uint8_t *xf, int b, int lane) {
     const half8_t *p = reinterpret_cast<const half8_t *>(xf) + static_cast<size_t>(b) * 512 + lane;
 #pragma unroll
@@ -174,8 +277,9 @@ __device__ __forceinline__ void load_xf(half8_t (&af)[8], const uint8_t *xf, int
 }
 
 // W: Q4W or Q6W.  R: tiles per wave and stage (they share the stage's activation fragments).
-// kMulti: several 16-row blocks per launch (a.n_blocks); the single-block instances keep the registers of a kernel without the loop.
-template <typename W, int R, bool kMulti>
+// kMulti: several 16-row blocks per launch (a.n_blocks): 1 = every wave has one stage (K of at most 16 super-blocks), 2 = one or
+// two; the single-block instances (0) keep the registers of a kernel without the loop.
+template <typename W, int R, int kMulti>
 __global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
     // [16 waves][R] partial tiles; Q6_K: then a staging area per wave
     extern __shared__ float4_t red[];
@@ -186,7 +290,7 @@ __global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
     const bool active = unit < a.n_units;
     const int n = lane & 15, g = lane >> 4;
     const int b0 = a.nb * kslice / a.ksplit, b1 = a.nb * (kslice + 1) / a.ksplit;  // one or two stages (host)
-    const bool two = b1 - b0 > 1;
+    const bool two = kMulti != 1 && b1 - b0 > 1;
     const int n_tiles = (a.n_out + 15) >> 4;
     int tile[R];
 #pragma unroll
@@ -210,13 +314,27 @@ __global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
     const int n_blocks = kMulti ? a.n_blocks : 1;
     half8_t af[8];
     if (kEarly && active) load_xf(af, a.xf, b0, lane);
+    // many row blocks, one tile per wave: the B operands are unpacked once and stay in registers in place of the raw weights
+    constexpr bool kFrags = kMulti != 0 && kEarly && R == 1;
+    typename FragsOf<W>::type f0, f1;
+    if (kFrags && active) {
+        unpack(w0[0], lane, area, sc_sel, magic, f0);
+        if (two) unpack(w1[0], lane, area, sc_sel, magic, f1);
+    }
     for (int blk = 0; blk < n_blocks; blk++) {
         const uint8_t *xf = a.xf + static_cast<size_t>(blk) * a.xf_stride;
         const int n_rows = blk + 1 == n_blocks ? a.rows_last : 16;
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] = acc_sub[r] = float4_t{0, 0, 0, 0};
         if (active) {
-            if constexpr (kEarly) {
+            if constexpr (kFrags) {
+                mma(f0, af, acc[0], acc_sub[0]);
+                if (two) {
+                    load_xf(af, xf, b0 + 1, lane);
+                    mma(f1, af, acc[0], acc_sub[0]);
+                }
+                if (blk + 1 < n_blocks) load_xf(af, xf + a.xf_stride, b0, lane);
+            } else if constexpr (kEarly) {
                 // (af holds this block's first stage: loaded above, or behind the previous block's products)
 #pragma unroll
                 for (int r = 0; r < R; r++) compute(w0[r], af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
@@ -226,7 +344,7 @@ __global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
                     for (int r = 0; r < R; r++) compute(w1[r], af, lane, area, sc_sel, magic, acc[r], acc_sub[r]);
                 }
                 // the next block's fragments travel while this block's partial tiles are summed and written
-                if (kMulti && blk + 1 < n_blocks) load_xf(af, xf + a.xf_stride, b0, lane);
+                if (kMulti != 0 && blk + 1 < n_blocks) load_xf(af, xf + a.xf_stride, b0, lane);
             } else {
                 for (int b = b0; b < b1; b++) {
                     load_xf(af, xf, b, lane);
@@ -396,11 +514,11 @@ int32_t dfl_gemm_whole_blocks(dflash_ctx *ctx, int32_t w_type, const void *w, co
     const size_t red_bytes = static_cast<size_t>(16) * p.R * 64 * sizeof(float4_t);
     const size_t lds = red_bytes + (p.kind == DFL_XF_Q6K ? static_cast<size_t>(16) * kQ6AreaBytes : 0);
     typedef void (*kernel_t)(WholeArgs);
-    const bool multi = n_blocks > 1;
-    const kernel_t fn = p.kind == DFL_XF_Q4K ? (p.R == 2 ? (multi ? gemm_whole_kernel<Q4W, 2, true> : gemm_whole_kernel<Q4W, 2, false>)
-                                                         : (multi ? gemm_whole_kernel<Q4W, 1, true> : gemm_whole_kernel<Q4W, 1, false>))
-                                             : (p.R == 2 ? (multi ? gemm_whole_kernel<Q6W, 2, true> : gemm_whole_kernel<Q6W, 2, false>)
-                                                         : (multi ? gemm_whole_kernel<Q6W, 1, true> : gemm_whole_kernel<Q6W, 1, false>));
+    const int multi = n_blocks > 1 ? (a.nb > p.ksplit ? 2 : 1) : 0;
+#define DFL_WHOLE_PICK(WT, RR) (multi == 0 ? gemm_whole_kernel<WT, RR, 0> : multi == 1 ? gemm_whole_kernel<WT, RR, 1> : gemm_whole_kernel<WT, RR, 2>)
+    const kernel_t fn = p.kind == DFL_XF_Q4K ? (p.R == 2 ? DFL_WHOLE_PICK(Q4W, 2) : DFL_WHOLE_PICK(Q4W, 1))
+                                             : (p.R == 2 ? DFL_WHOLE_PICK(Q6W, 2) : DFL_WHOLE_PICK(Q6W, 1));
+#undef DFL_WHOLE_PICK
     if (lds > ctx->lds_bytes) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: %zu bytes of LDS needed", lds);
     if (lds > 48 * 1024)
         if (const int32_t rc = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(fn), lds)) return rc;

@@ -154,15 +154,15 @@ def test_pipelined_prefill_on_the_moe_shape_equals_block_by_block(ctx, weights):
 
 
 def test_grouped_prefill_over_several_groups_equals_block_by_block(ctx, weights):
-    """A prompt longer than one group of the grouped prefill (256 rows a pass: every projection once for all of them, the
+    """A prompt longer than one group of the grouped prefill (512 rows a pass: every projection once for all of them, the
     experts regrouped by expert) with a ragged tail, started at a position that is not a multiple of 16: captured rows,
     and the logits of a block that follows (which read every K/V row written), equal block-by-block execution bit for bit."""
     model = dfl.TargetModel(ctx, C5, weights)
     rng = np.random.default_rng(23)
     head = rng.integers(0, C5.vocab, 5).tolist()
-    toks = rng.integers(0, C5.vocab, 256 + 16 * 2 + 5).tolist()
+    toks = rng.integers(0, C5.vocab, 512 + 16 * 2 + 5).tolist()
     probe = rng.integers(0, C5.vocab, 16).tolist()
-    ref, pipe = dfl.Session(ctx, model, 512, TAPS), dfl.Session(ctx, model, 512, TAPS)
+    ref, pipe = dfl.Session(ctx, model, 1024, TAPS), dfl.Session(ctx, model, 1024, TAPS)
     for s in (ref, pipe):
         s.encode_packed_verify_layer_major(head, 0, want_head=False)
     got = pipe.prefill_blocks(toks, len(head))
@@ -236,6 +236,45 @@ def test_norm_inside_the_router_launch_equals_the_norm_kernel(tmp_path):
     taken in the same order, so logits and captured rows are equal bit for bit."""
     on, off = _probe_under(tmp_path, "DFLASH_MOE_FUSED_NORM")
     assert np.array_equal(on, off)
+
+
+_LANES_PROBE = r"""
+import sys
+import numpy as np
+import qwen_llm_amd as dfl
+cfg = dfl.ModelConfig(n_layers=2, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=0, vocab=8192, n_expert=128,
+                      n_expert_used=8, ffn_expert=768, ffn_shared=768)
+ctx = dfl.Context(0, workspace_bytes=64 << 20)
+model = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_blocks(cfg, 47))
+rng = np.random.default_rng(13)
+toks = rng.integers(0, cfg.vocab, 16 * 6 + 3).tolist()
+probe = rng.integers(0, cfg.vocab, 16).tolist()
+sess = dfl.Session(ctx, model, 256, [0, 1])
+hid = sess.prefill_blocks(toks, 0).cpu().numpy().reshape(len(toks), -1)
+out = sess.encode_packed_verify_layer_major(probe, len(toks), want_logits=True)
+np.save(sys.argv[1], np.concatenate([hid.reshape(-1), out.logits.cpu().numpy().reshape(-1)]))
+"""
+
+
+def test_prefill_with_blocks_in_flight_on_lanes_equals_grouped_prefill(tmp_path):
+    """The two prefill schedules of a mixture-of-experts target - rows of many blocks per pass (the default) and, with
+    DFLASH_PREFILL_GROUP=0, four blocks in flight on lane streams, each routing and running its experts in its own
+    scratch - leave the same captured rows and the same logits for a block that follows, bit for bit.  (The switch is
+    read once per process: each setting runs in a short-lived process of its own, one after the other.)"""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    got = {}
+    for flag in ("32", "0"):
+        path = str(tmp_path / f"prefill_{flag}.npy")
+        env = dict(os.environ, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""), DFLASH_PREFILL_GROUP=flag)
+        r = subprocess.run([sys.executable, "-c", _LANES_PROBE, path], env=env, cwd=root, capture_output=True, text=True, timeout=240)
+        assert r.returncode == 0, r.stderr[-2000:]
+        got[flag] = np.load(path)
+    assert got["32"].shape == got["0"].shape and np.all(np.isfinite(got["32"]))
+    assert np.array_equal(got["32"], got["0"])
 
 
 def test_generate_on_the_moe_shape_equals_serial_greedy(ctx, weights):
