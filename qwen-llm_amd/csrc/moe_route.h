@@ -49,22 +49,23 @@ struct RowPicks {
     unsigned long long m[4];   // the row's picked experts (every lane)
 };
 
-// lg: the row's n_expert router logits.  Called by all 64 lanes of a wave.
-__device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int n_expert, int n_used, int lane) {
+// lg: the row's n_expert router logits (n_expert <= 64 kRegs: kRegs probabilities per lane).  Called by all 64 lanes of a wave.
+template <int kRegs>
+__device__ __forceinline__ RowPicks route_row_regs(const float *__restrict__ lg, int n_expert, int n_used, int lane) {
     RowPicks r;
     r.my_e = 0;
     r.m[0] = r.m[1] = r.m[2] = r.m[3] = 0;
-    float lgv[4];
+    float lgv[kRegs];
 #pragma unroll
-    for (int j = 0; j < 4; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
+    for (int j = 0; j < kRegs; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
     float mx = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 4; j++) mx = fmaxf(mx, lgv[j]);
+    for (int j = 0; j < kRegs; j++) mx = fmaxf(mx, lgv[j]);
     mx = wave_max_f32(mx);
-    float pv[4];
+    float pv[kRegs];
     float sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < kRegs; j++) {
         pv[j] = 0.0f;
         if (lane + 64 * j < n_expert) {
             pv[j] = expf(lgv[j] - mx);
@@ -74,7 +75,7 @@ __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int 
     sum = wave_sum_f32(sum);
     const float inv = 1.0f / sum;
 #pragma unroll
-    for (int j = 0; j < 4; j++) pv[j] = lane + 64 * j < n_expert ? pv[j] * inv : -1.0f;  // no such expert: never picked
+    for (int j = 0; j < kRegs; j++) pv[j] = lane + 64 * j < n_expert ? pv[j] * inv : -1.0f;  // no such expert: never picked
 
     // pick k = the highest remaining probability, equal probabilities to the lower id: a wave-wide float maximum
     // (one DPP instruction per step), then the first lane / register that holds it, found with compares into scalar
@@ -82,10 +83,13 @@ __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int 
     // falls back to an index in range.
     float my_p = 0.0f;
     for (int k = 0; k < n_used; k++) {
-        const float pmax = wave_max_f32(fmaxf(fmaxf(pv[0], pv[1]), fmaxf(pv[2], pv[3])));
+        float lmax = pv[0];
+#pragma unroll
+        for (int j = 1; j < kRegs; j++) lmax = fmaxf(lmax, pv[j]);
+        const float pmax = wave_max_f32(lmax);
         int e_win = -1;
 #pragma unroll
-        for (int j = 3; j >= 0; j--) {
+        for (int j = kRegs - 1; j >= 0; j--) {
             const unsigned long long hit = __builtin_amdgcn_ballot_w64(pv[j] == pmax);
             if (hit) e_win = 64 * j + __builtin_ctzll(hit);
         }
@@ -97,7 +101,7 @@ __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int 
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            if (lane + 64 * j == e_win) pv[j] = -1.0f;  // taken
+            if (j < kRegs && lane + 64 * j == e_win) pv[j < kRegs ? j : 0] = -1.0f;  // taken
             if ((e_win >> 6) == j) r.m[j] |= 1ull << (e_win & 63);
         }
     }
@@ -106,6 +110,14 @@ __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int 
     wsum = fmaxf(wsum, 6.103515625e-05f);  // 2^-14
     r.my_w = my_p / wsum;
     return r;
+}
+
+// n_expert <= 256.  The common 128-expert router keeps two probabilities per lane instead of four: the same
+// arithmetic on the same values in the same order (the registers it drops hold "no such expert"), half the
+// per-pick work, which every workgroup of the expert launch spends before its first weight byte.
+__device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int n_expert, int n_used, int lane) {
+    if (n_expert <= 128) return route_row_regs<2>(lg, n_expert, n_used, lane);
+    return route_row_regs<4>(lg, n_expert, n_used, lane);
 }
 
 // v[i & 3] without indexing the array by a run-time value (which would move it from registers to scratch memory)
