@@ -324,7 +324,7 @@ def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048):
     serial.prepare_prefill()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    # every block but the last without the output head, four blocks in flight (dflash_prefill_blocks); the last with it
+    # every block but the last without the output head (dflash_prefill_blocks: the rows of up to 32 blocks per pass); the last with it
     body = (prompt_len - 1) // 16 * 16
     serial.prefill_blocks(prompt[:body], 0, want_hidden=False)
     out = serial.encode_packed_verify_layer_major(prompt[body:], body, want_hidden=False)
@@ -342,6 +342,7 @@ def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048):
     log(f"e2e: prefill {res['prefill_tokens_per_s']:.0f} tok/s, serial decode {res['serial_tokens_per_s']:.1f} tok/s")
     for k in sweep:
         dec = dfl.SpeculativeDecoder(ctx, target, head, taps, cap, mask)
+        dec.session.prepare_prefill()  # the prefill's scratch is set-up, as for the serial session above: not timed
         torch.cuda.synchronize()
         tp = time.perf_counter()
         first = dec.prefill(prompt)  # target prefill with hidden capture + the drafter's pass over the prompt's columns

@@ -438,15 +438,20 @@ int32_t dflash_verify_block(dflash_ctx *ctx, const dflash_model *model, dflash_s
 int32_t dflash_restore(dflash_ctx *ctx, dflash_session *session, int64_t start_position, int32_t n, int32_t n_keep);
 
 /* The packed prefill with hidden capture (metal_dflash.rs:10779-15648; the reference walks the prompt in chunks of
- * layer_scratch.n rows, :10770-10778): tokens_host[n_tokens] at positions start_position .., in blocks of 16 rows
- * through the same layers as dflash_verify_block, without the output head; K/V rows are appended, the tapped hidden
- * rows go to hidden_capture[n_tokens][n_taps][hidden] (device; may be NULL with n_taps = 0).  Up to four consecutive
- * blocks are in flight on as many streams (DFLASH_PREFILL_LANES, 1..8; the extra streams, scratch sets and
- * contexts' workspaces belong to the session and are made on the first call), ordered by per-layer events where a
- * block reads the earlier blocks' K/V rows; the caller's stream continues behind all of them.  Results equal those
- * of the same blocks through dflash_verify_block bit for bit.  Guards as dflash_verify_block; on an error kv_n_pos
- * is unchanged. */
-/* Makes the extra streams, scratch sets and contexts of dflash_prefill_blocks ahead of its first call (which makes
+ * layer_scratch.n rows, :10770-10778): tokens_host[n_tokens] at positions start_position .., through the same layers
+ * as dflash_verify_block, without the output head; K/V rows are appended, the tapped hidden rows go to
+ * hidden_capture[n_tokens][n_taps][hidden] (device; may be NULL with n_taps = 0).  Two schedules, same results:
+ *   - a mixture-of-experts target whose expert stacks and shared expert are tiled Q4_K and whose q/k/v and output
+ *     projections take the one-launch GEMM: the rows of up to 32 consecutive blocks (DFLASH_PREFILL_GROUP, 2..32;
+ *     0 = never) pass through a layer together on the caller's stream - every projection once for all of them, the
+ *     experts regrouped by expert - so a pass reads a layer's weights about once;
+ *   - any other target: 16-row blocks, up to four in flight on as many streams (DFLASH_PREFILL_LANES, 1..8), ordered
+ *     by per-layer events where a block reads the earlier blocks' K/V rows; the caller's stream continues behind all
+ *     of them.
+ * The scratch of both (group buffers; extra streams, scratch sets and contexts' workspaces) belongs to the session and
+ * is made on the first call.  Results equal those of the same blocks through dflash_verify_block bit for bit.  Guards
+ * as dflash_verify_block; on an error kv_n_pos is unchanged. */
+/* Makes the group buffers, extra streams, scratch sets and contexts of dflash_prefill_blocks ahead of its first call (which makes
  * them otherwise): the allocations then stay out of the first prompt's latency.  No counterpart in the reference. */
 int32_t dflash_prefill_prepare(dflash_ctx *ctx, dflash_session *session);
 int32_t dflash_prefill_blocks(dflash_ctx *ctx, const dflash_model *model, dflash_session *session,

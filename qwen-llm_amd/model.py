@@ -515,14 +515,15 @@ class Session:
                             list(host[:n]) if sync else None)
 
     def prepare_prefill(self):
-        """Makes the extra lanes of prefill_blocks now instead of inside its first call."""
+        """Sets up the scratch of prefill_blocks (group buffers, extra lanes) now instead of inside its first call."""
         self._L.dflash_prefill_prepare.restype = C.c_int32
         self._L.dflash_prefill_prepare.argtypes = [C.c_void_p, C.c_void_p]
         self.ctx._check(self._L.dflash_prefill_prepare(self.ctx._h, self._h))
 
     def prefill_blocks(self, tokens, start_position: int, want_hidden=True):
-        """The prompt's blocks without the output head, several blocks in flight on the library's lane streams
-        (dflash_prefill_blocks); returns the tapped hidden rows [n_tokens][n_taps][hidden] (or None).  Enqueue only."""
+        """The prompt's blocks without the output head (dflash_prefill_blocks: a mixture-of-experts target takes the rows
+        of many blocks per pass, any other target several blocks in flight on the library's lane streams); returns the
+        tapped hidden rows [n_tokens][n_taps][hidden] (or None).  Enqueue only."""
         torch = _torch()
         cfg = self.model.cfg
         n = len(tokens)
@@ -782,7 +783,7 @@ class SpeculativeDecoder:
         """Run the prompt through the packed verify in blocks of 16, feed the tapped hidden rows to
         the drafter context, and return the argmax after the last prompt token."""
         assert len(prompt) > 0 and self.position == 0
-        # every block but the last: K/V and the tapped rows only, four blocks in flight; the last one with its head
+        # every block but the last: K/V and the tapped rows only (many blocks per pass, or several in flight); the last one with its head
         body = (len(prompt) - 1) // 16 * 16
         if body:
             hidden = self.session.prefill_blocks(list(prompt[:body]), 0)
