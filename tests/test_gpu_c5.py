@@ -153,18 +153,22 @@ def test_pipelined_prefill_on_the_moe_shape_equals_block_by_block(ctx, weights):
     pipe.close()
 
 
-def test_grouped_prefill_over_several_groups_equals_block_by_block(ctx, weights):
+@pytest.mark.parametrize("n_head,n_toks", [(5, 512 + 16 * 2 + 5), (0, 17), (250, 16 * 3), (9, 512)])
+def test_grouped_prefill_over_several_groups_equals_block_by_block(ctx, weights, n_head, n_toks):
     """A prompt longer than one group of the grouped prefill (512 rows a pass: every projection once for all of them, the
-    experts regrouped by expert) with a ragged tail, started at a position that is not a multiple of 16: captured rows,
-    and the logits of a block that follows (which read every K/V row written), equal block-by-block execution bit for bit."""
+    experts regrouped by expert) with a ragged tail, started at a position that is not a multiple of 16; one block and
+    a row; blocks on both sides of a boundary between attention's context-length buckets; exactly one full pass: captured
+    rows, and the logits of a block that follows (which read every K/V row written), equal block-by-block execution bit
+    for bit."""
     model = dfl.TargetModel(ctx, C5, weights)
     rng = np.random.default_rng(23)
-    head = rng.integers(0, C5.vocab, 5).tolist()
-    toks = rng.integers(0, C5.vocab, 512 + 16 * 2 + 5).tolist()
+    head = rng.integers(0, C5.vocab, n_head).tolist()
+    toks = rng.integers(0, C5.vocab, n_toks).tolist()
     probe = rng.integers(0, C5.vocab, 16).tolist()
     ref, pipe = dfl.Session(ctx, model, 1024, TAPS), dfl.Session(ctx, model, 1024, TAPS)
     for s in (ref, pipe):
-        s.encode_packed_verify_layer_major(head, 0, want_head=False)
+        for h0 in range(0, len(head), 16):
+            s.encode_packed_verify_layer_major(head[h0:h0 + 16], h0, want_head=False)
     got = pipe.prefill_blocks(toks, len(head))
     want = []
     for s0 in range(0, len(toks), 16):
