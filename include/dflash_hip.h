@@ -58,8 +58,9 @@ enum {
 
 /* ggml tensor type tags (crates/qwen-llm/src/tensor.rs:164-208) */
 enum { DFLASH_TYPE_F32 = 0, DFLASH_TYPE_F16 = 1, DFLASH_TYPE_Q8_0 = 8, DFLASH_TYPE_Q4_K = 12, DFLASH_TYPE_Q6_K = 14 };
-/* Not a ggml type: Q4_K blocks in this library's tiled order (dflash_repack_q4k_tiled). */
-enum { DFLASH_TYPE_Q4_K_TILED = 1012 };
+/* Not ggml types: Q4_K blocks in this library's tiled order (dflash_repack_q4k_tiled); Q6_K blocks in its tiled,
+ * field-planar order (dflash_repack_q6k_tiled), which only dflash_gemm_fewrow_xf and the model-level calls take. */
+enum { DFLASH_TYPE_Q4_K_TILED = 1012, DFLASH_TYPE_Q6_K_TILED = 1014 };
 
 /* ---- context ------------------------------------------------------------------
  * Replaces MetalContext + the per-call scratch the reference keeps in
@@ -149,6 +150,16 @@ int32_t dflash_check_scale_range(dflash_ctx *ctx, int32_t type, const void *bloc
 size_t dflash_q4k_tiled_bytes(int64_t n_in, int64_t n_out);
 int32_t dflash_repack_q4k_tiled(dflash_ctx *ctx, const void *w, void *w_tiled, int64_t n_in, int64_t n_out,
                                 dflash_stream_t stream);
+/* The same idea for Q6_K matrices that only the one-launch GEMM below (dflash_gemm_fewrow_xf and the model-level
+ * calls) reads - a 2048-wide model's attention projections: [tile group of 256 rows][super-block][tile 0..15][3360
+ * bytes], a tile's sixteen 210-byte blocks stored field by field (ql [row][128], qh [row][64], scales [row][16],
+ * d [row]) so that every 16-byte piece a lane fetches is aligned; same values, bit-identical Y.  w_type
+ * DFLASH_TYPE_Q6_K_TILED.  dflash_gemm_fewrow does NOT take this type (DFLASH_ERR_UNSUPPORTED): tile a matrix only
+ * where dflash_gemm_fewrow_xf_kind(ctx, DFLASH_TYPE_Q6_K_TILED, n_in, n_out) is not DFLASH_XF_NONE.  Source 2-byte,
+ * destination 128-byte aligned; range-checked first, as above.  Blocking. */
+size_t dflash_q6k_tiled_bytes(int64_t n_in, int64_t n_out);
+int32_t dflash_repack_q6k_tiled(dflash_ctx *ctx, const void *w, void *w_tiled, int64_t n_in, int64_t n_out,
+                                dflash_stream_t stream);
 
 /* ---- few-row quantised GEMM ---------------------------------------------------
  * encode_mat_mat_dispatch_dflash_verify(ctx, enc, weight, x, y, n_in, n_out, n_query)
@@ -194,8 +205,8 @@ const char *dflash_gemm_fewrow_noalloc_error(void);
  * calls expose it.
  *   dflash_xf_bytes: size of an XF buffer for n_in values per row (n_in % 256 == 0; 0 otherwise).
  *   dflash_gemm_fewrow_xf_kind: the XF kind (DFLASH_XF_Q4K / DFLASH_XF_Q6K) this (type, shape) reads, or
- *     DFLASH_XF_NONE where it is not taken: w_type must be DFLASH_TYPE_Q4_K_TILED or DFLASH_TYPE_Q6_K |
- *     DFLASH_TYPE_RANGE_CHECKED (these kernels scale in f16: a range-checked tensor only), n_in at most 8192, and
+ *     DFLASH_XF_NONE where it is not taken: w_type must be DFLASH_TYPE_Q4_K_TILED, DFLASH_TYPE_Q6_K_TILED or
+ *     DFLASH_TYPE_Q6_K | DFLASH_TYPE_RANGE_CHECKED (these kernels scale in f16: a range-checked tensor only), n_in at most 8192, and
  *     the matrix at most one round of the chip (about 320 workgroups of 16 or 32 rows).
  *   dflash_pack_xf: row-major x[n_rows][n_in] (f32 or f16) -> xf, rounding to f16 as every few-row kernel does.
  *   dflash_gemm_fewrow_xf: Y[n_rows][n_out] = X . W^T; same guards as dflash_gemm_fewrow; DFLASH_ERR_UNSUPPORTED

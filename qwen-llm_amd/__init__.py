@@ -19,6 +19,7 @@ from .binding import (  # noqa: F401
     TYPE_F32,
     TYPE_Q4_K,
     TYPE_Q4_K_TILED,
+    TYPE_Q6_K_TILED,
     TYPE_Q6_K,
     TYPE_Q8_0,
     TYPE_RANGE_CHECKED,

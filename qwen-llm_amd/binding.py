@@ -15,6 +15,7 @@ HEADER_PATH = os.path.join(PKG_DIR, "..", "include", "dflash_hip.h")
 
 TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q6_K = 0, 1, 8, 12, 14
 TYPE_Q4_K_TILED = 1012  # Q4_K blocks in the library's tiled order (Context.repack_q4k_tiled)
+TYPE_Q6_K_TILED = 1014  # Q6_K blocks in the library's tiled, field-planar order (Context.repack_q6k_tiled): gemm_fewrow_xf only
 XF_NONE, XF_Q4K, XF_Q6K = 0, 1, 2  # fragment orders of Context.pack_xf
 TYPE_RANGE_CHECKED = 0x10000  # OR-ed into a w_type: the tensor passed Context.check_scale_range (fast Q4_K / Q6_K kernels)
 QT_RANGE_CHECKED = 1  # the same fact in a dflash_qtensor's flags
@@ -127,6 +128,10 @@ def _declare(L):
     L.dflash_q4k_tiled_bytes.argtypes = [i64, i64]
     L.dflash_repack_q4k_tiled.restype = i32
     L.dflash_repack_q4k_tiled.argtypes = [vp, vp, vp, i64, i64, vp]
+    L.dflash_q6k_tiled_bytes.restype = sz
+    L.dflash_q6k_tiled_bytes.argtypes = [i64, i64]
+    L.dflash_repack_q6k_tiled.restype = i32
+    L.dflash_repack_q6k_tiled.argtypes = [vp, vp, vp, i64, i64, vp]
     L.dflash_xf_bytes.restype = sz
     L.dflash_xf_bytes.argtypes = [i64]
     L.dflash_gemm_fewrow_xf_kind.restype = i32
@@ -333,6 +338,17 @@ class Context:
             raise DFlashError(2, f"bad Q4_K shape {n_out} x {n_in}")
         out = _empty(nbytes, dtype=torch.uint8, device=weight.device)
         self._check(self._lib.dflash_repack_q4k_tiled(self._h, weight.data_ptr(), out.data_ptr(), n_in, n_out, _stream_ptr()))
+        return out
+
+    def repack_q6k_tiled(self, weight, n_in: int, n_out: int):
+        """Q6_K blocks in GGUF row order -> a new tensor in the tiled, field-planar order (w_type TYPE_Q6_K_TILED), which
+        gemm_fewrow_xf (and the model-level calls) read with aligned loads; bit-identical results."""
+        torch = _torch()
+        nbytes = self._lib.dflash_q6k_tiled_bytes(n_in, n_out)
+        if nbytes == 0:
+            raise DFlashError(2, f"bad Q6_K shape {n_out} x {n_in}")
+        out = _empty(nbytes, dtype=torch.uint8, device=weight.device)
+        self._check(self._lib.dflash_repack_q6k_tiled(self._h, weight.data_ptr(), out.data_ptr(), n_in, n_out, _stream_ptr()))
         return out
 
     def gemm_fewrow(self, weight, w_type: int, x, n_in: int, n_out: int):

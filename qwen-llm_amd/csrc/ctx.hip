@@ -169,7 +169,9 @@ size_t dflash_row_bytes(int32_t type, size_t n_in) {
     case DFLASH_TYPE_Q4_K:
     case DFLASH_TYPE_Q4_K_TILED:  // (a tiled matrix of a multiple of 256 rows is as long as its row-order original)
         return n_in % DFL_QK_K ? 0 : n_in / DFL_QK_K * DFL_Q4_K_BYTES;
-    case DFLASH_TYPE_Q6_K: return n_in % DFL_QK_K ? 0 : n_in / DFL_QK_K * DFL_Q6_K_BYTES;
+    case DFLASH_TYPE_Q6_K:
+    case DFLASH_TYPE_Q6_K_TILED:  // (likewise)
+        return n_in % DFL_QK_K ? 0 : n_in / DFL_QK_K * DFL_Q6_K_BYTES;
     case DFLASH_TYPE_Q8_0: return n_in % DFL_QK8_0 ? 0 : n_in / DFL_QK8_0 * DFL_Q8_0_BYTES;
     case DFLASH_TYPE_F32: return n_in * 4;
     case DFLASH_TYPE_F16: return n_in * 2;

@@ -2900,6 +2900,9 @@ int32_t gemm_fewrow_impl(dflash_ctx *ctx, int32_t w_type, const void *w, const v
     const bool plain = w_type == DFLASH_TYPE_F32 || w_type == DFLASH_TYPE_F16;
     const bool tiled = w_type == DFLASH_TYPE_Q4_K_TILED;
     if (tiled) w_type = DFLASH_TYPE_Q4_K;
+    if (w_type == DFLASH_TYPE_Q6_K_TILED)
+        return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED,
+                        "gemm_fewrow: a tiled Q6_K tensor is read by dflash_gemm_fewrow_xf (and the model-level calls) only");
     if (w_type != DFLASH_TYPE_Q4_K && w_type != DFLASH_TYPE_Q6_K && w_type != DFLASH_TYPE_Q8_0 && !plain)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow: weight type %d has no few-row kernel", w_type);
     const int64_t blk = (w_type == DFLASH_TYPE_Q8_0 || plain) ? DFL_QK8_0 : DFL_QK_K;

@@ -163,8 +163,15 @@ __device__ __forceinline__ void load_w(Q6W &r, const WholeArgs &a, int tile, int
     }
     r.d = *reinterpret_cast<const uint16_t *>(base + static_cast<size_t>(min(tile * 16 + (lane & 15), last)) * a.row_bytes + 208);
 }
-__device__ __forceinline__ void compute(const Q6W &r, const half8_t (&af)[8], int lane, uint8_t *area, uint32_t, Q4KMagic magic,
-                                        float4_t &acc, float4_t &acc_sub) {
+// A lane's operands of one super-block of one weight row (lane (n, g): half h = g / 2, quarters (g & 1) and 2 + (g & 1)):
+// 32 bytes of ql, 32 of qh, the four scales of its two quarters and d.
+struct Q6Ops {
+    u32x4_t qa, qb, ha, hb;
+    uint32_t sc4, sc4h;  // low 16 bits: the two int8 scales of the low (high) quarter
+    float d;
+};
+// The lane's operands out of a wave-private LDS area that holds the tile's sixteen raw 210-byte blocks, rows 240 bytes apart.
+__device__ __forceinline__ Q6Ops q6_stage_through_lds(const Q6W &r, int lane, uint8_t *area) {
     const int n = lane & 15, g = lane >> 4, h = g >> 1, odd = g & 1;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -174,27 +181,33 @@ __device__ __forceinline__ void compute(const Q6W &r, const half8_t (&af)[8], in
     if (lane < 16) *reinterpret_cast<uint16_t *>(area + lane * kQ6RowStride + 208) = static_cast<uint16_t>(r.d);
     __builtin_amdgcn_wave_barrier();
     const uint8_t *rowp = area + n * kQ6RowStride;
-    const u32x4_t qa = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd);
-    const u32x4_t qb = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd + 16);
-    const u32x4_t ha = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h);
-    const u32x4_t hb = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h + 16);
-    const uint32_t sc4 = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h) >> (16 * odd)) & 0xffffu;
-    const uint32_t sc4h = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h + 4) >> (16 * odd)) & 0xffffu;
-    const float d = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(rowp + 208)));
+    Q6Ops o;
+    o.qa = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd);
+    o.qb = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd + 16);
+    o.ha = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h);
+    o.hb = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h + 16);
+    o.sc4 = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h) >> (16 * odd)) & 0xffffu;
+    o.sc4h = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h + 4) >> (16 * odd)) & 0xffffu;
+    o.d = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(rowp + 208)));
     __builtin_amdgcn_wave_barrier();  // (the area is rewritten by this wave's next tile only after these reads: LDS runs a wave's accesses in order)
+    return o;
+}
+__device__ __forceinline__ void q6_compute(const Q6Ops &o, const half8_t (&af)[8], int lane, Q4KMagic magic, float4_t &acc, float4_t &acc_sub) {
+    const int odd = (lane >> 4) & 1;
     const int hs = 2 * odd;
-    const uint32_t hq[8] = {ha.x >> hs, ha.y >> hs, ha.z >> hs, ha.w >> hs, hb.x >> hs, hb.y >> hs, hb.z >> hs, hb.w >> hs};
-    const uint32_t ql[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+    const uint32_t hq[8] = {o.ha.x >> hs, o.ha.y >> hs, o.ha.z >> hs, o.ha.w >> hs, o.hb.x >> hs, o.hb.y >> hs, o.hb.z >> hs, o.hb.w >> hs};
+    const uint32_t ql[8] = {o.qa.x, o.qa.y, o.qa.z, o.qa.w, o.qb.x, o.qb.y, o.qb.z, o.qb.w};
+    const float d = o.d;
     auto scale = [&](uint32_t pair, int j) { return static_cast<_Float16>(d * static_cast<float>(static_cast<int8_t>(pair >> (8 * j)))); };
-    const _Float16 s_l0 = scale(sc4, 0), s_l1 = scale(sc4, 1), s_h0 = scale(sc4h, 0), s_h1 = scale(sc4h, 1);
+    const _Float16 s_l0 = scale(o.sc4, 0), s_l1 = scale(o.sc4, 1), s_h0 = scale(o.sc4h, 0), s_h1 = scale(o.sc4h, 1);
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         const _Float16 sl = (t >> 1) ? s_l1 : s_l0;
         const half8_t bl = unpack6<false>(ql[2 * t], ql[2 * t + 1], hq[2 * t], hq[2 * t + 1], splat(sl),
                                           splat(sl * static_cast<_Float16>(-1024.0f)), magic.lo);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bl, acc, 0, 0, 0);
-        const _Float16 o = sl * static_cast<_Float16>(32.0f);
-        const half8_t bo = {o, o, o, o, o, o, o, o};
+        const _Float16 of = sl * static_cast<_Float16>(32.0f);
+        const half8_t bo = {of, of, of, of, of, of, of, of};
         acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t], bo, acc_sub, 0, 0, 0);
     }
 #pragma unroll
@@ -203,39 +216,71 @@ __device__ __forceinline__ void compute(const Q6W &r, const half8_t (&af)[8], in
         const half8_t bh = unpack6<true>(ql[2 * t], ql[2 * t + 1], hq[2 * t] >> 4, hq[2 * t + 1] >> 4, splat(sh),
                                          splat(sh * static_cast<_Float16>(-64.0f)), magic.hi);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bh, acc, 0, 0, 0);
-        const _Float16 o = sh * static_cast<_Float16>(32.0f);
-        const half8_t bo = {o, o, o, o, o, o, o, o};
+        const _Float16 of = sh * static_cast<_Float16>(32.0f);
+        const half8_t bo = {of, of, of, of, of, of, of, of};
         acc_sub = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[4 + t], bo, acc_sub, 0, 0, 0);
     }
+}
+__device__ __forceinline__ void compute(const Q6W &r, const half8_t (&af)[8], int lane, uint8_t *area, uint32_t, Q4KMagic magic,
+                                        float4_t &acc, float4_t &acc_sub) {
+    q6_compute(q6_stage_through_lds(r, lane, area), af, lane, magic, acc, acc_sub);
+}
+
+// ---- Q6_K, tiled and field-planar: [tile group of 256 rows][super-block][tile 0..15][3360 bytes], a tile's sixteen
+// blocks as four sections - ql [row][128], qh [row][64], scales [row][16], d [row] (f16) - every 16-byte piece aligned.
+// The 16-byte pieces of a row's ql (qh) sit at piece index p ^ (row & 7) (p ^ ((row >> 1) & 3)): a layout that a wave
+// can also read from LDS without bank conflicts.  Lane (n, g) fetches exactly its operands: four 16-byte loads, one of
+// 8 bytes, one of 2, all aligned, a row's ql line shared by the four lanes of the row - no staging, no LDS.
+constexpr int kQ6TileBytes = 16 * DFL_Q6_K_BYTES;  // 3360
+constexpr int kQ6TQh = 2048, kQ6TSc = 3072, kQ6TD = 3328;
+struct Q6T {
+    u32x4_t qa, qb, ha, hb;
+    uint32_t s0, s1;
+    uint32_t d;
+};
+__host__ __device__ __forceinline__ int q6t_ql_piece(int row, int p) { return row * 128 + ((p ^ (row & 7)) << 4); }
+__host__ __device__ __forceinline__ int q6t_qh_piece(int row, int p) { return kQ6TQh + row * 64 + ((p ^ ((row >> 1) & 3)) << 4); }
+__device__ __forceinline__ void load_w(Q6T &r, const WholeArgs &a, int tile, int b, int lane) {
+    const int n = lane & 15, g = lane >> 4, h = g >> 1, odd = g & 1;
+    const uint8_t *p = a.w + ((static_cast<size_t>(tile >> 4) * a.nb + b) * 16 + (tile & 15)) * kQ6TileBytes;
+    r.qa = *reinterpret_cast<const u32x4_t *>(p + q6t_ql_piece(n, 4 * h + 2 * odd));
+    r.qb = *reinterpret_cast<const u32x4_t *>(p + q6t_ql_piece(n, 4 * h + 2 * odd + 1));
+    r.ha = *reinterpret_cast<const u32x4_t *>(p + q6t_qh_piece(n, 2 * h));
+    r.hb = *reinterpret_cast<const u32x4_t *>(p + q6t_qh_piece(n, 2 * h + 1));
+    const uint2 sc = *reinterpret_cast<const uint2 *>(p + kQ6TSc + n * 16 + 8 * h);
+    r.s0 = sc.x;
+    r.s1 = sc.y;
+    r.d = *reinterpret_cast<const uint16_t *>(p + kQ6TD + n * 2);
+}
+__device__ __forceinline__ Q6Ops q6_ops(const Q6T &r, int lane) {
+    const int odd = (lane >> 4) & 1;
+    Q6Ops o;
+    o.qa = r.qa;
+    o.qb = r.qb;
+    o.ha = r.ha;
+    o.hb = r.hb;
+    o.sc4 = (r.s0 >> (16 * odd)) & 0xffffu;
+    o.sc4h = (r.s1 >> (16 * odd)) & 0xffffu;
+    o.d = __half2float(__ushort_as_half(static_cast<uint16_t>(r.d)));
+    return o;
+}
+__device__ __forceinline__ void compute(const Q6T &r, const half8_t (&af)[8], int lane, uint8_t *, uint32_t, Q4KMagic magic, float4_t &acc,
+                                        float4_t &acc_sub) {
+    q6_compute(q6_ops(r, lane), af, lane, magic, acc, acc_sub);
 }
 
 struct Q6F {
     half8_t b[8];
     _Float16 o[4];  // 32 s of the four scale pairs: low quarter's two, high quarter's two
 };
-__device__ __forceinline__ void unpack(const Q6W &r, int lane, uint8_t *area, uint32_t, Q4KMagic magic, Q6F &f) {
-    const int n = lane & 15, g = lane >> 4, h = g >> 1, odd = g & 1;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int i = lane + 64 * j;
-        if (i < 208) *reinterpret_cast<u32x4_t *>(area + (i / 13) * kQ6RowStride + 16 * (i % 13)) = r.p[j];
-    }
-    if (lane < 16) *reinterpret_cast<uint16_t *>(area + lane * kQ6RowStride + 208) = static_cast<uint16_t>(r.d);
-    __builtin_amdgcn_wave_barrier();
-    const uint8_t *rowp = area + n * kQ6RowStride;
-    const u32x4_t qa = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd);
-    const u32x4_t qb = *reinterpret_cast<const u32x4_t *>(rowp + 64 * h + 32 * odd + 16);
-    const u32x4_t ha = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h);
-    const u32x4_t hb = *reinterpret_cast<const u32x4_t *>(rowp + 128 + 32 * h + 16);
-    const uint32_t sc4 = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h) >> (16 * odd)) & 0xffffu;
-    const uint32_t sc4h = (*reinterpret_cast<const uint32_t *>(rowp + 192 + 8 * h + 4) >> (16 * odd)) & 0xffffu;
-    const float d = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(rowp + 208)));
-    __builtin_amdgcn_wave_barrier();
+__device__ __forceinline__ void q6_unpack(const Q6Ops &o, int lane, Q4KMagic magic, Q6F &f) {
+    const int odd = (lane >> 4) & 1;
     const int hs = 2 * odd;
-    const uint32_t hq[8] = {ha.x >> hs, ha.y >> hs, ha.z >> hs, ha.w >> hs, hb.x >> hs, hb.y >> hs, hb.z >> hs, hb.w >> hs};
-    const uint32_t ql[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+    const uint32_t hq[8] = {o.ha.x >> hs, o.ha.y >> hs, o.ha.z >> hs, o.ha.w >> hs, o.hb.x >> hs, o.hb.y >> hs, o.hb.z >> hs, o.hb.w >> hs};
+    const uint32_t ql[8] = {o.qa.x, o.qa.y, o.qa.z, o.qa.w, o.qb.x, o.qb.y, o.qb.z, o.qb.w};
+    const float d = o.d;
     auto scale = [&](uint32_t pair, int j) { return static_cast<_Float16>(d * static_cast<float>(static_cast<int8_t>(pair >> (8 * j)))); };
-    const _Float16 s_l0 = scale(sc4, 0), s_l1 = scale(sc4, 1), s_h0 = scale(sc4h, 0), s_h1 = scale(sc4h, 1);
+    const _Float16 s_l0 = scale(o.sc4, 0), s_l1 = scale(o.sc4, 1), s_h0 = scale(o.sc4h, 0), s_h1 = scale(o.sc4h, 1);
     const _Float16 k32 = static_cast<_Float16>(32.0f);
     f.o[0] = s_l0 * k32;
     f.o[1] = s_l1 * k32;
@@ -249,6 +294,12 @@ __device__ __forceinline__ void unpack(const Q6W &r, int lane, uint8_t *area, ui
         f.b[4 + t] = unpack6<true>(ql[2 * t], ql[2 * t + 1], hq[2 * t] >> 4, hq[2 * t + 1] >> 4, splat(sh),
                                    splat(sh * static_cast<_Float16>(-64.0f)), magic.hi);
     }
+}
+__device__ __forceinline__ void unpack(const Q6W &r, int lane, uint8_t *area, uint32_t, Q4KMagic magic, Q6F &f) {
+    q6_unpack(q6_stage_through_lds(r, lane, area), lane, magic, f);
+}
+__device__ __forceinline__ void unpack(const Q6T &r, int lane, uint8_t *, uint32_t, Q4KMagic magic, Q6F &f) {
+    q6_unpack(q6_ops(r, lane), lane, magic, f);
 }
 __device__ __forceinline__ void mma(const Q6F &f, const half8_t (&af)[8], float4_t &acc, float4_t &acc_sub) {
 #pragma unroll
@@ -267,6 +318,10 @@ struct FragsOf<Q4W> {
 };
 template <>
 struct FragsOf<Q6W> {
+    typedef Q6F type;
+};
+template <>
+struct FragsOf<Q6T> {
     typedef Q6F type;
 };
 
@@ -444,7 +499,9 @@ struct WholePlan {
 WholePlan whole_plan(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out, int64_t pair_ffn) {
     WholePlan p = {DFL_XF_NONE, 0, 0, 0, 0, 0};
     if (!env_int("DFLASH_GEMM_WHOLE", 1)) return p;
-    const int kind = w_type == DFLASH_TYPE_Q4_K_TILED ? DFL_XF_Q4K : w_type == DFLASH_TYPE_Q6_K ? DFL_XF_Q6K : DFL_XF_NONE;
+    const int kind = w_type == DFLASH_TYPE_Q4_K_TILED ? DFL_XF_Q4K
+                     : (w_type == DFLASH_TYPE_Q6_K || w_type == DFLASH_TYPE_Q6_K_TILED) ? DFL_XF_Q6K
+                                                                                       : DFL_XF_NONE;
     if (kind == DFL_XF_NONE || n_in <= 0 || n_in % DFL_QK_K || n_out <= 0 || n_out >= (1 << 24)) return p;
     const int nb = static_cast<int>(n_in / DFL_QK_K);
     if (nb > 32) return p;  // more than two stages per wave
@@ -486,7 +543,8 @@ int32_t dfl_gemm_whole_blocks(dflash_ctx *ctx, int32_t w_type, const void *w, co
                                                static_cast<long long>(n_in), static_cast<long long>(n_out));
     if (!w || !xf || n_rows < 1 || n_rows > 16 || (!y && !(pair_ffn && y_xf)))
         return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "gemm_whole: null operand or n_rows %d", n_rows);
-    if (reinterpret_cast<uintptr_t>(xf) % 16 || reinterpret_cast<uintptr_t>(w) % (p.kind == DFL_XF_Q4K ? 16 : 2) ||
+    const bool q6_tiled = w_type == DFLASH_TYPE_Q6_K_TILED;
+    if (reinterpret_cast<uintptr_t>(xf) % 16 || reinterpret_cast<uintptr_t>(w) % ((p.kind == DFL_XF_Q4K || q6_tiled) ? 16 : 2) ||
         (y_xf && reinterpret_cast<uintptr_t>(y_xf) % 16))
         return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "gemm_whole: operand alignment");
     if (y_xf && (!pair_ffn || (y_xf_kind != DFL_XF_Q4K && y_xf_kind != DFL_XF_Q6K)))
@@ -512,11 +570,12 @@ int32_t dfl_gemm_whole_blocks(dflash_ctx *ctx, int32_t w_type, const void *w, co
     a.y_stride = static_cast<size_t>(16) * (pair_ffn ? pair_ffn : n_out);
     const int threads = 64 * p.ksplit * p.tl;
     const size_t red_bytes = static_cast<size_t>(16) * p.R * 64 * sizeof(float4_t);
-    const size_t lds = red_bytes + (p.kind == DFL_XF_Q6K ? static_cast<size_t>(16) * kQ6AreaBytes : 0);
+    const size_t lds = red_bytes + ((p.kind == DFL_XF_Q6K && !q6_tiled) ? static_cast<size_t>(16) * kQ6AreaBytes : 0);
     typedef void (*kernel_t)(WholeArgs);
     const int multi = n_blocks > 1 ? (a.nb > p.ksplit ? 2 : 1) : 0;
 #define DFL_WHOLE_PICK(WT, RR) (multi == 0 ? gemm_whole_kernel<WT, RR, 0> : multi == 1 ? gemm_whole_kernel<WT, RR, 1> : gemm_whole_kernel<WT, RR, 2>)
     const kernel_t fn = p.kind == DFL_XF_Q4K ? (p.R == 2 ? DFL_WHOLE_PICK(Q4W, 2) : DFL_WHOLE_PICK(Q4W, 1))
+                        : q6_tiled           ? (p.R == 2 ? DFL_WHOLE_PICK(Q6T, 2) : DFL_WHOLE_PICK(Q6T, 1))
                                              : (p.R == 2 ? DFL_WHOLE_PICK(Q6W, 2) : DFL_WHOLE_PICK(Q6W, 1));
 #undef DFL_WHOLE_PICK
     if (lds > ctx->lds_bytes) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: %zu bytes of LDS needed", lds);
@@ -528,13 +587,68 @@ int32_t dfl_gemm_whole_blocks(dflash_ctx *ctx, int32_t w_type, const void *w, co
     return DFLASH_OK;
 }
 
+namespace {
+// One thread per (row, super-block) of the tiled matrix: the row-order block's fields to their places (rows past the
+// matrix: zero blocks, d = 0).
+__global__ void __launch_bounds__(256)
+    q6k_repack_tiled_kernel(const uint8_t *__restrict__ w, uint8_t *__restrict__ out, int n_out, int nb, int64_t n_items) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n_items) return;
+    const int b = static_cast<int>(i % nb);
+    const int64_t row = i / nb;
+    const int tile = static_cast<int>(row >> 4), r = static_cast<int>(row & 15);
+    uint8_t *t = out + ((static_cast<size_t>(tile >> 4) * nb + b) * 16 + (tile & 15)) * kQ6TileBytes;
+    const bool live = row < n_out;
+    const uint8_t *src = w + (static_cast<size_t>(live ? row : 0) * nb + b) * DFL_Q6_K_BYTES;  // 2-byte aligned
+    const uint16_t *s16 = reinterpret_cast<const uint16_t *>(src);
+    auto put = [&](int dst_off, int src_off16) {  // one 16-byte piece
+        uint16_t *d16 = reinterpret_cast<uint16_t *>(t + dst_off);
+        for (int k = 0; k < 8; k++) d16[k] = live ? s16[src_off16 + k] : static_cast<uint16_t>(0);
+    };
+    for (int p = 0; p < 8; p++) put(q6t_ql_piece(r, p), 8 * p);
+    for (int p = 0; p < 4; p++) put(q6t_qh_piece(r, p), 64 + 8 * p);
+    put(kQ6TSc + r * 16, 96);
+    *reinterpret_cast<uint16_t *>(t + kQ6TD + r * 2) = live ? s16[104] : static_cast<uint16_t>(0);
+}
+}  // namespace
+
+extern "C" size_t dflash_q6k_tiled_bytes(int64_t n_in, int64_t n_out) {
+    if (n_in <= 0 || n_out <= 0 || n_in % DFL_QK_K) return 0;
+    const size_t groups = (static_cast<size_t>(n_out) + 255) / 256;
+    return groups * static_cast<size_t>(n_in / DFL_QK_K) * 16 * kQ6TileBytes;
+}
+
+extern "C" int32_t dflash_repack_q6k_tiled(dflash_ctx *ctx, const void *w, void *w_tiled, int64_t n_in, int64_t n_out,
+                                           dflash_stream_t stream) {
+    if (!ctx) return DFLASH_ERR_INVALID_INPUT;
+    if (!w || !w_tiled) return dfl_fail(ctx, DFLASH_ERR_INVALID_INPUT, "repack_q6k_tiled: null pointer");
+    if (n_in <= 0 || n_out <= 0 || n_in % DFL_QK_K || n_in > 0x7fffffffll || n_out > 0x7fffffffll)
+        return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "repack_q6k_tiled: n_in %lld / n_out %lld", static_cast<long long>(n_in),
+                        static_cast<long long>(n_out));
+    if (reinterpret_cast<uintptr_t>(w) % 2 || reinterpret_cast<uintptr_t>(w_tiled) % 128)
+        return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "repack_q6k_tiled: source must be 2-byte, destination 128-byte aligned");
+    const size_t out_bytes = dflash_q6k_tiled_bytes(n_in, n_out);
+    const int nb = static_cast<int>(n_in / DFL_QK_K);
+    const size_t in_bytes = static_cast<size_t>(n_out) * nb * DFL_Q6_K_BYTES;
+    if (dfl_ranges_overlap(w_tiled, out_bytes, w, in_bytes)) return dfl_fail(ctx, DFLASH_ERR_ALIAS, "repack_q6k_tiled: buffers overlap");
+    // a tiled tensor goes to the fast kernels unconditionally: it must be one they can take
+    if (const int32_t rc = dflash_check_scale_range(ctx, DFLASH_TYPE_Q6_K, w, in_bytes / DFL_Q6_K_BYTES, nullptr, stream)) return rc;
+    const int64_t n_items = static_cast<int64_t>((static_cast<size_t>(n_out) + 255) / 256 * 256) * nb;
+    const int64_t blocks = (n_items + 255) / 256;
+    if (blocks > 0x7fffffffll) return dfl_fail(ctx, DFLASH_ERR_BAD_SHAPE, "repack_q6k_tiled: matrix too large");
+    q6k_repack_tiled_kernel<<<static_cast<unsigned>(blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint8_t *>(w), static_cast<uint8_t *>(w_tiled), static_cast<int>(n_out), nb, n_items);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
+}
+
 extern "C" size_t dflash_xf_bytes(int64_t n_in) { return n_in > 0 && n_in % DFL_QK_K == 0 ? dfl_xf_bytes(n_in) : 0; }
 
 namespace {
 // The public entries take a range-checked tensor only (there is no f32 kernel behind them): the tiled order, or
 // DFLASH_TYPE_Q6_K | DFLASH_TYPE_RANGE_CHECKED.  Returns the bare type, or -1.
 int32_t xf_public_type(int32_t w_type) {
-    if (w_type == DFLASH_TYPE_Q4_K_TILED) return w_type;
+    if (w_type == DFLASH_TYPE_Q4_K_TILED || w_type == DFLASH_TYPE_Q6_K_TILED) return w_type;
     if (w_type == (DFLASH_TYPE_Q6_K | DFLASH_TYPE_RANGE_CHECKED)) return DFLASH_TYPE_Q6_K;
     return -1;
 }
@@ -573,14 +687,16 @@ extern "C" int32_t dflash_gemm_fewrow_xf(dflash_ctx *ctx, int32_t w_type, const 
     w_type = xf_public_type(tagged);
     if (w_type < 0)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED,
-                        "gemm_fewrow_xf: type tag %d: only DFLASH_TYPE_Q4_K_TILED and DFLASH_TYPE_Q6_K | DFLASH_TYPE_RANGE_CHECKED "
-                        "(a tensor that passed dflash_check_scale_range) are taken",
+                        "gemm_fewrow_xf: type tag %d: only DFLASH_TYPE_Q4_K_TILED, DFLASH_TYPE_Q6_K_TILED and DFLASH_TYPE_Q6_K | "
+                        "DFLASH_TYPE_RANGE_CHECKED (a tensor that passed dflash_check_scale_range) are taken",
                         tagged);
     if (dfl_whole_kind(ctx, w_type, n_in, n_out, 0) == DFL_XF_NONE)
         return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_fewrow_xf: type %d, %lld -> %lld is not taken by the whole-K kernels", w_type,
                         static_cast<long long>(n_in), static_cast<long long>(n_out));
     if (n_in > 0 && n_out > 0 && y && xf && w) {
-        const size_t wb = w_type == DFLASH_TYPE_Q4_K_TILED ? dflash_q4k_tiled_bytes(n_in, n_out) : dflash_row_bytes(w_type, n_in) * n_out;
+        const size_t wb = w_type == DFLASH_TYPE_Q4_K_TILED   ? dflash_q4k_tiled_bytes(n_in, n_out)
+                          : w_type == DFLASH_TYPE_Q6_K_TILED ? dflash_q6k_tiled_bytes(n_in, n_out)
+                                                             : dflash_row_bytes(w_type, n_in) * n_out;
         const size_t yb = static_cast<size_t>(n_rows > 0 ? n_rows : 1) * n_out * sizeof(float);
         if (dfl_ranges_overlap(y, yb, xf, dfl_xf_bytes(n_in)) || dfl_ranges_overlap(y, yb, w, wb))
             return dfl_fail(ctx, DFLASH_ERR_ALIAS, "gemm_fewrow_xf: y aliases an input");

@@ -16,7 +16,7 @@ import numpy as np
 
 from . import synth
 from . import binding as _binding
-from .binding import QT_RANGE_CHECKED, TYPE_Q4_K, TYPE_Q4_K_TILED, CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
+from .binding import QT_RANGE_CHECKED, TYPE_Q4_K, TYPE_Q4_K_TILED, TYPE_Q6_K, TYPE_Q6_K_TILED, XF_NONE, CodebookC, Context, DFlashError, _stream_ptr, _torch, lib
 
 
 @dataclass
@@ -314,14 +314,17 @@ def synth_draft_weights_device(cfg: DraftConfig, seed: int, device, wtype: int =
 # ---- device-resident weights ----
 
 class _Uploader:
-    def __init__(self, device, ctx=None, tiled=True):
+    def __init__(self, device, ctx=None, tiled=True, tile_q6k=False):
         """``ctx``: when given, every Q4_K / Q6_K tensor's super-block scales are range-checked on upload (a tensor the
         few-row kernels cannot take is declined with DFlashError) and, with ``tiled``, Q4_K matrices uploaded with a
-        tile shape are repacked into the tiled order."""
+        tile shape are repacked into the tiled order.  ``tile_q6k``: Q6_K matrices uploaded with a tile shape that the
+        one-launch GEMM takes (``Context.xf_kind``) go into the tiled Q6_K order as well (only that GEMM reads it: for
+        tensors nothing else multiplies, i.e. a target's attention projections)."""
         self.torch = _torch()
         self.device = device
         self.ctx = ctx
         self.tiled = tiled and ctx is not None and not os.environ.get("DFLASH_NO_TILED")  # (the variable: for A/B runs)
+        self.tile_q6k = tile_q6k and self.tiled and not os.environ.get("DFLASH_NO_TILED_Q6K")
         self.keep = []
         self.n_tiled = 0  # uploads that went into the tiled order
 
@@ -352,7 +355,7 @@ class _Uploader:
         self.keep.append(t)
         return t.data_ptr()
 
-    def q(self, pair, tile_shape=None):
+    def q(self, pair, tile_shape=None, allow_q6k=False):
         """``tile_shape`` = (n_out, n_in): a Q4_K matrix that only the few-row GEMM reads is repacked into the
         library's tiled order (a permutation of whole blocks, bit-identical products, faster streaming)."""
         if pair is None:
@@ -367,17 +370,22 @@ class _Uploader:
             t = self.ctx.repack_q4k_tiled(t, tile_shape[1], tile_shape[0])
             qtype = TYPE_Q4_K_TILED
             self.n_tiled += 1
+        elif (tile_shape is not None and allow_q6k and self.tile_q6k and int(qtype) == TYPE_Q6_K
+              and self.ctx.xf_kind(TYPE_Q6_K_TILED, tile_shape[1], tile_shape[0]) != XF_NONE):
+            t = self.ctx.repack_q6k_tiled(t, tile_shape[1], tile_shape[0])
+            qtype = TYPE_Q6_K_TILED
+            self.n_tiled += 1
         self.keep.append(t)
         return QTensorC(int(qtype), flags, t.data_ptr())
 
-    def q_adjacent(self, pairs, tile_shapes=None):
+    def q_adjacent(self, pairs, tile_shapes=None, allow_q6k=False):
         """Uploads matrices of one type and one row length back to back in a single allocation (rows of the
         first, then the second, ...): the library then runs a layer's wq/wk/wv (or gate/up) as ONE GEMM.
         Falls back to separate uploads when the types differ.  ``tile_shapes`` = [(n_out, n_in), ...]: Q4_K sets
         whose row counts are all multiples of 256 are repacked as one tiled matrix (tile groups are 256 rows, so
         every member still starts where its row-order address arithmetic says)."""
         if any(p is None for p in pairs) or len({int(p[0]) for p in pairs}) != 1:
-            return [self.q(p, ts) for p, ts in zip(pairs, tile_shapes or [None] * len(pairs))]
+            return [self.q(p, ts) for p, ts in zip(pairs, tile_shapes or [None] * len(pairs))]  # (never the tiled Q6_K order: separate launches)
         torch = self.torch
         flats = []
         for _, blocks in pairs:
@@ -392,6 +400,12 @@ class _Uploader:
                 and all(ts is not None and ts[0] % 256 == 0 for ts in tile_shapes)):
             whole = self.ctx.repack_q4k_tiled(whole, tile_shapes[0][1], sum(ts[0] for ts in tile_shapes))
             qtype = TYPE_Q4_K_TILED
+            self.n_tiled += 1
+        elif (tile_shapes is not None and allow_q6k and self.tile_q6k and qtype == TYPE_Q6_K
+              and all(ts is not None and ts[0] % 256 == 0 for ts in tile_shapes)
+              and self.ctx.xf_kind(TYPE_Q6_K_TILED, tile_shapes[0][1], sum(ts[0] for ts in tile_shapes)) != XF_NONE):
+            whole = self.ctx.repack_q6k_tiled(whole, tile_shapes[0][1], sum(ts[0] for ts in tile_shapes))
+            qtype = TYPE_Q6_K_TILED
             self.n_tiled += 1
         self.keep.append(whole)
         out, off = [], 0
@@ -411,7 +425,8 @@ class TargetModel:
         that are multiples of 256) into the library's tiled order at upload; the embedding table and the router stay
         in GGUF row order."""
         self.ctx, self.cfg = ctx, cfg
-        up = _Uploader(f"cuda:{ctx.device}", ctx, tiled)
+        # (Q6_K attention projections too, where the one-launch GEMM takes their shape: nothing else reads them)
+        up = _Uploader(f"cuda:{ctx.device}", ctx, tiled, tile_q6k=adjacent)
         self._up = up
         self._layers = (LayerC * cfg.n_layers)()
         H, qd, kvd = cfg.hidden, cfg.n_q * cfg.head_dim, cfg.n_kv * cfg.head_dim
@@ -435,11 +450,12 @@ class TargetModel:
             grouped = ()
             if adjacent:
                 grouped = ("wq", "wk", "wv", "gate", "up")
-                L.wq, L.wk, L.wv = up.q_adjacent([Lw.get("wq"), Lw.get("wk"), Lw.get("wv")], [shape["wq"], shape["wk"], shape["wv"]])
+                L.wq, L.wk, L.wv = up.q_adjacent([Lw.get("wq"), Lw.get("wk"), Lw.get("wv")], [shape["wq"], shape["wk"], shape["wv"]],
+                                                 allow_q6k=True)
                 L.gate, L.up = up.q_adjacent([Lw.get("gate"), Lw.get("up")], [shape.get("gate"), shape.get("up")])
             for k in ("wq", "wk", "wv", "wo", "gate", "up", "down", "router", "gate_exps", "up_exps", "down_exps"):
                 if k not in grouped:
-                    setattr(L, k, up.q(Lw.get(k), shape.get(k)))
+                    setattr(L, k, up.q(Lw.get(k), shape.get(k), allow_q6k=(k == "wo")))
             L.shexp_gate = up.f32(Lw["shexp_gate"]) if "shexp_gate" in Lw else None
         self.c = ModelC(ModelCfgC(**cfg.as_dict()), self._layers, up.q(weights["token_embd"]),
                         up.q(weights["output"], (cfg.vocab, H)), up.f32(weights["output_norm"]))

@@ -81,6 +81,40 @@ def test_whole_k_gemm_extreme_blocks(ctx, oracle, qtype):
     check(y, x.astype(np.float16).astype(np.float64) @ wf.T, "extreme")
 
 
+@pytest.mark.parametrize("n_in,n_out,rows", SHAPES)
+def test_q6k_tiled_order_is_bit_identical(ctx, n_in, n_out, rows):
+    """The tiled, field-planar Q6_K order holds the same blocks in other places: the one-launch GEMM on it equals the same
+    GEMM on the GGUF row order bit for bit (ragged tile and row counts, one and two stages per wave, two tiles per wave)."""
+    blocks = dfl.synth.random_weight(dfl.synth.Q6_K, n_out, n_in, seed=n_in * 3 + n_out)
+    wd = dev(blocks)
+    row_type = ctx.checked_type(dfl.TYPE_Q6_K, wd)
+    kind = ctx.xf_kind(row_type, n_in, n_out)
+    assert kind == dfl.XF_Q6K and ctx.xf_kind(dfl.TYPE_Q6_K_TILED, n_in, n_out) == dfl.XF_Q6K
+    wt = ctx.repack_q6k_tiled(wd, n_in, n_out)
+    x = dev(np.random.default_rng(rows + 1).standard_normal((rows, n_in)).astype(np.float32))
+    xf = ctx.pack_xf(x, kind)
+    a = ctx.gemm_fewrow_xf(wd, row_type, xf, rows, n_in, n_out).cpu().numpy()
+    b = ctx.gemm_fewrow_xf(wt, dfl.TYPE_Q6_K_TILED, xf, rows, n_in, n_out).cpu().numpy()
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_q6k_tiled_guards(ctx):
+    import torch
+
+    n_in, n_out = 2048, 512
+    blocks = dfl.synth.random_weight(dfl.synth.Q6_K, n_out, n_in, seed=3)
+    wt = ctx.repack_q6k_tiled(dev(blocks), n_in, n_out)
+    x = torch.zeros((16, n_in), device="cuda")
+    with pytest.raises(dfl.DFlashError) as e:   # the streaming kernels do not read this order
+        ctx.gemm_fewrow(wt, dfl.TYPE_Q6_K_TILED, x, n_in, n_out)
+    assert e.value.kind == "Unsupported" and "gemm_fewrow_xf" in str(e.value)
+    bad = dfl.synth.extreme_blocks(dfl.synth.Q6_K, n_out * n_in // 256, seed=1).reshape(n_out, -1).copy()
+    bad.view(np.uint8).reshape(-1, 210)[0, 208:210] = np.array([np.float16(128.0)]).view(np.uint8)   # |d| = 128: outside the f16 range
+    with pytest.raises(dfl.DFlashError) as e:
+        ctx.repack_q6k_tiled(dev(bad), n_in, n_out)
+    assert e.value.kind == "Unsupported"
+
+
 def test_rows_are_independent(ctx):
     """A row of the product depends on its own activation row only: a 16-row block and each row alone agree bit for
     bit (what makes a packed verify equal to token-by-token decoding through the same kernel)."""
