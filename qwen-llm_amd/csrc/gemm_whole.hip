@@ -23,6 +23,7 @@
 #include "common.h"
 #include "mfma_unpack.h"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace {
@@ -467,6 +468,133 @@ __global__ void __launch_bounds__(1024) gemm_whole_kernel(WholeArgs a) {
     }
 }
 
+// The same product for a matrix of many more tiles than one round of the chip (an output head: 151936 rows), K of at
+// most 16 super-blocks: a workgroup walks units blockIdx.x * tl + tlane, + gridDim.x * tl, ...  A wave's K slice is
+// the same super-block in every unit, so its eight activation fragments are loaded ONCE and stay in registers; the
+// weights of the next unit travel while the current one is unpacked and multiplied; the slices' partial tiles meet
+// in one of two LDS buffers in turn (one barrier per unit: a buffer is rewritten two units later, behind the barrier
+// of the unit in between).  Same sums, in the same order, as gemm_whole_kernel.
+template <typename W>
+__global__ void __launch_bounds__(1024) gemm_whole_loop_kernel(WholeArgs a) {
+    extern __shared__ float4_t red[];  // [2][16 waves][64]; Q6_K in row order: then a staging area per wave
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tlane = wave / a.ksplit, kslice = wave - tlane * a.ksplit;
+    const int n = lane & 15, g = lane >> 4;
+    const int b0 = a.nb * kslice / a.ksplit;  // one stage per wave (host: nb <= 16, so ksplit == nb and every slice is one super-block)
+    const bool has_stage = a.nb * (kslice + 1) / a.ksplit > b0;
+    const int n_tiles = (a.n_out + 15) >> 4;
+    const int stride = static_cast<int>(gridDim.x) * a.tl;
+    const uint32_t sc_sel = (lane & 16) ? 0x04030402u : 0x04010400u;
+    const Q4KMagic magic = q4k_magic();
+    uint8_t *area = reinterpret_cast<uint8_t *>(red + 2 * 16 * 64) + wave * kQ6AreaBytes;
+    int unit = static_cast<int>(blockIdx.x) * a.tl + tlane;
+    W w_cur, w_next;
+    if (unit < n_tiles && has_stage) load_w(w_cur, a, unit, b0, lane);
+    half8_t af[8];
+    if (has_stage) load_xf(af, a.xf, b0, lane);
+    for (int it = 0;; it++) {
+        const int next = unit + stride;
+        if (next < n_tiles && has_stage) load_w(w_next, a, next, b0, lane);
+        float4_t acc = {0, 0, 0, 0}, acc_sub = {0, 0, 0, 0};
+        if (unit < n_tiles && has_stage) compute(w_cur, af, lane, area, sc_sel, magic, acc, acc_sub);
+        float4_t *buf = red + (it & 1) * (16 * 64);
+        buf[wave * 64 + lane] = acc - acc_sub;
+        __syncthreads();
+        if (kslice == 0 && unit < n_tiles) {
+            float4_t sum = buf[wave * 64 + lane];
+            for (int s = 1; s < a.ksplit; s++) sum += buf[(wave + s) * 64 + lane];
+            const int col = unit * 16 + n;
+            if (col < a.n_out) {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (4 * g + i < a.n_rows) a.y[static_cast<size_t>(4 * g + i) * a.n_out + col] = sum[i];
+            }
+        }
+        // (the same decision in every wave of the workgroup: its first unit lane's next index)
+        if (static_cast<int>(blockIdx.x) * a.tl + (it + 1) * stride >= n_tiles) break;
+        unit = next;
+        w_cur = w_next;
+    }
+}
+
+// The looping kernel for the tiled Q6_K order with the weights brought in through LDS instead of registers: a wave
+// streams its (tile, super-block) pieces - 3360 contiguous bytes, 210 pieces of 16 - with direct-to-LDS loads into a
+// private ring of two buffers and picks its operands out of them with aligned, conflict-free reads (that is what the
+// order's piece rotation is for).  No registers are tied up by bytes in flight, so two units travel per wave (the
+// register version holds one and already spills); "landed" is an s_waitcnt vmcnt of the younger unit's four loads
+// (loads return in order; a Y store of the previous unit that is still in flight only makes the wait stricter).
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+constexpr int kQ6RingDepth = 2;
+constexpr int kVmcnt4 = (4 & 0xF) | 0x0F70, kVmcnt0 = 0x0F70;  // s_waitcnt vmcnt(n), the other counters left alone (gfx9 encoding)
+constexpr size_t kQ6LoopLds = static_cast<size_t>(2) * 16 * 64 * sizeof(float4_t) + static_cast<size_t>(16) * kQ6RingDepth * kQ6TileBytes;
+__global__ void __launch_bounds__(1024) gemm_q6t_loop_kernel(WholeArgs a) {
+    extern __shared__ float4_t red[];  // [2][16 waves][64], then the rings [16 waves][kQ6RingDepth][3360 bytes]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tlane = wave / a.ksplit, kslice = wave - tlane * a.ksplit;
+    const int n = lane & 15, g = lane >> 4, h = g >> 1, odd = g & 1;
+    const int b0 = kslice;  // (host: nb <= 16, so ksplit == nb and every slice is one super-block)
+    const int n_tiles = (a.n_out + 15) >> 4;
+    const int stride = static_cast<int>(gridDim.x) * a.tl;
+    const Q4KMagic magic = q4k_magic();
+    uint8_t *ring = reinterpret_cast<uint8_t *>(red + 2 * 16 * 64) + static_cast<size_t>(wave) * (kQ6RingDepth * kQ6TileBytes);
+    auto issue = [&](int unit, int slot) {  // the unit's 210 pieces into ring buffer `slot`
+        const uint8_t *src = a.w + ((static_cast<size_t>(unit >> 4) * a.nb + b0) * 16 + (unit & 15)) * kQ6TileBytes + lane * 16;
+        uint8_t *dst = ring + slot * kQ6TileBytes;
+        __builtin_amdgcn_global_load_lds((gptr_t)(src), (lptr_t)(dst), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(src + 1024), (lptr_t)(dst + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(src + 2048), (lptr_t)(dst + 2048), 16, 0, 0);
+        // (the fourth load carries the last 18 pieces: a lane's 16 bytes land at the buffer address + 16 lane whatever it
+        // reads, so the other lanes stay out of it; the wave still issues four loads, which is what the count below needs)
+        if (lane < 18) __builtin_amdgcn_global_load_lds((gptr_t)(src + 3072), (lptr_t)(dst + 3072), 16, 0, 0);
+    };
+    int unit = static_cast<int>(blockIdx.x) * a.tl + tlane;
+    half8_t af[8];
+    load_xf(af, a.xf, b0, lane);
+    __builtin_amdgcn_s_waitcnt(kVmcnt0);  // (the fragments are in registers: from here on only weight loads and Y stores are counted)
+    if (unit < n_tiles) issue(unit, 0);
+    for (int it = 0;; it++) {
+        const int next = unit + stride;
+        const int slot = it & 1;
+        if (next < n_tiles) issue(next, slot ^ 1);  // (that buffer's unit was consumed in the previous round: its reads are complete)
+        float4_t acc = {0, 0, 0, 0}, acc_sub = {0, 0, 0, 0};
+        if (unit < n_tiles) {
+            if (next < n_tiles)
+                __builtin_amdgcn_s_waitcnt(kVmcnt4);
+            else
+                __builtin_amdgcn_s_waitcnt(kVmcnt0);
+            const uint8_t *t = ring + slot * kQ6TileBytes;
+            Q6Ops o;
+            o.qa = *reinterpret_cast<const u32x4_t *>(t + q6t_ql_piece(n, 4 * h + 2 * odd));
+            o.qb = *reinterpret_cast<const u32x4_t *>(t + q6t_ql_piece(n, 4 * h + 2 * odd + 1));
+            o.ha = *reinterpret_cast<const u32x4_t *>(t + q6t_qh_piece(n, 2 * h));
+            o.hb = *reinterpret_cast<const u32x4_t *>(t + q6t_qh_piece(n, 2 * h + 1));
+            const uint2 sc = *reinterpret_cast<const uint2 *>(t + kQ6TSc + n * 16 + 8 * h);
+            o.sc4 = (sc.x >> (16 * odd)) & 0xffffu;
+            o.sc4h = (sc.y >> (16 * odd)) & 0xffffu;
+            o.d = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(t + kQ6TD + n * 2)));
+            q6_compute(o, af, lane, magic, acc, acc_sub);
+        }
+        float4_t *buf = red + slot * (16 * 64);
+        buf[wave * 64 + lane] = acc - acc_sub;
+        __syncthreads();
+        if (kslice == 0 && unit < n_tiles) {
+            float4_t sum = buf[wave * 64 + lane];
+            for (int s = 1; s < a.ksplit; s++) sum += buf[(wave + s) * 64 + lane];
+            const int col = unit * 16 + n;
+            if (col < a.n_out) {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (4 * g + i < a.n_rows) a.y[static_cast<size_t>(4 * g + i) * a.n_out + col] = sum[i];
+            }
+        }
+        if (static_cast<int>(blockIdx.x) * a.tl + (it + 1) * stride >= n_tiles) break;
+        unit = next;
+    }
+}
+
 // Row-major activations -> XF: one thread per (row, eight consecutive values).
 template <typename XT>
 __global__ void __launch_bounds__(256) pack_xf_kernel(const XT *__restrict__ x, int n_rows, int n_in, int kind, uint8_t *__restrict__ xf) {
@@ -493,11 +621,12 @@ struct EnvInt {
 
 struct WholePlan {
     int kind, ksplit, tl, R, n_units, n_wg;
+    bool loop;  // more units than one round: gemm_whole_loop_kernel (one stage per wave, plain product)
 };
 
 // The split of a matrix over waves, or kind == DFL_XF_NONE where this path does not take it.
 WholePlan whole_plan(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_t n_out, int64_t pair_ffn) {
-    WholePlan p = {DFL_XF_NONE, 0, 0, 0, 0, 0};
+    WholePlan p = {DFL_XF_NONE, 0, 0, 0, 0, 0, false};
     if (!env_int("DFLASH_GEMM_WHOLE", 1)) return p;
     const int kind = w_type == DFLASH_TYPE_Q4_K_TILED ? DFL_XF_Q4K
                      : (w_type == DFLASH_TYPE_Q6_K || w_type == DFLASH_TYPE_Q6_K_TILED) ? DFL_XF_Q6K
@@ -517,8 +646,13 @@ WholePlan whole_plan(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_
         n_units = (tiles + 1) / 2;
     }
     const int n_wg = (n_units + tl - 1) / tl;
-    if (n_wg > max_wg) return p;
-    p = {kind, ksplit, tl, R, n_units, n_wg};
+    if (n_wg > max_wg) {
+        // many rounds: the looping kernel, where every wave keeps one super-block of the activations (K <= 16 super-blocks)
+        if (pair_ffn || nb > 16 || !env_int("DFLASH_GEMM_WHOLE_LOOP", 1)) return p;
+        p = {kind, ksplit, tl, 1, tiles, std::min((tiles + tl - 1) / tl, ctx->n_cu), true};
+        return p;
+    }
+    p = {kind, ksplit, tl, R, n_units, n_wg, false};
     return p;
 }
 
@@ -572,6 +706,24 @@ int32_t dfl_gemm_whole_blocks(dflash_ctx *ctx, int32_t w_type, const void *w, co
     const size_t red_bytes = static_cast<size_t>(16) * p.R * 64 * sizeof(float4_t);
     const size_t lds = red_bytes + ((p.kind == DFL_XF_Q6K && !q6_tiled) ? static_cast<size_t>(16) * kQ6AreaBytes : 0);
     typedef void (*kernel_t)(WholeArgs);
+    if (p.loop) {
+        if (n_blocks > 1) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: a matrix of %d tiles takes one block of rows per call", p.n_units);
+        const bool q6_ring = q6_tiled && kQ6LoopLds <= ctx->lds_bytes && env_int("DFLASH_Q6T_RING", 1);
+        const kernel_t lf = p.kind == DFL_XF_Q4K ? gemm_whole_loop_kernel<Q4W>
+                            : q6_ring            ? gemm_q6t_loop_kernel
+                            : q6_tiled           ? gemm_whole_loop_kernel<Q6T>
+                                                 : gemm_whole_loop_kernel<Q6W>;
+        const size_t llds = q6_ring ? kQ6LoopLds
+                                    : static_cast<size_t>(2) * 16 * 64 * sizeof(float4_t) +
+                                          ((p.kind == DFL_XF_Q6K && !q6_tiled) ? static_cast<size_t>(16) * kQ6AreaBytes : 0);
+        if (llds > ctx->lds_bytes) return dfl_fail(ctx, DFLASH_ERR_UNSUPPORTED, "gemm_whole: %zu bytes of LDS needed", llds);
+        if (llds > 48 * 1024)
+            if (const int32_t rc = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(lf), llds)) return rc;
+        dfl_timed timer(ctx, st, DFL_T_GEMM);
+        lf<<<p.n_wg, 64 * p.ksplit * p.tl, llds, st>>>(a);
+        DFL_HIP_CHECK(ctx, hipGetLastError());
+        return DFLASH_OK;
+    }
     const int multi = n_blocks > 1 ? (a.nb > p.ksplit ? 2 : 1) : 0;
 #define DFL_WHOLE_PICK(WT, RR) (multi == 0 ? gemm_whole_kernel<WT, RR, 0> : multi == 1 ? gemm_whole_kernel<WT, RR, 1> : gemm_whole_kernel<WT, RR, 2>)
     const kernel_t fn = p.kind == DFL_XF_Q4K ? (p.R == 2 ? DFL_WHOLE_PICK(Q4W, 2) : DFL_WHOLE_PICK(Q4W, 1))

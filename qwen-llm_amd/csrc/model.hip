@@ -42,11 +42,11 @@ __device__ float block_sum(float v, float *sh) {
 
 // kernel_rms_norm_batched_f32 (attn.metal:35-69), optionally preceded by the residual add that
 // feeds it (kernel_add, elementwise.metal): x += add (add may be null), then
-// y = x * rsqrt(mean(x^2) + eps) * w.  One row per workgroup; a row of up to 4096 values (n a
+// y = x * rsqrt(mean(x^2) + eps) * w.  One row per workgroup; a row of up to 8192 values (n a
 // multiple of 4) is read once and stays in registers between the two passes.  With gate_w, the row's
 // sigmoid(y . gate_w) also goes to gate_out[row] (the shared-expert gate of a mixture-of-experts
 // layer, forward.rs:749-824: the normalised row is at hand here, in registers).  With y_xf (n a multiple of 256, at most
-// 4096), y also goes there as f16 in the fragment order a whole-K GEMM reads (common.h, "XF").
+// 8192: every width the whole-K GEMMs take), y also goes there as f16 in the fragment order a whole-K GEMM reads (common.h, "XF").
 __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, const float *__restrict__ add,
                                                        const float *__restrict__ w, float *__restrict__ y, int n,
                                                        float eps, const float *__restrict__ gate_w,
@@ -58,11 +58,13 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
     const float *ar = add ? add + static_cast<size_t>(blockIdx.x) * n : nullptr;
     float *yr = y + static_cast<size_t>(blockIdx.x) * n;
     const int tid = threadIdx.x;
-    if (n <= 4096 && n % 4 == 0) {
-        f4 v[4];
+    if (n <= 8192 && n % 4 == 0) {
+        // (vectors past the row are zeros and add nothing: a row of up to 4096 values sums exactly as with four vectors)
+        constexpr int kVec = 8;
+        f4 v[kVec];
         float s = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kVec; j++) {
             const int i = 4 * (tid + 256 * j);
             v[j] = f4{0, 0, 0, 0};
             if (i < n) {
@@ -78,7 +80,7 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
         const float scale = 1.0f / sqrtf(s / static_cast<float>(n) + eps);
         float dot = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kVec; j++) {
             const int i = 4 * (tid + 256 * j);
             if (i < n) {
                 const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
@@ -814,11 +816,15 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
     const size_t per_layer = static_cast<size_t>(s->capacity) * kv_dim;
     bool cur_ready = false;  // s->cur already holds this layer's normalised input
     const float *pending_resid = nullptr;  // a dense layer's FFN output still to be added to s->x
-    // which projections of a layer read their rows in fragment order (past the last layer: none, the head streams)
+    // which projections of a layer read their rows in fragment order (past the last layer: `qkv` stands for the output head)
+    const int head_kind = want_head ? dfl_whole_kind(ctx, model->output.type, H, c.vocab, 0) : DFL_XF_NONE;
     auto layer_kinds = [&](int il) {
-        return il < c.n_layers ? layer_xf(ctx, model->layers[il], s->pk != nullptr, H, static_cast<int64_t>(q_dim),
-                                          static_cast<int64_t>(kv_dim), c.ffn, c.n_expert == 0)
-                               : LayerXf();
+        if (il < c.n_layers)
+            return layer_xf(ctx, model->layers[il], s->pk != nullptr, H, static_cast<int64_t>(q_dim), static_cast<int64_t>(kv_dim), c.ffn,
+                            c.n_expert == 0);
+        LayerXf head;
+        head.qkv = head_kind;
+        return head;
     };
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_layer &L = model->layers[il];
@@ -901,8 +907,14 @@ int32_t verify_enqueue(dflash_ctx *ctx, const dflash_model *model, dflash_sessio
                 capture_kernel<<<dim3(blocks_for(H), n), 256, 0, st>>>(s->x, hidden_capture, H, n_taps, t);
     }
     if (want_head) {  // (not for a caller that asked for no output of it: a prefill block wants K/V and the taps only)
-        if (!cur_ready) rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, model->output_norm, s->cur, H, c.eps, nullptr, nullptr);
-        if ((rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st))) return rc;
+        if (!cur_ready)
+            rms_norm_kernel<<<n, 256, 0, st>>>(s->x, pending_resid, model->output_norm, s->cur, H, c.eps, nullptr, nullptr,
+                                               head_kind ? s->xf_cur : nullptr, head_kind);
+        if (head_kind)
+            rc = dfl_gemm_whole(ctx, model->output.type, model->output.data, s->xf_cur, lg, H, c.vocab, n, 0, nullptr, DFL_XF_NONE, st);
+        else
+            rc = gemm(ctx, model->output, s->cur, lg, H, c.vocab, n, st);
+        if (rc) return rc;
         if ((rc = dflash_argmax_top2(ctx, lg, n, c.vocab, c.vocab, am, gp, st))) return rc;
     }
     DFL_HIP_CHECK(ctx, hipGetLastError());
@@ -1666,8 +1678,14 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         }
         pending_resid = resid;  // residual 2: added by the norm that reads x next (same x + r, one launch fewer)
     }
-    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, head->output_norm, s->cur, H, c.eps, nullptr, nullptr);
-    if ((rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st))) return rc;
+    const int head_kind = dfl_whole_kind(ctx, target->output.type, H, V, 0);
+    rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, head->output_norm, s->cur, H, c.eps, nullptr, nullptr,
+                                       head_kind ? s->xf_cur : nullptr, head_kind);
+    if (head_kind)
+        rc = dfl_gemm_whole(ctx, target->output.type, target->output.data, s->xf_cur, lg, H, V, N, 0, nullptr, DFL_XF_NONE, st);
+    else
+        rc = gemm(ctx, target->output, s->cur, lg, H, V, N, st);
+    if (rc) return rc;
     if (c.selector_rank > 0) {
         // DFlash-2 tail (:17098-17130, select_draft_path :17176-17251): the 16 best candidates of every
         // row, the selector gate W_h . h of the output-normed hidden, and the predecessor-conditioned

@@ -458,7 +458,7 @@ class TargetModel:
                     setattr(L, k, up.q(Lw.get(k), shape.get(k), allow_q6k=(k == "wo")))
             L.shexp_gate = up.f32(Lw["shexp_gate"]) if "shexp_gate" in Lw else None
         self.c = ModelC(ModelCfgC(**cfg.as_dict()), self._layers, up.q(weights["token_embd"]),
-                        up.q(weights["output"], (cfg.vocab, H)), up.f32(weights["output_norm"]))
+                        up.q(weights["output"], (cfg.vocab, H), allow_q6k=True), up.f32(weights["output_norm"]))
 
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self._up.keep)

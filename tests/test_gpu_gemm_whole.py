@@ -115,6 +115,40 @@ def test_q6k_tiled_guards(ctx):
     assert e.value.kind == "Unsupported"
 
 
+@pytest.mark.parametrize("qtype,tiled", [(dfl.synth.Q4_K, True), (dfl.synth.Q6_K, True), (dfl.synth.Q6_K, False)])
+@pytest.mark.parametrize("n_in,n_out,rows", [(2048, 20000, 16), (1024, 9001, 5), (4096, 6000, 16)])
+def test_many_rounds_of_tiles_take_the_looping_kernel(ctx, oracle, qtype, tiled, n_in, n_out, rows):
+    """A matrix of many more tiles than one round of the chip (an output head) with K of at most 16 super-blocks: the
+    looping kernel against f64 of the oracle's dequant, and - the same sums in the same order - bit for bit against
+    the one-round kernel on the matrix's first rows."""
+    blocks = dfl.synth.random_weight(qtype, n_out, n_in, seed=n_out)
+    wd = dev(blocks)
+    if qtype == dfl.synth.Q4_K:
+        w, w_type = ctx.repack_q4k_tiled(wd, n_in, n_out), dfl.TYPE_Q4_K_TILED
+    elif tiled:
+        w, w_type = ctx.repack_q6k_tiled(wd, n_in, n_out), dfl.TYPE_Q6_K_TILED
+    else:
+        w, w_type = wd, ctx.checked_type(dfl.TYPE_Q6_K, wd)
+    kind = ctx.xf_kind(w_type, n_in, n_out)
+    assert kind != dfl.XF_NONE
+    x = np.random.default_rng(rows).standard_normal((rows, n_in)).astype(np.float32)
+    xf = ctx.pack_xf(dev(x), kind)
+    y = ctx.gemm_fewrow_xf(w, w_type, xf, rows, n_in, n_out).cpu().numpy()
+    wf = oracle.dequant(qtype, blocks, n_in * n_out).reshape(n_out, n_in).astype(np.float64)
+    check(y, x.astype(np.float16).astype(np.float64) @ wf.T, f"loop {n_in}->{n_out} x{rows}")
+    head_rows = 2048   # a matrix of the first rows alone fits one round
+    hb = np.ascontiguousarray(blocks[:head_rows])
+    hd = dev(hb)
+    if qtype == dfl.synth.Q4_K:
+        hw, ht = ctx.repack_q4k_tiled(hd, n_in, head_rows), dfl.TYPE_Q4_K_TILED
+    elif tiled:
+        hw, ht = ctx.repack_q6k_tiled(hd, n_in, head_rows), dfl.TYPE_Q6_K_TILED
+    else:
+        hw, ht = hd, ctx.checked_type(dfl.TYPE_Q6_K, hd)
+    y1 = ctx.gemm_fewrow_xf(hw, ht, xf, rows, n_in, head_rows).cpu().numpy()
+    assert np.array_equal(y1.view(np.uint32), y[:, :head_rows].view(np.uint32))
+
+
 def test_rows_are_independent(ctx):
     """A row of the product depends on its own activation row only: a 16-row block and each row alone agree bit for
     bit (what makes a packed verify equal to token-by-token decoding through the same kernel)."""
@@ -133,7 +167,8 @@ def test_shapes_outside_the_path_are_declined(ctx):
     import torch
 
     assert ctx.xf_kind(dfl.TYPE_Q4_K_TILED, 17408, 5120) == dfl.XF_NONE      # more than two stages per wave
-    assert ctx.xf_kind(dfl.TYPE_Q6_K | dfl.TYPE_RANGE_CHECKED, 2048, 151936) == dfl.XF_NONE  # more than one round of the chip
+    assert ctx.xf_kind(dfl.TYPE_Q6_K | dfl.TYPE_RANGE_CHECKED, 5120, 151936) == dfl.XF_NONE  # many rounds of the chip and K over 16 super-blocks
+    assert ctx.xf_kind(dfl.TYPE_Q6_K | dfl.TYPE_RANGE_CHECKED, 2048, 151936) == dfl.XF_Q6K   # many rounds, short K: the looping kernel
     assert ctx.xf_kind(dfl.TYPE_Q6_K | dfl.TYPE_RANGE_CHECKED, 2048, 2048) == dfl.XF_Q6K
     assert ctx.xf_kind(dfl.TYPE_Q6_K, 2048, 2048) == dfl.XF_NONE             # not range-checked: these kernels scale in f16
     assert ctx.xf_kind(dfl.TYPE_Q4_K, 2048, 2048) == dfl.XF_NONE             # GGUF row order Q4_K: streaming kernels only

@@ -163,6 +163,28 @@ def test_pipelined_prefill_equals_block_by_block(ctx, target):
     pipe.close()
 
 
+def test_wide_hidden_verify_matches_oracle(ctx, oracle):
+    """A 5120-wide dense layer pair (the width of the 27B-shaped benchmark matrices): rows wider than 4096 take the
+    norm kernel's in-register path with eight vectors per thread, and the norms hand their rows to the one-launch
+    projections in fragment order at that width too."""
+    cfg = dfl.ModelConfig(n_layers=2, hidden=5120, n_q=8, n_kv=2, head_dim=128, ffn=2048, vocab=4096)
+    w = dfl.synth_target_weights_blocks(cfg, 19)
+    model = dfl.TargetModel(ctx, cfg, w)
+    omodel, _keep = oracle.build_model(cfg.as_dict(), w)
+    sess = dfl.Session(ctx, model, 64, [0, 1])
+    ostate = oracle.TargetState(cfg.as_dict(), 64)
+    rng = np.random.default_rng(4)
+    pos = 0
+    for n in (16, 5):
+        blk = rng.integers(0, cfg.vocab, n).tolist()
+        out = sess.encode_packed_verify_layer_major(blk, pos, want_logits=True)
+        lo, hid = oracle.target_verify(omodel, ostate, blk, pos, [0, 1])
+        close(out.hidden_capture.cpu().numpy(), hid, f"wide hidden n={n}")
+        close(out.logits.cpu().numpy(), lo, f"wide logits n={n}")
+        pos += n
+    sess.close()
+
+
 def test_verify_guard_walls(ctx, target):
     model, _ = target
     sess = dfl.Session(ctx, model, 64, TAPS)
