@@ -111,12 +111,27 @@ def attention_section(ctx, with_cpu=True):
 
 
 def q6k_section(ctx):
-    """Few-row Q6_K GEMM, M=16, f32 activations: the output head of the end-to-end model (2048 -> 151936, 255 MB)
-    and a 5120 -> 5120 projection (21.5 MB); weights rotate over enough copies to stay out of the memory-side cache.
-    Microseconds per call (split-K reduction included) and weight GB/s."""
+    """Few-row Q6_K GEMM, M=16: the output head of the end-to-end model (2048 -> 151936, 255 MB) and a 5120 -> 5120
+    projection (21.5 MB); weights rotate over enough copies to stay out of the memory-side cache.  Microseconds per
+    call and weight GB/s, two ways: through dflash_gemm_fewrow on GGUF row order with f32 activations (the streaming
+    kernel and its split-K reduction launch), and - what the model-level calls run - through dflash_gemm_fewrow_xf on the
+    tiled Q6_K order with the activations already in fragment order (one launch; `tiled_xf_*`)."""
     import torch
 
     import qwen_llm_amd as dfl
+
+    def timed(fn, n_sets, reps=3):
+        for i in range(n_sets):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for i in range(n_sets):
+                fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (reps * n_sets) * 1e3
 
     out = []
     g = torch.Generator(device="cuda")
@@ -128,21 +143,20 @@ def q6k_section(ctx):
         x = torch.randn((16, n_in), device="cuda", generator=g)
         y = torch.empty((16, n_out), device="cuda")
         tag = ctx.checked_type(dfl.TYPE_Q6_K, ws[0])  # (every set comes from the same generator: one range check speaks for all)
-        for w in ws:
-            ctx.encode_mat_mat_dispatch_dflash_verify(w, tag, x, y, n_in, n_out, 16)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        reps = 3
-        e0.record()
-        for _ in range(reps):
-            for w in ws:
-                ctx.encode_mat_mat_dispatch_dflash_verify(w, tag, x, y, n_in, n_out, 16)
-        e1.record()
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / (reps * n_sets) * 1e3
-        out.append({"n_in": n_in, "n_out": n_out, "weight_bytes": nbytes, "us_per_call": us,
-                    "GBps": nbytes / (us * 1e-6) / 1e9, "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS})
-        del ws, x, y
+        us = timed(lambda i: ctx.encode_mat_mat_dispatch_dflash_verify(ws[i], tag, x, y, n_in, n_out, 16), n_sets)
+        row = {"n_in": n_in, "n_out": n_out, "weight_bytes": nbytes, "us_per_call": us,
+               "GBps": nbytes / (us * 1e-6) / 1e9, "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+               "rotating_copies": n_sets}
+        kind = ctx.xf_kind(dfl.TYPE_Q6_K_TILED, n_in, n_out)
+        if kind != dfl.XF_NONE:
+            wts = [ctx.repack_q6k_tiled(w, n_in, n_out) for w in ws]
+            del ws
+            xf = ctx.pack_xf(x, kind)
+            us_t = timed(lambda i: ctx.gemm_fewrow_xf(wts[i], dfl.TYPE_Q6_K_TILED, xf, 16, n_in, n_out, y=y), n_sets)
+            row.update({"tiled_xf_us_per_call": us_t, "tiled_xf_GBps": nbytes / (us_t * 1e-6) / 1e9,
+                        "tiled_xf_frac_of_hbm_peak": nbytes / (us_t * 1e-6) / 1e9 / HBM_PEAK_GBS})
+            del wts
+        out.append(row)
     return out
 
 

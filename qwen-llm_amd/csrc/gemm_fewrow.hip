@@ -1400,15 +1400,29 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     if constexpr (kRoute) {
         // The block's routing, by every workgroup for itself: wave w takes row w (dfl_route::route_row, the arithmetic
         // of the stand-alone kernel), the union of the rows' masks gives the ascending expert list, kept in LDS.
-        // The shared activations are on their way meanwhile.
-        load_x(0, 0);
+        // The row's logits are fetched FIRST and waited for before the shared activations are requested: a CU takes in
+        // 20-30 KB per microsecond, and behind the 64 KB of a chunk's f32 activations the 8 KB of logits arrived 2 us
+        // later than alone (loads return in order).  The activations then travel while the rows are routed.  The loads
+        // are asm loads with their own wait, like the activations': a wait the compiler placed at the logits' first use
+        // would stand behind the activation loads again.
         unsigned long long *row_mask = reinterpret_cast<unsigned long long *>(reinterpret_cast<uint8_t *>(lds) + kExpXchgEnd);
         const int E = bt.route_experts, used = bt.route_used;
+        float lgv[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        if (wave < n_rows) {
+            const float *lrow = bt.route_logits + static_cast<size_t>(wave) * E + lane;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (lane + 64 * j < E) asm volatile("global_load_dword %0, %1, off" : "+v"(lgv[j]) : "v"(lrow + 64 * j) : "memory");
+        }
+        __builtin_amdgcn_s_waitcnt(q4k_vmcnt(0));
+#pragma unroll
+        for (int j = 0; j < 4; j++) asm volatile("" : "+v"(lgv[j]));
+        load_x(0, 0);
         dfl_route::RowPicks pk;
         pk.my_e = 0;
         pk.my_w = 0.0f;
         pk.m[0] = pk.m[1] = pk.m[2] = pk.m[3] = 0;
-        if (wave < n_rows) pk = dfl_route::route_row(bt.route_logits + static_cast<size_t>(wave) * E, E, used, lane);
+        if (wave < n_rows) pk = dfl_route::route_row_from(lgv, E, used, lane);
         if (lane < 4) row_mask[wave * 4 + lane] = dfl_route::pick4(pk.m, lane);
         __builtin_amdgcn_s_waitcnt(kWaitLds);
         __builtin_amdgcn_s_barrier();

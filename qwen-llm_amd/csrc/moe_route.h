@@ -16,15 +16,19 @@ namespace dfl_route {
 // and 3, then lane 31 into rows 2 and 3; lane 63 has the result.  NaN operands are ignored, as v_max_f32 does; lanes
 // without a source keep their own value.  No LDS round trips, unlike a shuffle.
 __device__ __forceinline__ float wave_max_f32(float v) {
-#define DFL_FMAX_STEP(ctrl, row_mask)                                                                              \
-    v = fmaxf(v, __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(v), __float_as_uint(v), ctrl, row_mask, 0xf, false)))
-    DFL_FMAX_STEP(0x111, 0xf);
-    DFL_FMAX_STEP(0x112, 0xf);
-    DFL_FMAX_STEP(0x114, 0xf);
-    DFL_FMAX_STEP(0x118, 0xf);
-    DFL_FMAX_STEP(0x142, 0xa);
-    DFL_FMAX_STEP(0x143, 0xc);
-#undef DFL_FMAX_STEP
+    // One v_max_f32 with a DPP source per step.  (Written through update_dpp + fmaxf the compiler emits a copy, the
+    // move, a canonicalising maximum and the maximum: five instructions a step, thirty a call, and every workgroup of an
+    // expert launch makes eight calls per row with four waves on a SIMD before it can ask for its first weight byte.)
+    // A lane without a source keeps its value (bound_ctrl off); two wait states between a write of v and its DPP read.
+    asm volatile(
+        "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(v));
     return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
 }
 
@@ -50,14 +54,12 @@ struct RowPicks {
 };
 
 // lg: the row's n_expert router logits (n_expert <= 64 kRegs: kRegs probabilities per lane).  Called by all 64 lanes of a wave.
+// lgv[j]: logit of expert lane + 64 j, -infinity past n_expert.
 template <int kRegs>
-__device__ __forceinline__ RowPicks route_row_regs(const float *__restrict__ lg, int n_expert, int n_used, int lane) {
+__device__ __forceinline__ RowPicks route_row_loaded(const float (&lgv)[kRegs], int n_expert, int n_used, int lane) {
     RowPicks r;
     r.my_e = 0;
     r.m[0] = r.m[1] = r.m[2] = r.m[3] = 0;
-    float lgv[kRegs];
-#pragma unroll
-    for (int j = 0; j < kRegs; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < kRegs; j++) mx = fmaxf(mx, lgv[j]);
@@ -115,9 +117,24 @@ __device__ __forceinline__ RowPicks route_row_regs(const float *__restrict__ lg,
 // n_expert <= 256.  The common 128-expert router keeps two probabilities per lane instead of four: the same
 // arithmetic on the same values in the same order (the registers it drops hold "no such expert"), half the
 // per-pick work, which every workgroup of the expert launch spends before its first weight byte.
+template <int kRegs>
+__device__ __forceinline__ RowPicks route_row_regs(const float *__restrict__ lg, int n_expert, int n_used, int lane) {
+    float lgv[kRegs];
+#pragma unroll
+    for (int j = 0; j < kRegs; j++) lgv[j] = lane + 64 * j < n_expert ? lg[lane + 64 * j] : -INFINITY;
+    return route_row_loaded<kRegs>(lgv, n_expert, n_used, lane);
+}
 __device__ __forceinline__ RowPicks route_row(const float *__restrict__ lg, int n_expert, int n_used, int lane) {
     if (n_expert <= 128) return route_row_regs<2>(lg, n_expert, n_used, lane);
     return route_row_regs<4>(lg, n_expert, n_used, lane);
+}
+// The same from four logits per lane already in registers (a caller that loads them itself, ahead of other traffic).
+__device__ __forceinline__ RowPicks route_row_from(const float (&lgv)[4], int n_expert, int n_used, int lane) {
+    if (n_expert <= 128) {
+        const float two[2] = {lgv[0], lgv[1]};
+        return route_row_loaded<2>(two, n_expert, n_used, lane);
+    }
+    return route_row_loaded<4>(lgv, n_expert, n_used, lane);
 }
 
 // v[i & 3] without indexing the array by a run-time value (which would move it from registers to scratch memory)
