@@ -15,6 +15,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first 64 bytes of a kernel's arguments arrive in scalar registers with the wave instead of through scalar
+    # loads it has to wait for at its start (measured on the 40-layer verify: 3.53 -> 3.48 ms, nine dependent kernels a layer)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function",
 ]
 
