@@ -1556,6 +1556,9 @@ __global__ void __launch_bounds__(64 * kSlabWaves)
     const uint8_t *it_base0 = nullptr, *it_base1 = nullptr;
     auto it_seek = [&]() {  // the first round at or after it_r with a unit for this wave
         int slot = 0, tile = 0;
+        // (not unrolled: the first round almost always has a unit, and the compiler's four-at-a-time version spent a
+        // hundred scalar instructions, in all sixteen waves, before the first weight load of a launch)
+#pragma nounroll
         while (it_r < n_rounds && !unit_of(it_r, slot, tile)) it_r++;
         it_valid = it_r < n_rounds;
         if (it_valid) {
