@@ -387,6 +387,27 @@ __global__ void __launch_bounds__(256)
     const int tid = threadIdx.x;
     const int64_t slot0 = static_cast<int64_t>(head) * 16 + row;
     const int64_t slot_stride = static_cast<int64_t>(n_q) * 16;
+    // The partial outputs of the first kPre rounds of splits are asked for BEFORE the maxima: their addresses do not
+    // depend on the weights, so the two trips to memory (maxima, then outputs) are in flight together instead of one
+    // behind the other across two barriers.  The sums below take them in the same order as the loop that follows.
+    constexpr int kPre = 4;
+    const int sl = tid >> 5, dl = tid & 31;  // split lane, dim lane
+    const int n_vec = hd / 4;                // float4 per row: 16, 32 or 64
+    float4_t pre0[kPre], pre1[kPre];
+    float pre_l[kPre];
+#pragma unroll
+    for (int i = 0; i < kPre; i++) {
+        const int s = sl + 8 * i;
+        pre0[i] = float4_t{0, 0, 0, 0};
+        pre1[i] = float4_t{0, 0, 0, 0};
+        pre_l[i] = 0.0f;
+        if (s < n_splits) {
+            const float4_t *po = reinterpret_cast<const float4_t *>(part_o + (slot0 + s * slot_stride) * hd);
+            if (dl < n_vec) pre0[i] = po[dl];
+            if (dl + 32 < n_vec) pre1[i] = po[dl + 32];
+            if (dl == 0) pre_l[i] = part_ml[(slot0 + s * slot_stride) * 2 + 1];
+        }
+    }
     // m* = max over splits (a thread keeps the maxima it loaded: n_splits <= 1024 = 4 per thread)
     float m_loc = -INFINITY;
     float m_own[4];
@@ -406,11 +427,19 @@ __global__ void __launch_bounds__(256)
         if (s < n_splits) wgt[s] = (m_own[j] == -INFINITY) ? 0.0f : exp2f(m_own[j] - m_star);
     }
     __syncthreads();  // (also: every thread has read red_l before the split lanes write their sums into it)
-    const int sl = tid >> 5, dl = tid & 31;  // split lane, dim lane
-    const int n_vec = hd / 4;                // float4 per row: 16, 32 or 64
     float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
     float l = 0.0f;
-    for (int s = sl; s < n_splits; s += 8) {
+#pragma unroll
+    for (int i = 0; i < kPre; i++) {
+        const int s = sl + 8 * i;
+        if (s < n_splits) {
+            const float w = wgt[s];
+            if (dl < n_vec) acc0 += w * pre0[i];
+            if (dl + 32 < n_vec) acc1 += w * pre1[i];
+            if (dl == 0) l += w * pre_l[i];
+        }
+    }
+    for (int s = sl + 8 * kPre; s < n_splits; s += 8) {
         const float w = wgt[s];
         const float4_t *po = reinterpret_cast<const float4_t *>(part_o + (slot0 + s * slot_stride) * hd);
         if (dl < n_vec) acc0 += w * po[dl];

@@ -155,13 +155,34 @@ __global__ void __launch_bounds__(64)
                     : (k_dst ? nullptr : k_out + (static_cast<size_t>(row) * n_kv + (head - n_q)) * hd);
     const float *w = is_q ? q_w : k_w;
     const int half = hd / 2;
+    const int32_t pos_row = pos[row];
+    // heads of 128 or 256: a lane's two or four elements stay in registers between the two passes (element lane + 64 k
+    // in r[k]; the partner of element i is i + half = r[k + half / 64]); same sums in the same order as the loops
+    const bool in_regs = hd == 256 || hd == 128;
+    float r[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     float s = 0.0f;
-    for (int i = lane; i < hd; i += 64) s += v[i] * v[i];
+    if (in_regs) {
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (lane + 64 * k < hd) r[k] = v[lane + 64 * k];
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (lane + 64 * k < hd) s += r[k] * r[k];
+    } else {
+        for (int i = lane; i < hd; i += 64) s += v[i] * v[i];
+    }
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
     const float scale = 1.0f / sqrtf(s / static_cast<float>(hd) + eps);
-    const float p = static_cast<float>(pos[row]);
-    for (int i = lane; i < half; i += 64) {
-        float a = v[i] * scale, b = v[i + half] * scale;
+    const float p = static_cast<float>(pos_row);
+    for (int i = lane, k = 0; i < half; i += 64, k++) {
+        float a, b;
+        if (in_regs) {
+            a = (k == 0 ? r[0] : r[1]) * scale;
+            b = (hd == 256 ? (k == 0 ? r[2] : r[3]) : r[1]) * scale;
+        } else {
+            a = v[i] * scale;
+            b = v[i + half] * scale;
+        }
         if (w) {
             a *= w[i];
             b *= w[i + half];
@@ -174,7 +195,7 @@ __global__ void __launch_bounds__(64)
             o[i] = ra;
             o[i + half] = rb;
         } else {
-            _Float16 *dst = k_dst + (static_cast<size_t>(pos[row]) * n_kv + (head - n_q)) * hd;
+            _Float16 *dst = k_dst + (static_cast<size_t>(pos_row) * n_kv + (head - n_q)) * hd;
             dst[i] = static_cast<_Float16>(ra);
             dst[i + half] = static_cast<_Float16>(rb);
         }

@@ -378,6 +378,21 @@ __global__ void __launch_bounds__(256)
     __shared__ float w_k[64];
     __shared__ int32_t slot_k[64];  // row of eo that holds pick k of this row
     const int row = blockIdx.x, tid = threadIdx.x;
+    // Everything whose address depends on nothing this kernel reads is asked for first (the slot count, the gate, the
+    // residual row and the term to add to it), beside the picks: one trip to memory, then the picks' output rows.
+    const size_t n_slots_now = static_cast<size_t>(*n_slots);
+    const float gate = sg[row];
+    f4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int i = 4 * (tid + 256 * j);
+        v[j] = f4{0, 0, 0, 0};
+        if (i < hidden) {
+            v[j] = *reinterpret_cast<const f4 *>(x + static_cast<size_t>(row) * hidden + i);
+            // (a residual term the norm before this layer's experts left out: it goes in first, as it would have there)
+            if (pre_add) v[j] += *reinterpret_cast<const f4 *>(pre_add + static_cast<size_t>(row) * hidden + i);
+        }
+    }
     // grouped (rows of several 16-row blocks, moe_group_slots_kernel): slot_of is the eo row of a pick itself, and the
     // shared expert's slots are the last gridDim.x / 16 (rounded up) of the list, one per block of rows
     if (tid < n_used) {
@@ -385,15 +400,11 @@ __global__ void __launch_bounds__(256)
         slot_k[tid] = grouped ? slot_of[row * n_used + tid] : slot_of[row * n_used + tid] * 16 + row;
     }
     __syncthreads();
-    const float gate = sg[row];
-    const size_t last = grouped ? (static_cast<size_t>(*n_slots) - (gridDim.x + 15) / 16 + (row >> 4)) * 16 + (row & 15)
-                                : (static_cast<size_t>(*n_slots) - 1) * 16 + row;
-    f4 v[4];
+    const size_t last = grouped ? (n_slots_now - (gridDim.x + 15) / 16 + (row >> 4)) * 16 + (row & 15) : (n_slots_now - 1) * 16 + row;
     float s = 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int i = 4 * (tid + 256 * j);
-        v[j] = f4{0, 0, 0, 0};
         if (i < hidden) {
             f4 out = {0, 0, 0, 0};
             for (int k = 0; k < n_used; k++)
@@ -401,9 +412,6 @@ __global__ void __launch_bounds__(256)
             const f4 shv = shared ? *reinterpret_cast<const f4 *>(shared + static_cast<size_t>(row) * hidden + i)
                                   : *reinterpret_cast<const f4 *>(eo + last * hidden + i);
             out += gate * shv;
-            v[j] = *reinterpret_cast<const f4 *>(x + static_cast<size_t>(row) * hidden + i);
-            // (a residual term the norm before this layer's experts left out: it goes in first, as it would have there)
-            if (pre_add) v[j] += *reinterpret_cast<const f4 *>(pre_add + static_cast<size_t>(row) * hidden + i);
             v[j] += out;
             *reinterpret_cast<f4 *>(x + static_cast<size_t>(row) * hidden + i) = v[j];
         }
