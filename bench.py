@@ -305,7 +305,7 @@ def acceptance_table(hist):
     return {"alpha_pos1": at_least[0], "per_position_acceptance": at_least, "accept_len_hist": list(hist)}
 
 
-def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048):
+def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048, dflash2=True):
     """End-to-end DFlash speculative decode on the 35B-A3B-shaped synthetic MoE target (40 layers, hidden 2048,
     16 q / 2 kv heads of 256, 128 experts top-8 with F_exp 768 plus a shared expert; experts Q4_K, attention Q6_K,
     vocabulary 151936) with a 5-layer drafter fed by 3 tapped layers, batch 1, block 16, prompt 2048, greedy accept.
@@ -387,6 +387,36 @@ def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048):
             "tokens_equal_serial_greedy": agree, "tokens": len(tokens)})
         res["sweep"][-1].update(acceptance_table(st.get("accept_len_hist", [0] * 16)))
         log(f"e2e: forced k={k}: {res['sweep'][-1]}")
+
+    # The same run with a DFlash-2 drafter of that shape (what current drafters ship: a dynamic two-tap convolution
+    # before and after both sublayers of every layer, top-16 of the head's logits and the selector's walk over rank-256
+    # Q4_K codebooks in place of the argmax), greedy, forced k = 7.
+    if dflash2:
+        k = 7
+        d2cfg = dfl.DraftConfig(n_layers=5, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=6144, block_size=16, n_taps=3,
+                                conv_kernel_size=2, conv_group_size=64, selector_rank=256, selector_top_k=16)
+        head2 = dfl.DraftHead(ctx, d2cfg, dfl.synth_draft_weights_device(d2cfg, 1, "cuda", vocab=cfg.vocab))
+        dec = dfl.SpeculativeDecoder(ctx, target, head2, taps, cap, mask)
+        first = dec.prefill(prompt)
+
+        def override2(tokens, position):
+            done = len(tokens)
+            return cont[done:done + k] + [(t + 1) % (cfg.vocab - 1) for t in cont[done + k:done + 15]]
+
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        tokens, st = dec.generate(first, n_generate, draft_override_fn=override2)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        dec.close()
+        res["dflash2"] = {
+            "drafter": "DFlash-2: 5 layers, conv kernel 2 / group 64, selector rank 256 over Q4_K codebooks, top-16",
+            "forced_k": k, "accepted_tokens_per_s": (len(tokens) - 1) / dt, "steps": st["spec_steps"],
+            "ms_per_step": dt * 1e3 / max(st["spec_steps"], 1), "draft_ms": st["draft_ms"] / st["spec_steps"],
+            "verify_ms": st["verify_ms"] / st["spec_steps"],
+            "tokens_equal_serial_greedy": sum(int(a == b) for a, b in zip(tokens, cont)), "tokens": len(tokens)}
+        log(f"e2e: DFlash-2 drafter, forced k={k}: {res['dflash2']}")
+        del head2
 
     # Stochastic acceptance (sampler coupled to deterministic drafts), forced the same way: the serial sampler's own
     # stream (temperature 0.7, top-k 20, top-p 0.95, one draw per token, through the same kernels) supplies the first

@@ -72,24 +72,59 @@ struct SampledOut {
     dflash_weighted_candidate cands[15 * 16];    // [pos - 1][top_k], distribution order
 };
 
-// The walk, one workgroup.  Per position: all threads dequantise the candidates' successor rows and
-// form gate = pred * sel_h[pos] in LDS; thread b then scores candidate b with the reference's scalar
-// loop (products and additions rounded separately, rank order), thread 0 keeps the first strict
-// maximum (greedy) or samples from softmax(score / T) with the sampler chain and the position's
-// pre-drawn uniform (SAMPLED), and all threads fetch the winner's predecessor row.  status: 0, or 1
-// when a predecessor row is out of range (the walk stops there).
+// The walk's scores do not have to wait for the walk: the predecessor of position pos is one of the top_k candidates
+// of position pos - 1 (the carry token for pos = 1), so score(pos, a, b) for every candidate a of the previous position
+// and every candidate b of this one is known work up front: (n - 1) x top_k workgroups, all at once, each with the
+// reference's arithmetic for its sixteen scores.  Workgroup (a, pos): all threads dequantise the predecessor row of
+// candidate a and the successor rows of position pos's candidates and form gate = pred * sel_h[pos] in LDS; thread b
+// then scores candidate b with the reference's scalar loop (products and additions rounded separately, rank order):
+// table[pos - 1][a][b] = vals[pos][b] + sum_r gate[r] * succ_b[r], NaN for a candidate without a successor row.  A
+// previous candidate without a predecessor row gets no scores: the walk stops when it picks one.
+__global__ void __launch_bounds__(kSelThreads)
+    dflash2_scores_kernel(Codebook pred_cb, Codebook succ_cb, int top_k, int rank, int carry, int n,
+                          const int32_t *__restrict__ ids, const float *__restrict__ vals, const float *__restrict__ sel_h,
+                          float *__restrict__ table) {
+    extern __shared__ float lds[];  // gate[rank], succ[top_k][rank]
+    float *gate = lds, *succ = lds + rank;
+    const int tid = threadIdx.x;
+    const int a = blockIdx.x, pos = 1 + blockIdx.y;
+    if (pos == 1 && a != 0) return;  // (one predecessor only: the carry token)
+    const int32_t prev = pos == 1 ? carry : ids[(pos - 1) * top_k + a];
+    if (prev < 0 || prev >= pred_cb.n_rows) return;
+    const float *hrow = sel_h + static_cast<size_t>(pos) * rank;
+    for (int r = tid; r < rank; r += kSelThreads) gate[r] = codebook_elem(pred_cb, prev, r) * hrow[r];
+    for (int e = tid; e < top_k * rank; e += kSelThreads) {
+        const int b = e / rank, r = e - b * rank;
+        const int32_t cand = ids[pos * top_k + b];
+        if (cand >= 0 && cand < succ_cb.n_rows) succ[e] = codebook_elem(succ_cb, cand, r);
+    }
+    __syncthreads();
+    if (tid < top_k) {
+        const int32_t cand = ids[pos * top_k + tid];
+        float sc = __builtin_nanf("");  // skipped candidates never compare greater
+        if (cand >= 0 && cand < succ_cb.n_rows) {
+            float dot = 0.0f;
+            const float *sr = succ + tid * rank;
+            for (int r = 0; r < rank; r++) dot += gate[r] * sr[r];  // two roundings each (contraction is off in this file)
+            sc = vals[pos * top_k + tid] + dot;
+        }
+        table[(static_cast<size_t>(pos - 1) * top_k + a) * top_k + tid] = sc;
+    }
+}
+
+// The walk over the table, one workgroup: the table and the candidates go to LDS, thread 0 then follows the picks.
+// Per position it keeps the first strict maximum of the previous pick's row of scores (greedy) or samples from
+// softmax(score / T) with the sampler chain and the position's pre-drawn uniform (SAMPLED).  status: 0, or 1 when a
+// picked token has no predecessor row (the walk stops there).
 template <bool SAMPLED>
 __global__ void __launch_bounds__(kSelThreads)
-    dflash2_select_kernel(Codebook pred_cb, Codebook succ_cb, int top_k, int rank, int carry, int n,
-                          const int32_t *__restrict__ ids, const float *__restrict__ vals,
-                          const float *__restrict__ sel_h, int32_t *__restrict__ out, int32_t *__restrict__ status,
+    dflash2_select_kernel(int64_t n_pred_rows, int64_t n_succ_rows, int top_k, int carry, int n, const int32_t *__restrict__ ids,
+                          const float *__restrict__ table, int32_t *__restrict__ out, int32_t *__restrict__ status,
                           float temperature, const double *__restrict__ uniforms, SampledOut *__restrict__ sampled) {
-    extern __shared__ float lds[];  // pred[rank], gate[rank], succ[top_k][rank]
-    __shared__ float score[kSelMaxTopK];
-    __shared__ int chosen_s;
-    float *pred = lds, *gate = lds + rank, *succ = lds + 2 * rank;
-    const int tid = threadIdx.x;
+    __shared__ float table_s[15 * kSelMaxTopK * kSelMaxTopK];
+    __shared__ int32_t ids_s[16 * kSelMaxTopK];
     __shared__ RowDist dist;
+    const int tid = threadIdx.x;
     if (tid == 0) {
         out[0] = ids[0];
         *status = 0;
@@ -101,112 +136,109 @@ __global__ void __launch_bounds__(kSelThreads)
         }
     }
     if (n < 2) return;
-    if (carry < 0 || carry >= pred_cb.n_rows) {
+    if (carry < 0 || carry >= n_pred_rows) {
         if (tid == 0) *status = 1;
         return;
     }
-    for (int r = tid; r < rank; r += kSelThreads) pred[r] = codebook_elem(pred_cb, carry, r);
+    for (int e = tid; e < (n - 1) * top_k * top_k; e += kSelThreads) table_s[e] = table[e];
+    for (int e = tid; e < n * top_k; e += kSelThreads) ids_s[e] = ids[e];
     __syncthreads();
+    if (tid != 0) return;
+    int prev_a = 0;  // which candidate of the previous position was picked (the carry token's scores sit in row 0)
     for (int pos = 1; pos < n; pos++) {
-        const float *hrow = sel_h + static_cast<size_t>(pos) * rank;
-        for (int r = tid; r < rank; r += kSelThreads) gate[r] = pred[r] * hrow[r];
-        for (int e = tid; e < top_k * rank; e += kSelThreads) {
-            const int b = e / rank, r = e - b * rank;
-            const int32_t cand = ids[pos * top_k + b];
-            if (cand >= 0 && cand < succ_cb.n_rows) succ[e] = codebook_elem(succ_cb, cand, r);
-        }
-        __syncthreads();
-        if (tid < top_k) {
-            const int32_t cand = ids[pos * top_k + tid];
-            float s = __builtin_nanf("");  // skipped candidates never compare greater
-            if (cand >= 0 && cand < succ_cb.n_rows) {
-                float dot = 0.0f;
-                const float *sr = succ + tid * rank;
-                for (int r = 0; r < rank; r++) dot += gate[r] * sr[r];  // two roundings each (contraction is off in this file)
-                s = vals[pos * top_k + tid] + dot;
-            }
-            score[tid] = s;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            int best_b = 0;
-            if (!SAMPLED) {
-                float best = -INFINITY;
-                for (int b = 0; b < top_k; b++) {
-                    const int32_t cand = ids[pos * top_k + b];
-                    if (cand < 0 || cand >= succ_cb.n_rows) continue;
-                    if (score[b] > best) {
-                        best = score[b];
-                        best_b = b;
-                    }
+        const float *score = table_s + (static_cast<size_t>(pos - 1) * top_k + prev_a) * top_k;
+        const int32_t *cands = ids_s + pos * top_k;
+        int best_b = 0;
+        if (!SAMPLED) {
+            float best = -INFINITY;
+            for (int b = 0; b < top_k; b++) {
+                const int32_t cand = cands[b];
+                if (cand < 0 || cand >= n_succ_rows) continue;
+                if (score[b] > best) {
+                    best = score[b];
+                    best_b = b;
                 }
+            }
+        } else {
+            // scores of skipped candidates are -inf; the "tokens" of the distribution are candidate indices
+            uint64_t keys[kSelMaxTopK];
+            int nan_at = -1;
+            for (int b = 0; b < top_k; b++) {
+                const int32_t cand = cands[b];
+                const float sc = (cand < 0 || cand >= n_succ_rows) ? -INFINITY : score[b];
+                if (sc != sc && nan_at < 0) nan_at = b;
+                const uint64_t key = cand_key(static_cast<uint32_t>(b), sc);
+                int j = b;  // insertion sort, ascending keys = best first
+                while (j > 0 && keys[j - 1] > key) {
+                    keys[j] = keys[j - 1];
+                    j--;
+                }
+                keys[j] = key;
+            }
+            dist.err = 0;
+            if (nan_at >= 0) {
+                dist.err = DFLASH_ERR_NAN_LOGIT;
             } else {
-                // scores of skipped candidates are -inf; the "tokens" of the distribution are candidate indices
-                uint64_t keys[kSelMaxTopK];
-                int nan_at = -1;
-                for (int b = 0; b < top_k; b++) {
-                    const int32_t cand = ids[pos * top_k + b];
-                    const float sc = (cand < 0 || cand >= succ_cb.n_rows) ? -INFINITY : score[b];
-                    if (sc != sc && nan_at < 0) nan_at = b;
-                    const uint64_t key = cand_key(static_cast<uint32_t>(b), sc);
-                    int j = b;  // insertion sort, ascending keys = best first
-                    while (j > 0 && keys[j - 1] > key) {
-                        keys[j] = keys[j - 1];
-                        j--;
-                    }
-                    keys[j] = key;
-                }
-                dist.err = 0;
-                if (nan_at >= 0) {
-                    dist.err = DFLASH_ERR_NAN_LOGIT;
-                } else {
-                    ChainCfg cc = {};
-                    cc.temperature = temperature;
-                    cc.top_p = 1.0f;
-                    cc.min_p = 0.0f;
-                    cc.k = top_k;
-                    run_chain(keys, top_k, cc, &dist);
-                }
-                if (dist.err) {
-                    sampled->status = dist.err;
-                    sampled->err_pos = pos;
-                    *status = dist.err;
-                    chosen_s = -1;
-                } else {
-                    const int idx = pick_index(dist.weights, dist.n_keep, uniforms[pos - 1] * dist.total);
-                    best_b = dist.tokens[idx];
-                    sampled->n_sampled = pos;
-                    int cnt = 0;
-                    for (int i = 0; i < dist.n_keep; i++) {
-                        if (!(dist.weights[i] > 0.0)) continue;
-                        dflash_weighted_candidate &wc = sampled->cands[(pos - 1) * top_k + cnt++];
-                        wc.token = ids[pos * top_k + dist.tokens[i]];
-                        wc.weight = dist.weights[i];
-                    }
-                    sampled->counts[pos - 1] = cnt;
-                }
+                ChainCfg cc = {};
+                cc.temperature = temperature;
+                cc.top_p = 1.0f;
+                cc.min_p = 0.0f;
+                cc.k = top_k;
+                run_chain(keys, top_k, cc, &dist);
             }
-            if (SAMPLED && *status) {
-                // sampler error: stop the walk
-            } else {
-            const int32_t chosen = ids[pos * top_k + best_b];
-            out[pos] = chosen;
-            chosen_s = chosen;
-            if (chosen < 0 || chosen >= pred_cb.n_rows) {
-                *status = 1;
-                if (SAMPLED) {
-                    sampled->status = 1;
-                    sampled->err_pos = pos;
-                }
+            if (dist.err) {
+                sampled->status = dist.err;
+                sampled->err_pos = pos;
+                *status = dist.err;
+                return;  // sampler error: the walk stops
             }
+            const int idx = pick_index(dist.weights, dist.n_keep, uniforms[pos - 1] * dist.total);
+            best_b = dist.tokens[idx];
+            sampled->n_sampled = pos;
+            int cnt = 0;
+            for (int i = 0; i < dist.n_keep; i++) {
+                if (!(dist.weights[i] > 0.0)) continue;
+                dflash_weighted_candidate &wc = sampled->cands[(pos - 1) * top_k + cnt++];
+                wc.token = cands[dist.tokens[i]];
+                wc.weight = dist.weights[i];
             }
+            sampled->counts[pos - 1] = cnt;
         }
-        __syncthreads();
-        const int chosen = chosen_s;
-        if (chosen < 0 || chosen >= pred_cb.n_rows) return;
-        for (int r = tid; r < rank; r += kSelThreads) pred[r] = codebook_elem(pred_cb, chosen, r);
-        __syncthreads();
+        const int32_t chosen = cands[best_b];
+        out[pos] = chosen;
+        if (chosen < 0 || chosen >= n_pred_rows) {
+            *status = 1;
+            if (SAMPLED) {
+                sampled->status = 1;
+                sampled->err_pos = pos;
+            }
+            return;
+        }
+        prev_a = best_b;
     }
+}
+
+// Both launches of a walk: the score table ((n - 1) x top_k x top_k floats of context workspace behind *ws_off), then
+// the walk itself.
+template <bool SAMPLED>
+int32_t launch_walk(dflash_ctx *ctx, size_t *ws_off, const Codebook &pc, const Codebook &sc, int top_k, int rank, int carry, int n,
+                    const int32_t *ids, const float *vals, const float *sel_h, int32_t *out, int32_t *status, float temperature,
+                    const double *uniforms, SampledOut *sampled, hipStream_t st) {
+    float *table = dfl_ws_take<float>(ctx, ws_off, static_cast<size_t>(15) * kSelMaxTopK * kSelMaxTopK * sizeof(float));
+    if (!table) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "select_draft_path: workspace too small");
+    if (n > 1) {
+        const size_t lds = static_cast<size_t>(1 + top_k) * rank * sizeof(float);
+        if (lds > 48 * 1024) {
+            if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(dflash2_scores_kernel),
+                                                        (1 + kSelMaxTopK) * kSelMaxRank * sizeof(float)))
+                return rc_;
+        }
+        dflash2_scores_kernel<<<dim3(top_k, n - 1), kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry, n, ids, vals, sel_h, table);
+    }
+    dflash2_select_kernel<SAMPLED><<<1, kSelThreads, 0, st>>>(pc.n_rows, sc.n_rows, top_k, carry, n, ids, table, out, status, temperature,
+                                                               uniforms, sampled);
+    DFL_HIP_CHECK(ctx, hipGetLastError());
+    return DFLASH_OK;
 }
 
 int32_t check_codebook(dflash_ctx *ctx, const dflash_codebook *cb, int rank, Codebook *out, const char *what) {
@@ -269,15 +301,9 @@ extern "C" int32_t dflash_select_draft_path(dflash_ctx *ctx, const dflash_codebo
     int32_t *status = dfl_ws_take<int32_t>(ctx, &off, sizeof(int32_t));
     if (!status) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "select_draft_path: workspace too small");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const size_t lds = static_cast<size_t>(2 + top_k) * rank * sizeof(float);
-    if (lds > 48 * 1024) {
-        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(dflash2_select_kernel<false>),
-                                                    (2 + kSelMaxTopK) * kSelMaxRank * sizeof(float)))
-            return rc_;
-    }
-    dflash2_select_kernel<false><<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
-                                                              out_tokens, status, 0.0f, nullptr, nullptr);
-    DFL_HIP_CHECK(ctx, hipGetLastError());
+    if ((rc = launch_walk<false>(ctx, &off, pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h, out_tokens, status, 0.0f,
+                                 nullptr, nullptr, st)))
+        return rc;
     if (out_tokens_host) {
         // the blocking form also reports an invalid predecessor row, as the reference's CPU walk does
         int32_t status_host = 0;
@@ -321,15 +347,9 @@ extern "C" int32_t dflash_select_draft_path_sampled(dflash_ctx *ctx, const dflas
     double u_host[16] = {0};
     if (n > 1) dflash_sampler_peek(proposal_sampler, n - 1, u_host);
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(uniforms, u_host, sizeof(u_host), hipMemcpyHostToDevice, st));
-    const size_t lds = static_cast<size_t>(2 + top_k) * rank * sizeof(float);
-    if (lds > 48 * 1024) {
-        if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(dflash2_select_kernel<true>),
-                                                    (2 + kSelMaxTopK) * kSelMaxRank * sizeof(float)))
-            return rc_;
-    }
-    dflash2_select_kernel<true><<<1, kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h,
-                                                             out_dev, status, pc_cfg.temperature, uniforms, sampled);
-    DFL_HIP_CHECK(ctx, hipGetLastError());
+    if ((rc = launch_walk<true>(ctx, &off, pc, sc, top_k, rank, carry_token, n, topk_ids, topk_vals, sel_h, out_dev, status,
+                                pc_cfg.temperature, uniforms, sampled, st)))
+        return rc;
     static_assert(sizeof(SampledOut) <= DFL_PINNED_BYTES, "the walk's result is read back through the context's pinned page");
     const SampledOut &host = *static_cast<const SampledOut *>(ctx->pinned);
     DFL_HIP_CHECK(ctx, hipMemcpyAsync(ctx->pinned, sampled, sizeof(SampledOut), hipMemcpyDeviceToHost, st));

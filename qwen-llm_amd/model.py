@@ -290,7 +290,9 @@ def synth_target_weights_device(cfg: ModelConfig, seed: int, device, wtype: int 
     return w
 
 
-def synth_draft_weights_device(cfg: DraftConfig, seed: int, device, wtype: int = synth.Q4_K):
+def synth_draft_weights_device(cfg: DraftConfig, seed: int, device, wtype: int = synth.Q4_K, vocab=None):
+    """synth_draft_weights with every matrix generated on the device as random quant blocks (for timing; a DFlash-2
+    configuration gets its convolution and selector tensors too and needs ``vocab`` for the codebooks)."""
     torch = _torch()
     gen = torch.Generator(device=device)
     gen.manual_seed(seed + 7919)
@@ -308,6 +310,21 @@ def synth_draft_weights_device(cfg: DraftConfig, seed: int, device, wtype: int =
             "wv": _dev_mat(wtype, kv_dim, H, H ** -0.5, gen, device), "wo": _dev_mat(wtype, H, q_dim, q_dim ** -0.5, gen, device),
             "gate": _dev_mat(wtype, cfg.ffn, H, H ** -0.5, gen, device), "up": _dev_mat(wtype, cfg.ffn, H, H ** -0.5, gen, device),
             "down": _dev_mat(wtype, H, cfg.ffn, cfg.ffn ** -0.5, gen, device), "is_swa": 0})
+        if cfg.conv_kernel_size:
+            dyn_dim = 2 * cfg.conv_kernel_size * (H // cfg.conv_group_size)
+            L = w["layers"][-1]
+            L["conv_attn_proj"] = _dev_mat(wtype, dyn_dim, H, 0.1 * H ** -0.5, gen, device)
+            L["conv_ffn_proj"] = _dev_mat(wtype, dyn_dim, H, 0.1 * H ** -0.5, gen, device)
+            for name in ("conv_attn_base", "conv_ffn_base"):  # near the identity tap, f32 [2][kernel][hidden]
+                base = 0.1 * torch.randn((2, cfg.conv_kernel_size, H), generator=gen, device=device)
+                base[:, 0, :] += 1.0
+                L[name] = base
+    if cfg.selector_rank:
+        if vocab is None:
+            raise ValueError("a DFlash-2 selector needs the target vocabulary size")
+        w["selector_hidden"] = _dev_mat(wtype, cfg.selector_rank, H, H ** -0.5, gen, device)
+        w["selector_predecessor"] = _dev_mat(wtype, vocab, cfg.selector_rank, 1.0, gen, device)
+        w["selector_successor"] = _dev_mat(wtype, vocab, cfg.selector_rank, 1.0, gen, device)
     return w
 
 
