@@ -47,17 +47,68 @@ __device__ float block_sum(float v, float *sh) {
 // sigmoid(y . gate_w) also goes to gate_out[row] (the shared-expert gate of a mixture-of-experts
 // layer, forward.rs:749-824: the normalised row is at hand here, in registers).  With y_xf (n a multiple of 256, at most
 // 8192: every width the whole-K GEMMs take), y also goes there as f16 in the fragment order a whole-K GEMM reads (common.h, "XF").
+// With conv.dyn (a DFlash-2 drafter's residual adds, metal_dflash.rs:16795-16820, 17003-17022; rows of one block
+// only): what is added to row t is not add[t] but the side-1 dynamic convolution of the rows of add,
+//   sum_tap (base[1][tap][c] + dyn[t][1][tap][c / group_size]) * add[t - tap][c]   (rows before the block read as zeros),
+// taps accumulated in order with a fused multiply-add - the arithmetic of dflash2_conv_kernel, which a launch of its
+// own ran before.
+struct ConvResid {
+    const float *dyn = nullptr;   // [rows][2][kernel][n / group_size]
+    const float *base = nullptr;  // [2][kernel][n]
+    int kernel_size = 0, group_size = 1;
+};
 __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, const float *__restrict__ add,
                                                        const float *__restrict__ w, float *__restrict__ y, int n,
                                                        float eps, const float *__restrict__ gate_w,
                                                        float *__restrict__ gate_out, void *__restrict__ y_xf = nullptr,
-                                                       int y_xf_kind = 0, size_t xf_stride = 0) {
+                                                       int y_xf_kind = 0, size_t xf_stride = 0, ConvResid conv = ConvResid()) {
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float sh[4];
     float *xr = x + static_cast<size_t>(blockIdx.x) * n;
     const float *ar = add ? add + static_cast<size_t>(blockIdx.x) * n : nullptr;
     float *yr = y + static_cast<size_t>(blockIdx.x) * n;
     const int tid = threadIdx.x;
+    if (conv.dyn && ar && n <= 8192 && n % 4 == 0) {
+        // (the same two passes as below; the residual term is the convolution)
+        constexpr int kVec = 8;
+        const int t = blockIdx.x, ks = conv.kernel_size, n_groups = n / conv.group_size;
+        const float *dyn_t = conv.dyn + (static_cast<size_t>(t) * 2 + 1) * ks * n_groups;
+        const float *base1 = conv.base + static_cast<size_t>(ks) * n;
+        f4 v[kVec];
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kVec; j++) {
+            const int i = 4 * (tid + 256 * j);
+            v[j] = f4{0, 0, 0, 0};
+            if (i < n) {
+                f4 acc = {0, 0, 0, 0};
+                for (int tap = 0; tap < ks && tap <= t; tap++) {
+                    const f4 b = *reinterpret_cast<const f4 *>(base1 + static_cast<size_t>(tap) * n + i);
+                    const f4 src = *reinterpret_cast<const f4 *>(add + static_cast<size_t>(t - tap) * n + i);
+                    const float *dg = dyn_t + static_cast<size_t>(tap) * n_groups;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[e] = __builtin_fmaf(b[e] + dg[(i + e) / conv.group_size], src[e], acc[e]);
+                }
+                v[j] = *reinterpret_cast<const f4 *>(xr + i) + acc;
+                *reinterpret_cast<f4 *>(xr + i) = v[j];
+            }
+            s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
+        }
+        s = block_sum(s, sh);
+        const float scale = 1.0f / sqrtf(s / static_cast<float>(n) + eps);
+#pragma unroll
+        for (int j = 0; j < kVec; j++) {
+            const int i = 4 * (tid + 256 * j);
+            if (i < n) {
+                const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
+                *reinterpret_cast<f4 *>(yr + i) = o;
+                if (y_xf)
+                    dfl_xf_store_pair(static_cast<uint8_t *>(y_xf) + (blockIdx.x >> 4) * xf_stride, y_xf_kind, blockIdx.x & 15, i & ~7, o[0],
+                                      o[1], o[2], o[3]);
+            }
+        }
+        return;
+    }
     if (n <= 8192 && n % 4 == 0) {
         // (vectors past the row are zeros and add nothing: a row of up to 4096 values sums exactly as with four vectors)
         constexpr int kVec = 8;
@@ -1611,6 +1662,11 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
     if ((rc = embed_rows(ctx, target->token_embd, s->ids, N, H, s->x, st))) return rc;
 
     const float *pending_resid = nullptr;
+    // DFlash-2: the side-1 convolution of a sublayer's output is what gets added to the residual; the norm kernel that
+    // adds it computes it on the way (rms_norm_kernel's ConvResid), unless the width is one that kernel keeps no row in
+    // registers for (then a launch of dflash2_conv_kernel comes first, as for the side-0 convolutions)
+    const bool conv_in_norm = conv && H <= 8192 && H % 4 == 0;
+    ConvResid pending_conv;
     for (int il = 0; il < c.n_layers; il++) {
         const dflash_draft_layer &L = head->layers[il];
         float *kc = s->k_ctx + il * static_cast<size_t>(s->capacity) * kv_dim;
@@ -1620,13 +1676,21 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         // the previous layer's second residual (x += ffn output) is folded into this norm
         // (in a DFlash-2 layer the side-0 convolution sits between the norm and the projection: it writes the fragment-order rows)
         const LayerXf xk = layer_xf(ctx, L, fast && s->pk != nullptr, H, static_cast<int64_t>(q_dim), static_cast<int64_t>(kv_dim), c.ffn, true);
+        // (DFlash-2: the norm's fragment-order rows are for the coefficient projection when that is a one-launch product;
+        // the convolution then writes q/k/v's over them, later in the stream)
+        const int cp_attn = conv && fast ? dfl_whole_kind(ctx, L.conv_attn_proj.type, H, conv_dyn_dim, 0) : DFL_XF_NONE;
+        const int cp_ffn = conv && fast ? dfl_whole_kind(ctx, L.conv_ffn_proj.type, H, conv_dyn_dim, 0) : DFL_XF_NONE;
+        const int norm1_kind = conv ? cp_attn : xk.qkv;
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, L.attn_norm, s->cur, H, c.eps, nullptr, nullptr,
-                                           xk.qkv && !conv ? s->xf_cur : nullptr, xk.qkv);
+                                           norm1_kind ? s->xf_cur : nullptr, norm1_kind, 0, pending_conv);
         // DFlash-2 attention convolution (metal_dflash.rs:16210-16262): the dynamic coefficients come
         // from the normed input and serve both sides; q/k/v read the side-0 result
         const float *attn_src = s->cur;
         if (conv) {
-            if ((rc = gemm(ctx, L.conv_attn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st))) return rc;
+            rc = cp_attn ? dfl_gemm_whole(ctx, L.conv_attn_proj.type, L.conv_attn_proj.data, s->xf_cur, s->conv_dyn, H, conv_dyn_dim, N, 0,
+                                          nullptr, DFL_XF_NONE, st)
+                         : gemm(ctx, L.conv_attn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st);
+            if (rc) return rc;
             if ((rc = dfl_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_attn_base, s->conv_buf, N, H, c.conv_kernel_size,
                                        c.conv_group_size, 0, st, xk.qkv ? s->xf_cur : nullptr, xk.qkv)))
                 return rc;
@@ -1666,17 +1730,24 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
         // residual 1 (x += attn_output; DFlash-2: its side-1 convolution, same coefficients, :16795-16820),
         // folded into the norm that follows
         const float *resid = s->mix;
-        if (conv) {
+        ConvResid resid_conv;
+        if (conv_in_norm) {
+            resid_conv = ConvResid{s->conv_dyn, L.conv_attn_base, c.conv_kernel_size, c.conv_group_size};
+        } else if (conv) {
             if ((rc = dflash_dflash2_conv(ctx, s->mix, s->conv_dyn, L.conv_attn_base, s->conv_buf, N, H, c.conv_kernel_size,
                                           c.conv_group_size, 1, st)))
                 return rc;
             resid = s->conv_buf;
         }
+        const int norm2_kind = conv ? cp_ffn : xk.gate_up;
         rms_norm_kernel<<<N, 256, 0, st>>>(s->x, resid, L.post_norm, s->cur, H, c.eps, nullptr, nullptr,
-                                           xk.gate_up && !conv ? s->xf_cur : nullptr, xk.gate_up);
+                                           norm2_kind ? s->xf_cur : nullptr, norm2_kind, 0, resid_conv);
         const float *ffn_src = s->cur;
         if (conv) {  // the FFN pair (:16836-16885, 17003-17022)
-            if ((rc = gemm(ctx, L.conv_ffn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st))) return rc;
+            rc = cp_ffn ? dfl_gemm_whole(ctx, L.conv_ffn_proj.type, L.conv_ffn_proj.data, s->xf_cur, s->conv_dyn, H, conv_dyn_dim, N, 0,
+                                         nullptr, DFL_XF_NONE, st)
+                        : gemm(ctx, L.conv_ffn_proj, s->cur, s->conv_dyn, H, conv_dyn_dim, N, st);
+            if (rc) return rc;
             if ((rc = dfl_dflash2_conv(ctx, s->cur, s->conv_dyn, L.conv_ffn_base, s->conv_buf, N, H, c.conv_kernel_size,
                                        c.conv_group_size, 0, st, xk.gate_up ? s->xf_cur : nullptr, xk.gate_up)))
                 return rc;
@@ -1691,7 +1762,10 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
             rc = gemm(ctx, L.down, s->g, s->mix, c.ffn, H, N, st);
         if (rc) return rc;
         resid = s->mix;
-        if (conv) {
+        pending_conv = ConvResid();
+        if (conv_in_norm) {
+            pending_conv = ConvResid{s->conv_dyn, L.conv_ffn_base, c.conv_kernel_size, c.conv_group_size};
+        } else if (conv) {
             if ((rc = dflash_dflash2_conv(ctx, s->mix, s->conv_dyn, L.conv_ffn_base, s->conv_buf, N, H, c.conv_kernel_size,
                                           c.conv_group_size, 1, st)))
                 return rc;
@@ -1701,7 +1775,7 @@ int32_t draft_block_impl(dflash_ctx *ctx, const dflash_model *target, const dfla
     }
     const int head_kind = dfl_whole_kind(ctx, target->output.type, H, V, 0);
     rms_norm_kernel<<<N, 256, 0, st>>>(s->x, pending_resid, head->output_norm, s->cur, H, c.eps, nullptr, nullptr,
-                                       head_kind ? s->xf_cur : nullptr, head_kind);
+                                       head_kind ? s->xf_cur : nullptr, head_kind, 0, pending_conv);
     if (head_kind)
         rc = dfl_gemm_whole(ctx, target->output.type, target->output.data, s->xf_cur, lg, H, V, N, 0, nullptr, DFL_XF_NONE, st);
     else

@@ -616,7 +616,8 @@ class DraftHead:
                     setattr(L, k, up.q(Lw[k], shape[k]))
             L.is_swa = int(Lw.get("is_swa", 0))
             if cfg.conv_kernel_size:
-                L.conv_attn_proj, L.conv_ffn_proj = up.q(Lw["conv_attn_proj"]), up.q(Lw["conv_ffn_proj"])
+                dyn_dim = 2 * cfg.conv_kernel_size * (H // cfg.conv_group_size)
+                L.conv_attn_proj, L.conv_ffn_proj = up.q(Lw["conv_attn_proj"], (dyn_dim, H)), up.q(Lw["conv_ffn_proj"], (dyn_dim, H))
                 L.conv_attn_base, L.conv_ffn_base = up.f32(Lw["conv_attn_base"]), up.f32(Lw["conv_ffn_base"])
         self.c = DraftHeadC(DraftCfgC(**cfg.as_dict()), self._layers, up.q(weights["fc"], (H, cfg.n_taps * H)), up.f32(weights["hidden_norm"]),
                             up.f32(weights["output_norm"]))
