@@ -457,6 +457,44 @@ def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048, dflash2=True):
     return res
 
 
+def dense_verify_section(ctx, n_layers=64, context=2048, blocks=40):
+    """The 16-token verify step of a 27B-shaped dense Q4_K target as a whole: hidden 5120, 32 q / 8 kv heads of 128
+    (fused q|k|v 5120 -> 6144), SwiGLU FFN 17408 (the three matrix shapes of the headline are this layer's), `n_layers`
+    layers, output head 5120 -> 151936 in Q6_K; random quant blocks generated on the device.  Reports the time of one
+    packed verify of 16 rows at `context` (every layer's GEMMs with their reductions, norms, RoPE, attention, SwiGLU;
+    head and argmax included) and the rate at which it streams the model's weights."""
+    import numpy as np
+    import torch
+
+    import qwen_llm_amd as dfl
+
+    cfg = dfl.ModelConfig(n_layers=n_layers, hidden=5120, n_q=32, n_kv=8, head_dim=128, ffn=17408, vocab=151936)
+    target = dfl.TargetModel(ctx, cfg, dfl.synth_target_weights_device(cfg, 3, "cuda", attn_type=dfl.synth.Q4_K))
+    sess = dfl.Session(ctx, target, context + 64, [1])
+    prompt = np.random.default_rng(2).integers(0, cfg.vocab - 1, context + 16).tolist()
+    sess.prefill_blocks(prompt[:context], 0, want_hidden=False)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        sess.encode_packed_verify_layer_major(prompt[context:], context, want_hidden=False)
+        sess.encode_restore_after_partial_accept(context, 16, 0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(blocks):
+        sess.encode_packed_verify_layer_major(prompt[context:], context, want_hidden=False)
+        sess.encode_restore_after_partial_accept(context, 16, 0)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / blocks * 1e3
+    sess.close()
+    H, F, qkv = cfg.hidden, cfg.ffn, (cfg.n_q + 2 * cfg.n_kv) * cfg.head_dim
+    layer_bytes = (3 * H * F + H * qkv + cfg.n_q * cfg.head_dim * H) * 144 // 256
+    head_bytes = H * cfg.vocab * 210 // 256
+    streamed = n_layers * layer_bytes + head_bytes
+    return {"model": f"27B-shaped dense Q4_K target: {n_layers} layers, hidden 5120, 32 q / 8 kv heads of 128, FFN 17408, Q6_K head 151936",
+            "context": context, "rows": 16, "ms_per_verify": ms, "weight_bytes_per_verify": streamed,
+            "GBps": streamed / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": streamed / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "us_per_layer": (ms * 1e3) / n_layers, "weights_GB": target.weight_bytes() / 1e9}
+
+
 def moe_layer_probe(nd, blocks=60):
     """Verify blocks on a 4-layer 35B-A3B-shaped mixture-of-experts target (random quant blocks) whose 16 tokens are
     drawn from `nd` distinct ones: 16 distinct random tokens touch about 80 of the 128 experts per layer, 4 about 30,
@@ -547,6 +585,7 @@ def main():
     ap.add_argument("--gemm-only", action="store_true", help="skip the attention, acceptance and end-to-end sections")
     ap.add_argument("--moe-layer", metavar="N", type=int, help="only run the mixture-of-experts layer probe with blocks of N "
                                                                "distinct tokens (16, 4, 1 ...) and exit; for kernel traces")
+    ap.add_argument("--dense-verify", action="store_true", help="only run the 27B-shaped dense verify-step probe and print its result")
     ap.add_argument("--shapes", default="0,1,2", help="which of the three GEMM shapes take part (for per-shape profiles; the "
                                                       "metric is defined on all three)")
     args = ap.parse_args()
@@ -560,6 +599,11 @@ def main():
 
     if args.moe_layer:
         moe_layer_probe(max(1, min(16, args.moe_layer)))
+        return
+    if args.dense_verify:
+        import qwen_llm_amd as dfl
+
+        print(json.dumps({"dense_verify_27b": dense_verify_section(dfl.Context(0, workspace_bytes=256 << 20))}))
         return
 
     import numpy as np
@@ -745,6 +789,7 @@ def main():
             out["attention"] = attention_section(ctx, with_cpu)
             out["acceptance"] = acceptance_section(ctx, with_cpu)
             out["c1_verify"] = c1_section(ctx, with_cpu)
+            out["dense_verify_27b"] = dense_verify_section(ctx)
         except Exception as e:  # the GEMM line above stays valid
             out["sections_error"] = f"{type(e).__name__}: {e}"
     if not args.no_e2e and not args.gemm_only:

@@ -639,8 +639,11 @@ WholePlan whole_plan(const dflash_ctx *ctx, int32_t w_type, int64_t n_in, int64_
     const int tiles = static_cast<int>((n_out + 15) / 16);
     int R = pair_ffn ? 2 : 1;
     int n_units = pair_ffn ? static_cast<int>(pair_ffn / 16) : tiles;
-    // one round of the chip: at most one workgroup per CU (a wave's registers leave room for one), a quarter more tolerated
-    const int max_wg = ctx->n_cu + ctx->n_cu / 4;
+    // one round of the chip: at most one workgroup per CU (a wave's registers leave room for one)
+    // (a quarter of a round more, 320 workgroups on 256 CUs, measured slower than two tiles per wave on 160: 10.1 -> 8.6 us
+    // for 4096 -> 5120 Q4_K, 14.9 -> 14.0 us for 5120 -> 5120 Q6_K; DFLASH_WHOLE_TOL_PCT=25 for the former rule)
+    static const int env_tol = env_int("DFLASH_WHOLE_TOL_PCT", 0);
+    const int max_wg = ctx->n_cu + ctx->n_cu * env_tol / 100;
     if (!pair_ffn && (n_units + tl - 1) / tl > max_wg) {
         R = 2;
         n_units = (tiles + 1) / 2;
