@@ -558,7 +558,7 @@ __global__ void __launch_bounds__(1024) gemm_q6t_loop_kernel(WholeArgs a) {
     for (int it = 0;; it++) {
         const int next = unit + stride;
         const int slot = it & 1;
-        if (next < n_tiles) issue(next, slot ^ 1);  // (that buffer's unit was consumed in the previous round: its reads are complete)
+        if (next < n_tiles) issue(next, slot ^ 1);  // (that buffer's unit was consumed one iteration ago: its reads are complete)
         float4_t acc = {0, 0, 0, 0}, acc_sub = {0, 0, 0, 0};
         if (unit < n_tiles) {
             if (next < n_tiles)
