@@ -72,6 +72,10 @@ struct SampledOut {
     dflash_weighted_candidate cands[15 * 16];    // [pos - 1][top_k], distribution order
 };
 
+// where the raw rows sit in the scores kernel's LDS, behind the decoded ones (bytes)
+__host__ __device__ inline size_t sel_raw_pred_bytes(size_t row_bytes) { return (row_bytes + 15) / 16 * 16; }
+__host__ __device__ inline size_t sel_raw_succ_stride(size_t row_bytes) { return (row_bytes + 3) / 4 * 4; }
+
 // The walk's scores do not have to wait for the walk: the predecessor of position pos is one of the top_k candidates
 // of position pos - 1 (the carry token for pos = 1), so score(pos, a, b) for every candidate a of the previous position
 // and every candidate b of this one is known work up front: (n - 1) x top_k workgroups, all at once, each with the
@@ -84,19 +88,41 @@ __global__ void __launch_bounds__(kSelThreads)
     dflash2_scores_kernel(Codebook pred_cb, Codebook succ_cb, int top_k, int rank, int carry, int n,
                           const int32_t *__restrict__ ids, const float *__restrict__ vals, const float *__restrict__ sel_h,
                           float *__restrict__ table) {
-    extern __shared__ float lds[];  // gate[rank], succ[top_k][rank]
+    extern __shared__ float lds[];  // gate[rank], succ[top_k][rank], then the raw rows: predecessor, top_k successors
     float *gate = lds, *succ = lds + rank;
     const int tid = threadIdx.x;
     const int a = blockIdx.x, pos = 1 + blockIdx.y;
     if (pos == 1 && a != 0) return;  // (one predecessor only: the carry token)
     const int32_t prev = pos == 1 ? carry : ids[(pos - 1) * top_k + a];
     if (prev < 0 || prev >= pred_cb.n_rows) return;
+    // The rows' bytes come in with coalesced loads first (decoding element by element straight from memory cost a cold
+    // trip per field of every element).  Rows of every codebook type are a whole number of 2-byte words and start on
+    // one; in LDS the predecessor row sits first and the successor rows follow, each on a 4-byte boundary.
+    uint8_t *raw = reinterpret_cast<uint8_t *>(lds + static_cast<size_t>(1 + top_k) * rank);
+    const int pw = static_cast<int>(pred_cb.row_bytes / 2), sw = static_cast<int>(succ_cb.row_bytes / 2);
+    const size_t succ_at = sel_raw_pred_bytes(pred_cb.row_bytes), succ_stride = sel_raw_succ_stride(succ_cb.row_bytes);
+    {
+        const uint16_t *src = reinterpret_cast<const uint16_t *>(pred_cb.data + static_cast<size_t>(prev) * pred_cb.row_bytes);
+        for (int i = tid; i < pw; i += kSelThreads) reinterpret_cast<uint16_t *>(raw)[i] = src[i];
+    }
+    for (int e = tid; e < top_k * sw; e += kSelThreads) {
+        const int b = e / sw, i = e - b * sw;
+        const int32_t cand = ids[pos * top_k + b];
+        if (cand >= 0 && cand < succ_cb.n_rows)
+            reinterpret_cast<uint16_t *>(raw + succ_at + b * succ_stride)[i] =
+                reinterpret_cast<const uint16_t *>(succ_cb.data + static_cast<size_t>(cand) * succ_cb.row_bytes)[i];
+    }
+    __syncthreads();
+    Codebook pred_l = pred_cb, succ_l = succ_cb;  // the same rows, now rows of an LDS copy
+    pred_l.data = raw;
+    succ_l.data = raw + succ_at;
+    succ_l.row_bytes = succ_stride;
     const float *hrow = sel_h + static_cast<size_t>(pos) * rank;
-    for (int r = tid; r < rank; r += kSelThreads) gate[r] = codebook_elem(pred_cb, prev, r) * hrow[r];
+    for (int r = tid; r < rank; r += kSelThreads) gate[r] = codebook_elem(pred_l, 0, r) * hrow[r];
     for (int e = tid; e < top_k * rank; e += kSelThreads) {
         const int b = e / rank, r = e - b * rank;
         const int32_t cand = ids[pos * top_k + b];
-        if (cand >= 0 && cand < succ_cb.n_rows) succ[e] = codebook_elem(succ_cb, cand, r);
+        if (cand >= 0 && cand < succ_cb.n_rows) succ[e] = codebook_elem(succ_l, b, r);
     }
     __syncthreads();
     if (tid < top_k) {
@@ -143,6 +169,36 @@ __global__ void __launch_bounds__(kSelThreads)
     for (int e = tid; e < (n - 1) * top_k * top_k; e += kSelThreads) table_s[e] = table[e];
     for (int e = tid; e < n * top_k; e += kSelThreads) ids_s[e] = ids[e];
     __syncthreads();
+    if (!SAMPLED) {
+        // greedy: lane b holds candidate b of the position; the first strict maximum over the candidates with a successor
+        // row, as the scalar loop `if (score[b] > best)` from best = -inf keeps it (a NaN or -inf score is never greater:
+        // with none greater, candidate 0 stands)
+        if (tid >= 64) return;
+        int prev_a = 0;
+        for (int pos = 1; pos < n; pos++) {
+            float sc = -INFINITY;
+            int32_t cand = -1;
+            if (tid < top_k) {
+                cand = ids_s[pos * top_k + tid];
+                const float v = table_s[(static_cast<size_t>(pos - 1) * top_k + prev_a) * top_k + tid];
+                if (cand >= 0 && cand < n_succ_rows && v > -INFINITY) sc = v;
+            }
+            float best = sc;
+#pragma unroll
+            for (int off = 1; off < 16; off <<= 1) best = fmaxf(best, __shfl_xor(best, off, 64));
+            best = __shfl(best, 0, 64);  // (lanes 0..15 agree; the others hold -inf)
+            const unsigned long long at = __ballot(tid < top_k && sc == best && best > -INFINITY);
+            const int best_b = at ? __builtin_ctzll(at) : 0;
+            const int32_t chosen = __shfl(cand, best_b, 64);
+            if (tid == 0) out[pos] = chosen;
+            if (chosen < 0 || chosen >= n_pred_rows) {
+                if (tid == 0) *status = 1;
+                return;
+            }
+            prev_a = best_b;
+        }
+        return;
+    }
     if (tid != 0) return;
     int prev_a = 0;  // which candidate of the previous position was picked (the carry token's scores sit in row 0)
     for (int pos = 1; pos < n; pos++) {
@@ -227,11 +283,13 @@ int32_t launch_walk(dflash_ctx *ctx, size_t *ws_off, const Codebook &pc, const C
     float *table = dfl_ws_take<float>(ctx, ws_off, static_cast<size_t>(15) * kSelMaxTopK * kSelMaxTopK * sizeof(float));
     if (!table) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "select_draft_path: workspace too small");
     if (n > 1) {
-        const size_t lds = static_cast<size_t>(1 + top_k) * rank * sizeof(float);
+        // (decoded rows as floats + the same rows' bytes)
+        const size_t lds = static_cast<size_t>(1 + top_k) * rank * sizeof(float) + sel_raw_pred_bytes(pc.row_bytes) +
+                           static_cast<size_t>(top_k) * sel_raw_succ_stride(sc.row_bytes);
+        if (pc.row_bytes % 2 || sc.row_bytes % 2 || reinterpret_cast<uintptr_t>(pc.data) % 2 || reinterpret_cast<uintptr_t>(sc.data) % 2)
+            return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "select_draft_path: codebook rows must start on 2-byte boundaries");
         if (lds > 48 * 1024) {
-            if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(dflash2_scores_kernel),
-                                                        (1 + kSelMaxTopK) * kSelMaxRank * sizeof(float)))
-                return rc_;
+            if (const int32_t rc_ = dfl_raise_lds_limit(ctx, reinterpret_cast<const void *>(dflash2_scores_kernel), lds)) return rc_;
         }
         dflash2_scores_kernel<<<dim3(top_k, n - 1), kSelThreads, lds, st>>>(pc, sc, top_k, rank, carry, n, ids, vals, sel_h, table);
     }
