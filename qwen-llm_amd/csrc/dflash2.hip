@@ -75,6 +75,10 @@ struct SampledOut {
 // where the raw rows sit in the scores kernel's LDS, behind the decoded ones (bytes)
 __host__ __device__ inline size_t sel_raw_pred_bytes(size_t row_bytes) { return (row_bytes + 15) / 16 * 16; }
 __host__ __device__ inline size_t sel_raw_succ_stride(size_t row_bytes) { return (row_bytes + 3) / 4 * 4; }
+// floats of the decoded rows in front of them: gate[rank], succ[top_k][rank + 1], rounded up to a 16-byte boundary
+__host__ __device__ inline size_t sel_decoded_floats(int top_k, int rank) {
+    return (static_cast<size_t>(rank) + static_cast<size_t>(top_k) * (rank + 1) + 3) / 4 * 4;
+}
 
 // The walk's scores do not have to wait for the walk: the predecessor of position pos is one of the top_k candidates
 // of position pos - 1 (the carry token for pos = 1), so score(pos, a, b) for every candidate a of the previous position
@@ -88,8 +92,11 @@ __global__ void __launch_bounds__(kSelThreads)
     dflash2_scores_kernel(Codebook pred_cb, Codebook succ_cb, int top_k, int rank, int carry, int n,
                           const int32_t *__restrict__ ids, const float *__restrict__ vals, const float *__restrict__ sel_h,
                           float *__restrict__ table) {
-    extern __shared__ float lds[];  // gate[rank], succ[top_k][rank], then the raw rows: predecessor, top_k successors
+    extern __shared__ float lds[];  // gate[rank], succ[top_k][rank + 1], then the raw rows: predecessor, top_k successors
+    // (a successor row every rank + 1 floats: the sixteen scoring threads read element r of sixteen rows at once, and rows
+    // a power of two apart would all sit in one bank)
     float *gate = lds, *succ = lds + rank;
+    const int srow = rank + 1;
     const int tid = threadIdx.x;
     const int a = blockIdx.x, pos = 1 + blockIdx.y;
     if (pos == 1 && a != 0) return;  // (one predecessor only: the carry token)
@@ -98,7 +105,7 @@ __global__ void __launch_bounds__(kSelThreads)
     // The rows' bytes come in with coalesced loads first (decoding element by element straight from memory cost a cold
     // trip per field of every element).  Rows of every codebook type are a whole number of 2-byte words and start on
     // one; in LDS the predecessor row sits first and the successor rows follow, each on a 4-byte boundary.
-    uint8_t *raw = reinterpret_cast<uint8_t *>(lds + static_cast<size_t>(1 + top_k) * rank);
+    uint8_t *raw = reinterpret_cast<uint8_t *>(lds + sel_decoded_floats(top_k, rank));
     const int pw = static_cast<int>(pred_cb.row_bytes / 2), sw = static_cast<int>(succ_cb.row_bytes / 2);
     const size_t succ_at = sel_raw_pred_bytes(pred_cb.row_bytes), succ_stride = sel_raw_succ_stride(succ_cb.row_bytes);
     {
@@ -122,7 +129,7 @@ __global__ void __launch_bounds__(kSelThreads)
     for (int e = tid; e < top_k * rank; e += kSelThreads) {
         const int b = e / rank, r = e - b * rank;
         const int32_t cand = ids[pos * top_k + b];
-        if (cand >= 0 && cand < succ_cb.n_rows) succ[e] = codebook_elem(succ_l, b, r);
+        if (cand >= 0 && cand < succ_cb.n_rows) succ[b * srow + r] = codebook_elem(succ_l, b, r);
     }
     __syncthreads();
     if (tid < top_k) {
@@ -130,7 +137,7 @@ __global__ void __launch_bounds__(kSelThreads)
         float sc = __builtin_nanf("");  // skipped candidates never compare greater
         if (cand >= 0 && cand < succ_cb.n_rows) {
             float dot = 0.0f;
-            const float *sr = succ + tid * rank;
+            const float *sr = succ + tid * srow;
             for (int r = 0; r < rank; r++) dot += gate[r] * sr[r];  // two roundings each (contraction is off in this file)
             sc = vals[pos * top_k + tid] + dot;
         }
@@ -284,7 +291,7 @@ int32_t launch_walk(dflash_ctx *ctx, size_t *ws_off, const Codebook &pc, const C
     if (!table) return dfl_fail(ctx, DFLASH_ERR_WORKSPACE, "select_draft_path: workspace too small");
     if (n > 1) {
         // (decoded rows as floats + the same rows' bytes)
-        const size_t lds = static_cast<size_t>(1 + top_k) * rank * sizeof(float) + sel_raw_pred_bytes(pc.row_bytes) +
+        const size_t lds = sel_decoded_floats(top_k, rank) * sizeof(float) + sel_raw_pred_bytes(pc.row_bytes) +
                            static_cast<size_t>(top_k) * sel_raw_succ_stride(sc.row_bytes);
         if (pc.row_bytes % 2 || sc.row_bytes % 2 || reinterpret_cast<uintptr_t>(pc.data) % 2 || reinterpret_cast<uintptr_t>(sc.data) % 2)
             return dfl_fail(ctx, DFLASH_ERR_ALIGNMENT, "select_draft_path: codebook rows must start on 2-byte boundaries");

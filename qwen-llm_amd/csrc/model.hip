@@ -82,12 +82,21 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
             v[j] = f4{0, 0, 0, 0};
             if (i < n) {
                 f4 acc = {0, 0, 0, 0};
+                // (the four channels' groups, once per vector: one division when the group size is a multiple of four)
+                int grp[4];
+                grp[0] = i / conv.group_size;
+                if (conv.group_size % 4 == 0) {
+                    grp[1] = grp[2] = grp[3] = grp[0];
+                } else {
+#pragma unroll
+                    for (int e = 1; e < 4; e++) grp[e] = (i + e) / conv.group_size;
+                }
                 for (int tap = 0; tap < ks && tap <= t; tap++) {
                     const f4 b = *reinterpret_cast<const f4 *>(base1 + static_cast<size_t>(tap) * n + i);
                     const f4 src = *reinterpret_cast<const f4 *>(add + static_cast<size_t>(t - tap) * n + i);
                     const float *dg = dyn_t + static_cast<size_t>(tap) * n_groups;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) acc[e] = __builtin_fmaf(b[e] + dg[(i + e) / conv.group_size], src[e], acc[e]);
+                    for (int e = 0; e < 4; e++) acc[e] = __builtin_fmaf(b[e] + dg[grp[e]], src[e], acc[e]);
                 }
                 v[j] = *reinterpret_cast<const f4 *>(xr + i) + acc;
                 *reinterpret_cast<f4 *>(xr + i) = v[j];
