@@ -614,7 +614,14 @@ static int32_t attn_rows(dflash_ctx *ctx, const void *q, int32_t q_type, const v
     // KV splits: enough workgroups to cover the chip once or twice, chunks a multiple of 32 keys and at least
     // min_chunk keys long (a split costs a partial tile per head and row).  The policy is a function of the
     // bucket alone.
-    int per_cu = bucket >= 16384 ? 2 : 1;  // short contexts: fewer splits, fewer partial tiles to merge
+    // Workgroups per CU the split aims at, in halves.  Short contexts: one (fewer splits, fewer partial tiles to merge).
+    // Long contexts: two where two workgroups' LDS rings fit a CU side by side (heads of 64 or 128); with heads of 256 a
+    // ring is 96 KB, a CU holds one workgroup, and a second round of them only halves the chunk: a workgroup's partial
+    // tiles (16 rows x its heads x head_dim floats) are then as many bytes as the keys and values it read.  Half a
+    // workgroup per CU there (16 q / 2 kv heads of 256, 40-layer verify: 5.25 -> 4.79 ms at 16 k of context with chunks
+    // of 256 keys instead of 128, 6.21 -> 5.80 ms at 32 k with 512; a quarter measured slower again).
+    const size_t ring_bytes = static_cast<size_t>(kAttnBufs) * 2 * 32 * head_dim * sizeof(_Float16);
+    int per_cu_x2 = bucket >= 16384 ? (2 * ring_bytes <= static_cast<size_t>(ctx->lds_bytes) ? 4 : 1) : 2;
     int64_t min_chunk = bucket >= 8192 ? 128 : 64;
     // A workgroup serves hw heads of a GQA group (one wave each).  What a workgroup moves is its chunk of K and V,
     // its heads' queries and their partial outputs, and one CU takes in only 20-30 KB per microsecond: at short
@@ -632,13 +639,18 @@ static int32_t attn_rows(dflash_ctx *ctx, const void *q, int32_t q_type, const v
     static const int env_per_cu = [] { const char *e = getenv("DFLASH_ATTN_PER_CU"); return e ? atoi(e) : 0; }();
     static const int env_min_chunk = [] { const char *e = getenv("DFLASH_ATTN_MIN_CHUNK"); return e ? atoi(e) : 0; }();
     static const int env_hw = [] { const char *e = getenv("DFLASH_ATTN_HW"); return e ? atoi(e) : 0; }();
-    if (env_per_cu > 0) per_cu = env_per_cu;
+    if (env_per_cu > 0) per_cu_x2 = 2 * env_per_cu;
     if (env_min_chunk > 0) min_chunk = env_min_chunk;
     if (env_hw > 0 && group % env_hw == 0) hw = env_hw;
-    if (per_cu < 1) per_cu = 1;
+    if (per_cu_x2 < 1) per_cu_x2 = 1;
     if (min_chunk < 32) min_chunk = 32;
     int n_parts = group / hw;  // workgroups per (chunk, KV head)
-    const int want = static_cast<int>((static_cast<int64_t>(per_cu) * ctx->n_cu + n_kv * n_parts - 1) / (n_kv * n_parts));
+    int want = static_cast<int>(std::max<int64_t>(
+        1, (static_cast<int64_t>(per_cu_x2) * ctx->n_cu + 2 * n_kv * n_parts - 1) / (2 * n_kv * n_parts)));
+    // (one workgroup per CU at most: beyond half the chip the chunks stay at 512 to 1024 keys - at 64 k of context 256
+    // workgroups of 512 keys took 5.79 ms per 40-layer verify where 128 of 1024 took 6.70)
+    static const int env_long_chunk = [] { const char *e = getenv("DFLASH_ATTN_LONG_CHUNK"); return e ? atoi(e) : 0; }();
+    if (per_cu_x2 == 1) want = std::max<int>(want, static_cast<int>(bucket / (env_long_chunk >= 32 ? env_long_chunk : 512)));
     // Several blocks in one launch cover the chip between them: a workgroup then serves the whole GQA group, so a chunk
     // of keys is staged once instead of group / hw times (a workgroup's LDS ring leaves no room for a second one on
     // its CU, whatever its size).  The split of the keys (want, min_chunk) stays the single block's, and a head is one
