@@ -650,7 +650,9 @@ static int32_t attn_rows(dflash_ctx *ctx, const void *q, int32_t q_type, const v
     // (one workgroup per CU at most: beyond half the chip the chunks stay at 512 to 1024 keys - at 64 k of context 256
     // workgroups of 512 keys took 5.79 ms per 40-layer verify where 128 of 1024 took 6.70)
     static const int env_long_chunk = [] { const char *e = getenv("DFLASH_ATTN_LONG_CHUNK"); return e ? atoi(e) : 0; }();
-    if (per_cu_x2 == 1) want = std::max<int>(want, static_cast<int>(bucket / (env_long_chunk >= 32 ? env_long_chunk : 512)));
+    // (at most 256 splits, which two workgroups per CU would ask for as well: the partial tiles' share of the workspace stays what it was)
+    if (per_cu_x2 == 1)
+        want = std::max<int>(want, static_cast<int>(std::min<int64_t>(256, bucket / (env_long_chunk >= 32 ? env_long_chunk : 512))));
     // Several blocks in one launch cover the chip between them: a workgroup then serves the whole GQA group, so a chunk
     // of keys is staged once instead of group / hw times (a workgroup's LDS ring leaves no room for a second one on
     // its CU, whatever its size).  The split of the keys (want, min_chunk) stays the single block's, and a head is one
