@@ -269,7 +269,7 @@ int32_t dflash_top16(dflash_ctx *ctx, const float *logits, int32_t n_rows, int64
  *   products and additions rounded separately; strict >, so the first maximum wins and candidate 0
  *   when nothing compares greater; candidates below 0 or past the successor table are skipped);
  *   the winner's predecessor row conditions the next position.  Codebooks are [n_rows][rank] rows
- *   of F32, F16, Q8_0 or Q4_K in device memory; topk_ids/topk_vals [n][top_k], sel_h [n][rank] and
+ *   of F32, F16, Q8_0 or Q4_K in device memory (data on a 2-byte boundary); topk_ids/topk_vals [n][top_k], sel_h [n][rank] and
  *   out_tokens [n] are device pointers; top_k <= 16, rank <= 1024, n <= 16.  With out_tokens_host
  *   the call waits, copies the tokens and returns DFLASH_ERR_INVALID_TOKEN if a predecessor row was
  *   out of range (the reference's BadDrafter("selector codebook row out of range")); without it the
