@@ -124,6 +124,37 @@ def test_attn_long_context(ctx, oracle, L, canaries):
     assert (out1 - 0.75).abs().max().item() < 2e-3
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("L", [16500, 40000, 70001])
+def test_attn_long_context_wide_heads(ctx, oracle, L, canaries):
+    """the end-to-end model's shape, 16 q / 2 kv heads of 256, at contexts where one LDS ring fits a CU and the split
+    aims at half a workgroup per CU with chunks of 512 to 1024 keys; oracle on one KV head, constant V over all"""
+    import torch
+
+    n_rows, n_q, n_kv, hd = 16, 16, 2, 256
+    cap = (L + n_rows + 31) // 32 * 32
+    g = torch.Generator(device="cuda").manual_seed(11)
+    q = torch.randn((n_rows, n_q, hd), device="cuda", generator=g).half()
+    k = torch.randn((cap, n_kv, hd), device="cuda", generator=g).half()
+    vt = torch.randn((n_kv, hd, cap), device="cuda", generator=g).half()
+    scale = 1.0 / math.sqrt(hd)
+    got = ctx.attn_verify_block(q, k, vt, L, scale, v_transposed=True)
+    assert torch.isfinite(got).all()
+    h0 = 1
+    qn = q[:, 8 * h0: 8 * h0 + 8].float().cpu().numpy()
+    kn = k[: L + n_rows, h0: h0 + 1].cpu().numpy()
+    vn = vt[h0, :, : L + n_rows].t().contiguous().unsqueeze(1).cpu().numpy()
+    want = oracle.attn_verify_block(qn, kn, vn, L, scale)
+    check(got[:, 8 * h0: 8 * h0 + 8].cpu().numpy(), want, f"wide heads L={L}")
+    ones = torch.full_like(vt, -1.25)
+    out1 = ctx.attn_verify_block(q, k, ones, L, scale, v_transposed=True)
+    assert (out1 + 1.25).abs().max().item() < 2e-3
+    # a single row at the block's last position sees the same keys through the same split: the same bits
+    one = ctx.attn_verify_block(q[15:16].contiguous(), k, vt, L + 15, scale, v_transposed=True)
+    if (L + 16).bit_length() == (L + 15 + 1).bit_length():
+        assert torch.equal(one[0], got[15])
+
+
 def test_attn_guards(ctx, canaries):
     import torch
 
