@@ -577,6 +577,17 @@ __device__ unsigned long long *g_trace2 = nullptr;  // [n_wg][16 waves][4]: cycl
     do {          \
     } while (0)
 #endif
+// the norm + router kernel's stamps (debug build), one set per workgroup of its two-dimensional grid
+#ifdef DFLASH_TRACE
+#define DFL_TRR(i)                                                                                                            \
+    do {                                                                                                                      \
+        if (threadIdx.x == 0 && g_trace) g_trace[(blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();           \
+    } while (0)
+#else
+#define DFL_TRR(i) \
+    do {           \
+    } while (0)
+#endif
 
 template <int kWaves, typename XT>
 __global__ void __launch_bounds__(64 * kWaves)
@@ -2017,11 +2028,23 @@ __device__ __forceinline__ Raw8<DFLASH_TYPE_Q8_0> load_raw8<DFLASH_TYPE_Q8_0>(co
     return r;
 }
 
+// f16(d * q) for eight int8 quants.  d is an f16 value and q has eight bits, so d * q is exact in f32 and the one rounding
+// to f16 is the rounding of the exact product: a packed f16 multiply of d by q gives the same bits.  q itself is made
+// without conversions: byte q ^ 0x80 = q + 128 in the mantissa of f16 1024.0, minus 1152.0 (exact in f16), two at a time.
 template <>
 __device__ __forceinline__ half8_t convert_raw8<DFLASH_TYPE_Q8_0>(const Raw8<DFLASH_TYPE_Q8_0> &r) {
+    const uint32_t w[2] = {static_cast<uint32_t>(r.q), static_cast<uint32_t>(r.q >> 32)};
+    const half2_t d2 = splat(static_cast<_Float16>(r.d)), off = splat(static_cast<_Float16>(-1152.0f));
     half8_t v;
 #pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = static_cast<_Float16>(r.d * static_cast<float>(static_cast<int8_t>(r.q >> (8 * i))));
+    for (int j = 0; j < 2; j++) {
+        const half2_t lo = (as_half2(__builtin_amdgcn_perm(0x64646464u, w[j], 0x04010400u) ^ 0x00800080u) + off) * d2;
+        const half2_t hi = (as_half2(__builtin_amdgcn_perm(0x64646464u, w[j], 0x04030402u) ^ 0x00800080u) + off) * d2;
+        v[4 * j] = lo[0];
+        v[4 * j + 1] = lo[1];
+        v[4 * j + 2] = hi[0];
+        v[4 * j + 3] = hi[1];
+    }
     return v;
 }
 
@@ -2228,13 +2251,17 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
     const int hidden = 32 * n_steps;
     const bool first_tile = blockIdx.x == 0;
     const bool norm_wave = wave < 4;  // the norm is the work of 256 threads, as in rms_norm_kernel; the row's loads go out first
-    f4 v[2] = {f4{0, 0, 0, 0}, f4{0, 0, 0, 0}};
+    DFL_TRR(0);
+    f4 v[2] = {f4{0, 0, 0, 0}, f4{0, 0, 0, 0}}, nw[2] = {f4{0, 0, 0, 0}, f4{0, 0, 0, 0}};
     if (norm_wave) {
         const float *xr = x + static_cast<size_t>(r) * hidden, *ar = add + static_cast<size_t>(r) * hidden;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int i = 4 * (tid + 256 * j);
-            if (i < hidden) v[j] = *reinterpret_cast<const f4 *>(xr + i) + *reinterpret_cast<const f4 *>(ar + i);
+            if (i < hidden) {
+                v[j] = *reinterpret_cast<const f4 *>(xr + i) + *reinterpret_cast<const f4 *>(ar + i);
+                nw[j] = *reinterpret_cast<const f4 *>(norm_w + i);
+            }
         }
     }
     const int wp_row = n_steps * DFL_Q8_0_BYTES / 16;
@@ -2252,7 +2279,9 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
         for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
         if (lane == 0) sq_part[wave] = s;
     }
+    DFL_TRR(1);
     __syncthreads();
+    DFL_TRR(2);
     if (norm_wave) {
         float tot = 0.0f;
 #pragma unroll
@@ -2263,7 +2292,7 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
         for (int j = 0; j < 2; j++) {
             const int i = 4 * (tid + 256 * j);
             if (i < hidden) {
-                const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
+                const f4 o = v[j] * scale * nw[j];
                 if (first_tile) {
                     *reinterpret_cast<f4 *>(cur + static_cast<size_t>(r) * hidden + i) = o;
                     const f4 gw = *reinterpret_cast<const f4 *>(gate_w + i);
@@ -2280,7 +2309,9 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
             if (lane == 0) dot_part[wave] = dot;
         }
     }
+    DFL_TRR(3);
     __syncthreads();  // the row, the weight rows and the gate's partial sums are in LDS
+    DFL_TRR(4);
     if (first_tile && tid == 0) {
         float d = 0.0f;
         for (int k = 0; k < 4; k++) d += dot_part[k];
@@ -2304,12 +2335,15 @@ __global__ void __launch_bounds__(64 * kMaxSplit)
     const int ri = r & 3;
     const float mine = ri == 0 ? acc[0] : ri == 1 ? acc[1] : ri == 2 ? acc[2] : acc[3];
     if (g == ((r & 15) >> 2)) red[wave][n] = mine;
+    DFL_TRR(5);
     __syncthreads();
+    DFL_TRR(6);
     if (tid < 16 && n0 + tid < n_out) {
         float sum = 0.0f;
         for (int wv = 0; wv < kMaxSplit; wv++) sum += red[wv][tid];
         y[static_cast<size_t>(r) * n_out + n0 + tid] = sum;
     }
+    DFL_TRR(7);
 }
 
 // ----------------------------------------------------------------------------
