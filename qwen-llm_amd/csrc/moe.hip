@@ -417,6 +417,14 @@ __global__ void __launch_bounds__(256)
         }
         s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
     }
+    // (the next norm's weights are asked for here, behind the picks' rows in the order of issue - loads return in that
+    // order, and these come from further away than the rows the sum is waiting for - and ahead of the barrier)
+    f4 nw[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int i = 4 * (tid + 256 * j);
+        nw[j] = i < hidden ? *reinterpret_cast<const f4 *>(norm_w + i) : f4{0, 0, 0, 0};
+    }
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
     if ((tid & 63) == 0) sh[tid >> 6] = s;
     __syncthreads();
@@ -426,7 +434,7 @@ __global__ void __launch_bounds__(256)
     for (int j = 0; j < 4; j++) {
         const int i = 4 * (tid + 256 * j);
         if (i < hidden) {
-            const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(norm_w + i);
+            const f4 o = v[j] * scale * nw[j];
             *reinterpret_cast<f4 *>(y + static_cast<size_t>(row) * hidden + i) = o;
             // (hidden a multiple of 256 here: whole waves are inside or outside the row)
             if (y_xf)
