@@ -387,9 +387,17 @@ __global__ void __launch_bounds__(256)
     const int tid = threadIdx.x;
     const int64_t slot0 = static_cast<int64_t>(head) * 16 + row;
     const int64_t slot_stride = static_cast<int64_t>(n_q) * 16;
-    // The partial outputs of the first kPre rounds of splits are asked for BEFORE the maxima: their addresses do not
-    // depend on the weights, so the two trips to memory (maxima, then outputs) are in flight together instead of one
-    // behind the other across two barriers.  The sums below take them in the same order as the loop that follows.
+    // m* = max over splits (a thread keeps the maxima it loaded: n_splits <= 1024 = 4 per thread)
+    float m_own[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int s = tid + 256 * j;
+        m_own[j] = s < n_splits ? part_ml[(slot0 + s * slot_stride) * 2] : -INFINITY;
+    }
+    // The partial outputs of the first kPre rounds of splits are asked for right behind the maxima, before those are
+    // waited for: their addresses do not depend on the weights, so the two trips to memory are in flight together
+    // instead of one behind the other across two barriers (the maxima first: loads return in the order of their issue,
+    // and the maxima are what the first reduction needs).  The sums below take them in the order of the loop that follows.
     constexpr int kPre = 4;
     const int sl = tid >> 5, dl = tid & 31;  // split lane, dim lane
     const int n_vec = hd / 4;                // float4 per row: 16, 32 or 64
@@ -408,15 +416,7 @@ __global__ void __launch_bounds__(256)
             if (dl == 0) pre_l[i] = part_ml[(slot0 + s * slot_stride) * 2 + 1];
         }
     }
-    // m* = max over splits (a thread keeps the maxima it loaded: n_splits <= 1024 = 4 per thread)
-    float m_loc = -INFINITY;
-    float m_own[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int s = tid + 256 * j;
-        m_own[j] = s < n_splits ? part_ml[(slot0 + s * slot_stride) * 2] : -INFINITY;
-        m_loc = fmaxf(m_loc, m_own[j]);
-    }
+    float m_loc = fmaxf(fmaxf(m_own[0], m_own[1]), fmaxf(m_own[2], m_own[3]));
     for (int off = 32; off > 0; off >>= 1) m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off, 64));
     if ((tid & 63) == 0) red_l[tid >> 6] = m_loc;
     __syncthreads();
