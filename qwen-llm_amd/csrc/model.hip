@@ -121,7 +121,7 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
     if (n <= 8192 && n % 4 == 0) {
         // (vectors past the row are zeros and add nothing: a row of up to 4096 values sums exactly as with four vectors)
         constexpr int kVec = 8;
-        f4 v[kVec];
+        f4 v[kVec], wv[kVec];
         float s = 0.0f;
 #pragma unroll
         for (int j = 0; j < kVec; j++) {
@@ -129,11 +129,20 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
             v[j] = f4{0, 0, 0, 0};
             if (i < n) {
                 v[j] = *reinterpret_cast<const f4 *>(xr + i);
-                if (ar) {
-                    v[j] += *reinterpret_cast<const f4 *>(ar + i);
-                    *reinterpret_cast<f4 *>(xr + i) = v[j];
-                }
+                if (ar) v[j] += *reinterpret_cast<const f4 *>(ar + i);
             }
+        }
+        // (the weights are asked for ahead of the sum's barrier, but behind the row: vector loads return in the order of
+        // their issue, and the row is what the sum waits for)
+#pragma unroll
+        for (int j = 0; j < kVec; j++) {
+            const int i = 4 * (tid + 256 * j);
+            wv[j] = i < n ? *reinterpret_cast<const f4 *>(w + i) : f4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < kVec; j++) {
+            const int i = 4 * (tid + 256 * j);
+            if (i < n && ar) *reinterpret_cast<f4 *>(xr + i) = v[j];
             s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
         }
         s = block_sum(s, sh);
@@ -143,7 +152,7 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(float *__restrict__ x, co
         for (int j = 0; j < kVec; j++) {
             const int i = 4 * (tid + 256 * j);
             if (i < n) {
-                const f4 o = v[j] * scale * *reinterpret_cast<const f4 *>(w + i);
+                const f4 o = v[j] * scale * wv[j];
                 *reinterpret_cast<f4 *>(yr + i) = o;
                 // (the host passes y_xf only for n a multiple of 256: whole waves are inside or outside the row)
                 // (more than sixteen rows: block b of sixteen at y_xf + b * xf_stride bytes)
