@@ -107,6 +107,39 @@ def test_walk_matches_oracle_on_random_lattices(ctx, oracle, kind, n):
         assert got == want.tolist(), f"{kind} n={n} seed={seed}"
 
 
+@pytest.mark.parametrize("pred_kind,succ_kind,rank", [("q8_0", "q8_0", 32), ("q8_0", "f32", 96), ("f16", "q8_0", 160),
+                                                      ("f16", "f16", 33), ("f32", "f16", 7), ("q4_k", "q8_0", 1024)])
+def test_walk_with_rows_on_two_byte_boundaries_and_mixed_codebooks(ctx, oracle, pred_kind, succ_kind, rank):
+    """Q8_0 rows of an odd number of blocks (34 bytes each) and F16 rows of an odd rank start on 2-byte boundaries only;
+    the two codebooks may have different types; rank 1024 is the largest the walk takes."""
+    top_k, vocab, n = 16, 512, 16
+
+    def book(kind, seed, rng):
+        if kind in ("q4_k", "q8_0"):
+            qt = dfl.synth.Q4_K if kind == "q4_k" else dfl.synth.Q8_0
+            return ((dfl.TYPE_Q4_K if kind == "q4_k" else dfl.TYPE_Q8_0), (oracle.Q4_K if kind == "q4_k" else oracle.Q8_0),
+                    dfl.synth.random_weight(qt, vocab, rank, seed=seed))
+        dt = np.float16 if kind == "f16" else np.float32
+        return ((dfl.TYPE_F16 if kind == "f16" else dfl.TYPE_F32), (oracle.F16 if kind == "f16" else oracle.F32),
+                (rng.standard_normal((vocab, rank)) * 0.05).astype(dt))
+
+    for seed in range(3):
+        rng = np.random.default_rng(7000 + 10 * seed + rank)
+        pt, po, pred_rows = book(pred_kind, 2 * seed, rng)
+        st, so, succ_rows = book(succ_kind, 2 * seed + 1, rng)
+        ids = rng.integers(0, vocab, (n, top_k)).astype(np.int32)
+        ids[rng.random((n, top_k)) < 0.1] = -1
+        ids[:, 0] = rng.integers(0, vocab, n)
+        vals = np.sort(rng.standard_normal((n, top_k)).astype(np.float32), axis=1)[:, ::-1].copy()
+        sel_h = rng.standard_normal((n, rank)).astype(np.float32)
+        carry = int(rng.integers(0, vocab))
+        pc, k1 = oracle.make_codebook(po, pred_rows, rank)
+        sc, k2 = oracle.make_codebook(so, succ_rows, rank)
+        want, _, _ = oracle.select_draft_path(pc, sc, top_k, rank, carry, n, ids, vals, sel_h)
+        got = walk_gpu(ctx, (pt, pred_rows), (st, succ_rows), rank, carry, ids, vals, sel_h)
+        assert got == want.tolist(), f"{pred_kind}/{succ_kind} rank={rank} seed={seed}"
+
+
 @pytest.mark.parametrize("kind", ["q4_k", "f32"])
 def test_sampled_walk_matches_oracle(ctx, oracle, kind):
     """draft_block_sampled (metal_dflash.rs:17268-17415): tokens, the sparse proposals (candidate token ids in
