@@ -417,6 +417,27 @@ def e2e_speculative(ctx, n_generate, sweep, log, prompt_len=2048, dflash2=True):
             "tokens_equal_serial_greedy": sum(int(a == b) for a, b in zip(tokens, cont)), "tokens": len(tokens)}
         log(f"e2e: DFlash-2 drafter, forced k={k}: {res['dflash2']}")
         del head2
+        # ... and at the block size the released DFlash-2 drafters use, 8: all seven drafts of a block accepted
+        d8cfg = dfl.DraftConfig(n_layers=5, hidden=2048, n_q=16, n_kv=2, head_dim=256, ffn=6144, block_size=8, n_taps=3,
+                                conv_kernel_size=2, conv_group_size=64, selector_rank=256, selector_top_k=16)
+        head8 = dfl.DraftHead(ctx, d8cfg, dfl.synth_draft_weights_device(d8cfg, 1, "cuda", vocab=cfg.vocab))
+        dec = dfl.SpeculativeDecoder(ctx, target, head8, taps, cap, mask)
+        first = dec.prefill(prompt)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        tokens, st = dec.generate(first, n_generate, draft_override_fn=lambda tokens, position: cont[len(tokens):len(tokens) + 7])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        dec.close()
+        res["dflash2_block8"] = {
+            "drafter": "the same DFlash-2 drafter with blocks of 8", "forced_k": 7,
+            "accepted_tokens_per_s": (len(tokens) - 1) / dt, "steps": st["spec_steps"],
+            "mean_accept_len": st["accepted_drafts"] / max(st["spec_steps"], 1),
+            "ms_per_step": dt * 1e3 / max(st["spec_steps"], 1), "draft_ms": st["draft_ms"] / st["spec_steps"],
+            "verify_ms": st["verify_ms"] / st["spec_steps"],
+            "tokens_equal_serial_greedy": sum(int(a == b) for a, b in zip(tokens, cont)), "tokens": len(tokens)}
+        log(f"e2e: DFlash-2 drafter, blocks of 8: {res['dflash2_block8']}")
+        del head8
 
     # Stochastic acceptance (sampler coupled to deterministic drafts), forced the same way: the serial sampler's own
     # stream (temperature 0.7, top-k 20, top-p 0.95, one draw per token, through the same kernels) supplies the first
